@@ -1,0 +1,158 @@
+/*
+ * C ABI of the MI355X articulation-step library (libnuka_hip.so): the subset of the reference's stable C surface
+ * (src/include/nuka/nuka.h) that drives the batched articulation step, with the same names, argument meaning
+ * and error behaviour.  Plain pointers and sizes only.
+ *
+ * Each entry cites the reference interface it replaces.  `nuka_world_create_from_template` stands where
+ * `nuka_world_create_from_scene` stands in the reference: this library has no scene importer, so the caller
+ * passes the cooked-template inputs (what SceneIR -> CookToModel produces) directly.
+ */
+#ifndef NUKA_HIP_H_
+#define NUKA_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "nuka_phi.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* nuka.h:22-32 (the device-error code keeps the reference's numeric value 3) */
+typedef enum nuka_result_t {
+    NUKA_RESULT_OK = 0,
+    NUKA_RESULT_INVALID_ARG = 1,
+    NUKA_RESULT_NULL_HANDLE = 2,
+    NUKA_RESULT_DEVICE_ERROR = 3,
+    NUKA_RESULT_OUT_OF_MEMORY = 6,
+    NUKA_RESULT_NOT_SUPPORTED = 7,
+    NUKA_RESULT_INTERNAL = 100
+} nuka_result_t;
+
+typedef struct nuka_device_t* nuka_device_handle;
+typedef struct nuka_world_t* nuka_world_handle;
+
+/* nuka.h:40-44 */
+const char* nuka_result_message(nuka_result_t result);
+const char* nuka_last_error_message(void);
+
+/* nuka.h:46-55.  `stream` non-null is a borrowed hipStream_t; null creates an owned stream at default priority. */
+typedef struct nuka_device_desc_t {
+    uint32_t gpu_index;
+    void* stream;
+    uint8_t backend_selection_layer_enabled;
+} nuka_device_desc_t;
+nuka_result_t nuka_device_create(const nuka_device_desc_t* desc, nuka_device_handle* out);
+void nuka_device_destroy(nuka_device_handle device);
+/* The PHI backend a device owns (src/c_abi/internal.hpp:57-69 DeviceRecord). */
+nuka_phi_backend* nuka_device_backend(nuka_device_handle device);
+
+/* Cook inputs of one environment (src/runtime/articulation/articulation_state.cpp:345-435 BuildArticulationHostState,
+ * src/scene/cook/cook_to_model.cpp collidable rows).  Arrays are per link / per collidable row. */
+typedef struct nuka_template_desc_t {
+    uint32_t struct_size;
+    uint32_t link_count;
+    uint32_t body_count;
+    uint32_t profile_count;
+    uint32_t max_contacts_per_env;   /* contact slots per env; 0 => admitted collidable pairs of the template */
+    uint32_t reserved0;
+    const uint8_t* joint_type;       /* phi/articulation_contract.hpp:8-16; link 0 is the root */
+    const uint32_t* parent_link;     /* ~0u for the root */
+    const float* joint_axis;         /* [link][3], in the child joint frame */
+    const float* parent_offset;      /* [link][3], nullable */
+    const float* link_local_pose;    /* [link][7] px py pz qw qx qy qz, parent to child at q = 0 */
+    const float* link_inertial_frame;/* [link][7] */
+    const float* link_mass;          /* [link] */
+    const float* link_diag_inertia;  /* [link][3] */
+    const float* joint_damping;      /* [link], nullable */
+    const float* joint_armature;     /* [link], nullable */
+    const float* joint_stiffness;    /* [link], nullable */
+    const float* joint_spring_reference; /* [link], nullable */
+    const uint32_t* body_role;       /* 0 static, 1 the link's own body row, 2 extra collidable of a link */
+    const uint32_t* body_link;       /* owning link for roles 1 and 2 */
+    const float* body_local;         /* [row][7]: world pose (static) or pose in the owning link's frame */
+    const uint32_t* shape_kind;      /* collision/shape_kind.hpp:9-18; ~0u for no shape */
+    const float* shape_params;       /* [row][4] */
+    const uint32_t* shape_contype;
+    const uint32_t* shape_conaffinity;
+    const uint32_t* shape_group;
+    const uint32_t* shape_profile;   /* friction profile row, ~0u for the default (mu 1) */
+    const float* profile_mu;         /* [profile][2] */
+} nuka_template_desc_t;
+
+/* nuka.h:57-173 nuka_world_desc_t; zero keeps the default of the same reference field. */
+typedef struct nuka_world_desc_t {
+    uint32_t struct_size;
+    uint32_t env_count;
+    float fixed_dt;                  /* 0 => 1/240 */
+    float gravity[3];
+    uint32_t solver_vel_iters;       /* 0 => 10 (op_schema.hpp:598) */
+    uint32_t solver_pos_iters;       /* 0 => 4; ~0u => no position pass */
+    float solver_contact_margin;
+    float solver_pos_beta;           /* 0 => 0.3 */
+    float solver_pos_slop;           /* 0 => 1e-3 */
+    float solver_velocity_tolerance; /* 0 => 1e-5 (op_schema.hpp:663) */
+    float solver_baumgarte_max_velocity;   /* 0 => 3e38 */
+    float solver_overlap_recovery_velocity;
+} nuka_world_desc_t;
+
+/* nuka.h:175 nuka_world_create_from_scene */
+nuka_result_t nuka_world_create_from_template(nuka_device_handle device, const nuka_template_desc_t* tmpl,
+                                              const nuka_world_desc_t* desc, nuka_world_handle* out);
+void nuka_world_destroy(nuka_world_handle world);            /* nuka.h:253 */
+nuka_result_t nuka_world_step(nuka_world_handle world);      /* nuka.h:254, src/c_abi/world.cpp:696-698 */
+nuka_result_t nuka_world_step_n(nuka_world_handle world, uint32_t step_count);   /* nuka.h:255, world.cpp:700-731 */
+
+/* nuka.h:257-279 */
+typedef enum nuka_execution_mode_t { NUKA_EXECUTION_EAGER = 0, NUKA_EXECUTION_GRAPH = 1 } nuka_execution_mode_t;
+nuka_result_t nuka_world_set_execution_mode(nuka_world_handle world, nuka_execution_mode_t mode);
+nuka_result_t nuka_world_set_velocity_iterations(nuka_world_handle world, uint32_t iterations);   /* nuka.h:289 */
+nuka_result_t nuka_world_get_velocity_iterations(nuka_world_handle world, uint32_t* out_iterations);
+nuka_result_t nuka_world_synchronize(nuka_world_handle world);   /* nuka.h:376 */
+nuka_result_t nuka_world_reset(nuka_world_handle world);         /* nuka.h:380 */
+
+/* nk::World::DispatchOp (src/nk/pipeline/world.hpp): one op of the pipeline with the pipeline's own parameters.
+ * `variant` 1 on ArticulationDynamics dispatches it with integrate_velocity = 0, the probe
+ * tests/oracle/featherstone_oracle_harness.cpp:174-182 uses. */
+nuka_result_t nuka_world_dispatch_op(nuka_world_handle world, uint16_t op, uint32_t variant);
+
+/* Fields are named as in src/nk/model/fields.yaml. */
+typedef uint32_t nuka_state_field_t;
+/* ~0u when the library serves no field of that name. */
+nuka_state_field_t nuka_field_from_name(const char* name);
+const char* nuka_field_names(void);   /* comma separated */
+
+/* nuka.h:1158-1168 */
+typedef struct nuka_buffer_view_t {
+    void* device_ptr;
+    size_t element_count;
+    uint32_t element_stride_bytes;
+    uint8_t dtype;   /* 0 float32, 1 uint32, 2 uint64, 3 uint8 */
+} nuka_buffer_view_t;
+nuka_result_t nuka_world_get_buffer_view(nuka_world_handle world, nuka_state_field_t field, nuka_buffer_view_t* out);
+/* nuka.h:1181-1188: byte transfers relative to the field's base; out-of-range is INVALID_ARG, never a clamp. */
+nuka_result_t nuka_world_upload_field(nuka_world_handle world, nuka_state_field_t field, const void* bytes, size_t nbytes,
+                                      size_t byte_offset);
+nuka_result_t nuka_world_download_field(nuka_world_handle world, nuka_state_field_t field, void* bytes, size_t nbytes,
+                                        size_t byte_offset);
+
+/* Counts of the cooked world. */
+typedef struct nuka_world_info_t {
+    uint32_t env_count, links_per_env, bodies_per_env, dof, max_dof, contact_slots_per_env, rows_per_env, op_count;
+} nuka_world_info_t;
+nuka_result_t nuka_world_get_info(nuka_world_handle world, nuka_world_info_t* out);
+
+/* Timing on the world's own stream with device events, as tests/perf/test_go2_4096env_step_time.cpp:118-137
+ * (back-to-back steps, one wait at the end) and, per op, as the eager profiler behind NUKA_STEP_TIMING
+ * (src/phi/backend_cuda/cuda_backend.cu:78-120, 188-221). */
+nuka_result_t nuka_world_time_steps(nuka_world_handle world, uint32_t step_count, float* out_total_ms);
+/* out_ms has one slot per pipeline op (nuka_world_info_t::op_count); out_ops receives their op ids. */
+nuka_result_t nuka_world_profile_ops(nuka_world_handle world, uint32_t step_count, float* out_ms, uint16_t* out_ops);
+/* Device-to-device copy of `bytes` bytes repeated `repeats` times on the world's stream; the streaming-copy ceiling. */
+nuka_result_t nuka_device_copy_bandwidth(nuka_device_handle device, size_t bytes, uint32_t repeats, float* out_gb_per_s);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,203 @@
+"""MI355X-native batched articulation step for Nuka-Physics: Python host layer over the C ABI of libnuka_hip.so.
+
+The package directory name carries a hyphen, so load it by path (see __graft_entry__.load_package) or put its parent
+on sys.path under the module name ``nuka_physics_amd``.  Everything computes in the HIP library; there is no CPU
+fallback, and a missing library or GPU raises.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+from . import abi, synthetic  # noqa: F401
+from .abi import BufferViewC, TemplateDescC, WorldDescC
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libnuka_hip.so")
+
+_DTYPES = {0: np.float32, 1: np.uint32, 2: np.uint64, 3: np.uint8}
+
+
+class NukaError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(f"nuka result {code}: {message}")
+        self.code = code
+
+
+class WorldInfoC(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("env_count", "links_per_env", "bodies_per_env", "dof", "max_dof",
+                                          "contact_slots_per_env", "rows_per_env", "op_count")]
+
+
+class DeviceDescC(C.Structure):
+    _fields_ = [("gpu_index", C.c_uint32), ("stream", C.c_void_p), ("backend_selection_layer_enabled", C.c_uint8)]
+
+
+EXPORTS = [
+    "nuka_result_message", "nuka_last_error_message", "nuka_device_create", "nuka_device_destroy", "nuka_device_backend",
+    "nuka_world_create_from_template", "nuka_world_destroy", "nuka_world_step", "nuka_world_step_n",
+    "nuka_world_set_execution_mode", "nuka_world_set_velocity_iterations", "nuka_world_get_velocity_iterations",
+    "nuka_world_synchronize", "nuka_world_reset", "nuka_world_dispatch_op", "nuka_field_from_name", "nuka_field_names",
+    "nuka_world_get_buffer_view", "nuka_world_upload_field", "nuka_world_download_field", "nuka_world_get_info",
+    "nuka_world_time_steps", "nuka_world_profile_ops", "nuka_device_copy_bandwidth", "nuka_hip_register_backend_entry",
+    "nuka_hip_op_count", "nuka_hip_op_name", "nuka_hip_op_from_name",
+]
+
+
+def build(force=False):
+    """Compiles csrc/*.hip for gfx950 into lib/libnuka_hip.so (hipcc cross-compiles without a GPU)."""
+    cmd = ["make", "-C", os.path.join(HERE, "csrc"), "-j8"] + (["-B"] if force else [])
+    subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.PIPE)
+
+
+_lib = None
+
+
+def lib():
+    """The loaded C-ABI library; raises when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(f"{LIB_PATH} is missing: run __graft_entry__.build() first")
+        L = C.CDLL(LIB_PATH)
+        L.nuka_result_message.restype = C.c_char_p
+        L.nuka_last_error_message.restype = C.c_char_p
+        L.nuka_field_names.restype = C.c_char_p
+        L.nuka_hip_op_name.restype = C.c_char_p
+        L.nuka_hip_op_name.argtypes = [C.c_uint16]
+        L.nuka_hip_op_from_name.argtypes = [C.c_char_p]
+        L.nuka_hip_register_backend_entry.restype = C.c_void_p
+        L.nuka_device_backend.restype = C.c_void_p
+        L.nuka_device_backend.argtypes = [C.c_void_p]
+        L.nuka_device_create.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        L.nuka_device_destroy.argtypes = [C.c_void_p]
+        L.nuka_world_create_from_template.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]
+        L.nuka_world_destroy.argtypes = [C.c_void_p]
+        L.nuka_world_step.argtypes = [C.c_void_p]
+        L.nuka_world_step_n.argtypes = [C.c_void_p, C.c_uint32]
+        L.nuka_world_set_execution_mode.argtypes = [C.c_void_p, C.c_int]
+        L.nuka_world_set_velocity_iterations.argtypes = [C.c_void_p, C.c_uint32]
+        L.nuka_world_get_velocity_iterations.argtypes = [C.c_void_p, C.POINTER(C.c_uint32)]
+        L.nuka_world_synchronize.argtypes = [C.c_void_p]
+        L.nuka_world_reset.argtypes = [C.c_void_p]
+        L.nuka_world_dispatch_op.argtypes = [C.c_void_p, C.c_uint16, C.c_uint32]
+        L.nuka_field_from_name.argtypes = [C.c_char_p]
+        L.nuka_field_from_name.restype = C.c_uint32
+        L.nuka_world_get_buffer_view.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(BufferViewC)]
+        L.nuka_world_upload_field.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_size_t, C.c_size_t]
+        L.nuka_world_download_field.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_size_t, C.c_size_t]
+        L.nuka_world_get_info.argtypes = [C.c_void_p, C.POINTER(WorldInfoC)]
+        L.nuka_world_time_steps.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(C.c_float)]
+        L.nuka_world_profile_ops.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(C.c_float), C.POINTER(C.c_uint16)]
+        L.nuka_device_copy_bandwidth.argtypes = [C.c_void_p, C.c_size_t, C.c_uint32, C.POINTER(C.c_float)]
+        _lib = L
+    return _lib
+
+
+def _check(code):
+    if code != 0:
+        raise NukaError(code, lib().nuka_last_error_message().decode() or lib().nuka_result_message(code).decode())
+
+
+class Device:
+    """nuka_device_create / nuka_device_destroy."""
+
+    def __init__(self, gpu_index=0):
+        self._h = C.c_void_p()
+        desc = DeviceDescC(gpu_index, None, 0)
+        _check(lib().nuka_device_create(C.byref(desc), C.byref(self._h)))
+
+    def close(self):
+        if self._h:
+            lib().nuka_device_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def copy_bandwidth(self, nbytes=1 << 30, repeats=10):
+        out = C.c_float()
+        _check(lib().nuka_device_copy_bandwidth(self._h, nbytes, repeats, C.byref(out)))
+        return out.value
+
+
+class World:
+    """One cooked template stepped over `env_count` environments on the GPU (nuka_world_*)."""
+
+    def __init__(self, device, template, desc):
+        self.device = device
+        tdesc, keep = template.to_c()
+        self._h = C.c_void_p()
+        _check(lib().nuka_world_create_from_template(device._h, C.byref(tdesc), C.byref(desc), C.byref(self._h)))
+        del keep
+        info = WorldInfoC()
+        _check(lib().nuka_world_get_info(self._h, C.byref(info)))
+        self.info = info
+        self.env_count, self.link_count, self.dof = info.env_count, info.links_per_env, info.dof
+        self.rows_per_env, self.op_count = info.rows_per_env, info.op_count
+
+    def close(self):
+        if self._h:
+            lib().nuka_world_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def _field(self, name):
+        fid = lib().nuka_field_from_name(name.encode())
+        if fid == 0xFFFFFFFF:
+            raise KeyError(name)
+        view = BufferViewC()
+        _check(lib().nuka_world_get_buffer_view(self._h, fid, C.byref(view)))
+        return fid, view
+
+    def download(self, name):
+        fid, view = self._field(name)
+        out = np.empty(view.element_count, dtype=_DTYPES[view.dtype])
+        _check(lib().nuka_world_download_field(self._h, fid, out.ctypes.data, out.nbytes, 0))
+        return out
+
+    def upload(self, name, values):
+        fid, view = self._field(name)
+        arr = np.ascontiguousarray(np.asarray(values, dtype=_DTYPES[view.dtype]).reshape(-1))
+        if arr.size != view.element_count:
+            raise ValueError(f"{name}: expected {view.element_count} elements, got {arr.size}")
+        _check(lib().nuka_world_upload_field(self._h, fid, arr.ctypes.data, arr.nbytes, 0))
+
+    def set_state(self, state):
+        E, nl = self.env_count, self.link_count
+        self.upload("q", state["q"])
+        self.upload("qdot", state["qdot"])
+        self.upload("tau", state["tau"])
+        self.upload("base_pose", state["base_pose"])
+        lv = np.zeros((E, nl, 6), np.float32)
+        lv[:, 0, :] = state["root_twist"]
+        self.upload("link_velocity", lv)
+
+    def op(self, name, variant=0):
+        op = lib().nuka_hip_op_from_name(name.encode())
+        if op < 0:
+            raise KeyError(name)
+        _check(lib().nuka_world_dispatch_op(self._h, op, variant))
+
+    def step(self, n=1):
+        _check(lib().nuka_world_step_n(self._h, n))
+
+    def synchronize(self):
+        _check(lib().nuka_world_synchronize(self._h))
+
+    def reset(self):
+        _check(lib().nuka_world_reset(self._h))
+
+    def set_execution_mode(self, graph):
+        _check(lib().nuka_world_set_execution_mode(self._h, 1 if graph else 0))
+
+    def set_velocity_iterations(self, n):
+        _check(lib().nuka_world_set_velocity_iterations(self._h, n))
+
+    def time_steps(self, n):
+        out = C.c_float()
+        _check(lib().nuka_world_time_steps(self._h, n, C.byref(out)))
+        return out.value
+
+    def profile_ops(self, steps):
+        ms = (C.c_float * self.op_count)()
+        ops = (C.c_uint16 * self.op_count)()
+        _check(lib().nuka_world_profile_ops(self._h, steps, ms, ops))
+        return [(lib().nuka_hip_op_name(ops[i]).decode(), ms[i] / steps) for i in range(self.op_count)]

@@ -1,0 +1,149 @@
+"""ctypes mirror of include/nuka_hip.h: descriptor structs, result codes and the host-side template container.
+
+The structs are plain C layouts (pointers and sizes), the same ones the reference's ctypes caller style uses
+(examples/sim_val/nuka_cabi.py); nothing here touches torch.
+"""
+import ctypes as C
+
+import numpy as np
+
+INVALID = 0xFFFFFFFF
+
+# phi/articulation_contract.hpp:8-16
+JOINT_REVOLUTE, JOINT_PRISMATIC, JOINT_FIXED, JOINT_FLOATING = 0, 1, 2, 3
+# collision/shape_kind.hpp:9-18
+SHAPE_SPHERE, SHAPE_CAPSULE, SHAPE_BOX, SHAPE_PLANE, SHAPE_NONE = 0, 1, 2, 3, INVALID
+# collidable row roles of the template description
+ROLE_STATIC, ROLE_LINK_BODY, ROLE_PROXY = 0, 1, 2
+
+# nuka.h:22-32
+RESULT_OK, RESULT_INVALID_ARG, RESULT_NULL_HANDLE, RESULT_DEVICE_ERROR = 0, 1, 2, 3
+RESULT_OUT_OF_MEMORY, RESULT_NOT_SUPPORTED, RESULT_INTERNAL = 6, 7, 100
+
+_PF = C.POINTER(C.c_float)
+_PU = C.POINTER(C.c_uint32)
+_PB = C.POINTER(C.c_uint8)
+
+
+class TemplateDescC(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("link_count", C.c_uint32), ("body_count", C.c_uint32),
+        ("profile_count", C.c_uint32), ("max_contacts_per_env", C.c_uint32), ("reserved0", C.c_uint32),
+        ("joint_type", _PB), ("parent_link", _PU), ("joint_axis", _PF), ("parent_offset", _PF),
+        ("link_local_pose", _PF), ("link_inertial_frame", _PF), ("link_mass", _PF), ("link_diag_inertia", _PF),
+        ("joint_damping", _PF), ("joint_armature", _PF), ("joint_stiffness", _PF), ("joint_spring_reference", _PF),
+        ("body_role", _PU), ("body_link", _PU), ("body_local", _PF), ("shape_kind", _PU), ("shape_params", _PF),
+        ("shape_contype", _PU), ("shape_conaffinity", _PU), ("shape_group", _PU), ("shape_profile", _PU),
+        ("profile_mu", _PF),
+    ]
+
+
+class WorldDescC(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("env_count", C.c_uint32), ("fixed_dt", C.c_float), ("gravity", C.c_float * 3),
+        ("solver_vel_iters", C.c_uint32), ("solver_pos_iters", C.c_uint32), ("solver_contact_margin", C.c_float),
+        ("solver_pos_beta", C.c_float), ("solver_pos_slop", C.c_float), ("solver_velocity_tolerance", C.c_float),
+        ("solver_baumgarte_max_velocity", C.c_float), ("solver_overlap_recovery_velocity", C.c_float),
+    ]
+
+
+class BufferViewC(C.Structure):   # nuka.h:1158-1164
+    _fields_ = [("device_ptr", C.c_void_p), ("element_count", C.c_size_t), ("element_stride_bytes", C.c_uint32),
+                ("dtype", C.c_uint8)]
+
+
+IDENTITY7 = np.array([0, 0, 0, 1, 0, 0, 0], dtype=np.float32)
+
+
+class Template:
+    """Host-side authoring description of one environment: an articulation tree plus its collidable rows."""
+
+    def __init__(self):
+        self.links = []
+        self.bodies = []
+        self.profiles = []
+        self.max_contacts_per_env = 0
+
+    def add_link(self, joint_type, parent, axis=(0, 0, 1), local_pos=(0, 0, 0), local_rot=(1, 0, 0, 0), mass=1.0,
+                 diag_inertia=(0.01, 0.01, 0.01), com=(0, 0, 0), damping=0.0, armature=0.0, stiffness=0.0,
+                 spring_ref=0.0, parent_offset=(0, 0, 0)):
+        self.links.append(dict(joint_type=joint_type, parent=INVALID if parent is None else parent, axis=axis,
+                               local=list(local_pos) + list(local_rot), mass=mass, diag=diag_inertia,
+                               inertial=list(com) + [1, 0, 0, 0], damping=damping, armature=armature,
+                               stiffness=stiffness, spring_ref=spring_ref, parent_offset=parent_offset))
+        return len(self.links) - 1
+
+    def add_profile(self, mu1, mu2=None):
+        self.profiles.append((mu1, mu1 if mu2 is None else mu2))
+        return len(self.profiles) - 1
+
+    def add_body(self, role, link=None, kind=SHAPE_NONE, params=(0, 0, 0, 0), local_pos=(0, 0, 0),
+                 local_rot=(1, 0, 0, 0), contype=1, conaffinity=1, group=0, profile=INVALID):
+        self.bodies.append(dict(role=role, link=INVALID if link is None else link, kind=kind, params=params,
+                                local=list(local_pos) + list(local_rot), contype=contype, conaffinity=conaffinity,
+                                group=group, profile=profile))
+        return len(self.bodies) - 1
+
+    @property
+    def link_count(self):
+        return len(self.links)
+
+    @property
+    def dof(self):
+        width = {JOINT_REVOLUTE: 1, JOINT_PRISMATIC: 1, JOINT_FIXED: 0, JOINT_FLOATING: 6}
+        return sum(width[l["joint_type"]] for l in self.links)
+
+    def arrays(self):
+        f32, u32 = np.float32, np.uint32
+        L, B = self.links, self.bodies
+        return dict(
+            joint_type=np.array([l["joint_type"] for l in L], dtype=np.uint8),
+            parent_link=np.array([l["parent"] for l in L], dtype=u32),
+            joint_axis=np.array([l["axis"] for l in L], dtype=f32).reshape(-1),
+            parent_offset=np.array([l["parent_offset"] for l in L], dtype=f32).reshape(-1),
+            link_local_pose=np.array([l["local"] for l in L], dtype=f32).reshape(-1),
+            link_inertial_frame=np.array([l["inertial"] for l in L], dtype=f32).reshape(-1),
+            link_mass=np.array([l["mass"] for l in L], dtype=f32),
+            link_diag_inertia=np.array([l["diag"] for l in L], dtype=f32).reshape(-1),
+            joint_damping=np.array([l["damping"] for l in L], dtype=f32),
+            joint_armature=np.array([l["armature"] for l in L], dtype=f32),
+            joint_stiffness=np.array([l["stiffness"] for l in L], dtype=f32),
+            joint_spring_reference=np.array([l["spring_ref"] for l in L], dtype=f32),
+            body_role=np.array([b["role"] for b in B], dtype=u32),
+            body_link=np.array([b["link"] for b in B], dtype=u32),
+            body_local=np.array([b["local"] for b in B], dtype=f32).reshape(-1),
+            shape_kind=np.array([b["kind"] for b in B], dtype=u32),
+            shape_params=np.array([b["params"] for b in B], dtype=f32).reshape(-1),
+            shape_contype=np.array([b["contype"] for b in B], dtype=u32),
+            shape_conaffinity=np.array([b["conaffinity"] for b in B], dtype=u32),
+            shape_group=np.array([b["group"] for b in B], dtype=u32),
+            shape_profile=np.array([b["profile"] for b in B], dtype=u32),
+            profile_mu=np.array(self.profiles, dtype=f32).reshape(-1),
+        )
+
+    def to_c(self):
+        """Returns (TemplateDescC, keepalive) - the arrays must outlive the call that consumes the struct."""
+        a = self.arrays()
+        d = TemplateDescC()
+        d.struct_size = C.sizeof(TemplateDescC)
+        d.link_count, d.body_count, d.profile_count = len(self.links), len(self.bodies), len(self.profiles)
+        d.max_contacts_per_env = self.max_contacts_per_env
+        ctype = {np.dtype(np.float32): C.c_float, np.dtype(np.uint32): C.c_uint32, np.dtype(np.uint8): C.c_uint8}
+        for name, arr in a.items():
+            arr = np.ascontiguousarray(arr)
+            a[name] = arr
+            if arr.size:
+                setattr(d, name, arr.ctypes.data_as(C.POINTER(ctype[arr.dtype])))
+        return d, a
+
+
+def world_desc(env_count, dt, gravity=(0.0, 0.0, -9.81), vel_iters=0, pos_iters=0, contact_margin=0.0,
+               velocity_tolerance=0.0):
+    d = WorldDescC()
+    d.struct_size = C.sizeof(WorldDescC)
+    d.env_count, d.fixed_dt = env_count, dt
+    d.gravity[0], d.gravity[1], d.gravity[2] = gravity
+    d.solver_vel_iters, d.solver_pos_iters = vel_iters, pos_iters
+    d.solver_contact_margin = contact_margin
+    d.solver_velocity_tolerance = velocity_tolerance
+    return d

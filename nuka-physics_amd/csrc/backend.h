@@ -1,0 +1,22 @@
+// Internal interface between the PHI-shaped backend (backend.hip) and the host world (world.hip).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "../../include/nuka_phi.h"
+#include "nk_types.h"
+
+namespace nkh {
+
+// A backend on `device`; `borrowed_stream` non-null is used as is, else an owned stream at default priority.
+void* CreateBackend(int device, void* borrowed_stream);
+hipStream_t BackendStream(void* backend);
+nuka_phi_buffer_type* BackendDeviceBufferType(void* backend);
+nuka_phi_buffer_type* BackendHostBufferType(void* backend);
+bool BackendSupportsOp(NkOp op);
+// Raises the dynamic-LDS limit of the wide kernels once, outside any stream capture.
+void InitArticulationKernels();
+void InitSolverKernels();
+uint32_t SolverHeadCapacity(const ModelView& m, uint32_t slots, size_t lds_budget_bytes);
+
+}  // namespace nkh

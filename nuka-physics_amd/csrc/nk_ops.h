@@ -1,0 +1,30 @@
+// Op entry points of the HIP backend.  Each has the reference's OpFn shape
+// (src/phi/backend_cuda/ops/registry.cuh:27): Status(const ModelView&, const DataView&, const void* params, stream).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "nk_types.h"
+
+namespace nkh {
+
+using OpFn = Status (*)(const ModelView&, const DataView&, const void*, hipStream_t);
+
+Status OpFkWorldPoses(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpArticulationDynamics(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpIntegratePosition(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpFkLinkVelocities(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpApplyDrives(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpIntegrateVelocity(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpSyncLinkBodyPose(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpBuildAabbs(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpLbvhBuild(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpLbvhQueryPairs(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpNarrowphasePrimitives(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpNarrowphaseHeightfield(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpAssembleRows(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpContactWarmStart(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpBlockDescentSolve(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpSnapshotStepVelocity(const ModelView&, const DataView&, const void*, hipStream_t);
+
+}  // namespace nkh

@@ -1,0 +1,577 @@
+// Articulation ops for gfx950: forward kinematics, forward dynamics (RNEA bias + CRBA + LDL^T solve), position
+// integration and link twists.  One 64-lane wavefront owns one environment: lanes are links in the tree sweeps,
+// matrix entries in the 6x6 inertia pushes, and matrix rows in the factorisation; every per-link quantity of the
+// environment lives in LDS between the sweeps and reaches HBM once, in contiguous env-major blocks.
+//
+// Replaces src/phi/backend_cuda/ops/articulation.cu (UpdateWorldLinkPosesKernel :1561-1596,
+// ArticulationDynamicsKernel :505-645, IntegratePositionArticulationKernel :764-791, FkLinkVelocitiesKernel
+// :647-689) and articulation_mass.cuh (ComputeArticulationMass :124-253, FactorMass :269-335,
+// SolveMassBlock :357-396).
+#include "nk_device_math.h"
+#include "backend.h"
+#include "nk_ops.h"
+
+namespace nkh {
+
+namespace {
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ V3 load3(const float* p) { return V3{p[0], p[1], p[2]}; }
+
+// kinematics.cuh:25-42 JointRelativeFrame (revolute / prismatic / fixed)
+__device__ Xf joint_relative_frame(uint8_t type, V3 axis, Xf local, V3 parent_offset, float coordinate) {
+    Xf result = local;
+    result.p = add3(local.p, parent_offset);
+    const float l = dot3(axis, axis);
+    axis = l > 1.0e-12f ? scale3(axis, rsqrt_exact(l)) : V3{0.0f, 0.0f, 0.0f};
+    if (type == kRevolute) {
+        const float half = 0.5f * coordinate;
+        const float sine = sinf(half);
+        const Q4 turn{cosf(half), axis.x * sine, axis.y * sine, axis.z * sine};
+        result.r = qnormalize_le(qmul(local.r, turn), 1.0e-12f);
+    } else if (type == kPrismatic) {
+        result.p = add3(result.p, rotate_normalized(local.r, scale3(axis, coordinate)));
+    }
+    return result;
+}
+
+// articulation.cu:91-124
+__device__ void mat3_from_quat(Q4 q, float* m) {
+    const float n = q.w * q.w + q.x * q.x + q.y * q.y + q.z * q.z;
+    if (n <= 1.0e-12f) {
+        m[0] = 1; m[1] = 0; m[2] = 0; m[3] = 0; m[4] = 1; m[5] = 0; m[6] = 0; m[7] = 0; m[8] = 1;
+        return;
+    }
+    const float inv = rsqrt_exact(n);
+    q.w *= inv; q.x *= inv; q.y *= inv; q.z *= inv;
+    const float xx = q.x * q.x, yy = q.y * q.y, zz = q.z * q.z, xy = q.x * q.y, xz = q.x * q.z, yz = q.y * q.z;
+    const float wx = q.w * q.x, wy = q.w * q.y, wz = q.w * q.z;
+    m[0] = 1.0f - 2.0f * (yy + zz); m[1] = 2.0f * (xy - wz); m[2] = 2.0f * (xz + wy);
+    m[3] = 2.0f * (xy + wz); m[4] = 1.0f - 2.0f * (xx + zz); m[5] = 2.0f * (yz - wx);
+    m[6] = 2.0f * (xz - wy); m[7] = 2.0f * (yz + wx); m[8] = 1.0f - 2.0f * (xx + yy);
+}
+
+// articulation.cu:126-147
+__device__ void mat3_axis_angle(V3 axis, float angle, float* m) {
+    const float l = dot3(axis, axis);
+    if (l <= 1.0e-12f) {
+        m[0] = 1; m[1] = 0; m[2] = 0; m[3] = 0; m[4] = 1; m[5] = 0; m[6] = 0; m[7] = 0; m[8] = 1;
+        return;
+    }
+    axis = scale3(axis, rsqrt_exact(l));
+    const float c = cosf(angle), s = sinf(angle), t = 1.0f - c;
+    m[0] = t * axis.x * axis.x + c; m[1] = t * axis.x * axis.y - s * axis.z; m[2] = t * axis.x * axis.z + s * axis.y;
+    m[3] = t * axis.x * axis.y + s * axis.z; m[4] = t * axis.y * axis.y + c; m[5] = t * axis.y * axis.z - s * axis.x;
+    m[6] = t * axis.x * axis.z - s * axis.y; m[7] = t * axis.y * axis.z + s * axis.x; m[8] = t * axis.z * axis.z + c;
+}
+
+__device__ void mat3_mul(const float* a, const float* b, float* out) {
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int c = 0; c < 3; ++c) out[r * 3 + c] = a[r * 3] * b[c] + a[r * 3 + 1] * b[c + 3] + a[r * 3 + 2] * b[c + 6];
+}
+
+// articulation.cu:149-171: X = [[E, 0], [-E skew(t), E]] written to a 36-float LDS tile
+__device__ void store_motion_transform(const float* E, V3 t, float* X) {
+    const float skew[9] = {0.0f, -t.z, t.y, t.z, 0.0f, -t.x, -t.y, t.x, 0.0f};
+    float ll[9];
+    mat3_mul(E, skew, ll);
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int c = 0; c < 3; ++c) {
+            X[r * 6 + c] = E[r * 3 + c];
+            X[r * 6 + c + 3] = 0.0f;
+            X[(r + 3) * 6 + c] = -ll[r * 3 + c];
+            X[(r + 3) * 6 + c + 3] = E[r * 3 + c];
+        }
+}
+
+// articulation.cu:259-277 JointTransform
+__device__ void joint_transform(const ModelView& m, uint32_t link, float q, float* X) {
+    const uint8_t type = m.joint_type[link];
+    const V3 axis = load3(m.joint_axis + 3u * link);
+    const Xf local = load_xf(m.link_local_pose + 7u * link);
+    const V3 offset = load3(m.parent_offset + 3u * link);
+    float joint[9] = {1, 0, 0, 0, 1, 0, 0, 0, 1};
+    V3 translation = add3(local.p, offset);
+    if (type == kRevolute) mat3_axis_angle(axis, q, joint);
+    else if (type == kPrismatic) translation = joint_relative_frame(type, axis, local, offset, q).p;
+    float lr[9], rot[9], E[9];
+    mat3_from_quat(local.r, lr);
+    mat3_mul(lr, joint, rot);
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int c = 0; c < 3; ++c) E[r * 3 + c] = rot[c * 3 + r];
+    store_motion_transform(E, translation, X);
+}
+
+// articulation.cu:194-211
+__device__ void motion_subspace(uint8_t type, V3 axis, float* s) {
+#pragma unroll
+    for (int i = 0; i < 6; ++i) s[i] = 0.0f;
+    const float l = dot3(axis, axis);
+    if (l > 1.0e-12f) axis = scale3(axis, rsqrt_exact(l));
+    if (type == kRevolute) { s[0] = axis.x; s[1] = axis.y; s[2] = axis.z; }
+    else if (type == kPrismatic) { s[3] = axis.x; s[4] = axis.y; s[5] = axis.z; }
+}
+
+// ---- FkWorldPoses ---------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(kWave) FkWorldPosesKernel(ModelView m, DataView d, uint32_t env_count) {
+    extern __shared__ float lds[];
+    const uint32_t env = blockIdx.x, lane = threadIdx.x, nl = m.links_per_env;
+    if (env >= env_count) return;
+    float* pose = lds;   // nl * 7
+    const float* q = d.q + size_t{env} * nl;
+    for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
+        for (uint32_t l = lane; l < nl; l += kWave) {
+            if (m.link_tree_depth[l] != depth) continue;
+            const Xf relative = joint_relative_frame(m.joint_type[l], load3(m.joint_axis + 3u * l),
+                load_xf(m.link_local_pose + 7u * l), load3(m.parent_offset + 3u * l), q[l]);
+            const uint32_t parent = m.parent_link[l];
+            Xf out;
+            if (parent == kInvalid) out = m.joint_type[l] == kFloatingBase ? load_xf(d.base_pose + size_t{env} * 7u) : relative;
+            else out = compose_frame(load_xf(pose + 7u * parent), relative);
+            store_xf(pose + 7u * l, out);
+        }
+        __syncthreads();
+    }
+    float* out = d.link_pose + size_t{env} * nl * 7u;
+    for (uint32_t e = lane; e < nl * 7u; e += kWave) out[e] = pose[e];
+}
+
+// ---- ArticulationDynamics -------------------------------------------------------------------------------
+__host__ __device__ inline uint32_t DynamicsLdsFloats(uint32_t nl, uint32_t n) {
+    return nl * (36u + 36u + 5u * 6u) + n * (n + 1u) + 2u * n + 64u;
+}
+
+__global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m, DataView d, ArticulationDynamicsParams p,
+                                                                   uint32_t env_count) {
+    extern __shared__ float lds[];
+    const uint32_t env = blockIdx.x, lane = threadIdx.x, nl = m.links_per_env, n = m.dof, stride = m.max_dof;
+    if (env >= env_count) return;
+    float* xup = lds;
+    float* ic = xup + nl * 36u;
+    float* S = ic + nl * 36u;
+    float* vb = S + nl * 6u;
+    float* v = vb + nl * 6u;
+    float* a = v + nl * 6u;
+    float* pf = a + nl * 6u;
+    float* A = pf + nl * 6u;          // n x (n + 1): mass matrix, then its factor
+    float* vel = A + n * (n + 1u);
+    float* acc = vel + n;
+    float* tmp = acc + n;             // 36 floats of the inertia push, padded to 64
+    const uint32_t ld = n + 1u;
+    const size_t lbase = size_t{env} * nl;
+    const float* q = d.q + lbase;
+    float* qd = d.qdot + lbase;
+    const V3 gravity{p.gravity[0], p.gravity[1], p.gravity[2]};
+    const Q4 base_rot = load_xf(d.base_pose + size_t{env} * 7u).r;
+
+    // link twists of the state enter LDS (a floating root's twist is state; the rest is rebuilt)
+    for (uint32_t e = lane; e < nl * 6u; e += kWave) v[e] = d.link_velocity[lbase * 6u + e];
+    // joint transforms and motion subspaces (articulation.cu:318-332)
+    for (uint32_t l = lane; l < nl; l += kWave) {
+        if (m.parent_link[l] == kInvalid && m.joint_type[l] == kFloatingBase) {
+            const float id[9] = {1, 0, 0, 0, 1, 0, 0, 0, 1};
+            store_motion_transform(id, V3{0.0f, 0.0f, 0.0f}, xup + 36u * l);
+#pragma unroll
+            for (int i = 0; i < 6; ++i) { S[6u * l + i] = 0.0f; vb[6u * l + i] = 0.0f; }
+            continue;
+        }
+        joint_transform(m, l, q[l], xup + 36u * l);
+        motion_subspace(m.joint_type[l], load3(m.joint_axis + 3u * l), S + 6u * l);
+    }
+    __syncthreads();
+    // velocities root to leaf (:334-363)
+    for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
+        for (uint32_t l = lane; l < nl; l += kWave) {
+            if (m.link_tree_depth[l] != depth) continue;
+            const uint32_t parent = m.parent_link[l];
+            if (parent == kInvalid && m.joint_type[l] == kFloatingBase) continue;
+            float vp[6] = {0, 0, 0, 0, 0, 0}, tp[6], jv[6], vl[6];
+            if (parent != kInvalid) {
+#pragma unroll
+                for (int i = 0; i < 6; ++i) vp[i] = v[6u * parent + i];
+            }
+            mat66_vec(xup + 36u * l, vp, tp);
+            const float qdl = qd[l];
+#pragma unroll
+            for (int i = 0; i < 6; ++i) { jv[i] = S[6u * l + i] * qdl; vl[i] = tp[i] + jv[i]; }
+#pragma unroll
+            for (int i = 0; i < 6; ++i) v[6u * l + i] = vl[i];
+            motion_cross(vl, jv, vb + 6u * l);
+        }
+        __syncthreads();
+    }
+    // p = v x* (I v) - external wrench (:364-374, 279-295)
+    for (uint32_t l = lane; l < nl; l += kWave) {
+        float vl[6], iv[6], bf[6];
+#pragma unroll
+        for (int i = 0; i < 6; ++i) vl[i] = v[6u * l + i];
+        mat66_vec(m.link_inertia + 36u * l, vl, iv);
+        force_cross(vl, iv, bf);
+        if (p.apply_link_wrench != 0u) {
+            const float* wr = d.link_wrench + (lbase + l) * 6u;
+            if (wr[0] != 0.0f || wr[1] != 0.0f || wr[2] != 0.0f || wr[3] != 0.0f || wr[4] != 0.0f || wr[5] != 0.0f) {
+                const Q4 rot = load_xf(d.link_pose + (lbase + l) * 7u).r;
+                const V3 force = rotate_inverse(rot, V3{wr[0], wr[1], wr[2]});
+                const V3 torque = rotate_inverse(rot, V3{wr[3], wr[4], wr[5]});
+                const V3 moment = add3(torque, cross3(load_xf(m.link_inertial_frame + 7u * l).p, force));
+                bf[0] -= moment.x; bf[1] -= moment.y; bf[2] -= moment.z; bf[3] -= force.x; bf[4] -= force.y; bf[5] -= force.z;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 6; ++i) pf[6u * l + i] = bf[i];
+    }
+    __syncthreads();
+    // bias accelerations with gravity as base acceleration (:526-547)
+    for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
+        for (uint32_t l = lane; l < nl; l += kWave) {
+            if (m.link_tree_depth[l] != depth) continue;
+            float al[6];
+            const uint32_t parent = m.parent_link[l];
+            if (parent != kInvalid) {
+                float ap[6];
+#pragma unroll
+                for (int i = 0; i < 6; ++i) ap[i] = a[6u * parent + i];
+                mat66_vec(xup + 36u * l, ap, al);
+            } else if (m.joint_type[l] == kFloatingBase) {
+                const V3 g = rotate_inverse(base_rot, gravity);
+                al[0] = al[1] = al[2] = 0.0f; al[3] = -g.x; al[4] = -g.y; al[5] = -g.z;
+            } else {
+                const float world[6] = {0.0f, 0.0f, 0.0f, -gravity.x, -gravity.y, -gravity.z};
+                mat66_vec(xup + 36u * l, world, al);
+            }
+#pragma unroll
+            for (int i = 0; i < 6; ++i) a[6u * l + i] = al[i] + vb[6u * l + i];
+        }
+        __syncthreads();
+    }
+    // p += I a (:548-555)
+    for (uint32_t l = lane; l < nl; l += kWave) {
+        float al[6], f[6];
+#pragma unroll
+        for (int i = 0; i < 6; ++i) al[i] = a[6u * l + i];
+        mat66_vec(m.link_inertia + 36u * l, al, f);
+#pragma unroll
+        for (int i = 0; i < 6; ++i) pf[6u * l + i] += f[i];
+    }
+    __syncthreads();
+    // leaf to root, children in CSR order (:557-569)
+    for (uint32_t remaining = m.max_depth + 1u; remaining > 0u; --remaining) {
+        for (uint32_t l = lane; l < nl; l += kWave) {
+            if (m.link_tree_depth[l] != remaining - 1u) continue;
+            for (uint32_t i = m.link_child_range[2u * l]; i < m.link_child_range[2u * l + 1u]; ++i) {
+                const uint32_t child = m.link_children[i];
+                float pc[6], f[6];
+#pragma unroll
+                for (int c = 0; c < 6; ++c) pc[c] = pf[6u * child + c];
+                mat66t_vec(xup + 36u * child, pc, f);
+#pragma unroll
+                for (int c = 0; c < 6; ++c) pf[6u * l + c] += f[c];
+            }
+        }
+        __syncthreads();
+    }
+    // generalized bias and right-hand side, lane = DoF (:570-585)
+    float* bias = d.articulation_bias + size_t{env} * stride;
+    if (lane < stride) {
+        if (lane >= n) bias[lane] = 0.0f;
+        else {
+            const uint32_t link = m.dof_link[lane], component = m.dof_component[lane];
+            const bool scalar = component == kInvalid;
+            const float velocity = scalar ? qd[link] : v[6u * link + component];
+            float b = scalar ? dot6(S + 6u * link, pf + 6u * link) : pf[6u * link + component];
+            const float damping = scalar ? m.joint_damping[link] : 0.0f;
+            const float spring = scalar ? m.joint_stiffness[link] * (q[link] - m.joint_spring_reference[link]) : 0.0f;
+            vel[lane] = velocity;
+            bias[lane] = b;
+            acc[lane] = (scalar ? d.tau[lbase + link] : 0.0f) - b - damping * velocity - spring;
+        }
+    }
+    // CRBA: composite inertias leaf to root; the push X^T Ic X runs entry-parallel on 36 lanes (articulation_mass.cuh:146-165)
+    for (uint32_t e = lane; e < nl * 36u; e += kWave) ic[e] = m.link_inertia[e];
+    for (uint32_t e = lane; e < n * ld; e += kWave) A[e] = 0.0f;
+    __syncthreads();
+    for (uint32_t depth = m.max_depth; depth > 0u; --depth) {
+        for (uint32_t l = 0u; l < nl; ++l) {
+            if (m.link_tree_depth[l] + 1u != depth) continue;
+            for (uint32_t i = m.link_child_range[2u * l]; i < m.link_child_range[2u * l + 1u]; ++i) {
+                const uint32_t child = m.link_children[i];
+                const float* X = xup + 36u * child;
+                const float* C = ic + 36u * child;
+                const uint32_t row = lane / 6u, col = lane % 6u;
+                if (lane < 36u) {
+                    float value = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < 6; ++k) value += C[row * 6u + k] * X[k * 6u + col];
+                    tmp[lane] = value;
+                }
+                __syncthreads();
+                if (lane < 36u) {
+                    float value = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < 6; ++k) value += X[k * 6u + row] * tmp[k * 6u + col];
+                    ic[36u * l + lane] += value;
+                }
+                __syncthreads();
+            }
+        }
+    }
+    const bool floating_root = m.floating_root != 0u;
+    if (floating_root && lane < 36u) A[(lane / 6u) * ld + lane % 6u] = ic[lane];
+    __syncthreads();
+    // mass columns: each jointed link pushes Ic S to the root (:183-252)
+    for (uint32_t l = lane; l < nl; l += kWave) {
+        if (joint_dof(m.joint_type[l]) == 0u) continue;
+        if (l == 0u && floating_root) continue;
+        const uint32_t dof_i = m.link_dof[l];
+        float force[6], sl[6];
+#pragma unroll
+        for (int i = 0; i < 6; ++i) sl[i] = S[6u * l + i];
+        mat66_vec(ic + 36u * l, sl, force);
+        float diagonal = dot6(sl, force);
+        diagonal += m.joint_armature[l];
+        A[dof_i * ld + dof_i] = diagonal;
+        uint32_t walk = l;
+        for (;;) {
+            const uint32_t parent = m.parent_link[walk];
+            if (parent == kInvalid) break;
+            float pushed[6];
+            mat66t_vec(xup + 36u * walk, force, pushed);
+#pragma unroll
+            for (int i = 0; i < 6; ++i) force[i] = pushed[i];
+            walk = parent;
+            if (joint_dof(m.joint_type[walk]) == 0u) continue;
+            const uint32_t dof_j = m.link_dof[walk];
+            if (walk == 0u && floating_root) {
+#pragma unroll
+                for (int b = 0; b < 6; ++b) { A[dof_i * ld + b] = force[b]; A[b * ld + dof_i] = force[b]; }
+                continue;
+            }
+            const float entry = dot6(S + 6u * walk, force);
+            A[dof_i * ld + dof_j] = entry;
+            A[dof_j * ld + dof_i] = entry;
+        }
+    }
+    __syncthreads();
+    // the dense mass tile reaches HBM once, in row-major runs
+    float* M = d.m + size_t{env} * stride * stride;
+    for (uint32_t e = lane; e < stride * stride; e += kWave) {
+        const uint32_t i = e / stride, j = e % stride;
+        M[e] = i < n && j < n ? A[i * ld + j] : 0.0f;
+    }
+    // LDL^T, right-looking, lane = row; the strict lower triangle becomes L and the diagonal D (:269-335)
+    for (uint32_t k = 0u; k < n; ++k) {
+        const float diagonal = fmaxf(A[k * ld + k], 1.0e-6f);
+        float lik = 0.0f;
+        if (lane > k && lane < n) {
+            lik = A[lane * ld + k] / diagonal;
+            A[lane * ld + k] = lik;
+        }
+        __syncthreads();
+        if (lane > k && lane < n)
+            for (uint32_t j = k + 1u; j <= lane; ++j) A[lane * ld + j] -= lik * A[j * ld + k] * diagonal;
+        if (lane == k) A[k * ld + k] = diagonal;
+        __syncthreads();
+    }
+    float* factor = d.m_factor + size_t{env} * stride * stride;
+    for (uint32_t e = lane; e < stride * stride; e += kWave) {
+        const uint32_t i = e / stride, j = e % stride;
+        if (j <= i) factor[e] = i < n ? A[i * ld + j] : (i == j ? 1.0e-6f : 0.0f);
+    }
+    // solve L D L^T x = rhs: forward by rows, scale, backward by columns (:357-396)
+    float x = lane < n ? acc[lane] : 0.0f;
+    for (uint32_t j = 0u; j < n; ++j) {
+        const float solved = wave_bcast(x, int(j));
+        if (lane > j && lane < n) x -= A[lane * ld + j] * solved;
+    }
+    if (lane < n) x = x / A[lane * ld + lane];
+    for (uint32_t end = n; end > 0u; --end) {
+        const uint32_t i = end - 1u;
+        const float value = wave_bcast(x, int(i));
+        if (lane < i) x -= A[i * ld + lane] * value;
+    }
+    if (lane < stride) d.articulation_qdd[size_t{env} * stride + lane] = lane < n ? x : 0.0f;
+    if (lane < n) acc[lane] = x;
+    __syncthreads();
+    // write back accelerations and the unconstrained velocity update (:597-615)
+    for (uint32_t l = lane; l < nl; l += kWave) {
+        const uint8_t type = m.joint_type[l];
+        float qdd = 0.0f;
+        if (joint_dof(type) == 1u) {
+            const uint32_t dof = m.link_dof[l];
+            qdd = acc[dof];
+            if (p.integrate_velocity != 0u) qd[l] = vel[dof] + p.dt * qdd;
+        }
+        d.qddot[lbase + l] = qdd;
+        if (p.integrate_velocity != 0u) {
+            float* wr = d.link_wrench + (lbase + l) * 6u;
+#pragma unroll
+            for (int i = 0; i < 6; ++i) wr[i] = 0.0f;
+        }
+    }
+    if (floating_root && p.integrate_velocity != 0u && lane < 6u) {
+        const uint32_t component = lane, i = component % 3u, j = (i + 1u) % 3u, k = (i + 2u) % 3u;
+        const float transport = component < 3u ? 0.0f : vel[j] * vel[3u + k] - vel[k] * vel[3u + j];
+        v[component] = vel[lane] + p.dt * (acc[lane] + transport);
+    }
+    __syncthreads();
+    // final link accelerations (:617-644)
+    for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
+        for (uint32_t l = lane; l < nl; l += kWave) {
+            if (m.link_tree_depth[l] != depth) continue;
+            float al[6];
+            const uint32_t parent = m.parent_link[l];
+            if (m.joint_type[l] == kFloatingBase) {
+                const V3 g = rotate_inverse(base_rot, gravity);
+#pragma unroll
+                for (int c = 0; c < 6; ++c) al[c] = acc[c];
+                al[3] -= g.x; al[4] -= g.y; al[5] -= g.z;
+            } else {
+                if (parent != kInvalid) {
+                    float ap[6];
+#pragma unroll
+                    for (int i = 0; i < 6; ++i) ap[i] = a[6u * parent + i];
+                    mat66_vec(xup + 36u * l, ap, al);
+                } else {
+                    const float world[6] = {0.0f, 0.0f, 0.0f, -gravity.x, -gravity.y, -gravity.z};
+                    mat66_vec(xup + 36u * l, world, al);
+                }
+                const float qdd = joint_dof(m.joint_type[l]) == 1u ? acc[m.link_dof[l]] : 0.0f;
+#pragma unroll
+                for (int c = 0; c < 6; ++c) al[c] += vb[6u * l + c] + S[6u * l + c] * qdd;
+            }
+#pragma unroll
+            for (int c = 0; c < 6; ++c) a[6u * l + c] = al[c];
+        }
+        __syncthreads();
+    }
+    for (uint32_t e = lane; e < nl * 6u; e += kWave) {
+        d.link_velocity[lbase * 6u + e] = v[e];
+        d.link_acceleration[lbase * 6u + e] = a[e];
+    }
+}
+
+// ---- IntegratePosition: one thread per (env, link) (articulation.cu:732-791) ------------------------------
+__global__ void IntegratePositionKernel(ModelView m, DataView d, IntegratePositionParams p) {
+    const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= p.total_link_count) return;
+    const uint32_t nl = m.links_per_env, env = gid / nl, l = gid % nl;
+    const float dt = p.dt;
+    if (p.pos_pass != 0u) d.q[gid] += (d.qdot[gid] + d.qdot_pseudo[gid]) * dt;
+    else d.q[gid] += d.qdot[gid] * dt;
+    if (m.parent_link[l] == kInvalid && m.joint_type[l] == kFloatingBase) {
+        float* rv = d.link_velocity + size_t{gid} * 6u;
+        Xf pose = load_xf(d.base_pose + size_t{env} * 7u);
+        float vv[6];
+#pragma unroll
+        for (int i = 0; i < 6; ++i) vv[i] = p.pos_pass != 0u ? rv[i] + d.link_velocity_pseudo[size_t{gid} * 6u + i] : rv[i];
+        const V3 lin_world = rotate_forward(pose.r, V3{vv[3], vv[4], vv[5]});
+        pose.p = add3(pose.p, scale3(lin_world, dt));
+        const Q4 dq{1.0f, 0.5f * vv[0] * dt, 0.5f * vv[1] * dt, 0.5f * vv[2] * dt};
+        pose.r = qnormalize_lt(qmul(pose.r, dq), 1.0e-24f);
+        const V3 turned = rotate_inverse(qnormalize_lt(dq, 1.0e-24f), V3{rv[3], rv[4], rv[5]});
+        rv[3] = turned.x; rv[4] = turned.y; rv[5] = turned.z;
+        store_xf(d.base_pose + size_t{env} * 7u, pose);
+    }
+}
+
+// ---- FkLinkVelocities (articulation.cu:647-689) ---------------------------------------------------------
+__global__ void __launch_bounds__(kWave) FkLinkVelocitiesKernel(ModelView m, DataView d, uint32_t env_count) {
+    extern __shared__ float lds[];
+    const uint32_t env = blockIdx.x, lane = threadIdx.x, nl = m.links_per_env;
+    if (env >= env_count) return;
+    float* v = lds;   // nl * 6
+    const size_t lbase = size_t{env} * nl;
+    for (uint32_t e = lane; e < nl * 6u; e += kWave) v[e] = d.link_velocity[lbase * 6u + e];
+    __syncthreads();
+    for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
+        for (uint32_t l = lane; l < nl; l += kWave) {
+            if (m.link_tree_depth[l] != depth) continue;
+            const uint32_t parent = m.parent_link[l];
+            if (parent == kInvalid && m.joint_type[l] == kFloatingBase) continue;
+            float pv[6] = {0, 0, 0, 0, 0, 0}, X[36], s[6], vl[6];
+            if (parent != kInvalid) {
+#pragma unroll
+                for (int i = 0; i < 6; ++i) pv[i] = v[6u * parent + i];
+            }
+            joint_transform(m, l, d.q[lbase + l], X);
+            motion_subspace(m.joint_type[l], load3(m.joint_axis + 3u * l), s);
+            mat66_vec(X, pv, vl);
+            const float qdl = d.qdot[lbase + l];
+#pragma unroll
+            for (int c = 0; c < 6; ++c) v[6u * l + c] = vl[c] + s[c] * qdl;
+        }
+        __syncthreads();
+    }
+    for (uint32_t e = lane; e < nl * 6u; e += kWave) d.link_velocity[lbase * 6u + e] = v[e];
+}
+
+}  // namespace
+
+// ---- op entry points ------------------------------------------------------------------------------------
+Status OpFkWorldPoses(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const FkWorldPosesParams*>(params);
+    if (p == nullptr) return Status::Failed;
+    if (p->articulation_count == 0u || p->total_link_count == 0u) return Status::Ok;
+    if (m.links_per_env == 0u || p->total_link_count != p->articulation_count * m.links_per_env) return Status::InvalidArgument;
+    const size_t lds = size_t{m.links_per_env} * 7u * sizeof(float);
+    hipLaunchKernelGGL(FkWorldPosesKernel, dim3(p->articulation_count), dim3(kWave), lds, stream, m, d, p->articulation_count);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
+Status OpArticulationDynamics(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const ArticulationDynamicsParams*>(params);
+    if (p == nullptr) return Status::Failed;
+    if (p->articulation_count == 0u || p->total_link_count == 0u) return Status::Ok;
+    if (m.dof > kMaxDof || m.dof == 0u || p->max_dof != m.max_dof ||
+        p->total_link_count != p->articulation_count * m.links_per_env) return Status::InvalidArgument;
+    const size_t lds = size_t{DynamicsLdsFloats(m.links_per_env, m.dof)} * sizeof(float);
+    if (lds > 160u * 1024u) return Status::InvalidArgument;
+    hipLaunchKernelGGL(ArticulationDynamicsKernel, dim3(p->articulation_count), dim3(kWave), lds, stream, m, d, *p,
+                       p->articulation_count);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
+Status OpIntegratePosition(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const IntegratePositionParams*>(params);
+    if (p == nullptr) return Status::Failed;
+    if (p->dt <= 0.0f || p->total_link_count == 0u) return Status::Ok;
+    const uint32_t blocks = (p->total_link_count + 255u) / 256u;
+    hipLaunchKernelGGL(IntegratePositionKernel, dim3(blocks), dim3(256), 0, stream, m, d, *p);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
+Status OpFkLinkVelocities(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const FkLinkVelocitiesParams*>(params);
+    if (p == nullptr) return Status::InvalidArgument;
+    if (p->articulation_count == 0u || p->total_link_count == 0u) return Status::Ok;
+    const size_t lds = size_t{m.links_per_env} * 6u * sizeof(float);
+    hipLaunchKernelGGL(FkLinkVelocitiesKernel, dim3(p->articulation_count), dim3(kWave), lds, stream, m, d, p->articulation_count);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
+void InitArticulationKernels() {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(ArticulationDynamicsKernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              160 * 1024);
+    (void)hipGetLastError();
+}
+
+// Torque control leaves tau as applied; free bodies do not exist on this path, so both ops only validate.
+Status OpApplyDrives(const ModelView&, const DataView&, const void* params, hipStream_t) {
+    const auto* p = static_cast<const ApplyDrivesParams*>(params);
+    if (p == nullptr || p->mode != 1u) return p == nullptr ? Status::InvalidArgument : Status::Unsupported;
+    return Status::Ok;
+}
+Status OpIntegrateVelocity(const ModelView&, const DataView&, const void* params, hipStream_t) {
+    const auto* p = static_cast<const IntegrateVelocityParams*>(params);
+    if (p == nullptr) return Status::Failed;
+    return Status::Ok;
+}
+
+}  // namespace nkh

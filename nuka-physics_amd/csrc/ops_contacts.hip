@@ -1,0 +1,565 @@
+// Contact detection and row assembly for gfx950: collidable poses, AABBs, candidate pairs in canonical (a, b)
+// order, sphere/box x plane manifolds, pair-driven contact rows and chain Jacobians.
+//
+// Elementwise stages run one thread per (env, item) on contiguous env-major fields; the stages with an order
+// inside an environment (pair emission, row-range prefix, Jacobian rows) run one wavefront per environment so the
+// order comes from lane ranks and prefix counts - no atomics, no sort, identical output every run.
+//
+// Replaces src/phi/backend_cuda/ops/sync_body_pose.cu, broadphase.cu (BuildAabbsKernel :173-270, EnvAllPairsKernel
+// :408-474 plus the canonical radix sort :478-542, 630-680), narrowphase_prims.cu (PairDrivenNarrowphaseKernel<false>
+// :181-366) and assemble_rows.cu (:122-214, 325-801, 1479-1605).
+#include "nk_device_math.h"
+#include "nk_ops.h"
+
+namespace nkh {
+
+namespace {
+
+constexpr int kWave = 64;
+
+struct ShapeRow { uint32_t kind; float p[4]; uint32_t contype, conaffinity; int32_t body_id; uint32_t group, profile; };
+
+// prims_types.cuh:55-72
+__device__ __forceinline__ ShapeRow load_shape(const float* table, uint32_t row) {
+    const float* q = table + size_t{row} * kShapeStride;
+    ShapeRow s;
+    s.kind = __float_as_uint(q[0]);
+    s.p[0] = q[1]; s.p[1] = q[2]; s.p[2] = q[3]; s.p[3] = q[4];
+    s.contype = __float_as_uint(q[5]); s.conaffinity = __float_as_uint(q[6]);
+    s.body_id = int32_t(__float_as_uint(q[8])); s.group = __float_as_uint(q[9]); s.profile = __float_as_uint(q[12]);
+    return s;
+}
+
+// collision/contact_query.hpp:17-31
+__device__ __forceinline__ float motion_radius(float base, float dt, float sa, float sb, float relax) {
+    return base + dt * (sa + sb) * (2.0f / relax);
+}
+
+// ---- SyncLinkBodyPose (sync_body_pose.cu:23-83): link-owned rows only; static rows keep their cooked pose ----
+__global__ void SyncLinkBodyPoseKernel(ModelView m, DataView d, uint32_t total_bodies) {
+    const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= total_bodies) return;
+    const uint32_t nb = m.bodies_per_env, env = gid / nb, b = gid % nb;
+    const uint32_t own = m.body_to_link[b], proxy = m.body_collidable_link[b];
+    if (own != kInvalid) {
+        if (m.link_body[own] != b) return;
+        Xf world = load_xf(d.link_pose + (size_t{env} * m.links_per_env + own) * 7u);
+        if (m.link_geom_kind[own] != 0u) world = compose_collidable(world, load_xf(m.link_geom_local + 7u * own));
+        store_xf(d.body_pose + size_t{gid} * 7u, world);
+    } else if (proxy != kInvalid && proxy < m.links_per_env) {
+        store_xf(d.body_pose + size_t{gid} * 7u,
+                 compose_collidable(load_xf(d.link_pose + (size_t{env} * m.links_per_env + proxy) * 7u),
+                                    load_xf(m.body_collidable_local + 7u * b)));
+    }
+}
+
+// broadphase.cu:154-170
+__device__ V3 rot_abs(Q4 q, V3 v) {
+    const V3 cx = rotate_raw(q, V3{1, 0, 0}), cy = rotate_raw(q, V3{0, 1, 0}), cz = rotate_raw(q, V3{0, 0, 1});
+    return V3{fabsf(cx.x) * v.x + fabsf(cy.x) * v.y + fabsf(cz.x) * v.z, fabsf(cx.y) * v.x + fabsf(cy.y) * v.y + fabsf(cz.y) * v.z,
+              fabsf(cx.z) * v.x + fabsf(cy.z) * v.y + fabsf(cz.z) * v.z};
+}
+
+// ---- BuildAabbs (broadphase.cu:173-270).  Link-owned collidables carry no body velocity on this path, so the
+// motion term of the margin is zero. ----
+__global__ void BuildAabbsKernel(ModelView m, DataView d, BuildAabbsParams p) {
+    const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= p.env_count * p.bodies_per_env) return;
+    const uint32_t b = gid % p.bodies_per_env;
+    const ShapeRow s = load_shape(m.shape_table, b);
+    const Xf xf = load_xf(d.body_pose + size_t{gid} * 7u);
+    float* lo = d.body_aabb_lo + size_t{gid} * 3u;
+    float* hi = d.body_aabb_hi + size_t{gid} * 3u;
+    V3 he{0, 0, 0};
+    if (s.kind == kShapeSphere) he = V3{s.p[0], s.p[0], s.p[0]};
+    else if (s.kind == kShapeBox) he = rot_abs(xf.r, V3{s.p[0], s.p[1], s.p[2]});
+    else if (s.kind == kShapePlane) {
+        lo[0] = lo[1] = lo[2] = -FLT_MAX; hi[0] = hi[1] = hi[2] = FLT_MAX;
+        return;
+    } else {
+        lo[0] = lo[1] = lo[2] = FLT_MAX; hi[0] = hi[1] = hi[2] = -FLT_MAX;
+        return;
+    }
+    const float mg = fmaxf(p.margin, fminf(motion_radius(p.margin, p.dt, 0.0f, 0.0f, 0.9f), p.query_reach));
+    const V3 c = xf.p;
+    lo[0] = c.x - he.x - mg; lo[1] = c.y - he.y - mg; lo[2] = c.z - he.z - mg;
+    hi[0] = c.x + he.x + mg; hi[1] = c.y + he.y + mg; hi[2] = c.z + he.z + mg;
+}
+
+// collision/shape_kind.hpp:26-33
+__device__ __forceinline__ bool shape_filter_admits(uint32_t ta, uint32_t aa, uint32_t ga_, uint32_t tb, uint32_t ab, uint32_t gb_) {
+    if (((ta & ab) | (tb & aa)) == 0u) return false;
+    const int32_t ga = int32_t(ga_), gb = int32_t(gb_);
+    return !(ga != 0 && gb != 0 && (ga > 0 ? (ga != gb && gb > 0) : ga == gb));
+}
+
+// ---- candidate pairs: one wavefront per env walks the (i, j) grid in row-major order; the ballot rank of an
+// emitting lane is its slot, which is the ascending (a, b) order the reference reaches by sorting. ----
+__global__ void __launch_bounds__(kWave) QueryPairsKernel(ModelView m, DataView d, LbvhQueryPairsParams p) {
+    const uint32_t env = blockIdx.x, lane = threadIdx.x, N = p.bodies_per_env;
+    const size_t bbase = size_t{env} * N;
+    const uint32_t capacity = min(p.rigid_slot_cap, p.max_pairs);
+    uint32_t* pairs = d.candidate_pairs + size_t{env} * p.max_contacts_per_env * 2u;
+    uint32_t count = 0u;
+    bool overflow = false;
+    for (uint32_t base = 0u; base < N * N; base += kWave) {
+        const uint32_t item = base + lane, i = item / N, j = item % N;
+        bool emit = false;
+        if (i < j && i < N) {
+            const float* alo = d.body_aabb_lo + (bbase + i) * 3u, *ahi = d.body_aabb_hi + (bbase + i) * 3u;
+            const float* blo = d.body_aabb_lo + (bbase + j) * 3u, *bhi = d.body_aabb_hi + (bbase + j) * 3u;
+            const bool overlap = !(ahi[0] < blo[0] || alo[0] > bhi[0] || ahi[1] < blo[1] || alo[1] > bhi[1] ||
+                                   ahi[2] < blo[2] || alo[2] > bhi[2]);
+            if (overlap) {
+                const ShapeRow sa = load_shape(m.shape_table, i), sb = load_shape(m.shape_table, j);
+                emit = !(sa.body_id < 0 && sb.body_id < 0) &&
+                       shape_filter_admits(sa.contype, sa.conaffinity, sa.group, sb.contype, sb.conaffinity, sb.group);
+            }
+        }
+        const uint64_t mask = __ballot(emit);
+        if (emit) {
+            const uint32_t slot = count + __popcll(mask & ((uint64_t{1} << lane) - 1u));
+            if (slot < capacity) { pairs[2u * slot] = i; pairs[2u * slot + 1u] = j; }
+            else overflow = true;
+        }
+        count += __popcll(mask);
+    }
+    overflow = __any(overflow);
+    if (lane == 0u) {
+        d.pair_count[env] = min(count, capacity);
+        const uint32_t status = d.env_status[env] & ~kEnvStatusPairOverflow;
+        d.env_status[env] = overflow ? status | kEnvStatusPairOverflow : status;
+    }
+}
+
+// ---- manifolds (collision/analytical_manifold.hpp) ------------------------------------------------------
+struct Prim { V3 cx, cy, cz, t; float radius; V3 half; };
+struct Manifold { uint32_t count; V3 position[4]; V3 normal; float penetration[4]; uint32_t key[4]; };
+
+__device__ Prim make_prim(const ShapeRow& s, Xf xf) {   // narrowphase_prims.cu:34-46
+    Prim p;
+    p.cx = rotate_raw(xf.r, V3{1, 0, 0}); p.cy = rotate_raw(xf.r, V3{0, 1, 0}); p.cz = rotate_raw(xf.r, V3{0, 0, 1});
+    p.t = xf.p; p.radius = s.p[0]; p.half = V3{s.p[0], s.p[1], s.p[2]};
+    return p;
+}
+__device__ V3 plane_normal(const Prim& plane) {   // analytical_manifold.hpp:194-198 with the +Z fallback
+    const float len = sqrtf(plane.cz.x * plane.cz.x + plane.cz.y * plane.cz.y + plane.cz.z * plane.cz.z);
+    if (len < 1.0e-12f) return V3{0, 0, 1};
+    return V3{plane.cz.x / len, plane.cz.y / len, plane.cz.z / len};
+}
+__device__ void sphere_plane(const Prim& sph, const Prim& plane, float query, Manifold* out) {   // :451-463
+    out->count = 0u;
+    const V3 n = plane_normal(plane);
+    const float signed_dist = dot3(sub3(sph.t, plane.t), n);
+    const float pen = sph.radius - signed_dist;
+    if (pen <= -query) return;
+    out->position[0] = sub3(sph.t, scale3(n, sph.radius - 0.5f * pen));
+    out->normal = n; out->penetration[0] = pen; out->key[0] = 0u; out->count = 1u;
+}
+__device__ void box_plane(const Prim& box, const Prim& plane, float query, Manifold* out) {   // :469-493, 273-311
+    out->count = 0u;
+    const V3 n = plane_normal(plane);
+    V3 position[8]; float pen[8]; uint32_t feature[8];
+    int ncand = 0;
+    for (uint32_t c = 0u; c < 8u; ++c) {
+        const float sx = (c & 1u) ? 1.0f : -1.0f, sy = (c & 2u) ? 1.0f : -1.0f, sz = (c & 4u) ? 1.0f : -1.0f;
+        const V3 l{sx * box.half.x, sy * box.half.y, sz * box.half.z};
+        const V3 corner{box.cx.x * l.x + box.cy.x * l.y + box.cz.x * l.z + box.t.x,
+                        box.cx.y * l.x + box.cy.y * l.y + box.cz.y * l.z + box.t.y,
+                        box.cx.z * l.x + box.cy.z * l.y + box.cz.z * l.z + box.t.z};
+        const float sd = dot3(sub3(corner, plane.t), n);
+        if (sd < query) {
+            position[ncand] = sub3(corner, scale3(n, 0.5f * sd));
+            pen[ncand] = -sd; feature[ncand] = c; ++ncand;
+        }
+    }
+    if (ncand <= 0) return;
+    const int keep = ncand < 4 ? ncand : 4;
+    for (int s = 0; s < keep; ++s) {
+        int best = s;
+        for (int i = s + 1; i < ncand; ++i)
+            if (pen[i] > pen[best] || (pen[i] == pen[best] && feature[i] < feature[best])) best = i;
+        const V3 tp = position[s]; position[s] = position[best]; position[best] = tp;
+        const float tf = pen[s]; pen[s] = pen[best]; pen[best] = tf;
+        const uint32_t tk = feature[s]; feature[s] = feature[best]; feature[best] = tk;
+    }
+    for (int i = 1; i < keep; ++i) {
+        const V3 kp = position[i]; const float kf = pen[i]; const uint32_t kk = feature[i];
+        int j = i - 1;
+        while (j >= 0 && feature[j] > kk) { position[j + 1] = position[j]; pen[j + 1] = pen[j]; feature[j + 1] = feature[j]; --j; }
+        position[j + 1] = kp; pen[j + 1] = kf; feature[j + 1] = kk;
+    }
+    for (int i = 0; i < keep; ++i) { out->position[i] = position[i]; out->penetration[i] = pen[i]; out->key[i] = feature[i]; }
+    out->normal = n;
+    out->count = uint32_t(keep);
+}
+
+// nk/contact/contact_identity.hpp:98-157
+__device__ __forceinline__ int32_t quantize_coord(float value) {
+    const float scaled = value * 4096.0f;
+    return int32_t(scaled >= 0.0f ? scaled + 0.5f : scaled - 0.5f);
+}
+__device__ __forceinline__ uint64_t hash_word(uint64_t hash, uint64_t word) { hash ^= word; return hash * 1099511628211ull; }
+__device__ uint64_t feature_token(uint32_t feature, V3 p) {
+    if (feature != 0xffffffffu) return 0x8000000000000000ull | uint64_t{feature};
+    uint64_t h = 1469598103934665603ull;
+    h = hash_word(h, uint32_t(quantize_coord(p.x))); h = hash_word(h, uint32_t(quantize_coord(p.y)));
+    h = hash_word(h, uint32_t(quantize_coord(p.z)));
+    return h & 0x7fffffffffffffffull;
+}
+__device__ V3 inverse_transform_point(Xf xf, V3 wp) {   // prims_types.cuh:98-105
+    const V3 v = sub3(wp, xf.p);
+    const V3 qv{-xf.r.x, -xf.r.y, -xf.r.z};
+    const V3 t = scale3(cross3(qv, v), 2.0f);
+    return add3(add3(v, scale3(t, xf.r.w)), cross3(qv, t));
+}
+
+// ---- NarrowphasePrimitives: one thread per (env, slot) (narrowphase_prims.cu:181-366, analytic route) ----
+__global__ void NarrowphaseKernel(ModelView m, DataView d, NarrowphasePrimitivesParams p) {
+    const uint32_t item = blockIdx.x * blockDim.x + threadIdx.x;
+    if (item >= p.env_count * p.rigid_slot_cap) return;
+    const uint32_t env = item / p.rigid_slot_cap, slot = item - env * p.rigid_slot_cap;
+    const size_t gid = size_t{env} * p.union_slot_count + slot;
+    const size_t bbase = size_t{env} * p.bodies_per_env;
+    const float separation = fmaxf(p.contact_margin, 0.0005f);
+    const uint32_t live = d.pair_count[env];
+    Manifold mf; mf.count = 0u; mf.normal = V3{0, 0, 1};
+    uint32_t a = 0u, b = 0u;
+    Xf xa{}, xb{};
+    if (slot < live) {
+        a = d.candidate_pairs[gid * 2u]; b = d.candidate_pairs[gid * 2u + 1u];
+        const ShapeRow sa = load_shape(m.shape_table, a), sb = load_shape(m.shape_table, b);
+        xa = load_xf(d.body_pose + (bbase + a) * 7u); xb = load_xf(d.body_pose + (bbase + b) * 7u);
+        const Prim pa = make_prim(sa, xa), pb = make_prim(sb, xb);
+        const float query = fmaxf(separation, fminf(motion_radius(2.0f * separation, p.dt, 0.0f, 0.0f, 0.9f), p.query_reach));
+        if (sa.kind == kShapeSphere && sb.kind == kShapePlane) sphere_plane(pa, pb, query, &mf);
+        else if (sa.kind == kShapeBox && sb.kind == kShapePlane) box_plane(pa, pb, query, &mf);
+        else if (sa.kind == kShapePlane && (sb.kind == kShapeSphere || sb.kind == kShapeBox)) {
+            if (sb.kind == kShapeSphere) sphere_plane(pb, pa, query, &mf); else box_plane(pb, pa, query, &mf);
+            mf.normal = V3{-mf.normal.x, -mf.normal.y, -mf.normal.z};
+        }
+        for (uint32_t i = 0u; i < mf.count; ++i) mf.penetration[i] += separation;
+    }
+    d.ucontact_count[gid] = mf.count;
+    d.ucontact_law[gid] = kContactLawSpeculative;
+    for (uint32_t i = 0u; i < mf.count; ++i) {
+        const size_t at = gid * 4u + i;
+        d.ucontact_point[3u * at] = mf.position[i].x; d.ucontact_point[3u * at + 1u] = mf.position[i].y; d.ucontact_point[3u * at + 2u] = mf.position[i].z;
+        d.ucontact_normal[3u * at] = mf.normal.x; d.ucontact_normal[3u * at + 1u] = mf.normal.y; d.ucontact_normal[3u * at + 2u] = mf.normal.z;
+        d.ucontact_depth[at] = mf.penetration[i];
+        d.ucontact_a[at] = a; d.ucontact_b[at] = b;
+        const uint32_t feature = mf.key[i] == 0u ? 0xffffffffu : mf.key[i];
+        uint64_t h = 1469598103934665603ull;
+        h = hash_word(h, feature_token(feature, inverse_transform_point(xa, mf.position[i])));
+        h = hash_word(h, feature_token(feature, inverse_transform_point(xb, mf.position[i])));
+        h = hash_word(h, i); h = hash_word(h, 0u); h = hash_word(h, 0u);
+        d.ucontact_id_pair[at] = (uint64_t{a & 0x0fffffffu} << 32u) | uint64_t{b & 0x0fffffffu};
+        d.ucontact_id_feature[at] = h;
+    }
+}
+
+// math/cuda_vec_ops.cuh:150-183
+__device__ void contact_tangent_basis(V3 normal, V3* t1, V3* t2) {
+    V3 n = normal;
+    const float l = dot3(n, n);
+    if (l > 1.0e-10f) { const float inv = rsqrt_exact(l); n = V3{n.x * inv, n.y * inv, n.z * inv}; }
+    else n = V3{0.0f, 0.0f, 1.0f};
+    V3 reference{1.0f, 0.0f, 0.0f};
+    if (fabsf(n.x) > 0.9f) reference = V3{0.0f, 1.0f, 0.0f};
+    const float proj = dot3(reference, n);
+    V3 ta{reference.x - proj * n.x, reference.y - proj * n.y, reference.z - proj * n.z};
+    const float len_sq = dot3(ta, ta);
+    if (len_sq > 1.0e-12f) { const float s = rsqrt_exact(len_sq); ta = V3{ta.x * s, ta.y * s, ta.z * s}; }
+    else ta = V3{1.0f, 0.0f, 0.0f};
+    *t1 = ta;
+    *t2 = cross3(n, ta);
+}
+
+// union_types.cuh:187-193
+__device__ __forceinline__ uint32_t contact_row_bound(uint32_t previous, uint32_t current, uint32_t contact_rows) {
+    if (previous == 0u || current == 0u) return contact_rows;
+    return min(max(previous, current) - 1u, contact_rows);
+}
+
+// nk/solve/collidable_owner.hpp:25-62 for one articulation per environment
+__device__ uint32_t resolve_side(const ModelView& m, uint32_t env, uint32_t collidable, int32_t body_id, uint32_t* index,
+                                 uint32_t* link) {
+    *index = kInvalid; *link = kInvalid;
+    if (collidable >= m.bodies_per_env) return kInvalid;
+    uint32_t body = collidable;
+    if (body_id < 0) return kSideStatic;
+    const uint32_t proxy = m.body_collidable_body[body];
+    if (proxy != kInvalid) {
+        if (proxy >= m.bodies_per_env) return kInvalid;
+        body = proxy;
+        if (m.body_collidable_body[body] != kInvalid) return kInvalid;
+    }
+    const uint32_t l = m.body_to_link[body];
+    if (l == kInvalid) { *index = env * m.bodies_per_env + body; return kSideRigid; }
+    if (l >= m.links_per_env || m.body_to_articulation[body] >= 1u) return kInvalid;
+    *link = env * m.links_per_env + l; *index = env;
+    return kSideArtic;
+}
+
+struct RowSide { uint32_t kind, index; V3 jlin, jang; };
+struct Row { uint32_t flags, group_first, group_normal_count, env; float rhs, compliance_alpha, lower, upper, mu, friction_secondary; RowSide a, b; };
+static_assert(sizeof(Row) == kRowWords * sizeof(float), "row layout must stay 26 words");
+
+// ---- AssembleRows: one wavefront per environment (assemble_rows.cu:325-394, 200-214, 406-801, 122-186) ----
+__global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataView d, AssembleRowsParams p) {
+    extern __shared__ uint32_t lds_u[];
+    const uint32_t env = blockIdx.x, lane = threadIdx.x;
+    const uint32_t R = p.rows_per_env, S = p.union_slot_count, CR = p.contact_rows_per_env, md = p.max_dof, nl = m.links_per_env;
+    uint32_t* range_first = lds_u;        // S
+    uint32_t* range_points = lds_u + S;   // S
+    Row* rows = reinterpret_cast<Row*>(d.urows) + size_t{env} * R;
+    float* lambda = d.lambda + size_t{env} * R;
+    float* pen = d.row_penetration + size_t{env} * R;
+    uint32_t* cj_link = d.row_cj_link + size_t{env} * R, *cj_link_b = d.row_cj_link_b + size_t{env} * R;
+    float* cj_point = d.row_cj_point + size_t{env} * R * 3u, *cj_point_b = d.row_cj_point_b + size_t{env} * R * 3u;
+    // row ranges: exclusive prefix of the slots' point counts, four rows a point (:336-360)
+    const uint32_t previous_extent = d.contact_row_extent[2u * env + 1u];
+    uint32_t carry = 0u, extent = 1u;
+    for (uint32_t base = 0u; base < S; base += kWave) {
+        const uint32_t slot = base + lane;
+        const uint32_t points = slot < S ? d.ucontact_count[size_t{env} * S + slot] : 0u;
+        uint32_t through = points;
+#pragma unroll
+        for (int o = 1; o < kWave; o <<= 1) {
+            const uint32_t other = __shfl_up(through, o, kWave);
+            if (int(lane) >= o) through += other;
+        }
+        if (slot < S) {
+            const uint32_t first = (carry + through - points) * kRowsPerPoint;
+            range_first[slot] = first; range_points[slot] = points;
+            d.ucontact_row_range[(size_t{env} * S + slot) * 2u] = env * R + first;
+            d.ucontact_row_range[(size_t{env} * S + slot) * 2u + 1u] = points;
+            if (points > 0u) extent = max(extent, first + points * kRowsPerPoint + 1u);
+        }
+        carry += __shfl(through, kWave - 1, kWave);
+    }
+    extent = wave_max_u(extent);
+    // rows below the previous and current extents are cleared (:366-394)
+    const uint32_t clear_bound = contact_row_bound(previous_extent, 1u, CR);
+    for (uint32_t local = lane; local < min(clear_bound, R); local += kWave) {
+        lambda[local] = 0.0f; pen[local] = 0.0f; cj_link[local] = kInvalid; cj_link_b[local] = kInvalid;
+        rows[local].flags = 0u;
+    }
+    if (lane == 0u) {
+        d.contact_row_extent[2u * env] = previous_extent;
+        d.contact_row_extent[2u * env + 1u] = extent;
+    }
+    // padded generalized velocity tile (:200-214)
+    if (lane < md) {
+        float value = 0.0f;
+        if (lane < m.dof) {
+            const uint32_t link = m.dof_link[lane], c = m.dof_component[lane];
+            value = c == kInvalid ? d.qdot[size_t{env} * nl + link] : d.link_velocity[(size_t{env} * nl + link) * 6u + c];
+        }
+        d.qdot_flat[size_t{env} * md + lane] = value;
+    }
+    __syncthreads();
+    // contact rows, one lane per slot (:453-801; speculative law, condim 3)
+    uint32_t active_rows = 0u;
+    bool invalid_endpoint = false;
+    for (uint32_t slot = lane; slot < S; slot += kWave) {
+        const size_t gid = size_t{env} * S + slot;
+        const uint32_t base = range_first[slot], P = range_points[slot];
+        if (P == 0u) continue;
+        uint32_t n_active = P;
+        const uint32_t local_a = d.ucontact_a[gid * 4u], local_b = d.ucontact_b[gid * 4u];
+        ShapeRow sa{}, sb{};
+        sa.body_id = sb.body_id = -1; sa.profile = sb.profile = kInvalid;
+        if (local_a < m.bodies_per_env) sa = load_shape(m.shape_table, local_a);
+        if (local_b < m.bodies_per_env) sb = load_shape(m.shape_table, local_b);
+        uint32_t idx_a, idx_b, link_a, link_b;
+        uint32_t kind_a = resolve_side(m, env, local_a, sa.body_id, &idx_a, &link_a);
+        uint32_t kind_b = resolve_side(m, env, local_b, sb.body_id, &idx_b, &link_b);
+        if (kind_a == kInvalid || kind_b == kInvalid) {
+            invalid_endpoint = true;
+            n_active = 0u; kind_a = kind_b = kSideStatic;
+        }
+        if (kind_a == kSideStatic) idx_a = kInvalid;
+        if (kind_b == kSideStatic) idx_b = kInvalid;
+        // per-shape friction profile or the default 1.0, mixed by max at equal priority (scene/contact_filter.hpp:58-62, 108-111)
+        const float mu_a1 = sa.profile < m.profile_count ? m.profile_mu[2u * sa.profile] : 1.0f;
+        const float mu_a2 = sa.profile < m.profile_count ? m.profile_mu[2u * sa.profile + 1u] : 1.0f;
+        const float mu_b1 = sb.profile < m.profile_count ? m.profile_mu[2u * sb.profile] : 1.0f;
+        const float mu_b2 = sb.profile < m.profile_count ? m.profile_mu[2u * sb.profile + 1u] : 1.0f;
+        const float mu1 = fmaxf(mu_a1, mu_b1), mu2 = fmaxf(mu_a2, mu_b2);
+        for (uint32_t pt = 0u; pt < P; ++pt) {
+            const bool live = pt < n_active && pt < 4u;
+            const size_t mp = gid * 4u + pt;
+            const uint32_t row_of[3] = {base + pt, base + P + pt, base + 2u * P + pt};
+            V3 n{0, 0, 1}, point{0, 0, 0}, dirs[3];
+            dirs[1] = V3{1, 0, 0}; dirs[2] = V3{0, 1, 0};
+            float d0 = 0.0f;
+            if (live) {
+                const V3 raw{d.ucontact_normal[3u * mp], d.ucontact_normal[3u * mp + 1u], d.ucontact_normal[3u * mp + 2u]};
+                const float len = sqrtf(raw.x * raw.x + raw.y * raw.y + raw.z * raw.z);
+                n = len < 1e-12f ? V3{0, 0, 0} : V3{raw.x / len, raw.y / len, raw.z / len};
+                point = V3{d.ucontact_point[3u * mp], d.ucontact_point[3u * mp + 1u], d.ucontact_point[3u * mp + 2u]};
+                contact_tangent_basis(raw, &dirs[1], &dirs[2]);
+                d0 = d.ucontact_depth[mp];
+            }
+            dirs[0] = n;
+            for (uint32_t axis = 0u; axis < 3u; ++axis) {
+                const uint32_t rs = row_of[axis];
+                lambda[rs] = 0.0f; pen[rs] = 0.0f; cj_link[rs] = kInvalid; cj_link_b[rs] = kInvalid;
+                if (!live) { rows[rs].flags = 0u; continue; }
+                Row row{};
+                const V3 dir = dirs[axis];
+                row.group_first = env * R + base; row.group_normal_count = P; row.env = env;
+                row.mu = mu1; row.friction_secondary = mu2;
+                row.a.kind = kind_a; row.a.index = idx_a; row.a.jlin = dir; row.a.jang = V3{0, 0, 0};
+                row.b.kind = kind_b; row.b.index = idx_b; row.b.jlin = V3{-dir.x, -dir.y, -dir.z}; row.b.jang = V3{0, 0, 0};
+                if (axis == 0u) {
+                    // speculative rows reserve the rounding of their projected endpoint positions (:703-713)
+                    const V3 ext{fabsf(point.x) + fabsf(n.x * d0), fabsf(point.y) + fabsf(n.y * d0), fabsf(point.z) + fabsf(n.z * d0)};
+                    const double gamma = 3.0 * double(FLT_EPSILON) / (1.0 - 3.0 * double(FLT_EPSILON));
+                    const double roundoff = gamma * (fabs(double(n.x)) * (fabs(double(ext.x)) + fabs(double(ext.x))) +
+                                                     fabs(double(n.y)) * (fabs(double(ext.y)) + fabs(double(ext.y))) +
+                                                     fabs(double(n.z)) * (fabs(double(ext.z)) + fabs(double(ext.z))));
+                    const float clearance = roundoff > 0.0 ? nextafterf(float(roundoff), FLT_MAX) : 0.0f;
+                    const float depth = d0 + clearance;
+                    pen[rs] = depth;
+                    row.flags = kRowActive | kRowContactNormal | kRowBlockNormal | kRowSpeculative;
+                    row.rhs = (fminf(depth, 0.0f) + (p.position_pass != 0u ? 0.0f
+                               : fminf(fmaxf(d0, 0.0f), p.overlap_recovery_velocity * p.dt))) / (p.dt * p.dt);
+                    row.lower = 0.0f; row.upper = FLT_MAX;
+                } else {
+                    row.flags = kRowActive | kRowBlockTangent;
+                    row.lower = -FLT_MAX; row.upper = FLT_MAX;
+                }
+                if (kind_a == kSideArtic) { cj_link[rs] = link_a; cj_point[3u * rs] = point.x; cj_point[3u * rs + 1u] = point.y; cj_point[3u * rs + 2u] = point.z; }
+                if (kind_b == kSideArtic) { cj_link_b[rs] = link_b; cj_point_b[3u * rs] = point.x; cj_point_b[3u * rs + 1u] = point.y; cj_point_b[3u * rs + 2u] = point.z; }
+                rows[rs] = row;
+                ++active_rows;
+            }
+        }
+    }
+    active_rows = uint32_t(wave_sum(float(active_rows)));
+    invalid_endpoint = __any(invalid_endpoint);
+    if (lane == 0u) {
+        d.row_count[env] = active_rows;
+        if (invalid_endpoint) d.env_status[env] |= kEnvStatusInvalidEndpoint;
+    }
+    __syncthreads();
+    // chain Jacobians, lane = DoF: every row entry is the joint's own column when the joint lies on the path from
+    // the row's link to the root, which the cooked per-link DoF mask answers (assemble_rows.cu:122-169,
+    // articulation_types.cuh:193-238); both sides, then the shared-owner merge (:172-186).
+    if (md == 0u) return;
+    V3 axis_world{0, 0, 0}, origin{0, 0, 0};
+    uint32_t mode = 0u;   // 0 none, 1 revolute, 2 prismatic, 3 base angular, 4 base linear
+    if (lane < m.dof) {
+        const uint32_t link = m.dof_link[lane], component = m.dof_component[lane];
+        if (component == kInvalid) {
+            const Xf pose = load_xf(d.link_pose + (size_t{env} * nl + link) * 7u);
+            axis_world = rotate_normalized(pose.r, V3{m.joint_axis[3u * link], m.joint_axis[3u * link + 1u], m.joint_axis[3u * link + 2u]});
+            origin = pose.p;
+            mode = m.joint_type[link] == kPrismatic ? 2u : 1u;
+        } else {
+            const Xf base = load_xf(d.base_pose + size_t{env} * 7u);
+            const uint32_t k = component % 3u;
+            axis_world = rotate_normalized(base.r, V3{k == 0u ? 1.0f : 0.0f, k == 1u ? 1.0f : 0.0f, k == 2u ? 1.0f : 0.0f});
+            origin = base.p;
+            mode = component < 3u ? 3u : 4u;
+        }
+    }
+    const uint32_t bound = min(contact_row_bound(previous_extent, extent, CR) + (R - CR), R);
+    for (uint32_t r = 0u; r < bound; ++r) {
+        const Row* row = rows + r;
+        for (uint32_t side = 0u; side < 2u; ++side) {
+            const uint32_t link_global = side == 0u ? cj_link[r] : cj_link_b[r];
+            if (link_global == kInvalid) continue;
+            const uint32_t link = link_global - env * nl;
+            const float* cp = (side == 0u ? cj_point : cj_point_b) + 3u * r;
+            const V3 point{cp[0], cp[1], cp[2]};
+            const V3 dir = side == 0u ? row->a.jlin : row->b.jlin;
+            float entry = 0.0f;
+            if (lane < m.dof && ((m.link_dof_mask[link] >> lane) & 1ull) != 0ull) {
+                if (mode == 1u) entry = dot3(cross3(axis_world, sub3(point, origin)), dir) + dot3(axis_world, V3{0, 0, 0});
+                else if (mode == 2u) entry = dot3(axis_world, dir);
+                else if (mode == 3u) entry = dot3(cross3(axis_world, sub3(point, origin)), dir) + dot3(axis_world, V3{0, 0, 0});
+                else if (mode == 4u) entry = dot3(axis_world, dir);
+            }
+            if (lane < md) (side == 0u ? d.chain_jacobian : d.chain_jacobian_b)[(size_t{env} * R + r) * md + lane] = entry;
+        }
+        if ((row->flags & kRowActive) != 0u && row->a.kind == kSideArtic && row->b.kind == kSideArtic &&
+            row->a.index == row->b.index && lane < md) {
+            float* ja = d.chain_jacobian + (size_t{env} * R + r) * md;
+            float* jb = d.chain_jacobian_b + (size_t{env} * R + r) * md;
+            ja[lane] += jb[lane];
+            jb[lane] = 0.0f;
+        }
+    }
+}
+
+}  // namespace
+
+Status OpSyncLinkBodyPose(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const SyncLinkBodyPoseParams*>(params);
+    if (p == nullptr) return Status::Failed;
+    if (p->env_count == 0u || p->bodies_per_env == 0u) return Status::Ok;
+    if (p->selected_env_count != 0u) return Status::Unsupported;
+    const uint32_t total = p->env_count * p->bodies_per_env;
+    hipLaunchKernelGGL(SyncLinkBodyPoseKernel, dim3((total + 255u) / 256u), dim3(256), 0, stream, m, d, total);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
+Status OpBuildAabbs(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const BuildAabbsParams*>(params);
+    if (p == nullptr) return Status::Failed;
+    if (p->env_count == 0u || p->bodies_per_env == 0u) return Status::Ok;
+    const uint32_t total = p->env_count * p->bodies_per_env;
+    hipLaunchKernelGGL(BuildAabbsKernel, dim3((total + 255u) / 256u), dim3(256), 0, stream, m, d, *p);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
+// The pair query reads the body AABBs directly, so no tree is built (the reference skips its LBVH the same way for
+// small worlds, broadphase.cu:581-582).
+Status OpLbvhBuild(const ModelView&, const DataView&, const void* params, hipStream_t) {
+    return params == nullptr ? Status::Failed : Status::Ok;
+}
+
+Status OpLbvhQueryPairs(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const LbvhQueryPairsParams*>(params);
+    if (p == nullptr) return Status::Failed;
+    if (p->env_count == 0u) return Status::Ok;
+    if (p->excluded_count != 0u) return Status::Unsupported;
+    hipLaunchKernelGGL(QueryPairsKernel, dim3(p->env_count), dim3(kWave), 0, stream, m, d, *p);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
+Status OpNarrowphasePrimitives(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const NarrowphasePrimitivesParams*>(params);
+    if (p == nullptr) return Status::Failed;
+    if (p->env_count == 0u || p->union_slot_count == 0u || p->rigid_slot_cap == 0u) return Status::Ok;
+    const uint32_t total = p->env_count * p->rigid_slot_cap;
+    hipLaunchKernelGGL(NarrowphaseKernel, dim3((total + 127u) / 128u), dim3(128), 0, stream, m, d, *p);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
+Status OpNarrowphaseHeightfield(const ModelView&, const DataView&, const void* params, hipStream_t) {
+    return params == nullptr ? Status::Ok : Status::Ok;   // no heightfield on this path: a no-op, as in the reference
+}
+
+Status OpAssembleRows(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const AssembleRowsParams*>(params);
+    if (p == nullptr) return Status::Failed;
+    if (p->env_count == 0u || p->rows_per_env == 0u) return Status::Ok;
+    if (p->max_dof > kMaxDof) return Status::InvalidArgument;
+    const size_t lds = size_t{p->union_slot_count} * 2u * sizeof(uint32_t);
+    hipLaunchKernelGGL(AssembleRowsKernel, dim3(p->env_count), dim3(kWave), lds, stream, m, d, *p);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
+// With no contact cache carried between steps every multiplier starts at the zero AssembleRows wrote
+// (assemble_rows.cu:1393-1455 with an empty cache).
+Status OpContactWarmStart(const ModelView&, const DataView&, const void* params, hipStream_t) {
+    return params == nullptr ? Status::Failed : Status::Ok;
+}
+
+Status OpSnapshotStepVelocity(const ModelView&, const DataView&, const void*, hipStream_t) { return Status::Ok; }
+
+}  // namespace nkh

@@ -1,0 +1,771 @@
+// Host side of the library above the PHI seam: the template cook, the device arena with its named env-major
+// fields, the pipeline (the ordered op list of one step with its parameter PODs), the world that steps it eagerly or
+// as a captured plan, and the C ABI.  Counterpart, for the articulation-step path only, of src/nk/{model,data,
+// pipeline} and src/c_abi/{device,world,buffer}.cpp.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <exception>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/nuka_hip.h"
+#include "backend.h"
+#include "nk_types.h"
+
+namespace nkh {
+namespace {
+
+thread_local std::string g_last_error;   // nuka.h:42-44
+
+nuka_result_t Error(nuka_result_t code, const std::string& message) {
+    g_last_error = message;
+    return code;
+}
+
+// ---- host math for the cook (runtime/articulation/articulation_state.cpp:113-165, 307-343) ---------------
+void MakeSpatialInertia(float mass, const float* diag, const float* frame, float* I) {
+    std::memset(I, 0, 36 * sizeof(float));
+    if (mass <= 0.0f) return;
+    float qw = frame[3], qx = frame[4], qy = frame[5], qz = frame[6];
+    const float norm = std::sqrt(qw * qw + qx * qx + qy * qy + qz * qz);
+    if (norm > 0.0f) { const float inv = 1.0f / norm; qw *= inv; qx *= inv; qy *= inv; qz *= inv; }
+    const float xx = qx * qx, yy = qy * qy, zz = qz * qz, xy = qx * qy, xz = qx * qz, yz = qy * qz, wx = qw * qx, wy = qw * qy, wz = qw * qz;
+    const float r[9] = {1.0f - 2.0f * (yy + zz), 2.0f * (xy - wz), 2.0f * (xz + wy), 2.0f * (xy + wz), 1.0f - 2.0f * (xx + zz),
+                        2.0f * (yz - wx), 2.0f * (xz - wy), 2.0f * (yz + wx), 1.0f - 2.0f * (xx + yy)};
+    const float cx = frame[0], cy = frame[1], cz = frame[2];
+    const float c_dot = cx * cx + cy * cy + cz * cz;
+    const float parallel[9] = {c_dot - cx * cx, -cx * cy, -cx * cz, -cy * cx, c_dot - cy * cy, -cy * cz, -cz * cx, -cz * cy, c_dot - cz * cz};
+    const float cross[9] = {0.0f, -cz, cy, cz, 0.0f, -cx, -cy, cx, 0.0f};
+    for (int row = 0; row < 3; ++row)
+        for (int col = 0; col < 3; ++col) {
+            float com = 0.0f;
+            for (int k = 0; k < 3; ++k) com += r[row * 3 + k] * diag[k] * r[col * 3 + k];
+            I[row * 6 + col] = com + mass * parallel[row * 3 + col];
+            I[row * 6 + 3 + col] += mass * cross[row * 3 + col];
+            I[(3 + row) * 6 + col] += -mass * cross[row * 3 + col];
+            I[(3 + row) * 6 + 3 + col] = row == col ? mass : 0.0f;
+        }
+}
+
+uint32_t JointWidth(uint8_t type) { return type <= kPrismatic ? 1u : type == kFloatingBase ? 6u : 0u; }
+
+struct HostModel {
+    ModelView counts{};   // scalar members only
+    std::vector<uint8_t> joint_type;
+    std::vector<uint32_t> parent_link, link_body, link_tree_depth, link_child_range, link_children, link_dof, dof_link, dof_component,
+        link_geom_kind, body_to_link, body_to_articulation, body_collidable_link, body_collidable_body;
+    std::vector<uint64_t> link_dof_mask;
+    std::vector<float> joint_axis, parent_offset, link_local_pose, link_inertial_frame, link_inertia, joint_damping, joint_armature,
+        joint_stiffness, joint_spring_reference, link_geom_local, shape_table, body_collidable_local, body_init_pose, profile_mu;
+};
+
+std::vector<float> CopyOrZero(const float* src, size_t n) {
+    return src != nullptr ? std::vector<float>(src, src + n) : std::vector<float>(n, 0.0f);
+}
+
+// The cook: tree tables (fields.yaml:845-848), DoF maps (articulation_mass.cuh:64-90), spatial inertias, collidable rows
+// (prims_types.cuh:27-54) and owner tables (nk/solve/collidable_owner.hpp).
+void Cook(const nuka_template_desc_t& d, HostModel* out) {
+    const uint32_t nl = d.link_count, nb = d.body_count;
+    if (nl == 0u) throw std::invalid_argument("template has no links");
+    if (!d.joint_type || !d.parent_link || !d.joint_axis || !d.link_local_pose || !d.link_inertial_frame || !d.link_mass ||
+        !d.link_diag_inertia) throw std::invalid_argument("template link arrays are required");
+    if (nb > 0u && (!d.body_role || !d.body_link || !d.body_local || !d.shape_kind || !d.shape_params || !d.shape_contype ||
+                    !d.shape_conaffinity || !d.shape_group || !d.shape_profile)) throw std::invalid_argument("template body arrays are required");
+    HostModel& m = *out;
+    m.joint_type.assign(d.joint_type, d.joint_type + nl);
+    m.parent_link.assign(d.parent_link, d.parent_link + nl);
+    m.joint_axis.assign(d.joint_axis, d.joint_axis + 3u * nl);
+    m.parent_offset = CopyOrZero(d.parent_offset, 3u * nl);
+    m.link_local_pose.assign(d.link_local_pose, d.link_local_pose + 7u * nl);
+    m.link_inertial_frame.assign(d.link_inertial_frame, d.link_inertial_frame + 7u * nl);
+    m.joint_damping = CopyOrZero(d.joint_damping, nl);
+    m.joint_armature = CopyOrZero(d.joint_armature, nl);
+    m.joint_stiffness = CopyOrZero(d.joint_stiffness, nl);
+    m.joint_spring_reference = CopyOrZero(d.joint_spring_reference, nl);
+    m.link_inertia.resize(36u * nl);
+    m.link_dof.resize(nl);
+    m.link_body.assign(nl, kInvalid);
+    m.link_geom_kind.assign(nl, 0u);
+    m.link_geom_local.resize(7u * nl);
+    uint32_t nv = 0u;
+    for (uint32_t l = 0u; l < nl; ++l) {
+        const uint8_t type = m.joint_type[l];
+        if (type > kFloatingBase) throw std::invalid_argument("joint type not supported on this path");
+        if (type == kFloatingBase && (l != 0u || m.parent_link[l] != kInvalid)) throw std::invalid_argument("a floating base must be link 0");
+        if (m.parent_link[l] != kInvalid && m.parent_link[l] >= l) throw std::invalid_argument("parents must precede children");
+        if (l > 0u && m.parent_link[l] == kInvalid) throw std::invalid_argument("one articulation (one root) per environment");
+        MakeSpatialInertia(d.link_mass[l], d.link_diag_inertia + 3u * l, d.link_inertial_frame + 7u * l, m.link_inertia.data() + 36u * l);
+        m.link_dof[l] = nv;
+        nv += JointWidth(type);
+        const float id[7] = {0, 0, 0, 1, 0, 0, 0};
+        std::memcpy(m.link_geom_local.data() + 7u * l, id, sizeof(id));
+    }
+    if (nv == 0u || nv > kMaxDof) throw std::invalid_argument("articulation DoF must be in 1..64");
+    m.dof_link.resize(nv);
+    m.dof_component.resize(nv);
+    m.link_dof_mask.assign(nl, 0ull);
+    m.link_tree_depth.resize(nl);
+    uint32_t max_depth = 0u;
+    for (uint32_t l = 0u; l < nl; ++l) {
+        const uint32_t width = JointWidth(m.joint_type[l]);
+        uint64_t own = 0ull;
+        for (uint32_t c = 0u; c < width; ++c) {
+            m.dof_link[m.link_dof[l] + c] = l;
+            m.dof_component[m.link_dof[l] + c] = width == 1u ? kInvalid : c;
+            own |= 1ull << (m.link_dof[l] + c);
+        }
+        const uint32_t parent = m.parent_link[l];
+        m.link_dof_mask[l] = own | (parent == kInvalid ? 0ull : m.link_dof_mask[parent]);
+        m.link_tree_depth[l] = parent == kInvalid ? 0u : m.link_tree_depth[parent] + 1u;
+        max_depth = std::max(max_depth, m.link_tree_depth[l]);
+    }
+    m.link_child_range.resize(2u * nl);
+    m.link_children.clear();
+    for (uint32_t l = 0u; l < nl; ++l) {
+        m.link_child_range[2u * l] = uint32_t(m.link_children.size());
+        for (uint32_t c = 0u; c < nl; ++c) if (m.parent_link[c] == l) m.link_children.push_back(c);
+        m.link_child_range[2u * l + 1u] = uint32_t(m.link_children.size());
+    }
+    m.link_children.resize(nl, 0u);
+    m.shape_table.assign(size_t{nb} * kShapeStride, 0.0f);
+    m.body_to_link.assign(nb, kInvalid);
+    m.body_to_articulation.assign(nb, kInvalid);
+    m.body_collidable_link.assign(nb, kInvalid);
+    m.body_collidable_body.assign(nb, kInvalid);
+    m.body_collidable_local.resize(size_t{nb} * 7u);
+    m.body_init_pose.resize(size_t{nb} * 7u);
+    m.profile_mu.assign(d.profile_mu, d.profile_mu + 2u * d.profile_count);
+    auto bits = [](uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; };
+    bool any_box = false;
+    for (uint32_t b = 0u; b < nb; ++b) {
+        const uint32_t role = d.body_role[b], link = d.body_link[b];
+        float* row = m.shape_table.data() + size_t{b} * kShapeStride;
+        row[0] = bits(d.shape_kind[b]);
+        for (int k = 0; k < 4; ++k) row[1 + k] = d.shape_params[4u * b + k];
+        row[5] = bits(d.shape_contype[b]); row[6] = bits(d.shape_conaffinity[b]); row[7] = bits(0u);
+        row[8] = bits(role == 0u ? 0xFFFFFFFFu : b); row[9] = bits(d.shape_group[b]);
+        row[10] = bits(0u); row[11] = bits(0u); row[12] = bits(d.shape_profile[b]);
+        any_box = any_box || d.shape_kind[b] == kShapeBox;
+        const float id[7] = {0, 0, 0, 1, 0, 0, 0};
+        std::memcpy(m.body_collidable_local.data() + 7u * b, id, sizeof(id));
+        std::memcpy(m.body_init_pose.data() + 7u * b, id, sizeof(id));
+        if (role == 0u) std::memcpy(m.body_init_pose.data() + 7u * b, d.body_local + 7u * b, 7u * sizeof(float));
+        else if (role == 1u) {
+            if (link >= nl || m.link_body[link] != kInvalid) throw std::invalid_argument("each link owns at most one body row");
+            m.link_body[link] = b; m.body_to_link[b] = link; m.body_to_articulation[b] = 0u;
+            std::memcpy(m.link_geom_local.data() + 7u * link, d.body_local + 7u * b, 7u * sizeof(float));
+            m.link_geom_kind[link] = d.shape_kind[b] != kInvalid ? 1u : 0u;
+        } else if (role != 2u) throw std::invalid_argument("unknown collidable role");
+    }
+    for (uint32_t b = 0u; b < nb; ++b) {
+        if (d.body_role[b] != 2u) continue;
+        const uint32_t link = d.body_link[b];
+        if (link >= nl || m.link_body[link] == kInvalid) throw std::invalid_argument("an extra collidable needs its link's body row");
+        m.body_collidable_link[b] = link;
+        m.body_collidable_body[b] = m.link_body[link];
+        std::memcpy(m.body_collidable_local.data() + 7u * b, d.body_local + 7u * b, 7u * sizeof(float));
+    }
+    uint32_t slots = d.max_contacts_per_env;
+    if (slots == 0u)
+        for (uint32_t i = 0u; i < nb; ++i)
+            for (uint32_t j = i + 1u; j < nb; ++j) {
+                if (d.body_role[i] == 0u && d.body_role[j] == 0u) continue;
+                if (d.shape_kind[i] == kInvalid || d.shape_kind[j] == kInvalid) continue;
+                if (((d.shape_contype[i] & d.shape_conaffinity[j]) | (d.shape_contype[j] & d.shape_conaffinity[i])) == 0u) continue;
+                ++slots;
+            }
+    ModelView& c = m.counts;
+    c.links_per_env = nl; c.bodies_per_env = nb; c.dof = nv; c.max_dof = nv; c.max_depth = max_depth;
+    c.contact_slots = slots;
+    c.contact_rows_per_env = slots * kPointsPerSlot * kRowsPerPoint;   // nk_row.hpp:59-63
+    c.rows_per_env = c.contact_rows_per_env;
+    c.profile_count = d.profile_count;
+    c.floating_root = m.joint_type[0] == kFloatingBase ? 1u : 0u;
+    c.max_points_per_slot = any_box ? 4u : 1u;
+}
+
+enum Dtype : uint8_t { kF32 = 0, kU32 = 1, kU64 = 2, kU8 = 3 };
+struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count; size_t offset; bool is_template; };
+
+#define NKH_DATA_FIELDS(X) \
+    X(q, kF32, E * nl) X(qdot, kF32, E * nl) X(qddot, kF32, E * nl) X(tau, kF32, E * nl) X(base_pose, kF32, E * 7) \
+    X(link_pose, kF32, E * nl * 7) X(link_velocity, kF32, E * nl * 6) X(link_acceleration, kF32, E * nl * 6) \
+    X(link_wrench, kF32, E * nl * 6) X(articulation_bias, kF32, E * md) X(articulation_qdd, kF32, E * md) \
+    X(m, kF32, E * md * md) X(m_factor, kF32, E * md * md) X(qdot_flat, kF32, E * md) X(qdot_pseudo, kF32, E * nl) \
+    X(link_velocity_pseudo, kF32, E * nl * 6) X(body_pose, kF32, E * nb * 7) X(body_aabb_lo, kF32, E * nb * 3) \
+    X(body_aabb_hi, kF32, E * nb * 3) X(candidate_pairs, kU32, E * S * 2) X(pair_count, kU32, E) X(ucontact_count, kU32, E * S) \
+    X(ucontact_a, kU32, E * S * 4) X(ucontact_b, kU32, E * S * 4) X(ucontact_law, kU32, E * S) \
+    X(ucontact_row_range, kU32, E * S * 2) X(ucontact_point, kF32, E * S * 12) X(ucontact_normal, kF32, E * S * 12) \
+    X(ucontact_depth, kF32, E * S * 4) X(ucontact_id_pair, kU64, E * S * 4) X(ucontact_id_feature, kU64, E * S * 4) \
+    X(urows, kF32, E * R * 26) X(lambda, kF32, E * R) X(row_penetration, kF32, E * R) X(row_cj_point, kF32, E * R * 3) \
+    X(row_cj_point_b, kF32, E * R * 3) X(chain_jacobian, kF32, E * R * md) X(chain_jacobian_b, kF32, E * R * md) \
+    X(row_cj_link, kU32, E * R) X(row_cj_link_b, kU32, E * R) X(row_count, kU32, E) X(contact_count, kU32, E) \
+    X(contact_row_extent, kU32, E * 2) X(env_status, kU32, E) X(vbd_velocity_sweep_count, kU32, E) \
+    X(solver_residual, kF32, E * 4) X(solver_penalty, kF32, E * R) X(solver_velocity, kF32, E * md) X(solver_free, kF32, E * md)
+
+#define NKH_MODEL_FIELDS(X) \
+    X(joint_type, kU8) X(parent_link, kU32) X(joint_axis, kF32) X(parent_offset, kF32) X(link_local_pose, kF32) \
+    X(link_inertial_frame, kF32) X(link_inertia, kF32) X(joint_damping, kF32) X(joint_armature, kF32) X(joint_stiffness, kF32) \
+    X(joint_spring_reference, kF32) X(link_body, kU32) X(link_tree_depth, kU32) X(link_child_range, kU32) X(link_children, kU32) \
+    X(link_dof, kU32) X(dof_link, kU32) X(dof_component, kU32) X(link_dof_mask, kU64) X(link_geom_kind, kU32) \
+    X(link_geom_local, kF32) X(shape_table, kF32) X(body_to_link, kU32) X(body_to_articulation, kU32) \
+    X(body_collidable_link, kU32) X(body_collidable_body, kU32) X(body_collidable_local, kF32) X(profile_mu, kF32)
+
+uint32_t DtypeBytes(Dtype t) { return t == kU64 ? 8u : t == kU8 ? 1u : 4u; }
+
+struct DeviceRecord {   // src/c_abi/internal.hpp:57-69
+    void* backend = nullptr;
+    int gpu_index = 0;
+};
+
+struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
+    DeviceRecord* device = nullptr;
+    nuka_phi_backend* backend = nullptr;
+    const nuka_phi_backend_i* be = nullptr;
+    HostModel host;
+    nuka_world_desc_t cfg{};
+    uint32_t env_count = 0u;
+    nuka_phi_buffer* arena = nullptr;
+    nuka_phi_buffer* initial = nullptr;   // the state after creation, for nuka_world_reset
+    size_t arena_bytes = 0u;
+    std::vector<Field> fields;
+    ModelView model{};
+    DataView data{};
+    // the pipeline: ops in step order with their parameter PODs (src/nk/pipeline/pipeline.cpp:187-1020)
+    std::vector<nuka_phi_op_call> calls;
+    FkWorldPosesParams p_fk{};
+    FkLinkVelocitiesParams p_fk_velocity{};
+    ApplyDrivesParams p_drives{};
+    ArticulationDynamicsParams p_dynamics{}, p_dynamics_probe{};
+    IntegrateVelocityParams p_int_vel{};
+    IntegratePositionParams p_int_pos{};
+    SyncLinkBodyPoseParams p_sync{};
+    BuildAabbsParams p_aabbs{};
+    LbvhBuildParams p_lbvh{};
+    LbvhQueryPairsParams p_query{};
+    NarrowphasePrimitivesParams p_narrow{};
+    AssembleRowsParams p_assemble{};
+    ContactWarmStartParams p_warm0{}, p_warm1{};
+    BlockDescentSolveParams p_solve{};
+    SnapshotParams p_snapshot{};
+    nuka_execution_mode_t mode = NUKA_EXECUTION_EAGER;
+    nuka_phi_plan* plan = nullptr;
+
+    ~World() {
+        if (be != nullptr && plan != nullptr) be->plan_free(backend, plan);
+        if (arena != nullptr) reinterpret_cast<nuka_phi_buffer_head*>(arena)->iface->free(arena);
+        if (initial != nullptr) reinterpret_cast<nuka_phi_buffer_head*>(initial)->iface->free(initial);
+    }
+};
+
+const nuka_phi_buffer_i* Iface(nuka_phi_buffer* b) { return reinterpret_cast<nuka_phi_buffer_head*>(b)->iface; }
+
+void BuildPipeline(World& w) {
+    const ModelView& m = w.model;
+    const uint32_t E = w.env_count, nl = m.links_per_env, nb = m.bodies_per_env;
+    const nuka_world_desc_t& cfg = w.cfg;
+    const bool has_contacts = m.rows_per_env > 0u;
+    const float contact_margin = cfg.solver_contact_margin;
+    const float query_reach = std::fmax(0.02f, 2.0f * (2.0f * 0.0f + contact_margin));   // contact_query.hpp:20-22
+    w.p_fk = {E, E * nl};
+    w.p_fk_velocity = {E, E * nl};
+    w.p_drives = {};
+    w.p_drives.dt = cfg.fixed_dt; w.p_drives.total_link_count = E * nl; w.p_drives.links_per_env = nl;
+    w.p_drives.mode = 1u; w.p_drives.articulation_count = E;
+    std::memcpy(w.p_drives.gravity, cfg.gravity, sizeof(cfg.gravity));
+    ArticulationDynamicsParams& dyn = w.p_dynamics;   // pipeline.cpp:388-402
+    dyn = {};
+    dyn.dt = cfg.fixed_dt; dyn.max_dof = m.max_dof; dyn.integrate_velocity = 1u; dyn.fold_drive_damping = 0u; dyn.reuse_mass = 0u;
+    std::memcpy(dyn.gravity, cfg.gravity, sizeof(cfg.gravity));
+    dyn.articulation_count = E; dyn.total_link_count = E * nl; dyn.apply_link_wrench = 1u; dyn.max_links = nl;
+    dyn.links_per_env = nl; dyn.bodies_per_env = nb;
+    w.p_dynamics_probe = dyn;
+    w.p_dynamics_probe.integrate_velocity = 0u;
+    w.p_int_vel = {};
+    w.p_int_vel.dt = cfg.fixed_dt;
+    std::memcpy(w.p_int_vel.gravity, cfg.gravity, sizeof(cfg.gravity));
+    w.p_int_pos = {cfg.fixed_dt, E * nl, E, 0u, E, (has_contacts && cfg.solver_pos_iters > 0u) ? 1u : 0u, 0u};
+    w.p_sync = {E, nl, nb, 0u, 0u};
+    w.p_aabbs = {E, nb, 0u, std::fmax(contact_margin, 0.0005f), cfg.fixed_dt, query_reach};   // pipeline.cpp:613-615
+    w.p_lbvh = {E, nb, 0u};
+    w.p_query = {E, nb, 0u, m.contact_slots, m.contact_slots, m.contact_slots, 0u};
+    w.p_narrow = {E, nb, m.contact_slots, m.contact_slots, contact_margin, cfg.fixed_dt, query_reach};
+    AssembleRowsParams& as = w.p_assemble;   // pipeline.cpp:861-897
+    as = {};
+    as.env_count = E; as.articulation_count = E; as.total_link_count = E * nl; as.max_dof = m.max_dof;
+    as.union_slot_count = m.contact_slots; as.rows_per_env = m.rows_per_env; as.contact_rows_per_env = m.contact_rows_per_env;
+    as.full_row_slot_count = m.contact_slots; as.bodies_per_env = nb; as.base_link_count = nl;
+    as.position_pass = cfg.solver_pos_iters > 0u ? 1u : 0u;
+    as.dt = cfg.fixed_dt; as.overlap_recovery_velocity = cfg.solver_overlap_recovery_velocity; as.contact_margin = contact_margin;
+    w.p_warm0 = {0u, E, m.contact_slots, m.rows_per_env, m.contact_slots, 2u};
+    w.p_warm1 = w.p_warm0;
+    w.p_warm1.phase = 1u;
+    BlockDescentSolveParams& bd = w.p_solve;   // pipeline.cpp:471-497
+    bd = {};
+    bd.dt = cfg.fixed_dt; bd.env_count = E; bd.rows_per_env = m.rows_per_env; bd.total_body_count = E * nb; bd.articulation_count = E;
+    bd.max_dof = m.max_dof; bd.max_independent_dof = m.dof; bd.base_link_count = nl; bd.contact_rows_per_env = m.contact_rows_per_env;
+    bd.contact_slots_per_env = m.contact_slots; bd.iterations = cfg.solver_vel_iters;
+    bd.position_iterations = has_contacts ? cfg.solver_pos_iters : 0u;
+    bd.position_beta = cfg.solver_pos_beta; bd.position_slop = cfg.solver_pos_slop;
+    bd.position_max_velocity = cfg.solver_baumgarte_max_velocity; bd.velocity_tolerance = cfg.solver_velocity_tolerance;
+
+    // op order of one interval (pipeline.cpp:374, 428-430, 442, 605-639, 699, 746, 908-923, 967, 981-986)
+    w.calls.clear();
+    auto add = [&](NkOp op, const void* params) {
+        if (!BackendSupportsOp(op)) throw std::runtime_error(std::string("backend does not support op ") + OpName(op));
+        w.calls.push_back({uint16_t(op), params});
+    };
+    add(NkOp::SnapshotStepVelocity, &w.p_snapshot);
+    add(NkOp::FkWorldPoses, &w.p_fk);
+    add(NkOp::ApplyDrives, &w.p_drives);
+    add(NkOp::ArticulationDynamics, &w.p_dynamics);
+    add(NkOp::IntegrateVelocity, &w.p_int_vel);
+    if (has_contacts) {
+        add(NkOp::SyncLinkBodyPose, &w.p_sync);
+        add(NkOp::BuildAabbs, &w.p_aabbs);
+        add(NkOp::LbvhBuild, &w.p_lbvh);
+        add(NkOp::LbvhQueryPairs, &w.p_query);
+        add(NkOp::NarrowphasePrimitives, &w.p_narrow);
+        add(NkOp::NarrowphaseHeightfield, &w.p_narrow);
+        add(NkOp::AssembleRows, &w.p_assemble);
+        add(NkOp::ContactWarmStart, &w.p_warm0);
+        add(NkOp::BlockDescentSolve, &w.p_solve);
+        add(NkOp::ContactWarmStart, &w.p_warm1);
+    }
+    add(NkOp::IntegratePosition, &w.p_int_pos);
+    add(NkOp::FkWorldPoses, &w.p_fk);
+    add(NkOp::FkLinkVelocities, &w.p_fk_velocity);
+    if (nb > 0u) add(NkOp::SyncLinkBodyPose, &w.p_sync);
+}
+
+void InvalidatePlan(World& w) {
+    if (w.plan != nullptr) { w.be->plan_free(w.backend, w.plan); w.plan = nullptr; }
+}
+
+nuka_result_t MapStatus(uint8_t status) {
+    switch (static_cast<Status>(status)) {
+        case Status::Ok: return NUKA_RESULT_OK;
+        case Status::Unsupported: return NUKA_RESULT_NOT_SUPPORTED;
+        case Status::OutOfMemory: return NUKA_RESULT_OUT_OF_MEMORY;
+        case Status::InvalidArgument: return NUKA_RESULT_INVALID_ARG;
+        default: return NUKA_RESULT_DEVICE_ERROR;
+    }
+}
+
+// nk::World::Step (src/nk/pipeline/world.cpp:663-686): every op through the backend's dispatch
+nuka_result_t StepEager(World& w) {
+    for (const nuka_phi_op_call& call : w.calls) {
+        const uint8_t status = w.be->dispatch(w.backend, reinterpret_cast<const nuka_phi_model_view*>(&w.model),
+                                              reinterpret_cast<const nuka_phi_data_view*>(&w.data), &call);
+        if (status != uint8_t(Status::Ok))
+            return Error(MapStatus(status), std::string("step failed in op ") + OpName(static_cast<NkOp>(call.op)));
+    }
+    return NUKA_RESULT_OK;
+}
+
+// nk::World::PrepareGraph (world.cpp:688-705)
+nuka_result_t PreparePlan(World& w) {
+    if (w.plan != nullptr) return NUKA_RESULT_OK;
+    nuka_phi_execution_error error{};
+    w.plan = w.be->plan_create(w.backend, reinterpret_cast<const nuka_phi_model_view*>(&w.model),
+                               reinterpret_cast<const nuka_phi_data_view*>(&w.data), w.calls.data(), int(w.calls.size()), &error);
+    if (w.plan == nullptr) return Error(MapStatus(error.status), std::string("graph capture failed: ") + error.message);
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t StepN(World& w, uint32_t n) {
+    if (w.mode == NUKA_EXECUTION_GRAPH) {
+        const nuka_result_t prepared = PreparePlan(w);
+        if (prepared != NUKA_RESULT_OK) return prepared;
+        uint32_t submitted = 0u;
+        nuka_phi_execution_error error{};
+        const uint8_t status = w.be->plan_execute_repeated(w.backend, w.plan, n, &submitted, &error);
+        if (status != uint8_t(Status::Ok)) return Error(MapStatus(status), std::string("graph launch failed: ") + error.message);
+        return NUKA_RESULT_OK;
+    }
+    for (uint32_t i = 0u; i < n; ++i) {
+        const nuka_result_t r = StepEager(w);
+        if (r != NUKA_RESULT_OK) return r;
+    }
+    return NUKA_RESULT_OK;
+}
+
+template <typename T>
+size_t Place(std::vector<Field>& fields, const char* name, Dtype dtype, size_t count, size_t* cursor, bool is_template) {
+    (void)sizeof(T);
+    const size_t offset = *cursor;
+    fields.push_back({name, dtype, DtypeBytes(dtype), count, offset, is_template});
+    *cursor = (offset + count * DtypeBytes(dtype) + 255u) & ~size_t{255u};
+    return offset;
+}
+
+}  // namespace
+}  // namespace nkh
+
+using namespace nkh;
+
+extern "C" {
+
+const char* nuka_result_message(nuka_result_t result) {
+    switch (result) {
+        case NUKA_RESULT_OK: return "ok";
+        case NUKA_RESULT_INVALID_ARG: return "invalid argument";
+        case NUKA_RESULT_NULL_HANDLE: return "null handle";
+        case NUKA_RESULT_DEVICE_ERROR: return "device error";
+        case NUKA_RESULT_OUT_OF_MEMORY: return "out of memory";
+        case NUKA_RESULT_NOT_SUPPORTED: return "not supported";
+        default: return "internal error";
+    }
+}
+
+const char* nuka_last_error_message(void) {
+    static thread_local std::string held;
+    held.swap(g_last_error);
+    g_last_error.clear();
+    return held.c_str();
+}
+
+nuka_result_t nuka_device_create(const nuka_device_desc_t* desc, nuka_device_handle* out) {
+    if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    *out = nullptr;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count == 0) {
+        (void)hipGetLastError();
+        return Error(NUKA_RESULT_NOT_SUPPORTED, "no HIP device: the library has no CPU fallback");
+    }
+    const uint32_t index = desc != nullptr ? desc->gpu_index : 0u;
+    if (index >= uint32_t(count)) return Error(NUKA_RESULT_INVALID_ARG, "gpu_index out of range");
+    void* backend = CreateBackend(int(index), desc != nullptr ? desc->stream : nullptr);
+    if (backend == nullptr) return Error(NUKA_RESULT_DEVICE_ERROR, "backend creation failed");
+    auto* record = new DeviceRecord{backend, int(index)};
+    *out = reinterpret_cast<nuka_device_handle>(record);
+    return NUKA_RESULT_OK;
+}
+
+void nuka_device_destroy(nuka_device_handle device) {
+    auto* record = reinterpret_cast<DeviceRecord*>(device);
+    if (record == nullptr) return;
+    auto* backend = reinterpret_cast<nuka_phi_backend*>(record->backend);
+    reinterpret_cast<nuka_phi_backend_head*>(backend)->iface->free(backend);
+    delete record;
+}
+
+nuka_phi_backend* nuka_device_backend(nuka_device_handle device) {
+    auto* record = reinterpret_cast<DeviceRecord*>(device);
+    return record != nullptr ? reinterpret_cast<nuka_phi_backend*>(record->backend) : nullptr;
+}
+
+nuka_result_t nuka_world_create_from_template(nuka_device_handle device, const nuka_template_desc_t* tmpl,
+                                              const nuka_world_desc_t* desc, nuka_world_handle* out) {
+    if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    *out = nullptr;
+    if (device == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "device is null");
+    if (tmpl == nullptr || desc == nullptr || desc->env_count == 0u) return Error(NUKA_RESULT_INVALID_ARG, "template, desc and env_count are required");
+    if (tmpl->struct_size != sizeof(nuka_template_desc_t) || desc->struct_size != sizeof(nuka_world_desc_t))
+        return Error(NUKA_RESULT_INVALID_ARG, "struct_size mismatch");
+    try {
+        auto world = std::make_unique<World>();
+        World& w = *world;
+        w.device = reinterpret_cast<DeviceRecord*>(device);
+        w.backend = reinterpret_cast<nuka_phi_backend*>(w.device->backend);
+        w.be = reinterpret_cast<nuka_phi_backend_head*>(w.backend)->iface;
+        Cook(*tmpl, &w.host);
+        w.cfg = *desc;
+        nuka_world_desc_t& cfg = w.cfg;   // nuka.h:160-173 defaults; pipeline.hpp SolverConfig; op_schema.hpp:598, 663
+        if (cfg.fixed_dt <= 0.0f) cfg.fixed_dt = 1.0f / 240.0f;
+        if (cfg.solver_vel_iters == 0u) cfg.solver_vel_iters = 10u;
+        if (cfg.solver_pos_iters == 0u) cfg.solver_pos_iters = 4u;
+        if (cfg.solver_pos_iters == 0xFFFFFFFFu) cfg.solver_pos_iters = 0u;
+        if (cfg.solver_pos_beta <= 0.0f) cfg.solver_pos_beta = 0.3f;
+        if (cfg.solver_pos_slop <= 0.0f) cfg.solver_pos_slop = 1.0e-3f;
+        if (cfg.solver_velocity_tolerance <= 0.0f) cfg.solver_velocity_tolerance = 1.0e-5f;
+        if (cfg.solver_baumgarte_max_velocity <= 0.0f) cfg.solver_baumgarte_max_velocity = 3.0e38f;
+        w.env_count = desc->env_count;
+        const ModelView& hc = w.host.counts;
+        const size_t E = w.env_count, nl = hc.links_per_env, nb = hc.bodies_per_env, md = hc.max_dof, S = hc.contact_slots, R = hc.rows_per_env;
+        if (E * std::max<size_t>(R, 1u) > 0xFFFFFFFFull / 2u || E * nl * 7u > 0xFFFFFFFFull) throw std::invalid_argument("world too large for 32-bit row indices");
+        if (hc.rows_per_env > 0u && SolverHeadCapacity(hc, hc.contact_slots, 150u * 1024u) == 0u) throw std::invalid_argument("solver tile does not fit LDS");
+        // arena layout: template tables first, then the env-major fields, each on a 256-byte boundary (buffer.hpp:39)
+        size_t cursor = 0u;
+#define X(name, dtype) Place<int>(w.fields, #name, dtype, w.host.name.size(), &cursor, true);
+        NKH_MODEL_FIELDS(X)
+#undef X
+#define X(name, dtype, count) Place<int>(w.fields, #name, dtype, size_t(count), &cursor, false);
+        NKH_DATA_FIELDS(X)
+#undef X
+        w.arena_bytes = cursor;
+        uint8_t status = 0u;
+        nuka_phi_buffer_type* type = BackendDeviceBufferType(w.device->backend);
+        w.arena = reinterpret_cast<nuka_phi_buffer_type_head*>(type)->iface->alloc(type, w.arena_bytes, &status);
+        if (w.arena == nullptr) return Error(NUKA_RESULT_OUT_OF_MEMORY, "arena allocation failed");
+        w.initial = reinterpret_cast<nuka_phi_buffer_type_head*>(type)->iface->alloc(type, w.arena_bytes, &status);
+        if (w.initial == nullptr) return Error(NUKA_RESULT_OUT_OF_MEMORY, "reset snapshot allocation failed");
+        if (Iface(w.arena)->memset(w.arena, 0u, 0u, w.arena_bytes) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "arena clear failed");
+        char* base = static_cast<char*>(Iface(w.arena)->base(w.arena));
+        w.model = hc;
+        size_t f = 0u;
+#define X(name, dtype) { const Field& fld = w.fields[f++]; \
+            w.model.name = reinterpret_cast<decltype(w.model.name)>(base + fld.offset); \
+            if (fld.count > 0u && Iface(w.arena)->upload(w.arena, w.host.name.data(), fld.offset, fld.count * fld.elem_bytes) != uint8_t(Status::Ok)) \
+                return Error(NUKA_RESULT_DEVICE_ERROR, "template upload failed"); }
+        NKH_MODEL_FIELDS(X)
+#undef X
+#define X(name, dtype, count) { const Field& fld = w.fields[f++]; w.data.name = reinterpret_cast<decltype(w.data.name)>(base + fld.offset); }
+        NKH_DATA_FIELDS(X)
+#undef X
+        // initial state: identity poses, cooked static poses, no rows
+        {
+            std::vector<float> base_pose(E * 7u, 0.0f), link_pose(E * nl * 7u, 0.0f), body_pose(E * nb * 7u, 0.0f);
+            for (size_t e = 0u; e < E; ++e) {
+                base_pose[e * 7u + 3u] = 1.0f;
+                for (size_t l = 0u; l < nl; ++l) link_pose[(e * nl + l) * 7u + 3u] = 1.0f;
+                for (size_t b = 0u; b < nb; ++b) std::memcpy(&body_pose[(e * nb + b) * 7u], &w.host.body_init_pose[b * 7u], 7u * sizeof(float));
+            }
+            std::vector<uint32_t> invalid(E * R, kInvalid);
+            auto put = [&](void* field, const void* src, size_t bytes) {
+                if (bytes == 0u) return true;
+                return Iface(w.arena)->upload(w.arena, src, size_t(static_cast<char*>(field) - base), bytes) == uint8_t(Status::Ok);
+            };
+            if (!put(w.data.base_pose, base_pose.data(), base_pose.size() * 4u) || !put(w.data.link_pose, link_pose.data(), link_pose.size() * 4u) ||
+                !put(w.data.body_pose, body_pose.data(), body_pose.size() * 4u) || !put(w.data.row_cj_link, invalid.data(), invalid.size() * 4u) ||
+                !put(w.data.row_cj_link_b, invalid.data(), invalid.size() * 4u)) return Error(NUKA_RESULT_DEVICE_ERROR, "initial state upload failed");
+        }
+        if (Iface(w.initial)->copy_from(w.initial, w.arena, 0u, 0u, w.arena_bytes) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "snapshot failed");
+        BuildPipeline(w);
+        if (w.be->synchronize(w.backend, nullptr) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "device error during world creation");
+        *out = reinterpret_cast<nuka_world_handle>(world.release());
+        return NUKA_RESULT_OK;
+    } catch (const std::invalid_argument& e) {
+        return Error(NUKA_RESULT_INVALID_ARG, e.what());
+    } catch (const std::bad_alloc&) {
+        return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
+    } catch (const std::exception& e) {
+        return Error(NUKA_RESULT_INTERNAL, e.what());
+    }
+}
+
+void nuka_world_destroy(nuka_world_handle world) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return;
+    (void)w->be->synchronize(w->backend, nullptr);
+    delete w;
+}
+
+nuka_result_t nuka_world_step(nuka_world_handle world) { return nuka_world_step_n(world, 1u); }
+
+nuka_result_t nuka_world_step_n(nuka_world_handle world, uint32_t step_count) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    try {
+        return StepN(*w, step_count);
+    } catch (const std::exception& e) {
+        std::fprintf(stderr, "nuka_world_step_n: %s\n", e.what());
+        return Error(NUKA_RESULT_INTERNAL, e.what());
+    }
+}
+
+nuka_result_t nuka_world_set_execution_mode(nuka_world_handle world, nuka_execution_mode_t mode) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (mode != NUKA_EXECUTION_EAGER && mode != NUKA_EXECUTION_GRAPH) return Error(NUKA_RESULT_INVALID_ARG, "unknown execution mode");
+    if (mode == NUKA_EXECUTION_GRAPH) {   // capture without advancing state; fail explicitly if unavailable (nuka.h:275-277)
+        const nuka_result_t prepared = PreparePlan(*w);
+        if (prepared != NUKA_RESULT_OK) return prepared;
+    }
+    w->mode = mode;
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_set_velocity_iterations(nuka_world_handle world, uint32_t iterations) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (iterations == 0u || iterations > 65535u) return Error(NUKA_RESULT_INVALID_ARG, "iterations must be in 1..65535");
+    if (w->be->synchronize(w->backend, nullptr) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "device error");
+    w->cfg.solver_vel_iters = iterations;
+    w->p_solve.iterations = iterations;
+    InvalidatePlan(*w);   // a changed value invalidates the execution graph (nuka.h:287-288)
+    if (w->mode == NUKA_EXECUTION_GRAPH) return PreparePlan(*w);
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_get_velocity_iterations(nuka_world_handle world, uint32_t* out_iterations) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (out_iterations == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    *out_iterations = w->p_solve.iterations;
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_synchronize(nuka_world_handle world) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    nuka_phi_execution_error error{};
+    if (w->be->synchronize(w->backend, &error) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, error.message);
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_reset(nuka_world_handle world) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (Iface(w->arena)->copy_from(w->arena, w->initial, 0u, 0u, w->arena_bytes) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "reset copy failed");
+    return nuka_world_synchronize(world);
+}
+
+nuka_result_t nuka_world_dispatch_op(nuka_world_handle world, uint16_t op, uint32_t variant) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (op >= uint16_t(NkOp::Count)) return Error(NUKA_RESULT_INVALID_ARG, "unknown op");
+    const void* params = nullptr;
+    for (const nuka_phi_op_call& call : w->calls) if (call.op == op) { params = call.params; break; }
+    if (op == uint16_t(NkOp::ArticulationDynamics) && variant == 1u) params = &w->p_dynamics_probe;
+    if (op == uint16_t(NkOp::ContactWarmStart) && variant == 1u) params = &w->p_warm1;
+    if (params == nullptr) return Error(NUKA_RESULT_NOT_SUPPORTED, "op is not part of this world's pipeline");
+    const nuka_phi_op_call call{op, params};
+    const uint8_t status = w->be->dispatch(w->backend, reinterpret_cast<const nuka_phi_model_view*>(&w->model),
+                                           reinterpret_cast<const nuka_phi_data_view*>(&w->data), &call);
+    if (status != uint8_t(Status::Ok)) return Error(MapStatus(status), std::string("dispatch failed: ") + OpName(static_cast<NkOp>(op)));
+    return NUKA_RESULT_OK;
+}
+
+const char* nuka_field_names(void) {
+#define X(name, ...) #name ","
+    return NKH_MODEL_FIELDS(X) NKH_DATA_FIELDS(X) "";
+#undef X
+}
+
+nuka_state_field_t nuka_field_from_name(const char* name) {
+    if (name == nullptr) return 0xFFFFFFFFu;
+    uint32_t index = 0u;
+#define X(field, ...) if (std::strcmp(name, #field) == 0) return index; ++index;
+    NKH_MODEL_FIELDS(X)
+    NKH_DATA_FIELDS(X)
+#undef X
+    return 0xFFFFFFFFu;
+}
+
+nuka_result_t nuka_world_get_buffer_view(nuka_world_handle world, nuka_state_field_t field, nuka_buffer_view_t* out) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    if (field >= w->fields.size()) return Error(NUKA_RESULT_NOT_SUPPORTED, "unknown field");
+    const Field& f = w->fields[field];
+    out->device_ptr = static_cast<char*>(Iface(w->arena)->base(w->arena)) + f.offset;
+    out->element_count = f.count;
+    out->element_stride_bytes = f.elem_bytes;
+    out->dtype = uint8_t(f.dtype);
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_upload_field(nuka_world_handle world, nuka_state_field_t field, const void* bytes, size_t nbytes, size_t byte_offset) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (field >= w->fields.size()) return Error(NUKA_RESULT_NOT_SUPPORTED, "unknown field");
+    const Field& f = w->fields[field];
+    const size_t size = f.count * f.elem_bytes;
+    if (byte_offset > size || nbytes > size - byte_offset || (bytes == nullptr && nbytes > 0u)) return Error(NUKA_RESULT_INVALID_ARG, "range exceeds the field");
+    if (nbytes == 0u) return NUKA_RESULT_OK;
+    return MapStatus(Iface(w->arena)->upload(w->arena, bytes, f.offset + byte_offset, nbytes));
+}
+
+nuka_result_t nuka_world_download_field(nuka_world_handle world, nuka_state_field_t field, void* bytes, size_t nbytes, size_t byte_offset) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (field >= w->fields.size()) return Error(NUKA_RESULT_NOT_SUPPORTED, "unknown field");
+    const Field& f = w->fields[field];
+    const size_t size = f.count * f.elem_bytes;
+    if (byte_offset > size || nbytes > size - byte_offset || (bytes == nullptr && nbytes > 0u)) return Error(NUKA_RESULT_INVALID_ARG, "range exceeds the field");
+    if (nbytes == 0u) return NUKA_RESULT_OK;
+    return MapStatus(Iface(w->arena)->download(w->arena, bytes, f.offset + byte_offset, nbytes));
+}
+
+nuka_result_t nuka_world_get_info(nuka_world_handle world, nuka_world_info_t* out) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    const ModelView& m = w->model;
+    *out = {w->env_count, m.links_per_env, m.bodies_per_env, m.dof, m.max_dof, m.contact_slots, m.rows_per_env, uint32_t(w->calls.size())};
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_time_steps(nuka_world_handle world, uint32_t step_count, float* out_total_ms) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (out_total_ms == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    nuka_phi_event* start = w->be->event_new(w->backend);
+    nuka_phi_event* stop = w->be->event_new(w->backend);
+    if (start == nullptr || stop == nullptr) return Error(NUKA_RESULT_DEVICE_ERROR, "event creation failed");
+    w->be->event_record(w->backend, start);
+    const nuka_result_t r = StepN(*w, step_count);
+    w->be->event_record(w->backend, stop);
+    w->be->event_wait(w->backend, stop);
+    *out_total_ms = w->be->event_elapsed_ms(w->backend, start, stop);
+    w->be->event_free(w->backend, start);
+    w->be->event_free(w->backend, stop);
+    return r;
+}
+
+nuka_result_t nuka_world_profile_ops(nuka_world_handle world, uint32_t step_count, float* out_ms, uint16_t* out_ops) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (out_ms == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    const size_t n = w->calls.size();
+    std::vector<nuka_phi_event*> events(n + 1u, nullptr);
+    for (auto& e : events) e = w->be->event_new(w->backend);
+    for (size_t i = 0u; i < n; ++i) { out_ms[i] = 0.0f; if (out_ops != nullptr) out_ops[i] = w->calls[i].op; }
+    nuka_result_t result = NUKA_RESULT_OK;
+    for (uint32_t s = 0u; s < step_count && result == NUKA_RESULT_OK; ++s) {
+        w->be->event_record(w->backend, events[0]);
+        for (size_t i = 0u; i < n; ++i) {
+            const uint8_t status = w->be->dispatch(w->backend, reinterpret_cast<const nuka_phi_model_view*>(&w->model),
+                                                   reinterpret_cast<const nuka_phi_data_view*>(&w->data), &w->calls[i]);
+            if (status != uint8_t(Status::Ok)) { result = Error(MapStatus(status), "profile dispatch failed"); break; }
+            w->be->event_record(w->backend, events[i + 1u]);
+        }
+        w->be->event_wait(w->backend, events[n]);
+        if (result == NUKA_RESULT_OK)
+            for (size_t i = 0u; i < n; ++i) out_ms[i] += w->be->event_elapsed_ms(w->backend, events[i], events[i + 1u]);
+    }
+    (void)w->be->synchronize(w->backend, nullptr);
+    for (auto* e : events) w->be->event_free(w->backend, e);
+    return result;
+}
+
+nuka_result_t nuka_device_copy_bandwidth(nuka_device_handle device, size_t bytes, uint32_t repeats, float* out_gb_per_s) {
+    auto* record = reinterpret_cast<DeviceRecord*>(device);
+    if (record == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "device is null");
+    if (out_gb_per_s == nullptr || bytes == 0u || repeats == 0u) return Error(NUKA_RESULT_INVALID_ARG, "bytes, repeats and out are required");
+    auto* backend = reinterpret_cast<nuka_phi_backend*>(record->backend);
+    const nuka_phi_backend_i* be = reinterpret_cast<nuka_phi_backend_head*>(backend)->iface;
+    nuka_phi_buffer_type* type = BackendDeviceBufferType(record->backend);
+    uint8_t status = 0u;
+    nuka_phi_buffer* a = reinterpret_cast<nuka_phi_buffer_type_head*>(type)->iface->alloc(type, bytes, &status);
+    nuka_phi_buffer* b = reinterpret_cast<nuka_phi_buffer_type_head*>(type)->iface->alloc(type, bytes, &status);
+    if (a == nullptr || b == nullptr) {
+        if (a != nullptr) Iface(a)->free(a);
+        if (b != nullptr) Iface(b)->free(b);
+        return Error(NUKA_RESULT_OUT_OF_MEMORY, "copy buffers");
+    }
+    (void)Iface(a)->memset(a, 1u, 0u, bytes);
+    (void)Iface(b)->copy_from(b, a, 0u, 0u, bytes);
+    nuka_phi_event* start = be->event_new(backend);
+    nuka_phi_event* stop = be->event_new(backend);
+    be->event_record(backend, start);
+    for (uint32_t i = 0u; i < repeats; ++i) (void)Iface(b)->copy_from(b, a, 0u, 0u, bytes);
+    be->event_record(backend, stop);
+    be->event_wait(backend, stop);
+    const float ms = be->event_elapsed_ms(backend, start, stop);
+    be->event_free(backend, start);
+    be->event_free(backend, stop);
+    Iface(a)->free(a);
+    Iface(b)->free(b);
+    *out_gb_per_s = ms > 0.0f ? float(2.0 * double(bytes) * repeats / (double(ms) * 1.0e6)) : 0.0f;
+    return NUKA_RESULT_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,536 @@
+/*
+ * CPU oracle (test infrastructure; see nuka_oracle.h): collidable poses, AABBs, candidate pairs in
+ * canonical order, sphere/box x plane manifolds, pair-driven row assembly and chain Jacobians.
+ */
+#include "nko_internal.h"
+
+#define SHAPE_STRIDE 13u   /* phi/op_schema.hpp:26 kShapeTableRowStride */
+
+typedef struct {
+    uint32_t kind; float p[4]; uint32_t contype, conaffinity; int32_t body_id; uint32_t group, profile;
+} shape_row;
+
+/* prims_types.cuh:55-72 LoadPrimShape */
+static shape_row load_shape(const float* table, uint32_t row) {
+    const float* q = table + (size_t)row * SHAPE_STRIDE;
+    shape_row s;
+    s.kind = f2u(q[0]);
+    s.p[0] = q[1]; s.p[1] = q[2]; s.p[2] = q[3]; s.p[3] = q[4];
+    s.contype = f2u(q[5]); s.conaffinity = f2u(q[6]);
+    s.body_id = (int32_t)f2u(q[8]); s.group = f2u(q[9]); s.profile = f2u(q[12]);
+    return s;
+}
+
+/* ---- SyncLinkBodyPose (ops/sync_body_pose.cu:23-52, 54-83) -------------- */
+void nko_env_sync_body_pose(nko_world* w, uint32_t env) {
+    const nko_template* t = &w->t;
+    const size_t lbase = (size_t)env * t->nl, bbase = (size_t)env * t->nb;
+    for (uint32_t l = 0u; l < t->nl; ++l) {
+        const uint32_t b = t->link_body[l];
+        if (b >= t->nb) continue;
+        xform world = xform_load(w->link_pose + (lbase + l) * 7u);
+        if (t->link_geom_kind[l] != 0u) world = nko_compose_hd(world, xform_load(t->link_geom_local + 7u * l));
+        xform_store(w->body_pose + (bbase + b) * 7u, world);
+    }
+    for (uint32_t b = 0u; b < t->nb; ++b) {
+        const uint32_t link = t->body_collidable_link[b];
+        if (link != NKO_INVALID) {
+            if (link >= t->nl) continue;
+            xform_store(w->body_pose + (bbase + b) * 7u,
+                        nko_compose_hd(xform_load(w->link_pose + (lbase + link) * 7u), xform_load(t->body_collidable_local + 7u * b)));
+            continue;
+        }
+        const uint32_t owner = t->body_collidable_body[b];
+        if (owner == NKO_INVALID || owner >= t->nb) continue;
+        xform_store(w->body_pose + (bbase + b) * 7u,
+                    nko_compose_hd(xform_load(w->body_pose + (bbase + owner) * 7u), xform_load(t->body_collidable_local + 7u * b)));
+    }
+}
+
+/* broadphase.cu:154-170 RotAbs */
+static v3 rot_abs(quat q, v3 v) {
+    const v3 cx = nko_prim_rotate(q, v3_make(1, 0, 0)), cy = nko_prim_rotate(q, v3_make(0, 1, 0)), cz = nko_prim_rotate(q, v3_make(0, 0, 1));
+    return v3_make(fabsf(cx.x) * v.x + fabsf(cy.x) * v.y + fabsf(cz.x) * v.z,
+                   fabsf(cx.y) * v.x + fabsf(cy.y) * v.y + fabsf(cz.y) * v.z,
+                   fabsf(cx.z) * v.x + fabsf(cy.z) * v.y + fabsf(cz.z) * v.z);
+}
+
+/* collision/contact_query.hpp:17-31 */
+static float contact_query_reach(float thickness, float margin) { return fmaxf(0.02f, 2.0f * (2.0f * thickness + margin)); }
+static float contact_motion_radius(float base, float dt, float sa, float sb, float relax) { return base + dt * (sa + sb) * (2.0f / relax); }
+
+/* ---- BuildAabbs (broadphase.cu:173-270). Link-owned collidables keep zero body velocity and
+ * zero previous motion on this path (nothing writes them for inv_mass 0 rows), so speed = 0. ---- */
+void nko_env_aabbs(nko_world* w, uint32_t env) {
+    const nko_template* t = &w->t;
+    const size_t bbase = (size_t)env * t->nb;
+    const float margin = fmaxf(w->cfg.solver_contact_margin, 0.0005f);   /* pipeline.cpp:613 */
+    const float reach = contact_query_reach(0.0f, w->cfg.solver_contact_margin);   /* pipeline.cpp:202 */
+    for (uint32_t b = 0u; b < t->nb; ++b) {
+        const shape_row s = load_shape(t->shape_table, b);
+        const xform xf = xform_load(w->body_pose + (bbase + b) * 7u);
+        float* lo = w->body_aabb_lo + (bbase + b) * 3u;
+        float* hi = w->body_aabb_hi + (bbase + b) * 3u;
+        v3 he = v3_make(0, 0, 0);
+        if (s.kind == NKO_SPHERE) he = v3_make(s.p[0], s.p[0], s.p[0]);
+        else if (s.kind == NKO_BOX) he = rot_abs(xf.r, v3_make(s.p[0], s.p[1], s.p[2]));
+        else if (s.kind == NKO_PLANE) {
+            lo[0] = lo[1] = lo[2] = -FLT_MAX; hi[0] = hi[1] = hi[2] = FLT_MAX;
+            continue;
+        } else {
+            lo[0] = lo[1] = lo[2] = FLT_MAX; hi[0] = hi[1] = hi[2] = -FLT_MAX;
+            continue;
+        }
+        const float speed = 0.0f;
+        const float m = fmaxf(margin, fminf(contact_motion_radius(margin, w->cfg.fixed_dt, speed, 0.0f, 0.9f), reach));
+        const v3 c = xf.p;
+        lo[0] = c.x - he.x - m; lo[1] = c.y - he.y - m; lo[2] = c.z - he.z - m;
+        hi[0] = c.x + he.x + m; hi[1] = c.y + he.y + m; hi[2] = c.z + he.z + m;
+    }
+}
+
+/* collision/shape_kind.hpp:26-33 ShapeFilterAdmits */
+static int shape_filter_admits(uint32_t ta, uint32_t aa, uint32_t ga_, uint32_t tb, uint32_t ab, uint32_t gb_) {
+    if (((ta & ab) | (tb & aa)) == 0u) return 0;
+    const int32_t ga = (int32_t)ga_, gb = (int32_t)gb_;
+    return !(ga != 0 && gb != 0 && (ga > 0 ? (ga != gb && gb > 0) : ga == gb));
+}
+
+/* ---- candidate pairs (broadphase.cu:408-474 EnvAllPairsKernel, 478-542 canonical sort).
+ * Emission order is a race in the reference and is erased by the stable sort on (a, b); the
+ * oracle enumerates i<j ascending, which already is that order.  Overflow keeps the first
+ * `capacity` emitted pairs in the reference (racy); the oracle keeps the smallest keys. ---- */
+void nko_env_pairs(nko_world* w, uint32_t env) {
+    const nko_template* t = &w->t;
+    const size_t bbase = (size_t)env * t->nb;
+    uint32_t* pairs = w->candidate_pairs + (size_t)env * t->slots * 2u;
+    uint32_t count = 0u;
+    w->env_status[env] &= ~(uint32_t)NKO_STATUS_PAIR_OVERFLOW;
+    for (uint32_t i = 0u; i < t->nb; ++i)
+        for (uint32_t j = i + 1u; j < t->nb; ++j) {
+            const float* alo = w->body_aabb_lo + (bbase + i) * 3u, *ahi = w->body_aabb_hi + (bbase + i) * 3u;
+            const float* blo = w->body_aabb_lo + (bbase + j) * 3u, *bhi = w->body_aabb_hi + (bbase + j) * 3u;
+            if (ahi[0] < blo[0] || alo[0] > bhi[0]) continue;
+            if (ahi[1] < blo[1] || alo[1] > bhi[1]) continue;
+            if (ahi[2] < blo[2] || alo[2] > bhi[2]) continue;
+            const shape_row sa = load_shape(t->shape_table, i), sb = load_shape(t->shape_table, j);
+            if (sa.body_id < 0 && sb.body_id < 0) continue;
+            if (!shape_filter_admits(sa.contype, sa.conaffinity, sa.group, sb.contype, sb.conaffinity, sb.group)) continue;
+            if (count < t->slots) { pairs[2u * count] = i; pairs[2u * count + 1u] = j; ++count; }
+            else w->env_status[env] |= NKO_STATUS_PAIR_OVERFLOW;
+        }
+    w->pair_count[env] = count;
+}
+
+/* ---- manifolds (collision/analytical_manifold.hpp) ----------------------- */
+typedef struct { v3 cx, cy, cz, t; float radius; v3 half; } prim;
+
+static prim make_prim(shape_row s, xform xf) {   /* narrowphase_prims.cu:34-46 MakePrim */
+    prim p;
+    p.cx = nko_prim_rotate(xf.r, v3_make(1, 0, 0)); p.cy = nko_prim_rotate(xf.r, v3_make(0, 1, 0));
+    p.cz = nko_prim_rotate(xf.r, v3_make(0, 0, 1)); p.t = xf.p;
+    p.radius = s.p[0]; p.half = v3_make(s.p[0], s.p[1], s.p[2]);
+    return p;
+}
+static v3 norm_or(v3 v, v3 fallback) {   /* analytical_manifold.hpp:194-198 Norm */
+    const float len = sqrtf(v.x * v.x + v.y * v.y + v.z * v.z);
+    if (len < 1.0e-12f) return fallback;
+    return v3_make(v.x / len, v.y / len, v.z / len);
+}
+typedef struct { uint32_t count; v3 position[4]; v3 normal[4]; float penetration[4]; uint64_t key[4]; } manifold;
+
+/* analytical_manifold.hpp:451-463 SpherePlane */
+static void sphere_plane(const prim* sph, const prim* plane, float query, manifold* out) {
+    out->count = 0u;
+    const v3 n = norm_or(plane->cz, v3_make(0, 0, 1));
+    const float signed_dist = v3_dot(v3_sub(sph->t, plane->t), n);
+    const float pen = sph->radius - signed_dist;
+    if (pen <= -query) return;
+    out->position[0] = v3_sub(sph->t, v3_scale(n, sph->radius - 0.5f * pen));
+    out->normal[0] = n; out->penetration[0] = pen; out->key[0] = 0u; out->count = 1u;
+}
+
+/* analytical_manifold.hpp:469-493 BoxPlane + :273-311 ReduceAndEmit */
+static void box_plane(const prim* box, const prim* plane, float query, manifold* out) {
+    out->count = 0u;
+    const v3 n = norm_or(plane->cz, v3_make(0, 0, 1));
+    v3 position[8]; float pen[8]; uint32_t feature[8];
+    int ncand = 0;
+    for (uint32_t c = 0u; c < 8u; ++c) {
+        const float sx = (c & 1u) ? 1.0f : -1.0f, sy = (c & 2u) ? 1.0f : -1.0f, sz = (c & 4u) ? 1.0f : -1.0f;
+        const v3 l = v3_make(sx * box->half.x, sy * box->half.y, sz * box->half.z);
+        const v3 corner = v3_make(box->cx.x * l.x + box->cy.x * l.y + box->cz.x * l.z + box->t.x,
+                                  box->cx.y * l.x + box->cy.y * l.y + box->cz.y * l.z + box->t.y,
+                                  box->cx.z * l.x + box->cy.z * l.y + box->cz.z * l.z + box->t.z);
+        const float sd = v3_dot(v3_sub(corner, plane->t), n);
+        if (sd < query) {
+            position[ncand] = v3_sub(corner, v3_scale(n, 0.5f * sd));
+            pen[ncand] = -sd; feature[ncand] = c; ++ncand;
+        }
+    }
+    if (ncand <= 0) return;
+    const int keep = ncand < 4 ? ncand : 4;
+    for (int s = 0; s < keep; ++s) {
+        int best = s;
+        for (int i = s + 1; i < ncand; ++i)
+            if (pen[i] > pen[best] || (pen[i] == pen[best] && feature[i] < feature[best])) best = i;
+        const v3 tp = position[s]; position[s] = position[best]; position[best] = tp;
+        const float tf = pen[s]; pen[s] = pen[best]; pen[best] = tf;
+        const uint32_t tk = feature[s]; feature[s] = feature[best]; feature[best] = tk;
+    }
+    for (int i = 1; i < keep; ++i) {
+        const v3 kp = position[i]; const float kf = pen[i]; const uint32_t kk = feature[i];
+        int j = i - 1;
+        while (j >= 0 && feature[j] > kk) { position[j + 1] = position[j]; pen[j + 1] = pen[j]; feature[j + 1] = feature[j]; --j; }
+        position[j + 1] = kp; pen[j + 1] = kf; feature[j + 1] = kk;
+    }
+    for (int i = 0; i < keep; ++i) {
+        out->position[i] = position[i]; out->normal[i] = n; out->penetration[i] = pen[i]; out->key[i] = feature[i];
+    }
+    out->count = (uint32_t)keep;
+}
+
+/* analytical_manifold.hpp:934-966 PrimitivePair (sphere/box x plane subset) */
+static void primitive_pair(uint32_t ka, const prim* a, uint32_t kb, const prim* b, float query, manifold* out) {
+    out->count = 0u;
+    if (ka == NKO_SPHERE && kb == NKO_PLANE) { sphere_plane(a, b, query, out); return; }
+    if (ka == NKO_BOX && kb == NKO_PLANE) { box_plane(a, b, query, out); return; }
+    if (ka == NKO_PLANE && (kb == NKO_SPHERE || kb == NKO_BOX)) {
+        if (kb == NKO_SPHERE) sphere_plane(b, a, query, out); else box_plane(b, a, query, out);
+        for (uint32_t i = 0u; i < out->count; ++i) out->normal[i] = v3_make(-out->normal[i].x, -out->normal[i].y, -out->normal[i].z);
+    }
+}
+
+uint32_t nko_sphere_plane(const float sphere_pose[7], float radius, const float plane_pose[7], float query,
+                          float point[3], float normal[3], float* penetration) {
+    shape_row s; memset(&s, 0, sizeof(s)); s.p[0] = radius;
+    shape_row pl; memset(&pl, 0, sizeof(pl));
+    const prim a = make_prim(s, xform_load(sphere_pose)), b = make_prim(pl, xform_load(plane_pose));
+    manifold m; sphere_plane(&a, &b, query, &m);
+    if (m.count) {
+        point[0] = m.position[0].x; point[1] = m.position[0].y; point[2] = m.position[0].z;
+        normal[0] = m.normal[0].x; normal[1] = m.normal[0].y; normal[2] = m.normal[0].z; *penetration = m.penetration[0];
+    }
+    return m.count;
+}
+
+uint32_t nko_box_plane(const float box_pose[7], const float half[3], const float plane_pose[7], float query,
+                       float points[12], float normal[3], float penetration[4], uint32_t feature[4]) {
+    shape_row s; memset(&s, 0, sizeof(s)); s.p[0] = half[0]; s.p[1] = half[1]; s.p[2] = half[2];
+    shape_row pl; memset(&pl, 0, sizeof(pl));
+    const prim a = make_prim(s, xform_load(box_pose)), b = make_prim(pl, xform_load(plane_pose));
+    manifold m; box_plane(&a, &b, query, &m);
+    for (uint32_t i = 0u; i < m.count; ++i) {
+        points[3u * i] = m.position[i].x; points[3u * i + 1u] = m.position[i].y; points[3u * i + 2u] = m.position[i].z;
+        penetration[i] = m.penetration[i]; feature[i] = (uint32_t)m.key[i];
+        normal[0] = m.normal[i].x; normal[1] = m.normal[i].y; normal[2] = m.normal[i].z;
+    }
+    return m.count;
+}
+
+/* ---- contact identity (nk/contact/contact_identity.hpp:98-157) ----------- */
+static int32_t quantize_coord(float value) {
+    const float scaled = value * 4096.0f;
+    const float rounded = scaled >= 0.0f ? scaled + 0.5f : scaled - 0.5f;
+    return (int32_t)rounded;
+}
+static uint64_t hash_word(uint64_t hash, uint64_t word) { hash ^= word; hash *= 1099511628211ull; return hash; }
+static uint64_t feature_token(uint32_t feature, v3 p) {
+    if (feature != 0xffffffffu) return 0x8000000000000000ull | (uint64_t)feature;
+    uint64_t h = 1469598103934665603ull;
+    h = hash_word(h, (uint32_t)quantize_coord(p.x)); h = hash_word(h, (uint32_t)quantize_coord(p.y));
+    h = hash_word(h, (uint32_t)quantize_coord(p.z));
+    return h & 0x7fffffffffffffffull;
+}
+static v3 inverse_transform_point(xform xf, v3 wp) {   /* prims_types.cuh:98-105 */
+    const v3 v = v3_sub(wp, xf.p);
+    const v3 qv = v3_make(-xf.r.x, -xf.r.y, -xf.r.z);
+    const v3 t = v3_scale(v3_cross(qv, v), 2.0f);
+    return v3_add(v3_add(v, v3_scale(t, xf.r.w)), v3_cross(qv, t));
+}
+
+/* ---- NarrowphasePrimitives (narrowphase_prims.cu:181-366, analytic route) ---- */
+void nko_env_narrowphase(nko_world* w, uint32_t env) {
+    const nko_template* t = &w->t;
+    const size_t bbase = (size_t)env * t->nb;
+    const float separation = fmaxf(w->cfg.solver_contact_margin, 0.0005f);   /* :425 */
+    const float reach = contact_query_reach(0.0f, w->cfg.solver_contact_margin);
+    const uint32_t live = w->pair_count[env];
+    uint32_t contacts = 0u;
+    for (uint32_t slot = 0u; slot < t->slots; ++slot) {
+        const size_t gid = (size_t)env * t->slots + slot;
+        manifold m; m.count = 0u;
+        uint32_t a = 0u, b = 0u;
+        const uint32_t law = 2u;   /* kContactLawSpeculative: no MuJoCo-sourced profile on this path (:232) */
+        if (slot < live) {
+            a = w->candidate_pairs[gid * 2u]; b = w->candidate_pairs[gid * 2u + 1u];
+            const shape_row sa = load_shape(t->shape_table, a), sb = load_shape(t->shape_table, b);
+            const xform xa = xform_load(w->body_pose + (bbase + a) * 7u), xb = xform_load(w->body_pose + (bbase + b) * 7u);
+            const prim pa = make_prim(sa, xa), pb = make_prim(sb, xb);
+            /* :243-250 query band; both speeds are zero for link-owned collidables */
+            const float query = fmaxf(separation, fminf(contact_motion_radius(2.0f * separation, w->cfg.fixed_dt, 0.0f, 0.0f, 0.9f), reach));
+            primitive_pair(sa.kind, &pa, sb.kind, &pb, query, &m);
+            for (uint32_t i = 0u; i < m.count; ++i) m.penetration[i] += separation;   /* :295-296 */
+        }
+        w->ucontact_count[gid] = m.count;
+        w->ucontact_law[gid] = law;
+        for (uint32_t i = 0u; i < m.count; ++i) {
+            const size_t at = gid * 4u + i;
+            w->ucontact_point[3u * at] = m.position[i].x; w->ucontact_point[3u * at + 1u] = m.position[i].y; w->ucontact_point[3u * at + 2u] = m.position[i].z;
+            w->ucontact_normal[3u * at] = m.normal[i].x; w->ucontact_normal[3u * at + 1u] = m.normal[i].y; w->ucontact_normal[3u * at + 2u] = m.normal[i].z;
+            w->ucontact_depth[at] = m.penetration[i];
+            w->ucontact_a[at] = a; w->ucontact_b[at] = b;
+            /* MakeContactId with CollidableRef type 0: a < b already canonical (:108-157) */
+            const uint32_t feature = m.key[i] == 0u ? 0xffffffffu : (uint32_t)m.key[i];
+            const v3 la = inverse_transform_point(xform_load(w->body_pose + (bbase + a) * 7u), m.position[i]);
+            const v3 lb = inverse_transform_point(xform_load(w->body_pose + (bbase + b) * 7u), m.position[i]);
+            uint64_t h = 1469598103934665603ull;
+            h = hash_word(h, feature_token(feature, la)); h = hash_word(h, feature_token(feature, lb));
+            h = hash_word(h, i); h = hash_word(h, 0u); h = hash_word(h, 0u);
+            w->ucontact_id_pair[at] = ((uint64_t)(a & 0x0fffffffu) << 32u) | (uint64_t)(b & 0x0fffffffu);
+            w->ucontact_id_feature[at] = h;
+        }
+        contacts += m.count;
+    }
+    w->contact_count[env] = contacts;
+}
+
+/* math/cuda_vec_ops.cuh:150-183 NormalizeOrUp + ContactTangentBasis */
+void nko_contact_tangent_basis(const float normal[3], float t1[3], float t2[3]) {
+    v3 n = v3_make(normal[0], normal[1], normal[2]);
+    const float l = v3_dot(n, n);
+    if (l > 1.0e-10f) { const float inv = nko_rsqrt(l); n = v3_make(n.x * inv, n.y * inv, n.z * inv); }
+    else n = v3_make(0.0f, 0.0f, 1.0f);
+    v3 reference = v3_make(1.0f, 0.0f, 0.0f);
+    if (fabsf(n.x) > 0.9f) reference = v3_make(0.0f, 1.0f, 0.0f);
+    const float proj = v3_dot(reference, n);
+    v3 ta = v3_make(reference.x - proj * n.x, reference.y - proj * n.y, reference.z - proj * n.z);
+    const float len_sq = v3_dot(ta, ta);
+    if (len_sq > 1.0e-12f) { const float s = nko_rsqrt(len_sq); ta = v3_make(ta.x * s, ta.y * s, ta.z * s); }
+    else ta = v3_make(1.0f, 0.0f, 0.0f);
+    const v3 tb = v3_cross(n, ta);
+    t1[0] = ta.x; t1[1] = ta.y; t1[2] = ta.z; t2[0] = tb.x; t2[1] = tb.y; t2[2] = tb.z;
+}
+
+/* union_types.cuh:187-193 ContactRowBound */
+static uint32_t contact_row_bound(const uint32_t* extent, uint32_t env, uint32_t contact_rows) {
+    const uint32_t previous = extent[2u * env], current = extent[2u * env + 1u];
+    if (previous == 0u || current == 0u) return contact_rows;
+    const uint32_t m = (previous > current ? previous : current) - 1u;
+    return m < contact_rows ? m : contact_rows;
+}
+
+/* nk/solve/collidable_owner.hpp:25-62 ResolveCollidableOwner (one articulation per env) */
+static uint32_t resolve_side(const nko_template* t, uint32_t env, uint32_t collidable, int32_t body_id,
+                             uint32_t* index, uint32_t* link) {
+    *index = NKO_INVALID; *link = NKO_INVALID;
+    if (collidable >= t->nb) return NKO_INVALID;
+    uint32_t body = collidable;
+    if (body_id < 0) return NKO_SIDE_STATIC;
+    const uint32_t proxy = t->body_collidable_body[body];
+    if (proxy != NKO_INVALID) {
+        if (proxy >= t->nb) return NKO_INVALID;
+        body = proxy;
+        if (t->body_collidable_body[body] != NKO_INVALID) return NKO_INVALID;
+    }
+    const uint32_t l = t->body_to_link[body];
+    if (l == NKO_INVALID) { *index = env * t->nb + body; return NKO_SIDE_RIGID; }
+    if (l >= t->nl) return NKO_INVALID;
+    if (t->body_to_articulation[body] >= 1u) return NKO_INVALID;
+    *link = env * t->nl + l; *index = env;
+    return NKO_SIDE_ARTIC;
+}
+
+/* articulation_types.cuh:193-238 AccumulateChainJointForce with f = dir, tau = 0 */
+static void accumulate_chain(const nko_world* w, uint32_t env, uint32_t link_local, uint32_t dof_index, v3 point, v3 f, float* out) {
+    const nko_template* t = &w->t;
+    const uint32_t stride = t->max_dof;
+    const uint8_t type = t->joint_type[link_local];
+    const v3 zero = v3_make(0, 0, 0);
+    if (type == NKO_FLOATING) {
+        const xform base = xform_load(w->base_pose + (size_t)env * 7u);
+        const v3 lever = v3_sub(point, base.p);
+        const v3 ex = nko_rotate_normalized(base.r, v3_make(1, 0, 0)), ey = nko_rotate_normalized(base.r, v3_make(0, 1, 0)),
+                 ez = nko_rotate_normalized(base.r, v3_make(0, 0, 1));
+        const float ang[3] = {v3_dot(v3_cross(ex, lever), f) + v3_dot(ex, zero), v3_dot(v3_cross(ey, lever), f) + v3_dot(ey, zero),
+                              v3_dot(v3_cross(ez, lever), f) + v3_dot(ez, zero)};
+        const float lin[3] = {v3_dot(ex, f), v3_dot(ey, f), v3_dot(ez, f)};
+        for (uint32_t b = 0u; b < 3u; ++b) {
+            if (dof_index + b < stride) out[dof_index + b] += ang[b];
+            if (dof_index + 3u + b < stride) out[dof_index + 3u + b] += lin[b];
+        }
+        return;
+    }
+    const xform pose = xform_load(w->link_pose + ((size_t)env * t->nl + link_local) * 7u);
+    const v3 axis_world = nko_rotate_normalized(pose.r, v3_make(t->joint_axis[3u * link_local], t->joint_axis[3u * link_local + 1u],
+                                                                 t->joint_axis[3u * link_local + 2u]));
+    float entry;
+    if (type == NKO_PRISMATIC) entry = v3_dot(axis_world, f);
+    else {
+        const v3 lever = v3_sub(point, pose.p);
+        entry = v3_dot(v3_cross(axis_world, lever), f) + v3_dot(axis_world, zero);
+    }
+    if (dof_index < stride) out[dof_index] += entry;
+}
+
+/* assemble_rows.cu:122-169 ComputeContactChainJacobianKernel for one row side */
+static void chain_jacobian_row(const nko_world* w, uint32_t env, uint32_t link_global, v3 point, v3 dir, float* out) {
+    const nko_template* t = &w->t;
+    if (link_global == NKO_INVALID) return;
+    for (uint32_t k = 0u; k < t->max_dof; ++k) out[k] = 0.0f;
+    uint32_t link = link_global - env * t->nl;
+    while (link != NKO_INVALID) {
+        if (nko_joint_dof(t->joint_type[link]) != 0u) accumulate_chain(w, env, link, t->link_dof[link], point, dir, out);
+        link = t->parent_link[link];
+    }
+}
+
+/* ---- AssembleRows (assemble_rows.cu:325-394 ranges/clear, 406-801 emit, 1587-1605 chain J) ---- */
+void nko_env_assemble_rows(nko_world* w, uint32_t env) {
+    const nko_template* t = &w->t;
+    const uint32_t R = t->rows_per_env, S = t->slots, CR = t->contact_rows_per_env;
+    if (R == 0u) return;
+    const float dt = w->cfg.fixed_dt;
+    nko_row* rows = (nko_row*)w->urows + (size_t)env * R;
+    float* lambda = w->lambda + (size_t)env * R;
+    float* pen = w->row_penetration + (size_t)env * R;
+    uint32_t* cj_link = w->row_cj_link + (size_t)env * R, *cj_link_b = w->row_cj_link_b + (size_t)env * R;
+    float* cj_point = w->row_cj_point + (size_t)env * R * 3u, *cj_point_b = w->row_cj_point_b + (size_t)env * R * 3u;
+    uint32_t* extent = w->contact_row_extent;
+    /* InitializePairDrivenRangesKernel :336-360 */
+    w->row_count[env] = 0u;
+    extent[2u * env] = extent[2u * env + 1u];
+    extent[2u * env + 1u] = 1u;
+    uint32_t carry = 0u;
+    for (uint32_t slot = 0u; slot < S; ++slot) {
+        const uint32_t points = w->ucontact_count[(size_t)env * S + slot];
+        w->ucontact_row_range[((size_t)env * S + slot) * 2u] = env * R + carry * 4u;
+        w->ucontact_row_range[((size_t)env * S + slot) * 2u + 1u] = points;
+        carry += points;
+    }
+    /* ClearPairDrivenRowsKernel :366-394 */
+    {
+        const uint32_t bound = contact_row_bound(extent, env, CR);
+        for (uint32_t local = 0u; local < R; ++local)
+            if (local < bound) {
+                lambda[local] = 0.0f; pen[local] = 0.0f; cj_link[local] = NKO_INVALID; cj_link_b[local] = NKO_INVALID;
+                if (rows[local].flags != 0u) rows[local].flags = 0u;
+            }
+    }
+    /* PackQdotFlatMultiKernel :200-214 */
+    for (uint32_t d = 0u; d < t->max_dof; ++d) {
+        float v = 0.0f;
+        if (d < t->nv) {
+            const uint32_t link = t->dof_link[d], c = t->dof_component[d];
+            v = c == NKO_INVALID ? w->qdot[(size_t)env * t->nl + link] : w->link_velocity[((size_t)env * t->nl + link) * 6u + c];
+        }
+        w->qdot_flat[(size_t)env * t->max_dof + d] = v;
+    }
+    /* EmitPairDrivenRowsKernel :453-801, speculative law, condim 3 */
+    uint32_t active_rows = 0u;
+    for (uint32_t slot = 0u; slot < S; ++slot) {
+        const size_t gid = (size_t)env * S + slot;
+        const uint32_t base = w->ucontact_row_range[gid * 2u] - env * R, P = w->ucontact_row_range[gid * 2u + 1u];
+        const uint32_t n_active_in = w->ucontact_count[gid];
+        if (n_active_in > 0u) {
+            const uint32_t e = base + P * 4u + 1u;   /* :464-472 extent past the slot's rows */
+            if (e > extent[2u * env + 1u]) extent[2u * env + 1u] = e;
+        }
+        if (n_active_in == 0u) continue;
+        uint32_t n_active = n_active_in;
+        const uint32_t local_a = w->ucontact_a[gid * 4u], local_b = w->ucontact_b[gid * 4u];
+        shape_row sa, sb; memset(&sa, 0, sizeof(sa)); memset(&sb, 0, sizeof(sb)); sa.body_id = sb.body_id = -1;
+        if (local_a < t->nb) sa = load_shape(t->shape_table, local_a);
+        if (local_b < t->nb) sb = load_shape(t->shape_table, local_b);
+        uint32_t idx_a, idx_b, link_a, link_b;
+        uint32_t kind_a = resolve_side(t, env, local_a, sa.body_id, &idx_a, &link_a);
+        uint32_t kind_b = resolve_side(t, env, local_b, sb.body_id, &idx_b, &link_b);
+        if (kind_a == NKO_INVALID || kind_b == NKO_INVALID) {
+            w->env_status[env] |= NKO_STATUS_INVALID_ENDPOINT;
+            n_active = 0u; kind_a = kind_b = NKO_SIDE_STATIC;
+        }
+        if (kind_a == NKO_SIDE_STATIC) idx_a = NKO_INVALID;
+        if (kind_b == NKO_SIDE_STATIC) idx_b = NKO_INVALID;
+        /* friction: per-shape profile or the default 1.0; equal priority mixes by max (contact_filter.hpp:58-62, 108-111) */
+        const float mu_a1 = sa.profile < t->n_profiles ? t->profile_mu[2u * sa.profile] : 1.0f;
+        const float mu_a2 = sa.profile < t->n_profiles ? t->profile_mu[2u * sa.profile + 1u] : 1.0f;
+        const float mu_b1 = sb.profile < t->n_profiles ? t->profile_mu[2u * sb.profile] : 1.0f;
+        const float mu_b2 = sb.profile < t->n_profiles ? t->profile_mu[2u * sb.profile + 1u] : 1.0f;
+        const float mu1 = mu_a1 > mu_b1 ? mu_a1 : mu_b1, mu2 = mu_a2 > mu_b2 ? mu_a2 : mu_b2;
+        const int position_pass = w->cfg.solver_pos_iters > 0u;
+        for (uint32_t p = 0u; p < P; ++p) {
+            const int live = p < n_active && p < 4u;   /* velocity_only keeps every point (:625-626) */
+            const size_t mp = gid * 4u + p;
+            const uint32_t normal_row = base + p, t1_row = base + P + p, t2_row = base + 2u * P + p;
+            v3 n = v3_make(0, 0, 1), point = v3_make(0, 0, 0), t0 = v3_make(1, 0, 0), t1v = v3_make(0, 1, 0);
+            if (live) {
+                const v3 raw = v3_make(w->ucontact_normal[3u * mp], w->ucontact_normal[3u * mp + 1u], w->ucontact_normal[3u * mp + 2u]);
+                const float len = sqrtf(raw.x * raw.x + raw.y * raw.y + raw.z * raw.z);   /* :193-197 NormalizedHostExpr */
+                n = len < 1e-12f ? v3_make(0, 0, 0) : v3_make(raw.x / len, raw.y / len, raw.z / len);
+                point = v3_make(w->ucontact_point[3u * mp], w->ucontact_point[3u * mp + 1u], w->ucontact_point[3u * mp + 2u]);
+                float a[3], b[3];
+                nko_contact_tangent_basis(&w->ucontact_normal[3u * mp], a, b);
+                t0 = v3_make(a[0], a[1], a[2]); t1v = v3_make(b[0], b[1], b[2]);
+            }
+            {   /* normal row :692-755 */
+                nko_row row; memset(&row, 0, sizeof(row));
+                row.a.kind = row.b.kind = NKO_SIDE_STATIC; row.a.index = row.b.index = NKO_INVALID;
+                lambda[normal_row] = 0.0f; pen[normal_row] = 0.0f; cj_link[normal_row] = NKO_INVALID; cj_link_b[normal_row] = NKO_INVALID;
+                if (live) {
+                    const float d0 = w->ucontact_depth[mp];
+                    const v3 extent_v = v3_make(fabsf(point.x) + fabsf(n.x * d0), fabsf(point.y) + fabsf(n.y * d0), fabsf(point.z) + fabsf(n.z * d0));
+                    /* contact_query.hpp:33-40 ContactProjectionRoundoff(start = end = extent) */
+                    const double gamma = 3.0 * FLT_EPSILON / (1.0 - 3.0 * FLT_EPSILON);
+                    const double roundoff = gamma * (fabs((double)n.x) * (fabs((double)extent_v.x) + fabs((double)extent_v.x)) +
+                                                     fabs((double)n.y) * (fabs((double)extent_v.y) + fabs((double)extent_v.y)) +
+                                                     fabs((double)n.z) * (fabs((double)extent_v.z) + fabs((double)extent_v.z)));
+                    const float clearance = roundoff > 0.0 ? nextafterf((float)roundoff, FLT_MAX) : 0.0f;
+                    const float depth = d0 + clearance;
+                    pen[normal_row] = depth;
+                    row.flags = NKO_ROW_ACTIVE | NKO_ROW_CONTACT_NORMAL | NKO_ROW_BLOCK_NORMAL | NKO_ROW_SPECULATIVE;
+                    row.group_first = env * R + base; row.group_normal_count = P; row.env = env;
+                    row.rhs = (fminf(depth, 0.0f) + (position_pass ? 0.0f : fminf(fmaxf(d0, 0.0f), w->cfg.solver_overlap_recovery_velocity * dt))) / (dt * dt);
+                    row.compliance_alpha = 0.0f;   /* DiscretizeCompliantRow of a zero row: R = 0 (solref_solimp.hpp:40-44) */
+                    row.lower = 0.0f; row.upper = FLT_MAX; row.mu = mu1; row.friction_secondary = mu2;
+                    row.a.kind = kind_a; row.a.index = idx_a; row.a.jlin = n;
+                    row.b.kind = kind_b; row.b.index = idx_b; row.b.jlin = v3_make(-n.x, -n.y, -n.z);
+                    if (kind_a == NKO_SIDE_ARTIC) { cj_link[normal_row] = link_a; cj_point[3u * normal_row] = point.x; cj_point[3u * normal_row + 1u] = point.y; cj_point[3u * normal_row + 2u] = point.z; }
+                    if (kind_b == NKO_SIDE_ARTIC) { cj_link_b[normal_row] = link_b; cj_point_b[3u * normal_row] = point.x; cj_point_b[3u * normal_row + 1u] = point.y; cj_point_b[3u * normal_row + 2u] = point.z; }
+                    ++active_rows;
+                    rows[normal_row] = row;
+                } else rows[normal_row].flags = 0u;
+            }
+            const uint32_t trow[2] = {t1_row, t2_row};
+            const v3 tdir[2] = {t0, t1v};
+            for (uint32_t k = 0u; k < 2u; ++k) {   /* tangent rows :758-797 */
+                const uint32_t rs = trow[k];
+                nko_row row; memset(&row, 0, sizeof(row));
+                row.a.kind = row.b.kind = NKO_SIDE_STATIC; row.a.index = row.b.index = NKO_INVALID;
+                lambda[rs] = 0.0f; pen[rs] = 0.0f; cj_link[rs] = NKO_INVALID; cj_link_b[rs] = NKO_INVALID;
+                if (live) {
+                    const v3 dir = tdir[k];
+                    row.flags = NKO_ROW_ACTIVE | NKO_ROW_BLOCK_TANGENT;
+                    row.group_first = env * R + base; row.group_normal_count = P; row.env = env;
+                    row.lower = -FLT_MAX; row.upper = FLT_MAX; row.mu = mu1; row.friction_secondary = mu2;
+                    row.a.kind = kind_a; row.a.index = idx_a; row.a.jlin = dir;
+                    row.b.kind = kind_b; row.b.index = idx_b; row.b.jlin = v3_make(-dir.x, -dir.y, -dir.z);
+                    if (kind_a == NKO_SIDE_ARTIC) { cj_link[rs] = link_a; cj_point[3u * rs] = point.x; cj_point[3u * rs + 1u] = point.y; cj_point[3u * rs + 2u] = point.z; }
+                    if (kind_b == NKO_SIDE_ARTIC) { cj_link_b[rs] = link_b; cj_point_b[3u * rs] = point.x; cj_point_b[3u * rs + 1u] = point.y; cj_point_b[3u * rs + 2u] = point.z; }
+                    ++active_rows;
+                    rows[rs] = row;
+                } else rows[rs].flags = 0u;
+            }
+        }
+    }
+    w->row_count[env] += active_rows;
+    /* chain Jacobians for both sides, then the shared-owner merge (:1587-1605, 172-186) */
+    for (uint32_t r = 0u; r < R; ++r) {
+        float* ja = w->chain_jacobian + ((size_t)env * R + r) * t->max_dof;
+        float* jb = w->chain_jacobian_b + ((size_t)env * R + r) * t->max_dof;
+        chain_jacobian_row(w, env, cj_link[r], v3_make(cj_point[3u * r], cj_point[3u * r + 1u], cj_point[3u * r + 2u]), rows[r].a.jlin, ja);
+        chain_jacobian_row(w, env, cj_link_b[r], v3_make(cj_point_b[3u * r], cj_point_b[3u * r + 1u], cj_point_b[3u * r + 2u]), rows[r].b.jlin, jb);
+        if ((rows[r].flags & NKO_ROW_ACTIVE) && rows[r].a.kind == NKO_SIDE_ARTIC && rows[r].b.kind == NKO_SIDE_ARTIC &&
+            rows[r].a.index == rows[r].b.index)
+            for (uint32_t i = 0u; i < t->max_dof; ++i) { ja[i] += jb[i]; jb[i] = 0.0f; }
+    }
+}

@@ -1,0 +1,141 @@
+/* Internal declarations of the CPU oracle (test infrastructure; see nuka_oracle.h). */
+#ifndef NKO_INTERNAL_H_
+#define NKO_INTERNAL_H_
+
+#include <float.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "nuka_oracle.h"
+
+#define NKO_INVALID 0xFFFFFFFFu
+#define NKO_MAX_DOF 64u
+
+/* phi/articulation_contract.hpp:8-16 */
+enum { NKO_REVOLUTE = 0, NKO_PRISMATIC = 1, NKO_FIXED = 2, NKO_FLOATING = 3, NKO_SPHERICAL = 4 };
+/* collision/shape_kind.hpp:9-18 */
+enum { NKO_SPHERE = 0, NKO_CAPSULE = 1, NKO_BOX = 2, NKO_PLANE = 3 };
+/* nk/solve/nk_row.hpp:14-19 */
+enum { NKO_SIDE_RIGID = 0, NKO_SIDE_ARTIC = 1, NKO_SIDE_STATIC = 3 };
+/* nk/solve/nk_row.hpp:41-57 */
+enum {
+    NKO_ROW_ACTIVE = 1u << 0, NKO_ROW_BLOCK_NORMAL = 1u << 2, NKO_ROW_BLOCK_TANGENT = 1u << 3,
+    NKO_ROW_CONTACT_NORMAL = 1u << 6, NKO_ROW_VELOCITY_ONLY = 1u << 7, NKO_ROW_SPECULATIVE = 1u << 8,
+    NKO_ROW_MUJOCO = 1u << 11, NKO_ROW_FRICTION = 1u << 1
+};
+/* phi/op_schema.hpp:36-52 */
+enum { NKO_STATUS_PAIR_OVERFLOW = 1u << 0, NKO_STATUS_DOF_OVERFLOW = 1u << 2, NKO_STATUS_INVALID_ENDPOINT = 1u << 6,
+       NKO_STATUS_SOLVER_FAILURE = 1u << 13 };
+
+typedef struct { float x, y, z; } v3;
+typedef struct { float w, x, y, z; } quat;
+typedef struct { v3 p; quat r; } xform;
+
+/* nk/solve/nk_row.hpp:75-101: 26 words. */
+typedef struct {
+    uint32_t kind, index;
+    v3 jlin, jang;
+} nko_row_side;
+typedef struct {
+    uint32_t flags, group_first, group_normal_count, env;
+    float rhs, compliance_alpha, lower, upper, mu, friction_secondary;
+    nko_row_side a, b;
+} nko_row;
+
+/* Cooked template shared by every environment. */
+typedef struct {
+    uint32_t nl, nb, nv, max_dof, slots, rows_per_env, contact_rows_per_env, n_profiles, max_depth;
+    int floating;
+    uint8_t* joint_type;
+    uint32_t* parent_link;
+    float* joint_axis;          /* nl*3 */
+    float* parent_offset;       /* nl*3 */
+    float* link_local_pose;     /* nl*7 */
+    float* link_inertial_frame; /* nl*7 */
+    float* link_inertia;        /* nl*36 */
+    float* joint_damping, *joint_armature, *joint_stiffness, *joint_spring_reference;
+    uint32_t* link_body;        /* nl */
+    uint32_t* link_tree_depth;  /* nl */
+    uint32_t* link_child_range; /* nl*2 */
+    uint32_t* link_children;    /* nl */
+    uint32_t* link_dof;         /* nl: first dof of the link */
+    uint32_t* dof_link;         /* max_dof */
+    uint32_t* dof_component;    /* max_dof, ~0 for scalar joints */
+    float* link_geom_local;     /* nl*7 */
+    uint32_t* link_geom_kind;   /* nl */
+    float* shape_table;         /* nb*13 words */
+    uint32_t* body_to_link, *body_to_articulation, *body_collidable_link, *body_collidable_body;
+    float* body_collidable_local; /* nb*7 */
+    float* body_init_pose;        /* nb*7 */
+    float* profile_mu;            /* n_profiles*2 */
+} nko_template;
+
+struct nko_world {
+    nko_template t;
+    nko_world_desc cfg;
+    uint32_t env_count;
+    int threads;
+    uint64_t step_index;
+    /* env-major state */
+    float *q, *qdot, *qddot, *tau, *base_pose, *link_pose, *link_velocity, *link_acceleration, *link_wrench;
+    float *articulation_bias, *articulation_qdd, *m, *m_factor, *qdot_flat;
+    float *qdot_pseudo, *link_velocity_pseudo;
+    float *body_pose, *body_aabb_lo, *body_aabb_hi;
+    uint32_t *candidate_pairs, *pair_count;
+    uint32_t *ucontact_count, *ucontact_a, *ucontact_b, *ucontact_law, *ucontact_row_range;
+    float *ucontact_point, *ucontact_normal, *ucontact_depth;
+    uint64_t *ucontact_id_pair, *ucontact_id_feature;
+    float *urows, *lambda, *row_penetration, *row_cj_point, *row_cj_point_b, *chain_jacobian, *chain_jacobian_b;
+    uint32_t *row_cj_link, *row_cj_link_b, *row_count, *contact_count, *contact_row_extent;
+    uint32_t *env_status, *vbd_velocity_sweep_count;
+    float *solver_residual;
+    /* solver state kept between steps (block_descent.cu BlockScratch articulation_velocity/free) */
+    float *solver_velocity, *solver_free, *solver_penalty;
+};
+
+/* ---- math (nko_math.c) ------------------------------------------------- */
+static inline v3 v3_make(float x, float y, float z) { v3 r = {x, y, z}; return r; }
+static inline v3 v3_add(v3 a, v3 b) { return v3_make(a.x + b.x, a.y + b.y, a.z + b.z); }
+static inline v3 v3_sub(v3 a, v3 b) { return v3_make(a.x - b.x, a.y - b.y, a.z - b.z); }
+static inline v3 v3_scale(v3 a, float s) { return v3_make(a.x * s, a.y * s, a.z * s); }
+static inline float v3_dot(v3 a, v3 b) { return a.x * b.x + a.y * b.y + a.z * b.z; }
+static inline v3 v3_cross(v3 a, v3 b) {
+    return v3_make(a.y * b.z - a.z * b.y, a.z * b.x - a.x * b.z, a.x * b.y - a.y * b.x);
+}
+static inline float nko_rsqrt(float x) { return 1.0f / sqrtf(x); }
+static inline quat quat_make(float w, float x, float y, float z) { quat q = {w, x, y, z}; return q; }
+static inline xform xform_load(const float* p) {
+    xform t; t.p = v3_make(p[0], p[1], p[2]); t.r = quat_make(p[3], p[4], p[5], p[6]); return t;
+}
+static inline void xform_store(float* p, xform t) {
+    p[0] = t.p.x; p[1] = t.p.y; p[2] = t.p.z; p[3] = t.r.w; p[4] = t.r.x; p[5] = t.r.y; p[6] = t.r.z;
+}
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+quat nko_quat_mul(quat a, quat b);
+quat nko_quat_normalize_rsqrt(quat q, float eps);
+v3 nko_rotate_normalized(quat q, v3 v);
+v3 nko_rotate_inverse(quat q, v3 v);
+v3 nko_rotate_forward(quat q, v3 v);
+v3 nko_prim_rotate(quat q, v3 v);
+xform nko_compose_frame(xform parent, xform local);
+xform nko_compose_hd(xform parent, xform child);
+uint32_t nko_joint_dof(uint8_t type);
+
+void nko_env_fk(const nko_world* w, uint32_t env);
+void nko_env_dynamics(nko_world* w, uint32_t env, uint32_t integrate_velocity);
+void nko_env_integrate_position(nko_world* w, uint32_t env);
+void nko_env_link_velocities(nko_world* w, uint32_t env);
+void nko_env_sync_body_pose(nko_world* w, uint32_t env);
+void nko_env_aabbs(nko_world* w, uint32_t env);
+void nko_env_pairs(nko_world* w, uint32_t env);
+void nko_env_narrowphase(nko_world* w, uint32_t env);
+void nko_env_assemble_rows(nko_world* w, uint32_t env);
+void nko_env_solve(nko_world* w, uint32_t env);
+void nko_joint_transform(const nko_world* w, uint32_t env, uint32_t link, float X[36]);
+void nko_motion_subspace(uint8_t type, v3 axis, float s[6]);
+
+#endif

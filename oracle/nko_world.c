@@ -1,0 +1,286 @@
+/*
+ * CPU oracle (test infrastructure; see nuka_oracle.h): template cook, env-major storage, the named
+ * field table and the per-op drivers that loop environments (OpenMP when built with -fopenmp).
+ */
+#include <stdio.h>
+
+#include "nko_internal.h"
+
+#define ALLOC(type, count) ((type*)calloc((size_t)(count) + 1u, sizeof(type)))
+
+static void copy_or_zero(float* dst, const float* src, size_t n) {
+    if (src != NULL) memcpy(dst, src, n * sizeof(float));
+    else memset(dst, 0, n * sizeof(float));
+}
+
+/* Tree tables (fields.yaml:845-848; articulation_types.cuh:40-50): BFS depth, children CSR in link order;
+ * DOF maps as BuildDofMaps (articulation_mass.cuh:64-90). */
+static int cook_template(nko_template* t, const nko_template_desc* d) {
+    const uint32_t nl = d->link_count, nb = d->body_count;
+    memset(t, 0, sizeof(*t));
+    t->nl = nl; t->nb = nb; t->n_profiles = d->profile_count;
+    t->joint_type = ALLOC(uint8_t, nl); t->parent_link = ALLOC(uint32_t, nl);
+    t->joint_axis = ALLOC(float, nl * 3u); t->parent_offset = ALLOC(float, nl * 3u);
+    t->link_local_pose = ALLOC(float, nl * 7u); t->link_inertial_frame = ALLOC(float, nl * 7u);
+    t->link_inertia = ALLOC(float, nl * 36u);
+    t->joint_damping = ALLOC(float, nl); t->joint_armature = ALLOC(float, nl);
+    t->joint_stiffness = ALLOC(float, nl); t->joint_spring_reference = ALLOC(float, nl);
+    t->link_body = ALLOC(uint32_t, nl); t->link_tree_depth = ALLOC(uint32_t, nl);
+    t->link_child_range = ALLOC(uint32_t, nl * 2u); t->link_children = ALLOC(uint32_t, nl);
+    t->link_dof = ALLOC(uint32_t, nl);
+    t->link_geom_local = ALLOC(float, nl * 7u); t->link_geom_kind = ALLOC(uint32_t, nl);
+    memcpy(t->joint_type, d->joint_type, nl);
+    memcpy(t->parent_link, d->parent_link, nl * sizeof(uint32_t));
+    memcpy(t->joint_axis, d->joint_axis, nl * 3u * sizeof(float));
+    copy_or_zero(t->parent_offset, d->parent_offset, nl * 3u);
+    memcpy(t->link_local_pose, d->link_local_pose, nl * 7u * sizeof(float));
+    memcpy(t->link_inertial_frame, d->link_inertial_frame, nl * 7u * sizeof(float));
+    copy_or_zero(t->joint_damping, d->joint_damping, nl);
+    copy_or_zero(t->joint_armature, d->joint_armature, nl);
+    copy_or_zero(t->joint_stiffness, d->joint_stiffness, nl);
+    copy_or_zero(t->joint_spring_reference, d->joint_spring_reference, nl);
+    uint32_t nv = 0u;
+    for (uint32_t l = 0u; l < nl; ++l) {
+        nko_make_spatial_inertia(d->link_mass[l], d->link_diag_inertia + 3u * l, d->link_inertial_frame + 7u * l, t->link_inertia + 36u * l);
+        t->link_dof[l] = nv;
+        nv += nko_joint_dof(t->joint_type[l]);
+        t->link_body[l] = NKO_INVALID;
+        const float id[7] = {0, 0, 0, 1, 0, 0, 0};
+        memcpy(t->link_geom_local + 7u * l, id, sizeof(id));
+    }
+    if (nv > NKO_MAX_DOF) return -1;
+    t->nv = nv; t->max_dof = nv;
+    t->floating = nl > 0u && t->joint_type[0] == NKO_FLOATING && t->parent_link[0] == NKO_INVALID;
+    t->dof_link = ALLOC(uint32_t, nv); t->dof_component = ALLOC(uint32_t, nv);
+    for (uint32_t l = 0u; l < nl; ++l) {
+        const uint32_t width = nko_joint_dof(t->joint_type[l]);
+        for (uint32_t c = 0u; c < width; ++c) {
+            t->dof_link[t->link_dof[l] + c] = l;
+            t->dof_component[t->link_dof[l] + c] = width == 1u ? NKO_INVALID : c;
+        }
+    }
+    for (uint32_t l = 0u; l < nl; ++l) {
+        uint32_t depth = 0u, walk = l;
+        while (t->parent_link[walk] != NKO_INVALID) { walk = t->parent_link[walk]; ++depth; if (depth > nl) return -1; }
+        t->link_tree_depth[l] = depth;
+        if (depth > t->max_depth) t->max_depth = depth;
+    }
+    uint32_t cursor = 0u;
+    for (uint32_t l = 0u; l < nl; ++l) {
+        t->link_child_range[2u * l] = cursor;
+        for (uint32_t c = 0u; c < nl; ++c) if (t->parent_link[c] == l) t->link_children[cursor++] = c;
+        t->link_child_range[2u * l + 1u] = cursor;
+    }
+    /* collidable rows (scene/cook/cook_to_model.cpp:612-640; prims_types.cuh:27-54) */
+    t->shape_table = ALLOC(float, nb * 13u);
+    t->body_to_link = ALLOC(uint32_t, nb); t->body_to_articulation = ALLOC(uint32_t, nb);
+    t->body_collidable_link = ALLOC(uint32_t, nb); t->body_collidable_body = ALLOC(uint32_t, nb);
+    t->body_collidable_local = ALLOC(float, nb * 7u); t->body_init_pose = ALLOC(float, nb * 7u);
+    t->profile_mu = ALLOC(float, t->n_profiles * 2u);
+    if (t->n_profiles) memcpy(t->profile_mu, d->profile_mu, t->n_profiles * 2u * sizeof(float));
+    for (uint32_t b = 0u; b < nb; ++b) {
+        const uint32_t role = d->body_role[b], link = d->body_link[b];
+        float* row = t->shape_table + 13u * b;
+        row[0] = u2f(d->shape_kind[b]);
+        for (uint32_t k = 0u; k < 4u; ++k) row[1u + k] = d->shape_params[4u * b + k];
+        row[5] = u2f(d->shape_contype[b]); row[6] = u2f(d->shape_conaffinity[b]); row[7] = u2f(0u);
+        row[8] = u2f(role == 0u ? 0xFFFFFFFFu : b); row[9] = u2f(d->shape_group[b]);
+        row[10] = u2f(0u); row[11] = u2f(0u); row[12] = u2f(d->shape_profile[b]);
+        t->body_to_link[b] = NKO_INVALID; t->body_to_articulation[b] = NKO_INVALID;
+        t->body_collidable_link[b] = NKO_INVALID; t->body_collidable_body[b] = NKO_INVALID;
+        const float id[7] = {0, 0, 0, 1, 0, 0, 0};
+        memcpy(t->body_collidable_local + 7u * b, id, sizeof(id));
+        memcpy(t->body_init_pose + 7u * b, id, sizeof(id));
+        if (role == 0u) memcpy(t->body_init_pose + 7u * b, d->body_local + 7u * b, 7u * sizeof(float));
+        else if (role == 1u) {
+            if (link >= nl || t->link_body[link] != NKO_INVALID) return -1;
+            t->link_body[link] = b; t->body_to_link[b] = link; t->body_to_articulation[b] = 0u;
+            memcpy(t->link_geom_local + 7u * link, d->body_local + 7u * b, 7u * sizeof(float));
+            t->link_geom_kind[link] = d->shape_kind[b] != NKO_INVALID ? 1u : 0u;
+        }
+    }
+    for (uint32_t b = 0u; b < nb; ++b) {
+        if (d->body_role[b] != 2u) continue;
+        const uint32_t link = d->body_link[b];
+        if (link >= nl || t->link_body[link] == NKO_INVALID) return -1;
+        t->body_collidable_link[b] = link;
+        t->body_collidable_body[b] = t->link_body[link];
+        memcpy(t->body_collidable_local + 7u * b, d->body_local + 7u * b, 7u * sizeof(float));
+    }
+    uint32_t slots = d->max_contacts_per_env;
+    if (slots == 0u) {   /* admitted pairs of the template */
+        for (uint32_t i = 0u; i < nb; ++i)
+            for (uint32_t j = i + 1u; j < nb; ++j) {
+                const int si = d->body_role[i] == 0u, sj = d->body_role[j] == 0u;
+                if (si && sj) continue;
+                if (d->shape_kind[i] == NKO_INVALID || d->shape_kind[j] == NKO_INVALID) continue;
+                if (((d->shape_contype[i] & d->shape_conaffinity[j]) | (d->shape_contype[j] & d->shape_conaffinity[i])) == 0u) continue;
+                ++slots;
+            }
+    }
+    t->slots = slots;
+    t->contact_rows_per_env = slots * 16u;   /* nk_row.hpp:59-63: 4 points x 4 rows per rigid slot */
+    t->rows_per_env = t->contact_rows_per_env;
+    return 0;
+}
+
+static void free_template(nko_template* t) {
+    free(t->joint_type); free(t->parent_link); free(t->joint_axis); free(t->parent_offset); free(t->link_local_pose);
+    free(t->link_inertial_frame); free(t->link_inertia); free(t->joint_damping); free(t->joint_armature);
+    free(t->joint_stiffness); free(t->joint_spring_reference); free(t->link_body); free(t->link_tree_depth);
+    free(t->link_child_range); free(t->link_children); free(t->link_dof); free(t->dof_link); free(t->dof_component);
+    free(t->link_geom_local); free(t->link_geom_kind); free(t->shape_table); free(t->body_to_link);
+    free(t->body_to_articulation); free(t->body_collidable_link); free(t->body_collidable_body);
+    free(t->body_collidable_local); free(t->body_init_pose); free(t->profile_mu);
+}
+
+nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc* desc) {
+    if (tmpl == NULL || desc == NULL || desc->env_count == 0u) return NULL;
+    nko_world* w = (nko_world*)calloc(1, sizeof(nko_world));
+    if (cook_template(&w->t, tmpl) != 0) { free_template(&w->t); free(w); return NULL; }
+    w->cfg = *desc;
+    /* C-ABI defaults (nuka.h:160-173; pipeline.hpp SolverConfig; op_schema.hpp:598, 663) */
+    if (w->cfg.fixed_dt <= 0.0f) w->cfg.fixed_dt = 1.0f / 240.0f;
+    if (w->cfg.solver_vel_iters == 0u) w->cfg.solver_vel_iters = 10u;
+    if (w->cfg.solver_pos_iters == 0u) w->cfg.solver_pos_iters = 4u;
+    if (w->cfg.solver_pos_iters == 0xFFFFFFFFu) w->cfg.solver_pos_iters = 0u;
+    if (w->cfg.solver_pos_beta <= 0.0f) w->cfg.solver_pos_beta = 0.3f;
+    if (w->cfg.solver_pos_slop <= 0.0f) w->cfg.solver_pos_slop = 1.0e-3f;
+    if (w->cfg.solver_velocity_tolerance <= 0.0f) w->cfg.solver_velocity_tolerance = 1.0e-5f;
+    if (w->cfg.solver_baumgarte_max_velocity <= 0.0f) w->cfg.solver_baumgarte_max_velocity = 3.0e38f;
+    w->env_count = desc->env_count;
+    w->threads = 1;
+    const nko_template* t = &w->t;
+    const size_t E = w->env_count, nl = t->nl, nb = t->nb, md = t->max_dof, S = t->slots, R = t->rows_per_env;
+    w->q = ALLOC(float, E * nl); w->qdot = ALLOC(float, E * nl); w->qddot = ALLOC(float, E * nl); w->tau = ALLOC(float, E * nl);
+    w->base_pose = ALLOC(float, E * 7u); w->link_pose = ALLOC(float, E * nl * 7u);
+    w->link_velocity = ALLOC(float, E * nl * 6u); w->link_acceleration = ALLOC(float, E * nl * 6u); w->link_wrench = ALLOC(float, E * nl * 6u);
+    w->articulation_bias = ALLOC(float, E * md); w->articulation_qdd = ALLOC(float, E * md);
+    w->m = ALLOC(float, E * md * md); w->m_factor = ALLOC(float, E * md * md); w->qdot_flat = ALLOC(float, E * md);
+    w->qdot_pseudo = ALLOC(float, E * nl); w->link_velocity_pseudo = ALLOC(float, E * nl * 6u);
+    w->body_pose = ALLOC(float, E * nb * 7u); w->body_aabb_lo = ALLOC(float, E * nb * 3u); w->body_aabb_hi = ALLOC(float, E * nb * 3u);
+    w->candidate_pairs = ALLOC(uint32_t, E * S * 2u); w->pair_count = ALLOC(uint32_t, E);
+    w->ucontact_count = ALLOC(uint32_t, E * S); w->ucontact_a = ALLOC(uint32_t, E * S * 4u); w->ucontact_b = ALLOC(uint32_t, E * S * 4u);
+    w->ucontact_law = ALLOC(uint32_t, E * S); w->ucontact_row_range = ALLOC(uint32_t, E * S * 2u);
+    w->ucontact_point = ALLOC(float, E * S * 12u); w->ucontact_normal = ALLOC(float, E * S * 12u); w->ucontact_depth = ALLOC(float, E * S * 4u);
+    w->ucontact_id_pair = ALLOC(uint64_t, E * S * 4u); w->ucontact_id_feature = ALLOC(uint64_t, E * S * 4u);
+    w->urows = ALLOC(float, E * R * 26u); w->lambda = ALLOC(float, E * R); w->row_penetration = ALLOC(float, E * R);
+    w->row_cj_point = ALLOC(float, E * R * 3u); w->row_cj_point_b = ALLOC(float, E * R * 3u);
+    w->chain_jacobian = ALLOC(float, E * R * md); w->chain_jacobian_b = ALLOC(float, E * R * md);
+    w->row_cj_link = ALLOC(uint32_t, E * R); w->row_cj_link_b = ALLOC(uint32_t, E * R);
+    w->row_count = ALLOC(uint32_t, E); w->contact_count = ALLOC(uint32_t, E); w->contact_row_extent = ALLOC(uint32_t, E * 2u);
+    w->env_status = ALLOC(uint32_t, E); w->vbd_velocity_sweep_count = ALLOC(uint32_t, E);
+    w->solver_residual = ALLOC(float, E * 4u);
+    w->solver_velocity = ALLOC(float, E * md); w->solver_free = ALLOC(float, E * md); w->solver_penalty = ALLOC(float, E * R);
+    for (size_t i = 0u; i < E * R; ++i) { w->row_cj_link[i] = NKO_INVALID; w->row_cj_link_b[i] = NKO_INVALID; }
+    for (size_t e = 0u; e < E; ++e) {
+        const float id[7] = {0, 0, 0, 1, 0, 0, 0};
+        memcpy(w->base_pose + e * 7u, id, sizeof(id));
+        for (size_t l = 0u; l < nl; ++l) memcpy(w->link_pose + (e * nl + l) * 7u, id, sizeof(id));
+        for (size_t b = 0u; b < nb; ++b) memcpy(w->body_pose + (e * nb + b) * 7u, t->body_init_pose + 7u * b, sizeof(id));
+    }
+    return w;
+}
+
+void nko_world_destroy(nko_world* w) {
+    if (w == NULL) return;
+    free_template(&w->t);
+    free(w->q); free(w->qdot); free(w->qddot); free(w->tau); free(w->base_pose); free(w->link_pose); free(w->link_velocity);
+    free(w->link_acceleration); free(w->link_wrench); free(w->articulation_bias); free(w->articulation_qdd); free(w->m);
+    free(w->m_factor); free(w->qdot_flat); free(w->qdot_pseudo); free(w->link_velocity_pseudo); free(w->body_pose);
+    free(w->body_aabb_lo); free(w->body_aabb_hi); free(w->candidate_pairs); free(w->pair_count); free(w->ucontact_count);
+    free(w->ucontact_a); free(w->ucontact_b); free(w->ucontact_law); free(w->ucontact_row_range); free(w->ucontact_point);
+    free(w->ucontact_normal); free(w->ucontact_depth); free(w->ucontact_id_pair); free(w->ucontact_id_feature); free(w->urows);
+    free(w->lambda); free(w->row_penetration); free(w->row_cj_point); free(w->row_cj_point_b); free(w->chain_jacobian);
+    free(w->chain_jacobian_b); free(w->row_cj_link); free(w->row_cj_link_b); free(w->row_count); free(w->contact_count);
+    free(w->contact_row_extent); free(w->env_status); free(w->vbd_velocity_sweep_count); free(w->solver_residual);
+    free(w->solver_velocity); free(w->solver_free); free(w->solver_penalty);
+    free(w);
+}
+
+#define FIELD_LIST(X) \
+    X(q, float, E * nl) X(qdot, float, E * nl) X(qddot, float, E * nl) X(tau, float, E * nl) \
+    X(base_pose, float, E * 7u) X(link_pose, float, E * nl * 7u) X(link_velocity, float, E * nl * 6u) \
+    X(link_acceleration, float, E * nl * 6u) X(link_wrench, float, E * nl * 6u) \
+    X(articulation_bias, float, E * md) X(articulation_qdd, float, E * md) X(m, float, E * md * md) \
+    X(m_factor, float, E * md * md) X(qdot_flat, float, E * md) X(qdot_pseudo, float, E * nl) \
+    X(link_velocity_pseudo, float, E * nl * 6u) X(body_pose, float, E * nb * 7u) X(body_aabb_lo, float, E * nb * 3u) \
+    X(body_aabb_hi, float, E * nb * 3u) X(candidate_pairs, uint32_t, E * S * 2u) X(pair_count, uint32_t, E) \
+    X(ucontact_count, uint32_t, E * S) X(ucontact_a, uint32_t, E * S * 4u) X(ucontact_b, uint32_t, E * S * 4u) \
+    X(ucontact_law, uint32_t, E * S) X(ucontact_row_range, uint32_t, E * S * 2u) X(ucontact_point, float, E * S * 12u) \
+    X(ucontact_normal, float, E * S * 12u) X(ucontact_depth, float, E * S * 4u) X(ucontact_id_pair, uint64_t, E * S * 4u) \
+    X(ucontact_id_feature, uint64_t, E * S * 4u) X(urows, float, E * R * 26u) X(lambda, float, E * R) \
+    X(row_penetration, float, E * R) X(row_cj_point, float, E * R * 3u) X(row_cj_point_b, float, E * R * 3u) \
+    X(chain_jacobian, float, E * R * md) X(chain_jacobian_b, float, E * R * md) X(row_cj_link, uint32_t, E * R) \
+    X(row_cj_link_b, uint32_t, E * R) X(row_count, uint32_t, E) X(contact_count, uint32_t, E) \
+    X(contact_row_extent, uint32_t, E * 2u) X(env_status, uint32_t, E) X(vbd_velocity_sweep_count, uint32_t, E) \
+    X(solver_residual, float, E * 4u) X(solver_penalty, float, E * R)
+
+#define TEMPLATE_LIST(X) \
+    X(link_inertia, float, nl * 36u) X(link_tree_depth, uint32_t, nl) X(link_child_range, uint32_t, nl * 2u) \
+    X(link_children, uint32_t, nl) X(link_dof, uint32_t, nl) X(dof_link, uint32_t, md) X(dof_component, uint32_t, md) \
+    X(link_body, uint32_t, nl) X(shape_table, float, nb * 13u) X(body_to_link, uint32_t, nb) \
+    X(body_collidable_link, uint32_t, nb) X(body_collidable_body, uint32_t, nb)
+
+int nko_world_field(nko_world* w, const char* name, void** ptr, size_t* bytes) {
+    const nko_template* t = &w->t;
+    const size_t E = w->env_count, nl = t->nl, nb = t->nb, md = t->max_dof, S = t->slots, R = t->rows_per_env;
+#define X(field, type, count) if (strcmp(name, #field) == 0) { *ptr = w->field; *bytes = (size_t)(count) * sizeof(type); return 0; }
+    FIELD_LIST(X)
+#undef X
+#define X(field, type, count) if (strcmp(name, #field) == 0) { *ptr = w->t.field; *bytes = (size_t)(count) * sizeof(type); return 0; }
+    TEMPLATE_LIST(X)
+#undef X
+    (void)E; (void)nl; (void)nb; (void)md; (void)S; (void)R;
+    return -1;
+}
+
+const char* nko_world_field_names(void) {
+#define X(field, type, count) #field ","
+    return FIELD_LIST(X) TEMPLATE_LIST(X) "";
+#undef X
+}
+
+void nko_world_set_threads(nko_world* w, int threads) { w->threads = threads > 0 ? threads : 1; }
+uint32_t nko_world_dof(const nko_world* w) { return w->t.nv; }
+uint32_t nko_world_rows_per_env(const nko_world* w) { return w->t.rows_per_env; }
+
+#define FOR_ENVS(body) \
+    { const int threads_ = w->threads; (void)threads_; \
+      _Pragma("omp parallel for schedule(dynamic, 8) num_threads(threads_)") \
+      for (long env_ = 0; env_ < (long)w->env_count; ++env_) { const uint32_t env = (uint32_t)env_; body; } }
+
+void nko_fk_world_poses(nko_world* w) { FOR_ENVS(nko_env_fk(w, env)) }
+void nko_articulation_dynamics(nko_world* w, uint32_t integrate_velocity) { FOR_ENVS(nko_env_dynamics(w, env, integrate_velocity)) }
+void nko_sync_link_body_pose(nko_world* w) { FOR_ENVS(nko_env_sync_body_pose(w, env)) }
+void nko_build_aabbs(nko_world* w) { FOR_ENVS(nko_env_aabbs(w, env)) }
+void nko_query_pairs(nko_world* w) { FOR_ENVS(nko_env_pairs(w, env)) }
+void nko_narrowphase(nko_world* w) { FOR_ENVS(nko_env_narrowphase(w, env)) }
+void nko_assemble_rows(nko_world* w) { FOR_ENVS(nko_env_assemble_rows(w, env)) }
+/* assemble_rows.cu:1393-1455: with an empty cache (first step, or no persistence) every multiplier starts at 0,
+ * which AssembleRows already wrote; cache persistence across steps is not restated. */
+void nko_contact_warm_start(nko_world* w, uint32_t phase) { (void)w; (void)phase; }
+void nko_block_descent_solve(nko_world* w) { FOR_ENVS(nko_env_solve(w, env)) }
+void nko_integrate_position(nko_world* w) { FOR_ENVS(nko_env_integrate_position(w, env)) }
+void nko_fk_link_velocities(nko_world* w) { FOR_ENVS(nko_env_link_velocities(w, env)) }
+
+/* Op order of one step (src/nk/pipeline/pipeline.cpp:374-986) for an articulated world with ground contact. */
+void nko_world_step(nko_world* w) {
+    nko_fk_world_poses(w);
+    nko_articulation_dynamics(w, 1u);
+    if (w->t.rows_per_env > 0u) {
+        nko_sync_link_body_pose(w);
+        nko_build_aabbs(w);
+        nko_query_pairs(w);
+        nko_narrowphase(w);
+        nko_assemble_rows(w);
+        nko_contact_warm_start(w, 0u);
+        nko_block_descent_solve(w);
+        nko_contact_warm_start(w, 1u);
+    }
+    nko_integrate_position(w);
+    nko_fk_world_poses(w);
+    nko_fk_link_velocities(w);
+    if (w->t.nb > 0u) nko_sync_link_body_pose(w);
+    ++w->step_index;
+}

@@ -1,0 +1,136 @@
+/*
+ * CPU oracle for the batched articulation step: TEST INFRASTRUCTURE ONLY.
+ *
+ * A plain-C, one-environment-at-a-time fp32 restatement of the reference's CUDA kernels for
+ * forward kinematics, RNEA bias + CRBA + LDL^T forward dynamics, the sphere/box x plane contact
+ * pipeline (pairs, manifolds, rows, chain Jacobians) and the UABD tile block-descent solve with its
+ * split-impulse position pass.  Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline
+ * leg may load it, and only as the checker.  Nothing shipped links or calls it.
+ *
+ * Every function in nuka_oracle.c cites the reference file:line it follows.  Compile without
+ * fast-math and with -ffp-contract=off: fused multiply-adds appear only where the reference
+ * writes fmaf/__fmaf_rn itself.
+ *
+ * Parity status per function group (what pins it beyond "it restates the reference"):
+ *   cook / spatial inertia  : pinned (parallel-axis closed form, symmetry; tests/test_oracle_dynamics.py)
+ *   forward kinematics      : pinned (planar chain closed form, composition invariants)
+ *   dynamics (bias, M, LDL) : pinned (pendulum closed forms, RNEA column identity, kinetic energy,
+ *                             independent ABA recursion in tests, double-precision LDL reconstruction)
+ *   pairs / slots / rows    : pinned (brute-force O(B^2) enumeration + sort; integer exact)
+ *   manifolds               : pinned against oracle/_ref (the reference's own analytical_manifold.hpp)
+ *   row math (AL impulses)  : pinned against oracle/_ref (the reference's own augmented_row.hpp) and
+ *                             the known answers in tests/math/test_contact_tangent.cpp
+ *   chain Jacobian          : pinned (J qdot == contact point velocity from link twists)
+ *   UABD fixed point        : pinned (KKT invariants, momentum balance, frictionless closed form,
+ *                             brute-force PGS on <= 3 contacts)
+ *   UABD iterate path       : PARITY UNPINNED - penalty heuristic, first-sweep segment search, FISTA
+ *                             restart timing, secant relaxation and the 8-epsilon waivers decide the
+ *                             multipliers held after a fixed sweep budget; only a running reference
+ *                             could pin them and none can run here.
+ */
+#ifndef NUKA_ORACLE_H_
+#define NUKA_ORACLE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Layout-identical to nuka_template_desc_t / nuka_world_desc_t of include/nuka_hip.h so that one
+ * host-side description drives both the product library and this checker. */
+typedef struct nko_template_desc {
+    uint32_t struct_size;
+    uint32_t link_count;
+    uint32_t body_count;
+    uint32_t profile_count;
+    uint32_t max_contacts_per_env;
+    uint32_t reserved0;
+    const uint8_t* joint_type;
+    const uint32_t* parent_link;
+    const float* joint_axis;
+    const float* parent_offset;
+    const float* link_local_pose;
+    const float* link_inertial_frame;
+    const float* link_mass;
+    const float* link_diag_inertia;
+    const float* joint_damping;
+    const float* joint_armature;
+    const float* joint_stiffness;
+    const float* joint_spring_reference;
+    const uint32_t* body_role;
+    const uint32_t* body_link;
+    const float* body_local;
+    const uint32_t* shape_kind;
+    const float* shape_params;
+    const uint32_t* shape_contype;
+    const uint32_t* shape_conaffinity;
+    const uint32_t* shape_group;
+    const uint32_t* shape_profile;
+    const float* profile_mu;
+} nko_template_desc;
+
+typedef struct nko_world_desc {
+    uint32_t struct_size;
+    uint32_t env_count;
+    float fixed_dt;
+    float gravity[3];
+    uint32_t solver_vel_iters;
+    uint32_t solver_pos_iters;
+    float solver_contact_margin;
+    float solver_pos_beta;
+    float solver_pos_slop;
+    float solver_velocity_tolerance;
+    float solver_baumgarte_max_velocity;
+    float solver_overlap_recovery_velocity;
+} nko_world_desc;
+
+typedef struct nko_world nko_world;
+
+nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc* desc);
+void nko_world_destroy(nko_world* w);
+/* Host pointer and byte size of a named env-major field (or template table); 0 on success. */
+int nko_world_field(nko_world* w, const char* name, void** ptr, size_t* bytes);
+/* Comma-separated list of the field names nko_world_field serves. */
+const char* nko_world_field_names(void);
+void nko_world_set_threads(nko_world* w, int threads);
+uint32_t nko_world_dof(const nko_world* w);
+uint32_t nko_world_rows_per_env(const nko_world* w);
+
+/* One call per reference op (src/nk/pipeline/pipeline.cpp op order). */
+void nko_fk_world_poses(nko_world* w);
+void nko_articulation_dynamics(nko_world* w, uint32_t integrate_velocity);
+void nko_sync_link_body_pose(nko_world* w);
+void nko_build_aabbs(nko_world* w);
+void nko_query_pairs(nko_world* w);
+void nko_narrowphase(nko_world* w);
+void nko_assemble_rows(nko_world* w);
+void nko_contact_warm_start(nko_world* w, uint32_t phase);
+void nko_block_descent_solve(nko_world* w);
+void nko_integrate_position(nko_world* w);
+void nko_fk_link_velocities(nko_world* w);
+/* The whole op list of one step, in the reference's order. */
+void nko_world_step(nko_world* w);
+
+/* Stand-alone pieces exposed for unit pins. */
+void nko_make_spatial_inertia(float mass, const float diag[3], const float inertial_frame[7], float out[36]);
+void nko_factor_mass(const float* mass, float* factor, uint32_t n, uint32_t stride);
+void nko_solve_mass(const float* factor, float* value, uint32_t n, uint32_t stride);
+float nko_mass_coupling(const float* factor, uint32_t n, const float* v, const float* extra);
+void nko_scalar_impulse(float dual, float rho, float residual, float compliance, float lower, float upper,
+                        float out[2]);
+void nko_tangent_impulse(const float dual[3], float rho, const float residual[3], float normal_impulse,
+                         float mu_first, float mu_second, float impulse[3], float curvature[6]);
+void nko_relax_contact_impulse(const float dual[3], const float next[3], float last_step[3], float* last_weight,
+                               float last_point[3], float out[3]);
+uint32_t nko_sphere_plane(const float sphere_pose[7], float radius, const float plane_pose[7], float query,
+                          float point[3], float normal[3], float* penetration);
+uint32_t nko_box_plane(const float box_pose[7], const float half[3], const float plane_pose[7], float query,
+                       float points[12], float normal[3], float penetration[4], uint32_t feature[4]);
+void nko_contact_tangent_basis(const float normal[3], float t1[3], float t2[3]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,111 @@
+"""ctypes driver of the CPU oracle (test infrastructure: tests/, smoke() and bench.py's cpu_baseline leg only)."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "_build", "libnuka_oracle.so")
+REF_PATH = os.path.join(HERE, "_ref", "libnuka_ref.so")
+
+U32_FIELDS = {"candidate_pairs", "pair_count", "ucontact_count", "ucontact_a", "ucontact_b", "ucontact_law",
+              "ucontact_row_range", "row_cj_link", "row_cj_link_b", "row_count", "contact_count",
+              "contact_row_extent", "env_status", "vbd_velocity_sweep_count", "link_tree_depth",
+              "link_child_range", "link_children", "link_dof", "dof_link", "dof_component", "link_body",
+              "body_to_link", "body_collidable_link", "body_collidable_body"}
+U64_FIELDS = {"ucontact_id_pair", "ucontact_id_feature"}
+
+
+def build(force=False):
+    """Compiles the oracle (and, where the reference tree is mounted, the reference-header shim)."""
+    if force or not os.path.exists(LIB_PATH):
+        subprocess.run(["make", "-C", HERE, "_build/libnuka_oracle.so"] + (["-B"] if force else []), check=True,
+                       stdout=subprocess.DEVNULL)
+    if os.path.isdir("/root/reference/src") and (force or not os.path.exists(REF_PATH)):
+        subprocess.run(["make", "-C", HERE, "ref"], check=True, stdout=subprocess.DEVNULL)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        L = C.CDLL(LIB_PATH)
+        L.nko_world_create.restype = C.c_void_p
+        L.nko_world_create.argtypes = [C.c_void_p, C.c_void_p]
+        L.nko_world_destroy.argtypes = [C.c_void_p]
+        L.nko_world_field.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t)]
+        L.nko_world_field_names.restype = C.c_char_p
+        L.nko_world_set_threads.argtypes = [C.c_void_p, C.c_int]
+        L.nko_world_dof.argtypes = [C.c_void_p]
+        L.nko_world_dof.restype = C.c_uint32
+        L.nko_world_rows_per_env.argtypes = [C.c_void_p]
+        L.nko_world_rows_per_env.restype = C.c_uint32
+        for name in ("fk_world_poses", "sync_link_body_pose", "build_aabbs", "query_pairs", "narrowphase",
+                     "assemble_rows", "block_descent_solve", "integrate_position", "fk_link_velocities"):
+            getattr(L, "nko_" + name).argtypes = [C.c_void_p]
+        L.nko_articulation_dynamics.argtypes = [C.c_void_p, C.c_uint32]
+        L.nko_contact_warm_start.argtypes = [C.c_void_p, C.c_uint32]
+        L.nko_world_step.argtypes = [C.c_void_p]
+        L.nko_mass_coupling.restype = C.c_float
+        _lib = L
+    return _lib
+
+
+class OracleWorld:
+    def __init__(self, template, desc, threads=1):
+        L = lib()
+        tdesc, self._keep = template.to_c()
+        self._h = L.nko_world_create(C.byref(tdesc), C.byref(desc))
+        if not self._h:
+            raise RuntimeError("oracle: template rejected")
+        L.nko_world_set_threads(self._h, threads)
+        self.env_count = desc.env_count
+        self.link_count = template.link_count
+        self.dof = L.nko_world_dof(self._h)
+        self.rows_per_env = L.nko_world_rows_per_env(self._h)
+
+    def close(self):
+        if self._h:
+            lib().nko_world_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    def field(self, name):
+        ptr, nbytes = C.c_void_p(), C.c_size_t()
+        if lib().nko_world_field(self._h, name.encode(), C.byref(ptr), C.byref(nbytes)) != 0:
+            raise KeyError(name)
+        dtype = np.uint32 if name in U32_FIELDS else np.uint64 if name in U64_FIELDS else np.float32
+        count = nbytes.value // np.dtype(dtype).itemsize
+        if count == 0:
+            return np.zeros(0, dtype)
+        return np.ctypeslib.as_array(C.cast(ptr, C.POINTER(np.ctypeslib.as_ctypes_type(dtype))), shape=(count,))
+
+    def download(self, name):
+        return self.field(name).copy()
+
+    def upload(self, name, values):
+        f = self.field(name)
+        f[:] = np.asarray(values, dtype=f.dtype).reshape(-1)
+
+    def set_state(self, state):
+        E, nl = self.env_count, self.link_count
+        self.upload("q", state["q"])
+        self.upload("qdot", state["qdot"])
+        self.upload("tau", state["tau"])
+        self.upload("base_pose", state["base_pose"])
+        lv = self.field("link_velocity").reshape(E, nl, 6)
+        lv[:] = 0.0
+        lv[:, 0, :] = state["root_twist"]
+
+    def op(self, name, *args):
+        getattr(lib(), "nko_" + name)(self._h, *args)
+
+    def step(self, n=1):
+        for _ in range(n):
+            lib().nko_world_step(self._h)

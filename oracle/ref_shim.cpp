@@ -1,0 +1,137 @@
+// Test infrastructure: extern "C" entry points around the reference's own host-compilable headers, compiled
+// from /root/reference/src where they lie (never copied).  Used only to pin the CPU oracle's restatement of
+// the row math (nk/solve/augmented_row.hpp), the analytic manifolds (collision/analytical_manifold.hpp),
+// the compliant-row discretisation (constraint/solref_solimp.hpp), contact identity and filters.
+#include <cstdint>
+#include <cstring>
+
+#include "collision/analytical_manifold.hpp"
+#include "collision/contact_query.hpp"
+#include "collision/shape_kind.hpp"
+#include "constraint/solref_solimp.hpp"
+#include "nk/contact/contact_identity.hpp"
+#include "nk/solve/augmented_row.hpp"
+#include "scene/contact_filter.hpp"
+
+using namespace nuka;
+
+static math::Transform MakeTransform(const float* p) {
+    math::Transform t;
+    t.position = {p[0], p[1], p[2]};
+    t.rotation.w = p[3]; t.rotation.x = p[4]; t.rotation.y = p[5]; t.rotation.z = p[6];
+    return t;
+}
+
+extern "C" {
+
+void ref_scalar_impulse(float dual, float rho, float residual, float compliance, float lower, float upper, float* out) {
+    const auto term = nk::augmented::EvaluateScalarImpulse(dual, rho, residual, compliance, lower, upper,
+        nk::augmented::ComputeFloatScalarResponse(rho, compliance));
+    out[0] = term.impulse; out[1] = term.curvature;
+}
+
+void ref_tangent_impulse(const float* dual, float rho, const float* residual, float normal_impulse, float mu_first,
+                         float mu_second, float* impulse, float* curvature) {
+    const auto term = nk::augmented::EvaluateTangentImpulse({dual[0], dual[1], dual[2]}, rho,
+        {residual[0], residual[1], residual[2]}, normal_impulse, mu_first, mu_second);
+    impulse[0] = term.impulse.x; impulse[1] = term.impulse.y; impulse[2] = term.impulse.z;
+    curvature[0] = term.curvature.xx; curvature[1] = term.curvature.yy; curvature[2] = term.curvature.zz;
+    curvature[3] = term.curvature.xy; curvature[4] = term.curvature.xz; curvature[5] = term.curvature.yz;
+}
+
+void ref_relax_contact_impulse(const float* dual, const float* next, float* last_step, float* last_weight,
+                               float* last_point, float* out) {
+    nk::augmented::ContactRelaxation last{{last_step[0], last_step[1], last_step[2]}, *last_weight,
+                                          {last_point[0], last_point[1], last_point[2]}};
+    const auto r = nk::augmented::RelaxContactImpulse({dual[0], dual[1], dual[2]}, {next[0], next[1], next[2]}, &last);
+    last_step[0] = last.step.x; last_step[1] = last.step.y; last_step[2] = last.step.z; *last_weight = last.weight;
+    last_point[0] = last.point.x; last_point[1] = last.point.y; last_point[2] = last.point.z;
+    out[0] = r.x; out[1] = r.y; out[2] = r.z;
+}
+
+float ref_cone_argument(float dual, float rho, float mu, float residual) {
+    return nk::augmented::ConeArgument(dual, rho, mu, residual);
+}
+
+double ref_momentum_restart(const float* point, const float* next, const float* base, const float* scale) {
+    return nk::augmented::MultiplierMomentumRestart({point[0], point[1], point[2]}, {next[0], next[1], next[2]},
+                                                    {base[0], base[1], base[2]}, {scale[0], scale[1], scale[2]});
+}
+
+double ref_tangent_potential(const float* dual, float rho, const float* residual, float normal_impulse, float mu_first,
+                             float mu_second) {
+    return nk::augmented::EvaluateTangent({dual[0], dual[1], dual[2]}, rho, {residual[0], residual[1], residual[2]},
+                                          normal_impulse, mu_first, mu_second).potential;
+}
+
+float ref_tangent_potential_change(const float* dual, float rho, const float* residual, const float* drop,
+                                   float normal_impulse, float mu_first, float mu_second) {
+    return nk::augmented::TangentPotentialChange({dual[0], dual[1], dual[2]}, rho, {residual[0], residual[1], residual[2]},
+                                                 {drop[0], drop[1], drop[2]}, normal_impulse, mu_first, mu_second);
+}
+
+static collision::amf::PrimParams Prim(const float* pose, const float* params) {
+    collision::amf::PrimParams p;
+    p.frame = collision::amf::BuildPrimFrameDevice(MakeTransform(pose));
+    p.radius = params[0]; p.half_height = params[1]; p.half_extents = {params[0], params[1], params[2]};
+    return p;
+}
+
+uint32_t ref_primitive_pair(uint32_t kind_a, const float* pose_a, const float* params_a, uint32_t kind_b,
+                            const float* pose_b, const float* params_b, float query, float* points, float* normals,
+                            float* penetration, uint64_t* keys) {
+    constraint::ContactManifold m;
+    collision::amf::PrimitivePair(kind_a, Prim(pose_a, params_a), kind_b, Prim(pose_b, params_b), query, &m);
+    for (uint32_t i = 0; i < m.point_count; ++i) {
+        points[3 * i] = m.points[i].position.x; points[3 * i + 1] = m.points[i].position.y; points[3 * i + 2] = m.points[i].position.z;
+        normals[3 * i] = m.points[i].normal.x; normals[3 * i + 1] = m.points[i].normal.y; normals[3 * i + 2] = m.points[i].normal.z;
+        penetration[i] = m.points[i].penetration; keys[i] = m.points[i].stable_key;
+    }
+    return m.point_count;
+}
+
+void ref_compose_transform(const float* parent, const float* child, float* out) {
+    const auto t = collision::amf::ComposeTransformHD(MakeTransform(parent), MakeTransform(child));
+    out[0] = t.position.x; out[1] = t.position.y; out[2] = t.position.z;
+    out[3] = t.rotation.w; out[4] = t.rotation.x; out[5] = t.rotation.y; out[6] = t.rotation.z;
+}
+
+void ref_make_contact_id(uint32_t a, uint32_t b, const float* local_a, const float* local_b, const float* normal,
+                         uint32_t feature, uint32_t manifold_slot, uint64_t* out) {
+    nk::CanonicalContactDescriptor d;
+    d.a.handle = a; d.b.handle = b;
+    d.local_point_a = {local_a[0], local_a[1], local_a[2]}; d.local_point_b = {local_b[0], local_b[1], local_b[2]};
+    d.normal = {normal[0], normal[1], normal[2]};
+    d.feature_a = d.feature_b = feature; d.manifold_slot = manifold_slot;
+    const auto id = nk::MakeContactId(d);
+    out[0] = id.pair; out[1] = id.feature;
+}
+
+void ref_discretize_zero_row(float dt, float* out) {
+    const auto d = constraint::DiscretizeCompliantRow(constraint::CompliantContactRow{}, dt);
+    out[0] = d.R; out[1] = d.bias; out[2] = d.reference_gain;
+}
+
+void ref_merge_friction(float mu_a, float mu_b, float* out) {
+    scene::ContactParamsIn a, b;
+    a.mu1 = a.mu2 = mu_a; b.mu1 = b.mu2 = mu_b;
+    const auto m = scene::MergeContactParams(a, b);
+    out[0] = m.mu1; out[1] = m.mu2; out[2] = float(m.condim); out[3] = m.margin;
+}
+
+int ref_shape_filter_admits(uint32_t ta, uint32_t aa, uint32_t ga, uint32_t tb, uint32_t ab, uint32_t gb) {
+    return collision::ShapeFilterAdmits(ta, aa, ga, tb, ab, gb) ? 1 : 0;
+}
+
+double ref_contact_projection_roundoff(const float* start, const float* end, const float* axis) {
+    return collision::ContactProjectionRoundoff({start[0], start[1], start[2]}, {end[0], end[1], end[2]},
+                                                {axis[0], axis[1], axis[2]});
+}
+
+float ref_contact_query_reach(float thickness, float margin) { return collision::ContactQueryReach(thickness, margin); }
+float ref_contact_motion_radius(float base, float dt, float sa, float sb, float relaxation) {
+    return collision::ContactMotionRadius(base, dt, sa, sb, relaxation);
+}
+float ref_rigid_contact_query_margin() { return collision::kRigidContactQueryMargin; }
+
+}  // extern "C"
