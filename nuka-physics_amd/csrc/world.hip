@@ -434,14 +434,15 @@ const char* nuka_last_error_message(void) {
 nuka_result_t nuka_device_create(const nuka_device_desc_t* desc, nuka_device_handle* out) {
     if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
     *out = nullptr;
+    if (desc == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "desc is null");
     int count = 0;
     if (hipGetDeviceCount(&count) != hipSuccess || count == 0) {
         (void)hipGetLastError();
-        return Error(NUKA_RESULT_NOT_SUPPORTED, "no HIP device: the library has no CPU fallback");
+        return Error(NUKA_RESULT_DEVICE_ERROR, "no HIP device: the library has no CPU fallback");
     }
-    const uint32_t index = desc != nullptr ? desc->gpu_index : 0u;
-    if (index >= uint32_t(count)) return Error(NUKA_RESULT_INVALID_ARG, "gpu_index out of range");
-    void* backend = CreateBackend(int(index), desc != nullptr ? desc->stream : nullptr);
+    const uint32_t index = desc->gpu_index;
+    if (index >= uint32_t(count)) return Error(NUKA_RESULT_DEVICE_ERROR, "no HIP device with this gpu_index");
+    void* backend = CreateBackend(int(index), desc->stream);
     if (backend == nullptr) return Error(NUKA_RESULT_DEVICE_ERROR, "backend creation failed");
     auto* record = new DeviceRecord{backend, int(index)};
     *out = reinterpret_cast<nuka_device_handle>(record);

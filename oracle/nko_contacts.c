@@ -228,6 +228,33 @@ uint32_t nko_box_plane(const float box_pose[7], const float half[3], const float
     return m.count;
 }
 
+uint32_t nko_primitive_pair_frames(uint32_t kind_a, const float frame_a[12], const float params_a[4], uint32_t kind_b,
+                                   const float frame_b[12], const float params_b[4], float query, float points[12],
+                                   float normals[12], float penetration[4], uint64_t keys[4]) {
+    prim pr[2];
+    const float* f[2] = {frame_a, frame_b};
+    const float* s[2] = {params_a, params_b};
+    for (int k = 0; k < 2; ++k) {
+        pr[k].cx = v3_make(f[k][0], f[k][1], f[k][2]); pr[k].cy = v3_make(f[k][3], f[k][4], f[k][5]);
+        pr[k].cz = v3_make(f[k][6], f[k][7], f[k][8]); pr[k].t = v3_make(f[k][9], f[k][10], f[k][11]);
+        pr[k].radius = s[k][0]; pr[k].half = v3_make(s[k][0], s[k][1], s[k][2]);
+    }
+    manifold m; primitive_pair(kind_a, &pr[0], kind_b, &pr[1], query, &m);
+    for (uint32_t i = 0u; i < m.count; ++i) {
+        points[3u * i] = m.position[i].x; points[3u * i + 1u] = m.position[i].y; points[3u * i + 2u] = m.position[i].z;
+        normals[3u * i] = m.normal[i].x; normals[3u * i + 1u] = m.normal[i].y; normals[3u * i + 2u] = m.normal[i].z;
+        penetration[i] = m.penetration[i]; keys[i] = m.key[i];
+    }
+    return m.count;
+}
+
+void nko_prim_frame(const float pose[7], float frame[12]) {
+    shape_row s; memset(&s, 0, sizeof(s));
+    const prim p = make_prim(s, xform_load(pose));
+    const v3 c[4] = {p.cx, p.cy, p.cz, p.t};
+    for (int i = 0; i < 4; ++i) { frame[3 * i] = c[i].x; frame[3 * i + 1] = c[i].y; frame[3 * i + 2] = c[i].z; }
+}
+
 /* ---- contact identity (nk/contact/contact_identity.hpp:98-157) ----------- */
 static int32_t quantize_coord(float value) {
     const float scaled = value * 4096.0f;
@@ -241,6 +268,15 @@ static uint64_t feature_token(uint32_t feature, v3 p) {
     h = hash_word(h, (uint32_t)quantize_coord(p.x)); h = hash_word(h, (uint32_t)quantize_coord(p.y));
     h = hash_word(h, (uint32_t)quantize_coord(p.z));
     return h & 0x7fffffffffffffffull;
+}
+/* MakeContactId for two CollidableRefs of type 0 with a < b (:108-157): pair word, then the feature hash over
+ * both sides' tokens, the manifold slot and the two (zero) element words. */
+static void contact_id(uint32_t a, uint32_t b, v3 la, v3 lb, uint32_t feature, uint32_t manifold_slot, uint64_t out[2]) {
+    uint64_t h = 1469598103934665603ull;
+    h = hash_word(h, feature_token(feature, la)); h = hash_word(h, feature_token(feature, lb));
+    h = hash_word(h, manifold_slot); h = hash_word(h, 0u); h = hash_word(h, 0u);
+    out[0] = ((uint64_t)(a & 0x0fffffffu) << 32u) | (uint64_t)(b & 0x0fffffffu);
+    out[1] = h;
 }
 static v3 inverse_transform_point(xform xf, v3 wp) {   /* prims_types.cuh:98-105 */
     const v3 v = v3_sub(wp, xf.p);
@@ -284,15 +320,39 @@ void nko_env_narrowphase(nko_world* w, uint32_t env) {
             const uint32_t feature = m.key[i] == 0u ? 0xffffffffu : (uint32_t)m.key[i];
             const v3 la = inverse_transform_point(xform_load(w->body_pose + (bbase + a) * 7u), m.position[i]);
             const v3 lb = inverse_transform_point(xform_load(w->body_pose + (bbase + b) * 7u), m.position[i]);
-            uint64_t h = 1469598103934665603ull;
-            h = hash_word(h, feature_token(feature, la)); h = hash_word(h, feature_token(feature, lb));
-            h = hash_word(h, i); h = hash_word(h, 0u); h = hash_word(h, 0u);
-            w->ucontact_id_pair[at] = ((uint64_t)(a & 0x0fffffffu) << 32u) | (uint64_t)(b & 0x0fffffffu);
-            w->ucontact_id_feature[at] = h;
+            uint64_t id[2];
+            contact_id(a, b, la, lb, feature, i, id);
+            w->ucontact_id_pair[at] = id[0];
+            w->ucontact_id_feature[at] = id[1];
         }
         contacts += m.count;
     }
     w->contact_count[env] = contacts;
+}
+
+/* contact_query.hpp:33-40 ContactProjectionRoundoff */
+static double projection_roundoff(v3 start, v3 end, v3 axis) {
+    const double gamma = 3.0 * FLT_EPSILON / (1.0 - 3.0 * FLT_EPSILON);
+    return gamma * (fabs((double)axis.x) * (fabs((double)start.x) + fabs((double)end.x)) +
+                    fabs((double)axis.y) * (fabs((double)start.y) + fabs((double)end.y)) +
+                    fabs((double)axis.z) * (fabs((double)start.z) + fabs((double)end.z)));
+}
+
+/* ---- exported restatements for the unit pins ---- */
+double nko_contact_projection_roundoff(const float start[3], const float end[3], const float axis[3]) {
+    return projection_roundoff(v3_make(start[0], start[1], start[2]), v3_make(end[0], end[1], end[2]), v3_make(axis[0], axis[1], axis[2]));
+}
+float nko_contact_query_reach(float thickness, float margin) { return contact_query_reach(thickness, margin); }
+float nko_contact_motion_radius(float base, float dt, float sa, float sb, float relax) { return contact_motion_radius(base, dt, sa, sb, relax); }
+int nko_shape_filter_admits(uint32_t ta, uint32_t aa, uint32_t ga_, uint32_t tb, uint32_t ab, uint32_t gb_) {
+    return shape_filter_admits(ta, aa, ga_, tb, ab, gb_);
+}
+void nko_compose_transform(const float parent[7], const float child[7], float out[7]) {
+    xform_store(out, nko_compose_hd(xform_load(parent), xform_load(child)));
+}
+void nko_make_contact_id(uint32_t a, uint32_t b, const float local_a[3], const float local_b[3], uint32_t feature,
+                         uint32_t manifold_slot, uint64_t out[2]) {
+    contact_id(a, b, v3_make(local_a[0], local_a[1], local_a[2]), v3_make(local_b[0], local_b[1], local_b[2]), feature, manifold_slot, out);
 }
 
 /* math/cuda_vec_ops.cuh:150-183 NormalizeOrUp + ContactTangentBasis */
@@ -479,11 +539,7 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
                 if (live) {
                     const float d0 = w->ucontact_depth[mp];
                     const v3 extent_v = v3_make(fabsf(point.x) + fabsf(n.x * d0), fabsf(point.y) + fabsf(n.y * d0), fabsf(point.z) + fabsf(n.z * d0));
-                    /* contact_query.hpp:33-40 ContactProjectionRoundoff(start = end = extent) */
-                    const double gamma = 3.0 * FLT_EPSILON / (1.0 - 3.0 * FLT_EPSILON);
-                    const double roundoff = gamma * (fabs((double)n.x) * (fabs((double)extent_v.x) + fabs((double)extent_v.x)) +
-                                                     fabs((double)n.y) * (fabs((double)extent_v.y) + fabs((double)extent_v.y)) +
-                                                     fabs((double)n.z) * (fabs((double)extent_v.z) + fabs((double)extent_v.z)));
+                    const double roundoff = projection_roundoff(extent_v, extent_v, n);
                     const float clearance = roundoff > 0.0 ? nextafterf((float)roundoff, FLT_MAX) : 0.0f;
                     const float depth = d0 + clearance;
                     pen[normal_row] = depth;

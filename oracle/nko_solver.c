@@ -144,6 +144,11 @@ static double momentum_restart(v3 point, v3 next, v3 base, v3 scale) {
 
 /* ---- block_descent.cu helpers --------------------------------------------- */
 
+float nko_cone_argument(float dual, float rho, float mu, float residual) { return cone_argument(dual, rho, mu, residual); }
+double nko_momentum_restart(const float point[3], const float next[3], const float base[3], const float scale[3]) {
+    return momentum_restart(v3_make(point[0], point[1], point[2]), v3_make(next[0], next[1], next[2]),
+                            v3_make(base[0], base[1], base[2]), v3_make(scale[0], scale[1], scale[2]));
+}
 static uint32_t residual_bits(float value) { return f2u(value <= FLT_MAX ? fabsf(value) : FLT_MAX); }   /* :735 */
 static float along_axis(float impulse, float velocity) { return impulse > 0.0f ? velocity : impulse < 0.0f ? -velocity : 0.0f; }   /* :773-775 */
 

@@ -124,6 +124,21 @@ void nko_tangent_impulse(const float dual[3], float rho, const float residual[3]
                          float mu_first, float mu_second, float impulse[3], float curvature[6]);
 void nko_relax_contact_impulse(const float dual[3], const float next[3], float last_step[3], float* last_weight,
                                float last_point[3], float out[3]);
+float nko_cone_argument(float dual, float rho, float mu, float residual);
+double nko_momentum_restart(const float point[3], const float next[3], const float base[3], const float scale[3]);
+double nko_contact_projection_roundoff(const float start[3], const float end[3], const float axis[3]);
+float nko_contact_query_reach(float thickness, float margin);
+float nko_contact_motion_radius(float base, float dt, float sa, float sb, float relax);
+int nko_shape_filter_admits(uint32_t ta, uint32_t aa, uint32_t ga, uint32_t tb, uint32_t ab, uint32_t gb);
+void nko_compose_transform(const float parent[7], const float child[7], float out[7]);
+void nko_make_contact_id(uint32_t a, uint32_t b, const float local_a[3], const float local_b[3], uint32_t feature,
+                         uint32_t manifold_slot, uint64_t out[2]);
+/* analytical_manifold.hpp:931-966 PrimitivePair on two baked frames (cx, cy, cz, t) */
+uint32_t nko_primitive_pair_frames(uint32_t kind_a, const float frame_a[12], const float params_a[4], uint32_t kind_b,
+                                   const float frame_b[12], const float params_b[4], float query, float points[12],
+                                   float normals[12], float penetration[4], uint64_t keys[4]);
+/* cx, cy, cz, t of the baked prim frame (narrowphase_prims.cu:34-46 MakePrim) */
+void nko_prim_frame(const float pose[7], float frame[12]);
 uint32_t nko_sphere_plane(const float sphere_pose[7], float radius, const float plane_pose[7], float query,
                           float point[3], float normal[3], float* penetration);
 uint32_t nko_box_plane(const float box_pose[7], const float half[3], const float plane_pose[7], float query,

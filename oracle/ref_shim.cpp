@@ -77,6 +77,30 @@ static collision::amf::PrimParams Prim(const float* pose, const float* params) {
     return p;
 }
 
+// Same, with the two prim frames given as cx, cy, cz, t (12 floats): the pipeline bakes its frames in a device-only
+// helper, so the manifold math is compared on frames the caller supplies.
+static collision::amf::PrimParams PrimFromFrame(const float* f, const float* params) {
+    collision::amf::PrimParams p;
+    p.frame.cx = {f[0], f[1], f[2]}; p.frame.cy = {f[3], f[4], f[5]}; p.frame.cz = {f[6], f[7], f[8]};
+    p.frame.t = {f[9], f[10], f[11]};
+    p.radius = params[0]; p.half_height = params[1]; p.half_extents = {params[0], params[1], params[2]};
+    return p;
+}
+
+uint32_t ref_primitive_pair_frames(uint32_t kind_a, const float* frame_a, const float* params_a, uint32_t kind_b,
+                                   const float* frame_b, const float* params_b, float query, float* points,
+                                   float* normals, float* penetration, uint64_t* keys) {
+    constraint::ContactManifold m;
+    collision::amf::PrimitivePair(kind_a, PrimFromFrame(frame_a, params_a), kind_b, PrimFromFrame(frame_b, params_b),
+                                  query, &m);
+    for (uint32_t i = 0; i < m.point_count; ++i) {
+        points[3 * i] = m.points[i].position.x; points[3 * i + 1] = m.points[i].position.y; points[3 * i + 2] = m.points[i].position.z;
+        normals[3 * i] = m.points[i].normal.x; normals[3 * i + 1] = m.points[i].normal.y; normals[3 * i + 2] = m.points[i].normal.z;
+        penetration[i] = m.points[i].penetration; keys[i] = m.points[i].stable_key;
+    }
+    return m.point_count;
+}
+
 uint32_t ref_primitive_pair(uint32_t kind_a, const float* pose_a, const float* params_a, uint32_t kind_b,
                             const float* pose_b, const float* params_b, float query, float* points, float* normals,
                             float* penetration, uint64_t* keys) {

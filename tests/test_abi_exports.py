@@ -1,0 +1,62 @@
+"""The C-ABI library loads and exports every symbol include/*.h declares (no compute calls: runs without a GPU)."""
+import ctypes as C
+import os
+import re
+
+from conftest import ROOT, nk
+
+
+def declared_functions():
+    names = []
+    for header in ("nuka_hip.h", "nuka_phi.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        text = re.sub(r"typedef struct\s+\w+\s*\{.*?\}\s*\w+;", "", text, flags=re.S)
+        names += re.findall(r"\b(nuka_\w+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = C.CDLL(nk.LIB_PATH)
+    names = declared_functions()
+    assert len(names) >= 28
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, f"declared but not exported: {missing}"
+    assert set(nk.EXPORTS) <= set(names)
+
+
+def test_struct_layouts_match_the_header():
+    # 6 u32 + 22 pointers; 14 4-byte words
+    assert C.sizeof(nk.abi.TemplateDescC) == 6 * 4 + 22 * 8
+    assert C.sizeof(nk.abi.WorldDescC) == 14 * 4
+
+
+def test_op_catalog_names_round_trip():
+    lib = nk.lib()
+    count = lib.nuka_hip_op_count()
+    names = [lib.nuka_hip_op_name(i).decode() for i in range(count)]
+    for expected in ("FkWorldPoses", "ArticulationDynamics", "SyncLinkBodyPose", "BuildAabbs", "LbvhQueryPairs",
+                     "NarrowphasePrimitives", "AssembleRows", "ContactWarmStart", "BlockDescentSolve", "IntegratePosition",
+                     "FkLinkVelocities"):
+        assert expected in names
+        assert lib.nuka_hip_op_from_name(expected.encode()) == names.index(expected)
+    assert lib.nuka_hip_op_from_name(b"NoSuchOp") == -1
+
+
+def test_field_names_cover_the_seam_fields():
+    lib = nk.lib()
+    fields = lib.nuka_field_names().decode().strip(",").split(",")
+    for name in ("q", "qdot", "qddot", "tau", "base_pose", "link_pose", "link_velocity", "link_acceleration", "m",
+                 "m_factor", "articulation_bias", "candidate_pairs", "pair_count", "ucontact_count", "ucontact_point",
+                 "ucontact_normal", "ucontact_depth", "ucontact_row_range", "urows", "lambda", "chain_jacobian",
+                 "chain_jacobian_b", "env_status", "solver_residual", "vbd_velocity_sweep_count", "link_inertia",
+                 "shape_table"):
+        assert name in fields
+        assert lib.nuka_field_from_name(name.encode()) == fields.index(name)
+    assert lib.nuka_field_from_name(b"no_such_field") == 0xFFFFFFFF
+
+
+def test_result_messages():
+    lib = nk.lib()
+    assert lib.nuka_result_message(0) == b"ok"
+    assert lib.nuka_result_message(7) == b"not supported"
