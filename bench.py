@@ -1,0 +1,140 @@
+"""Headline benchmark: env-steps/s of the batched articulation step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 3] [--envs 4096] [--mode eager|graph]
+
+One "step" is one pass of the whole pipeline (FK, dynamics, contacts, block-descent solve, integration, FK) over
+every environment of the batch, state resident in HBM.  Every timed step starts from the same seeded batch: the
+state is put back by a device-side checkpoint restore INSIDE the timed region, so the figure is the cost of a step
+on the published input distribution and does not drift with the trajectory (left alone, the humanoids fall away
+from the plane within a few dozen steps and the contact solve has nothing left to do - that free-running figure
+is reported beside it as `free_running_ms_per_step`).  Prints ONE JSON line."""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+HBM_PEAK_GBPS = 8000.0
+DOMINANT_OP = "BlockDescentSolve"
+DOMINANT_KERNEL = "BlockDescentTileKernel"
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, scaled
+# by the same counters' reading of a plain copy of known size); keyed by (config, envs).  None where not measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def algorithmic_bytes(nl, nv, nc, floating):
+    """Bytes per env-step the step must move at least: state in/out (tier A) plus the fields the seam keeps in
+    HBM once per step - packed M, packed L.D, bias, contact Jacobians - written once and read once (tier B)."""
+    nj, f = nl - 1, 1 if floating else 0
+    tier_a = 4 * ((3 * nj + 13 * f) + (nv + nj + nv + 7 * f + 7 * nl + 3 * nc + 2 * nc + 1))
+    tier_b = 8 * (nv * (nv + 1) + nv + 3 * nc * nv)
+    return tier_a, tier_a + tier_b
+
+
+def solver_bytes(nv, nc):
+    """The solve's share of that figure: it reads packed M, packed L.D, the contact Jacobians and the free velocity,
+    and writes the velocity and the impulses."""
+    return 4 * (nv * (nv + 1) + 3 * nc * nv + 2 * nv + 3 * nc)
+
+
+def cpu_baseline(nk, cfg, desc, budget_s=12.0):
+    """The CPU oracle (a restatement of the reference algorithm, OpenMP over environments) on the same workload."""
+    oracle_py = entry.load_oracle()
+    threads = min(16, os.cpu_count() or 1)
+    world = oracle_py.OracleWorld(cfg.template, desc, threads=threads)
+    state = cfg.state()
+    world.set_state(state)
+    world.step()                      # first touch of every page
+    start = time.perf_counter()
+    steps = 0
+    while time.perf_counter() - start < budget_s:
+        world.set_state(state)        # every step from the seeded batch, as on the GPU
+        world.step()
+        steps += 1
+    elapsed = time.perf_counter() - start
+    world.close()
+    return {"value": cfg.env_count * steps / elapsed, "unit": "env-steps/s", "cores": threads, "kind": "port",
+            "sample": f"{steps} steps of the same seeded {cfg.env_count}-env batch in {elapsed:.1f} s, gcc -O2 -fopenmp"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--config", type=int, default=3)
+    ap.add_argument("--envs", type=int, default=0)
+    ap.add_argument("--mode", choices=("eager", "graph"), default="graph")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path runs on one GPU (one wavefront per environment, no cross-device state); "
+                 "--gpus must be 1")
+
+    nk = entry.load_package()
+    cfg = nk.synthetic.config(args.config, args.envs or None)
+    E = cfg.env_count
+    desc = nk.abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters)
+    device = nk.Device(0)
+    world = nk.World(device, cfg.template, desc)
+    world.set_state(cfg.state())
+    world.set_execution_mode(args.mode == "graph")
+
+    seeded = world.checkpoint()
+    world.step_from(seeded, args.warmup)
+    world.synchronize()
+    start = time.perf_counter()
+    world.step_from(seeded, args.steps)
+    world.synchronize()
+    wall_ms = (time.perf_counter() - start) * 1e3 / args.steps
+    event_ms = world.time_steps(args.steps, seeded) / args.steps  # device events on the world's own stream
+    world.restore(seeded)
+    world.step(100)                                               # the trajectory left alone, for comparison
+    free_ms = world.time_steps(args.steps) / args.steps
+
+    # per-op durations with device events on the launch stream (eager dispatch), for the dominant kernel
+    world.set_execution_mode(False)
+    per_op = {}
+    for name, ms in world.profile_ops(min(args.steps, 50), seeded):
+        per_op[name] = per_op.get(name, 0.0) + ms
+    dominant_ms = per_op.get(DOMINANT_OP, 0.0)
+    nl, nv = world.link_count, world.dof
+    nc = world.info.contact_slots_per_env
+    tier_a, b_alg = algorithmic_bytes(nl, nv, nc, cfg.floating)
+    if world.rows_per_env == 0 or dominant_ms == 0.0:             # contact-free worlds: dynamics is the step
+        kernel, kernel_ms, kernel_bytes = "ArticulationDynamicsKernel", per_op.get("ArticulationDynamics", 0.0), 8 * (nv * (nv + 1) + nv) + 4 * (3 * (nl - 1) + 2 * nv)
+    else:
+        kernel, kernel_ms, kernel_bytes = DOMINANT_KERNEL, dominant_ms, solver_bytes(nv, nc)
+    achieved = kernel_bytes * E / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
+    step_gbps = b_alg * E / (wall_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "env-steps/sec", "value": E * 1e3 / wall_ms, "unit": "env-steps/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall_ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{cfg.name}: {nl} links, {nv} DoF, {nc} contact spheres, {E} envs, dt {cfg.dt:.6f}, "
+                               f"{cfg.vel_iters} block-descent sweeps", "config_index": args.config, "envs": E,
+                   "execution": args.mode, "event_ms_per_step": event_ms,
+                   "each_step_from": "seeded batch (checkpoint restore inside the timed region)",
+                   "free_running_ms_per_step": free_ms},
+        "roofline": {"bound": "hbm", "kernel": kernel, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, E)),
+                     "algorithmic_bytes_per_launch": kernel_bytes * E, "kernel_ms": kernel_ms},
+        "roofline_step": {"algorithmic_bytes_per_env_step": b_alg, "state_io_bytes_per_env_step": tier_a,
+                          "achieved": step_gbps, "unit": "GB/s", "frac": step_gbps / HBM_PEAK_GBPS},
+        "per_op_ms": {k: round(v, 4) for k, v in per_op.items() if v >= 0.001},
+        "copy_ceiling_gbps": device.copy_bandwidth(1 << 28, 10),
+    }
+    world.close()
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(nk, cfg, desc)
+    device.close()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

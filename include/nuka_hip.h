@@ -112,6 +112,14 @@ nuka_result_t nuka_world_get_velocity_iterations(nuka_world_handle world, uint32
 nuka_result_t nuka_world_synchronize(nuka_world_handle world);   /* nuka.h:376 */
 nuka_result_t nuka_world_reset(nuka_world_handle world);         /* nuka.h:380 */
 
+/* nuka.h:386-398: a checkpoint holds the persistent physics of every environment, in device memory here.  Restore
+ * is enqueued on the world's stream (no host wait) and refuses a checkpoint of another world. */
+typedef struct nuka_checkpoint_t* nuka_checkpoint_handle;
+nuka_result_t nuka_world_checkpoint_capture(nuka_world_handle world, nuka_checkpoint_handle* out);
+nuka_result_t nuka_world_checkpoint_restore(nuka_world_handle world, nuka_checkpoint_handle checkpoint);
+void nuka_checkpoint_destroy(nuka_checkpoint_handle checkpoint);
+nuka_result_t nuka_checkpoint_byte_size(nuka_checkpoint_handle checkpoint, uint64_t* out_bytes);
+
 /* nk::World::DispatchOp (src/nk/pipeline/world.hpp): one op of the pipeline with the pipeline's own parameters.
  * `variant` 1 on ArticulationDynamics dispatches it with integrate_velocity = 0, the probe
  * tests/oracle/featherstone_oracle_harness.cpp:174-182 uses. */
@@ -146,9 +154,13 @@ nuka_result_t nuka_world_get_info(nuka_world_handle world, nuka_world_info_t* ou
 /* Timing on the world's own stream with device events, as tests/perf/test_go2_4096env_step_time.cpp:118-137
  * (back-to-back steps, one wait at the end) and, per op, as the eager profiler behind NUKA_STEP_TIMING
  * (src/phi/backend_cuda/cuda_backend.cu:78-120, 188-221). */
-nuka_result_t nuka_world_time_steps(nuka_world_handle world, uint32_t step_count, float* out_total_ms);
+/* `from` non-null: every step is preceded by a restore of that checkpoint (inside the timed region), so that each
+ * timed step runs on the same state; null: the steps follow one another. */
+nuka_result_t nuka_world_time_steps(nuka_world_handle world, nuka_checkpoint_handle from, uint32_t step_count,
+                                    float* out_total_ms);
 /* out_ms has one slot per pipeline op (nuka_world_info_t::op_count); out_ops receives their op ids. */
-nuka_result_t nuka_world_profile_ops(nuka_world_handle world, uint32_t step_count, float* out_ms, uint16_t* out_ops);
+nuka_result_t nuka_world_profile_ops(nuka_world_handle world, nuka_checkpoint_handle from, uint32_t step_count,
+                                     float* out_ms, uint16_t* out_ops);
 /* Device-to-device copy of `bytes` bytes repeated `repeats` times on the world's stream; the streaming-copy ceiling. */
 nuka_result_t nuka_device_copy_bandwidth(nuka_device_handle device, size_t bytes, uint32_t repeats, float* out_gb_per_s);
 

@@ -38,7 +38,8 @@ EXPORTS = [
     "nuka_result_message", "nuka_last_error_message", "nuka_device_create", "nuka_device_destroy", "nuka_device_backend",
     "nuka_world_create_from_template", "nuka_world_destroy", "nuka_world_step", "nuka_world_step_n",
     "nuka_world_set_execution_mode", "nuka_world_set_velocity_iterations", "nuka_world_get_velocity_iterations",
-    "nuka_world_synchronize", "nuka_world_reset", "nuka_world_dispatch_op", "nuka_field_from_name", "nuka_field_names",
+    "nuka_world_synchronize", "nuka_world_reset", "nuka_world_checkpoint_capture", "nuka_world_checkpoint_restore",
+    "nuka_checkpoint_destroy", "nuka_checkpoint_byte_size", "nuka_world_dispatch_op", "nuka_field_from_name", "nuka_field_names",
     "nuka_world_get_buffer_view", "nuka_world_upload_field", "nuka_world_download_field", "nuka_world_get_info",
     "nuka_world_time_steps", "nuka_world_profile_ops", "nuka_device_copy_bandwidth", "nuka_hip_register_backend_entry",
     "nuka_hip_op_count", "nuka_hip_op_name", "nuka_hip_op_from_name",
@@ -88,8 +89,12 @@ def lib():
         L.nuka_world_upload_field.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_size_t, C.c_size_t]
         L.nuka_world_download_field.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_size_t, C.c_size_t]
         L.nuka_world_get_info.argtypes = [C.c_void_p, C.POINTER(WorldInfoC)]
-        L.nuka_world_time_steps.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(C.c_float)]
-        L.nuka_world_profile_ops.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(C.c_float), C.POINTER(C.c_uint16)]
+        L.nuka_world_time_steps.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.POINTER(C.c_float)]
+        L.nuka_world_profile_ops.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.POINTER(C.c_float), C.POINTER(C.c_uint16)]
+        L.nuka_world_checkpoint_capture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        L.nuka_world_checkpoint_restore.argtypes = [C.c_void_p, C.c_void_p]
+        L.nuka_checkpoint_destroy.argtypes = [C.c_void_p]
+        L.nuka_checkpoint_byte_size.argtypes = [C.c_void_p, C.POINTER(C.c_uint64)]
         L.nuka_device_copy_bandwidth.argtypes = [C.c_void_p, C.c_size_t, C.c_uint32, C.POINTER(C.c_float)]
         _lib = L
     return _lib
@@ -182,6 +187,23 @@ class World:
     def synchronize(self):
         _check(lib().nuka_world_synchronize(self._h))
 
+    def checkpoint(self):
+        """nuka_world_checkpoint_capture: the persistent physics of every environment, kept in device memory."""
+        handle = C.c_void_p()
+        _check(lib().nuka_world_checkpoint_capture(self._h, C.byref(handle)))
+        return handle
+
+    def restore(self, checkpoint):
+        """nuka_world_checkpoint_restore, enqueued on the world's stream."""
+        _check(lib().nuka_world_checkpoint_restore(self._h, checkpoint))
+
+    def step_from(self, checkpoint, n=1):
+        """n times: restore the checkpoint, then one step - every step runs on the checkpointed state."""
+        L, h = lib(), self._h
+        for _ in range(n):
+            _check(L.nuka_world_checkpoint_restore(h, checkpoint))
+            _check(L.nuka_world_step(h))
+
     def reset(self):
         _check(lib().nuka_world_reset(self._h))
 
@@ -191,13 +213,14 @@ class World:
     def set_velocity_iterations(self, n):
         _check(lib().nuka_world_set_velocity_iterations(self._h, n))
 
-    def time_steps(self, n):
+    def time_steps(self, n, checkpoint=None):
+        """Milliseconds of n steps by device events on the world's stream; with a checkpoint every step starts from it."""
         out = C.c_float()
-        _check(lib().nuka_world_time_steps(self._h, n, C.byref(out)))
+        _check(lib().nuka_world_time_steps(self._h, checkpoint, n, C.byref(out)))
         return out.value
 
-    def profile_ops(self, steps):
+    def profile_ops(self, steps, checkpoint=None):
         ms = (C.c_float * self.op_count)()
         ops = (C.c_uint16 * self.op_count)()
-        _check(lib().nuka_world_profile_ops(self._h, steps, ms, ops))
+        _check(lib().nuka_world_profile_ops(self._h, checkpoint, steps, ms, ops))
         return [(lib().nuka_hip_op_name(ops[i]).decode(), ms[i] / steps) for i in range(self.op_count)]

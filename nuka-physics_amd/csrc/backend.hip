@@ -108,6 +108,7 @@ nuka_phi_buffer* BtAlloc(nuka_phi_buffer_type* t, size_t bytes, uint8_t* status)
     auto* buffer = new (std::nothrow) Buffer{&kBufferI, nullptr, bytes, type->host, type->stream};
     if (buffer == nullptr) { set(Status::OutOfMemory); return nullptr; }
     if (bytes > 0u) {
+        if (hipSetDevice(type->device) != hipSuccess) { (void)hipGetLastError(); delete buffer; set(Status::Failed); return nullptr; }
         const size_t padded = (bytes + 255u) & ~size_t{255u};
         const hipError_t e = type->host ? hipHostMalloc(&buffer->base, padded, hipHostMallocDefault) : hipMalloc(&buffer->base, padded);
         if (e != hipSuccess) { (void)hipGetLastError(); delete buffer; set(Status::OutOfMemory); return nullptr; }
@@ -274,7 +275,8 @@ const nuka_phi_backend_i kBackendI = {BeName, BeFree, BeDispatch, BeSynchronize,
                                       BePlanMetrics, BePlanExecuteRepeated};
 
 // ---- device and registry entry (device.cu, cuda_backend.cu:714) -----------------------------------------
-struct Device { const nuka_phi_device_i* iface; int index; char name[256]; };
+struct Device { const nuka_phi_device_i* iface; int index; char name[256]; BufferType device_type, host_type; };
+hipStream_t g_default_stream = nullptr;   // device-level buffer types move bytes on the default stream
 struct RegistryEntry { const nuka_phi_registry_entry_i* iface; Device devices[16]; size_t count; };
 
 const char* DevName(nuka_phi_device* d) { return reinterpret_cast<Device*>(d)->name; }
@@ -287,9 +289,8 @@ void DevMemory(nuka_phi_device* d, size_t* free_b, size_t* total_b) {
 nuka_phi_backend* DevInitBackend(nuka_phi_device* d, const char*) {
     return reinterpret_cast<nuka_phi_backend*>(CreateBackend(reinterpret_cast<Device*>(d)->index, nullptr));
 }
-// Buffer types belong to a backend (they allocate on its stream's device); the device-level query serves none.
-nuka_phi_buffer_type* DevBufferType(nuka_phi_device*) { return nullptr; }
-nuka_phi_buffer_type* DevHostBufferType(nuka_phi_device*) { return nullptr; }
+nuka_phi_buffer_type* DevBufferType(nuka_phi_device* d) { return reinterpret_cast<nuka_phi_buffer_type*>(&reinterpret_cast<Device*>(d)->device_type); }
+nuka_phi_buffer_type* DevHostBufferType(nuka_phi_device* d) { return reinterpret_cast<nuka_phi_buffer_type*>(&reinterpret_cast<Device*>(d)->host_type); }
 int DevSupportsOp(nuka_phi_device*, uint16_t op) {
     std::call_once(g_ops_once, RegisterOps);
     return op < uint16_t(NkOp::Count) && g_ops[op] != nullptr ? 1 : 0;
@@ -354,6 +355,8 @@ nuka_phi_registry_entry* nuka_hip_register_backend_entry(void) {
         for (size_t i = 0u; i < entry.count; ++i) {
             entry.devices[i].iface = &nkh::kDeviceI;
             entry.devices[i].index = int(i);
+            entry.devices[i].device_type = nkh::BufferType{&nkh::kBufferTypeI, false, &nkh::g_default_stream, int(i)};
+            entry.devices[i].host_type = nkh::BufferType{&nkh::kBufferTypeI, true, &nkh::g_default_stream, int(i)};
             hipDeviceProp_t prop;
             if (hipGetDeviceProperties(&prop, int(i)) == hipSuccess) std::snprintf(entry.devices[i].name, sizeof(entry.devices[i].name), "%s", prop.name);
             else std::snprintf(entry.devices[i].name, sizeof(entry.devices[i].name), "HIP device %zu", i);

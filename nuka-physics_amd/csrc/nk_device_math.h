@@ -172,6 +172,11 @@ __device__ __forceinline__ uint32_t wave_max_u(uint32_t v) {
     for (int o = 32; o > 0; o >>= 1) { const uint32_t other = __shfl_xor(v, o, 64); v = other > v ? other : v; }
     return v;
 }
+__device__ __forceinline__ uint32_t wave_sum_u(uint32_t v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += uint32_t(__shfl_xor(int(v), o, 64));
+    return v;
+}
 __device__ __forceinline__ bool wave_all(bool p) { return __all(p); }
 __device__ __forceinline__ bool wave_any(bool p) { return __any(p); }
 

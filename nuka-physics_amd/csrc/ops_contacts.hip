@@ -215,10 +215,8 @@ __device__ V3 inverse_transform_point(Xf xf, V3 wp) {   // prims_types.cuh:98-10
 }
 
 // ---- NarrowphasePrimitives: one thread per (env, slot) (narrowphase_prims.cu:181-366, analytic route) ----
-__global__ void NarrowphaseKernel(ModelView m, DataView d, NarrowphasePrimitivesParams p) {
-    const uint32_t item = blockIdx.x * blockDim.x + threadIdx.x;
-    if (item >= p.env_count * p.rigid_slot_cap) return;
-    const uint32_t env = item / p.rigid_slot_cap, slot = item - env * p.rigid_slot_cap;
+__device__ uint32_t NarrowphaseSlot(const ModelView& m, const DataView& d, const NarrowphasePrimitivesParams& p, uint32_t env,
+                                    uint32_t slot) {
     const size_t gid = size_t{env} * p.union_slot_count + slot;
     const size_t bbase = size_t{env} * p.bodies_per_env;
     const float separation = fmaxf(p.contact_margin, 0.0005f);
@@ -256,8 +254,21 @@ __global__ void NarrowphaseKernel(ModelView m, DataView d, NarrowphasePrimitives
         d.ucontact_id_pair[at] = (uint64_t{a & 0x0fffffffu} << 32u) | uint64_t{b & 0x0fffffffu};
         d.ucontact_id_feature[at] = h;
     }
+    return mf.count;
 }
 
+// One wavefront per environment; its lanes take the environment's slots in strides of 64, and the per-environment
+// contact count is a wave sum (no atomics).
+__global__ void __launch_bounds__(64) NarrowphaseKernel(ModelView m, DataView d, NarrowphasePrimitivesParams p) {
+    const uint32_t env = blockIdx.x, lane = threadIdx.x;
+    uint32_t contacts = 0u;
+    for (uint32_t first = 0u; first < p.rigid_slot_cap; first += 64u) {
+        const uint32_t slot = first + lane;
+        if (slot < p.rigid_slot_cap) contacts += NarrowphaseSlot(m, d, p, env, slot);
+    }
+    contacts = wave_sum_u(contacts);
+    if (lane == 0u) d.contact_count[env] = contacts;
+}
 // math/cuda_vec_ops.cuh:150-183
 __device__ void contact_tangent_basis(V3 normal, V3* t1, V3* t2) {
     V3 n = normal;
@@ -535,8 +546,7 @@ Status OpNarrowphasePrimitives(const ModelView& m, const DataView& d, const void
     const auto* p = static_cast<const NarrowphasePrimitivesParams*>(params);
     if (p == nullptr) return Status::Failed;
     if (p->env_count == 0u || p->union_slot_count == 0u || p->rigid_slot_cap == 0u) return Status::Ok;
-    const uint32_t total = p->env_count * p->rigid_slot_cap;
-    hipLaunchKernelGGL(NarrowphaseKernel, dim3((total + 127u) / 128u), dim3(128), 0, stream, m, d, *p);
+    hipLaunchKernelGGL(NarrowphaseKernel, dim3(p->env_count), dim3(64), 0, stream, m, d, *p);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 

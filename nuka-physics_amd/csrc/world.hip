@@ -64,6 +64,8 @@ struct HostModel {
         joint_stiffness, joint_spring_reference, link_geom_local, shape_table, body_collidable_local, body_init_pose, profile_mu;
 };
 
+struct NotSupported : std::runtime_error { using std::runtime_error::runtime_error; };
+
 std::vector<float> CopyOrZero(const float* src, size_t n) {
     return src != nullptr ? std::vector<float>(src, src + n) : std::vector<float>(n, 0.0f);
 }
@@ -171,15 +173,25 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
         m.body_collidable_body[b] = m.link_body[link];
         std::memcpy(m.body_collidable_local.data() + 7u * b, d.body_local + 7u * b, 7u * sizeof(float));
     }
-    uint32_t slots = d.max_contacts_per_env;
-    if (slots == 0u)
-        for (uint32_t i = 0u; i < nb; ++i)
-            for (uint32_t j = i + 1u; j < nb; ++j) {
-                if (d.body_role[i] == 0u && d.body_role[j] == 0u) continue;
-                if (d.shape_kind[i] == kInvalid || d.shape_kind[j] == kInvalid) continue;
-                if (((d.shape_contype[i] & d.shape_conaffinity[j]) | (d.shape_contype[j] & d.shape_conaffinity[i])) == 0u) continue;
-                ++slots;
-            }
+    // Manifolds built here: sphere and box against a plane, either order.  Any other admitted pair is refused at
+    // cook time instead of silently producing no contact.
+    uint32_t admitted = 0u;
+    for (uint32_t i = 0u; i < nb; ++i) {
+        const uint32_t kind = d.shape_kind[i];
+        if (kind != kInvalid && kind != kShapeSphere && kind != kShapeBox && kind != kShapePlane)
+            throw NotSupported("shape kind not supported on this path (sphere, box, plane)");
+        for (uint32_t j = i + 1u; j < nb; ++j) {
+            if (d.body_role[i] == 0u && d.body_role[j] == 0u) continue;
+            if (kind == kInvalid || d.shape_kind[j] == kInvalid) continue;
+            if (((d.shape_contype[i] & d.shape_conaffinity[j]) | (d.shape_contype[j] & d.shape_conaffinity[i])) == 0u) continue;
+            const int32_t ga = int32_t(d.shape_group[i]), gb = int32_t(d.shape_group[j]);   // shape_kind.hpp:26-33
+            if (ga != 0 && gb != 0 && (ga > 0 ? ga != gb && gb > 0 : ga == gb)) continue;
+            if ((kind == kShapePlane) == (d.shape_kind[j] == kShapePlane))
+                throw NotSupported("admitted collidable pair has no manifold on this path (one side must be a plane)");
+            ++admitted;
+        }
+    }
+    const uint32_t slots = d.max_contacts_per_env != 0u ? d.max_contacts_per_env : admitted;
     ModelView& c = m.counts;
     c.links_per_env = nl; c.bodies_per_env = nb; c.dof = nv; c.max_dof = nv; c.max_depth = max_depth;
     c.contact_slots = slots;
@@ -263,6 +275,35 @@ struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
         if (initial != nullptr) reinterpret_cast<nuka_phi_buffer_head*>(initial)->iface->free(initial);
     }
 };
+
+// Checkpoint of the persistent physics (src/include/nuka/nuka.h:388-392): every state field a step reads before it
+// writes it.  The mass matrix, its factor and the contact Jacobians are rebuilt by every step and stay out.
+constexpr uint32_t kMaxCheckpointSegments = 64u;
+struct CheckpointSegments {
+    uint32_t count;
+    uint32_t units[kMaxCheckpointSegments];          // 16-byte units
+    char* live[kMaxCheckpointSegments];
+    char* kept[kMaxCheckpointSegments];
+};
+struct Checkpoint {
+    World* owner = nullptr;
+    nuka_phi_buffer* store = nullptr;
+    CheckpointSegments segments{};
+    uint64_t bytes = 0u;
+};
+
+// blockIdx.y picks the segment, blockIdx.x strides over its 16-byte units.
+__global__ void __launch_bounds__(256) CheckpointCopyKernel(CheckpointSegments s, uint32_t restore) {
+    const uint32_t seg = blockIdx.y;
+    const uint4* src = reinterpret_cast<const uint4*>(restore != 0u ? s.kept[seg] : s.live[seg]);
+    uint4* dst = reinterpret_cast<uint4*>(restore != 0u ? s.live[seg] : s.kept[seg]);
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < s.units[seg]; i += gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
+bool CheckpointExcludes(const char* name) {
+    for (const char* rebuilt : {"m", "m_factor", "chain_jacobian", "chain_jacobian_b"}) if (std::strcmp(name, rebuilt) == 0) return true;
+    return false;
+}
 
 const nuka_phi_buffer_i* Iface(nuka_phi_buffer* b) { return reinterpret_cast<nuka_phi_buffer_head*>(b)->iface; }
 
@@ -544,6 +585,8 @@ nuka_result_t nuka_world_create_from_template(nuka_device_handle device, const n
         return NUKA_RESULT_OK;
     } catch (const std::invalid_argument& e) {
         return Error(NUKA_RESULT_INVALID_ARG, e.what());
+    } catch (const NotSupported& e) {
+        return Error(NUKA_RESULT_NOT_SUPPORTED, e.what());
     } catch (const std::bad_alloc&) {
         return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
     } catch (const std::exception& e) {
@@ -694,15 +737,22 @@ nuka_result_t nuka_world_get_info(nuka_world_handle world, nuka_world_info_t* ou
     return NUKA_RESULT_OK;
 }
 
-nuka_result_t nuka_world_time_steps(nuka_world_handle world, uint32_t step_count, float* out_total_ms) {
+nuka_result_t nuka_world_time_steps(nuka_world_handle world, nuka_checkpoint_handle from, uint32_t step_count, float* out_total_ms) {
     auto* w = reinterpret_cast<World*>(world);
     if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
     if (out_total_ms == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    if (from != nullptr && reinterpret_cast<Checkpoint*>(from)->owner != w) return Error(NUKA_RESULT_INVALID_ARG, "checkpoint belongs to another world");
     nuka_phi_event* start = w->be->event_new(w->backend);
     nuka_phi_event* stop = w->be->event_new(w->backend);
     if (start == nullptr || stop == nullptr) return Error(NUKA_RESULT_DEVICE_ERROR, "event creation failed");
     w->be->event_record(w->backend, start);
-    const nuka_result_t r = StepN(*w, step_count);
+    nuka_result_t r = NUKA_RESULT_OK;
+    if (from == nullptr) r = StepN(*w, step_count);
+    else
+        for (uint32_t s = 0u; s < step_count && r == NUKA_RESULT_OK; ++s) {
+            r = nuka_world_checkpoint_restore(world, from);
+            if (r == NUKA_RESULT_OK) r = StepN(*w, 1u);
+        }
     w->be->event_record(w->backend, stop);
     w->be->event_wait(w->backend, stop);
     *out_total_ms = w->be->event_elapsed_ms(w->backend, start, stop);
@@ -711,16 +761,19 @@ nuka_result_t nuka_world_time_steps(nuka_world_handle world, uint32_t step_count
     return r;
 }
 
-nuka_result_t nuka_world_profile_ops(nuka_world_handle world, uint32_t step_count, float* out_ms, uint16_t* out_ops) {
+nuka_result_t nuka_world_profile_ops(nuka_world_handle world, nuka_checkpoint_handle from, uint32_t step_count, float* out_ms,
+                                     uint16_t* out_ops) {
     auto* w = reinterpret_cast<World*>(world);
     if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
     if (out_ms == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    if (from != nullptr && reinterpret_cast<Checkpoint*>(from)->owner != w) return Error(NUKA_RESULT_INVALID_ARG, "checkpoint belongs to another world");
     const size_t n = w->calls.size();
     std::vector<nuka_phi_event*> events(n + 1u, nullptr);
     for (auto& e : events) e = w->be->event_new(w->backend);
     for (size_t i = 0u; i < n; ++i) { out_ms[i] = 0.0f; if (out_ops != nullptr) out_ops[i] = w->calls[i].op; }
     nuka_result_t result = NUKA_RESULT_OK;
     for (uint32_t s = 0u; s < step_count && result == NUKA_RESULT_OK; ++s) {
+        if (from != nullptr && (result = nuka_world_checkpoint_restore(world, from)) != NUKA_RESULT_OK) break;
         w->be->event_record(w->backend, events[0]);
         for (size_t i = 0u; i < n; ++i) {
             const uint8_t status = w->be->dispatch(w->backend, reinterpret_cast<const nuka_phi_model_view*>(&w->model),
@@ -766,6 +819,72 @@ nuka_result_t nuka_device_copy_bandwidth(nuka_device_handle device, size_t bytes
     Iface(a)->free(a);
     Iface(b)->free(b);
     *out_gb_per_s = ms > 0.0f ? float(2.0 * double(bytes) * repeats / (double(ms) * 1.0e6)) : 0.0f;
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_checkpoint_capture(nuka_world_handle world, nuka_checkpoint_handle* out) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    *out = nullptr;
+    auto cp = std::unique_ptr<Checkpoint>(new (std::nothrow) Checkpoint{});
+    if (!cp) return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
+    cp->owner = w;
+    size_t total = 0u;
+    for (const Field& f : w->fields) {
+        if (f.is_template || f.count == 0u || CheckpointExcludes(f.name)) continue;
+        if (cp->segments.count == kMaxCheckpointSegments) return Error(NUKA_RESULT_INTERNAL, "too many checkpoint segments");
+        total += (f.count * f.elem_bytes + 255u) & ~size_t{255u};
+        ++cp->segments.count;
+    }
+    uint8_t status = 0u;
+    nuka_phi_buffer_type* type = BackendDeviceBufferType(w->device->backend);
+    cp->store = reinterpret_cast<nuka_phi_buffer_type_head*>(type)->iface->alloc(type, total, &status);
+    if (cp->store == nullptr) return Error(NUKA_RESULT_OUT_OF_MEMORY, "checkpoint allocation failed");
+    char* arena = static_cast<char*>(Iface(w->arena)->base(w->arena));
+    char* kept = static_cast<char*>(Iface(cp->store)->base(cp->store));
+    uint32_t at = 0u;
+    size_t offset = 0u;
+    for (const Field& f : w->fields) {
+        if (f.is_template || f.count == 0u || CheckpointExcludes(f.name)) continue;
+        const size_t padded = (f.count * f.elem_bytes + 255u) & ~size_t{255u};    // arena fields are 256-byte aligned and padded
+        cp->segments.live[at] = arena + f.offset;
+        cp->segments.kept[at] = kept + offset;
+        cp->segments.units[at] = uint32_t(padded / 16u);
+        offset += padded;
+        ++at;
+    }
+    cp->bytes = total;
+    hipLaunchKernelGGL(CheckpointCopyKernel, dim3(256, cp->segments.count), dim3(256), 0, BackendStream(w->device->backend), cp->segments, 0u);
+    if (hipGetLastError() != hipSuccess || nuka_world_synchronize(world) != NUKA_RESULT_OK) {
+        Iface(cp->store)->free(cp->store);
+        return Error(NUKA_RESULT_DEVICE_ERROR, "checkpoint capture failed");
+    }
+    *out = reinterpret_cast<nuka_checkpoint_handle>(cp.release());
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_checkpoint_restore(nuka_world_handle world, nuka_checkpoint_handle checkpoint) {
+    auto* w = reinterpret_cast<World*>(world);
+    auto* cp = reinterpret_cast<Checkpoint*>(checkpoint);
+    if (w == nullptr || cp == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world or checkpoint is null");
+    if (cp->owner != w) return Error(NUKA_RESULT_INVALID_ARG, "checkpoint belongs to another world");
+    hipLaunchKernelGGL(CheckpointCopyKernel, dim3(256, cp->segments.count), dim3(256), 0, BackendStream(w->device->backend), cp->segments, 1u);
+    return hipGetLastError() == hipSuccess ? NUKA_RESULT_OK : Error(NUKA_RESULT_DEVICE_ERROR, "checkpoint restore failed");
+}
+
+void nuka_checkpoint_destroy(nuka_checkpoint_handle checkpoint) {
+    auto* cp = reinterpret_cast<Checkpoint*>(checkpoint);
+    if (cp == nullptr) return;
+    if (cp->store != nullptr) Iface(cp->store)->free(cp->store);
+    delete cp;
+}
+
+nuka_result_t nuka_checkpoint_byte_size(nuka_checkpoint_handle checkpoint, uint64_t* out_bytes) {
+    auto* cp = reinterpret_cast<Checkpoint*>(checkpoint);
+    if (cp == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "checkpoint is null");
+    if (out_bytes == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    *out_bytes = cp->bytes;
     return NUKA_RESULT_OK;
 }
 

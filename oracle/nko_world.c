@@ -114,7 +114,8 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
                 const int si = d->body_role[i] == 0u, sj = d->body_role[j] == 0u;
                 if (si && sj) continue;
                 if (d->shape_kind[i] == NKO_INVALID || d->shape_kind[j] == NKO_INVALID) continue;
-                if (((d->shape_contype[i] & d->shape_conaffinity[j]) | (d->shape_contype[j] & d->shape_conaffinity[i])) == 0u) continue;
+                if (!nko_shape_filter_admits(d->shape_contype[i], d->shape_conaffinity[i], d->shape_group[i],
+                                             d->shape_contype[j], d->shape_conaffinity[j], d->shape_group[j])) continue;
                 ++slots;
             }
     }

@@ -1,0 +1,244 @@
+"""Size-independent properties of the HIP path at the published sizes, edge cases and error paths (MI355X)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from conftest import nk, relative_error
+
+pytestmark = pytest.mark.gpu
+abi = nk.abi
+ROW_WORDS = 26
+IDENTITY7 = np.array([0, 0, 0, 1, 0, 0, 0], np.float32)
+
+
+def stepped(device, index, E, **kw):
+    cfg = nk.synthetic.config(index, E)
+    world = nk.World(device, cfg.template, abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters, **kw))
+    world.set_state(cfg.state())
+    return cfg, world
+
+
+def test_humanoid_4096_contact_solution_properties(device):
+    """The headline batch: cone, non-negative normal impulses, momentum balance M dv = J^T lambda with the GPU's own
+    M and J, finite state, and environments independent of the batch they run in."""
+    E = 4096
+    cfg, world = stepped(device, 3, E)
+    for name in ("FkWorldPoses", "ArticulationDynamics", "SyncLinkBodyPose", "BuildAabbs", "LbvhQueryPairs",
+                 "NarrowphasePrimitives", "AssembleRows"):
+        world.op(name)
+    world.synchronize()
+    n, R, nl = world.dof, world.rows_per_env, world.link_count
+    free = world.download("qdot_flat").reshape(E, -1)[:, :n].astype(np.float64)
+    world.op("BlockDescentSolve")
+    world.synchronize()
+    rows = world.download("urows").reshape(E, R, ROW_WORDS)
+    words = rows.view(np.uint32)
+    lam = world.download("lambda").reshape(E, R).astype(np.float64)
+    assert np.all(world.download("env_status") == 0) and np.all(np.isfinite(lam))
+    normal = (words[:, :, 0] & (1 << 6)) != 0
+    assert normal.sum() > E
+    assert np.all(lam[normal] >= 0)
+    e_idx, r_idx = np.nonzero(normal)
+    P = words[e_idx, r_idx, 2]
+    tangent = np.hypot(lam[e_idx, r_idx + P], lam[e_idx, r_idx + 2 * P])
+    mu = rows[e_idx, r_idx, 8]
+    assert np.all(tangent <= mu * lam[e_idx, r_idx] * (1 + 1e-5) + 1e-7)
+    assert np.all(lam[(words[:, :, 0] & 1) == 0] == 0)                         # dead rows hold no impulse
+    M = world.download("m").reshape(E, n, n).astype(np.float64)
+    J = (world.download("chain_jacobian").reshape(E, R, -1) + world.download("chain_jacobian_b").reshape(E, R, -1))[:, :, :n]
+    scalar = [i for i, l in enumerate(cfg.template.links) if l["joint_type"] in (abi.JOINT_REVOLUTE, abi.JOINT_PRISMATIC)]
+    v = np.concatenate([world.download("link_velocity").reshape(E, nl, 6)[:, 0, :], world.download("qdot").reshape(E, nl)[:, scalar]], 1)
+    impulse = np.einsum("eri,er->ei", J.astype(np.float64), lam)
+    balance = np.einsum("eij,ej->ei", M, v - free) - impulse
+    imbalance = np.abs(np.linalg.solve(M, balance[:, :, None])[:, :, 0]).max(1)        # in velocity units
+    residual = world.download("solver_residual").reshape(E, 4)
+    # environments that met the tolerance inside the sweep budget hold the balance to rounding; the others stop with
+    # the impulses one dual update ahead of the velocity, which solver_residual reports
+    converged = world.download("vbd_velocity_sweep_count") < cfg.vel_iters
+    assert converged.mean() > 0.5
+    assert np.all(imbalance[converged] < 1.2e-5)                                       # the velocity tolerance is 1e-5
+    assert np.all(np.isfinite(residual[:, :3])) and np.all(residual[converged].max(1) < 2e-5)
+    # batch independence: the first 64 environments of the 4096 equal a 64-environment world bit for bit
+    _, small = stepped(device, 3, 64)
+    small.step()
+    small.synchronize()
+    world.reset()
+    world.set_state(cfg.state())
+    world.step()
+    world.synchronize()
+    for name, per in (("q", nl), ("qdot", nl), ("lambda", R), ("link_pose", nl * 7)):
+        assert np.array_equal(world.download(name).reshape(E, per)[:64], small.download(name).reshape(64, per)), name
+    small.close()
+    world.close()
+
+
+@pytest.mark.parametrize("index,E", [(2, 4096), (4, 16384)])
+def test_full_size_batches_step_cleanly(device, index, E):
+    cfg, world = stepped(device, index, E)
+    world.step(2)
+    world.synchronize()
+    assert np.all(world.download("env_status") == 0)
+    for name in ("q", "qdot", "link_pose", "lambda"):
+        assert np.all(np.isfinite(world.download(name))), name
+    pose = world.download("link_pose").reshape(E, -1, 7)
+    assert np.abs(np.linalg.norm(pose[:, :, 3:], axis=2) - 1).max() < 1e-5      # unit quaternions
+    assert np.all(world.download("pair_count") <= world.info.contact_slots_per_env)
+    world.close()
+
+
+def test_rope_full_batch_steps(device):
+    E = 1024
+    cfg, world = stepped(device, 5, E)
+    world.step()
+    world.synchronize()
+    assert np.all(np.isfinite(world.download("q"))) and np.all(np.isfinite(world.download("link_pose")))
+    world.close()
+
+
+def test_single_environment_and_contact_free_worlds(oracle_py, device):
+    for index in (1, 3):
+        cfg = nk.synthetic.config(index, 1)
+        desc = abi.world_desc(1, cfg.dt, vel_iters=cfg.vel_iters)
+        world, oracle = nk.World(device, cfg.template, desc), oracle_py.OracleWorld(cfg.template, desc)
+        state = cfg.state()
+        world.set_state(state)
+        oracle.set_state(state)
+        world.step()
+        world.synchronize()
+        oracle.step()
+        for name in ("q", "qdot", "link_pose"):
+            assert relative_error(world.download(name), oracle.download(name)) <= 1e-4
+        world.close()
+        oracle.close()
+
+
+def box_template(plane_first):
+    t = abi.Template()
+    t.add_link(abi.JOINT_FLOATING, None, mass=1.2, diag_inertia=(0.004, 0.006, 0.005))
+    t.add_link(abi.JOINT_REVOLUTE, 0, axis=(0, 1, 0), local_pos=(0.1, 0, 0.05), mass=0.3, diag_inertia=(0.001,) * 3, com=(0.05, 0, 0))
+    profile = t.add_profile(0.6)
+    plane = dict(kind=abi.SHAPE_PLANE, contype=2, conaffinity=1, profile=profile)
+    if plane_first:
+        t.add_body(abi.ROLE_STATIC, **plane)
+    t.add_body(abi.ROLE_LINK_BODY, link=0, contype=0, conaffinity=0)
+    t.add_body(abi.ROLE_LINK_BODY, link=1, contype=0, conaffinity=0)
+    t.add_body(abi.ROLE_PROXY, link=0, kind=abi.SHAPE_BOX, params=(0.1, 0.06, 0.04, 0), contype=1, conaffinity=2, profile=profile)
+    t.add_body(abi.ROLE_PROXY, link=1, kind=abi.SHAPE_SPHERE, params=(0.03, 0, 0, 0), local_pos=(0.1, 0, 0), contype=1, conaffinity=2, profile=profile)
+    if not plane_first:
+        t.add_body(abi.ROLE_STATIC, **plane)
+    return t
+
+
+@pytest.mark.parametrize("plane_first", [True, False])
+def test_box_manifolds_and_either_side_order(oracle_py, device, plane_first):
+    """A tilted box (up to four points per slot) plus a sphere; with the plane as the last row it is side B."""
+    E = 64
+    t = box_template(plane_first)
+    g = np.random.default_rng(4)
+    quat = np.array([1, 0, 0, 0]) + g.normal(0, 0.04, (E, 4))
+    base = np.concatenate([g.normal(0, 0.2, (E, 2)), g.uniform(0.035, 0.05, (E, 1)), quat / np.linalg.norm(quat, axis=1, keepdims=True)], 1)
+    zero = np.zeros((E, 1), np.float32)
+    state = dict(q=np.concatenate([zero, g.uniform(-0.3, 0.6, (E, 1))], 1).astype(np.float32),
+                 qdot=np.concatenate([zero, g.normal(0, 1, (E, 1))], 1).astype(np.float32), tau=np.zeros((E, 2), np.float32),
+                 base_pose=base.astype(np.float32), root_twist=g.normal(0, 0.3, (E, 6)).astype(np.float32))
+    desc = abi.world_desc(E, 1.0 / 200.0, vel_iters=50)
+    world, oracle = nk.World(device, t, desc), oracle_py.OracleWorld(t, desc, threads=4)
+    world.set_state(state)
+    oracle.set_state(state)
+    world.step()
+    world.synchronize()
+    oracle.step()
+    for name in ("pair_count", "ucontact_count", "ucontact_row_range", "ucontact_id_pair", "row_count", "env_status"):
+        assert np.array_equal(world.download(name), oracle.download(name)), name
+    counts = oracle.download("ucontact_count")
+    assert counts.max() == 4 and (counts == 1).any()
+    S = world.info.contact_slots_per_env
+    mask = np.arange(4)[None, None, :] < counts.reshape(E, S)[:, :, None]
+    ids_g, ids_o = world.download("ucontact_id_feature").reshape(E, S, 4), oracle.download("ucontact_id_feature").reshape(E, S, 4)
+    assert np.mean(ids_g[mask] == ids_o[mask]) > 0.99       # box corners carry feature ids: exact; sphere points hash a quantised position
+    for name in ("qdot", "q", "link_pose", "link_velocity"):
+        assert relative_error(world.download(name), oracle.download(name)) <= 1e-4, name
+    world.close()
+    oracle.close()
+
+
+def test_error_paths(device):
+    lib = nk.lib()
+    cfg = nk.synthetic.config(2, 8)
+    world = nk.World(device, cfg.template, abi.world_desc(8, cfg.dt))
+    fid, view = world._field("q")
+    nbytes = view.element_count * 4
+    buf = (C.c_char * (nbytes + 8))()
+    assert lib.nuka_world_download_field(world._h, fid, buf, nbytes + 4, 0) == 1          # past the end: refused, not clamped
+    assert lib.nuka_world_upload_field(world._h, fid, buf, 8, nbytes - 4) == 1
+    assert lib.nuka_world_download_field(world._h, fid, buf, 8, nbytes - 8) == 0
+    assert lib.nuka_world_download_field(world._h, 10_000, buf, 4, 0) == 7
+    assert lib.nuka_world_dispatch_op(world._h, 60_000, 0) == 1
+    assert lib.nuka_world_set_velocity_iterations(world._h, 0) == 1
+    assert lib.nuka_world_set_execution_mode(world._h, 5) == 1
+    world.close()
+    # templates outside the path are refused at creation
+    t = abi.Template()
+    t.add_link(abi.JOINT_FLOATING, None)
+    t.add_body(abi.ROLE_STATIC, kind=abi.SHAPE_PLANE, contype=2, conaffinity=1)
+    t.add_body(abi.ROLE_LINK_BODY, link=0, kind=abi.SHAPE_CAPSULE, params=(0.1, 0.2, 0, 0), contype=1, conaffinity=2)
+    with pytest.raises(nk.NukaError) as info:
+        nk.World(device, t, abi.world_desc(4, 0.005))
+    assert info.value.code == 7
+    t = abi.Template()
+    t.add_link(abi.JOINT_FIXED, None)
+    t.add_link(abi.JOINT_REVOLUTE, 5)
+    with pytest.raises(nk.NukaError) as info:
+        nk.World(device, t, abi.world_desc(4, 0.005))
+    assert info.value.code == 1
+    with pytest.raises(nk.NukaError):
+        nk.World(device, nk.synthetic.config(1, 1).template, abi.world_desc(0, 0.005))
+
+
+def table(handle, count):
+    """The function-pointer table a seam handle starts with."""
+    iface = C.cast(handle, C.POINTER(C.c_void_p))[0]
+    return C.cast(iface, C.POINTER(C.c_void_p * count))[0]
+
+
+def test_backend_seam_walk_through_the_tables(device):
+    """Drives the PHI-shaped seam the way a foreign host would: only through the tables of include/nuka_phi.h."""
+    lib = nk.lib()
+    lib.nuka_hip_register_backend_entry.restype = C.c_void_p
+    entry = lib.nuka_hip_register_backend_entry()
+    e = table(entry, 4)
+    name = C.CFUNCTYPE(C.c_char_p, C.c_void_p)(e[0])(entry)
+    assert b"hip" in name.lower()
+    assert C.CFUNCTYPE(C.c_size_t, C.c_void_p)(e[1])(entry) >= 1
+    dev = C.CFUNCTYPE(C.c_void_p, C.c_void_p, C.c_size_t)(e[2])(entry, 0)
+    d = table(dev, 6)
+    supports = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_uint16)(d[5])
+    names = [lib.nuka_hip_op_name(i).decode() for i in range(lib.nuka_hip_op_count())]
+    for wanted in ("FkWorldPoses", "ArticulationDynamics", "AssembleRows", "BlockDescentSolve", "IntegratePosition"):
+        assert supports(dev, names.index(wanted)) == 1
+    assert supports(dev, 60_000) == 0
+    free_b, total_b = C.c_size_t(), C.c_size_t()
+    C.CFUNCTYPE(None, C.c_void_p, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t))(d[1])(dev, C.byref(free_b), C.byref(total_b))
+    assert total_b.value > 200 * 2**30 and free_b.value <= total_b.value       # 288 GB of HBM3E
+    # buffer type -> buffer -> upload / download round trip, and out-of-range transfers refused
+    btype = C.CFUNCTYPE(C.c_void_p, C.c_void_p)(d[3])(dev)
+    bt = table(btype, 4)
+    assert C.CFUNCTYPE(C.c_int, C.c_void_p)(bt[3])(btype) == 0
+    status = C.c_uint8(9)
+    buf = C.CFUNCTYPE(C.c_void_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_uint8))(bt[1])(btype, 4096, C.byref(status))
+    assert buf and status.value == 0
+    b = table(buf, 6)
+    src = np.arange(1024, dtype=np.uint32)
+    dst = np.zeros_like(src)
+    upload = C.CFUNCTYPE(C.c_uint8, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t)(b[2])
+    download = C.CFUNCTYPE(C.c_uint8, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t)(b[3])
+    assert upload(buf, src.ctypes.data, 0, 4096) == 0 and download(buf, dst.ctypes.data, 0, 4096) == 0
+    assert np.array_equal(src, dst)
+    assert upload(buf, src.ctypes.data, 8, 4096) != 0
+    C.CFUNCTYPE(None, C.c_void_p)(b[0])(buf)
+    # the backend a device handle owns answers through its own table
+    lib.nuka_device_backend.restype = C.c_void_p
+    backend = lib.nuka_device_backend(device._h)
+    k = table(backend, 15)
+    assert b"hip" in C.CFUNCTYPE(C.c_char_p, C.c_void_p)(k[0])(backend).lower()

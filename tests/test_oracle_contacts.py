@@ -59,7 +59,8 @@ def test_pairs_are_the_brute_force_overlaps_in_canonical_order(oracle_py, index)
                 if ra["kind"] == abi.SHAPE_NONE or rb["kind"] == abi.SHAPE_NONE:
                     continue
                 admits = (ra["contype"] & rb["conaffinity"]) or (rb["contype"] & ra["conaffinity"])
-                if ra["group"] != 0 and ra["group"] == rb["group"]:
+                ga, gb = ra["group"], rb["group"]
+                if ga != 0 and gb != 0 and ((ga != gb and gb > 0) if ga > 0 else ga == gb):
                     admits = 0
                 overlap = np.all(aabb[e, a, :3] <= aabb[e, b, 3:]) and np.all(aabb[e, b, :3] <= aabb[e, a, 3:])
                 if admits and overlap:
