@@ -70,6 +70,8 @@ def main():
     ap.add_argument("--envs", type=int, default=0)
     ap.add_argument("--mode", choices=("eager", "graph"), default="graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seeded-only", action="store_true",
+                    help="skip the free-running comparison, so that every launch of the run is a step from the seeded batch (for profiles)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (one wavefront per environment, no cross-device state); "
@@ -92,9 +94,11 @@ def main():
     world.synchronize()
     wall_ms = (time.perf_counter() - start) * 1e3 / args.steps
     event_ms = world.time_steps(args.steps, seeded) / args.steps  # device events on the world's own stream
-    world.restore(seeded)
-    world.step(100)                                               # the trajectory left alone, for comparison
-    free_ms = world.time_steps(args.steps) / args.steps
+    free_ms = None
+    if not args.seeded_only:
+        world.restore(seeded)
+        world.step(100)                                           # the trajectory left alone, for comparison
+        free_ms = world.time_steps(args.steps) / args.steps
 
     # per-op durations with device events on the launch stream (eager dispatch), for the dominant kernel
     world.set_execution_mode(False)
