@@ -150,17 +150,27 @@ __device__ __forceinline__ uint32_t joint_dof(uint8_t type) {
     return type <= 1u ? 1u : type == 3u ? 6u : type == 4u ? 3u : 0u;
 }
 
-// 64-lane wave helpers
+// 64-lane wave helpers.  Reductions run inside each row of 16 lanes with DPP moves (lane^1, lane^2, mirror of 8,
+// mirror of 16: every step pairs lanes that already hold equal partial results, so a commutative combine leaves all
+// 16 lanes equal), then the four row results are read as scalars and combined as (r0 + r1) + (r2 + r3).  The result
+// is uniform across the wave.
 __device__ __forceinline__ float wave_bcast(float v, int lane) { return __shfl(v, lane, 64); }
+template <int Ctrl>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), Ctrl, 0xF, 0xF, false));
+}
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140;
+__device__ __forceinline__ float row_value(float v, int row) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16 * row));
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
+    v = fmaxf(v, dpp_move<kDppXor1>(v)); v = fmaxf(v, dpp_move<kDppXor2>(v));
+    v = fmaxf(v, dpp_move<kDppHalfMirror>(v)); v = fmaxf(v, dpp_move<kDppMirror>(v));
+    return fmaxf(fmaxf(row_value(v, 0), row_value(v, 1)), fmaxf(row_value(v, 2), row_value(v, 3)));
 }
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
+    v += dpp_move<kDppXor1>(v); v += dpp_move<kDppXor2>(v); v += dpp_move<kDppHalfMirror>(v); v += dpp_move<kDppMirror>(v);
+    return (row_value(v, 0) + row_value(v, 1)) + (row_value(v, 2) + row_value(v, 3));
 }
 __device__ __forceinline__ double wave_sum_d(double v) {
 #pragma unroll
@@ -168,6 +178,7 @@ __device__ __forceinline__ double wave_sum_d(double v) {
     return v;
 }
 __device__ __forceinline__ uint32_t wave_max_u(uint32_t v) {
+    // non-negative floats order like their bit patterns, and every caller passes such bits or small counts
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) { const uint32_t other = __shfl_xor(v, o, 64); v = other > v ? other : v; }
     return v;

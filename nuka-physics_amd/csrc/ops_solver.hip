@@ -1,9 +1,12 @@
 // UABD block-descent contact solve for gfx950.  One 64-lane wavefront owns one environment for the whole solve:
 // every velocity sweep, the dual updates and the split-impulse position pass run in a single launch with the
-// block's mass matrix, Newton Hessian, staged Jacobian rows and per-head state resident in LDS.  A lane is a block
-// coordinate in the matrix phases (one Hessian row per lane; nv <= 64 fits one wavefront, so the reference's
-// helper-warp machinery for wide tiles has no counterpart) and a head row in the per-head phases.  Cross-lane sums
-// use the compensated two-float butterfly; nothing is exchanged between environments.
+// staged Jacobian rows and per-head state resident in LDS.  A lane is a block coordinate in the matrix phases and
+// owns one matrix row IN REGISTERS: the kernel is compiled per padded width N (a multiple of 4, nv <= N <= 64), the
+// mass row, the Newton Hessian row and its Cholesky factor row are fully unrolled register arrays, pivots and
+// multipliers travel between lanes as scalar lane reads, and LDS only carries what must be read transposed (the
+// factor columns of the backward substitution) or broadcast (Jacobian rows, small vectors, read as 16-byte words).
+// The mass matrix is constant over a solve, so its factor is built once.  A lane is a head row in the per-head
+// phases.  Cross-lane sums use the compensated two-float butterfly; nothing is exchanged between environments.
 //
 // Replaces src/phi/backend_cuda/ops/block_descent_tile.cuh (DescendTile :2941-3087 and everything it calls) and
 // the helpers it takes from block_descent.cu (:735-820, 1593-1621, 1726-1753) and nk/solve/augmented_row.hpp.
@@ -24,6 +27,18 @@ constexpr float kLineTolerance = 1.0e-6f;     // block_descent_dense.cuh:17
 constexpr float kRoundings = 8.0f;            // block_descent_dense.cuh:19
 constexpr float kPenaltyConditionCap = 1.0e2f;   // block_descent.cu:71
 
+// Phase timers for development builds (-DNKH_SOLVER_PROFILE): cycles per phase and event counts per environment,
+// written over the environment's solver_penalty words at the end of the solve.
+#ifdef NKH_SOLVER_PROFILE
+#define PROF_BEGIN(c, i) const long long prof_start_##i = clock64()
+#define PROF_END(c, i) (c).prof[i] += clock64() - prof_start_##i
+#define PROF_COUNT(c, i) (c).prof_count[i] += 1u
+#else
+#define PROF_BEGIN(c, i)
+#define PROF_END(c, i)
+#define PROF_COUNT(c, i)
+#endif
+
 struct TileSum { float value, error; };   // block_descent_tile.cuh:15-31
 __device__ __forceinline__ void tile_add(TileSum& s, float x) {
     const float sum = s.value + x;
@@ -36,15 +51,21 @@ __device__ __forceinline__ void tile_add_product(TileSum& s, float a, float b) {
     s.error += fmaf(a, b, -product);
     tile_add(s, product);
 }
-// block_descent_tile.cuh:34-46 over 64 lanes
+// block_descent_tile.cuh:34-46 over 64 lanes: rows of 16 by DPP, then the four rows as scalars; uniform result
+__device__ __forceinline__ void tile_merge(TileSum& s, float value, float error) {
+    s.error += error;
+    tile_add(s, value);
+}
 __device__ __forceinline__ float wave_total(TileSum s) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const float value = __shfl_xor(s.value, o, kWave);
-        s.error += __shfl_xor(s.error, o, kWave);
-        tile_add(s, value);
-    }
-    return s.value + s.error;
+    tile_merge(s, dpp_move<kDppXor1>(s.value), dpp_move<kDppXor1>(s.error));
+    tile_merge(s, dpp_move<kDppXor2>(s.value), dpp_move<kDppXor2>(s.error));
+    tile_merge(s, dpp_move<kDppHalfMirror>(s.value), dpp_move<kDppHalfMirror>(s.error));
+    tile_merge(s, dpp_move<kDppMirror>(s.value), dpp_move<kDppMirror>(s.error));
+    TileSum a{row_value(s.value, 0), row_value(s.error, 0)}, b{row_value(s.value, 2), row_value(s.error, 2)};
+    tile_merge(a, row_value(s.value, 1), row_value(s.error, 1));
+    tile_merge(b, row_value(s.value, 3), row_value(s.error, 3));
+    tile_merge(a, b.value, b.error);
+    return a.value + a.error;
 }
 
 struct Response { float dual_scale, residual_scale; };
@@ -127,14 +148,19 @@ enum HeadField : uint32_t {
 struct Tile {
     uint32_t env, lane, n, ld, ldj, heads, cap, iteration;
     float tolerance;
-    float* mass;     // n x ld
-    float* hmat;     // n x ld
-    float* jac;      // 3 * cap rows x ldj
+    float* mfac;     // N x ld: Cholesky factor of the mass matrix (rows; columns are read transposed)
+    float* hfac;     // N x ld: Cholesky factor of the current Newton Hessian
+    float* jac;      // 3 * cap rows x ldj, ldj = N
     float* fields;   // hFieldCount x cap
-    float* vec;      // 4 x 64 scratch vectors
-    float* ywork;    // n x 64 forward-substitution scratch (lane = head)
+    float* vec;      // 4 x 64 scratch vectors, 16-byte aligned
+    float mass_inverse;   // 1 / diagonal of the mass factor, lane = row
+    bool mass_valid;
     float momentum, residual;
     bool failed;
+#ifdef NKH_SOLVER_PROFILE
+    mutable long long prof[10];
+    mutable uint32_t prof_count[4];
+#endif
     __device__ float& F(uint32_t field, uint32_t h) const { return fields[field * cap + h]; }
     __device__ uint32_t& U(uint32_t field, uint32_t h) const { return reinterpret_cast<uint32_t*>(fields)[field * cap + h]; }
 };
@@ -152,54 +178,112 @@ __device__ void head_response(const Tile& c, uint32_t h, float mx, float my, flo
                     c.F(hNormalBound, h), c.F(hMu1, h), c.F(hMu2, h), &f[1], &f[2], &cv[1], &cv[2], &cv[5]);
 }
 
-// FactorTileBlock + SolveTileBlock (:1622-1666): Cholesky of the n x n matrix in `a` (lane = row), then d = a^-1 g.
-// Returns false (uniformly) on a non-positive pivot.
-__device__ bool cholesky_solve(const Tile& c, float* a, float g, float* d_out) {
-    const uint32_t n = c.n, ld = c.ld, lane = c.lane;
+// A lane's value of `v` for a lane index that is a compile-time constant at every call site: a scalar lane read.
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+// FactorTileBlock (:1622-1645) on register rows: lane i holds row i of the symmetric matrix; on return its entries
+// k <= i are row i of the Cholesky factor.  Element (i, j) loses L_ik L_jk for k = 0, 1, ... in that order, one
+// product and one subtraction each, as the reference's serial inner loop does.  Uniform result: false on a bad pivot.
+template <int N>
+__device__ __forceinline__ bool factor_rows(uint32_t lane, float (&row)[N], float* inverse_out) {
     bool valid = true;
     float inverse = 0.0f;
-    for (uint32_t k = 0u; k < n; ++k) {
-        float value = 0.0f;
-        if (lane >= k && lane < n) {
-            value = a[lane * ld + k];
-            for (uint32_t j = 0u; j < k; ++j) value -= a[lane * ld + j] * a[k * ld + j];
-        }
-        const float pivot = __shfl(value, int(k), kWave);
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+        const float pivot = lane_value(row[k], k);
         valid = valid && pivot > 0.0f && pivot <= FLT_MAX;
         const float root = sqrtf(valid ? pivot : 1.0f);
         const float scale = 1.0f / root;
-        if (lane >= k && lane < n) a[lane * ld + k] = lane == k ? root : value * scale;
-        if (lane == k) inverse = scale;
-        __syncthreads();
+        row[k] = lane == uint32_t(k) ? root : row[k] * scale;
+        if (lane == uint32_t(k)) inverse = scale;
+#pragma unroll
+        for (int j = k + 1; j < N; ++j) row[j] -= row[k] * lane_value(row[k], j);
     }
+    *inverse_out = inverse;
+    return valid;
+}
+
+// SolveTileBlock (:1647-1666): forward with the factor's rows, backward with its columns (col[j] = L_j,lane).
+template <int N>
+__device__ __forceinline__ float substitute(uint32_t lane, const float (&row)[N], const float (&col)[N], float inverse, float g) {
+    float r = g;
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        const float y = lane_value(r * inverse, j);
+        r = lane == uint32_t(j) ? y : (lane > uint32_t(j) ? fmaf(-row[j], y, r) : r);
+    }
+#pragma unroll
+    for (int j = N - 1; j >= 0; --j) {
+        const float x = lane_value(r * inverse, j);
+        r = lane == uint32_t(j) ? x : (lane < uint32_t(j) ? fmaf(-col[j], x, r) : r);
+    }
+    return r;
+}
+
+template <int N>
+__device__ __forceinline__ void store_rows(float* a, uint32_t lane, const float (&row)[N]) {
+    if (lane < uint32_t(N)) {
+#pragma unroll
+        for (int k = 0; k < N; ++k) a[lane * (N + 1) + k] = row[k];
+    }
+}
+template <int N>
+__device__ __forceinline__ void load_rows(const float* a, uint32_t lane, float (&row)[N]) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) row[k] = lane < uint32_t(N) ? a[lane * (N + 1) + k] : 0.0f;
+}
+template <int N>
+__device__ __forceinline__ void load_columns(const float* a, uint32_t lane, float (&col)[N]) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) col[j] = lane < uint32_t(N) ? a[j * (N + 1) + lane] : 0.0f;
+}
+
+// Cholesky of the Newton Hessian held in `hrow`, then d = H^-1 g.  The factor passes through LDS once, for the
+// transposed read of the backward substitution.
+template <int N>
+__device__ bool cholesky_solve(const Tile& c, float (&hrow)[N], float g, float* d_out) {
+    float inverse = 0.0f;
+    const bool valid = factor_rows<N>(c.lane, hrow, &inverse);
     if (!valid) return false;
-    float r = lane < n ? g : 0.0f;
-    for (uint32_t j = 0u; j < n; ++j) {
-        const float y = __shfl(r * inverse, int(j), kWave);
-        if (lane == j) r = y;
-        else if (lane > j && lane < n) r = fmaf(-a[lane * ld + j], y, r);
-    }
-    for (uint32_t k = n; k > 0u; --k) {
-        const uint32_t j = k - 1u;
-        const float x = __shfl(r * inverse, int(j), kWave);
-        if (lane == j) r = x;
-        else if (lane < j) r = fmaf(-a[j * ld + lane], x, r);
-    }
-    *d_out = r;
+    store_rows<N>(c.hfac, c.lane, hrow);
+    __syncthreads();
+    float col[N];
+    load_columns<N>(c.hfac, c.lane, col);
+    *d_out = substitute<N>(c.lane, hrow, col, inverse, c.lane < c.n ? g : 0.0f);
+    __syncthreads();
     return true;
 }
 
-// SolveTileMass (:1898-1931)
-__device__ bool solve_tile_mass(const Tile& c, float force, float* direction) {
-    for (uint32_t e = c.lane; e < c.n * c.ld; e += kWave) c.hmat[e] = c.mass[e];
+// SolveTileMass (:1898-1931).  The mass matrix does not change during a solve, so its factor (same arithmetic as the
+// reference's per-call factorisation, hence the same numbers) is built once by factor_mass and reused here.
+template <int N>
+__device__ bool factor_mass(Tile& c, const float (&mrow)[N]) {
+    float row[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k) row[k] = mrow[k];
+    float inverse = 0.0f;
+    const bool valid = factor_rows<N>(c.lane, row, &inverse);
+    c.mass_inverse = inverse;
+    store_rows<N>(c.mfac, c.lane, row);
     __syncthreads();
-    return cholesky_solve(c, c.hmat, force, direction);
+    return valid;
+}
+template <int N>
+__device__ float solve_tile_mass(const Tile& c, float force) {
+    float row[N], col[N];
+    load_rows<N>(c.mfac, c.lane, row);
+    load_columns<N>(c.mfac, c.lane, col);
+    return substitute<N>(c.lane, row, col, c.mass_inverse, c.lane < c.n ? force : 0.0f);
 }
 
-// AssembleTileBlock (:1507-1618): lane i assembles row i of H = M + sum J^T C J in hmat and its force g_i.
-__device__ bool assemble_block(const Tile& c, float u, float free_v, float* force, float* inertia, bool* converged) {
-    const uint32_t n = c.n, ld = c.ld, lane = c.lane;
-    const bool coordinate = lane < n;
+// AssembleTileBlock (:1507-1618): lane i assembles row i of H = M + sum J^T C J in `hrow` and its force g_i.
+template <int N>
+__device__ bool assemble_block(const Tile& c, const float (&mrow)[N], float u, float free_v, float (&hrow)[N], float* force,
+                               float* inertia, bool* converged) {
+    const uint32_t lane = c.lane;
+    const bool coordinate = lane < c.n;
     const float difference = u - free_v;
     const float part = difference - u;
     const float difference_error = (u - (difference - part)) + (-free_v - part);
@@ -225,32 +309,45 @@ __device__ bool assemble_block(const Tile& c, float u, float free_v, float* forc
         c.U(hContrib, h) = contributes ? 1u : 0u;
     }
     __syncthreads();
+    // Padded columns (k >= n) hold exact zeros in the mass row, the vectors and the Jacobian rows: their terms add
+    // nothing to any of the sums below.
     TileSum inertial{0.0f, 0.0f};
     float scale = 0.0f;
-    if (coordinate)
-        for (uint32_t k = 0u; k < n; ++k) {
-            const float mass = c.mass[lane * ld + k];
-            c.hmat[lane * ld + k] = mass;
-            tile_add_product(inertial, mass, dvec[k]);
-            tile_add_product(inertial, mass, evec[k]);
-            scale += fabsf(mass) * fabsf(dvec[k]);
+    const float4* d4 = reinterpret_cast<const float4*>(dvec);
+    const float4* e4 = reinterpret_cast<const float4*>(evec);
+#pragma unroll
+    for (int q = 0; q < N / 4; ++q) {
+        const float4 dv = d4[q], ev = e4[q];
+        const float dk[4] = {dv.x, dv.y, dv.z, dv.w}, ek[4] = {ev.x, ev.y, ev.z, ev.w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float mass = mrow[4 * q + t];
+            hrow[4 * q + t] = mass;
+            tile_add_product(inertial, mass, dk[t]);
+            tile_add_product(inertial, mass, ek[t]);
+            scale += fabsf(mass) * fabsf(dk[t]);
         }
+    }
     TileSum g{-inertial.value, -inertial.error};
     for (uint32_t h = 0u; h < c.heads; ++h) {
         if (c.U(hContrib, h) == 0u) continue;
-        if (!coordinate) continue;
-        const float* j0r = c.jac + (3u * h) * c.ldj;
-        const float j0 = j0r[lane];
+        const float* j0r = c.jac + (3u * h) * uint32_t(N);
+        const float j0 = coordinate ? j0r[lane] : 0.0f;
         const float fx = c.F(hF, h), cxx = c.F(hC, h);
         tile_add_product(g, j0, fx);
         scale += fabsf(j0) * c.F(hNoise, h);
+        const float4* r0 = reinterpret_cast<const float4*>(j0r);
         if (c.U(hAxes, h) == 1u) {
             const float a0 = j0 * cxx;
-            for (uint32_t k = 0u; k < n; ++k) c.hmat[lane * ld + k] += a0 * j0r[k];
+#pragma unroll
+            for (int q = 0; q < N / 4; ++q) {
+                const float4 x0 = r0[q];
+                hrow[4 * q] += a0 * x0.x; hrow[4 * q + 1] += a0 * x0.y; hrow[4 * q + 2] += a0 * x0.z; hrow[4 * q + 3] += a0 * x0.w;
+            }
             continue;
         }
-        const float* j1r = j0r + c.ldj, *j2r = j0r + 2u * c.ldj;
-        const float j1 = j1r[lane], j2 = j2r[lane];
+        const float* j1r = j0r + N, *j2r = j0r + 2 * N;
+        const float j1 = coordinate ? j1r[lane] : 0.0f, j2 = coordinate ? j2r[lane] : 0.0f;
         const float cyy = c.F(hC + 1, h), czz = c.F(hC + 2, h), cxy = c.F(hC + 3, h), cxz = c.F(hC + 4, h), cyz = c.F(hC + 5, h);
         tile_add_product(g, j1, c.F(hF + 1, h));
         tile_add_product(g, j2, c.F(hF + 2, h));
@@ -258,58 +355,95 @@ __device__ bool assemble_block(const Tile& c, float u, float free_v, float* forc
         const float a0 = (j0 * cxx + j1 * cxy) + j2 * cxz;
         const float a1 = (j1 * cyy + j2 * cyz) + j0 * cxy;
         const float a2 = (j2 * czz + j1 * cyz) + j0 * cxz;
-        for (uint32_t k = 0u; k < n; ++k) c.hmat[lane * ld + k] += a0 * j0r[k] + a1 * j1r[k] + a2 * j2r[k];
+        const float4* r1 = reinterpret_cast<const float4*>(j1r);
+        const float4* r2 = reinterpret_cast<const float4*>(j2r);
+#pragma unroll
+        for (int q = 0; q < N / 4; ++q) {
+            const float4 x0 = r0[q], x1 = r1[q], x2 = r2[q];
+            hrow[4 * q] += a0 * x0.x + a1 * x1.x + a2 * x2.x;
+            hrow[4 * q + 1] += a0 * x0.y + a1 * x1.y + a2 * x2.y;
+            hrow[4 * q + 2] += a0 * x0.z + a1 * x1.z + a2 * x2.z;
+            hrow[4 * q + 3] += a0 * x0.w + a1 * x1.w + a2 * x2.w;
+        }
     }
     *force = coordinate ? g.value + g.error : 0.0f;
     *inertia = coordinate ? inertial.value + inertial.error : 0.0f;
     bool finite = isfinite(*force);
-    if (coordinate)
-        for (uint32_t k = 0u; k < n; ++k) {
-            const float entry = c.hmat[lane * ld + k];
+    const float4* u4 = reinterpret_cast<const float4*>(uvec);
+#pragma unroll
+    for (int q = 0; q < N / 4; ++q) {
+        const float4 uv = u4[q];
+        const float uk[4] = {uv.x, uv.y, uv.z, uv.w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float entry = hrow[4 * q + t];
             finite = finite && isfinite(entry);
-            scale += fabsf(entry) * uvec[k];
+            scale += fabsf(entry) * uk[t];
         }
+    }
     *converged = __all(!coordinate || fabsf(*force) <= kRoundings * FLT_EPSILON * scale);
-    const bool ok = __all(finite);
+    const bool ok = __all(!coordinate || finite);
     __syncthreads();
     return ok;
 }
 
 enum Failure : uint32_t { kFailNone = 0u, kFailEquation, kFailFactor, kFailDirection, kFailCandidate };
 
-// TileNewtonDirection (:1935-1992), narrow form
-__device__ Failure newton_direction(const Tile& c, float u, float free_v, float* force, float* inertia, float* d, bool* converged) {
-    if (!assemble_block(c, u, free_v, force, inertia, converged)) return kFailEquation;
+// TileNewtonDirection (:1935-1992), narrow form.  The reference re-assembles the block after the mass-normalised
+// convergence test because its mass factor overwrites the Hessian storage; here the two live apart and the
+// assembled row, force and inertia (which the second assembly would reproduce bit for bit) are simply kept.
+template <int N>
+__device__ Failure newton_direction(const Tile& c, const float (&mrow)[N], float u, float free_v, float* force, float* inertia,
+                                    float* d, bool* converged) {
+    PROF_COUNT(c, 0);
+    float hrow[N];
+    PROF_BEGIN(c, 1);
+    const bool assembled = assemble_block<N>(c, mrow, u, free_v, hrow, force, inertia, converged);
+    PROF_END(c, 1);
+    if (!assembled) return kFailEquation;
     if (*converged && c.tolerance > 0.0f) {
-        // the Hessian is not needed again this step, so the mass factor may overwrite it
-        float direction = 0.0f;
-        if (!solve_tile_mass(c, *force, &direction)) return kFailFactor;
+        if (!c.mass_valid) return kFailFactor;
+        PROF_BEGIN(c, 3);
+        const float direction = solve_tile_mass<N>(c, *force);
+        PROF_END(c, 3);
         *d = direction;
         *converged = __all(c.lane >= c.n || fabsf(direction) < c.tolerance);
         if (*converged) return kFailNone;
-        bool rounded = false;
-        if (!assemble_block(c, u, free_v, force, inertia, &rounded)) return kFailEquation;
     }
     if (*converged) return kFailNone;
-    if (!cholesky_solve(c, c.hmat, *force, d)) return kFailFactor;
+    PROF_BEGIN(c, 2);
+    const bool factored = cholesky_solve<N>(c, hrow, *force, d);
+    PROF_END(c, 2);
+    if (!factored) return kFailFactor;
     return kFailNone;
 }
 
-// TileRowSteps (:2018-2044): step = J d per head axis by serial fused multiply-adds, lane = head
+// TileRowSteps (:2018-2044): step = J d per head axis by serial fused multiply-adds, lane = head.  The Jacobian row
+// and the direction come in as 16-byte words; padded columns are zeros on both sides.
+template <int N>
+__device__ __forceinline__ float row_dot_fma(const float* jrow, const float* dvec) {
+    const float4* j4 = reinterpret_cast<const float4*>(jrow);
+    const float4* d4 = reinterpret_cast<const float4*>(dvec);
+    float value = 0.0f;
+#pragma unroll
+    for (int q = 0; q < N / 4; ++q) {
+        const float4 j = j4[q], d = d4[q];
+        value = fmaf(j.x, d.x, value); value = fmaf(j.y, d.y, value); value = fmaf(j.z, d.z, value); value = fmaf(j.w, d.w, value);
+    }
+    return value;
+}
+template <int N>
 __device__ void row_steps(const Tile& c, float d) {
     float* dvec = c.vec;
-    dvec[c.lane] = d;
+    dvec[c.lane] = c.lane < c.n ? d : 0.0f;
     __syncthreads();
     for (uint32_t h = c.lane; h < c.heads; h += kWave) {
         if (c.U(hOwned, h) == 0u) continue;
-        const float* j = c.jac + (3u * h) * c.ldj;
+        const float* j = c.jac + (3u * h) * uint32_t(N);
         const uint32_t axes = c.U(hAxes, h);
-        for (uint32_t axis = 0u; axis < 3u; ++axis) {
-            float value = 0.0f;
-            if (axis < axes)
-                for (uint32_t i = 0u; i < c.n; ++i) value = fmaf(j[axis * c.ldj + i], dvec[i], value);
-            c.F(hStep + axis, h) = value;
-        }
+        c.F(hStep, h) = row_dot_fma<N>(j, dvec);
+        c.F(hStep + 1, h) = axes > 1u ? row_dot_fma<N>(j + N, dvec) : 0.0f;
+        c.F(hStep + 2, h) = axes > 2u ? row_dot_fma<N>(j + 2 * N, dvec) : 0.0f;
     }
     __syncthreads();
 }
@@ -317,6 +451,7 @@ __device__ void row_steps(const Tile& c, float d) {
 // TileLineDerivatives (:2048-2086)
 __device__ void line_derivatives(const Tile& c, float alpha, float inertial_slope, float inertial_curvature, float* slope,
                                  float* curvature, float* magnitude) {
+    PROF_COUNT(c, 1);
     TileSum row_slope{0.0f, 0.0f};
     float row_curvature = 0.0f, row_magnitude = 0.0f;
     for (uint32_t h = c.lane; h < c.heads; h += kWave) {
@@ -376,19 +511,25 @@ __device__ void apply_moves(const Tile& c, float alpha) {
 }
 
 // mass_step_i = sum_k M_ik d_k in coordinate order (:2177-2187, 2228-2238)
-__device__ float mass_times(const Tile& c, float d) {
+template <int N>
+__device__ float mass_times(const Tile& c, const float (&mrow)[N], float d) {
     float* dvec = c.vec + 192;
     dvec[c.lane] = d;
     __syncthreads();
     float out = 0.0f;
-    if (c.lane < c.n)
-        for (uint32_t k = 0u; k < c.n; ++k) out += c.mass[c.lane * c.ld + k] * dvec[k];
+    const float4* d4 = reinterpret_cast<const float4*>(dvec);
+#pragma unroll
+    for (int q = 0; q < N / 4; ++q) {
+        const float4 dv = d4[q];
+        out += mrow[4 * q] * dv.x; out += mrow[4 * q + 1] * dv.y; out += mrow[4 * q + 2] * dv.z; out += mrow[4 * q + 3] * dv.w;
+    }
     __syncthreads();
-    return out;
+    return c.lane < c.n ? out : 0.0f;
 }
 
 // DescendTileBlock (:2145-2301).  `u` is lane i's block coordinate; `has_free` is false in the position pass.
-__device__ void descend_block(Tile& c, float* u_io, float free_in, bool has_free, DataView d) {
+template <int N>
+__device__ void descend_block(Tile& c, const float (&mrow)[N], float* u_io, float free_in, bool has_free, DataView d) {
     const uint32_t lane = c.lane, n = c.n;
     const bool coordinate = lane < n;
     for (uint32_t h = lane; h < c.heads; h += kWave) {   // StartTileBlock (:1386-1397)
@@ -402,12 +543,12 @@ __device__ void descend_block(Tile& c, float* u_io, float free_in, bool has_free
     float u = start;
     if (c.iteration == 0u && has_free) {   // first-sweep segment search (:2165-2209)
         const float dd = coordinate ? free_v - u : 0.0f;
-        const float mass_step = mass_times(c, dd);
+        const float mass_step = mass_times<N>(c, mrow, dd);
         TileSum curvature{0.0f, 0.0f};
         if (coordinate) tile_add_product(curvature, dd, mass_step);
         const float inertial_curvature = wave_total(curvature);
         if (inertial_curvature > 0.0f && isfinite(inertial_curvature)) {
-            row_steps(c, dd);
+            row_steps<N>(c, dd);
             const float alpha = search_line(c, -inertial_curvature, inertial_curvature);
             if (alpha > 0.0f) {
                 u = fmaf(alpha, dd, u);
@@ -420,11 +561,13 @@ __device__ void descend_block(Tile& c, float* u_io, float free_in, bool has_free
     for (uint32_t step = 0u; step < kNewtonSteps; ++step) {
         float force = 0.0f, inertia = 0.0f, dd = 0.0f;
         bool converged = false;
-        failure = newton_direction(c, u, free_v, &force, &inertia, &dd, &converged);
+        failure = newton_direction<N>(c, mrow, u, free_v, &force, &inertia, &dd, &converged);
         if (converged) primal = 0.0f;
         if (failure != kFailNone || converged) break;
         if (!coordinate) dd = 0.0f;
-        const float mass_step = mass_times(c, dd);
+        PROF_BEGIN(c, 8);
+        const float mass_step = mass_times<N>(c, mrow, dd);
+        PROF_END(c, 8);
         TileSum decrement{0, 0}, slope{0, 0}, curvature{0, 0};
         if (coordinate) {
             tile_add_product(decrement, force, dd);
@@ -436,8 +579,12 @@ __device__ void descend_block(Tile& c, float* u_io, float free_in, bool has_free
         const float inertial_curvature = wave_total(curvature);
         if (!isfinite(total_decrement) || !isfinite(inertial_slope) || !isfinite(inertial_curvature)) { failure = kFailDirection; break; }
         if (!(total_decrement > 0.0f)) break;
-        row_steps(c, dd);
+        PROF_BEGIN(c, 4);
+        row_steps<N>(c, dd);
+        PROF_END(c, 4);
+        PROF_BEGIN(c, 5);
         const float alpha = search_line(c, inertial_slope, inertial_curvature);
+        PROF_END(c, 5);
         const float after = fmaf(alpha, dd, u);
         const bool rounded = __all(!coordinate || after == u);
         if (!__all(!coordinate || isfinite(after))) { failure = kFailCandidate; break; }
@@ -467,8 +614,9 @@ __device__ void descend_block(Tile& c, float* u_io, float free_in, bool has_free
 }
 
 // MeasureTilePrimal (:2378-2489): the mass-normalised momentum balance in double
-__device__ void measure_primal(Tile& c, float* velocity_io, float free_v, const float* lambda_env, uint32_t R, bool reconstruct,
-                               DataView d) {
+template <int N>
+__device__ void measure_primal(Tile& c, const float (&mrow)[N], float* velocity_io, float free_v, const float* lambda_env, uint32_t R,
+                               bool reconstruct, DataView d) {
     const uint32_t lane = c.lane, n = c.n;
     const bool coordinate = lane < n;
     float* dvec = c.vec;
@@ -476,8 +624,8 @@ __device__ void measure_primal(Tile& c, float* velocity_io, float free_v, const 
     c.vec[64 + lane] = coordinate ? free_v : 0.0f;
     __syncthreads();
     double balance = 0.0;
-    if (coordinate)
-        for (uint32_t j = 0u; j < n; ++j) balance -= double(c.mass[lane * c.ld + j]) * (double(dvec[j]) - c.vec[64 + j]);
+#pragma unroll
+    for (int j = 0; j < N; ++j) balance -= double(mrow[j]) * (double(dvec[j]) - c.vec[64 + j]);   // padded terms are exact zeros
     for (uint32_t h = 0u; h < c.heads; ++h) {
         if (c.U(hOwned, h) == 0u) continue;
         const uint32_t local = c.U(hSlot, h) - c.env * R, stride = c.U(hStride, h), axes = c.U(hAxes, h);
@@ -497,7 +645,10 @@ __device__ void measure_primal(Tile& c, float* velocity_io, float free_v, const 
     const bool finite = __all(!coordinate || fabs(balance) <= double(FLT_MAX));
     Failure failure = finite ? kFailNone : kFailEquation;
     float direction = 0.0f;
-    if (failure == kFailNone && !solve_tile_mass(c, force, &direction)) failure = kFailFactor;
+    if (failure == kFailNone) {
+        if (c.mass_valid) direction = solve_tile_mass<N>(c, force);
+        else failure = kFailFactor;
+    }
     float residual = failure == kFailNone ? 0.0f : FLT_MAX;
     if (failure != kFailNone && lane == 0u) d.env_status[c.env] |= kEnvStatusSolverFailure;
     if (failure == kFailNone && coordinate) residual = fmaxf(residual, isfinite(direction) ? fabsf(direction) : FLT_MAX);
@@ -511,19 +662,25 @@ __device__ void measure_primal(Tile& c, float* velocity_io, float free_v, const 
 }
 
 // InitializeTileResiduals (:890-930) on the staged rows: residual = fl(rhs dt) - J u, products summed in coordinate order
+template <int N>
 __device__ void initialize_residuals(const Tile& c, float velocity, const float* urows, float dt) {
     float* dvec = c.vec;
     dvec[c.lane] = c.lane < c.n ? velocity : 0.0f;
     __syncthreads();
+    const float4* d4 = reinterpret_cast<const float4*>(dvec);
     for (uint32_t h = c.lane; h < c.heads; h += kWave) {
         const uint32_t slot = c.U(hSlot, h), stride = c.U(hStride, h), axes = c.U(hAxes, h);
         for (uint32_t axis = 0u; axis < 3u; ++axis) {
             float residual = 0.0f;
             if (axis < axes) {
                 const float rhs = urows[size_t{slot + axis * stride} * kRowWords + 4u];
-                const float* j = c.jac + (3u * h + axis) * c.ldj;
+                const float4* j4 = reinterpret_cast<const float4*>(c.jac + (3u * h + axis) * uint32_t(N));
                 float along = 0.0f;
-                for (uint32_t i = 0u; i < c.n; ++i) along = along + j[i] * dvec[i];
+#pragma unroll
+                for (int q = 0; q < N / 4; ++q) {
+                    const float4 j = j4[q], dv = d4[q];
+                    along = along + j.x * dv.x; along = along + j.y * dv.y; along = along + j.z * dv.z; along = along + j.w * dv.w;
+                }
                 residual = rhs * dt - along;
             }
             c.F(hRes + axis, h) = residual;
@@ -592,8 +749,8 @@ __device__ void update_duals(const Tile& c, float* lambda_env, uint32_t R, const
             const float rate = -residual.x + compliance * physical.x;
             const float violation = physical.x > 0.0f ? fabsf(rate) : fmaxf(-rate, 0.0f);
             const float value = normal_row ? fmaxf(step_normal, violation) : step_normal;
-            const uint32_t kind = normal_row ? 0u : 2u;
-            steps[kind] = max(steps[kind], residual_bits(value));
+            if (normal_row) steps[0] = max(steps[0], residual_bits(value));
+            else steps[2] = max(steps[2], residual_bits(value));
         } else {
             if (commit) {
                 c.F(hRelaxStep, h) = rstep.x; c.F(hRelaxStep + 1, h) = rstep.y; c.F(hRelaxStep + 2, h) = rstep.z;
@@ -657,25 +814,38 @@ __device__ void update_duals(const Tile& c, float* lambda_env, uint32_t R, const
     __syncthreads();
 }
 
+__host__ __device__ inline uint32_t PaddedWidth(uint32_t n) { return (n + 3u) & ~3u; }
+__host__ __device__ inline uint32_t FactorRegionFloats(uint32_t n) {
+    const uint32_t N = PaddedWidth(n);
+    return 2u * N * (N + 1u);   // a multiple of 4 since N is
+}
 __host__ __device__ inline uint32_t SolverLdsFloats(uint32_t n, uint32_t cap) {
-    const uint32_t ld = n + 1u, ldj = n | 1u;
-    return 2u * n * ld + 3u * cap * ldj + hFieldCount * cap + 256u + n * 64u;
+    const uint32_t N = PaddedWidth(n);
+    return FactorRegionFloats(n) + 3u * cap * N + ((hFieldCount * cap + 3u) & ~3u) + 256u;
 }
 
 // DescendTile (:2941-3087)
-__global__ void __launch_bounds__(kWave) BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint32_t cap) {
-    extern __shared__ float lds[];
+template <int N>
+__global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(N <= 36 ? 2 : 1, N <= 36 ? 2 : 1)))
+BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint32_t cap) {
+    extern __shared__ __align__(16) float lds[];
     const uint32_t env = blockIdx.x, lane = threadIdx.x;
     const uint32_t R = p.rows_per_env, md = p.max_dof, n = m.dof, nl = m.links_per_env, S = p.contact_slots_per_env;
     Tile c;
-    c.env = env; c.lane = lane; c.n = n; c.ld = n + 1u; c.ldj = n | 1u; c.cap = cap; c.heads = 0u; c.iteration = 0u;
+    c.env = env; c.lane = lane; c.n = n; c.ld = uint32_t(N) + 1u; c.ldj = uint32_t(N); c.cap = cap; c.heads = 0u; c.iteration = 0u;
     c.tolerance = p.velocity_tolerance; c.failed = false; c.momentum = 0.0f; c.residual = 0.0f;
-    c.mass = lds;
-    c.hmat = c.mass + n * c.ld;
-    c.jac = c.hmat + n * c.ld;
+    c.mass_inverse = 0.0f; c.mass_valid = false;
+#ifdef NKH_SOLVER_PROFILE
+    for (int i = 0; i < 10; ++i) c.prof[i] = 0;
+    for (int i = 0; i < 4; ++i) c.prof_count[i] = 0u;
+#endif
+    PROF_BEGIN(c, 9);
+    PROF_BEGIN(c, 0);
+    c.mfac = lds;
+    c.hfac = c.mfac + uint32_t(N) * c.ld;
+    c.jac = lds + FactorRegionFloats(n);
     c.fields = c.jac + 3u * cap * c.ldj;
-    c.vec = c.fields + hFieldCount * cap;
-    c.ywork = c.vec + 256u;
+    c.vec = c.fields + ((hFieldCount * cap + 3u) & ~3u);
     const bool coordinate = lane < n;
     const float* urows = d.urows;
     float* lambda_env = d.lambda + size_t{env} * R;
@@ -690,8 +860,6 @@ __global__ void __launch_bounds__(kWave) BlockDescentTileKernel(ModelView m, Dat
         free_v = value;
         velocity = value + (isfinite(carried) ? carried : 0.0f);
     }
-    // StageTileMass (:2127-2142)
-    for (uint32_t e = lane; e < n * n; e += kWave) c.mass[(e / n) * c.ld + e % n] = d.m[size_t{env} * md * md + size_t{e / n} * md + e % n];
     // ListTileHeads (:1250-1296): active rows that are not block tangents, in slot order
     const uint32_t previous = d.contact_row_extent[2u * env], current = d.contact_row_extent[2u * env + 1u];
     const uint32_t bound = previous == 0u || current == 0u ? p.contact_rows_per_env : min(max(previous, current) - 1u, p.contact_rows_per_env);
@@ -734,12 +902,51 @@ __global__ void __launch_bounds__(kWave) BlockDescentTileKernel(ModelView m, Dat
                 if (kind_a == kSideArtic) value += d.chain_jacobian[size_t{rs} * md + lane];
                 if (kind_b == kSideArtic) value += d.chain_jacobian_b[size_t{rs} * md + lane];
             }
-            if (lane < c.ldj) c.jac[(3u * h + axis) * c.ldj + lane] = value;
+            if (lane < c.ldj) c.jac[(3u * h + axis) * c.ldj + lane] = value;   // padded columns hold zeros
         }
     }
     __syncthreads();
-    // InitializeTileHead (:743-797), lane = head; J M^-1 J^T through the stored LDL^T factor (TileInertialResponse :709-739)
-    const float* factor = d.m_factor + size_t{env} * md * md;
+    // TileInertialResponse (:709-739): J M^-1 J^T of every head's first row through the stored LDL^T factor
+    // (ForwardMass + MassDot, articulation_mass.cuh:414-431).  lane = DoF: the unit-lower factor row sits in
+    // registers with zeros from the diagonal on, each y_j travels as a scalar lane read, so row i subtracts
+    // L_ij y_j for j = 0, 1, ... exactly as the serial loop does; the ordered sum of y_i^2 / D_i follows the same way.
+    {
+        const float* factor = d.m_factor + size_t{env} * md * md;
+        for (uint32_t e = lane; e < n * n; e += kWave) c.hfac[(e / n) * c.ld + e % n] = factor[size_t{e / n} * md + e % n];
+        __syncthreads();
+        float lrow[N];
+#pragma unroll
+        for (int k = 0; k < N; ++k) lrow[k] = coordinate && uint32_t(k) < lane ? c.hfac[lane * c.ld + k] : 0.0f;
+        const float pivot = coordinate ? c.hfac[lane * c.ld + lane] : 1.0f;
+        __syncthreads();
+        for (uint32_t h = 0u; h < heads; ++h) {
+            const uint32_t slot = c.U(hSlot, h);
+            const float* row = urows + size_t{slot} * kRowWords;
+            const uint32_t kind_a = __float_as_uint(row[10]), index_a = __float_as_uint(row[11]);
+            const uint32_t kind_b = __float_as_uint(row[18]), index_b = __float_as_uint(row[19]);
+            const bool shared = kind_a == kind_b && index_a == index_b;
+            float shares[2] = {0.0f, 0.0f};
+            for (uint32_t side = 0u; side < (shared ? 1u : 2u); ++side) {
+                float contribution = 0.0f;
+                if ((side == 0u ? kind_a : kind_b) == kSideArtic) {
+                    float a = 0.0f;
+                    if (coordinate) {
+                        a = (side == 0u ? d.chain_jacobian : d.chain_jacobian_b)[size_t{slot} * md + lane];
+                        if (shared) a += d.chain_jacobian_b[size_t{slot} * md + lane];
+                    }
+#pragma unroll
+                    for (int j = 0; j < N; ++j) a -= lrow[j] * lane_value(a, j);
+                    const float term = coordinate ? a * a / pivot : 0.0f;
+#pragma unroll
+                    for (int i = 0; i < N; ++i) contribution += lane_value(term, i);
+                }
+                shares[side] = contribution;
+            }
+            if (lane == 0u) { c.F(hRes, h) = shares[0]; c.F(hRes + 1, h) = shares[1]; }
+        }
+        __syncthreads();
+    }
+    // InitializeTileHead (:743-797), lane = head
     for (uint32_t base = 0u; base < heads; base += kWave) {
         const uint32_t h = base + lane;
         if (h < heads) {
@@ -747,31 +954,10 @@ __global__ void __launch_bounds__(kWave) BlockDescentTileKernel(ModelView m, Dat
             const float* row = urows + size_t{slot} * kRowWords;
             const uint32_t flags = __float_as_uint(row[0]), stride = __float_as_uint(row[2]);
             const uint32_t axes = (flags & kRowBlockNormal) != 0u ? 3u : 1u;
-            const uint32_t kind_a = __float_as_uint(row[10]), index_a = __float_as_uint(row[11]);
-            const uint32_t kind_b = __float_as_uint(row[18]), index_b = __float_as_uint(row[19]);
-            const bool shared = kind_a == kind_b && index_a == index_b;
-            float shares[2] = {0.0f, 0.0f}, response = 0.0f;
-            bool valid = true;
-            for (uint32_t side = 0u; side < (shared ? 1u : 2u); ++side) {
-                float contribution = 0.0f;
-                if ((side == 0u ? kind_a : kind_b) == kSideArtic) {
-                    // ForwardMass + MassDot over max_dof (articulation_mass.cuh:414-431); y lives in LDS, one column per lane
-                    const float* v = (side == 0u ? d.chain_jacobian : d.chain_jacobian_b) + size_t{slot} * md;
-                    const float* extra = shared ? d.chain_jacobian_b + size_t{slot} * md : nullptr;
-                    for (uint32_t i = 0u; i < md; ++i) {
-                        float a = v[i] + (extra == nullptr ? 0.0f : extra[i]);
-                        for (uint32_t j = 0u; j < i; ++j) a -= factor[size_t{i} * md + j] * c.ywork[j * 64u + lane];
-                        c.ywork[i * 64u + lane] = a;
-                    }
-                    for (uint32_t i = 0u; i < md; ++i) {
-                        const float y = c.ywork[i * 64u + lane];
-                        contribution += y * y / factor[size_t{i} * md + i];
-                    }
-                }
-                valid = valid && contribution >= 0.0f && isfinite(contribution);
-                response += contribution;
-                shares[side] = contribution;
-            }
+            const uint32_t kind_a = __float_as_uint(row[10]), kind_b = __float_as_uint(row[18]);
+            const float shares[2] = {c.F(hRes, h), c.F(hRes + 1, h)};
+            const bool valid = shares[0] >= 0.0f && isfinite(shares[0]) && shares[1] >= 0.0f && isfinite(shares[1]);
+            float response = shares[0] + shares[1];
             const float coupling = shares[0] * shares[1], largest = fmaxf(shares[0], shares[1]);
             if (!(valid && isfinite(response))) response = nanf("");
             const float coupled = coupling > 0.0f ? (response + sqrtf(response * response + 12.0f * coupling)) / (6.0f * coupling) : FLT_MAX;
@@ -800,7 +986,18 @@ __global__ void __launch_bounds__(kWave) BlockDescentTileKernel(ModelView m, Dat
         }
     }
     __syncthreads();
-    initialize_residuals(c, velocity, urows, p.dt);
+    // StageTileMass (:2127-2142): the mass rows go to registers through a coalesced pass over LDS (the head setup's
+    // scratch is dead by now); rows and columns n..N-1 are those of the identity.  Then the one factorisation.
+    float mrow[N];
+    for (uint32_t e = lane; e < n * n; e += kWave) c.hfac[(e / n) * c.ld + e % n] = d.m[size_t{env} * md * md + size_t{e / n} * md + e % n];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < N; ++k)
+        mrow[k] = coordinate && uint32_t(k) < n ? c.hfac[lane * c.ld + k] : (lane == uint32_t(k) && lane < uint32_t(N) ? 1.0f : 0.0f);
+    __syncthreads();
+    c.mass_valid = factor_mass<N>(c, mrow);
+    initialize_residuals<N>(c, velocity, urows, p.dt);
+    PROF_END(c, 0);
     float residual4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     uint32_t sweeps = 0u;
     DualMomentum momentum{1.0f, 0.0f};
@@ -808,18 +1005,23 @@ __global__ void __launch_bounds__(kWave) BlockDescentTileKernel(ModelView m, Dat
     while (sweeps < p.iterations) {
         c.iteration = sweeps++;
         c.momentum = 0.0f; c.residual = 0.0f;
-        descend_block(c, &velocity, free_v, true, d);
+        PROF_COUNT(c, 2);
+        descend_block<N>(c, mrow, &velocity, free_v, true, d);
         float rowsr[3];
+        PROF_BEGIN(c, 6);
         update_duals(c, lambda_env, R, urows, &momentum, true, true, rowsr);
+        PROF_END(c, 6);
+        PROF_BEGIN(c, 7);
         if (sweeps == p.iterations || fmaxf(fmaxf(rowsr[0], rowsr[1]), fmaxf(rowsr[2], c.residual)) < tol)
-            measure_primal(c, &velocity, free_v, lambda_env, R, false, d);
+            measure_primal<N>(c, mrow, &velocity, free_v, lambda_env, R, false, d);
+        PROF_END(c, 7);
         if (fmaxf(fmaxf(rowsr[0], rowsr[1]), rowsr[2]) < tol && c.residual >= tol && c.residual < FLT_MAX) {
-            measure_primal(c, &velocity, free_v, lambda_env, R, true, d);
+            measure_primal<N>(c, mrow, &velocity, free_v, lambda_env, R, true, d);
             if (c.residual < FLT_MAX) {
-                initialize_residuals(c, velocity, urows, p.dt);
+                initialize_residuals<N>(c, velocity, urows, p.dt);
                 update_duals(c, lambda_env, R, urows, nullptr, true, false, rowsr);
                 c.residual = 0.0f;
-                measure_primal(c, &velocity, free_v, lambda_env, R, false, d);
+                measure_primal<N>(c, mrow, &velocity, free_v, lambda_env, R, false, d);
             }
         }
         residual4[0] = rowsr[0]; residual4[1] = rowsr[1]; residual4[2] = rowsr[2]; residual4[3] = c.residual;
@@ -830,6 +1032,13 @@ __global__ void __launch_bounds__(kWave) BlockDescentTileKernel(ModelView m, Dat
         d.solver_residual[size_t{env} * 4u + lane] =
             lane == 0u ? residual4[0] : lane == 1u ? residual4[1] : lane == 2u ? residual4[2] : residual4[3];
     if (lane == 0u) d.vbd_velocity_sweep_count[env] = sweeps;
+#ifdef NKH_SOLVER_PROFILE
+    PROF_END(c, 9);
+    if (lane == 0u) {
+        for (int i = 0; i < 10; ++i) d.solver_penalty[size_t{env} * R + i] = float(c.prof[i]);
+        for (int i = 0; i < 4; ++i) d.solver_penalty[size_t{env} * R + 10 + i] = float(c.prof_count[i]);
+    }
+#endif
     // the block velocities persist for the next solve's carried start
     if (lane < md) {
         d.solver_velocity[size_t{env} * md + lane] = coordinate ? velocity : 0.0f;
@@ -911,7 +1120,7 @@ __global__ void __launch_bounds__(kWave) BlockDescentTileKernel(ModelView m, Dat
             const uint32_t positions = 1u;   // no head couples two moving blocks here, so one solve (:2716)
             for (uint32_t iteration = 0u; iteration < positions; ++iteration) {
                 c.iteration = sweeps + iteration;
-                descend_block(c, &pseudo, 0.0f, false, d);
+                descend_block<N>(c, mrow, &pseudo, 0.0f, false, d);
             }
         }
         // FinishTilePositions (:2720-2744)
@@ -931,10 +1140,21 @@ uint32_t SolverHeadCapacity(const ModelView& m, uint32_t slots, size_t lds_budge
     return 0u;
 }
 
+namespace {
+using SolverKernel = void (*)(ModelView, DataView, BlockDescentSolveParams, uint32_t);
+// One instantiation per padded width.
+const SolverKernel kSolverKernels[16] = {
+    BlockDescentTileKernel<4>, BlockDescentTileKernel<8>, BlockDescentTileKernel<12>, BlockDescentTileKernel<16>,
+    BlockDescentTileKernel<20>, BlockDescentTileKernel<24>, BlockDescentTileKernel<28>, BlockDescentTileKernel<32>,
+    BlockDescentTileKernel<36>, BlockDescentTileKernel<40>, BlockDescentTileKernel<44>, BlockDescentTileKernel<48>,
+    BlockDescentTileKernel<52>, BlockDescentTileKernel<56>, BlockDescentTileKernel<60>, BlockDescentTileKernel<64>};
+}  // namespace
+
 void InitSolverKernels() {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(BlockDescentTileKernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              160 * 1024);
-    (void)hipGetLastError();
+    for (SolverKernel kernel : kSolverKernels) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipGetLastError();
+    }
 }
 
 Status OpBlockDescentSolve(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
@@ -947,7 +1167,7 @@ Status OpBlockDescentSolve(const ModelView& m, const DataView& d, const void* pa
     const uint32_t cap = SolverHeadCapacity(m, p->contact_slots_per_env == 0u ? 1u : p->contact_slots_per_env, budget);
     if (cap == 0u) return Status::InvalidArgument;
     const size_t lds = size_t{SolverLdsFloats(m.dof, cap)} * sizeof(float);
-    hipLaunchKernelGGL(BlockDescentTileKernel, dim3(p->env_count), dim3(kWave), lds, stream, m, d, *p, cap);
+    hipLaunchKernelGGL(kSolverKernels[PaddedWidth(m.dof) / 4u - 1u], dim3(p->env_count), dim3(kWave), lds, stream, m, d, *p, cap);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 
