@@ -106,17 +106,21 @@ __device__ __forceinline__ float cone_argument(float dual, float rho, float mu, 
     const float sum_low = (dd - (sum - t_part)) + (t - t_part);
     return sum + (sum_low + d_low + t_low);
 }
-// augmented_row.hpp:321-348; curvature entries yy, zz, yz
-__device__ void tangent_impulse(V3 dual, float rho, float res_y, float res_z, float normal_impulse, float mu_first, float mu_second,
+// augmented_row.hpp:321-348; curvature entries yy, zz, yz.  The friction ratios depend on the row only, so callers
+// that evaluate one row many times compute them once (tangent_ratios) and pass them in.
+struct TangentRatios { float mu_y, mu_z, scale; };
+__device__ __forceinline__ TangentRatios tangent_ratios(float mu_first, float mu_second) {
+    const float scale = fmaxf(mu_first, mu_second);
+    return TangentRatios{mu_first <= 0.0f ? 0.0f : mu_first / scale, mu_second <= 0.0f ? 0.0f : mu_second / scale, scale};
+}
+__device__ __forceinline__ void tangent_impulse(V3 dual, float rho, float res_y, float res_z, float normal_impulse, TangentRatios t,
                                 float* fy, float* fz, float* cyy, float* czz, float* cyz) {
     *fy = *fz = *cyy = *czz = *cyz = 0.0f;
     if (rho <= 0.0f) return;
-    const float scale = fmaxf(mu_first, mu_second);
-    const float mu_y = mu_first <= 0.0f ? 0.0f : mu_first / scale;
-    const float mu_z = mu_second <= 0.0f ? 0.0f : mu_second / scale;
+    const float mu_y = t.mu_y, mu_z = t.mu_z;
     const float q_y = mu_y == 0.0f ? 0.0f : cone_argument(dual.y, rho, mu_y, res_y);
     const float q_z = mu_z == 0.0f ? 0.0f : cone_argument(dual.z, rho, mu_z, res_z);
-    const float radius = (normal_impulse < 0.0f ? 0.0f : normal_impulse) * fmaxf(scale, 0.0f);
+    const float radius = (normal_impulse < 0.0f ? 0.0f : normal_impulse) * fmaxf(t.scale, 0.0f);
     if (q_y != q_y || q_z != q_z || radius != radius || rho != rho) {
         const float invalid = q_y + q_z + radius + rho;
         *fy = *fz = *cyy = *czz = *cyz = invalid;
@@ -132,6 +136,10 @@ __device__ void tangent_impulse(V3 dual, float rho, float res_y, float res_z, fl
     const float cs = rho * radius / norm;
     *fy = mu_y * radius * dy; *fz = mu_z * radius * dz;
     *cyy = cs * mu_y * mu_y * dz * dz; *czz = cs * mu_z * mu_z * dy * dy; *cyz = -cs * mu_y * mu_z * dy * dz;
+}
+__device__ __forceinline__ void tangent_impulse(V3 dual, float rho, float res_y, float res_z, float normal_impulse, float mu_first, float mu_second,
+                                float* fy, float* fz, float* cyy, float* czz, float* cyz) {
+    tangent_impulse(dual, rho, res_y, res_z, normal_impulse, tangent_ratios(mu_first, mu_second), fy, fz, cyy, czz, cyz);
 }
 
 __device__ __forceinline__ uint32_t residual_bits(float value) { return __float_as_uint(value <= FLT_MAX ? fabsf(value) : FLT_MAX); }
@@ -166,7 +174,7 @@ struct Tile {
 };
 
 // TileResponse (block_descent_tile.cuh:678-681) with the Coulomb branch of EvaluateAugmentedResponse (block_descent.cu:1593-1621)
-__device__ void head_response(const Tile& c, uint32_t h, float mx, float my, float mz, float* f, float* cv) {
+__device__ __forceinline__ void head_response(const Tile& c, uint32_t h, float mx, float my, float mz, float* f, float* cv) {
     const float rho = c.F(hRho, h);
     float ni, nc;
     scalar_impulse(c.F(hDual, h), rho, c.F(hRes, h) - mx, c.F(hCompliance, h), c.F(hLower, h), c.F(hUpper, h),
@@ -184,22 +192,32 @@ __device__ __forceinline__ float lane_value(float v, int lane) {
 }
 
 // FactorTileBlock (:1622-1645) on register rows: lane i holds row i of the symmetric matrix; on return its entries
-// k <= i are row i of the Cholesky factor.  Element (i, j) loses L_ik L_jk for k = 0, 1, ... in that order, one
-// product and one subtraction each, as the reference's serial inner loop does.  Uniform result: false on a bad pivot.
+// k <= i are row i of the Cholesky factor.  Element (i, j) loses L_ik L_jk for k = 0, 1, ... in that order, as the
+// reference's serial inner loop does; each product and subtraction is one fused multiply-add (the reference is
+// built with its compiler's default contraction, so it fuses these too).  Uniform result: false on a bad pivot.
 template <int N>
 __device__ __forceinline__ bool factor_rows(uint32_t lane, float (&row)[N], float* inverse_out) {
     bool valid = true;
     float inverse = 0.0f;
+    // The pivot's square root and reciprocal are a long dependent chain; column k + 1 is brought up to date first
+    // and its pivot chain started, so that it runs under the rest of step k's column updates.
+    float pivot = lane_value(row[0], 0);
+    valid = pivot > 0.0f && pivot <= FLT_MAX;
+    float root = sqrtf(valid ? pivot : 1.0f);
+    float scale = 1.0f / root;
 #pragma unroll
     for (int k = 0; k < N; ++k) {
-        const float pivot = lane_value(row[k], k);
-        valid = valid && pivot > 0.0f && pivot <= FLT_MAX;
-        const float root = sqrtf(valid ? pivot : 1.0f);
-        const float scale = 1.0f / root;
         row[k] = lane == uint32_t(k) ? root : row[k] * scale;
         if (lane == uint32_t(k)) inverse = scale;
+        if (k + 1 < N) {
+            row[k + 1] = fmaf(-row[k], lane_value(row[k], k + 1), row[k + 1]);
+            pivot = lane_value(row[k + 1], k + 1);
+            valid = valid && pivot > 0.0f && pivot <= FLT_MAX;
+            root = sqrtf(valid ? pivot : 1.0f);
+            scale = 1.0f / root;
+        }
 #pragma unroll
-        for (int j = k + 1; j < N; ++j) row[j] -= row[k] * lane_value(row[k], j);
+        for (int j = k + 2; j < N; ++j) row[j] = fmaf(-row[k], lane_value(row[k], j), row[j]);
     }
     *inverse_out = inverse;
     return valid;
@@ -243,7 +261,7 @@ __device__ __forceinline__ void load_columns(const float* a, uint32_t lane, floa
 // Cholesky of the Newton Hessian held in `hrow`, then d = H^-1 g.  The factor passes through LDS once, for the
 // transposed read of the backward substitution.
 template <int N>
-__device__ bool cholesky_solve(const Tile& c, float (&hrow)[N], float g, float* d_out) {
+__device__ __forceinline__ bool cholesky_solve(const Tile& c, float (&hrow)[N], float g, float* d_out) {
     float inverse = 0.0f;
     const bool valid = factor_rows<N>(c.lane, hrow, &inverse);
     if (!valid) return false;
@@ -259,7 +277,7 @@ __device__ bool cholesky_solve(const Tile& c, float (&hrow)[N], float g, float* 
 // SolveTileMass (:1898-1931).  The mass matrix does not change during a solve, so its factor (same arithmetic as the
 // reference's per-call factorisation, hence the same numbers) is built once by factor_mass and reused here.
 template <int N>
-__device__ bool factor_mass(Tile& c, const float (&mrow)[N]) {
+__device__ __forceinline__ bool factor_mass(Tile& c, const float (&mrow)[N]) {
     float row[N];
 #pragma unroll
     for (int k = 0; k < N; ++k) row[k] = mrow[k];
@@ -271,7 +289,7 @@ __device__ bool factor_mass(Tile& c, const float (&mrow)[N]) {
     return valid;
 }
 template <int N>
-__device__ float solve_tile_mass(const Tile& c, float force) {
+__device__ __forceinline__ float solve_tile_mass(const Tile& c, float force) {
     float row[N], col[N];
     load_rows<N>(c.mfac, c.lane, row);
     load_columns<N>(c.mfac, c.lane, col);
@@ -280,7 +298,7 @@ __device__ float solve_tile_mass(const Tile& c, float force) {
 
 // AssembleTileBlock (:1507-1618): lane i assembles row i of H = M + sum J^T C J in `hrow` and its force g_i.
 template <int N>
-__device__ bool assemble_block(const Tile& c, const float (&mrow)[N], float u, float free_v, float (&hrow)[N], float* force,
+__device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow)[N], float u, float free_v, float (&hrow)[N], float* force,
                                float* inertia, bool* converged) {
     const uint32_t lane = c.lane;
     const bool coordinate = lane < c.n;
@@ -342,7 +360,8 @@ __device__ bool assemble_block(const Tile& c, const float (&mrow)[N], float u, f
 #pragma unroll
             for (int q = 0; q < N / 4; ++q) {
                 const float4 x0 = r0[q];
-                hrow[4 * q] += a0 * x0.x; hrow[4 * q + 1] += a0 * x0.y; hrow[4 * q + 2] += a0 * x0.z; hrow[4 * q + 3] += a0 * x0.w;
+                hrow[4 * q] = fmaf(a0, x0.x, hrow[4 * q]); hrow[4 * q + 1] = fmaf(a0, x0.y, hrow[4 * q + 1]);
+                hrow[4 * q + 2] = fmaf(a0, x0.z, hrow[4 * q + 2]); hrow[4 * q + 3] = fmaf(a0, x0.w, hrow[4 * q + 3]);
             }
             continue;
         }
@@ -360,10 +379,10 @@ __device__ bool assemble_block(const Tile& c, const float (&mrow)[N], float u, f
 #pragma unroll
         for (int q = 0; q < N / 4; ++q) {
             const float4 x0 = r0[q], x1 = r1[q], x2 = r2[q];
-            hrow[4 * q] += a0 * x0.x + a1 * x1.x + a2 * x2.x;
-            hrow[4 * q + 1] += a0 * x0.y + a1 * x1.y + a2 * x2.y;
-            hrow[4 * q + 2] += a0 * x0.z + a1 * x1.z + a2 * x2.z;
-            hrow[4 * q + 3] += a0 * x0.w + a1 * x1.w + a2 * x2.w;
+            hrow[4 * q] += fmaf(a2, x2.x, fmaf(a1, x1.x, a0 * x0.x));
+            hrow[4 * q + 1] += fmaf(a2, x2.y, fmaf(a1, x1.y, a0 * x0.y));
+            hrow[4 * q + 2] += fmaf(a2, x2.z, fmaf(a1, x1.z, a0 * x0.z));
+            hrow[4 * q + 3] += fmaf(a2, x2.w, fmaf(a1, x1.w, a0 * x0.w));
         }
     }
     *force = coordinate ? g.value + g.error : 0.0f;
@@ -393,7 +412,7 @@ enum Failure : uint32_t { kFailNone = 0u, kFailEquation, kFailFactor, kFailDirec
 // convergence test because its mass factor overwrites the Hessian storage; here the two live apart and the
 // assembled row, force and inertia (which the second assembly would reproduce bit for bit) are simply kept.
 template <int N>
-__device__ Failure newton_direction(const Tile& c, const float (&mrow)[N], float u, float free_v, float* force, float* inertia,
+__device__ __forceinline__ Failure newton_direction(const Tile& c, const float (&mrow)[N], float u, float free_v, float* force, float* inertia,
                                     float* d, bool* converged) {
     PROF_COUNT(c, 0);
     float hrow[N];
@@ -433,7 +452,7 @@ __device__ __forceinline__ float row_dot_fma(const float* jrow, const float* dve
     return value;
 }
 template <int N>
-__device__ void row_steps(const Tile& c, float d) {
+__device__ __forceinline__ void row_steps(const Tile& c, float d) {
     float* dvec = c.vec;
     dvec[c.lane] = c.lane < c.n ? d : 0.0f;
     __syncthreads();
@@ -448,23 +467,52 @@ __device__ void row_steps(const Tile& c, float d) {
     __syncthreads();
 }
 
-// TileLineDerivatives (:2048-2086)
-__device__ void line_derivatives(const Tile& c, float alpha, float inertial_slope, float inertial_curvature, float* slope,
-                                 float* curvature, float* magnitude) {
+// One head's line-search inputs in registers: nothing in them changes between the probes of one search.
+struct HeadLine {
+    bool owned, contact;
+    float rho, compliance, lower, upper, bound;
+    Response response;
+    TangentRatios ratios;
+    float dual[3], res[3], move[3], step[3];
+};
+__device__ __forceinline__ HeadLine load_head_line(const Tile& c, uint32_t h) {
+    HeadLine l{};
+    l.owned = h < c.heads && c.U(hOwned, h) != 0u;
+    if (!l.owned) return l;
+    l.contact = c.U(hAxes, h) == 3u;
+    l.rho = c.F(hRho, h); l.compliance = c.F(hCompliance, h); l.lower = c.F(hLower, h); l.upper = c.F(hUpper, h);
+    l.bound = c.F(hNormalBound, h);
+    l.response = Response{c.F(hDualScale, h), c.F(hResidualScale, h)};
+    l.ratios = tangent_ratios(c.F(hMu1, h), c.F(hMu2, h));
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { l.dual[k] = c.F(hDual + k, h); l.res[k] = c.F(hRes + k, h); l.move[k] = c.F(hMove + k, h); l.step[k] = c.F(hStep + k, h); }
+    return l;
+}
+
+// TileLineDerivatives (:2048-2086); lane = head, heads beyond the first 64 go through `extra`
+__device__ __forceinline__ void line_terms(const HeadLine& l, float alpha, TileSum& row_slope, float& row_curvature, float& row_magnitude) {
+    const float sx = l.step[0], sy = l.step[1], sz = l.step[2];
+    float f[3] = {0.0f, 0.0f, 0.0f}, r[6] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    scalar_impulse(l.dual[0], l.rho, l.res[0] - fmaf(alpha, sx, l.move[0]), l.compliance, l.lower, l.upper, l.response, &f[0], &r[0]);
+    if (l.contact)
+        tangent_impulse(V3{l.dual[0], l.dual[1], l.dual[2]}, l.rho, l.res[1] - fmaf(alpha, sy, l.move[1]),
+                        l.res[2] - fmaf(alpha, sz, l.move[2]), l.bound, l.ratios, &f[1], &f[2], &r[1], &r[2], &r[5]);
+    tile_add_product(row_slope, f[0], sx);
+    tile_add_product(row_slope, f[1], sy);
+    tile_add_product(row_slope, f[2], sz);
+    row_magnitude += fabsf(f[0] * sx) + fabsf(f[1] * sy) + fabsf(f[2] * sz);
+    row_curvature += r[0] * sx * sx + r[1] * sy * sy + r[2] * sz * sz + 2.0f * r[5] * sy * sz + 2.0f * r[3] * sx * sy +
+                     2.0f * r[4] * sx * sz;
+}
+__device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& mine, float alpha, float inertial_slope, float inertial_curvature,
+                                 float* slope, float* curvature, float* magnitude) {
     PROF_COUNT(c, 1);
     TileSum row_slope{0.0f, 0.0f};
     float row_curvature = 0.0f, row_magnitude = 0.0f;
-    for (uint32_t h = c.lane; h < c.heads; h += kWave) {
-        if (c.U(hOwned, h) == 0u) continue;
-        const float sx = c.F(hStep, h), sy = c.F(hStep + 1, h), sz = c.F(hStep + 2, h);
-        float f[3], r[6];
-        head_response(c, h, fmaf(alpha, sx, c.F(hMove, h)), fmaf(alpha, sy, c.F(hMove + 1, h)), fmaf(alpha, sz, c.F(hMove + 2, h)), f, r);
-        tile_add_product(row_slope, f[0], sx);
-        tile_add_product(row_slope, f[1], sy);
-        tile_add_product(row_slope, f[2], sz);
-        row_magnitude += fabsf(f[0] * sx) + fabsf(f[1] * sy) + fabsf(f[2] * sz);
-        row_curvature += r[0] * sx * sx + r[1] * sy * sy + r[2] * sz * sz + 2.0f * r[5] * sy * sz + 2.0f * r[3] * sx * sy +
-                         2.0f * r[4] * sx * sz;
+    if (mine.owned) line_terms(mine, alpha, row_slope, row_curvature, row_magnitude);
+    for (uint32_t h = c.lane + kWave; h < c.heads; h += kWave) {
+        const HeadLine extra = load_head_line(c, h);
+        if (extra.owned) line_terms(extra, alpha, row_slope, row_curvature, row_magnitude);
     }
     TileSum total{-row_slope.value, -row_slope.error};
     if (c.lane == 0u) {
@@ -477,15 +525,16 @@ __device__ void line_derivatives(const Tile& c, float alpha, float inertial_slop
 }
 
 // SearchTileLine (:2089-2125)
-__device__ float search_line(const Tile& c, float inertial_slope, float inertial_curvature) {
+__device__ __forceinline__ float search_line(const Tile& c, float inertial_slope, float inertial_curvature) {
     float slope = 0.0f, curvature = 0.0f, magnitude = 0.0f;
-    line_derivatives(c, 0.0f, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
+    const HeadLine mine = load_head_line(c, c.lane);
+    line_derivatives(c, mine, 0.0f, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
     const float initial = slope;
     if (!(initial < 0.0f)) return 0.0f;
     float low = 0.0f, high = 0.0f, alpha = 1.0f;
     bool bounded = false;
     for (uint32_t step = 0u; step < kLineSearchSteps; ++step) {
-        line_derivatives(c, alpha, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
+        line_derivatives(c, mine, alpha, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
         if (!isfinite(slope) || !isfinite(curvature)) {
             high = alpha; bounded = true; alpha = 0.5f * (low + high);
             continue;
@@ -501,7 +550,7 @@ __device__ float search_line(const Tile& c, float inertial_slope, float inertial
     return low;
 }
 
-__device__ void apply_moves(const Tile& c, float alpha) {
+__device__ __forceinline__ void apply_moves(const Tile& c, float alpha) {
     for (uint32_t h = c.lane; h < c.heads; h += kWave) {
         if (c.U(hOwned, h) == 0u) continue;
 #pragma unroll
@@ -512,7 +561,7 @@ __device__ void apply_moves(const Tile& c, float alpha) {
 
 // mass_step_i = sum_k M_ik d_k in coordinate order (:2177-2187, 2228-2238)
 template <int N>
-__device__ float mass_times(const Tile& c, const float (&mrow)[N], float d) {
+__device__ __forceinline__ float mass_times(const Tile& c, const float (&mrow)[N], float d) {
     float* dvec = c.vec + 192;
     dvec[c.lane] = d;
     __syncthreads();
@@ -529,7 +578,7 @@ __device__ float mass_times(const Tile& c, const float (&mrow)[N], float d) {
 
 // DescendTileBlock (:2145-2301).  `u` is lane i's block coordinate; `has_free` is false in the position pass.
 template <int N>
-__device__ void descend_block(Tile& c, const float (&mrow)[N], float* u_io, float free_in, bool has_free, DataView d) {
+__device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], float* u_io, float free_in, bool has_free, DataView d) {
     const uint32_t lane = c.lane, n = c.n;
     const bool coordinate = lane < n;
     for (uint32_t h = lane; h < c.heads; h += kWave) {   // StartTileBlock (:1386-1397)
@@ -615,7 +664,7 @@ __device__ void descend_block(Tile& c, const float (&mrow)[N], float* u_io, floa
 
 // MeasureTilePrimal (:2378-2489): the mass-normalised momentum balance in double
 template <int N>
-__device__ void measure_primal(Tile& c, const float (&mrow)[N], float* velocity_io, float free_v, const float* lambda_env, uint32_t R,
+__device__ __forceinline__ void measure_primal(Tile& c, const float (&mrow)[N], float* velocity_io, float free_v, const float* lambda_env, uint32_t R,
                                bool reconstruct, DataView d) {
     const uint32_t lane = c.lane, n = c.n;
     const bool coordinate = lane < n;
@@ -663,7 +712,7 @@ __device__ void measure_primal(Tile& c, const float (&mrow)[N], float* velocity_
 
 // InitializeTileResiduals (:890-930) on the staged rows: residual = fl(rhs dt) - J u, products summed in coordinate order
 template <int N>
-__device__ void initialize_residuals(const Tile& c, float velocity, const float* urows, float dt) {
+__device__ __forceinline__ void initialize_residuals(const Tile& c, float velocity, const float* urows, float dt) {
     float* dvec = c.vec;
     dvec[c.lane] = c.lane < c.n ? velocity : 0.0f;
     __syncthreads();
@@ -692,7 +741,7 @@ __device__ void initialize_residuals(const Tile& c, float velocity, const float*
 struct DualMomentum { float t, beta; };
 
 // UpdateTileHeadDuals (:2493-2595); classes = {normal, tangent, joint}
-__device__ void update_duals(const Tile& c, float* lambda_env, uint32_t R, const float* urows, DualMomentum* momentum, bool velocity,
+__device__ __forceinline__ void update_duals(const Tile& c, float* lambda_env, uint32_t R, const float* urows, DualMomentum* momentum, bool velocity,
                              bool commit, float* classes) {
     uint32_t steps[3] = {0u, 0u, 0u};
     double restart = 0.0;
