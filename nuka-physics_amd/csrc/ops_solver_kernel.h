@@ -1,0 +1,1185 @@
+// UABD block-descent contact solve for gfx950.  One 64-lane wavefront owns one environment for the whole solve:
+// every velocity sweep, the dual updates and the split-impulse position pass run in a single launch with the
+// staged Jacobian rows and per-head state resident in LDS.  A lane is a block coordinate in the matrix phases and
+// owns one matrix row IN REGISTERS: the kernel is compiled per padded width N (a multiple of 4, nv <= N <= 64), the
+// mass row, the Newton Hessian row and its Cholesky factor row are fully unrolled register arrays, pivots and
+// multipliers travel between lanes as scalar lane reads, and LDS only carries what must be read transposed (the
+// factor columns of the backward substitution) or broadcast (Jacobian rows, small vectors, read as 16-byte words).
+// The mass matrix is constant over a solve, so its factor is built once.  A lane is a head row in the per-head
+// phases.  Cross-lane sums use the compensated two-float butterfly; nothing is exchanged between environments.
+//
+// Replaces src/phi/backend_cuda/ops/block_descent_tile.cuh (DescendTile :2941-3087 and everything it calls) and
+// the helpers it takes from block_descent.cu (:735-820, 1593-1621, 1726-1753) and nk/solve/augmented_row.hpp.
+// Blocks: one articulation per environment.  Not built: free rigid 6x6 blocks, mimic couplings, elliptic
+// (MuJoCo-law) cones, single-coordinate "unit" rows (only joint rows produce them, and joint rows are not emitted).
+#pragma once
+
+#include "nk_device_math.h"
+#include "backend.h"
+#include "nk_ops.h"
+
+namespace nkh {
+namespace solver {
+
+constexpr int kWave = 64;
+constexpr uint32_t kNewtonSteps = 16u;        // block_descent_dense.cuh:14
+constexpr uint32_t kLineSearchSteps = 32u;    // block_descent_dense.cuh:15
+constexpr float kLineTolerance = 1.0e-6f;     // block_descent_dense.cuh:17
+constexpr float kRoundings = 8.0f;            // block_descent_dense.cuh:19
+constexpr float kPenaltyConditionCap = 1.0e2f;   // block_descent.cu:71
+
+// Phase timers for development builds (-DNKH_SOLVER_PROFILE): cycles per phase and event counts per environment,
+// written over the environment's solver_penalty words at the end of the solve.
+#ifdef NKH_SOLVER_PROFILE
+#define PROF_BEGIN(c, i) const long long prof_start_##i = clock64()
+#define PROF_END(c, i) (c).prof[i] += clock64() - prof_start_##i
+#define PROF_COUNT(c, i) (c).prof_count[i] += 1u
+#else
+#define PROF_BEGIN(c, i)
+#define PROF_END(c, i)
+#define PROF_COUNT(c, i)
+#endif
+
+struct TileSum { float value, error; };   // block_descent_tile.cuh:15-31
+__device__ __forceinline__ void tile_add(TileSum& s, float x) {
+    const float sum = s.value + x;
+    const float part = sum - s.value;
+    s.error += (s.value - (sum - part)) + (x - part);
+    s.value = sum;
+}
+__device__ __forceinline__ void tile_add_product(TileSum& s, float a, float b) {
+    const float product = a * b;
+    s.error += fmaf(a, b, -product);
+    tile_add(s, product);
+}
+// block_descent_tile.cuh:34-46 over 64 lanes: rows of 16 by DPP, then the four rows as scalars; uniform result
+__device__ __forceinline__ void tile_merge(TileSum& s, float value, float error) {
+    s.error += error;
+    tile_add(s, value);
+}
+__device__ __forceinline__ float wave_total(TileSum s) {
+    tile_merge(s, dpp_move<kDppXor1>(s.value), dpp_move<kDppXor1>(s.error));
+    tile_merge(s, dpp_move<kDppXor2>(s.value), dpp_move<kDppXor2>(s.error));
+    tile_merge(s, dpp_move<kDppHalfMirror>(s.value), dpp_move<kDppHalfMirror>(s.error));
+    tile_merge(s, dpp_move<kDppMirror>(s.value), dpp_move<kDppMirror>(s.error));
+    TileSum a{row_value(s.value, 0), row_value(s.error, 0)}, b{row_value(s.value, 2), row_value(s.error, 2)};
+    tile_merge(a, row_value(s.value, 1), row_value(s.error, 1));
+    tile_merge(b, row_value(s.value, 3), row_value(s.error, 3));
+    tile_merge(a, b.value, b.error);
+    return a.value + a.error;
+}
+
+struct Response { float dual_scale, residual_scale; };
+// augmented_row.hpp:226-229
+__device__ __forceinline__ Response scalar_response(float cap, float compliance) {
+    const float product = cap * compliance;
+    return product >= 1.0f ? Response{0.0f, 1.0f / compliance} : Response{1.0f - product, cap};
+}
+// augmented_row.hpp:232-247
+__device__ __forceinline__ void scalar_impulse(float dual, float rho, float residual, float compliance, float lower, float upper,
+                                               Response r, float* impulse, float* curvature) {
+    *impulse = 0.0f; *curvature = 0.0f;
+    if (rho <= 0.0f) return;
+    if (dual != dual || rho != rho || residual != residual || compliance != compliance || lower != lower || upper != upper) {
+        const float invalid = dual + rho + residual + compliance + lower + upper;
+        *impulse = invalid; *curvature = invalid;
+        return;
+    }
+    const float k = r.residual_scale;
+    const float x = fmaf(k, residual, r.dual_scale * dual);
+    *impulse = x < lower ? lower : (x > upper ? upper : x);
+    *curvature = x != x ? x : (lower < upper && x >= lower && x <= upper ? k : 0.0f);
+}
+// augmented_row.hpp:302-318
+__device__ __forceinline__ float cone_argument(float dual, float rho, float mu, float residual) {
+    const bool dual_zero = dual == 0.0f;
+    const float dual_quotient = (dual + float(dual_zero)) / mu;
+    const float dd = dual_zero ? dual : dual_quotient;
+    const float low = fmaf(-dd, mu, dual);
+    const bool low_zero = low == 0.0f;
+    const float low_quotient = (low + float(low_zero)) / mu;
+    const float d_low = low_zero ? low : low_quotient;
+    const float p = rho * mu;
+    const float t = p * residual;
+    const float t_low = fmaf(p, residual, -t) + fmaf(rho, mu, -p) * residual;
+    const float sum = dd + t;
+    const float t_part = sum - dd;
+    const float sum_low = (dd - (sum - t_part)) + (t - t_part);
+    return sum + (sum_low + d_low + t_low);
+}
+// augmented_row.hpp:321-348; curvature entries yy, zz, yz.  The friction ratios depend on the row only, so callers
+// that evaluate one row many times compute them once (tangent_ratios) and pass them in.
+struct TangentRatios { float mu_y, mu_z, scale; };
+__device__ __forceinline__ TangentRatios tangent_ratios(float mu_first, float mu_second) {
+    const float scale = fmaxf(mu_first, mu_second);
+    return TangentRatios{mu_first <= 0.0f ? 0.0f : mu_first / scale, mu_second <= 0.0f ? 0.0f : mu_second / scale, scale};
+}
+__device__ __forceinline__ void tangent_impulse(V3 dual, float rho, float res_y, float res_z, float normal_impulse, TangentRatios t,
+                                float* fy, float* fz, float* cyy, float* czz, float* cyz) {
+    *fy = *fz = *cyy = *czz = *cyz = 0.0f;
+    if (rho <= 0.0f) return;
+    const float mu_y = t.mu_y, mu_z = t.mu_z;
+    const float q_y = mu_y == 0.0f ? 0.0f : cone_argument(dual.y, rho, mu_y, res_y);
+    const float q_z = mu_z == 0.0f ? 0.0f : cone_argument(dual.z, rho, mu_z, res_z);
+    const float radius = (normal_impulse < 0.0f ? 0.0f : normal_impulse) * fmaxf(t.scale, 0.0f);
+    if (q_y != q_y || q_z != q_z || radius != radius || rho != rho) {
+        const float invalid = q_y + q_z + radius + rho;
+        *fy = *fz = *cyy = *czz = *cyz = invalid;
+        return;
+    }
+    if (radius == 0.0f) return;
+    const float norm = hypotf(q_y, q_z);
+    if (norm <= radius) {
+        *fy = mu_y * q_y; *fz = mu_z * q_z; *cyy = rho * mu_y * mu_y; *czz = rho * mu_z * mu_z;
+        return;
+    }
+    const float dy = q_y / norm, dz = q_z / norm;
+    const float cs = rho * radius / norm;
+    *fy = mu_y * radius * dy; *fz = mu_z * radius * dz;
+    *cyy = cs * mu_y * mu_y * dz * dz; *czz = cs * mu_z * mu_z * dy * dy; *cyz = -cs * mu_y * mu_z * dy * dz;
+}
+__device__ __forceinline__ void tangent_impulse(V3 dual, float rho, float res_y, float res_z, float normal_impulse, float mu_first, float mu_second,
+                                float* fy, float* fz, float* cyy, float* czz, float* cyz) {
+    tangent_impulse(dual, rho, res_y, res_z, normal_impulse, tangent_ratios(mu_first, mu_second), fy, fz, cyy, czz, cyz);
+}
+
+__device__ __forceinline__ uint32_t residual_bits(float value) { return __float_as_uint(value <= FLT_MAX ? fabsf(value) : FLT_MAX); }
+__device__ __forceinline__ float along_axis(float impulse, float velocity) { return impulse > 0.0f ? velocity : impulse < 0.0f ? -velocity : 0.0f; }
+
+// Per-head state, field-major in LDS so lane = head reads without bank conflicts.
+enum HeadField : uint32_t {
+    hSlot, hStride, hAxes, hOwned, hRho, hCompliance, hLower, hUpper, hMu1, hMu2, hNormalBound,
+    hRes, hDual = hRes + 3, hMove = hDual + 3, hStep = hMove + 3, hBase = hStep + 3, hDualScale = hBase + 3, hResidualScale,
+    hRelaxStep, hRelaxWeight = hRelaxStep + 3, hRelaxPoint, hF = hRelaxPoint + 3, hC = hF + 3, hNoise = hC + 6, hContrib = hNoise + 3,
+    hFieldCount
+};
+
+struct Tile {
+    uint32_t env, lane, n, ld, ldj, heads, cap, iteration;
+    float tolerance;
+    float* mfac;     // N x ld: Cholesky factor of the mass matrix (rows; columns are read transposed)
+    float* hfac;     // N x ld: Cholesky factor of the current Newton Hessian
+    float* jac;      // 3 * cap rows x ldj, ldj = N
+    float* fields;   // hFieldCount x cap
+    float* vec;      // 4 x 64 scratch vectors, 16-byte aligned
+    float mass_inverse;   // 1 / diagonal of the mass factor, lane = row
+    bool mass_valid;
+    float momentum, residual;
+    bool failed;
+#ifdef NKH_SOLVER_PROFILE
+    mutable long long prof[10];
+    mutable uint32_t prof_count[4];
+#endif
+    __device__ float& F(uint32_t field, uint32_t h) const { return fields[field * cap + h]; }
+    __device__ uint32_t& U(uint32_t field, uint32_t h) const { return reinterpret_cast<uint32_t*>(fields)[field * cap + h]; }
+};
+
+// TileResponse (block_descent_tile.cuh:678-681) with the Coulomb branch of EvaluateAugmentedResponse (block_descent.cu:1593-1621)
+__device__ __forceinline__ void head_response(const Tile& c, uint32_t h, float mx, float my, float mz, float* f, float* cv) {
+    const float rho = c.F(hRho, h);
+    float ni, nc;
+    scalar_impulse(c.F(hDual, h), rho, c.F(hRes, h) - mx, c.F(hCompliance, h), c.F(hLower, h), c.F(hUpper, h),
+                   Response{c.F(hDualScale, h), c.F(hResidualScale, h)}, &ni, &nc);
+    f[0] = ni; f[1] = f[2] = 0.0f;
+    cv[0] = nc; cv[1] = cv[2] = cv[3] = cv[4] = cv[5] = 0.0f;
+    if (c.U(hAxes, h) != 3u) return;
+    tangent_impulse(V3{c.F(hDual, h), c.F(hDual + 1, h), c.F(hDual + 2, h)}, rho, c.F(hRes + 1, h) - my, c.F(hRes + 2, h) - mz,
+                    c.F(hNormalBound, h), c.F(hMu1, h), c.F(hMu2, h), &f[1], &f[2], &cv[1], &cv[2], &cv[5]);
+}
+
+// A lane's value of `v` for a lane index that is a compile-time constant at every call site: a scalar lane read.
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+// FactorTileBlock (:1622-1645) on register rows: lane i holds row i of the symmetric matrix; on return its entries
+// k <= i are row i of the Cholesky factor.  Element (i, j) loses L_ik L_jk for k = 0, 1, ... in that order, as the
+// reference's serial inner loop does; each product and subtraction is one fused multiply-add (the reference is
+// built with its compiler's default contraction, so it fuses these too).  Uniform result: false on a bad pivot.
+template <int N>
+__device__ __forceinline__ bool factor_rows(uint32_t lane, float (&row)[N], float* inverse_out) {
+    bool valid = true;
+    float inverse = 0.0f;
+    // The pivot's square root and reciprocal are a long dependent chain; column k + 1 is brought up to date first
+    // and its pivot chain started, so that it runs under the rest of step k's column updates.
+    float pivot = lane_value(row[0], 0);
+    valid = pivot > 0.0f && pivot <= FLT_MAX;
+    float root = sqrtf(valid ? pivot : 1.0f);
+    float scale = 1.0f / root;
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+        row[k] = lane == uint32_t(k) ? root : row[k] * scale;
+        if (lane == uint32_t(k)) inverse = scale;
+        if (k + 1 < N) {
+            row[k + 1] = fmaf(-row[k], lane_value(row[k], k + 1), row[k + 1]);
+            pivot = lane_value(row[k + 1], k + 1);
+            valid = valid && pivot > 0.0f && pivot <= FLT_MAX;
+            root = sqrtf(valid ? pivot : 1.0f);
+            scale = 1.0f / root;
+        }
+#pragma unroll
+        for (int j = k + 2; j < N; ++j) row[j] = fmaf(-row[k], lane_value(row[k], j), row[j]);
+    }
+    *inverse_out = inverse;
+    return valid;
+}
+
+// SolveTileBlock (:1647-1666): forward with the factor's rows, backward with its columns (col[j] = L_j,lane).
+template <int N>
+__device__ __forceinline__ float substitute(uint32_t lane, const float (&row)[N], const float (&col)[N], float inverse, float g) {
+    float r = g;
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        const float y = lane_value(r * inverse, j);
+        r = lane == uint32_t(j) ? y : (lane > uint32_t(j) ? fmaf(-row[j], y, r) : r);
+    }
+#pragma unroll
+    for (int j = N - 1; j >= 0; --j) {
+        const float x = lane_value(r * inverse, j);
+        r = lane == uint32_t(j) ? x : (lane < uint32_t(j) ? fmaf(-col[j], x, r) : r);
+    }
+    return r;
+}
+
+template <int N>
+__device__ __forceinline__ void store_rows(float* a, uint32_t lane, const float (&row)[N]) {
+    if (lane < uint32_t(N)) {
+#pragma unroll
+        for (int k = 0; k < N; ++k) a[lane * (N + 1) + k] = row[k];
+    }
+}
+template <int N>
+__device__ __forceinline__ void load_rows(const float* a, uint32_t lane, float (&row)[N]) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) row[k] = lane < uint32_t(N) ? a[lane * (N + 1) + k] : 0.0f;
+}
+template <int N>
+__device__ __forceinline__ void load_columns(const float* a, uint32_t lane, float (&col)[N]) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) col[j] = lane < uint32_t(N) ? a[j * (N + 1) + lane] : 0.0f;
+}
+
+// Cholesky of the Newton Hessian held in `hrow`, then d = H^-1 g.  The factor passes through LDS once, for the
+// transposed read of the backward substitution.
+template <int N>
+__device__ __forceinline__ bool cholesky_solve(const Tile& c, float (&hrow)[N], float g, float* d_out) {
+    float inverse = 0.0f;
+    const bool valid = factor_rows<N>(c.lane, hrow, &inverse);
+    if (!valid) return false;
+    store_rows<N>(c.hfac, c.lane, hrow);
+    __syncthreads();
+    float col[N];
+    load_columns<N>(c.hfac, c.lane, col);
+    *d_out = substitute<N>(c.lane, hrow, col, inverse, c.lane < c.n ? g : 0.0f);
+    __syncthreads();
+    return true;
+}
+
+// SolveTileMass (:1898-1931).  The mass matrix does not change during a solve, so its factor (same arithmetic as the
+// reference's per-call factorisation, hence the same numbers) is built once by factor_mass and reused here.
+template <int N>
+__device__ __forceinline__ bool factor_mass(Tile& c, const float (&mrow)[N]) {
+    float row[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k) row[k] = mrow[k];
+    float inverse = 0.0f;
+    const bool valid = factor_rows<N>(c.lane, row, &inverse);
+    c.mass_inverse = inverse;
+    store_rows<N>(c.mfac, c.lane, row);
+    __syncthreads();
+    return valid;
+}
+template <int N>
+__device__ __forceinline__ float solve_tile_mass(const Tile& c, float force) {
+    float row[N], col[N];
+    load_rows<N>(c.mfac, c.lane, row);
+    load_columns<N>(c.mfac, c.lane, col);
+    return substitute<N>(c.lane, row, col, c.mass_inverse, c.lane < c.n ? force : 0.0f);
+}
+
+// AssembleTileBlock (:1507-1618): lane i assembles row i of H = M + sum J^T C J in `hrow` and its force g_i.
+template <int N>
+__device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow)[N], float u, float free_v, float (&hrow)[N], float* force,
+                               float* inertia, bool* converged) {
+    const uint32_t lane = c.lane;
+    const bool coordinate = lane < c.n;
+    const float difference = u - free_v;
+    const float part = difference - u;
+    const float difference_error = (u - (difference - part)) + (-free_v - part);
+    float* dvec = c.vec, *evec = c.vec + 64, *uvec = c.vec + 128;
+    dvec[lane] = difference; evec[lane] = difference_error; uvec[lane] = fabsf(u);
+    // every head's response at its current move, lane = head
+    for (uint32_t h = lane; h < c.heads; h += kWave) {
+        float f[3] = {0, 0, 0}, cv[6] = {0, 0, 0, 0, 0, 0};
+        bool contributes = false;
+        if (c.U(hOwned, h) != 0u) {
+            head_response(c, h, c.F(hMove, h), c.F(hMove + 1, h), c.F(hMove + 2, h), f, cv);
+            const float n0 = fabsf(f[0]) + cv[0] * (fabsf(c.F(hRes, h)) + fabsf(c.F(hMove, h)));
+            const float n1 = fabsf(f[1]) + cv[1] * (fabsf(c.F(hRes + 1, h)) + fabsf(c.F(hMove + 1, h)));
+            const float n2 = fabsf(f[2]) + cv[2] * (fabsf(c.F(hRes + 2, h)) + fabsf(c.F(hMove + 2, h)));
+            c.F(hNoise, h) = n0; c.F(hNoise + 1, h) = n1; c.F(hNoise + 2, h) = n2;
+            contributes = f[0] != 0.0f || f[1] != 0.0f || f[2] != 0.0f || cv[0] != 0.0f || cv[1] != 0.0f || cv[2] != 0.0f ||
+                          cv[5] != 0.0f || cv[3] != 0.0f || cv[4] != 0.0f || n0 != 0.0f || n1 != 0.0f || n2 != 0.0f;
+        }
+#pragma unroll
+        for (int k = 0; k < 3; ++k) c.F(hF + k, h) = f[k];
+#pragma unroll
+        for (int k = 0; k < 6; ++k) c.F(hC + k, h) = cv[k];
+        c.U(hContrib, h) = contributes ? 1u : 0u;
+    }
+    __syncthreads();
+    // Padded columns (k >= n) hold exact zeros in the mass row, the vectors and the Jacobian rows: their terms add
+    // nothing to any of the sums below.
+    TileSum inertial{0.0f, 0.0f};
+    float scale = 0.0f;
+    const float4* d4 = reinterpret_cast<const float4*>(dvec);
+    const float4* e4 = reinterpret_cast<const float4*>(evec);
+#pragma unroll
+    for (int q = 0; q < N / 4; ++q) {
+        const float4 dv = d4[q], ev = e4[q];
+        const float dk[4] = {dv.x, dv.y, dv.z, dv.w}, ek[4] = {ev.x, ev.y, ev.z, ev.w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float mass = mrow[4 * q + t];
+            hrow[4 * q + t] = mass;
+            tile_add_product(inertial, mass, dk[t]);
+            tile_add_product(inertial, mass, ek[t]);
+            scale += fabsf(mass) * fabsf(dk[t]);
+        }
+    }
+    TileSum g{-inertial.value, -inertial.error};
+    for (uint32_t h = 0u; h < c.heads; ++h) {
+        if (c.U(hContrib, h) == 0u) continue;
+        const float* j0r = c.jac + (3u * h) * uint32_t(N);
+        const float j0 = coordinate ? j0r[lane] : 0.0f;
+        const float fx = c.F(hF, h), cxx = c.F(hC, h);
+        tile_add_product(g, j0, fx);
+        scale += fabsf(j0) * c.F(hNoise, h);
+        const float4* r0 = reinterpret_cast<const float4*>(j0r);
+        if (c.U(hAxes, h) == 1u) {
+            const float a0 = j0 * cxx;
+#pragma unroll
+            for (int q = 0; q < N / 4; ++q) {
+                const float4 x0 = r0[q];
+                hrow[4 * q] = fmaf(a0, x0.x, hrow[4 * q]); hrow[4 * q + 1] = fmaf(a0, x0.y, hrow[4 * q + 1]);
+                hrow[4 * q + 2] = fmaf(a0, x0.z, hrow[4 * q + 2]); hrow[4 * q + 3] = fmaf(a0, x0.w, hrow[4 * q + 3]);
+            }
+            continue;
+        }
+        const float* j1r = j0r + N, *j2r = j0r + 2 * N;
+        const float j1 = coordinate ? j1r[lane] : 0.0f, j2 = coordinate ? j2r[lane] : 0.0f;
+        const float cyy = c.F(hC + 1, h), czz = c.F(hC + 2, h), cxy = c.F(hC + 3, h), cxz = c.F(hC + 4, h), cyz = c.F(hC + 5, h);
+        tile_add_product(g, j1, c.F(hF + 1, h));
+        tile_add_product(g, j2, c.F(hF + 2, h));
+        scale += fabsf(j1) * c.F(hNoise + 1, h) + fabsf(j2) * c.F(hNoise + 2, h);
+        const float a0 = (j0 * cxx + j1 * cxy) + j2 * cxz;
+        const float a1 = (j1 * cyy + j2 * cyz) + j0 * cxy;
+        const float a2 = (j2 * czz + j1 * cyz) + j0 * cxz;
+        const float4* r1 = reinterpret_cast<const float4*>(j1r);
+        const float4* r2 = reinterpret_cast<const float4*>(j2r);
+#pragma unroll
+        for (int q = 0; q < N / 4; ++q) {
+            const float4 x0 = r0[q], x1 = r1[q], x2 = r2[q];
+            hrow[4 * q] += fmaf(a2, x2.x, fmaf(a1, x1.x, a0 * x0.x));
+            hrow[4 * q + 1] += fmaf(a2, x2.y, fmaf(a1, x1.y, a0 * x0.y));
+            hrow[4 * q + 2] += fmaf(a2, x2.z, fmaf(a1, x1.z, a0 * x0.z));
+            hrow[4 * q + 3] += fmaf(a2, x2.w, fmaf(a1, x1.w, a0 * x0.w));
+        }
+    }
+    *force = coordinate ? g.value + g.error : 0.0f;
+    *inertia = coordinate ? inertial.value + inertial.error : 0.0f;
+    bool finite = isfinite(*force);
+    const float4* u4 = reinterpret_cast<const float4*>(uvec);
+#pragma unroll
+    for (int q = 0; q < N / 4; ++q) {
+        const float4 uv = u4[q];
+        const float uk[4] = {uv.x, uv.y, uv.z, uv.w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float entry = hrow[4 * q + t];
+            finite = finite && isfinite(entry);
+            scale += fabsf(entry) * uk[t];
+        }
+    }
+    *converged = __all(!coordinate || fabsf(*force) <= kRoundings * FLT_EPSILON * scale);
+    const bool ok = __all(!coordinate || finite);
+    __syncthreads();
+    return ok;
+}
+
+enum Failure : uint32_t { kFailNone = 0u, kFailEquation, kFailFactor, kFailDirection, kFailCandidate };
+
+// TileNewtonDirection (:1935-1992), narrow form.  The reference re-assembles the block after the mass-normalised
+// convergence test because its mass factor overwrites the Hessian storage; here the two live apart and the
+// assembled row, force and inertia (which the second assembly would reproduce bit for bit) are simply kept.
+template <int N>
+__device__ __forceinline__ Failure newton_direction(const Tile& c, const float (&mrow)[N], float u, float free_v, float* force, float* inertia,
+                                    float* d, bool* converged) {
+    PROF_COUNT(c, 0);
+    float hrow[N];
+    PROF_BEGIN(c, 1);
+    const bool assembled = assemble_block<N>(c, mrow, u, free_v, hrow, force, inertia, converged);
+    PROF_END(c, 1);
+    if (!assembled) return kFailEquation;
+    if (*converged && c.tolerance > 0.0f) {
+        if (!c.mass_valid) return kFailFactor;
+        PROF_BEGIN(c, 3);
+        const float direction = solve_tile_mass<N>(c, *force);
+        PROF_END(c, 3);
+        *d = direction;
+        *converged = __all(c.lane >= c.n || fabsf(direction) < c.tolerance);
+        if (*converged) return kFailNone;
+    }
+    if (*converged) return kFailNone;
+    PROF_BEGIN(c, 2);
+    const bool factored = cholesky_solve<N>(c, hrow, *force, d);
+    PROF_END(c, 2);
+    if (!factored) return kFailFactor;
+    return kFailNone;
+}
+
+// TileRowSteps (:2018-2044): step = J d per head axis by serial fused multiply-adds, lane = head.  The Jacobian row
+// and the direction come in as 16-byte words; padded columns are zeros on both sides.
+template <int N>
+__device__ __forceinline__ float row_dot_fma(const float* jrow, const float* dvec) {
+    const float4* j4 = reinterpret_cast<const float4*>(jrow);
+    const float4* d4 = reinterpret_cast<const float4*>(dvec);
+    float value = 0.0f;
+#pragma unroll
+    for (int q = 0; q < N / 4; ++q) {
+        const float4 j = j4[q], d = d4[q];
+        value = fmaf(j.x, d.x, value); value = fmaf(j.y, d.y, value); value = fmaf(j.z, d.z, value); value = fmaf(j.w, d.w, value);
+    }
+    return value;
+}
+template <int N>
+__device__ __forceinline__ void row_steps(const Tile& c, float d) {
+    float* dvec = c.vec;
+    dvec[c.lane] = c.lane < c.n ? d : 0.0f;
+    __syncthreads();
+    for (uint32_t h = c.lane; h < c.heads; h += kWave) {
+        if (c.U(hOwned, h) == 0u) continue;
+        const float* j = c.jac + (3u * h) * uint32_t(N);
+        const uint32_t axes = c.U(hAxes, h);
+        c.F(hStep, h) = row_dot_fma<N>(j, dvec);
+        c.F(hStep + 1, h) = axes > 1u ? row_dot_fma<N>(j + N, dvec) : 0.0f;
+        c.F(hStep + 2, h) = axes > 2u ? row_dot_fma<N>(j + 2 * N, dvec) : 0.0f;
+    }
+    __syncthreads();
+}
+
+// One head's line-search inputs in registers: nothing in them changes between the probes of one search.
+struct HeadLine {
+    bool owned, contact;
+    float rho, compliance, lower, upper, bound;
+    Response response;
+    TangentRatios ratios;
+    float dual[3], res[3], move[3], step[3];
+};
+__device__ __forceinline__ HeadLine load_head_line(const Tile& c, uint32_t h) {
+    HeadLine l{};
+    l.owned = h < c.heads && c.U(hOwned, h) != 0u;
+    if (!l.owned) return l;
+    l.contact = c.U(hAxes, h) == 3u;
+    l.rho = c.F(hRho, h); l.compliance = c.F(hCompliance, h); l.lower = c.F(hLower, h); l.upper = c.F(hUpper, h);
+    l.bound = c.F(hNormalBound, h);
+    l.response = Response{c.F(hDualScale, h), c.F(hResidualScale, h)};
+    l.ratios = tangent_ratios(c.F(hMu1, h), c.F(hMu2, h));
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { l.dual[k] = c.F(hDual + k, h); l.res[k] = c.F(hRes + k, h); l.move[k] = c.F(hMove + k, h); l.step[k] = c.F(hStep + k, h); }
+    return l;
+}
+
+// TileLineDerivatives (:2048-2086); lane = head, heads beyond the first 64 go through `extra`
+__device__ __forceinline__ void line_terms(const HeadLine& l, float alpha, TileSum& row_slope, float& row_curvature, float& row_magnitude) {
+    const float sx = l.step[0], sy = l.step[1], sz = l.step[2];
+    float f[3] = {0.0f, 0.0f, 0.0f}, r[6] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    scalar_impulse(l.dual[0], l.rho, l.res[0] - fmaf(alpha, sx, l.move[0]), l.compliance, l.lower, l.upper, l.response, &f[0], &r[0]);
+    if (l.contact)
+        tangent_impulse(V3{l.dual[0], l.dual[1], l.dual[2]}, l.rho, l.res[1] - fmaf(alpha, sy, l.move[1]),
+                        l.res[2] - fmaf(alpha, sz, l.move[2]), l.bound, l.ratios, &f[1], &f[2], &r[1], &r[2], &r[5]);
+    tile_add_product(row_slope, f[0], sx);
+    tile_add_product(row_slope, f[1], sy);
+    tile_add_product(row_slope, f[2], sz);
+    row_magnitude += fabsf(f[0] * sx) + fabsf(f[1] * sy) + fabsf(f[2] * sz);
+    row_curvature += r[0] * sx * sx + r[1] * sy * sy + r[2] * sz * sz + 2.0f * r[5] * sy * sz + 2.0f * r[3] * sx * sy +
+                     2.0f * r[4] * sx * sz;
+}
+__device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& mine, float alpha, float inertial_slope, float inertial_curvature,
+                                 float* slope, float* curvature, float* magnitude) {
+    PROF_COUNT(c, 1);
+    TileSum row_slope{0.0f, 0.0f};
+    float row_curvature = 0.0f, row_magnitude = 0.0f;
+    if (mine.owned) line_terms(mine, alpha, row_slope, row_curvature, row_magnitude);
+    for (uint32_t h = c.lane + kWave; h < c.heads; h += kWave) {
+        const HeadLine extra = load_head_line(c, h);
+        if (extra.owned) line_terms(extra, alpha, row_slope, row_curvature, row_magnitude);
+    }
+    TileSum total{-row_slope.value, -row_slope.error};
+    if (c.lane == 0u) {
+        tile_add_product(total, alpha, inertial_curvature);
+        tile_add(total, inertial_slope);
+    }
+    *slope = wave_total(total);
+    *curvature = inertial_curvature + wave_sum(row_curvature);
+    *magnitude = fabsf(inertial_slope) + alpha * inertial_curvature + wave_sum(row_magnitude);
+}
+
+// SearchTileLine (:2089-2125)
+__device__ __forceinline__ float search_line(const Tile& c, float inertial_slope, float inertial_curvature) {
+    float slope = 0.0f, curvature = 0.0f, magnitude = 0.0f;
+    const HeadLine mine = load_head_line(c, c.lane);
+    line_derivatives(c, mine, 0.0f, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
+    const float initial = slope;
+    if (!(initial < 0.0f)) return 0.0f;
+    float low = 0.0f, high = 0.0f, alpha = 1.0f;
+    bool bounded = false;
+    for (uint32_t step = 0u; step < kLineSearchSteps; ++step) {
+        line_derivatives(c, mine, alpha, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
+        if (!isfinite(slope) || !isfinite(curvature)) {
+            high = alpha; bounded = true; alpha = 0.5f * (low + high);
+            continue;
+        }
+        if (fabsf(slope) <= fmaxf(kLineTolerance * -initial, kRoundings * FLT_EPSILON * magnitude)) return alpha;
+        if (slope < 0.0f) low = alpha;
+        else { high = alpha; bounded = true; }
+        if (bounded && high - low <= FLT_EPSILON * high) break;
+        float next = alpha - slope / curvature;
+        if (!(next > low && (!bounded || next < high))) next = bounded ? 0.5f * (low + high) : 2.0f * alpha;
+        alpha = next;
+    }
+    return low;
+}
+
+__device__ __forceinline__ void apply_moves(const Tile& c, float alpha) {
+    for (uint32_t h = c.lane; h < c.heads; h += kWave) {
+        if (c.U(hOwned, h) == 0u) continue;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) c.F(hMove + k, h) = fmaf(alpha, c.F(hStep + k, h), c.F(hMove + k, h));
+    }
+    __syncthreads();
+}
+
+// mass_step_i = sum_k M_ik d_k in coordinate order (:2177-2187, 2228-2238)
+template <int N>
+__device__ __forceinline__ float mass_times(const Tile& c, const float (&mrow)[N], float d) {
+    float* dvec = c.vec + 192;
+    dvec[c.lane] = d;
+    __syncthreads();
+    float out = 0.0f;
+    const float4* d4 = reinterpret_cast<const float4*>(dvec);
+#pragma unroll
+    for (int q = 0; q < N / 4; ++q) {
+        const float4 dv = d4[q];
+        out += mrow[4 * q] * dv.x; out += mrow[4 * q + 1] * dv.y; out += mrow[4 * q + 2] * dv.z; out += mrow[4 * q + 3] * dv.w;
+    }
+    __syncthreads();
+    return c.lane < c.n ? out : 0.0f;
+}
+
+// DescendTileBlock (:2145-2301).  `u` is lane i's block coordinate; `has_free` is false in the position pass.
+template <int N>
+__device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], float* u_io, float free_in, bool has_free, DataView d) {
+    const uint32_t lane = c.lane, n = c.n;
+    const bool coordinate = lane < n;
+    for (uint32_t h = lane; h < c.heads; h += kWave) {   // StartTileBlock (:1386-1397)
+        if (c.U(hOwned, h) == 0u) continue;
+        c.F(hNormalBound, h) = c.F(hDual, h);
+        c.F(hMove, h) = 0.0f; c.F(hMove + 1, h) = 0.0f; c.F(hMove + 2, h) = 0.0f;
+    }
+    __syncthreads();
+    const float start = coordinate ? *u_io : 0.0f;
+    const float free_v = coordinate && has_free ? free_in : 0.0f;
+    float u = start;
+    if (c.iteration == 0u && has_free) {   // first-sweep segment search (:2165-2209)
+        const float dd = coordinate ? free_v - u : 0.0f;
+        const float mass_step = mass_times<N>(c, mrow, dd);
+        TileSum curvature{0.0f, 0.0f};
+        if (coordinate) tile_add_product(curvature, dd, mass_step);
+        const float inertial_curvature = wave_total(curvature);
+        if (inertial_curvature > 0.0f && isfinite(inertial_curvature)) {
+            row_steps<N>(c, dd);
+            const float alpha = search_line(c, -inertial_curvature, inertial_curvature);
+            if (alpha > 0.0f) {
+                u = fmaf(alpha, dd, u);
+                apply_moves(c, alpha);
+            }
+        }
+    }
+    Failure failure = kFailNone;
+    float primal = FLT_MAX;
+    for (uint32_t step = 0u; step < kNewtonSteps; ++step) {
+        float force = 0.0f, inertia = 0.0f, dd = 0.0f;
+        bool converged = false;
+        failure = newton_direction<N>(c, mrow, u, free_v, &force, &inertia, &dd, &converged);
+        if (converged) primal = 0.0f;
+        if (failure != kFailNone || converged) break;
+        if (!coordinate) dd = 0.0f;
+        PROF_BEGIN(c, 8);
+        const float mass_step = mass_times<N>(c, mrow, dd);
+        PROF_END(c, 8);
+        TileSum decrement{0, 0}, slope{0, 0}, curvature{0, 0};
+        if (coordinate) {
+            tile_add_product(decrement, force, dd);
+            tile_add_product(slope, inertia, dd);
+            tile_add_product(curvature, dd, mass_step);
+        }
+        const float total_decrement = wave_total(decrement);
+        const float inertial_slope = wave_total(slope);
+        const float inertial_curvature = wave_total(curvature);
+        if (!isfinite(total_decrement) || !isfinite(inertial_slope) || !isfinite(inertial_curvature)) { failure = kFailDirection; break; }
+        if (!(total_decrement > 0.0f)) break;
+        PROF_BEGIN(c, 4);
+        row_steps<N>(c, dd);
+        PROF_END(c, 4);
+        PROF_BEGIN(c, 5);
+        const float alpha = search_line(c, inertial_slope, inertial_curvature);
+        PROF_END(c, 5);
+        const float after = fmaf(alpha, dd, u);
+        const bool rounded = __all(!coordinate || after == u);
+        if (!__all(!coordinate || isfinite(after))) { failure = kFailCandidate; break; }
+        primal = 0.0f;
+        if (coordinate && !rounded) primal = fmaxf(primal, fabsf(alpha * dd));
+        if (!(alpha > 0.0f)) break;
+        u = after;
+        apply_moves(c, alpha);
+        if (rounded) break;
+    }
+    for (uint32_t h = lane; h < c.heads; h += kWave) {   // EndTileBlock (:1400-1409)
+        if (c.U(hOwned, h) == 0u) continue;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) c.F(hRes + k, h) = c.F(hRes + k, h) - c.F(hMove + k, h);
+    }
+    __syncthreads();
+    if (failure != kFailNone) {
+        c.failed = true;
+        if (lane == 0u) d.env_status[c.env] |= kEnvStatusSolverFailure;
+    }
+    float moved = failure == kFailNone ? 0.0f : FLT_MAX;
+    if (coordinate) moved = fmaxf(moved, __uint_as_float(residual_bits(u - start)));
+    c.momentum = fmaxf(c.momentum, wave_max(moved));
+    if (failure != kFailNone) primal = FLT_MAX;
+    c.residual = fmaxf(c.residual, wave_max(primal));   // one block per environment: no coupled heads
+    if (coordinate) *u_io = u;
+}
+
+// MeasureTilePrimal (:2378-2489): the mass-normalised momentum balance in double
+template <int N>
+__device__ __forceinline__ void measure_primal(Tile& c, const float (&mrow)[N], float* velocity_io, float free_v, const float* lambda_env, uint32_t R,
+                               bool reconstruct, DataView d) {
+    const uint32_t lane = c.lane, n = c.n;
+    const bool coordinate = lane < n;
+    float* dvec = c.vec;
+    dvec[lane] = coordinate ? *velocity_io : 0.0f;
+    c.vec[64 + lane] = coordinate ? free_v : 0.0f;
+    __syncthreads();
+    double balance = 0.0;
+#pragma unroll
+    for (int j = 0; j < N; ++j) balance -= double(mrow[j]) * (double(dvec[j]) - c.vec[64 + j]);   // padded terms are exact zeros
+    for (uint32_t h = 0u; h < c.heads; ++h) {
+        if (c.U(hOwned, h) == 0u) continue;
+        const uint32_t local = c.U(hSlot, h) - c.env * R, stride = c.U(hStride, h), axes = c.U(hAxes, h);
+        const float ix = lambda_env[local], iy = axes == 3u ? lambda_env[local + stride] : 0.0f,
+                    iz = axes == 3u ? lambda_env[local + 2u * stride] : 0.0f;
+        if (!(ix != 0.0f || iy != 0.0f || iz != 0.0f)) continue;
+        if (!coordinate) continue;
+        const float* j = c.jac + (3u * h) * c.ldj;
+        balance += double(j[lane]) * ix;
+        if (axes == 3u) {
+            balance += double(j[c.ldj + lane]) * iy;
+            balance += double(j[2u * c.ldj + lane]) * iz;
+        }
+    }
+    __syncthreads();
+    const float force = float(balance);
+    const bool finite = __all(!coordinate || fabs(balance) <= double(FLT_MAX));
+    Failure failure = finite ? kFailNone : kFailEquation;
+    float direction = 0.0f;
+    if (failure == kFailNone) {
+        if (c.mass_valid) direction = solve_tile_mass<N>(c, force);
+        else failure = kFailFactor;
+    }
+    float residual = failure == kFailNone ? 0.0f : FLT_MAX;
+    if (failure != kFailNone && lane == 0u) d.env_status[c.env] |= kEnvStatusSolverFailure;
+    if (failure == kFailNone && coordinate) residual = fmaxf(residual, isfinite(direction) ? fabsf(direction) : FLT_MAX);
+    residual = wave_max(residual);
+    c.residual = fmaxf(c.residual, residual);
+    if (reconstruct && failure == kFailNone) {
+        if (!__all(!coordinate || isfinite(*velocity_io + direction))) { c.residual = FLT_MAX; return; }
+        if (coordinate) *velocity_io += direction;
+        c.momentum = fmaxf(c.momentum, residual);
+    }
+}
+
+// InitializeTileResiduals (:890-930) on the staged rows: residual = fl(rhs dt) - J u, products summed in coordinate order
+template <int N>
+__device__ __forceinline__ void initialize_residuals(const Tile& c, float velocity, const float* urows, float dt) {
+    float* dvec = c.vec;
+    dvec[c.lane] = c.lane < c.n ? velocity : 0.0f;
+    __syncthreads();
+    const float4* d4 = reinterpret_cast<const float4*>(dvec);
+    for (uint32_t h = c.lane; h < c.heads; h += kWave) {
+        const uint32_t slot = c.U(hSlot, h), stride = c.U(hStride, h), axes = c.U(hAxes, h);
+        for (uint32_t axis = 0u; axis < 3u; ++axis) {
+            float residual = 0.0f;
+            if (axis < axes) {
+                const float rhs = urows[size_t{slot + axis * stride} * kRowWords + 4u];
+                const float4* j4 = reinterpret_cast<const float4*>(c.jac + (3u * h + axis) * uint32_t(N));
+                float along = 0.0f;
+#pragma unroll
+                for (int q = 0; q < N / 4; ++q) {
+                    const float4 j = j4[q], dv = d4[q];
+                    along = along + j.x * dv.x; along = along + j.y * dv.y; along = along + j.z * dv.z; along = along + j.w * dv.w;
+                }
+                residual = rhs * dt - along;
+            }
+            c.F(hRes + axis, h) = residual;
+        }
+    }
+    __syncthreads();
+}
+
+struct DualMomentum { float t, beta; };
+
+// UpdateTileHeadDuals (:2493-2595); classes = {normal, tangent, joint}
+__device__ __forceinline__ void update_duals(const Tile& c, float* lambda_env, uint32_t R, const float* urows, DualMomentum* momentum, bool velocity,
+                             bool commit, float* classes) {
+    uint32_t steps[3] = {0u, 0u, 0u};
+    double restart = 0.0;
+    for (uint32_t h = c.lane; h < c.heads; h += kWave) {
+        const uint32_t slot = c.U(hSlot, h), local = slot - c.env * R, stride = c.U(hStride, h), axes = c.U(hAxes, h);
+        const bool contact = axes == 3u;
+        const float rho = c.F(hRho, h), compliance = c.F(hCompliance, h), lower = c.F(hLower, h), upper = c.F(hUpper, h);
+        const float mu1 = c.F(hMu1, h), mu2 = c.F(hMu2, h);
+        const Response response{c.F(hDualScale, h), c.F(hResidualScale, h)};
+        const V3 residual{c.F(hRes, h), c.F(hRes + 1, h), c.F(hRes + 2, h)};
+        const V3 base{c.F(hBase, h), c.F(hBase + 1, h), c.F(hBase + 2, h)};
+        const V3 tdual = commit ? V3{c.F(hDual, h), c.F(hDual + 1, h), c.F(hDual + 2, h)} : base;
+        float normal, ncurv;
+        scalar_impulse(tdual.x, rho, residual.x, compliance, lower, upper, response, &normal, &ncurv);
+        V3 dual{normal, 0.0f, 0.0f};
+        V3 rstep{0, 0, 0}, rpoint{0, 0, 0};
+        float rweight = 0.0f;
+        if (contact) {   // ProjectRowDual (block_descent.cu:799-804) with RelaxContactImpulse (augmented_row.hpp:128-138)
+            float fy, fz, cyy, czz, cyz;
+            tangent_impulse(tdual, rho, residual.y, residual.z, normal, mu1, mu2, &fy, &fz, &cyy, &czz, &cyz);
+            const V3 next{normal, fy, fz};
+            V3 last_step{0, 0, 0}, last_point{0, 0, 0};
+            float last_weight = 0.0f;
+            if (commit) {
+                last_step = V3{c.F(hRelaxStep, h), c.F(hRelaxStep + 1, h), c.F(hRelaxStep + 2, h)};
+                last_weight = c.F(hRelaxWeight, h);
+                last_point = V3{c.F(hRelaxPoint, h), c.F(hRelaxPoint + 1, h), c.F(hRelaxPoint + 2, h)};
+            }
+            const V3 step{next.x - tdual.x, next.y - tdual.y, next.z - tdual.z};
+            const V3 change{step.x - last_step.x, step.y - last_step.y, step.z - last_step.z};
+            const V3 moved = sub3(tdual, last_point);
+            const float square = change.x * change.x + change.y * change.y + change.z * change.z;
+            const float along = -(moved.x * change.x + moved.y * change.y + moved.z * change.z);
+            float weight = 1.0f;
+            if (last_weight > 0.0f && along > 0.0f && square > 0.0f) weight = fminf(1.0f, along / square);
+            rstep = step; rweight = weight; rpoint = tdual;
+            dual = V3{tdual.x + weight * step.x, tdual.y + weight * step.y, tdual.z + weight * step.z};
+        }
+        // MultiplierSteps (block_descent.cu:761-770)
+        float step_normal = response.residual_scale > 0.0f && response.dual_scale != 0.0f
+            ? fabsf(dual.x - tdual.x) / response.residual_scale : 0.0f;
+        float step_tangent = 0.0f;
+        if (contact) {
+            const float fs = fmaxf(mu1, mu2);
+            const float m1 = mu1 <= 0.0f ? 0.0f : mu1 / fs, m2 = mu2 <= 0.0f ? 0.0f : mu2 / fs;
+            const float first = m1 > 0.0f && rho > 0.0f ? (dual.y - tdual.y) / (rho * m1 * m1) : 0.0f;
+            const float second = m2 > 0.0f && rho > 0.0f ? (dual.z - tdual.z) / (rho * m2 * m2) : 0.0f;
+            step_tangent = hypotf(first, second);
+        }
+        if (!commit && response.residual_scale > 0.0f) step_normal = fabsf(dual.x - tdual.x) / response.residual_scale;
+        const V3 physical = commit ? dual : tdual;
+        if (!contact) {
+            const bool normal_row = (__float_as_uint(urows[size_t{slot} * kRowWords]) & kRowContactNormal) != 0u;
+            const float rate = -residual.x + compliance * physical.x;
+            const float violation = physical.x > 0.0f ? fabsf(rate) : fmaxf(-rate, 0.0f);
+            const float value = normal_row ? fmaxf(step_normal, violation) : step_normal;
+            if (normal_row) steps[0] = max(steps[0], residual_bits(value));
+            else steps[2] = max(steps[2], residual_bits(value));
+        } else {
+            if (commit) {
+                c.F(hRelaxStep, h) = rstep.x; c.F(hRelaxStep + 1, h) = rstep.y; c.F(hRelaxStep + 2, h) = rstep.z;
+                c.F(hRelaxWeight, h) = rweight;
+                c.F(hRelaxPoint, h) = rpoint.x; c.F(hRelaxPoint + 1, h) = rpoint.y; c.F(hRelaxPoint + 2, h) = rpoint.z;
+                lambda_env[local + stride] = dual.y;
+                lambda_env[local + 2u * stride] = dual.z;
+            }
+            const V3 v{-residual.x + compliance * physical.x, -residual.y, -residual.z};
+            steps[0] = max(steps[0], residual_bits(physical.x > 0.0f ? fabsf(v.x) : fmaxf(-v.x, 0.0f)));
+            steps[1] = max(steps[1], residual_bits(fmaxf(step_tangent, fmaxf(along_axis(physical.y, v.y), along_axis(physical.z, v.z)))));
+        }
+        if (!commit) continue;
+        if (velocity) lambda_env[local] = dual.x;
+        const bool extrapolate = contact || response.dual_scale != 0.0f;
+        if (extrapolate) {   // MultiplierMetric (block_descent.cu:790-795) and MultiplierMomentumRestart (augmented_row.hpp:119-124)
+            const float friction = fmaxf(mu1, mu2);
+            const float first = contact && mu1 > 0.0f ? mu1 / friction : 0.0f;
+            const float second = contact && mu2 > 0.0f ? mu2 / friction : 0.0f;
+            const V3 metric{response.residual_scale, rho * first * first, rho * second * second};
+            restart += (metric.x > 0.0f ? (double(tdual.x) - dual.x) * (double(dual.x) - base.x) / metric.x : 0.0) +
+                       (metric.y > 0.0f ? (double(tdual.y) - dual.y) * (double(dual.y) - base.y) / metric.y : 0.0) +
+                       (metric.z > 0.0f ? (double(tdual.z) - dual.z) * (double(dual.z) - base.z) / metric.z : 0.0);
+        }
+        if (momentum != nullptr) { c.F(hMove, h) = base.x; c.F(hMove + 1, h) = base.y; c.F(hMove + 2, h) = base.z; }
+        c.F(hDual, h) = dual.x; c.F(hDual + 1, h) = dual.y; c.F(hDual + 2, h) = dual.z;
+        c.F(hBase, h) = dual.x; c.F(hBase + 1, h) = dual.y; c.F(hBase + 2, h) = dual.z;
+    }
+    classes[0] = __uint_as_float(wave_max_u(steps[0]));
+    classes[1] = __uint_as_float(wave_max_u(steps[1]));
+    classes[2] = __uint_as_float(wave_max_u(steps[2]));
+    restart = wave_sum_d(restart);
+    if (momentum != nullptr) {
+        // AdvanceDualMomentum (block_descent.cu:780-788) and ExtrapolateDual (:808-820)
+        if (restart > 0.0) momentum->t = 1.0f;
+        const float t = 0.5f * (1.0f + sqrtf(fmaf(4.0f * momentum->t, momentum->t, 1.0f)));
+        momentum->beta = (momentum->t - 1.0f) / t;
+        momentum->t = t;
+        for (uint32_t h = c.lane; h < c.heads; h += kWave) {
+            const bool contact = c.U(hAxes, h) == 3u;
+            const bool extrapolate = contact || c.F(hDualScale, h) != 0.0f;
+            const float beta = extrapolate ? momentum->beta : 0.0f;
+            const V3 base{c.F(hMove, h), c.F(hMove + 1, h), c.F(hMove + 2, h)};
+            const V3 next{c.F(hBase, h), c.F(hBase + 1, h), c.F(hBase + 2, h)};
+            V3 out = next;
+            if (beta != 0.0f) {
+                V3 y{fmaf(beta, next.x - base.x, next.x), fmaf(beta, next.y - base.y, next.y), fmaf(beta, next.z - base.z, next.z)};
+                y.x = fminf(fmaxf(y.x, c.F(hLower, h)), c.F(hUpper, h));
+                if (!contact) out = V3{y.x, 0.0f, 0.0f};
+                else {
+                    const float mu1 = c.F(hMu1, h), mu2 = c.F(hMu2, h);
+                    const float first = mu1 > 0.0f ? y.y / mu1 : 0.0f, second = mu2 > 0.0f ? y.z / mu2 : 0.0f;
+                    const float slip = hypotf(first, second), radius = fmaxf(y.x, 0.0f);
+                    const float scale = slip > radius ? radius / slip : 1.0f;
+                    out = V3{y.x, mu1 > 0.0f ? y.y * scale : 0.0f, mu2 > 0.0f ? y.z * scale : 0.0f};
+                }
+            }
+            c.F(hDual, h) = out.x; c.F(hDual + 1, h) = out.y; c.F(hDual + 2, h) = out.z;
+        }
+    }
+    __syncthreads();
+}
+
+__host__ __device__ inline uint32_t PaddedWidth(uint32_t n) { return (n + 3u) & ~3u; }
+__host__ __device__ inline uint32_t FactorRegionFloats(uint32_t n) {
+    const uint32_t N = PaddedWidth(n);
+    return 2u * N * (N + 1u);   // a multiple of 4 since N is
+}
+__host__ __device__ inline uint32_t SolverLdsFloats(uint32_t n, uint32_t cap) {
+    const uint32_t N = PaddedWidth(n);
+    return FactorRegionFloats(n) + 3u * cap * N + ((hFieldCount * cap + 3u) & ~3u) + 256u;
+}
+
+// DescendTile (:2941-3087)
+template <int N>
+__global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(N <= 36 ? 2 : 1, N <= 36 ? 2 : 1)))
+BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint32_t cap) {
+    extern __shared__ __align__(16) float lds[];
+    const uint32_t env = blockIdx.x, lane = threadIdx.x;
+    const uint32_t R = p.rows_per_env, md = p.max_dof, n = m.dof, nl = m.links_per_env, S = p.contact_slots_per_env;
+    Tile c;
+    c.env = env; c.lane = lane; c.n = n; c.ld = uint32_t(N) + 1u; c.ldj = uint32_t(N); c.cap = cap; c.heads = 0u; c.iteration = 0u;
+    c.tolerance = p.velocity_tolerance; c.failed = false; c.momentum = 0.0f; c.residual = 0.0f;
+    c.mass_inverse = 0.0f; c.mass_valid = false;
+#ifdef NKH_SOLVER_PROFILE
+    for (int i = 0; i < 10; ++i) c.prof[i] = 0;
+    for (int i = 0; i < 4; ++i) c.prof_count[i] = 0u;
+#endif
+    PROF_BEGIN(c, 9);
+    PROF_BEGIN(c, 0);
+    c.mfac = lds;
+    c.hfac = c.mfac + uint32_t(N) * c.ld;
+    c.jac = lds + FactorRegionFloats(n);
+    c.fields = c.jac + 3u * cap * c.ldj;
+    c.vec = c.fields + ((hFieldCount * cap + 3u) & ~3u);
+    const bool coordinate = lane < n;
+    const float* urows = d.urows;
+    float* lambda_env = d.lambda + size_t{env} * R;
+    const size_t lbase = size_t{env} * nl;
+    // InitializeTile (:1327-1350): the free velocity and the constraint velocity carried from the previous solve
+    uint32_t my_link = 0u, my_component = kInvalid;
+    float free_v = 0.0f, velocity = 0.0f;
+    if (coordinate) {
+        my_link = m.dof_link[lane]; my_component = m.dof_component[lane];
+        const float value = my_component == kInvalid ? d.qdot[lbase + my_link] : d.link_velocity[(lbase + my_link) * 6u + my_component];
+        const float carried = d.solver_velocity[size_t{env} * md + lane] - d.solver_free[size_t{env} * md + lane];
+        free_v = value;
+        velocity = value + (isfinite(carried) ? carried : 0.0f);
+    }
+    // ListTileHeads (:1250-1296): active rows that are not block tangents, in slot order
+    const uint32_t previous = d.contact_row_extent[2u * env], current = d.contact_row_extent[2u * env + 1u];
+    const uint32_t bound = previous == 0u || current == 0u ? p.contact_rows_per_env : min(max(previous, current) - 1u, p.contact_rows_per_env);
+    const uint32_t total = bound + (R - p.contact_rows_per_env);
+    uint32_t heads = 0u;
+    bool overflow = false;
+    for (uint32_t base = 0u; base < total; base += kWave) {
+        const uint32_t index = base + lane;
+        const uint32_t slot = env * R + (index < bound ? index : p.contact_rows_per_env + (index - bound));
+        bool head = false;
+        if (index < total) {
+            const uint32_t flags = __float_as_uint(urows[size_t{slot} * kRowWords]);
+            head = (flags & kRowActive) != 0u && (flags & kRowBlockTangent) == 0u;
+        }
+        const uint64_t mask = __ballot(head);
+        if (head) {
+            const uint32_t at = heads + __popcll(mask & ((uint64_t{1} << lane) - 1u));
+            if (at < cap) c.U(hSlot, at) = slot; else overflow = true;
+        }
+        heads += __popcll(mask);
+    }
+    if (__any(overflow)) {   // more heads than the staged LDS holds: fail loudly, solve the ones that fit
+        heads = cap;
+        if (lane == 0u) d.env_status[env] |= kEnvStatusSolverFailure;
+    }
+    c.heads = heads;
+    __syncthreads();
+    // stage Jacobian rows: the sum of the articulated sides' chain rows (TileBlock::Jacobian :555-573, CopyTileRows :836-869)
+    for (uint32_t h = 0u; h < heads; ++h) {
+        const uint32_t slot = c.U(hSlot, h);
+        const uint32_t flags = __float_as_uint(urows[size_t{slot} * kRowWords]);
+        const uint32_t stride = __float_as_uint(urows[size_t{slot} * kRowWords + 2u]);
+        const uint32_t axes = (flags & kRowBlockNormal) != 0u ? 3u : 1u;
+        for (uint32_t axis = 0u; axis < 3u; ++axis) {
+            float value = 0.0f;
+            if (axis < axes && coordinate) {
+                const uint32_t rs = slot + axis * stride;
+                const uint32_t kind_a = __float_as_uint(urows[size_t{rs} * kRowWords + 10u]);
+                const uint32_t kind_b = __float_as_uint(urows[size_t{rs} * kRowWords + 18u]);
+                if (kind_a == kSideArtic) value += d.chain_jacobian[size_t{rs} * md + lane];
+                if (kind_b == kSideArtic) value += d.chain_jacobian_b[size_t{rs} * md + lane];
+            }
+            if (lane < c.ldj) c.jac[(3u * h + axis) * c.ldj + lane] = value;   // padded columns hold zeros
+        }
+    }
+    __syncthreads();
+    // TileInertialResponse (:709-739): J M^-1 J^T of every head's first row through the stored LDL^T factor
+    // (ForwardMass + MassDot, articulation_mass.cuh:414-431).  lane = DoF: the unit-lower factor row sits in
+    // registers with zeros from the diagonal on, each y_j travels as a scalar lane read, so row i subtracts
+    // L_ij y_j for j = 0, 1, ... exactly as the serial loop does; the ordered sum of y_i^2 / D_i follows the same way.
+    {
+        const float* factor = d.m_factor + size_t{env} * md * md;
+        for (uint32_t e = lane; e < n * n; e += kWave) c.hfac[(e / n) * c.ld + e % n] = factor[size_t{e / n} * md + e % n];
+        __syncthreads();
+        float lrow[N];
+#pragma unroll
+        for (int k = 0; k < N; ++k) lrow[k] = coordinate && uint32_t(k) < lane ? c.hfac[lane * c.ld + k] : 0.0f;
+        const float pivot = coordinate ? c.hfac[lane * c.ld + lane] : 1.0f;
+        __syncthreads();
+        for (uint32_t h = 0u; h < heads; ++h) {
+            const uint32_t slot = c.U(hSlot, h);
+            const float* row = urows + size_t{slot} * kRowWords;
+            const uint32_t kind_a = __float_as_uint(row[10]), index_a = __float_as_uint(row[11]);
+            const uint32_t kind_b = __float_as_uint(row[18]), index_b = __float_as_uint(row[19]);
+            const bool shared = kind_a == kind_b && index_a == index_b;
+            float shares[2] = {0.0f, 0.0f};
+            for (uint32_t side = 0u; side < (shared ? 1u : 2u); ++side) {
+                float contribution = 0.0f;
+                if ((side == 0u ? kind_a : kind_b) == kSideArtic) {
+                    float a = 0.0f;
+                    if (coordinate) {
+                        a = (side == 0u ? d.chain_jacobian : d.chain_jacobian_b)[size_t{slot} * md + lane];
+                        if (shared) a += d.chain_jacobian_b[size_t{slot} * md + lane];
+                    }
+#pragma unroll
+                    for (int j = 0; j < N; ++j) a -= lrow[j] * lane_value(a, j);
+                    const float term = coordinate ? a * a / pivot : 0.0f;
+#pragma unroll
+                    for (int i = 0; i < N; ++i) contribution += lane_value(term, i);
+                }
+                shares[side] = contribution;
+            }
+            if (lane == 0u) { c.F(hRes, h) = shares[0]; c.F(hRes + 1, h) = shares[1]; }
+        }
+        __syncthreads();
+    }
+    // InitializeTileHead (:743-797), lane = head
+    for (uint32_t base = 0u; base < heads; base += kWave) {
+        const uint32_t h = base + lane;
+        if (h < heads) {
+            const uint32_t slot = c.U(hSlot, h);
+            const float* row = urows + size_t{slot} * kRowWords;
+            const uint32_t flags = __float_as_uint(row[0]), stride = __float_as_uint(row[2]);
+            const uint32_t axes = (flags & kRowBlockNormal) != 0u ? 3u : 1u;
+            const uint32_t kind_a = __float_as_uint(row[10]), kind_b = __float_as_uint(row[18]);
+            const float shares[2] = {c.F(hRes, h), c.F(hRes + 1, h)};
+            const bool valid = shares[0] >= 0.0f && isfinite(shares[0]) && shares[1] >= 0.0f && isfinite(shares[1]);
+            float response = shares[0] + shares[1];
+            const float coupling = shares[0] * shares[1], largest = fmaxf(shares[0], shares[1]);
+            if (!(valid && isfinite(response))) response = nanf("");
+            const float coupled = coupling > 0.0f ? (response + sqrtf(response * response + 12.0f * coupling)) / (6.0f * coupling) : FLT_MAX;
+            const float capv = kPenaltyConditionCap / largest;
+            float rho = response > 0.0f ? fminf(capv, coupled) : 0.0f;
+            if (!(response == 0.0f || (response > 0.0f && rho > 0.0f && rho <= FLT_MAX))) {
+                atomicOr(d.env_status + env, kEnvStatusSolverFailure);
+                rho = nanf("");
+            }
+            d.solver_penalty[slot] = rho;
+            const float compliance = row[5];
+            const Response sr = scalar_response(rho, compliance);
+            const uint32_t local = slot - env * R;
+            c.U(hStride, h) = stride; c.U(hAxes, h) = axes;
+            c.U(hOwned, h) = (kind_a == kSideArtic || kind_b == kSideArtic) ? 1u : 0u;
+            c.F(hRho, h) = rho; c.F(hCompliance, h) = compliance; c.F(hLower, h) = row[6]; c.F(hUpper, h) = row[7];
+            c.F(hMu1, h) = row[8]; c.F(hMu2, h) = row[9]; c.F(hNormalBound, h) = 0.0f;
+            c.F(hDualScale, h) = sr.dual_scale; c.F(hResidualScale, h) = sr.residual_scale;
+            const float dx = lambda_env[local], dy = axes == 3u ? lambda_env[local + stride] : 0.0f,
+                        dz = axes == 3u ? lambda_env[local + 2u * stride] : 0.0f;
+            c.F(hDual, h) = dx; c.F(hDual + 1, h) = dy; c.F(hDual + 2, h) = dz;
+            c.F(hBase, h) = dx; c.F(hBase + 1, h) = dy; c.F(hBase + 2, h) = dz;
+#pragma unroll
+            for (int k = 0; k < 3; ++k) { c.F(hRes + k, h) = 0.0f; c.F(hMove + k, h) = 0.0f; c.F(hStep + k, h) = 0.0f; c.F(hRelaxStep + k, h) = 0.0f; c.F(hRelaxPoint + k, h) = 0.0f; }
+            c.F(hRelaxWeight, h) = 0.0f;
+        }
+    }
+    __syncthreads();
+    // StageTileMass (:2127-2142): the mass rows go to registers through a coalesced pass over LDS (the head setup's
+    // scratch is dead by now); rows and columns n..N-1 are those of the identity.  Then the one factorisation.
+    float mrow[N];
+    for (uint32_t e = lane; e < n * n; e += kWave) c.hfac[(e / n) * c.ld + e % n] = d.m[size_t{env} * md * md + size_t{e / n} * md + e % n];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < N; ++k)
+        mrow[k] = coordinate && uint32_t(k) < n ? c.hfac[lane * c.ld + k] : (lane == uint32_t(k) && lane < uint32_t(N) ? 1.0f : 0.0f);
+    __syncthreads();
+    c.mass_valid = factor_mass<N>(c, mrow);
+    initialize_residuals<N>(c, velocity, urows, p.dt);
+    PROF_END(c, 0);
+    float residual4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    uint32_t sweeps = 0u;
+    DualMomentum momentum{1.0f, 0.0f};
+    const float tol = c.tolerance;
+    while (sweeps < p.iterations) {
+        c.iteration = sweeps++;
+        c.momentum = 0.0f; c.residual = 0.0f;
+        PROF_COUNT(c, 2);
+        descend_block<N>(c, mrow, &velocity, free_v, true, d);
+        float rowsr[3];
+        PROF_BEGIN(c, 6);
+        update_duals(c, lambda_env, R, urows, &momentum, true, true, rowsr);
+        PROF_END(c, 6);
+        PROF_BEGIN(c, 7);
+        if (sweeps == p.iterations || fmaxf(fmaxf(rowsr[0], rowsr[1]), fmaxf(rowsr[2], c.residual)) < tol)
+            measure_primal<N>(c, mrow, &velocity, free_v, lambda_env, R, false, d);
+        PROF_END(c, 7);
+        if (fmaxf(fmaxf(rowsr[0], rowsr[1]), rowsr[2]) < tol && c.residual >= tol && c.residual < FLT_MAX) {
+            measure_primal<N>(c, mrow, &velocity, free_v, lambda_env, R, true, d);
+            if (c.residual < FLT_MAX) {
+                initialize_residuals<N>(c, velocity, urows, p.dt);
+                update_duals(c, lambda_env, R, urows, nullptr, true, false, rowsr);
+                c.residual = 0.0f;
+                measure_primal<N>(c, mrow, &velocity, free_v, lambda_env, R, false, d);
+            }
+        }
+        residual4[0] = rowsr[0]; residual4[1] = rowsr[1]; residual4[2] = rowsr[2]; residual4[3] = c.residual;
+        const float largest = fmaxf(fmaxf(rowsr[0], rowsr[1]), fmaxf(rowsr[2], c.residual));
+        if (largest < tol || largest == FLT_MAX) break;
+    }
+    if (lane < 4u)
+        d.solver_residual[size_t{env} * 4u + lane] =
+            lane == 0u ? residual4[0] : lane == 1u ? residual4[1] : lane == 2u ? residual4[2] : residual4[3];
+    if (lane == 0u) d.vbd_velocity_sweep_count[env] = sweeps;
+#ifdef NKH_SOLVER_PROFILE
+    PROF_END(c, 9);
+    if (lane == 0u) {
+        for (int i = 0; i < 10; ++i) d.solver_penalty[size_t{env} * R + i] = float(c.prof[i]);
+        for (int i = 0; i < 4; ++i) d.solver_penalty[size_t{env} * R + 10 + i] = float(c.prof_count[i]);
+    }
+#endif
+    // the block velocities persist for the next solve's carried start
+    if (lane < md) {
+        d.solver_velocity[size_t{env} * md + lane] = coordinate ? velocity : 0.0f;
+        d.solver_free[size_t{env} * md + lane] = coordinate ? free_v : 0.0f;
+    }
+    // FinishTile (:2607-2650)
+    const bool invalid = __any(coordinate && !(fabsf(velocity) <= FLT_MAX));
+    if (!invalid) {
+        if (lane < md) d.qdot_flat[size_t{env} * md + lane] = coordinate ? velocity : 0.0f;
+        if (coordinate) {
+            if (my_component == kInvalid) d.qdot[lbase + my_link] = velocity;
+            else d.link_velocity[(lbase + my_link) * 6u + my_component] = velocity;
+        }
+    } else if (lane == 0u) d.env_status[env] |= kEnvStatusSolverFailure;
+    // split-impulse position pass (:3059-3077; MarkTilePositions :2673-2708; PositionRowBias block_descent.cu:1734-1753)
+    if (p.position_iterations != 0u) {
+        float* qvec = c.vec + 128;
+        qvec[lane] = coordinate ? velocity : 0.0f;   // the final generalized velocity, as qdot_flat
+        __syncthreads();
+        bool push = false;
+        for (uint32_t h = lane; h < heads; h += kWave) {
+            const uint32_t slot = c.U(hSlot, h);
+            const float* row = urows + size_t{slot} * kRowWords;
+            const uint32_t flags = __float_as_uint(row[0]);
+            const float penetration = d.row_penetration[slot];
+            const bool speculative = (flags & kRowSpeculative) != 0u;
+            const float slop = speculative ? 0.0f : p.position_slop;
+            const bool position = (flags & (kRowFriction | kRowVelocityOnly | kRowMuJoCo)) == 0u &&
+                (speculative || penetration > slop || c.F(hDual, h) != 0.0f);
+            float bias = 0.0f, rounding = 0.0f;
+            if (position) {
+                const float pen = fmaxf(penetration - slop, 0.0f);
+                if (speculative) {
+                    // the contact slot whose normal rows hold this row (MapRowContactsKernel, block_descent.cu:1756-1767)
+                    const uint32_t group_first = __float_as_uint(row[1]), points = __float_as_uint(row[2]);
+                    uint32_t contact = 0u;
+                    for (uint32_t s = 0u; s < S; ++s)
+                        if (d.ucontact_row_range[(size_t{env} * S + s) * 2u] == group_first &&
+                            d.ucontact_row_range[(size_t{env} * S + s) * 2u + 1u] > 0u) contact = env * S + s;
+                    const size_t point = size_t{contact} * 4u + (slot - group_first) % points;
+                    const double depth = double(d.ucontact_depth[point]) - slop;
+                    const double reserve = double(penetration) - d.ucontact_depth[point];
+                    const double correction = p.position_beta * fmax(depth, 0.0) + reserve;
+                    const double target = fmin(depth, 0.0) + correction;
+                    double vel = 0.0;   // RowVelocity (block_descent.cu:1051-1082) per articulated side
+                    const uint32_t kind_a = __float_as_uint(row[10]), kind_b = __float_as_uint(row[18]);
+                    if (kind_a == kSideArtic) {
+                        double value = 0.0;
+                        for (uint32_t k = 0u; k < n; ++k) value += double(d.chain_jacobian[size_t{slot} * md + k]) * qvec[k];
+                        vel += value;
+                    }
+                    if (kind_b == kSideArtic) {
+                        double value = 0.0;
+                        for (uint32_t k = 0u; k < n; ++k) value += double(d.chain_jacobian_b[size_t{slot} * md + k]) * qvec[k];
+                        vel += value;
+                    }
+                    const double limit = fmin(correction / p.dt, double(p.position_max_velocity));
+                    const double absorbed = target > 0.0 ? 0.0 : fmax(reserve, 0.0) / p.dt;
+                    bias = float(fmin(target / p.dt - vel, limit));
+                    rounding = float(absorbed);
+                } else {
+                    const float correction = p.position_beta * pen + fmaxf(pen - pen, 0.0f);
+                    bias = fminf(correction / p.dt, p.position_max_velocity);
+                }
+            }
+            if (!position) c.U(hOwned, h) = 0u;
+            const Response sr = scalar_response(c.F(hRho, h), 0.0f);
+            c.U(hAxes, h) = 1u;
+            c.F(hCompliance, h) = 0.0f; c.F(hLower, h) = 0.0f; c.F(hUpper, h) = FLT_MAX;
+            c.F(hDualScale, h) = sr.dual_scale; c.F(hResidualScale, h) = sr.residual_scale;
+            c.F(hRes, h) = bias; c.F(hRes + 1, h) = 0.0f; c.F(hRes + 2, h) = 0.0f;
+            c.F(hDual, h) = 0.0f; c.F(hDual + 1, h) = 0.0f; c.F(hDual + 2, h) = 0.0f;
+            push = push || bias > rounding;
+        }
+        push = __any(push);
+        __syncthreads();
+        float pseudo = 0.0f;
+        if (push) {
+            const uint32_t positions = 1u;   // no head couples two moving blocks here, so one solve (:2716)
+            for (uint32_t iteration = 0u; iteration < positions; ++iteration) {
+                c.iteration = sweeps + iteration;
+                descend_block<N>(c, mrow, &pseudo, 0.0f, false, d);
+            }
+        }
+        // FinishTilePositions (:2720-2744)
+        if (coordinate) {
+            if (my_component == kInvalid) d.qdot_pseudo[lbase + my_link] = pseudo;
+            else d.link_velocity_pseudo[(lbase + my_link) * 6u + my_component] = pseudo;
+        }
+    }
+}
+
+}  // namespace solver
+}  // namespace nkh

@@ -1,0 +1,10 @@
+// Instantiations of the block-descent kernel for padded widths 28, 32, 36.
+#include "ops_solver_kernel.h"
+
+namespace nkh {
+namespace solver {
+template __global__ void BlockDescentTileKernel<28>(ModelView, DataView, BlockDescentSolveParams, uint32_t);
+template __global__ void BlockDescentTileKernel<32>(ModelView, DataView, BlockDescentSolveParams, uint32_t);
+template __global__ void BlockDescentTileKernel<36>(ModelView, DataView, BlockDescentSolveParams, uint32_t);
+}  // namespace solver
+}  // namespace nkh
