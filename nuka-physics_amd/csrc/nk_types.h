@@ -97,6 +97,7 @@ struct DataView {
     uint32_t *env_status, *vbd_velocity_sweep_count;
     float *solver_residual, *solver_penalty;
     float *solver_velocity, *solver_free;   // block velocities kept between solves (carried constraint velocity)
+    uint32_t *solver_cost, *tile_order;     // last solve's work per environment; launch order of the next solve (costliest first)
     float *snapshot;                        // SnapshotState / RestoreState storage
 };
 

@@ -23,6 +23,34 @@ uint32_t SolverHeadCapacity(const ModelView& m, uint32_t slots, size_t lds_budge
 
 namespace {
 using namespace solver;
+
+// OrderTilesKernel (block_descent_tile.cuh:3097-3121 orders tiles for its persistent kernel; here the order feeds the
+// grid): environments sorted by the work their previous solve took, costliest first, so that the few long solves
+// start at once instead of trailing the launch.  One workgroup, counting sort on a 256-level key; the order inside a
+// level is arbitrary, which changes when an environment runs and nothing it computes.
+__global__ void __launch_bounds__(1024) OrderTilesKernel(DataView d, uint32_t env_count) {
+    __shared__ uint32_t bins[256];
+    __shared__ uint32_t top;
+    const uint32_t t = threadIdx.x;
+    if (t < 256u) bins[t] = 0u;
+    if (t == 0u) top = 0u;
+    __syncthreads();
+    uint32_t largest = 0u;
+    for (uint32_t e = t; e < env_count; e += 1024u) largest = max(largest, d.solver_cost[e]);
+    atomicMax(&top, largest);
+    __syncthreads();
+    const uint32_t scale = top / 256u + 1u;
+    for (uint32_t e = t; e < env_count; e += 1024u) atomicAdd(&bins[255u - min(d.solver_cost[e] / scale, 255u)], 1u);
+    __syncthreads();
+    if (t == 0u) {
+        uint32_t running = 0u;
+        for (uint32_t b = 0u; b < 256u; ++b) { const uint32_t count = bins[b]; bins[b] = running; running += count; }
+    }
+    __syncthreads();
+    for (uint32_t e = t; e < env_count; e += 1024u) d.tile_order[atomicAdd(&bins[255u - min(d.solver_cost[e] / scale, 255u)], 1u)] = e;
+}
+
+
 using SolverKernel = void (*)(ModelView, DataView, BlockDescentSolveParams, uint32_t);
 // One instantiation per padded width.
 const SolverKernel kSolverKernels[16] = {
@@ -49,6 +77,7 @@ Status OpBlockDescentSolve(const ModelView& m, const DataView& d, const void* pa
     const uint32_t cap = SolverHeadCapacity(m, p->contact_slots_per_env == 0u ? 1u : p->contact_slots_per_env, budget);
     if (cap == 0u) return Status::InvalidArgument;
     const size_t lds = size_t{solver::SolverLdsFloats(m.dof, cap)} * sizeof(float);
+    hipLaunchKernelGGL(OrderTilesKernel, dim3(1), dim3(1024), 0, stream, d, p->env_count);
     hipLaunchKernelGGL(kSolverKernels[solver::PaddedWidth(m.dof) / 4u - 1u], dim3(p->env_count), dim3(solver::kWave), lds, stream, m, d, *p, cap);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }

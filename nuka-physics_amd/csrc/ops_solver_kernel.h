@@ -22,6 +22,11 @@ namespace nkh {
 namespace solver {
 
 constexpr int kWave = 64;
+// Widths up to this run two waves per SIMD (at most 256 registers each); wider rows need the whole register file.
+#ifndef NKH_TWO_WAVE_WIDTH
+#define NKH_TWO_WAVE_WIDTH 36
+#endif
+constexpr int kTwoWaveWidth = NKH_TWO_WAVE_WIDTH;
 constexpr uint32_t kNewtonSteps = 16u;        // block_descent_dense.cuh:14
 constexpr uint32_t kLineSearchSteps = 32u;    // block_descent_dense.cuh:15
 constexpr float kLineTolerance = 1.0e-6f;     // block_descent_dense.cuh:17
@@ -163,6 +168,7 @@ struct Tile {
     float* fields;   // hFieldCount x cap
     float* vec;      // 4 x 64 scratch vectors, 16-byte aligned
     float mass_inverse;   // 1 / diagonal of the mass factor, lane = row
+    mutable uint32_t work;   // Newton steps and line probes of this solve, the next solve's scheduling key
     bool mass_valid;
     float momentum, residual;
     bool failed;
@@ -187,6 +193,14 @@ __device__ __forceinline__ void head_response(const Tile& c, uint32_t h, float m
                     c.F(hNormalBound, h), c.F(hMu1, h), c.F(hMu2, h), &f[1], &f[2], &cv[1], &cv[2], &cv[5]);
 }
 
+// Lane predicates (lane == k, lane > j, ...) are invariant over the whole solve; hoisted out of its loops they would
+// occupy hundreds of scalar registers and spill.  Passing the lane index through this makes each use site compute
+// its own predicate where it needs it.
+__device__ __forceinline__ uint32_t local_lane(uint32_t lane) {
+    asm volatile("" : "+v"(lane));
+    return lane;
+}
+
 // A lane's value of `v` for a lane index that is a compile-time constant at every call site: a scalar lane read.
 __device__ __forceinline__ float lane_value(float v, int lane) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
@@ -198,6 +212,7 @@ __device__ __forceinline__ float lane_value(float v, int lane) {
 // built with its compiler's default contraction, so it fuses these too).  Uniform result: false on a bad pivot.
 template <int N>
 __device__ __forceinline__ bool factor_rows(uint32_t lane, float (&row)[N], float* inverse_out) {
+    lane = local_lane(lane);
     bool valid = true;
     float inverse = 0.0f;
     // The pivot's square root and reciprocal are a long dependent chain; column k + 1 is brought up to date first
@@ -217,8 +232,17 @@ __device__ __forceinline__ bool factor_rows(uint32_t lane, float (&row)[N], floa
             root = sqrtf(valid ? pivot : 1.0f);
             scale = 1.0f / root;
         }
+        // lane reads in batches of eight ahead of their multiply-adds: a scalar read has to settle for two cycles
+        // before an arithmetic instruction may use it, and the next reads fill that gap
 #pragma unroll
-        for (int j = k + 2; j < N; ++j) row[j] = fmaf(-row[k], lane_value(row[k], j), row[j]);
+        for (int j0 = k + 2; j0 < N; j0 += 8) {
+            float l[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) l[t] = j0 + t < N ? lane_value(row[k], j0 + t) : 0.0f;
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                if (j0 + t < N) row[j0 + t] = fmaf(-row[k], l[t], row[j0 + t]);
+        }
     }
     *inverse_out = inverse;
     return valid;
@@ -227,6 +251,7 @@ __device__ __forceinline__ bool factor_rows(uint32_t lane, float (&row)[N], floa
 // SolveTileBlock (:1647-1666): forward with the factor's rows, backward with its columns (col[j] = L_j,lane).
 template <int N>
 __device__ __forceinline__ float substitute(uint32_t lane, const float (&row)[N], const float (&col)[N], float inverse, float g) {
+    lane = local_lane(lane);
     float r = g;
 #pragma unroll
     for (int j = 0; j < N; ++j) {
@@ -243,6 +268,7 @@ __device__ __forceinline__ float substitute(uint32_t lane, const float (&row)[N]
 
 template <int N>
 __device__ __forceinline__ void store_rows(float* a, uint32_t lane, const float (&row)[N]) {
+    lane = local_lane(lane);
     if (lane < uint32_t(N)) {
 #pragma unroll
         for (int k = 0; k < N; ++k) a[lane * (N + 1) + k] = row[k];
@@ -250,11 +276,13 @@ __device__ __forceinline__ void store_rows(float* a, uint32_t lane, const float 
 }
 template <int N>
 __device__ __forceinline__ void load_rows(const float* a, uint32_t lane, float (&row)[N]) {
+    lane = local_lane(lane);
 #pragma unroll
     for (int k = 0; k < N; ++k) row[k] = lane < uint32_t(N) ? a[lane * (N + 1) + k] : 0.0f;
 }
 template <int N>
 __device__ __forceinline__ void load_columns(const float* a, uint32_t lane, float (&col)[N]) {
+    lane = local_lane(lane);
 #pragma unroll
     for (int j = 0; j < N; ++j) col[j] = lane < uint32_t(N) ? a[j * (N + 1) + lane] : 0.0f;
 }
@@ -416,6 +444,7 @@ template <int N>
 __device__ __forceinline__ Failure newton_direction(const Tile& c, const float (&mrow)[N], float u, float free_v, float* force, float* inertia,
                                     float* d, bool* converged) {
     PROF_COUNT(c, 0);
+    c.work += 16u;
     float hrow[N];
     PROF_BEGIN(c, 1);
     const bool assembled = assemble_block<N>(c, mrow, u, free_v, hrow, force, inertia, converged);
@@ -508,6 +537,7 @@ __device__ __forceinline__ void line_terms(const HeadLine& l, float alpha, TileS
 __device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& mine, float alpha, float inertial_slope, float inertial_curvature,
                                  float* slope, float* curvature, float* magnitude) {
     PROF_COUNT(c, 1);
+    c.work += 1u;
     TileSum row_slope{0.0f, 0.0f};
     float row_curvature = 0.0f, row_magnitude = 0.0f;
     if (mine.owned) line_terms(mine, alpha, row_slope, row_curvature, row_magnitude);
@@ -876,15 +906,15 @@ __host__ __device__ inline uint32_t SolverLdsFloats(uint32_t n, uint32_t cap) {
 
 // DescendTile (:2941-3087)
 template <int N>
-__global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(N <= 36 ? 2 : 1, N <= 36 ? 2 : 1)))
+__global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(N <= kTwoWaveWidth ? 2 : 1, N <= kTwoWaveWidth ? 2 : 1)))
 BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint32_t cap) {
     extern __shared__ __align__(16) float lds[];
-    const uint32_t env = blockIdx.x, lane = threadIdx.x;
+    const uint32_t env = d.tile_order[blockIdx.x], lane = threadIdx.x;
     const uint32_t R = p.rows_per_env, md = p.max_dof, n = m.dof, nl = m.links_per_env, S = p.contact_slots_per_env;
     Tile c;
     c.env = env; c.lane = lane; c.n = n; c.ld = uint32_t(N) + 1u; c.ldj = uint32_t(N); c.cap = cap; c.heads = 0u; c.iteration = 0u;
     c.tolerance = p.velocity_tolerance; c.failed = false; c.momentum = 0.0f; c.residual = 0.0f;
-    c.mass_inverse = 0.0f; c.mass_valid = false;
+    c.mass_inverse = 0.0f; c.mass_valid = false; c.work = 0u;
 #ifdef NKH_SOLVER_PROFILE
     for (int i = 0; i < 10; ++i) c.prof[i] = 0;
     for (int i = 0; i < 4; ++i) c.prof_count[i] = 0u;
@@ -1081,7 +1111,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     if (lane < 4u)
         d.solver_residual[size_t{env} * 4u + lane] =
             lane == 0u ? residual4[0] : lane == 1u ? residual4[1] : lane == 2u ? residual4[2] : residual4[3];
-    if (lane == 0u) d.vbd_velocity_sweep_count[env] = sweeps;
+    if (lane == 0u) { d.vbd_velocity_sweep_count[env] = sweeps; d.solver_cost[env] = c.work; }
 #ifdef NKH_SOLVER_PROFILE
     PROF_END(c, 9);
     if (lane == 0u) {

@@ -219,7 +219,8 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(row_cj_point_b, kF32, E * R * 3) X(chain_jacobian, kF32, E * R * md) X(chain_jacobian_b, kF32, E * R * md) \
     X(row_cj_link, kU32, E * R) X(row_cj_link_b, kU32, E * R) X(row_count, kU32, E) X(contact_count, kU32, E) \
     X(contact_row_extent, kU32, E * 2) X(env_status, kU32, E) X(vbd_velocity_sweep_count, kU32, E) \
-    X(solver_residual, kF32, E * 4) X(solver_penalty, kF32, E * R) X(solver_velocity, kF32, E * md) X(solver_free, kF32, E * md)
+    X(solver_residual, kF32, E * 4) X(solver_penalty, kF32, E * R) X(solver_velocity, kF32, E * md) X(solver_free, kF32, E * md) \
+    X(solver_cost, kU32, E) X(tile_order, kU32, E)
 
 #define NKH_MODEL_FIELDS(X) \
     X(joint_type, kU8) X(parent_link, kU32) X(joint_axis, kF32) X(parent_offset, kF32) X(link_local_pose, kF32) \
@@ -301,7 +302,8 @@ __global__ void __launch_bounds__(256) CheckpointCopyKernel(CheckpointSegments s
 }
 
 bool CheckpointExcludes(const char* name) {
-    for (const char* rebuilt : {"m", "m_factor", "chain_jacobian", "chain_jacobian_b"}) if (std::strcmp(name, rebuilt) == 0) return true;
+    // rebuilt by every step, or scheduling hints that are no part of the physics
+    for (const char* rebuilt : {"m", "m_factor", "chain_jacobian", "chain_jacobian_b", "solver_cost", "tile_order"}) if (std::strcmp(name, rebuilt) == 0) return true;
     return false;
 }
 
