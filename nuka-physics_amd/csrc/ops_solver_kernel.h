@@ -155,7 +155,7 @@ __device__ __forceinline__ float along_axis(float impulse, float velocity) { ret
 enum HeadField : uint32_t {
     hSlot, hStride, hAxes, hOwned, hRho, hCompliance, hLower, hUpper, hMu1, hMu2, hNormalBound,
     hRes, hDual = hRes + 3, hMove = hDual + 3, hStep = hMove + 3, hBase = hStep + 3, hDualScale = hBase + 3, hResidualScale,
-    hRelaxStep, hRelaxWeight = hRelaxStep + 3, hRelaxPoint, hF = hRelaxPoint + 3, hC = hF + 3, hNoise = hC + 6, hContrib = hNoise + 3,
+    hRelaxStep, hRelaxWeight = hRelaxStep + 3, hRelaxPoint, hF = hRelaxPoint + 3, hC = hF + 3, hNoise = hC + 6, hContrib = hNoise + 3, hColumnsLow, hColumnsHigh,
     hFieldCount
 };
 
@@ -173,7 +173,7 @@ struct Tile {
     float momentum, residual;
     bool failed;
 #ifdef NKH_SOLVER_PROFILE
-    mutable long long prof[10];
+    mutable long long prof[16];
     mutable uint32_t prof_count[4];
 #endif
     __device__ float& F(uint32_t field, uint32_t h) const { return fields[field * cap + h]; }
@@ -325,7 +325,71 @@ __device__ __forceinline__ float solve_tile_mass(const Tile& c, float force) {
     return substitute<N>(c.lane, row, col, c.mass_inverse, c.lane < c.n ? force : 0.0f);
 }
 
-// AssembleTileBlock (:1507-1618): lane i assembles row i of H = M + sum J^T C J in `hrow` and its force g_i.
+// One head's part of the block: g += J^T f and H += J^T C J for lane's row, skipping the column blocks the head's
+// Jacobian rows leave at exact zero.  All head values are uniform.
+template <int N>
+__device__ __forceinline__ void add_head(const Tile& c, uint32_t h, bool coordinate, const float (&f)[3], const float (&cv)[6],
+                                         const float (&noise)[3], uint32_t axes, uint64_t columns, float (&hrow)[N], TileSum& g,
+                                         float& scale) {
+    const float* j0r = c.jac + (3u * h) * uint32_t(N);
+    const float j0 = coordinate ? j0r[c.lane] : 0.0f;
+    tile_add_product(g, j0, f[0]);
+    scale += fabsf(j0) * noise[0];
+    const float4* r0 = reinterpret_cast<const float4*>(j0r);
+    if (axes == 1u) {
+        const float a0 = j0 * cv[0];
+#pragma unroll
+        for (int q = 0; q < N / 4; ++q) {
+            if (((columns >> (4 * q)) & 0xFull) == 0ull) continue;
+            const float4 x0 = r0[q];
+            hrow[4 * q] = fmaf(a0, x0.x, hrow[4 * q]); hrow[4 * q + 1] = fmaf(a0, x0.y, hrow[4 * q + 1]);
+            hrow[4 * q + 2] = fmaf(a0, x0.z, hrow[4 * q + 2]); hrow[4 * q + 3] = fmaf(a0, x0.w, hrow[4 * q + 3]);
+        }
+        return;
+    }
+    const float* j1r = j0r + N, *j2r = j0r + 2 * N;
+    const float j1 = coordinate ? j1r[c.lane] : 0.0f, j2 = coordinate ? j2r[c.lane] : 0.0f;
+    const float cxx = cv[0], cyy = cv[1], czz = cv[2], cxy = cv[3], cxz = cv[4], cyz = cv[5];
+    tile_add_product(g, j1, f[1]);
+    tile_add_product(g, j2, f[2]);
+    scale += fabsf(j1) * noise[1] + fabsf(j2) * noise[2];
+    const float a0 = (j0 * cxx + j1 * cxy) + j2 * cxz;
+    const float a1 = (j1 * cyy + j2 * cyz) + j0 * cxy;
+    const float a2 = (j2 * czz + j1 * cyz) + j0 * cxz;
+    const float4* r1 = reinterpret_cast<const float4*>(j1r);
+    const float4* r2 = reinterpret_cast<const float4*>(j2r);
+#pragma unroll
+    for (int q = 0; q < N / 4; ++q) {
+        if (((columns >> (4 * q)) & 0xFull) == 0ull) continue;
+        const float4 x0 = r0[q], x1 = r1[q], x2 = r2[q];
+        hrow[4 * q] += fmaf(a2, x2.x, fmaf(a1, x1.x, a0 * x0.x));
+        hrow[4 * q + 1] += fmaf(a2, x2.y, fmaf(a1, x1.y, a0 * x0.y));
+        hrow[4 * q + 2] += fmaf(a2, x2.z, fmaf(a1, x1.z, a0 * x0.z));
+        hrow[4 * q + 3] += fmaf(a2, x2.w, fmaf(a1, x1.w, a0 * x0.w));
+    }
+}
+
+// A head's response at its current move with the rounding noise of each axis; false when nothing of it is non-zero.
+__device__ __forceinline__ bool head_terms(const Tile& c, uint32_t h, float (&f)[3], float (&cv)[6], float (&noise)[3]) {
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { f[k] = 0.0f; noise[k] = 0.0f; }
+#pragma unroll
+    for (int k = 0; k < 6; ++k) cv[k] = 0.0f;
+    if (h >= c.heads || c.U(hOwned, h) == 0u) return false;
+    head_response(c, h, c.F(hMove, h), c.F(hMove + 1, h), c.F(hMove + 2, h), f, cv);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) noise[k] = fabsf(f[k]) + cv[k] * (fabsf(c.F(hRes + k, h)) + fabsf(c.F(hMove + k, h)));
+    return f[0] != 0.0f || f[1] != 0.0f || f[2] != 0.0f || cv[0] != 0.0f || cv[1] != 0.0f || cv[2] != 0.0f || cv[5] != 0.0f ||
+           cv[3] != 0.0f || cv[4] != 0.0f || noise[0] != 0.0f || noise[1] != 0.0f || noise[2] != 0.0f;
+}
+
+__device__ __forceinline__ float uniform_lane_value(float v, uint32_t lane) {   // `lane` is uniform, not a constant
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), int(lane)));
+}
+
+// AssembleTileBlock (:1507-1618): lane i assembles row i of H = M + sum J^T C J in `hrow` and its force g_i.  The
+// first 64 heads evaluate their response one per lane and hand it to the row lanes as scalar lane reads; heads beyond
+// 64 pass theirs through the head fields.
 template <int N>
 __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow)[N], float u, float free_v, float (&hrow)[N], float* force,
                                float* inertia, bool* converged) {
@@ -336,26 +400,23 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
     const float difference_error = (u - (difference - part)) + (-free_v - part);
     float* dvec = c.vec, *evec = c.vec + 64, *uvec = c.vec + 128;
     dvec[lane] = difference; evec[lane] = difference_error; uvec[lane] = fabsf(u);
-    // every head's response at its current move, lane = head
-    for (uint32_t h = lane; h < c.heads; h += kWave) {
-        float f[3] = {0, 0, 0}, cv[6] = {0, 0, 0, 0, 0, 0};
-        bool contributes = false;
-        if (c.U(hOwned, h) != 0u) {
-            head_response(c, h, c.F(hMove, h), c.F(hMove + 1, h), c.F(hMove + 2, h), f, cv);
-            const float n0 = fabsf(f[0]) + cv[0] * (fabsf(c.F(hRes, h)) + fabsf(c.F(hMove, h)));
-            const float n1 = fabsf(f[1]) + cv[1] * (fabsf(c.F(hRes + 1, h)) + fabsf(c.F(hMove + 1, h)));
-            const float n2 = fabsf(f[2]) + cv[2] * (fabsf(c.F(hRes + 2, h)) + fabsf(c.F(hMove + 2, h)));
-            c.F(hNoise, h) = n0; c.F(hNoise + 1, h) = n1; c.F(hNoise + 2, h) = n2;
-            contributes = f[0] != 0.0f || f[1] != 0.0f || f[2] != 0.0f || cv[0] != 0.0f || cv[1] != 0.0f || cv[2] != 0.0f ||
-                          cv[5] != 0.0f || cv[3] != 0.0f || cv[4] != 0.0f || n0 != 0.0f || n1 != 0.0f || n2 != 0.0f;
-        }
+    PROF_BEGIN(c, 10);
+    float mf[3], mc[6], mn[3];
+    const bool mine = head_terms(c, lane, mf, mc, mn);
+    const uint32_t my_axes = lane < c.heads ? c.U(hAxes, lane) : 0u;
+    const uint32_t my_low = lane < c.heads ? c.U(hColumnsLow, lane) : 0u, my_high = lane < c.heads ? c.U(hColumnsHigh, lane) : 0u;
+    for (uint32_t h = lane + kWave; h < c.heads; h += kWave) {
+        float f[3], cv[6], noise[3];
+        const bool contributes = head_terms(c, h, f, cv, noise);
 #pragma unroll
-        for (int k = 0; k < 3; ++k) c.F(hF + k, h) = f[k];
+        for (int k = 0; k < 3; ++k) { c.F(hF + k, h) = f[k]; c.F(hNoise + k, h) = noise[k]; }
 #pragma unroll
         for (int k = 0; k < 6; ++k) c.F(hC + k, h) = cv[k];
         c.U(hContrib, h) = contributes ? 1u : 0u;
     }
     __syncthreads();
+    PROF_END(c, 10);
+    PROF_BEGIN(c, 11);
     // Padded columns (k >= n) hold exact zeros in the mass row, the vectors and the Jacobian rows: their terms add
     // nothing to any of the sums below.
     TileSum inertial{0.0f, 0.0f};
@@ -376,44 +437,31 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
         }
     }
     TileSum g{-inertial.value, -inertial.error};
-    for (uint32_t h = 0u; h < c.heads; ++h) {
-        if (c.U(hContrib, h) == 0u) continue;
-        const float* j0r = c.jac + (3u * h) * uint32_t(N);
-        const float j0 = coordinate ? j0r[lane] : 0.0f;
-        const float fx = c.F(hF, h), cxx = c.F(hC, h);
-        tile_add_product(g, j0, fx);
-        scale += fabsf(j0) * c.F(hNoise, h);
-        const float4* r0 = reinterpret_cast<const float4*>(j0r);
-        if (c.U(hAxes, h) == 1u) {
-            const float a0 = j0 * cxx;
+    PROF_END(c, 11);
+    PROF_BEGIN(c, 12);
+    for (uint64_t rest = __ballot(mine); rest != 0ull; rest &= rest - 1ull) {
+        const uint32_t h = uint32_t(__builtin_ctzll(rest));
+        float f[3], cv[6], noise[3];
 #pragma unroll
-            for (int q = 0; q < N / 4; ++q) {
-                const float4 x0 = r0[q];
-                hrow[4 * q] = fmaf(a0, x0.x, hrow[4 * q]); hrow[4 * q + 1] = fmaf(a0, x0.y, hrow[4 * q + 1]);
-                hrow[4 * q + 2] = fmaf(a0, x0.z, hrow[4 * q + 2]); hrow[4 * q + 3] = fmaf(a0, x0.w, hrow[4 * q + 3]);
-            }
-            continue;
-        }
-        const float* j1r = j0r + N, *j2r = j0r + 2 * N;
-        const float j1 = coordinate ? j1r[lane] : 0.0f, j2 = coordinate ? j2r[lane] : 0.0f;
-        const float cyy = c.F(hC + 1, h), czz = c.F(hC + 2, h), cxy = c.F(hC + 3, h), cxz = c.F(hC + 4, h), cyz = c.F(hC + 5, h);
-        tile_add_product(g, j1, c.F(hF + 1, h));
-        tile_add_product(g, j2, c.F(hF + 2, h));
-        scale += fabsf(j1) * c.F(hNoise + 1, h) + fabsf(j2) * c.F(hNoise + 2, h);
-        const float a0 = (j0 * cxx + j1 * cxy) + j2 * cxz;
-        const float a1 = (j1 * cyy + j2 * cyz) + j0 * cxy;
-        const float a2 = (j2 * czz + j1 * cyz) + j0 * cxz;
-        const float4* r1 = reinterpret_cast<const float4*>(j1r);
-        const float4* r2 = reinterpret_cast<const float4*>(j2r);
+        for (int k = 0; k < 3; ++k) { f[k] = uniform_lane_value(mf[k], h); noise[k] = uniform_lane_value(mn[k], h); }
 #pragma unroll
-        for (int q = 0; q < N / 4; ++q) {
-            const float4 x0 = r0[q], x1 = r1[q], x2 = r2[q];
-            hrow[4 * q] += fmaf(a2, x2.x, fmaf(a1, x1.x, a0 * x0.x));
-            hrow[4 * q + 1] += fmaf(a2, x2.y, fmaf(a1, x1.y, a0 * x0.y));
-            hrow[4 * q + 2] += fmaf(a2, x2.z, fmaf(a1, x1.z, a0 * x0.z));
-            hrow[4 * q + 3] += fmaf(a2, x2.w, fmaf(a1, x1.w, a0 * x0.w));
-        }
+        for (int k = 0; k < 6; ++k) cv[k] = uniform_lane_value(mc[k], h);
+        const uint32_t axes = uint32_t(__builtin_amdgcn_readlane(int(my_axes), int(h)));
+        const uint64_t columns = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_high), int(h)))) << 32u) |
+                                 uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_low), int(h))));
+        add_head<N>(c, h, coordinate, f, cv, noise, axes, columns, hrow, g, scale);
     }
+    for (uint32_t h = kWave; h < c.heads; ++h) {
+        if (c.U(hContrib, h) == 0u) continue;
+        const float f[3] = {c.F(hF, h), c.F(hF + 1, h), c.F(hF + 2, h)};
+        const float cv[6] = {c.F(hC, h), c.F(hC + 1, h), c.F(hC + 2, h), c.F(hC + 3, h), c.F(hC + 4, h), c.F(hC + 5, h)};
+        const float noise[3] = {c.F(hNoise, h), c.F(hNoise + 1, h), c.F(hNoise + 2, h)};
+        const uint64_t columns = (uint64_t(__builtin_amdgcn_readfirstlane(c.U(hColumnsHigh, h))) << 32u) |
+                                 uint64_t(__builtin_amdgcn_readfirstlane(c.U(hColumnsLow, h)));
+        add_head<N>(c, h, coordinate, f, cv, noise, c.U(hAxes, h), columns, hrow, g, scale);
+    }
+    PROF_END(c, 12);
+    PROF_BEGIN(c, 13);
     *force = coordinate ? g.value + g.error : 0.0f;
     *inertia = coordinate ? inertial.value + inertial.error : 0.0f;
     bool finite = isfinite(*force);
@@ -432,6 +480,7 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
     *converged = __all(!coordinate || fabsf(*force) <= kRoundings * FLT_EPSILON * scale);
     const bool ok = __all(!coordinate || finite);
     __syncthreads();
+    PROF_END(c, 13);
     return ok;
 }
 
@@ -916,7 +965,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     c.tolerance = p.velocity_tolerance; c.failed = false; c.momentum = 0.0f; c.residual = 0.0f;
     c.mass_inverse = 0.0f; c.mass_valid = false; c.work = 0u;
 #ifdef NKH_SOLVER_PROFILE
-    for (int i = 0; i < 10; ++i) c.prof[i] = 0;
+    for (int i = 0; i < 16; ++i) c.prof[i] = 0;
     for (int i = 0; i < 4; ++i) c.prof_count[i] = 0u;
 #endif
     PROF_BEGIN(c, 9);
@@ -973,6 +1022,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         const uint32_t flags = __float_as_uint(urows[size_t{slot} * kRowWords]);
         const uint32_t stride = __float_as_uint(urows[size_t{slot} * kRowWords + 2u]);
         const uint32_t axes = (flags & kRowBlockNormal) != 0u ? 3u : 1u;
+        bool used = false;
         for (uint32_t axis = 0u; axis < 3u; ++axis) {
             float value = 0.0f;
             if (axis < axes && coordinate) {
@@ -983,7 +1033,12 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
                 if (kind_b == kSideArtic) value += d.chain_jacobian_b[size_t{rs} * md + lane];
             }
             if (lane < c.ldj) c.jac[(3u * h + axis) * c.ldj + lane] = value;   // padded columns hold zeros
+            used = used || value != 0.0f;
         }
+        // the columns this head touches at all: a contact on one limb leaves most coordinates out, and the Hessian
+        // update skips their exact-zero products four columns at a time
+        const uint64_t columns = __ballot(used);
+        if (lane == 0u) { c.U(hColumnsLow, h) = uint32_t(columns); c.U(hColumnsHigh, h) = uint32_t(columns >> 32u); }
     }
     __syncthreads();
     // TileInertialResponse (:709-739): J M^-1 J^T of every head's first row through the stored LDL^T factor
@@ -1117,6 +1172,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     if (lane == 0u) {
         for (int i = 0; i < 10; ++i) d.solver_penalty[size_t{env} * R + i] = float(c.prof[i]);
         for (int i = 0; i < 4; ++i) d.solver_penalty[size_t{env} * R + 10 + i] = float(c.prof_count[i]);
+        for (int i = 10; i < 16; ++i) d.solver_penalty[size_t{env} * R + 4 + i] = float(c.prof[i]);
     }
 #endif
     // the block velocities persist for the next solve's carried start
