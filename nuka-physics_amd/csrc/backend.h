@@ -17,6 +17,7 @@ bool BackendSupportsOp(NkOp op);
 // Raises the dynamic-LDS limit of the wide kernels once, outside any stream capture.
 void InitArticulationKernels();
 void InitSolverKernels();
+void InitContactKernels();
 uint32_t SolverHeadCapacity(const ModelView& m, uint32_t slots, size_t lds_budget_bytes);
 
 }  // namespace nkh

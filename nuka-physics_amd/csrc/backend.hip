@@ -327,6 +327,7 @@ void* CreateBackend(int device, void* borrowed_stream) {
     }
     InitArticulationKernels();
     InitSolverKernels();
+    InitContactKernels();
     be->device_type = BufferType{&kBufferTypeI, false, &be->stream, device};
     be->host_type = BufferType{&kBufferTypeI, true, &be->stream, device};
     return be;

@@ -323,6 +323,12 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
     const uint32_t R = p.rows_per_env, S = p.union_slot_count, CR = p.contact_rows_per_env, md = p.max_dof, nl = m.links_per_env;
     uint32_t* range_first = lds_u;        // S
     uint32_t* range_points = lds_u + S;   // S
+    // what the chain Jacobian pass needs of each row, kept here so that it does not read back what this block wrote
+    uint32_t* row_link_a = lds_u + 2u * S;             // R
+    uint32_t* row_link_b = row_link_a + R;              // R
+    uint32_t* row_merge = row_link_b + R;               // R: both sides articulated with the same owner
+    float* row_point = reinterpret_cast<float*>(row_merge + R);   // 3R
+    float* row_dir = row_point + 3u * R;                 // 3R, side A's direction (side B's is its negative)
     Row* rows = reinterpret_cast<Row*>(d.urows) + size_t{env} * R;
     float* lambda = d.lambda + size_t{env} * R;
     float* pen = d.row_penetration + size_t{env} * R;
@@ -356,6 +362,7 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
         lambda[local] = 0.0f; pen[local] = 0.0f; cj_link[local] = kInvalid; cj_link_b[local] = kInvalid;
         rows[local].flags = 0u;
     }
+    for (uint32_t local = lane; local < R; local += kWave) { row_link_a[local] = kInvalid; row_link_b[local] = kInvalid; row_merge[local] = 0u; }
     if (lane == 0u) {
         d.contact_row_extent[2u * env] = previous_extent;
         d.contact_row_extent[2u * env + 1u] = extent;
@@ -442,6 +449,11 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
                     row.flags = kRowActive | kRowBlockTangent;
                     row.lower = -FLT_MAX; row.upper = FLT_MAX;
                 }
+                row_point[3u * rs] = point.x; row_point[3u * rs + 1u] = point.y; row_point[3u * rs + 2u] = point.z;
+                row_dir[3u * rs] = dir.x; row_dir[3u * rs + 1u] = dir.y; row_dir[3u * rs + 2u] = dir.z;
+                if (kind_a == kSideArtic) row_link_a[rs] = link_a;
+                if (kind_b == kSideArtic) row_link_b[rs] = link_b;
+                row_merge[rs] = kind_a == kSideArtic && kind_b == kSideArtic && idx_a == idx_b ? 1u : 0u;
                 if (kind_a == kSideArtic) { cj_link[rs] = link_a; cj_point[3u * rs] = point.x; cj_point[3u * rs + 1u] = point.y; cj_point[3u * rs + 2u] = point.z; }
                 if (kind_b == kSideArtic) { cj_link_b[rs] = link_b; cj_point_b[3u * rs] = point.x; cj_point_b[3u * rs + 1u] = point.y; cj_point_b[3u * rs + 2u] = point.z; }
                 rows[rs] = row;
@@ -479,14 +491,15 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
     }
     const uint32_t bound = min(contact_row_bound(previous_extent, extent, CR) + (R - CR), R);
     for (uint32_t r = 0u; r < bound; ++r) {
-        const Row* row = rows + r;
+        const uint32_t links[2] = {row_link_a[r], row_link_b[r]};
+        if (links[0] == kInvalid && links[1] == kInvalid) continue;
+        const V3 point{row_point[3u * r], row_point[3u * r + 1u], row_point[3u * r + 2u]};
+        const V3 dir_a{row_dir[3u * r], row_dir[3u * r + 1u], row_dir[3u * r + 2u]};
+        float entries[2] = {0.0f, 0.0f};
         for (uint32_t side = 0u; side < 2u; ++side) {
-            const uint32_t link_global = side == 0u ? cj_link[r] : cj_link_b[r];
-            if (link_global == kInvalid) continue;
-            const uint32_t link = link_global - env * nl;
-            const float* cp = (side == 0u ? cj_point : cj_point_b) + 3u * r;
-            const V3 point{cp[0], cp[1], cp[2]};
-            const V3 dir = side == 0u ? row->a.jlin : row->b.jlin;
+            if (links[side] == kInvalid) continue;
+            const uint32_t link = links[side] - env * nl;
+            const V3 dir = side == 0u ? dir_a : V3{-dir_a.x, -dir_a.y, -dir_a.z};
             float entry = 0.0f;
             if (lane < m.dof && ((m.link_dof_mask[link] >> lane) & 1ull) != 0ull) {
                 if (mode == 1u) entry = dot3(cross3(axis_world, sub3(point, origin)), dir) + dot3(axis_world, V3{0, 0, 0});
@@ -494,14 +507,12 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
                 else if (mode == 3u) entry = dot3(cross3(axis_world, sub3(point, origin)), dir) + dot3(axis_world, V3{0, 0, 0});
                 else if (mode == 4u) entry = dot3(axis_world, dir);
             }
-            if (lane < md) (side == 0u ? d.chain_jacobian : d.chain_jacobian_b)[(size_t{env} * R + r) * md + lane] = entry;
+            entries[side] = entry;
         }
-        if ((row->flags & kRowActive) != 0u && row->a.kind == kSideArtic && row->b.kind == kSideArtic &&
-            row->a.index == row->b.index && lane < md) {
-            float* ja = d.chain_jacobian + (size_t{env} * R + r) * md;
-            float* jb = d.chain_jacobian_b + (size_t{env} * R + r) * md;
-            ja[lane] += jb[lane];
-            jb[lane] = 0.0f;
+        if (row_merge[r] != 0u) { entries[0] += entries[1]; entries[1] = 0.0f; }   // shared owner (:172-186)
+        if (lane < md) {
+            if (links[0] != kInvalid) d.chain_jacobian[(size_t{env} * R + r) * md + lane] = entries[0];
+            if (links[1] != kInvalid) d.chain_jacobian_b[(size_t{env} * R + r) * md + lane] = entries[1];
         }
     }
 }
@@ -554,12 +565,18 @@ Status OpNarrowphaseHeightfield(const ModelView&, const DataView&, const void* p
     return params == nullptr ? Status::Ok : Status::Ok;   // no heightfield on this path: a no-op, as in the reference
 }
 
+void InitContactKernels() {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(AssembleRowsKernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    (void)hipGetLastError();
+}
+
 Status OpAssembleRows(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
     const auto* p = static_cast<const AssembleRowsParams*>(params);
     if (p == nullptr) return Status::Failed;
     if (p->env_count == 0u || p->rows_per_env == 0u) return Status::Ok;
     if (p->max_dof > kMaxDof) return Status::InvalidArgument;
-    const size_t lds = size_t{p->union_slot_count} * 2u * sizeof(uint32_t);
+    const size_t lds = (size_t{p->union_slot_count} * 2u + size_t{p->rows_per_env} * 9u) * sizeof(uint32_t);
+    if (lds > 150u * 1024u) return Status::InvalidArgument;
     hipLaunchKernelGGL(AssembleRowsKernel, dim3(p->env_count), dim3(kWave), lds, stream, m, d, *p);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
