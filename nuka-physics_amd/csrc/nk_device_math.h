@@ -188,6 +188,17 @@ __device__ __forceinline__ uint32_t wave_sum_u(uint32_t v) {
     for (int o = 32; o > 0; o >>= 1) v += uint32_t(__shfl_xor(int(v), o, 64));
     return v;
 }
+// A lane's value of `v` for a lane index that is a compile-time constant at every call site: a scalar lane read.
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+// Lane predicates (lane == k, lane > j, ...) of fully unrolled loops are loop invariant; hoisted out of the enclosing
+// loops they would occupy hundreds of scalar registers and spill.  Passing the lane index through this makes each
+// use site compute its own predicate where it needs it.
+__device__ __forceinline__ uint32_t local_lane(uint32_t lane) {
+    asm volatile("" : "+v"(lane));
+    return lane;
+}
 __device__ __forceinline__ bool wave_all(bool p) { return __all(p); }
 __device__ __forceinline__ bool wave_any(bool p) { return __any(p); }
 

@@ -148,6 +148,9 @@ __host__ __device__ inline uint32_t DynamicsLdsFloats(uint32_t nl, uint32_t n) {
     return nl * (36u + 36u + 5u * 6u) + n * (n + 1u) + 2u * n + 64u;
 }
 
+// Compiled per padded DoF width N (a multiple of 4): the LDL^T factorisation and the solve keep one matrix row per
+// lane in registers, fully unrolled, and pass pivots and multipliers between lanes as scalar lane reads.
+template <int N>
 __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m, DataView d, ArticulationDynamicsParams p,
                                                                    uint32_t env_count) {
     extern __shared__ float lds[];
@@ -365,20 +368,41 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
         const uint32_t i = e / stride, j = e % stride;
         M[e] = i < n && j < n ? A[i * ld + j] : 0.0f;
     }
-    // LDL^T, right-looking, lane = row; the strict lower triangle becomes L and the diagonal D (:269-335)
-    for (uint32_t k = 0u; k < n; ++k) {
-        const float diagonal = fmaxf(A[k * ld + k], 1.0e-6f);
-        float lik = 0.0f;
-        if (lane > k && lane < n) {
-            lik = A[lane * ld + k] / diagonal;
-            A[lane * ld + k] = lik;
-        }
-        __syncthreads();
-        if (lane > k && lane < n)
-            for (uint32_t j = k + 1u; j <= lane; ++j) A[lane * ld + j] -= lik * A[j * ld + k] * diagonal;
-        if (lane == k) A[k * ld + k] = diagonal;
-        __syncthreads();
+    // LDL^T, right-looking, lane = row in registers; the strict lower triangle becomes L and the diagonal D (:269-335).
+    // Rows and columns n..N-1 are those of the identity.  Entry (i, j) loses (L_ik L_jk) D_k for k = 0, 1, ... as the
+    // serial loop does; what a lane computes above its diagonal is never read.
+    float row[N];
+    {
+        const uint32_t ll = local_lane(lane);
+#pragma unroll
+        for (int k = 0; k < N; ++k)
+            row[k] = ll < n && uint32_t(k) < n ? A[ll * ld + k] : (ll == uint32_t(k) ? 1.0f : 0.0f);
     }
+    __syncthreads();
+    {
+        const uint32_t ll = local_lane(lane);
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+            const float diagonal = fmaxf(lane_value(row[k], k), 1.0e-6f);
+            const float lik = row[k] / diagonal;
+            row[k] = ll > uint32_t(k) ? lik : (ll == uint32_t(k) ? diagonal : row[k]);
+#pragma unroll
+            for (int j0 = k + 1; j0 < N; j0 += 8) {
+                float l[8];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) l[t] = j0 + t < N ? lane_value(lik, j0 + t) : 0.0f;
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+                    if (j0 + t < N) row[j0 + t] -= lik * l[t] * diagonal;
+            }
+        }
+        if (ll < n) {
+#pragma unroll
+            for (int k = 0; k < N; ++k)
+                if (uint32_t(k) < n) A[ll * ld + k] = row[k];
+        }
+    }
+    __syncthreads();
     float* factor = d.m_factor + size_t{env} * stride * stride;
     for (uint32_t e = lane; e < stride * stride; e += kWave) {
         const uint32_t i = e / stride, j = e % stride;
@@ -386,15 +410,22 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
     }
     // solve L D L^T x = rhs: forward by rows, scale, backward by columns (:357-396)
     float x = lane < n ? acc[lane] : 0.0f;
-    for (uint32_t j = 0u; j < n; ++j) {
-        const float solved = wave_bcast(x, int(j));
-        if (lane > j && lane < n) x -= A[lane * ld + j] * solved;
-    }
-    if (lane < n) x = x / A[lane * ld + lane];
-    for (uint32_t end = n; end > 0u; --end) {
-        const uint32_t i = end - 1u;
-        const float value = wave_bcast(x, int(i));
-        if (lane < i) x -= A[i * ld + lane] * value;
+    {
+        const uint32_t ll = local_lane(lane);
+        float col[N];
+#pragma unroll
+        for (int i = 0; i < N; ++i) col[i] = ll < uint32_t(i) && uint32_t(i) < n ? A[i * ld + ll] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const float solved = lane_value(x, j);
+            if (ll > uint32_t(j) && ll < n) x -= row[j] * solved;
+        }
+        if (ll < n) x = x / A[ll * ld + ll];
+#pragma unroll
+        for (int i = N - 1; i >= 0; --i) {
+            const float value = lane_value(x, i);
+            if (ll < uint32_t(i)) x -= col[i] * value;
+        }
     }
     if (lane < stride) d.articulation_qdd[size_t{env} * stride + lane] = lane < n ? x : 0.0f;
     if (lane < n) acc[lane] = x;
@@ -525,6 +556,13 @@ Status OpFkWorldPoses(const ModelView& m, const DataView& d, const void* params,
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 
+using DynamicsKernel = void (*)(ModelView, DataView, ArticulationDynamicsParams, uint32_t);
+static const DynamicsKernel kDynamicsKernels[16] = {
+    ArticulationDynamicsKernel<4>, ArticulationDynamicsKernel<8>, ArticulationDynamicsKernel<12>, ArticulationDynamicsKernel<16>,
+    ArticulationDynamicsKernel<20>, ArticulationDynamicsKernel<24>, ArticulationDynamicsKernel<28>, ArticulationDynamicsKernel<32>,
+    ArticulationDynamicsKernel<36>, ArticulationDynamicsKernel<40>, ArticulationDynamicsKernel<44>, ArticulationDynamicsKernel<48>,
+    ArticulationDynamicsKernel<52>, ArticulationDynamicsKernel<56>, ArticulationDynamicsKernel<60>, ArticulationDynamicsKernel<64>};
+
 Status OpArticulationDynamics(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
     const auto* p = static_cast<const ArticulationDynamicsParams*>(params);
     if (p == nullptr) return Status::Failed;
@@ -533,8 +571,8 @@ Status OpArticulationDynamics(const ModelView& m, const DataView& d, const void*
         p->total_link_count != p->articulation_count * m.links_per_env) return Status::InvalidArgument;
     const size_t lds = size_t{DynamicsLdsFloats(m.links_per_env, m.dof)} * sizeof(float);
     if (lds > 160u * 1024u) return Status::InvalidArgument;
-    hipLaunchKernelGGL(ArticulationDynamicsKernel, dim3(p->articulation_count), dim3(kWave), lds, stream, m, d, *p,
-                       p->articulation_count);
+    hipLaunchKernelGGL(kDynamicsKernels[((m.dof + 3u) & ~3u) / 4u - 1u], dim3(p->articulation_count), dim3(kWave), lds, stream, m, d,
+                       *p, p->articulation_count);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 
@@ -557,9 +595,10 @@ Status OpFkLinkVelocities(const ModelView& m, const DataView& d, const void* par
 }
 
 void InitArticulationKernels() {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(ArticulationDynamicsKernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              160 * 1024);
-    (void)hipGetLastError();
+    for (DynamicsKernel kernel : kDynamicsKernels) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipGetLastError();
+    }
 }
 
 // Torque control leaves tau as applied; free bodies do not exist on this path, so both ops only validate.

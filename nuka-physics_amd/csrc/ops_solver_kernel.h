@@ -193,19 +193,6 @@ __device__ __forceinline__ void head_response(const Tile& c, uint32_t h, float m
                     c.F(hNormalBound, h), c.F(hMu1, h), c.F(hMu2, h), &f[1], &f[2], &cv[1], &cv[2], &cv[5]);
 }
 
-// Lane predicates (lane == k, lane > j, ...) are invariant over the whole solve; hoisted out of its loops they would
-// occupy hundreds of scalar registers and spill.  Passing the lane index through this makes each use site compute
-// its own predicate where it needs it.
-__device__ __forceinline__ uint32_t local_lane(uint32_t lane) {
-    asm volatile("" : "+v"(lane));
-    return lane;
-}
-
-// A lane's value of `v` for a lane index that is a compile-time constant at every call site: a scalar lane read.
-__device__ __forceinline__ float lane_value(float v, int lane) {
-    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
-}
-
 // FactorTileBlock (:1622-1645) on register rows: lane i holds row i of the symmetric matrix; on return its entries
 // k <= i are row i of the Cholesky factor.  Element (i, j) loses L_ik L_jk for k = 0, 1, ... in that order, as the
 // reference's serial inner loop does; each product and subtraction is one fused multiply-add (the reference is
