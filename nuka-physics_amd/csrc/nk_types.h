@@ -97,6 +97,11 @@ struct DataView {
     uint32_t *env_status, *vbd_velocity_sweep_count;
     float *solver_residual, *solver_penalty;
     float *solver_velocity, *solver_free;   // block velocities kept between solves (carried constraint velocity)
+    // contact cache carried between steps (fields.yaml:524-539, 155, 791, 844)
+    uint64_t *contact_material, *contact_cache_pair, *contact_cache_feature, *contact_cache_material;
+    float *contact_cache_lambda, *contact_cache_normal;
+    uint32_t *contact_cache_age, *contact_cache_current_owner, *contact_cache_old_keep, *contact_cache_extent;
+    uint32_t *contact_warm_start_counts, *contact_cache_match;
     uint32_t *solver_cost, *tile_order;     // last solve's work per environment; launch order of the next solve (costliest first)
     float *snapshot;                        // SnapshotState / RestoreState storage
 };

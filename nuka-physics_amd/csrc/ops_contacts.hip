@@ -316,6 +316,26 @@ struct RowSide { uint32_t kind, index; V3 jlin, jang; };
 struct Row { uint32_t flags, group_first, group_normal_count, env; float rhs, compliance_alpha, lower, upper, mu, friction_secondary; RowSide a, b; };
 static_assert(sizeof(Row) == kRowWords * sizeof(float), "row layout must stay 26 words");
 
+// HashMergedContactProfile (assemble_rows.cu:88-105) of two default-authored profiles that differ in friction only
+// (scene/contact_filter.hpp:16-31, 72-130: equal priorities and mixing weights leave every other term at its default),
+// then the contact law for velocity-only laws (:620-622).
+__device__ __forceinline__ uint64_t profile_word(uint64_t hash, uint32_t word) { hash ^= uint64_t{word}; hash *= 0x100000001b3ull; return hash; }
+__device__ uint64_t contact_material_key(float mu1, float mu2, uint32_t law) {
+    uint64_t h = 0x4e554b4150524f46ull;
+    h = profile_word(h, 2u);   // profile schema version
+    h = profile_word(h, 1u);   // reference-safe flag
+    h = profile_word(h, __float_as_uint(mu1)); h = profile_word(h, __float_as_uint(mu2));
+    h = profile_word(h, __float_as_uint(0.005f)); h = profile_word(h, __float_as_uint(0.0001f));
+    h = profile_word(h, __float_as_uint(0.02f)); h = profile_word(h, __float_as_uint(1.0f));
+    h = profile_word(h, __float_as_uint(0.9f)); h = profile_word(h, __float_as_uint(0.95f)); h = profile_word(h, __float_as_uint(0.001f));
+    h = profile_word(h, __float_as_uint(0.5f)); h = profile_word(h, __float_as_uint(2.0f));
+    h = profile_word(h, __float_as_uint(0.0f)); h = profile_word(h, __float_as_uint(0.0f));
+    h = profile_word(h, 3u);
+    if (h == 0ull) h = 0x9e3779b97f4a7c15ull;
+    if (law == 1u || law == 2u) { h ^= uint64_t{law}; h *= 1099511628211ull; }
+    return h;
+}
+
 // ---- AssembleRows: one wavefront per environment (assemble_rows.cu:325-394, 200-214, 406-801, 122-186) ----
 __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataView d, AssembleRowsParams p) {
     extern __shared__ uint32_t lds_u[];
@@ -351,6 +371,7 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
             range_first[slot] = first; range_points[slot] = points;
             d.ucontact_row_range[(size_t{env} * S + slot) * 2u] = env * R + first;
             d.ucontact_row_range[(size_t{env} * S + slot) * 2u + 1u] = points;
+            if (first < contact_row_bound(previous_extent, 1u, CR)) d.contact_material[size_t{env} * S + slot] = 0ull;   // :358
             if (points > 0u) extent = max(extent, first + points * kRowsPerPoint + 1u);
         }
         carry += __shfl(through, kWave - 1, kWave);
@@ -405,6 +426,7 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
         const float mu_b1 = sb.profile < m.profile_count ? m.profile_mu[2u * sb.profile] : 1.0f;
         const float mu_b2 = sb.profile < m.profile_count ? m.profile_mu[2u * sb.profile + 1u] : 1.0f;
         const float mu1 = fmaxf(mu_a1, mu_b1), mu2 = fmaxf(mu_a2, mu_b2);
+        d.contact_material[gid] = n_active > 0u ? contact_material_key(mu1, mu2, d.ucontact_law[gid]) : 0ull;   // :620-622
         for (uint32_t pt = 0u; pt < P; ++pt) {
             const bool live = pt < n_active && pt < 4u;
             const size_t mp = gid * 4u + pt;
@@ -565,10 +587,6 @@ Status OpNarrowphaseHeightfield(const ModelView&, const DataView&, const void* p
     return params == nullptr ? Status::Ok : Status::Ok;   // no heightfield on this path: a no-op, as in the reference
 }
 
-void InitContactKernels() {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(AssembleRowsKernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    (void)hipGetLastError();
-}
 
 Status OpAssembleRows(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
     const auto* p = static_cast<const AssembleRowsParams*>(params);
@@ -581,12 +599,216 @@ Status OpAssembleRows(const ModelView& m, const DataView& d, const void* params,
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 
-// With no contact cache carried between steps every multiplier starts at the zero AssembleRows wrote
-// (assemble_rows.cu:1393-1455 with an empty cache).
-Status OpContactWarmStart(const ModelView&, const DataView&, const void* params, hipStream_t) {
-    return params == nullptr ? Status::Failed : Status::Ok;
+namespace {
+
+// ---- ContactWarmStart (assemble_rows.cu:1393-1455): one wavefront per environment ------------------------------
+// The reference indexes equal keys (pair, feature, material) through a hash table sized for the whole batch
+// (contact_cache.cuh:167-284).  An environment holds at most a few hundred entries, so here a wavefront lists them
+// in LDS (current points first, then cache entries, both in point order) and compares keys directly: the head of a
+// key is its first entry, the warm point of a key is its lowest cache point that has not decayed.
+struct CacheEntries {
+    uint64_t* pair; uint64_t* feature; uint64_t* material;   // 2P each
+    uint32_t* point;                                          // 2P: point index; cache entries carry bit 31
+};
+constexpr uint32_t kCacheFlag = 0x80000000u;
+
+__device__ __forceinline__ uint32_t prefix_rank(uint64_t mask, uint32_t lane) { return uint32_t(__popcll(mask & ((uint64_t{1} << lane) - 1ull))); }
+
+__device__ __forceinline__ bool row_offsets(const DataView& d, uint32_t env, uint32_t S, uint32_t slot, uint32_t point, uint32_t* rn,
+                                            uint32_t* r1, uint32_t* r2) {
+    const uint32_t first = d.ucontact_row_range[(size_t{env} * S + slot) * 2u], points = d.ucontact_row_range[(size_t{env} * S + slot) * 2u + 1u];
+    if (point >= points) return false;
+    *rn = first + point; *r1 = first + points + point; *r2 = first + 2u * points + point;
+    return true;
+}
+
+// Phase 0: BuildIndex (contact_cache.cuh:286-338) and PrepareContactWarmStartKernel (assemble_rows.cu:1229-1272)
+__global__ void __launch_bounds__(kWave) WarmStartPrepareKernel(DataView d, ContactWarmStartParams p) {
+    extern __shared__ uint64_t lds64[];
+    const uint32_t env = blockIdx.x, lane = threadIdx.x, S = p.slot_count, P = S * 4u;
+    const size_t base = size_t{env} * P;
+    CacheEntries e{lds64, lds64 + 2u * P, lds64 + 4u * P, reinterpret_cast<uint32_t*>(lds64 + 6u * P)};
+    uint32_t count = 0u;
+    for (uint32_t first = 0u; first < P; first += kWave) {   // current points that exist, in point order
+        const uint32_t i = first + lane;
+        const bool valid = i < P && (i & 3u) < d.ucontact_count[size_t{env} * S + i / 4u];
+        if (i < P) { d.contact_cache_current_owner[base + i] = 0u; d.contact_cache_old_keep[base + i] = 0u; d.contact_cache_match[base + i] = kInvalid; }
+        const uint64_t mask = __ballot(valid);
+        if (valid) {
+            const uint32_t at = count + prefix_rank(mask, lane);
+            e.pair[at] = d.ucontact_id_pair[base + i]; e.feature[at] = d.ucontact_id_feature[base + i];
+            e.material[at] = d.contact_material[size_t{env} * S + i / 4u]; e.point[at] = i;
+        }
+        count += uint32_t(__popcll(mask));
+    }
+    const uint32_t current_count = count;
+    for (uint32_t first = 0u; first < P; first += kWave) {   // cache entries, in point order
+        const uint32_t j = first + lane;
+        const bool valid = j < P && d.contact_cache_pair[base + j] != 0ull;
+        const uint64_t mask = __ballot(valid);
+        if (valid) {
+            const uint32_t at = count + prefix_rank(mask, lane);
+            e.pair[at] = d.contact_cache_pair[base + j]; e.feature[at] = d.contact_cache_feature[base + j];
+            e.material[at] = d.contact_cache_material[base + j]; e.point[at] = j | kCacheFlag;
+        }
+        count += uint32_t(__popcll(mask));
+    }
+    __syncthreads();
+    uint32_t owned = 0u, matched = 0u;
+    for (uint32_t k = lane; k < count; k += kWave) {
+        const uint64_t pair = e.pair[k], feature = e.feature[k], material = e.material[k];
+        bool head = true;
+        for (uint32_t earlier = 0u; earlier < k && head; ++earlier)
+            head = !(e.pair[earlier] == pair && e.feature[earlier] == feature && e.material[earlier] == material);
+        const uint32_t tagged = e.point[k];
+        if ((tagged & kCacheFlag) == 0u) {
+            const uint32_t i = tagged;
+            uint32_t warm = kInvalid;
+            if (head)
+                for (uint32_t other = current_count; other < count; ++other) {
+                    const uint32_t point = e.point[other] & ~kCacheFlag;
+                    if (e.pair[other] == pair && e.feature[other] == feature && e.material[other] == material &&
+                        d.contact_cache_age[base + point] < p.decay_steps && point < warm) warm = point;
+                }
+            d.contact_cache_match[base + i] = warm;
+            if (warm != kInvalid) {
+                const float* n = d.ucontact_normal + 3u * (base + i);
+                const float* o = d.contact_cache_normal + 3u * (base + warm);
+                if (n[0] * o[0] + n[1] * o[1] + n[2] * o[2] > 0.25f) ++matched;
+            }
+            if (head) { d.contact_cache_current_owner[base + i] = 1u; owned = max(owned, i + 1u); }
+        } else if (head && p.decay_steps > 1u && d.contact_cache_age[base + (tagged & ~kCacheFlag)] < p.decay_steps - 1u) {
+            d.contact_cache_old_keep[base + (tagged & ~kCacheFlag)] = 1u;
+        }
+    }
+    owned = wave_max_u(owned);
+    matched = wave_sum_u(matched);
+    if (lane == 0u) {
+        d.contact_cache_extent[2u * env + 1u] = owned;
+        d.contact_warm_start_counts[2u * env] = current_count;
+        d.contact_warm_start_counts[2u * env + 1u] = matched;
+    }
+    __syncthreads();   // this block's match writes are read back below
+    // rows of matched points whose normal has kept its side start from the cached impulse, the tangential part carried
+    // over in the world frame
+    for (uint32_t i = lane; i < P; i += kWave) {
+        const uint32_t match = d.contact_cache_match[base + i];
+        if (match == kInvalid) continue;
+        const V3 n{d.ucontact_normal[3u * (base + i)], d.ucontact_normal[3u * (base + i) + 1u], d.ucontact_normal[3u * (base + i) + 2u]};
+        const V3 o{d.contact_cache_normal[3u * (base + match)], d.contact_cache_normal[3u * (base + match) + 1u],
+                   d.contact_cache_normal[3u * (base + match) + 2u]};
+        if (n.x * o.x + n.y * o.y + n.z * o.z <= 0.25f) continue;
+        uint32_t rn, r1, r2;
+        if (!row_offsets(d, env, S, i / 4u, i & 3u, &rn, &r1, &r2)) continue;
+        const float* cached = d.contact_cache_lambda + 4u * (base + match);
+        V3 ot1, ot2, t1, t2;
+        contact_tangent_basis(o, &ot1, &ot2);
+        contact_tangent_basis(n, &t1, &t2);
+        const V3 old = add3(scale3(ot1, cached[1]), scale3(ot2, cached[2]));
+        d.lambda[rn] = fmaxf(cached[0], 0.0f);
+        d.lambda[r1] = dot3(old, t1);
+        d.lambda[r2] = dot3(old, t2);
+    }
+}
+
+// Phase 1: BuildRanks, CacheExtentKernel (contact_cache.cuh:340-365) and RebuildContactCacheKernel
+// (assemble_rows.cu:1313-1391).  The retained old entries are copied to LDS before the cache is rewritten.
+__global__ void __launch_bounds__(kWave) WarmStartCommitKernel(DataView d, ContactWarmStartParams p) {
+    extern __shared__ uint64_t lds64[];
+    const uint32_t env = blockIdx.x, lane = threadIdx.x, S = p.slot_count, P = S * 4u;
+    const size_t base = size_t{env} * P;
+    uint64_t* kept_pair = lds64, *kept_feature = lds64 + P, *kept_material = lds64 + 2u * P;
+    float* kept_float = reinterpret_cast<float*>(lds64 + 3u * P);         // 7 per entry: impulse 4, normal 3
+    uint32_t* kept_age = reinterpret_cast<uint32_t*>(kept_float + 7u * P);
+    uint32_t* free_rank = kept_age + P;                                      // free points before each point
+    uint32_t retained = 0u, unowned = 0u;
+    for (uint32_t first = 0u; first < P; first += kWave) {
+        const uint32_t i = first + lane;
+        const bool keep = i < P && d.contact_cache_old_keep[base + i] != 0u;
+        const bool is_free = i < P && d.contact_cache_current_owner[base + i] == 0u;
+        const uint64_t keep_mask = __ballot(keep), free_mask = __ballot(is_free);
+        if (i < P) free_rank[i] = unowned + prefix_rank(free_mask, lane);
+        if (keep) {
+            const uint32_t at = retained + prefix_rank(keep_mask, lane);
+            kept_pair[at] = d.contact_cache_pair[base + i]; kept_feature[at] = d.contact_cache_feature[base + i];
+            kept_material[at] = d.contact_cache_material[base + i];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) kept_float[7u * at + k] = d.contact_cache_lambda[4u * (base + i) + k];
+#pragma unroll
+            for (int k = 0; k < 3; ++k) kept_float[7u * at + 4 + k] = d.contact_cache_normal[3u * (base + i) + k];
+            kept_age[at] = d.contact_cache_age[base + i];
+        }
+        retained += uint32_t(__popcll(keep_mask));
+        unowned += uint32_t(__popcll(free_mask));
+    }
+    const uint32_t extent_previous = d.contact_cache_extent[2u * env], extent_current = d.contact_cache_extent[2u * env + 1u];
+    const uint32_t previous = extent_previous == 0u ? P : min(extent_previous - 1u, P);
+    const uint32_t next = min(max(extent_current, P - unowned + retained), P);
+    const uint32_t bound = min(max(previous, next), P);
+    __syncthreads();
+    if (lane == 0u) { d.contact_cache_extent[2u * env] = next + 1u; d.contact_cache_extent[2u * env + 1u] = max(previous, next); }
+    for (uint32_t i = lane; i < bound; i += kWave) {
+        uint32_t rn, r1, r2;
+        if (d.contact_cache_current_owner[base + i] != 0u && row_offsets(d, env, S, i / 4u, i & 3u, &rn, &r1, &r2)) {
+            const uint32_t stride = r1 - rn;
+            d.contact_cache_pair[base + i] = d.ucontact_id_pair[base + i];
+            d.contact_cache_feature[base + i] = d.ucontact_id_feature[base + i];
+#pragma unroll
+            for (uint32_t k = 0u; k < 4u; ++k) d.contact_cache_lambda[4u * (base + i) + k] = k < 3u ? d.lambda[rn + k * stride] : 0.0f;
+#pragma unroll
+            for (int k = 0; k < 3; ++k) d.contact_cache_normal[3u * (base + i) + k] = d.ucontact_normal[3u * (base + i) + k];
+            d.contact_cache_material[base + i] = d.contact_material[size_t{env} * S + i / 4u];
+            d.contact_cache_age[base + i] = 0u;
+            continue;
+        }
+        const uint32_t rank = free_rank[i];
+        if (rank < retained) {
+            d.contact_cache_pair[base + i] = kept_pair[rank]; d.contact_cache_feature[base + i] = kept_feature[rank];
+            d.contact_cache_material[base + i] = kept_material[rank];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) d.contact_cache_lambda[4u * (base + i) + k] = kept_float[7u * rank + k];
+#pragma unroll
+            for (int k = 0; k < 3; ++k) d.contact_cache_normal[3u * (base + i) + k] = kept_float[7u * rank + 4 + k];
+            d.contact_cache_age[base + i] = kept_age[rank] + 1u;
+            continue;
+        }
+        d.contact_cache_pair[base + i] = 0ull; d.contact_cache_feature[base + i] = 0ull; d.contact_cache_material[base + i] = 0ull;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) d.contact_cache_lambda[4u * (base + i) + k] = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) d.contact_cache_normal[3u * (base + i) + k] = 0.0f;
+        d.contact_cache_age[base + i] = 0u;
+    }
+}
+
+}  // namespace
+
+Status OpContactWarmStart(const ModelView&, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const ContactWarmStartParams*>(params);
+    if (p == nullptr || p->phase > 1u) return Status::InvalidArgument;
+    if (p->slot_count == 0u || p->env_count == 0u) return Status::Ok;
+    const size_t points = size_t{p->slot_count} * 4u;
+    if (p->phase == 0u) {
+        const size_t lds = points * (6u * sizeof(uint64_t) + 2u * sizeof(uint32_t));
+        if (lds > 150u * 1024u) return Status::InvalidArgument;
+        hipLaunchKernelGGL(WarmStartPrepareKernel, dim3(p->env_count), dim3(kWave), lds, stream, d, *p);
+    } else {
+        const size_t lds = points * (3u * sizeof(uint64_t) + 7u * sizeof(float) + 2u * sizeof(uint32_t));
+        if (lds > 150u * 1024u) return Status::InvalidArgument;
+        hipLaunchKernelGGL(WarmStartCommitKernel, dim3(p->env_count), dim3(kWave), lds, stream, d, *p);
+    }
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 
 Status OpSnapshotStepVelocity(const ModelView&, const DataView&, const void*, hipStream_t) { return Status::Ok; }
+
+void InitContactKernels() {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(AssembleRowsKernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    (void)hipGetLastError();
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(WarmStartPrepareKernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    (void)hipGetLastError();
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(WarmStartCommitKernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    (void)hipGetLastError();
+}
 
 }  // namespace nkh

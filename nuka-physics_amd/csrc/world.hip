@@ -220,7 +220,11 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(row_cj_link, kU32, E * R) X(row_cj_link_b, kU32, E * R) X(row_count, kU32, E) X(contact_count, kU32, E) \
     X(contact_row_extent, kU32, E * 2) X(env_status, kU32, E) X(vbd_velocity_sweep_count, kU32, E) \
     X(solver_residual, kF32, E * 4) X(solver_penalty, kF32, E * R) X(solver_velocity, kF32, E * md) X(solver_free, kF32, E * md) \
-    X(solver_cost, kU32, E) X(tile_order, kU32, E)
+    X(solver_cost, kU32, E) X(tile_order, kU32, E) \
+    X(contact_material, kU64, E * S) X(contact_cache_pair, kU64, E * S * 4) X(contact_cache_feature, kU64, E * S * 4) \
+    X(contact_cache_material, kU64, E * S * 4) X(contact_cache_lambda, kF32, E * S * 16) X(contact_cache_normal, kF32, E * S * 12) \
+    X(contact_cache_age, kU32, E * S * 4) X(contact_cache_current_owner, kU32, E * S * 4) X(contact_cache_old_keep, kU32, E * S * 4) \
+    X(contact_cache_extent, kU32, E * 2) X(contact_warm_start_counts, kU32, E * 2) X(contact_cache_match, kU32, E * S * 4)
 
 #define NKH_MODEL_FIELDS(X) \
     X(joint_type, kU8) X(parent_link, kU32) X(joint_axis, kF32) X(parent_offset, kF32) X(link_local_pose, kF32) \

@@ -462,10 +462,12 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
     extent[2u * env] = extent[2u * env + 1u];
     extent[2u * env + 1u] = 1u;
     uint32_t carry = 0u;
+    const uint32_t range_bound = contact_row_bound(extent, env, CR);
     for (uint32_t slot = 0u; slot < S; ++slot) {
         const uint32_t points = w->ucontact_count[(size_t)env * S + slot];
         w->ucontact_row_range[((size_t)env * S + slot) * 2u] = env * R + carry * 4u;
         w->ucontact_row_range[((size_t)env * S + slot) * 2u + 1u] = points;
+        if (carry * 4u < range_bound) w->contact_material[(size_t)env * S + slot] = 0u;   /* :358 */
         carry += points;
     }
     /* ClearPairDrivenRowsKernel :366-394 */
@@ -518,6 +520,7 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
         const float mu_b2 = sb.profile < t->n_profiles ? t->profile_mu[2u * sb.profile + 1u] : 1.0f;
         const float mu1 = mu_a1 > mu_b1 ? mu_a1 : mu_b1, mu2 = mu_a2 > mu_b2 ? mu_a2 : mu_b2;
         const int position_pass = w->cfg.solver_pos_iters > 0u;
+        w->contact_material[gid] = n_active > 0u ? nko_contact_material(mu1, mu2, w->ucontact_law[gid]) : 0u;   /* :620-622 */
         for (uint32_t p = 0u; p < P; ++p) {
             const int live = p < n_active && p < 4u;   /* velocity_only keeps every point (:625-626) */
             const size_t mp = gid * 4u + p;

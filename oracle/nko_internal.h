@@ -93,6 +93,11 @@ struct nko_world {
     float *solver_residual;
     /* solver state kept between steps (block_descent.cu BlockScratch articulation_velocity/free) */
     float *solver_velocity, *solver_free, *solver_penalty;
+    /* contact cache carried between steps (fields.yaml:524-539, 155, 791, 844) */
+    uint64_t *contact_material, *contact_cache_pair, *contact_cache_feature, *contact_cache_material;
+    float *contact_cache_lambda, *contact_cache_normal;
+    uint32_t *contact_cache_age, *contact_cache_current_owner, *contact_cache_old_keep, *contact_cache_extent;
+    uint32_t *contact_warm_start_counts, *contact_cache_match;
 };
 
 /* ---- math (nko_math.c) ------------------------------------------------- */
@@ -134,6 +139,9 @@ void nko_env_aabbs(nko_world* w, uint32_t env);
 void nko_env_pairs(nko_world* w, uint32_t env);
 void nko_env_narrowphase(nko_world* w, uint32_t env);
 void nko_env_assemble_rows(nko_world* w, uint32_t env);
+void nko_env_warm_start_prepare(nko_world* w, uint32_t env);
+void nko_env_warm_start_commit(nko_world* w, uint32_t env);
+uint64_t nko_contact_material(float mu1, float mu2, uint32_t law);
 void nko_env_solve(nko_world* w, uint32_t env);
 void nko_joint_transform(const nko_world* w, uint32_t env, uint32_t link, float X[36]);
 void nko_motion_subspace(uint8_t type, v3 axis, float s[6]);

@@ -173,6 +173,12 @@ nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc*
     w->env_status = ALLOC(uint32_t, E); w->vbd_velocity_sweep_count = ALLOC(uint32_t, E);
     w->solver_residual = ALLOC(float, E * 4u);
     w->solver_velocity = ALLOC(float, E * md); w->solver_free = ALLOC(float, E * md); w->solver_penalty = ALLOC(float, E * R);
+    w->contact_material = ALLOC(uint64_t, E * S); w->contact_cache_pair = ALLOC(uint64_t, E * S * 4u);
+    w->contact_cache_feature = ALLOC(uint64_t, E * S * 4u); w->contact_cache_material = ALLOC(uint64_t, E * S * 4u);
+    w->contact_cache_lambda = ALLOC(float, E * S * 16u); w->contact_cache_normal = ALLOC(float, E * S * 12u);
+    w->contact_cache_age = ALLOC(uint32_t, E * S * 4u); w->contact_cache_current_owner = ALLOC(uint32_t, E * S * 4u);
+    w->contact_cache_old_keep = ALLOC(uint32_t, E * S * 4u); w->contact_cache_extent = ALLOC(uint32_t, E * 2u);
+    w->contact_warm_start_counts = ALLOC(uint32_t, E * 2u); w->contact_cache_match = ALLOC(uint32_t, E * S * 4u);
     for (size_t i = 0u; i < E * R; ++i) { w->row_cj_link[i] = NKO_INVALID; w->row_cj_link_b[i] = NKO_INVALID; }
     for (size_t e = 0u; e < E; ++e) {
         const float id[7] = {0, 0, 0, 1, 0, 0, 0};
@@ -196,6 +202,9 @@ void nko_world_destroy(nko_world* w) {
     free(w->chain_jacobian_b); free(w->row_cj_link); free(w->row_cj_link_b); free(w->row_count); free(w->contact_count);
     free(w->contact_row_extent); free(w->env_status); free(w->vbd_velocity_sweep_count); free(w->solver_residual);
     free(w->solver_velocity); free(w->solver_free); free(w->solver_penalty);
+    free(w->contact_material); free(w->contact_cache_pair); free(w->contact_cache_feature); free(w->contact_cache_material);
+    free(w->contact_cache_lambda); free(w->contact_cache_normal); free(w->contact_cache_age); free(w->contact_cache_current_owner);
+    free(w->contact_cache_old_keep); free(w->contact_cache_extent); free(w->contact_warm_start_counts); free(w->contact_cache_match);
     free(w);
 }
 
@@ -215,7 +224,12 @@ void nko_world_destroy(nko_world* w) {
     X(chain_jacobian, float, E * R * md) X(chain_jacobian_b, float, E * R * md) X(row_cj_link, uint32_t, E * R) \
     X(row_cj_link_b, uint32_t, E * R) X(row_count, uint32_t, E) X(contact_count, uint32_t, E) \
     X(contact_row_extent, uint32_t, E * 2u) X(env_status, uint32_t, E) X(vbd_velocity_sweep_count, uint32_t, E) \
-    X(solver_residual, float, E * 4u) X(solver_penalty, float, E * R)
+    X(solver_residual, float, E * 4u) X(solver_penalty, float, E * R) \
+    X(contact_material, uint64_t, E * S) X(contact_cache_pair, uint64_t, E * S * 4u) X(contact_cache_feature, uint64_t, E * S * 4u) \
+    X(contact_cache_material, uint64_t, E * S * 4u) X(contact_cache_lambda, float, E * S * 16u) \
+    X(contact_cache_normal, float, E * S * 12u) X(contact_cache_age, uint32_t, E * S * 4u) \
+    X(contact_cache_current_owner, uint32_t, E * S * 4u) X(contact_cache_old_keep, uint32_t, E * S * 4u) \
+    X(contact_cache_extent, uint32_t, E * 2u) X(contact_warm_start_counts, uint32_t, E * 2u)
 
 #define TEMPLATE_LIST(X) \
     X(link_inertia, float, nl * 36u) X(link_tree_depth, uint32_t, nl) X(link_child_range, uint32_t, nl * 2u) \
@@ -258,9 +272,11 @@ void nko_build_aabbs(nko_world* w) { FOR_ENVS(nko_env_aabbs(w, env)) }
 void nko_query_pairs(nko_world* w) { FOR_ENVS(nko_env_pairs(w, env)) }
 void nko_narrowphase(nko_world* w) { FOR_ENVS(nko_env_narrowphase(w, env)) }
 void nko_assemble_rows(nko_world* w) { FOR_ENVS(nko_env_assemble_rows(w, env)) }
-/* assemble_rows.cu:1393-1455: with an empty cache (first step, or no persistence) every multiplier starts at 0,
- * which AssembleRows already wrote; cache persistence across steps is not restated. */
-void nko_contact_warm_start(nko_world* w, uint32_t phase) { (void)w; (void)phase; }
+/* assemble_rows.cu:1393-1455: phase 0 seeds the rows from the cache, phase 1 rebuilds the cache from the solution */
+void nko_contact_warm_start(nko_world* w, uint32_t phase) {
+    if (phase == 0u) { FOR_ENVS(nko_env_warm_start_prepare(w, env)) }
+    else { FOR_ENVS(nko_env_warm_start_commit(w, env)) }
+}
 void nko_block_descent_solve(nko_world* w) { FOR_ENVS(nko_env_solve(w, env)) }
 void nko_integrate_position(nko_world* w) { FOR_ENVS(nko_env_integrate_position(w, env)) }
 void nko_fk_link_velocities(nko_world* w) { FOR_ENVS(nko_env_link_velocities(w, env)) }

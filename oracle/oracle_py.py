@@ -13,8 +13,10 @@ U32_FIELDS = {"candidate_pairs", "pair_count", "ucontact_count", "ucontact_a", "
               "ucontact_row_range", "row_cj_link", "row_cj_link_b", "row_count", "contact_count",
               "contact_row_extent", "env_status", "vbd_velocity_sweep_count", "link_tree_depth",
               "link_child_range", "link_children", "link_dof", "dof_link", "dof_component", "link_body",
-              "body_to_link", "body_collidable_link", "body_collidable_body"}
-U64_FIELDS = {"ucontact_id_pair", "ucontact_id_feature"}
+              "body_to_link", "body_collidable_link", "body_collidable_body", "contact_cache_age",
+              "contact_cache_current_owner", "contact_cache_old_keep", "contact_cache_extent", "contact_warm_start_counts"}
+U64_FIELDS = {"ucontact_id_pair", "ucontact_id_feature", "contact_material", "contact_cache_pair", "contact_cache_feature",
+              "contact_cache_material"}
 
 
 def build(force=False):

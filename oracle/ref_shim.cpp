@@ -143,6 +143,17 @@ void ref_merge_friction(float mu_a, float mu_b, float* out) {
     out[0] = m.mu1; out[1] = m.mu2; out[2] = float(m.condim); out[3] = m.margin;
 }
 
+// MergeContactParams of two default-authored profiles that differ in friction: every field the slot material key hashes.
+void ref_merged_profile(float mu_a, float mu_b, float* out) {
+    scene::ContactParamsIn a, b;
+    a.mu1 = a.mu2 = mu_a; b.mu1 = b.mu2 = mu_b;
+    const auto m = scene::MergeContactParams(a, b);
+    out[0] = m.mu1; out[1] = m.mu2; out[2] = m.friction_spin; out[3] = m.friction_roll; out[4] = m.solref[0]; out[5] = m.solref[1];
+    for (int i = 0; i < 5; ++i) out[6 + i] = m.solimp[i];
+    out[11] = m.margin; out[12] = m.gap; out[13] = float(m.condim); out[14] = m.friction_stiffness;
+    out[15] = m.solreffriction[0]; out[16] = m.solreffriction[1];
+}
+
 int ref_shape_filter_admits(uint32_t ta, uint32_t aa, uint32_t ga, uint32_t tb, uint32_t ab, uint32_t gb) {
     return collision::ShapeFilterAdmits(ta, aa, ga, tb, ab, gb) ? 1 : 0;
 }

@@ -302,3 +302,52 @@ def test_checkpoint_restore_replays_the_same_step(oracle_py, device):
     nk.lib().nuka_checkpoint_destroy(seeded)
     world.close()
     oracle.close()
+
+
+def test_contact_cache_follows_the_oracle_over_steps(oracle_py, device):
+    """ContactWarmStart over several steps of tilted boxes (feature-id corners persist, so the cache matches and
+    seeds): keys, ages, owners, retained entries, extents and match counts bit-exact; cached impulses to TOL."""
+    from test_gpu_properties import box_template
+    E = 64
+    t = box_template(True)
+    g = np.random.default_rng(4)
+    quat = np.array([1, 0, 0, 0]) + g.normal(0, 0.04, (E, 4))
+    base = np.concatenate([g.normal(0, 0.2, (E, 2)), g.uniform(0.035, 0.05, (E, 1)), quat / np.linalg.norm(quat, axis=1, keepdims=True)], 1)
+    zero = np.zeros((E, 1), np.float32)
+    state = dict(q=np.concatenate([zero, g.uniform(-0.3, 0.6, (E, 1))], 1).astype(np.float32), qdot=np.zeros((E, 2), np.float32),
+                 tau=np.zeros((E, 2), np.float32), base_pose=base.astype(np.float32), root_twist=np.zeros((E, 6), np.float32))
+    desc = nk.abi.world_desc(E, 1.0 / 200.0, vel_iters=30)
+    world, oracle = nk.World(device, t, desc), oracle_py.OracleWorld(t, desc, threads=4)
+    world.set_state(state)
+    oracle.set_state(state)
+    matched = 0
+    for step in range(5):
+        world.step()
+        world.synchronize()
+        oracle.step()
+        for name in ("contact_material", "contact_cache_current_owner", "contact_cache_old_keep", "contact_cache_extent",
+                     "contact_warm_start_counts", "contact_cache_age"):
+            assert np.array_equal(world.download(name), oracle.download(name)), f"step {step}: {name}"
+        same = world.download("contact_cache_pair") == oracle.download("contact_cache_pair")
+        assert same.all()
+        # sphere points hash a quantised position into their feature word; box corners carry exact ids
+        assert np.mean(world.download("contact_cache_feature") == oracle.download("contact_cache_feature")) > 0.99
+        assert relative_error(world.download("contact_cache_lambda"), oracle.download("contact_cache_lambda")) <= TOL
+        assert relative_error(world.download("contact_cache_normal"), oracle.download("contact_cache_normal")) <= TOL
+        assert relative_error(world.download("qdot"), oracle.download("qdot")) <= TOL
+        matched += int(oracle.download("contact_warm_start_counts").reshape(E, 2)[:, 1].sum())
+    assert matched > E
+    # the seeding itself: phase 0 on both sides from the same cache
+    for name, oname in (("FkWorldPoses", "fk_world_poses"), ("ArticulationDynamics", "articulation_dynamics")):
+        oracle.op(oname, *((1,) if oname == "articulation_dynamics" else ()))
+        world.op(name)
+    for name in UPSTREAM[2:]:
+        both(oracle, world, name)
+    oracle.op("contact_warm_start", 0)
+    world.op("ContactWarmStart", 0)
+    world.synchronize()
+    seeds = oracle.download("lambda")
+    assert np.count_nonzero(seeds) > E
+    assert relative_error(world.download("lambda"), seeds) <= TOL
+    world.close()
+    oracle.close()
