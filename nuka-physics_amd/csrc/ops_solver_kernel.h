@@ -62,16 +62,23 @@ __device__ __forceinline__ void tile_merge(TileSum& s, float value, float error)
     s.error += error;
     tile_add(s, value);
 }
-__device__ __forceinline__ float wave_total(TileSum s) {
+__device__ __forceinline__ float wave_total(TileSum s, bool first_row_only = false) {
     tile_merge(s, dpp_move<kDppXor1>(s.value), dpp_move<kDppXor1>(s.error));
     tile_merge(s, dpp_move<kDppXor2>(s.value), dpp_move<kDppXor2>(s.error));
     tile_merge(s, dpp_move<kDppHalfMirror>(s.value), dpp_move<kDppHalfMirror>(s.error));
     tile_merge(s, dpp_move<kDppMirror>(s.value), dpp_move<kDppMirror>(s.error));
-    TileSum a{row_value(s.value, 0), row_value(s.error, 0)}, b{row_value(s.value, 2), row_value(s.error, 2)};
+    TileSum a{row_value(s.value, 0), row_value(s.error, 0)};
+    // lanes 16..63 hold exact zeros when only the first sixteen lanes carry terms: merging them changes nothing
+    if (first_row_only) return a.value + a.error;
+    TileSum b{row_value(s.value, 2), row_value(s.error, 2)};
     tile_merge(a, row_value(s.value, 1), row_value(s.error, 1));
     tile_merge(b, row_value(s.value, 3), row_value(s.error, 3));
     tile_merge(a, b.value, b.error);
     return a.value + a.error;
+}
+__device__ __forceinline__ float first_row_sum(float v) {
+    v += dpp_move<kDppXor1>(v); v += dpp_move<kDppXor2>(v); v += dpp_move<kDppHalfMirror>(v); v += dpp_move<kDppMirror>(v);
+    return row_value(v, 0);
 }
 
 struct Response { float dual_scale, residual_scale; };
@@ -97,12 +104,14 @@ __device__ __forceinline__ void scalar_impulse(float dual, float rho, float resi
 }
 // augmented_row.hpp:302-318
 __device__ __forceinline__ float cone_argument(float dual, float rho, float mu, float residual) {
+    // a friction ratio of exactly one (equal coefficients) divides to the dividend itself: skip the two divisions
+    const bool unit = mu == 1.0f;
     const bool dual_zero = dual == 0.0f;
-    const float dual_quotient = (dual + float(dual_zero)) / mu;
+    const float dual_quotient = unit ? dual + float(dual_zero) : (dual + float(dual_zero)) / mu;
     const float dd = dual_zero ? dual : dual_quotient;
     const float low = fmaf(-dd, mu, dual);
     const bool low_zero = low == 0.0f;
-    const float low_quotient = (low + float(low_zero)) / mu;
+    const float low_quotient = unit ? low + float(low_zero) : (low + float(low_zero)) / mu;
     const float d_low = low_zero ? low : low_quotient;
     const float p = rho * mu;
     const float t = p * residual;
@@ -586,9 +595,11 @@ __device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& 
         tile_add_product(total, alpha, inertial_curvature);
         tile_add(total, inertial_slope);
     }
-    *slope = wave_total(total);
-    *curvature = inertial_curvature + wave_sum(row_curvature);
-    *magnitude = fabsf(inertial_slope) + alpha * inertial_curvature + wave_sum(row_magnitude);
+    // with at most sixteen heads every term sits in the first row of lanes; (t + 0) + (0 + 0) is t, so the sums agree
+    const bool narrow = c.heads <= 16u;
+    *slope = wave_total(total, narrow);
+    *curvature = inertial_curvature + (narrow ? first_row_sum(row_curvature) : wave_sum(row_curvature));
+    *magnitude = fabsf(inertial_slope) + alpha * inertial_curvature + (narrow ? first_row_sum(row_magnitude) : wave_sum(row_magnitude));
 }
 
 // SearchTileLine (:2089-2125)
