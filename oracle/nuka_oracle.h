@@ -7,22 +7,31 @@
  * split-impulse position pass.  Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline
  * leg may load it, and only as the checker.  Nothing shipped links or calls it.
  *
- * Every function in nuka_oracle.c cites the reference file:line it follows.  Compile without
- * fast-math and with -ffp-contract=off: fused multiply-adds appear only where the reference
- * writes fmaf/__fmaf_rn itself.
+ * Every function in nko_*.c cites the reference file:line it follows.  Compile without fast-math and
+ * with -ffp-contract=off: fused multiply-adds appear only where the reference writes fmaf itself.
  *
- * Parity status per function group (what pins it beyond "it restates the reference"):
- *   cook / spatial inertia  : pinned (parallel-axis closed form, symmetry; tests/test_oracle_dynamics.py)
- *   forward kinematics      : pinned (planar chain closed form, composition invariants)
- *   dynamics (bias, M, LDL) : pinned (pendulum closed forms, RNEA column identity, kinetic energy,
- *                             independent ABA recursion in tests, double-precision LDL reconstruction)
- *   pairs / slots / rows    : pinned (brute-force O(B^2) enumeration + sort; integer exact)
- *   manifolds               : pinned against oracle/_ref (the reference's own analytical_manifold.hpp)
- *   row math (AL impulses)  : pinned against oracle/_ref (the reference's own augmented_row.hpp) and
+ * Parity status per function group (what pins it beyond "it restates the reference"; tests/ holds each check):
+ *   cook / spatial inertia  : pinned (parallel-axis closed form)
+ *   forward kinematics      : pinned (float64 rotation-matrix kinematics on all four configurations)
+ *   dynamics (bias, M, LDL) : pinned (pendulum closed form with damping, spring, armature; M as the kinetic-energy
+ *                             form and the bias as the Euler-Lagrange bias of an independent float64 model built
+ *                             from finite differences of poses; first-order energy drift and momentum laws of
+ *                             free motion, fixed and floating base; LDL^T reconstruction and dense solves)
+ *   link velocities, integration : pinned (pose rates of the float64 model; the conservation runs above)
+ *   pairs / slots / rows    : pinned (brute-force O(B^2) overlap enumeration in canonical order; integer exact)
+ *   manifolds, compose, contact id, query band, filter, projection roundoff :
+ *                             pinned bit-exact against oracle/_ref (the reference's own host headers) and the
+ *                             committed vectors tests/golden/rowmath_vectors.npz; the prim-frame bake is device-only
+ *                             code and is pinned by the rotation-matrix closed form instead
+ *   row math (AL impulses)  : pinned bit-exact against oracle/_ref (augmented_row.hpp), the committed vectors, and
  *                             the known answers in tests/math/test_contact_tangent.cpp
- *   chain Jacobian          : pinned (J qdot == contact point velocity from link twists)
- *   UABD fixed point        : pinned (KKT invariants, momentum balance, frictionless closed form,
- *                             brute-force PGS on <= 3 contacts)
+ *   chain Jacobian          : pinned (J qdot == contact point velocity of the float64 model)
+ *   contact cache           : pinned by behaviour (seeding of a persisting contact, one-step retention and decay,
+ *                             layout invariants); the merged profile terms of the material key against the
+ *                             reference's MergeContactParams.  The key's hash routine is device-only code:
+ *                             PARITY UNPINNED for its constants.
+ *   UABD fixed point        : pinned (closed-form resting, falling, sticking and sliding ball; Coulomb / KKT
+ *                             conditions and momentum balance of converged solves)
  *   UABD iterate path       : PARITY UNPINNED - penalty heuristic, first-sweep segment search, FISTA
  *                             restart timing, secant relaxation and the 8-epsilon waivers decide the
  *                             multipliers held after a fixed sweep budget; only a running reference
