@@ -281,8 +281,12 @@ struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
     }
 };
 
-// Checkpoint of the persistent physics (src/include/nuka/nuka.h:388-392): every state field a step reads before it
-// writes it.  The mass matrix, its factor and the contact Jacobians are rebuilt by every step and stay out.
+// Checkpoint of the persistent physics (src/include/nuka/nuka.h:388-392): the fields the reference keeps in its
+// persistent arena (fields.yaml: q, qdot, qddot, tau, base_pose, link_pose, link_velocity, body_pose, lambda and the
+// contact cache) plus the applied link wrench.  Everything else is per-step scratch; a restore puts the scratch a
+// step reads before writing into its cleared state - row and cache extents of zero make the next assembly clear
+// every row, carried solver velocities of zero start the solve from the free velocity, status words are cleared -
+// the lifecycle of a reset (op_schema.hpp:936 RestoreStateParams).
 constexpr uint32_t kMaxCheckpointSegments = 64u;
 struct CheckpointSegments {
     uint32_t count;
@@ -300,14 +304,27 @@ struct Checkpoint {
 // blockIdx.y picks the segment, blockIdx.x strides over its 16-byte units.
 __global__ void __launch_bounds__(256) CheckpointCopyKernel(CheckpointSegments s, uint32_t restore) {
     const uint32_t seg = blockIdx.y;
+    if (s.kept[seg] == nullptr) {   // a scratch field a restore clears; a capture leaves it alone
+        if (restore == 0u) return;
+        uint4* cleared = reinterpret_cast<uint4*>(s.live[seg]);
+        for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < s.units[seg]; i += gridDim.x * blockDim.x) cleared[i] = uint4{0u, 0u, 0u, 0u};
+        return;
+    }
     const uint4* src = reinterpret_cast<const uint4*>(restore != 0u ? s.kept[seg] : s.live[seg]);
     uint4* dst = reinterpret_cast<uint4*>(restore != 0u ? s.live[seg] : s.kept[seg]);
     for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < s.units[seg]; i += gridDim.x * blockDim.x) dst[i] = src[i];
 }
 
-bool CheckpointExcludes(const char* name) {
-    // rebuilt by every step, or scheduling hints that are no part of the physics
-    for (const char* rebuilt : {"m", "m_factor", "chain_jacobian", "chain_jacobian_b", "solver_cost", "tile_order"}) if (std::strcmp(name, rebuilt) == 0) return true;
+bool CheckpointKeeps(const char* name) {
+    for (const char* kept : {"q", "qdot", "qddot", "tau", "base_pose", "link_pose", "link_velocity", "body_pose", "lambda", "link_wrench",
+                             "contact_cache_pair", "contact_cache_feature", "contact_cache_material", "contact_cache_lambda",
+                             "contact_cache_normal", "contact_cache_age"})
+        if (std::strcmp(name, kept) == 0) return true;
+    return false;
+}
+bool CheckpointClears(const char* name) {
+    for (const char* cleared : {"contact_row_extent", "contact_cache_extent", "solver_velocity", "solver_free", "env_status"})
+        if (std::strcmp(name, cleared) == 0) return true;
     return false;
 }
 
@@ -838,9 +855,9 @@ nuka_result_t nuka_world_checkpoint_capture(nuka_world_handle world, nuka_checkp
     cp->owner = w;
     size_t total = 0u;
     for (const Field& f : w->fields) {
-        if (f.is_template || f.count == 0u || CheckpointExcludes(f.name)) continue;
+        if (f.is_template || f.count == 0u || !(CheckpointKeeps(f.name) || CheckpointClears(f.name))) continue;
         if (cp->segments.count == kMaxCheckpointSegments) return Error(NUKA_RESULT_INTERNAL, "too many checkpoint segments");
-        total += (f.count * f.elem_bytes + 255u) & ~size_t{255u};
+        if (CheckpointKeeps(f.name)) total += (f.count * f.elem_bytes + 255u) & ~size_t{255u};
         ++cp->segments.count;
     }
     uint8_t status = 0u;
@@ -852,12 +869,12 @@ nuka_result_t nuka_world_checkpoint_capture(nuka_world_handle world, nuka_checkp
     uint32_t at = 0u;
     size_t offset = 0u;
     for (const Field& f : w->fields) {
-        if (f.is_template || f.count == 0u || CheckpointExcludes(f.name)) continue;
+        if (f.is_template || f.count == 0u || !(CheckpointKeeps(f.name) || CheckpointClears(f.name))) continue;
         const size_t padded = (f.count * f.elem_bytes + 255u) & ~size_t{255u};    // arena fields are 256-byte aligned and padded
         cp->segments.live[at] = arena + f.offset;
-        cp->segments.kept[at] = kept + offset;
         cp->segments.units[at] = uint32_t(padded / 16u);
-        offset += padded;
+        if (CheckpointKeeps(f.name)) { cp->segments.kept[at] = kept + offset; offset += padded; }
+        else cp->segments.kept[at] = nullptr;
         ++at;
     }
     cp->bytes = total;

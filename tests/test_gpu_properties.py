@@ -242,3 +242,26 @@ def test_backend_seam_walk_through_the_tables(device):
     backend = lib.nuka_device_backend(device._h)
     k = table(backend, 15)
     assert b"hip" in C.CFUNCTYPE(C.c_char_p, C.c_void_p)(k[0])(backend).lower()
+
+
+@pytest.mark.parametrize("index,E", [(2, 4096), (3, 4096)])
+def test_published_batch_sizes_match_the_oracle_directly(oracle_py, device, index, E):
+    """The whole published batch, not a sample: one step of all 4096 environments against the oracle (the oracle takes
+    a fraction of a second for this on a few threads)."""
+    cfg = nk.synthetic.config(index, E)
+    desc = abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters)
+    world, oracle = nk.World(device, cfg.template, desc), oracle_py.OracleWorld(cfg.template, desc, threads=16)
+    state = cfg.state()
+    world.set_state(state)
+    oracle.set_state(state)
+    world.step()
+    world.synchronize()
+    oracle.step()
+    for name in ("pair_count", "ucontact_count", "ucontact_row_range", "row_count", "env_status", "contact_cache_pair",
+                 "contact_cache_age", "contact_warm_start_counts"):
+        assert np.array_equal(world.download(name), oracle.download(name)), name
+    for name in ("articulation_qdd", "link_pose", "body_pose", "q", "qdot", "link_velocity"):
+        error = relative_error(world.download(name), oracle.download(name))
+        assert error <= 1e-4, f"{name}: {error:.2e}"
+    world.close()
+    oracle.close()
