@@ -111,6 +111,8 @@ nuka_result_t nuka_world_set_velocity_iterations(nuka_world_handle world, uint32
 nuka_result_t nuka_world_get_velocity_iterations(nuka_world_handle world, uint32_t* out_iterations);
 nuka_result_t nuka_world_synchronize(nuka_world_handle world);   /* nuka.h:376 */
 nuka_result_t nuka_world_reset(nuka_world_handle world);         /* nuka.h:380 */
+/* nuka.h:381-385: duplicates are ignored, count 0 is a no-op, an id out of range returns INVALID_ARG and changes nothing */
+nuka_result_t nuka_world_reset_envs(nuka_world_handle world, const uint32_t* env_ids, uint32_t count);
 
 /* nuka.h:386-398: a checkpoint holds the persistent physics of every environment, in device memory here.  Restore
  * is enqueued on the world's stream (no host wait) and refuses a checkpoint of another world. */

@@ -38,7 +38,7 @@ EXPORTS = [
     "nuka_result_message", "nuka_last_error_message", "nuka_device_create", "nuka_device_destroy", "nuka_device_backend",
     "nuka_world_create_from_template", "nuka_world_destroy", "nuka_world_step", "nuka_world_step_n",
     "nuka_world_set_execution_mode", "nuka_world_set_velocity_iterations", "nuka_world_get_velocity_iterations",
-    "nuka_world_synchronize", "nuka_world_reset", "nuka_world_checkpoint_capture", "nuka_world_checkpoint_restore",
+    "nuka_world_synchronize", "nuka_world_reset", "nuka_world_reset_envs", "nuka_world_checkpoint_capture", "nuka_world_checkpoint_restore",
     "nuka_checkpoint_destroy", "nuka_checkpoint_byte_size", "nuka_world_dispatch_op", "nuka_field_from_name", "nuka_field_names",
     "nuka_world_get_buffer_view", "nuka_world_upload_field", "nuka_world_download_field", "nuka_world_get_info",
     "nuka_world_time_steps", "nuka_world_profile_ops", "nuka_device_copy_bandwidth", "nuka_hip_register_backend_entry",
@@ -82,6 +82,7 @@ def lib():
         L.nuka_world_get_velocity_iterations.argtypes = [C.c_void_p, C.POINTER(C.c_uint32)]
         L.nuka_world_synchronize.argtypes = [C.c_void_p]
         L.nuka_world_reset.argtypes = [C.c_void_p]
+        L.nuka_world_reset_envs.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32]
         L.nuka_world_dispatch_op.argtypes = [C.c_void_p, C.c_uint16, C.c_uint32]
         L.nuka_field_from_name.argtypes = [C.c_char_p]
         L.nuka_field_from_name.restype = C.c_uint32
@@ -206,6 +207,10 @@ class World:
 
     def reset(self):
         _check(lib().nuka_world_reset(self._h))
+
+    def reset_envs(self, env_ids):
+        ids = np.ascontiguousarray(np.asarray(env_ids, dtype=np.uint32))
+        _check(lib().nuka_world_reset_envs(self._h, ids.ctypes.data, ids.size))
 
     def set_execution_mode(self, graph):
         _check(lib().nuka_world_set_execution_mode(self._h, 1 if graph else 0))

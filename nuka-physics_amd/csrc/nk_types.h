@@ -102,6 +102,7 @@ struct DataView {
     float *contact_cache_lambda, *contact_cache_normal;
     uint32_t *contact_cache_age, *contact_cache_current_owner, *contact_cache_old_keep, *contact_cache_extent;
     uint32_t *contact_warm_start_counts, *contact_cache_match;
+    uint32_t *reset_env_ids;                // staging of nuka_world_reset_envs
     uint32_t *solver_cost, *tile_order;     // last solve's work per environment; launch order of the next solve (costliest first)
     float *snapshot;                        // SnapshotState / RestoreState storage
 };

@@ -224,7 +224,8 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(contact_material, kU64, E * S) X(contact_cache_pair, kU64, E * S * 4) X(contact_cache_feature, kU64, E * S * 4) \
     X(contact_cache_material, kU64, E * S * 4) X(contact_cache_lambda, kF32, E * S * 16) X(contact_cache_normal, kF32, E * S * 12) \
     X(contact_cache_age, kU32, E * S * 4) X(contact_cache_current_owner, kU32, E * S * 4) X(contact_cache_old_keep, kU32, E * S * 4) \
-    X(contact_cache_extent, kU32, E * 2) X(contact_warm_start_counts, kU32, E * 2) X(contact_cache_match, kU32, E * S * 4)
+    X(contact_cache_extent, kU32, E * 2) X(contact_warm_start_counts, kU32, E * 2) X(contact_cache_match, kU32, E * S * 4) \
+    X(reset_env_ids, kU32, E)
 
 #define NKH_MODEL_FIELDS(X) \
     X(joint_type, kU8) X(parent_link, kU32) X(joint_axis, kF32) X(parent_offset, kF32) X(link_local_pose, kF32) \
@@ -313,6 +314,23 @@ __global__ void __launch_bounds__(256) CheckpointCopyKernel(CheckpointSegments s
     const uint4* src = reinterpret_cast<const uint4*>(restore != 0u ? s.kept[seg] : s.live[seg]);
     uint4* dst = reinterpret_cast<uint4*>(restore != 0u ? s.live[seg] : s.kept[seg]);
     for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < s.units[seg]; i += gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
+// ResetEnvs (op_schema.hpp:904-926): the selected environments get their slice of every persistent field back from
+// the snapshot taken at creation, and their per-step history cleared.  blockIdx.x = selected environment,
+// blockIdx.y = field; words of four bytes, since an environment's slice of a field need not be 16-byte aligned.
+struct ResetSegments {
+    uint32_t count;
+    uint32_t words_per_env[kMaxCheckpointSegments];
+    uint32_t* live[kMaxCheckpointSegments];
+    const uint32_t* initial[kMaxCheckpointSegments];   // null: clear
+};
+__global__ void __launch_bounds__(256) ResetEnvsKernel(ResetSegments s, const uint32_t* ids, uint32_t env_count) {
+    const uint32_t env = ids[blockIdx.x], seg = blockIdx.y;
+    if (env >= env_count) return;
+    const size_t first = size_t{env} * s.words_per_env[seg];
+    for (uint32_t i = threadIdx.x; i < s.words_per_env[seg]; i += blockDim.x)
+        s.live[seg][first + i] = s.initial[seg] != nullptr ? s.initial[seg][first + i] : 0u;
 }
 
 bool CheckpointKeeps(const char* name) {
@@ -682,6 +700,38 @@ nuka_result_t nuka_world_reset(nuka_world_handle world) {
     if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
     if (Iface(w->arena)->copy_from(w->arena, w->initial, 0u, 0u, w->arena_bytes) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "reset copy failed");
     return nuka_world_synchronize(world);
+}
+
+nuka_result_t nuka_world_reset_envs(nuka_world_handle world, const uint32_t* env_ids, uint32_t count) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (count == 0u) return NUKA_RESULT_OK;
+    if (env_ids == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "env_ids is null");
+    // an invalid id changes nothing; duplicates are dropped so that no two workgroups write one slice
+    std::vector<uint8_t> seen(w->env_count, 0u);
+    std::vector<uint32_t> unique;
+    for (uint32_t i = 0u; i < count; ++i) {
+        if (env_ids[i] >= w->env_count) return Error(NUKA_RESULT_INVALID_ARG, "environment id out of range");
+        if (seen[env_ids[i]] == 0u) { seen[env_ids[i]] = 1u; unique.push_back(env_ids[i]); }
+    }
+    ResetSegments segments{};
+    char* arena = static_cast<char*>(Iface(w->arena)->base(w->arena));
+    const char* initial = static_cast<const char*>(Iface(w->initial)->base(w->initial));
+    for (const Field& f : w->fields) {
+        if (f.is_template || f.count == 0u || !(CheckpointKeeps(f.name) || CheckpointClears(f.name))) continue;
+        if (segments.count == kMaxCheckpointSegments) return Error(NUKA_RESULT_INTERNAL, "too many reset segments");
+        const uint32_t at = segments.count++;
+        segments.words_per_env[at] = uint32_t(f.count * f.elem_bytes / 4u / w->env_count);
+        segments.live[at] = reinterpret_cast<uint32_t*>(arena + f.offset);
+        segments.initial[at] = CheckpointKeeps(f.name) ? reinterpret_cast<const uint32_t*>(initial + f.offset) : nullptr;
+    }
+    if (nuka_world_synchronize(world) != NUKA_RESULT_OK) return NUKA_RESULT_DEVICE_ERROR;
+    if (hipMemcpyAsync(w->data.reset_env_ids, unique.data(), unique.size() * sizeof(uint32_t), hipMemcpyHostToDevice,
+                       BackendStream(w->device->backend)) != hipSuccess) return Error(NUKA_RESULT_DEVICE_ERROR, "id upload failed");
+    hipLaunchKernelGGL(ResetEnvsKernel, dim3(uint32_t(unique.size()), segments.count), dim3(256), 0, BackendStream(w->device->backend),
+                       segments, w->data.reset_env_ids, w->env_count);
+    if (hipGetLastError() != hipSuccess) return Error(NUKA_RESULT_DEVICE_ERROR, "reset launch failed");
+    return nuka_world_synchronize(world);   // the host copy of the ids must outlive the upload
 }
 
 nuka_result_t nuka_world_dispatch_op(nuka_world_handle world, uint16_t op, uint32_t variant) {

@@ -265,3 +265,49 @@ def test_published_batch_sizes_match_the_oracle_directly(oracle_py, device, inde
         assert error <= 1e-4, f"{name}: {error:.2e}"
     world.close()
     oracle.close()
+
+
+def test_reset_envs_restores_the_selected_environments_only(device):
+    """nuka_world_reset_envs: the chosen environments return to the state the world was created with and lose their
+    contact and solver history; the others are untouched; duplicates are ignored and a bad id changes nothing."""
+    E = 64
+    cfg = nk.synthetic.config(2, E)
+    desc = abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters)
+    world = nk.World(device, cfg.template, desc)
+    created = {n: world.download(n) for n in ("q", "qdot", "base_pose", "link_pose", "lambda")}
+    state = cfg.state()
+    world.set_state(state)
+    world.step(3)
+    world.synchronize()
+    before = {n: world.download(n) for n in ("q", "qdot", "base_pose", "link_pose", "lambda", "contact_cache_pair", "contact_row_extent")}
+    assert nk.lib().nuka_world_reset_envs(world._h, np.array([2, 99], np.uint32).ctypes.data, 2) == 1
+    assert all(np.array_equal(world.download(n), v) for n, v in before.items())
+    assert nk.lib().nuka_world_reset_envs(world._h, None, 0) == 0
+    chosen = [3, 17, 3, 40]
+    world.reset_envs(chosen)
+    picked = np.zeros(E, bool)
+    picked[chosen] = True
+    for n in ("q", "qdot", "base_pose", "link_pose", "lambda"):
+        now, was, new = (a.reshape(E, -1) for a in (world.download(n), before[n], created[n]))
+        assert np.array_equal(now[~picked], was[~picked]) and np.array_equal(now[picked], new[picked]), n
+    assert np.all(world.download("contact_cache_pair").reshape(E, -1)[picked] == 0)
+    assert np.all(world.download("contact_row_extent").reshape(E, 2)[picked] == 0)
+    assert np.array_equal(world.download("contact_cache_pair").reshape(E, -1)[~picked], before["contact_cache_pair"].reshape(E, -1)[~picked])
+    # a reset environment, given its seeded state again, steps exactly as it did in a fresh world
+    fresh = nk.World(device, cfg.template, desc)
+    fresh.set_state(state)
+    fresh.step()
+    fresh.synchronize()
+    for name, key in (("q", "q"), ("qdot", "qdot"), ("tau", "tau"), ("base_pose", "base_pose")):
+        current = world.download(name).reshape(E, -1)
+        current[picked] = np.asarray(state[key], np.float32).reshape(E, -1)[picked]
+        world.upload(name, current)
+    twist = world.download("link_velocity").reshape(E, -1, 6)
+    twist[picked, 0, :] = state["root_twist"][picked]
+    world.upload("link_velocity", twist)
+    world.step()
+    world.synchronize()
+    for n in ("q", "qdot", "lambda", "link_pose"):
+        assert np.array_equal(world.download(n).reshape(E, -1)[picked], fresh.download(n).reshape(E, -1)[picked]), n
+    fresh.close()
+    world.close()
