@@ -164,7 +164,7 @@ __device__ __forceinline__ float along_axis(float impulse, float velocity) { ret
 enum HeadField : uint32_t {
     hSlot, hStride, hAxes, hOwned, hRho, hCompliance, hLower, hUpper, hMu1, hMu2, hNormalBound,
     hRes, hDual = hRes + 3, hMove = hDual + 3, hStep = hMove + 3, hBase = hStep + 3, hDualScale = hBase + 3, hResidualScale,
-    hRelaxStep, hRelaxWeight = hRelaxStep + 3, hRelaxPoint, hF = hRelaxPoint + 3, hC = hF + 3, hNoise = hC + 6, hContrib = hNoise + 3, hColumnsLow, hColumnsHigh,
+    hRelaxStep, hRelaxWeight = hRelaxStep + 3, hRelaxPoint, hF = hRelaxPoint + 3, hC = hF + 3, hNoise = hC + 6, hContrib = hNoise + 3, hColumnsLow, hColumnsHigh, hSourceA, hSourceB = hSourceA + 3, hSourceEnd = hSourceB + 3,
     hFieldCount
 };
 
@@ -1014,28 +1014,40 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     }
     c.heads = heads;
     __syncthreads();
-    // stage Jacobian rows: the sum of the articulated sides' chain rows (TileBlock::Jacobian :555-573, CopyTileRows :836-869)
-    for (uint32_t h = 0u; h < heads; ++h) {
+    // stage Jacobian rows: the sum of the articulated sides' chain rows (TileBlock::Jacobian :555-573, CopyTileRows :836-869).
+    // First every (head, axis) row finds its source rows, one per lane; then the copies run with their loads in flight
+    // together instead of one row's latency after another.
+    for (uint32_t r = lane; r < 3u * heads; r += kWave) {
+        const uint32_t h = r / 3u, axis = r - 3u * h;
         const uint32_t slot = c.U(hSlot, h);
         const uint32_t flags = __float_as_uint(urows[size_t{slot} * kRowWords]);
         const uint32_t stride = __float_as_uint(urows[size_t{slot} * kRowWords + 2u]);
         const uint32_t axes = (flags & kRowBlockNormal) != 0u ? 3u : 1u;
-        bool used = false;
-        for (uint32_t axis = 0u; axis < 3u; ++axis) {
-            float value = 0.0f;
-            if (axis < axes && coordinate) {
-                const uint32_t rs = slot + axis * stride;
-                const uint32_t kind_a = __float_as_uint(urows[size_t{rs} * kRowWords + 10u]);
-                const uint32_t kind_b = __float_as_uint(urows[size_t{rs} * kRowWords + 18u]);
-                if (kind_a == kSideArtic) value += d.chain_jacobian[size_t{rs} * md + lane];
-                if (kind_b == kSideArtic) value += d.chain_jacobian_b[size_t{rs} * md + lane];
-            }
-            if (lane < c.ldj) c.jac[(3u * h + axis) * c.ldj + lane] = value;   // padded columns hold zeros
-            used = used || value != 0.0f;
+        uint32_t source_a = kInvalid, source_b = kInvalid;
+        if (axis < axes) {
+            const uint32_t rs = slot + axis * stride;
+            if (__float_as_uint(urows[size_t{rs} * kRowWords + 10u]) == kSideArtic) source_a = rs;
+            if (__float_as_uint(urows[size_t{rs} * kRowWords + 18u]) == kSideArtic) source_b = rs;
         }
+        c.U(hSourceA + axis, h) = source_a; c.U(hSourceB + axis, h) = source_b;
+    }
+    __syncthreads();
+#pragma unroll 2
+    for (uint32_t h = 0u; h < heads; ++h) {
+        float value[3];
+#pragma unroll
+        for (uint32_t axis = 0u; axis < 3u; ++axis) {
+            const uint32_t source_a = c.U(hSourceA + axis, h), source_b = c.U(hSourceB + axis, h);
+            value[axis] = 0.0f;
+            if (coordinate && source_a != kInvalid) value[axis] += d.chain_jacobian[size_t{source_a} * md + lane];
+            if (coordinate && source_b != kInvalid) value[axis] += d.chain_jacobian_b[size_t{source_b} * md + lane];
+        }
+#pragma unroll
+        for (uint32_t axis = 0u; axis < 3u; ++axis)
+            if (lane < c.ldj) c.jac[(3u * h + axis) * c.ldj + lane] = value[axis];   // padded columns hold zeros
         // the columns this head touches at all: a contact on one limb leaves most coordinates out, and the Hessian
         // update skips their exact-zero products four columns at a time
-        const uint64_t columns = __ballot(used);
+        const uint64_t columns = __ballot(value[0] != 0.0f || value[1] != 0.0f || value[2] != 0.0f);
         if (lane == 0u) { c.U(hColumnsLow, h) = uint32_t(columns); c.U(hColumnsHigh, h) = uint32_t(columns >> 32u); }
     }
     __syncthreads();
