@@ -182,7 +182,7 @@ struct Tile {
     float momentum, residual;
     bool failed;
 #ifdef NKH_SOLVER_PROFILE
-    mutable long long prof[16];
+    mutable long long prof[22];
     mutable uint32_t prof_count[4];
 #endif
     __device__ float& F(uint32_t field, uint32_t h) const { return fields[field * cap + h]; }
@@ -963,7 +963,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     c.tolerance = p.velocity_tolerance; c.failed = false; c.momentum = 0.0f; c.residual = 0.0f;
     c.mass_inverse = 0.0f; c.mass_valid = false; c.work = 0u;
 #ifdef NKH_SOLVER_PROFILE
-    for (int i = 0; i < 16; ++i) c.prof[i] = 0;
+    for (int i = 0; i < 22; ++i) c.prof[i] = 0;
     for (int i = 0; i < 4; ++i) c.prof_count[i] = 0u;
 #endif
     PROF_BEGIN(c, 9);
@@ -987,6 +987,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         free_v = value;
         velocity = value + (isfinite(carried) ? carried : 0.0f);
     }
+    PROF_BEGIN(c, 16);
     // ListTileHeads (:1250-1296): active rows that are not block tangents, in slot order
     const uint32_t previous = d.contact_row_extent[2u * env], current = d.contact_row_extent[2u * env + 1u];
     const uint32_t bound = previous == 0u || current == 0u ? p.contact_rows_per_env : min(max(previous, current) - 1u, p.contact_rows_per_env);
@@ -1014,6 +1015,8 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     }
     c.heads = heads;
     __syncthreads();
+    PROF_END(c, 16);
+    PROF_BEGIN(c, 17);
     // stage Jacobian rows: the sum of the articulated sides' chain rows (TileBlock::Jacobian :555-573, CopyTileRows :836-869).
     // First every (head, axis) row finds its source rows, one per lane; then the copies run with their loads in flight
     // together instead of one row's latency after another.
@@ -1051,46 +1054,87 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         if (lane == 0u) { c.U(hColumnsLow, h) = uint32_t(columns); c.U(hColumnsHigh, h) = uint32_t(columns >> 32u); }
     }
     __syncthreads();
+    PROF_END(c, 17);
+    PROF_BEGIN(c, 18);
     // TileInertialResponse (:709-739): J M^-1 J^T of every head's first row through the stored LDL^T factor
     // (ForwardMass + MassDot, articulation_mass.cuh:414-431).  lane = DoF: the unit-lower factor row sits in
     // registers with zeros from the diagonal on, each y_j travels as a scalar lane read, so row i subtracts
     // L_ij y_j for j = 0, 1, ... exactly as the serial loop does; the ordered sum of y_i^2 / D_i follows the same way.
+    float mrow[N];
     {
         const float* factor = d.m_factor + size_t{env} * md * md;
-        for (uint32_t e = lane; e < n * n; e += kWave) c.hfac[(e / n) * c.ld + e % n] = factor[size_t{e / n} * md + e % n];
+        // the mass rows ride along (StageTileMass :2127-2142), so that both matrices' loads are in flight together
+        for (uint32_t e = lane; e < n * n; e += kWave) {
+            c.hfac[(e / n) * c.ld + e % n] = factor[size_t{e / n} * md + e % n];
+            c.mfac[(e / n) * c.ld + e % n] = d.m[size_t{env} * md * md + size_t{e / n} * md + e % n];
+        }
         __syncthreads();
         float lrow[N];
 #pragma unroll
-        for (int k = 0; k < N; ++k) lrow[k] = coordinate && uint32_t(k) < lane ? c.hfac[lane * c.ld + k] : 0.0f;
+        for (int k = 0; k < N; ++k) {
+            lrow[k] = coordinate && uint32_t(k) < lane ? c.hfac[lane * c.ld + k] : 0.0f;
+            // rows and columns n..N-1 of the mass matrix are those of the identity
+            mrow[k] = coordinate && uint32_t(k) < n ? c.mfac[lane * c.ld + k] : (lane == uint32_t(k) && lane < uint32_t(N) ? 1.0f : 0.0f);
+        }
         const float pivot = coordinate ? c.hfac[lane * c.ld + lane] : 1.0f;
         __syncthreads();
-        for (uint32_t h = 0u; h < heads; ++h) {
-            const uint32_t slot = c.U(hSlot, h);
-            const float* row = urows + size_t{slot} * kRowWords;
-            const uint32_t kind_a = __float_as_uint(row[10]), index_a = __float_as_uint(row[11]);
-            const uint32_t kind_b = __float_as_uint(row[18]), index_b = __float_as_uint(row[19]);
-            const bool shared = kind_a == kind_b && index_a == index_b;
-            float shares[2] = {0.0f, 0.0f};
-            for (uint32_t side = 0u; side < (shared ? 1u : 2u); ++side) {
-                float contribution = 0.0f;
-                if ((side == 0u ? kind_a : kind_b) == kSideArtic) {
-                    float a = 0.0f;
-                    if (coordinate) {
-                        a = (side == 0u ? d.chain_jacobian : d.chain_jacobian_b)[size_t{slot} * md + lane];
-                        if (shared) a += d.chain_jacobian_b[size_t{slot} * md + lane];
-                    }
+        // y = L^-1 a, then the ordered sum of y_i^2 / D_i
+        auto response = [&](float a) -> float {
 #pragma unroll
-                    for (int j = 0; j < N; ++j) a -= lrow[j] * lane_value(a, j);
-                    const float term = coordinate ? a * a / pivot : 0.0f;
+            for (int j = 0; j < N; ++j) a -= lrow[j] * lane_value(a, j);
+            const float term = coordinate ? a * a / pivot : 0.0f;
+            float total = 0.0f;
 #pragma unroll
-                    for (int i = 0; i < N; ++i) contribution += lane_value(term, i);
+            for (int i = 0; i < N; ++i) total += lane_value(term, i);
+            return total;
+        };
+        // Four heads at a time: their substitution chains are independent, and side by side each one's lane reads
+        // settle under the others' arithmetic.  A head with one moving side, or with both sides on one owner (:752),
+        // wants exactly the staged sum of its two sides' rows.
+        for (uint32_t h0 = 0u; h0 < heads; h0 += 4u) {
+            float a[4], term[4], total[4];
+            bool second[4], apart[4];
+#pragma unroll
+            for (uint32_t t = 0u; t < 4u; ++t) {
+                const uint32_t h = h0 + t;
+                a[t] = 0.0f; second[t] = false; apart[t] = false;
+                if (h >= heads) continue;
+                const bool artic_a = c.U(hSourceA, h) != kInvalid, artic_b = c.U(hSourceB, h) != kInvalid;
+                if (artic_a && artic_b) {
+                    const float* row = urows + size_t{c.U(hSlot, h)} * kRowWords;
+                    apart[t] = __float_as_uint(row[11]) != __float_as_uint(row[19]);
                 }
-                shares[side] = contribution;
+                second[t] = artic_b && !artic_a;
+                if (coordinate && (artic_a || artic_b) && !apart[t]) a[t] = c.jac[(3u * h) * c.ldj + lane];
             }
-            if (lane == 0u) { c.F(hRes, h) = shares[0]; c.F(hRes + 1, h) = shares[1]; }
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) a[t] -= lrow[j] * lane_value(a[t], j);
+            }
+#pragma unroll
+            for (int t = 0; t < 4; ++t) { term[t] = coordinate ? a[t] * a[t] / pivot : 0.0f; total[t] = 0.0f; }
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) total[t] += lane_value(term[t], i);
+            }
+#pragma unroll
+            for (uint32_t t = 0u; t < 4u; ++t) {
+                const uint32_t h = h0 + t;
+                if (h >= heads) continue;
+                float shares[2] = {second[t] ? 0.0f : total[t], second[t] ? total[t] : 0.0f};
+                if (apart[t]) {   // two owners: one response each
+                    shares[0] = response(coordinate ? d.chain_jacobian[size_t{c.U(hSourceA, h)} * md + lane] : 0.0f);
+                    shares[1] = response(coordinate ? d.chain_jacobian_b[size_t{c.U(hSourceB, h)} * md + lane] : 0.0f);
+                }
+                if (lane == 0u) { c.F(hRes, h) = shares[0]; c.F(hRes + 1, h) = shares[1]; }
+            }
         }
         __syncthreads();
     }
+    PROF_END(c, 18);
+    PROF_BEGIN(c, 19);
     // InitializeTileHead (:743-797), lane = head
     for (uint32_t base = 0u; base < heads; base += kWave) {
         const uint32_t h = base + lane;
@@ -1131,17 +1175,14 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         }
     }
     __syncthreads();
-    // StageTileMass (:2127-2142): the mass rows go to registers through a coalesced pass over LDS (the head setup's
-    // scratch is dead by now); rows and columns n..N-1 are those of the identity.  Then the one factorisation.
-    float mrow[N];
-    for (uint32_t e = lane; e < n * n; e += kWave) c.hfac[(e / n) * c.ld + e % n] = d.m[size_t{env} * md * md + size_t{e / n} * md + e % n];
-    __syncthreads();
-#pragma unroll
-    for (int k = 0; k < N; ++k)
-        mrow[k] = coordinate && uint32_t(k) < n ? c.hfac[lane * c.ld + k] : (lane == uint32_t(k) && lane < uint32_t(N) ? 1.0f : 0.0f);
-    __syncthreads();
+    PROF_END(c, 19);
+    PROF_BEGIN(c, 20);
+    // the one factorisation of the mass matrix
     c.mass_valid = factor_mass<N>(c, mrow);
+    PROF_END(c, 20);
+    PROF_BEGIN(c, 21);
     initialize_residuals<N>(c, velocity, urows, p.dt);
+    PROF_END(c, 21);
     PROF_END(c, 0);
     float residual4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     uint32_t sweeps = 0u;
@@ -1182,7 +1223,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     if (lane == 0u) {
         for (int i = 0; i < 10; ++i) d.solver_penalty[size_t{env} * R + i] = float(c.prof[i]);
         for (int i = 0; i < 4; ++i) d.solver_penalty[size_t{env} * R + 10 + i] = float(c.prof_count[i]);
-        for (int i = 10; i < 16; ++i) d.solver_penalty[size_t{env} * R + 4 + i] = float(c.prof[i]);
+        for (int i = 10; i < 22; ++i) d.solver_penalty[size_t{env} * R + 4 + i] = float(c.prof[i]);
     }
 #endif
     // the block velocities persist for the next solve's carried start
