@@ -79,6 +79,17 @@ typedef struct nuka_template_desc_t {
     const uint32_t* shape_group;
     const uint32_t* shape_profile;   /* friction profile row, ~0u for the default (mu 1) */
     const float* profile_mu;         /* [profile][2] */
+    /* Joint rows and drives (src/scene/cook/cook_to_model.cpp:696-719); read only when struct_size covers them. */
+    const float* joint_limit_lower;  /* [link], nullable */
+    const float* joint_limit_upper;  /* [link], nullable */
+    const uint8_t* joint_limit_flags;/* [link] bit 0: lower bound authored, bit 1: upper; nullable.  Any bit set gives
+                                        every link its two limit row slots */
+    const float* joint_frictionloss; /* [link], nullable; any positive entry gives every link a friction row slot */
+    uint32_t drive_mode;             /* phi/articulation_contract.hpp:16-23: 0 PD position, 1 torque, 2 velocity, 5 actuator */
+    uint32_t drive_rows;             /* 0: the field `tau` is the applied generalized force and no drive rows exist;
+                                        1: the reference's actuation - ApplyDrives turns the drive_* fields into one
+                                        bounded-effort row per link, overwrites `tau` with `joint_f` and ReadoutDrives
+                                        reports the applied effort (src/nk/pipeline/world.cpp:61) */
 } nuka_template_desc_t;
 
 /* nuka.h:57-173 nuka_world_desc_t; zero keeps the default of the same reference field. */
@@ -95,6 +106,9 @@ typedef struct nuka_world_desc_t {
     float solver_velocity_tolerance; /* 0 => 1e-5 (op_schema.hpp:663) */
     float solver_baumgarte_max_velocity;   /* 0 => 3e38 */
     float solver_overlap_recovery_velocity;
+    uint32_t solver_fold_drive_damping;    /* 0 => on (pipeline.hpp:48-49): a drive's velocity feedback is solved
+                                              implicitly through the mass matrix; ~0u => off.  Read only when
+                                              struct_size covers it */
 } nuka_world_desc_t;
 
 /* nuka.h:175 nuka_world_create_from_scene */

@@ -16,6 +16,9 @@ SHAPE_SPHERE, SHAPE_CAPSULE, SHAPE_BOX, SHAPE_PLANE, SHAPE_NONE = 0, 1, 2, 3, IN
 # collidable row roles of the template description
 ROLE_STATIC, ROLE_LINK_BODY, ROLE_PROXY = 0, 1, 2
 
+# phi/articulation_contract.hpp:16-23
+DRIVE_PD_POSITION, DRIVE_TORQUE, DRIVE_VELOCITY, DRIVE_COMPUTED_TORQUE, DRIVE_OSC, DRIVE_ACTUATOR = 0, 1, 2, 3, 4, 5
+
 # nuka.h:22-32
 RESULT_OK, RESULT_INVALID_ARG, RESULT_NULL_HANDLE, RESULT_DEVICE_ERROR = 0, 1, 2, 3
 RESULT_OUT_OF_MEMORY, RESULT_NOT_SUPPORTED, RESULT_INTERNAL = 6, 7, 100
@@ -35,6 +38,8 @@ class TemplateDescC(C.Structure):
         ("body_role", _PU), ("body_link", _PU), ("body_local", _PF), ("shape_kind", _PU), ("shape_params", _PF),
         ("shape_contype", _PU), ("shape_conaffinity", _PU), ("shape_group", _PU), ("shape_profile", _PU),
         ("profile_mu", _PF),
+        ("joint_limit_lower", _PF), ("joint_limit_upper", _PF), ("joint_limit_flags", _PB), ("joint_frictionloss", _PF),
+        ("drive_mode", C.c_uint32), ("drive_rows", C.c_uint32),
     ]
 
 
@@ -44,6 +49,7 @@ class WorldDescC(C.Structure):
         ("solver_vel_iters", C.c_uint32), ("solver_pos_iters", C.c_uint32), ("solver_contact_margin", C.c_float),
         ("solver_pos_beta", C.c_float), ("solver_pos_slop", C.c_float), ("solver_velocity_tolerance", C.c_float),
         ("solver_baumgarte_max_velocity", C.c_float), ("solver_overlap_recovery_velocity", C.c_float),
+        ("solver_fold_drive_damping", C.c_uint32),
     ]
 
 
@@ -63,14 +69,17 @@ class Template:
         self.bodies = []
         self.profiles = []
         self.max_contacts_per_env = 0
+        self.drive_mode = DRIVE_TORQUE
+        self.drive_rows = False   # True: affine drives through joint drive rows; False: `tau` is the applied force
 
     def add_link(self, joint_type, parent, axis=(0, 0, 1), local_pos=(0, 0, 0), local_rot=(1, 0, 0, 0), mass=1.0,
                  diag_inertia=(0.01, 0.01, 0.01), com=(0, 0, 0), damping=0.0, armature=0.0, stiffness=0.0,
-                 spring_ref=0.0, parent_offset=(0, 0, 0)):
+                 spring_ref=0.0, parent_offset=(0, 0, 0), lower=None, upper=None, frictionloss=0.0):
         self.links.append(dict(joint_type=joint_type, parent=INVALID if parent is None else parent, axis=axis,
                                local=list(local_pos) + list(local_rot), mass=mass, diag=diag_inertia,
                                inertial=list(com) + [1, 0, 0, 0], damping=damping, armature=armature,
-                               stiffness=stiffness, spring_ref=spring_ref, parent_offset=parent_offset))
+                               stiffness=stiffness, spring_ref=spring_ref, parent_offset=parent_offset,
+                               lower=lower, upper=upper, frictionloss=frictionloss))
         return len(self.links) - 1
 
     def add_profile(self, mu1, mu2=None):
@@ -109,6 +118,10 @@ class Template:
             joint_armature=np.array([l["armature"] for l in L], dtype=f32),
             joint_stiffness=np.array([l["stiffness"] for l in L], dtype=f32),
             joint_spring_reference=np.array([l["spring_ref"] for l in L], dtype=f32),
+            joint_limit_lower=np.array([0.0 if l["lower"] is None else l["lower"] for l in L], dtype=f32),
+            joint_limit_upper=np.array([0.0 if l["upper"] is None else l["upper"] for l in L], dtype=f32),
+            joint_limit_flags=np.array([(l["lower"] is not None) + 2 * (l["upper"] is not None) for l in L], dtype=np.uint8),
+            joint_frictionloss=np.array([l["frictionloss"] for l in L], dtype=f32),
             body_role=np.array([b["role"] for b in B], dtype=u32),
             body_link=np.array([b["link"] for b in B], dtype=u32),
             body_local=np.array([b["local"] for b in B], dtype=f32).reshape(-1),
@@ -128,6 +141,7 @@ class Template:
         d.struct_size = C.sizeof(TemplateDescC)
         d.link_count, d.body_count, d.profile_count = len(self.links), len(self.bodies), len(self.profiles)
         d.max_contacts_per_env = self.max_contacts_per_env
+        d.drive_mode, d.drive_rows = self.drive_mode, 1 if self.drive_rows else 0
         ctype = {np.dtype(np.float32): C.c_float, np.dtype(np.uint32): C.c_uint32, np.dtype(np.uint8): C.c_uint8}
         for name, arr in a.items():
             arr = np.ascontiguousarray(arr)
@@ -138,7 +152,7 @@ class Template:
 
 
 def world_desc(env_count, dt, gravity=(0.0, 0.0, -9.81), vel_iters=0, pos_iters=0, contact_margin=0.0,
-               velocity_tolerance=0.0):
+               velocity_tolerance=0.0, fold_drive_damping=True):
     d = WorldDescC()
     d.struct_size = C.sizeof(WorldDescC)
     d.env_count, d.fixed_dt = env_count, dt
@@ -146,4 +160,5 @@ def world_desc(env_count, dt, gravity=(0.0, 0.0, -9.81), vel_iters=0, pos_iters=
     d.solver_vel_iters, d.solver_pos_iters = vel_iters, pos_iters
     d.solver_contact_margin = contact_margin
     d.solver_velocity_tolerance = velocity_tolerance
+    d.solver_fold_drive_damping = 0 if fold_drive_damping else INVALID
     return d

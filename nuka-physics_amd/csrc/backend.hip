@@ -18,7 +18,7 @@ const char* OpName(NkOp op) {
         "ApplyDrives", "ArticulationDynamics", "IntegrateVelocity", "FkWorldPoses", "IntegratePosition", "BuildAabbs",
         "LbvhBuild", "LbvhQueryPairs", "NarrowphasePrimitives", "AssembleRows", "SyncLinkBodyPose", "NarrowphaseHeightfield",
         "ContactWarmStart", "SnapshotStepVelocity", "FkLinkVelocities", "BlockDescentSolve", "ResetEnvs", "SnapshotState",
-        "RestoreState", "FusedStep"};
+        "RestoreState", "ReadoutDrives"};
     return op < NkOp::Count ? names[static_cast<uint16_t>(op)] : "?";
 }
 
@@ -46,6 +46,7 @@ void RegisterOps() {
     set(NkOp::SnapshotStepVelocity, &OpSnapshotStepVelocity);
     set(NkOp::FkLinkVelocities, &OpFkLinkVelocities);
     set(NkOp::BlockDescentSolve, &OpBlockDescentSolve);
+    set(NkOp::ReadoutDrives, &OpReadoutDrives);
 }
 
 void Fail(nuka_phi_execution_error* error, Status status, uint16_t op, int native, const char* message) {

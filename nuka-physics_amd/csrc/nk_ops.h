@@ -25,6 +25,7 @@ Status OpNarrowphaseHeightfield(const ModelView&, const DataView&, const void*, 
 Status OpAssembleRows(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpContactWarmStart(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpBlockDescentSolve(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpReadoutDrives(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpSnapshotStepVelocity(const ModelView&, const DataView&, const void*, hipStream_t);
 
 }  // namespace nkh

@@ -15,7 +15,7 @@ enum class NkOp : uint16_t {
     ApplyDrives, ArticulationDynamics, IntegrateVelocity, FkWorldPoses, IntegratePosition, BuildAabbs, LbvhBuild,
     LbvhQueryPairs, NarrowphasePrimitives, AssembleRows, SyncLinkBodyPose, NarrowphaseHeightfield, ContactWarmStart,
     SnapshotStepVelocity, FkLinkVelocities, BlockDescentSolve, ResetEnvs, SnapshotState, RestoreState,
-    FusedStep,   // extension: the whole step in the fused launches (plan path)
+    ReadoutDrives,
     Count
 };
 
@@ -37,13 +37,16 @@ enum : uint32_t { kSideRigid = 0, kSideArtic = 1, kSideStatic = 3 };
 // src/nk/solve/nk_row.hpp:41-57
 enum : uint32_t {
     kRowActive = 1u << 0, kRowFriction = 1u << 1, kRowBlockNormal = 1u << 2, kRowBlockTangent = 1u << 3,
+    kRowJointLimitLower = 1u << 4, kRowJointLimitUpper = 1u << 5,
     kRowContactNormal = 1u << 6, kRowVelocityOnly = 1u << 7, kRowSpeculative = 1u << 8, kRowMuJoCo = 1u << 11
 };
 // src/phi/op_schema.hpp:36-52
 enum : uint32_t {
     kEnvStatusPairOverflow = 1u << 0, kEnvStatusDofOverflow = 1u << 2, kEnvStatusInvalidEndpoint = 1u << 6,
-    kEnvStatusSolverFailure = 1u << 13
+    kEnvStatusControlFailure = 1u << 10, kEnvStatusSolverFailure = 1u << 13
 };
+// src/phi/articulation_contract.hpp:16-23
+enum : uint32_t { kDrivePdPosition = 0, kDriveTorque = 1, kDriveVelocity = 2, kDriveComputedTorque = 3, kDriveOsc = 4, kDriveActuator = 5 };
 constexpr uint32_t kContactLawSpeculative = 2u;   // src/nk/solve/nk_row.hpp:37
 
 // Template tables, stored once and shared by every environment (the reference replicates them per env,
@@ -52,6 +55,8 @@ struct ModelView {
     uint32_t links_per_env, bodies_per_env, dof, max_dof, max_depth, contact_slots, rows_per_env, contact_rows_per_env;
     uint32_t profile_count, floating_root;
     uint32_t max_points_per_slot;   // 1 when no box can meet a plane, else 4 (sizes the solver's staged rows)
+    // joint row slots after the contact rows: 2 per link, 1 per link, 1 per link, or 0 (scene/cook/cook_to_model.cpp:706-719)
+    uint32_t joint_limit_rows, joint_friction_rows, joint_drive_rows, drive_mode;
     const uint8_t* joint_type;
     const uint32_t* parent_link;
     const float* joint_axis;
@@ -63,6 +68,10 @@ struct ModelView {
     const float* joint_armature;
     const float* joint_stiffness;
     const float* joint_spring_reference;
+    const float* joint_limit_lower;
+    const float* joint_limit_upper;
+    const float* joint_frictionloss;
+    const uint8_t* joint_limit_flags;   // bit 0: lower bound authored, bit 1: upper
     const uint32_t* link_body;
     const uint32_t* link_tree_depth;
     const uint32_t* link_child_range;
@@ -102,6 +111,11 @@ struct DataView {
     float *contact_cache_lambda, *contact_cache_normal;
     uint32_t *contact_cache_age, *contact_cache_current_owner, *contact_cache_old_keep, *contact_cache_extent;
     uint32_t *contact_warm_start_counts, *contact_cache_match;
+    // drives (fields.yaml:49-53, 328, 658-668, 548-551, 906)
+    float *drive_target, *drive_stiffness, *drive_damping, *drive_force_limit, *drive_joint_force_limit;
+    float *velocity_target, *actuator_noload_speed, *joint_f, *joint_gravity_force;
+    float *drive_command, *drive_dissipation, *drive_lower, *drive_upper;
+    float *joint_limit_impulse, *actuator_effort_requested, *actuator_effort, *actuator_saturated;
     uint32_t *reset_env_ids;                // staging of nuka_world_reset_envs
     uint32_t *solver_cost, *tile_order;     // last solve's work per environment; launch order of the next solve (costliest first)
     float *snapshot;                        // SnapshotState / RestoreState storage
@@ -110,7 +124,13 @@ struct DataView {
 // --- parameter PODs (field names follow src/phi/op_schema.hpp) -------------------------------------------
 struct FkWorldPosesParams { uint32_t articulation_count, total_link_count; };
 struct FkLinkVelocitiesParams { uint32_t articulation_count, total_link_count; };
-struct ApplyDrivesParams { float dt; uint32_t total_link_count, links_per_env, mode, articulation_count; float gravity[3]; };
+struct ApplyDrivesParams {   // op_schema.hpp:79-88
+    float dt;
+    uint32_t total_link_count, defer_velocity_damping, mode, links_per_env, bodies_per_env, articulation_count;
+    float gravity[3];
+    uint32_t affine;   // this backend's own: 0 leaves `tau` as the applied generalized force (no drive rows cooked)
+};
+struct ReadoutDrivesParams { float dt; uint32_t total_link_count, links_per_env, rows_per_env, first_drive_row; };   // op_schema.hpp:100-106
 struct ArticulationDynamicsParams {   // op_schema.hpp:108-121
     float dt;
     uint32_t max_dof;
@@ -136,6 +156,8 @@ struct AssembleRowsParams {
     uint32_t env_count, articulation_count, total_link_count, max_dof, union_slot_count, rows_per_env, contact_rows_per_env;
     uint32_t full_row_slot_count, bodies_per_env, base_link_count, position_pass, family;
     float dt, overlap_recovery_velocity, contact_margin;
+    uint32_t joint_limit_rows_per_env, joint_friction_rows_per_env, joint_drive_rows_per_env;
+    float baumgarte_max_velocity;
 };
 struct ContactWarmStartParams { uint32_t phase, env_count, slot_count, rows_per_env, full_row_slot_count, decay_steps; };
 struct BlockDescentSolveParams {   // op_schema.hpp:549-636 (the tile-route subset)
@@ -146,15 +168,8 @@ struct BlockDescentSolveParams {   // op_schema.hpp:549-636 (the tile-route subs
     uint32_t position_iterations;
     float position_beta, position_slop, position_max_velocity;
     float velocity_tolerance;
+    uint32_t joint_limit_rows_per_env;
 };
 struct SnapshotParams { uint32_t env_count, selected_env_count; };
-struct FusedStepParams {
-    ArticulationDynamicsParams dynamics;
-    BuildAabbsParams aabbs;
-    NarrowphasePrimitivesParams narrowphase;
-    AssembleRowsParams assemble;
-    BlockDescentSolveParams solve;
-    IntegratePositionParams integrate;
-};
 
 }  // namespace nkh

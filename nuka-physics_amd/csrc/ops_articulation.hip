@@ -289,7 +289,8 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
             const bool scalar = component == kInvalid;
             const float velocity = scalar ? qd[link] : v[6u * link + component];
             float b = scalar ? dot6(S + 6u * link, pf + 6u * link) : pf[6u * link + component];
-            const float damping = scalar ? m.joint_damping[link] : 0.0f;
+            if (scalar) b += d.joint_gravity_force[lbase + link];   // zero unless uploaded
+            const float damping = scalar ? m.joint_damping[link] + (p.fold_drive_damping != 0u ? d.drive_dissipation[lbase + link] : 0.0f) : 0.0f;
             const float spring = scalar ? m.joint_stiffness[link] * (q[link] - m.joint_spring_reference[link]) : 0.0f;
             vel[lane] = velocity;
             bias[lane] = b;
@@ -339,6 +340,7 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
         mat66_vec(ic + 36u * l, sl, force);
         float diagonal = dot6(sl, force);
         diagonal += m.joint_armature[l];
+        if (p.fold_drive_damping != 0u) diagonal += p.dt * d.drive_dissipation[lbase + l];   // articulation_mass.cuh:206-208
         A[dof_i * ld + dof_i] = diagonal;
         uint32_t walk = l;
         for (;;) {
@@ -601,11 +603,123 @@ void InitArticulationKernels() {
     }
 }
 
-// Torque control leaves tau as applied; free bodies do not exist on this path, so both ops only validate.
-Status OpApplyDrives(const ModelView&, const DataView&, const void* params, hipStream_t) {
+// ApplyAffineDriveKernel (articulation.cu:836-940): one thread per link turns the controller fields into an affine
+// effort `command - dissipation * qdot` and its bounds for the drive row, and overwrites tau with the feedforward
+// load.  Gravity compensation (ProjectGravityCompensationKernel :393-423) is not authored on this path:
+// joint_gravity_force stays as uploaded.  The inverse-dynamics modes (ComputedTorque, Osc) are not built.
+__global__ void __launch_bounds__(256) ApplyAffineDriveKernel(ModelView m, DataView d, ApplyDrivesParams p) {
+    const uint32_t link = blockIdx.x * blockDim.x + threadIdx.x;
+    if (link >= p.total_link_count) return;
+    d.drive_command[link] = d.drive_dissipation[link] = 0.0f;
+    d.drive_lower[link] = d.drive_upper[link] = 0.0f;
+    d.tau[link] = 0.0f;
+    const uint32_t local = link % p.links_per_env;
+    if (joint_dof(m.joint_type[local]) != 1u) return;
+    const uint32_t mode = p.mode;
+    const bool implicit = p.defer_velocity_damping != 0u;
+    const bool position_control = mode == kDrivePdPosition, velocity_control = mode == kDriveVelocity;
+    const float kp = d.drive_stiffness[link], kd = d.drive_damping[link];
+    if ((position_control && (!isfinite(d.drive_target[link]) || !isfinite(kp) || kp < 0.0f || !isfinite(kd) || (implicit && kd < 0.0f))) ||
+        ((position_control || velocity_control) && !isfinite(d.velocity_target[link])) ||
+        (velocity_control && (!isfinite(kp) || kp < 0.0f)) ||
+        (mode == kDriveActuator && !isfinite(d.actuator_noload_speed[link]))) {
+        atomicOr(d.env_status + link / p.links_per_env, kEnvStatusControlFailure);
+        return;
+    }
+    const float velocity = d.qdot[link];
+    const float limit = d.drive_force_limit[link];
+    float lower = limit > 0.0f ? -limit : -FLT_MAX;
+    float upper = limit > 0.0f ? limit : FLT_MAX;
+    float bias = 0.0f, damping = 0.0f;
+    if (mode == kDrivePdPosition) {
+        // an implicit spring is evaluated at the end of the step, adding dt kp to the damping
+        damping = kd + (implicit ? p.dt * kp : 0.0f);
+        bias = kp * (d.drive_target[link] - d.q[link]) + damping * d.velocity_target[link];
+    } else if (mode == kDriveVelocity) {
+        damping = kp;
+        bias = damping * d.velocity_target[link];
+    } else {   // torque, actuator
+        bias = d.drive_target[link];
+        if (mode == kDriveActuator && limit > 0.0f && d.actuator_noload_speed[link] > 0.0f) {
+            const float speed_bias = limit * velocity / d.actuator_noload_speed[link];
+            lower = fminf(fmaxf(-limit - speed_bias, -limit), limit);
+            upper = fminf(fmaxf(limit - speed_bias, -limit), limit);
+        }
+    }
+    const float effort = bias - damping * velocity;
+    const float gravity_force = d.joint_gravity_force[link];
+    const bool saturated = effort < lower || effort > upper;
+    const float joint_limit = d.drive_joint_force_limit[link];
+    if (implicit && joint_limit > 0.0f) {
+        bias = fminf(fmaxf(fminf(fmaxf(effort, lower), upper) + gravity_force, -joint_limit), joint_limit);
+        damping = saturated ? 0.0f : damping;
+        bias += damping * velocity;
+        lower = -FLT_MAX;
+        upper = FLT_MAX;
+    } else if (!implicit || saturated) {
+        bias = effort + gravity_force;
+        damping = 0.0f;
+        lower += gravity_force;
+        upper += gravity_force;
+        if (joint_limit > 0.0f) {
+            lower = fminf(fmaxf(lower, -joint_limit), joint_limit);
+            upper = fminf(fmaxf(upper, -joint_limit), joint_limit);
+        }
+    } else {   // the row clamps the command bias = effort + damping * velocity
+        bias += gravity_force;
+        lower += gravity_force + damping * velocity;
+        upper += gravity_force + damping * velocity;
+    }
+    const float feedforward = d.joint_f[link];
+    if (!isfinite(bias) || !isfinite(damping) || damping < 0.0f || !isfinite(limit) || !isfinite(feedforward) || !isfinite(velocity) ||
+        !isfinite(d.q[link])) {
+        atomicOr(d.env_status + link / p.links_per_env, kEnvStatusControlFailure);
+        return;
+    }
+    d.drive_command[link] = bias;
+    d.drive_dissipation[link] = damping;
+    d.drive_lower[link] = lower;
+    d.drive_upper[link] = upper;
+    d.tau[link] = feedforward;
+}
+
+// ReadoutDrivesKernel (articulation.cu:999-1016)
+__global__ void __launch_bounds__(256) ReadoutDrivesKernel(ModelView m, DataView d, ReadoutDrivesParams p) {
+    const uint32_t link = blockIdx.x * blockDim.x + threadIdx.x;
+    if (link >= p.total_link_count) return;
+    d.actuator_effort_requested[link] = d.actuator_effort[link] = d.actuator_saturated[link] = 0.0f;
+    const uint32_t env = link / p.links_per_env, local = link - env * p.links_per_env;
+    if (joint_dof(m.joint_type[local]) != 1u) return;
+    const size_t row = size_t{env} * p.rows_per_env + p.first_drive_row + local;
+    const float effort = d.drive_command[link] - d.drive_dissipation[link] * d.qdot[link];
+    d.actuator_effort_requested[link] = effort;
+    const float applied = d.lambda[row] / p.dt - d.drive_dissipation[link] * d.qdot[link];
+    d.actuator_effort[link] = applied;
+    d.actuator_saturated[link] = d.drive_command[link] < d.drive_lower[link] || d.drive_command[link] > d.drive_upper[link] ? 1.0f : 0.0f;
+    d.tau[link] += applied;
+}
+
+// OpApplyDrives (articulation.cu:1604-1620).  Without drive rows in the cooked world tau is the applied generalized
+// force and the op only validates; free bodies do not exist on this path, so IntegrateVelocity only validates too.
+Status OpApplyDrives(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
     const auto* p = static_cast<const ApplyDrivesParams*>(params);
-    if (p == nullptr || p->mode != 1u) return p == nullptr ? Status::InvalidArgument : Status::Unsupported;
-    return Status::Ok;
+    if (p == nullptr || p->mode > kDriveActuator) return Status::InvalidArgument;
+    if (p->affine == 0u) return p->mode == kDriveTorque ? Status::Ok : Status::Unsupported;
+    if (p->mode == kDriveComputedTorque || p->mode == kDriveOsc) return Status::Unsupported;
+    if (p->total_link_count == 0u) return Status::Ok;
+    if (p->links_per_env == 0u || p->links_per_env != m.links_per_env) return Status::InvalidArgument;
+    hipLaunchKernelGGL(ApplyAffineDriveKernel, dim3((p->total_link_count + 255u) / 256u), dim3(256), 0, stream, m, d, *p);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+// OpReadoutDrives (articulation.cu:1654-1667)
+Status OpReadoutDrives(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const ReadoutDrivesParams*>(params);
+    if (p == nullptr || p->dt <= 0.0f) return Status::InvalidArgument;
+    if (p->total_link_count == 0u) return Status::Ok;
+    if (p->links_per_env == 0u || p->links_per_env != m.links_per_env || p->first_drive_row + p->links_per_env > p->rows_per_env)
+        return Status::InvalidArgument;
+    hipLaunchKernelGGL(ReadoutDrivesKernel, dim3((p->total_link_count + 255u) / 256u), dim3(256), 0, stream, m, d, *p);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 Status OpIntegrateVelocity(const ModelView&, const DataView&, const void* params, hipStream_t) {
     const auto* p = static_cast<const IntegrateVelocityParams*>(params);

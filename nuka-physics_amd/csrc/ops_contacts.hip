@@ -344,11 +344,11 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
     uint32_t* range_first = lds_u;        // S
     uint32_t* range_points = lds_u + S;   // S
     // what the chain Jacobian pass needs of each row, kept here so that it does not read back what this block wrote
-    uint32_t* row_link_a = lds_u + 2u * S;             // R
-    uint32_t* row_link_b = row_link_a + R;              // R
-    uint32_t* row_merge = row_link_b + R;               // R: both sides articulated with the same owner
-    float* row_point = reinterpret_cast<float*>(row_merge + R);   // 3R
-    float* row_dir = row_point + 3u * R;                 // 3R, side A's direction (side B's is its negative)
+    uint32_t* row_link_a = lds_u + 2u * S;             // CR (contact rows only; joint rows need no chain walk)
+    uint32_t* row_link_b = row_link_a + CR;             // CR
+    uint32_t* row_merge = row_link_b + CR;              // CR: both sides articulated with the same owner
+    float* row_point = reinterpret_cast<float*>(row_merge + CR);   // 3 CR
+    float* row_dir = row_point + 3u * CR;                // 3 CR, side A's direction (side B's is its negative)
     Row* rows = reinterpret_cast<Row*>(d.urows) + size_t{env} * R;
     float* lambda = d.lambda + size_t{env} * R;
     float* pen = d.row_penetration + size_t{env} * R;
@@ -379,11 +379,11 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
     extent = wave_max_u(extent);
     // rows below the previous and current extents are cleared (:366-394)
     const uint32_t clear_bound = contact_row_bound(previous_extent, 1u, CR);
-    for (uint32_t local = lane; local < min(clear_bound, R); local += kWave) {
+    for (uint32_t local = lane; local < min(clear_bound, CR); local += kWave) {
         lambda[local] = 0.0f; pen[local] = 0.0f; cj_link[local] = kInvalid; cj_link_b[local] = kInvalid;
         rows[local].flags = 0u;
     }
-    for (uint32_t local = lane; local < R; local += kWave) { row_link_a[local] = kInvalid; row_link_b[local] = kInvalid; row_merge[local] = 0u; }
+    for (uint32_t local = lane; local < CR; local += kWave) { row_link_a[local] = kInvalid; row_link_b[local] = kInvalid; row_merge[local] = 0u; }
     if (lane == 0u) {
         d.contact_row_extent[2u * env] = previous_extent;
         d.contact_row_extent[2u * env + 1u] = extent;
@@ -483,6 +483,63 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
             }
         }
     }
+    // joint rows (EmitJointRowsKernel, assemble_rows.cu:803-1026): stable per-link slots after the contact rows - lower
+    // and upper limit (two a link), dry friction, drive.  Each acts on one coordinate, J = +-e_joint; the rest of
+    // its Jacobian row is never written and stays at the zeros it was allocated with.  Native law only.
+    {
+        const uint32_t limit_rows = p.joint_limit_rows_per_env, friction_rows = p.joint_friction_rows_per_env;
+        const uint32_t joint_slots = limit_rows + friction_rows + p.joint_drive_rows_per_env;
+        const size_t lbase = size_t{env} * nl;
+        for (uint32_t slot = lane; slot < joint_slots; slot += kWave) {
+            const uint32_t rs = CR + slot;
+            Row row{};
+            cj_link[rs] = kInvalid; cj_link_b[rs] = kInvalid; pen[rs] = 0.0f;
+            float jacobian = 0.0f, impulse = 0.0f;
+            uint32_t l;
+            if (slot < limit_rows) {   // EmitJointLimitRow :805-882
+                l = slot / 2u;
+                const uint32_t side = slot & 1u;
+                if (joint_dof(m.joint_type[l]) == 1u && (m.joint_limit_flags[l] & (1u << side)) != 0u && p.dt > 0.0f) {
+                    const float bound = side == 0u ? m.joint_limit_lower[l] : m.joint_limit_upper[l];
+                    const float q = d.q[lbase + l];
+                    const float signed_distance = side == 0u ? q - bound : bound - q;
+                    // with a position pass the row only stops further violation; that pass removes it
+                    const float target_velocity = -(p.position_pass != 0u ? fmaxf(signed_distance, 0.0f) : signed_distance) / p.dt;
+                    row.flags = kRowActive | (side == 0u ? kRowJointLimitLower : kRowJointLimitUpper);
+                    row.rhs = fminf(target_velocity, p.baumgarte_max_velocity) / p.dt;
+                    row.lower = 0.0f; row.upper = FLT_MAX;
+                    jacobian = side == 0u ? 1.0f : -1.0f;
+                    pen[rs] = fmaxf(-signed_distance, 0.0f);
+                    impulse = lambda[rs];   // an active limit row keeps its multiplier
+                }
+            } else if (slot < limit_rows + friction_rows) {   // EmitJointFrictionRows :886-934
+                l = slot - limit_rows;
+                const float friction = m.joint_frictionloss[l];
+                if (joint_dof(m.joint_type[l]) == 1u && friction > 0.0f && p.dt > 0.0f) {
+                    row.flags = kRowActive | kRowVelocityOnly;
+                    row.lower = -friction * p.dt; row.upper = friction * p.dt;
+                    jacobian = 1.0f;
+                }
+            } else {   // EmitJointDriveRows :938-971
+                l = slot - limit_rows - friction_rows;
+                const float effort = fminf(fmaxf(d.drive_command[lbase + l], d.drive_lower[lbase + l]), d.drive_upper[lbase + l]);
+                if (joint_dof(m.joint_type[l]) == 1u && effort != 0.0f) {
+                    row.flags = kRowActive | kRowVelocityOnly;
+                    row.lower = row.upper = effort * p.dt;
+                    jacobian = 1.0f;
+                    impulse = row.lower;   // the row admits one impulse, so the first sweep already descends against it
+                }
+            }
+            if (row.flags != 0u) {
+                row.group_first = env * R + rs; row.group_normal_count = 1u; row.env = env;
+                row.a.kind = kSideArtic; row.a.index = env;
+                ++active_rows;
+            }
+            lambda[rs] = impulse;
+            if (joint_dof(m.joint_type[l]) == 1u) d.chain_jacobian[(size_t{env} * R + rs) * md + m.link_dof[l]] = jacobian;
+            rows[rs] = row;
+        }
+    }
     active_rows = uint32_t(wave_sum(float(active_rows)));
     invalid_endpoint = __any(invalid_endpoint);
     if (lane == 0u) {
@@ -511,7 +568,7 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
             mode = component < 3u ? 3u : 4u;
         }
     }
-    const uint32_t bound = min(contact_row_bound(previous_extent, extent, CR) + (R - CR), R);
+    const uint32_t bound = min(contact_row_bound(previous_extent, extent, CR), CR);
     for (uint32_t r = 0u; r < bound; ++r) {
         const uint32_t links[2] = {row_link_a[r], row_link_b[r]};
         if (links[0] == kInvalid && links[1] == kInvalid) continue;
@@ -593,7 +650,7 @@ Status OpAssembleRows(const ModelView& m, const DataView& d, const void* params,
     if (p == nullptr) return Status::Failed;
     if (p->env_count == 0u || p->rows_per_env == 0u) return Status::Ok;
     if (p->max_dof > kMaxDof) return Status::InvalidArgument;
-    const size_t lds = (size_t{p->union_slot_count} * 2u + size_t{p->rows_per_env} * 9u) * sizeof(uint32_t);
+    const size_t lds = (size_t{p->union_slot_count} * 2u + size_t{p->contact_rows_per_env} * 9u) * sizeof(uint32_t);
     if (lds > 150u * 1024u) return Status::InvalidArgument;
     hipLaunchKernelGGL(AssembleRowsKernel, dim3(p->env_count), dim3(kWave), lds, stream, m, d, *p);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;

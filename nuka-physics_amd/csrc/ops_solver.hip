@@ -6,7 +6,7 @@
 namespace nkh {
 namespace solver {
 #define NKH_DECLARE_WIDTH(N) \
-    extern template __global__ void BlockDescentTileKernel<N>(ModelView, DataView, BlockDescentSolveParams, uint32_t);
+    extern template __global__ void BlockDescentTileKernel<N>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
 NKH_DECLARE_WIDTH(4) NKH_DECLARE_WIDTH(8) NKH_DECLARE_WIDTH(12) NKH_DECLARE_WIDTH(16) NKH_DECLARE_WIDTH(20) NKH_DECLARE_WIDTH(24)
 NKH_DECLARE_WIDTH(28) NKH_DECLARE_WIDTH(32) NKH_DECLARE_WIDTH(36) NKH_DECLARE_WIDTH(40) NKH_DECLARE_WIDTH(44) NKH_DECLARE_WIDTH(48)
 NKH_DECLARE_WIDTH(52) NKH_DECLARE_WIDTH(56) NKH_DECLARE_WIDTH(60) NKH_DECLARE_WIDTH(64)
@@ -14,10 +14,13 @@ NKH_DECLARE_WIDTH(52) NKH_DECLARE_WIDTH(56) NKH_DECLARE_WIDTH(60) NKH_DECLARE_WI
 }  // namespace solver
 
 
+// Heads the solver's LDS holds: the contact heads (each stages three Jacobian rows) plus one unit head per joint row
+// slot.  Returns the contact-head capacity that fits `lds_budget_bytes`, 0 when not even one does.
 uint32_t SolverHeadCapacity(const ModelView& m, uint32_t slots, size_t lds_budget_bytes) {
     const uint32_t want = slots * (m.max_points_per_slot == 0u ? kPointsPerSlot : m.max_points_per_slot);
-    for (uint32_t cap = want; cap >= 1u; --cap)
-        if (size_t{solver::SolverLdsFloats(m.dof, cap)} * sizeof(float) <= lds_budget_bytes) return cap;
+    const uint32_t joint_heads = m.joint_limit_rows + m.joint_friction_rows + m.joint_drive_rows;
+    for (uint32_t staged = want; staged >= 1u; --staged)
+        if (size_t{solver::SolverLdsFloats(m.dof, staged + joint_heads, staged)} * sizeof(float) <= lds_budget_bytes) return staged;
     return 0u;
 }
 
@@ -51,7 +54,7 @@ __global__ void __launch_bounds__(1024) OrderTilesKernel(DataView d, uint32_t en
 }
 
 
-using SolverKernel = void (*)(ModelView, DataView, BlockDescentSolveParams, uint32_t);
+using SolverKernel = void (*)(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
 // One instantiation per padded width.
 const SolverKernel kSolverKernels[16] = {
     BlockDescentTileKernel<4>, BlockDescentTileKernel<8>, BlockDescentTileKernel<12>, BlockDescentTileKernel<16>,
@@ -74,11 +77,13 @@ Status OpBlockDescentSolve(const ModelView& m, const DataView& d, const void* pa
     if (p->articulation_count != p->env_count || m.dof == 0u || m.dof > kMaxDof || p->max_dof != m.max_dof ||
         p->iterations == 0u) return Status::InvalidArgument;
     const size_t budget = 150u * 1024u;
-    const uint32_t cap = SolverHeadCapacity(m, p->contact_slots_per_env == 0u ? 1u : p->contact_slots_per_env, budget);
-    if (cap == 0u) return Status::InvalidArgument;
-    const size_t lds = size_t{solver::SolverLdsFloats(m.dof, cap)} * sizeof(float);
+    const uint32_t staged = SolverHeadCapacity(m, p->contact_slots_per_env == 0u ? 1u : p->contact_slots_per_env, budget);
+    if (staged == 0u) return Status::InvalidArgument;
+    const uint32_t cap = staged + m.joint_limit_rows + m.joint_friction_rows + m.joint_drive_rows;
+    const size_t lds = size_t{solver::SolverLdsFloats(m.dof, cap, staged)} * sizeof(float);
     hipLaunchKernelGGL(OrderTilesKernel, dim3(1), dim3(1024), 0, stream, d, p->env_count);
-    hipLaunchKernelGGL(kSolverKernels[solver::PaddedWidth(m.dof) / 4u - 1u], dim3(p->env_count), dim3(solver::kWave), lds, stream, m, d, *p, cap);
+    hipLaunchKernelGGL(kSolverKernels[solver::PaddedWidth(m.dof) / 4u - 1u], dim3(p->env_count), dim3(solver::kWave), lds, stream, m, d, *p, cap,
+                       staged);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 

@@ -10,8 +10,9 @@
 //
 // Replaces src/phi/backend_cuda/ops/block_descent_tile.cuh (DescendTile :2941-3087 and everything it calls) and
 // the helpers it takes from block_descent.cu (:735-820, 1593-1621, 1726-1753) and nk/solve/augmented_row.hpp.
-// Blocks: one articulation per environment.  Not built: free rigid 6x6 blocks, mimic couplings, elliptic
-// (MuJoCo-law) cones, single-coordinate "unit" rows (only joint rows produce them, and joint rows are not emitted).
+// Blocks: one articulation per environment.  Rows on a single coordinate (joint limit, friction and drive rows) are
+// "unit" rows (:799-833): they stage no Jacobian row and touch one diagonal entry and one force entry.
+// Not built: free rigid 6x6 blocks, mimic couplings, elliptic (MuJoCo-law) cones.
 #pragma once
 
 #include "nk_device_math.h"
@@ -165,6 +166,9 @@ enum HeadField : uint32_t {
     hSlot, hStride, hAxes, hOwned, hRho, hCompliance, hLower, hUpper, hMu1, hMu2, hNormalBound,
     hRes, hDual = hRes + 3, hMove = hDual + 3, hStep = hMove + 3, hBase = hStep + 3, hDualScale = hBase + 3, hResidualScale,
     hRelaxStep, hRelaxWeight = hRelaxStep + 3, hRelaxPoint, hF = hRelaxPoint + 3, hC = hF + 3, hNoise = hC + 6, hContrib = hNoise + 3, hColumnsLow, hColumnsHigh, hSourceA, hSourceB = hSourceA + 3, hSourceEnd = hSourceB + 3,
+    hRow = hSourceEnd,   // first of the head's three staged Jacobian rows; kInvalid for a unit head
+    hUnit,               // the one coordinate a unit head acts on; kInvalid for a staged head
+    hUnitValue,          // its Jacobian entry there
     hFieldCount
 };
 
@@ -173,12 +177,13 @@ struct Tile {
     float tolerance;
     float* mfac;     // N x ld: Cholesky factor of the mass matrix (rows; columns are read transposed)
     float* hfac;     // N x ld: Cholesky factor of the current Newton Hessian
-    float* jac;      // 3 * cap rows x ldj, ldj = N
+    float* jac;      // 3 * staged capacity rows x ldj, ldj = N
     float* fields;   // hFieldCount x cap
     float* vec;      // 4 x 64 scratch vectors, 16-byte aligned
     float mass_inverse;   // 1 / diagonal of the mass factor, lane = row
     mutable uint32_t work;   // Newton steps and line probes of this solve, the next solve's scheduling key
     bool mass_valid;
+    bool units;      // some head is a unit head
     float momentum, residual;
     bool failed;
 #ifdef NKH_SOLVER_PROFILE
@@ -327,7 +332,7 @@ template <int N>
 __device__ __forceinline__ void add_head(const Tile& c, uint32_t h, bool coordinate, const float (&f)[3], const float (&cv)[6],
                                          const float (&noise)[3], uint32_t axes, uint64_t columns, float (&hrow)[N], TileSum& g,
                                          float& scale) {
-    const float* j0r = c.jac + (3u * h) * uint32_t(N);
+    const float* j0r = c.jac + c.U(hRow, h) * uint32_t(N);
     const float j0 = coordinate ? j0r[c.lane] : 0.0f;
     tile_add_product(g, j0, f[0]);
     scale += fabsf(j0) * noise[0];
@@ -435,26 +440,87 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
     TileSum g{-inertial.value, -inertial.error};
     PROF_END(c, 11);
     PROF_BEGIN(c, 12);
-    for (uint64_t rest = __ballot(mine); rest != 0ull; rest &= rest - 1ull) {
-        const uint32_t h = uint32_t(__builtin_ctzll(rest));
-        float f[3], cv[6], noise[3];
+    if (!c.units) {   // staged heads only: plain head order
+        for (uint64_t rest = __ballot(mine); rest != 0ull; rest &= rest - 1ull) {
+            const uint32_t h = uint32_t(__builtin_ctzll(rest));
+            float f[3], cv[6], noise[3];
 #pragma unroll
-        for (int k = 0; k < 3; ++k) { f[k] = uniform_lane_value(mf[k], h); noise[k] = uniform_lane_value(mn[k], h); }
+            for (int k = 0; k < 3; ++k) { f[k] = uniform_lane_value(mf[k], h); noise[k] = uniform_lane_value(mn[k], h); }
 #pragma unroll
-        for (int k = 0; k < 6; ++k) cv[k] = uniform_lane_value(mc[k], h);
-        const uint32_t axes = uint32_t(__builtin_amdgcn_readlane(int(my_axes), int(h)));
-        const uint64_t columns = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_high), int(h)))) << 32u) |
-                                 uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_low), int(h))));
-        add_head<N>(c, h, coordinate, f, cv, noise, axes, columns, hrow, g, scale);
-    }
-    for (uint32_t h = kWave; h < c.heads; ++h) {
-        if (c.U(hContrib, h) == 0u) continue;
-        const float f[3] = {c.F(hF, h), c.F(hF + 1, h), c.F(hF + 2, h)};
-        const float cv[6] = {c.F(hC, h), c.F(hC + 1, h), c.F(hC + 2, h), c.F(hC + 3, h), c.F(hC + 4, h), c.F(hC + 5, h)};
-        const float noise[3] = {c.F(hNoise, h), c.F(hNoise + 1, h), c.F(hNoise + 2, h)};
-        const uint64_t columns = (uint64_t(__builtin_amdgcn_readfirstlane(c.U(hColumnsHigh, h))) << 32u) |
-                                 uint64_t(__builtin_amdgcn_readfirstlane(c.U(hColumnsLow, h)));
-        add_head<N>(c, h, coordinate, f, cv, noise, c.U(hAxes, h), columns, hrow, g, scale);
+            for (int k = 0; k < 6; ++k) cv[k] = uniform_lane_value(mc[k], h);
+            const uint32_t axes = uint32_t(__builtin_amdgcn_readlane(int(my_axes), int(h)));
+            const uint64_t columns = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_high), int(h)))) << 32u) |
+                                     uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_low), int(h))));
+            add_head<N>(c, h, coordinate, f, cv, noise, axes, columns, hrow, g, scale);
+        }
+        for (uint32_t h = kWave; h < c.heads; ++h) {
+            if (c.U(hContrib, h) == 0u) continue;
+            const float f[3] = {c.F(hF, h), c.F(hF + 1, h), c.F(hF + 2, h)};
+            const float cv[6] = {c.F(hC, h), c.F(hC + 1, h), c.F(hC + 2, h), c.F(hC + 3, h), c.F(hC + 4, h), c.F(hC + 5, h)};
+            const float noise[3] = {c.F(hNoise, h), c.F(hNoise + 1, h), c.F(hNoise + 2, h)};
+            const uint64_t columns = (uint64_t(__builtin_amdgcn_readfirstlane(c.U(hColumnsHigh, h))) << 32u) |
+                                     uint64_t(__builtin_amdgcn_readfirstlane(c.U(hColumnsLow, h)));
+            add_head<N>(c, h, coordinate, f, cv, noise, c.U(hAxes, h), columns, hrow, g, scale);
+        }
+    } else {
+        // The heads add in the reference's order (:1533-1603): 32 at a time, and within each 32 the unit heads - a row on
+        // one coordinate adds to that coordinate's diagonal and force only - before the staged ones.
+        float diagonal = 0.0f;
+        const uint32_t my_unit = lane < c.heads ? c.U(hUnit, lane) : kInvalid;
+        const float my_unit_value = lane < c.heads ? c.F(hUnitValue, lane) : 0.0f;
+        const uint64_t contributing = __ballot(mine), unit_heads = __ballot(my_unit != kInvalid);
+        for (uint32_t chunk = 0u; chunk < uint32_t(kWave) && chunk < c.heads; chunk += 32u) {
+            const uint64_t here = contributing & (0xFFFFFFFFull << chunk);
+            for (uint64_t rest = here & unit_heads; rest != 0ull; rest &= rest - 1ull) {
+                const uint32_t h = uint32_t(__builtin_ctzll(rest));
+                const uint32_t target = uint32_t(__builtin_amdgcn_readlane(int(my_unit), int(h)));
+                const float v = uniform_lane_value(my_unit_value, h), fx = uniform_lane_value(mf[0], h);
+                const float cxx = uniform_lane_value(mc[0], h), nx = uniform_lane_value(mn[0], h);
+                if (lane == target) {
+                    diagonal += v * cxx * v;
+                    tile_add_product(g, v, fx);
+                    scale += fabsf(v) * nx;
+                }
+            }
+            for (uint64_t rest = here & ~unit_heads; rest != 0ull; rest &= rest - 1ull) {
+                const uint32_t h = uint32_t(__builtin_ctzll(rest));
+                float f[3], cv[6], noise[3];
+    #pragma unroll
+                for (int k = 0; k < 3; ++k) { f[k] = uniform_lane_value(mf[k], h); noise[k] = uniform_lane_value(mn[k], h); }
+    #pragma unroll
+                for (int k = 0; k < 6; ++k) cv[k] = uniform_lane_value(mc[k], h);
+                const uint32_t axes = uint32_t(__builtin_amdgcn_readlane(int(my_axes), int(h)));
+                const uint64_t columns = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_high), int(h)))) << 32u) |
+                                         uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_low), int(h))));
+                add_head<N>(c, h, coordinate, f, cv, noise, axes, columns, hrow, g, scale);
+            }
+        }
+        for (uint32_t chunk = kWave; chunk < c.heads; chunk += 32u) {
+            const uint32_t end = min(chunk + 32u, c.heads);
+            for (uint32_t h = chunk; h < end; ++h) {
+                const uint32_t target = c.U(hUnit, h);
+                if (c.U(hContrib, h) == 0u || target == kInvalid) continue;
+                const float v = c.F(hUnitValue, h);
+                if (lane == target) {
+                    diagonal += v * c.F(hC, h) * v;
+                    tile_add_product(g, v, c.F(hF, h));
+                    scale += fabsf(v) * c.F(hNoise, h);
+                }
+            }
+            for (uint32_t h = chunk; h < end; ++h) {
+                if (c.U(hContrib, h) == 0u || c.U(hUnit, h) != kInvalid) continue;
+                const float f[3] = {c.F(hF, h), c.F(hF + 1, h), c.F(hF + 2, h)};
+                const float cv[6] = {c.F(hC, h), c.F(hC + 1, h), c.F(hC + 2, h), c.F(hC + 3, h), c.F(hC + 4, h), c.F(hC + 5, h)};
+                const float noise[3] = {c.F(hNoise, h), c.F(hNoise + 1, h), c.F(hNoise + 2, h)};
+                const uint64_t columns = (uint64_t(__builtin_amdgcn_readfirstlane(c.U(hColumnsHigh, h))) << 32u) |
+                                         uint64_t(__builtin_amdgcn_readfirstlane(c.U(hColumnsLow, h)));
+                add_head<N>(c, h, coordinate, f, cv, noise, c.U(hAxes, h), columns, hrow, g, scale);
+            }
+        }
+        if (c.units) {   // the unit heads' curvature lands on the diagonal after every staged head (:1605-1606)
+    #pragma unroll
+            for (int k = 0; k < N; ++k) hrow[k] += local_lane(lane) == uint32_t(k) ? diagonal : 0.0f;
+        }
     }
     PROF_END(c, 12);
     PROF_BEGIN(c, 13);
@@ -533,7 +599,12 @@ __device__ __forceinline__ void row_steps(const Tile& c, float d) {
     __syncthreads();
     for (uint32_t h = c.lane; h < c.heads; h += kWave) {
         if (c.U(hOwned, h) == 0u) continue;
-        const float* j = c.jac + (3u * h) * uint32_t(N);
+        const uint32_t unit = c.U(hUnit, h);
+        if (unit != kInvalid) {   // :2028-2032
+            c.F(hStep, h) = c.F(hUnitValue, h) * dvec[unit]; c.F(hStep + 1, h) = 0.0f; c.F(hStep + 2, h) = 0.0f;
+            continue;
+        }
+        const float* j = c.jac + c.U(hRow, h) * uint32_t(N);
         const uint32_t axes = c.U(hAxes, h);
         c.F(hStep, h) = row_dot_fma<N>(j, dvec);
         c.F(hStep + 1, h) = axes > 1u ? row_dot_fma<N>(j + N, dvec) : 0.0f;
@@ -760,7 +831,12 @@ __device__ __forceinline__ void measure_primal(Tile& c, const float (&mrow)[N], 
                     iz = axes == 3u ? lambda_env[local + 2u * stride] : 0.0f;
         if (!(ix != 0.0f || iy != 0.0f || iz != 0.0f)) continue;
         if (!coordinate) continue;
-        const float* j = c.jac + (3u * h) * c.ldj;
+        const uint32_t unit = c.U(hUnit, h);
+        if (unit != kInvalid) {   // :2428
+            if (lane == unit) balance += double(c.F(hUnitValue, h)) * ix;
+            continue;
+        }
+        const float* j = c.jac + c.U(hRow, h) * c.ldj;
         balance += double(j[lane]) * ix;
         if (axes == 3u) {
             balance += double(j[c.ldj + lane]) * iy;
@@ -797,11 +873,18 @@ __device__ __forceinline__ void initialize_residuals(const Tile& c, float veloci
     const float4* d4 = reinterpret_cast<const float4*>(dvec);
     for (uint32_t h = c.lane; h < c.heads; h += kWave) {
         const uint32_t slot = c.U(hSlot, h), stride = c.U(hStride, h), axes = c.U(hAxes, h);
+        const uint32_t unit = c.U(hUnit, h), first = c.U(hRow, h);
+        if (unit != kInvalid || first == kInvalid) {   // one coordinate (or none): every other product is an exact zero
+            const float along = unit != kInvalid ? c.F(hUnitValue, h) * dvec[unit] : 0.0f;
+            c.F(hRes, h) = urows[size_t{slot} * kRowWords + 4u] * dt - (0.0f + along);
+            c.F(hRes + 1, h) = 0.0f; c.F(hRes + 2, h) = 0.0f;
+            continue;
+        }
         for (uint32_t axis = 0u; axis < 3u; ++axis) {
             float residual = 0.0f;
             if (axis < axes) {
                 const float rhs = urows[size_t{slot + axis * stride} * kRowWords + 4u];
-                const float4* j4 = reinterpret_cast<const float4*>(c.jac + (3u * h + axis) * uint32_t(N));
+                const float4* j4 = reinterpret_cast<const float4*>(c.jac + (first + axis) * uint32_t(N));
                 float along = 0.0f;
 #pragma unroll
                 for (int q = 0; q < N / 4; ++q) {
@@ -946,22 +1029,23 @@ __host__ __device__ inline uint32_t FactorRegionFloats(uint32_t n) {
     const uint32_t N = PaddedWidth(n);
     return 2u * N * (N + 1u);   // a multiple of 4 since N is
 }
-__host__ __device__ inline uint32_t SolverLdsFloats(uint32_t n, uint32_t cap) {
+// `cap` heads carry fields; `staged` of them (the contact heads) carry three Jacobian rows each.
+__host__ __device__ inline uint32_t SolverLdsFloats(uint32_t n, uint32_t cap, uint32_t staged) {
     const uint32_t N = PaddedWidth(n);
-    return FactorRegionFloats(n) + 3u * cap * N + ((hFieldCount * cap + 3u) & ~3u) + 256u;
+    return FactorRegionFloats(n) + 3u * staged * N + ((hFieldCount * cap + 3u) & ~3u) + 256u;
 }
 
 // DescendTile (:2941-3087)
 template <int N>
 __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(N <= kTwoWaveWidth ? 2 : 1, N <= kTwoWaveWidth ? 2 : 1)))
-BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint32_t cap) {
+BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint32_t cap, uint32_t staged_cap) {
     extern __shared__ __align__(16) float lds[];
     const uint32_t env = d.tile_order[blockIdx.x], lane = threadIdx.x;
     const uint32_t R = p.rows_per_env, md = p.max_dof, n = m.dof, nl = m.links_per_env, S = p.contact_slots_per_env;
     Tile c;
     c.env = env; c.lane = lane; c.n = n; c.ld = uint32_t(N) + 1u; c.ldj = uint32_t(N); c.cap = cap; c.heads = 0u; c.iteration = 0u;
     c.tolerance = p.velocity_tolerance; c.failed = false; c.momentum = 0.0f; c.residual = 0.0f;
-    c.mass_inverse = 0.0f; c.mass_valid = false; c.work = 0u;
+    c.mass_inverse = 0.0f; c.mass_valid = false; c.work = 0u; c.units = false;
 #ifdef NKH_SOLVER_PROFILE
     for (int i = 0; i < 22; ++i) c.prof[i] = 0;
     for (int i = 0; i < 4; ++i) c.prof_count[i] = 0u;
@@ -971,7 +1055,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     c.mfac = lds;
     c.hfac = c.mfac + uint32_t(N) * c.ld;
     c.jac = lds + FactorRegionFloats(n);
-    c.fields = c.jac + 3u * cap * c.ldj;
+    c.fields = c.jac + 3u * staged_cap * c.ldj;
     c.vec = c.fields + ((hFieldCount * cap + 3u) & ~3u);
     const bool coordinate = lane < n;
     const float* urows = d.urows;
@@ -1035,8 +1119,58 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         c.U(hSourceA + axis, h) = source_a; c.U(hSourceB + axis, h) = source_b;
     }
     __syncthreads();
+    // FindTileRowSupport (:801-833), lane = head: a single-axis head whose Jacobian row has at most one entry is a unit
+    // head and stages nothing; every other owned head stages three rows, placed in head order (PlaceTileRows).
+    {
+        uint32_t staged = 0u;
+        bool overflow_rows = false, any_unit = false;
+        for (uint32_t base = 0u; base < heads; base += kWave) {
+            const uint32_t h = base + lane;
+            bool stage = false;
+            uint32_t unit = kInvalid;
+            float unit_value = 0.0f;
+            if (h < heads) {
+                const uint32_t source_a = c.U(hSourceA, h), source_b = c.U(hSourceB, h);
+                const bool owned = source_a != kInvalid || source_b != kInvalid;
+                const bool single_axis = (__float_as_uint(urows[size_t{c.U(hSlot, h)} * kRowWords]) & kRowBlockNormal) == 0u;
+                if (owned && single_axis) {
+                    uint32_t supported = 0u, last = 0u;
+                    float last_value = 0.0f;
+                    for (uint32_t i = 0u; i < n; ++i) {
+                        float value = 0.0f;
+                        if (source_a != kInvalid) value += d.chain_jacobian[size_t{source_a} * md + i];
+                        if (source_b != kInvalid) value += d.chain_jacobian_b[size_t{source_b} * md + i];
+                        if (value != 0.0f) { ++supported; last = i; last_value = value; }
+                    }
+                    if (supported <= 1u) { unit = last; unit_value = last_value; }
+                }
+                stage = owned && unit == kInvalid;
+            }
+            const uint64_t mask = __ballot(stage);
+            if (h < heads) {
+                uint32_t row = kInvalid;
+                if (stage) {
+                    const uint32_t at = staged + uint32_t(__popcll(mask & ((uint64_t{1} << lane) - 1ull)));
+                    if (at < staged_cap) row = 3u * at;
+                    else { overflow_rows = true; unit = 0u; unit_value = 0.0f; }   // no room: the head acts on nothing, and the solve is flagged
+                }
+                c.U(hRow, h) = row; c.U(hUnit, h) = unit; c.F(hUnitValue, h) = unit_value;
+            }
+            staged += uint32_t(__popcll(mask));
+            any_unit = any_unit || unit != kInvalid;
+        }
+        c.units = __any(any_unit);
+        if (__any(overflow_rows) && lane == 0u) d.env_status[env] |= kEnvStatusSolverFailure;
+    }
+    __syncthreads();
+    // CopyTileRows (:836-869): the staged heads' rows, their loads in flight together
 #pragma unroll 2
     for (uint32_t h = 0u; h < heads; ++h) {
+        const uint32_t first = c.U(hRow, h);
+        if (first == kInvalid) {
+            if (lane == 0u) { c.U(hColumnsLow, h) = 0u; c.U(hColumnsHigh, h) = 0u; }
+            continue;
+        }
         float value[3];
 #pragma unroll
         for (uint32_t axis = 0u; axis < 3u; ++axis) {
@@ -1047,7 +1181,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         }
 #pragma unroll
         for (uint32_t axis = 0u; axis < 3u; ++axis)
-            if (lane < c.ldj) c.jac[(3u * h + axis) * c.ldj + lane] = value[axis];   // padded columns hold zeros
+            if (lane < c.ldj) c.jac[(first + axis) * c.ldj + lane] = value[axis];   // padded columns hold zeros
         // the columns this head touches at all: a contact on one limb leaves most coordinates out, and the Hessian
         // update skips their exact-zero products four columns at a time
         const uint64_t columns = __ballot(value[0] != 0.0f || value[1] != 0.0f || value[2] != 0.0f);
@@ -1105,7 +1239,10 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
                     apart[t] = __float_as_uint(row[11]) != __float_as_uint(row[19]);
                 }
                 second[t] = artic_b && !artic_a;
-                if (coordinate && (artic_a || artic_b) && !apart[t]) a[t] = c.jac[(3u * h) * c.ldj + lane];
+                if (coordinate && (artic_a || artic_b) && !apart[t]) {
+                    const uint32_t first = c.U(hRow, h);
+                    a[t] = first != kInvalid ? c.jac[first * c.ldj + lane] : (lane == c.U(hUnit, h) ? c.F(hUnitValue, h) : 0.0f);
+                }
             }
 #pragma unroll
             for (int j = 0; j < N; ++j) {
@@ -1240,6 +1377,14 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
             else d.link_velocity[(lbase + my_link) * 6u + my_component] = velocity;
         }
     } else if (lane == 0u) d.env_status[env] |= kEnvStatusSolverFailure;
+    // joint limit impulses (:2658-2668)
+    if (p.base_link_count != 0u && p.joint_limit_rows_per_env >= 2u * p.base_link_count) {
+        for (uint32_t l = lane; l < nl; l += kWave) {
+            const size_t lower = size_t{env} * R + p.contact_rows_per_env + size_t{l} * 2u;
+            d.joint_limit_impulse[2u * (lbase + l)] = (__float_as_uint(urows[lower * kRowWords]) & kRowActive) != 0u ? d.lambda[lower] : 0.0f;
+            d.joint_limit_impulse[2u * (lbase + l) + 1u] = (__float_as_uint(urows[(lower + 1u) * kRowWords]) & kRowActive) != 0u ? d.lambda[lower + 1u] : 0.0f;
+        }
+    }
     // split-impulse position pass (:3059-3077; MarkTilePositions :2673-2708; PositionRowBias block_descent.cu:1734-1753)
     if (p.position_iterations != 0u) {
         float* qvec = c.vec + 128;

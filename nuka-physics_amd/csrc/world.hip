@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <cstddef>
 #include <cstdio>
 #include <cstring>
 #include <exception>
@@ -56,12 +57,12 @@ uint32_t JointWidth(uint8_t type) { return type <= kPrismatic ? 1u : type == kFl
 
 struct HostModel {
     ModelView counts{};   // scalar members only
-    std::vector<uint8_t> joint_type;
+    std::vector<uint8_t> joint_type, joint_limit_flags;
     std::vector<uint32_t> parent_link, link_body, link_tree_depth, link_child_range, link_children, link_dof, dof_link, dof_component,
         link_geom_kind, body_to_link, body_to_articulation, body_collidable_link, body_collidable_body;
     std::vector<uint64_t> link_dof_mask;
     std::vector<float> joint_axis, parent_offset, link_local_pose, link_inertial_frame, link_inertia, joint_damping, joint_armature,
-        joint_stiffness, joint_spring_reference, link_geom_local, shape_table, body_collidable_local, body_init_pose, profile_mu;
+        joint_stiffness, joint_spring_reference, joint_limit_lower, joint_limit_upper, joint_frictionloss, link_geom_local, shape_table, body_collidable_local, body_init_pose, profile_mu;
 };
 
 struct NotSupported : std::runtime_error { using std::runtime_error::runtime_error; };
@@ -90,6 +91,10 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
     m.joint_armature = CopyOrZero(d.joint_armature, nl);
     m.joint_stiffness = CopyOrZero(d.joint_stiffness, nl);
     m.joint_spring_reference = CopyOrZero(d.joint_spring_reference, nl);
+    m.joint_limit_lower = CopyOrZero(d.joint_limit_lower, nl);
+    m.joint_limit_upper = CopyOrZero(d.joint_limit_upper, nl);
+    m.joint_frictionloss = CopyOrZero(d.joint_frictionloss, nl);
+    m.joint_limit_flags = d.joint_limit_flags != nullptr ? std::vector<uint8_t>(d.joint_limit_flags, d.joint_limit_flags + nl) : std::vector<uint8_t>(nl, 0u);
     m.link_inertia.resize(36u * nl);
     m.link_dof.resize(nl);
     m.link_body.assign(nl, kInvalid);
@@ -196,7 +201,24 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
     c.links_per_env = nl; c.bodies_per_env = nb; c.dof = nv; c.max_dof = nv; c.max_depth = max_depth;
     c.contact_slots = slots;
     c.contact_rows_per_env = slots * kPointsPerSlot * kRowsPerPoint;   // nk_row.hpp:59-63
-    c.rows_per_env = c.contact_rows_per_env;
+    // joint row slots (scene/cook/cook_to_model.cpp:696-719; nk/pipeline/world.cpp:61, 96)
+    bool any_limit = false, any_friction = false;
+    for (uint32_t l = 0u; l < nl; ++l) {
+        const uint8_t flags = m.joint_limit_flags[l];
+        if (((flags & 1u) != 0u && !std::isfinite(m.joint_limit_lower[l])) || ((flags & 2u) != 0u && !std::isfinite(m.joint_limit_upper[l])) ||
+            ((flags & 3u) == 3u && m.joint_limit_lower[l] > m.joint_limit_upper[l])) throw std::invalid_argument("invalid authored joint limit");
+        if (!std::isfinite(m.joint_frictionloss[l]) || m.joint_frictionloss[l] < 0.0f) throw std::invalid_argument("invalid joint frictionloss");
+        any_limit = any_limit || flags != 0u;
+        any_friction = any_friction || m.joint_frictionloss[l] > 0.0f;
+    }
+    if (d.drive_rows != 0u && (d.drive_mode == kDriveComputedTorque || d.drive_mode == kDriveOsc))
+        throw NotSupported("inverse-dynamics drive modes are not built on this path");
+    if (d.drive_rows != 0u && d.drive_mode > kDriveActuator) throw std::invalid_argument("unknown drive mode");
+    c.joint_limit_rows = any_limit ? nl * 2u : 0u;
+    c.joint_friction_rows = any_friction ? nl : 0u;
+    c.joint_drive_rows = d.drive_rows != 0u ? nl : 0u;
+    c.drive_mode = d.drive_rows != 0u ? d.drive_mode : uint32_t(kDriveTorque);
+    c.rows_per_env = c.contact_rows_per_env + c.joint_limit_rows + c.joint_friction_rows + c.joint_drive_rows;
     c.profile_count = d.profile_count;
     c.floating_root = m.joint_type[0] == kFloatingBase ? 1u : 0u;
     c.max_points_per_slot = any_box ? 4u : 1u;
@@ -225,12 +247,18 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(contact_cache_material, kU64, E * S * 4) X(contact_cache_lambda, kF32, E * S * 16) X(contact_cache_normal, kF32, E * S * 12) \
     X(contact_cache_age, kU32, E * S * 4) X(contact_cache_current_owner, kU32, E * S * 4) X(contact_cache_old_keep, kU32, E * S * 4) \
     X(contact_cache_extent, kU32, E * 2) X(contact_warm_start_counts, kU32, E * 2) X(contact_cache_match, kU32, E * S * 4) \
-    X(reset_env_ids, kU32, E)
+    X(reset_env_ids, kU32, E) \
+    X(drive_target, kF32, E * nl) X(drive_stiffness, kF32, E * nl) X(drive_damping, kF32, E * nl) X(drive_force_limit, kF32, E * nl) \
+    X(drive_joint_force_limit, kF32, E * nl) X(velocity_target, kF32, E * nl) X(actuator_noload_speed, kF32, E * nl) \
+    X(joint_f, kF32, E * nl) X(joint_gravity_force, kF32, E * nl) X(drive_command, kF32, E * nl) X(drive_dissipation, kF32, E * nl) \
+    X(drive_lower, kF32, E * nl) X(drive_upper, kF32, E * nl) X(joint_limit_impulse, kF32, E * nl * 2) \
+    X(actuator_effort_requested, kF32, E * nl) X(actuator_effort, kF32, E * nl) X(actuator_saturated, kF32, E * nl)
 
 #define NKH_MODEL_FIELDS(X) \
     X(joint_type, kU8) X(parent_link, kU32) X(joint_axis, kF32) X(parent_offset, kF32) X(link_local_pose, kF32) \
     X(link_inertial_frame, kF32) X(link_inertia, kF32) X(joint_damping, kF32) X(joint_armature, kF32) X(joint_stiffness, kF32) \
-    X(joint_spring_reference, kF32) X(link_body, kU32) X(link_tree_depth, kU32) X(link_child_range, kU32) X(link_children, kU32) \
+    X(joint_spring_reference, kF32) X(joint_limit_lower, kF32) X(joint_limit_upper, kF32) X(joint_frictionloss, kF32) \
+    X(joint_limit_flags, kU8) X(link_body, kU32) X(link_tree_depth, kU32) X(link_child_range, kU32) X(link_children, kU32) \
     X(link_dof, kU32) X(dof_link, kU32) X(dof_component, kU32) X(link_dof_mask, kU64) X(link_geom_kind, kU32) \
     X(link_geom_local, kF32) X(shape_table, kF32) X(body_to_link, kU32) X(body_to_articulation, kU32) \
     X(body_collidable_link, kU32) X(body_collidable_body, kU32) X(body_collidable_local, kF32) X(profile_mu, kF32)
@@ -260,6 +288,7 @@ struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
     FkWorldPosesParams p_fk{};
     FkLinkVelocitiesParams p_fk_velocity{};
     ApplyDrivesParams p_drives{};
+    ReadoutDrivesParams p_readout_drives{};
     ArticulationDynamicsParams p_dynamics{}, p_dynamics_probe{};
     IntegrateVelocityParams p_int_vel{};
     IntegratePositionParams p_int_pos{};
@@ -359,11 +388,16 @@ void BuildPipeline(World& w) {
     w.p_fk_velocity = {E, E * nl};
     w.p_drives = {};
     w.p_drives.dt = cfg.fixed_dt; w.p_drives.total_link_count = E * nl; w.p_drives.links_per_env = nl;
-    w.p_drives.mode = 1u; w.p_drives.articulation_count = E;
+    w.p_drives.mode = m.drive_mode; w.p_drives.articulation_count = E; w.p_drives.bodies_per_env = nb;
+    const bool drives = m.joint_drive_rows > 0u;
+    const bool fold = drives && cfg.solver_fold_drive_damping != 0xFFFFFFFFu;   // pipeline.cpp:380-381
+    w.p_drives.affine = drives ? 1u : 0u;
+    w.p_drives.defer_velocity_damping = fold ? 1u : 0u;
     std::memcpy(w.p_drives.gravity, cfg.gravity, sizeof(cfg.gravity));
+    w.p_readout_drives = {cfg.fixed_dt, E * nl, nl, m.rows_per_env, m.contact_rows_per_env + m.joint_limit_rows + m.joint_friction_rows};
     ArticulationDynamicsParams& dyn = w.p_dynamics;   // pipeline.cpp:388-402
     dyn = {};
-    dyn.dt = cfg.fixed_dt; dyn.max_dof = m.max_dof; dyn.integrate_velocity = 1u; dyn.fold_drive_damping = 0u; dyn.reuse_mass = 0u;
+    dyn.dt = cfg.fixed_dt; dyn.max_dof = m.max_dof; dyn.integrate_velocity = 1u; dyn.fold_drive_damping = fold ? 1u : 0u; dyn.reuse_mass = 0u;
     std::memcpy(dyn.gravity, cfg.gravity, sizeof(cfg.gravity));
     dyn.articulation_count = E; dyn.total_link_count = E * nl; dyn.apply_link_wrench = 1u; dyn.max_links = nl;
     dyn.links_per_env = nl; dyn.bodies_per_env = nb;
@@ -385,6 +419,8 @@ void BuildPipeline(World& w) {
     as.full_row_slot_count = m.contact_slots; as.bodies_per_env = nb; as.base_link_count = nl;
     as.position_pass = cfg.solver_pos_iters > 0u ? 1u : 0u;
     as.dt = cfg.fixed_dt; as.overlap_recovery_velocity = cfg.solver_overlap_recovery_velocity; as.contact_margin = contact_margin;
+    as.joint_limit_rows_per_env = m.joint_limit_rows; as.joint_friction_rows_per_env = m.joint_friction_rows;
+    as.joint_drive_rows_per_env = m.joint_drive_rows; as.baumgarte_max_velocity = cfg.solver_baumgarte_max_velocity;
     w.p_warm0 = {0u, E, m.contact_slots, m.rows_per_env, m.contact_slots, 2u};
     w.p_warm1 = w.p_warm0;
     w.p_warm1.phase = 1u;
@@ -396,6 +432,7 @@ void BuildPipeline(World& w) {
     bd.position_iterations = has_contacts ? cfg.solver_pos_iters : 0u;
     bd.position_beta = cfg.solver_pos_beta; bd.position_slop = cfg.solver_pos_slop;
     bd.position_max_velocity = cfg.solver_baumgarte_max_velocity; bd.velocity_tolerance = cfg.solver_velocity_tolerance;
+    bd.joint_limit_rows_per_env = m.joint_limit_rows;
 
     // op order of one interval (pipeline.cpp:374, 428-430, 442, 605-639, 699, 746, 908-923, 967, 981-986)
     w.calls.clear();
@@ -408,18 +445,21 @@ void BuildPipeline(World& w) {
     add(NkOp::ApplyDrives, &w.p_drives);
     add(NkOp::ArticulationDynamics, &w.p_dynamics);
     add(NkOp::IntegrateVelocity, &w.p_int_vel);
-    if (has_contacts) {
-        add(NkOp::SyncLinkBodyPose, &w.p_sync);
-        add(NkOp::BuildAabbs, &w.p_aabbs);
-        add(NkOp::LbvhBuild, &w.p_lbvh);
-        add(NkOp::LbvhQueryPairs, &w.p_query);
-        add(NkOp::NarrowphasePrimitives, &w.p_narrow);
-        add(NkOp::NarrowphaseHeightfield, &w.p_narrow);
+    if (has_contacts) {   // rows of any kind: contact slots, joint limits, joint friction, drives (pipeline.cpp:207)
+        if (m.contact_slots > 0u) {
+            add(NkOp::SyncLinkBodyPose, &w.p_sync);
+            add(NkOp::BuildAabbs, &w.p_aabbs);
+            add(NkOp::LbvhBuild, &w.p_lbvh);
+            add(NkOp::LbvhQueryPairs, &w.p_query);
+            add(NkOp::NarrowphasePrimitives, &w.p_narrow);
+            add(NkOp::NarrowphaseHeightfield, &w.p_narrow);
+        }
         add(NkOp::AssembleRows, &w.p_assemble);
-        add(NkOp::ContactWarmStart, &w.p_warm0);
+        if (m.contact_slots > 0u) add(NkOp::ContactWarmStart, &w.p_warm0);
         add(NkOp::BlockDescentSolve, &w.p_solve);
-        add(NkOp::ContactWarmStart, &w.p_warm1);
+        if (m.contact_slots > 0u) add(NkOp::ContactWarmStart, &w.p_warm1);
     }
+    if (drives) add(NkOp::ReadoutDrives, &w.p_readout_drives);   // pipeline.cpp:929-937
     add(NkOp::IntegratePosition, &w.p_int_pos);
     add(NkOp::FkWorldPoses, &w.p_fk);
     add(NkOp::FkLinkVelocities, &w.p_fk_velocity);
@@ -550,8 +590,18 @@ nuka_result_t nuka_world_create_from_template(nuka_device_handle device, const n
     *out = nullptr;
     if (device == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "device is null");
     if (tmpl == nullptr || desc == nullptr || desc->env_count == 0u) return Error(NUKA_RESULT_INVALID_ARG, "template, desc and env_count are required");
-    if (tmpl->struct_size != sizeof(nuka_template_desc_t) || desc->struct_size != sizeof(nuka_world_desc_t))
+    // a caller built against the header before the joint-row members passes the shorter size; those members read as zero
+    constexpr size_t kTemplateBase = offsetof(nuka_template_desc_t, joint_limit_lower);
+    constexpr size_t kWorldBase = offsetof(nuka_world_desc_t, solver_fold_drive_damping);
+    if ((tmpl->struct_size != sizeof(nuka_template_desc_t) && tmpl->struct_size != kTemplateBase) ||
+        (desc->struct_size != sizeof(nuka_world_desc_t) && desc->struct_size != kWorldBase))
         return Error(NUKA_RESULT_INVALID_ARG, "struct_size mismatch");
+    nuka_template_desc_t template_copy{};
+    std::memcpy(&template_copy, tmpl, tmpl->struct_size);
+    nuka_world_desc_t desc_copy{};
+    std::memcpy(&desc_copy, desc, desc->struct_size);
+    tmpl = &template_copy;
+    desc = &desc_copy;
     try {
         auto world = std::make_unique<World>();
         World& w = *world;
@@ -573,7 +623,7 @@ nuka_result_t nuka_world_create_from_template(nuka_device_handle device, const n
         const ModelView& hc = w.host.counts;
         const size_t E = w.env_count, nl = hc.links_per_env, nb = hc.bodies_per_env, md = hc.max_dof, S = hc.contact_slots, R = hc.rows_per_env;
         if (E * std::max<size_t>(R, 1u) > 0xFFFFFFFFull / 2u || E * nl * 7u > 0xFFFFFFFFull) throw std::invalid_argument("world too large for 32-bit row indices");
-        if (hc.rows_per_env > 0u && SolverHeadCapacity(hc, hc.contact_slots, 150u * 1024u) == 0u) throw std::invalid_argument("solver tile does not fit LDS");
+        if (hc.rows_per_env > 0u && SolverHeadCapacity(hc, std::max(hc.contact_slots, 1u), 150u * 1024u) == 0u) throw std::invalid_argument("solver tile does not fit LDS");
         // arena layout: template tables first, then the env-major fields, each on a 256-byte boundary (buffer.hpp:39)
         size_t cursor = 0u;
 #define X(name, dtype) Place<int>(w.fields, #name, dtype, w.host.name.size(), &cursor, true);

@@ -446,6 +446,75 @@ static void chain_jacobian_row(const nko_world* w, uint32_t env, uint32_t link_g
 }
 
 /* ---- AssembleRows (assemble_rows.cu:325-394 ranges/clear, 406-801 emit, 1587-1605 chain J) ---- */
+/* EmitJointRowsKernel (assemble_rows.cu:803-1026): stable per-link slots after the contact rows - lower and upper
+ * limit (2 per link), dry friction (1 per link), drive (1 per link).  Every row acts on one coordinate: J = +-e_joint
+ * over a zeroed Jacobian row.  Only the native (non-MuJoCo) law is built. */
+void nko_env_joint_rows(nko_world* w, uint32_t env) {
+    const nko_template* t = &w->t;
+    const uint32_t R = t->rows_per_env, CR = t->contact_rows_per_env, nl = t->nl, md = t->max_dof;
+    const uint32_t limit_rows = t->joint_limit_rows, friction_rows = t->joint_friction_rows, drive_rows = t->joint_drive_rows;
+    if (limit_rows + friction_rows + drive_rows == 0u) return;
+    const float dt = w->cfg.fixed_dt;
+    const int position_pass = w->cfg.solver_pos_iters > 0u;
+    nko_row* rows = (nko_row*)w->urows;
+    const size_t lbase = (size_t)env * nl;
+    for (uint32_t slot = 0u; slot < limit_rows + friction_rows + drive_rows; ++slot) {
+        const size_t rs = (size_t)env * R + CR + slot;
+        float* J = w->chain_jacobian + rs * md;
+        for (uint32_t k = 0u; k < md; ++k) J[k] = 0.0f;   /* :1000-1004 */
+        nko_row row; memset(&row, 0, sizeof(row));
+        w->row_cj_link[rs] = NKO_INVALID; w->row_cj_link_b[rs] = NKO_INVALID;
+        w->row_penetration[rs] = 0.0f;
+        if (slot < limit_rows) {   /* EmitJointLimitRow :805-882 */
+            const uint32_t l = slot / 2u, side = slot & 1u;
+            const size_t link = lbase + l;
+            const int scalar = nko_joint_dof(t->joint_type[l]) == 1u;
+            if (scalar && (t->joint_limit_flags[l] & (1u << side)) != 0u && dt > 0.0f) {
+                const float sign = side == 0u ? 1.0f : -1.0f;
+                const float bound = side == 0u ? t->joint_limit_lower[l] : t->joint_limit_upper[l];
+                const float signed_distance = side == 0u ? w->q[link] - bound : bound - w->q[link];
+                const float target_velocity = -(position_pass ? fmaxf(signed_distance, 0.0f) : signed_distance) / dt;
+                const float capped_velocity = fminf(target_velocity, w->cfg.solver_baumgarte_max_velocity);
+                row.flags = NKO_ROW_ACTIVE | (side == 0u ? NKO_ROW_JOINT_LIMIT_LOWER : NKO_ROW_JOINT_LIMIT_UPPER);
+                row.group_first = (uint32_t)rs; row.group_normal_count = 1u; row.env = env;
+                row.rhs = capped_velocity / dt;
+                row.lower = 0.0f; row.upper = FLT_MAX;
+                row.a.kind = NKO_SIDE_ARTIC; row.a.index = env;
+                J[t->link_dof[l]] = sign;
+                w->row_penetration[rs] = fmaxf(-signed_distance, 0.0f);
+                w->row_count[env] += 1u;
+            } else w->lambda[rs] = 0.0f;
+        } else if (slot < limit_rows + friction_rows) {   /* EmitJointFrictionRows :886-934 */
+            const uint32_t l = slot - limit_rows;
+            w->lambda[rs] = 0.0f;
+            const float friction = t->joint_frictionloss[l];
+            if (nko_joint_dof(t->joint_type[l]) == 1u && friction > 0.0f && dt > 0.0f) {
+                row.flags = NKO_ROW_ACTIVE | NKO_ROW_VELOCITY_ONLY;
+                row.group_first = (uint32_t)rs; row.group_normal_count = 1u; row.env = env;
+                row.lower = -friction * dt; row.upper = friction * dt;
+                row.a.kind = NKO_SIDE_ARTIC; row.a.index = env;
+                J[t->link_dof[l]] = 1.0f;
+                w->row_count[env] += 1u;
+            }
+        } else {   /* EmitJointDriveRows :938-971 */
+            const uint32_t l = slot - limit_rows - friction_rows;
+            const size_t link = lbase + l;
+            w->lambda[rs] = 0.0f;
+            const float effort = fminf(fmaxf(w->drive_command[link], w->drive_lower[link]), w->drive_upper[link]);
+            if (nko_joint_dof(t->joint_type[l]) == 1u && effort != 0.0f) {
+                row.flags = NKO_ROW_ACTIVE | NKO_ROW_VELOCITY_ONLY;
+                row.group_first = (uint32_t)rs; row.group_normal_count = 1u; row.env = env;
+                row.a.kind = NKO_SIDE_ARTIC; row.a.index = env;
+                J[t->link_dof[l]] = 1.0f;
+                row.lower = row.upper = effort * dt;
+                w->lambda[rs] = row.lower;   /* the row admits one impulse */
+                w->row_count[env] += 1u;
+            }
+        }
+        rows[rs] = row;
+    }
+}
+
 void nko_env_assemble_rows(nko_world* w, uint32_t env) {
     const nko_template* t = &w->t;
     const uint32_t R = t->rows_per_env, S = t->slots, CR = t->contact_rows_per_env;
@@ -582,6 +651,7 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
         }
     }
     w->row_count[env] += active_rows;
+    nko_env_joint_rows(w, env);
     /* chain Jacobians for both sides, then the shared-owner merge (:1587-1605, 172-186) */
     for (uint32_t r = 0u; r < R; ++r) {
         float* ja = w->chain_jacobian + ((size_t)env * R + r) * t->max_dof;

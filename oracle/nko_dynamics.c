@@ -488,8 +488,9 @@ void nko_env_dynamics(nko_world* w, uint32_t env, uint32_t integrate_velocity) {
         const int scalar = component == NKO_INVALID;
         velocity[d] = scalar ? qd[link] : lv[6u * link + component];
         bias[d] = scalar ? dot6(S + 6u * link, pf + 6u * link) : pf[6u * link + component];
-        if (scalar) bias[d] += 0.0f;
-        const float damping = scalar ? t->joint_damping[link] + 0.0f : 0.0f;
+        if (scalar) bias[d] += w->joint_gravity_force[lbase + link];
+        const int fold = w->fold_drive_damping && t->joint_drive_rows > 0u;   /* pipeline.cpp:380-381, 400 */
+        const float damping = scalar ? t->joint_damping[link] + (fold ? w->drive_dissipation[lbase + link] : 0.0f) : 0.0f;
         const float spring = scalar ? t->joint_stiffness[link] * (q[link] - t->joint_spring_reference[link]) : 0.0f;
         acceleration[d] = (scalar ? w->tau[lbase + link] : 0.0f) - bias[d] - damping * velocity[d] - spring;
     }
@@ -519,6 +520,7 @@ void nko_env_dynamics(nko_world* w, uint32_t env, uint32_t integrate_velocity) {
         mat66_mul_vec6(comp + 36u * l, S + 6u * l, force);
         float diagonal = dot6(S + 6u * l, force);
         diagonal += t->joint_armature[l];
+        if (w->fold_drive_damping && t->joint_drive_rows > 0u) diagonal += dt * w->drive_dissipation[lbase + l];   /* :206-208 */
         M[(size_t)dof_i * stride + dof_i] = diagonal;
         uint32_t walk = l;
         for (;;) {
@@ -634,4 +636,115 @@ void nko_env_link_velocities(nko_world* w, uint32_t env) {
             for (uint32_t c = 0u; c < 6u; ++c) v[c] += s[c] * w->qdot[lbase + l];
             memcpy(lv + 6u * l, v, sizeof(v));
         }
+}
+
+/* ---- ApplyDrives (articulation.cu:836-940 ApplyAffineDriveKernel) --------
+ * Controllers hand the row solver an affine effort `command - dissipation * qdot` and its bounds; the dissipation
+ * is folded into the articulation mass and bias when the velocity feedback is solved implicitly.  Gravity
+ * compensation (ProjectGravityCompensationKernel :393-423) is not authored on this path: joint_gravity_force
+ * stays as uploaded (zero by default).  The inverse-dynamics modes (ComputedTorque, Osc) are not built. */
+void nko_env_apply_drives(nko_world* w, uint32_t env) {
+    const nko_template* t = &w->t;
+    const uint32_t nl = t->nl, mode = t->drive_mode;
+    const size_t lbase = (size_t)env * nl;
+    const int implicit = w->fold_drive_damping;
+    const float dt = w->cfg.fixed_dt;
+    for (uint32_t l = 0u; l < nl; ++l) {
+        const size_t link = lbase + l;
+        w->drive_command[link] = w->drive_dissipation[link] = 0.0f;
+        w->drive_lower[link] = w->drive_upper[link] = 0.0f;
+        w->tau[link] = 0.0f;
+        if (nko_joint_dof(t->joint_type[l]) != 1u) continue;
+        const int position_control = mode == NKO_DRIVE_PD_POSITION;
+        const int velocity_control = mode == NKO_DRIVE_VELOCITY;
+        const float kp = w->drive_stiffness[link], kd = w->drive_damping[link];
+        if ((position_control && (!isfinite(w->drive_target[link]) || !isfinite(kp) || kp < 0.0f || !isfinite(kd) ||
+                                  (implicit && kd < 0.0f))) ||
+            ((position_control || velocity_control) && !isfinite(w->velocity_target[link])) ||
+            (velocity_control && (!isfinite(kp) || kp < 0.0f)) ||
+            (mode == NKO_DRIVE_ACTUATOR && !isfinite(w->actuator_noload_speed[link]))) {
+            w->env_status[env] |= NKO_STATUS_CONTROL_FAILURE;
+            continue;
+        }
+        const float velocity = w->qdot[link];
+        const float limit = w->drive_force_limit[link];
+        float lower = limit > 0.0f ? -limit : -FLT_MAX;
+        float upper = limit > 0.0f ? limit : FLT_MAX;
+        float bias = 0.0f, damping = 0.0f;
+        switch (mode) {
+            case NKO_DRIVE_PD_POSITION:
+                damping = kd + (implicit ? dt * kp : 0.0f);
+                bias = kp * (w->drive_target[link] - w->q[link]) + damping * w->velocity_target[link];
+                break;
+            case NKO_DRIVE_VELOCITY:
+                damping = kp;
+                bias = damping * w->velocity_target[link];
+                break;
+            case NKO_DRIVE_TORQUE:
+            case NKO_DRIVE_ACTUATOR:
+                bias = w->drive_target[link];
+                if (mode == NKO_DRIVE_ACTUATOR && limit > 0.0f && w->actuator_noload_speed[link] > 0.0f) {
+                    const float speed_bias = limit * velocity / w->actuator_noload_speed[link];
+                    lower = fminf(fmaxf(-limit - speed_bias, -limit), limit);
+                    upper = fminf(fmaxf(limit - speed_bias, -limit), limit);
+                }
+                break;
+            default: break;
+        }
+        const float effort = bias - damping * velocity;
+        const float gravity_force = w->joint_gravity_force[link];
+        const int saturated = effort < lower || effort > upper;
+        const float joint_limit = w->drive_joint_force_limit[link];
+        if (implicit && joint_limit > 0.0f) {
+            bias = fminf(fmaxf(fminf(fmaxf(effort, lower), upper) + gravity_force, -joint_limit), joint_limit);
+            damping = saturated ? 0.0f : damping;
+            bias += damping * velocity;
+            lower = -FLT_MAX;
+            upper = FLT_MAX;
+        } else if (!implicit || saturated) {
+            bias = effort + gravity_force;
+            damping = 0.0f;
+            lower += gravity_force;
+            upper += gravity_force;
+            if (joint_limit > 0.0f) {
+                lower = fminf(fmaxf(lower, -joint_limit), joint_limit);
+                upper = fminf(fmaxf(upper, -joint_limit), joint_limit);
+            }
+        } else {
+            bias += gravity_force;
+            lower += gravity_force + damping * velocity;
+            upper += gravity_force + damping * velocity;
+        }
+        const float feedforward = w->joint_f[link];
+        if (!isfinite(bias) || !isfinite(damping) || damping < 0.0f || !isfinite(limit) || !isfinite(feedforward) ||
+            !isfinite(velocity) || !isfinite(w->q[link])) {
+            w->env_status[env] |= NKO_STATUS_CONTROL_FAILURE;
+            continue;
+        }
+        w->drive_command[link] = bias;
+        w->drive_dissipation[link] = damping;
+        w->drive_lower[link] = lower;
+        w->drive_upper[link] = upper;
+        w->tau[link] = feedforward;
+    }
+}
+
+/* ---- ReadoutDrives (articulation.cu:999-1016) ---------------------------- */
+void nko_env_readout_drives(nko_world* w, uint32_t env) {
+    const nko_template* t = &w->t;
+    const uint32_t nl = t->nl, R = t->rows_per_env;
+    const uint32_t first_drive_row = t->contact_rows_per_env + t->joint_limit_rows + t->joint_friction_rows;
+    const float dt = w->cfg.fixed_dt;
+    for (uint32_t l = 0u; l < nl; ++l) {
+        const size_t link = (size_t)env * nl + l;
+        w->actuator_effort_requested[link] = w->actuator_effort[link] = w->actuator_saturated[link] = 0.0f;
+        if (nko_joint_dof(t->joint_type[l]) != 1u) continue;
+        const size_t row = (size_t)env * R + first_drive_row + l;
+        const float effort = w->drive_command[link] - w->drive_dissipation[link] * w->qdot[link];
+        w->actuator_effort_requested[link] = effort;
+        w->actuator_effort[link] = w->lambda[row] / dt - w->drive_dissipation[link] * w->qdot[link];
+        w->actuator_saturated[link] =
+            w->drive_command[link] < w->drive_lower[link] || w->drive_command[link] > w->drive_upper[link] ? 1.0f : 0.0f;
+        w->tau[link] += w->actuator_effort[link];
+    }
 }

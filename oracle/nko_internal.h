@@ -22,12 +22,16 @@ enum { NKO_SIDE_RIGID = 0, NKO_SIDE_ARTIC = 1, NKO_SIDE_STATIC = 3 };
 /* nk/solve/nk_row.hpp:41-57 */
 enum {
     NKO_ROW_ACTIVE = 1u << 0, NKO_ROW_BLOCK_NORMAL = 1u << 2, NKO_ROW_BLOCK_TANGENT = 1u << 3,
+    NKO_ROW_JOINT_LIMIT_LOWER = 1u << 4, NKO_ROW_JOINT_LIMIT_UPPER = 1u << 5,
     NKO_ROW_CONTACT_NORMAL = 1u << 6, NKO_ROW_VELOCITY_ONLY = 1u << 7, NKO_ROW_SPECULATIVE = 1u << 8,
     NKO_ROW_MUJOCO = 1u << 11, NKO_ROW_FRICTION = 1u << 1
 };
 /* phi/op_schema.hpp:36-52 */
 enum { NKO_STATUS_PAIR_OVERFLOW = 1u << 0, NKO_STATUS_DOF_OVERFLOW = 1u << 2, NKO_STATUS_INVALID_ENDPOINT = 1u << 6,
-       NKO_STATUS_SOLVER_FAILURE = 1u << 13 };
+       NKO_STATUS_CONTROL_FAILURE = 1u << 10, NKO_STATUS_SOLVER_FAILURE = 1u << 13 };
+/* phi/articulation_contract.hpp:16-23 */
+enum { NKO_DRIVE_PD_POSITION = 0, NKO_DRIVE_TORQUE = 1, NKO_DRIVE_VELOCITY = 2, NKO_DRIVE_COMPUTED_TORQUE = 3,
+       NKO_DRIVE_OSC = 4, NKO_DRIVE_ACTUATOR = 5 };
 
 typedef struct { float x, y, z; } v3;
 typedef struct { float w, x, y, z; } quat;
@@ -47,6 +51,8 @@ typedef struct {
 /* Cooked template shared by every environment. */
 typedef struct {
     uint32_t nl, nb, nv, max_dof, slots, rows_per_env, contact_rows_per_env, n_profiles, max_depth;
+    /* joint row slots after the contact rows: 2 per link, 1 per link, 1 per link, or 0 (cook_to_model.cpp:706-719) */
+    uint32_t joint_limit_rows, joint_friction_rows, joint_drive_rows, drive_mode;
     int floating;
     uint8_t* joint_type;
     uint32_t* parent_link;
@@ -56,6 +62,8 @@ typedef struct {
     float* link_inertial_frame; /* nl*7 */
     float* link_inertia;        /* nl*36 */
     float* joint_damping, *joint_armature, *joint_stiffness, *joint_spring_reference;
+    float* joint_limit_lower, *joint_limit_upper, *joint_frictionloss;   /* nl */
+    uint8_t* joint_limit_flags;                                          /* nl: bit 0 lower, bit 1 upper */
     uint32_t* link_body;        /* nl */
     uint32_t* link_tree_depth;  /* nl */
     uint32_t* link_child_range; /* nl*2 */
@@ -98,6 +106,12 @@ struct nko_world {
     float *contact_cache_lambda, *contact_cache_normal;
     uint32_t *contact_cache_age, *contact_cache_current_owner, *contact_cache_old_keep, *contact_cache_extent;
     uint32_t *contact_warm_start_counts, *contact_cache_match;
+    /* drives (fields.yaml:49-53, 328, 658-668, 548-551, 906) */
+    float *drive_target, *drive_stiffness, *drive_damping, *drive_force_limit, *drive_joint_force_limit;
+    float *velocity_target, *actuator_noload_speed, *joint_f, *joint_gravity_force;
+    float *drive_command, *drive_dissipation, *drive_lower, *drive_upper;
+    float *joint_limit_impulse, *actuator_effort_requested, *actuator_effort, *actuator_saturated;
+    int fold_drive_damping;
 };
 
 /* ---- math (nko_math.c) ------------------------------------------------- */
@@ -131,6 +145,9 @@ xform nko_compose_hd(xform parent, xform child);
 uint32_t nko_joint_dof(uint8_t type);
 
 void nko_env_fk(const nko_world* w, uint32_t env);
+void nko_env_apply_drives(nko_world* w, uint32_t env);
+void nko_env_readout_drives(nko_world* w, uint32_t env);
+void nko_env_joint_rows(nko_world* w, uint32_t env);
 void nko_env_dynamics(nko_world* w, uint32_t env, uint32_t integrate_velocity);
 void nko_env_integrate_position(nko_world* w, uint32_t env);
 void nko_env_link_velocities(nko_world* w, uint32_t env);

@@ -845,6 +845,13 @@ void nko_env_solve(nko_world* w, uint32_t env) {
             }
         else w->env_status[env] |= NKO_STATUS_SOLVER_FAILURE;
     }
+    /* joint limit impulses (FinishTile :2658-2668) */
+    if (tp->joint_limit_rows >= 2u * nl)
+        for (uint32_t l = 0u; l < nl; ++l) {
+            const size_t lower = (size_t)env * R + tp->contact_rows_per_env + (size_t)l * 2u;
+            w->joint_limit_impulse[2u * (lbase + l)] = (rows[lower].flags & NKO_ROW_ACTIVE) != 0u ? w->lambda[lower] : 0.0f;
+            w->joint_limit_impulse[2u * (lbase + l) + 1u] = (rows[lower + 1u].flags & NKO_ROW_ACTIVE) != 0u ? w->lambda[lower + 1u] : 0.0f;
+        }
     /* split-impulse position pass (:3059-3077, MarkTilePositions :2673-2708) */
     if (w->cfg.solver_pos_iters != 0u) {
         float pseudo[NKO_MAX_DOF];

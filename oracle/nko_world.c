@@ -25,6 +25,8 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
     t->link_inertia = ALLOC(float, nl * 36u);
     t->joint_damping = ALLOC(float, nl); t->joint_armature = ALLOC(float, nl);
     t->joint_stiffness = ALLOC(float, nl); t->joint_spring_reference = ALLOC(float, nl);
+    t->joint_limit_lower = ALLOC(float, nl); t->joint_limit_upper = ALLOC(float, nl);
+    t->joint_frictionloss = ALLOC(float, nl); t->joint_limit_flags = ALLOC(uint8_t, nl);
     t->link_body = ALLOC(uint32_t, nl); t->link_tree_depth = ALLOC(uint32_t, nl);
     t->link_child_range = ALLOC(uint32_t, nl * 2u); t->link_children = ALLOC(uint32_t, nl);
     t->link_dof = ALLOC(uint32_t, nl);
@@ -39,6 +41,12 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
     copy_or_zero(t->joint_armature, d->joint_armature, nl);
     copy_or_zero(t->joint_stiffness, d->joint_stiffness, nl);
     copy_or_zero(t->joint_spring_reference, d->joint_spring_reference, nl);
+    const int has_joint_rows = d->struct_size >= sizeof(nko_template_desc);
+    copy_or_zero(t->joint_limit_lower, has_joint_rows ? d->joint_limit_lower : NULL, nl);
+    copy_or_zero(t->joint_limit_upper, has_joint_rows ? d->joint_limit_upper : NULL, nl);
+    copy_or_zero(t->joint_frictionloss, has_joint_rows ? d->joint_frictionloss : NULL, nl);
+    if (has_joint_rows && d->joint_limit_flags != NULL) memcpy(t->joint_limit_flags, d->joint_limit_flags, nl);
+    t->drive_mode = has_joint_rows ? d->drive_mode : NKO_DRIVE_TORQUE;
     uint32_t nv = 0u;
     for (uint32_t l = 0u; l < nl; ++l) {
         nko_make_spatial_inertia(d->link_mass[l], d->link_diag_inertia + 3u * l, d->link_inertial_frame + 7u * l, t->link_inertia + 36u * l);
@@ -121,14 +129,28 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
     }
     t->slots = slots;
     t->contact_rows_per_env = slots * 16u;   /* nk_row.hpp:59-63: 4 points x 4 rows per rigid slot */
-    t->rows_per_env = t->contact_rows_per_env;
+    /* joint row slots (cook_to_model.cpp:696-719, nk/pipeline/world.cpp:61, 96) */
+    int any_limit = 0, any_friction = 0;
+    for (uint32_t l = 0u; l < nl; ++l) {
+        const uint8_t flags = t->joint_limit_flags[l];
+        if (((flags & 1u) && !isfinite(t->joint_limit_lower[l])) || ((flags & 2u) && !isfinite(t->joint_limit_upper[l])) ||
+            ((flags & 3u) == 3u && t->joint_limit_lower[l] > t->joint_limit_upper[l])) return -1;
+        if (!isfinite(t->joint_frictionloss[l]) || t->joint_frictionloss[l] < 0.0f) return -1;
+        any_limit = any_limit || flags != 0u;
+        any_friction = any_friction || t->joint_frictionloss[l] > 0.0f;
+    }
+    t->joint_limit_rows = any_limit ? nl * 2u : 0u;
+    t->joint_friction_rows = any_friction ? nl : 0u;
+    t->joint_drive_rows = has_joint_rows && d->drive_rows != 0u ? nl : 0u;
+    t->rows_per_env = t->contact_rows_per_env + t->joint_limit_rows + t->joint_friction_rows + t->joint_drive_rows;
     return 0;
 }
 
 static void free_template(nko_template* t) {
     free(t->joint_type); free(t->parent_link); free(t->joint_axis); free(t->parent_offset); free(t->link_local_pose);
     free(t->link_inertial_frame); free(t->link_inertia); free(t->joint_damping); free(t->joint_armature);
-    free(t->joint_stiffness); free(t->joint_spring_reference); free(t->link_body); free(t->link_tree_depth);
+    free(t->joint_stiffness); free(t->joint_spring_reference); free(t->joint_limit_lower); free(t->joint_limit_upper);
+    free(t->joint_frictionloss); free(t->joint_limit_flags); free(t->link_body); free(t->link_tree_depth);
     free(t->link_child_range); free(t->link_children); free(t->link_dof); free(t->dof_link); free(t->dof_component);
     free(t->link_geom_local); free(t->link_geom_kind); free(t->shape_table); free(t->body_to_link);
     free(t->body_to_articulation); free(t->body_collidable_link); free(t->body_collidable_body);
@@ -149,6 +171,9 @@ nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc*
     if (w->cfg.solver_pos_slop <= 0.0f) w->cfg.solver_pos_slop = 1.0e-3f;
     if (w->cfg.solver_velocity_tolerance <= 0.0f) w->cfg.solver_velocity_tolerance = 1.0e-5f;
     if (w->cfg.solver_baumgarte_max_velocity <= 0.0f) w->cfg.solver_baumgarte_max_velocity = 3.0e38f;
+    /* pipeline.hpp:48-49: velocity feedback of a drive is solved implicitly unless switched off */
+    w->fold_drive_damping = 1;
+    if (desc->struct_size >= sizeof(nko_world_desc) && desc->solver_fold_drive_damping == 0xFFFFFFFFu) w->fold_drive_damping = 0;
     w->env_count = desc->env_count;
     w->threads = 1;
     const nko_template* t = &w->t;
@@ -179,6 +204,14 @@ nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc*
     w->contact_cache_age = ALLOC(uint32_t, E * S * 4u); w->contact_cache_current_owner = ALLOC(uint32_t, E * S * 4u);
     w->contact_cache_old_keep = ALLOC(uint32_t, E * S * 4u); w->contact_cache_extent = ALLOC(uint32_t, E * 2u);
     w->contact_warm_start_counts = ALLOC(uint32_t, E * 2u); w->contact_cache_match = ALLOC(uint32_t, E * S * 4u);
+    w->drive_target = ALLOC(float, E * nl); w->drive_stiffness = ALLOC(float, E * nl); w->drive_damping = ALLOC(float, E * nl);
+    w->drive_force_limit = ALLOC(float, E * nl); w->drive_joint_force_limit = ALLOC(float, E * nl);
+    w->velocity_target = ALLOC(float, E * nl); w->actuator_noload_speed = ALLOC(float, E * nl); w->joint_f = ALLOC(float, E * nl);
+    w->joint_gravity_force = ALLOC(float, E * nl);
+    w->drive_command = ALLOC(float, E * nl); w->drive_dissipation = ALLOC(float, E * nl); w->drive_lower = ALLOC(float, E * nl);
+    w->drive_upper = ALLOC(float, E * nl); w->joint_limit_impulse = ALLOC(float, E * nl * 2u);
+    w->actuator_effort_requested = ALLOC(float, E * nl); w->actuator_effort = ALLOC(float, E * nl);
+    w->actuator_saturated = ALLOC(float, E * nl);
     for (size_t i = 0u; i < E * R; ++i) { w->row_cj_link[i] = NKO_INVALID; w->row_cj_link_b[i] = NKO_INVALID; }
     for (size_t e = 0u; e < E; ++e) {
         const float id[7] = {0, 0, 0, 1, 0, 0, 0};
@@ -205,6 +238,10 @@ void nko_world_destroy(nko_world* w) {
     free(w->contact_material); free(w->contact_cache_pair); free(w->contact_cache_feature); free(w->contact_cache_material);
     free(w->contact_cache_lambda); free(w->contact_cache_normal); free(w->contact_cache_age); free(w->contact_cache_current_owner);
     free(w->contact_cache_old_keep); free(w->contact_cache_extent); free(w->contact_warm_start_counts); free(w->contact_cache_match);
+    free(w->drive_target); free(w->drive_stiffness); free(w->drive_damping); free(w->drive_force_limit);
+    free(w->drive_joint_force_limit); free(w->velocity_target); free(w->actuator_noload_speed); free(w->joint_f);
+    free(w->joint_gravity_force); free(w->drive_command); free(w->drive_dissipation); free(w->drive_lower); free(w->drive_upper);
+    free(w->joint_limit_impulse); free(w->actuator_effort_requested); free(w->actuator_effort); free(w->actuator_saturated);
     free(w);
 }
 
@@ -229,7 +266,13 @@ void nko_world_destroy(nko_world* w) {
     X(contact_cache_material, uint64_t, E * S * 4u) X(contact_cache_lambda, float, E * S * 16u) \
     X(contact_cache_normal, float, E * S * 12u) X(contact_cache_age, uint32_t, E * S * 4u) \
     X(contact_cache_current_owner, uint32_t, E * S * 4u) X(contact_cache_old_keep, uint32_t, E * S * 4u) \
-    X(contact_cache_extent, uint32_t, E * 2u) X(contact_warm_start_counts, uint32_t, E * 2u)
+    X(contact_cache_extent, uint32_t, E * 2u) X(contact_warm_start_counts, uint32_t, E * 2u) \
+    X(drive_target, float, E * nl) X(drive_stiffness, float, E * nl) X(drive_damping, float, E * nl) \
+    X(drive_force_limit, float, E * nl) X(drive_joint_force_limit, float, E * nl) X(velocity_target, float, E * nl) \
+    X(actuator_noload_speed, float, E * nl) X(joint_f, float, E * nl) X(joint_gravity_force, float, E * nl) \
+    X(drive_command, float, E * nl) X(drive_dissipation, float, E * nl) X(drive_lower, float, E * nl) \
+    X(drive_upper, float, E * nl) X(joint_limit_impulse, float, E * nl * 2u) X(actuator_effort_requested, float, E * nl) \
+    X(actuator_effort, float, E * nl) X(actuator_saturated, float, E * nl)
 
 #define TEMPLATE_LIST(X) \
     X(link_inertia, float, nl * 36u) X(link_tree_depth, uint32_t, nl) X(link_child_range, uint32_t, nl * 2u) \
@@ -266,6 +309,8 @@ uint32_t nko_world_rows_per_env(const nko_world* w) { return w->t.rows_per_env; 
       for (long env_ = 0; env_ < (long)w->env_count; ++env_) { const uint32_t env = (uint32_t)env_; body; } }
 
 void nko_fk_world_poses(nko_world* w) { FOR_ENVS(nko_env_fk(w, env)) }
+void nko_apply_drives(nko_world* w) { FOR_ENVS(nko_env_apply_drives(w, env)) }
+void nko_readout_drives(nko_world* w) { FOR_ENVS(nko_env_readout_drives(w, env)) }
 void nko_articulation_dynamics(nko_world* w, uint32_t integrate_velocity) { FOR_ENVS(nko_env_dynamics(w, env, integrate_velocity)) }
 void nko_sync_link_body_pose(nko_world* w) { FOR_ENVS(nko_env_sync_body_pose(w, env)) }
 void nko_build_aabbs(nko_world* w) { FOR_ENVS(nko_env_aabbs(w, env)) }
@@ -284,17 +329,21 @@ void nko_fk_link_velocities(nko_world* w) { FOR_ENVS(nko_env_link_velocities(w, 
 /* Op order of one step (src/nk/pipeline/pipeline.cpp:374-986) for an articulated world with ground contact. */
 void nko_world_step(nko_world* w) {
     nko_fk_world_poses(w);
+    if (w->t.joint_drive_rows > 0u) nko_apply_drives(w);
     nko_articulation_dynamics(w, 1u);
     if (w->t.rows_per_env > 0u) {
-        nko_sync_link_body_pose(w);
-        nko_build_aabbs(w);
-        nko_query_pairs(w);
-        nko_narrowphase(w);
+        if (w->t.slots > 0u) {
+            nko_sync_link_body_pose(w);
+            nko_build_aabbs(w);
+            nko_query_pairs(w);
+            nko_narrowphase(w);
+        }
         nko_assemble_rows(w);
         nko_contact_warm_start(w, 0u);
         nko_block_descent_solve(w);
         nko_contact_warm_start(w, 1u);
     }
+    if (w->t.joint_drive_rows > 0u) nko_readout_drives(w);   /* pipeline.cpp:929-937 */
     nko_integrate_position(w);
     nko_fk_world_poses(w);
     nko_fk_link_velocities(w);

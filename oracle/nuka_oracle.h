@@ -78,6 +78,13 @@ typedef struct nko_template_desc {
     const uint32_t* shape_group;
     const uint32_t* shape_profile;
     const float* profile_mu;
+    /* joint rows and drives; read only when struct_size covers them */
+    const float* joint_limit_lower;
+    const float* joint_limit_upper;
+    const uint8_t* joint_limit_flags;
+    const float* joint_frictionloss;
+    uint32_t drive_mode;
+    uint32_t drive_rows;
 } nko_template_desc;
 
 typedef struct nko_world_desc {
@@ -93,6 +100,7 @@ typedef struct nko_world_desc {
     float solver_velocity_tolerance;
     float solver_baumgarte_max_velocity;
     float solver_overlap_recovery_velocity;
+    uint32_t solver_fold_drive_damping;   /* read only when struct_size covers it */
 } nko_world_desc;
 
 typedef struct nko_world nko_world;
@@ -109,6 +117,7 @@ uint32_t nko_world_rows_per_env(const nko_world* w);
 
 /* One call per reference op (src/nk/pipeline/pipeline.cpp op order). */
 void nko_fk_world_poses(nko_world* w);
+void nko_apply_drives(nko_world* w);
 void nko_articulation_dynamics(nko_world* w, uint32_t integrate_velocity);
 void nko_sync_link_body_pose(nko_world* w);
 void nko_build_aabbs(nko_world* w);
@@ -117,6 +126,7 @@ void nko_narrowphase(nko_world* w);
 void nko_assemble_rows(nko_world* w);
 void nko_contact_warm_start(nko_world* w, uint32_t phase);
 void nko_block_descent_solve(nko_world* w);
+void nko_readout_drives(nko_world* w);
 void nko_integrate_position(nko_world* w);
 void nko_fk_link_velocities(nko_world* w);
 /* The whole op list of one step, in the reference's order. */

@@ -26,9 +26,9 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_struct_layouts_match_the_header():
-    # 6 u32 + 22 pointers; 14 4-byte words
-    assert C.sizeof(nk.abi.TemplateDescC) == 6 * 4 + 22 * 8
-    assert C.sizeof(nk.abi.WorldDescC) == 14 * 4
+    # 6 u32 + 22 pointers, then 4 pointers + 2 u32 of joint rows; 15 4-byte words
+    assert C.sizeof(nk.abi.TemplateDescC) == 6 * 4 + 22 * 8 + 4 * 8 + 2 * 4
+    assert C.sizeof(nk.abi.WorldDescC) == 15 * 4
 
 
 def test_op_catalog_names_round_trip():
@@ -37,7 +37,7 @@ def test_op_catalog_names_round_trip():
     names = [lib.nuka_hip_op_name(i).decode() for i in range(count)]
     for expected in ("FkWorldPoses", "ArticulationDynamics", "SyncLinkBodyPose", "BuildAabbs", "LbvhQueryPairs",
                      "NarrowphasePrimitives", "AssembleRows", "ContactWarmStart", "BlockDescentSolve", "IntegratePosition",
-                     "FkLinkVelocities"):
+                     "FkLinkVelocities", "ApplyDrives", "ReadoutDrives"):
         assert expected in names
         assert lib.nuka_hip_op_from_name(expected.encode()) == names.index(expected)
     assert lib.nuka_hip_op_from_name(b"NoSuchOp") == -1
@@ -50,7 +50,8 @@ def test_field_names_cover_the_seam_fields():
                  "m_factor", "articulation_bias", "candidate_pairs", "pair_count", "ucontact_count", "ucontact_point",
                  "ucontact_normal", "ucontact_depth", "ucontact_row_range", "urows", "lambda", "chain_jacobian",
                  "chain_jacobian_b", "env_status", "solver_residual", "vbd_velocity_sweep_count", "link_inertia",
-                 "shape_table"):
+                 "shape_table", "drive_target", "drive_stiffness", "drive_damping", "drive_force_limit", "velocity_target",
+                 "joint_f", "drive_command", "actuator_effort", "joint_limit_impulse"):
         assert name in fields
         assert lib.nuka_field_from_name(name.encode()) == fields.index(name)
     assert lib.nuka_field_from_name(b"no_such_field") == 0xFFFFFFFF
