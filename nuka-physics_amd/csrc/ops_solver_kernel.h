@@ -1132,7 +1132,8 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
             if (h < heads) {
                 const uint32_t source_a = c.U(hSourceA, h), source_b = c.U(hSourceB, h);
                 const bool owned = source_a != kInvalid || source_b != kInvalid;
-                const bool single_axis = (__float_as_uint(urows[size_t{c.U(hSlot, h)} * kRowWords]) & kRowBlockNormal) == 0u;
+                // a block head has found the sources of its tangent rows on the sides that move
+                const bool single_axis = c.U(hSourceA + 1u, h) == kInvalid && c.U(hSourceB + 1u, h) == kInvalid;
                 if (owned && single_axis) {
                     uint32_t supported = 0u, last = 0u;
                     float last_value = 0.0f;
