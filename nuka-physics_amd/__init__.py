@@ -225,6 +225,9 @@ class World:
         return out.value
 
     def profile_ops(self, steps, checkpoint=None):
+        info = WorldInfoC()
+        _check(lib().nuka_world_get_info(self._h, C.byref(info)))
+        self.op_count = info.op_count   # a demanded readout joins the pipeline
         ms = (C.c_float * self.op_count)()
         ops = (C.c_uint16 * self.op_count)()
         _check(lib().nuka_world_profile_ops(self._h, checkpoint, steps, ms, ops))

@@ -18,7 +18,7 @@ const char* OpName(NkOp op) {
         "ApplyDrives", "ArticulationDynamics", "IntegrateVelocity", "FkWorldPoses", "IntegratePosition", "BuildAabbs",
         "LbvhBuild", "LbvhQueryPairs", "NarrowphasePrimitives", "AssembleRows", "SyncLinkBodyPose", "NarrowphaseHeightfield",
         "ContactWarmStart", "SnapshotStepVelocity", "FkLinkVelocities", "BlockDescentSolve", "ResetEnvs", "SnapshotState",
-        "RestoreState", "ReadoutDrives"};
+        "RestoreState", "ReadoutDrives", "ReadoutContactWrench"};
     return op < NkOp::Count ? names[static_cast<uint16_t>(op)] : "?";
 }
 
@@ -47,6 +47,7 @@ void RegisterOps() {
     set(NkOp::FkLinkVelocities, &OpFkLinkVelocities);
     set(NkOp::BlockDescentSolve, &OpBlockDescentSolve);
     set(NkOp::ReadoutDrives, &OpReadoutDrives);
+    set(NkOp::ReadoutContactWrench, &OpReadoutContactWrench);
 }
 
 void Fail(nuka_phi_execution_error* error, Status status, uint16_t op, int native, const char* message) {

@@ -26,6 +26,7 @@ Status OpAssembleRows(const ModelView&, const DataView&, const void*, hipStream_
 Status OpContactWarmStart(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpBlockDescentSolve(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpReadoutDrives(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpReadoutContactWrench(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpSnapshotStepVelocity(const ModelView&, const DataView&, const void*, hipStream_t);
 
 }  // namespace nkh

@@ -15,7 +15,7 @@ enum class NkOp : uint16_t {
     ApplyDrives, ArticulationDynamics, IntegrateVelocity, FkWorldPoses, IntegratePosition, BuildAabbs, LbvhBuild,
     LbvhQueryPairs, NarrowphasePrimitives, AssembleRows, SyncLinkBodyPose, NarrowphaseHeightfield, ContactWarmStart,
     SnapshotStepVelocity, FkLinkVelocities, BlockDescentSolve, ResetEnvs, SnapshotState, RestoreState,
-    ReadoutDrives,
+    ReadoutDrives, ReadoutContactWrench,
     Count
 };
 
@@ -116,6 +116,9 @@ struct DataView {
     float *velocity_target, *actuator_noload_speed, *joint_f, *joint_gravity_force;
     float *drive_command, *drive_dissipation, *drive_lower, *drive_upper;
     float *joint_limit_impulse, *actuator_effort_requested, *actuator_effort, *actuator_saturated;
+    // contact readout (fields.yaml contact_point .. link_contact_wrench), written by ReadoutContactWrench on demand
+    float *contact_point, *contact_normal, *contact_force, *ucontact_impulse, *link_contact_wrench;
+    uint32_t *contact_side_a_kind, *contact_side_b_kind, *contact_side_a_index, *contact_side_b_index, *contact_link;
     uint32_t *reset_env_ids;                // staging of nuka_world_reset_envs
     uint32_t *solver_cost, *tile_order;     // last solve's work per environment; launch order of the next solve (costliest first)
     float *snapshot;                        // SnapshotState / RestoreState storage
@@ -169,6 +172,10 @@ struct BlockDescentSolveParams {   // op_schema.hpp:549-636 (the tile-route subs
     float position_beta, position_slop, position_max_velocity;
     float velocity_tolerance;
     uint32_t joint_limit_rows_per_env;
+};
+struct ReadoutContactWrenchParams {   // op_schema.hpp:746-755
+    float dt;
+    uint32_t env_count, base_link_count, max_contacts_per_env, rows_per_env, full_row_slot_count, contact_rows_per_env;
 };
 struct SnapshotParams { uint32_t env_count, selected_env_count; };
 

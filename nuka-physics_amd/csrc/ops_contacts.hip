@@ -857,6 +857,91 @@ Status OpContactWarmStart(const ModelView&, const DataView& d, const void* param
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 
+namespace {
+// ReadoutContactWrench (ops/readout.cu:59-220, 559-626): per contact slot the first manifold point and normal, the
+// summed {normal, tangent, tangent} force, each point's world impulse, the two sides' owners and the contact's link;
+// per link the world-frame wrench of every active row ending on it.  One wavefront per environment.  The reference
+// sorts (link, row, side) keys to list a link's endpoints; here a lane per link walks the environment's rows in that
+// same order - ascending row, side A before B - so the sums add in the same sequence.
+__global__ void __launch_bounds__(kWave) ReadoutContactWrenchKernel(ModelView m, DataView d, ReadoutContactWrenchParams p) {
+    const uint32_t env = blockIdx.x, lane = threadIdx.x;
+    const uint32_t S = p.max_contacts_per_env, R = p.rows_per_env, nl = p.base_link_count;
+    const float inv_dt = p.dt > 0.0f ? 1.0f / p.dt : 0.0f;
+    const Row* rows = reinterpret_cast<const Row*>(d.urows);
+    for (uint32_t s = lane; s < S; s += kWave) {
+        const size_t slot = size_t{env} * S + s;
+        const uint32_t points = d.ucontact_count[slot];
+        for (uint32_t k = 0u; k < 3u; ++k) {   // LegacyContactGeometryKernel :59-77
+            d.contact_point[slot * 3u + k] = points > 0u ? d.ucontact_point[slot * 12u + k] : 0.0f;
+            d.contact_normal[slot * 3u + k] = points > 0u ? d.ucontact_normal[slot * 12u + k] : 0.0f;
+        }
+        const uint32_t first = d.ucontact_row_range[slot * 2u], pts = d.ucontact_row_range[slot * 2u + 1u];   // ContactForceKernel :80-123
+        float fn = 0.0f, ft1 = 0.0f, ft2 = 0.0f;
+        for (uint32_t i = 0u; i < pts; ++i) {
+            fn += d.lambda[first + i]; ft1 += d.lambda[first + i + pts]; ft2 += d.lambda[first + i + 2u * pts];
+        }
+        for (uint32_t i = 0u; i < kPointsPerSlot; ++i) {   // ContactPointWorldImpulse, nk/contact/row_readout.hpp:38-48
+            V3 impulse{0.0f, 0.0f, 0.0f};
+            if (i < pts && (rows[first + i].flags & kRowActive) != 0u)
+                for (uint32_t axis = 0u; axis < 3u; ++axis) {
+                    const uint32_t index = first + i + axis * pts;
+                    const float l = d.lambda[index];
+                    impulse.x += rows[index].a.jlin.x * l; impulse.y += rows[index].a.jlin.y * l; impulse.z += rows[index].a.jlin.z * l;
+                }
+            float* out = d.ucontact_impulse + (slot * kPointsPerSlot + i) * 3u;
+            out[0] = impulse.x; out[1] = impulse.y; out[2] = impulse.z;
+        }
+        d.contact_force[slot * 3u] = fn * inv_dt; d.contact_force[slot * 3u + 1u] = ft1 * inv_dt; d.contact_force[slot * 3u + 2u] = ft2 * inv_dt;
+        const bool active = pts > 0u && (rows[first].flags & kRowActive) != 0u;
+        const uint32_t kind_a = active ? rows[first].a.kind : uint32_t(kSideStatic), kind_b = active ? rows[first].b.kind : uint32_t(kSideStatic);
+        d.contact_side_a_kind[slot] = kind_a; d.contact_side_b_kind[slot] = kind_b;
+        d.contact_side_a_index[slot] = !active || kind_a == kSideStatic ? kInvalid : kind_a == kSideArtic ? d.row_cj_link[first] : rows[first].a.index;
+        d.contact_side_b_index[slot] = !active || kind_b == kSideStatic ? kInvalid : kind_b == kSideArtic ? d.row_cj_link_b[first] : rows[first].b.index;
+        uint32_t link = kInvalid;   // ContactLinkKernel :127-149
+        for (uint32_t i = 0u; i < pts && link == kInvalid; ++i) link = d.row_cj_link[first + i];
+        for (uint32_t i = 0u; i < pts && link == kInvalid; ++i) link = d.row_cj_link_b[first + i];
+        d.contact_link[slot] = link;
+    }
+    // LinkContactWrenchKernel :154-220
+    const uint32_t previous = d.contact_row_extent[2u * env], current = d.contact_row_extent[2u * env + 1u];
+    const uint32_t bound = contact_row_bound(previous, current, p.contact_rows_per_env);
+    for (uint32_t base = 0u; base < nl; base += kWave) {
+        const uint32_t l = base + lane;
+        const uint32_t link = env * nl + l;
+        V3 origin{0.0f, 0.0f, 0.0f}, force{0.0f, 0.0f, 0.0f}, torque{0.0f, 0.0f, 0.0f};
+        if (l < nl) origin = V3{d.link_pose[size_t{link} * 7u], d.link_pose[size_t{link} * 7u + 1u], d.link_pose[size_t{link} * 7u + 2u]};
+        for (uint32_t r = 0u; r < bound; ++r) {
+            const size_t rs = size_t{env} * R + r;
+            if ((rows[rs].flags & kRowActive) == 0u) continue;
+            const uint32_t ends[2] = {d.row_cj_link[rs], d.row_cj_link_b[rs]};
+            const float scale = d.lambda[rs] * inv_dt;
+            for (uint32_t side = 0u; side < 2u; ++side) {
+                if (l >= nl || ends[side] != link) continue;
+                const V3 dir = side == 0u ? rows[rs].a.jlin : rows[rs].b.jlin;
+                const float* point = (side == 0u ? d.row_cj_point : d.row_cj_point_b) + rs * 3u;
+                const V3 f{dir.x * scale, dir.y * scale, dir.z * scale};
+                const V3 moment = cross3(sub3(V3{point[0], point[1], point[2]}, origin), f);
+                force = V3{force.x + f.x, force.y + f.y, force.z + f.z};
+                torque = V3{torque.x + moment.x, torque.y + moment.y, torque.z + moment.z};
+            }
+        }
+        if (l < nl) {
+            float* out = d.link_contact_wrench + size_t{link} * 6u;
+            out[0] = force.x; out[1] = force.y; out[2] = force.z; out[3] = torque.x; out[4] = torque.y; out[5] = torque.z;
+        }
+    }
+}
+}  // namespace
+
+Status OpReadoutContactWrench(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const ReadoutContactWrenchParams*>(params);
+    if (p == nullptr) return Status::InvalidArgument;
+    if (p->full_row_slot_count > p->max_contacts_per_env || p->contact_rows_per_env > p->rows_per_env) return Status::InvalidArgument;
+    if (p->env_count == 0u || p->max_contacts_per_env == 0u) return Status::Ok;
+    hipLaunchKernelGGL(ReadoutContactWrenchKernel, dim3(p->env_count), dim3(kWave), 0, stream, m, d, *p);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
 Status OpSnapshotStepVelocity(const ModelView&, const DataView&, const void*, hipStream_t) { return Status::Ok; }
 
 void InitContactKernels() {

@@ -252,7 +252,11 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(drive_joint_force_limit, kF32, E * nl) X(velocity_target, kF32, E * nl) X(actuator_noload_speed, kF32, E * nl) \
     X(joint_f, kF32, E * nl) X(joint_gravity_force, kF32, E * nl) X(drive_command, kF32, E * nl) X(drive_dissipation, kF32, E * nl) \
     X(drive_lower, kF32, E * nl) X(drive_upper, kF32, E * nl) X(joint_limit_impulse, kF32, E * nl * 2) \
-    X(actuator_effort_requested, kF32, E * nl) X(actuator_effort, kF32, E * nl) X(actuator_saturated, kF32, E * nl)
+    X(actuator_effort_requested, kF32, E * nl) X(actuator_effort, kF32, E * nl) X(actuator_saturated, kF32, E * nl) \
+    X(contact_point, kF32, E * S * 3) X(contact_normal, kF32, E * S * 3) X(contact_force, kF32, E * S * 3) \
+    X(ucontact_impulse, kF32, E * S * 12) X(link_contact_wrench, kF32, E * nl * 6) X(contact_side_a_kind, kU32, E * S) \
+    X(contact_side_b_kind, kU32, E * S) X(contact_side_a_index, kU32, E * S) X(contact_side_b_index, kU32, E * S) \
+    X(contact_link, kU32, E * S)
 
 #define NKH_MODEL_FIELDS(X) \
     X(joint_type, kU8) X(parent_link, kU32) X(joint_axis, kF32) X(parent_offset, kF32) X(link_local_pose, kF32) \
@@ -289,6 +293,8 @@ struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
     FkLinkVelocitiesParams p_fk_velocity{};
     ApplyDrivesParams p_drives{};
     ReadoutDrivesParams p_readout_drives{};
+    ReadoutContactWrenchParams p_readout_contacts{};
+    bool contact_readout_demanded = false;   // nk/pipeline/pipeline.hpp:60 kReadoutContactWrench
     ArticulationDynamicsParams p_dynamics{}, p_dynamics_probe{};
     IntegrateVelocityParams p_int_vel{};
     IntegratePositionParams p_int_pos{};
@@ -464,6 +470,9 @@ void BuildPipeline(World& w) {
     add(NkOp::FkWorldPoses, &w.p_fk);
     add(NkOp::FkLinkVelocities, &w.p_fk_velocity);
     if (nb > 0u) add(NkOp::SyncLinkBodyPose, &w.p_sync);
+    // a pure readout, part of the step only once a consumer has asked for one of its fields (pipeline.cpp:990-1005)
+    w.p_readout_contacts = {cfg.fixed_dt, E, nl, m.contact_slots, m.rows_per_env, m.contact_slots, m.contact_rows_per_env};
+    if (w.contact_readout_demanded && has_contacts && m.contact_slots > 0u) add(NkOp::ReadoutContactWrench, &w.p_readout_contacts);
 }
 
 void InvalidatePlan(World& w) {
@@ -816,12 +825,37 @@ nuka_state_field_t nuka_field_from_name(const char* name) {
     return 0xFFFFFFFFu;
 }
 
+namespace nkh {
+namespace {
+// nk::World::DemandReadout (src/nk/pipeline/world.cpp:905-975): the first request for a contact readout field waits
+// for the device, runs the readout once on the current solution and makes it part of every later step.
+nuka_result_t DemandReadout(World& w, const Field& f) {
+    static const char* const kContactReadout[] = {"contact_point", "contact_normal", "contact_force", "ucontact_impulse",
+        "link_contact_wrench", "contact_side_a_kind", "contact_side_b_kind", "contact_side_a_index", "contact_side_b_index", "contact_link"};
+    bool wanted = false;
+    for (const char* name : kContactReadout) wanted = wanted || std::strcmp(f.name, name) == 0;
+    if (!wanted || w.contact_readout_demanded || w.model.contact_slots == 0u) return NUKA_RESULT_OK;
+    if (w.be->synchronize(w.backend, nullptr) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "device error before the readout");
+    const nuka_phi_op_call call{uint16_t(NkOp::ReadoutContactWrench), &w.p_readout_contacts};
+    const uint8_t status = w.be->dispatch(w.backend, reinterpret_cast<const nuka_phi_model_view*>(&w.model),
+                                          reinterpret_cast<const nuka_phi_data_view*>(&w.data), &call);
+    if (status != uint8_t(Status::Ok)) return Error(MapStatus(status), "contact readout failed");
+    if (w.be->synchronize(w.backend, nullptr) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "device error in the readout");
+    w.contact_readout_demanded = true;
+    InvalidatePlan(w);
+    BuildPipeline(w);
+    return NUKA_RESULT_OK;
+}
+}  // namespace
+}  // namespace nkh
+
 nuka_result_t nuka_world_get_buffer_view(nuka_world_handle world, nuka_state_field_t field, nuka_buffer_view_t* out) {
     auto* w = reinterpret_cast<World*>(world);
     if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
     if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
     if (field >= w->fields.size()) return Error(NUKA_RESULT_NOT_SUPPORTED, "unknown field");
     const Field& f = w->fields[field];
+    if (const nuka_result_t demanded = DemandReadout(*w, f); demanded != NUKA_RESULT_OK) return demanded;
     out->device_ptr = static_cast<char*>(Iface(w->arena)->base(w->arena)) + f.offset;
     out->element_count = f.count;
     out->element_stride_bytes = f.elem_bytes;
@@ -848,6 +882,7 @@ nuka_result_t nuka_world_download_field(nuka_world_handle world, nuka_state_fiel
     const size_t size = f.count * f.elem_bytes;
     if (byte_offset > size || nbytes > size - byte_offset || (bytes == nullptr && nbytes > 0u)) return Error(NUKA_RESULT_INVALID_ARG, "range exceeds the field");
     if (nbytes == 0u) return NUKA_RESULT_OK;
+    if (const nuka_result_t demanded = DemandReadout(*w, f); demanded != NUKA_RESULT_OK) return demanded;
     return MapStatus(Iface(w->arena)->download(w->arena, bytes, f.offset + byte_offset, nbytes));
 }
 

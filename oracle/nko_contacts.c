@@ -663,3 +663,66 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
             for (uint32_t i = 0u; i < t->max_dof; ++i) { ja[i] += jb[i]; jb[i] = 0.0f; }
     }
 }
+
+/* ---- ReadoutContactWrench (ops/readout.cu:59-220, 559-626) ---------------
+ * Per slot: first manifold point and normal, the summed {normal, tangent, tangent} force, each point's world impulse
+ * (nk/contact/row_readout.hpp:17-48), the sides' owners, the contact's link.  Per link: the world wrench of the
+ * active rows ending on it, added by ascending row then side A before B (contact_index.cuh:85-110 key order). */
+void nko_env_readout_contact_wrench(nko_world* w, uint32_t env) {
+    const nko_template* t = &w->t;
+    const uint32_t S = t->slots, R = t->rows_per_env, nl = t->nl;
+    const float dt = w->cfg.fixed_dt, inv_dt = dt > 0.0f ? 1.0f / dt : 0.0f;
+    const nko_row* rows = (const nko_row*)w->urows;
+    for (uint32_t s = 0u; s < S; ++s) {
+        const size_t slot = (size_t)env * S + s;
+        const uint32_t points = w->ucontact_count[slot];
+        for (uint32_t k = 0u; k < 3u; ++k) {
+            w->contact_point[slot * 3u + k] = points > 0u ? w->ucontact_point[slot * 12u + k] : 0.0f;
+            w->contact_normal[slot * 3u + k] = points > 0u ? w->ucontact_normal[slot * 12u + k] : 0.0f;
+        }
+        const uint32_t first = w->ucontact_row_range[slot * 2u], pts = w->ucontact_row_range[slot * 2u + 1u];
+        float fn = 0.0f, ft1 = 0.0f, ft2 = 0.0f;
+        for (uint32_t i = 0u; i < pts; ++i) {
+            fn += w->lambda[first + i]; ft1 += w->lambda[first + i + pts]; ft2 += w->lambda[first + i + 2u * pts];
+        }
+        for (uint32_t i = 0u; i < 4u; ++i) {
+            v3 impulse = v3_make(0, 0, 0);
+            if (i < pts && (rows[first + i].flags & NKO_ROW_ACTIVE) != 0u)
+                for (uint32_t axis = 0u; axis < 3u; ++axis) {
+                    const uint32_t index = first + i + axis * pts;
+                    impulse = v3_add(impulse, v3_scale(rows[index].a.jlin, w->lambda[index]));
+                }
+            float* out = w->ucontact_impulse + (slot * 4u + i) * 3u;
+            out[0] = impulse.x; out[1] = impulse.y; out[2] = impulse.z;
+        }
+        w->contact_force[slot * 3u] = fn * inv_dt; w->contact_force[slot * 3u + 1u] = ft1 * inv_dt; w->contact_force[slot * 3u + 2u] = ft2 * inv_dt;
+        const int active = pts > 0u && (rows[first].flags & NKO_ROW_ACTIVE) != 0u;
+        const uint32_t kind_a = active ? rows[first].a.kind : NKO_SIDE_STATIC, kind_b = active ? rows[first].b.kind : NKO_SIDE_STATIC;
+        w->contact_side_a_kind[slot] = kind_a; w->contact_side_b_kind[slot] = kind_b;
+        w->contact_side_a_index[slot] = !active || kind_a == NKO_SIDE_STATIC ? NKO_INVALID : kind_a == NKO_SIDE_ARTIC ? w->row_cj_link[first] : rows[first].a.index;
+        w->contact_side_b_index[slot] = !active || kind_b == NKO_SIDE_STATIC ? NKO_INVALID : kind_b == NKO_SIDE_ARTIC ? w->row_cj_link_b[first] : rows[first].b.index;
+        uint32_t link = NKO_INVALID;
+        for (uint32_t i = 0u; i < pts && link == NKO_INVALID; ++i) link = w->row_cj_link[first + i];
+        for (uint32_t i = 0u; i < pts && link == NKO_INVALID; ++i) link = w->row_cj_link_b[first + i];
+        w->contact_link[slot] = link;
+    }
+    for (uint32_t l = 0u; l < nl; ++l) {
+        const uint32_t link = env * nl + l;
+        const v3 origin = v3_make(w->link_pose[(size_t)link * 7u], w->link_pose[(size_t)link * 7u + 1u], w->link_pose[(size_t)link * 7u + 2u]);
+        v3 force = v3_make(0, 0, 0), torque = v3_make(0, 0, 0);
+        for (uint32_t r = 0u; r < R; ++r) {
+            const size_t rs = (size_t)env * R + r;
+            if ((rows[rs].flags & NKO_ROW_ACTIVE) == 0u) continue;
+            for (uint32_t side = 0u; side < 2u; ++side) {
+                if ((side == 0u ? w->row_cj_link[rs] : w->row_cj_link_b[rs]) != link) continue;
+                const v3 dir = side == 0u ? rows[rs].a.jlin : rows[rs].b.jlin;
+                const float* point = (side == 0u ? w->row_cj_point : w->row_cj_point_b) + rs * 3u;
+                const v3 f = v3_scale(dir, w->lambda[rs] * inv_dt);
+                force = v3_add(force, f);
+                torque = v3_add(torque, v3_cross(v3_sub(v3_make(point[0], point[1], point[2]), origin), f));
+            }
+        }
+        float* out = w->link_contact_wrench + (size_t)link * 6u;
+        out[0] = force.x; out[1] = force.y; out[2] = force.z; out[3] = torque.x; out[4] = torque.y; out[5] = torque.z;
+    }
+}

@@ -111,6 +111,9 @@ struct nko_world {
     float *velocity_target, *actuator_noload_speed, *joint_f, *joint_gravity_force;
     float *drive_command, *drive_dissipation, *drive_lower, *drive_upper;
     float *joint_limit_impulse, *actuator_effort_requested, *actuator_effort, *actuator_saturated;
+    /* contact readout (ops/readout.cu ReadoutContactWrench) */
+    float *contact_point, *contact_normal, *contact_force, *ucontact_impulse, *link_contact_wrench;
+    uint32_t *contact_side_a_kind, *contact_side_b_kind, *contact_side_a_index, *contact_side_b_index, *contact_link;
     int fold_drive_damping;
 };
 
@@ -148,6 +151,7 @@ void nko_env_fk(const nko_world* w, uint32_t env);
 void nko_env_apply_drives(nko_world* w, uint32_t env);
 void nko_env_readout_drives(nko_world* w, uint32_t env);
 void nko_env_joint_rows(nko_world* w, uint32_t env);
+void nko_env_readout_contact_wrench(nko_world* w, uint32_t env);
 void nko_env_dynamics(nko_world* w, uint32_t env, uint32_t integrate_velocity);
 void nko_env_integrate_position(nko_world* w, uint32_t env);
 void nko_env_link_velocities(nko_world* w, uint32_t env);

@@ -212,6 +212,11 @@ nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc*
     w->drive_upper = ALLOC(float, E * nl); w->joint_limit_impulse = ALLOC(float, E * nl * 2u);
     w->actuator_effort_requested = ALLOC(float, E * nl); w->actuator_effort = ALLOC(float, E * nl);
     w->actuator_saturated = ALLOC(float, E * nl);
+    w->contact_point = ALLOC(float, E * S * 3u); w->contact_normal = ALLOC(float, E * S * 3u); w->contact_force = ALLOC(float, E * S * 3u);
+    w->ucontact_impulse = ALLOC(float, E * S * 12u); w->link_contact_wrench = ALLOC(float, E * nl * 6u);
+    w->contact_side_a_kind = ALLOC(uint32_t, E * S); w->contact_side_b_kind = ALLOC(uint32_t, E * S);
+    w->contact_side_a_index = ALLOC(uint32_t, E * S); w->contact_side_b_index = ALLOC(uint32_t, E * S);
+    w->contact_link = ALLOC(uint32_t, E * S);
     for (size_t i = 0u; i < E * R; ++i) { w->row_cj_link[i] = NKO_INVALID; w->row_cj_link_b[i] = NKO_INVALID; }
     for (size_t e = 0u; e < E; ++e) {
         const float id[7] = {0, 0, 0, 1, 0, 0, 0};
@@ -242,6 +247,9 @@ void nko_world_destroy(nko_world* w) {
     free(w->drive_joint_force_limit); free(w->velocity_target); free(w->actuator_noload_speed); free(w->joint_f);
     free(w->joint_gravity_force); free(w->drive_command); free(w->drive_dissipation); free(w->drive_lower); free(w->drive_upper);
     free(w->joint_limit_impulse); free(w->actuator_effort_requested); free(w->actuator_effort); free(w->actuator_saturated);
+    free(w->contact_point); free(w->contact_normal); free(w->contact_force); free(w->ucontact_impulse); free(w->link_contact_wrench);
+    free(w->contact_side_a_kind); free(w->contact_side_b_kind); free(w->contact_side_a_index); free(w->contact_side_b_index);
+    free(w->contact_link);
     free(w);
 }
 
@@ -272,7 +280,11 @@ void nko_world_destroy(nko_world* w) {
     X(actuator_noload_speed, float, E * nl) X(joint_f, float, E * nl) X(joint_gravity_force, float, E * nl) \
     X(drive_command, float, E * nl) X(drive_dissipation, float, E * nl) X(drive_lower, float, E * nl) \
     X(drive_upper, float, E * nl) X(joint_limit_impulse, float, E * nl * 2u) X(actuator_effort_requested, float, E * nl) \
-    X(actuator_effort, float, E * nl) X(actuator_saturated, float, E * nl)
+    X(actuator_effort, float, E * nl) X(actuator_saturated, float, E * nl) \
+    X(contact_point, float, E * S * 3u) X(contact_normal, float, E * S * 3u) X(contact_force, float, E * S * 3u) \
+    X(ucontact_impulse, float, E * S * 12u) X(link_contact_wrench, float, E * nl * 6u) \
+    X(contact_side_a_kind, uint32_t, E * S) X(contact_side_b_kind, uint32_t, E * S) X(contact_side_a_index, uint32_t, E * S) \
+    X(contact_side_b_index, uint32_t, E * S) X(contact_link, uint32_t, E * S)
 
 #define TEMPLATE_LIST(X) \
     X(link_inertia, float, nl * 36u) X(link_tree_depth, uint32_t, nl) X(link_child_range, uint32_t, nl * 2u) \
@@ -311,6 +323,7 @@ uint32_t nko_world_rows_per_env(const nko_world* w) { return w->t.rows_per_env; 
 void nko_fk_world_poses(nko_world* w) { FOR_ENVS(nko_env_fk(w, env)) }
 void nko_apply_drives(nko_world* w) { FOR_ENVS(nko_env_apply_drives(w, env)) }
 void nko_readout_drives(nko_world* w) { FOR_ENVS(nko_env_readout_drives(w, env)) }
+void nko_readout_contact_wrench(nko_world* w) { FOR_ENVS(nko_env_readout_contact_wrench(w, env)) }
 void nko_articulation_dynamics(nko_world* w, uint32_t integrate_velocity) { FOR_ENVS(nko_env_dynamics(w, env, integrate_velocity)) }
 void nko_sync_link_body_pose(nko_world* w) { FOR_ENVS(nko_env_sync_body_pose(w, env)) }
 void nko_build_aabbs(nko_world* w) { FOR_ENVS(nko_env_aabbs(w, env)) }

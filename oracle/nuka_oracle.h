@@ -127,6 +127,7 @@ void nko_assemble_rows(nko_world* w);
 void nko_contact_warm_start(nko_world* w, uint32_t phase);
 void nko_block_descent_solve(nko_world* w);
 void nko_readout_drives(nko_world* w);
+void nko_readout_contact_wrench(nko_world* w);   /* on demand; not part of nko_world_step */
 void nko_integrate_position(nko_world* w);
 void nko_fk_link_velocities(nko_world* w);
 /* The whole op list of one step, in the reference's order. */

@@ -162,3 +162,40 @@ def test_invalid_gains_and_modes(device):
     with pytest.raises(nk.NukaError) as err:
         nk.World(device, t, abi.world_desc(2, 0.005))
     assert err.value.code == abi.RESULT_INVALID_ARG
+
+
+READOUT_F32 = ("contact_point", "contact_normal", "contact_force", "ucontact_impulse", "link_contact_wrench")
+READOUT_U32 = ("contact_side_a_kind", "contact_side_b_kind", "contact_side_a_index", "contact_side_b_index", "contact_link")
+
+
+@pytest.mark.parametrize("index,E", [(2, 256), (3, 256)])
+def test_contact_readout_matches_the_oracle_and_joins_the_step_on_demand(oracle_py, device, index, E):
+    """ReadoutContactWrench: not part of the step until a consumer asks for one of its fields; the first request runs
+    it on the current solution, and from then on every step ends with it (nk/pipeline/world.cpp:905-975)."""
+    cfg = nk.synthetic.config(index, E)
+    desc = abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters)
+    oracle = oracle_py.OracleWorld(cfg.template, desc, threads=8)
+    world = nk.World(device, cfg.template, desc)
+    for w in (oracle, world):
+        w.set_state(cfg.state())
+    ops_before = world.info.op_count
+    world.step(); world.synchronize()
+    oracle.step(); oracle.op("readout_contact_wrench")
+    for name in READOUT_U32:                       # the first download demands the readout
+        assert np.array_equal(world.download(name), oracle.download(name)), name
+    for name in READOUT_F32[:2]:
+        assert relative_error(world.download(name), oracle.download(name)) <= TOL, name
+    # the generalized impulse is the well-determined quantity (see test_gpu_parity): per-slot forces of the humanoid's
+    # redundant foot spheres inherit the indeterminacy of the individual multipliers, the per-link wrench does not
+    assert relative_error(world.download("link_contact_wrench"), oracle.download("link_contact_wrench")) <= (TOL if index == 2 else 5 * TOL)
+    if index == 2:
+        for name in ("contact_force", "ucontact_impulse"):
+            assert relative_error(world.download(name), oracle.download(name)) <= TOL, name
+    info = nk.WorldInfoC()
+    nk._check(nk.lib().nuka_world_get_info(world._h, __import__("ctypes").byref(info)))
+    assert info.op_count == ops_before + 1
+    world.step(); world.synchronize()              # now the step itself refreshes the readout
+    oracle.step(); oracle.op("readout_contact_wrench")
+    assert np.array_equal(world.download("contact_link"), oracle.download("contact_link"))
+    assert relative_error(world.download("link_contact_wrench"), oracle.download("link_contact_wrench")) <= 10 * TOL
+    world.close(); oracle.close()
