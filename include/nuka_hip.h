@@ -111,6 +111,39 @@ typedef struct nuka_world_desc_t {
                                               struct_size covers it */
 } nuka_world_desc_t;
 
+/* Scene files (src/import/mjcf_importer.cpp LoadMjcf, then the articulation part of the cook): a MuJoCo XML robot
+ * description read into the cook inputs of one environment.  One articulation per file; bodies, default classes,
+ * hinge / slide / free joints (several per body), inertial elements or geom-derived mass, sphere / box / plane
+ * collision geoms, joint ranges, damping, armature, frictionloss, springs, and position / velocity / motor actuators.
+ * Joint and contact rows use this library's native laws (no solref / solimp compliance). */
+typedef struct nuka_scene_t* nuka_scene_handle;
+/* Keep sphere and box geoms against planes only: other colliding geoms are dropped and counted, and the robot's geoms
+ * share one negative collision group, so that they meet the ground and not each other. */
+#define NUKA_SCENE_PLANE_CONTACTS_ONLY 1u
+nuka_result_t nuka_scene_load_mjcf(const char* path, uint32_t flags, nuka_scene_handle* out);
+void nuka_scene_destroy(nuka_scene_handle scene);
+/* The cook inputs; the arrays live as long as the scene. */
+const nuka_template_desc_t* nuka_scene_template(nuka_scene_handle scene);
+typedef struct nuka_scene_info_t {
+    uint32_t link_count, body_count, actuator_count, dropped_geom_count, floating_root, drive_mode;
+    float timestep;
+    float gravity[3];
+} nuka_scene_info_t;
+nuka_result_t nuka_scene_get_info(nuka_scene_handle scene, nuka_scene_info_t* out);
+/* The MJCF body behind a link ("<body>_anchor" for the static anchor of a jointed root, "<body>/<joint>" for the
+ * massless links between several joints of one body) and the joint that moves it ("" for a welded body). */
+const char* nuka_scene_link_name(nuka_scene_handle scene, uint32_t link);
+const char* nuka_scene_joint_name(nuka_scene_handle scene, uint32_t link);
+/* What the file authors beyond the template, per link: initial coordinate, drive stiffness / damping / force limit from
+ * its actuators and the joint's actuator force range; base_pose[7] of a floating root.  Null outputs are skipped. */
+nuka_result_t nuka_scene_initial_state(nuka_scene_handle scene, float* q, float* base_pose, float* drive_stiffness,
+                                       float* drive_damping, float* drive_force_limit, float* drive_joint_force_limit);
+/* nuka.h:175 nuka_world_create_from_scene: the scene's template in every environment, its initial state and drive
+ * parameters uploaded (PD targets hold the initial pose), and that state kept as what nuka_world_reset returns to.
+ * `desc->fixed_dt` of 0 takes the file's timestep; gravity of all zeros takes the file's. */
+nuka_result_t nuka_world_create_from_scene(nuka_device_handle device, nuka_scene_handle scene, const nuka_world_desc_t* desc,
+                                           nuka_world_handle* out);
+
 /* nuka.h:175 nuka_world_create_from_scene */
 nuka_result_t nuka_world_create_from_template(nuka_device_handle device, const nuka_template_desc_t* tmpl,
                                               const nuka_world_desc_t* desc, nuka_world_handle* out);

@@ -30,6 +30,14 @@ class WorldInfoC(C.Structure):
                                           "contact_slots_per_env", "rows_per_env", "op_count")]
 
 
+class SceneInfoC(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("link_count", "body_count", "actuator_count", "dropped_geom_count", "floating_root",
+                                          "drive_mode")] + [("timestep", C.c_float), ("gravity", C.c_float * 3)]
+
+
+SCENE_PLANE_CONTACTS_ONLY = 1
+
+
 class DeviceDescC(C.Structure):
     _fields_ = [("gpu_index", C.c_uint32), ("stream", C.c_void_p), ("backend_selection_layer_enabled", C.c_uint8)]
 
@@ -43,6 +51,8 @@ EXPORTS = [
     "nuka_world_get_buffer_view", "nuka_world_upload_field", "nuka_world_download_field", "nuka_world_get_info",
     "nuka_world_time_steps", "nuka_world_profile_ops", "nuka_device_copy_bandwidth", "nuka_hip_register_backend_entry",
     "nuka_hip_op_count", "nuka_hip_op_name", "nuka_hip_op_from_name",
+    "nuka_scene_load_mjcf", "nuka_scene_destroy", "nuka_scene_template", "nuka_scene_get_info", "nuka_scene_link_name",
+    "nuka_scene_joint_name", "nuka_scene_initial_state", "nuka_world_create_from_scene",
 ]
 
 
@@ -97,6 +107,17 @@ def lib():
         L.nuka_checkpoint_destroy.argtypes = [C.c_void_p]
         L.nuka_checkpoint_byte_size.argtypes = [C.c_void_p, C.POINTER(C.c_uint64)]
         L.nuka_device_copy_bandwidth.argtypes = [C.c_void_p, C.c_size_t, C.c_uint32, C.POINTER(C.c_float)]
+        L.nuka_scene_load_mjcf.argtypes = [C.c_char_p, C.c_uint32, C.POINTER(C.c_void_p)]
+        L.nuka_scene_destroy.argtypes = [C.c_void_p]
+        L.nuka_scene_template.argtypes = [C.c_void_p]
+        L.nuka_scene_template.restype = C.POINTER(TemplateDescC)
+        L.nuka_scene_get_info.argtypes = [C.c_void_p, C.POINTER(SceneInfoC)]
+        L.nuka_scene_link_name.argtypes = [C.c_void_p, C.c_uint32]
+        L.nuka_scene_link_name.restype = C.c_char_p
+        L.nuka_scene_joint_name.argtypes = [C.c_void_p, C.c_uint32]
+        L.nuka_scene_joint_name.restype = C.c_char_p
+        L.nuka_scene_initial_state.argtypes = [C.c_void_p] + [C.c_void_p] * 6
+        L.nuka_world_create_from_scene.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]
         _lib = L
     return _lib
 
@@ -125,15 +146,65 @@ class Device:
         return out.value
 
 
+class Scene:
+    """A robot description file read into the cook inputs of one environment (nuka_scene_*; host code, no GPU)."""
+
+    def __init__(self, path, flags=0):
+        self._h = C.c_void_p()
+        _check(lib().nuka_scene_load_mjcf(os.fsencode(path), flags, C.byref(self._h)))
+        info = SceneInfoC()
+        _check(lib().nuka_scene_get_info(self._h, C.byref(info)))
+        self.info = info
+        self.link_count = info.link_count
+        self.link_names = [lib().nuka_scene_link_name(self._h, l).decode() for l in range(info.link_count)]
+        self.joint_names = [lib().nuka_scene_joint_name(self._h, l).decode() for l in range(info.link_count)]
+
+    def close(self):
+        if self._h:
+            lib().nuka_scene_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        self.close()
+
+    def to_c(self):
+        """(TemplateDescC, keepalive), as abi.Template.to_c(): the arrays belong to the scene."""
+        return lib().nuka_scene_template(self._h).contents, self
+
+    def template_arrays(self):
+        """The template description as numpy copies, keyed like abi.Template.arrays()."""
+        d = lib().nuka_scene_template(self._h).contents
+        nl, nb, npf = d.link_count, d.body_count, d.profile_count
+        shapes = dict(joint_type=nl, parent_link=nl, joint_axis=3 * nl, link_local_pose=7 * nl, link_inertial_frame=7 * nl, link_mass=nl,
+                      link_diag_inertia=3 * nl, joint_damping=nl, joint_armature=nl, joint_stiffness=nl, joint_spring_reference=nl,
+                      body_role=nb, body_link=nb, body_local=7 * nb, shape_kind=nb, shape_params=4 * nb, shape_contype=nb,
+                      shape_conaffinity=nb, shape_group=nb, shape_profile=nb, profile_mu=2 * npf, joint_limit_lower=nl,
+                      joint_limit_upper=nl, joint_limit_flags=nl, joint_frictionloss=nl)
+        out = {name: np.ctypeslib.as_array(getattr(d, name), shape=(count,)).copy() if count else np.zeros(0, np.float32)
+               for name, count in shapes.items()}
+        out.update(drive_mode=d.drive_mode, drive_rows=d.drive_rows)
+        return out
+
+    def initial_state(self):
+        nl = self.link_count
+        names = ("q", "base_pose", "drive_stiffness", "drive_damping", "drive_force_limit", "drive_joint_force_limit")
+        out = {n: np.zeros(7 if n == "base_pose" else nl, np.float32) for n in names}
+        _check(lib().nuka_scene_initial_state(self._h, *[out[n].ctypes.data for n in names]))
+        return out
+
+
 class World:
     """One cooked template stepped over `env_count` environments on the GPU (nuka_world_*)."""
 
     def __init__(self, device, template, desc):
         self.device = device
-        tdesc, keep = template.to_c()
         self._h = C.c_void_p()
-        _check(lib().nuka_world_create_from_template(device._h, C.byref(tdesc), C.byref(desc), C.byref(self._h)))
-        del keep
+        if isinstance(template, Scene):
+            _check(lib().nuka_world_create_from_scene(device._h, template._h, C.byref(desc), C.byref(self._h)))
+        else:
+            tdesc, keep = template.to_c()
+            _check(lib().nuka_world_create_from_template(device._h, C.byref(tdesc), C.byref(desc), C.byref(self._h)))
+            del keep
         info = WorldInfoC()
         _check(lib().nuka_world_get_info(self._h, C.byref(info)))
         self.info = info

@@ -1,0 +1,40 @@
+// The MJCF template loader's result: the arrays behind a nuka_template_desc_t plus what else the file authors
+// for the articulation-step path (names, initial state, drive parameters).  Host code only.
+#pragma once
+
+#include <array>
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "../../include/nuka_hip.h"
+
+namespace nkh {
+namespace mjcf {
+
+// Keep sphere and box geoms against planes only: other colliding geoms are dropped (and counted), and the robot's
+// geoms share one negative collision group so that they meet the ground and not each other.
+constexpr uint32_t kPlaneContactsOnly = 1u;
+
+struct Scene {
+    nuka_template_desc_t desc{};
+    std::vector<std::string> link_names, joint_names;
+    std::vector<uint8_t> joint_type, joint_limit_flags;
+    std::vector<uint32_t> parent_link, body_role, body_link, shape_kind, shape_contype, shape_conaffinity, shape_group, shape_profile;
+    std::vector<float> joint_axis, link_local_pose, link_inertial_frame, link_mass, link_diag_inertia, joint_damping, joint_armature,
+        joint_stiffness, joint_spring_reference, joint_frictionloss, joint_limit_lower, joint_limit_upper, body_local, shape_params, profile_mu;
+    std::vector<float> initial_q, drive_stiffness, drive_damping, drive_force_limit, drive_joint_force_limit;
+    std::array<float, 7> base_pose{0, 0, 0, 1, 0, 0, 0};
+    bool floating_root = false;
+    uint32_t actuator_count = 0u, dropped_geom_count = 0u, drive_mode = 1u;
+    float timestep = 0.002f;
+    float gravity[3] = {0.0f, 0.0f, -9.81f};
+    void Bind();   // points `desc` at the arrays
+};
+
+// Throws std::runtime_error with the reason when the file cannot be read or uses what this path does not build.
+std::unique_ptr<Scene> LoadMjcf(const std::string& path, uint32_t flags);
+
+}  // namespace mjcf
+}  // namespace nkh

@@ -1165,24 +1165,21 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     }
     __syncthreads();
     // CopyTileRows (:836-869): the staged heads' rows, their loads in flight together
-#pragma unroll 2
+
     for (uint32_t h = 0u; h < heads; ++h) {
         const uint32_t first = c.U(hRow, h);
-        if (first == kInvalid) {
-            if (lane == 0u) { c.U(hColumnsLow, h) = 0u; c.U(hColumnsHigh, h) = 0u; }
-            continue;
-        }
+        const bool staged = first != kInvalid;   // a unit head stages nothing and touches no column block
         float value[3];
 #pragma unroll
         for (uint32_t axis = 0u; axis < 3u; ++axis) {
             const uint32_t source_a = c.U(hSourceA + axis, h), source_b = c.U(hSourceB + axis, h);
             value[axis] = 0.0f;
-            if (coordinate && source_a != kInvalid) value[axis] += d.chain_jacobian[size_t{source_a} * md + lane];
-            if (coordinate && source_b != kInvalid) value[axis] += d.chain_jacobian_b[size_t{source_b} * md + lane];
+            if (staged && coordinate && source_a != kInvalid) value[axis] += d.chain_jacobian[size_t{source_a} * md + lane];
+            if (staged && coordinate && source_b != kInvalid) value[axis] += d.chain_jacobian_b[size_t{source_b} * md + lane];
         }
 #pragma unroll
         for (uint32_t axis = 0u; axis < 3u; ++axis)
-            if (lane < c.ldj) c.jac[(first + axis) * c.ldj + lane] = value[axis];   // padded columns hold zeros
+            if (staged && lane < c.ldj) c.jac[(first + axis) * c.ldj + lane] = value[axis];   // padded columns hold zeros
         // the columns this head touches at all: a contact on one limb leaves most coordinates out, and the Hessian
         // update skips their exact-zero products four columns at a time
         const uint64_t columns = __ballot(value[0] != 0.0f || value[1] != 0.0f || value[2] != 0.0f);

@@ -16,6 +16,7 @@
 
 #include "../../include/nuka_hip.h"
 #include "backend.h"
+#include "mjcf_loader.h"
 #include "nk_types.h"
 
 namespace nkh {
@@ -593,8 +594,10 @@ nuka_phi_backend* nuka_device_backend(nuka_device_handle device) {
     return record != nullptr ? reinterpret_cast<nuka_phi_backend*>(record->backend) : nullptr;
 }
 
-nuka_result_t nuka_world_create_from_template(nuka_device_handle device, const nuka_template_desc_t* tmpl,
-                                              const nuka_world_desc_t* desc, nuka_world_handle* out) {
+namespace nkh {
+namespace {
+nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t* tmpl, const nuka_world_desc_t* desc,
+                          const mjcf::Scene* scene, nuka_world_handle* out) {
     if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
     *out = nullptr;
     if (device == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "device is null");
@@ -678,6 +681,24 @@ nuka_result_t nuka_world_create_from_template(nuka_device_handle device, const n
                 !put(w.data.body_pose, body_pose.data(), body_pose.size() * 4u) || !put(w.data.row_cj_link, invalid.data(), invalid.size() * 4u) ||
                 !put(w.data.row_cj_link_b, invalid.data(), invalid.size() * 4u)) return Error(NUKA_RESULT_DEVICE_ERROR, "initial state upload failed");
         }
+        if (scene != nullptr) {   // the state and drive parameters the scene file authors, in every environment
+            auto tile = [&](const std::vector<float>& per_link) {
+                std::vector<float> all(E * nl);
+                for (size_t e = 0u; e < E; ++e) std::copy(per_link.begin(), per_link.end(), all.begin() + e * nl);
+                return all;
+            };
+            auto put = [&](void* field, const std::vector<float>& values) {
+                return Iface(w.arena)->upload(w.arena, values.data(), size_t(static_cast<char*>(field) - base), values.size() * 4u) == uint8_t(Status::Ok);
+            };
+            std::vector<float> base_pose(E * 7u);
+            for (size_t e = 0u; e < E; ++e) std::copy(scene->base_pose.begin(), scene->base_pose.end(), base_pose.begin() + e * 7u);
+            bool ok = put(w.data.q, tile(scene->initial_q)) && put(w.data.drive_stiffness, tile(scene->drive_stiffness)) &&
+                      put(w.data.drive_damping, tile(scene->drive_damping)) && put(w.data.drive_force_limit, tile(scene->drive_force_limit)) &&
+                      put(w.data.drive_joint_force_limit, tile(scene->drive_joint_force_limit));
+            if (hc.floating_root != 0u) ok = ok && put(w.data.base_pose, base_pose);
+            if (hc.drive_mode == kDrivePdPosition) ok = ok && put(w.data.drive_target, tile(scene->initial_q));   // hold the authored pose
+            if (!ok) return Error(NUKA_RESULT_DEVICE_ERROR, "scene state upload failed");
+        }
         if (Iface(w.initial)->copy_from(w.initial, w.arena, 0u, 0u, w.arena_bytes) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "snapshot failed");
         BuildPipeline(w);
         if (w.be->synchronize(w.backend, nullptr) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "device error during world creation");
@@ -692,6 +713,80 @@ nuka_result_t nuka_world_create_from_template(nuka_device_handle device, const n
     } catch (const std::exception& e) {
         return Error(NUKA_RESULT_INTERNAL, e.what());
     }
+}
+}  // namespace
+}  // namespace nkh
+
+nuka_result_t nuka_world_create_from_template(nuka_device_handle device, const nuka_template_desc_t* tmpl,
+                                              const nuka_world_desc_t* desc, nuka_world_handle* out) {
+    return CreateWorld(device, tmpl, desc, nullptr, out);
+}
+
+nuka_result_t nuka_scene_load_mjcf(const char* path, uint32_t flags, nuka_scene_handle* out) {
+    if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    *out = nullptr;
+    if (path == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "path is null");
+    if ((flags & ~uint32_t(NUKA_SCENE_PLANE_CONTACTS_ONLY)) != 0u) return Error(NUKA_RESULT_INVALID_ARG, "unknown scene flag");
+    try {
+        *out = reinterpret_cast<nuka_scene_handle>(mjcf::LoadMjcf(path, flags).release());
+        return NUKA_RESULT_OK;
+    } catch (const std::bad_alloc&) {
+        return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
+    } catch (const std::exception& e) {
+        return Error(NUKA_RESULT_INVALID_ARG, e.what());
+    }
+}
+
+void nuka_scene_destroy(nuka_scene_handle scene) { delete reinterpret_cast<mjcf::Scene*>(scene); }
+
+const nuka_template_desc_t* nuka_scene_template(nuka_scene_handle scene) {
+    return scene != nullptr ? &reinterpret_cast<mjcf::Scene*>(scene)->desc : nullptr;
+}
+
+nuka_result_t nuka_scene_get_info(nuka_scene_handle scene, nuka_scene_info_t* out) {
+    const auto* s = reinterpret_cast<const mjcf::Scene*>(scene);
+    if (s == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "scene is null");
+    if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    *out = {s->desc.link_count, s->desc.body_count, s->actuator_count, s->dropped_geom_count, s->floating_root ? 1u : 0u, s->drive_mode,
+            s->timestep, {s->gravity[0], s->gravity[1], s->gravity[2]}};
+    return NUKA_RESULT_OK;
+}
+
+const char* nuka_scene_link_name(nuka_scene_handle scene, uint32_t link) {
+    const auto* s = reinterpret_cast<const mjcf::Scene*>(scene);
+    return s != nullptr && link < s->link_names.size() ? s->link_names[link].c_str() : nullptr;
+}
+
+const char* nuka_scene_joint_name(nuka_scene_handle scene, uint32_t link) {
+    const auto* s = reinterpret_cast<const mjcf::Scene*>(scene);
+    return s != nullptr && link < s->joint_names.size() ? s->joint_names[link].c_str() : nullptr;
+}
+
+nuka_result_t nuka_scene_initial_state(nuka_scene_handle scene, float* q, float* base_pose, float* drive_stiffness, float* drive_damping,
+                                       float* drive_force_limit, float* drive_joint_force_limit) {
+    const auto* s = reinterpret_cast<const mjcf::Scene*>(scene);
+    if (s == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "scene is null");
+    auto copy = [](float* out, const std::vector<float>& values) { if (out != nullptr) std::copy(values.begin(), values.end(), out); };
+    copy(q, s->initial_q);
+    copy(drive_stiffness, s->drive_stiffness);
+    copy(drive_damping, s->drive_damping);
+    copy(drive_force_limit, s->drive_force_limit);
+    copy(drive_joint_force_limit, s->drive_joint_force_limit);
+    if (base_pose != nullptr) std::copy(s->base_pose.begin(), s->base_pose.end(), base_pose);
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_create_from_scene(nuka_device_handle device, nuka_scene_handle scene, const nuka_world_desc_t* desc,
+                                           nuka_world_handle* out) {
+    const auto* s = reinterpret_cast<const mjcf::Scene*>(scene);
+    if (s == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "scene is null");
+    if (desc == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "desc is null");
+    if (desc->struct_size != sizeof(nuka_world_desc_t)) return Error(NUKA_RESULT_INVALID_ARG, "struct_size mismatch");
+    nuka_world_desc_t with_file = *desc;
+    if (with_file.fixed_dt <= 0.0f) with_file.fixed_dt = s->timestep;
+    if (with_file.gravity[0] == 0.0f && with_file.gravity[1] == 0.0f && with_file.gravity[2] == 0.0f)
+        std::copy(s->gravity, s->gravity + 3, with_file.gravity);
+    return CreateWorld(device, &s->desc, &with_file, s, out);
 }
 
 void nuka_world_destroy(nuka_world_handle world) {

@@ -1,0 +1,215 @@
+"""The MJCF template loader (host code, no GPU): the expectations the reference's own importer tests assert on its
+fixtures (tests/golden/mjcf), and MuJoCo's kinematic conventions checked independently on a small biped - body
+frames composed straight from the XML with ElementTree, hinges turning about their anchors - against the oracle's
+forward kinematics run on the loaded template."""
+import os
+import xml.etree.ElementTree as ET
+
+import numpy as np
+import pytest
+
+from conftest import ROOT, nk
+
+abi = nk.abi
+GOLDEN = os.path.join(ROOT, "tests", "golden", "mjcf")
+BIPED = os.path.join(ROOT, "tests", "data", "biped.xml")
+
+
+def quat_mul(a, b):
+    return np.array([a[0] * b[0] - a[1] * b[1] - a[2] * b[2] - a[3] * b[3], a[0] * b[1] + a[1] * b[0] + a[2] * b[3] - a[3] * b[2],
+                     a[0] * b[2] - a[1] * b[3] + a[2] * b[0] + a[3] * b[1], a[0] * b[3] + a[1] * b[2] - a[2] * b[1] + a[3] * b[0]])
+
+
+def rotate(q, v):
+    u = np.asarray(q[1:], float)
+    t = 2.0 * np.cross(u, v)
+    return np.asarray(v, float) + q[0] * t + np.cross(u, t)
+
+
+def test_minimal_arm_bodies_joint_and_shapes():      # test_mjcf_importer.cpp:8-57
+    s = nk.Scene(os.path.join(GOLDEN, "minimal_arm.xml"))
+    a = s.template_arrays()
+    assert s.link_names == ["base", "link1"] and s.joint_names == ["", "joint0"]
+    assert list(a["joint_type"]) == [abi.JOINT_FIXED, abi.JOINT_REVOLUTE]       # a jointless root body is static
+    assert list(a["link_mass"]) == [1.0, 0.5]
+    assert list(a["shape_kind"]) == [abi.SHAPE_BOX, abi.SHAPE_CAPSULE]
+    assert np.allclose(a["link_local_pose"].reshape(2, 7)[1], [0, 0, 0.5, 1, 0, 0, 0])
+    assert np.allclose(a["link_inertial_frame"].reshape(2, 7)[1, :3], [0, 0, 0.25])
+    assert np.allclose(a["shape_params"].reshape(2, 4)[1, :2], [0.05, 0.25])     # capsule radius, half height from fromto
+
+
+def test_joint_dynamics_respect_defaults_and_overrides():      # test_mjcf_importer.cpp:59-77
+    s = nk.Scene(os.path.join(GOLDEN, "mjcf_joint_dynamics.xml"))
+    a = s.template_arrays()
+    expected = np.array([[0.3, 0.01, 0.075], [10.0, 0.2, 0.4], [100.0, 1.0, 1.0], [0.0, 0.0, 0.0], [4.0, 0.2, 0.4]], np.float32)
+    assert s.joint_names[1:] == ["root_defaults", "class_defaults", "explicit_values", "explicit_zero", "partial_override"]
+    got = np.stack([a["joint_damping"], a["joint_armature"], a["joint_frictionloss"]], 1)[1:]
+    assert np.array_equal(got, expected)
+
+
+def test_geometry_defaults_and_fromto_preserve_endpoints():      # test_mjcf_importer.cpp:106-131
+    s = nk.Scene(os.path.join(GOLDEN, "mjcf_geom_frames.xml"))
+    a = s.template_arrays()
+    assert list(a["joint_type"]) == [abi.JOINT_FLOATING]
+    local, params = a["body_local"].reshape(-1, 7), a["shape_params"].reshape(-1, 4)
+    ends = lambda row, z: local[row, :3] + rotate(local[row, 3:], [0, 0, z])
+    assert params[0, 0] == np.float32(0.01) and params[0, 1] == pytest.approx(0.2)
+    assert np.allclose(ends(0, -params[0, 1]), [-0.2, 0, 0.1], atol=1e-7) and np.allclose(ends(0, params[0, 1]), [0.2, 0, 0.1], atol=1e-7)
+    assert params[1, 0] == np.float32(0.02) and params[1, 1] == np.float32(0.15)
+    assert np.allclose(ends(1, 0.15), [0.15, 0.3, 0.0], atol=1e-7)            # euler="0 90 0" in degrees
+    assert params[2, 0] == np.float32(0.03) and params[2, 1] == pytest.approx(0.25)
+    assert np.allclose(ends(2, -0.25), [0, 0, 0], atol=1e-7) and np.allclose(ends(2, 0.25), [0, 0.3, 0.4], atol=1e-7)
+
+
+def test_inertial_sources():      # test_mjcf_mass_pipeline.cpp:27-60
+    s = nk.Scene(os.path.join(GOLDEN, "mjcf_inertial_sources.xml"))
+    a = s.template_arrays()
+    assert s.link_names == ["empty_wrapper", "explicit_inertial", "geom_only"]
+    mass, inertia = a["link_mass"], a["link_diag_inertia"].reshape(3, 3)
+    assert mass[0] == 0.0 and not inertia[0].any()
+    assert mass[1] == 2.5 and np.array_equal(inertia[1], np.array([0.1, 0.2, 0.3], np.float32))
+    assert mass[2] == pytest.approx(24.0, abs=1e-5)
+    box = 24.0 / 3.0 * np.array([0.2 ** 2 + 0.3 ** 2, 0.1 ** 2 + 0.3 ** 2, 0.1 ** 2 + 0.2 ** 2])
+    frame = a["link_inertial_frame"].reshape(3, 7)[2]
+    # the principal moments come back in the order the diagonalisation leaves them, with the rotation that undoes it
+    R = np.stack([rotate(frame[3:], e) for e in np.eye(3)], 1)
+    assert np.allclose(R @ np.diag(inertia[2]) @ R.T, np.diag(box), atol=1e-5)
+
+
+def test_rotated_slider_types_axes_and_motors():
+    s = nk.Scene(os.path.join(GOLDEN, "rotated_slider.xml"))
+    a = s.template_arrays()
+    assert s.link_names == ["base", "arm", "slider"] and s.joint_names == ["", "hinge", "slide"]
+    assert list(a["joint_type"]) == [abi.JOINT_FIXED, abi.JOINT_REVOLUTE, abi.JOINT_PRISMATIC]
+    assert np.allclose(a["link_local_pose"].reshape(3, 7)[2], [0.3, 0, 0, 0.70710678, 0, 0, 0.70710678])
+    assert s.info.actuator_count == 2 and s.info.drive_mode == abi.DRIVE_TORQUE
+    assert list(s.initial_state()["drive_force_limit"]) == [0.0, 100.0, 100.0]
+    assert s.info.timestep == np.float32(0.0001) and list(s.info.gravity) == [0.0, 0.0, 0.0]
+    assert not (a["shape_contype"].any() or a["shape_conaffinity"].any()) or s.info.body_count == 3   # geoms with contype 0 carry no collidable rows
+
+
+# ---- the biped: MuJoCo's conventions, checked independently ----------------------------------------------------
+def xml_body_frames(path):
+    """World frames of every <body> at q = 0, composed from pos / quat as MuJoCo does (mj_kinematics)."""
+    root = ET.parse(path).getroot()
+    frames = {}
+
+    def walk(element, position, rotation):
+        for body in element.findall("body"):
+            p = np.array([float(x) for x in body.get("pos", "0 0 0").split()])
+            q = np.array([float(x) for x in body.get("quat", "1 0 0 0").split()])
+            q = q / np.linalg.norm(q)
+            world_p, world_q = position + rotate(rotation, p), quat_mul(rotation, q)
+            frames[body.get("name")] = (world_p, world_q, body)
+            walk(body, world_p, world_q)
+
+    walk(root.find("worldbody"), np.zeros(3), np.array([1.0, 0, 0, 0]))
+    return frames
+
+
+def oracle_fk(oracle_py, scene, q=None):
+    state = scene.initial_state()
+    w = oracle_py.OracleWorld(scene, abi.world_desc(1, 0.005), threads=1)
+    w.upload("q", state["q"] if q is None else q)
+    w.upload("base_pose", state["base_pose"])
+    w.op("fk_world_poses")
+    pose = w.download("link_pose").reshape(-1, 7)
+    w.close()
+    return pose
+
+
+def test_biped_link_frames_sit_on_the_joint_anchors(oracle_py):
+    scene = nk.Scene(BIPED)
+    frames = xml_body_frames(BIPED)
+    pose = oracle_fk(oracle_py, scene)
+    for l, name in enumerate(scene.link_names):
+        body_name = name.split("/")[0]
+        world_p, world_q, body = frames[body_name]
+        joints = body.findall("joint")
+        if "/" in name:                       # the massless link of a body's earlier joint sits on that joint's anchor
+            anchor = next(j for j in joints if j.get("name") == name.split("/")[1]).get("pos")
+        else:                                 # the body's own link sits on its last hinge's anchor
+            anchor = joints[-1].get("pos", "0 0 0") if joints else "0 0 0"
+        anchor = np.array([float(x) for x in anchor.split()])
+        assert np.allclose(pose[l, :3], world_p + rotate(world_q, anchor), atol=2e-6), name
+        assert np.allclose(np.abs(pose[l, 3:] @ world_q), 1.0, atol=1e-6), name
+
+
+def test_biped_hinges_turn_about_their_anchors(oracle_py):
+    scene = nk.Scene(BIPED)
+    frames = xml_body_frames(BIPED)
+    rest = oracle_fk(oracle_py, scene)
+    knee = scene.joint_names.index("l_knee")
+    foot = scene.link_names.index("l_foot")
+    angle = 0.7
+    q = np.zeros(scene.link_count, np.float32)
+    q[knee] = angle
+    turned = oracle_fk(oracle_py, scene, q)
+    shin_p, shin_q, shin = frames["l_shin"]
+    anchor = shin_p + rotate(shin_q, [0.01, 0, 0.01])
+    axis = rotate(shin_q, [0, 1, 0])
+    rot = np.concatenate([[np.cos(angle / 2)], np.sin(angle / 2) * axis])
+    for link in (knee, foot):                 # every point of the shin and the foot swings about the knee's anchor line
+        assert np.allclose(turned[link, :3], anchor + rotate(rot, rest[link, :3] - anchor), atol=2e-6)
+    assert np.allclose(turned[: knee], rest[: knee], atol=1e-7)      # nothing above the knee moves
+
+
+def test_biped_masses_limits_profiles_and_drives():
+    scene = nk.Scene(BIPED)
+    a, state = scene.template_arrays(), scene.initial_state()
+    assert a["link_mass"].sum() == pytest.approx(6 + 2 * (1.5 + 0.3 + 800 * 8 * 0.02 * 0.02 * 0.11), rel=1e-6)
+    assert scene.info.floating_root == 1 and scene.info.actuator_count == 6 and scene.info.drive_mode == abi.DRIVE_PD_POSITION
+    names = scene.joint_names
+    knee, hip_x = names.index("l_knee"), names.index("r_hip_x")
+    assert (a["joint_limit_lower"][knee], a["joint_limit_upper"][knee], a["joint_limit_flags"][knee]) == (0.0, np.float32(2.2), 3)
+    assert (a["joint_limit_lower"][hip_x], a["joint_limit_upper"][hip_x]) == (np.float32(-0.5), np.float32(0.5))
+    assert a["joint_damping"][knee] == np.float32(0.6) and a["joint_frictionloss"][knee] == np.float32(0.05) and a["joint_armature"][knee] == np.float32(0.02)
+    assert a["joint_stiffness"][knee] == 1.5 and a["joint_spring_reference"][knee] == np.float32(0.3)
+    assert state["drive_stiffness"][knee] == 80.0 and state["drive_damping"][knee] == 3.0
+    assert state["drive_force_limit"][knee] == 25.0 and state["drive_force_limit"][names.index("r_knee")] == 90.0 and state["drive_force_limit"][hip_x] == 40.0
+    assert np.allclose(state["base_pose"], [0, 0, 0.62, 0.9987503, 0, 0.0499792, 0], atol=1e-6)
+    # collidable rows: the floor, one body row a link (its first colliding geom, if any), further geoms as extra rows
+    assert list(a["body_role"]) == [0, 1, 1, 1, 1, 1, 2, 1, 1, 1, 1, 2]
+    assert list(a["shape_kind"][[0, 1, 5, 6]]) == [abi.SHAPE_PLANE, abi.SHAPE_BOX, abi.SHAPE_SPHERE, abi.SHAPE_SPHERE]
+    assert list(a["profile_mu"]) == [np.float32(0.9)] * 2 + [np.float32(0.6)] * 2 and list(a["shape_profile"][[5, 6]]) == [0, 1]
+    # a full inertia tensor is diagonalised: R diag(principal) R^T gives the authored tensor back
+    thigh = scene.link_names.index("l_thigh")
+    frame, principal = a["link_inertial_frame"].reshape(-1, 7)[thigh], a["link_diag_inertia"].reshape(-1, 3)[thigh]
+    R = np.stack([rotate(frame[3:], e) for e in np.eye(3)], 1)
+    assert np.allclose(R @ np.diag(principal) @ R.T, [[0.012, 0.0005, 0], [0.0005, 0.011, 0.0003], [0, 0.0003, 0.002]], atol=1e-8)
+    assert np.allclose(frame[:3], [0, 0, -0.12 + 0.01], atol=1e-7)       # the centre of mass moves with the link frame onto the last anchor
+
+
+def test_biped_stands_on_its_feet_in_the_oracle(oracle_py):
+    scene = nk.Scene(BIPED, nk.SCENE_PLANE_CONTACTS_ONLY)
+    state = scene.initial_state()
+    w = oracle_py.OracleWorld(scene, abi.world_desc(2, 0.005, vel_iters=8), threads=2)
+    for name, values in (("q", state["q"]), ("drive_target", state["q"]), ("drive_stiffness", state["drive_stiffness"]),
+                         ("drive_damping", state["drive_damping"]), ("drive_force_limit", state["drive_force_limit"])):
+        w.upload(name, np.tile(values, 2))
+    w.upload("base_pose", np.tile(state["base_pose"], 2))
+    w.step(100)
+    assert not w.download("env_status").any()
+    base = w.download("base_pose").reshape(2, 7)
+    assert 0.45 < base[0, 2] < 0.65                       # it settled onto its feet and the servos hold it up
+    assert np.array_equal(base[0], base[1])               # identical environments stay identical
+    assert w.download("contact_count")[0] >= 2
+    w.close()
+
+
+def test_errors(tmp_path):
+    with pytest.raises(nk.NukaError) as err:
+        nk.Scene(str(tmp_path / "nonexistent.xml"))
+    assert err.value.code == abi.RESULT_INVALID_ARG and "failed to load" in str(err.value)
+    cases = {
+        "ball": '<mujoco><worldbody><body><joint type="ball"/><inertial mass="1" pos="0 0 0" diaginertia="1 1 1"/></body></worldbody></mujoco>',
+        "two": '<mujoco><worldbody><body name="a"><freejoint/></body><body name="b"><freejoint/></body></worldbody></mujoco>',
+        "xml": '<mujoco><worldbody><body></worldbody></mujoco>',
+        "root": '<robot/>',
+    }
+    for name, text in cases.items():
+        path = tmp_path / f"{name}.xml"
+        path.write_text(text)
+        with pytest.raises(nk.NukaError) as err:
+            nk.Scene(str(path))
+        assert err.value.code == abi.RESULT_INVALID_ARG, name
