@@ -30,6 +30,10 @@
  *                             layout invariants); the merged profile terms of the material key against the
  *                             reference's MergeContactParams.  The key's hash routine is device-only code:
  *                             PARITY UNPINNED for its constants.
+ *   drives, joint rows      : pinned (gravity-free pendulum: implicit-Euler PD step, force-limit clamp, limit stop and
+ *                             push-out, dry friction hold / slip; torque-mode drive rows against the direct-torque path)
+ *   contact readout         : pinned (weight of a resting ball, Coulomb friction and its moment, link wrenches adding up
+ *                             to the generalized impulse the solve applied)
  *   UABD fixed point        : pinned (closed-form resting, falling, sticking and sliding ball; Coulomb / KKT
  *                             conditions and momentum balance of converged solves)
  *   UABD iterate path       : PARITY UNPINNED - penalty heuristic, first-sweep segment search, FISTA
