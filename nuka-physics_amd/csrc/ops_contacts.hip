@@ -537,6 +537,9 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
             }
             lambda[rs] = impulse;
             if (joint_dof(m.joint_type[l]) == 1u) d.chain_jacobian[(size_t{env} * R + rs) * md + m.link_dof[l]] = jacobian;
+            // the solve takes a row on one coordinate from here instead of scanning its Jacobian row for it
+            d.row_unit[size_t{env} * R + rs] = row.flags != 0u ? m.link_dof[l] : kInvalid;
+            d.row_unit_value[size_t{env} * R + rs] = jacobian;
             rows[rs] = row;
         }
     }

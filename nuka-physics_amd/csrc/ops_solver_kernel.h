@@ -33,6 +33,9 @@ constexpr uint32_t kLineSearchSteps = 32u;    // block_descent_dense.cuh:15
 constexpr float kLineTolerance = 1.0e-6f;     // block_descent_dense.cuh:17
 constexpr float kRoundings = 8.0f;            // block_descent_dense.cuh:19
 constexpr float kPenaltyConditionCap = 1.0e2f;   // block_descent.cu:71
+// Unit heads a coordinate can list for itself (lower limit, upper limit, friction, drive, and room to spare); a block
+// with more on one coordinate walks its unit heads serially instead.
+constexpr uint32_t kUnitSlots = 6u;
 
 // Phase timers for development builds (-DNKH_SOLVER_PROFILE): cycles per phase and event counts per environment,
 // written over the environment's solver_penalty words at the end of the solve.
@@ -184,10 +187,15 @@ struct Tile {
     mutable uint32_t work;   // Newton steps and line probes of this solve, the next solve's scheduling key
     bool mass_valid;
     bool units;      // some head is a unit head
+    bool unit_lists; // every coordinate's unit heads fit its list
+    uint32_t* unit_list;      // kUnitSlots x 64: lane's unit heads in head order, slot-major
+    uint32_t unit_count;      // lane's own count
+    uint32_t staged_end;      // one past the last staged head
+    uint32_t individual_end;  // one past the last head whose inertial response is computed for itself
     float momentum, residual;
     bool failed;
 #ifdef NKH_SOLVER_PROFILE
-    mutable long long prof[22];
+    mutable long long prof[26];
     mutable uint32_t prof_count[4];
 #endif
     __device__ float& F(uint32_t field, uint32_t h) const { return fields[field * cap + h]; }
@@ -415,6 +423,10 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
         for (int k = 0; k < 6; ++k) c.F(hC + k, h) = cv[k];
         c.U(hContrib, h) = contributes ? 1u : 0u;
     }
+    if (c.units && lane < c.heads && c.U(hUnit, lane) != kInvalid) {   // a coordinate reads its unit heads' responses from the fields
+        c.F(hF, lane) = mf[0]; c.F(hC, lane) = mc[0]; c.F(hNoise, lane) = mn[0];
+        c.U(hContrib, lane) = mine ? 1u : 0u;
+    }
     __syncthreads();
     PROF_END(c, 10);
     PROF_BEGIN(c, 11);
@@ -464,63 +476,65 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
         }
     } else {
         // The heads add in the reference's order (:1533-1603): 32 at a time, and within each 32 the unit heads - a row on
-        // one coordinate adds to that coordinate's diagonal and force only - before the staged ones.
+        // one coordinate adds to that coordinate's diagonal and force only - before the staged ones.  Chunks past the
+        // last staged head hold unit heads only and go in one pass.
         float diagonal = 0.0f;
-        const uint32_t my_unit = lane < c.heads ? c.U(hUnit, lane) : kInvalid;
-        const float my_unit_value = lane < c.heads ? c.F(hUnitValue, lane) : 0.0f;
-        const uint64_t contributing = __ballot(mine), unit_heads = __ballot(my_unit != kInvalid);
-        for (uint32_t chunk = 0u; chunk < uint32_t(kWave) && chunk < c.heads; chunk += 32u) {
-            const uint64_t here = contributing & (0xFFFFFFFFull << chunk);
-            for (uint64_t rest = here & unit_heads; rest != 0ull; rest &= rest - 1ull) {
-                const uint32_t h = uint32_t(__builtin_ctzll(rest));
-                const uint32_t target = uint32_t(__builtin_amdgcn_readlane(int(my_unit), int(h)));
-                const float v = uniform_lane_value(my_unit_value, h), fx = uniform_lane_value(mf[0], h);
-                const float cxx = uniform_lane_value(mc[0], h), nx = uniform_lane_value(mn[0], h);
-                if (lane == target) {
-                    diagonal += v * cxx * v;
-                    tile_add_product(g, v, fx);
-                    scale += fabsf(v) * nx;
+        uint32_t next = 0u;
+        const uint64_t contributing = __ballot(mine);
+        const uint64_t unit_heads = __ballot(lane < c.heads && c.U(hUnit, lane) != kInvalid);
+        auto add_unit = [&](uint32_t h) {
+            const float v = c.F(hUnitValue, h);
+            diagonal += v * c.F(hC, h) * v;
+            tile_add_product(g, v, c.F(hF, h));
+            scale += fabsf(v) * c.F(hNoise, h);
+        };
+        // unit heads below `below`: lane = coordinate walks its own short list, or, when some coordinate's list
+        // overflowed, the wave walks every unit head in turn
+        auto add_units = [&](uint32_t from, uint32_t below) {
+            if (c.unit_lists) {
+                while (next < c.unit_count) {
+                    const uint32_t h = c.unit_list[next * uint32_t(kWave) + lane];
+                    if (h >= below) break;
+                    ++next;
+                    if (c.U(hContrib, h) != 0u) add_unit(h);
                 }
+                return;
             }
-            for (uint64_t rest = here & ~unit_heads; rest != 0ull; rest &= rest - 1ull) {
-                const uint32_t h = uint32_t(__builtin_ctzll(rest));
-                float f[3], cv[6], noise[3];
-    #pragma unroll
-                for (int k = 0; k < 3; ++k) { f[k] = uniform_lane_value(mf[k], h); noise[k] = uniform_lane_value(mn[k], h); }
-    #pragma unroll
-                for (int k = 0; k < 6; ++k) cv[k] = uniform_lane_value(mc[k], h);
-                const uint32_t axes = uint32_t(__builtin_amdgcn_readlane(int(my_axes), int(h)));
-                const uint64_t columns = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_high), int(h)))) << 32u) |
-                                         uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_low), int(h))));
-                add_head<N>(c, h, coordinate, f, cv, noise, axes, columns, hrow, g, scale);
-            }
-        }
-        for (uint32_t chunk = kWave; chunk < c.heads; chunk += 32u) {
+            for (uint32_t h = from; h < below; ++h)
+                if (c.U(hContrib, h) != 0u && c.U(hUnit, h) == lane) add_unit(h);
+        };
+        for (uint32_t chunk = 0u; chunk < c.staged_end; chunk += 32u) {
             const uint32_t end = min(chunk + 32u, c.heads);
-            for (uint32_t h = chunk; h < end; ++h) {
-                const uint32_t target = c.U(hUnit, h);
-                if (c.U(hContrib, h) == 0u || target == kInvalid) continue;
-                const float v = c.F(hUnitValue, h);
-                if (lane == target) {
-                    diagonal += v * c.F(hC, h) * v;
-                    tile_add_product(g, v, c.F(hF, h));
-                    scale += fabsf(v) * c.F(hNoise, h);
+            add_units(chunk, end);
+            if (chunk < uint32_t(kWave)) {
+                for (uint64_t rest = contributing & ~unit_heads & (0xFFFFFFFFull << chunk); rest != 0ull; rest &= rest - 1ull) {
+                    const uint32_t h = uint32_t(__builtin_ctzll(rest));
+                    float f[3], cv[6], noise[3];
+#pragma unroll
+                    for (int k = 0; k < 3; ++k) { f[k] = uniform_lane_value(mf[k], h); noise[k] = uniform_lane_value(mn[k], h); }
+#pragma unroll
+                    for (int k = 0; k < 6; ++k) cv[k] = uniform_lane_value(mc[k], h);
+                    const uint32_t axes = uint32_t(__builtin_amdgcn_readlane(int(my_axes), int(h)));
+                    const uint64_t columns = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_high), int(h)))) << 32u) |
+                                             uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_low), int(h))));
+                    add_head<N>(c, h, coordinate, f, cv, noise, axes, columns, hrow, g, scale);
+                }
+            } else {
+                for (uint32_t h = chunk; h < end; ++h) {
+                    if (c.U(hContrib, h) == 0u || c.U(hUnit, h) != kInvalid) continue;
+                    const float f[3] = {c.F(hF, h), c.F(hF + 1, h), c.F(hF + 2, h)};
+                    const float cv[6] = {c.F(hC, h), c.F(hC + 1, h), c.F(hC + 2, h), c.F(hC + 3, h), c.F(hC + 4, h), c.F(hC + 5, h)};
+                    const float noise[3] = {c.F(hNoise, h), c.F(hNoise + 1, h), c.F(hNoise + 2, h)};
+                    const uint64_t columns = (uint64_t(__builtin_amdgcn_readfirstlane(c.U(hColumnsHigh, h))) << 32u) |
+                                             uint64_t(__builtin_amdgcn_readfirstlane(c.U(hColumnsLow, h)));
+                    add_head<N>(c, h, coordinate, f, cv, noise, c.U(hAxes, h), columns, hrow, g, scale);
                 }
             }
-            for (uint32_t h = chunk; h < end; ++h) {
-                if (c.U(hContrib, h) == 0u || c.U(hUnit, h) != kInvalid) continue;
-                const float f[3] = {c.F(hF, h), c.F(hF + 1, h), c.F(hF + 2, h)};
-                const float cv[6] = {c.F(hC, h), c.F(hC + 1, h), c.F(hC + 2, h), c.F(hC + 3, h), c.F(hC + 4, h), c.F(hC + 5, h)};
-                const float noise[3] = {c.F(hNoise, h), c.F(hNoise + 1, h), c.F(hNoise + 2, h)};
-                const uint64_t columns = (uint64_t(__builtin_amdgcn_readfirstlane(c.U(hColumnsHigh, h))) << 32u) |
-                                         uint64_t(__builtin_amdgcn_readfirstlane(c.U(hColumnsLow, h)));
-                add_head<N>(c, h, coordinate, f, cv, noise, c.U(hAxes, h), columns, hrow, g, scale);
-            }
         }
-        if (c.units) {   // the unit heads' curvature lands on the diagonal after every staged head (:1605-1606)
-    #pragma unroll
-            for (int k = 0; k < N; ++k) hrow[k] += local_lane(lane) == uint32_t(k) ? diagonal : 0.0f;
-        }
+        add_units((c.staged_end + 31u) & ~31u, c.heads);
+        // the unit heads' curvature lands on the diagonal after every staged head (:1605-1606)
+#pragma unroll
+        for (int k = 0; k < N; ++k) hrow[k] += local_lane(lane) == uint32_t(k) ? diagonal : 0.0f;
     }
     PROF_END(c, 12);
     PROF_BEGIN(c, 13);
@@ -824,25 +838,42 @@ __device__ __forceinline__ void measure_primal(Tile& c, const float (&mrow)[N], 
     double balance = 0.0;
 #pragma unroll
     for (int j = 0; j < N; ++j) balance -= double(mrow[j]) * (double(dvec[j]) - c.vec[64 + j]);   // padded terms are exact zeros
-    for (uint32_t h = 0u; h < c.heads; ++h) {
-        if (c.U(hOwned, h) == 0u) continue;
+    // heads with an impulse add J^T lambda in head order (:2402-2436).  A unit head touches one coordinate: that
+    // lane takes it from its own list when it comes up between the staged heads
+    uint32_t next = 0u;
+    auto add_units = [&](uint32_t from, uint32_t below) {
+        if (!c.units) return;
+        if (c.unit_lists) {
+            while (next < c.unit_count) {
+                const uint32_t h = c.unit_list[next * uint32_t(kWave) + lane];
+                if (h >= below) break;
+                ++next;
+                if (c.U(hOwned, h) != 0u) balance += double(c.F(hUnitValue, h)) * lambda_env[c.U(hSlot, h) - c.env * R];
+            }
+            return;
+        }
+        for (uint32_t h = from; h < below; ++h)
+            if (c.U(hOwned, h) != 0u && c.U(hUnit, h) == lane) balance += double(c.F(hUnitValue, h)) * lambda_env[c.U(hSlot, h) - c.env * R];
+    };
+    uint32_t done = 0u;
+    for (uint32_t h = 0u; h < c.staged_end; ++h) {
+        const uint32_t first = c.U(hRow, h);
+        if (first == kInvalid || c.U(hOwned, h) == 0u) continue;
+        add_units(done, h);
+        done = h + 1u;
         const uint32_t local = c.U(hSlot, h) - c.env * R, stride = c.U(hStride, h), axes = c.U(hAxes, h);
         const float ix = lambda_env[local], iy = axes == 3u ? lambda_env[local + stride] : 0.0f,
                     iz = axes == 3u ? lambda_env[local + 2u * stride] : 0.0f;
         if (!(ix != 0.0f || iy != 0.0f || iz != 0.0f)) continue;
         if (!coordinate) continue;
-        const uint32_t unit = c.U(hUnit, h);
-        if (unit != kInvalid) {   // :2428
-            if (lane == unit) balance += double(c.F(hUnitValue, h)) * ix;
-            continue;
-        }
-        const float* j = c.jac + c.U(hRow, h) * c.ldj;
+        const float* j = c.jac + first * c.ldj;
         balance += double(j[lane]) * ix;
         if (axes == 3u) {
             balance += double(j[c.ldj + lane]) * iy;
             balance += double(j[2u * c.ldj + lane]) * iz;
         }
     }
+    add_units(done, c.heads);
     __syncthreads();
     const float force = float(balance);
     const bool finite = __all(!coordinate || fabs(balance) <= double(FLT_MAX));
@@ -1032,7 +1063,7 @@ __host__ __device__ inline uint32_t FactorRegionFloats(uint32_t n) {
 // `cap` heads carry fields; `staged` of them (the contact heads) carry three Jacobian rows each.
 __host__ __device__ inline uint32_t SolverLdsFloats(uint32_t n, uint32_t cap, uint32_t staged) {
     const uint32_t N = PaddedWidth(n);
-    return FactorRegionFloats(n) + 3u * staged * N + ((hFieldCount * cap + 3u) & ~3u) + 256u;
+    return FactorRegionFloats(n) + 3u * staged * N + ((hFieldCount * cap + 3u) & ~3u) + 256u + kUnitSlots * uint32_t(kWave);
 }
 
 // DescendTile (:2941-3087)
@@ -1047,7 +1078,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     c.tolerance = p.velocity_tolerance; c.failed = false; c.momentum = 0.0f; c.residual = 0.0f;
     c.mass_inverse = 0.0f; c.mass_valid = false; c.work = 0u; c.units = false;
 #ifdef NKH_SOLVER_PROFILE
-    for (int i = 0; i < 22; ++i) c.prof[i] = 0;
+    for (int i = 0; i < 26; ++i) c.prof[i] = 0;
     for (int i = 0; i < 4; ++i) c.prof_count[i] = 0u;
 #endif
     PROF_BEGIN(c, 9);
@@ -1057,6 +1088,8 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     c.jac = lds + FactorRegionFloats(n);
     c.fields = c.jac + 3u * staged_cap * c.ldj;
     c.vec = c.fields + ((hFieldCount * cap + 3u) & ~3u);
+    c.unit_list = reinterpret_cast<uint32_t*>(c.vec + 256);
+    c.unit_lists = true; c.unit_count = 0u; c.staged_end = 0u; c.individual_end = 0u;
     const bool coordinate = lane < n;
     const float* urows = d.urows;
     float* lambda_env = d.lambda + size_t{env} * R;
@@ -1119,54 +1152,73 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         c.U(hSourceA + axis, h) = source_a; c.U(hSourceB + axis, h) = source_b;
     }
     __syncthreads();
+    PROF_BEGIN(c, 22);
     // FindTileRowSupport (:801-833), lane = head: a single-axis head whose Jacobian row has at most one entry is a unit
     // head and stages nothing; every other owned head stages three rows, placed in head order (PlaceTileRows).
     {
-        uint32_t staged = 0u;
+        // a single-axis head acting on one coordinate is a unit head; the rows carry that coordinate and its entry
+        // from where they were emitted (row_unit, row_unit_value), which is what a scan of the head's Jacobian row
+        // for its entries would find
+        for (uint32_t base = 0u; base < heads; base += kWave) {
+            const uint32_t h = base + lane;
+            if (h >= heads) continue;
+            const uint32_t source_a = c.U(hSourceA, h), source_b = c.U(hSourceB, h);
+            const bool owned = source_a != kInvalid || source_b != kInvalid;
+            // a block head has found the sources of its tangent rows on the sides that move
+            const bool single_axis = c.U(hSourceA + 1u, h) == kInvalid && c.U(hSourceB + 1u, h) == kInvalid;
+            const uint32_t slot = c.U(hSlot, h);
+            uint32_t unit = kInvalid;
+            float unit_value = 0.0f;
+            if (owned && single_axis && d.row_unit[slot] != kInvalid) { unit = d.row_unit[slot]; unit_value = d.row_unit_value[slot]; }
+            c.U(hUnit, h) = unit; c.F(hUnitValue, h) = unit_value; c.U(hRow, h) = owned && unit == kInvalid ? 0u : kInvalid;
+            c.U(hColumnsLow, h) = 0u; c.U(hColumnsHigh, h) = 0u;
+        }
+        __syncthreads();
+        PROF_END(c, 22);
+        PROF_BEGIN(c, 23);
+        // PlaceTileRows: the staged heads take their rows in head order
+        uint32_t staged = 0u, staged_end = 0u, individual_end = 0u, my_units = 0u;
         bool overflow_rows = false, any_unit = false;
         for (uint32_t base = 0u; base < heads; base += kWave) {
             const uint32_t h = base + lane;
-            bool stage = false;
-            uint32_t unit = kInvalid;
-            float unit_value = 0.0f;
-            if (h < heads) {
-                const uint32_t source_a = c.U(hSourceA, h), source_b = c.U(hSourceB, h);
-                const bool owned = source_a != kInvalid || source_b != kInvalid;
-                // a block head has found the sources of its tangent rows on the sides that move
-                const bool single_axis = c.U(hSourceA + 1u, h) == kInvalid && c.U(hSourceB + 1u, h) == kInvalid;
-                if (owned && single_axis) {
-                    uint32_t supported = 0u, last = 0u;
-                    float last_value = 0.0f;
-                    for (uint32_t i = 0u; i < n; ++i) {
-                        float value = 0.0f;
-                        if (source_a != kInvalid) value += d.chain_jacobian[size_t{source_a} * md + i];
-                        if (source_b != kInvalid) value += d.chain_jacobian_b[size_t{source_b} * md + i];
-                        if (value != 0.0f) { ++supported; last = i; last_value = value; }
-                    }
-                    if (supported <= 1u) { unit = last; unit_value = last_value; }
-                }
-                stage = owned && unit == kInvalid;
-            }
+            const bool stage = h < heads && c.U(hRow, h) != kInvalid;
             const uint64_t mask = __ballot(stage);
-            if (h < heads) {
-                uint32_t row = kInvalid;
-                if (stage) {
-                    const uint32_t at = staged + uint32_t(__popcll(mask & ((uint64_t{1} << lane) - 1ull)));
-                    if (at < staged_cap) row = 3u * at;
-                    else { overflow_rows = true; unit = 0u; unit_value = 0.0f; }   // no room: the head acts on nothing, and the solve is flagged
+            if (stage) {
+                const uint32_t at = staged + uint32_t(__popcll(mask & ((uint64_t{1} << lane) - 1ull)));
+                if (at < staged_cap) c.U(hRow, h) = 3u * at;
+                else {   // no room: the head acts on nothing, and the solve is flagged
+                    overflow_rows = true;
+                    c.U(hRow, h) = kInvalid; c.U(hUnit, h) = 0u; c.F(hUnitValue, h) = 0.0f;
                 }
-                c.U(hRow, h) = row; c.U(hUnit, h) = unit; c.F(hUnitValue, h) = unit_value;
             }
             staged += uint32_t(__popcll(mask));
-            any_unit = any_unit || unit != kInvalid;
+            if (mask != 0ull) staged_end = base + uint32_t(64 - __builtin_clzll(mask));
+            any_unit = any_unit || (h < heads && c.U(hUnit, h) != kInvalid);
+            // heads that need a response of their own: staged ones, and unit heads whose entry is not +-1
+            const uint64_t own = __ballot(h < heads && (c.U(hUnit, h) == kInvalid || fabsf(c.F(hUnitValue, h)) != 1.0f));
+            if (own != 0ull) individual_end = base + uint32_t(64 - __builtin_clzll(own));
         }
         c.units = __any(any_unit);
+        c.staged_end = staged_end;
+        c.individual_end = individual_end;
         if (__any(overflow_rows) && lane == 0u) d.env_status[env] |= kEnvStatusSolverFailure;
+        __syncthreads();
+        // every coordinate lists its own unit heads, in head order
+        if (c.units) {
+            for (uint32_t h = 0u; h < heads; ++h) {
+                if (c.U(hUnit, h) != lane) continue;
+                if (my_units < kUnitSlots) c.unit_list[my_units * uint32_t(kWave) + lane] = h;
+                ++my_units;
+            }
+            c.unit_lists = !__any(my_units > kUnitSlots);
+            c.unit_count = min(my_units, kUnitSlots);
+        }
+        PROF_END(c, 23);
     }
     __syncthreads();
     // CopyTileRows (:836-869): the staged heads' rows, their loads in flight together
 
-    for (uint32_t h = 0u; h < heads; ++h) {
+    for (uint32_t h = 0u; h < c.staged_end; ++h) {
         const uint32_t first = c.U(hRow, h);
         const bool staged = first != kInvalid;   // a unit head stages nothing and touches no column block
         float value[3];
@@ -1222,14 +1274,16 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         };
         // Four heads at a time: their substitution chains are independent, and side by side each one's lane reads
         // settle under the others' arithmetic.  A head with one moving side, or with both sides on one owner (:752),
-        // wants exactly the staged sum of its two sides' rows.
-        for (uint32_t h0 = 0u; h0 < heads; h0 += 4u) {
+        // wants exactly the staged sum of its two sides' rows.  Unit heads with an entry of +-1 are left to the
+        // per-coordinate pass below: y(-e) = -y(e), so every such head of one coordinate has the same response.
+        const bool share_units = c.units && c.unit_lists;
+        for (uint32_t h0 = 0u; h0 < (share_units ? c.individual_end : heads); h0 += 4u) {
             float a[4], term[4], total[4];
-            bool second[4], apart[4];
+            bool second[4], apart[4], skip[4];
 #pragma unroll
             for (uint32_t t = 0u; t < 4u; ++t) {
                 const uint32_t h = h0 + t;
-                a[t] = 0.0f; second[t] = false; apart[t] = false;
+                a[t] = 0.0f; second[t] = false; apart[t] = false; skip[t] = true;
                 if (h >= heads) continue;
                 const bool artic_a = c.U(hSourceA, h) != kInvalid, artic_b = c.U(hSourceB, h) != kInvalid;
                 if (artic_a && artic_b) {
@@ -1237,11 +1291,13 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
                     apart[t] = __float_as_uint(row[11]) != __float_as_uint(row[19]);
                 }
                 second[t] = artic_b && !artic_a;
-                if (coordinate && (artic_a || artic_b) && !apart[t]) {
-                    const uint32_t first = c.U(hRow, h);
-                    a[t] = first != kInvalid ? c.jac[first * c.ldj + lane] : (lane == c.U(hUnit, h) ? c.F(hUnitValue, h) : 0.0f);
-                }
+                const uint32_t first = c.U(hRow, h), unit = c.U(hUnit, h);
+                const float unit_value = c.F(hUnitValue, h);
+                skip[t] = share_units && unit != kInvalid && fabsf(unit_value) == 1.0f && !apart[t];
+                if (coordinate && (artic_a || artic_b) && !apart[t] && !skip[t])
+                    a[t] = first != kInvalid ? c.jac[first * c.ldj + lane] : (lane == unit ? unit_value : 0.0f);
             }
+            if (skip[0] && skip[1] && skip[2] && skip[3]) continue;
 #pragma unroll
             for (int j = 0; j < N; ++j) {
 #pragma unroll
@@ -1257,13 +1313,55 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
 #pragma unroll
             for (uint32_t t = 0u; t < 4u; ++t) {
                 const uint32_t h = h0 + t;
-                if (h >= heads) continue;
+                if (h >= heads || skip[t]) continue;
                 float shares[2] = {second[t] ? 0.0f : total[t], second[t] ? total[t] : 0.0f};
                 if (apart[t]) {   // two owners: one response each
                     shares[0] = response(coordinate ? d.chain_jacobian[size_t{c.U(hSourceA, h)} * md + lane] : 0.0f);
                     shares[1] = response(coordinate ? d.chain_jacobian_b[size_t{c.U(hSourceB, h)} * md + lane] : 0.0f);
                 }
                 if (lane == 0u) { c.F(hRes, h) = shares[0]; c.F(hRes + 1, h) = shares[1]; }
+            }
+        }
+        if (share_units) {   // (M^-1)_uu of every coordinate that has unit heads, four coordinates at a time
+            float mine = 0.0f;
+            for (uint64_t rest = __ballot(c.unit_count > 0u); rest != 0ull;) {
+                uint32_t target[4];
+                float a[4], term[4], total[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    target[t] = rest != 0ull ? uint32_t(__builtin_ctzll(rest)) : kInvalid;
+                    rest &= rest - 1ull;   // zero stays zero
+                    a[t] = lane == target[t] ? 1.0f : 0.0f;
+                }
+                // below the group's first coordinate every y_j is an exact zero: those steps subtract and add nothing
+                const int first = int(target[0]);
+#pragma unroll
+                for (int j = 0; j < N; ++j) {
+                    if (j < first) continue;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) a[t] -= lrow[j] * lane_value(a[t], j);
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t) { term[t] = coordinate ? a[t] * a[t] / pivot : 0.0f; total[t] = 0.0f; }
+#pragma unroll
+                for (int i = 0; i < N; ++i) {
+                    if (i < first) continue;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) total[t] += lane_value(term[t], i);
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t) if (lane == target[t]) mine = total[t];
+            }
+            for (uint32_t k = 0u; k < c.unit_count; ++k) {   // lane = coordinate hands its response to its own unit heads
+                const uint32_t h = c.unit_list[k * uint32_t(kWave) + lane];
+                if (fabsf(c.F(hUnitValue, h)) != 1.0f) continue;
+                const bool artic_a = c.U(hSourceA, h) != kInvalid, artic_b = c.U(hSourceB, h) != kInvalid;
+                if (artic_a && artic_b) {   // both sides on one owner (two owners were answered above)
+                    const float* row = urows + size_t{c.U(hSlot, h)} * kRowWords;
+                    if (__float_as_uint(row[11]) != __float_as_uint(row[19])) continue;
+                }
+                const bool second = artic_b && !artic_a;
+                c.F(hRes, h) = second ? 0.0f : mine; c.F(hRes + 1, h) = second ? mine : 0.0f;
             }
         }
         __syncthreads();
@@ -1358,7 +1456,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     if (lane == 0u) {
         for (int i = 0; i < 10; ++i) d.solver_penalty[size_t{env} * R + i] = float(c.prof[i]);
         for (int i = 0; i < 4; ++i) d.solver_penalty[size_t{env} * R + 10 + i] = float(c.prof_count[i]);
-        for (int i = 10; i < 22; ++i) d.solver_penalty[size_t{env} * R + 4 + i] = float(c.prof[i]);
+        for (int i = 10; i < 26; ++i) d.solver_penalty[size_t{env} * R + 4 + i] = float(c.prof[i]);
     }
 #endif
     // the block velocities persist for the next solve's carried start

@@ -243,7 +243,7 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(row_cj_link, kU32, E * R) X(row_cj_link_b, kU32, E * R) X(row_count, kU32, E) X(contact_count, kU32, E) \
     X(contact_row_extent, kU32, E * 2) X(env_status, kU32, E) X(vbd_velocity_sweep_count, kU32, E) \
     X(solver_residual, kF32, E * 4) X(solver_penalty, kF32, E * R) X(solver_velocity, kF32, E * md) X(solver_free, kF32, E * md) \
-    X(solver_cost, kU32, E) X(tile_order, kU32, E) \
+    X(solver_cost, kU32, E) X(tile_order, kU32, E) X(row_unit, kU32, E * R) X(row_unit_value, kF32, E * R) \
     X(contact_material, kU64, E * S) X(contact_cache_pair, kU64, E * S * 4) X(contact_cache_feature, kU64, E * S * 4) \
     X(contact_cache_material, kU64, E * S * 4) X(contact_cache_lambda, kF32, E * S * 16) X(contact_cache_normal, kF32, E * S * 12) \
     X(contact_cache_age, kU32, E * S * 4) X(contact_cache_current_owner, kU32, E * S * 4) X(contact_cache_old_keep, kU32, E * S * 4) \
@@ -679,7 +679,8 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
             };
             if (!put(w.data.base_pose, base_pose.data(), base_pose.size() * 4u) || !put(w.data.link_pose, link_pose.data(), link_pose.size() * 4u) ||
                 !put(w.data.body_pose, body_pose.data(), body_pose.size() * 4u) || !put(w.data.row_cj_link, invalid.data(), invalid.size() * 4u) ||
-                !put(w.data.row_cj_link_b, invalid.data(), invalid.size() * 4u)) return Error(NUKA_RESULT_DEVICE_ERROR, "initial state upload failed");
+                !put(w.data.row_cj_link_b, invalid.data(), invalid.size() * 4u) || !put(w.data.row_unit, invalid.data(), invalid.size() * 4u))
+                return Error(NUKA_RESULT_DEVICE_ERROR, "initial state upload failed");
         }
         if (scene != nullptr) {   // the state and drive parameters the scene file authors, in every environment
             auto tile = [&](const std::vector<float>& per_link) {
