@@ -175,13 +175,34 @@ enum HeadField : uint32_t {
     hFieldCount
 };
 
+// A head on one axis uses the first component of every three-component field and none of the block-only fields;
+// only block heads (three axes: contact points, which are listed first) use the rest.  The fields are therefore kept
+// in two tables: "wide" fields have room for every head, "narrow" fields for the first `narrow` heads and one more
+// word that every later head shares.  That word reads as zero and swallows what is written to it, which is always
+// zero: a single-axis head keeps its second and third components, its relaxation state and its column masks at zero
+// throughout.  A head's place in a narrow field is min(h, narrow), one operation whatever the number of fields read.
+__host__ __device__ constexpr uint32_t clamped_span(uint32_t f, uint32_t first, uint32_t end) {   // fields of [first, end) below f
+    return f <= first ? 0u : (f >= end ? end - first : f - first);
+}
+// the narrow fields are these ranges of field ids
+__host__ __device__ constexpr uint32_t narrow_below(uint32_t f) {
+    return clamped_span(f, hRes + 1, hRes + 3) + clamped_span(f, hDual + 1, hDual + 3) + clamped_span(f, hMove + 1, hMove + 3) +
+           clamped_span(f, hStep + 1, hStep + 3) + clamped_span(f, hBase + 1, hBase + 3) + clamped_span(f, hRelaxStep, hF) +
+           clamped_span(f, hF + 1, hF + 3) + clamped_span(f, hC + 1, hNoise) + clamped_span(f, hNoise + 1, hNoise + 3) +
+           clamped_span(f, hColumnsLow, hColumnsHigh + 1);
+}
+__host__ __device__ constexpr bool narrow_field(uint32_t f) { return narrow_below(f + 1u) != narrow_below(f); }
+constexpr uint32_t kNarrowFields = narrow_below(hFieldCount);
+constexpr uint32_t kWideFields = hFieldCount - kNarrowFields;
+static_assert(kNarrowFields <= 64u, "one lane clears the shared word of each narrow field");
+
 struct Tile {
-    uint32_t env, lane, n, ld, ldj, heads, cap, iteration;
+    uint32_t env, lane, n, ld, ldj, heads, cap, narrow, iteration;
     float tolerance;
     float* mfac;     // N x ld: Cholesky factor of the mass matrix (rows; columns are read transposed)
     float* hfac;     // N x ld: Cholesky factor of the current Newton Hessian
     float* jac;      // 3 * staged capacity rows x ldj, ldj = N
-    float* fields;   // hFieldCount x cap
+    float* fields;   // kWideFields x cap, then kNarrowFields x (narrow + 1)
     float* vec;      // 4 x 64 scratch vectors, 16-byte aligned
     float mass_inverse;   // 1 / diagonal of the mass factor, lane = row
     mutable uint32_t work;   // Newton steps and line probes of this solve, the next solve's scheduling key
@@ -198,8 +219,14 @@ struct Tile {
     mutable long long prof[26];
     mutable uint32_t prof_count[4];
 #endif
-    __device__ float& F(uint32_t field, uint32_t h) const { return fields[field * cap + h]; }
-    __device__ uint32_t& U(uint32_t field, uint32_t h) const { return reinterpret_cast<uint32_t*>(fields)[field * cap + h]; }
+    // with a constant field, as at nearly every call, the place of the field folds to a constant
+    __device__ __forceinline__ uint32_t at(uint32_t field, uint32_t h) const {
+        const uint32_t below = narrow_below(field);
+        if (!narrow_field(field)) return (field - below) * cap + h;
+        return kWideFields * cap + below * (narrow + 1u) + min(h, narrow);
+    }
+    __device__ __forceinline__ float& F(uint32_t field, uint32_t h) const { return fields[at(field, h)]; }
+    __device__ __forceinline__ uint32_t& U(uint32_t field, uint32_t h) const { return reinterpret_cast<uint32_t*>(fields)[at(field, h)]; }
 };
 
 // TileResponse (block_descent_tile.cuh:678-681) with the Coulomb branch of EvaluateAugmentedResponse (block_descent.cu:1593-1621)
@@ -1060,10 +1087,15 @@ __host__ __device__ inline uint32_t FactorRegionFloats(uint32_t n) {
     const uint32_t N = PaddedWidth(n);
     return 2u * N * (N + 1u);   // a multiple of 4 since N is
 }
+__host__ __device__ inline uint32_t HeadFieldFloats(uint32_t cap, uint32_t narrow) {
+    return (kWideFields * cap + kNarrowFields * (narrow + 1u) + 3u) & ~3u;
+}
 // `cap` heads carry fields; `staged` of them (the contact heads) carry three Jacobian rows each.
 __host__ __device__ inline uint32_t SolverLdsFloats(uint32_t n, uint32_t cap, uint32_t staged) {
     const uint32_t N = PaddedWidth(n);
-    return FactorRegionFloats(n) + 3u * staged * N + ((hFieldCount * cap + 3u) & ~3u) + 256u + kUnitSlots * uint32_t(kWave);
+    // the per-coordinate unit lists exist only when some head beyond the staged ones can be listed; without joint rows
+    // the block keeps the footprint that lets eight of them share a compute unit's LDS
+    return FactorRegionFloats(n) + 3u * staged * N + HeadFieldFloats(cap, staged) + 256u + (cap > staged ? kUnitSlots * uint32_t(kWave) : 0u);
 }
 
 // DescendTile (:2941-3087)
@@ -1074,7 +1106,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     const uint32_t env = d.tile_order[blockIdx.x], lane = threadIdx.x;
     const uint32_t R = p.rows_per_env, md = p.max_dof, n = m.dof, nl = m.links_per_env, S = p.contact_slots_per_env;
     Tile c;
-    c.env = env; c.lane = lane; c.n = n; c.ld = uint32_t(N) + 1u; c.ldj = uint32_t(N); c.cap = cap; c.heads = 0u; c.iteration = 0u;
+    c.env = env; c.lane = lane; c.n = n; c.ld = uint32_t(N) + 1u; c.ldj = uint32_t(N); c.cap = cap; c.narrow = staged_cap; c.heads = 0u; c.iteration = 0u;
     c.tolerance = p.velocity_tolerance; c.failed = false; c.momentum = 0.0f; c.residual = 0.0f;
     c.mass_inverse = 0.0f; c.mass_valid = false; c.work = 0u; c.units = false;
 #ifdef NKH_SOLVER_PROFILE
@@ -1087,7 +1119,8 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     c.hfac = c.mfac + uint32_t(N) * c.ld;
     c.jac = lds + FactorRegionFloats(n);
     c.fields = c.jac + 3u * staged_cap * c.ldj;
-    c.vec = c.fields + ((hFieldCount * cap + 3u) & ~3u);
+    c.vec = c.fields + HeadFieldFloats(cap, staged_cap);
+    if (lane < kNarrowFields) c.fields[kWideFields * cap + lane * (staged_cap + 1u) + staged_cap] = 0.0f;   // what a narrow field reads beyond its heads
     c.unit_list = reinterpret_cast<uint32_t*>(c.vec + 256);
     c.unit_lists = true; c.unit_count = 0u; c.staged_end = 0u; c.individual_end = 0u;
     const bool coordinate = lane < n;
@@ -1198,7 +1231,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
             const uint64_t own = __ballot(h < heads && (c.U(hUnit, h) == kInvalid || fabsf(c.F(hUnitValue, h)) != 1.0f));
             if (own != 0ull) individual_end = base + uint32_t(64 - __builtin_clzll(own));
         }
-        c.units = __any(any_unit);
+        c.units = __any(any_unit) && cap > staged_cap;   // the lists have room only when the world has joint heads
         c.staged_end = staged_end;
         c.individual_end = individual_end;
         if (__any(overflow_rows) && lane == 0u) d.env_status[env] |= kEnvStatusSolverFailure;
@@ -1319,7 +1352,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
                     shares[0] = response(coordinate ? d.chain_jacobian[size_t{c.U(hSourceA, h)} * md + lane] : 0.0f);
                     shares[1] = response(coordinate ? d.chain_jacobian_b[size_t{c.U(hSourceB, h)} * md + lane] : 0.0f);
                 }
-                if (lane == 0u) { c.F(hRes, h) = shares[0]; c.F(hRes + 1, h) = shares[1]; }
+                if (lane == 0u) { c.F(hStep, h) = shares[0]; c.F(hMove, h) = shares[1]; }
             }
         }
         if (share_units) {   // (M^-1)_uu of every coordinate that has unit heads, four coordinates at a time
@@ -1361,7 +1394,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
                     if (__float_as_uint(row[11]) != __float_as_uint(row[19])) continue;
                 }
                 const bool second = artic_b && !artic_a;
-                c.F(hRes, h) = second ? 0.0f : mine; c.F(hRes + 1, h) = second ? mine : 0.0f;
+                c.F(hStep, h) = second ? 0.0f : mine; c.F(hMove, h) = second ? mine : 0.0f;
             }
         }
         __syncthreads();
@@ -1377,7 +1410,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
             const uint32_t flags = __float_as_uint(row[0]), stride = __float_as_uint(row[2]);
             const uint32_t axes = (flags & kRowBlockNormal) != 0u ? 3u : 1u;
             const uint32_t kind_a = __float_as_uint(row[10]), kind_b = __float_as_uint(row[18]);
-            const float shares[2] = {c.F(hRes, h), c.F(hRes + 1, h)};
+            const float shares[2] = {c.F(hStep, h), c.F(hMove, h)};
             const bool valid = shares[0] >= 0.0f && isfinite(shares[0]) && shares[1] >= 0.0f && isfinite(shares[1]);
             float response = shares[0] + shares[1];
             const float coupling = shares[0] * shares[1], largest = fmaxf(shares[0], shares[1]);
