@@ -72,8 +72,9 @@ typedef struct nuka_template_desc_t {
     const uint32_t* body_role;       /* 0 static, 1 the link's own body row, 2 extra collidable of a link */
     const uint32_t* body_link;       /* owning link for roles 1 and 2 */
     const float* body_local;         /* [row][7]: world pose (static) or pose in the owning link's frame */
-    const uint32_t* shape_kind;      /* collision/shape_kind.hpp:9-18; ~0u for no shape */
-    const float* shape_params;       /* [row][4] */
+    const uint32_t* shape_kind;      /* collision/shape_kind.hpp:9-18: sphere 0, capsule 1, box 2, plane 3, cylinder 7;
+                                        ~0u for no shape */
+    const float* shape_params;       /* [row][4]: radius | radius, half length along local z | half extents */
     const uint32_t* shape_contype;
     const uint32_t* shape_conaffinity;
     const uint32_t* shape_group;
@@ -90,6 +91,12 @@ typedef struct nuka_template_desc_t {
                                         1: the reference's actuation - ApplyDrives turns the drive_* fields into one
                                         bounded-effort row per link, overwrites `tau` with `joint_f` and ReadoutDrives
                                         reports the applied effort (src/nk/pipeline/world.cpp:61) */
+    /* Collidable rows that never pair (src/scene/cooker.cpp:470-538 excluded_body_pairs, carried to collidable rows
+     * at src/scene/cook/cook_to_model.cpp:1468-1490); read only when struct_size covers them.  Two rows of one link
+     * are excluded by the cook itself. */
+    const uint32_t* excluded_pairs;  /* [pair][2] collidable rows, either order; nullable */
+    uint32_t excluded_pair_count;
+    uint32_t reserved1;
 } nuka_template_desc_t;
 
 /* nuka.h:57-173 nuka_world_desc_t; zero keeps the default of the same reference field. */

@@ -179,7 +179,7 @@ class Scene:
                       link_diag_inertia=3 * nl, joint_damping=nl, joint_armature=nl, joint_stiffness=nl, joint_spring_reference=nl,
                       body_role=nb, body_link=nb, body_local=7 * nb, shape_kind=nb, shape_params=4 * nb, shape_contype=nb,
                       shape_conaffinity=nb, shape_group=nb, shape_profile=nb, profile_mu=2 * npf, joint_limit_lower=nl,
-                      joint_limit_upper=nl, joint_limit_flags=nl, joint_frictionloss=nl)
+                      joint_limit_upper=nl, joint_limit_flags=nl, joint_frictionloss=nl, excluded_pairs=2 * d.excluded_pair_count)
         out = {name: np.ctypeslib.as_array(getattr(d, name), shape=(count,)).copy() if count else np.zeros(0, np.float32)
                for name, count in shapes.items()}
         out.update(drive_mode=d.drive_mode, drive_rows=d.drive_rows)

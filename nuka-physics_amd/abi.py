@@ -12,7 +12,7 @@ INVALID = 0xFFFFFFFF
 # phi/articulation_contract.hpp:8-16
 JOINT_REVOLUTE, JOINT_PRISMATIC, JOINT_FIXED, JOINT_FLOATING = 0, 1, 2, 3
 # collision/shape_kind.hpp:9-18
-SHAPE_SPHERE, SHAPE_CAPSULE, SHAPE_BOX, SHAPE_PLANE, SHAPE_NONE = 0, 1, 2, 3, INVALID
+SHAPE_SPHERE, SHAPE_CAPSULE, SHAPE_BOX, SHAPE_PLANE, SHAPE_CYLINDER, SHAPE_NONE = 0, 1, 2, 3, 7, INVALID
 # collidable row roles of the template description
 ROLE_STATIC, ROLE_LINK_BODY, ROLE_PROXY = 0, 1, 2
 
@@ -40,6 +40,7 @@ class TemplateDescC(C.Structure):
         ("profile_mu", _PF),
         ("joint_limit_lower", _PF), ("joint_limit_upper", _PF), ("joint_limit_flags", _PB), ("joint_frictionloss", _PF),
         ("drive_mode", C.c_uint32), ("drive_rows", C.c_uint32),
+        ("excluded_pairs", _PU), ("excluded_pair_count", C.c_uint32), ("reserved1", C.c_uint32),
     ]
 
 
@@ -71,6 +72,7 @@ class Template:
         self.max_contacts_per_env = 0
         self.drive_mode = DRIVE_TORQUE
         self.drive_rows = False   # True: affine drives through joint drive rows; False: `tau` is the applied force
+        self.excluded = []        # pairs of collidable rows that never pair (rows of one link are excluded by the cook)
 
     def add_link(self, joint_type, parent, axis=(0, 0, 1), local_pos=(0, 0, 0), local_rot=(1, 0, 0, 0), mass=1.0,
                  diag_inertia=(0.01, 0.01, 0.01), com=(0, 0, 0), damping=0.0, armature=0.0, stiffness=0.0,
@@ -92,6 +94,9 @@ class Template:
                                 local=list(local_pos) + list(local_rot), contype=contype, conaffinity=conaffinity,
                                 group=group, profile=profile))
         return len(self.bodies) - 1
+
+    def exclude(self, row_a, row_b):
+        self.excluded.append((row_a, row_b))
 
     @property
     def link_count(self):
@@ -132,6 +137,7 @@ class Template:
             shape_group=np.array([b["group"] for b in B], dtype=u32),
             shape_profile=np.array([b["profile"] for b in B], dtype=u32),
             profile_mu=np.array(self.profiles, dtype=f32).reshape(-1),
+            excluded_pairs=np.array(self.excluded, dtype=u32).reshape(-1),
         )
 
     def to_c(self):
@@ -142,6 +148,7 @@ class Template:
         d.link_count, d.body_count, d.profile_count = len(self.links), len(self.bodies), len(self.profiles)
         d.max_contacts_per_env = self.max_contacts_per_env
         d.drive_mode, d.drive_rows = self.drive_mode, 1 if self.drive_rows else 0
+        d.excluded_pair_count = len(self.excluded)
         ctype = {np.dtype(np.float32): C.c_float, np.dtype(np.uint32): C.c_uint32, np.dtype(np.uint8): C.c_uint8}
         for name, arr in a.items():
             arr = np.ascontiguousarray(arr)

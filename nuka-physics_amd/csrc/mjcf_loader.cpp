@@ -3,8 +3,8 @@
 // followed by the articulation part of the cook (src/runtime/articulation/articulation_state.cpp:345-435): the
 // same body -> link rules, default classes, joint anchors, inertial sources and actuator mapping.  Host code only.
 //
-// Not read: meshes, height fields, materials, cameras, lights, sensors, sites, equalities, <contact> pairs and
-// excludes, ball joints (rejected), tendons.  The joint and contact laws are this library's native ones: the
+// Not read: meshes, height fields, materials, cameras, lights, sensors, sites, equalities, <contact> pairs, ball
+// joints (rejected), tendons.  The joint and contact laws are this library's native ones: the
 // solref / solimp compliant rows the reference attaches to MJCF joints and geoms are not built.
 #include "mjcf_loader.h"
 
@@ -466,6 +466,7 @@ struct Link {
     V3 anchor_shift;   // what the body authors in its own frame moves by this: minus its joint anchor
     std::vector<Geom> geoms;
     float drive_stiffness = 0.0f, drive_damping = 0.0f, drive_force_limit = 0.0f;
+    bool intermediate = false;   // a massless link that carries one of several joints of a body
 };
 
 constexpr uint32_t kShapeSphere = 0u, kShapeCapsule = 1u, kShapeBox = 2u, kShapePlane = 3u, kShapeCylinder = 7u, kShapeUnknown = 0xFFFFFFFEu;
@@ -537,6 +538,7 @@ struct Builder {
     Context context;
     std::vector<Link> links;
     std::vector<Geom> world_geoms;   // static collidables, world frame
+    std::vector<std::pair<std::string, std::string>> excluded_bodies;   // <contact><exclude body1 body2>
     std::map<std::string, uint32_t> joint_links;   // joint name -> the link it moves
     bool floating_root = false;
     V3 base_position;
@@ -646,6 +648,7 @@ struct Builder {
             link.rotation = k == 0u ? rec.rotation : Quat{};
             link.mass = 1.0e-6f;
             link.inertia = {1.0e-9f, 1.0e-9f, 1.0e-9f};
+            link.intermediate = true;
             links.push_back(link);
             joint_link[k] = uint32_t(links.size() - 1u);
             walk_parent = joint_link[k];
@@ -847,6 +850,12 @@ std::unique_ptr<Scene> LoadMjcf(const std::string& path, uint32_t flags) {
         worldbody.Each("body", [&](const Element& e) { b.ParseBody(e, 0xFFFFFFFFu, nullptr); });
     });
     if (b.links.empty()) throw std::runtime_error("MJCF: no body under <worldbody> in " + path);
+    mujoco->Each("contact", [&](const Element& contact) {
+        contact.Each("exclude", [&](const Element& e) {
+            if (e.Attribute("body1") == nullptr || e.Attribute("body2") == nullptr) throw std::runtime_error("MJCF: <exclude> needs body1 and body2");
+            b.excluded_bodies.emplace_back(e.Attribute("body1"), e.Attribute("body2"));
+        });
+    });
     uint32_t drive_mode = 1u;
     b.ParseActuators(*mujoco, &drive_mode);
 
@@ -881,7 +890,9 @@ std::unique_ptr<Scene> LoadMjcf(const std::string& path, uint32_t flags) {
     }
     // collidable rows: the static geoms, then per link its own body row (with its first geom) and its further geoms
     const bool plane_only = (flags & kPlaneContactsOnly) != 0u;
-    auto supported = [](const Geom& g) { return g.kind == kShapeSphere || g.kind == kShapeBox || g.kind == kShapePlane; };
+    auto supported = [](const Geom& g) {
+        return g.kind == kShapeSphere || g.kind == kShapeCapsule || g.kind == kShapeBox || g.kind == kShapePlane || g.kind == kShapeCylinder;
+    };
     auto collides = [](const Geom& g) { return g.contype != 0u || g.conaffinity != 0u; };
     auto profile_of = [&](const Geom& g) -> uint32_t {
         if (!g.friction_authored) return 0xFFFFFFFFu;
@@ -910,13 +921,46 @@ std::unique_ptr<Scene> LoadMjcf(const std::string& path, uint32_t flags) {
         return false;
     };
     for (const Geom& g : b.world_geoms) if (keep(g)) add_row(0u, 0xFFFFFFFFu, &g, 0);
+    std::vector<std::vector<uint32_t>> link_rows(nl);
     for (uint32_t l = 0u; l < nl; ++l) {
         std::vector<const Geom*> kept;
         for (const Geom& g : b.links[l].geoms) if (keep(g)) kept.push_back(&g);
         // with plane contacts only, the robot's geoms share one negative group: they meet the ground, not each other
         const int32_t group = plane_only ? -1 : 0;
+        link_rows[l].push_back(uint32_t(s.body_role.size()));
         add_row(1u, l, kept.empty() ? nullptr : kept[0], group);
-        for (size_t i = 1u; i < kept.size(); ++i) add_row(2u, l, kept[i], group);
+        for (size_t i = 1u; i < kept.size(); ++i) { link_rows[l].push_back(uint32_t(s.body_role.size())); add_row(2u, l, kept[i], group); }
+    }
+    // Excluded pairs (src/scene/cooker.cpp:470-538): bodies welded together by fixed joints form a cluster; no two
+    // bodies of a cluster collide, nor a cluster with the cluster of its parent body, nor the bodies an <exclude>
+    // names.  The massless links that carry the earlier joints of a several-joint body stand for no body of the file:
+    // the parent of such a body is the body above them.
+    {
+        auto weld = [&](uint32_t link) {
+            while (b.links[link].parent != 0xFFFFFFFFu && (b.links[link].joint_type == 2u || b.links[link].intermediate)) link = b.links[link].parent;
+            return link;
+        };
+        std::vector<std::vector<uint32_t>> clusters(nl);
+        for (uint32_t l = 0u; l < nl; ++l) clusters[weld(l)].push_back(l);
+        auto exclude_links = [&](uint32_t la, uint32_t lb) {
+            if (la == lb) return;   // the rows of one link are excluded by the cook
+            for (uint32_t ra : link_rows[la]) for (uint32_t rb : link_rows[lb]) {
+                if (s.shape_kind[ra] == 0xFFFFFFFFu || s.shape_kind[rb] == 0xFFFFFFFFu) continue;   // a row without a shape meets nothing
+                s.excluded_pairs.push_back(ra); s.excluded_pairs.push_back(rb);
+            }
+        };
+        for (uint32_t root = 0u; root < nl; ++root) {
+            const auto& members = clusters[root];
+            for (size_t i = 0u; i < members.size(); ++i) for (size_t k = i + 1u; k < members.size(); ++k) exclude_links(members[i], members[k]);
+            if (members.empty() || b.links[root].parent == 0xFFFFFFFFu) continue;
+            for (uint32_t other : clusters[weld(b.links[root].parent)]) for (uint32_t member : members) exclude_links(member, other);
+        }
+        for (const auto& names : b.excluded_bodies) {
+            uint32_t found[2] = {0xFFFFFFFFu, 0xFFFFFFFFu};
+            for (uint32_t l = 0u; l < nl; ++l) for (int k = 0; k < 2; ++k) if (!b.links[l].intermediate && b.links[l].name == (k == 0 ? names.first : names.second)) found[k] = l;
+            if (found[0] == 0xFFFFFFFFu || found[1] == 0xFFFFFFFFu) throw std::runtime_error("MJCF: <exclude> names an unknown body");
+            exclude_links(found[0], found[1]);
+        }
     }
     (void)any_friction_profile;
     s.dropped_geom_count = b.dropped_geoms;
@@ -944,6 +988,8 @@ void Scene::Bind() {
     desc.joint_limit_flags = joint_limit_flags.data(); desc.joint_frictionloss = joint_frictionloss.data();
     desc.drive_mode = drive_mode;
     desc.drive_rows = 1u;   // the reference always cooks one drive row per link (src/nk/pipeline/world.cpp:61)
+    desc.excluded_pairs = excluded_pairs.data();
+    desc.excluded_pair_count = uint32_t(excluded_pairs.size() / 2u);
 }
 
 }  // namespace mjcf

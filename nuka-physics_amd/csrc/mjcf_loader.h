@@ -21,7 +21,8 @@ struct Scene {
     nuka_template_desc_t desc{};
     std::vector<std::string> link_names, joint_names;
     std::vector<uint8_t> joint_type, joint_limit_flags;
-    std::vector<uint32_t> parent_link, body_role, body_link, shape_kind, shape_contype, shape_conaffinity, shape_group, shape_profile;
+    std::vector<uint32_t> parent_link, body_role, body_link, shape_kind, shape_contype, shape_conaffinity, shape_group, shape_profile,
+        excluded_pairs;   // [pair][2] collidable rows that never pair
     std::vector<float> joint_axis, link_local_pose, link_inertial_frame, link_mass, link_diag_inertia, joint_damping, joint_armature,
         joint_stiffness, joint_spring_reference, joint_frictionloss, joint_limit_lower, joint_limit_upper, body_local, shape_params, profile_mu;
     std::vector<float> initial_q, drive_stiffness, drive_damping, drive_force_limit, drive_joint_force_limit;

@@ -31,7 +31,7 @@ constexpr uint32_t kRowsPerPoint = 4u;     // src/nk/solve/nk_row.hpp:61
 // src/phi/articulation_contract.hpp:8-16
 enum : uint8_t { kRevolute = 0, kPrismatic = 1, kFixed = 2, kFloatingBase = 3, kSpherical = 4 };
 // src/collision/shape_kind.hpp:9-18
-enum : uint32_t { kShapeSphere = 0, kShapeCapsule = 1, kShapeBox = 2, kShapePlane = 3 };
+enum : uint32_t { kShapeSphere = 0, kShapeCapsule = 1, kShapeBox = 2, kShapePlane = 3, kShapeCylinder = 7 };
 // src/nk/solve/nk_row.hpp:14-19
 enum : uint32_t { kSideRigid = 0, kSideArtic = 1, kSideStatic = 3 };
 // src/nk/solve/nk_row.hpp:41-57
@@ -54,7 +54,8 @@ constexpr uint32_t kContactLawSpeculative = 2u;   // src/nk/solve/nk_row.hpp:37
 struct ModelView {
     uint32_t links_per_env, bodies_per_env, dof, max_dof, max_depth, contact_slots, rows_per_env, contact_rows_per_env;
     uint32_t profile_count, floating_root;
-    uint32_t max_points_per_slot;   // 1 when no box can meet a plane, else 4 (sizes the solver's staged rows)
+    uint32_t max_points_per_slot;   // most points a manifold of the template's admitted pairs can hold (sizes the solver's staged rows)
+    uint32_t excluded_pair_count;
     // joint row slots after the contact rows: 2 per link, 1 per link, 1 per link, or 0 (scene/cook/cook_to_model.cpp:706-719)
     uint32_t joint_limit_rows, joint_friction_rows, joint_drive_rows, drive_mode;
     const uint8_t* joint_type;
@@ -89,6 +90,7 @@ struct ModelView {
     const uint32_t* body_collidable_body;
     const float* body_collidable_local;
     const float* profile_mu;
+    const uint64_t* excluded_pairs;   // sorted (a << 32 | b) keys of collidable rows that never pair, a < b
 };
 
 // Mutable per-environment fields, env-major with the element layout of the reference's public fields

@@ -1,5 +1,6 @@
 // Contact detection and row assembly for gfx950: collidable poses, AABBs, candidate pairs in canonical (a, b)
-// order, sphere/box x plane manifolds, pair-driven contact rows and chain Jacobians.
+// order, the analytic manifolds of sphere, capsule, box, plane and cylinder pairs, pair-driven contact rows and chain
+// Jacobians.
 //
 // Elementwise stages run one thread per (env, item) on contiguous env-major fields; the stages with an order
 // inside an environment (pair emission, row-range prefix, Jacobian rows) run one wavefront per environment so the
@@ -72,8 +73,16 @@ __global__ void BuildAabbsKernel(ModelView m, DataView d, BuildAabbsParams p) {
     float* hi = d.body_aabb_hi + size_t{gid} * 3u;
     V3 he{0, 0, 0};
     if (s.kind == kShapeSphere) he = V3{s.p[0], s.p[0], s.p[0]};
+    else if (s.kind == kShapeCapsule) he = rot_abs(xf.r, V3{s.p[0], s.p[0], s.p[0] + s.p[1]});
     else if (s.kind == kShapeBox) he = rot_abs(xf.r, V3{s.p[0], s.p[1], s.p[2]});
-    else if (s.kind == kShapePlane) {
+    else if (s.kind == kShapeCylinder) {   // per world axis hh |a_i| + r sqrt(1 - a_i^2) for the cylinder's axis a
+        const V3 qv{xf.r.x, xf.r.y, xf.r.z}, ez{0, 0, 1};
+        const V3 tz = scale3(cross3(qv, ez), 2.0f);
+        const V3 a = add3(add3(ez, scale3(tz, xf.r.w)), cross3(qv, tz));
+        he = V3{s.p[1] * fabsf(a.x) + s.p[0] * sqrtf(fmaxf(0.0f, 1.0f - a.x * a.x)),
+                s.p[1] * fabsf(a.y) + s.p[0] * sqrtf(fmaxf(0.0f, 1.0f - a.y * a.y)),
+                s.p[1] * fabsf(a.z) + s.p[0] * sqrtf(fmaxf(0.0f, 1.0f - a.z * a.z))};
+    } else if (s.kind == kShapePlane) {
         lo[0] = lo[1] = lo[2] = -FLT_MAX; hi[0] = hi[1] = hi[2] = FLT_MAX;
         return;
     } else {
@@ -91,6 +100,17 @@ __device__ __forceinline__ bool shape_filter_admits(uint32_t ta, uint32_t aa, ui
     if (((ta & ab) | (tb & aa)) == 0u) return false;
     const int32_t ga = int32_t(ga_), gb = int32_t(gb_);
     return !(ga != 0 && gb != 0 && (ga > 0 ? (ga != gb && gb > 0) : ga == gb));
+}
+
+// broadphase.cu:87-99 IsExcluded: binary search of the sorted (a << 32 | b) keys, a < b
+__device__ bool pair_excluded(const ModelView& m, uint32_t a, uint32_t b) {
+    const uint64_t key = (uint64_t{a} << 32u) | uint64_t{b};
+    uint32_t lo = 0u, hi = m.excluded_pair_count;
+    while (lo < hi) {
+        const uint32_t mid = lo + (hi - lo) / 2u;
+        if (m.excluded_pairs[mid] < key) lo = mid + 1u; else hi = mid;
+    }
+    return lo < m.excluded_pair_count && m.excluded_pairs[lo] == key;
 }
 
 // ---- candidate pairs: one wavefront per env walks the (i, j) grid in row-major order; the ballot rank of an
@@ -113,7 +133,8 @@ __global__ void __launch_bounds__(kWave) QueryPairsKernel(ModelView m, DataView 
             if (overlap) {
                 const ShapeRow sa = load_shape(m.shape_table, i), sb = load_shape(m.shape_table, j);
                 emit = !(sa.body_id < 0 && sb.body_id < 0) &&
-                       shape_filter_admits(sa.contype, sa.conaffinity, sa.group, sb.contype, sb.conaffinity, sb.group);
+                       shape_filter_admits(sa.contype, sa.conaffinity, sa.group, sb.contype, sb.conaffinity, sb.group) &&
+                       !pair_excluded(m, i, j);
             }
         }
         const uint64_t mask = __ballot(emit);
@@ -133,46 +154,38 @@ __global__ void __launch_bounds__(kWave) QueryPairsKernel(ModelView m, DataView 
 }
 
 // ---- manifolds (collision/analytical_manifold.hpp) ------------------------------------------------------
-struct Prim { V3 cx, cy, cz, t; float radius; V3 half; };
+struct Prim { V3 cx, cy, cz, t; float radius, half_height; V3 half; };
 struct Manifold { uint32_t count; V3 position[4]; V3 normal; float penetration[4]; uint32_t key[4]; };
 
 __device__ Prim make_prim(const ShapeRow& s, Xf xf) {   // narrowphase_prims.cu:34-46
     Prim p;
     p.cx = rotate_raw(xf.r, V3{1, 0, 0}); p.cy = rotate_raw(xf.r, V3{0, 1, 0}); p.cz = rotate_raw(xf.r, V3{0, 0, 1});
-    p.t = xf.p; p.radius = s.p[0]; p.half = V3{s.p[0], s.p[1], s.p[2]};
+    p.t = xf.p; p.radius = s.p[0]; p.half_height = s.p[1]; p.half = V3{s.p[0], s.p[1], s.p[2]};
     return p;
 }
-__device__ V3 plane_normal(const Prim& plane) {   // analytical_manifold.hpp:194-198 with the +Z fallback
-    const float len = sqrtf(plane.cz.x * plane.cz.x + plane.cz.y * plane.cz.y + plane.cz.z * plane.cz.z);
-    if (len < 1.0e-12f) return V3{0, 0, 1};
-    return V3{plane.cz.x / len, plane.cz.y / len, plane.cz.z / len};
+__device__ V3 norm_or(V3 v, V3 fallback) {   // analytical_manifold.hpp:194-198 Norm
+    const float len = sqrtf(v.x * v.x + v.y * v.y + v.z * v.z);
+    if (len < 1.0e-12f) return fallback;
+    return V3{v.x / len, v.y / len, v.z / len};
 }
-__device__ void sphere_plane(const Prim& sph, const Prim& plane, float query, Manifold* out) {   // :451-463
-    out->count = 0u;
-    const V3 n = plane_normal(plane);
-    const float signed_dist = dot3(sub3(sph.t, plane.t), n);
-    const float pen = sph.radius - signed_dist;
-    if (pen <= -query) return;
-    out->position[0] = sub3(sph.t, scale3(n, sph.radius - 0.5f * pen));
-    out->normal = n; out->penetration[0] = pen; out->key[0] = 0u; out->count = 1u;
+// analytical_manifold.hpp:69-93 PrimFrame
+__device__ V3 frame_local_to_world(const Prim& f, V3 l) {
+    return V3{f.cx.x * l.x + f.cy.x * l.y + f.cz.x * l.z + f.t.x, f.cx.y * l.x + f.cy.y * l.y + f.cz.y * l.z + f.t.y,
+              f.cx.z * l.x + f.cy.z * l.y + f.cz.z * l.z + f.t.z};
 }
-__device__ void box_plane(const Prim& box, const Prim& plane, float query, Manifold* out) {   // :469-493, 273-311
+__device__ V3 frame_world_to_local(const Prim& f, V3 w) {
+    const V3 d = sub3(w, f.t);
+    return V3{dot3(d, f.cx), dot3(d, f.cy), dot3(d, f.cz)};
+}
+__device__ V3 frame_dir_to_world(const Prim& f, V3 l) {
+    return V3{f.cx.x * l.x + f.cy.x * l.y + f.cz.x * l.z, f.cx.y * l.x + f.cy.y * l.y + f.cz.y * l.z,
+              f.cx.z * l.x + f.cy.z * l.y + f.cz.z * l.z};
+}
+
+// analytical_manifold.hpp:273-311 ReduceAndEmit: the four deepest candidates (ties to the smaller feature id), emitted
+// in ascending feature order
+__device__ void reduce_and_emit(V3* position, float* pen, uint32_t* feature, int ncand, V3 n, Manifold* out) {
     out->count = 0u;
-    const V3 n = plane_normal(plane);
-    V3 position[8]; float pen[8]; uint32_t feature[8];
-    int ncand = 0;
-    for (uint32_t c = 0u; c < 8u; ++c) {
-        const float sx = (c & 1u) ? 1.0f : -1.0f, sy = (c & 2u) ? 1.0f : -1.0f, sz = (c & 4u) ? 1.0f : -1.0f;
-        const V3 l{sx * box.half.x, sy * box.half.y, sz * box.half.z};
-        const V3 corner{box.cx.x * l.x + box.cy.x * l.y + box.cz.x * l.z + box.t.x,
-                        box.cx.y * l.x + box.cy.y * l.y + box.cz.y * l.z + box.t.y,
-                        box.cx.z * l.x + box.cy.z * l.y + box.cz.z * l.z + box.t.z};
-        const float sd = dot3(sub3(corner, plane.t), n);
-        if (sd < query) {
-            position[ncand] = sub3(corner, scale3(n, 0.5f * sd));
-            pen[ncand] = -sd; feature[ncand] = c; ++ncand;
-        }
-    }
     if (ncand <= 0) return;
     const int keep = ncand < 4 ? ncand : 4;
     for (int s = 0; s < keep; ++s) {
@@ -192,6 +205,270 @@ __device__ void box_plane(const Prim& box, const Prim& plane, float query, Manif
     for (int i = 0; i < keep; ++i) { out->position[i] = position[i]; out->penetration[i] = pen[i]; out->key[i] = feature[i]; }
     out->normal = n;
     out->count = uint32_t(keep);
+}
+
+// analytical_manifold.hpp:337-405 ReduceAndEmitSpread: up to four candidates as they are; of more, the deepest and then,
+// three times, the one farthest from those kept (ties to the lower index); ascending feature order
+__device__ void reduce_and_emit_spread(const V3* position, const float* pen, const uint32_t* feature, int n, V3 normal, Manifold* out) {
+    out->count = 0u;
+    if (n <= 0) return;
+    int kept[4] = {0, 1, 2, 3};
+    int count = n;
+    if (n > 4) {
+        uint32_t used = 0u;
+        int seed = 0;
+        for (int i = 1; i < n; ++i) if (pen[i] > pen[seed]) seed = i;
+        kept[0] = seed; used |= 1u << seed;
+        for (int s = 1; s < 4; ++s) {
+            int best = -1; float best_mind = -1.0f;
+            for (int i = 0; i < n; ++i) {
+                if ((used >> i) & 1u) continue;
+                float mind = 3.4e38f;
+                for (int t = 0; t < s; ++t) {
+                    const V3 d = sub3(position[i], position[kept[t]]);
+                    const float dd = dot3(d, d);
+                    if (dd < mind) mind = dd;
+                }
+                if (mind > best_mind) { best_mind = mind; best = i; }
+            }
+            kept[s] = best; used |= 1u << best;   // more than four candidates: every round finds one
+        }
+        count = 4;
+    }
+    for (int i = 1; i < count; ++i) {
+        const int key = kept[i]; int j = i - 1;
+        while (j >= 0 && feature[kept[j]] > feature[key]) { kept[j + 1] = kept[j]; --j; }
+        kept[j + 1] = key;
+    }
+    for (int i = 0; i < count; ++i) { out->position[i] = position[kept[i]]; out->penetration[i] = pen[kept[i]]; out->key[i] = feature[kept[i]]; }
+    out->normal = normal;
+    out->count = uint32_t(count);
+}
+
+// collision/primitive_surface.hpp:28-122 QueryPrimitiveSurface: signed distance (positive outside), outward normal,
+// closest surface point and feature of a point in the primitive's own frame
+struct Surface { float distance; V3 normal, point; uint32_t feature; bool valid; };
+__device__ Surface query_surface(uint32_t kind, V3 par, V3 pos) {
+    Surface r{0.0f, V3{1, 0, 0}, V3{0, 0, 0}, 0u, false};
+    if (kind == kShapeSphere || kind == kShapeCapsule) {
+        if (!(par.x >= 0.0f)) return r;
+        V3 offset = pos;
+        if (kind == kShapeCapsule) {
+            if (!(par.y >= 0.0f)) return r;
+            offset.z -= fmaxf(-par.y, fminf(pos.z, par.y));
+            r.feature = pos.z < -par.y ? 0u : pos.z > par.y ? 2u : 1u;
+        }
+        const float length = sqrtf(dot3(offset, offset));
+        if (length > 0.0f) r.normal = V3{offset.x / length, offset.y / length, offset.z / length};
+        r.distance = length - par.x;
+    } else if (kind == kShapeBox) {
+        if (!(par.x >= 0.0f && par.y >= 0.0f && par.z >= 0.0f)) return r;
+        const V3 closest{fmaxf(-par.x, fminf(pos.x, par.x)), fmaxf(-par.y, fminf(pos.y, par.y)), fmaxf(-par.z, fminf(pos.z, par.z))};
+        const V3 offset = sub3(pos, closest);
+        const float length = sqrtf(dot3(offset, offset));
+        if (length > 0.0f) {
+            r.distance = length;
+            r.normal = V3{offset.x / length, offset.y / length, offset.z / length};
+            if (offset.x != 0.0f) r.feature |= 1u << (pos.x < 0.0f ? 0u : 1u);
+            if (offset.y != 0.0f) r.feature |= 1u << (pos.y < 0.0f ? 2u : 3u);
+            if (offset.z != 0.0f) r.feature |= 1u << (pos.z < 0.0f ? 4u : 5u);
+        } else {
+            const V3 dist{fabsf(pos.x) - par.x, fabsf(pos.y) - par.y, fabsf(pos.z) - par.z};
+            if (dist.x >= dist.y && dist.x >= dist.z) {
+                r.distance = dist.x; r.normal = V3{pos.x < 0.0f ? -1.0f : 1.0f, 0, 0}; r.feature = 1u << (pos.x < 0.0f ? 0u : 1u);
+            } else if (dist.y >= dist.z) {
+                r.distance = dist.y; r.normal = V3{0, pos.y < 0.0f ? -1.0f : 1.0f, 0}; r.feature = 1u << (pos.y < 0.0f ? 2u : 3u);
+            } else {
+                r.distance = dist.z; r.normal = V3{0, 0, pos.z < 0.0f ? -1.0f : 1.0f}; r.feature = 1u << (pos.z < 0.0f ? 4u : 5u);
+            }
+        }
+    } else if (kind == kShapeCylinder) {   // features: 0 bottom cap, 1 side, 2 top cap, 3 bottom rim, 4 top rim
+        if (!(par.x >= 0.0f && par.y >= 0.0f)) return r;
+        const float rho = sqrtf(pos.x * pos.x + pos.y * pos.y);
+        const V3 radial = rho > 0.0f ? V3{pos.x / rho, pos.y / rho, 0.0f} : V3{1, 0, 0};
+        const V3 axial{0, 0, pos.z < 0.0f ? -1.0f : 1.0f};
+        const float side = rho - par.x, cap = fabsf(pos.z) - par.y;
+        if (side > 0.0f && cap > 0.0f) {
+            r.distance = sqrtf(side * side + cap * cap);
+            const V3 sum = add3(scale3(radial, side), scale3(axial, cap));
+            r.normal = V3{sum.x / r.distance, sum.y / r.distance, sum.z / r.distance};
+            r.feature = pos.z < 0.0f ? 3u : 4u;
+        } else if (side > cap) {
+            r.distance = side; r.normal = radial; r.feature = 1u;
+        } else {
+            r.distance = cap; r.normal = axial; r.feature = pos.z < 0.0f ? 0u : 2u;
+        }
+    } else return r;
+    r.point = sub3(pos, scale3(r.normal, r.distance));
+    r.valid = true;
+    return r;
+}
+
+__device__ void emit_one(Manifold* out, V3 position, V3 normal, float pen, uint32_t key) {
+    out->position[0] = position; out->normal = normal; out->penetration[0] = pen; out->key[0] = key; out->count = 1u;
+}
+__device__ void sphere_sphere(const Prim& a, const Prim& b, float query, Manifold* out) {   // :416-429
+    out->count = 0u;
+    const V3 delta = sub3(a.t, b.t);
+    const float dist = sqrtf(delta.x * delta.x + delta.y * delta.y + delta.z * delta.z);
+    const float pen = (a.radius + b.radius) - dist;
+    if (pen <= -query) return;
+    const V3 n = norm_or(delta, V3{0, 1, 0});
+    emit_one(out, add3(b.t, scale3(n, b.radius - 0.5f * pen)), n, pen, 0u);
+}
+__device__ void sphere_box(const Prim& sph, const Prim& box, float query, Manifold* out) {   // :434-448
+    out->count = 0u;
+    const Surface s = query_surface(kShapeBox, box.half, frame_world_to_local(box, sph.t));
+    if (!s.valid) return;
+    const float pen = sph.radius - s.distance;
+    if (pen <= -query) return;
+    const V3 normal = frame_dir_to_world(box, s.normal);
+    emit_one(out, sub3(frame_local_to_world(box, s.point), scale3(normal, 0.5f * pen)), normal, pen, 0u);
+}
+__device__ void sphere_plane(const Prim& sph, const Prim& plane, float query, Manifold* out) {   // :451-463
+    out->count = 0u;
+    const V3 n = norm_or(plane.cz, V3{0, 0, 1});
+    const float signed_dist = dot3(sub3(sph.t, plane.t), n);
+    const float pen = sph.radius - signed_dist;
+    if (pen <= -query) return;
+    emit_one(out, sub3(sph.t, scale3(n, sph.radius - 0.5f * pen)), n, pen, 0u);
+}
+__device__ void box_plane(const Prim& box, const Prim& plane, float query, Manifold* out) {   // :469-493
+    out->count = 0u;
+    const V3 n = norm_or(plane.cz, V3{0, 0, 1});
+    V3 position[8]; float pen[8]; uint32_t feature[8];
+    int ncand = 0;
+    for (uint32_t c = 0u; c < 8u; ++c) {
+        const float sx = (c & 1u) ? 1.0f : -1.0f, sy = (c & 2u) ? 1.0f : -1.0f, sz = (c & 4u) ? 1.0f : -1.0f;
+        const V3 corner = frame_local_to_world(box, V3{sx * box.half.x, sy * box.half.y, sz * box.half.z});
+        const float sd = dot3(sub3(corner, plane.t), n);
+        if (sd < query) {
+            position[ncand] = sub3(corner, scale3(n, 0.5f * sd));
+            pen[ncand] = -sd; feature[ncand] = c; ++ncand;
+        }
+    }
+    reduce_and_emit(position, pen, feature, ncand, n, out);
+}
+__device__ void capsule_plane(const Prim& cap, const Prim& plane, float query, Manifold* out) {   // :738-759
+    out->count = 0u;
+    const V3 n = norm_or(plane.cz, V3{0, 0, 1});
+    const V3 ends[2] = {add3(cap.t, scale3(cap.cz, cap.half_height)), sub3(cap.t, scale3(cap.cz, cap.half_height))};
+    V3 position[2]; float pen[2]; uint32_t feature[2];
+    int ncand = 0;
+    for (uint32_t k = 0u; k < 2u; ++k) {
+        const float sd = dot3(sub3(ends[k], plane.t), n) - cap.radius;
+        if (sd < query) {
+            position[ncand] = sub3(ends[k], scale3(n, cap.radius + 0.5f * sd));
+            pen[ncand] = -sd; feature[ncand] = k; ++ncand;
+        }
+    }
+    reduce_and_emit(position, pen, feature, ncand, n, out);
+}
+__device__ void capsule_sphere(const Prim& cap, const Prim& sph, float query, Manifold* out) {   // :764-778
+    out->count = 0u;
+    const Surface s = query_surface(kShapeCapsule, V3{cap.radius, cap.half_height, 0.0f}, frame_world_to_local(cap, sph.t));
+    if (!s.valid) return;
+    const float pen = sph.radius - s.distance;
+    if (pen <= -query) return;
+    const V3 normal = scale3(frame_dir_to_world(cap, s.normal), -1.0f);
+    emit_one(out, add3(frame_local_to_world(cap, s.point), scale3(normal, 0.5f * pen)), normal, pen, 0u);
+}
+// :780-815: the lower cap's octagon and deepest point when a cap faces the plane, else each cap's deepest point
+__device__ void cylinder_plane(const Prim& cyl, const Prim& plane, float query, Manifold* out) {
+    out->count = 0u;
+    constexpr float kS = 0.70710678f;
+    const float rc[8] = {1.0f, kS, 0.0f, -kS, -1.0f, -kS, 0.0f, kS};
+    const float rs[8] = {0.0f, kS, 1.0f, kS, 0.0f, -kS, -1.0f, -kS};
+    const V3 n = norm_or(plane.cz, V3{0, 0, 1});
+    const V3 axis = cyl.cz;
+    const float d = dot3(axis, n);
+    const bool on_cap = fabsf(d) >= 0.95f;
+    const V3 down = norm_or(sub3(scale3(axis, d), n), cyl.cx);
+    V3 position[10]; float pen[10]; uint32_t feature[10];
+    int ncand = 0;
+    for (int cap = 0; cap < 2; ++cap) {
+        if (on_cap && (cap == 0) == (d > 0.0f)) continue;
+        const V3 center = add3(cyl.t, scale3(axis, cap == 0 ? cyl.half_height : -cyl.half_height));
+        for (int k = -1; k < (on_cap ? 8 : 0); ++k) {
+            const V3 dir = k < 0 ? down : add3(scale3(cyl.cx, rc[k]), scale3(cyl.cy, rs[k]));
+            const V3 p = add3(center, scale3(dir, cyl.radius));
+            const float sd = dot3(sub3(p, plane.t), n);
+            if (sd >= query) continue;
+            position[ncand] = sub3(p, scale3(n, sd * 0.5f));
+            pen[ncand] = -sd;
+            feature[ncand] = uint32_t(k < 0 ? cap : 2 + cap * 8 + k);
+            ++ncand;
+        }
+    }
+    reduce_and_emit_spread(position, pen, feature, ncand, n, out);
+}
+__device__ void cylinder_sphere(const Prim& cyl, const Prim& sph, float query, Manifold* out) {   // :819-834
+    out->count = 0u;
+    const Surface s = query_surface(kShapeCylinder, V3{cyl.radius, cyl.half_height, 0.0f}, frame_world_to_local(cyl, sph.t));
+    if (!s.valid) return;
+    const float pen = sph.radius - s.distance;
+    if (pen <= -query) return;
+    const V3 normal = scale3(frame_dir_to_world(cyl, s.normal), -1.0f);
+    emit_one(out, add3(frame_local_to_world(cyl, s.point), scale3(normal, 0.5f * pen)), normal, pen, s.feature);
+}
+// :841-896 ClosestPtSegmentSegment (fixed branch order)
+__device__ __forceinline__ float clamp01(float v) { return v < 0.0f ? 0.0f : (v > 1.0f ? 1.0f : v); }
+__device__ float closest_segment_segment(V3 p1, V3 q1, V3 p2, V3 q2, V3* c1_out, V3* c2_out) {
+    const V3 d1 = sub3(q1, p1), d2 = sub3(q2, p2), r = sub3(p1, p2);
+    const float a = dot3(d1, d1), e = dot3(d2, d2), f = dot3(d2, r);
+    float s = 0.0f, t = 0.0f;
+    const float eps = 1.0e-12f;
+    if (a <= eps && e <= eps) { s = 0.0f; t = 0.0f; }
+    else if (a <= eps) { s = 0.0f; t = clamp01(f / e); }
+    else {
+        const float c = dot3(d1, r);
+        if (e <= eps) { t = 0.0f; s = clamp01(-c / a); }
+        else {
+            const float b = dot3(d1, d2);
+            const float denom = a * e - b * b;
+            s = denom > eps ? clamp01((b * f - c * e) / denom) : 0.0f;
+            t = (b * s + f) / e;
+            if (t < 0.0f) { t = 0.0f; s = clamp01(-c / a); }
+            else if (t > 1.0f) { t = 1.0f; s = clamp01((b - c) / a); }
+        }
+    }
+    const V3 c1 = add3(p1, scale3(d1, s)), c2 = add3(p2, scale3(d2, t));
+    *c1_out = c1; *c2_out = c2;
+    const V3 dv = sub3(c1, c2);
+    return dot3(dv, dv);
+}
+__device__ void capsule_capsule(const Prim& a, const Prim& b, float query, Manifold* out) {   // :905-932
+    out->count = 0u;
+    const V3 a0 = add3(a.t, scale3(a.cz, a.half_height)), a1 = sub3(a.t, scale3(a.cz, a.half_height));
+    const V3 b0 = add3(b.t, scale3(b.cz, b.half_height)), b1 = sub3(b.t, scale3(b.cz, b.half_height));
+    V3 ca, cb;
+    const float dist = sqrtf(closest_segment_segment(a0, a1, b0, b1, &ca, &cb));
+    const float pen = (a.radius + b.radius) - dist;
+    if (pen <= -query) return;
+    const V3 n = norm_or(sub3(ca, cb), norm_or(cross3(a.cz, b.cz), V3{0, 1, 0}));
+    const V3 sa = sub3(ca, scale3(n, a.radius)), sb = add3(cb, scale3(n, b.radius));
+    emit_one(out, scale3(add3(sa, sb), 0.5f), n, pen, 0u);
+}
+// :934-971 PrimitivePair, every analytic pair but box x box; a flipped pair negates the normal
+__device__ void primitive_pair(uint32_t ka, const Prim& a, uint32_t kb, const Prim& b, float query, Manifold* out) {
+    out->count = 0u;
+    if (ka == kShapeSphere && kb == kShapeSphere) { sphere_sphere(a, b, query, out); return; }
+    if (ka == kShapeSphere && kb == kShapeBox) { sphere_box(a, b, query, out); return; }
+    if (ka == kShapeSphere && kb == kShapePlane) { sphere_plane(a, b, query, out); return; }
+    if (ka == kShapeBox && kb == kShapePlane) { box_plane(a, b, query, out); return; }
+    if (ka == kShapeCapsule && kb == kShapePlane) { capsule_plane(a, b, query, out); return; }
+    if (ka == kShapeCapsule && kb == kShapeSphere) { capsule_sphere(a, b, query, out); return; }
+    if (ka == kShapeCapsule && kb == kShapeCapsule) { capsule_capsule(a, b, query, out); return; }
+    if (ka == kShapeCylinder && kb == kShapePlane) { cylinder_plane(a, b, query, out); return; }
+    if (ka == kShapeCylinder && kb == kShapeSphere) { cylinder_sphere(a, b, query, out); return; }
+    if (ka == kShapeBox && kb == kShapeSphere) sphere_box(b, a, query, out);
+    else if (ka == kShapePlane && kb == kShapeSphere) sphere_plane(b, a, query, out);
+    else if (ka == kShapePlane && kb == kShapeBox) box_plane(b, a, query, out);
+    else if (ka == kShapePlane && kb == kShapeCapsule) capsule_plane(b, a, query, out);
+    else if (ka == kShapeSphere && kb == kShapeCapsule) capsule_sphere(b, a, query, out);
+    else if (ka == kShapePlane && kb == kShapeCylinder) cylinder_plane(b, a, query, out);
+    else if (ka == kShapeSphere && kb == kShapeCylinder) cylinder_sphere(b, a, query, out);
+    out->normal = V3{-out->normal.x, -out->normal.y, -out->normal.z};
 }
 
 // nk/contact/contact_identity.hpp:98-157
@@ -230,12 +507,7 @@ __device__ uint32_t NarrowphaseSlot(const ModelView& m, const DataView& d, const
         xa = load_xf(d.body_pose + (bbase + a) * 7u); xb = load_xf(d.body_pose + (bbase + b) * 7u);
         const Prim pa = make_prim(sa, xa), pb = make_prim(sb, xb);
         const float query = fmaxf(separation, fminf(motion_radius(2.0f * separation, p.dt, 0.0f, 0.0f, 0.9f), p.query_reach));
-        if (sa.kind == kShapeSphere && sb.kind == kShapePlane) sphere_plane(pa, pb, query, &mf);
-        else if (sa.kind == kShapeBox && sb.kind == kShapePlane) box_plane(pa, pb, query, &mf);
-        else if (sa.kind == kShapePlane && (sb.kind == kShapeSphere || sb.kind == kShapeBox)) {
-            if (sb.kind == kShapeSphere) sphere_plane(pb, pa, query, &mf); else box_plane(pb, pa, query, &mf);
-            mf.normal = V3{-mf.normal.x, -mf.normal.y, -mf.normal.z};
-        }
+        primitive_pair(sa.kind, pa, sb.kind, pb, query, &mf);
         for (uint32_t i = 0u; i < mf.count; ++i) mf.penetration[i] += separation;
     }
     d.ucontact_count[gid] = mf.count;

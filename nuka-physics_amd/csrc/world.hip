@@ -4,6 +4,7 @@
 // pipeline} and src/c_abi/{device,world,buffer}.cpp.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstddef>
 #include <cstdio>
@@ -61,7 +62,7 @@ struct HostModel {
     std::vector<uint8_t> joint_type, joint_limit_flags;
     std::vector<uint32_t> parent_link, link_body, link_tree_depth, link_child_range, link_children, link_dof, dof_link, dof_component,
         link_geom_kind, body_to_link, body_to_articulation, body_collidable_link, body_collidable_body;
-    std::vector<uint64_t> link_dof_mask;
+    std::vector<uint64_t> link_dof_mask, excluded_pairs;
     std::vector<float> joint_axis, parent_offset, link_local_pose, link_inertial_frame, link_inertia, joint_damping, joint_armature,
         joint_stiffness, joint_spring_reference, joint_limit_lower, joint_limit_upper, joint_frictionloss, link_geom_local, shape_table, body_collidable_local, body_init_pose, profile_mu;
 };
@@ -150,7 +151,6 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
     m.body_init_pose.resize(size_t{nb} * 7u);
     m.profile_mu.assign(d.profile_mu, d.profile_mu + 2u * d.profile_count);
     auto bits = [](uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; };
-    bool any_box = false;
     for (uint32_t b = 0u; b < nb; ++b) {
         const uint32_t role = d.body_role[b], link = d.body_link[b];
         float* row = m.shape_table.data() + size_t{b} * kShapeStride;
@@ -159,7 +159,6 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
         row[5] = bits(d.shape_contype[b]); row[6] = bits(d.shape_conaffinity[b]); row[7] = bits(0u);
         row[8] = bits(role == 0u ? 0xFFFFFFFFu : b); row[9] = bits(d.shape_group[b]);
         row[10] = bits(0u); row[11] = bits(0u); row[12] = bits(d.shape_profile[b]);
-        any_box = any_box || d.shape_kind[b] == kShapeBox;
         const float id[7] = {0, 0, 0, 1, 0, 0, 0};
         std::memcpy(m.body_collidable_local.data() + 7u * b, id, sizeof(id));
         std::memcpy(m.body_init_pose.data() + 7u * b, id, sizeof(id));
@@ -179,21 +178,50 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
         m.body_collidable_body[b] = m.link_body[link];
         std::memcpy(m.body_collidable_local.data() + 7u * b, d.body_local + 7u * b, 7u * sizeof(float));
     }
-    // Manifolds built here: sphere and box against a plane, either order.  Any other admitted pair is refused at
-    // cook time instead of silently producing no contact.
-    uint32_t admitted = 0u;
+    // Excluded pairs (scene/cook/cook_to_model.cpp:1468-1490): the authored ones and every two rows of one link, as
+    // sorted (a << 32 | b) keys with a < b.
+    m.excluded_pairs.clear();
+    if (d.excluded_pairs != nullptr)
+        for (uint32_t k = 0u; k < d.excluded_pair_count; ++k) {
+            const uint32_t a = d.excluded_pairs[2u * k], b = d.excluded_pairs[2u * k + 1u];
+            if (a >= nb || b >= nb || a == b) throw std::invalid_argument("excluded pair names no two collidable rows");
+            m.excluded_pairs.push_back((uint64_t{std::min(a, b)} << 32u) | uint64_t{std::max(a, b)});
+        }
+    for (uint32_t i = 0u; i < nb; ++i)
+        for (uint32_t j = i + 1u; j < nb; ++j)
+            if (d.body_role[i] != 0u && d.body_role[j] != 0u && d.body_link[i] == d.body_link[j])
+                m.excluded_pairs.push_back((uint64_t{i} << 32u) | uint64_t{j});
+    std::sort(m.excluded_pairs.begin(), m.excluded_pairs.end());
+    m.excluded_pairs.erase(std::unique(m.excluded_pairs.begin(), m.excluded_pairs.end()), m.excluded_pairs.end());
+    // Manifolds built here: every analytic pair of the reference's PrimitivePair but box x box
+    // (collision/analytical_manifold.hpp:934-971).  Any other admitted pair is refused at cook time instead of
+    // silently producing no contact.
+    const auto points_of = [](uint32_t ka, uint32_t kb) -> uint32_t {   // most points of the pair's manifold, 0 for none
+        if (ka > kb) std::swap(ka, kb);
+        if (kb == kShapePlane) return ka == kShapeSphere ? 1u : ka == kShapeCapsule ? 2u : ka == kShapeBox ? 4u : 0u;
+        if (kb == kShapeCylinder) return ka == kShapeSphere ? 1u : ka == kShapePlane ? 4u : 0u;
+        if (ka == kShapeSphere) return kb <= kShapeBox ? 1u : 0u;                      // sphere x sphere, capsule, box
+        return ka == kShapeCapsule && kb == kShapeCapsule ? 1u : 0u;
+    };
+    uint32_t admitted = 0u, max_points = 1u;
     for (uint32_t i = 0u; i < nb; ++i) {
         const uint32_t kind = d.shape_kind[i];
-        if (kind != kInvalid && kind != kShapeSphere && kind != kShapeBox && kind != kShapePlane)
-            throw NotSupported("shape kind not supported on this path (sphere, box, plane)");
+        if (kind != kInvalid && kind != kShapeSphere && kind != kShapeCapsule && kind != kShapeBox && kind != kShapePlane && kind != kShapeCylinder)
+            throw NotSupported("shape kind not supported on this path (sphere, capsule, box, plane, cylinder)");
+        if ((kind == kShapeSphere || kind == kShapeCapsule || kind == kShapeCylinder) && !(d.shape_params[4u * i] >= 0.0f))
+            throw std::invalid_argument("negative shape radius");
+        if ((kind == kShapeCapsule || kind == kShapeCylinder) && !(d.shape_params[4u * i + 1u] >= 0.0f))
+            throw std::invalid_argument("negative shape half length");
         for (uint32_t j = i + 1u; j < nb; ++j) {
             if (d.body_role[i] == 0u && d.body_role[j] == 0u) continue;
             if (kind == kInvalid || d.shape_kind[j] == kInvalid) continue;
             if (((d.shape_contype[i] & d.shape_conaffinity[j]) | (d.shape_contype[j] & d.shape_conaffinity[i])) == 0u) continue;
             const int32_t ga = int32_t(d.shape_group[i]), gb = int32_t(d.shape_group[j]);   // shape_kind.hpp:26-33
             if (ga != 0 && gb != 0 && (ga > 0 ? ga != gb && gb > 0 : ga == gb)) continue;
-            if ((kind == kShapePlane) == (d.shape_kind[j] == kShapePlane))
-                throw NotSupported("admitted collidable pair has no manifold on this path (one side must be a plane)");
+            if (std::binary_search(m.excluded_pairs.begin(), m.excluded_pairs.end(), (uint64_t{i} << 32u) | uint64_t{j})) continue;
+            const uint32_t points = points_of(kind, d.shape_kind[j]);
+            if (points == 0u) throw NotSupported("admitted collidable pair has no manifold on this path (box x box, and capsule or cylinder against box, capsule x cylinder, cylinder x cylinder)");
+            max_points = std::max(max_points, points);
             ++admitted;
         }
     }
@@ -222,7 +250,8 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
     c.rows_per_env = c.contact_rows_per_env + c.joint_limit_rows + c.joint_friction_rows + c.joint_drive_rows;
     c.profile_count = d.profile_count;
     c.floating_root = m.joint_type[0] == kFloatingBase ? 1u : 0u;
-    c.max_points_per_slot = any_box ? 4u : 1u;
+    c.max_points_per_slot = max_points;
+    c.excluded_pair_count = uint32_t(m.excluded_pairs.size());
 }
 
 enum Dtype : uint8_t { kF32 = 0, kU32 = 1, kU64 = 2, kU8 = 3 };
@@ -266,7 +295,8 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(joint_limit_flags, kU8) X(link_body, kU32) X(link_tree_depth, kU32) X(link_child_range, kU32) X(link_children, kU32) \
     X(link_dof, kU32) X(dof_link, kU32) X(dof_component, kU32) X(link_dof_mask, kU64) X(link_geom_kind, kU32) \
     X(link_geom_local, kF32) X(shape_table, kF32) X(body_to_link, kU32) X(body_to_articulation, kU32) \
-    X(body_collidable_link, kU32) X(body_collidable_body, kU32) X(body_collidable_local, kF32) X(profile_mu, kF32)
+    X(body_collidable_link, kU32) X(body_collidable_body, kU32) X(body_collidable_local, kF32) X(profile_mu, kF32) \
+    X(excluded_pairs, kU64)
 
 uint32_t DtypeBytes(Dtype t) { return t == kU64 ? 8u : t == kU8 ? 1u : 4u; }
 
@@ -604,8 +634,9 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
     if (tmpl == nullptr || desc == nullptr || desc->env_count == 0u) return Error(NUKA_RESULT_INVALID_ARG, "template, desc and env_count are required");
     // a caller built against the header before the joint-row members passes the shorter size; those members read as zero
     constexpr size_t kTemplateBase = offsetof(nuka_template_desc_t, joint_limit_lower);
+    constexpr size_t kTemplateJointRows = offsetof(nuka_template_desc_t, excluded_pairs);
     constexpr size_t kWorldBase = offsetof(nuka_world_desc_t, solver_fold_drive_damping);
-    if ((tmpl->struct_size != sizeof(nuka_template_desc_t) && tmpl->struct_size != kTemplateBase) ||
+    if ((tmpl->struct_size != sizeof(nuka_template_desc_t) && tmpl->struct_size != kTemplateJointRows && tmpl->struct_size != kTemplateBase) ||
         (desc->struct_size != sizeof(nuka_world_desc_t) && desc->struct_size != kWorldBase))
         return Error(NUKA_RESULT_INVALID_ARG, "struct_size mismatch");
     nuka_template_desc_t template_copy{};

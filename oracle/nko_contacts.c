@@ -73,8 +73,16 @@ void nko_env_aabbs(nko_world* w, uint32_t env) {
         float* hi = w->body_aabb_hi + (bbase + b) * 3u;
         v3 he = v3_make(0, 0, 0);
         if (s.kind == NKO_SPHERE) he = v3_make(s.p[0], s.p[0], s.p[0]);
+        else if (s.kind == NKO_CAPSULE) he = rot_abs(xf.r, v3_make(s.p[0], s.p[0], s.p[0] + s.p[1]));
         else if (s.kind == NKO_BOX) he = rot_abs(xf.r, v3_make(s.p[0], s.p[1], s.p[2]));
-        else if (s.kind == NKO_PLANE) {
+        else if (s.kind == NKO_CYLINDER) {   /* per world axis hh |a_i| + r sqrt(1 - a_i^2) for the cylinder's axis a */
+            const v3 qv = v3_make(xf.r.x, xf.r.y, xf.r.z), ez = v3_make(0, 0, 1);
+            const v3 tz = v3_scale(v3_cross(qv, ez), 2.0f);
+            const v3 a = v3_add(v3_add(ez, v3_scale(tz, xf.r.w)), v3_cross(qv, tz));
+            he = v3_make(s.p[1] * fabsf(a.x) + s.p[0] * sqrtf(fmaxf(0.0f, 1.0f - a.x * a.x)),
+                         s.p[1] * fabsf(a.y) + s.p[0] * sqrtf(fmaxf(0.0f, 1.0f - a.y * a.y)),
+                         s.p[1] * fabsf(a.z) + s.p[0] * sqrtf(fmaxf(0.0f, 1.0f - a.z * a.z)));
+        } else if (s.kind == NKO_PLANE) {
             lo[0] = lo[1] = lo[2] = -FLT_MAX; hi[0] = hi[1] = hi[2] = FLT_MAX;
             continue;
         } else {
@@ -100,6 +108,18 @@ static int shape_filter_admits(uint32_t ta, uint32_t aa, uint32_t ga_, uint32_t 
  * Emission order is a race in the reference and is erased by the stable sort on (a, b); the
  * oracle enumerates i<j ascending, which already is that order.  Overflow keeps the first
  * `capacity` emitted pairs in the reference (racy); the oracle keeps the smallest keys. ---- */
+/* broadphase.cu:87-99 IsExcluded: binary search of the sorted (a << 32 | b) keys, a < b */
+int nko_template_pair_excluded(const nko_template* t, uint32_t a, uint32_t b) {
+    const uint64_t key = ((uint64_t)a << 32u) | (uint64_t)b;
+    uint32_t lo = 0u, hi = t->excluded_count;
+    while (lo < hi) {
+        const uint32_t mid = lo + (hi - lo) / 2u;
+        if (t->excluded_pairs[mid] < key) lo = mid + 1u; else hi = mid;
+    }
+    return lo < t->excluded_count && t->excluded_pairs[lo] == key;
+}
+int nko_pair_excluded(const nko_world* w, uint32_t a, uint32_t b) { return nko_template_pair_excluded(&w->t, a < b ? a : b, a < b ? b : a); }
+
 void nko_env_pairs(nko_world* w, uint32_t env) {
     const nko_template* t = &w->t;
     const size_t bbase = (size_t)env * t->nb;
@@ -116,6 +136,7 @@ void nko_env_pairs(nko_world* w, uint32_t env) {
             const shape_row sa = load_shape(t->shape_table, i), sb = load_shape(t->shape_table, j);
             if (sa.body_id < 0 && sb.body_id < 0) continue;
             if (!shape_filter_admits(sa.contype, sa.conaffinity, sa.group, sb.contype, sb.conaffinity, sb.group)) continue;
+            if (nko_template_pair_excluded(t, i, j)) continue;
             if (count < t->slots) { pairs[2u * count] = i; pairs[2u * count + 1u] = j; ++count; }
             else w->env_status[env] |= NKO_STATUS_PAIR_OVERFLOW;
         }
@@ -123,13 +144,13 @@ void nko_env_pairs(nko_world* w, uint32_t env) {
 }
 
 /* ---- manifolds (collision/analytical_manifold.hpp) ----------------------- */
-typedef struct { v3 cx, cy, cz, t; float radius; v3 half; } prim;
+typedef struct { v3 cx, cy, cz, t; float radius, half_height; v3 half; } prim;
 
 static prim make_prim(shape_row s, xform xf) {   /* narrowphase_prims.cu:34-46 MakePrim */
     prim p;
     p.cx = nko_prim_rotate(xf.r, v3_make(1, 0, 0)); p.cy = nko_prim_rotate(xf.r, v3_make(0, 1, 0));
     p.cz = nko_prim_rotate(xf.r, v3_make(0, 0, 1)); p.t = xf.p;
-    p.radius = s.p[0]; p.half = v3_make(s.p[0], s.p[1], s.p[2]);
+    p.radius = s.p[0]; p.half_height = s.p[1]; p.half = v3_make(s.p[0], s.p[1], s.p[2]);
     return p;
 }
 static v3 norm_or(v3 v, v3 fallback) {   /* analytical_manifold.hpp:194-198 Norm */
@@ -150,24 +171,10 @@ static void sphere_plane(const prim* sph, const prim* plane, float query, manifo
     out->normal[0] = n; out->penetration[0] = pen; out->key[0] = 0u; out->count = 1u;
 }
 
-/* analytical_manifold.hpp:469-493 BoxPlane + :273-311 ReduceAndEmit */
-static void box_plane(const prim* box, const prim* plane, float query, manifold* out) {
+/* analytical_manifold.hpp:273-311 ReduceAndEmit: the four deepest candidates (ties to the smaller feature id),
+ * emitted in ascending feature order */
+static void reduce_and_emit(v3* position, float* pen, uint32_t* feature, int ncand, v3 n, manifold* out) {
     out->count = 0u;
-    const v3 n = norm_or(plane->cz, v3_make(0, 0, 1));
-    v3 position[8]; float pen[8]; uint32_t feature[8];
-    int ncand = 0;
-    for (uint32_t c = 0u; c < 8u; ++c) {
-        const float sx = (c & 1u) ? 1.0f : -1.0f, sy = (c & 2u) ? 1.0f : -1.0f, sz = (c & 4u) ? 1.0f : -1.0f;
-        const v3 l = v3_make(sx * box->half.x, sy * box->half.y, sz * box->half.z);
-        const v3 corner = v3_make(box->cx.x * l.x + box->cy.x * l.y + box->cz.x * l.z + box->t.x,
-                                  box->cx.y * l.x + box->cy.y * l.y + box->cz.y * l.z + box->t.y,
-                                  box->cx.z * l.x + box->cy.z * l.y + box->cz.z * l.z + box->t.z);
-        const float sd = v3_dot(v3_sub(corner, plane->t), n);
-        if (sd < query) {
-            position[ncand] = v3_sub(corner, v3_scale(n, 0.5f * sd));
-            pen[ncand] = -sd; feature[ncand] = c; ++ncand;
-        }
-    }
     if (ncand <= 0) return;
     const int keep = ncand < 4 ? ncand : 4;
     for (int s = 0; s < keep; ++s) {
@@ -190,15 +197,325 @@ static void box_plane(const prim* box, const prim* plane, float query, manifold*
     out->count = (uint32_t)keep;
 }
 
-/* analytical_manifold.hpp:934-966 PrimitivePair (sphere/box x plane subset) */
-static void primitive_pair(uint32_t ka, const prim* a, uint32_t kb, const prim* b, float query, manifold* out) {
+/* analytical_manifold.hpp:337-405 ReduceAndEmitSpread: up to four candidates as they are; of more, the deepest
+ * and then, three times, the one farthest from those kept (ties to the lower index); ascending feature order */
+static void reduce_and_emit_spread(v3* position, float* pen, uint32_t* feature, int n, v3 normal, manifold* out) {
     out->count = 0u;
-    if (ka == NKO_SPHERE && kb == NKO_PLANE) { sphere_plane(a, b, query, out); return; }
-    if (ka == NKO_BOX && kb == NKO_PLANE) { box_plane(a, b, query, out); return; }
-    if (ka == NKO_PLANE && (kb == NKO_SPHERE || kb == NKO_BOX)) {
-        if (kb == NKO_SPHERE) sphere_plane(b, a, query, out); else box_plane(b, a, query, out);
-        for (uint32_t i = 0u; i < out->count; ++i) out->normal[i] = v3_make(-out->normal[i].x, -out->normal[i].y, -out->normal[i].z);
+    if (n <= 0) return;
+    int kept[4];
+    int count = n;
+    if (n <= 4) {
+        for (int i = 0; i < n; ++i) kept[i] = i;
+    } else {
+        int used[24] = {0};
+        int seed = 0;
+        for (int i = 1; i < n; ++i) if (pen[i] > pen[seed]) seed = i;
+        kept[0] = seed; used[seed] = 1;
+        count = 1;
+        for (int s = 1; s < 4; ++s) {
+            int best = -1; float best_mind = -1.0f;
+            for (int i = 0; i < n; ++i) {
+                if (used[i]) continue;
+                float mind = 3.4e38f;
+                for (int t = 0; t < s; ++t) {
+                    const v3 d = v3_sub(position[i], position[kept[t]]);
+                    const float dd = v3_dot(d, d);
+                    if (dd < mind) mind = dd;
+                }
+                if (mind > best_mind) { best_mind = mind; best = i; }
+            }
+            if (best < 0) break;
+            kept[s] = best; used[best] = 1; count = s + 1;
+        }
+        /* the reference sorts and emits four entries once more than four candidates exist; with n > 4 every
+         * round finds one, so count is 4 here */
     }
+    for (int i = 1; i < count; ++i) {
+        const int key = kept[i]; int j = i - 1;
+        while (j >= 0 && feature[kept[j]] > feature[key]) { kept[j + 1] = kept[j]; --j; }
+        kept[j + 1] = key;
+    }
+    for (int i = 0; i < count; ++i) {
+        out->position[i] = position[kept[i]]; out->normal[i] = normal; out->penetration[i] = pen[kept[i]]; out->key[i] = feature[kept[i]];
+    }
+    out->count = (uint32_t)count;
+}
+
+/* analytical_manifold.hpp:69-93 PrimFrame */
+static v3 frame_local_to_world(const prim* f, v3 l) {
+    return v3_make(f->cx.x * l.x + f->cy.x * l.y + f->cz.x * l.z + f->t.x,
+                   f->cx.y * l.x + f->cy.y * l.y + f->cz.y * l.z + f->t.y,
+                   f->cx.z * l.x + f->cy.z * l.y + f->cz.z * l.z + f->t.z);
+}
+static v3 frame_world_to_local(const prim* f, v3 w) {
+    const v3 d = v3_make(w.x - f->t.x, w.y - f->t.y, w.z - f->t.z);
+    return v3_make(d.x * f->cx.x + d.y * f->cx.y + d.z * f->cx.z,
+                   d.x * f->cy.x + d.y * f->cy.y + d.z * f->cy.z,
+                   d.x * f->cz.x + d.y * f->cz.y + d.z * f->cz.z);
+}
+static v3 frame_dir_to_world(const prim* f, v3 l) {
+    return v3_make(f->cx.x * l.x + f->cy.x * l.y + f->cz.x * l.z,
+                   f->cx.y * l.x + f->cy.y * l.y + f->cz.y * l.z,
+                   f->cx.z * l.x + f->cy.z * l.y + f->cz.z * l.z);
+}
+
+/* collision/primitive_surface.hpp:28-122 QueryPrimitiveSurface: signed distance (positive outside), outward normal,
+ * closest surface point and feature of a point in the primitive's own frame */
+typedef struct { float distance; v3 normal, point; uint32_t feature; int valid; } surface;
+static surface query_surface(uint32_t kind, v3 par, v3 pos) {
+    surface r; r.distance = 0.0f; r.normal = v3_make(1, 0, 0); r.point = v3_make(0, 0, 0); r.feature = 0u; r.valid = 0;
+    if (kind == NKO_SPHERE || kind == NKO_CAPSULE) {
+        if (!(par.x >= 0.0f)) return r;
+        v3 offset = pos;
+        if (kind == NKO_CAPSULE) {
+            if (!(par.y >= 0.0f)) return r;
+            const float axis = fmaxf(-par.y, fminf(pos.z, par.y));
+            offset.z -= axis;
+            r.feature = pos.z < -par.y ? 0u : pos.z > par.y ? 2u : 1u;
+        }
+        const float length = sqrtf(v3_dot(offset, offset));
+        if (length > 0.0f) r.normal = v3_make(offset.x / length, offset.y / length, offset.z / length);
+        r.distance = length - par.x;
+    } else if (kind == NKO_BOX) {
+        if (!(par.x >= 0.0f && par.y >= 0.0f && par.z >= 0.0f)) return r;
+        const v3 closest = v3_make(fmaxf(-par.x, fminf(pos.x, par.x)), fmaxf(-par.y, fminf(pos.y, par.y)), fmaxf(-par.z, fminf(pos.z, par.z)));
+        const v3 offset = v3_sub(pos, closest);
+        const float length = sqrtf(v3_dot(offset, offset));
+        if (length > 0.0f) {
+            r.distance = length;
+            r.normal = v3_make(offset.x / length, offset.y / length, offset.z / length);
+            if (offset.x != 0.0f) r.feature |= 1u << (pos.x < 0.0f ? 0u : 1u);
+            if (offset.y != 0.0f) r.feature |= 1u << (pos.y < 0.0f ? 2u : 3u);
+            if (offset.z != 0.0f) r.feature |= 1u << (pos.z < 0.0f ? 4u : 5u);
+        } else {
+            const v3 dist = v3_make(fabsf(pos.x) - par.x, fabsf(pos.y) - par.y, fabsf(pos.z) - par.z);
+            if (dist.x >= dist.y && dist.x >= dist.z) {
+                r.distance = dist.x; r.normal = v3_make(pos.x < 0.0f ? -1.0f : 1.0f, 0, 0); r.feature = 1u << (pos.x < 0.0f ? 0u : 1u);
+            } else if (dist.y >= dist.z) {
+                r.distance = dist.y; r.normal = v3_make(0, pos.y < 0.0f ? -1.0f : 1.0f, 0); r.feature = 1u << (pos.y < 0.0f ? 2u : 3u);
+            } else {
+                r.distance = dist.z; r.normal = v3_make(0, 0, pos.z < 0.0f ? -1.0f : 1.0f); r.feature = 1u << (pos.z < 0.0f ? 4u : 5u);
+            }
+        }
+    } else if (kind == NKO_PLANE) {
+        r.distance = pos.z; r.normal = v3_make(0, 0, 1);
+    } else if (kind == NKO_CYLINDER) {
+        if (!(par.x >= 0.0f && par.y >= 0.0f)) return r;
+        /* features: 0 bottom cap, 1 side, 2 top cap, 3 bottom rim, 4 top rim */
+        const float rho = sqrtf(pos.x * pos.x + pos.y * pos.y);
+        const v3 radial = rho > 0.0f ? v3_make(pos.x / rho, pos.y / rho, 0.0f) : v3_make(1, 0, 0);
+        const v3 axial = v3_make(0, 0, pos.z < 0.0f ? -1.0f : 1.0f);
+        const float side = rho - par.x;
+        const float cap = fabsf(pos.z) - par.y;
+        if (side > 0.0f && cap > 0.0f) {
+            r.distance = sqrtf(side * side + cap * cap);
+            const v3 sum = v3_add(v3_scale(radial, side), v3_scale(axial, cap));
+            r.normal = v3_make(sum.x / r.distance, sum.y / r.distance, sum.z / r.distance);
+            r.feature = pos.z < 0.0f ? 3u : 4u;
+        } else if (side > cap) {
+            r.distance = side; r.normal = radial; r.feature = 1u;
+        } else {
+            r.distance = cap; r.normal = axial; r.feature = pos.z < 0.0f ? 0u : 2u;
+        }
+    } else return r;
+    r.point = v3_sub(pos, v3_scale(r.normal, r.distance));
+    r.valid = 1;
+    return r;
+}
+
+static void emit_one(manifold* out, v3 position, v3 normal, float pen, uint64_t key) {
+    out->position[0] = position; out->normal[0] = normal; out->penetration[0] = pen; out->key[0] = key; out->count = 1u;
+}
+
+/* analytical_manifold.hpp:416-429 SphereSphere: the normal points from b to a, the point lies midway between the surfaces */
+static void sphere_sphere(const prim* a, const prim* b, float query, manifold* out) {
+    out->count = 0u;
+    const v3 delta = v3_sub(a->t, b->t);
+    const float dist = sqrtf(delta.x * delta.x + delta.y * delta.y + delta.z * delta.z);
+    const float pen = (a->radius + b->radius) - dist;
+    if (pen <= -query) return;
+    const v3 n = norm_or(delta, v3_make(0, 1, 0));
+    emit_one(out, v3_add(b->t, v3_scale(n, b->radius - 0.5f * pen)), n, pen, 0u);
+}
+
+/* analytical_manifold.hpp:434-448 SphereBox (a = sphere) */
+static void sphere_box(const prim* sph, const prim* box, float query, manifold* out) {
+    out->count = 0u;
+    const surface s = query_surface(NKO_BOX, box->half, frame_world_to_local(box, sph->t));
+    if (!s.valid) return;
+    const float pen = sph->radius - s.distance;
+    if (pen <= -query) return;
+    const v3 normal = frame_dir_to_world(box, s.normal);
+    emit_one(out, v3_sub(frame_local_to_world(box, s.point), v3_scale(normal, 0.5f * pen)), normal, pen, 0u);
+}
+
+/* analytical_manifold.hpp:469-493 BoxPlane */
+static void box_plane(const prim* box, const prim* plane, float query, manifold* out) {
+    out->count = 0u;
+    const v3 n = norm_or(plane->cz, v3_make(0, 0, 1));
+    v3 position[8]; float pen[8]; uint32_t feature[8];
+    int ncand = 0;
+    for (uint32_t c = 0u; c < 8u; ++c) {
+        const float sx = (c & 1u) ? 1.0f : -1.0f, sy = (c & 2u) ? 1.0f : -1.0f, sz = (c & 4u) ? 1.0f : -1.0f;
+        const v3 corner = frame_local_to_world(box, v3_make(sx * box->half.x, sy * box->half.y, sz * box->half.z));
+        const float sd = v3_dot(v3_sub(corner, plane->t), n);
+        if (sd < query) {
+            position[ncand] = v3_sub(corner, v3_scale(n, 0.5f * sd));
+            pen[ncand] = -sd; feature[ncand] = c; ++ncand;
+        }
+    }
+    reduce_and_emit(position, pen, feature, ncand, n, out);
+}
+
+/* analytical_manifold.hpp:738-759 CapsulePlane: both ends of the segment along the capsule's local z */
+static void capsule_plane(const prim* cap, const prim* plane, float query, manifold* out) {
+    out->count = 0u;
+    const v3 n = norm_or(plane->cz, v3_make(0, 0, 1));
+    const v3 axis = cap->cz;
+    const v3 ends[2] = {v3_add(cap->t, v3_scale(axis, cap->half_height)), v3_sub(cap->t, v3_scale(axis, cap->half_height))};
+    v3 position[2]; float pen[2]; uint32_t feature[2];
+    int ncand = 0;
+    for (uint32_t k = 0u; k < 2u; ++k) {
+        const float sd = v3_dot(v3_sub(ends[k], plane->t), n) - cap->radius;
+        if (sd < query) {
+            position[ncand] = v3_sub(ends[k], v3_scale(n, cap->radius + 0.5f * sd));
+            pen[ncand] = -sd; feature[ncand] = k; ++ncand;
+        }
+    }
+    reduce_and_emit(position, pen, feature, ncand, n, out);
+}
+
+/* analytical_manifold.hpp:764-778 CapsuleSphere (a = capsule): the normal points from the sphere to the capsule */
+static void capsule_sphere(const prim* cap, const prim* sph, float query, manifold* out) {
+    out->count = 0u;
+    const surface s = query_surface(NKO_CAPSULE, v3_make(cap->radius, cap->half_height, 0.0f), frame_world_to_local(cap, sph->t));
+    if (!s.valid) return;
+    const float pen = sph->radius - s.distance;
+    if (pen <= -query) return;
+    const v3 normal = v3_scale(frame_dir_to_world(cap, s.normal), -1.0f);
+    emit_one(out, v3_add(frame_local_to_world(cap, s.point), v3_scale(normal, 0.5f * pen)), normal, pen, 0u);
+}
+
+/* analytical_manifold.hpp:780-815 CylinderPlane: the lower cap's octagon and deepest point when a cap faces the
+ * plane, else each cap's deepest point */
+static void cylinder_plane(const prim* cyl, const prim* plane, float query, manifold* out) {
+    out->count = 0u;
+    static const float kS = 0.70710678f;
+    const float rc[8] = {1.0f, kS, 0.0f, -kS, -1.0f, -kS, 0.0f, kS};
+    const float rs[8] = {0.0f, kS, 1.0f, kS, 0.0f, -kS, -1.0f, -kS};
+    const v3 n = norm_or(plane->cz, v3_make(0, 0, 1));
+    const v3 axis = cyl->cz;
+    const float d = v3_dot(axis, n);
+    const int on_cap = (d < 0.0f ? -d : d) >= 0.95f;
+    const v3 down = norm_or(v3_sub(v3_scale(axis, d), n), cyl->cx);
+    v3 position[10]; float pen[10]; uint32_t feature[10];
+    int ncand = 0;
+    for (int cap = 0; cap < 2; ++cap) {
+        if (on_cap && (cap == 0) == (d > 0.0f)) continue;
+        const v3 center = v3_add(cyl->t, v3_scale(axis, cap == 0 ? cyl->half_height : -cyl->half_height));
+        for (int k = -1; k < (on_cap ? 8 : 0); ++k) {
+            const v3 dir = k < 0 ? down : v3_add(v3_scale(cyl->cx, rc[k]), v3_scale(cyl->cy, rs[k]));
+            const v3 p = v3_add(center, v3_scale(dir, cyl->radius));
+            const float sd = v3_dot(v3_sub(p, plane->t), n);
+            if (sd >= query) continue;
+            position[ncand] = v3_sub(p, v3_scale(n, sd * 0.5f));
+            pen[ncand] = -sd;
+            feature[ncand] = (uint32_t)(k < 0 ? cap : 2 + cap * 8 + k);
+            ++ncand;
+        }
+    }
+    reduce_and_emit_spread(position, pen, feature, ncand, n, out);
+}
+
+/* analytical_manifold.hpp:819-834 CylinderSphere (a = cylinder) */
+static void cylinder_sphere(const prim* cyl, const prim* sph, float query, manifold* out) {
+    out->count = 0u;
+    const surface s = query_surface(NKO_CYLINDER, v3_make(cyl->radius, cyl->half_height, 0.0f), frame_world_to_local(cyl, sph->t));
+    if (!s.valid) return;
+    const float pen = sph->radius - s.distance;
+    if (pen <= -query) return;
+    const v3 normal = v3_scale(frame_dir_to_world(cyl, s.normal), -1.0f);
+    emit_one(out, v3_add(frame_local_to_world(cyl, s.point), v3_scale(normal, 0.5f * pen)), normal, pen, (uint64_t)s.feature);
+}
+
+/* analytical_manifold.hpp:841-896 ClosestPtSegmentSegment (fixed branch order) */
+static float clamp01(float v) { return v < 0.0f ? 0.0f : (v > 1.0f ? 1.0f : v); }
+static float closest_segment_segment(v3 p1, v3 q1, v3 p2, v3 q2, v3* c1_out, v3* c2_out) {
+    const v3 d1 = v3_sub(q1, p1), d2 = v3_sub(q2, p2), r = v3_sub(p1, p2);
+    const float a = v3_dot(d1, d1), e = v3_dot(d2, d2), f = v3_dot(d2, r);
+    float s = 0.0f, t = 0.0f;
+    const float eps = 1.0e-12f;
+    if (a <= eps && e <= eps) { s = 0.0f; t = 0.0f; }
+    else if (a <= eps) { s = 0.0f; t = clamp01(f / e); }
+    else {
+        const float c = v3_dot(d1, r);
+        if (e <= eps) { t = 0.0f; s = clamp01(-c / a); }
+        else {
+            const float b = v3_dot(d1, d2);
+            const float denom = a * e - b * b;
+            if (denom > eps) s = clamp01((b * f - c * e) / denom); else s = 0.0f;
+            t = (b * s + f) / e;
+            if (t < 0.0f) { t = 0.0f; s = clamp01(-c / a); }
+            else if (t > 1.0f) { t = 1.0f; s = clamp01((b - c) / a); }
+        }
+    }
+    const v3 c1 = v3_add(p1, v3_scale(d1, s)), c2 = v3_add(p2, v3_scale(d2, t));
+    *c1_out = c1; *c2_out = c2;
+    const v3 dv = v3_sub(c1, c2);
+    return v3_dot(dv, dv);
+}
+
+/* analytical_manifold.hpp:905-932 CapsuleCapsule: closest points of the two axes, inflated by the radii */
+static void capsule_capsule(const prim* a, const prim* b, float query, manifold* out) {
+    out->count = 0u;
+    const v3 axa = a->cz, axb = b->cz;
+    const v3 a0 = v3_add(a->t, v3_scale(axa, a->half_height)), a1 = v3_sub(a->t, v3_scale(axa, a->half_height));
+    const v3 b0 = v3_add(b->t, v3_scale(axb, b->half_height)), b1 = v3_sub(b->t, v3_scale(axb, b->half_height));
+    v3 ca, cb;
+    const float dist = sqrtf(closest_segment_segment(a0, a1, b0, b1, &ca, &cb));
+    const float pen = (a->radius + b->radius) - dist;
+    if (pen <= -query) return;
+    const v3 n = norm_or(v3_sub(ca, cb), norm_or(v3_cross(axa, axb), v3_make(0, 1, 0)));
+    const v3 sa = v3_sub(ca, v3_scale(n, a->radius)), sb = v3_add(cb, v3_scale(n, b->radius));
+    emit_one(out, v3_scale(v3_add(sa, sb), 0.5f), n, pen, 0u);
+}
+
+/* analytical_manifold.hpp:934-971 PrimitivePair, every analytic pair but box x box; a flipped pair negates the
+ * normals.  Returns 0 for a pair that has no analytic manifold. */
+static int primitive_pair(uint32_t ka, const prim* a, uint32_t kb, const prim* b, float query, manifold* out) {
+    out->count = 0u;
+    if (ka == NKO_SPHERE && kb == NKO_SPHERE) { sphere_sphere(a, b, query, out); return 1; }
+    if (ka == NKO_SPHERE && kb == NKO_BOX) { sphere_box(a, b, query, out); return 1; }
+    if (ka == NKO_SPHERE && kb == NKO_PLANE) { sphere_plane(a, b, query, out); return 1; }
+    if (ka == NKO_BOX && kb == NKO_PLANE) { box_plane(a, b, query, out); return 1; }
+    if (ka == NKO_CAPSULE && kb == NKO_PLANE) { capsule_plane(a, b, query, out); return 1; }
+    if (ka == NKO_CAPSULE && kb == NKO_SPHERE) { capsule_sphere(a, b, query, out); return 1; }
+    if (ka == NKO_CAPSULE && kb == NKO_CAPSULE) { capsule_capsule(a, b, query, out); return 1; }
+    if (ka == NKO_CYLINDER && kb == NKO_PLANE) { cylinder_plane(a, b, query, out); return 1; }
+    if (ka == NKO_CYLINDER && kb == NKO_SPHERE) { cylinder_sphere(a, b, query, out); return 1; }
+    int flipped = 1;
+    if (ka == NKO_BOX && kb == NKO_SPHERE) sphere_box(b, a, query, out);
+    else if (ka == NKO_PLANE && kb == NKO_SPHERE) sphere_plane(b, a, query, out);
+    else if (ka == NKO_PLANE && kb == NKO_BOX) box_plane(b, a, query, out);
+    else if (ka == NKO_PLANE && kb == NKO_CAPSULE) capsule_plane(b, a, query, out);
+    else if (ka == NKO_SPHERE && kb == NKO_CAPSULE) capsule_sphere(b, a, query, out);
+    else if (ka == NKO_PLANE && kb == NKO_CYLINDER) cylinder_plane(b, a, query, out);
+    else if (ka == NKO_SPHERE && kb == NKO_CYLINDER) cylinder_sphere(b, a, query, out);
+    else flipped = 0;
+    for (uint32_t i = 0u; i < out->count; ++i) out->normal[i] = v3_make(-out->normal[i].x, -out->normal[i].y, -out->normal[i].z);
+    return flipped;
+}
+int nko_pair_has_manifold(uint32_t ka, uint32_t kb) {
+    static const uint32_t kinds[5] = {NKO_SPHERE, NKO_CAPSULE, NKO_BOX, NKO_PLANE, NKO_CYLINDER};
+    int known_a = 0, known_b = 0;
+    for (int i = 0; i < 5; ++i) { known_a |= ka == kinds[i]; known_b |= kb == kinds[i]; }
+    if (!known_a || !known_b) return 0;
+    if (ka == NKO_PLANE && kb == NKO_PLANE) return 0;
+    if (ka == NKO_BOX && kb == NKO_BOX) return 0;
+    if ((ka == NKO_CYLINDER && (kb == NKO_CYLINDER || kb == NKO_BOX || kb == NKO_CAPSULE)) ||
+        (kb == NKO_CYLINDER && (ka == NKO_BOX || ka == NKO_CAPSULE))) return 0;
+    if ((ka == NKO_CAPSULE && kb == NKO_BOX) || (ka == NKO_BOX && kb == NKO_CAPSULE)) return 0;
+    return 1;
 }
 
 uint32_t nko_sphere_plane(const float sphere_pose[7], float radius, const float plane_pose[7], float query,
@@ -237,7 +554,7 @@ uint32_t nko_primitive_pair_frames(uint32_t kind_a, const float frame_a[12], con
     for (int k = 0; k < 2; ++k) {
         pr[k].cx = v3_make(f[k][0], f[k][1], f[k][2]); pr[k].cy = v3_make(f[k][3], f[k][4], f[k][5]);
         pr[k].cz = v3_make(f[k][6], f[k][7], f[k][8]); pr[k].t = v3_make(f[k][9], f[k][10], f[k][11]);
-        pr[k].radius = s[k][0]; pr[k].half = v3_make(s[k][0], s[k][1], s[k][2]);
+        pr[k].radius = s[k][0]; pr[k].half_height = s[k][1]; pr[k].half = v3_make(s[k][0], s[k][1], s[k][2]);
     }
     manifold m; primitive_pair(kind_a, &pr[0], kind_b, &pr[1], query, &m);
     for (uint32_t i = 0u; i < m.count; ++i) {

@@ -16,7 +16,7 @@
 /* phi/articulation_contract.hpp:8-16 */
 enum { NKO_REVOLUTE = 0, NKO_PRISMATIC = 1, NKO_FIXED = 2, NKO_FLOATING = 3, NKO_SPHERICAL = 4 };
 /* collision/shape_kind.hpp:9-18 */
-enum { NKO_SPHERE = 0, NKO_CAPSULE = 1, NKO_BOX = 2, NKO_PLANE = 3 };
+enum { NKO_SPHERE = 0, NKO_CAPSULE = 1, NKO_BOX = 2, NKO_PLANE = 3, NKO_CYLINDER = 7 };
 /* nk/solve/nk_row.hpp:14-19 */
 enum { NKO_SIDE_RIGID = 0, NKO_SIDE_ARTIC = 1, NKO_SIDE_STATIC = 3 };
 /* nk/solve/nk_row.hpp:41-57 */
@@ -74,6 +74,8 @@ typedef struct {
     float* link_geom_local;     /* nl*7 */
     uint32_t* link_geom_kind;   /* nl */
     float* shape_table;         /* nb*13 words */
+    uint64_t* excluded_pairs;   /* sorted (a << 32 | b) keys of collidable rows that never pair, a < b */
+    uint32_t excluded_count;
     uint32_t* body_to_link, *body_to_articulation, *body_collidable_link, *body_collidable_body;
     float* body_collidable_local; /* nb*7 */
     float* body_init_pose;        /* nb*7 */
@@ -158,6 +160,7 @@ void nko_env_link_velocities(nko_world* w, uint32_t env);
 void nko_env_sync_body_pose(nko_world* w, uint32_t env);
 void nko_env_aabbs(nko_world* w, uint32_t env);
 void nko_env_pairs(nko_world* w, uint32_t env);
+int nko_template_pair_excluded(const nko_template* t, uint32_t a, uint32_t b);   /* a < b */
 void nko_env_narrowphase(nko_world* w, uint32_t env);
 void nko_env_assemble_rows(nko_world* w, uint32_t env);
 void nko_env_warm_start_prepare(nko_world* w, uint32_t env);

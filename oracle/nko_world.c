@@ -5,6 +5,7 @@
 #include <stdio.h>
 
 #include "nko_internal.h"
+#include <stddef.h>
 
 #define ALLOC(type, count) ((type*)calloc((size_t)(count) + 1u, sizeof(type)))
 
@@ -41,7 +42,8 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
     copy_or_zero(t->joint_armature, d->joint_armature, nl);
     copy_or_zero(t->joint_stiffness, d->joint_stiffness, nl);
     copy_or_zero(t->joint_spring_reference, d->joint_spring_reference, nl);
-    const int has_joint_rows = d->struct_size >= sizeof(nko_template_desc);
+    const int has_joint_rows = d->struct_size >= offsetof(nko_template_desc, excluded_pairs);
+    const int has_excluded = d->struct_size >= sizeof(nko_template_desc);
     copy_or_zero(t->joint_limit_lower, has_joint_rows ? d->joint_limit_lower : NULL, nl);
     copy_or_zero(t->joint_limit_upper, has_joint_rows ? d->joint_limit_upper : NULL, nl);
     copy_or_zero(t->joint_frictionloss, has_joint_rows ? d->joint_frictionloss : NULL, nl);
@@ -115,6 +117,38 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
         t->body_collidable_body[b] = t->link_body[link];
         memcpy(t->body_collidable_local + 7u * b, d->body_local + 7u * b, 7u * sizeof(float));
     }
+    /* excluded pairs (scene/cook/cook_to_model.cpp:1468-1490): the authored ones and every two rows of one link,
+     * as sorted (a << 32 | b) keys with a < b */
+    {
+        const uint32_t authored = has_excluded && d->excluded_pairs != NULL ? d->excluded_pair_count : 0u;
+        size_t cap = authored;
+        for (uint32_t i = 0u; i < nb; ++i)
+            for (uint32_t j = i + 1u; j < nb; ++j)
+                if (d->body_role[i] != 0u && d->body_role[j] != 0u && d->body_link[i] == d->body_link[j]) ++cap;
+        t->excluded_pairs = ALLOC(uint64_t, cap ? cap : 1u);
+        uint32_t n = 0u;
+        for (uint32_t k = 0u; k < authored; ++k) {
+            const uint32_t a = d->excluded_pairs[2u * k], b = d->excluded_pairs[2u * k + 1u];
+            if (a >= nb || b >= nb || a == b) return -1;
+            t->excluded_pairs[n++] = ((uint64_t)(a < b ? a : b) << 32u) | (uint64_t)(a < b ? b : a);
+        }
+        for (uint32_t i = 0u; i < nb; ++i)
+            for (uint32_t j = i + 1u; j < nb; ++j)
+                if (d->body_role[i] != 0u && d->body_role[j] != 0u && d->body_link[i] == d->body_link[j])
+                    t->excluded_pairs[n++] = ((uint64_t)i << 32u) | (uint64_t)j;
+        for (uint32_t i = 1u; i < n; ++i) {   /* insertion sort, then drop repeats */
+            const uint64_t key = t->excluded_pairs[i]; uint32_t j = i;
+            while (j > 0u && t->excluded_pairs[j - 1u] > key) { t->excluded_pairs[j] = t->excluded_pairs[j - 1u]; --j; }
+            t->excluded_pairs[j] = key;
+        }
+        uint32_t unique = 0u;
+        for (uint32_t i = 0u; i < n; ++i) if (unique == 0u || t->excluded_pairs[unique - 1u] != t->excluded_pairs[i]) t->excluded_pairs[unique++] = t->excluded_pairs[i];
+        t->excluded_count = unique;
+    }
+    for (uint32_t i = 0u; i < nb; ++i) {
+        const uint32_t kind = d->shape_kind[i];
+        if (kind != NKO_INVALID && kind != NKO_SPHERE && kind != NKO_CAPSULE && kind != NKO_BOX && kind != NKO_PLANE && kind != NKO_CYLINDER) return -1;
+    }
     uint32_t slots = d->max_contacts_per_env;
     if (slots == 0u) {   /* admitted pairs of the template */
         for (uint32_t i = 0u; i < nb; ++i)
@@ -124,6 +158,7 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
                 if (d->shape_kind[i] == NKO_INVALID || d->shape_kind[j] == NKO_INVALID) continue;
                 if (!nko_shape_filter_admits(d->shape_contype[i], d->shape_conaffinity[i], d->shape_group[i],
                                              d->shape_contype[j], d->shape_conaffinity[j], d->shape_group[j])) continue;
+                if (nko_template_pair_excluded(t, i, j)) continue;
                 ++slots;
             }
     }
@@ -152,7 +187,7 @@ static void free_template(nko_template* t) {
     free(t->joint_stiffness); free(t->joint_spring_reference); free(t->joint_limit_lower); free(t->joint_limit_upper);
     free(t->joint_frictionloss); free(t->joint_limit_flags); free(t->link_body); free(t->link_tree_depth);
     free(t->link_child_range); free(t->link_children); free(t->link_dof); free(t->dof_link); free(t->dof_component);
-    free(t->link_geom_local); free(t->link_geom_kind); free(t->shape_table); free(t->body_to_link);
+    free(t->link_geom_local); free(t->link_geom_kind); free(t->shape_table); free(t->excluded_pairs); free(t->body_to_link);
     free(t->body_to_articulation); free(t->body_collidable_link); free(t->body_collidable_body);
     free(t->body_collidable_local); free(t->body_init_pose); free(t->profile_mu);
 }

@@ -89,6 +89,10 @@ typedef struct nko_template_desc {
     const float* joint_frictionloss;
     uint32_t drive_mode;
     uint32_t drive_rows;
+    /* collidable rows that never pair; read only when struct_size covers them */
+    const uint32_t* excluded_pairs;
+    uint32_t excluded_pair_count;
+    uint32_t reserved1;
 } nko_template_desc;
 
 typedef struct nko_world_desc {
@@ -154,6 +158,8 @@ double nko_contact_projection_roundoff(const float start[3], const float end[3],
 float nko_contact_query_reach(float thickness, float margin);
 float nko_contact_motion_radius(float base, float dt, float sa, float sb, float relax);
 int nko_shape_filter_admits(uint32_t ta, uint32_t aa, uint32_t ga, uint32_t tb, uint32_t ab, uint32_t gb);
+int nko_pair_excluded(const nko_world* w, uint32_t a, uint32_t b);
+int nko_pair_has_manifold(uint32_t kind_a, uint32_t kind_b);   /* every analytic pair of PrimitivePair but box x box */
 void nko_compose_transform(const float parent[7], const float child[7], float out[7]);
 void nko_make_contact_id(uint32_t a, uint32_t b, const float local_a[3], const float local_b[3], uint32_t feature,
                          uint32_t manifold_slot, uint64_t out[2]);

@@ -33,6 +33,59 @@ def frame(pose):
     return np.concatenate([R[:, 0], R[:, 1], R[:, 2], pose[:3]]).astype(np.float32)
 
 
+# every ordered kind pair PrimitivePair answers analytically, box x box aside (sphere 0, capsule 1, box 2, plane 3,
+# cylinder 7)
+PAIR_ORDERS = [(0, 0), (0, 2), (2, 0), (1, 3), (3, 1), (1, 0), (0, 1), (1, 1), (7, 3), (3, 7), (7, 0), (0, 7)]
+
+
+def pair_shape(g, kind):
+    if kind == 0:
+        return [g.uniform(0.02, 0.06), 0, 0, 0]
+    if kind in (1, 7):
+        return [g.uniform(0.02, 0.05), g.uniform(0.03, 0.1), 0, 0]
+    if kind == 2:
+        return list(g.uniform(0.02, 0.08, 3)) + [0]
+    return [0, 0, 0, 0]
+
+
+def pair_case(g, ka, kb):
+    """Two poses a few centimetres apart, so that about half the cases touch, and the shapes' parameters."""
+    pose = np.zeros((2, 7), np.float32)
+    for side, kind in enumerate((ka, kb)):
+        if kind == 3:
+            q = np.array([1, 0, 0, 0]) + g.normal(0, 0.05, 4)
+            pose[side] = np.concatenate([[0, 0, g.uniform(-0.01, 0.01)], q / np.linalg.norm(q)])
+        else:
+            q = unit_quat(g)
+            if kind == 7 and g.uniform() < 0.5:   # a cylinder standing on a cap, or nearly
+                q = np.array([1, 0, 0, 0]) + g.normal(0, 0.08, 4)
+                q /= np.linalg.norm(q)
+                if g.uniform() < 0.5:
+                    q = np.array([-q[1], q[0], q[3], -q[2]])   # turned over
+            pose[side] = np.concatenate([g.normal(0, 0.04, 3), q])
+            if 3 in (ka, kb):
+                pose[side, 2] = g.uniform(-0.02, 0.12)
+    return pose, np.array([pair_shape(g, ka), pair_shape(g, kb)], np.float32), g.choice([0.0, 1e-3, 5e-4])
+
+
+def pair_cases(L, g):
+    m = 100 * len(PAIR_ORDERS)
+    kinds = np.zeros((m, 2), np.uint32)
+    poses, params, query = np.zeros((m, 2, 7), np.float32), np.zeros((m, 2, 4), np.float32), np.zeros(m, np.float32)
+    count = np.zeros(m, np.uint32)
+    points, normals, pen, keys = np.zeros((m, 12), np.float32), np.zeros((m, 12), np.float32), np.zeros((m, 4), np.float32), np.zeros((m, 4), np.uint64)
+    for i in range(m):
+        ka, kb = PAIR_ORDERS[i % len(PAIR_ORDERS)]
+        kinds[i] = (ka, kb)
+        poses[i], params[i], query[i] = pair_case(g, ka, kb)
+        p, nr, pe, ke = (F * 12)(), (F * 12)(), (F * 4)(), (C.c_uint64 * 4)()
+        count[i] = L.ref_primitive_pair_frames(ka, farr(frame(poses[i, 0])), farr(params[i, 0]), kb, farr(frame(poses[i, 1])),
+                                               farr(params[i, 1]), F(float(query[i])), p, nr, pe, ke)
+        points[i], normals[i], pen[i], keys[i] = list(p), list(nr), list(pe), list(ke)
+    return dict(pair_kinds=kinds, pair_poses=poses, pair_params=params, pair_query=query, pair_count=count,
+                pair_points=points, pair_normals=normals, pair_penetration=pen, pair_keys=keys)
+
+
 def main():
     oracle_py.build()
     L = C.CDLL(oracle_py.REF_PATH)
@@ -134,6 +187,8 @@ def main():
         cases[i] = g.normal(0, 1, 9)
         results[i] = L.ref_contact_projection_roundoff(farr(cases[i, :3]), farr(cases[i, 3:6]), farr(cases[i, 6:]))
     out["roundoff_in"], out["roundoff_out"] = cases, results
+
+    out.update(pair_cases(L, g))
 
     np.savez_compressed(os.path.join(HERE, "rowmath_vectors.npz"), **out)
     print("wrote", os.path.join(HERE, "rowmath_vectors.npz"))

@@ -81,6 +81,26 @@ def test_manifolds(oracle_py, vectors):
     assert hits > 100
 
 
+def test_every_analytic_pair(oracle_py, vectors):
+    """Sphere, capsule, box, plane and cylinder pairs of the reference's PrimitivePair (box x box aside), both orders."""
+    from golden.make_rowmath_vectors import frame
+    L = oracle_py.lib()
+    hits = {}
+    for i in range(len(vectors["pair_count"])):
+        ka, kb = [int(k) for k in vectors["pair_kinds"][i]]
+        p, n, pe, ke = (F * 12)(), (F * 12)(), (F * 4)(), (C.c_uint64 * 4)()
+        count = L.nko_primitive_pair_frames(ka, farr(frame(vectors["pair_poses"][i, 0])), farr(vectors["pair_params"][i, 0]), kb,
+                                            farr(frame(vectors["pair_poses"][i, 1])), farr(vectors["pair_params"][i, 1]),
+                                            F(float(vectors["pair_query"][i])), p, n, pe, ke)
+        assert count == vectors["pair_count"][i], (ka, kb, i)
+        hits[(ka, kb)] = hits.get((ka, kb), 0) + int(count > 0)
+        assert same(list(p)[:3 * count], vectors["pair_points"][i, :3 * count]), (ka, kb, i)
+        assert same(list(n)[:3 * count], vectors["pair_normals"][i, :3 * count]), (ka, kb, i)
+        assert same(list(pe)[:count], vectors["pair_penetration"][i, :count]), (ka, kb, i)
+        assert list(ke)[:count] == list(vectors["pair_keys"][i, :count]), (ka, kb, i)
+    assert len(hits) == 12 and min(hits.values()) >= 15, hits
+
+
 def test_compose_contact_id_and_roundoff(oracle_py, vectors):
     L = oracle_py.lib()
     L.nko_contact_projection_roundoff.restype = C.c_double

@@ -179,13 +179,18 @@ def test_error_paths(device):
     assert lib.nuka_world_set_execution_mode(world._h, 5) == 1
     world.close()
     # templates outside the path are refused at creation
-    t = abi.Template()
-    t.add_link(abi.JOINT_FLOATING, None)
-    t.add_body(abi.ROLE_STATIC, kind=abi.SHAPE_PLANE, contype=2, conaffinity=1)
-    t.add_body(abi.ROLE_LINK_BODY, link=0, kind=abi.SHAPE_CAPSULE, params=(0.1, 0.2, 0, 0), contype=1, conaffinity=2)
-    with pytest.raises(nk.NukaError) as info:
-        nk.World(device, t, abi.world_desc(4, 0.005))
-    assert info.value.code == 7
+    for kinds in ((abi.SHAPE_BOX, abi.SHAPE_BOX), (abi.SHAPE_CAPSULE, abi.SHAPE_BOX), (abi.SHAPE_CYLINDER, abi.SHAPE_CAPSULE), (4, abi.SHAPE_PLANE)):
+        t = abi.Template()   # an admitted pair without an analytic manifold, or a shape kind outside the path
+        t.add_link(abi.JOINT_FLOATING, None)
+        t.add_link(abi.JOINT_REVOLUTE, 0)
+        t.add_body(abi.ROLE_LINK_BODY, link=0, kind=kinds[0], params=(0.1, 0.2, 0.1, 0))
+        t.add_body(abi.ROLE_STATIC if kinds[1] == abi.SHAPE_PLANE else abi.ROLE_LINK_BODY, link=1, kind=kinds[1], params=(0.1, 0.2, 0.1, 0))
+        with pytest.raises(nk.NukaError) as info:
+            nk.World(device, t, abi.world_desc(4, 0.005))
+        assert info.value.code == 7
+    t.exclude(0, 1)          # the same pair, excluded: nothing left to refuse
+    t.bodies[0]["kind"] = abi.SHAPE_BOX
+    nk.World(device, t, abi.world_desc(4, 0.005)).close()
     t = abi.Template()
     t.add_link(abi.JOINT_FIXED, None)
     t.add_link(abi.JOINT_REVOLUTE, 5)

@@ -51,10 +51,59 @@ def test_scene_world_matches_the_oracle_and_resets_to_the_authored_state(oracle_
     world.close(); oracle.close()
 
 
+WALKER = os.path.join(ROOT, "tests", "data", "capsule_walker.xml")
+
+
+def test_capsule_walker_matches_the_oracle(oracle_py, device):
+    """A robot file whose links collide with capsules, a cylinder and spheres, with each other and with the floor:
+    loaded without the plane-contacts-only relaxation, stepped on the device and by the oracle from the same pushes."""
+    E, steps = 128, 12
+    scene = nk.Scene(WALKER)
+    assert scene.info.dropped_geom_count == 0
+    desc = abi.world_desc(E, scene.info.timestep, gravity=tuple(scene.info.gravity), vel_iters=8)
+    world, oracle = nk.World(device, scene, desc), oracle_py.OracleWorld(scene, desc, threads=8)
+    state = scene.initial_state()
+    rng = np.random.default_rng(23)
+    nl = scene.link_count
+    joint = {name: scene.joint_names.index(name) for name in ("l_hip_x", "r_hip_x", "l_hip_y", "r_hip_y")}
+    # the legs swing towards each other, one a little forward and one a little back, so that the thighs meet at an angle
+    q, qdot = np.tile(state["q"], (E, 1)), np.zeros((E, nl), np.float32)
+    cross, push = rng.uniform(0.05, 0.2, E), rng.uniform(0.0, 2.5, E)
+    q[:, joint["l_hip_x"]], q[:, joint["r_hip_x"]] = -cross, cross
+    q[:, joint["l_hip_y"]], q[:, joint["r_hip_y"]] = 0.12 + rng.normal(0, 0.02, E), -0.12 + rng.normal(0, 0.02, E)
+    qdot[:, joint["l_hip_x"]], qdot[:, joint["r_hip_x"]] = -push, push
+    base = np.tile(state["base_pose"], (E, 1))
+    base[:, 2] -= rng.uniform(0.03, 0.045, E)                  # the soles at the floor
+    for name in ("drive_stiffness", "drive_damping", "drive_force_limit", "drive_joint_force_limit"):
+        oracle.upload(name, np.tile(state[name], E))
+    for w in (oracle, world):
+        w.upload("q", q); w.upload("qdot", qdot); w.upload("drive_target", q); w.upload("base_pose", base)
+    world.step(steps); world.synchronize()
+    oracle.step(steps)
+    assert np.array_equal(world.download("env_status"), oracle.download("env_status")) and not world.download("env_status").any()
+    S = world.info.contact_slots_per_env
+    count = oracle.download("ucontact_count").reshape(E, S)
+    plane_row = 0
+    side_a = oracle.download("ucontact_a").reshape(E, S, 4)[:, :, 0]
+    link_pairs = (count > 0) & (side_a != plane_row)
+    assert link_pairs.any(1).sum() >= E // 4 and ((count > 0) & (side_a == plane_row)).any(1).sum() >= E // 4   # links meet links, soles the floor
+    # closest points of two capsules jump where the axes are parallel (legs side by side): environments whose manifolds
+    # differ by more than rounding are set aside, the rest has to meet the tolerance
+    point_g, point_o = world.download("ucontact_point").reshape(E, S, 4, 3), oracle.download("ucontact_point").reshape(E, S, 4, 3)
+    live = np.arange(4)[None, None, :] < count[:, :, None]
+    same = ~((np.abs(point_g - point_o).max(3) > 1e-3) & live).any((1, 2))
+    same &= (world.download("ucontact_count").reshape(E, S) == count).all(1)
+    assert same.mean() >= 0.85, same.mean()
+    for name in ("q", "qdot", "base_pose", "link_pose", "actuator_effort"):
+        error = relative_error(world.download(name).reshape(E, -1)[same], oracle.download(name).reshape(E, -1)[same])
+        assert error <= 5 * TOL, f"{name}: {error:.2e}"        # a dozen steps of accumulated rounding
+    world.close(); oracle.close()
+
+
 def test_scene_with_unsupported_collision_geometry_is_refused(device, tmp_path):
-    path = tmp_path / "capsule.xml"
+    path = tmp_path / "ellipsoid.xml"
     path.write_text('<mujoco><worldbody><geom type="plane" size="1 1 1"/><body pos="0 0 1"><freejoint/>'
-                    '<geom type="capsule" size="0.05 0.2"/></body></worldbody></mujoco>')
+                    '<inertial pos="0 0 0" mass="1" diaginertia="0.01 0.01 0.01"/><geom type="ellipsoid" size="0.05 0.2 0.1"/></body></worldbody></mujoco>')
     strict = nk.Scene(str(path))
     with pytest.raises(nk.NukaError) as err:
         nk.World(device, strict, abi.world_desc(4, 0.005))

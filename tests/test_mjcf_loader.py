@@ -197,6 +197,53 @@ def test_biped_stands_on_its_feet_in_the_oracle(oracle_py):
     w.close()
 
 
+WALKER = os.path.join(ROOT, "tests", "data", "capsule_walker.xml")
+
+
+def test_capsule_walker_links_meet_each_other_but_not_their_parents(oracle_py, tmp_path):
+    """Capsule, cylinder and sphere geoms become collidable rows; a body never pairs with its parent body (through the
+    massless links of a two-joint hip too), nor with a body welded to it, nor with one an <exclude> names - the
+    reference's cook-time policy (src/scene/cooker.cpp:470-538), which is MuJoCo's."""
+    scene = nk.Scene(WALKER)
+    a = scene.template_arrays()
+    owner = [scene.link_names[l] if l < scene.link_count else "world" for l in a["body_link"]]
+    kinds = {(owner[r], int(k)) for r, k in enumerate(a["shape_kind"]) if k != abi.INVALID}
+    assert kinds == {("world", abi.SHAPE_PLANE), ("torso", abi.SHAPE_CAPSULE), ("torso", abi.SHAPE_CYLINDER), ("l_thigh", abi.SHAPE_CAPSULE),
+                     ("l_shin", abi.SHAPE_CAPSULE), ("l_foot", abi.SHAPE_SPHERE), ("r_thigh", abi.SHAPE_CAPSULE), ("r_shin", abi.SHAPE_CAPSULE),
+                     ("r_foot", abi.SHAPE_SPHERE)}
+    trunk = a["shape_params"].reshape(-1, 4)[owner.index("torso")]
+    assert np.allclose(trunk[:2], [0.07, 0.12])                                     # radius, half length of the fromto segment
+    excluded = {frozenset((owner[p[0]], owner[p[1]])) for p in a["excluded_pairs"].reshape(-1, 2)}
+    assert excluded == {frozenset(p) for p in (("torso", "l_thigh"), ("torso", "r_thigh"), ("l_thigh", "l_shin"), ("r_thigh", "r_shin"),
+                                               ("l_shin", "l_foot"), ("r_shin", "r_foot"), ("l_thigh", "l_foot"), ("r_thigh", "r_foot"),
+                                               ("torso", "l_shin"), ("torso", "r_shin"))}
+    # it stands on its soles; crossing the legs makes the thighs meet each other (capsule against capsule)
+    state = scene.initial_state()
+    w = oracle_py.OracleWorld(scene, abi.world_desc(2, scene.info.timestep, vel_iters=8), threads=2)
+    for name in ("q", "drive_stiffness", "drive_damping", "drive_force_limit", "drive_joint_force_limit"):
+        w.upload(name, np.tile(state[name], 2))
+    w.upload("base_pose", np.tile(state["base_pose"], 2))
+    w.upload("drive_target", np.tile(state["q"], 2))
+    w.step(80)
+    assert not w.download("env_status").any() and w.download("contact_count")[0] == 2
+    assert 0.5 < w.download("base_pose").reshape(2, 7)[0, 2] < 0.6
+    q = w.download("q").reshape(2, -1).copy()
+    q[1, scene.joint_names.index("l_hip_x")], q[1, scene.joint_names.index("r_hip_x")] = -0.35, 0.35
+    w.upload("q", q)
+    w.step(1)
+    a_rows, b_rows = w.download("ucontact_a").reshape(2, -1, 4)[:, :, 0], w.download("ucontact_b").reshape(2, -1, 4)[:, :, 0]
+    live = w.download("ucontact_count").reshape(2, -1) > 0
+    met = {frozenset((owner[x], owner[y])) for x, y in zip(a_rows[1][live[1]], b_rows[1][live[1]])}
+    assert frozenset(("l_thigh", "r_thigh")) in met or frozenset(("l_shin", "r_shin")) in met
+    assert all("world" in pair for pair in ({frozenset((owner[x], owner[y])) for x, y in zip(a_rows[0][live[0]], b_rows[0][live[0]])}))
+    w.close()
+    bad = tmp_path / "exclude.xml"
+    bad.write_text('<mujoco><worldbody><body name="a"><freejoint/><geom size="0.1"/></body></worldbody>'
+                   '<contact><exclude body1="a" body2="nobody"/></contact></mujoco>')
+    with pytest.raises(nk.NukaError):
+        nk.Scene(str(bad))
+
+
 def test_errors(tmp_path):
     with pytest.raises(nk.NukaError) as err:
         nk.Scene(str(tmp_path / "nonexistent.xml"))
