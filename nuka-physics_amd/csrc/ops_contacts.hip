@@ -449,13 +449,139 @@ __device__ void capsule_capsule(const Prim& a, const Prim& b, float query, Manif
     const V3 sa = sub3(ca, scale3(n, a.radius)), sb = add3(cb, scale3(n, b.radius));
     emit_one(out, scale3(add3(sa, sb), 0.5f), n, pen, 0u);
 }
-// :934-971 PrimitivePair, every analytic pair but box x box; a flipped pair negates the normal
+// :224-260 ClipAgainstPlane: Sutherland-Hodgman against one half-space, edges in fixed order; an intersection
+// inherits the feature of the edge's first vertex
+struct ClipPoly { V3 v[8]; uint32_t feat[8]; int count; };
+__device__ __forceinline__ void clip_add(ClipPoly* p, V3 v, uint32_t f) { if (p->count < 8) { p->v[p->count] = v; p->feat[p->count] = f; ++p->count; } }
+__device__ void clip_against_plane(const ClipPoly& in, V3 plane_pt, V3 plane_n, ClipPoly* out) {
+    out->count = 0;
+    for (int i = 0; i < in.count; ++i) {
+        const int j = i + 1 == in.count ? 0 : i + 1;
+        const V3 cur = in.v[i], nxt = in.v[j];
+        const float dc = dot3(sub3(cur, plane_pt), plane_n), dn = dot3(sub3(nxt, plane_pt), plane_n);
+        const bool cur_in = dc <= 0.0f, nxt_in = dn <= 0.0f;
+        if (cur_in) clip_add(out, cur, in.feat[i]);
+        if (cur_in != nxt_in) {
+            const float t = dc / (dc - dn);
+            clip_add(out, V3{cur.x + (nxt.x - cur.x) * t, cur.y + (nxt.y - cur.y) * t, cur.z + (nxt.z - cur.z) * t}, in.feat[i]);
+        }
+    }
+}
+__device__ __forceinline__ V3 neg3(V3 a) { return V3{-a.x, -a.y, -a.z}; }
+__device__ __forceinline__ float comp3(V3 v, int k) { return k == 0 ? v.x : (k == 1 ? v.y : v.z); }
+__device__ __forceinline__ V3 axis3(const Prim& f, int k) { return k == 0 ? f.cx : (k == 1 ? f.cy : f.cz); }
+
+// :503-736 BoxBox: the axis of least penetration among the 15 separating-axis candidates in fixed order (faces preferred
+// by a 1e-5 bias); an edge pair gives one point between the closest edge points, a face gives the incident face clipped
+// against the reference face's sides, reduced by ReduceAndEmitSpread
+__device__ void box_box(const Prim& A, const Prim& B, float query, Manifold* out) {
+    out->count = 0u;
+    const V3 dpos = sub3(B.t, A.t);
+    float AbsR[3][3];
+    for (int i = 0; i < 3; ++i)
+        for (int j = 0; j < 3; ++j) AbsR[i][j] = fabsf(dot3(axis3(A, i), axis3(B, j))) + 1.0e-6f;
+    const float ea[3] = {A.half.x, A.half.y, A.half.z}, eb[3] = {B.half.x, B.half.y, B.half.z};
+    float min_pen = 3.4e38f;
+    int best_axis = -1;
+    V3 best_n{0, 1, 0};
+    const float bias = 1.0e-5f;
+    for (int i = 0; i < 3; ++i) {
+        const float d = dot3(dpos, axis3(A, i));
+        const float pen = (ea[i] + (eb[0] * AbsR[i][0] + eb[1] * AbsR[i][1] + eb[2] * AbsR[i][2])) - fabsf(d);
+        if (pen <= -query) return;
+        if (pen < min_pen - bias) { min_pen = pen; best_axis = i; best_n = d < 0.0f ? neg3(axis3(A, i)) : axis3(A, i); }
+    }
+    for (int j = 0; j < 3; ++j) {
+        const float d = dot3(dpos, axis3(B, j));
+        const float pen = ((ea[0] * AbsR[0][j] + ea[1] * AbsR[1][j] + ea[2] * AbsR[2][j]) + eb[j]) - fabsf(d);
+        if (pen <= -query) return;
+        if (pen < min_pen - bias) { min_pen = pen; best_axis = 3 + j; best_n = d < 0.0f ? neg3(axis3(B, j)) : axis3(B, j); }
+    }
+    for (int i = 0; i < 3; ++i)
+        for (int j = 0; j < 3; ++j) {
+            V3 L = cross3(axis3(A, i), axis3(B, j));
+            const float Llen = sqrtf(L.x * L.x + L.y * L.y + L.z * L.z);
+            if (Llen < 1.0e-6f) continue;
+            L = V3{L.x / Llen, L.y / Llen, L.z / Llen};
+            const float ra = ea[0] * fabsf(dot3(A.cx, L)) + ea[1] * fabsf(dot3(A.cy, L)) + ea[2] * fabsf(dot3(A.cz, L));
+            const float rb = eb[0] * fabsf(dot3(B.cx, L)) + eb[1] * fabsf(dot3(B.cy, L)) + eb[2] * fabsf(dot3(B.cz, L));
+            const float s = dot3(dpos, L);
+            const float pen = (ra + rb) - fabsf(s);
+            if (pen <= -query) return;
+            if (pen < min_pen - bias) { min_pen = pen; best_axis = 6 + i * 3 + j; best_n = s < 0.0f ? neg3(L) : L; }
+        }
+    if (best_axis < 0) return;
+    if (best_axis >= 6) {   // edge against edge: one point between the closest points of the two edges
+        const int i = (best_axis - 6) / 3, j = (best_axis - 6) % 3;
+        V3 pa = A.t, pb = B.t;
+        for (int k = 0; k < 3; ++k) {
+            if (k != i) pa = add3(pa, scale3(axis3(A, k), (dot3(axis3(A, k), best_n) >= 0.0f ? 1.0f : -1.0f) * ea[k]));
+            if (k != j) pb = add3(pb, scale3(axis3(B, k), (dot3(axis3(B, k), best_n) >= 0.0f ? -1.0f : 1.0f) * eb[k]));
+        }
+        const V3 da = axis3(A, i), db = axis3(B, j), r = sub3(pa, pb);
+        const float bb = dot3(da, db), dd = dot3(da, r), ee = dot3(db, r);
+        const float denom = 1.0f - bb * bb;
+        float sN = 0.0f, tN = 0.0f;
+        if (denom > 1.0e-9f) { sN = (bb * ee - dd) / denom; tN = (ee - bb * dd) / denom; }
+        const float sCl = fminf(fmaxf(sN, -ea[i]), ea[i]), tCl = fminf(fmaxf(tN, -eb[j]), eb[j]);
+        const V3 ca = add3(pa, scale3(da, sCl)), cb = add3(pb, scale3(db, tCl));
+        emit_one(out, scale3(add3(ca, cb), 0.5f), best_n, min_pen, 0xE0000000u | (uint32_t(i) << 4) | uint32_t(j));
+        return;
+    }
+    const bool ref_is_A = best_axis < 3;
+    const int ref_axis = ref_is_A ? best_axis : best_axis - 3;
+    const Prim& Rf = ref_is_A ? A : B;
+    const Prim& If = ref_is_A ? B : A;
+    V3 refN = axis3(Rf, ref_axis);
+    if (dot3(sub3(If.t, Rf.t), refN) < 0.0f) refN = neg3(refN);
+    int inc_axis = 0; float best_dot = 3.4e38f, inc_sign = 1.0f;
+    for (int k = 0; k < 3; ++k) {
+        const float d = dot3(axis3(If, k), refN);
+        if (-fabsf(d) < best_dot) { best_dot = -fabsf(d); inc_axis = k; inc_sign = d < 0.0f ? 1.0f : -1.0f; }
+    }
+    const int iu = (inc_axis + 1) % 3, iv = (inc_axis + 2) % 3;
+    const V3 inc_face_center = add3(If.t, scale3(axis3(If, inc_axis), inc_sign * comp3(If.half, inc_axis)));
+    const V3 iu_w = axis3(If, iu), iv_w = axis3(If, iv);
+    const float iu_e = comp3(If.half, iu), iv_e = comp3(If.half, iv);
+    ClipPoly poly, next;
+    poly.count = 0;
+    for (uint32_t k = 0u; k < 4u; ++k) {
+        const float su = (k == 1u || k == 2u) ? 1.0f : -1.0f, sv = k >= 2u ? 1.0f : -1.0f;
+        clip_add(&poly, add3(add3(inc_face_center, scale3(iu_w, su * iu_e)), scale3(iv_w, sv * iv_e)), (uint32_t(inc_axis) << 4) | k);
+    }
+    const int ru = (ref_axis + 1) % 3, rv = (ref_axis + 2) % 3;
+    const V3 ru_w = axis3(Rf, ru), rv_w = axis3(Rf, rv);
+    const float ru_e = comp3(Rf.half, ru), rv_e = comp3(Rf.half, rv);
+    const V3 ref_face_center = add3(Rf.t, scale3(refN, comp3(Rf.half, ref_axis)));
+    clip_against_plane(poly, add3(ref_face_center, scale3(ru_w, ru_e)), ru_w, &next);
+    clip_against_plane(next, sub3(ref_face_center, scale3(ru_w, ru_e)), neg3(ru_w), &poly);
+    clip_against_plane(poly, add3(ref_face_center, scale3(rv_w, rv_e)), rv_w, &next);
+    clip_against_plane(next, sub3(ref_face_center, scale3(rv_w, rv_e)), neg3(rv_w), &poly);
+    V3 position[8]; float pen[8]; uint32_t feature[8];
+    int ncand = 0;
+    for (int k = 0; k < poly.count; ++k) {
+        const float depth = dot3(sub3(ref_face_center, poly.v[k]), refN);
+        if (depth >= -query) {
+            const V3 onref = add3(poly.v[k], scale3(refN, depth));
+            position[ncand] = scale3(add3(poly.v[k], onref), 0.5f);
+            pen[ncand] = depth; feature[ncand] = uint32_t(k); ++ncand;
+        }
+    }
+    const V3 normalA = ref_is_A ? neg3(refN) : refN;
+    if (ncand == 0) {
+        emit_one(out, add3(inc_face_center, scale3(refN, min_pen * 0.5f)), normalA, min_pen, uint32_t(inc_axis) << 4);
+        return;
+    }
+    reduce_and_emit_spread(position, pen, feature, ncand, normalA, out);
+}
+// :934-971 PrimitivePair; a flipped pair negates the normal
 __device__ void primitive_pair(uint32_t ka, const Prim& a, uint32_t kb, const Prim& b, float query, Manifold* out) {
     out->count = 0u;
     if (ka == kShapeSphere && kb == kShapeSphere) { sphere_sphere(a, b, query, out); return; }
     if (ka == kShapeSphere && kb == kShapeBox) { sphere_box(a, b, query, out); return; }
     if (ka == kShapeSphere && kb == kShapePlane) { sphere_plane(a, b, query, out); return; }
     if (ka == kShapeBox && kb == kShapePlane) { box_plane(a, b, query, out); return; }
+    if (ka == kShapeBox && kb == kShapeBox) { box_box(a, b, query, out); return; }
     if (ka == kShapeCapsule && kb == kShapePlane) { capsule_plane(a, b, query, out); return; }
     if (ka == kShapeCapsule && kb == kShapeSphere) { capsule_sphere(a, b, query, out); return; }
     if (ka == kShapeCapsule && kb == kShapeCapsule) { capsule_capsule(a, b, query, out); return; }

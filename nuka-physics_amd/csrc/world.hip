@@ -193,14 +193,14 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
                 m.excluded_pairs.push_back((uint64_t{i} << 32u) | uint64_t{j});
     std::sort(m.excluded_pairs.begin(), m.excluded_pairs.end());
     m.excluded_pairs.erase(std::unique(m.excluded_pairs.begin(), m.excluded_pairs.end()), m.excluded_pairs.end());
-    // Manifolds built here: every analytic pair of the reference's PrimitivePair but box x box
-    // (collision/analytical_manifold.hpp:934-971).  Any other admitted pair is refused at cook time instead of
+    // Manifolds built here: the analytic pairs of the reference's PrimitivePair (collision/analytical_manifold.hpp:934-971).  Any other admitted pair is refused at cook time instead of
     // silently producing no contact.
     const auto points_of = [](uint32_t ka, uint32_t kb) -> uint32_t {   // most points of the pair's manifold, 0 for none
         if (ka > kb) std::swap(ka, kb);
         if (kb == kShapePlane) return ka == kShapeSphere ? 1u : ka == kShapeCapsule ? 2u : ka == kShapeBox ? 4u : 0u;
         if (kb == kShapeCylinder) return ka == kShapeSphere ? 1u : ka == kShapePlane ? 4u : 0u;
         if (ka == kShapeSphere) return kb <= kShapeBox ? 1u : 0u;                      // sphere x sphere, capsule, box
+        if (ka == kShapeBox && kb == kShapeBox) return 4u;
         return ka == kShapeCapsule && kb == kShapeCapsule ? 1u : 0u;
     };
     uint32_t admitted = 0u, max_points = 1u;
@@ -220,7 +220,7 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
             if (ga != 0 && gb != 0 && (ga > 0 ? ga != gb && gb > 0 : ga == gb)) continue;
             if (std::binary_search(m.excluded_pairs.begin(), m.excluded_pairs.end(), (uint64_t{i} << 32u) | uint64_t{j})) continue;
             const uint32_t points = points_of(kind, d.shape_kind[j]);
-            if (points == 0u) throw NotSupported("admitted collidable pair has no manifold on this path (box x box, and capsule or cylinder against box, capsule x cylinder, cylinder x cylinder)");
+            if (points == 0u) throw NotSupported("admitted collidable pair has no analytic manifold (capsule or cylinder against box, capsule x cylinder, cylinder x cylinder)");
             max_points = std::max(max_points, points);
             ++admitted;
         }

@@ -480,7 +480,147 @@ static void capsule_capsule(const prim* a, const prim* b, float query, manifold*
     emit_one(out, v3_scale(v3_add(sa, sb), 0.5f), n, pen, 0u);
 }
 
-/* analytical_manifold.hpp:934-971 PrimitivePair, every analytic pair but box x box; a flipped pair negates the
+/* analytical_manifold.hpp:224-260 ClipAgainstPlane: Sutherland-Hodgman against one half-space, edges in fixed order;
+ * an intersection inherits the feature of the edge's first vertex */
+typedef struct { v3 v[8]; uint32_t feat[8]; int count; } clip_poly;
+static void clip_add(clip_poly* p, v3 v, uint32_t f) { if (p->count < 8) { p->v[p->count] = v; p->feat[p->count] = f; ++p->count; } }
+static clip_poly clip_against_plane(const clip_poly* in, v3 plane_pt, v3 plane_n) {
+    clip_poly out; out.count = 0;
+    for (int i = 0; i < in->count; ++i) {
+        const int j = (i + 1) % in->count;
+        const v3 cur = in->v[i], nxt = in->v[j];
+        const float dc = v3_dot(v3_sub(cur, plane_pt), plane_n), dn = v3_dot(v3_sub(nxt, plane_pt), plane_n);
+        const int cur_in = dc <= 0.0f, nxt_in = dn <= 0.0f;
+        if (cur_in) clip_add(&out, cur, in->feat[i]);
+        if (cur_in != nxt_in) {
+            const float t = dc / (dc - dn);
+            clip_add(&out, v3_make(cur.x + (nxt.x - cur.x) * t, cur.y + (nxt.y - cur.y) * t, cur.z + (nxt.z - cur.z) * t), in->feat[i]);
+        }
+    }
+    return out;
+}
+static v3 v3_neg(v3 a) { return v3_make(-a.x, -a.y, -a.z); }
+static float comp(v3 v, int k) { return k == 0 ? v.x : (k == 1 ? v.y : v.z); }
+
+/* analytical_manifold.hpp:503-736 BoxBox: the axis of least penetration among the 15 separating-axis candidates in
+ * fixed order (faces preferred by a 1e-5 bias); an edge pair gives one point between the closest edge points, a face
+ * gives the incident face clipped against the reference face's sides, reduced by ReduceAndEmitSpread */
+static void box_box(const prim* A, const prim* B, float query, manifold* out) {
+    out->count = 0u;
+    const v3 dpos = v3_sub(B->t, A->t);
+    const v3 ax[3] = {A->cx, A->cy, A->cz}, bx[3] = {B->cx, B->cy, B->cz};
+    float AbsR[3][3];
+    for (int i = 0; i < 3; ++i)
+        for (int j = 0; j < 3; ++j) { const float r = v3_dot(ax[i], bx[j]); AbsR[i][j] = (r < 0.0f ? -r : r) + 1.0e-6f; }
+    const float ea[3] = {A->half.x, A->half.y, A->half.z}, eb[3] = {B->half.x, B->half.y, B->half.z};
+    const float dA[3] = {v3_dot(dpos, ax[0]), v3_dot(dpos, ax[1]), v3_dot(dpos, ax[2])};
+    float min_pen = 3.4e38f;
+    int best_axis = -1;
+    v3 best_n = v3_make(0, 1, 0);
+    const float bias = 1.0e-5f;
+    for (int i = 0; i < 3; ++i) {
+        const float ra = ea[i], rb = eb[0] * AbsR[i][0] + eb[1] * AbsR[i][1] + eb[2] * AbsR[i][2];
+        const float s = dA[i] < 0.0f ? -dA[i] : dA[i];
+        const float pen = (ra + rb) - s;
+        if (pen <= -query) return;
+        if (pen < min_pen - bias) { min_pen = pen; best_axis = i; best_n = dA[i] < 0.0f ? v3_neg(ax[i]) : ax[i]; }
+    }
+    for (int j = 0; j < 3; ++j) {
+        const float ra = ea[0] * AbsR[0][j] + ea[1] * AbsR[1][j] + ea[2] * AbsR[2][j], rb = eb[j];
+        const float dBj = v3_dot(dpos, bx[j]);
+        const float s = dBj < 0.0f ? -dBj : dBj;
+        const float pen = (ra + rb) - s;
+        if (pen <= -query) return;
+        if (pen < min_pen - bias) { min_pen = pen; best_axis = 3 + j; best_n = dBj < 0.0f ? v3_neg(bx[j]) : bx[j]; }
+    }
+    for (int i = 0; i < 3; ++i)
+        for (int j = 0; j < 3; ++j) {
+            v3 L = v3_cross(ax[i], bx[j]);
+            const float Llen = sqrtf(L.x * L.x + L.y * L.y + L.z * L.z);
+            if (Llen < 1.0e-6f) continue;
+            L = v3_make(L.x / Llen, L.y / Llen, L.z / Llen);
+            const float ra = ea[0] * fabsf(v3_dot(ax[0], L)) + ea[1] * fabsf(v3_dot(ax[1], L)) + ea[2] * fabsf(v3_dot(ax[2], L));
+            const float rb = eb[0] * fabsf(v3_dot(bx[0], L)) + eb[1] * fabsf(v3_dot(bx[1], L)) + eb[2] * fabsf(v3_dot(bx[2], L));
+            const float s = v3_dot(dpos, L);
+            const float pen = (ra + rb) - (s < 0.0f ? -s : s);
+            if (pen <= -query) return;
+            if (pen < min_pen - bias) { min_pen = pen; best_axis = 6 + i * 3 + j; best_n = s < 0.0f ? v3_neg(L) : L; }
+        }
+    if (best_axis < 0) return;
+    if (best_axis >= 6) {   /* edge against edge: one point between the closest points of the two edges */
+        const int i = (best_axis - 6) / 3, j = (best_axis - 6) % 3;
+        v3 pa = A->t, pb = B->t;
+        for (int k = 0; k < 3; ++k) {
+            if (k == i) continue;
+            const float sgn = v3_dot(ax[k], best_n) >= 0.0f ? 1.0f : -1.0f;
+            pa = v3_add(pa, v3_scale(ax[k], sgn * ea[k]));
+        }
+        for (int k = 0; k < 3; ++k) {
+            if (k == j) continue;
+            const float sgn = v3_dot(bx[k], best_n) >= 0.0f ? -1.0f : 1.0f;
+            pb = v3_add(pb, v3_scale(bx[k], sgn * eb[k]));
+        }
+        const v3 r = v3_sub(pa, pb);
+        const float aa = 1.0f, bb = v3_dot(ax[i], bx[j]), cc = 1.0f;
+        const float dd = v3_dot(ax[i], r), ee = v3_dot(bx[j], r);
+        const float denom = aa * cc - bb * bb;
+        float sN = 0.0f, tN = 0.0f;
+        if (denom > 1.0e-9f) { sN = (bb * ee - cc * dd) / denom; tN = (aa * ee - bb * dd) / denom; }
+        const float sCl = sN < -ea[i] ? -ea[i] : (sN > ea[i] ? ea[i] : sN);
+        const float tCl = tN < -eb[j] ? -eb[j] : (tN > eb[j] ? eb[j] : tN);
+        const v3 ca = v3_add(pa, v3_scale(ax[i], sCl)), cb = v3_add(pb, v3_scale(bx[j], tCl));
+        emit_one(out, v3_scale(v3_add(ca, cb), 0.5f), best_n, min_pen, 0xE0000000ull | ((uint64_t)i << 4) | (uint64_t)j);
+        return;
+    }
+    const int ref_is_A = best_axis < 3;
+    const int ref_axis = ref_is_A ? best_axis : best_axis - 3;
+    const prim* Rf = ref_is_A ? A : B;
+    const prim* If = ref_is_A ? B : A;
+    const v3 rax[3] = {Rf->cx, Rf->cy, Rf->cz}, iax[3] = {If->cx, If->cy, If->cz};
+    const v3 rhe = Rf->half, ihe = If->half;
+    v3 refN = rax[ref_axis];
+    if (v3_dot(v3_sub(If->t, Rf->t), refN) < 0.0f) refN = v3_neg(refN);
+    int inc_axis = 0; float best_dot = 3.4e38f, inc_sign = 1.0f;
+    for (int k = 0; k < 3; ++k) {
+        const float d = v3_dot(iax[k], refN);
+        const float ad = d < 0.0f ? -d : d;
+        if (-ad < best_dot) { best_dot = -ad; inc_axis = k; inc_sign = d < 0.0f ? 1.0f : -1.0f; }
+    }
+    const int iu = (inc_axis + 1) % 3, iv = (inc_axis + 2) % 3;
+    const v3 inc_face_center = v3_add(If->t, v3_scale(iax[inc_axis], inc_sign * comp(ihe, inc_axis)));
+    const v3 iu_w = iax[iu], iv_w = iax[iv];
+    const float iu_e = comp(ihe, iu), iv_e = comp(ihe, iv);
+    clip_poly poly; poly.count = 0;
+    const float su[4] = {-1.0f, 1.0f, 1.0f, -1.0f}, sv[4] = {-1.0f, -1.0f, 1.0f, 1.0f};
+    for (uint32_t k = 0u; k < 4u; ++k)
+        clip_add(&poly, v3_add(v3_add(inc_face_center, v3_scale(iu_w, su[k] * iu_e)), v3_scale(iv_w, sv[k] * iv_e)), ((uint32_t)inc_axis << 4) | k);
+    const int ru = (ref_axis + 1) % 3, rv = (ref_axis + 2) % 3;
+    const v3 ru_w = rax[ru], rv_w = rax[rv];
+    const float ru_e = comp(rhe, ru), rv_e = comp(rhe, rv);
+    const v3 ref_face_center = v3_add(Rf->t, v3_scale(refN, comp(rhe, ref_axis)));
+    poly = clip_against_plane(&poly, v3_add(ref_face_center, v3_scale(ru_w, ru_e)), ru_w);
+    poly = clip_against_plane(&poly, v3_sub(ref_face_center, v3_scale(ru_w, ru_e)), v3_neg(ru_w));
+    poly = clip_against_plane(&poly, v3_add(ref_face_center, v3_scale(rv_w, rv_e)), rv_w);
+    poly = clip_against_plane(&poly, v3_sub(ref_face_center, v3_scale(rv_w, rv_e)), v3_neg(rv_w));
+    v3 position[8]; float pen[8]; uint32_t feature[8];
+    int ncand = 0;
+    for (int k = 0; k < poly.count; ++k) {
+        const float depth = v3_dot(v3_sub(ref_face_center, poly.v[k]), refN);
+        if (depth >= -query) {
+            const v3 onref = v3_add(poly.v[k], v3_scale(refN, depth));
+            position[ncand] = v3_scale(v3_add(poly.v[k], onref), 0.5f);
+            pen[ncand] = depth; feature[ncand] = (uint32_t)k; ++ncand;
+        }
+    }
+    const v3 normalA = ref_is_A ? v3_neg(refN) : refN;
+    if (ncand == 0) {
+        emit_one(out, v3_add(inc_face_center, v3_scale(refN, min_pen * 0.5f)), normalA, min_pen, (uint64_t)inc_axis << 4);
+        return;
+    }
+    reduce_and_emit_spread(position, pen, feature, ncand, normalA, out);
+}
+
+/* analytical_manifold.hpp:934-971 PrimitivePair, every analytic pair; a flipped pair negates the
  * normals.  Returns 0 for a pair that has no analytic manifold. */
 static int primitive_pair(uint32_t ka, const prim* a, uint32_t kb, const prim* b, float query, manifold* out) {
     out->count = 0u;
@@ -488,6 +628,7 @@ static int primitive_pair(uint32_t ka, const prim* a, uint32_t kb, const prim* b
     if (ka == NKO_SPHERE && kb == NKO_BOX) { sphere_box(a, b, query, out); return 1; }
     if (ka == NKO_SPHERE && kb == NKO_PLANE) { sphere_plane(a, b, query, out); return 1; }
     if (ka == NKO_BOX && kb == NKO_PLANE) { box_plane(a, b, query, out); return 1; }
+    if (ka == NKO_BOX && kb == NKO_BOX) { box_box(a, b, query, out); return 1; }
     if (ka == NKO_CAPSULE && kb == NKO_PLANE) { capsule_plane(a, b, query, out); return 1; }
     if (ka == NKO_CAPSULE && kb == NKO_SPHERE) { capsule_sphere(a, b, query, out); return 1; }
     if (ka == NKO_CAPSULE && kb == NKO_CAPSULE) { capsule_capsule(a, b, query, out); return 1; }
@@ -511,7 +652,6 @@ int nko_pair_has_manifold(uint32_t ka, uint32_t kb) {
     for (int i = 0; i < 5; ++i) { known_a |= ka == kinds[i]; known_b |= kb == kinds[i]; }
     if (!known_a || !known_b) return 0;
     if (ka == NKO_PLANE && kb == NKO_PLANE) return 0;
-    if (ka == NKO_BOX && kb == NKO_BOX) return 0;
     if ((ka == NKO_CYLINDER && (kb == NKO_CYLINDER || kb == NKO_BOX || kb == NKO_CAPSULE)) ||
         (kb == NKO_CYLINDER && (ka == NKO_BOX || ka == NKO_CAPSULE))) return 0;
     if ((ka == NKO_CAPSULE && kb == NKO_BOX) || (ka == NKO_BOX && kb == NKO_CAPSULE)) return 0;

@@ -2,8 +2,8 @@
  * CPU oracle for the batched articulation step: TEST INFRASTRUCTURE ONLY.
  *
  * A plain-C, one-environment-at-a-time fp32 restatement of the reference's CUDA kernels for
- * forward kinematics, RNEA bias + CRBA + LDL^T forward dynamics, the sphere/box x plane contact
- * pipeline (pairs, manifolds, rows, chain Jacobians) and the UABD tile block-descent solve with its
+ * forward kinematics, RNEA bias + CRBA + LDL^T forward dynamics, the contact pipeline of analytic
+ * primitive pairs (pairs, manifolds, rows, chain Jacobians) and the UABD tile block-descent solve with its
  * split-impulse position pass.  Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline
  * leg may load it, and only as the checker.  Nothing shipped links or calls it.
  *
@@ -22,7 +22,8 @@
  *   manifolds, compose, contact id, query band, filter, projection roundoff :
  *                             pinned bit-exact against oracle/_ref (the reference's own host headers) and the
  *                             committed vectors tests/golden/rowmath_vectors.npz; the prim-frame bake is device-only
- *                             code and is pinned by the rotation-matrix closed form instead
+ *                             code and is pinned by the rotation-matrix closed form instead.  Every pair kind of
+ *                             PrimitivePair is covered (sphere, capsule, box, plane, cylinder; box x box included)
  *   row math (AL impulses)  : pinned bit-exact against oracle/_ref (augmented_row.hpp), the committed vectors, and
  *                             the known answers in tests/math/test_contact_tangent.cpp
  *   chain Jacobian          : pinned (J qdot == contact point velocity of the float64 model)
@@ -159,7 +160,7 @@ float nko_contact_query_reach(float thickness, float margin);
 float nko_contact_motion_radius(float base, float dt, float sa, float sb, float relax);
 int nko_shape_filter_admits(uint32_t ta, uint32_t aa, uint32_t ga, uint32_t tb, uint32_t ab, uint32_t gb);
 int nko_pair_excluded(const nko_world* w, uint32_t a, uint32_t b);
-int nko_pair_has_manifold(uint32_t kind_a, uint32_t kind_b);   /* every analytic pair of PrimitivePair but box x box */
+int nko_pair_has_manifold(uint32_t kind_a, uint32_t kind_b);   /* the analytic pairs of PrimitivePair */
 void nko_compose_transform(const float parent[7], const float child[7], float out[7]);
 void nko_make_contact_id(uint32_t a, uint32_t b, const float local_a[3], const float local_b[3], uint32_t feature,
                          uint32_t manifold_slot, uint64_t out[2]);

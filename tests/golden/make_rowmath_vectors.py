@@ -33,9 +33,9 @@ def frame(pose):
     return np.concatenate([R[:, 0], R[:, 1], R[:, 2], pose[:3]]).astype(np.float32)
 
 
-# every ordered kind pair PrimitivePair answers analytically, box x box aside (sphere 0, capsule 1, box 2, plane 3,
-# cylinder 7)
-PAIR_ORDERS = [(0, 0), (0, 2), (2, 0), (1, 3), (3, 1), (1, 0), (0, 1), (1, 1), (7, 3), (3, 7), (7, 0), (0, 7)]
+# every ordered kind pair PrimitivePair answers analytically beyond those of the first block (sphere 0, capsule 1, box 2,
+# plane 3, cylinder 7); box x box twice over, for its many branches
+PAIR_ORDERS = [(0, 0), (0, 2), (2, 0), (1, 3), (3, 1), (1, 0), (0, 1), (1, 1), (7, 3), (3, 7), (7, 0), (0, 7), (2, 2), (2, 2)]
 
 
 def pair_shape(g, kind):
@@ -62,6 +62,9 @@ def pair_case(g, ka, kb):
                 q /= np.linalg.norm(q)
                 if g.uniform() < 0.5:
                     q = np.array([-q[1], q[0], q[3], -q[2]])   # turned over
+            if (ka, kb) == (2, 2) and g.uniform() < 0.5:   # boxes nearly aligned, or aligned: faces meet faces
+                q = np.array([1, 0, 0, 0]) + g.normal(0, g.choice([0.0, 0.02]), 4)
+                q /= np.linalg.norm(q)
             pose[side] = np.concatenate([g.normal(0, 0.04, 3), q])
             if 3 in (ka, kb):
                 pose[side, 2] = g.uniform(-0.02, 0.12)

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 from conftest import nk, relative_error
-from test_oracle_pairs import floating, floating_state, rail_state, rails
+from test_oracle_pairs import box_on_slab, floating, floating_state, rail_state, rails
 
 pytestmark = pytest.mark.gpu
 abi = nk.abi
@@ -69,7 +69,7 @@ def pair_state(t, E, seed, kinds):
 
 
 PAIRS = [(SPHERE, SPHERE), (SPHERE, BOX), (BOX, SPHERE), (CAPSULE, PLANE), (PLANE, CAPSULE), (CAPSULE, SPHERE), (SPHERE, CAPSULE),
-         (CAPSULE, CAPSULE), (CYLINDER, PLANE), (PLANE, CYLINDER), (CYLINDER, SPHERE), (SPHERE, CYLINDER)]
+         (CAPSULE, CAPSULE), (CYLINDER, PLANE), (PLANE, CYLINDER), (CYLINDER, SPHERE), (SPHERE, CYLINDER), (BOX, BOX)]
 
 
 @pytest.mark.parametrize("ka,kb", PAIRS)
@@ -87,7 +87,8 @@ def test_every_analytic_pair_matches_the_oracle(oracle_py, device, ka, kb):
                         ("NarrowphasePrimitives", "narrowphase"), ("AssembleRows", "assemble_rows")):
         oracle.op(oname); world.op(name)
     world.synchronize()
-    for name in ("pair_count", "candidate_pairs", "ucontact_count", "ucontact_row_range", "ucontact_id_pair", "row_count"):
+    exact = ("pair_count", "candidate_pairs") if (ka, kb) == (BOX, BOX) else ("pair_count", "candidate_pairs", "ucontact_count", "ucontact_row_range", "ucontact_id_pair", "row_count")
+    for name in exact:
         assert np.array_equal(world.download(name), oracle.download(name)), name
     counts = oracle.download("ucontact_count").reshape(E, -1)
     assert (counts > 0).sum() >= E // 5 and (counts == 0).sum() >= E // 10          # touching and apart both occur
@@ -108,6 +109,9 @@ def test_every_analytic_pair_matches_the_oracle(oracle_py, device, ka, kb):
     same = np.ones(E, bool)
     if CYLINDER in (ka, kb) and PLANE in (ka, kb):
         same &= ~((keys_g != keys_o) & live).any(1)
+    if (ka, kb) == (BOX, BOX):       # the winning axis of fifteen, and the clipped polygon's vertices, change with the last bits
+        same &= ~(((keys_g != keys_o) | (np.abs(point_g - point_o).max(2) > 1e-4)) & live).any(1)
+        same &= world.download("ucontact_count") == counts.reshape(-1)
     if (ka, kb) == (CAPSULE, CAPSULE):
         same &= ~((np.abs(point_g - point_o).max(2) > 1e-4) & live).any(1)
         # the normal is the difference of the closest axis points over its length: within two centimetres the
@@ -133,7 +137,7 @@ def test_every_analytic_pair_matches_the_oracle(oracle_py, device, ka, kb):
     oracle.op("contact_warm_start", 0); world.op("ContactWarmStart", 0)
     oracle.op("block_descent_solve"); world.op("BlockDescentSolve")
     world.synchronize()
-    assert np.array_equal(world.download("env_status"), oracle.download("env_status"))
+    assert np.array_equal(world.download("env_status")[same], oracle.download("env_status")[same])
     for name in ("qdot", "lambda"):
         assert relative_error(world.download(name).reshape(E, -1)[same], oracle.download(name).reshape(E, -1)[same]) <= TOL, name
     world.close()
@@ -169,16 +173,19 @@ def test_rows_of_one_link_and_excluded_rows_never_pair(device):
         world.close()
 
 
-@pytest.mark.parametrize("shape", ["capsule_lying", "cylinder_standing"])
+@pytest.mark.parametrize("shape", ["capsule_lying", "cylinder_standing", "box_on_box"])
 def test_supports_carry_the_weight(oracle_py, device, shape):
-    """A capsule lying on the plane (two points) and a cylinder standing on it (four): the normal impulses add up to
-    the weight, the body stays at rest, and the device agrees with the oracle."""
+    """A capsule lying on the plane (two points), a cylinder standing on it (four) and a box on a static box (four):
+    the normal impulses add up to the weight, the body stays at rest, and the device agrees with the oracle."""
     mass, radius, half, dt, g = 1.3, 0.04, 0.1, 1.0 / 200.0, 9.81
     if shape == "capsule_lying":
         kind, pose, points = CAPSULE, [0, 0, radius - 1e-3, np.sqrt(0.5), 0, np.sqrt(0.5), 0], 2
-    else:
+    elif shape == "cylinder_standing":
         kind, pose, points = CYLINDER, [0, 0, half - 1e-3, 1, 0, 0, 0], 4
-    t, desc = floating(kind, (radius, half, 0, 0), mass, (0.01, 0.01, 0.01)), abi.world_desc(1, dt, vel_iters=100)
+    else:
+        kind, pose, points = BOX, [0.02, -0.01, 0.05 - 1e-3, np.cos(0.15), 0, 0, np.sin(0.15)], 4
+    t = box_on_slab(mass) if kind == BOX else floating(kind, (radius, half, 0, 0), mass, (0.01, 0.01, 0.01))
+    desc = abi.world_desc(1, dt, vel_iters=100)
     world, oracle = nk.World(device, t, desc), oracle_py.OracleWorld(t, desc, threads=1)
     for w in (world, oracle):
         w.set_state(floating_state(pose))

@@ -179,7 +179,7 @@ def test_error_paths(device):
     assert lib.nuka_world_set_execution_mode(world._h, 5) == 1
     world.close()
     # templates outside the path are refused at creation
-    for kinds in ((abi.SHAPE_BOX, abi.SHAPE_BOX), (abi.SHAPE_CAPSULE, abi.SHAPE_BOX), (abi.SHAPE_CYLINDER, abi.SHAPE_CAPSULE), (4, abi.SHAPE_PLANE)):
+    for kinds in ((abi.SHAPE_CYLINDER, abi.SHAPE_CYLINDER), (abi.SHAPE_CAPSULE, abi.SHAPE_BOX), (abi.SHAPE_CYLINDER, abi.SHAPE_CAPSULE), (4, abi.SHAPE_PLANE)):
         t = abi.Template()   # an admitted pair without an analytic manifold, or a shape kind outside the path
         t.add_link(abi.JOINT_FLOATING, None)
         t.add_link(abi.JOINT_REVOLUTE, 0)

@@ -124,3 +124,28 @@ def test_supports_carry_the_weight(oracle_py, shape):
     assert np.abs(out["twist"][0]).max() < 3e-5
     if points == 2:
         assert np.abs(lam - lam.mean()).max() < 1e-3 * lam.mean()
+
+
+def box_on_slab(mass):
+    """A floating box over a static slab (a box as well) whose top face lies in the plane z = 0."""
+    t = abi.Template()
+    t.add_link(abi.JOINT_FLOATING, None, mass=mass, diag_inertia=(0.01, 0.012, 0.009))
+    profile = t.add_profile(0.8)
+    t.add_body(abi.ROLE_STATIC, kind=abi.SHAPE_BOX, params=(0.5, 0.4, 0.1, 0), local_pos=(0, 0, -0.1), contype=2, conaffinity=1, profile=profile)
+    t.add_body(abi.ROLE_LINK_BODY, link=0, contype=0, conaffinity=0)
+    t.add_body(abi.ROLE_PROXY, link=0, kind=abi.SHAPE_BOX, params=(0.08, 0.06, 0.05, 0), contype=1, conaffinity=2, profile=profile)
+    return t
+
+
+def test_box_rests_on_a_box(oracle_py):
+    """Face on face: the clipped incident face gives four points that carry the weight between them; turned about
+    the vertical by any angle the box still rests (the clip polygon changes, the support does not)."""
+    mass, dt, g = 2.1, 1.0 / 200.0, 9.81
+    for angle in (0.0, 0.3, 0.7853982):
+        pose = [0.02, -0.01, 0.05 - 1e-3, np.cos(angle / 2), 0, 0, np.sin(angle / 2)]
+        out = contact_step(oracle_py, box_on_slab(mass), abi.world_desc(1, dt, vel_iters=100), floating_state(pose))
+        assert out["pairs"][0] == 1 and out["count"][0, 0] == 4 and out["status"][0] == 0
+        normal = np.nonzero(out["rows"].view(np.uint32)[0, :, 0] & CONTACT_NORMAL)[0]
+        lam = out["lambda"][0, normal]
+        assert len(normal) == 4 and abs(lam.sum() - mass * g * dt) < 3e-5 * mass and lam.min() > 0.1 * lam.mean()
+        assert np.abs(out["twist"][0]).max() < 3e-5
