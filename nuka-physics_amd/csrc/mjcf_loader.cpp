@@ -543,7 +543,7 @@ struct Builder {
     bool floating_root = false;
     V3 base_position;
     Quat base_rotation;
-    uint32_t dropped_geoms = 0u, actuator_count = 0u, articulation_roots = 0u;
+    uint32_t dropped_geoms = 0u, actuator_count = 0u;
 
     // ParseGeoms (mjcf_importer.cpp:779-1036), collision attributes and mass only
     void ParseGeoms(const Element& body, const char* child_class, V3 shift, std::vector<Geom>* out, BodyMass* mass) {
@@ -616,9 +616,8 @@ struct Builder {
             chain.push_back({&joint, anchor});
         });
         const bool is_free = free_joint != nullptr || free_by_type;
-        if (is_free && (!root || !chain.empty())) throw std::runtime_error("MJCF freejoint must be the only joint of a root body");
+        if (is_free && (!root || !chain.empty())) throw std::runtime_error("MJCF: a free joint must be the only joint of the only body under <worldbody>");
         if (root) {
-            if (articulation_roots++ > 0u) throw std::runtime_error("MJCF: more than one articulation under <worldbody> is not supported on this path");
             // articulations root at static bodies, so a root hinge or slide turns against a static anchor
             if (!chain.empty()) {
                 Link anchor_link;
@@ -845,9 +844,20 @@ std::unique_ptr<Scene> LoadMjcf(const std::string& path, uint32_t flags) {
     }
     mujoco->Each("default", [&](const Element& e) { ParseDefaultElement(e, b.context.root, &b.context); });
     // geoms placed straight in <worldbody> are static collidables; included files bring worldbody sections of their own
+    // Several bodies straight under <worldbody> (a robot beside a table, say) hang off one static link that stands for
+    // the world; a single one is the articulation's root itself.  A floating body has to be that single root.
+    uint32_t top_level_bodies = 0u;
+    mujoco->Each("worldbody", [&](const Element& worldbody) { worldbody.Each("body", [&](const Element&) { ++top_level_bodies; }); });
+    uint32_t top_parent = 0xFFFFFFFFu;
+    if (top_level_bodies > 1u) {
+        Link world;
+        world.name = "world";
+        b.links.push_back(world);
+        top_parent = 0u;
+    }
     mujoco->Each("worldbody", [&](const Element& worldbody) {
         b.ParseGeoms(worldbody, nullptr, V3{}, &b.world_geoms, nullptr);
-        worldbody.Each("body", [&](const Element& e) { b.ParseBody(e, 0xFFFFFFFFu, nullptr); });
+        worldbody.Each("body", [&](const Element& e) { b.ParseBody(e, top_parent, nullptr); });
     });
     if (b.links.empty()) throw std::runtime_error("MJCF: no body under <worldbody> in " + path);
     mujoco->Each("contact", [&](const Element& contact) {
@@ -958,7 +968,7 @@ std::unique_ptr<Scene> LoadMjcf(const std::string& path, uint32_t flags) {
         for (const auto& names : b.excluded_bodies) {
             uint32_t found[2] = {0xFFFFFFFFu, 0xFFFFFFFFu};
             for (uint32_t l = 0u; l < nl; ++l) for (int k = 0; k < 2; ++k) if (!b.links[l].intermediate && b.links[l].name == (k == 0 ? names.first : names.second)) found[k] = l;
-            if (found[0] == 0xFFFFFFFFu || found[1] == 0xFFFFFFFFu) throw std::runtime_error("MJCF: <exclude> names an unknown body");
+            if (found[0] == 0xFFFFFFFFu || found[1] == 0xFFFFFFFFu) continue;   // an unknown body name is skipped, as the reference's importer does
             exclude_links(found[0], found[1]);
         }
     }

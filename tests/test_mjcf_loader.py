@@ -237,11 +237,29 @@ def test_capsule_walker_links_meet_each_other_but_not_their_parents(oracle_py, t
     assert frozenset(("l_thigh", "r_thigh")) in met or frozenset(("l_shin", "r_shin")) in met
     assert all("world" in pair for pair in ({frozenset((owner[x], owner[y])) for x, y in zip(a_rows[0][live[0]], b_rows[0][live[0]])}))
     w.close()
-    bad = tmp_path / "exclude.xml"
-    bad.write_text('<mujoco><worldbody><body name="a"><freejoint/><geom size="0.1"/></body></worldbody>'
-                   '<contact><exclude body1="a" body2="nobody"/></contact></mujoco>')
-    with pytest.raises(nk.NukaError):
-        nk.Scene(str(bad))
+
+
+def test_contact_filtering_fixture_of_the_reference():
+    """tests/data/contact_filtering.xml with the expectations of tests/import/test_mjcf_contact_filtering.cpp that bear
+    on pairing: explicit and class-inherited contype / conaffinity / group, the geom that collides with nothing, the
+    friction kept from a geom's first coefficient, the body pair excluded and the unknown body name skipped.  Its two
+    jointless bodies both sit under <worldbody>: they hang off one static world link."""
+    scene = nk.Scene(os.path.join(GOLDEN, "contact_filtering.xml"))
+    assert scene.link_names == ["world", "b1", "b2"]
+    a = scene.template_arrays()
+    assert list(a["joint_type"]) == [abi.JOINT_FIXED] * 3 and list(a["parent_link"]) == [abi.INVALID, 0, 0]
+    owner = [scene.link_names[l] for l in a["body_link"]]
+    rows = [(owner[r], int(a["shape_kind"][r]), int(a["shape_contype"][r]), int(a["shape_conaffinity"][r]), int(a["shape_group"][r]))
+            for r in range(len(owner)) if a["shape_kind"][r] != abi.INVALID]
+    assert rows == [("b1", abi.SHAPE_BOX, 2, 4, 3),         # g_explicit
+                    ("b1", abi.SHAPE_SPHERE, 1, 1, 0),      # g_default; g_visual (contype 0, conaffinity 0) has no row
+                    ("b2", abi.SHAPE_BOX, 8, 1, 0),         # g_class inherits contype 8
+                    ("b2", abi.SHAPE_BOX, 10, 1, 0)]        # g_class_override: its own contype wins
+    explicit = [r for r in range(len(owner)) if a["shape_kind"][r] != abi.INVALID][0]
+    assert a["profile_mu"].reshape(-1, 2)[a["shape_profile"][explicit]][0] == np.float32(0.7)
+    assert a["shape_profile"][explicit + 1] == abi.INVALID                              # friction never authored: the default
+    excluded = {frozenset((owner[p[0]], owner[p[1]])) for p in a["excluded_pairs"].reshape(-1, 2)}
+    assert excluded == {frozenset(("b1", "b2"))}
 
 
 def test_errors(tmp_path):
