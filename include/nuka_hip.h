@@ -118,16 +118,26 @@ typedef struct nuka_world_desc_t {
                                               struct_size covers it */
 } nuka_world_desc_t;
 
-/* Scene files (src/import/mjcf_importer.cpp LoadMjcf, then the articulation part of the cook): a MuJoCo XML robot
- * description read into the cook inputs of one environment.  One articulation per file; bodies, default classes,
- * hinge / slide / free joints (several per body), inertial elements or geom-derived mass, sphere / box / plane
- * collision geoms, joint ranges, damping, armature, frictionloss, springs, and position / velocity / motor actuators.
- * Joint and contact rows use this library's native laws (no solref / solimp compliance). */
+/* Scene files (src/import/mjcf_importer.cpp LoadMjcf and src/import/urdf_importer.cpp LoadUrdf, then the articulation
+ * part of the cook): a robot description read into the cook inputs of one environment.  One articulation per file.
+ * MJCF: bodies, default classes, hinge / slide / free joints (several per body), inertial elements or geom-derived
+ * mass, sphere / capsule / box / cylinder / plane collision geoms, joint ranges, damping, armature, frictionloss,
+ * springs, <contact><exclude>, and position / velocity / motor actuators.  URDF: links with inertial and collision
+ * elements (box, sphere, cylinder, capsule), revolute / continuous / prismatic / fixed joints with origin, axis, limits,
+ * dynamics and effort (a bounded torque motor), nuka:exclude.  A body never pairs with its parent body or with a body
+ * welded to it (src/scene/cooker.cpp:470-538).  Joint and contact rows use this library's native laws (no solref /
+ * solimp compliance). */
 typedef struct nuka_scene_t* nuka_scene_handle;
-/* Keep sphere and box geoms against planes only: other colliding geoms are dropped and counted, and the robot's geoms
- * share one negative collision group, so that they meet the ground and not each other. */
+/* Keep the shapes this library has manifolds for and drop (and count) the other colliding geoms; the robot's geoms
+ * share one negative collision group, so that they meet static shapes and not each other. */
 #define NUKA_SCENE_PLANE_CONTACTS_ONLY 1u
+/* URDF only: the root link is welded to the world (the importer's fix_base option, src/import/urdf_importer.cpp:655-661);
+ * without it the root link floats. */
+#define NUKA_SCENE_FIXED_BASE 2u
+/* A static ground plane z = 0 joins the file's collidables (a URDF describes the robot only). */
+#define NUKA_SCENE_GROUND_PLANE 4u
 nuka_result_t nuka_scene_load_mjcf(const char* path, uint32_t flags, nuka_scene_handle* out);
+nuka_result_t nuka_scene_load_urdf(const char* path, uint32_t flags, nuka_scene_handle* out);
 void nuka_scene_destroy(nuka_scene_handle scene);
 /* The cook inputs; the arrays live as long as the scene. */
 const nuka_template_desc_t* nuka_scene_template(nuka_scene_handle scene);

@@ -36,6 +36,8 @@ class SceneInfoC(C.Structure):
 
 
 SCENE_PLANE_CONTACTS_ONLY = 1
+SCENE_FIXED_BASE = 2
+SCENE_GROUND_PLANE = 4
 
 
 class DeviceDescC(C.Structure):
@@ -51,7 +53,7 @@ EXPORTS = [
     "nuka_world_get_buffer_view", "nuka_world_upload_field", "nuka_world_download_field", "nuka_world_get_info",
     "nuka_world_time_steps", "nuka_world_profile_ops", "nuka_device_copy_bandwidth", "nuka_hip_register_backend_entry",
     "nuka_hip_op_count", "nuka_hip_op_name", "nuka_hip_op_from_name",
-    "nuka_scene_load_mjcf", "nuka_scene_destroy", "nuka_scene_template", "nuka_scene_get_info", "nuka_scene_link_name",
+    "nuka_scene_load_mjcf", "nuka_scene_load_urdf", "nuka_scene_destroy", "nuka_scene_template", "nuka_scene_get_info", "nuka_scene_link_name",
     "nuka_scene_joint_name", "nuka_scene_initial_state", "nuka_world_create_from_scene",
 ]
 
@@ -108,6 +110,7 @@ def lib():
         L.nuka_checkpoint_byte_size.argtypes = [C.c_void_p, C.POINTER(C.c_uint64)]
         L.nuka_device_copy_bandwidth.argtypes = [C.c_void_p, C.c_size_t, C.c_uint32, C.POINTER(C.c_float)]
         L.nuka_scene_load_mjcf.argtypes = [C.c_char_p, C.c_uint32, C.POINTER(C.c_void_p)]
+        L.nuka_scene_load_urdf.argtypes = [C.c_char_p, C.c_uint32, C.POINTER(C.c_void_p)]
         L.nuka_scene_destroy.argtypes = [C.c_void_p]
         L.nuka_scene_template.argtypes = [C.c_void_p]
         L.nuka_scene_template.restype = C.POINTER(TemplateDescC)
@@ -147,11 +150,13 @@ class Device:
 
 
 class Scene:
-    """A robot description file read into the cook inputs of one environment (nuka_scene_*; host code, no GPU)."""
+    """A robot description file (MJCF, or URDF by its extension) read into the cook inputs of one environment
+    (nuka_scene_*; host code, no GPU)."""
 
     def __init__(self, path, flags=0):
         self._h = C.c_void_p()
-        _check(lib().nuka_scene_load_mjcf(os.fsencode(path), flags, C.byref(self._h)))
+        load = lib().nuka_scene_load_urdf if str(path).lower().endswith(".urdf") else lib().nuka_scene_load_mjcf
+        _check(load(os.fsencode(path), flags, C.byref(self._h)))
         info = SceneInfoC()
         _check(lib().nuka_scene_get_info(self._h, C.byref(info)))
         self.info = info

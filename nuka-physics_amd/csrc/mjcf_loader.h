@@ -1,4 +1,4 @@
-// The MJCF template loader's result: the arrays behind a nuka_template_desc_t plus what else the file authors
+// The robot-description loaders' result: the arrays behind a nuka_template_desc_t plus what else the file authors
 // for the articulation-step path (names, initial state, drive parameters).  Host code only.
 #pragma once
 
@@ -16,6 +16,10 @@ namespace mjcf {
 // Keep sphere and box geoms against planes only: other colliding geoms are dropped (and counted), and the robot's
 // geoms share one negative collision group so that they meet the ground and not each other.
 constexpr uint32_t kPlaneContactsOnly = 1u;
+// URDF: the root link is welded to the world instead of floating.
+constexpr uint32_t kFixedBase = 2u;
+// A static ground plane z = 0 is added to the file's collidables (a URDF names none).
+constexpr uint32_t kGroundPlane = 4u;
 
 struct Scene {
     nuka_template_desc_t desc{};
@@ -36,6 +40,7 @@ struct Scene {
 
 // Throws std::runtime_error with the reason when the file cannot be read or uses what this path does not build.
 std::unique_ptr<Scene> LoadMjcf(const std::string& path, uint32_t flags);
+std::unique_ptr<Scene> LoadUrdf(const std::string& path, uint32_t flags);
 
 }  // namespace mjcf
 }  // namespace nkh

@@ -758,9 +758,24 @@ nuka_result_t nuka_scene_load_mjcf(const char* path, uint32_t flags, nuka_scene_
     if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
     *out = nullptr;
     if (path == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "path is null");
-    if ((flags & ~uint32_t(NUKA_SCENE_PLANE_CONTACTS_ONLY)) != 0u) return Error(NUKA_RESULT_INVALID_ARG, "unknown scene flag");
+    if ((flags & ~uint32_t(NUKA_SCENE_PLANE_CONTACTS_ONLY | NUKA_SCENE_GROUND_PLANE)) != 0u) return Error(NUKA_RESULT_INVALID_ARG, "unknown scene flag");
     try {
         *out = reinterpret_cast<nuka_scene_handle>(mjcf::LoadMjcf(path, flags).release());
+        return NUKA_RESULT_OK;
+    } catch (const std::bad_alloc&) {
+        return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
+    } catch (const std::exception& e) {
+        return Error(NUKA_RESULT_INVALID_ARG, e.what());
+    }
+}
+
+nuka_result_t nuka_scene_load_urdf(const char* path, uint32_t flags, nuka_scene_handle* out) {
+    if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    *out = nullptr;
+    if (path == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "path is null");
+    if ((flags & ~uint32_t(NUKA_SCENE_PLANE_CONTACTS_ONLY | NUKA_SCENE_FIXED_BASE | NUKA_SCENE_GROUND_PLANE)) != 0u) return Error(NUKA_RESULT_INVALID_ARG, "unknown scene flag");
+    try {
+        *out = reinterpret_cast<nuka_scene_handle>(mjcf::LoadUrdf(path, flags).release());
         return NUKA_RESULT_OK;
     } catch (const std::bad_alloc&) {
         return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");

@@ -100,6 +100,44 @@ def test_capsule_walker_matches_the_oracle(oracle_py, device):
     world.close(); oracle.close()
 
 
+LEGGED = os.path.join(ROOT, "tests", "data", "legged.urdf")
+
+
+def test_urdf_world_matches_the_oracle(oracle_py, device):
+    """A URDF walker on the added ground plane: box trunk, cylinder thighs, capsule shins, sphere feet, torque motors
+    bounded by the joints' efforts, knee limits and friction.  Environments start at different heights and tilts and
+    with different motor commands; the device and the oracle step the same loaded template."""
+    E, steps = 96, 16
+    with pytest.raises(nk.NukaError) as err:      # cylinder thighs could meet capsule shins and the box trunk: no analytic manifold
+        nk.World(device, nk.Scene(LEGGED, nk.SCENE_GROUND_PLANE), abi.world_desc(2, 1.0 / 240.0))
+    assert err.value.code == abi.RESULT_NOT_SUPPORTED
+    scene = nk.Scene(LEGGED, nk.SCENE_GROUND_PLANE | nk.SCENE_PLANE_CONTACTS_ONLY)     # the links meet the ground, not each other
+    assert scene.info.dropped_geom_count == 0
+    desc = abi.world_desc(E, 1.0 / 240.0, vel_iters=8)
+    world, oracle = nk.World(device, scene, desc), oracle_py.OracleWorld(scene, desc, threads=8)
+    state = scene.initial_state()
+    rng = np.random.default_rng(31)
+    nl = scene.link_count
+    tilt = np.array([1, 0, 0, 0]) + rng.normal(0, 0.03, (E, 4))
+    base = np.concatenate([rng.normal(0, 0.1, (E, 2)), rng.uniform(0.46, 0.5, (E, 1)), tilt / np.linalg.norm(tilt, axis=1, keepdims=True)], 1).astype(np.float32)
+    q = rng.normal(0, 0.15, (E, nl)).astype(np.float32) * (state["drive_force_limit"] >= 0)
+    command = (rng.normal(0, 20.0, (E, nl)) * (state["drive_force_limit"] > 0)).astype(np.float32)     # beyond the 30 N m effort now and then
+    for name in ("drive_force_limit", "drive_joint_force_limit"):
+        oracle.upload(name, np.tile(state[name], E))
+    for w in (oracle, world):
+        w.upload("q", q); w.upload("base_pose", base); w.upload("drive_target", command)
+    assert np.array_equal(world.download("drive_force_limit").reshape(E, nl)[7], state["drive_force_limit"])
+    world.step(steps); world.synchronize()
+    oracle.step(steps)
+    assert np.array_equal(world.download("env_status"), oracle.download("env_status")) and not world.download("env_status").any()
+    assert np.array_equal(world.download("contact_count"), oracle.download("contact_count")) and world.download("contact_count").max() >= 2
+    assert np.abs(oracle.download("actuator_effort")).max() <= 30.0 + 1e-3 and (oracle.download("actuator_saturated") != 0).any()
+    for name in ("q", "qdot", "base_pose", "link_pose", "actuator_effort", "joint_limit_impulse"):
+        error = relative_error(world.download(name), oracle.download(name))
+        assert error <= 5 * TOL, f"{name}: {error:.2e}"
+    world.close(); oracle.close()
+
+
 def test_scene_with_unsupported_collision_geometry_is_refused(device, tmp_path):
     path = tmp_path / "ellipsoid.xml"
     path.write_text('<mujoco><worldbody><geom type="plane" size="1 1 1"/><body pos="0 0 1"><freejoint/>'
