@@ -205,6 +205,8 @@ struct Tile {
     float* fields;   // kWideFields x cap, then kNarrowFields x (narrow + 1)
     float* vec;      // 4 x 64 scratch vectors, 16-byte aligned
     float mass_inverse;   // 1 / diagonal of the mass factor, lane = row
+    mutable float hessian_inverse;   // 1 / diagonal of the Hessian factor held in hfac, lane = row
+    mutable bool factor_current;     // no head's curvature has changed since hfac was factored: the Hessian is the same
     mutable uint32_t work;   // Newton steps and line probes of this solve, the next solve's scheduling key
     bool mass_valid;
     bool units;      // some head is a unit head
@@ -327,14 +329,20 @@ __device__ __forceinline__ void load_columns(const float* a, uint32_t lane, floa
 // transposed read of the backward substitution.
 template <int N>
 __device__ __forceinline__ bool cholesky_solve(const Tile& c, float (&hrow)[N], float g, float* d_out) {
-    float inverse = 0.0f;
-    const bool valid = factor_rows<N>(c.lane, hrow, &inverse);
-    if (!valid) return false;
-    store_rows<N>(c.hfac, c.lane, hrow);
-    __syncthreads();
+    if (c.factor_current) {   // the same Hessian as at the last factorisation: its factor is still in hfac
+        load_rows<N>(c.hfac, c.lane, hrow);
+    } else {
+        float inverse = 0.0f;
+        const bool valid = factor_rows<N>(c.lane, hrow, &inverse);
+        if (!valid) return false;
+        c.hessian_inverse = inverse;
+        store_rows<N>(c.hfac, c.lane, hrow);
+        __syncthreads();
+        c.factor_current = true;
+    }
     float col[N];
     load_columns<N>(c.hfac, c.lane, col);
-    *d_out = substitute<N>(c.lane, hrow, col, inverse, c.lane < c.n ? g : 0.0f);
+    *d_out = substitute<N>(c.lane, hrow, col, c.hessian_inverse, c.lane < c.n ? g : 0.0f);
     __syncthreads();
     return true;
 }
@@ -441,17 +449,25 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
     const bool mine = head_terms(c, lane, mf, mc, mn);
     const uint32_t my_axes = lane < c.heads ? c.U(hAxes, lane) : 0u;
     const uint32_t my_low = lane < c.heads ? c.U(hColumnsLow, lane) : 0u, my_high = lane < c.heads ? c.U(hColumnsHigh, lane) : 0u;
+    // The Hessian M + sum J^T C J changes only through the heads' curvatures: every head keeps the curvature of its
+    // last assembly in its fields, and while none differs the factor of the last factorisation still stands.
+    bool changed = false;
     for (uint32_t h = lane + kWave; h < c.heads; h += kWave) {
         float f[3], cv[6], noise[3];
         const bool contributes = head_terms(c, h, f, cv, noise);
 #pragma unroll
         for (int k = 0; k < 3; ++k) { c.F(hF + k, h) = f[k]; c.F(hNoise + k, h) = noise[k]; }
 #pragma unroll
-        for (int k = 0; k < 6; ++k) c.F(hC + k, h) = cv[k];
+        for (int k = 0; k < 6; ++k) { changed = changed || __float_as_uint(c.F(hC + k, h)) != __float_as_uint(cv[k]); c.F(hC + k, h) = cv[k]; }
         c.U(hContrib, h) = contributes ? 1u : 0u;
     }
+    if (lane < c.heads) {
+#pragma unroll
+        for (int k = 0; k < 6; ++k) { changed = changed || __float_as_uint(c.F(hC + k, lane)) != __float_as_uint(mc[k]); c.F(hC + k, lane) = mc[k]; }
+    }
+    if (__any(changed)) c.factor_current = false;
     if (c.units && lane < c.heads && c.U(hUnit, lane) != kInvalid) {   // a coordinate reads its unit heads' responses from the fields
-        c.F(hF, lane) = mf[0]; c.F(hC, lane) = mc[0]; c.F(hNoise, lane) = mn[0];
+        c.F(hF, lane) = mf[0]; c.F(hNoise, lane) = mn[0];
         c.U(hContrib, lane) = mine ? 1u : 0u;
     }
     __syncthreads();
@@ -1109,6 +1125,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     c.env = env; c.lane = lane; c.n = n; c.ld = uint32_t(N) + 1u; c.ldj = uint32_t(N); c.cap = cap; c.narrow = staged_cap; c.heads = 0u; c.iteration = 0u;
     c.tolerance = p.velocity_tolerance; c.failed = false; c.momentum = 0.0f; c.residual = 0.0f;
     c.mass_inverse = 0.0f; c.mass_valid = false; c.work = 0u; c.units = false;
+    c.hessian_inverse = 0.0f; c.factor_current = false;
 #ifdef NKH_SOLVER_PROFILE
     for (int i = 0; i < 26; ++i) c.prof[i] = 0;
     for (int i = 0; i < 4; ++i) c.prof_count[i] = 0u;
