@@ -205,7 +205,6 @@ struct Tile {
     float* fields;   // kWideFields x cap, then kNarrowFields x (narrow + 1)
     float* vec;      // 4 x 64 scratch vectors, 16-byte aligned
     float mass_inverse;   // 1 / diagonal of the mass factor, lane = row
-    mutable float hessian_inverse;   // 1 / diagonal of the Hessian factor held in hfac, lane = row
     mutable bool factor_current;     // no head's curvature has changed since hfac was factored: the Hessian is the same
     mutable uint32_t work;   // Newton steps and line probes of this solve, the next solve's scheduling key
     bool mass_valid;
@@ -329,20 +328,22 @@ __device__ __forceinline__ void load_columns(const float* a, uint32_t lane, floa
 // transposed read of the backward substitution.
 template <int N>
 __device__ __forceinline__ bool cholesky_solve(const Tile& c, float (&hrow)[N], float g, float* d_out) {
-    if (c.factor_current) {   // the same Hessian as at the last factorisation: its factor is still in hfac
-        load_rows<N>(c.hfac, c.lane, hrow);
-    } else {
+    if (!c.factor_current) {   // otherwise the Hessian is the one factored last: its factor is still in hfac
         float inverse = 0.0f;
         const bool valid = factor_rows<N>(c.lane, hrow, &inverse);
         if (!valid) return false;
-        c.hessian_inverse = inverse;
         store_rows<N>(c.hfac, c.lane, hrow);
         __syncthreads();
         c.factor_current = true;
     }
+    // rows, columns and the reciprocal diagonal come back from hfac on either path (the factor's own reciprocal is
+    // 1 / its diagonal entry, the same division)
+    const uint32_t row = local_lane(c.lane);
+    const float inverse = row < uint32_t(N) ? 1.0f / c.hfac[row * (N + 1) + row] : 0.0f;
     float col[N];
+    load_rows<N>(c.hfac, c.lane, hrow);
     load_columns<N>(c.hfac, c.lane, col);
-    *d_out = substitute<N>(c.lane, hrow, col, c.hessian_inverse, c.lane < c.n ? g : 0.0f);
+    *d_out = substitute<N>(c.lane, hrow, col, inverse, c.lane < c.n ? g : 0.0f);
     __syncthreads();
     return true;
 }
@@ -1125,7 +1126,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     c.env = env; c.lane = lane; c.n = n; c.ld = uint32_t(N) + 1u; c.ldj = uint32_t(N); c.cap = cap; c.narrow = staged_cap; c.heads = 0u; c.iteration = 0u;
     c.tolerance = p.velocity_tolerance; c.failed = false; c.momentum = 0.0f; c.residual = 0.0f;
     c.mass_inverse = 0.0f; c.mass_valid = false; c.work = 0u; c.units = false;
-    c.hessian_inverse = 0.0f; c.factor_current = false;
+    c.factor_current = false;
 #ifdef NKH_SOLVER_PROFILE
     for (int i = 0; i < 26; ++i) c.prof[i] = 0;
     for (int i = 0; i < 4; ++i) c.prof_count[i] = 0u;
