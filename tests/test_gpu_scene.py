@@ -97,6 +97,12 @@ def test_capsule_walker_matches_the_oracle(oracle_py, device):
     for name in ("q", "qdot", "base_pose", "link_pose", "actuator_effort"):
         error = relative_error(world.download(name).reshape(E, -1)[same], oracle.download(name).reshape(E, -1)[same])
         assert error <= 5 * TOL, f"{name}: {error:.2e}"        # a dozen steps of accumulated rounding
+    # the readout of link against link contacts: asked for, it runs on the current solution
+    oracle.op("readout_contact_wrench")
+    wrench_g, wrench_o = world.download("link_contact_wrench").reshape(E, nl, 6)[same], oracle.download("link_contact_wrench").reshape(E, nl, 6)[same]
+    assert np.abs(wrench_o).max() > 1.0 and relative_error(wrench_g, wrench_o) <= 10 * TOL
+    for name in ("contact_side_a_kind", "contact_side_b_kind", "contact_side_a_index", "contact_side_b_index"):
+        assert np.array_equal(world.download(name).reshape(E, S)[same], oracle.download(name).reshape(E, S)[same]), name
     world.close(); oracle.close()
 
 

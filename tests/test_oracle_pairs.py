@@ -149,3 +149,24 @@ def test_box_rests_on_a_box(oracle_py):
         lam = out["lambda"][0, normal]
         assert len(normal) == 4 and abs(lam.sum() - mass * g * dt) < 3e-5 * mass and lam.min() > 0.1 * lam.mean()
         assert np.abs(out["twist"][0]).max() < 3e-5
+
+
+def test_readout_of_a_link_pair_is_action_and_reaction(oracle_py):
+    """Two sliders pressed together by opposite forces: the contact readout gives each link the other's push - equal,
+    opposite, of the size that holds the forces apart - and names both owners."""
+    m1, m2, radius, dt = 0.8, 2.0, 0.05, 1.0 / 200.0
+    state = rail_state([[0.0, 2 * radius - 1e-3]], [[0.0, 0.0]])
+    state["tau"] = np.array([[0.0, 3.0, -3.0]], np.float32)
+    w = oracle_py.OracleWorld(rails(m1, m2, radius), abi.world_desc(1, dt, gravity=(0, 0, 0), vel_iters=50, pos_iters=0xFFFFFFFF), threads=1)
+    w.set_state(state)
+    w.step(1)
+    w.op("readout_contact_wrench")
+    wrench = w.download("link_contact_wrench").reshape(3, 6)
+    assert np.abs(w.download("qdot")).max() < 2e-5                                  # the pair stays put
+    assert wrench[1, 0] == pytest.approx(-3.0, rel=1e-3) and wrench[2, 0] == pytest.approx(3.0, rel=1e-3)
+    assert np.abs(wrench[1, :3] + wrench[2, :3]).max() < 1e-5 and np.abs(wrench[0]).max() == 0
+    # equal and opposite about the world origin as well: the two forces share a line of action
+    assert np.abs(wrench[1, 3:] + wrench[2, 3:]).max() < 1e-5
+    assert w.download("contact_side_a_kind")[0] == 1 and w.download("contact_side_b_kind")[0] == 1     # both sides on the articulation
+    assert sorted([int(w.download("contact_side_a_index")[0]), int(w.download("contact_side_b_index")[0])]) == [1, 2]
+    w.close()
