@@ -149,6 +149,75 @@ double nko_momentum_restart(const float point[3], const float next[3], const flo
     return momentum_restart(v3_make(point[0], point[1], point[2]), v3_make(next[0], next[1], next[2]),
                             v3_make(base[0], base[1], base[2]), v3_make(scale[0], scale[1], scale[2]));
 }
+/* ---- the compliant (MuJoCo-law) row terms and the elliptic cone.  The product builds rows of the native law only
+ * (compliance 0, Coulomb disc): these restatements have no device counterpart and exist so that the reference's known
+ * answers for them (tests/constraint/test_solref_solimp.cpp) are held and checked here too. ---- */
+static float clampf(float v, float lo, float hi) { return fminf(fmaxf(v, lo), hi); }
+/* constraint/solref_solimp.hpp:55-86 ComputeCompliantRowTerms -> k, b, imp, D, R, aref */
+void nko_compliant_row_terms(const float solref[2], const float solimp[5], float pos_imp, float pos_aref, float vel, float invweight,
+                             float dt, int refsafe, float out[6]) {
+    float timeconst = solref[0];
+    const float dampratio = solref[1];
+    if (refsafe) timeconst = fmaxf(timeconst, 2.0f * dt);
+    const float dmin = clampf(solimp[0], 1.0e-4f, 0.9999f), dmax = clampf(solimp[1], 1.0e-4f, 0.9999f);
+    const float width = fmaxf(1.0e-15f, solimp[2]);
+    const float mid = clampf(solimp[3], 1.0e-4f, 0.9999f);
+    const float power = fmaxf(1.0f, solimp[4]);
+    const float dmax_sq = dmax * dmax;
+    float k = 1.0f / (dmax_sq * timeconst * timeconst * dampratio * dampratio);
+    float b = 2.0f / (dmax * timeconst);
+    if (solref[0] <= 0.0f) k = -solref[0] / dmax_sq;
+    if (solref[1] <= 0.0f) b = -solref[1] / dmax;
+    const float x = fabsf(pos_imp) / width;
+    const float rising = (1.0f / powf(mid, power - 1.0f)) * powf(x, power);
+    const float falling = 1.0f - (1.0f / powf(1.0f - mid, power - 1.0f)) * powf(1.0f - x, power);
+    const float y = x < mid ? rising : falling;
+    float imp = clampf(dmin + y * (dmax - dmin), dmin, dmax);
+    if (x > 1.0f) imp = dmax;
+    const float D = 1.0f / fmaxf(invweight * (1.0f - imp) / imp, 1.0e-15f);
+    out[0] = k; out[1] = b; out[2] = imp; out[3] = D; out[4] = 1.0f / D; out[5] = -k * imp * pos_aref - b * vel;
+}
+/* constraint/solref_solimp.hpp:40-44 DiscretizeCompliantRow -> R, bias, reference gain (midpoint damping) */
+void nko_discretize_compliant_row(float R, float aref_bias, float damping, float dt, float out[3]) {
+    const double scale = 1.0 + 0.5 * (double)dt * damping;
+    out[0] = (float)(R / scale); out[1] = (float)(aref_bias / scale); out[2] = (float)((1.0 / (double)dt - 0.5 * damping) / scale);
+}
+/* augmented_row.hpp:48-55 ComputeEllipticResponse -> residual scale k[3], dual scale s[3] */
+static void elliptic_response(float cap, v3 compliance, v3* k, v3* s) {
+    const double tangent = fmin((double)compliance.y, (double)compliance.z);
+    const double normal_scale = 1.0 / (1.0 + (double)cap * compliance.x);
+    const double tangent_scale = 1.0 / (1.0 + (double)cap * tangent);
+    *k = v3_make((float)(cap * normal_scale), (float)(cap * tangent_scale * tangent / compliance.y), (float)(cap * tangent_scale * tangent / compliance.z));
+    *s = v3_make((float)normal_scale, (float)tangent_scale, (float)tangent_scale);
+}
+/* augmented_row.hpp:58-80 EvaluateEllipticImpulse -> impulse[3], curvature xx yy zz xy xz yz: the projection onto the
+ * friction cone in the metric that makes its cross section a circle */
+void nko_elliptic_impulse(const float dual[3], float cap, const float residual[3], const float compliance[3], float mu_first, float out[9]) {
+    v3 k, s;
+    elliptic_response(cap, v3_make(compliance[0], compliance[1], compliance[2]), &k, &s);
+    const v3 x = v3_make(fmaf(k.x, residual[0], s.x * dual[0]), fmaf(k.y, residual[1], s.y * dual[1]), fmaf(k.z, residual[2], s.z * dual[2]));
+    const v3 root = v3_make(sqrtf(k.x), sqrtf(k.y), sqrtf(k.z));
+    const float m = mu_first * root.x / root.y;
+    const float p = x.x / root.x, q1 = x.y / root.y, q2 = x.z / root.z;
+    const float t = hypotf(q1, q2);
+    for (int i = 0; i < 9; ++i) out[i] = 0.0f;
+    if (t <= m * p) { out[0] = x.x; out[1] = x.y; out[2] = x.z; out[3] = k.x; out[4] = k.y; out[5] = k.z; return; }
+    if (m * t + p <= 0.0f) return;
+    const float a = 1.0f / (1.0f + m * m);
+    const float projected = (p + m * t) * a;
+    const float u1 = q1 / t, u2 = q2 / t;
+    const float b = m * projected / t, along = m * m * a;
+    out[0] = projected * root.x; out[1] = m * projected * u1 * root.y; out[2] = m * projected * u2 * root.z;
+    out[3] = k.x * a; out[4] = k.y * (along * u1 * u1 + b * u2 * u2); out[5] = k.z * (along * u2 * u2 + b * u1 * u1);
+    out[6] = root.x * root.y * m * a * u1; out[7] = root.x * root.z * m * a * u2; out[8] = root.y * root.z * (along - b) * u1 * u2;
+}
+/* augmented_row.hpp:104-108 EllipticMultiplierStep */
+void nko_elliptic_multiplier_step(const float dual[3], const float next[3], float cap, const float compliance[3], float out[3]) {
+    v3 k, s;
+    elliptic_response(cap, v3_make(compliance[0], compliance[1], compliance[2]), &k, &s);
+    out[0] = fabsf(next[0] - dual[0]) / k.x; out[1] = fabsf(next[1] - dual[1]) / k.y; out[2] = fabsf(next[2] - dual[2]) / k.z;
+}
+
 static uint32_t residual_bits(float value) { return f2u(value <= FLT_MAX ? fabsf(value) : FLT_MAX); }   /* :735 */
 static float along_axis(float impulse, float velocity) { return impulse > 0.0f ? velocity : impulse < 0.0f ? -velocity : 0.0f; }   /* :773-775 */
 

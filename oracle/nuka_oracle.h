@@ -25,7 +25,9 @@
  *                             code and is pinned by the rotation-matrix closed form instead.  Every pair kind of
  *                             PrimitivePair is covered (sphere, capsule, box, plane, cylinder; box x box included)
  *   row math (AL impulses)  : pinned bit-exact against oracle/_ref (augmented_row.hpp), the committed vectors, and
- *                             the known answers in tests/math/test_contact_tangent.cpp
+ *                             the known answers in tests/math/test_contact_tangent.cpp; the compliant-row terms and
+ *                             the elliptic cone (no device counterpart) likewise, with the hand-evaluated table of
+ *                             tests/constraint/test_solref_solimp.cpp
  *   chain Jacobian          : pinned (J qdot == contact point velocity of the float64 model)
  *   contact cache           : pinned by behaviour (seeding of a persisting contact, one-step retention and decay,
  *                             layout invariants); the merged profile terms of the material key against the
@@ -154,6 +156,13 @@ void nko_tangent_impulse(const float dual[3], float rho, const float residual[3]
 void nko_relax_contact_impulse(const float dual[3], const float next[3], float last_step[3], float* last_weight,
                                float last_point[3], float out[3]);
 float nko_cone_argument(float dual, float rho, float mu, float residual);
+/* The compliant (MuJoCo-law) row terms and the elliptic cone of the reference's row math.  No device counterpart: the
+ * product builds rows of the native law only.  Held so the reference's known answers for them are checked here too. */
+void nko_compliant_row_terms(const float solref[2], const float solimp[5], float pos_imp, float pos_aref, float vel, float invweight,
+                             float dt, int refsafe, float out[6]);
+void nko_discretize_compliant_row(float R, float aref_bias, float damping, float dt, float out[3]);
+void nko_elliptic_impulse(const float dual[3], float cap, const float residual[3], const float compliance[3], float mu_first, float out[9]);
+void nko_elliptic_multiplier_step(const float dual[3], const float next[3], float cap, const float compliance[3], float out[3]);
 double nko_momentum_restart(const float point[3], const float next[3], const float base[3], const float scale[3]);
 double nko_contact_projection_roundoff(const float start[3], const float end[3], const float axis[3]);
 float nko_contact_query_reach(float thickness, float margin);

@@ -131,6 +131,32 @@ void ref_make_contact_id(uint32_t a, uint32_t b, const float* local_a, const flo
     out[0] = id.pair; out[1] = id.feature;
 }
 
+// constraint/solref_solimp.hpp ComputeCompliantRowTerms -> k, b, imp, D, R, aref; DiscretizeCompliantRow -> R, bias, gain
+void ref_compliant_row_terms(const float* solref, const float* solimp, float pos_imp, float pos_aref, float vel, float invweight,
+                             float dt, int refsafe, float* out) {
+    const auto t = constraint::ComputeCompliantRowTerms(solref, solimp, pos_imp, pos_aref, vel, invweight, dt, refsafe != 0);
+    out[0] = t.k; out[1] = t.b; out[2] = t.imp; out[3] = t.D; out[4] = t.R; out[5] = t.aref;
+}
+void ref_discretize_row(float R, float aref_bias, float damping, float dt, float* out) {
+    constraint::CompliantContactRow row;
+    row.R = R; row.aref_bias = aref_bias; row.damping = damping;
+    const auto d = constraint::DiscretizeCompliantRow(row, dt);
+    out[0] = d.R; out[1] = d.bias; out[2] = d.reference_gain;
+}
+// nk/solve/augmented_row.hpp EvaluateEllipticImpulse -> impulse[3], curvature xx yy zz xy xz yz; EllipticMultiplierStep
+void ref_elliptic_impulse(const float* dual, float cap, const float* residual, const float* compliance, float mu_first, float* out) {
+    const auto t = nk::augmented::EvaluateEllipticImpulse({dual[0], dual[1], dual[2]}, cap, {residual[0], residual[1], residual[2]},
+                                                          {compliance[0], compliance[1], compliance[2]}, mu_first);
+    out[0] = t.impulse.x; out[1] = t.impulse.y; out[2] = t.impulse.z;
+    out[3] = t.curvature.xx; out[4] = t.curvature.yy; out[5] = t.curvature.zz;
+    out[6] = t.curvature.xy; out[7] = t.curvature.xz; out[8] = t.curvature.yz;
+}
+void ref_elliptic_multiplier_step(const float* dual, const float* next, float cap, const float* compliance, float* out) {
+    const auto d = nk::augmented::EllipticMultiplierStep({dual[0], dual[1], dual[2]}, {next[0], next[1], next[2]}, cap,
+                                                         {compliance[0], compliance[1], compliance[2]});
+    out[0] = d.x; out[1] = d.y; out[2] = d.z;
+}
+
 void ref_discretize_zero_row(float dt, float* out) {
     const auto d = constraint::DiscretizeCompliantRow(constraint::CompliantContactRow{}, dt);
     out[0] = d.R; out[1] = d.bias; out[2] = d.reference_gain;

@@ -193,6 +193,31 @@ def main():
 
     out.update(pair_cases(L, g))
 
+    # compliant-row terms and their discretisation: solref[2], solimp[5], pos_imp, pos_aref, vel, invweight, dt, refsafe
+    n = 300
+    cases, results = np.zeros((n, 13), np.float32), np.zeros((n, 9), np.float32)
+    for i in range(n):
+        cases[i] = [g.choice([0.02, 0.005, -50.0, 0.1]), g.choice([1.0, 0.5, -10.0]), g.uniform(0.5, 0.95), g.uniform(0.9, 0.999),
+                    g.choice([0.001, 0.01]), g.uniform(0.2, 0.8), g.choice([1.0, 2.0, 3.0]), -abs(g.normal(0, 0.002)), g.normal(0, 0.002),
+                    g.normal(0, 0.5), g.uniform(0.1, 5), g.choice([0.005, 0.002]), g.integers(0, 2)]
+        c = cases[i]
+        terms, discrete = (F * 6)(), (F * 3)()
+        L.ref_compliant_row_terms(farr(c[0:2]), farr(c[2:7]), F(float(c[7])), F(float(c[8])), F(float(c[9])), F(float(c[10])), F(float(c[11])), int(c[12]), terms)
+        L.ref_discretize_row(F(terms[4]), F(terms[5]), F(terms[1]), F(float(c[11])), discrete)
+        results[i] = list(terms) + list(discrete)
+    out["compliant_in"], out["compliant_out"] = cases, results
+
+    # elliptic cone: dual[3], cap, residual[3], compliance[3], mu, next[3] -> impulse[3], curvature[6], multiplier step[3]
+    cases, results = np.zeros((n, 14), np.float32), np.zeros((n, 12), np.float32)
+    for i in range(n):
+        cases[i] = list(g.normal(0, 1, 3)) + [np.exp(g.normal(0, 2))] + list(g.normal(0, 1, 3)) + list(np.exp(g.normal(-3, 2, 3))) + [g.uniform(0.1, 1.5)] + list(g.normal(0, 1, 3))
+        c = cases[i]
+        impulse, step = (F * 9)(), (F * 3)()
+        L.ref_elliptic_impulse(farr(c[0:3]), F(float(c[3])), farr(c[4:7]), farr(c[7:10]), F(float(c[10])), impulse)
+        L.ref_elliptic_multiplier_step(farr(c[0:3]), farr(c[11:14]), F(float(c[3])), farr(c[7:10]), step)
+        results[i] = list(impulse) + list(step)
+    out["elliptic_in"], out["elliptic_out"] = cases, results
+
     np.savez_compressed(os.path.join(HERE, "rowmath_vectors.npz"), **out)
     print("wrote", os.path.join(HERE, "rowmath_vectors.npz"))
 

@@ -101,6 +101,21 @@ def test_every_analytic_pair(oracle_py, vectors):
     assert len(hits) == 13 and min(hits.values()) >= 15, hits
 
 
+def test_compliant_rows_and_elliptic_cone(oracle_py, vectors):
+    """The compliant-row terms, their discretisation and the elliptic cone projection (no device counterpart)."""
+    L = oracle_py.lib()
+    for c, expect in zip(vectors["compliant_in"], vectors["compliant_out"]):
+        terms, discrete = (F * 6)(), (F * 3)()
+        L.nko_compliant_row_terms(farr(c[0:2]), farr(c[2:7]), F(float(c[7])), F(float(c[8])), F(float(c[9])), F(float(c[10])), F(float(c[11])), int(c[12]), terms)
+        L.nko_discretize_compliant_row(F(terms[4]), F(terms[5]), F(terms[1]), F(float(c[11])), discrete)
+        assert same(list(terms) + list(discrete), expect)
+    for c, expect in zip(vectors["elliptic_in"], vectors["elliptic_out"]):
+        impulse, step = (F * 9)(), (F * 3)()
+        L.nko_elliptic_impulse(farr(c[0:3]), F(float(c[3])), farr(c[4:7]), farr(c[7:10]), F(float(c[10])), impulse)
+        L.nko_elliptic_multiplier_step(farr(c[0:3]), farr(c[11:14]), F(float(c[3])), farr(c[7:10]), step)
+        assert same(list(impulse) + list(step), expect)
+
+
 def test_compose_contact_id_and_roundoff(oracle_py, vectors):
     L = oracle_py.lib()
     L.nko_contact_projection_roundoff.restype = C.c_double

@@ -227,3 +227,71 @@ def test_contact_id_matches_reference(oracle_py, ref_lib):
         L.nko_make_contact_id(a, b, la, lb, feature, slot, x)
         ref_lib.ref_make_contact_id(a, b, la, lb, n, feature, slot, y)
         assert list(x) == list(y)
+
+
+# the hand-evaluated table of tests/constraint/test_solref_solimp.cpp: solref, solimp, pos_imp, pos_aref, vel, invweight, dt,
+# then the expected k, b, imp, D, R, aref
+COMPLIANT_TABLE = [
+    ((0.02, 1.0), (0.9, 0.95, 0.001, 0.5, 2.0), -0.001, -0.001, 0.0, 1.0, 0.005, (2770.0835, 105.26316, 0.95, 18.999996, 0.05263159, 2.6315794)),
+    ((0.02, 1.0), (0.9, 0.95, 0.001, 0.5, 2.0), -0.0003, -0.0003, -0.1, 1.0, 0.005, (2770.0835, 105.26316, 0.909, 9.989008, 0.10011004, 11.281718)),
+    ((0.02, 1.0), (0.9, 0.95, 0.001, 0.5, 2.0), -0.0007, -0.0007, 0.2, 1.0, 0.005, (2770.0835, 105.26316, 0.941, 15.949148, 0.06269927, -19.22798)),
+    ((0.02, 1.0), (0.9, 0.95, 0.001, 0.5, 2.0), -0.002, -0.002, 0.5, 2.0, 0.005, (2770.0835, 105.26316, 0.95, 9.499998, 0.10526318, -47.368423)),
+    ((0.02, 1.0), (0.9, 0.95, 0.001, 0.5, 1.0), -0.0004, -0.0004, 0.0, 1.0, 0.005, (2770.0835, 105.26316, 0.92, 11.499993, 0.086956576, 1.0193907)),
+    ((-50.0, 1.0), (0.9, 0.95, 0.001, 0.5, 2.0), -0.0005, -0.0005, 0.3, 1.0, 0.005, (55.401665, 210.52632, 0.92499995, 12.333324, 0.08108114, -63.132275)),
+    ((0.02, -10.0), (0.9, 0.95, 0.001, 0.5, 2.0), -0.0005, -0.0005, 0.4, 1.0, 0.005, (27.700834, 10.526316, 0.92499995, 12.333324, 0.08108114, -4.197715)),
+    ((0.005, 1.0), (0.9, 0.95, 0.001, 0.5, 2.0), -0.0006, -0.0006, 0.0, 1.0, 0.01, (2770.0835, 105.26316, 0.934, 14.151519, 0.070663795, 1.5523549)),
+    ((0.02, 1.0), (0.9, 0.95, 0.001, 0.5, 2.0), -1.0e-7, -1.0e-7, 0.0, 1.0, 0.005, (2770.0835, 105.26316, 0.9, 8.999997, 0.11111115, 0.00024930752)),
+]
+
+
+def test_compliant_row_terms_match_the_hand_evaluated_table(oracle_py):
+    """ComputeCompliantRowTerms against the reference test's own table, with that test's tolerances; R D = 1 and a deeper
+    contact is stiffer (its DAndRNotSwapped case)."""
+    L = oracle_py.lib()
+    for solref, solimp, pos_imp, pos_aref, vel, invweight, dt, expect in COMPLIANT_TABLE:
+        out = (F * 6)()
+        L.nko_compliant_row_terms(farr(solref), farr(solimp), F(pos_imp), F(pos_aref), F(vel), F(invweight), F(dt), 1, out)
+        k, b, imp, D, R, aref = list(out)
+        assert abs(k - expect[0]) <= 1e-3 * (1 + abs(expect[0])) and abs(b - expect[1]) <= 1e-3 * (1 + abs(expect[1]))
+        assert abs(imp - expect[2]) <= 1e-5 and abs(D - expect[3]) <= 1e-3 * (1 + abs(expect[3])) and abs(R - expect[4]) <= 1e-5
+        assert abs(aref - expect[5]) <= 1e-3 * (1 + abs(expect[5]))
+    shallow, deep = (F * 6)(), (F * 6)()
+    default = (farr((0.02, 1.0)), farr((0.9, 0.95, 0.001, 0.5, 2.0)))
+    L.nko_compliant_row_terms(*default, F(-0.0002), F(-0.0002), F(0.0), F(1.0), F(0.005), 1, shallow)
+    L.nko_compliant_row_terms(*default, F(-0.0009), F(-0.0009), F(0.0), F(1.0), F(0.005), 1, deep)
+    assert abs(shallow[3] * shallow[4] - 1) < 1e-4 and abs(deep[3] * deep[4] - 1) < 1e-4
+    assert deep[2] > shallow[2] and deep[4] < shallow[4] and deep[3] > shallow[3]
+
+
+def test_compliant_rows_and_elliptic_cone_match_reference_bitwise(oracle_py, ref_lib):
+    L, g = oracle_py.lib(), np.random.default_rng(12)
+    for _ in range(1500):
+        solref = (float(g.choice([0.02, 0.005, -50.0, 0.1])), float(g.choice([1.0, 0.5, -10.0])))
+        solimp = (g.uniform(0.5, 0.95), g.uniform(0.9, 0.999), float(g.choice([0.001, 0.01])), g.uniform(0.2, 0.8), float(g.choice([1.0, 2.0, 3.0])))
+        args = (farr(solref), farr(solimp), F(-abs(g.normal(0, 0.002))), F(g.normal(0, 0.002)), F(g.normal(0, 0.5)), F(g.uniform(0.1, 5)),
+                F(float(g.choice([0.005, 0.002]))), int(g.integers(0, 2)))
+        a, b = (F * 6)(), (F * 6)()
+        L.nko_compliant_row_terms(*args, a)
+        ref_lib.ref_compliant_row_terms(*args, b)
+        assert list(a) == list(b)
+        c, d = (F * 3)(), (F * 3)()
+        L.nko_discretize_compliant_row(F(a[4]), F(a[5]), F(a[1]), args[6], c)
+        ref_lib.ref_discretize_row(F(a[4]), F(a[5]), F(a[1]), args[6], d)
+        assert list(c) == list(d)
+    inside = projected = polar = 0
+    for _ in range(3000):
+        dual, residual = farr(g.normal(0, 1, 3)), farr(g.normal(0, 1, 3))
+        cap, mu = F(float(np.exp(g.normal(0, 2)))), F(g.uniform(0.1, 1.5))
+        compliance = farr(np.exp(g.normal(-3, 2, 3)))
+        a, b = (F * 9)(), (F * 9)()
+        L.nko_elliptic_impulse(dual, cap, residual, compliance, mu, a)
+        ref_lib.ref_elliptic_impulse(dual, cap, residual, compliance, mu, b)
+        assert list(a) == list(b)
+        inside += a[6] == 0 and a[3] != 0
+        polar += not any(a)
+        projected += a[6] != 0 or a[7] != 0
+        nxt, c, d = farr(g.normal(0, 1, 3)), (F * 3)(), (F * 3)()
+        L.nko_elliptic_multiplier_step(dual, nxt, cap, compliance, c)
+        ref_lib.ref_elliptic_multiplier_step(dual, nxt, cap, compliance, d)
+        assert list(c) == list(d)
+    assert inside > 300 and projected > 300 and polar > 100
