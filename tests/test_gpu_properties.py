@@ -87,6 +87,37 @@ def test_full_size_batches_step_cleanly(device, index, E):
     world.close()
 
 
+def test_scene_files_at_full_batch_size(device):
+    """The capsule walker (links meeting links and the floor) and the URDF walker at 4096 environments, a hundred
+    steps from the authored pose with per-environment pushes: no status bit, finite state, unit quaternions, the
+    identical environments 0 and 1 stay identical, and the robots end up carried by contacts rather than falling."""
+    import os
+    from conftest import ROOT
+    E = 4096
+    for path, flags in ((os.path.join(ROOT, "tests", "data", "capsule_walker.xml"), 0),
+                        (os.path.join(ROOT, "tests", "data", "legged.urdf"), nk.SCENE_GROUND_PLANE | nk.SCENE_PLANE_CONTACTS_ONLY)):
+        scene = nk.Scene(path, flags)
+        world = nk.World(device, scene, abi.world_desc(E, 0.0 if path.endswith(".xml") else 1.0 / 240.0, vel_iters=8))
+        nl = scene.link_count
+        rng = np.random.default_rng(5)
+        twist = np.zeros((E, nl, 6), np.float32)
+        twist[2:, 0] = rng.normal(0, 0.2, (E - 2, 6))
+        base = world.download("base_pose").reshape(E, 7).copy()
+        base[:, 2] = 0.545 if path.endswith(".xml") else 0.488          # soles on the floor
+        world.upload("base_pose", base)
+        world.upload("link_velocity", twist)
+        world.step(100)
+        world.synchronize()
+        assert not world.download("env_status").any()
+        for name in ("q", "qdot", "link_pose", "lambda"):
+            assert np.all(np.isfinite(world.download(name))), name
+        pose = world.download("link_pose").reshape(E, nl, 7)
+        assert np.abs(np.linalg.norm(pose[:, :, 3:], axis=2) - 1).max() < 1e-5
+        assert np.array_equal(pose[0], pose[1])
+        assert (world.download("contact_count") >= 1).mean() > 0.9 and np.median(pose[:, 0, 2]) > 0.15
+        world.close()
+
+
 def test_rope_full_batch_steps(device):
     E = 1024
     cfg, world = stepped(device, 5, E)
