@@ -6,12 +6,12 @@
 // Not read: meshes, height fields, materials, cameras, lights, sensors, sites, equalities, <contact> pairs, ball
 // joints (rejected), tendons.  The joint and contact laws are this library's native ones: the
 // solref / solimp compliant rows the reference attaches to MJCF joints and geoms are not built.
-#include "mjcf_loader.h"
+#include "scene_loader.h"
 
 #include "scene_build.h"
 
 namespace nkh {
-namespace mjcf {
+namespace scene_file {
 namespace {
 
 // ---- default classes (mjcf_importer.cpp:104-190, 309-430, 522-556) --------------------------------------------
@@ -700,5 +700,5 @@ void Scene::Bind() {
     desc.excluded_pair_count = uint32_t(excluded_pairs.size() / 2u);
 }
 
-}  // namespace mjcf
+}  // namespace scene_file
 }  // namespace nkh

@@ -16,10 +16,10 @@
 #include <utility>
 #include <vector>
 
-#include "mjcf_loader.h"
+#include "scene_loader.h"
 
 namespace nkh {
-namespace mjcf {
+namespace scene_file {
 
 // ---- a small XML reader: elements, attributes, comments, declarations ---------------------------------------
 struct Element {
@@ -332,5 +332,5 @@ struct SceneParts {
 // policy, and binds its descriptor.
 void FlattenScene(const SceneParts& parts, uint32_t flags, uint32_t drive_mode, Scene* scene);
 
-}  // namespace mjcf
+}  // namespace scene_file
 }  // namespace nkh

@@ -11,7 +11,7 @@
 #include "../../include/nuka_hip.h"
 
 namespace nkh {
-namespace mjcf {
+namespace scene_file {
 
 // Keep sphere and box geoms against planes only: other colliding geoms are dropped (and counted), and the robot's
 // geoms share one negative collision group so that they meet the ground and not each other.
@@ -42,5 +42,5 @@ struct Scene {
 std::unique_ptr<Scene> LoadMjcf(const std::string& path, uint32_t flags);
 std::unique_ptr<Scene> LoadUrdf(const std::string& path, uint32_t flags);
 
-}  // namespace mjcf
+}  // namespace scene_file
 }  // namespace nkh

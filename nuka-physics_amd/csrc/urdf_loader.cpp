@@ -5,12 +5,12 @@
 //
 // Not read: visuals and materials, meshes (a mesh collision is a shape this library has no manifold for), mimic,
 // planar and floating joints (rejected), transmissions, gazebo extensions.
-#include "mjcf_loader.h"
+#include "scene_loader.h"
 
 #include "scene_build.h"
 
 namespace nkh {
-namespace mjcf {
+namespace scene_file {
 namespace {
 
 // urdf_importer.cpp:45-56 ParseOrigin: xyz, and fixed-axis roll-pitch-yaw composed as Rz(yaw) Ry(pitch) Rx(roll)
@@ -184,5 +184,5 @@ std::unique_ptr<Scene> LoadUrdf(const std::string& path, uint32_t flags) {
     return scene;
 }
 
-}  // namespace mjcf
+}  // namespace scene_file
 }  // namespace nkh

@@ -17,7 +17,7 @@
 
 #include "../../include/nuka_hip.h"
 #include "backend.h"
-#include "mjcf_loader.h"
+#include "scene_loader.h"
 #include "nk_types.h"
 
 namespace nkh {
@@ -627,7 +627,7 @@ nuka_phi_backend* nuka_device_backend(nuka_device_handle device) {
 namespace nkh {
 namespace {
 nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t* tmpl, const nuka_world_desc_t* desc,
-                          const mjcf::Scene* scene, nuka_world_handle* out) {
+                          const scene_file::Scene* scene, nuka_world_handle* out) {
     if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
     *out = nullptr;
     if (device == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "device is null");
@@ -760,7 +760,7 @@ nuka_result_t nuka_scene_load_mjcf(const char* path, uint32_t flags, nuka_scene_
     if (path == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "path is null");
     if ((flags & ~uint32_t(NUKA_SCENE_PLANE_CONTACTS_ONLY | NUKA_SCENE_GROUND_PLANE)) != 0u) return Error(NUKA_RESULT_INVALID_ARG, "unknown scene flag");
     try {
-        *out = reinterpret_cast<nuka_scene_handle>(mjcf::LoadMjcf(path, flags).release());
+        *out = reinterpret_cast<nuka_scene_handle>(scene_file::LoadMjcf(path, flags).release());
         return NUKA_RESULT_OK;
     } catch (const std::bad_alloc&) {
         return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
@@ -775,7 +775,7 @@ nuka_result_t nuka_scene_load_urdf(const char* path, uint32_t flags, nuka_scene_
     if (path == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "path is null");
     if ((flags & ~uint32_t(NUKA_SCENE_PLANE_CONTACTS_ONLY | NUKA_SCENE_FIXED_BASE | NUKA_SCENE_GROUND_PLANE)) != 0u) return Error(NUKA_RESULT_INVALID_ARG, "unknown scene flag");
     try {
-        *out = reinterpret_cast<nuka_scene_handle>(mjcf::LoadUrdf(path, flags).release());
+        *out = reinterpret_cast<nuka_scene_handle>(scene_file::LoadUrdf(path, flags).release());
         return NUKA_RESULT_OK;
     } catch (const std::bad_alloc&) {
         return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
@@ -784,14 +784,14 @@ nuka_result_t nuka_scene_load_urdf(const char* path, uint32_t flags, nuka_scene_
     }
 }
 
-void nuka_scene_destroy(nuka_scene_handle scene) { delete reinterpret_cast<mjcf::Scene*>(scene); }
+void nuka_scene_destroy(nuka_scene_handle scene) { delete reinterpret_cast<scene_file::Scene*>(scene); }
 
 const nuka_template_desc_t* nuka_scene_template(nuka_scene_handle scene) {
-    return scene != nullptr ? &reinterpret_cast<mjcf::Scene*>(scene)->desc : nullptr;
+    return scene != nullptr ? &reinterpret_cast<scene_file::Scene*>(scene)->desc : nullptr;
 }
 
 nuka_result_t nuka_scene_get_info(nuka_scene_handle scene, nuka_scene_info_t* out) {
-    const auto* s = reinterpret_cast<const mjcf::Scene*>(scene);
+    const auto* s = reinterpret_cast<const scene_file::Scene*>(scene);
     if (s == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "scene is null");
     if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
     *out = {s->desc.link_count, s->desc.body_count, s->actuator_count, s->dropped_geom_count, s->floating_root ? 1u : 0u, s->drive_mode,
@@ -800,18 +800,18 @@ nuka_result_t nuka_scene_get_info(nuka_scene_handle scene, nuka_scene_info_t* ou
 }
 
 const char* nuka_scene_link_name(nuka_scene_handle scene, uint32_t link) {
-    const auto* s = reinterpret_cast<const mjcf::Scene*>(scene);
+    const auto* s = reinterpret_cast<const scene_file::Scene*>(scene);
     return s != nullptr && link < s->link_names.size() ? s->link_names[link].c_str() : nullptr;
 }
 
 const char* nuka_scene_joint_name(nuka_scene_handle scene, uint32_t link) {
-    const auto* s = reinterpret_cast<const mjcf::Scene*>(scene);
+    const auto* s = reinterpret_cast<const scene_file::Scene*>(scene);
     return s != nullptr && link < s->joint_names.size() ? s->joint_names[link].c_str() : nullptr;
 }
 
 nuka_result_t nuka_scene_initial_state(nuka_scene_handle scene, float* q, float* base_pose, float* drive_stiffness, float* drive_damping,
                                        float* drive_force_limit, float* drive_joint_force_limit) {
-    const auto* s = reinterpret_cast<const mjcf::Scene*>(scene);
+    const auto* s = reinterpret_cast<const scene_file::Scene*>(scene);
     if (s == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "scene is null");
     auto copy = [](float* out, const std::vector<float>& values) { if (out != nullptr) std::copy(values.begin(), values.end(), out); };
     copy(q, s->initial_q);
@@ -825,7 +825,7 @@ nuka_result_t nuka_scene_initial_state(nuka_scene_handle scene, float* q, float*
 
 nuka_result_t nuka_world_create_from_scene(nuka_device_handle device, nuka_scene_handle scene, const nuka_world_desc_t* desc,
                                            nuka_world_handle* out) {
-    const auto* s = reinterpret_cast<const mjcf::Scene*>(scene);
+    const auto* s = reinterpret_cast<const scene_file::Scene*>(scene);
     if (s == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "scene is null");
     if (desc == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "desc is null");
     if (desc->struct_size != sizeof(nuka_world_desc_t)) return Error(NUKA_RESULT_INVALID_ARG, "struct_size mismatch");
