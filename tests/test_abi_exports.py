@@ -31,6 +31,28 @@ def test_struct_layouts_match_the_header():
     assert C.sizeof(nk.abi.WorldDescC) == 15 * 4
 
 
+def test_headers_compile_as_c_and_agree_with_the_ctypes_mirror(tmp_path):
+    """include/*.h are plain C: a C99 program that includes them reports the size of each descriptor and the offset of
+    every member the ctypes mirror declares, and the two layouts agree."""
+    import subprocess
+    members = {"nuka_template_desc_t": nk.abi.TemplateDescC, "nuka_world_desc_t": nk.abi.WorldDescC, "nuka_scene_info_t": nk.SceneInfoC}
+    lines = ['#include <stddef.h>', '#include <stdio.h>', '#include "nuka_phi.h"', '#include "nuka_hip.h"', 'int main(void) {']
+    for name, mirror in members.items():
+        lines.append(f'    printf("{name} %zu\\n", sizeof({name}));')
+        for field, _ in mirror._fields_:
+            lines.append(f'    printf("{name}.{field} %zu\\n", offsetof({name}, {field}));')
+    lines += ['    return 0;', '}']
+    source = tmp_path / "layout.c"
+    source.write_text("\n".join(lines) + "\n")
+    binary = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"), str(source), "-o", str(binary)], check=True)
+    reported = dict(line.split() for line in subprocess.run([str(binary)], check=True, capture_output=True, text=True).stdout.splitlines())
+    for name, mirror in members.items():
+        assert int(reported[name]) == C.sizeof(mirror), name
+        for field, _ in mirror._fields_:
+            assert int(reported[f"{name}.{field}"]) == getattr(mirror, field).offset, f"{name}.{field}"
+
+
 def test_op_catalog_names_round_trip():
     lib = nk.lib()
     count = lib.nuka_hip_op_count()
