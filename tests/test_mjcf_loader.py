@@ -239,6 +239,26 @@ def test_capsule_walker_links_meet_each_other_but_not_their_parents(oracle_py, t
     w.close()
 
 
+def test_inertia_and_friction_fixture_of_the_reference():
+    """tests/data/inertia_friction.xml with the expectations of tests/import/test_inertia_friction.cpp: a full inertia
+    tensor comes back from its principal moments and axes, the centre of mass is kept, frictionloss / damping /
+    armature inherit from the class and an element's own attribute wins."""
+    scene = nk.Scene(os.path.join(GOLDEN, "inertia_friction.xml"))
+    a = scene.template_arrays()
+    link1, link2 = scene.link_names.index("link1"), scene.link_names.index("link2")
+    frame, principal = a["link_inertial_frame"].reshape(-1, 7)[link1], a["link_diag_inertia"].reshape(-1, 3)[link1]
+    R = np.stack([rotate(frame[3:], e) for e in np.eye(3)], 1)
+    full = R @ np.diag(principal) @ R.T
+    assert np.allclose(full, [[2, 0.5, 0.3], [0.5, 3, 0.2], [0.3, 0.2, 4]], atol=1e-4)
+    assert np.abs(R - np.eye(3)).max() > 1e-3 and abs(frame[2] - 0.1) < 1e-6            # rotated principal axes, the authored z of the centre
+    assert a["link_mass"][link1] == 1.5
+    assert np.isclose(a["joint_frictionloss"][link1], 0.075) and np.isclose(a["joint_damping"][link1], 0.3) and np.isclose(a["joint_armature"][link1], 0.01)
+    assert np.isclose(a["joint_frictionloss"][link2], 0.02) and np.isclose(a["joint_damping"][link2], 0.3)
+    kinds = [int(k) for k in a["shape_kind"] if k != abi.INVALID]
+    assert kinds == [abi.SHAPE_BOX, abi.SHAPE_CAPSULE, abi.SHAPE_CAPSULE]
+    assert np.allclose(a["shape_params"].reshape(-1, 4)[1, :2], [0.02, 0.05])
+
+
 def test_contact_filtering_fixture_of_the_reference():
     """tests/data/contact_filtering.xml with the expectations of tests/import/test_mjcf_contact_filtering.cpp that bear
     on pairing: explicit and class-inherited contype / conaffinity / group, the geom that collides with nothing, the
