@@ -144,8 +144,11 @@ __global__ void __launch_bounds__(kWave) FkWorldPosesKernel(ModelView m, DataVie
 }
 
 // ---- ArticulationDynamics -------------------------------------------------------------------------------
+// The link accelerations and bias forces are dead while the composite inertias live (mass-matrix assembly) and the
+// other way round, so the two share their words: less LDS a block, more blocks a compute unit for a kernel that
+// waits on tree sweeps.
 __host__ __device__ inline uint32_t DynamicsLdsFloats(uint32_t nl, uint32_t n) {
-    return nl * (36u + 36u + 5u * 6u) + n * (n + 1u) + 2u * n + 64u;
+    return nl * (36u + 36u + 3u * 6u) + n * (n + 1u) + 2u * n + 64u;
 }
 
 // Compiled per padded DoF width N (a multiple of 4): the LDL^T factorisation and the solve keep one matrix row per
@@ -157,13 +160,13 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
     const uint32_t env = blockIdx.x, lane = threadIdx.x, nl = m.links_per_env, n = m.dof, stride = m.max_dof;
     if (env >= env_count) return;
     float* xup = lds;
-    float* ic = xup + nl * 36u;
-    float* S = ic + nl * 36u;
+    float* S = xup + nl * 36u;
     float* vb = S + nl * 6u;
     float* v = vb + nl * 6u;
-    float* a = v + nl * 6u;
-    float* pf = a + nl * 6u;
-    float* A = pf + nl * 6u;          // n x (n + 1): mass matrix, then its factor
+    float* ic = v + nl * 6u;          // composite inertias, from the mass-matrix assembly until its columns are done
+    float* a = ic;                    // link accelerations: bias pass, and again the final pass
+    float* pf = a + nl * 6u;          // bias forces: until the generalized bias is taken
+    float* A = ic + nl * 36u;         // n x (n + 1): mass matrix, then its factor
     float* vel = A + n * (n + 1u);
     float* acc = vel + n;
     float* tmp = acc + n;             // 36 floats of the inertia push, padded to 64
@@ -297,6 +300,7 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
             acc[lane] = (scalar ? d.tau[lbase + link] : 0.0f) - b - damping * velocity - spring;
         }
     }
+    __syncthreads();   // the bias forces have been read: their words now take the composite inertias
     // CRBA: composite inertias leaf to root; the push X^T Ic X runs entry-parallel on 36 lanes (articulation_mass.cuh:146-165)
     for (uint32_t e = lane; e < nl * 36u; e += kWave) ic[e] = m.link_inertia[e];
     for (uint32_t e = lane; e < n * ld; e += kWave) A[e] = 0.0f;
