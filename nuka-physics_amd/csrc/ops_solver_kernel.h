@@ -288,19 +288,22 @@ __device__ __forceinline__ bool factor_rows(uint32_t lane, float (&row)[N], floa
 // SolveTileBlock (:1647-1666): forward with the factor's rows, backward with its columns (col[j] = L_j,lane).
 template <int N>
 __device__ __forceinline__ float substitute(uint32_t lane, const float (&row)[N], const float (&col)[N], float inverse, float g) {
+    // Lane j's entry is final once the steps before it have run, so it is scaled by its reciprocal pivot where it is
+    // read (the same product that would be stored back) and the lanes take it in one multiplication after the sweep.
     lane = local_lane(lane);
     float r = g;
 #pragma unroll
     for (int j = 0; j < N; ++j) {
         const float y = lane_value(r * inverse, j);
-        r = lane == uint32_t(j) ? y : (lane > uint32_t(j) ? fmaf(-row[j], y, r) : r);
+        r = lane > uint32_t(j) ? fmaf(-row[j], y, r) : r;
     }
+    r *= inverse;
 #pragma unroll
     for (int j = N - 1; j >= 0; --j) {
         const float x = lane_value(r * inverse, j);
-        r = lane == uint32_t(j) ? x : (lane < uint32_t(j) ? fmaf(-col[j], x, r) : r);
+        r = lane < uint32_t(j) ? fmaf(-col[j], x, r) : r;
     }
-    return r;
+    return r * inverse;
 }
 
 template <int N>
