@@ -191,6 +191,6 @@ def rope(env_count=8192):
 
 
 def config(index, env_count=None):
-    """BASELINE configuration by number 1..5; 4 is the humanoid at a swept environment count."""
+    """Benchmark configuration by number 1..5; 4 is the humanoid at a swept environment count."""
     makers = {1: chain7, 2: quadruped, 3: humanoid, 4: lambda e=4096: humanoid(e, 4), 5: rope}
     return makers[index]() if env_count is None else makers[index](env_count)
