@@ -185,6 +185,49 @@ nuka_result_t nuka_world_checkpoint_capture(nuka_world_handle world, nuka_checkp
 nuka_result_t nuka_world_checkpoint_restore(nuka_world_handle world, nuka_checkpoint_handle checkpoint);
 void nuka_checkpoint_destroy(nuka_checkpoint_handle checkpoint);
 nuka_result_t nuka_checkpoint_byte_size(nuka_checkpoint_handle checkpoint, uint64_t* out_bytes);
+/* nuka.h:401-402: 1 when both checkpoints were taken of worlds of one layout and hold the same persistent bytes, else 0 */
+nuka_result_t nuka_checkpoint_equal(nuka_checkpoint_handle a, nuka_checkpoint_handle b, uint32_t* out_equal);
+/* nuka.h:403-404, src/c_abi/checkpoint.cpp:601-636: 64-bit FNV-1a over a domain string, the byte count and the
+ * persistent physics bytes in field order.  Waits for the device.  Two runs of one build from the same inputs hash
+ * alike; the value is not comparable with the reference's, whose persistent arena holds other fields. */
+nuka_result_t nuka_world_state_hash(nuka_world_handle world, uint64_t* out_hash);
+
+/* nuka.h:433-434, nk::World::RefreshPoses (src/nk/pipeline/world.cpp:778-793): link and body poses from the joint
+ * coordinates and base poses, without advancing time. */
+nuka_result_t nuka_world_forward_kinematics(nuka_world_handle world);
+
+/* The tunable parameters of a world (nuka.h:281-285, 304-341; src/c_abi/params.cpp): world options and values of one
+ * template link that hold in every environment.  Indices, keys, units and ranges are the reference's:
+ *   0 gravity_z            1 velocity_iterations   2 link_mass        3 joint_damping
+ *   4 joint_armature       5 joint_frictionloss    6 drive_stiffness  7 drive_force_limit
+ * Parameters 0 and 1 have one element, the others one per template link.  A LIVE value applies at the next step and
+ * survives nuka_world_reset.  link_mass keeps the link's centre of mass and its rotational inertia about it;
+ * drive_stiffness also sets the drive's damping to 2 sqrt(stiffness), as the cook derives it.  joint_frictionloss is
+ * REBUILD (set returns NOT_SUPPORTED) in a world cooked without joint friction rows.  NOT_SUPPORTED also for a joint
+ * parameter of a link whose joint has no scalar coordinate (the root, a fixed joint) and for a drive parameter in a
+ * world without drive rows. */
+typedef enum nuka_param_type_t { NUKA_PARAM_F32 = 0, NUKA_PARAM_U32 = 1 } nuka_param_type_t;
+typedef enum nuka_param_tier_t { NUKA_PARAM_LIVE = 0, NUKA_PARAM_REBUILD = 1 } nuka_param_tier_t;
+enum { NUKA_PARAM_INFO_VERSION = 1 };
+typedef struct nuka_param_info_t {
+    uint32_t struct_size;
+    uint32_t schema_version;
+    char key[48];
+    char unit[16];
+    char scene_field[48];
+    nuka_param_type_t type;
+    nuka_param_tier_t tier;
+    uint32_t count;
+    double min_value;
+    double max_value;
+} nuka_param_info_t;
+nuka_result_t nuka_world_param_count(nuka_world_handle world, uint32_t* out_count);
+/* every entry carries struct_size and schema_version on entry; capacity covers the count */
+nuka_result_t nuka_world_get_param_infos(nuka_world_handle world, nuka_param_info_t* infos, uint32_t capacity);
+nuka_result_t nuka_world_get_param(nuka_world_handle world, uint32_t param, uint32_t element, double* out_value);
+nuka_result_t nuka_world_set_param(nuka_world_handle world, uint32_t param, uint32_t element, double value);
+nuka_result_t nuka_world_set_link_mass(nuka_world_handle world, uint32_t link_index, float mass);   /* nuka.h:282 */
+nuka_result_t nuka_world_set_gravity_z(nuka_world_handle world, float gravity_z);                   /* nuka.h:285 */
 
 /* nk::World::DispatchOp (src/nk/pipeline/world.hpp): one op of the pipeline with the pipeline's own parameters.
  * `variant` 1 on ArticulationDynamics dispatches it with integrate_velocity = 0, the probe

@@ -40,6 +40,19 @@ SCENE_FIXED_BASE = 2
 SCENE_GROUND_PLANE = 4
 
 
+class ParamInfoC(C.Structure):
+    """nuka_param_info_t"""
+    _fields_ = [("struct_size", C.c_uint32), ("schema_version", C.c_uint32), ("key", C.c_char * 48), ("unit", C.c_char * 16),
+                ("scene_field", C.c_char * 48), ("type", C.c_int), ("tier", C.c_int), ("count", C.c_uint32),
+                ("min_value", C.c_double), ("max_value", C.c_double)]
+
+
+PARAM_INFO_VERSION = 1
+PARAM_LIVE, PARAM_REBUILD = 0, 1
+PARAMS = ("gravity_z", "velocity_iterations", "link_mass", "joint_damping", "joint_armature", "joint_frictionloss", "drive_stiffness",
+          "drive_force_limit")
+
+
 class DeviceDescC(C.Structure):
     _fields_ = [("gpu_index", C.c_uint32), ("stream", C.c_void_p), ("backend_selection_layer_enabled", C.c_uint8)]
 
@@ -55,6 +68,8 @@ EXPORTS = [
     "nuka_hip_op_count", "nuka_hip_op_name", "nuka_hip_op_from_name",
     "nuka_scene_load_mjcf", "nuka_scene_load_urdf", "nuka_scene_destroy", "nuka_scene_template", "nuka_scene_get_info", "nuka_scene_link_name",
     "nuka_scene_joint_name", "nuka_scene_initial_state", "nuka_world_create_from_scene",
+    "nuka_checkpoint_equal", "nuka_world_state_hash", "nuka_world_forward_kinematics", "nuka_world_param_count", "nuka_world_get_param_infos",
+    "nuka_world_get_param", "nuka_world_set_param", "nuka_world_set_link_mass", "nuka_world_set_gravity_z",
 ]
 
 
@@ -121,6 +136,15 @@ def lib():
         L.nuka_scene_joint_name.restype = C.c_char_p
         L.nuka_scene_initial_state.argtypes = [C.c_void_p] + [C.c_void_p] * 6
         L.nuka_world_create_from_scene.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]
+        L.nuka_checkpoint_equal.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_uint32)]
+        L.nuka_world_state_hash.argtypes = [C.c_void_p, C.POINTER(C.c_uint64)]
+        L.nuka_world_forward_kinematics.argtypes = [C.c_void_p]
+        L.nuka_world_param_count.argtypes = [C.c_void_p, C.POINTER(C.c_uint32)]
+        L.nuka_world_get_param_infos.argtypes = [C.c_void_p, C.POINTER(ParamInfoC), C.c_uint32]
+        L.nuka_world_get_param.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(C.c_double)]
+        L.nuka_world_set_param.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.c_double]
+        L.nuka_world_set_link_mass.argtypes = [C.c_void_p, C.c_uint32, C.c_float]
+        L.nuka_world_set_gravity_z.argtypes = [C.c_void_p, C.c_float]
         _lib = L
     return _lib
 
@@ -293,6 +317,46 @@ class World:
 
     def set_velocity_iterations(self, n):
         _check(lib().nuka_world_set_velocity_iterations(self._h, n))
+
+    def forward_kinematics(self):
+        """nuka_world_forward_kinematics: link and body poses from the joint coordinates, no time advanced."""
+        _check(lib().nuka_world_forward_kinematics(self._h))
+
+    def state_hash(self):
+        out = C.c_uint64()
+        _check(lib().nuka_world_state_hash(self._h, C.byref(out)))
+        return out.value
+
+    def checkpoints_equal(self, a, b):
+        out = C.c_uint32()
+        _check(lib().nuka_checkpoint_equal(a, b, C.byref(out)))
+        return bool(out.value)
+
+    def param_infos(self):
+        """nuka_world_get_param_infos as a list of dicts, in parameter order."""
+        count = C.c_uint32()
+        _check(lib().nuka_world_param_count(self._h, C.byref(count)))
+        infos = (ParamInfoC * count.value)()
+        for info in infos:
+            info.struct_size, info.schema_version = C.sizeof(ParamInfoC), PARAM_INFO_VERSION
+        _check(lib().nuka_world_get_param_infos(self._h, infos, count.value))
+        return [{"key": i.key.decode(), "unit": i.unit.decode(), "scene_field": i.scene_field.decode(), "type": i.type, "tier": i.tier,
+                 "count": i.count, "min": i.min_value, "max": i.max_value} for i in infos]
+
+    def get_param(self, key, element=0):
+        out = C.c_double()
+        _check(lib().nuka_world_get_param(self._h, PARAMS.index(key), element, C.byref(out)))
+        return out.value
+
+    def set_param(self, key, element, value):
+        """nuka_world_set_param: a world option or one template link's value, in every environment, from the next step on."""
+        _check(lib().nuka_world_set_param(self._h, PARAMS.index(key), element, float(value)))
+
+    def set_link_mass(self, link, mass):
+        _check(lib().nuka_world_set_link_mass(self._h, link, mass))
+
+    def set_gravity_z(self, gravity_z):
+        _check(lib().nuka_world_set_gravity_z(self._h, gravity_z))
 
     def time_steps(self, n, checkpoint=None):
         """Milliseconds of n steps by device events on the world's stream; with a checkpoint every step starts from it."""

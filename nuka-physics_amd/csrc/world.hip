@@ -65,6 +65,7 @@ struct HostModel {
     std::vector<uint64_t> link_dof_mask, excluded_pairs;
     std::vector<float> joint_axis, parent_offset, link_local_pose, link_inertial_frame, link_inertia, joint_damping, joint_armature,
         joint_stiffness, joint_spring_reference, joint_limit_lower, joint_limit_upper, joint_frictionloss, link_geom_local, shape_table, body_collidable_local, body_init_pose, profile_mu;
+    std::vector<float> link_mass, link_diag_inertia;   // kept for nuka_world_set_param: a new mass rebuilds the spatial inertia
 };
 
 struct NotSupported : std::runtime_error { using std::runtime_error::runtime_error; };
@@ -98,6 +99,8 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
     m.joint_frictionloss = CopyOrZero(d.joint_frictionloss, nl);
     m.joint_limit_flags = d.joint_limit_flags != nullptr ? std::vector<uint8_t>(d.joint_limit_flags, d.joint_limit_flags + nl) : std::vector<uint8_t>(nl, 0u);
     m.link_inertia.resize(36u * nl);
+    m.link_mass.assign(d.link_mass, d.link_mass + nl);
+    m.link_diag_inertia.assign(d.link_diag_inertia, d.link_diag_inertia + 3u * nl);
     m.link_dof.resize(nl);
     m.link_body.assign(nl, kInvalid);
     m.link_geom_kind.assign(nl, 0u);
@@ -340,6 +343,7 @@ struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
     SnapshotParams p_snapshot{};
     nuka_execution_mode_t mode = NUKA_EXECUTION_EAGER;
     nuka_phi_plan* plan = nullptr;
+    std::vector<float> drive_stiffness, drive_force_limit;   // per template link: what nuka_world_get_param reports
 
     ~World() {
         if (be != nullptr && plan != nullptr) be->plan_free(backend, plan);
@@ -713,6 +717,9 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
                 !put(w.data.row_cj_link_b, invalid.data(), invalid.size() * 4u) || !put(w.data.row_unit, invalid.data(), invalid.size() * 4u))
                 return Error(NUKA_RESULT_DEVICE_ERROR, "initial state upload failed");
         }
+        w.drive_stiffness.assign(nl, 0.0f);
+        w.drive_force_limit.assign(nl, 0.0f);
+        if (scene != nullptr) { w.drive_stiffness = scene->drive_stiffness; w.drive_force_limit = scene->drive_force_limit; }
         if (scene != nullptr) {   // the state and drive parameters the scene file authors, in every environment
             auto tile = [&](const std::vector<float>& per_link) {
                 std::vector<float> all(E * nl);
@@ -1186,6 +1193,244 @@ nuka_result_t nuka_checkpoint_byte_size(nuka_checkpoint_handle checkpoint, uint6
     if (out_bytes == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
     *out_bytes = cp->bytes;
     return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_checkpoint_equal(nuka_checkpoint_handle a, nuka_checkpoint_handle b, uint32_t* out_equal) {
+    auto* x = reinterpret_cast<Checkpoint*>(a);
+    auto* y = reinterpret_cast<Checkpoint*>(b);
+    if (x == nullptr || y == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "checkpoint is null");
+    if (out_equal == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    *out_equal = 0u;
+    bool same_layout = x->bytes == y->bytes && x->segments.count == y->segments.count;
+    for (uint32_t s = 0u; same_layout && s < x->segments.count; ++s)
+        same_layout = x->segments.units[s] == y->segments.units[s] && (x->segments.kept[s] == nullptr) == (y->segments.kept[s] == nullptr);
+    if (!same_layout) return NUKA_RESULT_OK;
+    try {
+        std::vector<uint8_t> left(x->bytes), right(y->bytes);
+        if (x->bytes > 0u && (Iface(x->store)->download(x->store, left.data(), 0u, x->bytes) != uint8_t(Status::Ok) ||
+                              Iface(y->store)->download(y->store, right.data(), 0u, y->bytes) != uint8_t(Status::Ok)))
+            return Error(NUKA_RESULT_DEVICE_ERROR, "checkpoint download failed");
+        *out_equal = left == right ? 1u : 0u;
+    } catch (const std::bad_alloc&) {
+        return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
+    }
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_state_hash(nuka_world_handle world, uint64_t* out_hash) {
+    if (out_hash == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    *out_hash = 0u;
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (nuka_world_synchronize(world) != NUKA_RESULT_OK) return NUKA_RESULT_DEVICE_ERROR;
+    uint64_t hash = 14695981039346656037ull;   // FNV-1a (src/c_abi/checkpoint.cpp:47-57)
+    auto mix = [&hash](const void* bytes, size_t count) {
+        const auto* p = static_cast<const uint8_t*>(bytes);
+        for (size_t i = 0u; i < count; ++i) { hash ^= p[i]; hash *= 1099511628211ull; }
+    };
+    constexpr char domain[] = "NukaHipStateHashV1";
+    mix(domain, sizeof(domain));
+    uint64_t byte_count = 0u;
+    for (const Field& f : w->fields) if (!f.is_template && CheckpointKeeps(f.name)) byte_count += f.count * f.elem_bytes;
+    mix(&byte_count, sizeof(byte_count));
+    try {
+        std::vector<uint8_t> bytes;
+        for (const Field& f : w->fields) {
+            if (f.is_template || f.count == 0u || !CheckpointKeeps(f.name)) continue;
+            bytes.resize(f.count * f.elem_bytes);
+            if (Iface(w->arena)->download(w->arena, bytes.data(), f.offset, bytes.size()) != uint8_t(Status::Ok))
+                return Error(NUKA_RESULT_DEVICE_ERROR, "state download failed");
+            mix(bytes.data(), bytes.size());
+        }
+    } catch (const std::bad_alloc&) {
+        return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
+    }
+    *out_hash = hash;
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_forward_kinematics(nuka_world_handle world) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    const nuka_phi_op_call fk{uint16_t(NkOp::FkWorldPoses), &w->p_fk}, sync{uint16_t(NkOp::SyncLinkBodyPose), &w->p_sync};
+    for (const nuka_phi_op_call* call : {&fk, &sync}) {
+        if (call == &sync && w->model.bodies_per_env == 0u) break;
+        const uint8_t status = w->be->dispatch(w->backend, reinterpret_cast<const nuka_phi_model_view*>(&w->model),
+                                               reinterpret_cast<const nuka_phi_data_view*>(&w->data), call);
+        if (status != uint8_t(Status::Ok)) return Error(MapStatus(status), std::string("dispatch failed: ") + OpName(static_cast<NkOp>(call->op)));
+    }
+    return NUKA_RESULT_OK;
+}
+
+extern "C++" {
+namespace nkh {
+namespace {
+// src/c_abi/params.cpp:24-57
+enum Param : uint32_t { kGravityZ, kVelocityIterations, kLinkMass, kJointDamping, kJointArmature, kJointFrictionloss, kDriveStiffness, kDriveForceLimit, kParamCount };
+struct ParamDef { const char* key; const char* unit; const char* scene_field; nuka_param_type_t type; double min_value, max_value; };
+constexpr double kFloatMin = 1.1754943508222875e-38, kFloatMax = 3.4028234663852886e38;
+constexpr ParamDef kParams[kParamCount] = {
+    {"gravity_z", "m/s^2", "", NUKA_PARAM_F32, -1000.0, 1000.0},
+    {"velocity_iterations", "", "", NUKA_PARAM_U32, 1.0, 65535.0},
+    {"link_mass", "kg", "body.mass", NUKA_PARAM_F32, kFloatMin, kFloatMax},
+    {"joint_damping", "N*m*s/rad", "joint.damping", NUKA_PARAM_F32, 0.0, kFloatMax},
+    {"joint_armature", "kg*m^2", "joint.armature", NUKA_PARAM_F32, 0.0, kFloatMax},
+    {"joint_frictionloss", "N*m", "joint.frictionloss", NUKA_PARAM_F32, 0.0, kFloatMax},
+    {"drive_stiffness", "N*m/rad", "actuator.gain", NUKA_PARAM_F32, 0.0, kFloatMax},
+    {"drive_force_limit", "N*m", "actuator.force_limit", NUKA_PARAM_F32, 0.0, kFloatMax},
+};
+uint32_t ParamElements(const World& w, uint32_t p) { return p >= kLinkMass ? w.model.links_per_env : 1u; }
+nuka_param_tier_t ParamTier(const World& w, uint32_t p) {   // params.cpp:66-72
+    return p == kJointFrictionloss && w.model.joint_friction_rows == 0u ? NUKA_PARAM_REBUILD : NUKA_PARAM_LIVE;
+}
+
+const Field* FindField(const World& w, const char* name) {
+    for (const Field& f : w.fields) if (std::strcmp(f.name, name) == 0) return &f;
+    return nullptr;
+}
+
+// One value of a template table: the live arena and the snapshot a reset copies back.
+bool PutTemplate(World& w, const char* name, size_t first, const float* values, size_t count) {
+    const Field* f = FindField(w, name);
+    if (f == nullptr || (first + count) > f->count) return false;
+    const size_t offset = f->offset + first * sizeof(float), bytes = count * sizeof(float);
+    return Iface(w.arena)->upload(w.arena, values, offset, bytes) == uint8_t(Status::Ok) &&
+           Iface(w.initial)->upload(w.initial, values, offset, bytes) == uint8_t(Status::Ok);
+}
+
+// One link's column of an environment-major field, in the live arena and in the reset snapshot.
+__global__ void __launch_bounds__(256) FillLinkColumnKernel(float* live, float* initial, uint32_t env_count, uint32_t links, uint32_t link, float value) {
+    for (uint32_t env = blockIdx.x * blockDim.x + threadIdx.x; env < env_count; env += gridDim.x * blockDim.x) {
+        live[size_t{env} * links + link] = value;
+        initial[size_t{env} * links + link] = value;
+    }
+}
+bool PutColumn(World& w, const char* name, uint32_t link, float value) {
+    const Field* f = FindField(w, name);
+    if (f == nullptr || f->count != size_t{w.env_count} * w.model.links_per_env) return false;
+    char* live = static_cast<char*>(Iface(w.arena)->base(w.arena));
+    char* initial = static_cast<char*>(Iface(w.initial)->base(w.initial));
+    hipLaunchKernelGGL(FillLinkColumnKernel, dim3(std::min((w.env_count + 255u) / 256u, 1024u)), dim3(256), 0, BackendStream(w.device->backend),
+                       reinterpret_cast<float*>(live + f->offset), reinterpret_cast<float*>(initial + f->offset), w.env_count, w.model.links_per_env, link, value);
+    return hipGetLastError() == hipSuccess;
+}
+
+nuka_result_t SetParam(World& w, nuka_world_handle handle, uint32_t p, uint32_t element, double value) {   // params.cpp:149-190
+    const ParamDef& def = kParams[p];
+    if (element >= ParamElements(w, p) || !std::isfinite(value) || value < def.min_value || value > def.max_value ||
+        (def.type == NUKA_PARAM_U32 && value != std::floor(value))) return Error(NUKA_RESULT_INVALID_ARG, std::string("value or element out of range for ") + def.key);
+    if (ParamTier(w, p) != NUKA_PARAM_LIVE) return Error(NUKA_RESULT_NOT_SUPPORTED, std::string(def.key) + " changes through a rebuild in this world");
+    const float f = float(value);
+    if (p == kVelocityIterations) return nuka_world_set_velocity_iterations(handle, uint32_t(value));
+    if (p == kGravityZ) {   // nk::World::SetGravity (src/nk/pipeline/world.cpp:804-828): the parameter blocks are rebuilt, a captured graph dropped
+        if (f == w.cfg.gravity[2]) return NUKA_RESULT_OK;
+        if (w.be->synchronize(w.backend, nullptr) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "device error");
+        w.cfg.gravity[2] = f;
+        InvalidatePlan(w);
+        BuildPipeline(w);
+        return w.mode == NUKA_EXECUTION_GRAPH ? PreparePlan(w) : NUKA_RESULT_OK;
+    }
+    const bool scalar_joint = w.host.joint_type[element] <= kPrismatic;
+    if ((p == kJointDamping || p == kJointArmature || p == kJointFrictionloss) && !scalar_joint)
+        return Error(NUKA_RESULT_NOT_SUPPORTED, "the link's joint has no scalar coordinate");
+    if ((p == kDriveStiffness || p == kDriveForceLimit) && (!scalar_joint || w.model.joint_drive_rows == 0u))
+        return Error(NUKA_RESULT_NOT_SUPPORTED, "the link has no drive in this world");
+    if (w.be->synchronize(w.backend, nullptr) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "device error");
+    bool ok = false;
+    switch (p) {
+        case kLinkMass: {   // the centre of mass and the rotational inertia about it stay (params.cpp:112-121)
+            float inertia[36];
+            MakeSpatialInertia(f, w.host.link_diag_inertia.data() + 3u * element, w.host.link_inertial_frame.data() + 7u * element, inertia);
+            ok = PutTemplate(w, "link_inertia", size_t{36u} * element, inertia, 36u);
+            if (ok) { std::memcpy(w.host.link_inertia.data() + 36u * element, inertia, sizeof(inertia)); w.host.link_mass[element] = f; }
+            break;
+        }
+        case kJointDamping: ok = PutTemplate(w, "joint_damping", element, &f, 1u); if (ok) w.host.joint_damping[element] = f; break;
+        case kJointArmature: ok = PutTemplate(w, "joint_armature", element, &f, 1u); if (ok) w.host.joint_armature[element] = f; break;
+        case kJointFrictionloss: ok = PutTemplate(w, "joint_frictionloss", element, &f, 1u); if (ok) w.host.joint_frictionloss[element] = f; break;
+        case kDriveStiffness:   // the cook derives a position drive's damping from its gain the same way (params.cpp:135-141)
+            ok = PutColumn(w, "drive_stiffness", element, f) && PutColumn(w, "drive_damping", element, 2.0f * std::sqrt(f));
+            if (ok) w.drive_stiffness[element] = f;
+            break;
+        case kDriveForceLimit: ok = PutColumn(w, "drive_force_limit", element, f); if (ok) w.drive_force_limit[element] = f; break;
+        default: break;
+    }
+    if (!ok || w.be->synchronize(w.backend, nullptr) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, std::string("write of ") + def.key + " failed");
+    return NUKA_RESULT_OK;
+}
+}  // namespace
+}  // namespace nkh
+}  // extern "C++"
+
+nuka_result_t nuka_world_param_count(nuka_world_handle world, uint32_t* out_count) {
+    if (out_count == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    if (world == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    *out_count = kParamCount;
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_get_param_infos(nuka_world_handle world, nuka_param_info_t* infos, uint32_t capacity) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (infos == nullptr || capacity < kParamCount) return Error(NUKA_RESULT_INVALID_ARG, "infos must hold every parameter");
+    for (uint32_t i = 0u; i < kParamCount; ++i)
+        if (infos[i].struct_size != sizeof(nuka_param_info_t) || infos[i].schema_version != NUKA_PARAM_INFO_VERSION)
+            return Error(NUKA_RESULT_INVALID_ARG, "struct_size or schema_version mismatch");
+    for (uint32_t i = 0u; i < kParamCount; ++i) {
+        const ParamDef& def = kParams[i];
+        nuka_param_info_t& info = infos[i];
+        info = {};
+        info.struct_size = sizeof(info);
+        info.schema_version = NUKA_PARAM_INFO_VERSION;
+        std::snprintf(info.key, sizeof(info.key), "%s", def.key);
+        std::snprintf(info.unit, sizeof(info.unit), "%s", def.unit);
+        std::snprintf(info.scene_field, sizeof(info.scene_field), "%s", def.scene_field);
+        info.type = def.type;
+        info.tier = ParamTier(*w, i);
+        info.count = ParamElements(*w, i);
+        info.min_value = def.min_value;
+        info.max_value = def.max_value;
+    }
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_get_param(nuka_world_handle world, uint32_t param, uint32_t element, double* out_value) {
+    if (out_value == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (param >= kParamCount || element >= ParamElements(*w, param)) return Error(NUKA_RESULT_INVALID_ARG, "unknown parameter or element");
+    switch (param) {   // params.cpp:74-90
+        case kGravityZ: *out_value = w->cfg.gravity[2]; break;
+        case kVelocityIterations: *out_value = w->p_solve.iterations; break;
+        case kLinkMass: *out_value = w->host.link_inertia[size_t{36u} * element + 3u * 6u + 3u]; break;   // (3,3) of the row-major 6x6
+        case kJointDamping: *out_value = w->host.joint_damping[element]; break;
+        case kJointArmature: *out_value = w->host.joint_armature[element]; break;
+        case kJointFrictionloss: *out_value = w->host.joint_frictionloss[element]; break;
+        case kDriveStiffness: *out_value = w->drive_stiffness[element]; break;
+        default: *out_value = w->drive_force_limit[element]; break;
+    }
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_set_param(nuka_world_handle world, uint32_t param, uint32_t element, double value) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (param >= kParamCount) return Error(NUKA_RESULT_INVALID_ARG, "unknown parameter");
+    try {
+        return SetParam(*w, world, param, element, value);
+    } catch (const std::bad_alloc&) {
+        return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
+    } catch (const std::exception& e) {
+        return Error(NUKA_RESULT_INTERNAL, e.what());
+    }
+}
+
+nuka_result_t nuka_world_set_link_mass(nuka_world_handle world, uint32_t link_index, float mass) {
+    return nuka_world_set_param(world, kLinkMass, link_index, mass);
+}
+
+nuka_result_t nuka_world_set_gravity_z(nuka_world_handle world, float gravity_z) {
+    return nuka_world_set_param(world, kGravityZ, 0u, gravity_z);
 }
 
 }  // extern "C"
