@@ -116,6 +116,11 @@ typedef struct nuka_world_desc_t {
     uint32_t solver_fold_drive_damping;    /* 0 => on (pipeline.hpp:48-49): a drive's velocity feedback is solved
                                               implicitly through the mass matrix; ~0u => off.  Read only when
                                               struct_size covers it */
+    uint32_t solver_substeps;              /* nuka.h:171: substeps of dt / substeps each step runs; 0 => 1.  Status words
+                                              are or-ed over the substeps, joint limit impulses summed, the links'
+                                              contact wrenches averaged over the step (src/nk/pipeline/pipeline.cpp:118-180).
+                                              Read, like the next member, only when struct_size covers it */
+    uint32_t contact_detection_substeps;   /* nuka.h:172: 0 or 1; substeps that share a detection are NOT_SUPPORTED */
 } nuka_world_desc_t;
 
 /* Scene files (src/import/mjcf_importer.cpp LoadMjcf and src/import/urdf_importer.cpp LoadUrdf, then the articulation

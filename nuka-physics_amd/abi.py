@@ -50,7 +50,7 @@ class WorldDescC(C.Structure):
         ("solver_vel_iters", C.c_uint32), ("solver_pos_iters", C.c_uint32), ("solver_contact_margin", C.c_float),
         ("solver_pos_beta", C.c_float), ("solver_pos_slop", C.c_float), ("solver_velocity_tolerance", C.c_float),
         ("solver_baumgarte_max_velocity", C.c_float), ("solver_overlap_recovery_velocity", C.c_float),
-        ("solver_fold_drive_damping", C.c_uint32),
+        ("solver_fold_drive_damping", C.c_uint32), ("solver_substeps", C.c_uint32), ("contact_detection_substeps", C.c_uint32),
     ]
 
 
@@ -159,7 +159,7 @@ class Template:
 
 
 def world_desc(env_count, dt, gravity=(0.0, 0.0, -9.81), vel_iters=0, pos_iters=0, contact_margin=0.0,
-               velocity_tolerance=0.0, fold_drive_damping=True):
+               velocity_tolerance=0.0, fold_drive_damping=True, substeps=0):
     d = WorldDescC()
     d.struct_size = C.sizeof(WorldDescC)
     d.env_count, d.fixed_dt = env_count, dt
@@ -168,4 +168,5 @@ def world_desc(env_count, dt, gravity=(0.0, 0.0, -9.81), vel_iters=0, pos_iters=
     d.solver_contact_margin = contact_margin
     d.solver_velocity_tolerance = velocity_tolerance
     d.solver_fold_drive_damping = 0 if fold_drive_damping else INVALID
+    d.solver_substeps = substeps
     return d

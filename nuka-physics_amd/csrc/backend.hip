@@ -18,7 +18,7 @@ const char* OpName(NkOp op) {
         "ApplyDrives", "ArticulationDynamics", "IntegrateVelocity", "FkWorldPoses", "IntegratePosition", "BuildAabbs",
         "LbvhBuild", "LbvhQueryPairs", "NarrowphasePrimitives", "AssembleRows", "SyncLinkBodyPose", "NarrowphaseHeightfield",
         "ContactWarmStart", "SnapshotStepVelocity", "FkLinkVelocities", "BlockDescentSolve", "ResetEnvs", "SnapshotState",
-        "RestoreState", "ReadoutDrives", "ReadoutContactWrench"};
+        "RestoreState", "ReadoutDrives", "ReadoutContactWrench", "AccumulateStep"};
     return op < NkOp::Count ? names[static_cast<uint16_t>(op)] : "?";
 }
 
@@ -48,6 +48,7 @@ void RegisterOps() {
     set(NkOp::BlockDescentSolve, &OpBlockDescentSolve);
     set(NkOp::ReadoutDrives, &OpReadoutDrives);
     set(NkOp::ReadoutContactWrench, &OpReadoutContactWrench);
+    set(NkOp::AccumulateStep, &OpAccumulateStep);
 }
 
 void Fail(nuka_phi_execution_error* error, Status status, uint16_t op, int native, const char* message) {

@@ -27,6 +27,7 @@ Status OpContactWarmStart(const ModelView&, const DataView&, const void*, hipStr
 Status OpBlockDescentSolve(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpReadoutDrives(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpReadoutContactWrench(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpAccumulateStep(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpSnapshotStepVelocity(const ModelView&, const DataView&, const void*, hipStream_t);
 
 }  // namespace nkh

@@ -15,7 +15,7 @@ enum class NkOp : uint16_t {
     ApplyDrives, ArticulationDynamics, IntegrateVelocity, FkWorldPoses, IntegratePosition, BuildAabbs, LbvhBuild,
     LbvhQueryPairs, NarrowphasePrimitives, AssembleRows, SyncLinkBodyPose, NarrowphaseHeightfield, ContactWarmStart,
     SnapshotStepVelocity, FkLinkVelocities, BlockDescentSolve, ResetEnvs, SnapshotState, RestoreState,
-    ReadoutDrives, ReadoutContactWrench,
+    ReadoutDrives, ReadoutContactWrench, AccumulateStep,
     Count
 };
 
@@ -126,6 +126,9 @@ struct DataView {
     uint32_t *row_unit;                     // per row: the one coordinate a single-coordinate row acts on, ~0u otherwise
     float *row_unit_value;                  // its Jacobian entry there
     float *snapshot;                        // SnapshotState / RestoreState storage
+    // sums over the substeps of one step (fields.yaml:627-632), written by AccumulateStep
+    uint32_t *step_env_status;
+    float *step_link_impulse, *step_link_moment, *step_joint_limit_impulse;
 };
 
 // --- parameter PODs (field names follow src/phi/op_schema.hpp) -------------------------------------------
@@ -182,5 +185,8 @@ struct ReadoutContactWrenchParams {   // op_schema.hpp:746-755
     uint32_t env_count, base_link_count, max_contacts_per_env, rows_per_env, full_row_slot_count, contact_rows_per_env;
 };
 struct SnapshotParams { uint32_t env_count, selected_env_count; };
+// op_schema.hpp:170-180; the flags this path uses (the particle and free-body ones have no counterpart here)
+constexpr uint32_t kAccumulateOutputs = 1u, kAccumulateLinkWrench = 2u, kAccumulateJointLimit = 4u, kFinalizeLinkWrench = 8u;
+struct AccumulateStepParams { uint32_t env_count, links_per_env, flags, first, last; float substep_dt, inv_outer_dt; };
 
 }  // namespace nkh

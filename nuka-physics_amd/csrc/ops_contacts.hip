@@ -1343,6 +1343,63 @@ Status OpReadoutContactWrench(const ModelView& m, const DataView& d, const void*
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 
+namespace {
+// AccumulateStepKernel (ops/readout.cu:222-300), the outputs of a step of several substeps: status words are or-ed,
+// joint limit impulses summed, the links' contact wrenches averaged as impulses and moments about the world origin
+// over the whole step, and the applied link wrenches cleared after the last substep.  One thread per link.
+__global__ void __launch_bounds__(256) AccumulateStepKernel(DataView d, AccumulateStepParams p) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t links = p.env_count * p.links_per_env;
+    if (i < p.env_count) {
+        const uint32_t status = d.env_status[i];
+        const uint32_t combined = p.first != 0u ? status : d.step_env_status[i] | status;
+        d.step_env_status[i] = combined;
+        if (p.last != 0u) d.env_status[i] = combined;
+    }
+    if (i >= links) return;
+    if ((p.flags & kAccumulateLinkWrench) != 0u) {
+        float* wrench = d.link_contact_wrench + size_t{i} * 6u;
+        const V3 impulse = scale3(V3{wrench[0], wrench[1], wrench[2]}, p.substep_dt);
+        const V3 origin{d.link_pose[size_t{i} * 7u], d.link_pose[size_t{i} * 7u + 1u], d.link_pose[size_t{i} * 7u + 2u]};
+        const V3 moment = add3(scale3(V3{wrench[3], wrench[4], wrench[5]}, p.substep_dt), cross3(origin, impulse));
+        float* sum_impulse = d.step_link_impulse + size_t{i} * 3u, *sum_moment = d.step_link_moment + size_t{i} * 3u;
+        V3 total_impulse = impulse, total_moment = moment;
+        if (p.first == 0u) {
+            total_impulse = add3(V3{sum_impulse[0], sum_impulse[1], sum_impulse[2]}, impulse);
+            total_moment = add3(V3{sum_moment[0], sum_moment[1], sum_moment[2]}, moment);
+        }
+        sum_impulse[0] = total_impulse.x; sum_impulse[1] = total_impulse.y; sum_impulse[2] = total_impulse.z;
+        sum_moment[0] = total_moment.x; sum_moment[1] = total_moment.y; sum_moment[2] = total_moment.z;
+        if (p.last != 0u) {
+            const V3 force = scale3(total_impulse, p.inv_outer_dt);
+            const V3 torque = scale3(sub3(total_moment, cross3(origin, total_impulse)), p.inv_outer_dt);
+            wrench[0] = force.x; wrench[1] = force.y; wrench[2] = force.z; wrench[3] = torque.x; wrench[4] = torque.y; wrench[5] = torque.z;
+        }
+    }
+    if ((p.flags & kAccumulateJointLimit) != 0u) {
+        for (uint32_t side = 0u; side < 2u; ++side) {
+            const size_t slot = size_t{i} * 2u + side;
+            const float impulse = d.joint_limit_impulse[slot];
+            const float total = p.first != 0u ? impulse : d.step_joint_limit_impulse[slot] + impulse;
+            d.step_joint_limit_impulse[slot] = total;
+            if (p.last != 0u) d.joint_limit_impulse[slot] = total;
+        }
+    }
+    if (p.last != 0u && (p.flags & kFinalizeLinkWrench) != 0u)
+        for (uint32_t k = 0u; k < 6u; ++k) d.link_wrench[size_t{i} * 6u + k] = 0.0f;
+}
+}  // namespace
+
+Status OpAccumulateStep(const ModelView&, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const AccumulateStepParams*>(params);
+    if (p == nullptr || (p->flags & ~(kAccumulateOutputs | kAccumulateLinkWrench | kAccumulateJointLimit | kFinalizeLinkWrench)) != 0u ||
+        (p->flags & kAccumulateOutputs) == 0u) return Status::InvalidArgument;
+    const uint32_t count = p->env_count * (p->links_per_env > 0u ? p->links_per_env : 1u);
+    if (count == 0u) return Status::Ok;
+    hipLaunchKernelGGL(AccumulateStepKernel, dim3((count + 255u) / 256u), dim3(256), 0, stream, d, *p);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
 Status OpSnapshotStepVelocity(const ModelView&, const DataView&, const void*, hipStream_t) { return Status::Ok; }
 
 void InitContactKernels() {

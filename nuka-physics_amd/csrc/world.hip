@@ -289,7 +289,9 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(contact_point, kF32, E * S * 3) X(contact_normal, kF32, E * S * 3) X(contact_force, kF32, E * S * 3) \
     X(ucontact_impulse, kF32, E * S * 12) X(link_contact_wrench, kF32, E * nl * 6) X(contact_side_a_kind, kU32, E * S) \
     X(contact_side_b_kind, kU32, E * S) X(contact_side_a_index, kU32, E * S) X(contact_side_b_index, kU32, E * S) \
-    X(contact_link, kU32, E * S)
+    X(contact_link, kU32, E * S) \
+    X(step_env_status, kU32, E) X(step_link_impulse, kF32, E * nl * 3) X(step_link_moment, kF32, E * nl * 3) \
+    X(step_joint_limit_impulse, kF32, E * nl * 2)
 
 #define NKH_MODEL_FIELDS(X) \
     X(joint_type, kU8) X(parent_link, kU32) X(joint_axis, kF32) X(parent_offset, kF32) X(link_local_pose, kF32) \
@@ -341,6 +343,7 @@ struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
     ContactWarmStartParams p_warm0{}, p_warm1{};
     BlockDescentSolveParams p_solve{};
     SnapshotParams p_snapshot{};
+    std::vector<AccumulateStepParams> p_accumulate;   // one per substep (pipeline.cpp:128-152)
     nuka_execution_mode_t mode = NUKA_EXECUTION_EAGER;
     nuka_phi_plan* plan = nullptr;
     std::vector<float> drive_stiffness, drive_force_limit;   // per template link: what nuka_world_get_param reports
@@ -423,43 +426,46 @@ void BuildPipeline(World& w) {
     const uint32_t E = w.env_count, nl = m.links_per_env, nb = m.bodies_per_env;
     const nuka_world_desc_t& cfg = w.cfg;
     const bool has_contacts = m.rows_per_env > 0u;
+    // A step of several substeps runs the interval below that many times at dt / substeps (pipeline.cpp:63-69).
+    const uint32_t substeps = std::max(1u, cfg.solver_substeps);
+    const float dt = cfg.fixed_dt / float(substeps);
     const float contact_margin = cfg.solver_contact_margin;
     const float query_reach = std::fmax(0.02f, 2.0f * (2.0f * 0.0f + contact_margin));   // contact_query.hpp:20-22
     w.p_fk = {E, E * nl};
     w.p_fk_velocity = {E, E * nl};
     w.p_drives = {};
-    w.p_drives.dt = cfg.fixed_dt; w.p_drives.total_link_count = E * nl; w.p_drives.links_per_env = nl;
+    w.p_drives.dt = dt; w.p_drives.total_link_count = E * nl; w.p_drives.links_per_env = nl;
     w.p_drives.mode = m.drive_mode; w.p_drives.articulation_count = E; w.p_drives.bodies_per_env = nb;
     const bool drives = m.joint_drive_rows > 0u;
     const bool fold = drives && cfg.solver_fold_drive_damping != 0xFFFFFFFFu;   // pipeline.cpp:380-381
     w.p_drives.affine = drives ? 1u : 0u;
     w.p_drives.defer_velocity_damping = fold ? 1u : 0u;
     std::memcpy(w.p_drives.gravity, cfg.gravity, sizeof(cfg.gravity));
-    w.p_readout_drives = {cfg.fixed_dt, E * nl, nl, m.rows_per_env, m.contact_rows_per_env + m.joint_limit_rows + m.joint_friction_rows};
+    w.p_readout_drives = {dt, E * nl, nl, m.rows_per_env, m.contact_rows_per_env + m.joint_limit_rows + m.joint_friction_rows};
     ArticulationDynamicsParams& dyn = w.p_dynamics;   // pipeline.cpp:388-402
     dyn = {};
-    dyn.dt = cfg.fixed_dt; dyn.max_dof = m.max_dof; dyn.integrate_velocity = 1u; dyn.fold_drive_damping = fold ? 1u : 0u; dyn.reuse_mass = 0u;
+    dyn.dt = dt; dyn.max_dof = m.max_dof; dyn.integrate_velocity = 1u; dyn.fold_drive_damping = fold ? 1u : 0u; dyn.reuse_mass = 0u;
     std::memcpy(dyn.gravity, cfg.gravity, sizeof(cfg.gravity));
     dyn.articulation_count = E; dyn.total_link_count = E * nl; dyn.apply_link_wrench = 1u; dyn.max_links = nl;
     dyn.links_per_env = nl; dyn.bodies_per_env = nb;
     w.p_dynamics_probe = dyn;
     w.p_dynamics_probe.integrate_velocity = 0u;
     w.p_int_vel = {};
-    w.p_int_vel.dt = cfg.fixed_dt;
+    w.p_int_vel.dt = dt;
     std::memcpy(w.p_int_vel.gravity, cfg.gravity, sizeof(cfg.gravity));
-    w.p_int_pos = {cfg.fixed_dt, E * nl, E, 0u, E, (has_contacts && cfg.solver_pos_iters > 0u) ? 1u : 0u, 0u};
+    w.p_int_pos = {dt, E * nl, E, 0u, E, (has_contacts && cfg.solver_pos_iters > 0u) ? 1u : 0u, 0u};
     w.p_sync = {E, nl, nb, 0u, 0u};
-    w.p_aabbs = {E, nb, 0u, std::fmax(contact_margin, 0.0005f), cfg.fixed_dt, query_reach};   // pipeline.cpp:613-615
+    w.p_aabbs = {E, nb, 0u, std::fmax(contact_margin, 0.0005f), dt, query_reach};   // pipeline.cpp:613-615
     w.p_lbvh = {E, nb, 0u};
     w.p_query = {E, nb, 0u, m.contact_slots, m.contact_slots, m.contact_slots, 0u};
-    w.p_narrow = {E, nb, m.contact_slots, m.contact_slots, contact_margin, cfg.fixed_dt, query_reach};
+    w.p_narrow = {E, nb, m.contact_slots, m.contact_slots, contact_margin, dt, query_reach};
     AssembleRowsParams& as = w.p_assemble;   // pipeline.cpp:861-897
     as = {};
     as.env_count = E; as.articulation_count = E; as.total_link_count = E * nl; as.max_dof = m.max_dof;
     as.union_slot_count = m.contact_slots; as.rows_per_env = m.rows_per_env; as.contact_rows_per_env = m.contact_rows_per_env;
     as.full_row_slot_count = m.contact_slots; as.bodies_per_env = nb; as.base_link_count = nl;
     as.position_pass = cfg.solver_pos_iters > 0u ? 1u : 0u;
-    as.dt = cfg.fixed_dt; as.overlap_recovery_velocity = cfg.solver_overlap_recovery_velocity; as.contact_margin = contact_margin;
+    as.dt = dt; as.overlap_recovery_velocity = cfg.solver_overlap_recovery_velocity; as.contact_margin = contact_margin;
     as.joint_limit_rows_per_env = m.joint_limit_rows; as.joint_friction_rows_per_env = m.joint_friction_rows;
     as.joint_drive_rows_per_env = m.joint_drive_rows; as.baumgarte_max_velocity = cfg.solver_baumgarte_max_velocity;
     w.p_warm0 = {0u, E, m.contact_slots, m.rows_per_env, m.contact_slots, 2u};
@@ -467,7 +473,7 @@ void BuildPipeline(World& w) {
     w.p_warm1.phase = 1u;
     BlockDescentSolveParams& bd = w.p_solve;   // pipeline.cpp:471-497
     bd = {};
-    bd.dt = cfg.fixed_dt; bd.env_count = E; bd.rows_per_env = m.rows_per_env; bd.total_body_count = E * nb; bd.articulation_count = E;
+    bd.dt = dt; bd.env_count = E; bd.rows_per_env = m.rows_per_env; bd.total_body_count = E * nb; bd.articulation_count = E;
     bd.max_dof = m.max_dof; bd.max_independent_dof = m.dof; bd.base_link_count = nl; bd.contact_rows_per_env = m.contact_rows_per_env;
     bd.contact_slots_per_env = m.contact_slots; bd.iterations = cfg.solver_vel_iters;
     bd.position_iterations = has_contacts ? cfg.solver_pos_iters : 0u;
@@ -506,8 +512,25 @@ void BuildPipeline(World& w) {
     add(NkOp::FkLinkVelocities, &w.p_fk_velocity);
     if (nb > 0u) add(NkOp::SyncLinkBodyPose, &w.p_sync);
     // a pure readout, part of the step only once a consumer has asked for one of its fields (pipeline.cpp:990-1005)
-    w.p_readout_contacts = {cfg.fixed_dt, E, nl, m.contact_slots, m.rows_per_env, m.contact_slots, m.contact_rows_per_env};
-    if (w.contact_readout_demanded && has_contacts && m.contact_slots > 0u) add(NkOp::ReadoutContactWrench, &w.p_readout_contacts);
+    w.p_readout_contacts = {dt, E, nl, m.contact_slots, m.rows_per_env, m.contact_slots, m.contact_rows_per_env};
+    const bool reads_contacts = w.contact_readout_demanded && has_contacts && m.contact_slots > 0u;
+    if (reads_contacts) add(NkOp::ReadoutContactWrench, &w.p_readout_contacts);
+    if (substeps == 1u) return;
+    // pipeline.cpp:118-180: the interval once per substep, each followed by the accumulation of the step's outputs
+    const std::vector<nuka_phi_op_call> interval = w.calls;
+    w.calls.clear();
+    w.p_accumulate.assign(substeps, AccumulateStepParams{});
+    for (uint32_t step = 0u; step < substeps; ++step) {
+        AccumulateStepParams& outputs = w.p_accumulate[step];
+        outputs.env_count = E; outputs.links_per_env = nl;
+        outputs.flags = kAccumulateOutputs | kFinalizeLinkWrench;
+        if (reads_contacts) outputs.flags |= kAccumulateLinkWrench;
+        if (m.joint_limit_rows != 0u) outputs.flags |= kAccumulateJointLimit;
+        outputs.first = step == 0u ? 1u : 0u; outputs.last = step + 1u == substeps ? 1u : 0u;
+        outputs.substep_dt = dt; outputs.inv_outer_dt = 1.0f / cfg.fixed_dt;
+        for (const nuka_phi_op_call& call : interval) w.calls.push_back(call);
+        add(NkOp::AccumulateStep, &outputs);
+    }
 }
 
 void InvalidatePlan(World& w) {
@@ -640,8 +663,9 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
     constexpr size_t kTemplateBase = offsetof(nuka_template_desc_t, joint_limit_lower);
     constexpr size_t kTemplateJointRows = offsetof(nuka_template_desc_t, excluded_pairs);
     constexpr size_t kWorldBase = offsetof(nuka_world_desc_t, solver_fold_drive_damping);
+    constexpr size_t kWorldDrives = offsetof(nuka_world_desc_t, solver_substeps);
     if ((tmpl->struct_size != sizeof(nuka_template_desc_t) && tmpl->struct_size != kTemplateJointRows && tmpl->struct_size != kTemplateBase) ||
-        (desc->struct_size != sizeof(nuka_world_desc_t) && desc->struct_size != kWorldBase))
+        (desc->struct_size != sizeof(nuka_world_desc_t) && desc->struct_size != kWorldDrives && desc->struct_size != kWorldBase))
         return Error(NUKA_RESULT_INVALID_ARG, "struct_size mismatch");
     nuka_template_desc_t template_copy{};
     std::memcpy(&template_copy, tmpl, tmpl->struct_size);
@@ -666,6 +690,9 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
         if (cfg.solver_pos_slop <= 0.0f) cfg.solver_pos_slop = 1.0e-3f;
         if (cfg.solver_velocity_tolerance <= 0.0f) cfg.solver_velocity_tolerance = 1.0e-5f;
         if (cfg.solver_baumgarte_max_velocity <= 0.0f) cfg.solver_baumgarte_max_velocity = 3.0e38f;
+        if (cfg.solver_substeps == 0u) cfg.solver_substeps = 1u;
+        if (cfg.solver_substeps > 64u) throw std::invalid_argument("solver_substeps must be at most 64");
+        if (cfg.contact_detection_substeps > 1u) throw NotSupported("substeps that share one contact detection are not built on this path");
         w.env_count = desc->env_count;
         const ModelView& hc = w.host.counts;
         const size_t E = w.env_count, nl = hc.links_per_env, nb = hc.bodies_per_env, md = hc.max_dof, S = hc.contact_slots, R = hc.rows_per_env;

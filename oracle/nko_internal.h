@@ -117,6 +117,12 @@ struct nko_world {
     float *contact_point, *contact_normal, *contact_force, *ucontact_impulse, *link_contact_wrench;
     uint32_t *contact_side_a_kind, *contact_side_b_kind, *contact_side_a_index, *contact_side_b_index, *contact_link;
     int fold_drive_damping;
+    /* a step of several substeps (nk/pipeline/pipeline.cpp:56-180; ops/readout.cu AccumulateStepKernel) */
+    uint32_t substeps;
+    float outer_dt;
+    int readout_in_step;
+    uint32_t* step_env_status;
+    float *step_link_impulse, *step_link_moment, *step_joint_limit_impulse;
 };
 
 /* ---- math (nko_math.c) ------------------------------------------------- */

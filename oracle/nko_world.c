@@ -208,7 +208,11 @@ nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc*
     if (w->cfg.solver_baumgarte_max_velocity <= 0.0f) w->cfg.solver_baumgarte_max_velocity = 3.0e38f;
     /* pipeline.hpp:48-49: velocity feedback of a drive is solved implicitly unless switched off */
     w->fold_drive_damping = 1;
-    if (desc->struct_size >= sizeof(nko_world_desc) && desc->solver_fold_drive_damping == 0xFFFFFFFFu) w->fold_drive_damping = 0;
+    if (desc->struct_size >= offsetof(nko_world_desc, solver_substeps) && desc->solver_fold_drive_damping == 0xFFFFFFFFu) w->fold_drive_damping = 0;
+    /* pipeline.cpp:63-69: every op of the interval runs at dt / substeps */
+    w->substeps = desc->struct_size >= sizeof(nko_world_desc) && desc->solver_substeps > 1u ? desc->solver_substeps : 1u;
+    w->outer_dt = w->cfg.fixed_dt;
+    w->cfg.fixed_dt = w->cfg.fixed_dt / (float)w->substeps;
     w->env_count = desc->env_count;
     w->threads = 1;
     const nko_template* t = &w->t;
@@ -230,6 +234,8 @@ nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc*
     w->chain_jacobian = ALLOC(float, E * R * md); w->chain_jacobian_b = ALLOC(float, E * R * md);
     w->row_cj_link = ALLOC(uint32_t, E * R); w->row_cj_link_b = ALLOC(uint32_t, E * R);
     w->row_count = ALLOC(uint32_t, E); w->contact_count = ALLOC(uint32_t, E); w->contact_row_extent = ALLOC(uint32_t, E * 2u);
+    w->step_env_status = ALLOC(uint32_t, E); w->step_link_impulse = ALLOC(float, E * nl * 3u);
+    w->step_link_moment = ALLOC(float, E * nl * 3u); w->step_joint_limit_impulse = ALLOC(float, E * nl * 2u);
     w->env_status = ALLOC(uint32_t, E); w->vbd_velocity_sweep_count = ALLOC(uint32_t, E);
     w->solver_residual = ALLOC(float, E * 4u);
     w->solver_velocity = ALLOC(float, E * md); w->solver_free = ALLOC(float, E * md); w->solver_penalty = ALLOC(float, E * R);
@@ -275,6 +281,7 @@ void nko_world_destroy(nko_world* w) {
     free(w->chain_jacobian_b); free(w->row_cj_link); free(w->row_cj_link_b); free(w->row_count); free(w->contact_count);
     free(w->contact_row_extent); free(w->env_status); free(w->vbd_velocity_sweep_count); free(w->solver_residual);
     free(w->solver_velocity); free(w->solver_free); free(w->solver_penalty);
+    free(w->step_env_status); free(w->step_link_impulse); free(w->step_link_moment); free(w->step_joint_limit_impulse);
     free(w->contact_material); free(w->contact_cache_pair); free(w->contact_cache_feature); free(w->contact_cache_material);
     free(w->contact_cache_lambda); free(w->contact_cache_normal); free(w->contact_cache_age); free(w->contact_cache_current_owner);
     free(w->contact_cache_old_keep); free(w->contact_cache_extent); free(w->contact_warm_start_counts); free(w->contact_cache_match);
@@ -358,7 +365,7 @@ uint32_t nko_world_rows_per_env(const nko_world* w) { return w->t.rows_per_env; 
 void nko_fk_world_poses(nko_world* w) { FOR_ENVS(nko_env_fk(w, env)) }
 void nko_apply_drives(nko_world* w) { FOR_ENVS(nko_env_apply_drives(w, env)) }
 void nko_readout_drives(nko_world* w) { FOR_ENVS(nko_env_readout_drives(w, env)) }
-void nko_readout_contact_wrench(nko_world* w) { FOR_ENVS(nko_env_readout_contact_wrench(w, env)) }
+void nko_readout_contact_wrench(nko_world* w) { w->readout_in_step = 1; FOR_ENVS(nko_env_readout_contact_wrench(w, env)) }
 void nko_articulation_dynamics(nko_world* w, uint32_t integrate_velocity) { FOR_ENVS(nko_env_dynamics(w, env, integrate_velocity)) }
 void nko_sync_link_body_pose(nko_world* w) { FOR_ENVS(nko_env_sync_body_pose(w, env)) }
 void nko_build_aabbs(nko_world* w) { FOR_ENVS(nko_env_aabbs(w, env)) }
@@ -375,7 +382,7 @@ void nko_integrate_position(nko_world* w) { FOR_ENVS(nko_env_integrate_position(
 void nko_fk_link_velocities(nko_world* w) { FOR_ENVS(nko_env_link_velocities(w, env)) }
 
 /* Op order of one step (src/nk/pipeline/pipeline.cpp:374-986) for an articulated world with ground contact. */
-void nko_world_step(nko_world* w) {
+static void step_interval(nko_world* w) {
     nko_fk_world_poses(w);
     if (w->t.joint_drive_rows > 0u) nko_apply_drives(w);
     nko_articulation_dynamics(w, 1u);
@@ -396,5 +403,63 @@ void nko_world_step(nko_world* w) {
     nko_fk_world_poses(w);
     nko_fk_link_velocities(w);
     if (w->t.nb > 0u) nko_sync_link_body_pose(w);
+    /* pipeline.cpp:990-1005: a readout a consumer has asked for closes every interval */
+    if (w->readout_in_step && w->t.rows_per_env > 0u && w->t.slots > 0u) nko_readout_contact_wrench(w);
+}
+
+/* AccumulateStepKernel (ops/readout.cu:222-300) for the outputs this path has: status words or-ed over the substeps,
+ * joint limit impulses summed, link contact wrenches averaged as impulses and moments about the world origin, the
+ * applied link wrenches cleared after the last substep. */
+static void accumulate_step(nko_world* w, int first, int last) {
+    const size_t E = w->env_count, nl = w->t.nl;
+    const float substep_dt = w->cfg.fixed_dt, inv_outer_dt = 1.0f / w->outer_dt;
+    const int wrenches = w->readout_in_step && w->t.rows_per_env > 0u && w->t.slots > 0u;
+    for (size_t e = 0u; e < E; ++e) {
+        const uint32_t status = w->env_status[e];
+        const uint32_t combined = first ? status : (w->step_env_status[e] | status);
+        w->step_env_status[e] = combined;
+        if (last) w->env_status[e] = combined;
+    }
+    for (size_t i = 0u; i < E * nl; ++i) {
+        if (wrenches) {
+            float* wrench = w->link_contact_wrench + i * 6u;
+            const v3 impulse = v3_scale(v3_make(wrench[0], wrench[1], wrench[2]), substep_dt);
+            const v3 origin = v3_make(w->link_pose[i * 7u], w->link_pose[i * 7u + 1u], w->link_pose[i * 7u + 2u]);
+            const v3 moment = v3_add(v3_scale(v3_make(wrench[3], wrench[4], wrench[5]), substep_dt), v3_cross(origin, impulse));
+            float* si = w->step_link_impulse + i * 3u, *sm = w->step_link_moment + i * 3u;
+            v3 total_impulse = impulse, total_moment = moment;
+            if (!first) {
+                total_impulse = v3_add(v3_make(si[0], si[1], si[2]), impulse);
+                total_moment = v3_add(v3_make(sm[0], sm[1], sm[2]), moment);
+            }
+            si[0] = total_impulse.x; si[1] = total_impulse.y; si[2] = total_impulse.z;
+            sm[0] = total_moment.x; sm[1] = total_moment.y; sm[2] = total_moment.z;
+            if (last) {
+                const v3 force = v3_scale(total_impulse, inv_outer_dt);
+                const v3 torque = v3_scale(v3_sub(total_moment, v3_cross(origin, total_impulse)), inv_outer_dt);
+                wrench[0] = force.x; wrench[1] = force.y; wrench[2] = force.z; wrench[3] = torque.x; wrench[4] = torque.y; wrench[5] = torque.z;
+            }
+        }
+        if (w->t.joint_limit_rows != 0u)
+            for (size_t side = 0u; side < 2u; ++side) {
+                const size_t slot = i * 2u + side;
+                const float impulse = w->joint_limit_impulse[slot];
+                const float total = first ? impulse : w->step_joint_limit_impulse[slot] + impulse;
+                w->step_joint_limit_impulse[slot] = total;
+                if (last) w->joint_limit_impulse[slot] = total;
+            }
+        if (last) for (size_t k = 0u; k < 6u; ++k) w->link_wrench[i * 6u + k] = 0.0f;
+    }
+}
+
+void nko_world_step(nko_world* w) {
+    if (w->substeps <= 1u) {
+        step_interval(w);
+    } else {
+        for (uint32_t s = 0u; s < w->substeps; ++s) {
+            step_interval(w);
+            accumulate_step(w, s == 0u, s + 1u == w->substeps);
+        }
+    }
     ++w->step_index;
 }

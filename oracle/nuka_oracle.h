@@ -112,6 +112,8 @@ typedef struct nko_world_desc {
     float solver_baumgarte_max_velocity;
     float solver_overlap_recovery_velocity;
     uint32_t solver_fold_drive_damping;   /* read only when struct_size covers it */
+    uint32_t solver_substeps;             /* 0 => 1; read, like the next member, only when struct_size covers it */
+    uint32_t contact_detection_substeps;  /* 0 or 1 */
 } nko_world_desc;
 
 typedef struct nko_world nko_world;
@@ -138,7 +140,8 @@ void nko_assemble_rows(nko_world* w);
 void nko_contact_warm_start(nko_world* w, uint32_t phase);
 void nko_block_descent_solve(nko_world* w);
 void nko_readout_drives(nko_world* w);
-void nko_readout_contact_wrench(nko_world* w);   /* on demand; not part of nko_world_step */
+void nko_readout_contact_wrench(nko_world* w);   /* on demand: not part of nko_world_step until it has been called once,
+                                                    then every interval ends with it (nk/pipeline/world.cpp:905-975) */
 void nko_integrate_position(nko_world* w);
 void nko_fk_link_velocities(nko_world* w);
 /* The whole op list of one step, in the reference's order. */

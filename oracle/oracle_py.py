@@ -22,9 +22,9 @@ U64_FIELDS = {"ucontact_id_pair", "ucontact_id_feature", "contact_material", "co
 
 def build(force=False):
     """Compiles the oracle (and, where the reference tree is mounted, the reference-header shim)."""
-    if force or not os.path.exists(LIB_PATH):
-        subprocess.run(["make", "-C", HERE, "_build/libnuka_oracle.so"] + (["-B"] if force else []), check=True,
-                       stdout=subprocess.DEVNULL)
+    # make compares the sources' and headers' times with the library's: an up-to-date library costs nothing
+    subprocess.run(["make", "-C", HERE, "_build/libnuka_oracle.so"] + (["-B"] if force else []), check=True,
+                   stdout=subprocess.DEVNULL)
     if os.path.isdir("/root/reference/src") and (force or not os.path.exists(REF_PATH)):
         subprocess.run(["make", "-C", HERE, "ref"], check=True, stdout=subprocess.DEVNULL)
 
