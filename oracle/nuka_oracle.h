@@ -37,6 +37,8 @@
  *                             push-out, dry friction hold / slip; torque-mode drive rows against the direct-torque path)
  *   contact readout         : pinned (weight of a resting ball, Coulomb friction and its moment, link wrenches adding up
  *                             to the generalized impulse the solve applied)
+ *   substeps                : pinned (n substeps of dt are n steps of dt / n bit for bit; the step's status, joint limit
+ *                             impulses and link contact wrenches are the or, the sum and the time average of those steps')
  *   UABD fixed point        : pinned (closed-form resting, falling, sticking and sliding ball; Coulomb / KKT
  *                             conditions and momentum balance of converged solves)
  *   UABD iterate path       : PARITY UNPINNED - penalty heuristic, first-sweep segment search, FISTA
