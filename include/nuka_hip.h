@@ -176,6 +176,22 @@ nuka_result_t nuka_world_step_n(nuka_world_handle world, uint32_t step_count);  
 /* nuka.h:257-279 */
 typedef enum nuka_execution_mode_t { NUKA_EXECUTION_EAGER = 0, NUKA_EXECUTION_GRAPH = 1 } nuka_execution_mode_t;
 nuka_result_t nuka_world_set_execution_mode(nuka_world_handle world, nuka_execution_mode_t mode);
+/* nuka.h:261-275, 342: how the world executes - mode, whether a captured graph stands, captures and graph replays so
+ * far, and the last failure of a dispatch, capture or replay (status mapped to a result, the op, the HIP error code). */
+enum { NUKA_EXECUTION_INFO_VERSION = 1 };
+typedef struct nuka_world_execution_info_t {
+    uint32_t struct_size;
+    uint32_t schema_version;
+    nuka_execution_mode_t mode;
+    uint32_t graph_ready;
+    uint64_t capture_attempts;
+    uint64_t graph_replays;
+    nuka_result_t last_result;
+    uint32_t failed_op;
+    int32_t native_error;
+    char message[256];
+} nuka_world_execution_info_t;
+nuka_result_t nuka_world_get_execution_info(nuka_world_handle world, nuka_world_execution_info_t* out);
 nuka_result_t nuka_world_set_velocity_iterations(nuka_world_handle world, uint32_t iterations);   /* nuka.h:289 */
 nuka_result_t nuka_world_get_velocity_iterations(nuka_world_handle world, uint32_t* out_iterations);
 nuka_result_t nuka_world_synchronize(nuka_world_handle world);   /* nuka.h:376 */
@@ -190,6 +206,12 @@ nuka_result_t nuka_world_checkpoint_capture(nuka_world_handle world, nuka_checkp
 nuka_result_t nuka_world_checkpoint_restore(nuka_world_handle world, nuka_checkpoint_handle checkpoint);
 void nuka_checkpoint_destroy(nuka_checkpoint_handle checkpoint);
 nuka_result_t nuka_checkpoint_byte_size(nuka_checkpoint_handle checkpoint, uint64_t* out_bytes);
+/* nuka.h:394-398: a checkpoint as a file - a header with the layout hash of the world it was taken of (environment
+ * count, names and sizes of the persistent fields) and the persistent bytes.  Reading makes a checkpoint of `world`
+ * from the file; a file of another layout, a truncated one or one that is no checkpoint is INVALID_ARG.  The format is
+ * this library's own, not the reference's. */
+nuka_result_t nuka_checkpoint_write(nuka_checkpoint_handle checkpoint, const char* path);
+nuka_result_t nuka_world_checkpoint_read(nuka_world_handle world, const char* path, nuka_checkpoint_handle* out);
 /* nuka.h:401-402: 1 when both checkpoints were taken of worlds of one layout and hold the same persistent bytes, else 0 */
 nuka_result_t nuka_checkpoint_equal(nuka_checkpoint_handle a, nuka_checkpoint_handle b, uint32_t* out_equal);
 /* nuka.h:403-404, src/c_abi/checkpoint.cpp:601-636: 64-bit FNV-1a over a domain string, the byte count and the

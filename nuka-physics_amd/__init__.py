@@ -47,6 +47,13 @@ class ParamInfoC(C.Structure):
                 ("min_value", C.c_double), ("max_value", C.c_double)]
 
 
+class ExecutionInfoC(C.Structure):
+    """nuka_world_execution_info_t"""
+    _fields_ = [("struct_size", C.c_uint32), ("schema_version", C.c_uint32), ("mode", C.c_int), ("graph_ready", C.c_uint32),
+                ("capture_attempts", C.c_uint64), ("graph_replays", C.c_uint64), ("last_result", C.c_int), ("failed_op", C.c_uint32),
+                ("native_error", C.c_int32), ("message", C.c_char * 256)]
+
+
 PARAM_INFO_VERSION = 1
 PARAM_LIVE, PARAM_REBUILD = 0, 1
 PARAMS = ("gravity_z", "velocity_iterations", "link_mass", "joint_damping", "joint_armature", "joint_frictionloss", "drive_stiffness",
@@ -70,6 +77,7 @@ EXPORTS = [
     "nuka_scene_joint_name", "nuka_scene_initial_state", "nuka_world_create_from_scene",
     "nuka_checkpoint_equal", "nuka_world_state_hash", "nuka_world_forward_kinematics", "nuka_world_param_count", "nuka_world_get_param_infos",
     "nuka_world_get_param", "nuka_world_set_param", "nuka_world_set_link_mass", "nuka_world_set_gravity_z",
+    "nuka_checkpoint_write", "nuka_world_checkpoint_read", "nuka_world_get_execution_info",
 ]
 
 
@@ -145,6 +153,9 @@ def lib():
         L.nuka_world_set_param.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.c_double]
         L.nuka_world_set_link_mass.argtypes = [C.c_void_p, C.c_uint32, C.c_float]
         L.nuka_world_set_gravity_z.argtypes = [C.c_void_p, C.c_float]
+        L.nuka_checkpoint_write.argtypes = [C.c_void_p, C.c_char_p]
+        L.nuka_world_checkpoint_read.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]
+        L.nuka_world_get_execution_info.argtypes = [C.c_void_p, C.POINTER(ExecutionInfoC)]
         _lib = L
     return _lib
 
@@ -331,6 +342,21 @@ class World:
         out = C.c_uint32()
         _check(lib().nuka_checkpoint_equal(a, b, C.byref(out)))
         return bool(out.value)
+
+    def write_checkpoint(self, checkpoint, path):
+        _check(lib().nuka_checkpoint_write(checkpoint, str(path).encode()))
+
+    def read_checkpoint(self, path):
+        """nuka_world_checkpoint_read: a checkpoint of this world from a file a world of the same layout wrote."""
+        handle = C.c_void_p()
+        _check(lib().nuka_world_checkpoint_read(self._h, str(path).encode(), C.byref(handle)))
+        return handle
+
+    def execution_info(self):
+        info = ExecutionInfoC()
+        info.struct_size, info.schema_version = C.sizeof(ExecutionInfoC), 1
+        _check(lib().nuka_world_get_execution_info(self._h, C.byref(info)))
+        return info
 
     def param_infos(self):
         """nuka_world_get_param_infos as a list of dicts, in parameter order."""

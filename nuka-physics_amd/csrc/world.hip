@@ -347,6 +347,8 @@ struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
     nuka_execution_mode_t mode = NUKA_EXECUTION_EAGER;
     nuka_phi_plan* plan = nullptr;
     std::vector<float> drive_stiffness, drive_force_limit;   // per template link: what nuka_world_get_param reports
+    uint64_t capture_attempts = 0u, graph_replays = 0u;      // nuka_world_get_execution_info
+    nuka_phi_execution_error last_error{};
 
     ~World() {
         if (be != nullptr && plan != nullptr) be->plan_free(backend, plan);
@@ -552,8 +554,12 @@ nuka_result_t StepEager(World& w) {
     for (const nuka_phi_op_call& call : w.calls) {
         const uint8_t status = w.be->dispatch(w.backend, reinterpret_cast<const nuka_phi_model_view*>(&w.model),
                                               reinterpret_cast<const nuka_phi_data_view*>(&w.data), &call);
-        if (status != uint8_t(Status::Ok))
-            return Error(MapStatus(status), std::string("step failed in op ") + OpName(static_cast<NkOp>(call.op)));
+        if (status != uint8_t(Status::Ok)) {
+            w.last_error = {};
+            w.last_error.status = status; w.last_error.failed_op = call.op;
+            std::snprintf(w.last_error.message, sizeof(w.last_error.message), "step failed in op %s", OpName(static_cast<NkOp>(call.op)));
+            return Error(MapStatus(status), w.last_error.message);
+        }
     }
     return NUKA_RESULT_OK;
 }
@@ -562,9 +568,10 @@ nuka_result_t StepEager(World& w) {
 nuka_result_t PreparePlan(World& w) {
     if (w.plan != nullptr) return NUKA_RESULT_OK;
     nuka_phi_execution_error error{};
+    ++w.capture_attempts;
     w.plan = w.be->plan_create(w.backend, reinterpret_cast<const nuka_phi_model_view*>(&w.model),
                                reinterpret_cast<const nuka_phi_data_view*>(&w.data), w.calls.data(), int(w.calls.size()), &error);
-    if (w.plan == nullptr) return Error(MapStatus(error.status), std::string("graph capture failed: ") + error.message);
+    if (w.plan == nullptr) { w.last_error = error; return Error(MapStatus(error.status), std::string("graph capture failed: ") + error.message); }
     return NUKA_RESULT_OK;
 }
 
@@ -575,7 +582,8 @@ nuka_result_t StepN(World& w, uint32_t n) {
         uint32_t submitted = 0u;
         nuka_phi_execution_error error{};
         const uint8_t status = w.be->plan_execute_repeated(w.backend, w.plan, n, &submitted, &error);
-        if (status != uint8_t(Status::Ok)) return Error(MapStatus(status), std::string("graph launch failed: ") + error.message);
+        w.graph_replays += submitted;
+        if (status != uint8_t(Status::Ok)) { w.last_error = error; return Error(MapStatus(status), std::string("graph launch failed: ") + error.message); }
         return NUKA_RESULT_OK;
     }
     for (uint32_t i = 0u; i < n; ++i) {
@@ -1156,11 +1164,10 @@ nuka_result_t nuka_device_copy_bandwidth(nuka_device_handle device, size_t bytes
     return NUKA_RESULT_OK;
 }
 
-nuka_result_t nuka_world_checkpoint_capture(nuka_world_handle world, nuka_checkpoint_handle* out) {
-    auto* w = reinterpret_cast<World*>(world);
-    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
-    if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
-    *out = nullptr;
+namespace nkh {
+namespace {
+// A checkpoint's storage and segment table for `w`, nothing copied yet.
+nuka_result_t NewCheckpoint(World* w, std::unique_ptr<Checkpoint>* out) {
     auto cp = std::unique_ptr<Checkpoint>(new (std::nothrow) Checkpoint{});
     if (!cp) return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
     cp->owner = w;
@@ -1189,12 +1196,119 @@ nuka_result_t nuka_world_checkpoint_capture(nuka_world_handle world, nuka_checkp
         ++at;
     }
     cp->bytes = total;
+    *out = std::move(cp);
+    return NUKA_RESULT_OK;
+}
+
+// What a checkpoint file has to agree on with the world that reads it: the environment count and every kept field's
+// name and size, FNV-1a hashed.
+uint64_t CheckpointLayoutHash(const World& w) {
+    uint64_t hash = 14695981039346656037ull;
+    auto mix = [&hash](const void* bytes, size_t count) {
+        const auto* p = static_cast<const uint8_t*>(bytes);
+        for (size_t i = 0u; i < count; ++i) { hash ^= p[i]; hash *= 1099511628211ull; }
+    };
+    const uint64_t envs = w.env_count;
+    mix(&envs, sizeof(envs));
+    for (const Field& f : w.fields) {
+        if (f.is_template || f.count == 0u || !CheckpointKeeps(f.name)) continue;
+        const uint64_t bytes = f.count * f.elem_bytes;
+        mix(f.name, std::strlen(f.name) + 1u);
+        mix(&bytes, sizeof(bytes));
+    }
+    return hash;
+}
+struct CheckpointFileHeader { char magic[8]; uint64_t layout_hash, bytes; };
+constexpr char kCheckpointMagic[8] = {'N', 'K', 'H', 'C', 'K', 'P', 'T', '1'};
+}  // namespace
+}  // namespace nkh
+
+nuka_result_t nuka_world_checkpoint_capture(nuka_world_handle world, nuka_checkpoint_handle* out) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    *out = nullptr;
+    std::unique_ptr<Checkpoint> cp;
+    if (const nuka_result_t made = NewCheckpoint(w, &cp); made != NUKA_RESULT_OK) return made;
     hipLaunchKernelGGL(CheckpointCopyKernel, dim3(256, cp->segments.count), dim3(256), 0, BackendStream(w->device->backend), cp->segments, 0u);
     if (hipGetLastError() != hipSuccess || nuka_world_synchronize(world) != NUKA_RESULT_OK) {
         Iface(cp->store)->free(cp->store);
         return Error(NUKA_RESULT_DEVICE_ERROR, "checkpoint capture failed");
     }
     *out = reinterpret_cast<nuka_checkpoint_handle>(cp.release());
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_checkpoint_write(nuka_checkpoint_handle checkpoint, const char* path) {
+    auto* cp = reinterpret_cast<Checkpoint*>(checkpoint);
+    if (cp == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "checkpoint is null");
+    if (path == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "path is null");
+    try {
+        std::vector<uint8_t> bytes(cp->bytes);
+        if (cp->bytes > 0u && Iface(cp->store)->download(cp->store, bytes.data(), 0u, cp->bytes) != uint8_t(Status::Ok))
+            return Error(NUKA_RESULT_DEVICE_ERROR, "checkpoint download failed");
+        CheckpointFileHeader header{};
+        std::memcpy(header.magic, kCheckpointMagic, sizeof(header.magic));
+        header.layout_hash = CheckpointLayoutHash(*cp->owner);
+        header.bytes = cp->bytes;
+        std::FILE* file = std::fopen(path, "wb");
+        if (file == nullptr) return Error(NUKA_RESULT_INVALID_ARG, std::string("cannot open ") + path);
+        const bool ok = std::fwrite(&header, sizeof(header), 1u, file) == 1u && (bytes.empty() || std::fwrite(bytes.data(), bytes.size(), 1u, file) == 1u);
+        if (std::fclose(file) != 0 || !ok) return Error(NUKA_RESULT_INTERNAL, std::string("write failed: ") + path);
+    } catch (const std::bad_alloc&) {
+        return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
+    }
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_checkpoint_read(nuka_world_handle world, const char* path, nuka_checkpoint_handle* out) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (path == nullptr || out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "path and out are required");
+    *out = nullptr;
+    std::FILE* file = std::fopen(path, "rb");
+    if (file == nullptr) return Error(NUKA_RESULT_INVALID_ARG, std::string("cannot open ") + path);
+    nuka_result_t result = NUKA_RESULT_OK;
+    try {
+        CheckpointFileHeader header{};
+        std::unique_ptr<Checkpoint> cp;
+        if (std::fread(&header, sizeof(header), 1u, file) != 1u || std::memcmp(header.magic, kCheckpointMagic, sizeof(header.magic)) != 0)
+            result = Error(NUKA_RESULT_INVALID_ARG, "not a checkpoint file");
+        else if (header.layout_hash != CheckpointLayoutHash(*w))
+            result = Error(NUKA_RESULT_INVALID_ARG, "the checkpoint was written by a world of another layout");
+        else if ((result = NewCheckpoint(w, &cp)) == NUKA_RESULT_OK) {
+            std::vector<uint8_t> bytes(cp->bytes);
+            if (header.bytes != cp->bytes || (!bytes.empty() && std::fread(bytes.data(), bytes.size(), 1u, file) != 1u))
+                result = Error(NUKA_RESULT_INVALID_ARG, "truncated checkpoint file");
+            else if (!bytes.empty() && Iface(cp->store)->upload(cp->store, bytes.data(), 0u, bytes.size()) != uint8_t(Status::Ok))
+                result = Error(NUKA_RESULT_DEVICE_ERROR, "checkpoint upload failed");
+            if (result == NUKA_RESULT_OK && nuka_world_synchronize(world) != NUKA_RESULT_OK) result = NUKA_RESULT_DEVICE_ERROR;
+            if (result != NUKA_RESULT_OK) Iface(cp->store)->free(cp->store);
+            else *out = reinterpret_cast<nuka_checkpoint_handle>(cp.release());
+        }
+    } catch (const std::bad_alloc&) {
+        result = Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
+    }
+    std::fclose(file);
+    return result;
+}
+
+nuka_result_t nuka_world_get_execution_info(nuka_world_handle world, nuka_world_execution_info_t* out) {   // src/c_abi/world.cpp:890-909
+    if (out == nullptr || out->struct_size != sizeof(*out) || out->schema_version != NUKA_EXECUTION_INFO_VERSION)
+        return Error(NUKA_RESULT_INVALID_ARG, "struct_size or schema_version mismatch");
+    *out = {};
+    out->struct_size = sizeof(*out);
+    out->schema_version = NUKA_EXECUTION_INFO_VERSION;
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    out->mode = w->mode;
+    out->graph_ready = w->plan != nullptr ? 1u : 0u;
+    out->capture_attempts = w->capture_attempts;
+    out->graph_replays = w->graph_replays;
+    out->last_result = MapStatus(w->last_error.status);
+    out->failed_op = w->last_error.failed_op;
+    out->native_error = w->last_error.native_code;
+    std::snprintf(out->message, sizeof(out->message), "%s", w->last_error.message);
     return NUKA_RESULT_OK;
 }
 

@@ -5,6 +5,7 @@ A parameter written into a live world has to act exactly as the same value cooke
 gets its values through nuka_world_set_param, the oracle world is created from a template (and a world description)
 that holds them from the start.  fp32 fields to norm-wise relative error 1e-4 a step, as in test_gpu_parity."""
 import copy
+import ctypes as C
 
 import numpy as np
 import pytest
@@ -165,4 +166,50 @@ def test_pose_refresh_state_hash_and_checkpoint_equality(oracle_py, device):
     for handle in (kept, again, moved, other):
         nk.lib().nuka_checkpoint_destroy(handle)
     for w in (world, twin, oracle):
+        w.close()
+
+
+def test_checkpoint_files_and_execution_info(device, tmp_path):
+    E = 32
+    cfg = nk.synthetic.config(2, E)
+    desc = abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters)
+    world, other = nk.World(device, cfg.template, desc), nk.World(device, cfg.template, desc)
+    world.set_state(cfg.state())
+    info = world.execution_info()
+    assert (info.mode, info.graph_ready, info.capture_attempts, info.graph_replays, info.last_result) == (0, 0, 0, 0, 0)
+    world.set_execution_mode(True)
+    world.step(3); world.synchronize()
+    info = world.execution_info()
+    assert (info.mode, info.graph_ready, info.capture_attempts, info.graph_replays) == (1, 1, 1, 3)
+    world.set_velocity_iterations(5)                       # a changed op sequence: the graph is captured again
+    assert world.execution_info().capture_attempts == 2
+    # a checkpoint written by one world, read by another of the same layout, continues bit for bit
+    kept = world.checkpoint()
+    path = tmp_path / "quadruped.ckpt"
+    world.write_checkpoint(kept, path)
+    size = C.c_uint64()
+    nk.lib().nuka_checkpoint_byte_size(kept, C.byref(size))
+    assert path.stat().st_size == 24 + size.value
+    read = other.read_checkpoint(path)
+    other.set_velocity_iterations(5)
+    other.restore(read); other.synchronize()
+    assert other.state_hash() == world.state_hash()
+    world.restore(kept)                                    # a restore also clears the solver's carried history: both start from it
+    world.step(2); other.step(2)
+    assert other.state_hash() == world.state_hash() and np.array_equal(other.download("qdot"), world.download("qdot"))
+    # files that are no checkpoint of this layout are refused
+    bigger = nk.World(device, cfg.template, abi.world_desc(E + 1, cfg.dt))
+    for reader, file in ((bigger, path), (other, tmp_path / "absent.ckpt")):
+        with pytest.raises(nk.NukaError) as err:
+            reader.read_checkpoint(file)
+        assert err.value.code == abi.RESULT_INVALID_ARG
+    (tmp_path / "short.ckpt").write_bytes(path.read_bytes()[:100])
+    (tmp_path / "noise.ckpt").write_bytes(b"x" * 64)
+    for name in ("short.ckpt", "noise.ckpt"):
+        with pytest.raises(nk.NukaError) as err:
+            other.read_checkpoint(tmp_path / name)
+        assert err.value.code == abi.RESULT_INVALID_ARG
+    for handle in (kept, read):
+        nk.lib().nuka_checkpoint_destroy(handle)
+    for w in (world, other, bigger):
         w.close()
