@@ -24,6 +24,10 @@ DOMINANT_KERNEL = "BlockDescentTileKernel"
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, scaled
 # by the same counters' reading of a plain copy of known size); keyed by (config, envs).  None where not measured.
 MEASURED_TRAFFIC_BYTES = {(3, 4096): 224.9e6}   # profiles/counters_humanoid_4096.txt
+# What the same counter runs say limits the dominant kernel (not measured by this script): vector instructions a
+# launch issues and the share of a wave's resident cycles spent issuing them, at two waves a SIMD.
+MEASURED_ISSUE = {(3, 4096): {"limiter": "valu_issue", "valu_instructions_per_env": 185000, "wave_cycles_issuing_valu": 0.45,
+                              "waves_per_simd": 2, "source": "profiles/counters_humanoid_4096.txt"}}
 
 
 def algorithmic_bytes(nl, nv, nc, floating):
@@ -127,7 +131,8 @@ def main():
                    "free_running_ms_per_step": free_ms},
         "roofline": {"bound": "hbm", "kernel": kernel, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, E)),
-                     "algorithmic_bytes_per_launch": kernel_bytes * E, "kernel_ms": kernel_ms},
+                     "algorithmic_bytes_per_launch": kernel_bytes * E, "kernel_ms": kernel_ms,
+                     "profiled": MEASURED_ISSUE.get((args.config, E))},
         "roofline_step": {"algorithmic_bytes_per_env_step": b_alg, "state_io_bytes_per_env_step": tier_a,
                           "achieved": step_gbps, "unit": "GB/s", "frac": step_gbps / HBM_PEAK_GBPS},
         "per_op_ms": {k: round(v, 4) for k, v in per_op.items() if v >= 0.001},
