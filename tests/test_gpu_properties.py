@@ -118,6 +118,37 @@ def test_scene_files_at_full_batch_size(device):
         world.close()
 
 
+def test_long_run_of_an_authored_robot_stays_bounded(device):
+    """Ten simulated seconds of the capsule walker holding its authored pose on damped, driven joints (graph replay):
+    every environment stays finite and flagged clean, velocities stay small and the robots stay carried by their
+    contacts.  (The benchmark configurations are no such test: their seeded torques act on undamped joints.)"""
+    import os
+    from conftest import ROOT
+    E, steps = 1024, 2000
+    scene = nk.Scene(os.path.join(ROOT, "tests", "data", "capsule_walker.xml"))
+    world = nk.World(device, scene, abi.world_desc(E, 0.0, vel_iters=8))
+    nl = scene.link_count
+    rng = np.random.default_rng(11)
+    twist = np.zeros((E, nl, 6), np.float32)
+    twist[:, 0] = rng.normal(0, 0.3, (E, 6))
+    base = world.download("base_pose").reshape(E, 7).copy()
+    base[:, 2] = 0.545
+    world.upload("base_pose", base)
+    world.upload("link_velocity", twist)
+    world.set_execution_mode(True)
+    peak = 0.0
+    for _ in range(4):
+        world.step(steps // 4); world.synchronize()
+        qdot = world.download("qdot")
+        assert np.all(np.isfinite(qdot)) and not world.download("env_status").any()
+        peak = max(peak, float(np.abs(qdot).max()))
+    assert peak < 50.0, peak
+    pose = world.download("link_pose").reshape(E, nl, 7)
+    assert np.all(np.isfinite(pose)) and np.abs(np.linalg.norm(pose[:, :, 3:], axis=2) - 1).max() < 1e-5
+    assert (world.download("contact_count") >= 1).mean() > 0.9 and pose[:, 0, 2].min() > 0.0
+    world.close()
+
+
 def test_rope_full_batch_steps(device):
     E = 1024
     cfg, world = stepped(device, 5, E)
