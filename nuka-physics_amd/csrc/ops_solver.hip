@@ -6,7 +6,7 @@
 namespace nkh {
 namespace solver {
 #define NKH_DECLARE_WIDTH(N) \
-    extern template __global__ void BlockDescentTileKernel<N>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
+    extern template __global__ void BlockDescentTileKernel<N>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
 NKH_DECLARE_WIDTH(4) NKH_DECLARE_WIDTH(8) NKH_DECLARE_WIDTH(12) NKH_DECLARE_WIDTH(16) NKH_DECLARE_WIDTH(20) NKH_DECLARE_WIDTH(24)
 NKH_DECLARE_WIDTH(28) NKH_DECLARE_WIDTH(32) NKH_DECLARE_WIDTH(36) NKH_DECLARE_WIDTH(40) NKH_DECLARE_WIDTH(44) NKH_DECLARE_WIDTH(48)
 NKH_DECLARE_WIDTH(52) NKH_DECLARE_WIDTH(56) NKH_DECLARE_WIDTH(60) NKH_DECLARE_WIDTH(64)
@@ -54,7 +54,7 @@ __global__ void __launch_bounds__(1024) OrderTilesKernel(DataView d, uint32_t en
 }
 
 
-using SolverKernel = void (*)(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
+using SolverKernel = void (*)(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
 // One instantiation per padded width.
 const SolverKernel kSolverKernels[16] = {
     BlockDescentTileKernel<4>, BlockDescentTileKernel<8>, BlockDescentTileKernel<12>, BlockDescentTileKernel<16>,
@@ -79,11 +79,24 @@ Status OpBlockDescentSolve(const ModelView& m, const DataView& d, const void* pa
     const size_t budget = 150u * 1024u;
     const uint32_t staged = SolverHeadCapacity(m, p->contact_slots_per_env == 0u ? 1u : p->contact_slots_per_env, budget);
     if (staged == 0u) return Status::InvalidArgument;
-    const uint32_t cap = staged + m.joint_limit_rows + m.joint_friction_rows + m.joint_drive_rows;
-    const size_t lds = size_t{solver::SolverLdsFloats(m.dof, cap, staged)} * sizeof(float);
+    const uint32_t joint_heads = m.joint_limit_rows + m.joint_friction_rows + m.joint_drive_rows;
+    const auto lds_bytes = [&](uint32_t contact_heads) { return size_t{solver::SolverLdsFloats(m.dof, contact_heads + joint_heads, contact_heads)} * sizeof(float); };
+    const auto blocks_per_unit = [&](uint32_t contact_heads) { return std::min<size_t>(8u, (160u * 1024u) / lds_bytes(contact_heads)); };
+    // The LDS a block needs grows with the contact heads it can stage, and a scene's slots (every pair that may ever
+    // touch, at its largest manifold) outnumber the contacts an environment usually has.  Where a smaller capacity
+    // lets more blocks share a compute unit, environments with few contact points go to a launch of that capacity
+    // and only the others to the full one; an environment's results do not depend on which launch solves it.
+    uint32_t few = staged;
+    while (few > 8u && blocks_per_unit(few) < 8u) --few;
+    const bool split = p->contact_slots_per_env != 0u && few < staged && blocks_per_unit(few) > blocks_per_unit(staged);
+    const SolverKernel kernel = kSolverKernels[solver::PaddedWidth(m.dof) / 4u - 1u];
     hipLaunchKernelGGL(OrderTilesKernel, dim3(1), dim3(1024), 0, stream, d, p->env_count);
-    hipLaunchKernelGGL(kSolverKernels[solver::PaddedWidth(m.dof) / 4u - 1u], dim3(p->env_count), dim3(solver::kWave), lds, stream, m, d, *p, cap,
-                       staged);
+    if (split) {
+        hipLaunchKernelGGL(kernel, dim3(p->env_count), dim3(solver::kWave), lds_bytes(few), stream, m, d, *p, few + joint_heads, few, 0u, few);
+        hipLaunchKernelGGL(kernel, dim3(p->env_count), dim3(solver::kWave), lds_bytes(staged), stream, m, d, *p, staged + joint_heads, staged, few + 1u, kInvalid);
+    } else {
+        hipLaunchKernelGGL(kernel, dim3(p->env_count), dim3(solver::kWave), lds_bytes(staged), stream, m, d, *p, staged + joint_heads, staged, 0u, kInvalid);
+    }
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 

@@ -1121,9 +1121,16 @@ __host__ __device__ inline uint32_t SolverLdsFloats(uint32_t n, uint32_t cap, ui
 // DescendTile (:2941-3087)
 template <int N>
 __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(N <= kTwoWaveWidth ? 2 : 1, N <= kTwoWaveWidth ? 2 : 1)))
-BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint32_t cap, uint32_t staged_cap) {
+BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint32_t cap, uint32_t staged_cap, uint32_t points_lo,
+                       uint32_t points_hi) {
     extern __shared__ __align__(16) float lds[];
     const uint32_t env = d.tile_order[blockIdx.x], lane = threadIdx.x;
+    // A world whose contact slots outnumber the contacts it usually has is solved by two launches of different LDS
+    // capacity; each takes the environments whose contact points fall in its range and leaves the others at once.
+    if (points_lo != 0u || points_hi != kInvalid) {
+        const uint32_t points = d.contact_count[env];
+        if (points < points_lo || points > points_hi) return;
+    }
     const uint32_t R = p.rows_per_env, md = p.max_dof, n = m.dof, nl = m.links_per_env, S = p.contact_slots_per_env;
     Tile c;
     c.env = env; c.lane = lane; c.n = n; c.ld = uint32_t(N) + 1u; c.ldj = uint32_t(N); c.cap = cap; c.narrow = staged_cap; c.heads = 0u; c.iteration = 0u;
@@ -1133,6 +1140,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
 #ifdef NKH_SOLVER_PROFILE
     for (int i = 0; i < 26; ++i) c.prof[i] = 0;
     for (int i = 0; i < 4; ++i) c.prof_count[i] = 0u;
+    const long long prof_wall_start = wall_clock64();
 #endif
     PROF_BEGIN(c, 9);
     PROF_BEGIN(c, 0);
@@ -1511,6 +1519,10 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         for (int i = 0; i < 10; ++i) d.solver_penalty[size_t{env} * R + i] = float(c.prof[i]);
         for (int i = 0; i < 4; ++i) d.solver_penalty[size_t{env} * R + 10 + i] = float(c.prof_count[i]);
         for (int i = 10; i < 26; ++i) d.solver_penalty[size_t{env} * R + 4 + i] = float(c.prof[i]);
+        // launch slot and the wave's first and last moment on the constant 100 MHz clock, as raw words
+        d.solver_penalty[size_t{env} * R + 30] = __uint_as_float(uint32_t(prof_wall_start));
+        d.solver_penalty[size_t{env} * R + 31] = __uint_as_float(uint32_t(wall_clock64()));
+        d.solver_penalty[size_t{env} * R + 32] = __uint_as_float(blockIdx.x);
     }
 #endif
     // the block velocities persist for the next solve's carried start

@@ -3,11 +3,11 @@
 
 namespace nkh {
 namespace solver {
-template __global__ void BlockDescentTileKernel<4>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
-template __global__ void BlockDescentTileKernel<8>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
-template __global__ void BlockDescentTileKernel<12>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
-template __global__ void BlockDescentTileKernel<16>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
-template __global__ void BlockDescentTileKernel<20>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
-template __global__ void BlockDescentTileKernel<24>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<4>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<8>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<12>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<16>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<20>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<24>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
 }  // namespace solver
 }  // namespace nkh

@@ -3,8 +3,8 @@
 
 namespace nkh {
 namespace solver {
-template __global__ void BlockDescentTileKernel<28>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
-template __global__ void BlockDescentTileKernel<32>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
-template __global__ void BlockDescentTileKernel<36>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<28>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<32>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<36>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
 }  // namespace solver
 }  // namespace nkh

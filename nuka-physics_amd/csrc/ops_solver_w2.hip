@@ -3,8 +3,8 @@
 
 namespace nkh {
 namespace solver {
-template __global__ void BlockDescentTileKernel<40>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
-template __global__ void BlockDescentTileKernel<44>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
-template __global__ void BlockDescentTileKernel<48>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<40>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<44>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<48>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
 }  // namespace solver
 }  // namespace nkh

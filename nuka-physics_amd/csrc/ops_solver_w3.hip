@@ -3,7 +3,7 @@
 
 namespace nkh {
 namespace solver {
-template __global__ void BlockDescentTileKernel<52>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
-template __global__ void BlockDescentTileKernel<56>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<52>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<56>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
 }  // namespace solver
 }  // namespace nkh

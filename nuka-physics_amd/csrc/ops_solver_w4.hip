@@ -3,7 +3,7 @@
 
 namespace nkh {
 namespace solver {
-template __global__ void BlockDescentTileKernel<60>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
-template __global__ void BlockDescentTileKernel<64>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<60>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<64>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
 }  // namespace solver
 }  // namespace nkh

@@ -4,7 +4,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from conftest import nk, relative_error
+from conftest import per_env_error, nk, relative_error
 
 pytestmark = pytest.mark.gpu
 abi = nk.abi
@@ -221,6 +221,51 @@ def test_box_manifolds_and_either_side_order(oracle_py, device, plane_first):
     assert np.mean(ids_g[mask] == ids_o[mask]) > 0.99       # box corners carry feature ids: exact; sphere points hash a quantised position
     for name in ("qdot", "q", "link_pose", "link_velocity"):
         assert relative_error(world.download(name), oracle.download(name)) <= 1e-4, name
+    world.close()
+    oracle.close()
+
+
+def test_environments_on_either_side_of_the_capacity_split_match_the_oracle(oracle_py, device):
+    """A raft of a hundred spheres over the plane: a hundred contact slots, of which a tilted raft fills a few and a
+    level one all.  The solve sends environments with few contact points to a launch with a small LDS capacity and
+    the others to a full-capacity launch; either way an environment's result is the oracle's, which knows no such
+    split.  Heads beyond the first sixty-four go through the head fields instead of lane registers."""
+    E = 96
+    t = abi.Template()
+    t.add_link(abi.JOINT_FLOATING, None, mass=5.0, diag_inertia=(0.2, 0.2, 0.4))
+    profile = t.add_profile(0.7)
+    t.add_body(abi.ROLE_STATIC, kind=abi.SHAPE_PLANE, contype=2, conaffinity=1, profile=profile)
+    t.add_body(abi.ROLE_LINK_BODY, link=0, contype=0, conaffinity=0)
+    for i in range(10):
+        for j in range(10):
+            t.add_body(abi.ROLE_PROXY, link=0, kind=abi.SHAPE_SPHERE, params=(0.02, 0, 0, 0), local_pos=(0.05 * (i - 4.5), 0.05 * (j - 4.5), 0.0),
+                       contype=1, conaffinity=2, profile=profile)
+    g = np.random.default_rng(8)
+    tilt = g.uniform(0.0, 0.12, E)
+    tilt[:8] = 0.0                                               # level rafts: every sphere touches
+    height = 0.02 + 0.225 * np.sin(tilt) - 0.001
+    base = np.stack([g.normal(0, 0.1, E), g.normal(0, 0.1, E), height, np.cos(tilt / 2), np.sin(tilt / 2), 0 * tilt, 0 * tilt], 1)
+    state = dict(q=np.zeros((E, 1), np.float32), qdot=np.zeros((E, 1), np.float32), tau=np.zeros((E, 1), np.float32),
+                 base_pose=base.astype(np.float32), root_twist=(g.normal(0, 0.2, (E, 6)) * [1, 1, 1, 1, 1, 0.2]).astype(np.float32))
+    desc = abi.world_desc(E, 1.0 / 200.0, vel_iters=8)
+    world, oracle = nk.World(device, t, desc), oracle_py.OracleWorld(t, desc, threads=8)
+    assert world.info.contact_slots_per_env == 100
+    world.set_state(state)
+    oracle.set_state(state)
+    world.step(2); world.synchronize()
+    oracle.step(2)
+    counts = oracle.download("contact_count")
+    assert counts.min() <= 30 and counts.max() == 100 and ((counts > 56) & (counts < 100)).any(), np.sort(counts)
+    for name in ("contact_count", "ucontact_count", "row_count", "env_status", "vbd_velocity_sweep_count"):
+        assert np.array_equal(world.download(name), oracle.download(name)), name
+    assert not world.download("env_status").any()
+    for name in ("qdot", "link_velocity", "base_pose"):
+        error = per_env_error(world.download(name), oracle.download(name), E)
+        assert error.max() <= 2e-4, (name, float(error.max()), int(counts[error.argmax()]))       # two steps
+    # spheres in a row share a load in no unique way: the multipliers are compared through what they add up to
+    oracle.op("readout_contact_wrench")
+    error = per_env_error(world.download("link_contact_wrench"), oracle.download("link_contact_wrench"), E)
+    assert np.abs(oracle.download("link_contact_wrench")).max() > 10.0 and error.max() <= 1e-3, float(error.max())
     world.close()
     oracle.close()
 
