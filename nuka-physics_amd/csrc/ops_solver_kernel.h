@@ -1512,7 +1512,13 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     if (lane < 4u)
         d.solver_residual[size_t{env} * 4u + lane] =
             lane == 0u ? residual4[0] : lane == 1u ? residual4[1] : lane == 2u ? residual4[2] : residual4[3];
-    if (lane == 0u) { d.vbd_velocity_sweep_count[env] = sweeps; d.solver_cost[env] = c.work; }
+    if (lane == 0u) {
+        d.vbd_velocity_sweep_count[env] = sweeps;
+        // the scheduling key of the next solves: this solve's work, or what is left of an earlier, longer one - an
+        // environment whose solves are long every other step or so keeps its early place in the launch order
+        const uint32_t earlier = d.solver_cost[env];
+        d.solver_cost[env] = max(c.work, earlier - earlier / 4u);
+    }
 #ifdef NKH_SOLVER_PROFILE
     PROF_END(c, 9);
     if (lane == 0u) {
