@@ -35,7 +35,9 @@ def test_headers_compile_as_c_and_agree_with_the_ctypes_mirror(tmp_path):
     """include/*.h are plain C: a C99 program that includes them reports the size of each descriptor and the offset of
     every member the ctypes mirror declares, and the two layouts agree."""
     import subprocess
-    members = {"nuka_template_desc_t": nk.abi.TemplateDescC, "nuka_world_desc_t": nk.abi.WorldDescC, "nuka_scene_info_t": nk.SceneInfoC}
+    members = {"nuka_template_desc_t": nk.abi.TemplateDescC, "nuka_world_desc_t": nk.abi.WorldDescC, "nuka_scene_info_t": nk.SceneInfoC,
+               "nuka_param_info_t": nk.ParamInfoC, "nuka_world_execution_info_t": nk.ExecutionInfoC, "nuka_world_info_t": nk.WorldInfoC,
+               "nuka_buffer_view_t": nk.abi.BufferViewC}
     lines = ['#include <stddef.h>', '#include <stdio.h>', '#include "nuka_phi.h"', '#include "nuka_hip.h"', 'int main(void) {']
     for name, mirror in members.items():
         lines.append(f'    printf("{name} %zu\\n", sizeof({name}));')
@@ -59,7 +61,7 @@ def test_op_catalog_names_round_trip():
     names = [lib.nuka_hip_op_name(i).decode() for i in range(count)]
     for expected in ("FkWorldPoses", "ArticulationDynamics", "SyncLinkBodyPose", "BuildAabbs", "LbvhQueryPairs",
                      "NarrowphasePrimitives", "AssembleRows", "ContactWarmStart", "BlockDescentSolve", "IntegratePosition",
-                     "FkLinkVelocities", "ApplyDrives", "ReadoutDrives"):
+                     "FkLinkVelocities", "ApplyDrives", "ReadoutDrives", "ReadoutContactWrench", "AccumulateStep"):
         assert expected in names
         assert lib.nuka_hip_op_from_name(expected.encode()) == names.index(expected)
     assert lib.nuka_hip_op_from_name(b"NoSuchOp") == -1
