@@ -46,6 +46,52 @@ def solver_bytes(nv, nc):
     return 4 * (nv * (nv + 1) + 3 * nc * nv + 2 * nv + 3 * nc)
 
 
+def scene_run(nk, args):
+    """Not the headline: a scene file's robot (MJCF or URDF, damped and driven joints) left to itself.  The batch
+    settles for --settle steps from the authored pose with a small random push per environment, then --steps
+    free-running steps are timed; environments that are flagged or not finite are counted, not hidden."""
+    import numpy as np
+    scene = nk.Scene(args.scene, nk.SCENE_GROUND_PLANE | nk.SCENE_PLANE_CONTACTS_ONLY if args.scene.endswith(".urdf") else 0)
+    E = args.envs or 4096
+    device = nk.Device(0)
+    world = nk.World(device, scene, nk.abi.world_desc(E, 0.0, vel_iters=8))
+    nl = scene.link_count
+    twist = np.zeros((E, nl, 6), np.float32)
+    twist[:, 0] = np.random.default_rng(11).normal(0, 0.3, (E, 6))
+    world.upload("link_velocity", twist)
+    if args.base_height > 0.0:
+        base = world.download("base_pose").reshape(E, 7).copy()
+        base[:, 2] = args.base_height
+        world.upload("base_pose", base)
+    world.set_execution_mode(args.mode == "graph")
+    world.step(args.settle)
+    world.synchronize()
+    start = time.perf_counter()
+    world.step(args.steps)
+    world.synchronize()
+    wall_ms = (time.perf_counter() - start) * 1e3 / args.steps
+    event_ms = world.time_steps(args.steps) / args.steps
+    world.set_execution_mode(False)
+    per_op = {}
+    for name, ms in world.profile_ops(min(args.steps, 50)):
+        per_op[name] = per_op.get(name, 0.0) + ms
+    failed = int(((world.download("env_status") != 0) | ~np.isfinite(world.download("qdot").reshape(E, -1)).all(1)).sum())
+    sweeps = world.download("vbd_velocity_sweep_count")
+    result = {
+        "metric": "env-steps/sec", "value": E * 1e3 / wall_ms, "unit": "env-steps/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.settle, "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{os.path.basename(args.scene)}: {nl} links, {world.dof} DoF, {world.info.contact_slots_per_env} contact slots, "
+                               f"{E} envs, free-running after {args.settle} settling steps", "envs": E, "execution": args.mode,
+                   "event_ms_per_step": event_ms, "failed_envs": failed, "contacts_mean": float(world.download("contact_count").mean()),
+                   "sweeps_mean": float(sweeps.mean()), "envs_using_every_sweep": int((sweeps == sweeps.max()).sum())},
+        "per_op_ms": {k: round(v, 4) for k, v in per_op.items() if v >= 0.001},
+    }
+    world.close()
+    device.close()
+    print(json.dumps(result))
+
+
 def cpu_baseline(nk, cfg, desc, budget_s=12.0):
     """The CPU oracle (a restatement of the reference algorithm, OpenMP over environments) on the same workload."""
     oracle_py = entry.load_oracle()
@@ -77,12 +123,18 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seeded-only", action="store_true",
                     help="kept for the profile commands: every launch of a run is a step from the seeded batch")
+    ap.add_argument("--scene", default="", help="a scene file instead of a benchmark configuration: its robot left to itself (see scene_run)")
+    ap.add_argument("--settle", type=int, default=600)
+    ap.add_argument("--base-height", type=float, default=0.0, help="with --scene: height of the root link at the start, 0 keeps the file's")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (one wavefront per environment, no cross-device state); "
                  "--gpus must be 1")
 
     nk = entry.load_package()
+    if args.scene:
+        scene_run(nk, args)
+        return
     cfg = nk.synthetic.config(args.config, args.envs or None)
     E = cfg.env_count
     desc = nk.abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters)
