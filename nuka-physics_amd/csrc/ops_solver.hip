@@ -84,19 +84,25 @@ Status OpBlockDescentSolve(const ModelView& m, const DataView& d, const void* pa
     const auto blocks_per_unit = [&](uint32_t contact_heads) { return std::min<size_t>(8u, (160u * 1024u) / lds_bytes(contact_heads)); };
     // The LDS a block needs grows with the contact heads it can stage, and a scene's slots (every pair that may ever
     // touch, at its largest manifold) outnumber the contacts an environment usually has.  Where a smaller capacity
-    // lets more blocks share a compute unit, environments with few contact points go to a launch of that capacity
-    // and only the others to the full one; an environment's results do not depend on which launch solves it.
-    uint32_t few = staged;
-    while (few > 8u && blocks_per_unit(few) < 8u) --few;
-    const bool split = p->contact_slots_per_env != 0u && few < staged && blocks_per_unit(few) > blocks_per_unit(staged);
+    // lets more blocks share a compute unit, environments with few contact points go to a launch of that capacity:
+    // up to three such launches, for eight, four and two blocks a unit, before the full one.  Each launch takes the
+    // environments whose contact points fall in its range; an environment's results do not depend on its launch.
     const SolverKernel kernel = kSolverKernels[solver::PaddedWidth(m.dof) / 4u - 1u];
     hipLaunchKernelGGL(OrderTilesKernel, dim3(1), dim3(1024), 0, stream, d, p->env_count);
-    if (split) {
-        hipLaunchKernelGGL(kernel, dim3(p->env_count), dim3(solver::kWave), lds_bytes(few), stream, m, d, *p, few + joint_heads, few, 0u, few);
-        hipLaunchKernelGGL(kernel, dim3(p->env_count), dim3(solver::kWave), lds_bytes(staged), stream, m, d, *p, staged + joint_heads, staged, few + 1u, kInvalid);
-    } else {
-        hipLaunchKernelGGL(kernel, dim3(p->env_count), dim3(solver::kWave), lds_bytes(staged), stream, m, d, *p, staged + joint_heads, staged, 0u, kInvalid);
+    uint32_t first_points = 0u;
+    if (p->contact_slots_per_env != 0u) {
+        for (const size_t blocks : {size_t{8u}, size_t{4u}, size_t{2u}}) {
+            if (blocks_per_unit(staged) >= blocks) break;                  // the full capacity does as well
+            uint32_t few = staged;
+            while (few > 8u && blocks_per_unit(few) < blocks) --few;
+            if (blocks_per_unit(few) < blocks || few < first_points) continue;   // not even eight heads fit that often
+            hipLaunchKernelGGL(kernel, dim3(p->env_count), dim3(solver::kWave), lds_bytes(few), stream, m, d, *p, few + joint_heads, few,
+                               first_points, few);
+            first_points = few + 1u;
+        }
     }
+    hipLaunchKernelGGL(kernel, dim3(p->env_count), dim3(solver::kWave), lds_bytes(staged), stream, m, d, *p, staged + joint_heads, staged,
+                       first_points, kInvalid);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 

@@ -225,44 +225,54 @@ def test_box_manifolds_and_either_side_order(oracle_py, device, plane_first):
     oracle.close()
 
 
-def test_environments_on_either_side_of_the_capacity_split_match_the_oracle(oracle_py, device):
-    """A raft of a hundred spheres over the plane: a hundred contact slots, of which a tilted raft fills a few and a
-    level one all.  The solve sends environments with few contact points to a launch with a small LDS capacity and
-    the others to a full-capacity launch; either way an environment's result is the oracle's, which knows no such
-    split.  Heads beyond the first sixty-four go through the head fields instead of lane registers."""
+@pytest.mark.parametrize("shape", ["spheres", "boxes"])
+def test_environments_on_either_side_of_the_capacity_split_match_the_oracle(oracle_py, device, shape):
+    """A raft of a hundred spheres (or thirty boxes of four points each) over the plane: a tilted raft fills a few of
+    its contact slots and a level one all.  The solve sends environments with few contact points to launches with
+    a small LDS capacity and the others to fuller ones - two launches for the spheres, three for the boxes; either
+    way an environment's result is the oracle's, which knows no such split.  Heads beyond the first sixty-four go
+    through the head fields instead of lane registers."""
     E = 96
     t = abi.Template()
     t.add_link(abi.JOINT_FLOATING, None, mass=5.0, diag_inertia=(0.2, 0.2, 0.4))
     profile = t.add_profile(0.7)
     t.add_body(abi.ROLE_STATIC, kind=abi.SHAPE_PLANE, contype=2, conaffinity=1, profile=profile)
     t.add_body(abi.ROLE_LINK_BODY, link=0, contype=0, conaffinity=0)
-    for i in range(10):
-        for j in range(10):
-            t.add_body(abi.ROLE_PROXY, link=0, kind=abi.SHAPE_SPHERE, params=(0.02, 0, 0, 0), local_pos=(0.05 * (i - 4.5), 0.05 * (j - 4.5), 0.0),
+    if shape == "spheres":
+        rows, cols, pitch, kind, params, reach, bounds = 10, 10, 0.05, abi.SHAPE_SPHERE, (0.02, 0, 0, 0), 0.225, (56, 100, 100)
+    else:
+        rows, cols, pitch, kind, params, reach, bounds = 6, 5, 0.08, abi.SHAPE_BOX, (0.02, 0.02, 0.02, 0), 0.18, (56, 118, 120)
+    for i in range(rows):
+        for j in range(cols):
+            t.add_body(abi.ROLE_PROXY, link=0, kind=kind, params=params, local_pos=(pitch * (i - (rows - 1) / 2), pitch * (j - (cols - 1) / 2), 0.0),
                        contype=1, conaffinity=2, profile=profile)
     g = np.random.default_rng(8)
     tilt = g.uniform(0.0, 0.12, E)
-    tilt[:8] = 0.0                                               # level rafts: every sphere touches
-    height = 0.02 + 0.225 * np.sin(tilt) - 0.001
+    tilt[:8] = 0.0                                               # level rafts: every shape touches
+    tilt[8:32] = np.linspace(0.001, 0.03, 24)                    # nearly level ones: most do
+    height = 0.02 * np.cos(tilt) + reach * np.sin(tilt) - 0.001
     base = np.stack([g.normal(0, 0.1, E), g.normal(0, 0.1, E), height, np.cos(tilt / 2), np.sin(tilt / 2), 0 * tilt, 0 * tilt], 1)
     state = dict(q=np.zeros((E, 1), np.float32), qdot=np.zeros((E, 1), np.float32), tau=np.zeros((E, 1), np.float32),
                  base_pose=base.astype(np.float32), root_twist=(g.normal(0, 0.2, (E, 6)) * [1, 1, 1, 1, 1, 0.2]).astype(np.float32))
     desc = abi.world_desc(E, 1.0 / 200.0, vel_iters=8)
     world, oracle = nk.World(device, t, desc), oracle_py.OracleWorld(t, desc, threads=8)
-    assert world.info.contact_slots_per_env == 100
+    assert world.info.contact_slots_per_env == rows * cols
     world.set_state(state)
     oracle.set_state(state)
     world.step(2); world.synchronize()
     oracle.step(2)
     counts = oracle.download("contact_count")
-    assert counts.min() <= 30 and counts.max() == 100 and ((counts > 56) & (counts < 100)).any(), np.sort(counts)
-    for name in ("contact_count", "ucontact_count", "row_count", "env_status", "vbd_velocity_sweep_count"):
+    small, middle, full = bounds
+    assert (counts <= small).any() and ((counts > small) & (counts <= middle)).any() and counts.max() == full, np.sort(counts)
+    for name in ("contact_count", "ucontact_count", "row_count", "env_status"):
         assert np.array_equal(world.download(name), oracle.download(name)), name
     assert not world.download("env_status").any()
+    # an environment whose residual sits at the tolerance may stop a sweep earlier or later under other rounding
+    assert np.mean(world.download("vbd_velocity_sweep_count") != oracle.download("vbd_velocity_sweep_count")) <= 0.03
     for name in ("qdot", "link_velocity", "base_pose"):
         error = per_env_error(world.download(name), oracle.download(name), E)
         assert error.max() <= 2e-4, (name, float(error.max()), int(counts[error.argmax()]))       # two steps
-    # spheres in a row share a load in no unique way: the multipliers are compared through what they add up to
+    # shapes in a row share a load in no unique way: the multipliers are compared through what they add up to
     oracle.op("readout_contact_wrench")
     error = per_env_error(world.download("link_contact_wrench"), oracle.download("link_contact_wrench"), E)
     assert np.abs(oracle.download("link_contact_wrench")).max() > 10.0 and error.max() <= 1e-3, float(error.max())
