@@ -285,6 +285,80 @@ __device__ __forceinline__ bool factor_rows(uint32_t lane, float (&row)[N], floa
     return valid;
 }
 
+// Past 32 coordinates the reference's tile is "wide" (TileSpan > 1, :71-73) and factors H = U U^T from the last
+// coordinate down, "so a tree's leaves go first" (FactorTileColumns :209-252); its substitutions run up the columns of
+// U and then down its rows (SolveWideTileBlock :1866-1895).  Which end the elimination starts from decides whether a
+// long chain's block can be factored in single precision at all, so the order is part of the path's arithmetic.
+template <int N>
+constexpr bool kLeavesFirst = N > 32;
+
+// FactorTileColumns on register rows: lane i holds row i of the symmetric matrix; on return its entries k >= i are
+// row i of U.  Column k leaves exact zeros in the rows of other branches of the tree, and the update of a column by
+// an exact zero changes nothing: such columns are skipped four at a time.
+template <int N>
+__device__ __forceinline__ bool factor_rows_up(uint32_t lane, float (&row)[N], float* inverse_out) {
+    lane = local_lane(lane);
+    bool valid = true;
+    float inverse = 0.0f;
+    float pivot = lane_value(row[N - 1], N - 1);
+    valid = pivot > 0.0f && pivot <= FLT_MAX;
+    float root = sqrtf(valid ? pivot : 1.0f);
+    float scale = 1.0f / root;
+#pragma unroll
+    for (int k = N - 1; k >= 0; --k) {
+        row[k] = lane == uint32_t(k) ? root : row[k] * scale;
+        if (lane == uint32_t(k)) inverse = scale;
+        const uint64_t reach = __ballot(lane < uint32_t(k) && row[k] != 0.0f);
+        if (k >= 1) {
+            row[k - 1] = fmaf(-row[k], lane_value(row[k], k - 1), row[k - 1]);
+            pivot = lane_value(row[k - 1], k - 1);
+            valid = valid && pivot > 0.0f && pivot <= FLT_MAX;
+            root = sqrtf(valid ? pivot : 1.0f);
+            scale = 1.0f / root;
+        }
+#pragma unroll
+        for (int q = (k - 2) / 4; q >= 0 && k >= 2; --q) {
+            if (((reach >> (4 * q)) & 0xFull) == 0ull) continue;
+            float u[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) u[t] = 4 * q + t <= k - 2 ? lane_value(row[k], 4 * q + t) : 0.0f;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                if (4 * q + t <= k - 2) row[4 * q + t] = fmaf(-row[k], u[t], row[4 * q + t]);
+        }
+    }
+    *inverse_out = inverse;
+    return valid;
+}
+
+// SolveWideTileBlock: U w = g with lane's own row (entries right of the diagonal), then U^T d = w with the columns,
+// read from the factor in LDS eight at a time.
+template <int N>
+__device__ __forceinline__ float substitute_up(uint32_t lane, const float (&row)[N], const float* factor, float inverse, float g) {
+    lane = local_lane(lane);
+    float r = g;
+#pragma unroll
+    for (int j = N - 1; j >= 0; --j) {
+        const float y = lane_value(r * inverse, j);
+        r = lane < uint32_t(j) ? fmaf(-row[j], y, r) : r;
+    }
+    r *= inverse;
+    const float* column = factor + (lane < uint32_t(N) ? lane : 0u);
+#pragma unroll
+    for (int j0 = 0; j0 < N; j0 += 8) {
+        float u[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) u[t] = j0 + t < N ? column[(j0 + t) * (N + 1)] : 0.0f;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            if (j0 + t >= N) continue;
+            const float x = lane_value(r * inverse, j0 + t);
+            r = lane > uint32_t(j0 + t) && lane < uint32_t(N) ? fmaf(-u[t], x, r) : r;
+        }
+    }
+    return r * inverse;
+}
+
 // SolveTileBlock (:1647-1666): forward with the factor's rows, backward with its columns (col[j] = L_j,lane).
 template <int N>
 __device__ __forceinline__ float substitute(uint32_t lane, const float (&row)[N], const float (&col)[N], float inverse, float g) {
@@ -333,7 +407,7 @@ template <int N>
 __device__ __forceinline__ bool cholesky_solve(const Tile& c, float (&hrow)[N], float g, float* d_out) {
     if (!c.factor_current) {   // otherwise the Hessian is the one factored last: its factor is still in hfac
         float inverse = 0.0f;
-        const bool valid = factor_rows<N>(c.lane, hrow, &inverse);
+        const bool valid = kLeavesFirst<N> ? factor_rows_up<N>(c.lane, hrow, &inverse) : factor_rows<N>(c.lane, hrow, &inverse);
         if (!valid) return false;
         store_rows<N>(c.hfac, c.lane, hrow);
         __syncthreads();
@@ -343,10 +417,14 @@ __device__ __forceinline__ bool cholesky_solve(const Tile& c, float (&hrow)[N], 
     // 1 / its diagonal entry, the same division)
     const uint32_t row = local_lane(c.lane);
     const float inverse = row < uint32_t(N) ? 1.0f / c.hfac[row * (N + 1) + row] : 0.0f;
-    float col[N];
     load_rows<N>(c.hfac, c.lane, hrow);
-    load_columns<N>(c.hfac, c.lane, col);
-    *d_out = substitute<N>(c.lane, hrow, col, inverse, c.lane < c.n ? g : 0.0f);
+    if constexpr (kLeavesFirst<N>) {
+        *d_out = substitute_up<N>(c.lane, hrow, c.hfac, inverse, c.lane < c.n ? g : 0.0f);
+    } else {
+        float col[N];
+        load_columns<N>(c.hfac, c.lane, col);
+        *d_out = substitute<N>(c.lane, hrow, col, inverse, c.lane < c.n ? g : 0.0f);
+    }
     __syncthreads();
     return true;
 }
@@ -359,7 +437,7 @@ __device__ __forceinline__ bool factor_mass(Tile& c, const float (&mrow)[N]) {
 #pragma unroll
     for (int k = 0; k < N; ++k) row[k] = mrow[k];
     float inverse = 0.0f;
-    const bool valid = factor_rows<N>(c.lane, row, &inverse);
+    const bool valid = kLeavesFirst<N> ? factor_rows_up<N>(c.lane, row, &inverse) : factor_rows<N>(c.lane, row, &inverse);
     c.mass_inverse = inverse;
     store_rows<N>(c.mfac, c.lane, row);
     __syncthreads();
@@ -367,8 +445,10 @@ __device__ __forceinline__ bool factor_mass(Tile& c, const float (&mrow)[N]) {
 }
 template <int N>
 __device__ __forceinline__ float solve_tile_mass(const Tile& c, float force) {
-    float row[N], col[N];
+    float row[N];
     load_rows<N>(c.mfac, c.lane, row);
+    if constexpr (kLeavesFirst<N>) return substitute_up<N>(c.lane, row, c.mfac, c.mass_inverse, c.lane < c.n ? force : 0.0f);
+    float col[N];
     load_columns<N>(c.mfac, c.lane, col);
     return substitute<N>(c.lane, row, col, c.mass_inverse, c.lane < c.n ? force : 0.0f);
 }
@@ -609,7 +689,7 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
 
 enum Failure : uint32_t { kFailNone = 0u, kFailEquation, kFailFactor, kFailDirection, kFailCandidate };
 
-// TileNewtonDirection (:1935-1992), narrow form.  The reference re-assembles the block after the mass-normalised
+// TileNewtonDirection (:1935-1992).  The reference re-assembles the block after the mass-normalised
 // convergence test because its mass factor overwrites the Hessian storage; here the two live apart and the
 // assembled row, force and inertia (which the second assembly would reproduce bit for bit) are simply kept.
 template <int N>

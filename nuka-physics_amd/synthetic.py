@@ -167,22 +167,62 @@ def humanoid(env_count=4096, index=3):
     return Config(index, "humanoid", t, 1.0 / 200.0, 8, env_count, sample, nominal, True)
 
 
+ROPE_RADIUS, ROPE_LINK, ROPE_REST_DEPTH = 0.01, 0.05, 5.0e-4
+# Sixty-four links of 50 to 200 g, each pressed on the plane by a penalty of a hundred times its own inverse
+# response, give a Newton block whose condition number (about 1e9) is past what a single-precision Cholesky can
+# factor from either end of the chain.  A reflected rotor inertia on every joint, the one term that adds to the whole
+# diagonal of the mass matrix, brings it to about 1e5.
+ROPE_ARMATURE = 0.01
+
+
+def _rope_lie(draw):
+    """Joint angles of a rope that lies on the plane, from one N(0, 0.3) draw per joint.
+
+    Joints alternate pitch (y, even links) and yaw (z, odd links).  A yaw joint takes its draw as its angle.  Sixty-four
+    independent pitch angles of that size would carry the rope metres above and below the plane (the height is the
+    double sum of the pitch angles), where no contact problem is posed; a pitch joint therefore takes the angle that
+    brings the joint two links on back to the rope's rest height plus its own draw read in millimetres, so that every
+    sphere rests on the plane within a millimetre of the nominal penetration and each environment has its own lie.
+    """
+    E = draw.shape[0]
+    q = np.zeros((E, 64))
+    rot = np.tile(np.eye(3), (E, 1, 1))            # world rotation of the parent link
+    origin = np.zeros((E, 3))                      # world position of the current joint, relative to the anchor
+    for i in range(0, 64, 2):
+        psi = draw[:, i + 1]
+        a, b, c = rot[:, 2, 0], rot[:, 2, 1], rot[:, 2, 2]
+        target = 1.0e-3 * draw[:, i] - origin[:, 2]
+        k = (target / ROPE_LINK - np.sin(psi) * b) / (1.0 + np.cos(psi))
+        theta = np.arctan2(a, c) - np.arcsin(np.clip(k / np.hypot(a, c), -1.0, 1.0))
+        q[:, i], q[:, i + 1] = theta, psi
+        ct, st, cp, sp = np.cos(theta), np.sin(theta), np.cos(psi), np.sin(psi)
+        zero, one = np.zeros(E), np.ones(E)
+        ry = np.stack([ct, zero, st, zero, one, zero, -st, zero, ct], 1).reshape(E, 3, 3)
+        rz = np.stack([cp, -sp, zero, sp, cp, zero, zero, zero, one], 1).reshape(E, 3, 3)
+        rot = rot @ ry
+        origin = origin + ROPE_LINK * rot[:, :, 0]
+        rot = rot @ rz
+        origin = origin + ROPE_LINK * rot[:, :, 0]
+    return q
+
+
 def rope(env_count=8192):
     g = _rng(5, 0)
     t = Template()
-    t.add_link(JOINT_FIXED, None, local_pos=(0, 0, 0.012), mass=1.0)
+    t.add_link(JOINT_FIXED, None, local_pos=(0, 0, ROPE_RADIUS - ROPE_REST_DEPTH), mass=1.0)
     spheres = []
     for i in range(64):
         m = g.uniform(0.05, 0.2)
-        link = t.add_link(JOINT_REVOLUTE, i, axis=Y if i % 2 == 0 else Z, local_pos=(0.05 if i else 0.0, 0, 0), mass=m,
-                          diag_inertia=(m * 2.5e-5, m * 2.3e-4, m * 2.3e-4), com=(0.025, 0, 0))
-        spheres.append((link, (0.025, 0, 0), 0.01))
+        link = t.add_link(JOINT_REVOLUTE, i, axis=Y if i % 2 == 0 else Z, local_pos=(ROPE_LINK if i else 0.0, 0, 0),
+                          mass=m, diag_inertia=(m * 2.5e-5, m * 2.3e-4, m * 2.3e-4), com=(0.5 * ROPE_LINK, 0, 0),
+                          armature=ROPE_ARMATURE)
+        spheres.append((link, (0.5 * ROPE_LINK, 0, 0), ROPE_RADIUS))
     _add_collidable_rows(t, spheres, 0.5)
     nl = t.link_count
 
     def sample(E):
         q = np.zeros((E, nl), np.float32)
-        q[:, 1:] = _rng(5, 1).normal(0.0, 0.3, size=(E, 64))
+        q[:, 1:] = _rope_lie(_rng(5, 1).normal(0.0, 0.3, size=(E, 64)))
         base = np.tile(np.array([0, 0, 0, 1, 0, 0, 0], np.float32), (E, 1))
         return dict(q=q, qdot=np.zeros((E, nl), np.float32), tau=np.zeros((E, nl), np.float32), base_pose=base,
                     root_twist=np.zeros((E, 6), np.float32))

@@ -7,6 +7,8 @@
  * order; the compensated TileSum arithmetic, fmaf uses and branch structure are kept.  Free rigid
  * bodies (6x6 blocks), mimic couplings and elliptic (MuJoCo-law) cones are outside this restatement.
  */
+#include <stdio.h>
+
 #include "nko_internal.h"
 
 typedef struct { float value, error; } tile_sum;   /* block_descent_tile.cuh:15-31 */
@@ -310,6 +312,8 @@ static int cholesky_solve(float h[NKO_MAX_DOF][NKO_MAX_DOF + 1], uint32_t n, con
             column[i] = value;
             if (i == k) pivot = value;
         }
+        if (valid && !(pivot > 0.0f && pivot <= FLT_MAX) && getenv("NKO_TRACE_FAILURES") != NULL)
+            fprintf(stderr, "nko: pivot %u of %u is %g (diagonal entry %g)\n", k, n, pivot, h[k][k]);
         valid = valid && pivot > 0.0f && pivot <= FLT_MAX;
         const float root = sqrtf(valid ? pivot : 1.0f);
         const float scale = 1.0f / root;
@@ -332,6 +336,78 @@ static int cholesky_solve(float h[NKO_MAX_DOF][NKO_MAX_DOF + 1], uint32_t n, con
     }
     for (uint32_t i = 0u; i < n; ++i) d[i] = r[i];
     return 1;
+}
+
+/* Past a warp of coordinates (TileSpan > 1: more than 32) the reference factors H = U U^T from the last coordinate
+ * down, "so a tree's leaves go first".  FactorTileColumns (:212-252): left-looking; the dot of row i with the pivot row
+ * over the finished columns k+2.. is split over four partial sums in runs of eight columns, the first of which takes
+ * the still unscaled column k+1 last, and the four are added pairwise.  SolveWideTileBlock (:1866-1895): U w = g up
+ * the columns, then U^T d = w down the rows.  Only the upper triangle of h is read. */
+static int cholesky_solve_wide(float h[NKO_MAX_DOF][NKO_MAX_DOF + 1], uint32_t n, const float* g, float* d) {
+    float inverse[NKO_MAX_DOF], raw[2][NKO_MAX_DOF];
+    int valid = 1;
+    for (uint32_t kk = n; kk > 0u; --kk) {
+        const uint32_t k = kk - 1u;
+        const float* last = raw[(k + 1u) % 2u];
+        float* next = raw[k % 2u];
+        const int scaled = k + 1u < n;
+        const float scale = scaled ? inverse[k + 1u] : 0.0f;
+        float pivot = 0.0f;
+        for (uint32_t i = 0u; i <= k; ++i) {
+            float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (uint32_t p = 0u; p < 4u; ++p) {
+                for (uint32_t m = 0u; m < 16u; ++m) {
+                    const uint32_t j = k + 2u + 8u * p + m % 8u + 32u * (m / 8u);
+                    if (j < n) part[p] = fmaf(h[i][j], h[k][j], part[p]);
+                }
+                if (p == 0u && scaled) part[p] = fmaf(last[i] * scale, last[k] * scale, part[p]);
+            }
+            const float sum = (part[0] + part[1]) + (part[2] + part[3]);
+            if (i < k) next[i] = h[i][k] - sum;
+            else pivot = h[i][k] - sum;
+        }
+        if (scaled) for (uint32_t i = 0u; i <= k; ++i) h[i][k + 1u] = last[i] * scale;
+        /* a failed pivot leaves every later root at one */
+        if (valid && !(pivot > 0.0f && pivot <= FLT_MAX) && getenv("NKO_TRACE_FAILURES") != NULL)
+            fprintf(stderr, "nko: pivot %u of %u is %g (diagonal entry %g)\n", k, n, pivot, h[k][k]);
+        valid = valid && pivot > 0.0f && pivot <= FLT_MAX;
+        const float root = sqrtf(valid ? pivot : 1.0f);
+        h[k][k] = root;
+        inverse[k] = 1.0f / root;
+    }
+    if (!valid) return 0;
+    float r[NKO_MAX_DOF];
+    for (uint32_t i = 0u; i < n; ++i) r[i] = g[i];
+    for (uint32_t jj = n; jj > 0u; --jj) {
+        const uint32_t j = jj - 1u;
+        const float y = r[j] * inverse[j];
+        r[j] = y;
+        for (uint32_t i = 0u; i < j; ++i) r[i] = fmaf(-h[i][j], y, r[i]);
+    }
+    for (uint32_t j = 0u; j < n; ++j) {
+        const float x = r[j] * inverse[j];
+        r[j] = x;
+        for (uint32_t i = j + 1u; i < n; ++i) r[i] = fmaf(-h[j][i], x, r[i]);
+    }
+    for (uint32_t i = 0u; i < n; ++i) d[i] = r[i];
+    return 1;
+}
+
+/* the reference's tile width decides the route: TileSpan (:71-73) over 32-lane warps */
+static int wide_tile(uint32_t n) { return n > 32u; }
+
+/* The block factorisation by itself, for unit pins: h is n x n row-major; on return factor (n x n) holds the
+ * triangular factor the route of this width builds (lower L with h = L L^T up to 32 coordinates, upper U with
+ * h = U U^T past them) and d the solution of h d = g.  Returns 0 when a pivot fails. */
+int nko_tile_cholesky_solve(const float* h_in, uint32_t n, const float* g, float* factor, float* d) {
+    static _Thread_local float h[NKO_MAX_DOF][NKO_MAX_DOF + 1];
+    if (n == 0u || n > NKO_MAX_DOF) return 0;
+    for (uint32_t i = 0u; i < n; ++i) for (uint32_t j = 0u; j < n; ++j) h[i][j] = h_in[(size_t)i * n + j];
+    const int valid = wide_tile(n) ? cholesky_solve_wide(h, n, g, d) : cholesky_solve(h, n, g, d);
+    for (uint32_t i = 0u; i < n; ++i)
+        for (uint32_t j = 0u; j < n; ++j)
+            factor[(size_t)i * n + j] = (wide_tile(n) ? j >= i : j <= i) ? h[i][j] : 0.0f;
+    return valid;
 }
 
 /* AssembleTileBlock (:1507-1618) */
@@ -388,7 +464,8 @@ static int assemble_block(tile* c, const float* u, const float* free_v, float h[
                     scale[i] += fabsf(j0) * noise.x;
                     if (t->axes == 1u) {
                         const float a0 = j0 * cv[0];
-                        for (uint32_t kk = 0u; kk < n; ++kk) h[i][kk] += a0 * j0r[kk];
+                        if (wide_tile(n)) for (uint32_t kk = i; kk < n; ++kk) h[i][kk] = fmaf(a0, j0r[kk], h[i][kk]);
+                        else for (uint32_t kk = 0u; kk < n; ++kk) h[i][kk] += a0 * j0r[kk];
                         continue;
                     }
                     const float j1 = j1r[i], j2 = j2r[i];
@@ -398,11 +475,17 @@ static int assemble_block(tile* c, const float* u, const float* free_v, float h[
                     const float a0 = (j0 * cv[0] + j1 * cv[3]) + j2 * cv[4];
                     const float a1 = (j1 * cv[1] + j2 * cv[5]) + j0 * cv[3];
                     const float a2 = (j2 * cv[2] + j1 * cv[5]) + j0 * cv[4];
+                    if (wide_tile(n)) {   /* AssembleTileChunk (:170-190): the upper triangle, one fused product per staged row */
+                        for (uint32_t kk = i; kk < n; ++kk) h[i][kk] = fmaf(a2, j2r[kk], fmaf(a1, j1r[kk], fmaf(a0, j0r[kk], h[i][kk])));
+                        continue;
+                    }
                     for (uint32_t kk = 0u; kk < n; ++kk) h[i][kk] += a0 * j0r[kk] + a1 * j1r[kk] + a2 * j2r[kk];
                 }
             }
     }
     int finite = 1, settled = 1;
+    /* ScaleTileRows (:194-207) reads the wide block's entry (i, k) from the upper triangle */
+    if (wide_tile(n)) for (uint32_t i = 0u; i < n; ++i) for (uint32_t k = 0u; k < i; ++k) h[i][k] = h[k][i];
     for (uint32_t i = 0u; i < n; ++i) {
         h[i][i] += diagonal[i];
         force[i] = g[i].value + g[i].error;
@@ -424,12 +507,13 @@ static int assemble_block(tile* c, const float* u, const float* free_v, float h[
 static int solve_tile_mass(tile* c, const float* force, float* d) {
     float m[NKO_MAX_DOF][NKO_MAX_DOF + 1];
     for (uint32_t i = 0u; i < c->n; ++i) for (uint32_t j = 0u; j < c->n; ++j) m[i][j] = c->mass[i][j];
-    return cholesky_solve(m, c->n, force, d);
+    return wide_tile(c->n) ? cholesky_solve_wide(m, c->n, force, d) : cholesky_solve(m, c->n, force, d);
 }
 
 enum { FAIL_NONE = 0, FAIL_EQUATION, FAIL_FACTOR, FAIL_DIRECTION, FAIL_CANDIDATE };
 
-/* TileNewtonDirection (:1935-1992), narrow form */
+/* TileNewtonDirection (:1935-1992): the narrow form up to 32 coordinates, the wide form (its second assembly
+ * reproduces the first bit for bit and is not repeated) past them */
 static int newton_direction(tile* c, const float* u, const float* free_v, float* force, float* inertia, float* d, int* converged) {
     float h[NKO_MAX_DOF][NKO_MAX_DOF + 1];
     if (!assemble_block(c, u, free_v, h, force, inertia, converged)) return FAIL_EQUATION;
@@ -440,7 +524,7 @@ static int newton_direction(tile* c, const float* u, const float* free_v, float*
         *converged = stationary;
     }
     if (*converged) return FAIL_NONE;
-    if (!cholesky_solve(h, c->n, force, d)) return FAIL_FACTOR;
+    if (!(wide_tile(c->n) ? cholesky_solve_wide(h, c->n, force, d) : cholesky_solve(h, c->n, force, d))) return FAIL_FACTOR;
     return FAIL_NONE;
 }
 
@@ -600,6 +684,8 @@ static void descend_block(tile* c, float* velocity, const float* free_in) {
         t->residual = v3_make(t->residual.x - t->move.x, t->residual.y - t->move.y, t->residual.z - t->move.z);
     }
     if (failure != FAIL_NONE) { c->failed = 1; c->w->env_status[c->env] |= NKO_STATUS_SOLVER_FAILURE; }
+    if (failure != FAIL_NONE && getenv("NKO_TRACE_FAILURES") != NULL)
+        fprintf(stderr, "nko: env %u sweep %u block descent failure kind %d\n", c->env, c->iteration, failure);
     float moved = failure == FAIL_NONE ? 0.0f : FLT_MAX;
     for (uint32_t i = 0u; i < n; ++i) moved = fmaxf(moved, u2f(residual_bits(u[i] - start[i])));
     c->momentum = fmaxf(c->momentum, moved);
@@ -639,6 +725,8 @@ static void measure_primal(tile* c, float* velocity, const float* free_v, const 
     if (failure == FAIL_NONE && !solve_tile_mass(c, force, direction)) failure = FAIL_FACTOR;
     float residual = failure == FAIL_NONE ? 0.0f : FLT_MAX;
     if (failure != FAIL_NONE) c->w->env_status[c->env] |= NKO_STATUS_SOLVER_FAILURE;
+    if (failure != FAIL_NONE && getenv("NKO_TRACE_FAILURES") != NULL)
+        fprintf(stderr, "nko: env %u sweep %u primal measure failure kind %d\n", c->env, c->iteration, failure);
     for (uint32_t i = 0u; i < n && failure == FAIL_NONE; ++i)
         residual = fmaxf(residual, isfinite(direction[i]) ? fabsf(direction[i]) : FLT_MAX);
     c->residual = fmaxf(c->residual, residual);
@@ -821,6 +909,8 @@ void nko_env_solve(nko_world* w, uint32_t env) {
         float rho = response > 0.0f ? fminf(cap, coupled) : 0.0f;
         if (!(response == 0.0f || (response > 0.0f && rho > 0.0f && rho <= FLT_MAX))) {
             w->env_status[env] |= NKO_STATUS_SOLVER_FAILURE;
+            if (getenv("NKO_TRACE_FAILURES") != NULL)
+                fprintf(stderr, "nko: env %u head %u inertial response %g (shares %g %g) rejected\n", env, h, response, shares[0], shares[1]);
             rho = NAN;
         }
         w->solver_penalty[slot] = rho;

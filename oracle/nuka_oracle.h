@@ -161,6 +161,9 @@ void nko_tangent_impulse(const float dual[3], float rho, const float residual[3]
 void nko_relax_contact_impulse(const float dual[3], const float next[3], float last_step[3], float* last_weight,
                                float last_point[3], float out[3]);
 float nko_cone_argument(float dual, float rho, float mu, float residual);
+/* FactorTileBlock + SolveTileBlock (block_descent_tile.cuh:1622-1666) up to 32 coordinates, FactorTileColumns +
+ * SolveWideTileBlock (:209-252, 1866-1895) past them; see nko_solver.c */
+int nko_tile_cholesky_solve(const float* h, uint32_t n, const float* g, float* factor, float* d);
 /* The compliant (MuJoCo-law) row terms and the elliptic cone of the reference's row math.  No device counterpart: the
  * product builds rows of the native law only.  Held so the reference's known answers for them are checked here too. */
 void nko_compliant_row_terms(const float solref[2], const float solimp[5], float pos_imp, float pos_aref, float vel, float invweight,

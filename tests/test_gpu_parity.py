@@ -34,9 +34,23 @@ def both(oracle, world, name):
 
 
 def close(world, oracle, name, tol=TOL):
-    error = relative_error(world.download(name), oracle.download(name))
-    assert error <= tol, f"{name}: relative error {error:.3e} > {tol:.1e}"
-    return error
+    """Norm-wise relative error of a field, environment by environment: no environment may hide behind another's
+    larger values."""
+    E = world.env_count
+    got, expect = world.download(name), oracle.download(name)
+    if got.size == 0 and expect.size == 0:
+        return 0.0
+    errors = per_env_error(got, expect, E)
+    worst = float(errors.max()) if errors.size else 0.0
+    assert worst <= tol, f"{name}: {int((errors > tol).sum())} of {E} environments above {tol:.1e}, worst {worst:.3e}"
+    return worst
+
+
+def close_masked(got, expect, mask, E, tol, what):
+    """Per-environment relative error over the entries `mask` selects (leading axis = environment)."""
+    got, expect = np.where(mask, got, 0.0).reshape(E, -1), np.where(mask, expect, 0.0).reshape(E, -1)
+    errors = per_env_error(got, expect, E)
+    assert errors.max() <= tol, f"{what}: {int((errors > tol).sum())} of {E} environments above {tol:.1e}, worst {errors.max():.3e}"
 
 
 def equal(world, oracle, name):
@@ -69,14 +83,91 @@ def oracle_sensitivity(oracle_py, index, E, fields, steps=1, **kw):
     return {f: relative_error(outputs[1][f], outputs[0][f]) for f in fields}
 
 
-@pytest.mark.parametrize("index,E", [(1, 64), (2, 256), (3, 256)])
-def test_every_op_matches_the_oracle(oracle_py, device, index, E):
-    cfg, oracle, world, _ = make_pair(oracle_py, device, index, E)
+def velocity_scale(world, oracle, E):
+    """Per-environment size of the velocities the solve works with: the free velocity it starts from, or the result.
+    A body that the contacts bring to rest ends near zero; its error is measured against what the solve removed."""
+    free = np.abs(oracle.download("qdot_flat")).reshape(E, -1).max(1)
+    return np.maximum(free, 1e-6)
+
+
+def scaled_errors(got, expect, scale, E):
+    return np.abs(np.asarray(got, np.float64).reshape(E, -1) - np.asarray(expect, np.float64).reshape(E, -1)).max(1) / scale
+
+
+def one_ulp_sensitivity(oracle_py, template, desc, state, threads=8):
+    """How far the oracle's own outputs move when q, qdot and tau move by one ulp: the worst environment's relative
+    change of the joint accelerations, of the generalized contact impulse and of the post-solve velocity (against the
+    free velocity), and the batch-wide relative change of lambda.  An ill-conditioned mass matrix or Newton block
+    shows here, and no other fp32 evaluation of the same formulas can be expected to agree more closely than this."""
+    E = desc.env_count
+    runs = []
+    for perturb in (False, True):
+        w = oracle_py.OracleWorld(template, desc, threads=threads)
+        moved = {k: v.copy() for k, v in state.items()}
+        if perturb:
+            g = np.random.default_rng(99)
+            for key in ("q", "qdot", "tau"):
+                toward = moved[key] + g.choice([-1.0, 1.0], moved[key].shape).astype(np.float32)
+                moved[key] = np.nextafter(moved[key], toward).astype(np.float32)
+        w.set_state(moved)
+        for name in UPSTREAM if w.rows_per_env else UPSTREAM[:2]:
+            w.op(*ORACLE_OPS[name])
+        out = {"qdd": w.download("articulation_qdd").reshape(E, -1).astype(np.float64)}
+        if w.rows_per_env:
+            out["free"] = np.abs(w.download("qdot_flat")).reshape(E, -1).max(1)
+            w.op("block_descent_solve")
+            out["impulse"] = generalized_impulse(w, E)
+            out["velocity"] = w.download("qdot_flat").reshape(E, -1).astype(np.float64)
+            out["lambda"] = w.download("lambda")
+        w.op("integrate_position")       # with the push-out of the position pass, a block descent of its own
+        out["q"] = w.download("q").reshape(E, -1).astype(np.float64)
+        runs.append(out)
+        w.close()
+    a, b = runs
+    sens = {"qdd": float((np.abs(b["qdd"] - a["qdd"]).max(1) / np.maximum(np.abs(a["qdd"]).max(1), 1e-6)).max()),
+            "q": float((np.abs(b["q"] - a["q"]).max(1) / np.maximum(np.abs(a["q"]).max(1), 1e-6)).max())}
+    if "impulse" in a:
+        sens["impulse"] = float((np.abs(b["impulse"] - a["impulse"]).max(1) / np.maximum(np.abs(a["impulse"]).max(1), 1e-9)).max())
+        sens["velocity"] = float((np.abs(b["velocity"] - a["velocity"]).max(1) / np.maximum(a["free"], 1e-6)).max())
+        sens["lambda"] = relative_error(b["lambda"], a["lambda"])
+    return sens
+
+
+def bar(sens, key):
+    """The stated tolerance, or four times the oracle's own one-ulp sensitivity where that is larger."""
+    return max(TOL, 4.0 * sens.get(key, 0.0)) if sens else TOL
+
+
+def acceleration_residual(w, state, E):
+    """Backward error of the joint accelerations: |M qdd + bias - tau| against |M||qdd| + |bias| + |tau|, per environment."""
+    n = w.dof
+    M = w.download("m").reshape(E, n, n).astype(np.float64)
+    qdd = w.download("articulation_qdd").reshape(E, -1)[:, :n].astype(np.float64)
+    bias = w.download("articulation_bias").reshape(E, -1)[:, :n].astype(np.float64)
+    nl = state["tau"].shape[1]
+    tau = np.zeros((E, n))
+    tau[:, n - (nl - 1):] = state["tau"][:, 1:]          # joint torques follow the root's coordinates
+    residual = np.abs(np.einsum("eij,ej->ei", M, qdd) + bias - tau).max(1)
+    scale = (np.einsum("eij,ej->ei", np.abs(M), np.abs(qdd)) + np.abs(bias) + np.abs(tau)).max(1)
+    return residual / np.maximum(scale, 1e-30)
+
+
+def compare_ops(oracle, world, E, sens=None, state=None):
+    """Every op of one step on both sides, outputs compared after each.  Returns the per-environment errors of the
+    solve's outputs (generalized impulse, velocity) for the caller's report."""
     both(oracle, world, "FkWorldPoses")
     close(world, oracle, "link_pose")
     both(oracle, world, "ArticulationDynamics")
-    for name in ("m", "m_factor", "articulation_bias", "articulation_qdd", "qddot", "qdot", "link_acceleration"):
+    for name in ("m", "articulation_bias"):
         close(world, oracle, name)
+    # the accelerations solve M qdd = tau - bias: forward to the bar the oracle's own conditioning allows, and
+    # backward (the residual of the device's own solution) to 1e-5 whatever the conditioning
+    for name in ("m_factor", "articulation_qdd", "qddot", "qdot", "link_acceleration"):
+        close(world, oracle, name, tol=bar(sens, "qdd"))
+    if state is not None:
+        residual = acceleration_residual(world, state, E)
+        assert residual.max() <= 1e-5, f"M qdd + bias - tau: worst environment {residual.max():.2e}"
+    report = {}
     if world.rows_per_env:
         R, S = world.rows_per_env, world.info.contact_slots_per_env
         for name in UPSTREAM[2:]:
@@ -92,7 +183,7 @@ def test_every_op_matches_the_oracle(oracle_py, device, index, E):
         mask = np.arange(4)[None, None, :] < points[:, :, None]
         for name, width in (("ucontact_point", 3), ("ucontact_normal", 3), ("ucontact_depth", 1)):
             g, o = world.download(name).reshape(E, S, 4, width), oracle.download(name).reshape(E, S, 4, width)
-            assert relative_error(g[mask], o[mask]) <= TOL, name
+            close_masked(g, o, mask[..., None], E, TOL, name)
         for name in ("ucontact_a", "ucontact_b"):
             g, o = world.download(name).reshape(E, S, 4), oracle.download(name).reshape(E, S, 4)
             assert np.array_equal(g[mask], o[mask]), name
@@ -103,39 +194,62 @@ def test_every_op_matches_the_oracle(oracle_py, device, index, E):
         for word in (1, 2, 3, 10, 11, 18, 19):                             # group, env, side kinds and indices
             assert np.array_equal(gw[:, :, word][active], ow[:, :, word][active]), f"row word {word}"
         for lo, hi in ((4, 10), (12, 18), (20, 26)):                       # rhs..mu, both sides' directions
-            assert relative_error(grow[:, :, lo:hi][active], orow[:, :, lo:hi][active]) <= TOL
+            close_masked(grow[:, :, lo:hi], orow[:, :, lo:hi], active[..., None], E, TOL, f"row words {lo}..{hi}")
         for name in ("chain_jacobian", "chain_jacobian_b"):
             g, o = world.download(name).reshape(E, R, -1), oracle.download(name).reshape(E, R, -1)
-            assert relative_error(g[active], o[active]) <= TOL, name
+            close_masked(g, o, active[..., None], E, TOL, name)
         g, o = world.download("row_penetration").reshape(E, R), oracle.download("row_penetration").reshape(E, R)
-        assert relative_error(g[active], o[active]) <= TOL
-        close(world, oracle, "qdot_flat")
+        close_masked(g, o, active, E, TOL, "row_penetration")
+        close(world, oracle, "qdot_flat", tol=bar(sens, "qdd"))
+        scale = velocity_scale(world, oracle, E)
         both(oracle, world, "BlockDescentSolve")
         assert np.array_equal(world.download("env_status"), oracle.download("env_status"))
-        assert relative_error(generalized_impulse(world, E), generalized_impulse(oracle, E)) <= TOL
-        close(world, oracle, "qdot")
-        close(world, oracle, "link_velocity")
+        impulse_o = generalized_impulse(oracle, E)
+        impulse = scaled_errors(generalized_impulse(world, E), impulse_o, np.maximum(np.abs(impulse_o).max(1), 1e-9), E)
+        velocity = scaled_errors(world.download("qdot_flat"), oracle.download("qdot_flat"), scale, E)
+        report = {"impulse": impulse, "velocity": velocity}
+        for what, errors in report.items():
+            assert errors.max() <= bar(sens, what), \
+                f"{what} after the solve: {int((errors > bar(sens, what)).sum())} of {E} environments above {bar(sens, what):.1e}, worst {errors.max():.3e}"
     for name in ("IntegratePosition", "FkWorldPoses", "FkLinkVelocities"):
         both(oracle, world, name)
-    for name in ("q", "base_pose", "link_pose", "link_velocity"):
-        close(world, oracle, name)
+    for name in ("q", "base_pose", "link_pose"):
+        close(world, oracle, name, tol=bar(sens, "q"))
+    return report
+
+
+@pytest.mark.parametrize("index,E", [(1, 64), (2, 256), (3, 256)])
+def test_every_op_matches_the_oracle(oracle_py, device, index, E):
+    cfg, oracle, world, state = make_pair(oracle_py, device, index, E)
+    desc = nk.abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters)
+    sens = one_ulp_sensitivity(oracle_py, cfg.template, desc, state)
+    print(cfg.name, "one-ulp sensitivity of the oracle:", {k: f"{v:.2e}" for k, v in sens.items()})
+    report = compare_ops(oracle, world, E, sens, state)
+    print(cfg.name, "worst environment:", {k: f"{v.max():.2e}" for k, v in report.items()},
+          "environments above 1e-4:", {k: int((v > TOL).sum()) for k, v in report.items()})
+    close(world, oracle, "link_velocity", tol=bar(sens, "velocity"))
     world.close()
     oracle.close()
 
 
 @pytest.mark.parametrize("index,E", [(1, 64), (2, 512), (3, 512)])
 def test_whole_step_matches_the_oracle(oracle_py, device, index, E):
-    cfg, oracle, world, _ = make_pair(oracle_py, device, index, E)
+    cfg, oracle, world, state = make_pair(oracle_py, device, index, E)
+    sens = one_ulp_sensitivity(oracle_py, cfg.template, nk.abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters), state)
     world.step()
     world.synchronize()
     oracle.step()
-    errors = {n: close(world, oracle, n) for n in ("articulation_qdd", "link_pose", "q", "qdot", "link_velocity", "base_pose", "body_pose")}
-    print(cfg.name, {k: f"{v:.2e}" for k, v in errors.items()})
+    errors = {n: close(world, oracle, n) for n in ("articulation_qdd", "link_pose", "q", "base_pose", "body_pose")}
+    errors.update({n: close(world, oracle, n, tol=bar(sens, "velocity")) for n in ("qdot", "link_velocity")})
+    print(cfg.name, "worst environment:", {k: f"{v:.2e}" for k, v in errors.items()})
     if world.rows_per_env:
-        R = world.rows_per_env
         assert np.array_equal(world.download("env_status"), oracle.download("env_status"))
-        assert relative_error(generalized_impulse(world, E), generalized_impulse(oracle, E)) <= TOL
-        bound = max(TOL, 4.0 * oracle_sensitivity(oracle_py, index, E, ["lambda"])["lambda"])
+        impulse_o = generalized_impulse(oracle, E)
+        impulse = scaled_errors(generalized_impulse(world, E), impulse_o, np.maximum(np.abs(impulse_o).max(1), 1e-9), E)
+        print(cfg.name, f"J^T lambda: worst environment {impulse.max():.2e}, {int((impulse > TOL).sum())} of {E} above 1e-4; "
+              f"the oracle's own one-ulp sensitivity {sens['impulse']:.2e}")
+        assert impulse.max() <= bar(sens, "impulse")
+        bound = bar(sens, "lambda")
         lam_error = relative_error(world.download("lambda"), oracle.download("lambda"))
         print(cfg.name, f"lambda error {lam_error:.2e} against bound {bound:.2e}")
         assert lam_error <= bound
@@ -178,38 +292,27 @@ def test_several_steps_stay_with_the_oracle(oracle_py, device):
     oracle.close()
 
 
-def test_rope_backward_error(oracle_py, device):
-    """The 64-link rope's mass matrix has a condition number near 5e6, so qdd moves by ~1e-2 under one-ulp input
-    changes in the oracle itself: a forward bar of 1e-4 means nothing there.  What fp32 does fix: M, the bias and
-    the poses to 1e-4, the factorisation by reconstruction, and qdd by its residual M qdd + bias - tau."""
-    E = 32
+def test_rope_step_matches_the_oracle(oracle_py, device):
+    """Config 5 through every op, the block descent included.  The 64-link rope's mass matrix has a condition number
+    of about 2e4 (with its joint armature) and its Newton block about 1e6, so accelerations and the solve's outputs
+    move by more than 1e-4 under a one-ulp change of the inputs in the oracle itself; their bar is max(1e-4, 4 x that
+    measured sensitivity), and the accelerations are also held by their residual.  The resulting joint angles carry
+    the push-out of the position pass, one more block descent over 64 one-sided rows that stops at its Newton-step
+    budget in a few environments: they get the same kind of bar.  Everything else - poses, M, the bias, the contact
+    integers, rows and Jacobians, status words - is held as on the other configurations."""
+    E = 64
     cfg, oracle, world, state = make_pair(oracle_py, device, 5, E)
-    both(oracle, world, "FkWorldPoses")
-    close(world, oracle, "link_pose")
-    oracle.op("articulation_dynamics", 0)
-    world.op("ArticulationDynamics", 1)
-    world.synchronize()
-    close(world, oracle, "m")
-    close(world, oracle, "articulation_bias")
-    n = world.dof
-    M = world.download("m").reshape(E, n, n).astype(np.float64)
-    factor = world.download("m_factor").reshape(E, n, n).astype(np.float64)
-    lower = np.tril(factor, -1) + np.eye(n)
-    rebuilt = lower @ (np.einsum("eii->ei", factor)[:, :, None] * lower.transpose(0, 2, 1))
-    assert np.abs(rebuilt - M).max() <= 1e-5 * np.abs(M).max()
-    qdd = world.download("articulation_qdd").reshape(E, n).astype(np.float64)
-    bias = world.download("articulation_bias").reshape(E, n)
-    tau = state["tau"][:, 1:].astype(np.float64)
-    residual = np.einsum("eij,ej->ei", M, qdd) + bias - tau
-    scale = np.abs(np.einsum("eij,ej->ei", np.abs(M), np.abs(qdd))).max()
-    assert np.abs(residual).max() <= 1e-5 * scale
-    forward = relative_error(world.download("articulation_qdd"), oracle.download("articulation_qdd"))
-    print(f"rope qdd forward error {forward:.2e} (ill conditioned; not a bar)")
-    # contact pipeline integers stay exact on the rope
-    for name in UPSTREAM[2:]:
-        both(oracle, world, name)
-    for name in ("pair_count", "ucontact_count", "ucontact_row_range", "row_count"):
-        equal(world, oracle, name)
+    sens = one_ulp_sensitivity(oracle_py, cfg.template, nk.abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters), state)
+    print("rope one-ulp sensitivity of the oracle:", {k: f"{v:.2e}" for k, v in sens.items()})
+    report = compare_ops(oracle, world, E, sens, state)
+    status = oracle.download("env_status")
+    assert np.all(status == 0) and np.all(oracle.download("contact_count") == 64)
+    gs, os_ = world.download("vbd_velocity_sweep_count"), oracle.download("vbd_velocity_sweep_count")
+    lam = relative_error(world.download("lambda"), oracle.download("lambda"))
+    print("rope sweeps (oracle)", np.bincount(os_), "same count on", float(np.mean(gs == os_)), "worst environment:",
+          {k: f"{v.max():.2e}" for k, v in report.items()}, f"lambda {lam:.2e}")
+    assert np.mean(gs == os_) >= 0.9 and np.all(gs <= cfg.vel_iters)
+    assert lam <= bar(sens, "lambda")
     world.close()
     oracle.close()
 

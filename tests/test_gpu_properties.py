@@ -150,11 +150,45 @@ def test_long_run_of_an_authored_robot_stays_bounded(device):
 
 
 def test_rope_full_batch_steps(device):
-    E = 1024
+    """All 8192 environments of the rope for several steps: no environment may raise a status bit (a failed
+    factorisation, a non-finite velocity), every link keeps its contact, and the step's own result balances momentum:
+    M (v - v_free) = J^T lambda to the solve's tolerance, the size-independent check of the whole batch."""
+    E = 8192
     cfg, world = stepped(device, 5, E)
-    world.step()
-    world.synchronize()
-    assert np.all(np.isfinite(world.download("q"))) and np.all(np.isfinite(world.download("link_pose")))
+    n, R = world.dof, world.rows_per_env
+    for step in range(3):
+        for name in ("FkWorldPoses", "ArticulationDynamics", "SyncLinkBodyPose", "BuildAabbs", "LbvhQueryPairs",
+                     "NarrowphasePrimitives", "AssembleRows"):
+            world.op(name)
+        world.op("ContactWarmStart", 0)
+        world.synchronize()
+        free = world.download("qdot_flat").reshape(E, -1)[:, :n].astype(np.float64)
+        world.op("BlockDescentSolve")
+        world.synchronize()
+        status = world.download("env_status")
+        assert not status.any(), f"step {step}: {int((status != 0).sum())} of {E} environments raised a status bit"
+        contacts = world.download("contact_count")
+        assert contacts.mean() > 56.0 and contacts.min() >= 32        # links pushed out of the plane leave their contact
+        sweeps = world.download("vbd_velocity_sweep_count")
+        assert sweeps.min() >= 1 and sweeps.max() <= cfg.vel_iters
+        velocity = world.download("qdot_flat").reshape(E, -1)[:, :n].astype(np.float64)
+        M = world.download("m").reshape(E, n, n).astype(np.float64)
+        J = (world.download("chain_jacobian").reshape(E, R, -1) + world.download("chain_jacobian_b").reshape(E, R, -1))[:, :, :n]
+        impulse = np.einsum("eri,er->ei", J.astype(np.float64), world.download("lambda").reshape(E, R).astype(np.float64))
+        momentum = np.einsum("eij,ej->ei", M, velocity - free)
+        # the solve's own measure (MeasureTilePrimal): the velocity that the unbalanced momentum stands for
+        balance = np.abs(np.linalg.solve(M, (momentum - impulse)[:, :, None])[:, :, 0]).max(1)
+        converged = sweeps < cfg.vel_iters
+        print(f"rope step {step}: sweeps mean {sweeps.mean():.2f}, at the cap {int((~converged).sum())}, "
+              f"momentum balance worst {balance[converged].max():.2e} m/s against free velocities of {np.abs(free).max():.2e}")
+        assert balance[converged].max() <= 1e-4
+        world.op("ContactWarmStart", 1)
+        for name in ("IntegratePosition", "FkWorldPoses", "FkLinkVelocities"):
+            world.op(name)
+        world.synchronize()
+    pose = world.download("link_pose").reshape(E, -1, 7)
+    assert np.all(np.isfinite(world.download("q"))) and np.all(np.isfinite(pose))
+    assert pose[:, 1:, 2].min() > 0.005 and pose[:, 1:, 2].max() < 0.02        # the rope stays on the plane
     world.close()
 
 
@@ -382,9 +416,13 @@ def test_published_batch_sizes_match_the_oracle_directly(oracle_py, device, inde
     for name in ("pair_count", "ucontact_count", "ucontact_row_range", "row_count", "env_status", "contact_cache_pair",
                  "contact_cache_age", "contact_warm_start_counts"):
         assert np.array_equal(world.download(name), oracle.download(name)), name
+    from test_gpu_parity import bar, one_ulp_sensitivity
+    sens = one_ulp_sensitivity(oracle_py, cfg.template, desc, state, threads=16)
     for name in ("articulation_qdd", "link_pose", "body_pose", "q", "qdot", "link_velocity"):
-        error = relative_error(world.download(name), oracle.download(name))
-        assert error <= 1e-4, f"{name}: {error:.2e}"
+        errors = per_env_error(world.download(name), oracle.download(name), E)
+        tol = bar(sens, "velocity") if name in ("qdot", "link_velocity") else 1e-4
+        print(f"{cfg.name} {E} envs {name}: worst environment {errors.max():.2e}, {int((errors > 1e-4).sum())} above 1e-4 (bar {tol:.1e})")
+        assert errors.max() <= tol, f"{name}: {errors.max():.2e}"
     world.close()
     oracle.close()
 

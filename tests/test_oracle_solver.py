@@ -160,3 +160,34 @@ def test_iteration_budget_is_respected_and_reported(oracle_py):
     assert early.any() and (~early).any()
     # environments that met the tolerance inside the budget are untouched by a larger budget
     assert np.array_equal(few["lambda"][early], many["lambda"][early]) and np.array_equal(few["sweeps"][early], many["sweeps"][early])
+
+
+@pytest.mark.parametrize("n", [7, 18, 32, 33, 36, 48, 64])
+def test_block_factor_follows_the_route_of_its_width(oracle_py, n):
+    """Up to 32 coordinates the block is factored L L^T from the first coordinate (block_descent_tile.cuh:1622-1645);
+    past them U U^T from the last one (FactorTileColumns :209-252).  Either factor must reproduce the matrix and
+    solve the system; which triangle it fills tells the order of elimination."""
+    import ctypes as C
+    L = oracle_py.lib()
+    L.nko_tile_cholesky_solve.restype = C.c_int
+    rng = np.random.default_rng(n)
+    a = rng.normal(size=(n, n + 5))
+    h = (a @ a.T + 0.5 * np.eye(n)).astype(np.float32)
+    g = rng.normal(size=n).astype(np.float32)
+    factor = np.zeros((n, n), np.float32)
+    d = np.zeros(n, np.float32)
+    ok = L.nko_tile_cholesky_solve(h.ctypes.data_as(C.c_void_p), C.c_uint32(n), g.ctypes.data_as(C.c_void_p),
+                                   factor.ctypes.data_as(C.c_void_p), d.ctypes.data_as(C.c_void_p))
+    assert ok == 1
+    f = factor.astype(np.float64)
+    if n > 32:
+        assert np.all(np.tril(f, -1) == 0.0) and np.all(np.diag(f) > 0.0)
+    else:
+        assert np.all(np.triu(f, 1) == 0.0) and np.all(np.diag(f) > 0.0)
+    assert np.abs(f @ f.T - h).max() <= 2e-6 * np.abs(h).max()
+    exact = np.linalg.solve(h.astype(np.float64), g.astype(np.float64))
+    assert np.abs(d - exact).max() <= 1e-4 * np.abs(exact).max()
+    # an indefinite matrix is refused on either route
+    h[n // 2, n // 2] = -1.0
+    assert L.nko_tile_cholesky_solve(h.ctypes.data_as(C.c_void_p), C.c_uint32(n), g.ctypes.data_as(C.c_void_p),
+                                     factor.ctypes.data_as(C.c_void_p), d.ctypes.data_as(C.c_void_p)) == 0
