@@ -64,11 +64,13 @@ class DeviceDescC(C.Structure):
     _fields_ = [("gpu_index", C.c_uint32), ("stream", C.c_void_p), ("backend_selection_layer_enabled", C.c_uint8)]
 
 
+RESET_ENVS_STATIC_MAX = 16384   # NUKA_RESET_ENVS_STATIC_MAX of include/nuka_hip.h
+
 EXPORTS = [
     "nuka_result_message", "nuka_last_error_message", "nuka_device_create", "nuka_device_destroy", "nuka_device_backend",
     "nuka_world_create_from_template", "nuka_world_destroy", "nuka_world_step", "nuka_world_step_n",
     "nuka_world_set_execution_mode", "nuka_world_set_velocity_iterations", "nuka_world_get_velocity_iterations",
-    "nuka_world_synchronize", "nuka_world_reset", "nuka_world_reset_envs", "nuka_world_checkpoint_capture", "nuka_world_checkpoint_restore",
+    "nuka_world_synchronize", "nuka_world_reset", "nuka_world_reset_envs", "nuka_world_reset_envs_static", "nuka_world_checkpoint_capture", "nuka_world_checkpoint_restore",
     "nuka_checkpoint_destroy", "nuka_checkpoint_byte_size", "nuka_world_dispatch_op", "nuka_field_from_name", "nuka_field_names",
     "nuka_world_get_buffer_view", "nuka_world_upload_field", "nuka_world_download_field", "nuka_world_get_info",
     "nuka_world_time_steps", "nuka_world_profile_ops", "nuka_device_copy_bandwidth", "nuka_hip_register_backend_entry",
@@ -319,9 +321,11 @@ class World:
     def reset(self):
         _check(lib().nuka_world_reset(self._h))
 
-    def reset_envs(self, env_ids):
+    def reset_envs(self, env_ids, static=False):
+        """Masked reset; `static` takes the entry point that stages the ids in the library's static device array."""
         ids = np.ascontiguousarray(np.asarray(env_ids, dtype=np.uint32))
-        _check(lib().nuka_world_reset_envs(self._h, ids.ctypes.data, ids.size))
+        call = lib().nuka_world_reset_envs_static if static else lib().nuka_world_reset_envs
+        _check(call(self._h, C.c_void_p(ids.ctypes.data), C.c_uint32(ids.size)))
 
     def set_execution_mode(self, graph):
         _check(lib().nuka_world_set_execution_mode(self._h, 1 if graph else 0))

@@ -11,6 +11,7 @@
 #include <cstring>
 #include <exception>
 #include <memory>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -408,6 +409,16 @@ __global__ void __launch_bounds__(256) ResetEnvsKernel(ResetSegments s, const ui
         s.live[seg][first + i] = s.initial[seg] != nullptr ? s.initial[seg][first + i] : 0u;
 }
 
+// Staging of nuka_world_reset_envs_static: the environment ids of one call.  A file-scope device array, so the call
+// takes no device memory of its own; every GPU the library runs on holds its own copy, at its own address, until the
+// process ends.  In host code the array's name is only a stand-in: its device address on a GPU is asked for once, with
+// that GPU current, when a device handle is created there, and kept in g_static_reset_ids.
+constexpr int kMaxGpus = 64;
+static __device__ __align__(256) uint32_t scratch[NUKA_RESET_ENVS_STATIC_MAX];
+uint32_t* g_static_reset_ids[kMaxGpus] = {};
+uint32_t g_static_reset_host[NUKA_RESET_ENVS_STATIC_MAX];   // the sorted, deduplicated ids of the call in flight
+std::mutex g_static_reset_mutex;                            // guards the host staging above
+
 bool CheckpointKeeps(const char* name) {
     for (const char* kept : {"q", "qdot", "qddot", "tau", "base_pose", "link_pose", "link_velocity", "body_pose", "lambda", "link_wrench",
                              "contact_cache_pair", "contact_cache_feature", "contact_cache_material", "contact_cache_lambda",
@@ -641,6 +652,17 @@ nuka_result_t nuka_device_create(const nuka_device_desc_t* desc, nuka_device_han
     if (index >= uint32_t(count)) return Error(NUKA_RESULT_DEVICE_ERROR, "no HIP device with this gpu_index");
     void* backend = CreateBackend(int(index), desc->stream);
     if (backend == nullptr) return Error(NUKA_RESULT_DEVICE_ERROR, "backend creation failed");
+    // CreateBackend has made this GPU current: its copy of the static staging array is looked up once
+    if (index < uint32_t(kMaxGpus) && g_static_reset_ids[index] == nullptr) {
+        void* address = nullptr;
+        if (hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)) != hipSuccess || address == nullptr) {
+            (void)hipGetLastError();
+            auto* made = reinterpret_cast<nuka_phi_backend*>(backend);
+            reinterpret_cast<nuka_phi_backend_head*>(made)->iface->free(made);
+            return Error(NUKA_RESULT_DEVICE_ERROR, "the static staging array has no address on this device");
+        }
+        g_static_reset_ids[index] = static_cast<uint32_t*>(address);
+    }
     auto* record = new DeviceRecord{backend, int(index)};
     *out = reinterpret_cast<nuka_device_handle>(record);
     return NUKA_RESULT_OK;
@@ -945,6 +967,27 @@ nuka_result_t nuka_world_reset(nuka_world_handle world) {
     return nuka_world_synchronize(world);
 }
 
+namespace nkh {
+namespace {
+// The arena slices a masked reset copies back or clears, one segment per field.
+nuka_result_t ResetSegmentsOf(World* w, ResetSegments* out) {
+    ResetSegments segments{};
+    char* arena = static_cast<char*>(Iface(w->arena)->base(w->arena));
+    const char* initial = static_cast<const char*>(Iface(w->initial)->base(w->initial));
+    for (const Field& f : w->fields) {
+        if (f.is_template || f.count == 0u || !(CheckpointKeeps(f.name) || CheckpointClears(f.name))) continue;
+        if (segments.count == kMaxCheckpointSegments) return NUKA_RESULT_INTERNAL;
+        const uint32_t at = segments.count++;
+        segments.words_per_env[at] = uint32_t(f.count * f.elem_bytes / 4u / w->env_count);
+        segments.live[at] = reinterpret_cast<uint32_t*>(arena + f.offset);
+        segments.initial[at] = CheckpointKeeps(f.name) ? reinterpret_cast<const uint32_t*>(initial + f.offset) : nullptr;
+    }
+    *out = segments;
+    return NUKA_RESULT_OK;
+}
+}  // namespace
+}  // namespace nkh
+
 nuka_result_t nuka_world_reset_envs(nuka_world_handle world, const uint32_t* env_ids, uint32_t count) {
     auto* w = reinterpret_cast<World*>(world);
     if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
@@ -958,16 +1001,7 @@ nuka_result_t nuka_world_reset_envs(nuka_world_handle world, const uint32_t* env
         if (seen[env_ids[i]] == 0u) { seen[env_ids[i]] = 1u; unique.push_back(env_ids[i]); }
     }
     ResetSegments segments{};
-    char* arena = static_cast<char*>(Iface(w->arena)->base(w->arena));
-    const char* initial = static_cast<const char*>(Iface(w->initial)->base(w->initial));
-    for (const Field& f : w->fields) {
-        if (f.is_template || f.count == 0u || !(CheckpointKeeps(f.name) || CheckpointClears(f.name))) continue;
-        if (segments.count == kMaxCheckpointSegments) return Error(NUKA_RESULT_INTERNAL, "too many reset segments");
-        const uint32_t at = segments.count++;
-        segments.words_per_env[at] = uint32_t(f.count * f.elem_bytes / 4u / w->env_count);
-        segments.live[at] = reinterpret_cast<uint32_t*>(arena + f.offset);
-        segments.initial[at] = CheckpointKeeps(f.name) ? reinterpret_cast<const uint32_t*>(initial + f.offset) : nullptr;
-    }
+    if (ResetSegmentsOf(w, &segments) != NUKA_RESULT_OK) return Error(NUKA_RESULT_INTERNAL, "too many reset segments");
     if (nuka_world_synchronize(world) != NUKA_RESULT_OK) return NUKA_RESULT_DEVICE_ERROR;
     if (hipMemcpyAsync(w->data.reset_env_ids, unique.data(), unique.size() * sizeof(uint32_t), hipMemcpyHostToDevice,
                        BackendStream(w->device->backend)) != hipSuccess) return Error(NUKA_RESULT_DEVICE_ERROR, "id upload failed");
@@ -975,6 +1009,38 @@ nuka_result_t nuka_world_reset_envs(nuka_world_handle world, const uint32_t* env
                        segments, w->data.reset_env_ids, w->env_count);
     if (hipGetLastError() != hipSuccess) return Error(NUKA_RESULT_DEVICE_ERROR, "reset launch failed");
     return nuka_world_synchronize(world);   // the host copy of the ids must outlive the upload
+}
+
+// nuka_world_reset_envs for callers that cannot allocate: same kernel, same result, but the ids are staged in the
+// static device array (at most NUKA_RESET_ENVS_STATIC_MAX of them) and in a static host array, so the call takes no
+// device or host memory.  The array is shared by every call on one GPU: calls that overlap there race.
+nuka_result_t nuka_world_reset_envs_static(nuka_world_handle world, const uint32_t* env_ids, uint32_t count) {
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (count == 0u) return NUKA_RESULT_OK;
+    if (env_ids == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "env_ids is null");
+    if (count > NUKA_RESET_ENVS_STATIC_MAX)
+        return Error(NUKA_RESULT_INVALID_ARG, "more environment ids than NUKA_RESET_ENVS_STATIC_MAX in one static reset");
+    const int gpu = w->device->gpu_index;
+    uint32_t* staged = gpu >= 0 && gpu < kMaxGpus ? g_static_reset_ids[gpu] : nullptr;
+    if (staged == nullptr) return Error(NUKA_RESULT_DEVICE_ERROR, "no static staging array on this device");
+    for (uint32_t i = 0u; i < count; ++i)
+        if (env_ids[i] >= w->env_count) return Error(NUKA_RESULT_INVALID_ARG, "environment id out of range");
+    ResetSegments segments{};
+    if (ResetSegmentsOf(w, &segments) != NUKA_RESULT_OK) return Error(NUKA_RESULT_INTERNAL, "too many reset segments");
+    std::lock_guard<std::mutex> lock(g_static_reset_mutex);
+    // duplicates are dropped so that no two workgroups write one slice; the order of the ids does not matter
+    std::memcpy(g_static_reset_host, env_ids, size_t{count} * sizeof(uint32_t));
+    std::sort(g_static_reset_host, g_static_reset_host + count);
+    const uint32_t unique = uint32_t(std::unique(g_static_reset_host, g_static_reset_host + count) - g_static_reset_host);
+    if (nuka_world_synchronize(world) != NUKA_RESULT_OK) return NUKA_RESULT_DEVICE_ERROR;
+    hipStream_t stream = BackendStream(w->device->backend);
+    // only the first `unique` words are read by this call; what an earlier, longer call left behind them is ignored
+    if (hipMemcpyAsync(staged, g_static_reset_host, size_t{unique} * sizeof(uint32_t), hipMemcpyHostToDevice, stream) != hipSuccess)
+        return Error(NUKA_RESULT_DEVICE_ERROR, "id upload failed");
+    hipLaunchKernelGGL(ResetEnvsKernel, dim3(unique, segments.count), dim3(256), 0, stream, segments, staged, w->env_count);
+    if (hipGetLastError() != hipSuccess) return Error(NUKA_RESULT_DEVICE_ERROR, "reset launch failed");
+    return nuka_world_synchronize(world);   // the host staging is free again once the upload has run
 }
 
 nuka_result_t nuka_world_dispatch_op(nuka_world_handle world, uint16_t op, uint32_t variant) {
