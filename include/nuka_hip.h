@@ -1,11 +1,16 @@
 /*
- * C ABI of the MI355X articulation-step library (libnuka_hip.so): the subset of the reference's stable C surface
- * (src/include/nuka/nuka.h) that drives the batched articulation step, with the same names, argument meaning
- * and error behaviour.  Plain pointers and sizes only.
+ * C ABI of the MI355X articulation-step library (libnuka_hip.so).  Plain pointers and sizes only.
  *
- * Each entry cites the reference interface it replaces.  `nuka_world_create_from_template` stands where
- * `nuka_world_create_from_scene` stands in the reference: this library has no scene importer, so the caller
- * passes the cooked-template inputs (what SceneIR -> CookToModel produces) directly.
+ * Two groups of declarations:
+ *   - what the reference's stable C surface (src/include/nuka/nuka.h) declares for the batched articulation step, under
+ *     the reference's own names and with its layouts, signatures and numeric values: result codes, device and world
+ *     descriptors, nuka_world_create_from_scene, step / reset / checkpoint / parameter / execution-mode calls, the
+ *     NUKA_FIELD_* ids of the fields this library serves, buffer views and byte transfers.  A caller compiled against
+ *     nuka.h that uses only these links against this library unchanged; every such entry cites the lines it matches.
+ *   - the library's own additions, which no reference name is reused for: the cooked-template creator
+ *     (nuka_hip_world_desc_t, nuka_world_create_from_template), scene handles (nuka_scene_*,
+ *     nuka_hip_world_create_from_scene_handle), per-op dispatch, the extended field ids (every internal field by
+ *     name, from NUKA_HIP_FIELD_BASE up) and the timing helpers the benchmark uses.
  */
 #ifndef NUKA_HIP_H_
 #define NUKA_HIP_H_
@@ -19,12 +24,15 @@
 extern "C" {
 #endif
 
-/* nuka.h:22-32 (the device-error code keeps the reference's numeric value 3) */
+/* nuka.h:22-32.  Code 3 is the reference's device-runtime error; NUKA_RESULT_DEVICE_ERROR names the same value. */
 typedef enum nuka_result_t {
     NUKA_RESULT_OK = 0,
     NUKA_RESULT_INVALID_ARG = 1,
     NUKA_RESULT_NULL_HANDLE = 2,
+    NUKA_RESULT_CUDA_ERROR = 3,
     NUKA_RESULT_DEVICE_ERROR = 3,
+    NUKA_RESULT_FILE_NOT_FOUND = 4,
+    NUKA_RESULT_PARSE_ERROR = 5,
     NUKA_RESULT_OUT_OF_MEMORY = 6,
     NUKA_RESULT_NOT_SUPPORTED = 7,
     NUKA_RESULT_INTERNAL = 100
@@ -37,10 +45,11 @@ typedef struct nuka_world_t* nuka_world_handle;
 const char* nuka_result_message(nuka_result_t result);
 const char* nuka_last_error_message(void);
 
-/* nuka.h:46-55.  `stream` non-null is a borrowed hipStream_t; null creates an owned stream at default priority. */
+/* nuka.h:46-51, member for member.  `cuda_stream` (the reference's name for the member) non-null is a borrowed
+ * hipStream_t; null creates an owned stream at default priority. */
 typedef struct nuka_device_desc_t {
     uint32_t gpu_index;
-    void* stream;
+    void* cuda_stream;
     uint8_t backend_selection_layer_enabled;
 } nuka_device_desc_t;
 nuka_result_t nuka_device_create(const nuka_device_desc_t* desc, nuka_device_handle* out);
@@ -99,8 +108,9 @@ typedef struct nuka_template_desc_t {
     uint32_t reserved1;
 } nuka_template_desc_t;
 
-/* nuka.h:57-173 nuka_world_desc_t; zero keeps the default of the same reference field. */
-typedef struct nuka_world_desc_t {
+/* The world options of the cooked-template creator (the library's own descriptor; the reference's nuka_world_desc_t
+ * follows below).  Zero keeps the default of the reference field of the same name (nuka.h:160-173). */
+typedef struct nuka_hip_world_desc_t {
     uint32_t struct_size;
     uint32_t env_count;
     float fixed_dt;                  /* 0 => 1/240 */
@@ -121,6 +131,55 @@ typedef struct nuka_world_desc_t {
                                               contact wrenches averaged over the step (src/nk/pipeline/pipeline.cpp:118-180).
                                               Read, like the next member, only when struct_size covers it */
     uint32_t contact_detection_substeps;   /* nuka.h:172: 0 or 1; substeps that share a detection are NOT_SUPPORTED */
+} nuka_hip_world_desc_t;
+
+/* nuka.h:57-173, member for member: same names, types, order and therefore offsets.  nuka_world_create_from_scene reads
+ * scene_path, env_count, fixed_dt, determinism, control_mode, gravity_*, solver_vel_iters, solver_pos_iters,
+ * solver_contact_margin, solver_baumgarte_max_velocity, solver_overlap_recovery_velocity, solver_substeps and
+ * contact_detection_substeps.  The members that ask for what this library does not build must be zero (null), else the
+ * creation is refused with NUKA_RESULT_NOT_SUPPORTED: terrain_*, instance_count above 1, contact_family,
+ * heightfield_*, curric_*, terrain_feature_cell, cloth_integrator, ogc_contact_capacity, control modes 3 and 4.
+ * solver_max_pairs is accepted and has no effect (every admitted pair of an environment has its own slot here). */
+typedef struct nuka_world_desc_t {
+    const char* scene_path;
+    uint32_t env_count;
+    float fixed_dt;
+    uint8_t determinism;             /* 0 or 1; both run the same deterministic kernels */
+    uint8_t control_mode;            /* 0 PD position, 1 torque, 2 velocity, 3 computed torque, 4 OSC, 5 actuator */
+    uint32_t osc_task_link;
+    float terrain_step_height;
+    float terrain_step_width;
+    float terrain_platform_width;
+    float terrain_grid_width;
+    float terrain_grid_height_max;
+    uint32_t instance_count;
+    float instance_spacing;
+    uint32_t contact_family;
+    uint32_t heightfield_terrain_type;
+    uint32_t heightfield_nrow;
+    uint32_t heightfield_ncol;
+    float heightfield_cell;
+    const char* heightfield_image_path;
+    float heightfield_radius_x;
+    float heightfield_radius_y;
+    float heightfield_elevation_z;
+    float heightfield_base_z;
+    float gravity_x;                 /* all three zero => {0, 0, -9.81} */
+    float gravity_y;
+    float gravity_z;
+    uint32_t curric_levels;
+    uint32_t curric_types;
+    float terrain_feature_cell;
+    uint32_t solver_vel_iters;       /* 0 => 10 */
+    uint32_t solver_pos_iters;       /* 0 => 4 */
+    float solver_contact_margin;
+    uint32_t solver_max_pairs;
+    float solver_baumgarte_max_velocity;
+    uint32_t cloth_integrator;
+    uint32_t ogc_contact_capacity;
+    float solver_overlap_recovery_velocity;
+    uint32_t solver_substeps;
+    uint32_t contact_detection_substeps;
 } nuka_world_desc_t;
 
 /* Scene files (src/import/mjcf_importer.cpp LoadMjcf and src/import/urdf_importer.cpp LoadUrdf, then the articulation
@@ -160,15 +219,24 @@ const char* nuka_scene_joint_name(nuka_scene_handle scene, uint32_t link);
  * its actuators and the joint's actuator force range; base_pose[7] of a floating root.  Null outputs are skipped. */
 nuka_result_t nuka_scene_initial_state(nuka_scene_handle scene, float* q, float* base_pose, float* drive_stiffness,
                                        float* drive_damping, float* drive_force_limit, float* drive_joint_force_limit);
-/* nuka.h:175 nuka_world_create_from_scene: the scene's template in every environment, its initial state and drive
- * parameters uploaded (PD targets hold the initial pose), and that state kept as what nuka_world_reset returns to.
- * `desc->fixed_dt` of 0 takes the file's timestep; gravity of all zeros takes the file's. */
-nuka_result_t nuka_world_create_from_scene(nuka_device_handle device, nuka_scene_handle scene, const nuka_world_desc_t* desc,
-                                           nuka_world_handle* out);
+/* A loaded scene's template in every environment, its initial state and drive parameters uploaded (PD targets hold
+ * the initial pose), and that state kept as what nuka_world_reset returns to.  `desc->fixed_dt` of 0 takes the file's
+ * timestep; gravity of all zeros takes the file's. */
+nuka_result_t nuka_hip_world_create_from_scene_handle(nuka_device_handle device, nuka_scene_handle scene,
+                                                      const nuka_hip_world_desc_t* desc, nuka_world_handle* out);
 
-/* nuka.h:175 nuka_world_create_from_scene */
+/* nuka.h:175-177, src/c_abi/world.cpp:590-635: the file at desc->scene_path read by its extension (.xml or .mjcf as
+ * MJCF, .urdf as URDF; .nks and OpenUSD files are NUKA_RESULT_NOT_SUPPORTED, as is any other extension) and stepped in
+ * desc->env_count environments.  As in the reference a null desc, a null scene_path, fixed_dt <= 0, env_count 0,
+ * determinism above 1 or an unknown control mode is NUKA_RESULT_INVALID_ARG and a null device NUKA_RESULT_NULL_HANDLE;
+ * a file that cannot be opened is NUKA_RESULT_FILE_NOT_FOUND and one that cannot be read as its format, or holds what
+ * this library has no path for (meshes, several articulations), NUKA_RESULT_PARSE_ERROR or NUKA_RESULT_NOT_SUPPORTED
+ * with the reason in nuka_last_error_message.  The control mode is the descriptor's, the drive gains the file's. */
+nuka_result_t nuka_world_create_from_scene(nuka_device_handle device, const nuka_world_desc_t* desc, nuka_world_handle* out);
+
+/* The cooked-template creator: what SceneIR -> CookToModel produces for one environment, passed directly. */
 nuka_result_t nuka_world_create_from_template(nuka_device_handle device, const nuka_template_desc_t* tmpl,
-                                              const nuka_world_desc_t* desc, nuka_world_handle* out);
+                                              const nuka_hip_world_desc_t* desc, nuka_world_handle* out);
 void nuka_world_destroy(nuka_world_handle world);            /* nuka.h:253 */
 nuka_result_t nuka_world_step(nuka_world_handle world);      /* nuka.h:254, src/c_abi/world.cpp:696-698 */
 nuka_result_t nuka_world_step_n(nuka_world_handle world, uint32_t step_count);   /* nuka.h:255, world.cpp:700-731 */
@@ -269,9 +337,62 @@ nuka_result_t nuka_world_set_gravity_z(nuka_world_handle world, float gravity_z)
  * tests/oracle/featherstone_oracle_harness.cpp:174-182 uses. */
 nuka_result_t nuka_world_dispatch_op(nuka_world_handle world, uint16_t op, uint32_t variant);
 
-/* Fields are named as in src/nk/model/fields.yaml. */
-typedef uint32_t nuka_state_field_t;
-/* ~0u when the library serves no field of that name. */
+/* nuka.h:496-958: the public field ids, with the reference's numeric values, for the fields this library serves
+ * (any other value below NUKA_HIP_FIELD_BASE is NUKA_RESULT_NOT_SUPPORTED, as the reference answers for a field a world
+ * does not hold).  A view of one of these has the reference's element stride (src/c_abi/dlpack_table.hpp:101-330): 28
+ * bytes for a pose, 24 for a spatial vector, 12 for a vector, the field's element size otherwise. */
+typedef enum nuka_state_field_t {
+    NUKA_FIELD_RIGID_BODY_TRANSFORM = 0,        /* body_pose */
+    NUKA_FIELD_ARTICULATION_LINK_POSE = 1,      /* link_pose */
+    NUKA_FIELD_JOINT_POSITION = 2,              /* q */
+    NUKA_FIELD_JOINT_VELOCITY = 3,              /* qdot */
+    NUKA_FIELD_CONTACT_POINTS = 5,              /* contact_point */
+    NUKA_FIELD_DRIVE_TARGET = 6,
+    NUKA_FIELD_LINK_VELOCITY = 7,
+    NUKA_FIELD_DRIVE_STIFFNESS = 8,
+    NUKA_FIELD_DRIVE_DAMPING = 9,
+    NUKA_FIELD_DRIVE_FORCE_LIMIT = 10,
+    NUKA_FIELD_BASE_POSE = 11,
+    NUKA_FIELD_TORQUE_INPUT = 12,               /* the storage of DRIVE_TARGET, as in the reference */
+    NUKA_FIELD_VELOCITY_TARGET = 13,
+    NUKA_FIELD_ACTUATOR_NOLOAD_SPEED = 14,
+    NUKA_FIELD_LINK_CONTACT_WRENCH = 16,
+    NUKA_FIELD_CONTACT_NORMAL = 17,
+    NUKA_FIELD_CONTACT_FORCE = 18,
+    NUKA_FIELD_CONTACT_LINK = 19,
+    NUKA_FIELD_JOINT_FEEDFORWARD = 22,          /* joint_f */
+    NUKA_FIELD_JOINT_LIMIT_IMPULSE = 27,
+    NUKA_FIELD_ACTUATOR_EFFORT_REQUESTED = 28,
+    NUKA_FIELD_ACTUATOR_EFFORT = 29,
+    NUKA_FIELD_ACTUATOR_SATURATED = 30,
+    NUKA_FIELD_CONTACT_SIDE_A_KIND = 33,
+    NUKA_FIELD_CONTACT_SIDE_B_KIND = 34,
+    NUKA_FIELD_CONTACT_SIDE_A_INDEX = 35,
+    NUKA_FIELD_CONTACT_SIDE_B_INDEX = 36,
+    NUKA_FIELD_ENV_STATUS = 39,
+    NUKA_FIELD_CONTACT_WARM_START_COUNTS = 70,
+    NUKA_FIELD_VBD_VELOCITY_SWEEP_COUNT = 79,
+    NUKA_FIELD_UCONTACT_ROW_RANGE = 103,
+    NUKA_FIELD_LINK_WRENCH = 105,
+    NUKA_FIELD_UCONTACT_COUNT = 107,
+    NUKA_FIELD_UCONTACT_POINT = 108,
+    NUKA_FIELD_SOLVER_RESIDUAL = 109,
+    NUKA_FIELD_UCONTACT_NORMAL = 128,
+    NUKA_FIELD_UCONTACT_DEPTH = 129,
+    NUKA_FIELD_UCONTACT_LAW = 132,
+    NUKA_FIELD_UCONTACT_SIDE_A = 134,
+    NUKA_FIELD_UCONTACT_SIDE_B = 135,
+    NUKA_FIELD_UCONTACT_IMPULSE = 138,
+    NUKA_FIELD_JOINT_GRAVITY_FORCE = 157,
+    NUKA_FIELD_ROW_PENETRATION = 161,
+    NUKA_FIELD_ROW_LAMBDA = 162,
+    /* The library's own ids: every field of the world by its name in src/nk/model/fields.yaml (m, m_factor, urows,
+     * chain_jacobian, ...), NUKA_HIP_FIELD_BASE + its place in nuka_field_names().  Views of these count 4- or 8-byte
+     * scalars. */
+    NUKA_HIP_FIELD_BASE = 0x10000,
+    NUKA_HIP_FIELD_NONE = 0x7FFFFFFF
+} nuka_state_field_t;
+/* NUKA_HIP_FIELD_NONE when the library serves no field of that name. */
 nuka_state_field_t nuka_field_from_name(const char* name);
 const char* nuka_field_names(void);   /* comma separated */
 

@@ -60,10 +60,11 @@ PARAMS = ("gravity_z", "velocity_iterations", "link_mass", "joint_damping", "joi
           "drive_force_limit")
 
 
-class DeviceDescC(C.Structure):
-    _fields_ = [("gpu_index", C.c_uint32), ("stream", C.c_void_p), ("backend_selection_layer_enabled", C.c_uint8)]
+class DeviceDescC(C.Structure):   # nuka.h:46-51
+    _fields_ = [("gpu_index", C.c_uint32), ("cuda_stream", C.c_void_p), ("backend_selection_layer_enabled", C.c_uint8)]
 
 
+FIELD_BASE, FIELD_NONE = 0x10000, 0x7FFFFFFF   # NUKA_HIP_FIELD_BASE, NUKA_HIP_FIELD_NONE
 RESET_ENVS_STATIC_MAX = 16384   # NUKA_RESET_ENVS_STATIC_MAX of include/nuka_hip.h
 
 EXPORTS = [
@@ -76,7 +77,7 @@ EXPORTS = [
     "nuka_world_time_steps", "nuka_world_profile_ops", "nuka_device_copy_bandwidth", "nuka_hip_register_backend_entry",
     "nuka_hip_op_count", "nuka_hip_op_name", "nuka_hip_op_from_name",
     "nuka_scene_load_mjcf", "nuka_scene_load_urdf", "nuka_scene_destroy", "nuka_scene_template", "nuka_scene_get_info", "nuka_scene_link_name",
-    "nuka_scene_joint_name", "nuka_scene_initial_state", "nuka_world_create_from_scene",
+    "nuka_scene_joint_name", "nuka_scene_initial_state", "nuka_world_create_from_scene", "nuka_hip_world_create_from_scene_handle",
     "nuka_checkpoint_equal", "nuka_world_state_hash", "nuka_world_forward_kinematics", "nuka_world_param_count", "nuka_world_get_param_infos",
     "nuka_world_get_param", "nuka_world_set_param", "nuka_world_set_link_mass", "nuka_world_set_gravity_z",
     "nuka_checkpoint_write", "nuka_world_checkpoint_read", "nuka_world_get_execution_info",
@@ -145,7 +146,8 @@ def lib():
         L.nuka_scene_joint_name.argtypes = [C.c_void_p, C.c_uint32]
         L.nuka_scene_joint_name.restype = C.c_char_p
         L.nuka_scene_initial_state.argtypes = [C.c_void_p] + [C.c_void_p] * 6
-        L.nuka_world_create_from_scene.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]
+        L.nuka_hip_world_create_from_scene_handle.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]
+        L.nuka_world_create_from_scene.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]
         L.nuka_checkpoint_equal.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_uint32)]
         L.nuka_world_state_hash.argtypes = [C.c_void_p, C.POINTER(C.c_uint64)]
         L.nuka_world_forward_kinematics.argtypes = [C.c_void_p]
@@ -241,8 +243,10 @@ class World:
     def __init__(self, device, template, desc):
         self.device = device
         self._h = C.c_void_p()
-        if isinstance(template, Scene):
-            _check(lib().nuka_world_create_from_scene(device._h, template._h, C.byref(desc), C.byref(self._h)))
+        if isinstance(desc, abi.SceneWorldDescC):      # the reference's entry point: the descriptor names the scene file
+            _check(lib().nuka_world_create_from_scene(device._h, C.byref(desc), C.byref(self._h)))
+        elif isinstance(template, Scene):
+            _check(lib().nuka_hip_world_create_from_scene_handle(device._h, template._h, C.byref(desc), C.byref(self._h)))
         else:
             tdesc, keep = template.to_c()
             _check(lib().nuka_world_create_from_template(device._h, C.byref(tdesc), C.byref(desc), C.byref(self._h)))
@@ -260,11 +264,20 @@ class World:
 
     def _field(self, name):
         fid = lib().nuka_field_from_name(name.encode())
-        if fid == 0xFFFFFFFF:
+        if fid == FIELD_NONE:
             raise KeyError(name)
         view = BufferViewC()
         _check(lib().nuka_world_get_buffer_view(self._h, fid, C.byref(view)))
         return fid, view
+
+    def public_view(self, public_name):
+        """The buffer view of a NUKA_FIELD_* id (its numeric value from nuka.h) and the bytes behind it."""
+        fid = abi.PUBLIC_FIELDS[public_name][0]
+        view = BufferViewC()
+        _check(lib().nuka_world_get_buffer_view(self._h, fid, C.byref(view)))
+        raw = np.empty(view.element_count * view.element_stride_bytes, np.uint8)
+        _check(lib().nuka_world_download_field(self._h, fid, raw.ctypes.data, raw.nbytes, 0))
+        return view, raw
 
     def download(self, name):
         fid, view = self._field(name)

@@ -54,6 +54,48 @@ class WorldDescC(C.Structure):
     ]
 
 
+class SceneWorldDescC(C.Structure):
+    """nuka_world_desc_t of nuka.h:57-173, member for member (the descriptor nuka_world_create_from_scene takes)."""
+    _fields_ = [
+        ("scene_path", C.c_char_p), ("env_count", C.c_uint32), ("fixed_dt", C.c_float), ("determinism", C.c_uint8),
+        ("control_mode", C.c_uint8), ("osc_task_link", C.c_uint32), ("terrain_step_height", C.c_float),
+        ("terrain_step_width", C.c_float), ("terrain_platform_width", C.c_float), ("terrain_grid_width", C.c_float),
+        ("terrain_grid_height_max", C.c_float), ("instance_count", C.c_uint32), ("instance_spacing", C.c_float),
+        ("contact_family", C.c_uint32), ("heightfield_terrain_type", C.c_uint32), ("heightfield_nrow", C.c_uint32),
+        ("heightfield_ncol", C.c_uint32), ("heightfield_cell", C.c_float), ("heightfield_image_path", C.c_char_p),
+        ("heightfield_radius_x", C.c_float), ("heightfield_radius_y", C.c_float), ("heightfield_elevation_z", C.c_float),
+        ("heightfield_base_z", C.c_float), ("gravity_x", C.c_float), ("gravity_y", C.c_float), ("gravity_z", C.c_float),
+        ("curric_levels", C.c_uint32), ("curric_types", C.c_uint32), ("terrain_feature_cell", C.c_float),
+        ("solver_vel_iters", C.c_uint32), ("solver_pos_iters", C.c_uint32), ("solver_contact_margin", C.c_float),
+        ("solver_max_pairs", C.c_uint32), ("solver_baumgarte_max_velocity", C.c_float), ("cloth_integrator", C.c_uint32),
+        ("ogc_contact_capacity", C.c_uint32), ("solver_overlap_recovery_velocity", C.c_float), ("solver_substeps", C.c_uint32),
+        ("contact_detection_substeps", C.c_uint32),
+    ]
+
+
+# nuka.h:496-958: the public field ids this library serves, by the name of the world field behind each
+PUBLIC_FIELDS = {
+    "RIGID_BODY_TRANSFORM": (0, "body_pose", 28), "ARTICULATION_LINK_POSE": (1, "link_pose", 28), "JOINT_POSITION": (2, "q", 4),
+    "JOINT_VELOCITY": (3, "qdot", 4), "CONTACT_POINTS": (5, "contact_point", 12), "DRIVE_TARGET": (6, "drive_target", 4),
+    "LINK_VELOCITY": (7, "link_velocity", 24), "DRIVE_STIFFNESS": (8, "drive_stiffness", 4), "DRIVE_DAMPING": (9, "drive_damping", 4),
+    "DRIVE_FORCE_LIMIT": (10, "drive_force_limit", 4), "BASE_POSE": (11, "base_pose", 28), "TORQUE_INPUT": (12, "drive_target", 4),
+    "VELOCITY_TARGET": (13, "velocity_target", 4), "ACTUATOR_NOLOAD_SPEED": (14, "actuator_noload_speed", 4),
+    "LINK_CONTACT_WRENCH": (16, "link_contact_wrench", 24), "CONTACT_NORMAL": (17, "contact_normal", 12),
+    "CONTACT_FORCE": (18, "contact_force", 12), "CONTACT_LINK": (19, "contact_link", 4), "JOINT_FEEDFORWARD": (22, "joint_f", 4),
+    "JOINT_LIMIT_IMPULSE": (27, "joint_limit_impulse", 8), "ACTUATOR_EFFORT_REQUESTED": (28, "actuator_effort_requested", 4),
+    "ACTUATOR_EFFORT": (29, "actuator_effort", 4), "ACTUATOR_SATURATED": (30, "actuator_saturated", 4),
+    "CONTACT_SIDE_A_KIND": (33, "contact_side_a_kind", 4), "CONTACT_SIDE_B_KIND": (34, "contact_side_b_kind", 4),
+    "CONTACT_SIDE_A_INDEX": (35, "contact_side_a_index", 4), "CONTACT_SIDE_B_INDEX": (36, "contact_side_b_index", 4),
+    "ENV_STATUS": (39, "env_status", 4), "CONTACT_WARM_START_COUNTS": (70, "contact_warm_start_counts", 8),
+    "VBD_VELOCITY_SWEEP_COUNT": (79, "vbd_velocity_sweep_count", 4), "UCONTACT_ROW_RANGE": (103, "ucontact_row_range", 8),
+    "LINK_WRENCH": (105, "link_wrench", 24), "UCONTACT_COUNT": (107, "ucontact_count", 4), "UCONTACT_POINT": (108, "ucontact_point", 48),
+    "SOLVER_RESIDUAL": (109, "solver_residual", 16), "UCONTACT_NORMAL": (128, "ucontact_normal", 48),
+    "UCONTACT_DEPTH": (129, "ucontact_depth", 16), "UCONTACT_LAW": (132, "ucontact_law", 4), "UCONTACT_SIDE_A": (134, "ucontact_a", 16),
+    "UCONTACT_SIDE_B": (135, "ucontact_b", 16), "UCONTACT_IMPULSE": (138, "ucontact_impulse", 48),
+    "JOINT_GRAVITY_FORCE": (157, "joint_gravity_force", 4), "ROW_PENETRATION": (161, "row_penetration", 4), "ROW_LAMBDA": (162, "lambda", 4),
+}
+
+
 class BufferViewC(C.Structure):   # nuka.h:1158-1164
     _fields_ = [("device_ptr", C.c_void_p), ("element_count", C.c_size_t), ("element_stride_bytes", C.c_uint32),
                 ("dtype", C.c_uint8)]

@@ -300,7 +300,7 @@ struct Builder : SceneParts {
                                                                       : context.Class(joint_class != nullptr ? joint_class : child_class).joint.type;
             if (kind == JointKind::Free) { free_by_type = true; return; }
             if (kind == JointKind::Fixed) return;
-            if (kind == JointKind::Ball) throw std::runtime_error("MJCF: ball joint on body '" + body_name + "' is not supported on this path");
+            if (kind == JointKind::Ball) throw Unsupported("MJCF: ball joint on body '" + body_name + "' is not supported on this path");
             if (kind != JointKind::Slide && joint.Attribute("pos") != nullptr) anchor = ParseV3(joint.Attribute("pos"));
             chain.push_back({&joint, anchor});
         });
@@ -468,7 +468,7 @@ struct Builder : SceneParts {
                 ParseFloats(actuator->Attribute("gainprm"), &gain, 1);
                 ParseFloats(actuator->Attribute("biasprm"), bias, 3);
                 if (const char* type = actuator->Attribute("biastype")) affine = std::string(type) == "affine";
-            } else throw std::runtime_error("MJCF: actuator '" + name + "' of type '" + tag + "' is not supported on this path");
+            } else throw Unsupported("MJCF: actuator '" + name + "' of type '" + tag + "' is not supported on this path");
             const char* joint_name = actuator->Attribute("joint");
             const auto found = joint_name != nullptr ? joint_links.find(joint_name) : joint_links.end();
             if (found == joint_links.end()) throw std::runtime_error("MJCF: actuator '" + name + "' needs a known joint transmission");

@@ -5,6 +5,7 @@
 #include <array>
 #include <cstdint>
 #include <memory>
+#include <stdexcept>
 #include <string>
 #include <vector>
 
@@ -38,7 +39,13 @@ struct Scene {
     void Bind();   // points `desc` at the arrays
 };
 
-// Throws std::runtime_error with the reason when the file cannot be read or uses what this path does not build.
+// A well-formed file that uses what this path does not build (a ball joint, a mimic joint, an actuator kind).
+struct Unsupported : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+
+// Throws std::runtime_error with the reason when the file cannot be read, Unsupported when it uses what this path does
+// not build.
 std::unique_ptr<Scene> LoadMjcf(const std::string& path, uint32_t flags);
 std::unique_ptr<Scene> LoadUrdf(const std::string& path, uint32_t flags);
 

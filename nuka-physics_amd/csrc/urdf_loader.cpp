@@ -112,7 +112,7 @@ std::unique_ptr<Scene> LoadUrdf(const std::string& path, uint32_t flags) {
         if (type == "revolute" || type == "continuous") link.joint_type = 0u;
         else if (type == "prismatic") link.joint_type = 1u;
         else if (type == "fixed") link.joint_type = 2u;
-        else throw std::runtime_error("URDF: joint '" + name + "' of type '" + type + "' is not supported on this path");
+        else throw Unsupported("URDF: joint '" + name + "' of type '" + type + "' is not supported on this path");
         ParseOrigin(e.First("origin"), &link.position, &link.rotation);
         link.axis = V3{1.0f, 0.0f, 0.0f};
         if (const Element* axis = e.First("axis")) if (axis->Attribute("xyz")) link.axis = ParseV3(axis->Attribute("xyz"));
@@ -132,7 +132,7 @@ std::unique_ptr<Scene> LoadUrdf(const std::string& path, uint32_t flags) {
             QueryFloat(*dynamics, "friction", &link.frictionloss);
         }
         if (link.damping < 0.0f || link.frictionloss < 0.0f || effort < 0.0f) throw std::runtime_error("URDF: joint '" + name + "' has a negative damping, friction or effort");
-        if (e.First("mimic") != nullptr) throw std::runtime_error("URDF: mimic joint '" + name + "' is not supported on this path");
+        if (e.First("mimic") != nullptr) throw Unsupported("URDF: mimic joint '" + name + "' is not supported on this path");
         if (effort > 0.0f && link.joint_type <= 1u) {   // a torque motor bounded by the effort (urdf_importer.cpp:631-638)
             link.drive_force_limit = effort;
             ++parts.actuator_count;

@@ -316,7 +316,7 @@ struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
     nuka_phi_backend* backend = nullptr;
     const nuka_phi_backend_i* be = nullptr;
     HostModel host;
-    nuka_world_desc_t cfg{};
+    nuka_hip_world_desc_t cfg{};
     uint32_t env_count = 0u;
     nuka_phi_buffer* arena = nullptr;
     nuka_phi_buffer* initial = nullptr;   // the state after creation, for nuka_world_reset
@@ -437,7 +437,7 @@ const nuka_phi_buffer_i* Iface(nuka_phi_buffer* b) { return reinterpret_cast<nuk
 void BuildPipeline(World& w) {
     const ModelView& m = w.model;
     const uint32_t E = w.env_count, nl = m.links_per_env, nb = m.bodies_per_env;
-    const nuka_world_desc_t& cfg = w.cfg;
+    const nuka_hip_world_desc_t& cfg = w.cfg;
     const bool has_contacts = m.rows_per_env > 0u;
     // A step of several substeps runs the interval below that many times at dt / substeps (pipeline.cpp:63-69).
     const uint32_t substeps = std::max(1u, cfg.solver_substeps);
@@ -650,7 +650,7 @@ nuka_result_t nuka_device_create(const nuka_device_desc_t* desc, nuka_device_han
     }
     const uint32_t index = desc->gpu_index;
     if (index >= uint32_t(count)) return Error(NUKA_RESULT_DEVICE_ERROR, "no HIP device with this gpu_index");
-    void* backend = CreateBackend(int(index), desc->stream);
+    void* backend = CreateBackend(int(index), desc->cuda_stream);
     if (backend == nullptr) return Error(NUKA_RESULT_DEVICE_ERROR, "backend creation failed");
     // CreateBackend has made this GPU current: its copy of the static staging array is looked up once
     if (index < uint32_t(kMaxGpus) && g_static_reset_ids[index] == nullptr) {
@@ -683,7 +683,7 @@ nuka_phi_backend* nuka_device_backend(nuka_device_handle device) {
 
 namespace nkh {
 namespace {
-nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t* tmpl, const nuka_world_desc_t* desc,
+nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t* tmpl, const nuka_hip_world_desc_t* desc,
                           const scene_file::Scene* scene, nuka_world_handle* out) {
     if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
     *out = nullptr;
@@ -692,14 +692,14 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
     // a caller built against the header before the joint-row members passes the shorter size; those members read as zero
     constexpr size_t kTemplateBase = offsetof(nuka_template_desc_t, joint_limit_lower);
     constexpr size_t kTemplateJointRows = offsetof(nuka_template_desc_t, excluded_pairs);
-    constexpr size_t kWorldBase = offsetof(nuka_world_desc_t, solver_fold_drive_damping);
-    constexpr size_t kWorldDrives = offsetof(nuka_world_desc_t, solver_substeps);
+    constexpr size_t kWorldBase = offsetof(nuka_hip_world_desc_t, solver_fold_drive_damping);
+    constexpr size_t kWorldDrives = offsetof(nuka_hip_world_desc_t, solver_substeps);
     if ((tmpl->struct_size != sizeof(nuka_template_desc_t) && tmpl->struct_size != kTemplateJointRows && tmpl->struct_size != kTemplateBase) ||
-        (desc->struct_size != sizeof(nuka_world_desc_t) && desc->struct_size != kWorldDrives && desc->struct_size != kWorldBase))
+        (desc->struct_size != sizeof(nuka_hip_world_desc_t) && desc->struct_size != kWorldDrives && desc->struct_size != kWorldBase))
         return Error(NUKA_RESULT_INVALID_ARG, "struct_size mismatch");
     nuka_template_desc_t template_copy{};
     std::memcpy(&template_copy, tmpl, tmpl->struct_size);
-    nuka_world_desc_t desc_copy{};
+    nuka_hip_world_desc_t desc_copy{};
     std::memcpy(&desc_copy, desc, desc->struct_size);
     tmpl = &template_copy;
     desc = &desc_copy;
@@ -711,7 +711,7 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
         w.be = reinterpret_cast<nuka_phi_backend_head*>(w.backend)->iface;
         Cook(*tmpl, &w.host);
         w.cfg = *desc;
-        nuka_world_desc_t& cfg = w.cfg;   // nuka.h:160-173 defaults; pipeline.hpp SolverConfig; op_schema.hpp:598, 663
+        nuka_hip_world_desc_t& cfg = w.cfg;   // nuka.h:160-173 defaults; pipeline.hpp SolverConfig; op_schema.hpp:598, 663
         if (cfg.fixed_dt <= 0.0f) cfg.fixed_dt = 1.0f / 240.0f;
         if (cfg.solver_vel_iters == 0u) cfg.solver_vel_iters = 10u;
         if (cfg.solver_pos_iters == 0u) cfg.solver_pos_iters = 4u;
@@ -814,7 +814,7 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
 }  // namespace nkh
 
 nuka_result_t nuka_world_create_from_template(nuka_device_handle device, const nuka_template_desc_t* tmpl,
-                                              const nuka_world_desc_t* desc, nuka_world_handle* out) {
+                                              const nuka_hip_world_desc_t* desc, nuka_world_handle* out) {
     return CreateWorld(device, tmpl, desc, nullptr, out);
 }
 
@@ -887,17 +887,79 @@ nuka_result_t nuka_scene_initial_state(nuka_scene_handle scene, float* q, float*
     return NUKA_RESULT_OK;
 }
 
-nuka_result_t nuka_world_create_from_scene(nuka_device_handle device, nuka_scene_handle scene, const nuka_world_desc_t* desc,
-                                           nuka_world_handle* out) {
+nuka_result_t nuka_hip_world_create_from_scene_handle(nuka_device_handle device, nuka_scene_handle scene,
+                                                      const nuka_hip_world_desc_t* desc, nuka_world_handle* out) {
     const auto* s = reinterpret_cast<const scene_file::Scene*>(scene);
     if (s == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "scene is null");
     if (desc == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "desc is null");
-    if (desc->struct_size != sizeof(nuka_world_desc_t)) return Error(NUKA_RESULT_INVALID_ARG, "struct_size mismatch");
-    nuka_world_desc_t with_file = *desc;
+    if (desc->struct_size != sizeof(nuka_hip_world_desc_t)) return Error(NUKA_RESULT_INVALID_ARG, "struct_size mismatch");
+    nuka_hip_world_desc_t with_file = *desc;
     if (with_file.fixed_dt <= 0.0f) with_file.fixed_dt = s->timestep;
     if (with_file.gravity[0] == 0.0f && with_file.gravity[1] == 0.0f && with_file.gravity[2] == 0.0f)
         std::copy(s->gravity, s->gravity + 3, with_file.gravity);
     return CreateWorld(device, &s->desc, &with_file, s, out);
+}
+
+// nuka_world_create_from_scene (nuka.h:175-177; src/c_abi/world.cpp:493-527, 590-635): the reference's descriptor, the
+// scene file read by its extension (LoadSceneByExtension, world.cpp:60-82).
+nuka_result_t nuka_world_create_from_scene(nuka_device_handle device, const nuka_world_desc_t* desc, nuka_world_handle* out) {
+    if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    *out = nullptr;
+    if (desc == nullptr || desc->scene_path == nullptr || !(desc->fixed_dt > 0.0f) || desc->env_count == 0u)
+        return Error(NUKA_RESULT_INVALID_ARG, "desc, scene_path, a positive fixed_dt and env_count are required");
+    if (desc->determinism > 1u) return Error(NUKA_RESULT_INVALID_ARG, "determinism is 0 or 1");
+    if (desc->control_mode > 5u) return Error(NUKA_RESULT_INVALID_ARG, "unknown control mode");
+    if (device == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "device is null");
+    if (desc->control_mode == 3u || desc->control_mode == 4u)
+        return Error(NUKA_RESULT_NOT_SUPPORTED, "the computed-torque and OSC control modes are not built");
+    const bool terrain = desc->terrain_step_height != 0.0f || desc->terrain_step_width != 0.0f || desc->terrain_platform_width != 0.0f ||
+                         desc->terrain_grid_width != 0.0f || desc->terrain_grid_height_max != 0.0f || desc->contact_family != 0u ||
+                         desc->heightfield_terrain_type != 0u || desc->heightfield_nrow != 0u || desc->heightfield_ncol != 0u ||
+                         desc->heightfield_cell != 0.0f || (desc->heightfield_image_path != nullptr && desc->heightfield_image_path[0] != '\0') ||
+                         desc->heightfield_radius_x != 0.0f || desc->heightfield_radius_y != 0.0f || desc->heightfield_elevation_z != 0.0f ||
+                         desc->heightfield_base_z != 0.0f || desc->curric_levels != 0u || desc->curric_types != 0u ||
+                         desc->terrain_feature_cell != 0.0f;
+    if (terrain) return Error(NUKA_RESULT_NOT_SUPPORTED, "terrain and heightfield members must be zero: no heightfield path is built");
+    if (desc->instance_count > 1u) return Error(NUKA_RESULT_NOT_SUPPORTED, "one articulation per environment: instance_count must be 0 or 1");
+    if (desc->cloth_integrator != 0u || desc->ogc_contact_capacity != 0u)
+        return Error(NUKA_RESULT_NOT_SUPPORTED, "cloth_integrator and ogc_contact_capacity must be zero: no particle path is built");
+    const std::string path(desc->scene_path);
+    const size_t dot = path.find_last_of('.');
+    const size_t slash = path.find_last_of("/\\");
+    const std::string extension = dot == std::string::npos || (slash != std::string::npos && dot < slash) ? std::string() : path.substr(dot);
+    const bool mjcf = extension == ".xml" || extension == ".mjcf", urdf = extension == ".urdf";
+    if (!mjcf && !urdf) return Error(NUKA_RESULT_NOT_SUPPORTED, "scene files are read as MJCF (.xml, .mjcf) or URDF (.urdf)");
+    {
+        std::FILE* probe = std::fopen(path.c_str(), "rb");
+        if (probe == nullptr) return Error(NUKA_RESULT_FILE_NOT_FOUND, "cannot open " + path);
+        std::fclose(probe);
+    }
+    std::unique_ptr<scene_file::Scene> scene;
+    try {
+        scene = mjcf ? scene_file::LoadMjcf(path.c_str(), 0u) : scene_file::LoadUrdf(path.c_str(), 0u);
+    } catch (const std::bad_alloc&) {
+        return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
+    } catch (const scene_file::Unsupported& e) {
+        return Error(NUKA_RESULT_NOT_SUPPORTED, e.what());
+    } catch (const std::exception& e) {
+        return Error(NUKA_RESULT_PARSE_ERROR, e.what());
+    }
+    nuka_template_desc_t tmpl = scene->desc;
+    tmpl.drive_mode = desc->control_mode;
+    nuka_hip_world_desc_t options{};
+    options.struct_size = sizeof(options);
+    options.env_count = desc->env_count;
+    options.fixed_dt = desc->fixed_dt;
+    const bool no_gravity = desc->gravity_x == 0.0f && desc->gravity_y == 0.0f && desc->gravity_z == 0.0f;
+    options.gravity[0] = desc->gravity_x; options.gravity[1] = desc->gravity_y; options.gravity[2] = no_gravity ? -9.81f : desc->gravity_z;
+    options.solver_vel_iters = desc->solver_vel_iters;
+    options.solver_pos_iters = desc->solver_pos_iters;
+    options.solver_contact_margin = desc->solver_contact_margin;
+    options.solver_baumgarte_max_velocity = desc->solver_baumgarte_max_velocity;
+    options.solver_overlap_recovery_velocity = desc->solver_overlap_recovery_velocity;
+    options.solver_substeps = desc->solver_substeps;
+    options.contact_detection_substeps = desc->contact_detection_substeps;
+    return CreateWorld(device, &tmpl, &options, scene.get(), out);
 }
 
 void nuka_world_destroy(nuka_world_handle world) {
@@ -1066,14 +1128,63 @@ const char* nuka_field_names(void) {
 }
 
 nuka_state_field_t nuka_field_from_name(const char* name) {
-    if (name == nullptr) return 0xFFFFFFFFu;
+    if (name == nullptr) return NUKA_HIP_FIELD_NONE;
     uint32_t index = 0u;
-#define X(field, ...) if (std::strcmp(name, #field) == 0) return index; ++index;
+#define X(field, ...) if (std::strcmp(name, #field) == 0) return nuka_state_field_t(uint32_t(NUKA_HIP_FIELD_BASE) + index); ++index;
     NKH_MODEL_FIELDS(X)
     NKH_DATA_FIELDS(X)
 #undef X
-    return 0xFFFFFFFFu;
+    return NUKA_HIP_FIELD_NONE;
 }
+
+namespace nkh {
+namespace {
+// The public field ids this library serves: the world's field behind each and the element stride of its view
+// (src/c_abi/dlpack_table.hpp:101-330; element sizes of src/nk/model/fields.yaml).
+struct PublicField { nuka_state_field_t id; const char* name; uint32_t stride; };
+constexpr PublicField kPublicFields[] = {
+    {NUKA_FIELD_RIGID_BODY_TRANSFORM, "body_pose", 28u}, {NUKA_FIELD_ARTICULATION_LINK_POSE, "link_pose", 28u},
+    {NUKA_FIELD_JOINT_POSITION, "q", 4u}, {NUKA_FIELD_JOINT_VELOCITY, "qdot", 4u}, {NUKA_FIELD_CONTACT_POINTS, "contact_point", 12u},
+    {NUKA_FIELD_DRIVE_TARGET, "drive_target", 4u}, {NUKA_FIELD_LINK_VELOCITY, "link_velocity", 24u},
+    {NUKA_FIELD_DRIVE_STIFFNESS, "drive_stiffness", 4u}, {NUKA_FIELD_DRIVE_DAMPING, "drive_damping", 4u},
+    {NUKA_FIELD_DRIVE_FORCE_LIMIT, "drive_force_limit", 4u}, {NUKA_FIELD_BASE_POSE, "base_pose", 28u},
+    {NUKA_FIELD_TORQUE_INPUT, "drive_target", 4u}, {NUKA_FIELD_VELOCITY_TARGET, "velocity_target", 4u},
+    {NUKA_FIELD_ACTUATOR_NOLOAD_SPEED, "actuator_noload_speed", 4u}, {NUKA_FIELD_LINK_CONTACT_WRENCH, "link_contact_wrench", 24u},
+    {NUKA_FIELD_CONTACT_NORMAL, "contact_normal", 12u}, {NUKA_FIELD_CONTACT_FORCE, "contact_force", 12u},
+    {NUKA_FIELD_CONTACT_LINK, "contact_link", 4u}, {NUKA_FIELD_JOINT_FEEDFORWARD, "joint_f", 4u},
+    {NUKA_FIELD_JOINT_LIMIT_IMPULSE, "joint_limit_impulse", 8u}, {NUKA_FIELD_ACTUATOR_EFFORT_REQUESTED, "actuator_effort_requested", 4u},
+    {NUKA_FIELD_ACTUATOR_EFFORT, "actuator_effort", 4u}, {NUKA_FIELD_ACTUATOR_SATURATED, "actuator_saturated", 4u},
+    {NUKA_FIELD_CONTACT_SIDE_A_KIND, "contact_side_a_kind", 4u}, {NUKA_FIELD_CONTACT_SIDE_B_KIND, "contact_side_b_kind", 4u},
+    {NUKA_FIELD_CONTACT_SIDE_A_INDEX, "contact_side_a_index", 4u}, {NUKA_FIELD_CONTACT_SIDE_B_INDEX, "contact_side_b_index", 4u},
+    {NUKA_FIELD_ENV_STATUS, "env_status", 4u}, {NUKA_FIELD_CONTACT_WARM_START_COUNTS, "contact_warm_start_counts", 8u},
+    {NUKA_FIELD_VBD_VELOCITY_SWEEP_COUNT, "vbd_velocity_sweep_count", 4u}, {NUKA_FIELD_UCONTACT_ROW_RANGE, "ucontact_row_range", 8u},
+    {NUKA_FIELD_LINK_WRENCH, "link_wrench", 24u}, {NUKA_FIELD_UCONTACT_COUNT, "ucontact_count", 4u},
+    {NUKA_FIELD_UCONTACT_POINT, "ucontact_point", 48u}, {NUKA_FIELD_SOLVER_RESIDUAL, "solver_residual", 16u},
+    {NUKA_FIELD_UCONTACT_NORMAL, "ucontact_normal", 48u}, {NUKA_FIELD_UCONTACT_DEPTH, "ucontact_depth", 16u},
+    {NUKA_FIELD_UCONTACT_LAW, "ucontact_law", 4u}, {NUKA_FIELD_UCONTACT_SIDE_A, "ucontact_a", 16u},
+    {NUKA_FIELD_UCONTACT_SIDE_B, "ucontact_b", 16u}, {NUKA_FIELD_UCONTACT_IMPULSE, "ucontact_impulse", 48u},
+    {NUKA_FIELD_JOINT_GRAVITY_FORCE, "joint_gravity_force", 4u}, {NUKA_FIELD_ROW_PENETRATION, "row_penetration", 4u},
+    {NUKA_FIELD_ROW_LAMBDA, "lambda", 4u},
+};
+
+// The world's field a public or library id stands for and the stride of its view; null when the id is not served.
+const Field* ResolveField(const World& w, nuka_state_field_t field, uint32_t* stride) {
+    const uint32_t id = uint32_t(field);
+    if (id >= uint32_t(NUKA_HIP_FIELD_BASE)) {
+        const uint32_t index = id - uint32_t(NUKA_HIP_FIELD_BASE);
+        if (index >= w.fields.size()) return nullptr;
+        *stride = w.fields[index].elem_bytes;
+        return &w.fields[index];
+    }
+    for (const PublicField& entry : kPublicFields) {
+        if (uint32_t(entry.id) != id) continue;
+        for (const Field& f : w.fields)
+            if (std::strcmp(f.name, entry.name) == 0) { *stride = entry.stride; return &f; }
+    }
+    return nullptr;
+}
+}  // namespace
+}  // namespace nkh
 
 namespace nkh {
 namespace {
@@ -1103,12 +1214,14 @@ nuka_result_t nuka_world_get_buffer_view(nuka_world_handle world, nuka_state_fie
     auto* w = reinterpret_cast<World*>(world);
     if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
     if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
-    if (field >= w->fields.size()) return Error(NUKA_RESULT_NOT_SUPPORTED, "unknown field");
-    const Field& f = w->fields[field];
+    uint32_t stride = 0u;
+    const Field* resolved = ResolveField(*w, field, &stride);
+    if (resolved == nullptr) return Error(NUKA_RESULT_NOT_SUPPORTED, "this world serves no field of that id");
+    const Field& f = *resolved;
     if (const nuka_result_t demanded = DemandReadout(*w, f); demanded != NUKA_RESULT_OK) return demanded;
     out->device_ptr = static_cast<char*>(Iface(w->arena)->base(w->arena)) + f.offset;
-    out->element_count = f.count;
-    out->element_stride_bytes = f.elem_bytes;
+    out->element_count = f.count * f.elem_bytes / stride;
+    out->element_stride_bytes = stride;
     out->dtype = uint8_t(f.dtype);
     return NUKA_RESULT_OK;
 }
@@ -1116,8 +1229,10 @@ nuka_result_t nuka_world_get_buffer_view(nuka_world_handle world, nuka_state_fie
 nuka_result_t nuka_world_upload_field(nuka_world_handle world, nuka_state_field_t field, const void* bytes, size_t nbytes, size_t byte_offset) {
     auto* w = reinterpret_cast<World*>(world);
     if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
-    if (field >= w->fields.size()) return Error(NUKA_RESULT_NOT_SUPPORTED, "unknown field");
-    const Field& f = w->fields[field];
+    uint32_t stride = 0u;
+    const Field* resolved = ResolveField(*w, field, &stride);
+    if (resolved == nullptr) return Error(NUKA_RESULT_NOT_SUPPORTED, "this world serves no field of that id");
+    const Field& f = *resolved;
     const size_t size = f.count * f.elem_bytes;
     if (byte_offset > size || nbytes > size - byte_offset || (bytes == nullptr && nbytes > 0u)) return Error(NUKA_RESULT_INVALID_ARG, "range exceeds the field");
     if (nbytes == 0u) return NUKA_RESULT_OK;
@@ -1127,8 +1242,10 @@ nuka_result_t nuka_world_upload_field(nuka_world_handle world, nuka_state_field_
 nuka_result_t nuka_world_download_field(nuka_world_handle world, nuka_state_field_t field, void* bytes, size_t nbytes, size_t byte_offset) {
     auto* w = reinterpret_cast<World*>(world);
     if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
-    if (field >= w->fields.size()) return Error(NUKA_RESULT_NOT_SUPPORTED, "unknown field");
-    const Field& f = w->fields[field];
+    uint32_t stride = 0u;
+    const Field* resolved = ResolveField(*w, field, &stride);
+    if (resolved == nullptr) return Error(NUKA_RESULT_NOT_SUPPORTED, "this world serves no field of that id");
+    const Field& f = *resolved;
     const size_t size = f.count * f.elem_bytes;
     if (byte_offset > size || nbytes > size - byte_offset || (bytes == nullptr && nbytes > 0u)) return Error(NUKA_RESULT_INVALID_ARG, "range exceeds the field");
     if (nbytes == 0u) return NUKA_RESULT_OK;

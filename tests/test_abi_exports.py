@@ -35,7 +35,7 @@ def test_headers_compile_as_c_and_agree_with_the_ctypes_mirror(tmp_path):
     """include/*.h are plain C: a C99 program that includes them reports the size of each descriptor and the offset of
     every member the ctypes mirror declares, and the two layouts agree."""
     import subprocess
-    members = {"nuka_template_desc_t": nk.abi.TemplateDescC, "nuka_world_desc_t": nk.abi.WorldDescC, "nuka_scene_info_t": nk.SceneInfoC,
+    members = {"nuka_template_desc_t": nk.abi.TemplateDescC, "nuka_hip_world_desc_t": nk.abi.WorldDescC, "nuka_world_desc_t": nk.abi.SceneWorldDescC, "nuka_device_desc_t": nk.DeviceDescC, "nuka_scene_info_t": nk.SceneInfoC,
                "nuka_param_info_t": nk.ParamInfoC, "nuka_world_execution_info_t": nk.ExecutionInfoC, "nuka_world_info_t": nk.WorldInfoC,
                "nuka_buffer_view_t": nk.abi.BufferViewC}
     lines = ['#include <stddef.h>', '#include <stdio.h>', '#include "nuka_phi.h"', '#include "nuka_hip.h"', 'int main(void) {']
@@ -77,8 +77,13 @@ def test_field_names_cover_the_seam_fields():
                  "shape_table", "drive_target", "drive_stiffness", "drive_damping", "drive_force_limit", "velocity_target",
                  "joint_f", "drive_command", "actuator_effort", "joint_limit_impulse"):
         assert name in fields
-        assert lib.nuka_field_from_name(name.encode()) == fields.index(name)
-    assert lib.nuka_field_from_name(b"no_such_field") == 0xFFFFFFFF
+        assert lib.nuka_field_from_name(name.encode()) == nk.FIELD_BASE + fields.index(name)     # the library's own ids
+    assert lib.nuka_field_from_name(b"no_such_field") == nk.FIELD_NONE
+    # every public id the header declares names a field of the world, and no library id collides with a public one
+    header = open(os.path.join(ROOT, "include", "nuka_hip.h")).read()
+    declared = {m.group(1): int(m.group(2)) for m in re.finditer(r"NUKA_FIELD_(\w+) = (\d+)", header)}
+    assert declared == {k: v[0] for k, v in nk.abi.PUBLIC_FIELDS.items()}
+    assert all(v[1] in fields for v in nk.abi.PUBLIC_FIELDS.values()) and max(declared.values()) < nk.FIELD_BASE
 
 
 def test_result_messages():

@@ -158,3 +158,70 @@ def test_scene_with_unsupported_collision_geometry_is_refused(device, tmp_path):
     world.step(2); world.synchronize()
     assert not world.download("env_status").any()
     world.close()
+
+
+def test_reference_entry_point_reads_the_scene_file_named_by_the_descriptor(device, tmp_path):
+    """nuka_world_create_from_scene(device, desc, out) with the reference's descriptor layout: the file is read by its
+    extension, the world steps exactly as one made from the loaded scene handle with the same options, and the public
+    field ids give views with the reference's element strides over the same bytes."""
+    import ctypes as C
+    E = 64
+    ref_desc = abi.SceneWorldDescC()
+    ref_desc.scene_path = WALKER.encode()
+    ref_desc.env_count, ref_desc.fixed_dt, ref_desc.solver_vel_iters = E, 0.004, 8
+    ref_desc.control_mode = abi.DRIVE_PD_POSITION
+    world = nk.World(device, None, ref_desc)
+    scene = nk.Scene(WALKER, 0)
+    twin = nk.World(device, scene, abi.world_desc(E, 0.004, gravity=(0.0, 0.0, -9.81), vel_iters=8))
+    rng = np.random.default_rng(3)
+    target = rng.normal(0, 0.2, (E, scene.link_count)).astype(np.float32)
+    for w in (world, twin):
+        w.upload("drive_target", target)
+        w.step(5)
+        w.synchronize()
+    for name in ("q", "qdot", "link_pose", "base_pose", "lambda", "env_status", "contact_count"):
+        assert np.array_equal(world.download(name), twin.download(name)), name
+    nl = scene.link_count
+    for public, (fid, name, stride) in abi.PUBLIC_FIELDS.items():
+        view, raw = world.public_view(public)
+        assert view.element_stride_bytes == stride, public
+        inner = world.download(name)
+        assert view.element_count * stride == inner.nbytes and np.array_equal(raw, inner.view(np.uint8)), public
+    view, _ = world.public_view("ARTICULATION_LINK_POSE")
+    assert view.element_count == E * nl and view.dtype == 0
+    view, _ = world.public_view("ENV_STATUS")
+    assert view.element_count == E and view.dtype == 1
+    # a public id this library does not serve, and the write path through a public id
+    out = abi.BufferViewC()
+    assert nk.lib().nuka_world_get_buffer_view(world._h, 4, C.byref(out)) == abi.RESULT_NOT_SUPPORTED      # OBSERVATIONS
+    q = np.full(E * nl, 0.25, np.float32)
+    assert nk.lib().nuka_world_upload_field(world._h, abi.PUBLIC_FIELDS["JOINT_POSITION"][0], q.ctypes.data, q.nbytes, 0) == 0
+    assert np.array_equal(world.download("q"), q)
+    world.close()
+    twin.close()
+    # the descriptor's own error contract (src/c_abi/world.cpp:493-527, 60-82)
+    handle = C.c_void_p()
+    lib = nk.lib()
+
+    def create(**changes):
+        d = abi.SceneWorldDescC()
+        d.scene_path, d.env_count, d.fixed_dt = WALKER.encode(), 4, 0.004
+        for k, v in changes.items():
+            setattr(d, k, v)
+        code = lib.nuka_world_create_from_scene(device._h, C.byref(d), C.byref(handle))
+        if code == 0:
+            lib.nuka_world_destroy(handle)
+        return code
+
+    assert create() == 0
+    assert create(fixed_dt=0.0) == abi.RESULT_INVALID_ARG and create(env_count=0) == abi.RESULT_INVALID_ARG
+    assert create(determinism=2) == abi.RESULT_INVALID_ARG and create(control_mode=6) == abi.RESULT_INVALID_ARG
+    assert create(scene_path=None) == abi.RESULT_INVALID_ARG
+    assert create(control_mode=4) == abi.RESULT_NOT_SUPPORTED and create(instance_count=2) == abi.RESULT_NOT_SUPPORTED
+    assert create(contact_family=1) == abi.RESULT_NOT_SUPPORTED and create(terrain_step_height=0.1) == abi.RESULT_NOT_SUPPORTED
+    assert create(scene_path=b"/no/such/file.xml") == 4                                     # NUKA_RESULT_FILE_NOT_FOUND
+    assert create(scene_path=b"/tmp/robot.usda") == abi.RESULT_NOT_SUPPORTED and create(scene_path=b"/tmp/robot.nks") == abi.RESULT_NOT_SUPPORTED
+    broken = tmp_path / "broken.xml"
+    broken.write_text("<mujoco><worldbody><body>")
+    assert create(scene_path=str(broken).encode()) == 5                                      # NUKA_RESULT_PARSE_ERROR
+    assert lib.nuka_world_create_from_scene(None, C.byref(abi.SceneWorldDescC(WALKER.encode(), 4, 0.004)), C.byref(handle)) == abi.RESULT_NULL_HANDLE
