@@ -14,6 +14,7 @@
 #ifndef NUKA_PHI_H_
 #define NUKA_PHI_H_
 
+#include <stdbool.h>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -102,7 +103,7 @@ typedef struct nuka_phi_device_i {
     nuka_phi_backend* (*init_backend)(nuka_phi_device*, const char* params_json);
     nuka_phi_buffer_type* (*get_buffer_type)(nuka_phi_device*);
     nuka_phi_buffer_type* (*get_host_buffer_type)(nuka_phi_device*);
-    int (*supports_op)(nuka_phi_device*, uint16_t op);
+    bool (*supports_op)(nuka_phi_device*, uint16_t op);   /* bool, as DeviceI::supports_op (src/phi/backend.hpp:114) */
 } nuka_phi_device_i;
 
 typedef struct nuka_phi_registry_entry_i {

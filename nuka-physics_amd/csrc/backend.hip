@@ -15,10 +15,10 @@ namespace nkh {
 
 const char* OpName(NkOp op) {
     static const char* const names[] = {
-        "ApplyDrives", "ArticulationDynamics", "IntegrateVelocity", "FkWorldPoses", "IntegratePosition", "BuildAabbs",
-        "LbvhBuild", "LbvhQueryPairs", "NarrowphasePrimitives", "AssembleRows", "SyncLinkBodyPose", "NarrowphaseHeightfield",
-        "ContactWarmStart", "SnapshotStepVelocity", "FkLinkVelocities", "BlockDescentSolve", "ResetEnvs", "SnapshotState",
-        "RestoreState", "ReadoutDrives", "ReadoutContactWrench", "AccumulateStep"};
+#define X(name) #name,
+        NKH_OP_CATALOG(X)
+#undef X
+    };
     return op < NkOp::Count ? names[static_cast<uint16_t>(op)] : "?";
 }
 
@@ -294,7 +294,7 @@ nuka_phi_backend* DevInitBackend(nuka_phi_device* d, const char*) {
 }
 nuka_phi_buffer_type* DevBufferType(nuka_phi_device* d) { return reinterpret_cast<nuka_phi_buffer_type*>(&reinterpret_cast<Device*>(d)->device_type); }
 nuka_phi_buffer_type* DevHostBufferType(nuka_phi_device* d) { return reinterpret_cast<nuka_phi_buffer_type*>(&reinterpret_cast<Device*>(d)->host_type); }
-int DevSupportsOp(nuka_phi_device*, uint16_t op) {
+bool DevSupportsOp(nuka_phi_device*, uint16_t op) {
     std::call_once(g_ops_once, RegisterOps);
     return op < uint16_t(NkOp::Count) && g_ops[op] != nullptr ? 1 : 0;
 }

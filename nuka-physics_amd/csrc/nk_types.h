@@ -10,12 +10,24 @@ namespace nkh {
 // src/phi/status.hpp
 enum class Status : uint8_t { Ok, Unsupported, Failed, OutOfMemory, InvalidArgument };
 
-// Subset of src/phi/op_catalog.inc in catalog order; ids are this backend's own.
+// The closed op set of src/phi/op_catalog.inc, in the catalog's order, so that an op id here is the reference's
+// NkOp value (src/phi/op_schema.hpp:60-65).  This backend serves the ops of the articulation step; the others have a
+// null slot in its table: supports_op answers 0 and a dispatch answers Unsupported.
+#define NKH_OP_CATALOG(X) \
+    X(ApplyDrives) X(ApplyDynamicsDrives) X(ArticulationDynamics) X(IntegrateVelocity) X(FkWorldPoses) X(IntegratePosition) \
+    X(BuildAabbs) X(LbvhBuild) X(LbvhQueryPairs) X(NarrowphasePrimitives) X(NarrowphaseSdf) X(AssembleRows) X(ParticleAeroDrag) \
+    X(ParticlePredict) X(ParticleFinalize) X(MpmPredict) X(MpmExchange) X(MpmCommit) X(ReadoutContactWrench) X(ExportObs) \
+    X(ResetEnvs) X(SnapshotState) X(RestoreState) X(RandomizeMaterialBuckets) X(RandomizeBodyParams) X(SyncLinkBodyPose) \
+    X(NarrowphaseBodyParticle) X(NarrowphaseHeightfield) X(ContactWarmStart) X(SnapshotStepVelocity) \
+    X(ParticleProjectionVelocity) X(ParticleContactDelta) X(AccumulateStep) X(FkLinkVelocities) X(ReadoutDrives) \
+    X(RefitParticleSurfaces) X(SampleObservation) X(ResetObservation) X(ReadoutMotion) X(SampleStateSensor) X(AdvanceSensorTime) \
+    X(ReadoutSensorWrenches) X(ReadoutContactRegion) X(ClothPredict) X(ClothContactRestart) X(ClothFinalize) X(OgcDetect) \
+    X(ReadoutEnergyLedger) X(ReadoutContactAudit) X(MimicReduce) X(BlockDescentSolve) X(RecordTelemetry) X(ReferenceWeights) \
+    X(ArticulationDamping) X(ReadoutIntervalState) X(ContactRefresh)
 enum class NkOp : uint16_t {
-    ApplyDrives, ArticulationDynamics, IntegrateVelocity, FkWorldPoses, IntegratePosition, BuildAabbs, LbvhBuild,
-    LbvhQueryPairs, NarrowphasePrimitives, AssembleRows, SyncLinkBodyPose, NarrowphaseHeightfield, ContactWarmStart,
-    SnapshotStepVelocity, FkLinkVelocities, BlockDescentSolve, ResetEnvs, SnapshotState, RestoreState,
-    ReadoutDrives, ReadoutContactWrench, AccumulateStep,
+#define X(name) name,
+    NKH_OP_CATALOG(X)
+#undef X
     Count
 };
 
@@ -131,16 +143,29 @@ struct DataView {
     float *step_link_impulse, *step_link_moment, *step_joint_limit_impulse;
 };
 
-// --- parameter PODs (field names follow src/phi/op_schema.hpp) -------------------------------------------
-struct FkWorldPosesParams { uint32_t articulation_count, total_link_count; };
-struct FkLinkVelocitiesParams { uint32_t articulation_count, total_link_count; };
+// --- parameter PODs ----------------------------------------------------------------------------------------
+// Layout-identical to src/phi/op_schema.hpp for every op this backend serves: same members, order and types, so an
+// OpCall filled by the reference's Pipeline (src/nk/pipeline/pipeline.cpp:187-1020) reads correctly here.  Members
+// that describe what this path does not build (particles, grids, hulls, heightfields, cloth, telemetry) are carried and
+// must be zero where a nonzero value would ask for that work; an op answers Unsupported otherwise.  What the kernels
+// need beyond these members they derive from the ModelView.
 struct ApplyDrivesParams {   // op_schema.hpp:79-88
     float dt;
-    uint32_t total_link_count, defer_velocity_damping, mode, links_per_env, bodies_per_env, articulation_count;
-    float gravity[3];
-    uint32_t affine;   // this backend's own: 0 leaves `tau` as the applied generalized force (no drive rows cooked)
+    uint32_t total_link_count;
+    uint32_t defer_velocity_damping;
+    uint32_t mode;
+    uint32_t links_per_env;
+    uint32_t bodies_per_env = 0u;
+    uint32_t articulation_count = 0u;
+    float gravity[3] = {};
 };
-struct ReadoutDrivesParams { float dt; uint32_t total_link_count, links_per_env, rows_per_env, first_drive_row; };   // op_schema.hpp:100-106
+struct ReadoutDrivesParams {   // op_schema.hpp:100-106
+    float dt;
+    uint32_t total_link_count;
+    uint32_t links_per_env;
+    uint32_t rows_per_env;
+    uint32_t first_drive_row;
+};
 struct ArticulationDynamicsParams {   // op_schema.hpp:108-121
     float dt;
     uint32_t max_dof;
@@ -155,38 +180,229 @@ struct ArticulationDynamicsParams {   // op_schema.hpp:108-121
     uint32_t links_per_env = 0u;
     uint32_t bodies_per_env = 0u;
 };
-struct IntegrateVelocityParams { float dt; float gravity[3]; uint32_t total_body_count, clear_body_forces; };
-struct IntegratePositionParams { float dt; uint32_t total_link_count, articulation_count, total_body_count, env_count, pos_pass, mimic_couplings; };
-struct SyncLinkBodyPoseParams { uint32_t env_count, links_per_env, bodies_per_env, family, selected_env_count; };
-struct BuildAabbsParams { uint32_t env_count, bodies_per_env, family; float margin, dt, query_reach; };
-struct LbvhBuildParams { uint32_t env_count, bodies_per_env, family; };
-struct LbvhQueryPairsParams { uint32_t env_count, bodies_per_env, family, max_contacts_per_env, rigid_slot_cap, max_pairs, excluded_count; };
-struct NarrowphasePrimitivesParams { uint32_t env_count, bodies_per_env, union_slot_count, rigid_slot_cap; float contact_margin, dt, query_reach; };
-struct AssembleRowsParams {
-    uint32_t env_count, articulation_count, total_link_count, max_dof, union_slot_count, rows_per_env, contact_rows_per_env;
-    uint32_t full_row_slot_count, bodies_per_env, base_link_count, position_pass, family;
-    float dt, overlap_recovery_velocity, contact_margin;
-    uint32_t joint_limit_rows_per_env, joint_friction_rows_per_env, joint_drive_rows_per_env;
-    float baumgarte_max_velocity;
-};
-struct ContactWarmStartParams { uint32_t phase, env_count, slot_count, rows_per_env, full_row_slot_count, decay_steps; };
-struct BlockDescentSolveParams {   // op_schema.hpp:549-636 (the tile-route subset)
+struct IntegrateVelocityParams {   // op_schema.hpp:143-150
     float dt;
-    uint32_t env_count, rows_per_env, total_body_count, articulation_count, max_dof, max_independent_dof;
-    uint32_t base_link_count, contact_rows_per_env, contact_slots_per_env;
-    uint32_t iterations = 10u;
-    uint32_t position_iterations;
-    float position_beta, position_slop, position_max_velocity;
-    float velocity_tolerance;
+    float gravity[3];
+    uint32_t total_link_count;
+    uint32_t articulation_count;
+    uint32_t total_body_count;
+    uint32_t clear_body_forces = 1u;
+};
+struct SnapshotStepVelocityParams {   // op_schema.hpp:153-160
+    uint32_t env_count;
+    uint32_t articulation_count;
+    uint32_t max_dof;
+    uint32_t base_link_count;
+    uint32_t total_body_count;
+    uint32_t total_particle_count;
+};
+// op_schema.hpp:162-168; the flags this path uses (the particle and free-body ones have no counterpart here)
+constexpr uint32_t kAccumulateOutputs = 1u, kAccumulateLinkWrench = 2u, kAccumulateJointLimit = 4u, kFinalizeLinkWrench = 8u;
+struct AccumulateStepParams {   // op_schema.hpp:170-180
+    uint32_t env_count = 0u;
+    uint32_t bodies_per_env = 0u;
+    uint32_t links_per_env = 0u;
+    uint32_t artics_per_env = 0u;
+    uint32_t flags = 0u;
+    uint32_t first = 0u;
+    uint32_t last = 0u;
+    float substep_dt = 0.0f;
+    float inv_outer_dt = 0.0f;
+};
+struct FkWorldPosesParams {   // op_schema.hpp:182-187
+    uint32_t articulation_count;
+    uint32_t total_link_count;
+    uint32_t articulations_per_env;
+    uint32_t selected_env_count;
+};
+struct FkLinkVelocitiesParams {   // op_schema.hpp:189-192
+    uint32_t articulation_count;
+    uint32_t total_link_count;
+};
+struct IntegratePositionParams {   // op_schema.hpp:194-202
+    float dt;
+    uint32_t total_link_count;
+    uint32_t articulation_count;
+    uint32_t total_body_count;
+    uint32_t pos_pass;
+    uint32_t env_count = 1u;
+    uint32_t mimic_couplings = 0u;
+};
+struct BuildAabbsParams {   // op_schema.hpp:221-228
+    float dt = 0.0f;
+    float query_reach = 0.02f;   // collision/contact_query.hpp:16
+    float margin;
+    uint32_t family;
+    uint32_t env_count;
+    uint32_t bodies_per_env;
+};
+struct LbvhBuildParams {   // op_schema.hpp:230-236
+    uint32_t family;
+    uint32_t env_count;
+    uint32_t bodies_per_env;
+    uint64_t workspace_bytes = 0u;
+    uint32_t tree_queries = 0u;
+};
+struct LbvhQueryPairsParams {   // op_schema.hpp:238-249
+    uint32_t max_pairs;
+    uint32_t family;
+    uint32_t env_count;
+    uint32_t bodies_per_env;
+    uint32_t max_contacts_per_env;
+    uint32_t filter_cross_env;
+    uint32_t excluded_count;
+    uint32_t contact_pair_count = 0u;
+    uint32_t rigid_slot_cap;
+    uint64_t workspace_bytes;
+};
+struct NarrowphasePrimitivesParams {   // op_schema.hpp:392-413
+    float contact_margin;
+    uint32_t num_material_buckets;
+    uint32_t contact_pairs = 0u;
+    float dt = 0.0f;
+    float query_reach = 0.02f;
+    uint8_t max_contacts_per_pair;
+    float ground_height;
+    uint32_t foot_count;
+    uint32_t env_count;
+    uint32_t base_link_count;
+    uint32_t family;
+    uint32_t union_slot_count;
+    uint32_t rigid_slot_cap;
+    uint32_t bodies_per_env;
+    uint32_t hull_vert_count;
+    uint32_t particles_per_env;
+    uint32_t articulations_per_env;
+    uint32_t max_foot_contacts;
+    uint32_t max_body_samples;
+    uint32_t convex_pairs;
+};
+struct SyncLinkBodyPoseParams {   // op_schema.hpp:434-440
+    uint32_t family;
+    uint32_t env_count;
+    uint32_t links_per_env;
+    uint32_t bodies_per_env;
+    uint32_t selected_env_count;
+};
+struct NarrowphaseHeightfieldParams {   // op_schema.hpp:442-457
+    uint32_t family;
+    uint32_t env_count;
+    uint32_t slot_stride;
+    uint32_t rigid_slot_cap;
+    uint32_t bodies_per_env;
+    uint32_t hull_vert_count;
+    float contact_margin;
+    uint32_t has_heightfield;
+    float origin_x, origin_y, origin_z;
+    float cell_size;
+    uint32_t nrow, ncol;
+    float min_z, max_z;
+    uint32_t data_offset;
+    uint32_t hf_body_row;
+};
+struct VertexBlockLayout {   // op_schema.hpp:535-547; all zero on this path
+    uint32_t begin = 0u;
+    uint32_t vertices = 0u;
+    uint32_t dynamic_vertices = 0u;
+    uint32_t colors = 0u;
+    uint32_t particles_per_env = 0u;
+    uint32_t env_count = 0u;
+    uint32_t elements = 0u;
+    uint32_t coarse_levels = 0u;
+    uint32_t coarse_nodes = 0u;
+    uint32_t coarse_dense_nodes = 0u;
+};
+struct AssembleRowsParams {   // op_schema.hpp:549-594
+    uint32_t grid_nodes_per_env = 0u;
+    float dt;
+    uint32_t slot_count;
+    uint32_t max_dof;
+    uint32_t env_count;
+    uint32_t articulation_count;
+    uint32_t total_link_count;
+    uint32_t family;
+    uint32_t union_slot_count;
+    uint32_t rows_per_env;
+    uint32_t contact_rows_per_env;
     uint32_t joint_limit_rows_per_env;
+    uint32_t joint_friction_rows_per_env;
+    uint32_t joint_drive_rows_per_env;
+    uint32_t mimic_couplings_per_env;
+    uint32_t full_row_slot_count;
+    uint32_t ogc_slot_count = 0u;
+    uint32_t bodies_per_env;
+    uint32_t base_link_count;
+    float solref[2];
+    float solimp[5];
+    float impratio;
+    bool refsafe;
+    uint32_t cone;
+    uint32_t particles_per_env;
+    uint32_t num_material_buckets;
+    uint32_t contact_pairs = 0u;
+    float baumgarte_max_velocity;
+    float contact_margin;
+    uint32_t position_pass = 0u;
+    float overlap_recovery_velocity = 0.0f;
+    uint32_t point_endpoints_per_env = 0u;
+    uint32_t point_endpoint_terms_per_env = 0u;
+    VertexBlockLayout vertex_blocks{};
+    uint32_t measure_contact_response = 0u;
+};
+struct BlockDescentSolveParams {   // op_schema.hpp:596-640
+    float dt;
+    uint32_t iterations = 10u;
+    uint32_t env_count = 0u;
+    uint32_t rows_per_env = 0u;
+    uint32_t total_particle_count = 0u;
+    uint32_t total_body_count = 0u;
+    uint32_t total_grid_count = 0u;
+    uint32_t articulation_count = 0u;
+    uint32_t max_dof = 0u;
+    uint32_t base_link_count = 0u;
+    uint32_t contact_rows_per_env = 0u;
+    uint32_t contact_slots_per_env = 0u;
+    uint32_t distinct_owner_rows_per_env = 0u;
+    uint32_t joint_limit_rows_per_env = 0u;
+    uint64_t incidence_per_env = 0u;
+    uint32_t measure_contact_residual = 0u;
+    uint64_t workspace_words = 0u;
+    VertexBlockLayout vertex_blocks{};
+    uint32_t measure_vertex_audit = 0u;
+    uint32_t mimic_couplings = 0u;
+    uint32_t max_independent_dof = kMaxDof;
+    uint32_t material_cells_per_env = 0u;
+    uint32_t grid_particles_per_env = 0u;
+    uint32_t grid_dims[3] = {};
+    uint32_t clear_failure_diagnostics = 1u;
+    uint32_t substep_index = 0u;
+    uint32_t position_iterations = 0u;
+    float position_beta = 0.0f;
+    float position_slop = 0.0f;
+    float position_max_velocity = 0.0f;
+    float velocity_tolerance = 0.0f;
+    uint32_t trace_sweeps = 0u;
+    uint32_t telemetry = 0u;
+    uint32_t contact_anchors = 0u;
 };
 struct ReadoutContactWrenchParams {   // op_schema.hpp:746-755
     float dt;
-    uint32_t env_count, base_link_count, max_contacts_per_env, rows_per_env, full_row_slot_count, contact_rows_per_env;
+    uint32_t env_count;
+    uint32_t base_link_count;
+    uint32_t max_contacts_per_env;
+    uint32_t rows_per_env;
+    uint32_t full_row_slot_count;
+    uint32_t contact_rows_per_env;
+    uint64_t workspace_bytes;
 };
-struct SnapshotParams { uint32_t env_count, selected_env_count; };
-// op_schema.hpp:170-180; the flags this path uses (the particle and free-body ones have no counterpart here)
-constexpr uint32_t kAccumulateOutputs = 1u, kAccumulateLinkWrench = 2u, kAccumulateJointLimit = 4u, kFinalizeLinkWrench = 8u;
-struct AccumulateStepParams { uint32_t env_count, links_per_env, flags, first, last; float substep_dt, inv_outer_dt; };
+struct ContactWarmStartParams {   // op_schema.hpp:951-959
+    uint32_t phase;
+    uint32_t env_count;
+    uint32_t slot_count;
+    uint32_t rows_per_env;
+    uint32_t full_row_slot_count;
+    uint32_t decay_steps;
+    uint64_t workspace_bytes = 0u;
+};
 
 }  // namespace nkh

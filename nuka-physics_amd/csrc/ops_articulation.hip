@@ -708,7 +708,8 @@ __global__ void __launch_bounds__(256) ReadoutDrivesKernel(ModelView m, DataView
 Status OpApplyDrives(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
     const auto* p = static_cast<const ApplyDrivesParams*>(params);
     if (p == nullptr || p->mode > kDriveActuator) return Status::InvalidArgument;
-    if (p->affine == 0u) return p->mode == kDriveTorque ? Status::Ok : Status::Unsupported;
+    // a world cooked without drive rows leaves `tau` as the applied generalized force: nothing to turn into rows
+    if (m.joint_drive_rows == 0u) return p->mode == kDriveTorque ? Status::Ok : Status::Unsupported;
     if (p->mode == kDriveComputedTorque || p->mode == kDriveOsc) return Status::Unsupported;
     if (p->total_link_count == 0u) return Status::Ok;
     if (p->links_per_env == 0u || p->links_per_env != m.links_per_env) return Status::InvalidArgument;

@@ -343,7 +343,8 @@ struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
     AssembleRowsParams p_assemble{};
     ContactWarmStartParams p_warm0{}, p_warm1{};
     BlockDescentSolveParams p_solve{};
-    SnapshotParams p_snapshot{};
+    SnapshotStepVelocityParams p_snapshot{};
+    NarrowphaseHeightfieldParams p_heightfield{};
     std::vector<AccumulateStepParams> p_accumulate;   // one per substep (pipeline.cpp:128-152)
     nuka_execution_mode_t mode = NUKA_EXECUTION_EAGER;
     nuka_phi_plan* plan = nullptr;
@@ -444,14 +445,14 @@ void BuildPipeline(World& w) {
     const float dt = cfg.fixed_dt / float(substeps);
     const float contact_margin = cfg.solver_contact_margin;
     const float query_reach = std::fmax(0.02f, 2.0f * (2.0f * 0.0f + contact_margin));   // contact_query.hpp:20-22
-    w.p_fk = {E, E * nl};
+    w.p_fk = {};
+    w.p_fk.articulation_count = E; w.p_fk.total_link_count = E * nl; w.p_fk.articulations_per_env = 1u;
     w.p_fk_velocity = {E, E * nl};
     w.p_drives = {};
     w.p_drives.dt = dt; w.p_drives.total_link_count = E * nl; w.p_drives.links_per_env = nl;
     w.p_drives.mode = m.drive_mode; w.p_drives.articulation_count = E; w.p_drives.bodies_per_env = nb;
     const bool drives = m.joint_drive_rows > 0u;
     const bool fold = drives && cfg.solver_fold_drive_damping != 0xFFFFFFFFu;   // pipeline.cpp:380-381
-    w.p_drives.affine = drives ? 1u : 0u;
     w.p_drives.defer_velocity_damping = fold ? 1u : 0u;
     std::memcpy(w.p_drives.gravity, cfg.gravity, sizeof(cfg.gravity));
     w.p_readout_drives = {dt, E * nl, nl, m.rows_per_env, m.contact_rows_per_env + m.joint_limit_rows + m.joint_friction_rows};
@@ -464,14 +465,29 @@ void BuildPipeline(World& w) {
     w.p_dynamics_probe = dyn;
     w.p_dynamics_probe.integrate_velocity = 0u;
     w.p_int_vel = {};
-    w.p_int_vel.dt = dt;
+    w.p_int_vel.dt = dt; w.p_int_vel.total_link_count = E * nl; w.p_int_vel.articulation_count = E;
     std::memcpy(w.p_int_vel.gravity, cfg.gravity, sizeof(cfg.gravity));
-    w.p_int_pos = {dt, E * nl, E, 0u, E, (has_contacts && cfg.solver_pos_iters > 0u) ? 1u : 0u, 0u};
-    w.p_sync = {E, nl, nb, 0u, 0u};
-    w.p_aabbs = {E, nb, 0u, std::fmax(contact_margin, 0.0005f), dt, query_reach};   // pipeline.cpp:613-615
-    w.p_lbvh = {E, nb, 0u};
-    w.p_query = {E, nb, 0u, m.contact_slots, m.contact_slots, m.contact_slots, 0u};
-    w.p_narrow = {E, nb, m.contact_slots, m.contact_slots, contact_margin, dt, query_reach};
+    w.p_int_pos = {};
+    w.p_int_pos.dt = dt; w.p_int_pos.total_link_count = E * nl; w.p_int_pos.articulation_count = E; w.p_int_pos.env_count = E;
+    w.p_int_pos.pos_pass = (has_contacts && cfg.solver_pos_iters > 0u) ? 1u : 0u;
+    w.p_sync = {};
+    w.p_sync.env_count = E; w.p_sync.links_per_env = nl; w.p_sync.bodies_per_env = nb;
+    w.p_aabbs = {};   // pipeline.cpp:613-615
+    w.p_aabbs.env_count = E; w.p_aabbs.bodies_per_env = nb; w.p_aabbs.margin = std::fmax(contact_margin, 0.0005f);
+    w.p_aabbs.dt = dt; w.p_aabbs.query_reach = query_reach;
+    w.p_lbvh = {};
+    w.p_lbvh.env_count = E; w.p_lbvh.bodies_per_env = nb;
+    w.p_query = {};
+    w.p_query.env_count = E; w.p_query.bodies_per_env = nb; w.p_query.max_contacts_per_env = m.contact_slots;
+    w.p_query.rigid_slot_cap = m.contact_slots; w.p_query.max_pairs = m.contact_slots;
+    w.p_narrow = {};
+    w.p_narrow.env_count = E; w.p_narrow.bodies_per_env = nb; w.p_narrow.union_slot_count = m.contact_slots;
+    w.p_narrow.rigid_slot_cap = m.contact_slots; w.p_narrow.contact_margin = contact_margin; w.p_narrow.dt = dt;
+    w.p_narrow.query_reach = query_reach; w.p_narrow.base_link_count = nl; w.p_narrow.articulations_per_env = 1u;
+    w.p_narrow.max_contacts_per_pair = 4u;
+    w.p_heightfield = {};   // has_heightfield 0: the op has nothing to add
+    w.p_heightfield.env_count = E; w.p_heightfield.bodies_per_env = nb; w.p_heightfield.rigid_slot_cap = m.contact_slots;
+    w.p_heightfield.slot_stride = m.contact_slots; w.p_heightfield.contact_margin = contact_margin;
     AssembleRowsParams& as = w.p_assemble;   // pipeline.cpp:861-897
     as = {};
     as.env_count = E; as.articulation_count = E; as.total_link_count = E * nl; as.max_dof = m.max_dof;
@@ -481,7 +497,9 @@ void BuildPipeline(World& w) {
     as.dt = dt; as.overlap_recovery_velocity = cfg.solver_overlap_recovery_velocity; as.contact_margin = contact_margin;
     as.joint_limit_rows_per_env = m.joint_limit_rows; as.joint_friction_rows_per_env = m.joint_friction_rows;
     as.joint_drive_rows_per_env = m.joint_drive_rows; as.baumgarte_max_velocity = cfg.solver_baumgarte_max_velocity;
-    w.p_warm0 = {0u, E, m.contact_slots, m.rows_per_env, m.contact_slots, 2u};
+    w.p_warm0 = {};
+    w.p_warm0.env_count = E; w.p_warm0.slot_count = m.contact_slots; w.p_warm0.rows_per_env = m.rows_per_env;
+    w.p_warm0.full_row_slot_count = m.contact_slots; w.p_warm0.decay_steps = 2u;
     w.p_warm1 = w.p_warm0;
     w.p_warm1.phase = 1u;
     BlockDescentSolveParams& bd = w.p_solve;   // pipeline.cpp:471-497
@@ -512,7 +530,7 @@ void BuildPipeline(World& w) {
             add(NkOp::LbvhBuild, &w.p_lbvh);
             add(NkOp::LbvhQueryPairs, &w.p_query);
             add(NkOp::NarrowphasePrimitives, &w.p_narrow);
-            add(NkOp::NarrowphaseHeightfield, &w.p_narrow);
+            add(NkOp::NarrowphaseHeightfield, &w.p_heightfield);
         }
         add(NkOp::AssembleRows, &w.p_assemble);
         if (m.contact_slots > 0u) add(NkOp::ContactWarmStart, &w.p_warm0);
@@ -525,7 +543,10 @@ void BuildPipeline(World& w) {
     add(NkOp::FkLinkVelocities, &w.p_fk_velocity);
     if (nb > 0u) add(NkOp::SyncLinkBodyPose, &w.p_sync);
     // a pure readout, part of the step only once a consumer has asked for one of its fields (pipeline.cpp:990-1005)
-    w.p_readout_contacts = {dt, E, nl, m.contact_slots, m.rows_per_env, m.contact_slots, m.contact_rows_per_env};
+    w.p_readout_contacts = {};
+    w.p_readout_contacts.dt = dt; w.p_readout_contacts.env_count = E; w.p_readout_contacts.base_link_count = nl;
+    w.p_readout_contacts.max_contacts_per_env = m.contact_slots; w.p_readout_contacts.rows_per_env = m.rows_per_env;
+    w.p_readout_contacts.full_row_slot_count = m.contact_slots; w.p_readout_contacts.contact_rows_per_env = m.contact_rows_per_env;
     const bool reads_contacts = w.contact_readout_demanded && has_contacts && m.contact_slots > 0u;
     if (reads_contacts) add(NkOp::ReadoutContactWrench, &w.p_readout_contacts);
     if (substeps == 1u) return;
