@@ -25,6 +25,35 @@ __device__ __forceinline__ V3 cross3(V3 a, V3 b) {
 // Full-precision reciprocal square root: v_rsq_f32 alone is 1 ulp-approximate, sqrt then divide is exact-rounded.
 __device__ __forceinline__ float rsqrt_exact(float x) { return 1.0f / sqrtf(x); }
 
+// Correctly rounded square root and quotient for operands in the normal range, without the range scaling, special-value
+// fix-ups and second reciprocal that the general sqrtf and operator/ carry.  sqrt_rn_normal corrects v_sqrt_f32 (at
+// most one ulp off) by the residuals of its two neighbours; make_recip / div_by are the Newton reciprocal and the two
+// quotient corrections of the general division, so one reciprocal serves every quotient with the same divisor.  Both
+// give the bits of sqrtf and a / b whenever |x|, |a|, |b| and the result lie between 2^-90 and 2^90 (compared on the
+// device over 5e8 random operands each); outside that range they stay within an ulp.
+__device__ __forceinline__ float sqrt_rn_normal(float x) {
+    const float s = __builtin_amdgcn_sqrtf(x);
+    const float down = __uint_as_float(__float_as_uint(s) - 1u), up = __uint_as_float(__float_as_uint(s) + 1u);
+    const float below = fmaf(-down, s, x), above = fmaf(-up, s, x);
+    float root = below <= 0.0f ? down : s;
+    root = above > 0.0f ? up : root;
+    return root;
+}
+struct Recip { float divisor, value; };
+__device__ __forceinline__ Recip make_recip(float divisor) {
+    float r = __builtin_amdgcn_rcpf(divisor);
+    const float e = fmaf(-divisor, r, 1.0f);
+    r = fmaf(e, r, r);
+    return Recip{divisor, r};
+}
+__device__ __forceinline__ float div_by(float a, Recip d) {
+    float q = a * d.value;
+    float e = fmaf(-d.divisor, q, a);
+    q = fmaf(e, d.value, q);
+    e = fmaf(-d.divisor, q, a);
+    return fmaf(e, d.value, q);
+}
+
 __device__ __forceinline__ Xf load_xf(const float* p) { return Xf{V3{p[0], p[1], p[2]}, Q4{p[3], p[4], p[5], p[6]}}; }
 __device__ __forceinline__ void store_xf(float* p, Xf t) {
     p[0] = t.p.x; p[1] = t.p.y; p[2] = t.p.z; p[3] = t.r.w; p[4] = t.r.x; p[5] = t.r.y; p[6] = t.r.z;
@@ -182,6 +211,11 @@ __device__ __forceinline__ uint32_t wave_max_u(uint32_t v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) { const uint32_t other = __shfl_xor(v, o, 64); v = other > v ? other : v; }
     return v;
+}
+__device__ __forceinline__ uint32_t wave_or_u(uint32_t v) {   // uniform result
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v |= uint32_t(__shfl_xor(int(v), o, 64));
+    return uint32_t(__builtin_amdgcn_readfirstlane(int(v)));
 }
 __device__ __forceinline__ uint32_t wave_sum_u(uint32_t v) {
 #pragma unroll

@@ -1,12 +1,13 @@
 // Launch side of the block-descent solve: head capacity, LDS sizing and the table of kernels, one per padded width.
-// The kernel template lives in ops_solver_kernel.h; its instantiations are spread over ops_solver_w*.hip so that
-// they compile in parallel.
+// The kernel template lives in ops_solver_kernel.h; its instantiations are spread over ops_solver_w*.hip (general)
+// and ops_solver_s*.hip (contact heads only) so that they compile in parallel.
 #include "ops_solver_kernel.h"
 
 namespace nkh {
 namespace solver {
 #define NKH_DECLARE_WIDTH(N) \
-    extern template __global__ void BlockDescentTileKernel<N>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+    extern template __global__ void BlockDescentTileKernel<N, false>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t); \
+    extern template __global__ void BlockDescentTileKernel<N, true>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
 NKH_DECLARE_WIDTH(4) NKH_DECLARE_WIDTH(8) NKH_DECLARE_WIDTH(12) NKH_DECLARE_WIDTH(16) NKH_DECLARE_WIDTH(20) NKH_DECLARE_WIDTH(24)
 NKH_DECLARE_WIDTH(28) NKH_DECLARE_WIDTH(32) NKH_DECLARE_WIDTH(36) NKH_DECLARE_WIDTH(40) NKH_DECLARE_WIDTH(44) NKH_DECLARE_WIDTH(48)
 NKH_DECLARE_WIDTH(52) NKH_DECLARE_WIDTH(56) NKH_DECLARE_WIDTH(60) NKH_DECLARE_WIDTH(64)
@@ -55,18 +56,23 @@ __global__ void __launch_bounds__(1024) OrderTilesKernel(DataView d, uint32_t en
 
 
 using SolverKernel = void (*)(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
-// One instantiation per padded width.
-const SolverKernel kSolverKernels[16] = {
-    BlockDescentTileKernel<4>, BlockDescentTileKernel<8>, BlockDescentTileKernel<12>, BlockDescentTileKernel<16>,
-    BlockDescentTileKernel<20>, BlockDescentTileKernel<24>, BlockDescentTileKernel<28>, BlockDescentTileKernel<32>,
-    BlockDescentTileKernel<36>, BlockDescentTileKernel<40>, BlockDescentTileKernel<44>, BlockDescentTileKernel<48>,
-    BlockDescentTileKernel<52>, BlockDescentTileKernel<56>, BlockDescentTileKernel<60>, BlockDescentTileKernel<64>};
+// Two instantiations per padded width: the general one, and the one for worlds whose heads are contact heads only,
+// at most one a lane.
+#define NKH_WIDTHS(V) \
+    BlockDescentTileKernel<4, V>, BlockDescentTileKernel<8, V>, BlockDescentTileKernel<12, V>, BlockDescentTileKernel<16, V>, \
+    BlockDescentTileKernel<20, V>, BlockDescentTileKernel<24, V>, BlockDescentTileKernel<28, V>, BlockDescentTileKernel<32, V>, \
+    BlockDescentTileKernel<36, V>, BlockDescentTileKernel<40, V>, BlockDescentTileKernel<44, V>, BlockDescentTileKernel<48, V>, \
+    BlockDescentTileKernel<52, V>, BlockDescentTileKernel<56, V>, BlockDescentTileKernel<60, V>, BlockDescentTileKernel<64, V>
+const SolverKernel kSolverKernels[2][16] = {{NKH_WIDTHS(false)}, {NKH_WIDTHS(true)}};
+#undef NKH_WIDTHS
 }  // namespace
 
 void InitSolverKernels() {
-    for (SolverKernel kernel : kSolverKernels) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        (void)hipGetLastError();
+    for (const auto& variant : kSolverKernels) {
+        for (SolverKernel kernel : variant) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipGetLastError();
+        }
     }
 }
 
@@ -81,17 +87,21 @@ Status OpBlockDescentSolve(const ModelView& m, const DataView& d, const void* pa
     if (staged == 0u) return Status::InvalidArgument;
     const uint32_t joint_heads = m.joint_limit_rows + m.joint_friction_rows + m.joint_drive_rows;
     const auto lds_bytes = [&](uint32_t contact_heads) { return size_t{solver::SolverLdsFloats(m.dof, contact_heads + joint_heads, contact_heads)} * sizeof(float); };
-    const auto blocks_per_unit = [&](uint32_t contact_heads) { return std::min<size_t>(8u, (160u * 1024u) / lds_bytes(contact_heads)); };
+    // widths past kTwoWaveWidth run one wave a SIMD: four blocks a compute unit at most, whatever their LDS
+    const size_t most_blocks = solver::PaddedWidth(m.dof) > uint32_t(solver::kTwoWaveWidth) ? 4u : 8u;
+    const auto blocks_per_unit = [&](uint32_t contact_heads) { return std::min<size_t>(most_blocks, (160u * 1024u) / lds_bytes(contact_heads)); };
     // The LDS a block needs grows with the contact heads it can stage, and a scene's slots (every pair that may ever
     // touch, at its largest manifold) outnumber the contacts an environment usually has.  Where a smaller capacity
     // lets more blocks share a compute unit, environments with few contact points go to a launch of that capacity:
     // up to three such launches, for eight, four and two blocks a unit, before the full one.  Each launch takes the
     // environments whose contact points fall in its range; an environment's results do not depend on its launch.
-    const SolverKernel kernel = kSolverKernels[solver::PaddedWidth(m.dof) / 4u - 1u];
+    const bool contacts_only = joint_heads == 0u && staged <= uint32_t(solver::kWave);
+    const SolverKernel kernel = kSolverKernels[contacts_only ? 1 : 0][solver::PaddedWidth(m.dof) / 4u - 1u];
     hipLaunchKernelGGL(OrderTilesKernel, dim3(1), dim3(1024), 0, stream, d, p->env_count);
     uint32_t first_points = 0u;
     if (p->contact_slots_per_env != 0u) {
         for (const size_t blocks : {size_t{8u}, size_t{4u}, size_t{2u}}) {
+            if (blocks > most_blocks) continue;                            // more blocks than the waves allow
             if (blocks_per_unit(staged) >= blocks) break;                  // the full capacity does as well
             uint32_t few = staged;
             while (few > 8u && blocks_per_unit(few) < blocks) --few;

@@ -106,24 +106,33 @@ __device__ __forceinline__ void scalar_impulse(float dual, float rho, float resi
     *impulse = x < lower ? lower : (x > upper ? upper : x);
     *curvature = x != x ? x : (lower < upper && x >= lower && x <= upper ? k : 0.0f);
 }
-// augmented_row.hpp:302-318
-__device__ __forceinline__ float cone_argument(float dual, float rho, float mu, float residual) {
+// augmented_row.hpp:302-318, in two parts: what depends on the dual, the penalty and the friction ratio only, and
+// the rest, which takes the residual.  A line search evaluates the second part at every probe and the first once.
+struct ConeAxis { float dd, d_low, p, p_low; };
+__device__ __forceinline__ ConeAxis cone_axis(float dual, float rho, float mu) {
     // a friction ratio of exactly one (equal coefficients) divides to the dividend itself: skip the two divisions
     const bool unit = mu == 1.0f;
     const bool dual_zero = dual == 0.0f;
-    const float dual_quotient = unit ? dual + float(dual_zero) : (dual + float(dual_zero)) / mu;
+    const Recip by_mu = make_recip(mu);   // a ratio of zero gives values that every caller discards
+    const float dual_quotient = unit ? dual + float(dual_zero) : div_by(dual + float(dual_zero), by_mu);
     const float dd = dual_zero ? dual : dual_quotient;
     const float low = fmaf(-dd, mu, dual);
     const bool low_zero = low == 0.0f;
-    const float low_quotient = unit ? low + float(low_zero) : (low + float(low_zero)) / mu;
+    const float low_quotient = unit ? low + float(low_zero) : div_by(low + float(low_zero), by_mu);
     const float d_low = low_zero ? low : low_quotient;
     const float p = rho * mu;
-    const float t = p * residual;
-    const float t_low = fmaf(p, residual, -t) + fmaf(rho, mu, -p) * residual;
-    const float sum = dd + t;
-    const float t_part = sum - dd;
-    const float sum_low = (dd - (sum - t_part)) + (t - t_part);
-    return sum + (sum_low + d_low + t_low);
+    return ConeAxis{dd, d_low, p, fmaf(rho, mu, -p)};
+}
+__device__ __forceinline__ float cone_value(ConeAxis a, float residual) {
+    const float t = a.p * residual;
+    const float t_low = fmaf(a.p, residual, -t) + a.p_low * residual;
+    const float sum = a.dd + t;
+    const float t_part = sum - a.dd;
+    const float sum_low = (a.dd - (sum - t_part)) + (t - t_part);
+    return sum + (sum_low + a.d_low + t_low);
+}
+__device__ __forceinline__ float cone_argument(float dual, float rho, float mu, float residual) {
+    return cone_value(cone_axis(dual, rho, mu), residual);
 }
 // augmented_row.hpp:321-348; curvature entries yy, zz, yz.  The friction ratios depend on the row only, so callers
 // that evaluate one row many times compute them once (tangent_ratios) and pass them in.
@@ -252,27 +261,19 @@ __device__ __forceinline__ bool factor_rows(uint32_t lane, float (&row)[N], floa
     lane = local_lane(lane);
     bool valid = true;
     float inverse = 0.0f;
-    // The pivot's square root and reciprocal are a long dependent chain; column k + 1 is brought up to date first
-    // and its pivot chain started, so that it runs under the rest of step k's column updates.
-    float pivot = lane_value(row[0], 0);
-    valid = pivot > 0.0f && pivot <= FLT_MAX;
-    float root = sqrtf(valid ? pivot : 1.0f);
-    float scale = 1.0f / root;
 #pragma unroll
     for (int k = 0; k < N; ++k) {
+        // the pivot's square root and reciprocal: every pivot of a valid block lies in the normal range
+        const float pivot = lane_value(row[k], k);
+        valid = valid && pivot > 0.0f && pivot <= FLT_MAX;
+        const float root = sqrt_rn_normal(valid ? pivot : 1.0f);
+        const float scale = div_by(1.0f, make_recip(root));
         row[k] = lane == uint32_t(k) ? root : row[k] * scale;
         if (lane == uint32_t(k)) inverse = scale;
-        if (k + 1 < N) {
-            row[k + 1] = fmaf(-row[k], lane_value(row[k], k + 1), row[k + 1]);
-            pivot = lane_value(row[k + 1], k + 1);
-            valid = valid && pivot > 0.0f && pivot <= FLT_MAX;
-            root = sqrtf(valid ? pivot : 1.0f);
-            scale = 1.0f / root;
-        }
         // lane reads in batches of eight ahead of their multiply-adds: a scalar read has to settle for two cycles
         // before an arithmetic instruction may use it, and the next reads fill that gap
 #pragma unroll
-        for (int j0 = k + 2; j0 < N; j0 += 8) {
+        for (int j0 = k + 1; j0 < N; j0 += 8) {
             float l[8];
 #pragma unroll
             for (int t = 0; t < 8; ++t) l[t] = j0 + t < N ? lane_value(row[k], j0 + t) : 0.0f;
@@ -300,31 +301,24 @@ __device__ __forceinline__ bool factor_rows_up(uint32_t lane, float (&row)[N], f
     lane = local_lane(lane);
     bool valid = true;
     float inverse = 0.0f;
-    float pivot = lane_value(row[N - 1], N - 1);
-    valid = pivot > 0.0f && pivot <= FLT_MAX;
-    float root = sqrtf(valid ? pivot : 1.0f);
-    float scale = 1.0f / root;
 #pragma unroll
     for (int k = N - 1; k >= 0; --k) {
+        const float pivot = lane_value(row[k], k);
+        valid = valid && pivot > 0.0f && pivot <= FLT_MAX;
+        const float root = sqrt_rn_normal(valid ? pivot : 1.0f);
+        const float scale = div_by(1.0f, make_recip(root));
         row[k] = lane == uint32_t(k) ? root : row[k] * scale;
         if (lane == uint32_t(k)) inverse = scale;
         const uint64_t reach = __ballot(lane < uint32_t(k) && row[k] != 0.0f);
-        if (k >= 1) {
-            row[k - 1] = fmaf(-row[k], lane_value(row[k], k - 1), row[k - 1]);
-            pivot = lane_value(row[k - 1], k - 1);
-            valid = valid && pivot > 0.0f && pivot <= FLT_MAX;
-            root = sqrtf(valid ? pivot : 1.0f);
-            scale = 1.0f / root;
-        }
 #pragma unroll
-        for (int q = (k - 2) / 4; q >= 0 && k >= 2; --q) {
+        for (int q = (k - 1) / 4; q >= 0 && k >= 1; --q) {
             if (((reach >> (4 * q)) & 0xFull) == 0ull) continue;
             float u[4];
 #pragma unroll
-            for (int t = 0; t < 4; ++t) u[t] = 4 * q + t <= k - 2 ? lane_value(row[k], 4 * q + t) : 0.0f;
+            for (int t = 0; t < 4; ++t) u[t] = 4 * q + t <= k - 1 ? lane_value(row[k], 4 * q + t) : 0.0f;
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-                if (4 * q + t <= k - 2) row[4 * q + t] = fmaf(-row[k], u[t], row[4 * q + t]);
+                if (4 * q + t <= k - 1) row[4 * q + t] = fmaf(-row[k], u[t], row[4 * q + t]);
         }
     }
     *inverse_out = inverse;
@@ -405,19 +399,25 @@ __device__ __forceinline__ void load_columns(const float* a, uint32_t lane, floa
 // transposed read of the backward substitution.
 template <int N>
 __device__ __forceinline__ bool cholesky_solve(const Tile& c, float (&hrow)[N], float g, float* d_out) {
+    const uint32_t row = local_lane(c.lane);
+    float inverse = 0.0f;
     if (!c.factor_current) {   // otherwise the Hessian is the one factored last: its factor is still in hfac
-        float inverse = 0.0f;
+        PROF_BEGIN(c, 14);
         const bool valid = kLeavesFirst<N> ? factor_rows_up<N>(c.lane, hrow, &inverse) : factor_rows<N>(c.lane, hrow, &inverse);
+        PROF_END(c, 14);
         if (!valid) return false;
+        PROF_BEGIN(c, 24);
         store_rows<N>(c.hfac, c.lane, hrow);
         __syncthreads();
+        PROF_END(c, 24);
         c.factor_current = true;
+    } else {
+        // rows and the reciprocal diagonal come back from hfac (the factor's own reciprocal is 1 / its diagonal
+        // entry, the same division)
+        inverse = row < uint32_t(N) ? 1.0f / c.hfac[row * (N + 1) + row] : 0.0f;
+        load_rows<N>(c.hfac, c.lane, hrow);
     }
-    // rows, columns and the reciprocal diagonal come back from hfac on either path (the factor's own reciprocal is
-    // 1 / its diagonal entry, the same division)
-    const uint32_t row = local_lane(c.lane);
-    const float inverse = row < uint32_t(N) ? 1.0f / c.hfac[row * (N + 1) + row] : 0.0f;
-    load_rows<N>(c.hfac, c.lane, hrow);
+    PROF_BEGIN(c, 15);
     if constexpr (kLeavesFirst<N>) {
         *d_out = substitute_up<N>(c.lane, hrow, c.hfac, inverse, c.lane < c.n ? g : 0.0f);
     } else {
@@ -426,6 +426,7 @@ __device__ __forceinline__ bool cholesky_solve(const Tile& c, float (&hrow)[N], 
         *d_out = substitute<N>(c.lane, hrow, col, inverse, c.lane < c.n ? g : 0.0f);
     }
     __syncthreads();
+    PROF_END(c, 15);
     return true;
 }
 
@@ -754,13 +755,16 @@ __device__ __forceinline__ void row_steps(const Tile& c, float d) {
     __syncthreads();
 }
 
-// One head's line-search inputs in registers: nothing in them changes between the probes of one search.
+// One head's line-search inputs in registers: nothing in them changes between the probes of one search, and neither
+// do the parts of its response that do not depend on the probe (plain_line).
 struct HeadLine {
-    bool owned, contact;
+    bool owned, contact, bounded, cone;
     float rho, compliance, lower, upper, bound;
     Response response;
     TangentRatios ratios;
     float dual[3], res[3], move[3], step[3];
+    float dual_part, radius, rho_radius, radius_y, radius_z, inside_yy, inside_zz;
+    ConeAxis y, z;
 };
 __device__ __forceinline__ HeadLine load_head_line(const Tile& c, uint32_t h) {
     HeadLine l{};
@@ -773,9 +777,29 @@ __device__ __forceinline__ HeadLine load_head_line(const Tile& c, uint32_t h) {
     l.ratios = tangent_ratios(c.F(hMu1, h), c.F(hMu2, h));
 #pragma unroll
     for (int k = 0; k < 3; ++k) { l.dual[k] = c.F(hDual + k, h); l.res[k] = c.F(hRes + k, h); l.move[k] = c.F(hMove + k, h); l.step[k] = c.F(hStep + k, h); }
+    l.bounded = l.lower < l.upper;
+    l.dual_part = l.response.dual_scale * l.dual[0];
+    if (l.contact) {
+        l.radius = (l.bound < 0.0f ? 0.0f : l.bound) * fmaxf(l.ratios.scale, 0.0f);
+        l.cone = l.radius != 0.0f;
+        l.y = cone_axis(l.dual[1], l.rho, l.ratios.mu_y);
+        l.z = cone_axis(l.dual[2], l.rho, l.ratios.mu_z);
+        l.rho_radius = l.rho * l.radius;
+        l.radius_y = l.ratios.mu_y * l.radius; l.radius_z = l.ratios.mu_z * l.radius;
+        l.inside_yy = l.rho * l.ratios.mu_y * l.ratios.mu_y; l.inside_zz = l.rho * l.ratios.mu_z * l.ratios.mu_z;
+    }
     return l;
 }
 
+__device__ __forceinline__ void add_line_terms(const float (&f)[3], const float (&r)[6], float sx, float sy, float sz, TileSum& row_slope,
+                                               float& row_curvature, float& row_magnitude) {
+    tile_add_product(row_slope, f[0], sx);
+    tile_add_product(row_slope, f[1], sy);
+    tile_add_product(row_slope, f[2], sz);
+    row_magnitude += fabsf(f[0] * sx) + fabsf(f[1] * sy) + fabsf(f[2] * sz);
+    row_curvature += r[0] * sx * sx + r[1] * sy * sy + r[2] * sz * sz + 2.0f * r[5] * sy * sz + 2.0f * r[3] * sx * sy +
+                     2.0f * r[4] * sx * sz;
+}
 // TileLineDerivatives (:2048-2086); lane = head, heads beyond the first 64 go through `extra`
 __device__ __forceinline__ void line_terms(const HeadLine& l, float alpha, TileSum& row_slope, float& row_curvature, float& row_magnitude) {
     const float sx = l.step[0], sy = l.step[1], sz = l.step[2];
@@ -784,24 +808,75 @@ __device__ __forceinline__ void line_terms(const HeadLine& l, float alpha, TileS
     if (l.contact)
         tangent_impulse(V3{l.dual[0], l.dual[1], l.dual[2]}, l.rho, l.res[1] - fmaf(alpha, sy, l.move[1]),
                         l.res[2] - fmaf(alpha, sz, l.move[2]), l.bound, l.ratios, &f[1], &f[2], &r[1], &r[2], &r[5]);
-    tile_add_product(row_slope, f[0], sx);
-    tile_add_product(row_slope, f[1], sy);
-    tile_add_product(row_slope, f[2], sz);
-    row_magnitude += fabsf(f[0] * sx) + fabsf(f[1] * sy) + fabsf(f[2] * sz);
-    row_curvature += r[0] * sx * sx + r[1] * sy * sy + r[2] * sz * sz + 2.0f * r[5] * sy * sz + 2.0f * r[3] * sx * sy +
-                     2.0f * r[4] * sx * sz;
+    add_line_terms(f, r, sx, sy, sz, row_slope, row_curvature, row_magnitude);
 }
-__device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& mine, float alpha, float inertial_slope, float inertial_curvature,
-                                 float* slope, float* curvature, float* magnitude) {
+// A head's line-search constants as numbers only, so that the probes run without a branch: every selection the
+// response makes on a constant of the head (a single-axis head has no tangent part, a friction ratio of zero takes no
+// cone argument, a cone of radius zero gives no tangent impulse and no curvature) is made here once, by handing the
+// probe constants on which the general formulas give those results exactly - zeros for what must come out as zero.
+// A lane without an owned head gets zeros throughout and adds exact zeros to every sum.
+struct PlainLine {
+    float k, k_bounded, dual_part, lower, upper;
+    float res[3], move[3], step[3];
+    ConeAxis y, z;
+    float mu_y, mu_z, radius, rho_radius, radius_y, radius_z, inside_yy, inside_zz;
+};
+__device__ __forceinline__ PlainLine plain_line(const HeadLine& l) {
+    PlainLine p{};
+    if (!l.owned || l.rho <= 0.0f) return p;   // no penalty: no impulse and no curvature (scalar_impulse, tangent_impulse)
+    p.k = l.response.residual_scale; p.k_bounded = l.bounded ? p.k : 0.0f; p.dual_part = l.dual_part; p.lower = l.lower; p.upper = l.upper;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { p.res[k] = l.res[k]; p.move[k] = l.move[k]; p.step[k] = l.step[k]; }
+    // a constant that is not a number makes the general response not a number; here it is handed on through the sum
+    if (!(l.rho == l.rho && l.dual[0] == l.dual[0] && l.compliance == l.compliance && l.lower == l.lower && l.upper == l.upper)) p.dual_part = nanf("");
+    if (!l.contact) return p;
+    p.mu_y = l.ratios.mu_y; p.mu_z = l.ratios.mu_z;
+    if (p.mu_y != 0.0f) p.y = l.y;
+    if (p.mu_z != 0.0f) p.z = l.z;
+    p.radius = l.radius; p.rho_radius = l.rho_radius; p.radius_y = l.radius_y; p.radius_z = l.radius_z;
+    if (l.cone) { p.inside_yy = l.inside_yy; p.inside_zz = l.inside_zz; }
+    return p;
+}
+// TileLineDerivatives (:2048-2086) with at most one head a lane: scalar_impulse and tangent_impulse operation
+// for operation, both sides of the cone computed and one selected, the three quotients by the tangent norm sharing
+// one reciprocal.  A residual that is not a number comes out as a slope that is not a number, as in the general path.
+__device__ __forceinline__ void plain_line_terms(const PlainLine& p, float alpha, TileSum& row_slope, float& row_curvature, float& row_magnitude) {
+    const float sx = p.step[0], sy = p.step[1], sz = p.step[2];
+    const float x = fmaf(p.k, p.res[0] - fmaf(alpha, sx, p.move[0]), p.dual_part);
+    const float f0 = x < p.lower ? p.lower : (x > p.upper ? p.upper : x);
+    const float r0 = x >= p.lower && x <= p.upper ? p.k_bounded : 0.0f;
+    const float q_y = cone_value(p.y, p.res[1] - fmaf(alpha, sy, p.move[1]));
+    const float q_z = cone_value(p.z, p.res[2] - fmaf(alpha, sz, p.move[2]));
+    const float norm = hypotf(q_y, q_z);
+    const bool inside = norm <= p.radius;
+    const Recip by_norm = make_recip(inside ? 1.0f : norm);
+    const float dy = div_by(q_y, by_norm), dz = div_by(q_z, by_norm), cs = div_by(p.rho_radius, by_norm);
+    const float f1 = inside ? p.mu_y * q_y : p.radius_y * dy, f2 = inside ? p.mu_z * q_z : p.radius_z * dz;
+    const float r1 = inside ? p.inside_yy : cs * p.mu_y * p.mu_y * dz * dz, r2 = inside ? p.inside_zz : cs * p.mu_z * p.mu_z * dy * dy;
+    const float r5 = inside ? 0.0f : -cs * p.mu_y * p.mu_z * dy * dz;
+    tile_add_product(row_slope, f0, sx);
+    tile_add_product(row_slope, f1, sy);
+    tile_add_product(row_slope, f2, sz);
+    row_magnitude += fabsf(f0 * sx) + fabsf(f1 * sy) + fabsf(f2 * sz);
+    row_curvature += r0 * sx * sx + r1 * sy * sy + r2 * sz * sz + 2.0f * r5 * sy * sz;
+}
+// `general` (uniform): the block has more heads than lanes
+__device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& mine, const PlainLine& plain, bool general, float alpha,
+                                 float inertial_slope, float inertial_curvature, float* slope, float* curvature, float* magnitude) {
     PROF_COUNT(c, 1);
     c.work += 1u;
     TileSum row_slope{0.0f, 0.0f};
     float row_curvature = 0.0f, row_magnitude = 0.0f;
-    if (mine.owned) line_terms(mine, alpha, row_slope, row_curvature, row_magnitude);
-    for (uint32_t h = c.lane + kWave; h < c.heads; h += kWave) {
-        const HeadLine extra = load_head_line(c, h);
-        if (extra.owned) line_terms(extra, alpha, row_slope, row_curvature, row_magnitude);
+    if (general) {
+        if (mine.owned) line_terms(mine, alpha, row_slope, row_curvature, row_magnitude);
+        for (uint32_t h = c.lane + kWave; h < c.heads; h += kWave) {
+            const HeadLine extra = load_head_line(c, h);
+            if (extra.owned) line_terms(extra, alpha, row_slope, row_curvature, row_magnitude);
+        }
+    } else {
+        plain_line_terms(plain, alpha, row_slope, row_curvature, row_magnitude);
     }
+    PROF_BEGIN(c, 25);
     TileSum total{-row_slope.value, -row_slope.error};
     if (c.lane == 0u) {
         tile_add_product(total, alpha, inertial_curvature);
@@ -812,19 +887,22 @@ __device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& 
     *slope = wave_total(total, narrow);
     *curvature = inertial_curvature + (narrow ? first_row_sum(row_curvature) : wave_sum(row_curvature));
     *magnitude = fabsf(inertial_slope) + alpha * inertial_curvature + (narrow ? first_row_sum(row_magnitude) : wave_sum(row_magnitude));
+    PROF_END(c, 25);
 }
 
 // SearchTileLine (:2089-2125)
 __device__ __forceinline__ float search_line(const Tile& c, float inertial_slope, float inertial_curvature) {
     float slope = 0.0f, curvature = 0.0f, magnitude = 0.0f;
     const HeadLine mine = load_head_line(c, c.lane);
-    line_derivatives(c, mine, 0.0f, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
+    const bool general = c.heads > uint32_t(kWave);
+    const PlainLine plain = plain_line(mine);
+    line_derivatives(c, mine, plain, general, 0.0f, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
     const float initial = slope;
     if (!(initial < 0.0f)) return 0.0f;
     float low = 0.0f, high = 0.0f, alpha = 1.0f;
     bool bounded = false;
     for (uint32_t step = 0u; step < kLineSearchSteps; ++step) {
-        line_derivatives(c, mine, alpha, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
+        line_derivatives(c, mine, plain, general, alpha, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
         if (!isfinite(slope) || !isfinite(curvature)) {
             high = alpha; bounded = true; alpha = 0.5f * (low + high);
             continue;
@@ -1198,8 +1276,10 @@ __host__ __device__ inline uint32_t SolverLdsFloats(uint32_t n, uint32_t cap, ui
     return FactorRegionFloats(n) + 3u * staged * N + HeadFieldFloats(cap, staged) + 256u + (cap > staged ? kUnitSlots * uint32_t(kWave) : 0u);
 }
 
-// DescendTile (:2941-3087)
-template <int N>
+// DescendTile (:2941-3087).  kContactsOnly is the instantiation for worlds without joint rows whose heads fit one a
+// lane (cap <= 64, every head a staged contact head): the unit-head paths and the loops over heads beyond the first
+// 64 are compiled out, which leaves the hot loop shorter and with fewer values to keep live.
+template <int N, bool kContactsOnly>
 __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(N <= kTwoWaveWidth ? 2 : 1, N <= kTwoWaveWidth ? 2 : 1)))
 BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint32_t cap, uint32_t staged_cap, uint32_t points_lo,
                        uint32_t points_hi) {
@@ -1272,6 +1352,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         heads = cap;
         if (lane == 0u) d.env_status[env] |= kEnvStatusSolverFailure;
     }
+    if constexpr (kContactsOnly) __builtin_assume(heads <= uint32_t(kWave));
     c.heads = heads;
     __syncthreads();
     PROF_END(c, 16);
@@ -1340,7 +1421,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
             const uint64_t own = __ballot(h < heads && (c.U(hUnit, h) == kInvalid || fabsf(c.F(hUnitValue, h)) != 1.0f));
             if (own != 0ull) individual_end = base + uint32_t(64 - __builtin_clzll(own));
         }
-        c.units = __any(any_unit) && cap > staged_cap;   // the lists have room only when the world has joint heads
+        c.units = !kContactsOnly && __any(any_unit) && cap > staged_cap;   // the lists have room only when the world has joint heads
         c.staged_end = staged_end;
         c.individual_end = individual_end;
         if (__any(overflow_rows) && lane == 0u) d.env_status[env] |= kEnvStatusSolverFailure;

@@ -1,10 +1,9 @@
-// Instantiations of the block-descent kernel for padded widths 28, 32, 36.
+// Instantiations of the block-descent kernel (general variant) for padded widths 28, 32, 36.
 #include "ops_solver_kernel.h"
-
 namespace nkh {
 namespace solver {
-template __global__ void BlockDescentTileKernel<28>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
-template __global__ void BlockDescentTileKernel<32>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
-template __global__ void BlockDescentTileKernel<36>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<28, false>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<32, false>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+template __global__ void BlockDescentTileKernel<36, false>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
 }  // namespace solver
 }  // namespace nkh
