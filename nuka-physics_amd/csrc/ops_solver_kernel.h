@@ -498,6 +498,109 @@ __device__ __forceinline__ void add_head(const Tile& c, uint32_t h, bool coordin
     }
 }
 
+// One head's line-search inputs in registers: nothing in them changes between the probes of one search, and neither
+// do the parts of its response that do not depend on the probe (plain_line).
+struct HeadLine {
+    bool owned, contact, bounded, cone;
+    float rho, compliance, lower, upper, bound;
+    Response response;
+    TangentRatios ratios;
+    float dual[3], res[3], move[3], step[3];
+    float dual_part, radius, rho_radius, radius_y, radius_z, inside_yy, inside_zz;
+    ConeAxis y, z;
+};
+__device__ __forceinline__ HeadLine load_head_line(const Tile& c, uint32_t h) {
+    HeadLine l{};
+    l.owned = h < c.heads && c.U(hOwned, h) != 0u;
+    if (!l.owned) return l;
+    l.contact = c.U(hAxes, h) == 3u;
+    l.rho = c.F(hRho, h); l.compliance = c.F(hCompliance, h); l.lower = c.F(hLower, h); l.upper = c.F(hUpper, h);
+    l.bound = c.F(hNormalBound, h);
+    l.response = Response{c.F(hDualScale, h), c.F(hResidualScale, h)};
+    l.ratios = tangent_ratios(c.F(hMu1, h), c.F(hMu2, h));
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { l.dual[k] = c.F(hDual + k, h); l.res[k] = c.F(hRes + k, h); l.move[k] = c.F(hMove + k, h); l.step[k] = c.F(hStep + k, h); }
+    l.bounded = l.lower < l.upper;
+    l.dual_part = l.response.dual_scale * l.dual[0];
+    if (l.contact) {
+        l.radius = (l.bound < 0.0f ? 0.0f : l.bound) * fmaxf(l.ratios.scale, 0.0f);
+        l.cone = l.radius != 0.0f;
+        l.y = cone_axis(l.dual[1], l.rho, l.ratios.mu_y);
+        l.z = cone_axis(l.dual[2], l.rho, l.ratios.mu_z);
+        l.rho_radius = l.rho * l.radius;
+        l.radius_y = l.ratios.mu_y * l.radius; l.radius_z = l.ratios.mu_z * l.radius;
+        l.inside_yy = l.rho * l.ratios.mu_y * l.ratios.mu_y; l.inside_zz = l.rho * l.ratios.mu_z * l.ratios.mu_z;
+    }
+    return l;
+}
+
+__device__ __forceinline__ void add_line_terms(const float (&f)[3], const float (&r)[6], float sx, float sy, float sz, TileSum& row_slope,
+                                               float& row_curvature, float& row_magnitude) {
+    tile_add_product(row_slope, f[0], sx);
+    tile_add_product(row_slope, f[1], sy);
+    tile_add_product(row_slope, f[2], sz);
+    row_magnitude += fabsf(f[0] * sx) + fabsf(f[1] * sy) + fabsf(f[2] * sz);
+    row_curvature += r[0] * sx * sx + r[1] * sy * sy + r[2] * sz * sz + 2.0f * r[5] * sy * sz + 2.0f * r[3] * sx * sy +
+                     2.0f * r[4] * sx * sz;
+}
+// TileLineDerivatives (:2048-2086); lane = head, heads beyond the first 64 go through `extra`
+__device__ __forceinline__ void line_terms(const HeadLine& l, float alpha, TileSum& row_slope, float& row_curvature, float& row_magnitude) {
+    const float sx = l.step[0], sy = l.step[1], sz = l.step[2];
+    float f[3] = {0.0f, 0.0f, 0.0f}, r[6] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    scalar_impulse(l.dual[0], l.rho, l.res[0] - fmaf(alpha, sx, l.move[0]), l.compliance, l.lower, l.upper, l.response, &f[0], &r[0]);
+    if (l.contact)
+        tangent_impulse(V3{l.dual[0], l.dual[1], l.dual[2]}, l.rho, l.res[1] - fmaf(alpha, sy, l.move[1]),
+                        l.res[2] - fmaf(alpha, sz, l.move[2]), l.bound, l.ratios, &f[1], &f[2], &r[1], &r[2], &r[5]);
+    add_line_terms(f, r, sx, sy, sz, row_slope, row_curvature, row_magnitude);
+}
+// A head's line-search constants as numbers only, so that the probes run without a branch: every selection the
+// response makes on a constant of the head (a single-axis head has no tangent part, a friction ratio of zero takes no
+// cone argument, a cone of radius zero gives no tangent impulse and no curvature) is made here once, by handing the
+// probe constants on which the general formulas give those results exactly - zeros for what must come out as zero.
+// A lane without an owned head gets zeros throughout and adds exact zeros to every sum.
+struct PlainLine {
+    float k, k_bounded, dual_part, lower, upper;
+    float res[3], move[3], step[3];
+    ConeAxis y, z;
+    float mu_y, mu_z, radius, rho_radius, radius_y, radius_z, inside_yy, inside_zz;
+};
+__device__ __forceinline__ PlainLine plain_line(const HeadLine& l) {
+    PlainLine p{};
+    if (!l.owned || l.rho <= 0.0f) return p;   // no penalty: no impulse and no curvature (scalar_impulse, tangent_impulse)
+    p.k = l.response.residual_scale; p.k_bounded = l.bounded ? p.k : 0.0f; p.dual_part = l.dual_part; p.lower = l.lower; p.upper = l.upper;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { p.res[k] = l.res[k]; p.move[k] = l.move[k]; p.step[k] = l.step[k]; }
+    // a constant that is not a number makes the general response not a number; here it is handed on through the sum
+    if (!(l.rho == l.rho && l.dual[0] == l.dual[0] && l.compliance == l.compliance && l.lower == l.lower && l.upper == l.upper)) p.dual_part = nanf("");
+    if (!l.contact) return p;
+    p.mu_y = l.ratios.mu_y; p.mu_z = l.ratios.mu_z;
+    if (p.mu_y != 0.0f) p.y = l.y;
+    if (p.mu_z != 0.0f) p.z = l.z;
+    p.radius = l.radius; p.rho_radius = l.rho_radius; p.radius_y = l.radius_y; p.radius_z = l.radius_z;
+    if (l.cone) { p.inside_yy = l.inside_yy; p.inside_zz = l.inside_zz; }
+    return p;
+}
+// The response of a head from its constants: scalar_impulse and tangent_impulse operation for operation, both sides
+// of the cone computed and one selected, the three quotients by the tangent norm sharing one reciprocal.  A residual
+// that is not a number comes out as an impulse that is not a number, as in the general functions.  plain_line_terms
+// is TileLineDerivatives (:2048-2086) on it, with at most one head a lane.
+__device__ __forceinline__ void plain_response(const PlainLine& p, float mx, float my, float mz, float (&f)[3], float (&r)[6]) {
+    const float x = fmaf(p.k, p.res[0] - mx, p.dual_part);
+    f[0] = x < p.lower ? p.lower : (x > p.upper ? p.upper : x);
+    r[0] = x >= p.lower && x <= p.upper ? p.k_bounded : 0.0f;
+    const float q_y = cone_value(p.y, p.res[1] - my);
+    const float q_z = cone_value(p.z, p.res[2] - mz);
+    const float norm = hypotf(q_y, q_z);
+    const bool inside = norm <= p.radius;
+    const Recip by_norm = make_recip(inside ? 1.0f : norm);
+    const float dy = div_by(q_y, by_norm), dz = div_by(q_z, by_norm), cs = div_by(p.rho_radius, by_norm);
+    f[1] = inside ? p.mu_y * q_y : p.radius_y * dy;
+    f[2] = inside ? p.mu_z * q_z : p.radius_z * dz;
+    r[1] = inside ? p.inside_yy : cs * p.mu_y * p.mu_y * dz * dz;
+    r[2] = inside ? p.inside_zz : cs * p.mu_z * p.mu_z * dy * dy;
+    r[3] = 0.0f; r[4] = 0.0f;
+    r[5] = inside ? 0.0f : -cs * p.mu_y * p.mu_z * dy * dz;
+}
 // A head's response at its current move with the rounding noise of each axis; false when nothing of it is non-zero.
 __device__ __forceinline__ bool head_terms(const Tile& c, uint32_t h, float (&f)[3], float (&cv)[6], float (&noise)[3]) {
 #pragma unroll
@@ -530,8 +633,16 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
     float* dvec = c.vec, *evec = c.vec + 64, *uvec = c.vec + 128;
     dvec[lane] = difference; evec[lane] = difference_error; uvec[lane] = fabsf(u);
     PROF_BEGIN(c, 10);
+    // lane's own head (the first 64 heads) from its constants, without a branch; a lane without an owned head gets zeros
     float mf[3], mc[6], mn[3];
-    const bool mine = head_terms(c, lane, mf, mc, mn);
+    {
+        const PlainLine own = plain_line(load_head_line(c, lane));
+        plain_response(own, own.move[0], own.move[1], own.move[2], mf, mc);
+#pragma unroll
+        for (int k = 0; k < 3; ++k) mn[k] = fabsf(mf[k]) + mc[k] * (fabsf(own.res[k]) + fabsf(own.move[k]));
+    }
+    const bool mine = mf[0] != 0.0f || mf[1] != 0.0f || mf[2] != 0.0f || mc[0] != 0.0f || mc[1] != 0.0f || mc[2] != 0.0f || mc[5] != 0.0f ||
+                      mn[0] != 0.0f || mn[1] != 0.0f || mn[2] != 0.0f;
     const uint32_t my_axes = lane < c.heads ? c.U(hAxes, lane) : 0u;
     const uint32_t my_low = lane < c.heads ? c.U(hColumnsLow, lane) : 0u, my_high = lane < c.heads ? c.U(hColumnsHigh, lane) : 0u;
     // The Hessian M + sum J^T C J changes only through the heads' curvatures: every head keeps the curvature of its
@@ -755,110 +866,15 @@ __device__ __forceinline__ void row_steps(const Tile& c, float d) {
     __syncthreads();
 }
 
-// One head's line-search inputs in registers: nothing in them changes between the probes of one search, and neither
-// do the parts of its response that do not depend on the probe (plain_line).
-struct HeadLine {
-    bool owned, contact, bounded, cone;
-    float rho, compliance, lower, upper, bound;
-    Response response;
-    TangentRatios ratios;
-    float dual[3], res[3], move[3], step[3];
-    float dual_part, radius, rho_radius, radius_y, radius_z, inside_yy, inside_zz;
-    ConeAxis y, z;
-};
-__device__ __forceinline__ HeadLine load_head_line(const Tile& c, uint32_t h) {
-    HeadLine l{};
-    l.owned = h < c.heads && c.U(hOwned, h) != 0u;
-    if (!l.owned) return l;
-    l.contact = c.U(hAxes, h) == 3u;
-    l.rho = c.F(hRho, h); l.compliance = c.F(hCompliance, h); l.lower = c.F(hLower, h); l.upper = c.F(hUpper, h);
-    l.bound = c.F(hNormalBound, h);
-    l.response = Response{c.F(hDualScale, h), c.F(hResidualScale, h)};
-    l.ratios = tangent_ratios(c.F(hMu1, h), c.F(hMu2, h));
-#pragma unroll
-    for (int k = 0; k < 3; ++k) { l.dual[k] = c.F(hDual + k, h); l.res[k] = c.F(hRes + k, h); l.move[k] = c.F(hMove + k, h); l.step[k] = c.F(hStep + k, h); }
-    l.bounded = l.lower < l.upper;
-    l.dual_part = l.response.dual_scale * l.dual[0];
-    if (l.contact) {
-        l.radius = (l.bound < 0.0f ? 0.0f : l.bound) * fmaxf(l.ratios.scale, 0.0f);
-        l.cone = l.radius != 0.0f;
-        l.y = cone_axis(l.dual[1], l.rho, l.ratios.mu_y);
-        l.z = cone_axis(l.dual[2], l.rho, l.ratios.mu_z);
-        l.rho_radius = l.rho * l.radius;
-        l.radius_y = l.ratios.mu_y * l.radius; l.radius_z = l.ratios.mu_z * l.radius;
-        l.inside_yy = l.rho * l.ratios.mu_y * l.ratios.mu_y; l.inside_zz = l.rho * l.ratios.mu_z * l.ratios.mu_z;
-    }
-    return l;
-}
-
-__device__ __forceinline__ void add_line_terms(const float (&f)[3], const float (&r)[6], float sx, float sy, float sz, TileSum& row_slope,
-                                               float& row_curvature, float& row_magnitude) {
+__device__ __forceinline__ void plain_line_terms(const PlainLine& p, float alpha, TileSum& row_slope, float& row_curvature, float& row_magnitude) {
+    const float sx = p.step[0], sy = p.step[1], sz = p.step[2];
+    float f[3], r[6];
+    plain_response(p, fmaf(alpha, sx, p.move[0]), fmaf(alpha, sy, p.move[1]), fmaf(alpha, sz, p.move[2]), f, r);
     tile_add_product(row_slope, f[0], sx);
     tile_add_product(row_slope, f[1], sy);
     tile_add_product(row_slope, f[2], sz);
     row_magnitude += fabsf(f[0] * sx) + fabsf(f[1] * sy) + fabsf(f[2] * sz);
-    row_curvature += r[0] * sx * sx + r[1] * sy * sy + r[2] * sz * sz + 2.0f * r[5] * sy * sz + 2.0f * r[3] * sx * sy +
-                     2.0f * r[4] * sx * sz;
-}
-// TileLineDerivatives (:2048-2086); lane = head, heads beyond the first 64 go through `extra`
-__device__ __forceinline__ void line_terms(const HeadLine& l, float alpha, TileSum& row_slope, float& row_curvature, float& row_magnitude) {
-    const float sx = l.step[0], sy = l.step[1], sz = l.step[2];
-    float f[3] = {0.0f, 0.0f, 0.0f}, r[6] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-    scalar_impulse(l.dual[0], l.rho, l.res[0] - fmaf(alpha, sx, l.move[0]), l.compliance, l.lower, l.upper, l.response, &f[0], &r[0]);
-    if (l.contact)
-        tangent_impulse(V3{l.dual[0], l.dual[1], l.dual[2]}, l.rho, l.res[1] - fmaf(alpha, sy, l.move[1]),
-                        l.res[2] - fmaf(alpha, sz, l.move[2]), l.bound, l.ratios, &f[1], &f[2], &r[1], &r[2], &r[5]);
-    add_line_terms(f, r, sx, sy, sz, row_slope, row_curvature, row_magnitude);
-}
-// A head's line-search constants as numbers only, so that the probes run without a branch: every selection the
-// response makes on a constant of the head (a single-axis head has no tangent part, a friction ratio of zero takes no
-// cone argument, a cone of radius zero gives no tangent impulse and no curvature) is made here once, by handing the
-// probe constants on which the general formulas give those results exactly - zeros for what must come out as zero.
-// A lane without an owned head gets zeros throughout and adds exact zeros to every sum.
-struct PlainLine {
-    float k, k_bounded, dual_part, lower, upper;
-    float res[3], move[3], step[3];
-    ConeAxis y, z;
-    float mu_y, mu_z, radius, rho_radius, radius_y, radius_z, inside_yy, inside_zz;
-};
-__device__ __forceinline__ PlainLine plain_line(const HeadLine& l) {
-    PlainLine p{};
-    if (!l.owned || l.rho <= 0.0f) return p;   // no penalty: no impulse and no curvature (scalar_impulse, tangent_impulse)
-    p.k = l.response.residual_scale; p.k_bounded = l.bounded ? p.k : 0.0f; p.dual_part = l.dual_part; p.lower = l.lower; p.upper = l.upper;
-#pragma unroll
-    for (int k = 0; k < 3; ++k) { p.res[k] = l.res[k]; p.move[k] = l.move[k]; p.step[k] = l.step[k]; }
-    // a constant that is not a number makes the general response not a number; here it is handed on through the sum
-    if (!(l.rho == l.rho && l.dual[0] == l.dual[0] && l.compliance == l.compliance && l.lower == l.lower && l.upper == l.upper)) p.dual_part = nanf("");
-    if (!l.contact) return p;
-    p.mu_y = l.ratios.mu_y; p.mu_z = l.ratios.mu_z;
-    if (p.mu_y != 0.0f) p.y = l.y;
-    if (p.mu_z != 0.0f) p.z = l.z;
-    p.radius = l.radius; p.rho_radius = l.rho_radius; p.radius_y = l.radius_y; p.radius_z = l.radius_z;
-    if (l.cone) { p.inside_yy = l.inside_yy; p.inside_zz = l.inside_zz; }
-    return p;
-}
-// TileLineDerivatives (:2048-2086) with at most one head a lane: scalar_impulse and tangent_impulse operation
-// for operation, both sides of the cone computed and one selected, the three quotients by the tangent norm sharing
-// one reciprocal.  A residual that is not a number comes out as a slope that is not a number, as in the general path.
-__device__ __forceinline__ void plain_line_terms(const PlainLine& p, float alpha, TileSum& row_slope, float& row_curvature, float& row_magnitude) {
-    const float sx = p.step[0], sy = p.step[1], sz = p.step[2];
-    const float x = fmaf(p.k, p.res[0] - fmaf(alpha, sx, p.move[0]), p.dual_part);
-    const float f0 = x < p.lower ? p.lower : (x > p.upper ? p.upper : x);
-    const float r0 = x >= p.lower && x <= p.upper ? p.k_bounded : 0.0f;
-    const float q_y = cone_value(p.y, p.res[1] - fmaf(alpha, sy, p.move[1]));
-    const float q_z = cone_value(p.z, p.res[2] - fmaf(alpha, sz, p.move[2]));
-    const float norm = hypotf(q_y, q_z);
-    const bool inside = norm <= p.radius;
-    const Recip by_norm = make_recip(inside ? 1.0f : norm);
-    const float dy = div_by(q_y, by_norm), dz = div_by(q_z, by_norm), cs = div_by(p.rho_radius, by_norm);
-    const float f1 = inside ? p.mu_y * q_y : p.radius_y * dy, f2 = inside ? p.mu_z * q_z : p.radius_z * dz;
-    const float r1 = inside ? p.inside_yy : cs * p.mu_y * p.mu_y * dz * dz, r2 = inside ? p.inside_zz : cs * p.mu_z * p.mu_z * dy * dy;
-    const float r5 = inside ? 0.0f : -cs * p.mu_y * p.mu_z * dy * dz;
-    tile_add_product(row_slope, f0, sx);
-    tile_add_product(row_slope, f1, sy);
-    tile_add_product(row_slope, f2, sz);
-    row_magnitude += fabsf(f0 * sx) + fabsf(f1 * sy) + fabsf(f2 * sz);
-    row_curvature += r0 * sx * sx + r1 * sy * sy + r2 * sz * sz + 2.0f * r5 * sy * sz;
+    row_curvature += r[0] * sx * sx + r[1] * sy * sy + r[2] * sz * sz + 2.0f * r[5] * sy * sz;
 }
 // `general` (uniform): the block has more heads than lanes
 __device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& mine, const PlainLine& plain, bool general, float alpha,
@@ -1441,24 +1457,35 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     __syncthreads();
     // CopyTileRows (:836-869): the staged heads' rows, their loads in flight together
 
-    for (uint32_t h = 0u; h < c.staged_end; ++h) {
-        const uint32_t first = c.U(hRow, h);
-        const bool staged = first != kInvalid;   // a unit head stages nothing and touches no column block
-        float value[3];
+    for (uint32_t h0 = 0u; h0 < c.staged_end; h0 += 4u) {   // four heads at a time: 24 reads in flight
+        uint32_t first[4];
+        float value[4][3];
 #pragma unroll
-        for (uint32_t axis = 0u; axis < 3u; ++axis) {
-            const uint32_t source_a = c.U(hSourceA + axis, h), source_b = c.U(hSourceB + axis, h);
-            value[axis] = 0.0f;
-            if (staged && coordinate && source_a != kInvalid) value[axis] += d.chain_jacobian[size_t{source_a} * md + lane];
-            if (staged && coordinate && source_b != kInvalid) value[axis] += d.chain_jacobian_b[size_t{source_b} * md + lane];
+        for (uint32_t t = 0u; t < 4u; ++t) {
+            const uint32_t h = h0 + t;
+            first[t] = h < c.staged_end ? c.U(hRow, h) : kInvalid;   // a unit head stages nothing and touches no column block
+            const bool staged = first[t] != kInvalid;
+#pragma unroll
+            for (uint32_t axis = 0u; axis < 3u; ++axis) {
+                const uint32_t source_a = staged ? c.U(hSourceA + axis, h) : kInvalid, source_b = staged ? c.U(hSourceB + axis, h) : kInvalid;
+                const float from_a = coordinate && source_a != kInvalid ? d.chain_jacobian[size_t{source_a} * md + lane] : 0.0f;
+                const float from_b = coordinate && source_b != kInvalid ? d.chain_jacobian_b[size_t{source_b} * md + lane] : 0.0f;
+                value[t][axis] = (0.0f + from_a) + from_b;
+            }
         }
 #pragma unroll
-        for (uint32_t axis = 0u; axis < 3u; ++axis)
-            if (staged && lane < c.ldj) c.jac[(first + axis) * c.ldj + lane] = value[axis];   // padded columns hold zeros
-        // the columns this head touches at all: a contact on one limb leaves most coordinates out, and the Hessian
-        // update skips their exact-zero products four columns at a time
-        const uint64_t columns = __ballot(value[0] != 0.0f || value[1] != 0.0f || value[2] != 0.0f);
-        if (lane == 0u) { c.U(hColumnsLow, h) = uint32_t(columns); c.U(hColumnsHigh, h) = uint32_t(columns >> 32u); }
+        for (uint32_t t = 0u; t < 4u; ++t) {
+            const uint32_t h = h0 + t;
+            if (h >= c.staged_end) break;
+            const bool staged = first[t] != kInvalid;
+#pragma unroll
+            for (uint32_t axis = 0u; axis < 3u; ++axis)
+                if (staged && lane < c.ldj) c.jac[(first[t] + axis) * c.ldj + lane] = value[t][axis];   // padded columns hold zeros
+            // the columns this head touches at all: a contact on one limb leaves most coordinates out, and the Hessian
+            // update skips their exact-zero products four columns at a time
+            const uint64_t columns = __ballot(value[t][0] != 0.0f || value[t][1] != 0.0f || value[t][2] != 0.0f);
+            if (lane == 0u) { c.U(hColumnsLow, h) = uint32_t(columns); c.U(hColumnsHigh, h) = uint32_t(columns >> 32u); }
+        }
     }
     __syncthreads();
     PROF_END(c, 17);
@@ -1469,22 +1496,35 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     // L_ij y_j for j = 0, 1, ... exactly as the serial loop does; the ordered sum of y_i^2 / D_i follows the same way.
     float mrow[N];
     {
-        const float* factor = d.m_factor + size_t{env} * md * md;
-        // the mass rows ride along (StageTileMass :2127-2142), so that both matrices' loads are in flight together
-        for (uint32_t e = lane; e < n * n; e += kWave) {
-            c.hfac[(e / n) * c.ld + e % n] = factor[size_t{e / n} * md + e % n];
-            c.mfac[(e / n) * c.ld + e % n] = d.m[size_t{env} * md * md + size_t{e / n} * md + e % n];
+        // Lane's own rows of the mass matrix and of its LDL^T factor (StageTileMass :2127-2142) straight into registers:
+        // one row is md contiguous words, so every read of both rows is in flight at once, as 16-byte words where the
+        // rows are long enough and aligned for that.
+        const size_t tile = size_t{env} * md * md + size_t{coordinate ? lane : 0u} * md;
+        const float* factor = d.m_factor + tile;
+        const float* mass = d.m + tile;
+        float lrow[N], fetched[N];
+        if (md % 4u == 0u && md >= uint32_t(N)) {
+#pragma unroll
+            for (int q = 0; q < N / 4; ++q) {
+                const float4 f4 = reinterpret_cast<const float4*>(factor)[q], m4 = reinterpret_cast<const float4*>(mass)[q];
+                lrow[4 * q] = f4.x; lrow[4 * q + 1] = f4.y; lrow[4 * q + 2] = f4.z; lrow[4 * q + 3] = f4.w;
+                fetched[4 * q] = m4.x; fetched[4 * q + 1] = m4.y; fetched[4 * q + 2] = m4.z; fetched[4 * q + 3] = m4.w;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < N; ++k) {
+                lrow[k] = uint32_t(k) < n ? factor[k] : 0.0f;
+                fetched[k] = uint32_t(k) < n ? mass[k] : 0.0f;
+            }
         }
-        __syncthreads();
-        float lrow[N];
+        float pivot = 1.0f;
 #pragma unroll
         for (int k = 0; k < N; ++k) {
-            lrow[k] = coordinate && uint32_t(k) < lane ? c.hfac[lane * c.ld + k] : 0.0f;
+            if (coordinate && lane == uint32_t(k)) pivot = lrow[k];
             // rows and columns n..N-1 of the mass matrix are those of the identity
-            mrow[k] = coordinate && uint32_t(k) < n ? c.mfac[lane * c.ld + k] : (lane == uint32_t(k) && lane < uint32_t(N) ? 1.0f : 0.0f);
+            mrow[k] = coordinate && uint32_t(k) < n ? fetched[k] : (lane == uint32_t(k) && lane < uint32_t(N) ? 1.0f : 0.0f);
+            lrow[k] = coordinate && uint32_t(k) < lane ? lrow[k] : 0.0f;
         }
-        const float pivot = coordinate ? c.hfac[lane * c.ld + lane] : 1.0f;
-        __syncthreads();
         // y = L^-1 a, then the ordered sum of y_i^2 / D_i
         auto response = [&](float a) -> float {
 #pragma unroll
