@@ -233,6 +233,12 @@ __device__ __forceinline__ uint32_t local_lane(uint32_t lane) {
     asm volatile("" : "+v"(lane));
     return lane;
 }
+// The value itself, through a barrier the optimiser cannot look across: what is computed from it stays where it is
+// written instead of being hoisted out of the enclosing loops.
+__device__ __forceinline__ float opaque(float v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
 __device__ __forceinline__ bool wave_all(bool p) { return __all(p); }
 __device__ __forceinline__ bool wave_any(bool p) { return __any(p); }
 

@@ -173,7 +173,7 @@ __device__ __forceinline__ void tangent_impulse(V3 dual, float rho, float res_y,
 __device__ __forceinline__ uint32_t residual_bits(float value) { return __float_as_uint(value <= FLT_MAX ? fabsf(value) : FLT_MAX); }
 __device__ __forceinline__ float along_axis(float impulse, float velocity) { return impulse > 0.0f ? velocity : impulse < 0.0f ? -velocity : 0.0f; }
 
-// Per-head state, field-major in LDS so lane = head reads without bank conflicts.
+// Per-head state in LDS, head-major with an odd stride so lane = head reads without bank conflicts.
 enum HeadField : uint32_t {
     hSlot, hStride, hAxes, hOwned, hRho, hCompliance, hLower, hUpper, hMu1, hMu2, hNormalBound,
     hRes, hDual = hRes + 3, hMove = hDual + 3, hStep = hMove + 3, hBase = hStep + 3, hDualScale = hBase + 3, hResidualScale,
@@ -204,6 +204,10 @@ __host__ __device__ constexpr bool narrow_field(uint32_t f) { return narrow_belo
 constexpr uint32_t kNarrowFields = narrow_below(hFieldCount);
 constexpr uint32_t kWideFields = hFieldCount - kNarrowFields;
 static_assert(kNarrowFields <= 64u, "one lane clears the shared word of each narrow field");
+// Both tables are head-major with an odd number of words a head: a field of head h sits at h * stride + its index, so
+// every access is one base register (the head's) plus a constant offset, and lanes that read one field of consecutive
+// heads fall on different banks.
+constexpr uint32_t kWideStride = kWideFields | 1u, kNarrowStride = kNarrowFields | 1u;
 
 struct Tile {
     uint32_t env, lane, n, ld, ldj, heads, cap, narrow, iteration;
@@ -211,7 +215,7 @@ struct Tile {
     float* mfac;     // N x ld: Cholesky factor of the mass matrix (rows; columns are read transposed)
     float* hfac;     // N x ld: Cholesky factor of the current Newton Hessian
     float* jac;      // 3 * staged capacity rows x ldj, ldj = N
-    float* fields;   // kWideFields x cap, then kNarrowFields x (narrow + 1)
+    float* fields;   // cap x kWideStride, then (narrow + 1) x kNarrowStride
     float* vec;      // 4 x 64 scratch vectors, 16-byte aligned
     float mass_inverse;   // 1 / diagonal of the mass factor, lane = row
     mutable bool factor_current;     // no head's curvature has changed since hfac was factored: the Hessian is the same
@@ -232,8 +236,8 @@ struct Tile {
     // with a constant field, as at nearly every call, the place of the field folds to a constant
     __device__ __forceinline__ uint32_t at(uint32_t field, uint32_t h) const {
         const uint32_t below = narrow_below(field);
-        if (!narrow_field(field)) return (field - below) * cap + h;
-        return kWideFields * cap + below * (narrow + 1u) + min(h, narrow);
+        if (!narrow_field(field)) return h * kWideStride + (field - below);
+        return kWideStride * cap + min(h, narrow) * kNarrowStride + below;
     }
     __device__ __forceinline__ float& F(uint32_t field, uint32_t h) const { return fields[at(field, h)]; }
     __device__ __forceinline__ uint32_t& U(uint32_t field, uint32_t h) const { return reinterpret_cast<uint32_t*>(fields)[at(field, h)]; }
@@ -1058,7 +1062,12 @@ __device__ __forceinline__ void measure_primal(Tile& c, const float (&mrow)[N], 
     __syncthreads();
     double balance = 0.0;
 #pragma unroll
-    for (int j = 0; j < N; ++j) balance -= double(mrow[j]) * (double(dvec[j]) - c.vec[64 + j]);   // padded terms are exact zeros
+    for (int j = 0; j < N; ++j) {
+        // the mass row does not change over the solve: left to itself the compiler widens all of it to double once,
+        // ahead of the sweeps, and holds two registers an entry from there on
+        const float mass = opaque(mrow[j]);
+        balance -= double(mass) * (double(dvec[j]) - c.vec[64 + j]);   // padded terms are exact zeros
+    }
     // heads with an impulse add J^T lambda in head order (:2402-2436).  A unit head touches one coordinate: that
     // lane takes it from its own list when it comes up between the staged heads
     uint32_t next = 0u;
@@ -1282,7 +1291,7 @@ __host__ __device__ inline uint32_t FactorRegionFloats(uint32_t n) {
     return 2u * N * (N + 1u);   // a multiple of 4 since N is
 }
 __host__ __device__ inline uint32_t HeadFieldFloats(uint32_t cap, uint32_t narrow) {
-    return (kWideFields * cap + kNarrowFields * (narrow + 1u) + 3u) & ~3u;
+    return (kWideStride * cap + kNarrowStride * (narrow + 1u) + 3u) & ~3u;
 }
 // `cap` heads carry fields; `staged` of them (the contact heads) carry three Jacobian rows each.
 __host__ __device__ inline uint32_t SolverLdsFloats(uint32_t n, uint32_t cap, uint32_t staged) {
@@ -1325,7 +1334,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     c.jac = lds + FactorRegionFloats(n);
     c.fields = c.jac + 3u * staged_cap * c.ldj;
     c.vec = c.fields + HeadFieldFloats(cap, staged_cap);
-    if (lane < kNarrowFields) c.fields[kWideFields * cap + lane * (staged_cap + 1u) + staged_cap] = 0.0f;   // what a narrow field reads beyond its heads
+    if (lane < kNarrowFields) c.fields[kWideStride * cap + staged_cap * kNarrowStride + lane] = 0.0f;   // what a narrow field reads beyond its heads
     c.unit_list = reinterpret_cast<uint32_t*>(c.vec + 256);
     c.unit_lists = true; c.unit_count = 0u; c.staged_end = 0u; c.individual_end = 0u;
     const bool coordinate = lane < n;
