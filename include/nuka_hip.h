@@ -106,6 +106,16 @@ typedef struct nuka_template_desc_t {
     const uint32_t* excluded_pairs;  /* [pair][2] collidable rows, either order; nullable */
     uint32_t excluded_pair_count;
     uint32_t reserved1;
+    /* The MuJoCo contact law (src/constraint/law_source.hpp; src/scene/contact_filter.hpp:20-37 ContactParamsIn), read
+     * only when struct_size covers it.  A pair with a MuJoCo-sourced profile on either side builds compliant rows from
+     * the merged solref/solimp of both sides (src/phi/backend_cuda/ops/assemble_rows.cu:540-800) in place of the
+     * native velocity rows. */
+    const uint32_t* profile_law;     /* [profile] 0 native, 1 MuJoCo-sourced; nullable */
+    const float* profile_solref;     /* [profile][2] timeconst, dampratio (or -stiffness, -damping); nullable => 0.02, 1 */
+    const float* profile_solimp;     /* [profile][5] dmin dmax width midpoint power; nullable => 0.9 0.95 0.001 0.5 2 */
+    const float* profile_margin;     /* [profile][2] margin, gap; nullable => 0, 0 */
+    uint32_t contact_cone;           /* <option cone>: 0 pyramidal (four edge rows a point), 1 elliptic */
+    float contact_impratio;          /* <option impratio>; 0 => 1 */
 } nuka_template_desc_t;
 
 /* The world options of the cooked-template creator (the library's own descriptor; the reference's nuka_world_desc_t

@@ -16,6 +16,10 @@ SHAPE_SPHERE, SHAPE_CAPSULE, SHAPE_BOX, SHAPE_PLANE, SHAPE_CYLINDER, SHAPE_NONE 
 # collidable row roles of the template description
 ROLE_STATIC, ROLE_LINK_BODY, ROLE_PROXY = 0, 1, 2
 
+# constraint/law_source.hpp: where a shape's contact law comes from; nk/solve/row_types.hpp cone of the MuJoCo law
+LAW_NATIVE, LAW_MUJOCO = 0, 1
+CONE_PYRAMIDAL, CONE_ELLIPTIC = 0, 1
+
 # phi/articulation_contract.hpp:16-23
 DRIVE_PD_POSITION, DRIVE_TORQUE, DRIVE_VELOCITY, DRIVE_COMPUTED_TORQUE, DRIVE_OSC, DRIVE_ACTUATOR = 0, 1, 2, 3, 4, 5
 
@@ -41,6 +45,8 @@ class TemplateDescC(C.Structure):
         ("joint_limit_lower", _PF), ("joint_limit_upper", _PF), ("joint_limit_flags", _PB), ("joint_frictionloss", _PF),
         ("drive_mode", C.c_uint32), ("drive_rows", C.c_uint32),
         ("excluded_pairs", _PU), ("excluded_pair_count", C.c_uint32), ("reserved1", C.c_uint32),
+        ("profile_law", _PU), ("profile_solref", _PF), ("profile_solimp", _PF), ("profile_margin", _PF),
+        ("contact_cone", C.c_uint32), ("contact_impratio", C.c_float),
     ]
 
 
@@ -115,6 +121,8 @@ class Template:
         self.drive_mode = DRIVE_TORQUE
         self.drive_rows = False   # True: affine drives through joint drive rows; False: `tau` is the applied force
         self.excluded = []        # pairs of collidable rows that never pair (rows of one link are excluded by the cook)
+        self.contact_cone = CONE_PYRAMIDAL   # friction cone of MuJoCo-law contacts (<option cone>)
+        self.contact_impratio = 1.0          # <option impratio>
 
     def add_link(self, joint_type, parent, axis=(0, 0, 1), local_pos=(0, 0, 0), local_rot=(1, 0, 0, 0), mass=1.0,
                  diag_inertia=(0.01, 0.01, 0.01), com=(0, 0, 0), damping=0.0, armature=0.0, stiffness=0.0,
@@ -126,8 +134,12 @@ class Template:
                                lower=lower, upper=upper, frictionloss=frictionloss))
         return len(self.links) - 1
 
-    def add_profile(self, mu1, mu2=None):
-        self.profiles.append((mu1, mu1 if mu2 is None else mu2))
+    def add_profile(self, mu1, mu2=None, law=LAW_NATIVE, solref=(0.02, 1.0), solimp=(0.9, 0.95, 0.001, 0.5, 2.0), margin=0.0,
+                    gap=0.0):
+        """A contact profile; `law`, `solref`, `solimp`, `margin` and `gap` matter to MuJoCo-law contacts only
+        (scene/contact_filter.hpp:20-37 holds the defaults)."""
+        self.profiles.append(dict(mu=(mu1, mu1 if mu2 is None else mu2), law=law, solref=tuple(solref), solimp=tuple(solimp),
+                                  margin=(margin, gap)))
         return len(self.profiles) - 1
 
     def add_body(self, role, link=None, kind=SHAPE_NONE, params=(0, 0, 0, 0), local_pos=(0, 0, 0),
@@ -178,7 +190,11 @@ class Template:
             shape_conaffinity=np.array([b["conaffinity"] for b in B], dtype=u32),
             shape_group=np.array([b["group"] for b in B], dtype=u32),
             shape_profile=np.array([b["profile"] for b in B], dtype=u32),
-            profile_mu=np.array(self.profiles, dtype=f32).reshape(-1),
+            profile_mu=np.array([p["mu"] for p in self.profiles], dtype=f32).reshape(-1),
+            profile_law=np.array([p["law"] for p in self.profiles], dtype=u32),
+            profile_solref=np.array([p["solref"] for p in self.profiles], dtype=f32).reshape(-1),
+            profile_solimp=np.array([p["solimp"] for p in self.profiles], dtype=f32).reshape(-1),
+            profile_margin=np.array([p["margin"] for p in self.profiles], dtype=f32).reshape(-1),
             excluded_pairs=np.array(self.excluded, dtype=u32).reshape(-1),
         )
 
@@ -191,6 +207,7 @@ class Template:
         d.max_contacts_per_env = self.max_contacts_per_env
         d.drive_mode, d.drive_rows = self.drive_mode, 1 if self.drive_rows else 0
         d.excluded_pair_count = len(self.excluded)
+        d.contact_cone, d.contact_impratio = self.contact_cone, self.contact_impratio
         ctype = {np.dtype(np.float32): C.c_float, np.dtype(np.uint32): C.c_uint32, np.dtype(np.uint8): C.c_uint8}
         for name, arr in a.items():
             arr = np.ascontiguousarray(arr)

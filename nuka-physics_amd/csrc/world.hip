@@ -713,9 +713,11 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
     // a caller built against the header before the joint-row members passes the shorter size; those members read as zero
     constexpr size_t kTemplateBase = offsetof(nuka_template_desc_t, joint_limit_lower);
     constexpr size_t kTemplateJointRows = offsetof(nuka_template_desc_t, excluded_pairs);
+    constexpr size_t kTemplateExcluded = offsetof(nuka_template_desc_t, profile_law);
     constexpr size_t kWorldBase = offsetof(nuka_hip_world_desc_t, solver_fold_drive_damping);
     constexpr size_t kWorldDrives = offsetof(nuka_hip_world_desc_t, solver_substeps);
-    if ((tmpl->struct_size != sizeof(nuka_template_desc_t) && tmpl->struct_size != kTemplateJointRows && tmpl->struct_size != kTemplateBase) ||
+    if ((tmpl->struct_size != sizeof(nuka_template_desc_t) && tmpl->struct_size != kTemplateExcluded && tmpl->struct_size != kTemplateJointRows &&
+         tmpl->struct_size != kTemplateBase) ||
         (desc->struct_size != sizeof(nuka_hip_world_desc_t) && desc->struct_size != kWorldDrives && desc->struct_size != kWorldBase))
         return Error(NUKA_RESULT_INVALID_ARG, "struct_size mismatch");
     nuka_template_desc_t template_copy{};

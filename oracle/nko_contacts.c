@@ -754,16 +754,24 @@ void nko_env_narrowphase(nko_world* w, uint32_t env) {
         const size_t gid = (size_t)env * t->slots + slot;
         manifold m; m.count = 0u;
         uint32_t a = 0u, b = 0u;
-        const uint32_t law = 2u;   /* kContactLawSpeculative: no MuJoCo-sourced profile on this path (:232) */
+        uint32_t law = 2u;   /* kContactLawSpeculative unless a side's profile is MuJoCo-sourced (:232, 268-276) */
         if (slot < live) {
             a = w->candidate_pairs[gid * 2u]; b = w->candidate_pairs[gid * 2u + 1u];
             const shape_row sa = load_shape(t->shape_table, a), sb = load_shape(t->shape_table, b);
             const xform xa = xform_load(w->body_pose + (bbase + a) * 7u), xb = xform_load(w->body_pose + (bbase + b) * 7u);
             const prim pa = make_prim(sa, xa), pb = make_prim(sb, xb);
+            const int has_a = sa.profile < t->n_profiles, has_b = sb.profile < t->n_profiles;
+            if ((has_a && t->profile_law[sa.profile] == 1u) || (has_b && t->profile_law[sb.profile] == 1u)) law = 0u;   /* kContactLawCompliant */
+            float query_margin = separation;
+            if (law == 0u) {   /* :277-281: the profiles' margin + gap */
+                const float margin_a = has_a ? t->profile_margin[2u * sa.profile] + t->profile_margin[2u * sa.profile + 1u] : 0.0f;
+                const float margin_b = has_b ? t->profile_margin[2u * sb.profile] + t->profile_margin[2u * sb.profile + 1u] : 0.0f;
+                query_margin = margin_a + margin_b;
+            }
             /* :243-250 query band; both speeds are zero for link-owned collidables */
-            const float query = fmaxf(separation, fminf(contact_motion_radius(2.0f * separation, w->cfg.fixed_dt, 0.0f, 0.0f, 0.9f), reach));
+            const float query = fmaxf(query_margin, fminf(contact_motion_radius(2.0f * separation, w->cfg.fixed_dt, 0.0f, 0.0f, 0.9f), reach));
             primitive_pair(sa.kind, &pa, sb.kind, &pb, query, &m);
-            for (uint32_t i = 0u; i < m.count; ++i) m.penetration[i] += separation;   /* :295-296 */
+            if (law != 0u) for (uint32_t i = 0u; i < m.count; ++i) m.penetration[i] += separation;   /* :295-296 */
         }
         w->ucontact_count[gid] = m.count;
         w->ucontact_law[gid] = law;
@@ -858,12 +866,11 @@ static uint32_t resolve_side(const nko_template* t, uint32_t env, uint32_t colli
     return NKO_SIDE_ARTIC;
 }
 
-/* articulation_types.cuh:193-238 AccumulateChainJointForce with f = dir, tau = 0 */
-static void accumulate_chain(const nko_world* w, uint32_t env, uint32_t link_local, uint32_t dof_index, v3 point, v3 f, float* out) {
+/* articulation_types.cuh:193-238 AccumulateChainJointForce */
+void nko_accumulate_chain(const nko_world* w, uint32_t env, uint32_t link_local, uint32_t dof_index, v3 point, v3 f, v3 zero, float* out) {
     const nko_template* t = &w->t;
     const uint32_t stride = t->max_dof;
     const uint8_t type = t->joint_type[link_local];
-    const v3 zero = v3_make(0, 0, 0);
     if (type == NKO_FLOATING) {
         const xform base = xform_load(w->base_pose + (size_t)env * 7u);
         const v3 lever = v3_sub(point, base.p);
@@ -897,9 +904,49 @@ static void chain_jacobian_row(const nko_world* w, uint32_t env, uint32_t link_g
     for (uint32_t k = 0u; k < t->max_dof; ++k) out[k] = 0.0f;
     uint32_t link = link_global - env * t->nl;
     while (link != NKO_INVALID) {
-        if (nko_joint_dof(t->joint_type[link]) != 0u) accumulate_chain(w, env, link, t->link_dof[link], point, dir, out);
+        if (nko_joint_dof(t->joint_type[link]) != 0u) nko_accumulate_chain(w, env, link, t->link_dof[link], point, dir, v3_make(0, 0, 0), out);
         link = t->parent_link[link];
     }
+}
+
+/* One shape's contact parameters as MergeContactParams takes them: mu1, mu2, solref[2], solimp[5], margin, gap; a
+ * shape without a profile has the defaults (assemble_rows.cu:41-52 DefaultProfile, mu 1). */
+static void profile_terms(const nko_template* t, uint32_t profile, float out[11]) {
+    const float defaults[11] = {1.0f, 1.0f, 0.02f, 1.0f, 0.9f, 0.95f, 0.001f, 0.5f, 2.0f, 0.0f, 0.0f};
+    memcpy(out, defaults, sizeof(defaults));
+    if (profile >= t->n_profiles) return;
+    out[0] = t->profile_mu[2u * profile]; out[1] = t->profile_mu[2u * profile + 1u];
+    out[2] = t->profile_solref[2u * profile]; out[3] = t->profile_solref[2u * profile + 1u];
+    for (uint32_t k = 0u; k < 5u; ++k) out[4u + k] = t->profile_solimp[5u * profile + k];
+    out[9] = t->profile_margin[2u * profile]; out[10] = t->profile_margin[2u * profile + 1u];
+}
+/* scene/contact_filter.hpp:100-137 MergeContactParams at equal priority and solmix 1 on both sides (mix 1/2), arithmetic
+ * friction mixing: friction by max, solref mixed (or the minimum when one is in direct form), solimp mixed, margins
+ * and gaps added */
+void nko_merge_contact_params(const float a[11], const float b[11], float out[11]) {
+    const float mix = 1.0f / (1.0f + 1.0f), imix = 1.0f - mix;
+    out[0] = a[0] > b[0] ? a[0] : b[0];
+    out[1] = a[1] > b[1] ? a[1] : b[1];
+    if (a[2] > 0.0f && b[2] > 0.0f) { out[2] = mix * a[2] + imix * b[2]; out[3] = mix * a[3] + imix * b[3]; }
+    else { out[2] = a[2] < b[2] ? a[2] : b[2]; out[3] = a[3] < b[3] ? a[3] : b[3]; }
+    for (int i = 0; i < 5; ++i) out[4 + i] = mix * a[4 + i] + imix * b[4 + i];
+    out[9] = a[9] + b[9];
+    out[10] = a[10] + b[10];
+}
+/* math/cuda_vec_ops.cuh:187-196 MuJoCoContactFrame */
+static void mujoco_contact_frame(const float normal[3], v3 axis, float t1[3], float t2[3]) {
+    v3 n = v3_make(normal[0], normal[1], normal[2]);
+    const float l = v3_dot(n, n);
+    if (l > 1.0e-10f) { const float inv = nko_rsqrt(l); n = v3_make(n.x * inv, n.y * inv, n.z * inv); }
+    else n = v3_make(0.0f, 0.0f, 1.0f);
+    v3 tangent = v3_sub(axis, v3_scale(n, v3_dot(n, axis)));
+    if (v3_dot(tangent, tangent) < 0.25f) {
+        const v3 reference = n.y > -0.5f && n.y < 0.5f ? v3_make(0.0f, 1.0f, 0.0f) : v3_make(0.0f, 0.0f, 1.0f);
+        tangent = v3_sub(reference, v3_scale(n, v3_dot(n, reference)));
+    }
+    const v3 a = v3_scale(tangent, nko_rsqrt(v3_dot(tangent, tangent)));
+    const v3 b = v3_cross(n, a);
+    t1[0] = a.x; t1[1] = a.y; t1[2] = a.z; t2[0] = b.x; t2[1] = b.y; t2[2] = b.z;
 }
 
 /* ---- AssembleRows (assemble_rows.cu:325-394 ranges/clear, 406-801 emit, 1587-1605 chain J) ---- */
@@ -1046,9 +1093,28 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
         const float mu_b2 = sb.profile < t->n_profiles ? t->profile_mu[2u * sb.profile + 1u] : 1.0f;
         const float mu1 = mu_a1 > mu_b1 ? mu_a1 : mu_b1, mu2 = mu_a2 > mu_b2 ? mu_a2 : mu_b2;
         const int position_pass = w->cfg.solver_pos_iters > 0u;
-        w->contact_material[gid] = n_active > 0u ? nko_contact_material(mu1, mu2, w->ucontact_law[gid]) : 0u;   /* :620-622 */
+        const uint32_t law = w->ucontact_law[gid];
+        const int mujoco = law == 0u;   /* kContactLawCompliant (:480) */
+        /* the two sides' profiles merged (:540-594; contact_filter.hpp:100-137), a side without one at the defaults */
+        float side_a[11], side_b[11], merged[11];
+        profile_terms(t, sa.profile, side_a); profile_terms(t, sb.profile, side_b);
+        nko_merge_contact_params(side_a, side_b, merged);
+        const float* solref = merged + 2, *solimp = merged + 4;
+        const float margin = merged[9];
+        const uint32_t weight_a = kind_a == NKO_SIDE_ARTIC ? t->link_body[link_a - env * t->nl] : local_a;
+        const uint32_t weight_b = kind_b == NKO_SIDE_ARTIC ? t->link_body[link_b - env * t->nl] : local_b;
+        const float* invweight0 = w->body_invweight0 + (size_t)env * t->nb * 2u;
+        const float invweight = mujoco ? invweight0[2u * weight_a] + invweight0[2u * weight_b] : 0.0f;   /* :597 */
+        const int pyramidal = mujoco && t->cone == 0u;   /* condim 3 (:598) */
+        const float impratio = t->impratio;
+        v3 frame_axis = v3_make(0, 0, 0);   /* :601-605: a capsule on a plane aligns the pyramid with the capsule's axis */
+        if (pyramidal && sa.kind == 1u && sb.kind == 3u) frame_axis = nko_prim_rotate(xform_load(w->body_pose + ((size_t)env * t->nb + local_a) * 7u).r, v3_make(0, 0, 1));
+        if (pyramidal && sb.kind == 1u && sa.kind == 3u) frame_axis = nko_prim_rotate(xform_load(w->body_pose + ((size_t)env * t->nb + local_b) * 7u).r, v3_make(0, 0, 1));
+        w->contact_material[gid] = n_active > 0u ? (mujoco ? nko_contact_material_merged(merged, law, t->cone)
+                                                           : nko_contact_material(mu1, mu2, law)) : 0u;   /* :620-623 */
         for (uint32_t p = 0u; p < P; ++p) {
-            const int live = p < n_active && p < 4u;   /* velocity_only keeps every point (:625-626) */
+            /* velocity_only keeps every point; a compliant point lives inside its margin (:625-626) */
+            const int live = p < n_active && p < 4u && (!mujoco || w->ucontact_depth[gid * 4u + p] + margin > 0.0f);
             const size_t mp = gid * 4u + p;
             const uint32_t normal_row = base + p, t1_row = base + P + p, t2_row = base + 2u * P + p;
             v3 n = v3_make(0, 0, 1), point = v3_make(0, 0, 0), t0 = v3_make(1, 0, 0), t1v = v3_make(0, 1, 0);
@@ -1061,6 +1127,42 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
                 nko_contact_tangent_basis(&w->ucontact_normal[3u * mp], a, b);
                 t0 = v3_make(a[0], a[1], a[2]); t1v = v3_make(b[0], b[1], b[2]);
             }
+            if (pyramidal) {   /* :651-690: four scalar edges n +- mu t of the friction pyramid */
+                if (live) {
+                    float a[3], b[3];
+                    mujoco_contact_frame(&w->ucontact_normal[3u * mp], frame_axis, a, b);
+                    t0 = v3_make(a[0], a[1], a[2]); t1v = v3_make(b[0], b[1], b[2]);
+                }
+                const float d0 = w->ucontact_depth[mp];
+                const float edge_invweight = (invweight + mu1 * mu1 * invweight) * 2.0f * mu1 * mu1 / impratio;
+                const float pos = -d0 - margin;
+                float terms[6], discrete[3];
+                nko_compliant_row_terms(solref, solimp, pos, pos, 0.0f, edge_invweight, dt, 1, terms);
+                nko_discretize_compliant_row(terms[4], terms[5], terms[1], dt, discrete);
+                for (uint32_t edge = 0u; edge < 4u; ++edge) {
+                    const uint32_t rs = base + edge * P + p;
+                    nko_row row; memset(&row, 0, sizeof(row));
+                    lambda[rs] = 0.0f; pen[rs] = 0.0f; cj_link[rs] = NKO_INVALID; cj_link_b[rs] = NKO_INVALID;
+                    if (live) {
+                        const float mu = edge < 2u ? mu1 : mu2;
+                        const v3 tangent = edge < 2u ? t0 : t1v;
+                        const v3 dir = v3_add(n, v3_scale(tangent, (edge & 1u) ? -mu : mu));
+                        row.flags = NKO_ROW_ACTIVE | NKO_ROW_MUJOCO | NKO_ROW_PYRAMIDAL | (edge == 0u ? NKO_ROW_CONTACT_NORMAL : 0u);
+                        row.group_first = env * R + rs; row.group_normal_count = 1u; row.env = env;
+                        row.rhs = discrete[1]; row.compliance_alpha = discrete[0];
+                        row.lower = 0.0f; row.upper = FLT_MAX; row.mu = mu1; row.friction_secondary = mu2;
+                        row.a.kind = kind_a; row.a.index = idx_a; row.a.jlin = dir;
+                        row.b.kind = kind_b; row.b.index = idx_b; row.b.jlin = v3_scale(dir, -1.0f);
+                        if (kind_a == NKO_SIDE_ARTIC) { cj_link[rs] = link_a; cj_point[3u * rs] = point.x; cj_point[3u * rs + 1u] = point.y; cj_point[3u * rs + 2u] = point.z; }
+                        if (kind_b == NKO_SIDE_ARTIC) { cj_link_b[rs] = link_b; cj_point_b[3u * rs] = point.x; cj_point_b[3u * rs + 1u] = point.y; cj_point_b[3u * rs + 2u] = point.z; }
+                        w->row_reference_velocity_gain[(size_t)env * R + rs] = discrete[2];
+                        w->row_invweight[(size_t)env * R + rs] = edge_invweight;
+                        ++active_rows;
+                    }
+                    rows[rs] = row;
+                }
+                continue;
+            }
             {   /* normal row :692-755 */
                 nko_row row; memset(&row, 0, sizeof(row));
                 row.a.kind = row.b.kind = NKO_SIDE_STATIC; row.a.index = row.b.index = NKO_INVALID;
@@ -1071,11 +1173,20 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
                     const double roundoff = projection_roundoff(extent_v, extent_v, n);
                     const float clearance = roundoff > 0.0 ? nextafterf((float)roundoff, FLT_MAX) : 0.0f;
                     const float depth = d0 + clearance;
-                    pen[normal_row] = depth;
-                    row.flags = NKO_ROW_ACTIVE | NKO_ROW_CONTACT_NORMAL | NKO_ROW_BLOCK_NORMAL | NKO_ROW_SPECULATIVE;
+                    pen[normal_row] = mujoco ? fmaxf(d0, 0.0f) : depth;
+                    row.flags = NKO_ROW_ACTIVE | NKO_ROW_CONTACT_NORMAL | NKO_ROW_BLOCK_NORMAL | (mujoco ? NKO_ROW_MUJOCO : NKO_ROW_SPECULATIVE);
                     row.group_first = env * R + base; row.group_normal_count = P; row.env = env;
                     row.rhs = (fminf(depth, 0.0f) + (position_pass ? 0.0f : fminf(fmaxf(d0, 0.0f), w->cfg.solver_overlap_recovery_velocity * dt))) / (dt * dt);
                     row.compliance_alpha = 0.0f;   /* DiscretizeCompliantRow of a zero row: R = 0 (solref_solimp.hpp:40-44) */
+                    if (mujoco) {   /* :714-731: the spring-damper reference of the merged solref / solimp at this depth */
+                        const float pos = -d0 - margin;
+                        float terms[6], discrete[3];
+                        nko_compliant_row_terms(solref, solimp, pos, pos, 0.0f, invweight, dt, 1, terms);
+                        nko_discretize_compliant_row(terms[4], terms[5], terms[1], dt, discrete);
+                        row.rhs = discrete[1]; row.compliance_alpha = discrete[0];
+                        w->row_reference_velocity_gain[(size_t)env * R + normal_row] = discrete[2];
+                        w->row_invweight[(size_t)env * R + normal_row] = invweight;
+                    }
                     row.lower = 0.0f; row.upper = FLT_MAX; row.mu = mu1; row.friction_secondary = mu2;
                     row.a.kind = kind_a; row.a.index = idx_a; row.a.jlin = n;
                     row.b.kind = kind_b; row.b.index = idx_b; row.b.jlin = v3_make(-n.x, -n.y, -n.z);
@@ -1096,6 +1207,17 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
                     const v3 dir = tdir[k];
                     row.flags = NKO_ROW_ACTIVE | NKO_ROW_BLOCK_TANGENT;
                     row.group_first = env * R + base; row.group_normal_count = P; row.env = env;
+                    if (mujoco) {   /* :771-782: the tangent rows' compliance, which shapes the elliptic cone's metric */
+                        const float mu = k == 0u ? mu1 : mu2;
+                        const float tangent_invweight = invweight / impratio * (mu1 * mu1) / (mu * mu);
+                        float terms[6], discrete[3];
+                        nko_compliant_row_terms(solref, solimp, -w->ucontact_depth[mp] - margin, 0.0f, 0.0f, tangent_invweight, dt, 1, terms);
+                        nko_discretize_compliant_row(terms[4], terms[5], terms[1], dt, discrete);
+                        row.flags |= NKO_ROW_MUJOCO;
+                        row.compliance_alpha = discrete[0];
+                        w->row_reference_velocity_gain[(size_t)env * R + rs] = discrete[2];
+                        w->row_invweight[(size_t)env * R + rs] = tangent_invweight;
+                    }
                     row.lower = -FLT_MAX; row.upper = FLT_MAX; row.mu = mu1; row.friction_secondary = mu2;
                     row.a.kind = kind_a; row.a.index = idx_a; row.a.jlin = dir;
                     row.b.kind = kind_b; row.b.index = idx_b; row.b.jlin = v3_make(-dir.x, -dir.y, -dir.z);
@@ -1118,6 +1240,18 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
         if ((rows[r].flags & NKO_ROW_ACTIVE) && rows[r].a.kind == NKO_SIDE_ARTIC && rows[r].b.kind == NKO_SIDE_ARTIC &&
             rows[r].a.index == rows[r].b.index)
             for (uint32_t i = 0u; i < t->max_dof; ++i) { ja[i] += jb[i]; jb[i] = 0.0f; }
+    }
+    /* PrepareContactRowsKernel (:1134-1140): a compliant row's reference acceleration includes the damping of the
+     * velocity the step started from, ContactReferenceVelocity (:1072-1100) side A then side B */
+    const float* start = w->step_qdot_flat + (size_t)env * t->max_dof;
+    for (uint32_t r = 0u; r < R; ++r) {
+        if ((rows[r].flags & NKO_ROW_ACTIVE) == 0u || (rows[r].flags & NKO_ROW_MUJOCO) == 0u) continue;
+        float velocity = 0.0f;
+        if (rows[r].a.kind == NKO_SIDE_ARTIC)
+            for (uint32_t i = 0u; i < t->max_dof; ++i) velocity += w->chain_jacobian[((size_t)env * R + r) * t->max_dof + i] * start[i];
+        if (rows[r].b.kind == NKO_SIDE_ARTIC)
+            for (uint32_t i = 0u; i < t->max_dof; ++i) velocity += w->chain_jacobian_b[((size_t)env * R + r) * t->max_dof + i] * start[i];
+        rows[r].rhs += w->row_reference_velocity_gain[(size_t)env * R + r] * velocity;
     }
 }
 

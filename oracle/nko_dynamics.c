@@ -748,3 +748,50 @@ void nko_env_readout_drives(nko_world* w, uint32_t env) {
         w->tau[link] += w->actuator_effort[link];
     }
 }
+
+/* ArticulationReferenceWeightsKernel and BodyReferenceWeightsKernel (articulation.cu:425-500): the mass matrix at the
+ * current pose (armature included, no damping folded in), its factor, the diagonal of its inverse, and for every link
+ * the mean translational and rotational response of its centre of mass to a unit force and a unit moment. */
+void nko_env_reference_weights(nko_world* w, uint32_t env) {
+    const nko_template* t = &w->t;
+    const uint32_t nl = t->nl, nb = t->nb, md = t->max_dof, dof = t->nv;
+    float* weights = w->body_invweight0 + (size_t)env * nb * 2u;
+    for (uint32_t b = 0u; b < nb; ++b) weights[2u * b] = weights[2u * b + 1u] = 0.0f;   /* static rows: inverse mass zero */
+    if (dof == 0u) return;
+    nko_env_dynamics(w, env, 0u);   /* m, m_factor at the current pose; the caller has switched the damping fold off */
+    const float* factor = w->m_factor + (size_t)env * md * md;
+    float* diagonal = w->dof_invweight0 + (size_t)env * md;
+    float row[NKO_MAX_DOF], solution[NKO_MAX_DOF];
+    for (uint32_t d = 0u; d < dof; ++d) {
+        for (uint32_t i = 0u; i < dof; ++i) solution[i] = i == d ? 1.0f : 0.0f;
+        nko_solve_mass(factor, solution, dof, md);
+        diagonal[d] = solution[d];
+    }
+    if (t->joint_type[0] == NKO_FLOATING) {
+        const float rotation = (diagonal[0] + diagonal[1] + diagonal[2]) / 3.0f;
+        const float translation = (diagonal[3] + diagonal[4] + diagonal[5]) / 3.0f;
+        for (uint32_t i = 0u; i < 3u; ++i) { diagonal[i] = rotation; diagonal[i + 3u] = translation; }
+    }
+    for (uint32_t link = 0u; link < nl; ++link) {
+        const xform pose = xform_load(w->link_pose + ((size_t)env * nl + link) * 7u);
+        const v3 com = v3_make(t->link_inertial_frame[7u * link], t->link_inertial_frame[7u * link + 1u], t->link_inertial_frame[7u * link + 2u]);
+        const v3 point = v3_add(pose.p, nko_rotate_normalized(pose.r, com));
+        float weight[2] = {0.0f, 0.0f};
+        for (uint32_t axis = 0u; axis < 6u; ++axis) {
+            for (uint32_t d = 0u; d < dof; ++d) row[d] = 0.0f;
+            const v3 unit = v3_make(axis % 3u == 0u ? 1.0f : 0.0f, axis % 3u == 1u ? 1.0f : 0.0f, axis % 3u == 2u ? 1.0f : 0.0f);
+            const v3 none = v3_make(0.0f, 0.0f, 0.0f);
+            uint32_t walk = link;
+            while (walk != NKO_INVALID) {
+                if (nko_joint_dof(t->joint_type[walk]) != 0u)
+                    nko_accumulate_chain(w, env, walk, t->link_dof[walk], point, axis < 3u ? unit : none, axis < 3u ? none : unit, row);
+                walk = t->parent_link[walk];
+            }
+            for (uint32_t d = 0u; d < dof; ++d) solution[d] = row[d];
+            nko_solve_mass(factor, solution, dof, md);
+            for (uint32_t d = 0u; d < dof; ++d) weight[axis / 3u] += row[d] * solution[d];
+        }
+        const uint32_t body = t->link_body[link];
+        if (body < nb) { weights[2u * body] = weight[0] / 3.0f; weights[2u * body + 1u] = weight[1] / 3.0f; }
+    }
+}

@@ -24,7 +24,7 @@ enum {
     NKO_ROW_ACTIVE = 1u << 0, NKO_ROW_BLOCK_NORMAL = 1u << 2, NKO_ROW_BLOCK_TANGENT = 1u << 3,
     NKO_ROW_JOINT_LIMIT_LOWER = 1u << 4, NKO_ROW_JOINT_LIMIT_UPPER = 1u << 5,
     NKO_ROW_CONTACT_NORMAL = 1u << 6, NKO_ROW_VELOCITY_ONLY = 1u << 7, NKO_ROW_SPECULATIVE = 1u << 8,
-    NKO_ROW_MUJOCO = 1u << 11, NKO_ROW_FRICTION = 1u << 1
+    NKO_ROW_MUJOCO = 1u << 11, NKO_ROW_PYRAMIDAL = 1u << 12, NKO_ROW_FRICTION = 1u << 1
 };
 /* phi/op_schema.hpp:36-52 */
 enum { NKO_STATUS_PAIR_OVERFLOW = 1u << 0, NKO_STATUS_DOF_OVERFLOW = 1u << 2, NKO_STATUS_INVALID_ENDPOINT = 1u << 6,
@@ -80,6 +80,14 @@ typedef struct {
     float* body_collidable_local; /* nb*7 */
     float* body_init_pose;        /* nb*7 */
     float* profile_mu;            /* n_profiles*2 */
+    /* MuJoCo-law profiles (scene_ir.hpp:116; contact_filter.hpp:20-37): law source, solref, solimp, margin and gap */
+    uint32_t* profile_law;        /* n_profiles */
+    float* profile_solref;        /* n_profiles*2 */
+    float* profile_solimp;        /* n_profiles*5 */
+    float* profile_margin;        /* n_profiles*2 */
+    uint32_t cone;                /* constraint::FrictionCone: 0 pyramidal, 1 elliptic */
+    float impratio;
+    int any_mujoco;
 } nko_template;
 
 struct nko_world {
@@ -103,6 +111,8 @@ struct nko_world {
     float *solver_residual;
     /* solver state kept between steps (block_descent.cu BlockScratch articulation_velocity/free) */
     float *solver_velocity, *solver_free, *solver_penalty;
+    /* MuJoCo-law reference weights and per-row records (fields.yaml:863, 168-169) */
+    float *body_invweight0, *dof_invweight0, *row_invweight, *row_reference_velocity_gain, *step_qdot_flat;
     /* contact cache carried between steps (fields.yaml:524-539, 155, 791, 844) */
     uint64_t *contact_material, *contact_cache_pair, *contact_cache_feature, *contact_cache_material;
     float *contact_cache_lambda, *contact_cache_normal;
@@ -163,6 +173,9 @@ void nko_env_readout_contact_wrench(nko_world* w, uint32_t env);
 void nko_env_dynamics(nko_world* w, uint32_t env, uint32_t integrate_velocity);
 void nko_env_integrate_position(nko_world* w, uint32_t env);
 void nko_env_link_velocities(nko_world* w, uint32_t env);
+void nko_env_reference_weights(nko_world* w, uint32_t env);
+/* the generalized force of a force f and a moment tau applied at `point`, added into one link's coordinates */
+void nko_accumulate_chain(const nko_world* w, uint32_t env, uint32_t link_local, uint32_t dof_index, v3 point, v3 f, v3 tau, float* out);
 void nko_env_sync_body_pose(nko_world* w, uint32_t env);
 void nko_env_aabbs(nko_world* w, uint32_t env);
 void nko_env_pairs(nko_world* w, uint32_t env);

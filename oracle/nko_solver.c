@@ -5,7 +5,7 @@
  *
  * Where the reference reduces across a 32-lane warp with a shuffle tree, the oracle adds in index
  * order; the compensated TileSum arithmetic, fmaf uses and branch structure are kept.  Free rigid
- * bodies (6x6 blocks), mimic couplings and elliptic (MuJoCo-law) cones are outside this restatement.
+ * bodies (6x6 blocks) and mimic couplings are outside this restatement.
  */
 #include <stdio.h>
 
@@ -268,6 +268,8 @@ typedef struct {
     uint32_t slot, stride, axes, owner[2], unit[2], row[2];
     float unit_value[2];
     float rho, compliance, lower, upper, mu_first, mu_second, normal_bound;
+    int elliptic;            /* three axes of a MuJoCo-law contact: the elliptic cone (block_descent_tile.cuh:645, 778) */
+    v3 cone_compliance;      /* the compliances of the normal row and of its two tangent rows */
     v3 residual, dual, move, step, base;
     scalar_response response;
     relaxation relax;
@@ -287,6 +289,16 @@ typedef struct {
 
 /* TileResponse (block_descent_tile.cuh:678-681) with EvaluateAugmentedResponse (block_descent.cu:1593-1621), Coulomb cone */
 static void tile_response(const tile_head* t, v3 move, v3* f, float* c) {
+    if (t->elliptic) {   /* block_descent.cu:1595-1601 */
+        const float dual[3] = {t->dual.x, t->dual.y, t->dual.z};
+        const float residual[3] = {t->residual.x - move.x, t->residual.y - move.y, t->residual.z - move.z};
+        const float compliance[3] = {t->cone_compliance.x, t->cone_compliance.y, t->cone_compliance.z};
+        float out[9];
+        nko_elliptic_impulse(dual, t->rho, residual, compliance, t->mu_first, out);
+        *f = v3_make(out[0], out[1], out[2]);
+        for (int i = 0; i < 6; ++i) c[i] = out[3 + i];
+        return;
+    }
     float ni, nc;
     scalar_impulse(t->dual.x, t->rho, t->residual.x - move.x, t->compliance, t->lower, t->upper, t->response, &ni, &nc);
     *f = v3_make(ni, 0.0f, 0.0f);
@@ -779,7 +791,13 @@ static void update_duals(tile* c, float* lambda_env, dual_momentum* momentum, in
         relaxation relax = t.relax;
         if (!commit) memset(&relax, 0, sizeof(relax));
         v3 dual;
-        if (!contact) dual = v3_make(normal, 0.0f, 0.0f);   /* ProjectRowDual block_descent.cu:799-804 */
+        const float t_dual[3] = {t.dual.x, t.dual.y, t.dual.z}, t_residual[3] = {t.residual.x, t.residual.y, t.residual.z};
+        const float t_compliance[3] = {t.cone_compliance.x, t.cone_compliance.y, t.cone_compliance.z};
+        if (t.elliptic) {   /* :2509-2510 */
+            float out[9];
+            nko_elliptic_impulse(t_dual, t.rho, t_residual, t_compliance, t.mu_first, out);
+            dual = v3_make(out[0], out[1], out[2]);
+        } else if (!contact) dual = v3_make(normal, 0.0f, 0.0f);   /* ProjectRowDual block_descent.cu:799-804 */
         else {
             v3 f; float cv[6];
             tangent_impulse(t.dual, t.rho, t.residual, normal, t.mu_first, t.mu_second, &f, cv);
@@ -789,6 +807,12 @@ static void update_duals(tile* c, float* lambda_env, dual_momentum* momentum, in
         multiplier_steps(t.dual, dual, t.response.residual_scale, t.response.dual_scale, t.rho, contact ? t.mu_first : 0.0f,
                          contact ? t.mu_second : 0.0f, step);
         if (!commit && t.response.residual_scale > 0.0f) step[0] = fabsf(dual.x - t.dual.x) / t.response.residual_scale;
+        if (t.elliptic) {   /* :2516-2519 */
+            const float next[3] = {dual.x, dual.y, dual.z};
+            float delta[3];
+            nko_elliptic_multiplier_step(t_dual, next, t.rho, t_compliance, delta);
+            step[0] = delta[0]; step[1] = fmaxf(delta[1], delta[2]);
+        }
         const v3 physical = commit ? dual : t.dual;
         if (!contact) {
             const int normal_row = (rows[t.slot].flags & NKO_ROW_CONTACT_NORMAL) != 0u;
@@ -803,17 +827,23 @@ static void update_duals(tile* c, float* lambda_env, dual_momentum* momentum, in
                 lambda_env[local + t.stride] = dual.y;
                 lambda_env[local + 2u * t.stride] = dual.z;
             }
-            const v3 v = v3_make(-t.residual.x + t.compliance * physical.x, -t.residual.y, -t.residual.z);
-            const uint32_t nb = residual_bits(physical.x > 0.0f ? fabsf(v.x) : fmaxf(-v.x, 0.0f));
-            if (nb > steps[0]) steps[0] = nb;
-            const uint32_t tb = residual_bits(fmaxf(step[1], fmaxf(along_axis(physical.y, v.y), along_axis(physical.z, v.z))));
-            if (tb > steps[1]) steps[1] = tb;
+            if (t.elliptic) {   /* :2540-2542 */
+                if (residual_bits(step[0]) > steps[0]) steps[0] = residual_bits(step[0]);
+                if (residual_bits(step[1]) > steps[1]) steps[1] = residual_bits(step[1]);
+            } else {
+                const v3 v = v3_make(-t.residual.x + t.compliance * physical.x, -t.residual.y, -t.residual.z);
+                const uint32_t nb = residual_bits(physical.x > 0.0f ? fabsf(v.x) : fmaxf(-v.x, 0.0f));
+                if (nb > steps[0]) steps[0] = nb;
+                const uint32_t tb = residual_bits(fmaxf(step[1], fmaxf(along_axis(physical.y, v.y), along_axis(physical.z, v.z))));
+                if (tb > steps[1]) steps[1] = tb;
+            }
         }
         if (!commit) continue;
         if (velocity) lambda_env[local] = dual.x;
         const int extrapolate = contact || t.response.dual_scale != 0.0f;
         const v3 base = t.base;
-        const v3 metric = multiplier_metric(t.response.residual_scale, t.rho, contact, t.mu_first, t.mu_second);
+        v3 metric = multiplier_metric(t.response.residual_scale, t.rho, contact, t.mu_first, t.mu_second);
+        if (t.elliptic) { v3 unused; elliptic_response(t.rho, t.cone_compliance, &metric, &unused); }   /* :2555-2557 */
         if (extrapolate) restart += momentum_restart(t.dual, dual, base, metric);
         if (momentum != NULL) th->move = base;
         th->dual = dual;
@@ -919,6 +949,9 @@ void nko_env_solve(nko_world* w, uint32_t env) {
         t->response = float_scalar_response(rho, t->compliance);
         t->lower = row->lower; t->upper = row->upper; t->mu_first = row->mu; t->mu_second = row->friction_secondary;
         t->normal_bound = 0.0f;
+        t->elliptic = t->axes == 3u && (row->flags & NKO_ROW_MUJOCO) != 0u;   /* :778-780 */
+        t->cone_compliance = v3_make(t->compliance, t->axes == 3u ? rows[slot + t->stride].compliance_alpha : 0.0f,
+                                     t->axes == 3u ? rows[slot + 2u * t->stride].compliance_alpha : 0.0f);
         const uint32_t local = slot - env * R;
         t->dual = v3_make(lambda_env[local], t->axes == 3u ? lambda_env[local + t->stride] : 0.0f, t->axes == 3u ? lambda_env[local + 2u * t->stride] : 0.0f);
         t->base = t->dual;
@@ -1064,6 +1097,7 @@ void nko_env_solve(nko_world* w, uint32_t env) {
             if (!position) t->owner[0] = t->owner[1] = NO_BLOCK;
             coupled = coupled || (t->owner[0] != NO_BLOCK && t->owner[1] != NO_BLOCK);
             t->axes = 1u;
+            t->elliptic = 0;   /* :2691 */
             t->compliance = 0.0f; t->lower = 0.0f; t->upper = FLT_MAX;
             t->response = float_scalar_response(t->rho, 0.0f);
             t->residual = v3_make(bias, 0.0f, 0.0f);

@@ -43,7 +43,7 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
     copy_or_zero(t->joint_stiffness, d->joint_stiffness, nl);
     copy_or_zero(t->joint_spring_reference, d->joint_spring_reference, nl);
     const int has_joint_rows = d->struct_size >= offsetof(nko_template_desc, excluded_pairs);
-    const int has_excluded = d->struct_size >= sizeof(nko_template_desc);
+    const int has_excluded = d->struct_size >= offsetof(nko_template_desc, profile_law);
     copy_or_zero(t->joint_limit_lower, has_joint_rows ? d->joint_limit_lower : NULL, nl);
     copy_or_zero(t->joint_limit_upper, has_joint_rows ? d->joint_limit_upper : NULL, nl);
     copy_or_zero(t->joint_frictionloss, has_joint_rows ? d->joint_frictionloss : NULL, nl);
@@ -88,6 +88,22 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
     t->body_collidable_local = ALLOC(float, nb * 7u); t->body_init_pose = ALLOC(float, nb * 7u);
     t->profile_mu = ALLOC(float, t->n_profiles * 2u);
     if (t->n_profiles) memcpy(t->profile_mu, d->profile_mu, t->n_profiles * 2u * sizeof(float));
+    {   /* MuJoCo-law profile terms, defaults of ContactParamsIn (contact_filter.hpp:20-37) where not authored */
+        const int has = d->struct_size >= sizeof(nko_template_desc);
+        t->profile_law = ALLOC(uint32_t, t->n_profiles); t->profile_solref = ALLOC(float, t->n_profiles * 2u);
+        t->profile_solimp = ALLOC(float, t->n_profiles * 5u); t->profile_margin = ALLOC(float, t->n_profiles * 2u);
+        const float solimp[5] = {0.9f, 0.95f, 0.001f, 0.5f, 2.0f};
+        for (uint32_t i = 0u; i < t->n_profiles; ++i) {
+            t->profile_law[i] = has && d->profile_law ? d->profile_law[i] : 0u;
+            t->profile_solref[2u * i] = has && d->profile_solref ? d->profile_solref[2u * i] : 0.02f;
+            t->profile_solref[2u * i + 1u] = has && d->profile_solref ? d->profile_solref[2u * i + 1u] : 1.0f;
+            for (uint32_t k = 0u; k < 5u; ++k) t->profile_solimp[5u * i + k] = has && d->profile_solimp ? d->profile_solimp[5u * i + k] : solimp[k];
+            for (uint32_t k = 0u; k < 2u; ++k) t->profile_margin[2u * i + k] = has && d->profile_margin ? d->profile_margin[2u * i + k] : 0.0f;
+            t->any_mujoco = t->any_mujoco || t->profile_law[i] == 1u;
+        }
+        t->cone = has ? d->contact_cone : 0u;
+        t->impratio = has && d->contact_impratio > 0.0f ? d->contact_impratio : 1.0f;
+    }
     for (uint32_t b = 0u; b < nb; ++b) {
         const uint32_t role = d->body_role[b], link = d->body_link[b];
         float* row = t->shape_table + 13u * b;
@@ -190,6 +206,7 @@ static void free_template(nko_template* t) {
     free(t->link_geom_local); free(t->link_geom_kind); free(t->shape_table); free(t->excluded_pairs); free(t->body_to_link);
     free(t->body_to_articulation); free(t->body_collidable_link); free(t->body_collidable_body);
     free(t->body_collidable_local); free(t->body_init_pose); free(t->profile_mu);
+    free(t->profile_law); free(t->profile_solref); free(t->profile_solimp); free(t->profile_margin);
 }
 
 nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc* desc) {
@@ -239,6 +256,9 @@ nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc*
     w->env_status = ALLOC(uint32_t, E); w->vbd_velocity_sweep_count = ALLOC(uint32_t, E);
     w->solver_residual = ALLOC(float, E * 4u);
     w->solver_velocity = ALLOC(float, E * md); w->solver_free = ALLOC(float, E * md); w->solver_penalty = ALLOC(float, E * R);
+    w->body_invweight0 = ALLOC(float, E * nb * 2u); w->dof_invweight0 = ALLOC(float, E * md);
+    w->row_invweight = ALLOC(float, E * R); w->row_reference_velocity_gain = ALLOC(float, E * R);
+    w->step_qdot_flat = ALLOC(float, E * md);
     w->contact_material = ALLOC(uint64_t, E * S); w->contact_cache_pair = ALLOC(uint64_t, E * S * 4u);
     w->contact_cache_feature = ALLOC(uint64_t, E * S * 4u); w->contact_cache_material = ALLOC(uint64_t, E * S * 4u);
     w->contact_cache_lambda = ALLOC(float, E * S * 16u); w->contact_cache_normal = ALLOC(float, E * S * 12u);
@@ -265,6 +285,11 @@ nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc*
         for (size_t l = 0u; l < nl; ++l) memcpy(w->link_pose + (e * nl + l) * 7u, id, sizeof(id));
         for (size_t b = 0u; b < nb; ++b) memcpy(w->body_pose + (e * nb + b) * 7u, t->body_init_pose + 7u * b, sizeof(id));
     }
+    /* nk/pipeline/world.cpp:553-561: creation exposes the poses of the rest state and the reference weights at them */
+    if (t->any_mujoco) {
+        nko_fk_world_poses(w);
+        nko_reference_weights(w);
+    }
     return w;
 }
 
@@ -281,6 +306,7 @@ void nko_world_destroy(nko_world* w) {
     free(w->chain_jacobian_b); free(w->row_cj_link); free(w->row_cj_link_b); free(w->row_count); free(w->contact_count);
     free(w->contact_row_extent); free(w->env_status); free(w->vbd_velocity_sweep_count); free(w->solver_residual);
     free(w->solver_velocity); free(w->solver_free); free(w->solver_penalty);
+    free(w->body_invweight0); free(w->dof_invweight0); free(w->row_invweight); free(w->row_reference_velocity_gain); free(w->step_qdot_flat);
     free(w->step_env_status); free(w->step_link_impulse); free(w->step_link_moment); free(w->step_joint_limit_impulse);
     free(w->contact_material); free(w->contact_cache_pair); free(w->contact_cache_feature); free(w->contact_cache_material);
     free(w->contact_cache_lambda); free(w->contact_cache_normal); free(w->contact_cache_age); free(w->contact_cache_current_owner);
@@ -312,6 +338,8 @@ void nko_world_destroy(nko_world* w) {
     X(row_cj_link_b, uint32_t, E * R) X(row_count, uint32_t, E) X(contact_count, uint32_t, E) \
     X(contact_row_extent, uint32_t, E * 2u) X(env_status, uint32_t, E) X(vbd_velocity_sweep_count, uint32_t, E) \
     X(solver_residual, float, E * 4u) X(solver_penalty, float, E * R) \
+    X(body_invweight0, float, E * nb * 2u) X(dof_invweight0, float, E * md) X(row_invweight, float, E * R) \
+    X(row_reference_velocity_gain, float, E * R) X(step_qdot_flat, float, E * md) \
     X(contact_material, uint64_t, E * S) X(contact_cache_pair, uint64_t, E * S * 4u) X(contact_cache_feature, uint64_t, E * S * 4u) \
     X(contact_cache_material, uint64_t, E * S * 4u) X(contact_cache_lambda, float, E * S * 16u) \
     X(contact_cache_normal, float, E * S * 12u) X(contact_cache_age, uint32_t, E * S * 4u) \
@@ -380,9 +408,31 @@ void nko_contact_warm_start(nko_world* w, uint32_t phase) {
 void nko_block_descent_solve(nko_world* w) { FOR_ENVS(nko_env_solve(w, env)) }
 void nko_integrate_position(nko_world* w) { FOR_ENVS(nko_env_integrate_position(w, env)) }
 void nko_fk_link_velocities(nko_world* w) { FOR_ENVS(nko_env_link_velocities(w, env)) }
+void nko_reference_weights(nko_world* w) {
+    const int fold = w->fold_drive_damping;
+    w->fold_drive_damping = 0;   /* ComputeArticulationMass without drive damping (articulation.cu:452-453) */
+    FOR_ENVS(nko_env_reference_weights(w, env))
+    w->fold_drive_damping = fold;
+}
 
 /* Op order of one step (src/nk/pipeline/pipeline.cpp:374-986) for an articulated world with ground contact. */
+/* OpSnapshotStepVelocity (assemble_rows.cu:1457-1477, PackQdotFlatMultiKernel :200-214): the generalized velocity the
+ * step starts from, which the compliant rows' reference acceleration is taken at (pipeline.cpp:367-375) */
+void nko_snapshot_step_velocity(nko_world* w) {
+    const nko_template* t = &w->t;
+    for (size_t env = 0u; env < w->env_count; ++env)
+        for (uint32_t d = 0u; d < t->max_dof; ++d) {
+            float value = 0.0f;
+            if (d < t->nv) {
+                const uint32_t link = t->dof_link[d], component = t->dof_component[d];
+                value = component == NKO_INVALID ? w->qdot[env * t->nl + link] : w->link_velocity[(env * t->nl + link) * 6u + component];
+            }
+            w->step_qdot_flat[env * t->max_dof + d] = value;
+        }
+}
+
 static void step_interval(nko_world* w) {
+    if (w->t.rows_per_env > 0u) nko_snapshot_step_velocity(w);
     nko_fk_world_poses(w);
     if (w->t.joint_drive_rows > 0u) nko_apply_drives(w);
     nko_articulation_dynamics(w, 1u);

@@ -98,6 +98,13 @@ typedef struct nko_template_desc {
     const uint32_t* excluded_pairs;
     uint32_t excluded_pair_count;
     uint32_t reserved1;
+    /* MuJoCo-law contact profiles; read only when struct_size covers them */
+    const uint32_t* profile_law;
+    const float* profile_solref;
+    const float* profile_solimp;
+    const float* profile_margin;
+    uint32_t contact_cone;
+    float contact_impratio;
 } nko_template_desc;
 
 typedef struct nko_world_desc {
@@ -148,6 +155,14 @@ void nko_integrate_position(nko_world* w);
 void nko_fk_link_velocities(nko_world* w);
 /* The whole op list of one step, in the reference's order. */
 void nko_world_step(nko_world* w);
+/* ReferenceWeights (articulation.cu:425-500): body_invweight0 and dof_invweight0 at the current poses; creation runs it
+ * once at the template's rest pose. */
+void nko_reference_weights(nko_world* w);
+void nko_snapshot_step_velocity(nko_world* w);
+/* scene/contact_filter.hpp:100-137 MergeContactParams of two profiles of equal priority and solmix:
+ * out = mu1, mu2, solref[2], solimp[5], margin, gap */
+void nko_merge_contact_params(const float a[11], const float b[11], float out[11]);
+uint64_t nko_contact_material_merged(const float merged[11], uint32_t law, uint32_t cone);
 
 /* Stand-alone pieces exposed for unit pins. */
 void nko_make_spatial_inertia(float mass, const float diag[3], const float inertial_frame[7], float out[36]);
@@ -164,8 +179,8 @@ float nko_cone_argument(float dual, float rho, float mu, float residual);
 /* FactorTileBlock + SolveTileBlock (block_descent_tile.cuh:1622-1666) up to 32 coordinates, FactorTileColumns +
  * SolveWideTileBlock (:209-252, 1866-1895) past them; see nko_solver.c */
 int nko_tile_cholesky_solve(const float* h, uint32_t n, const float* g, float* factor, float* d);
-/* The compliant (MuJoCo-law) row terms and the elliptic cone of the reference's row math.  No device counterpart: the
- * product builds rows of the native law only.  Held so the reference's known answers for them are checked here too. */
+/* The compliant (MuJoCo-law) row terms and the elliptic cone of the reference's row math (constraint/solref_solimp.hpp,
+ * nk/solve/augmented_row.hpp:48-108), as the contact rows of a MuJoCo-sourced profile and the block descent use them. */
 void nko_compliant_row_terms(const float solref[2], const float solimp[5], float pos_imp, float pos_aref, float vel, float invweight,
                              float dt, int refsafe, float out[6]);
 void nko_discretize_compliant_row(float R, float aref_bias, float damping, float dt, float out[3]);
