@@ -210,6 +210,10 @@ typedef struct nuka_scene_t* nuka_scene_handle;
 #define NUKA_SCENE_FIXED_BASE 2u
 /* A static ground plane z = 0 joins the file's collidables (a URDF describes the robot only). */
 #define NUKA_SCENE_GROUND_PLANE 4u
+/* MJCF only: the geoms keep the native contact law (speculative velocity rows).  Without it every geom is
+ * MuJoCo-sourced, as in the reference's importer (src/import/mjcf_importer.cpp:790): its friction, solref, solimp,
+ * margin and gap make a contact profile of the MuJoCo law, with the cone and impratio of <option>. */
+#define NUKA_SCENE_NATIVE_CONTACT_LAW 8u
 nuka_result_t nuka_scene_load_mjcf(const char* path, uint32_t flags, nuka_scene_handle* out);
 nuka_result_t nuka_scene_load_urdf(const char* path, uint32_t flags, nuka_scene_handle* out);
 void nuka_scene_destroy(nuka_scene_handle scene);

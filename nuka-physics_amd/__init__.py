@@ -38,6 +38,7 @@ class SceneInfoC(C.Structure):
 SCENE_PLANE_CONTACTS_ONLY = 1
 SCENE_FIXED_BASE = 2
 SCENE_GROUND_PLANE = 4
+SCENE_NATIVE_CONTACT_LAW = 8
 
 
 class ParamInfoC(C.Structure):
@@ -223,10 +224,12 @@ class Scene:
                       link_diag_inertia=3 * nl, joint_damping=nl, joint_armature=nl, joint_stiffness=nl, joint_spring_reference=nl,
                       body_role=nb, body_link=nb, body_local=7 * nb, shape_kind=nb, shape_params=4 * nb, shape_contype=nb,
                       shape_conaffinity=nb, shape_group=nb, shape_profile=nb, profile_mu=2 * npf, joint_limit_lower=nl,
+                      profile_law=npf if d.profile_law else 0, profile_solref=2 * npf if d.profile_solref else 0,
+                      profile_solimp=5 * npf if d.profile_solimp else 0, profile_margin=2 * npf if d.profile_margin else 0,
                       joint_limit_upper=nl, joint_limit_flags=nl, joint_frictionloss=nl, excluded_pairs=2 * d.excluded_pair_count)
         out = {name: np.ctypeslib.as_array(getattr(d, name), shape=(count,)).copy() if count else np.zeros(0, np.float32)
                for name, count in shapes.items()}
-        out.update(drive_mode=d.drive_mode, drive_rows=d.drive_rows)
+        out.update(drive_mode=d.drive_mode, drive_rows=d.drive_rows, contact_cone=d.contact_cone, contact_impratio=d.contact_impratio)
         return out
 
     def initial_state(self):

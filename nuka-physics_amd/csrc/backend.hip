@@ -49,6 +49,7 @@ void RegisterOps() {
     set(NkOp::ReadoutDrives, &OpReadoutDrives);
     set(NkOp::ReadoutContactWrench, &OpReadoutContactWrench);
     set(NkOp::AccumulateStep, &OpAccumulateStep);
+    set(NkOp::ReferenceWeights, &OpReferenceWeights);
 }
 
 void Fail(nuka_phi_execution_error* error, Status status, uint16_t op, int native, const char* message) {

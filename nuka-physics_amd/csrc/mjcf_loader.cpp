@@ -4,8 +4,10 @@
 // same body -> link rules, default classes, joint anchors, inertial sources and actuator mapping.  Host code only.
 //
 // Not read: meshes, height fields, materials, cameras, lights, sensors, sites, equalities, <contact> pairs, ball
-// joints (rejected), tendons.  The joint and contact laws are this library's native ones: the
-// solref / solimp compliant rows the reference attaches to MJCF joints and geoms are not built.
+// joints (rejected), tendons.  Geoms carry the MuJoCo contact law as in the reference's importer (every MJCF shape is
+// MuJoCo-sourced, mjcf_importer.cpp:790): friction, solref, solimp, margin and gap go into contact profiles, and
+// <option cone impratio> selects the cone.  The joint rows keep this library's native law: the solref / solimp
+// compliant limit and friction rows the reference attaches to MJCF joints are not built.
 #include "scene_loader.h"
 
 #include "scene_build.h"
@@ -44,6 +46,9 @@ struct GeomDefaults : Frame {
     bool has_conaffinity = false; uint32_t conaffinity = 1u;
     bool has_group = false;       int32_t group = 0;
     float friction[3] = {1.0f, 0.005f, 0.0001f};
+    float solref[2] = {0.02f, 1.0f};
+    float solimp[5] = {0.9f, 0.95f, 0.001f, 0.5f, 2.0f};
+    float margin = 0.0f, gap = 0.0f;
     float density = 1000.0f, mass = -1.0f;
 };
 struct GeneralDefaults {
@@ -98,6 +103,10 @@ void ApplyGeomAttributes(const Element& e, GeomDefaults* g) {
     if (QueryInt(e, "conaffinity", &value)) { g->conaffinity = uint32_t(value); g->has_conaffinity = true; }
     if (QueryInt(e, "group", &value)) { g->group = int32_t(value); g->has_group = true; }
     ParseFloats(e.Attribute("friction"), g->friction, 3);
+    ParseFloats(e.Attribute("solref"), g->solref, 2);
+    ParseFloats(e.Attribute("solimp"), g->solimp, 5);
+    QueryFloat(e, "margin", &g->margin);
+    QueryFloat(e, "gap", &g->gap);
     QueryFloat(e, "density", &g->density);
     QueryFloat(e, "mass", &g->mass);
 }
@@ -275,6 +284,13 @@ struct Builder : SceneParts {
             ParseFloats(e.Attribute("friction"), friction, 3);
             g.friction = friction[0];
             g.friction_authored = g.friction != 1.0f;
+            g.solref[0] = gd.solref[0]; g.solref[1] = gd.solref[1];
+            for (int k = 0; k < 5; ++k) g.solimp[k] = gd.solimp[k];
+            g.margin = gd.margin; g.gap = gd.gap;
+            ParseFloats(e.Attribute("solref"), g.solref, 2);
+            ParseFloats(e.Attribute("solimp"), g.solimp, 5);
+            QueryFloat(e, "margin", &g.margin);
+            QueryFloat(e, "gap", &g.gap);
             float density = gd.density, geom_mass = gd.mass;
             QueryFloat(e, "density", &density);
             QueryFloat(e, "mass", &geom_mass);
@@ -515,6 +531,12 @@ std::unique_ptr<Scene> LoadMjcf(const std::string& path, uint32_t flags) {
     if (const Element* option = mujoco->First("option")) {
         QueryFloat(*option, "timestep", &scene->timestep);
         ParseFloats(option->Attribute("gravity"), scene->gravity, 3);
+        if (const char* cone = option->Attribute("cone")) {   // mjcf_importer.cpp:1724-1728
+            if (std::string(cone) == "elliptic") scene->contact_cone = 1u;
+            else if (std::string(cone) == "pyramidal") scene->contact_cone = 0u;
+            else throw std::runtime_error("MJCF: invalid option cone");
+        }
+        QueryFloat(*option, "impratio", &scene->contact_impratio);
     }
     if (const Element* compiler = mujoco->First("compiler")) {
         if (const char* angle = compiler->Attribute("angle")) {
@@ -598,12 +620,25 @@ void FlattenScene(const SceneParts& b, uint32_t flags, uint32_t drive_mode, Scen
         return g.kind == kShapeSphere || g.kind == kShapeCapsule || g.kind == kShapeBox || g.kind == kShapePlane || g.kind == kShapeCylinder;
     };
     auto collides = [](const Geom& g) { return g.contype != 0u || g.conaffinity != 0u; };
+    // Every geom's contact terms are one profile, shared by the geoms that agree on all of them.  Under the native law
+    // only an authored friction needs one (the other terms are not read).
+    const bool native_law = (flags & kNativeContactLaw) != 0u;
     auto profile_of = [&](const Geom& g) -> uint32_t {
-        if (!g.friction_authored) return 0xFFFFFFFFu;
-        for (size_t i = 0u; i < s.profile_mu.size() / 2u; ++i) if (s.profile_mu[2u * i] == g.friction) return uint32_t(i);
+        if (native_law && !g.friction_authored) return 0xFFFFFFFFu;
+        const uint32_t law = native_law ? 0u : 1u;
+        for (size_t i = 0u; i < s.profile_law.size(); ++i) {
+            bool same = s.profile_mu[2u * i] == g.friction && s.profile_law[i] == law && s.profile_solref[2u * i] == g.solref[0] &&
+                        s.profile_solref[2u * i + 1u] == g.solref[1] && s.profile_margin[2u * i] == g.margin && s.profile_margin[2u * i + 1u] == g.gap;
+            for (size_t k = 0u; k < 5u; ++k) same = same && s.profile_solimp[5u * i + k] == g.solimp[k];
+            if (same) return uint32_t(i);
+        }
         s.profile_mu.push_back(g.friction); s.profile_mu.push_back(g.friction);
+        s.profile_law.push_back(law);
+        s.profile_solref.push_back(g.solref[0]); s.profile_solref.push_back(g.solref[1]);
+        for (float v : g.solimp) s.profile_solimp.push_back(v);
+        s.profile_margin.push_back(g.margin); s.profile_margin.push_back(g.gap);
         any_friction_profile = true;
-        return uint32_t(s.profile_mu.size() / 2u - 1u);
+        return uint32_t(s.profile_law.size() - 1u);
     };
     auto add_row = [&](uint32_t role, uint32_t link, const Geom* g, int32_t group_override) {
         s.body_role.push_back(role); s.body_link.push_back(link);
@@ -698,6 +733,12 @@ void Scene::Bind() {
     desc.drive_rows = 1u;   // the reference always cooks one drive row per link (src/nk/pipeline/world.cpp:61)
     desc.excluded_pairs = excluded_pairs.data();
     desc.excluded_pair_count = uint32_t(excluded_pairs.size() / 2u);
+    if (!profile_law.empty()) {   // a loader that authors no law leaves every profile native
+        desc.profile_law = profile_law.data(); desc.profile_solref = profile_solref.data();
+        desc.profile_solimp = profile_solimp.data(); desc.profile_margin = profile_margin.data();
+    }
+    desc.contact_cone = contact_cone;
+    desc.contact_impratio = contact_impratio;
 }
 
 }  // namespace scene_file

@@ -50,7 +50,8 @@ enum : uint32_t { kSideRigid = 0, kSideArtic = 1, kSideStatic = 3 };
 enum : uint32_t {
     kRowActive = 1u << 0, kRowFriction = 1u << 1, kRowBlockNormal = 1u << 2, kRowBlockTangent = 1u << 3,
     kRowJointLimitLower = 1u << 4, kRowJointLimitUpper = 1u << 5,
-    kRowContactNormal = 1u << 6, kRowVelocityOnly = 1u << 7, kRowSpeculative = 1u << 8, kRowMuJoCo = 1u << 11
+    kRowContactNormal = 1u << 6, kRowVelocityOnly = 1u << 7, kRowSpeculative = 1u << 8, kRowMuJoCo = 1u << 11,
+    kRowPyramidal = 1u << 12
 };
 // src/phi/op_schema.hpp:36-52
 enum : uint32_t {
@@ -59,7 +60,7 @@ enum : uint32_t {
 };
 // src/phi/articulation_contract.hpp:16-23
 enum : uint32_t { kDrivePdPosition = 0, kDriveTorque = 1, kDriveVelocity = 2, kDriveComputedTorque = 3, kDriveOsc = 4, kDriveActuator = 5 };
-constexpr uint32_t kContactLawSpeculative = 2u;   // src/nk/solve/nk_row.hpp:37
+constexpr uint32_t kContactLawCompliant = 0u, kContactLawVelocity = 1u, kContactLawSpeculative = 2u;   // src/nk/solve/nk_row.hpp:35-37
 
 // Template tables, stored once and shared by every environment (the reference replicates them per env,
 // src/nk/model/model.hpp:154-157).  Counts are per environment.
@@ -70,6 +71,9 @@ struct ModelView {
     uint32_t excluded_pair_count;
     // joint row slots after the contact rows: 2 per link, 1 per link, 1 per link, or 0 (scene/cook/cook_to_model.cpp:706-719)
     uint32_t joint_limit_rows, joint_friction_rows, joint_drive_rows, drive_mode;
+    // the MuJoCo contact law: some profile is MuJoCo-sourced; the cone of its contacts (0 pyramidal, 1 elliptic) and impratio
+    uint32_t any_mujoco, contact_cone;
+    float contact_impratio;
     const uint8_t* joint_type;
     const uint32_t* parent_link;
     const float* joint_axis;
@@ -102,6 +106,10 @@ struct ModelView {
     const uint32_t* body_collidable_body;
     const float* body_collidable_local;
     const float* profile_mu;
+    const uint32_t* profile_law;      // [profile] 1: MuJoCo-sourced (constraint/law_source.hpp)
+    const float* profile_solref;      // [profile][2]
+    const float* profile_solimp;      // [profile][5]
+    const float* profile_margin;      // [profile][2] margin, gap
     const uint64_t* excluded_pairs;   // sorted (a << 32 | b) keys of collidable rows that never pair, a < b
 };
 
@@ -120,6 +128,9 @@ struct DataView {
     uint32_t *env_status, *vbd_velocity_sweep_count;
     float *solver_residual, *solver_penalty;
     float *solver_velocity, *solver_free;   // block velocities kept between solves (carried constraint velocity)
+    // the MuJoCo contact law (fields.yaml body_invweight0, dof_invweight0, row_invweight, row_reference_velocity_gain,
+    // step_qdot_flat): reference weights at the creation pose, per row the weight and the gain on the start velocity
+    float *body_invweight0, *dof_invweight0, *row_invweight, *row_reference_velocity_gain, *step_qdot_flat;
     // contact cache carried between steps (fields.yaml:524-539, 155, 791, 844)
     uint64_t *contact_material, *contact_cache_pair, *contact_cache_feature, *contact_cache_material;
     float *contact_cache_lambda, *contact_cache_normal;
@@ -179,6 +190,14 @@ struct ArticulationDynamicsParams {   // op_schema.hpp:108-121
     uint32_t max_links = 0u;
     uint32_t links_per_env = 0u;
     uint32_t bodies_per_env = 0u;
+};
+struct ReferenceWeightsParams {   // op_schema.hpp:123-130
+    uint32_t max_dof;
+    uint32_t articulation_count;
+    uint32_t total_link_count;
+    uint32_t articulations_per_env;
+    uint32_t bodies_per_env;
+    uint32_t total_body_count;
 };
 struct IntegrateVelocityParams {   // op_schema.hpp:143-150
     float dt;

@@ -582,6 +582,111 @@ Status OpArticulationDynamics(const ModelView& m, const DataView& d, const void*
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 
+namespace {
+// SolveMassBlock (articulation_mass.cuh:357-396) by one thread: forward by columns, divide, backward
+__device__ void solve_mass_serial(const float* factor, float* value, uint32_t n, uint32_t stride) {
+    for (uint32_t j = 0u; j < n; ++j) {
+        const float solved = value[j];
+        for (uint32_t i = j + 1u; i < n; ++i) value[i] -= factor[size_t{i} * stride + j] * solved;
+    }
+    for (uint32_t i = 0u; i < n; ++i) value[i] = value[i] / factor[size_t{i} * stride + i];
+    for (uint32_t end = n; end > 0u; --end) {
+        const uint32_t i = end - 1u;
+        float sum = value[i];
+        for (uint32_t j = i + 1u; j < n; ++j) sum -= factor[size_t{j} * stride + i] * value[j];
+        value[i] = sum;
+    }
+}
+
+// AccumulateChainJointForce (articulation_types.cuh:193-238): what a force f and a moment at `point` add to the
+// generalized force of the joint of `link`
+__device__ void accumulate_chain(const ModelView& m, const DataView& d, uint32_t env, uint32_t link, V3 point, V3 f, V3 moment, float* out) {
+    const uint32_t dof_index = m.link_dof[link], stride = m.max_dof;
+    const uint8_t type = m.joint_type[link];
+    if (type == kFloatingBase) {
+        const Xf base = load_xf(d.base_pose + size_t{env} * 7u);
+        const V3 lever = sub3(point, base.p);
+        const V3 e[3] = {rotate_normalized(base.r, V3{1, 0, 0}), rotate_normalized(base.r, V3{0, 1, 0}), rotate_normalized(base.r, V3{0, 0, 1})};
+        for (uint32_t b = 0u; b < 3u; ++b) {
+            const float angular = dot3(cross3(e[b], lever), f) + dot3(e[b], moment), linear = dot3(e[b], f);
+            if (dof_index + b < stride) out[dof_index + b] += angular;
+            if (dof_index + 3u + b < stride) out[dof_index + 3u + b] += linear;
+        }
+        return;
+    }
+    const Xf pose = load_xf(d.link_pose + (size_t{env} * m.links_per_env + link) * 7u);
+    const V3 axis_world = rotate_normalized(pose.r, load3(m.joint_axis + 3u * link));
+    float entry;
+    if (type == kPrismatic) entry = dot3(axis_world, f);
+    else entry = dot3(cross3(axis_world, sub3(point, pose.p)), f) + dot3(axis_world, moment);
+    if (dof_index < stride) out[dof_index] += entry;
+}
+
+// ArticulationReferenceWeightsKernel (articulation.cu:434-501), one thread an environment as in the reference: the
+// diagonal of M^-1 (a floating base's six entries averaged over its rotations and its translations), and for every
+// link the mean response of its centre of mass to a unit force and to a unit moment along the three world axes.
+// `m_factor` holds the factor of the mass matrix at the current pose (no drive damping folded in).
+__global__ void __launch_bounds__(kWave) ReferenceWeightsKernel(ModelView m, DataView d, uint32_t env_count) {
+    const uint32_t env = blockIdx.x * kWave + threadIdx.x;
+    if (env >= env_count) return;
+    const uint32_t nl = m.links_per_env, nb = m.bodies_per_env, md = m.max_dof, dof = m.dof;
+    float* weights = d.body_invweight0 + size_t{env} * nb * 2u;
+    for (uint32_t b = 0u; b < nb; ++b) weights[2u * b] = weights[2u * b + 1u] = 0.0f;   // static rows move under nothing
+    const float* factor = d.m_factor + size_t{env} * md * md;
+    float* diagonal = d.dof_invweight0 + size_t{env} * md;
+    float row[kMaxDof], solution[kMaxDof];
+    for (uint32_t k = 0u; k < dof; ++k) {
+        for (uint32_t i = 0u; i < dof; ++i) solution[i] = i == k ? 1.0f : 0.0f;
+        solve_mass_serial(factor, solution, dof, md);
+        diagonal[k] = solution[k];
+    }
+    if (m.joint_type[0] == kFloatingBase) {
+        const float rotation = (diagonal[0] + diagonal[1] + diagonal[2]) / 3.0f;
+        const float translation = (diagonal[3] + diagonal[4] + diagonal[5]) / 3.0f;
+        for (uint32_t i = 0u; i < 3u; ++i) { diagonal[i] = rotation; diagonal[i + 3u] = translation; }
+    }
+    for (uint32_t link = 0u; link < nl; ++link) {
+        const Xf pose = load_xf(d.link_pose + (size_t{env} * nl + link) * 7u);
+        const V3 point = add3(pose.p, rotate_normalized(pose.r, load3(m.link_inertial_frame + 7u * link)));
+        float weight[2] = {0.0f, 0.0f};
+        for (uint32_t axis = 0u; axis < 6u; ++axis) {
+            for (uint32_t k = 0u; k < dof; ++k) row[k] = 0.0f;
+            const V3 unit{axis % 3u == 0u ? 1.0f : 0.0f, axis % 3u == 1u ? 1.0f : 0.0f, axis % 3u == 2u ? 1.0f : 0.0f};
+            const V3 none{0.0f, 0.0f, 0.0f};
+            for (uint32_t walk = link; walk != kInvalid; walk = m.parent_link[walk])
+                if (joint_dof(m.joint_type[walk]) != 0u) accumulate_chain(m, d, env, walk, point, axis < 3u ? unit : none, axis < 3u ? none : unit, row);
+            for (uint32_t k = 0u; k < dof; ++k) solution[k] = row[k];
+            solve_mass_serial(factor, solution, dof, md);
+            for (uint32_t k = 0u; k < dof; ++k) weight[axis / 3u] += row[k] * solution[k];
+        }
+        const uint32_t body = m.link_body[link];
+        if (body < nb) { weights[2u * body] = weight[0] / 3.0f; weights[2u * body + 1u] = weight[1] / 3.0f; }
+    }
+}
+}  // namespace
+
+// ReferenceWeights (op_schema.hpp:123-130; articulation.cu:425-500): the mass matrix at the current poses without
+// drive damping, its factor, and the reference weights from it.  World creation and reset dispatch it after the poses
+// are refreshed (nk/pipeline/world.cpp:553-561).
+Status OpReferenceWeights(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const ReferenceWeightsParams*>(params);
+    if (p == nullptr) return Status::Failed;
+    if (p->articulation_count == 0u || p->total_link_count == 0u) return Status::Ok;
+    if (p->articulations_per_env != 1u || p->max_dof != m.max_dof || p->bodies_per_env != m.bodies_per_env ||
+        p->total_link_count != p->articulation_count * m.links_per_env) return Status::InvalidArgument;
+    ArticulationDynamicsParams mass{};   // no velocity update, no wrench, nothing folded into the diagonal
+    mass.max_dof = p->max_dof; mass.integrate_velocity = 0u; mass.articulation_count = p->articulation_count;
+    mass.total_link_count = p->total_link_count; mass.max_links = m.links_per_env; mass.links_per_env = m.links_per_env;
+    mass.bodies_per_env = m.bodies_per_env;
+    if (m.dof != 0u) {
+        const Status status = OpArticulationDynamics(m, d, &mass, stream);
+        if (status != Status::Ok) return status;
+    }
+    hipLaunchKernelGGL(ReferenceWeightsKernel, dim3((p->articulation_count + kWave - 1u) / kWave), dim3(kWave), 0, stream, m, d,
+                       p->articulation_count);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
 Status OpIntegratePosition(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
     const auto* p = static_cast<const IntegratePositionParams*>(params);
     if (p == nullptr) return Status::Failed;

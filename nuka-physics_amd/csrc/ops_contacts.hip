@@ -625,19 +625,29 @@ __device__ uint32_t NarrowphaseSlot(const ModelView& m, const DataView& d, const
     const float separation = fmaxf(p.contact_margin, 0.0005f);
     const uint32_t live = d.pair_count[env];
     Manifold mf; mf.count = 0u; mf.normal = V3{0, 0, 1};
-    uint32_t a = 0u, b = 0u;
+    uint32_t a = 0u, b = 0u, law = kContactLawSpeculative;
     Xf xa{}, xb{};
     if (slot < live) {
         a = d.candidate_pairs[gid * 2u]; b = d.candidate_pairs[gid * 2u + 1u];
         const ShapeRow sa = load_shape(m.shape_table, a), sb = load_shape(m.shape_table, b);
         xa = load_xf(d.body_pose + (bbase + a) * 7u); xb = load_xf(d.body_pose + (bbase + b) * 7u);
         const Prim pa = make_prim(sa, xa), pb = make_prim(sb, xb);
-        const float query = fmaxf(separation, fminf(motion_radius(2.0f * separation, p.dt, 0.0f, 0.0f, 0.9f), p.query_reach));
+        // a MuJoCo-sourced profile on either side makes the contact compliant; its query band is the profiles' margin
+        // and gap, and its depth stays the geometric one (narrowphase_prims.cu:232, 268-281, 295-296)
+        const bool has_a = sa.profile < m.profile_count, has_b = sb.profile < m.profile_count;
+        float query_margin = separation;
+        if ((has_a && m.profile_law[sa.profile] == 1u) || (has_b && m.profile_law[sb.profile] == 1u)) {
+            law = kContactLawCompliant;
+            const float margin_a = has_a ? m.profile_margin[2u * sa.profile] + m.profile_margin[2u * sa.profile + 1u] : 0.0f;
+            const float margin_b = has_b ? m.profile_margin[2u * sb.profile] + m.profile_margin[2u * sb.profile + 1u] : 0.0f;
+            query_margin = margin_a + margin_b;
+        }
+        const float query = fmaxf(query_margin, fminf(motion_radius(2.0f * separation, p.dt, 0.0f, 0.0f, 0.9f), p.query_reach));
         primitive_pair(sa.kind, pa, sb.kind, pb, query, &mf);
-        for (uint32_t i = 0u; i < mf.count; ++i) mf.penetration[i] += separation;
+        if (law != kContactLawCompliant) for (uint32_t i = 0u; i < mf.count; ++i) mf.penetration[i] += separation;
     }
     d.ucontact_count[gid] = mf.count;
-    d.ucontact_law[gid] = kContactLawSpeculative;
+    d.ucontact_law[gid] = law;
     for (uint32_t i = 0u; i < mf.count; ++i) {
         const size_t at = gid * 4u + i;
         d.ucontact_point[3u * at] = mf.position[i].x; d.ucontact_point[3u * at + 1u] = mf.position[i].y; d.ucontact_point[3u * at + 2u] = mf.position[i].z;
@@ -734,6 +744,95 @@ __device__ uint64_t contact_material_key(float mu1, float mu2, uint32_t law) {
     return h;
 }
 
+// The same hash of any merged profile (mu1, mu2, solref[2], solimp[5], margin, gap; condim 3, no friction slope),
+// then the law word for the velocity-only laws and the cone for the compliant law (:620-623).
+__device__ uint64_t merged_material_key(const float (&merged)[11], uint32_t law, uint32_t cone) {
+    uint64_t h = 0x4e554b4150524f46ull;
+    h = profile_word(h, 2u);
+    h = profile_word(h, 1u);
+    h = profile_word(h, __float_as_uint(merged[0])); h = profile_word(h, __float_as_uint(merged[1]));
+    h = profile_word(h, __float_as_uint(0.005f)); h = profile_word(h, __float_as_uint(0.0001f));
+    for (int i = 2; i < 11; ++i) h = profile_word(h, __float_as_uint(merged[i]));
+    h = profile_word(h, 3u);
+    if (h == 0ull) h = 0x9e3779b97f4a7c15ull;
+    if (law == kContactLawVelocity || law == kContactLawSpeculative) { h ^= uint64_t{law}; h *= 1099511628211ull; }
+    if (law == kContactLawCompliant) { h ^= uint64_t{cone}; h *= 1099511628211ull; }
+    return h;
+}
+// One shape's contact parameters as the merge takes them: mu1, mu2, solref[2], solimp[5], margin, gap; a shape without
+// a profile has the defaults of scene/contact_filter.hpp:20-37.
+__device__ void profile_terms(const ModelView& m, uint32_t profile, float (&out)[11]) {
+    out[0] = 1.0f; out[1] = 1.0f; out[2] = 0.02f; out[3] = 1.0f; out[4] = 0.9f; out[5] = 0.95f; out[6] = 0.001f; out[7] = 0.5f; out[8] = 2.0f;
+    out[9] = 0.0f; out[10] = 0.0f;
+    if (profile >= m.profile_count) return;
+    out[0] = m.profile_mu[2u * profile]; out[1] = m.profile_mu[2u * profile + 1u];
+    out[2] = m.profile_solref[2u * profile]; out[3] = m.profile_solref[2u * profile + 1u];
+    for (uint32_t k = 0u; k < 5u; ++k) out[4u + k] = m.profile_solimp[5u * profile + k];
+    out[9] = m.profile_margin[2u * profile]; out[10] = m.profile_margin[2u * profile + 1u];
+}
+// MergeContactParams (scene/contact_filter.hpp:100-137) at equal priority and mixing weight: friction by max, solref
+// mixed half and half (or the minimum when either is in direct form), solimp mixed, margins and gaps added.
+__device__ void merge_contact_params(const float (&a)[11], const float (&b)[11], float (&out)[11]) {
+    const float mix = 1.0f / (1.0f + 1.0f), imix = 1.0f - mix;
+    out[0] = a[0] > b[0] ? a[0] : b[0];
+    out[1] = a[1] > b[1] ? a[1] : b[1];
+    if (a[2] > 0.0f && b[2] > 0.0f) { out[2] = mix * a[2] + imix * b[2]; out[3] = mix * a[3] + imix * b[3]; }
+    else { out[2] = a[2] < b[2] ? a[2] : b[2]; out[3] = a[3] < b[3] ? a[3] : b[3]; }
+    for (int i = 0; i < 5; ++i) out[4 + i] = mix * a[4 + i] + imix * b[4 + i];
+    out[9] = a[9] + b[9];
+    out[10] = a[10] + b[10];
+}
+// ComputeCompliantRow (constraint/solref_solimp.hpp:55-86) followed by DiscretizeCompliantRow (:40-44): the row's
+// regularisation R, its reference acceleration and the gain on the start velocity, for the step dt with the
+// damping taken at the midpoint.
+struct CompliantRow { float R, bias, gain; };
+__device__ __forceinline__ float clampf(float v, float lo, float hi) { return fminf(fmaxf(v, lo), hi); }
+__device__ CompliantRow compliant_row(const float* solref, const float* solimp, float pos_imp, float pos_aref, float vel, float invweight,
+                                      float dt, bool refsafe) {
+    float timeconst = solref[0];
+    const float dampratio = solref[1];
+    if (refsafe) timeconst = fmaxf(timeconst, 2.0f * dt);
+    const float dmin = clampf(solimp[0], 1.0e-4f, 0.9999f), dmax = clampf(solimp[1], 1.0e-4f, 0.9999f);
+    const float width = fmaxf(1.0e-15f, solimp[2]);
+    const float mid = clampf(solimp[3], 1.0e-4f, 0.9999f);
+    const float power = fmaxf(1.0f, solimp[4]);
+    const float dmax_sq = dmax * dmax;
+    float k = 1.0f / (dmax_sq * timeconst * timeconst * dampratio * dampratio);
+    float b = 2.0f / (dmax * timeconst);
+    if (solref[0] <= 0.0f) k = -solref[0] / dmax_sq;
+    if (solref[1] <= 0.0f) b = -solref[1] / dmax;
+    const float x = fabsf(pos_imp) / width;
+    const float rising = (1.0f / powf(mid, power - 1.0f)) * powf(x, power);
+    const float falling = 1.0f - (1.0f / powf(1.0f - mid, power - 1.0f)) * powf(1.0f - x, power);
+    const float y = x < mid ? rising : falling;
+    float imp = clampf(dmin + y * (dmax - dmin), dmin, dmax);
+    if (x > 1.0f) imp = dmax;
+    const float D = 1.0f / fmaxf(invweight * (1.0f - imp) / imp, 1.0e-15f);
+    const float R = 1.0f / D, aref = -k * imp * pos_aref - b * vel;
+    const double scale = 1.0 + 0.5 * double(dt) * b;
+    return CompliantRow{float(R / scale), float(aref / scale), float((1.0 / double(dt) - 0.5 * b) / scale)};
+}
+// math/cuda_vec_ops.cuh:187-196 MuJoCoContactFrame: the first tangent along `axis` where that is far enough from the
+// normal, else along a world axis
+__device__ void mujoco_contact_frame(V3 normal, V3 axis, V3* t1, V3* t2) {
+    V3 n = normal;
+    const float l = dot3(n, n);
+    if (l > 1.0e-10f) { const float inv = rsqrt_exact(l); n = V3{n.x * inv, n.y * inv, n.z * inv}; }
+    else n = V3{0.0f, 0.0f, 1.0f};
+    V3 tangent = sub3(axis, scale3(n, dot3(n, axis)));
+    if (dot3(tangent, tangent) < 0.25f) {
+        const V3 reference = n.y > -0.5f && n.y < 0.5f ? V3{0.0f, 1.0f, 0.0f} : V3{0.0f, 0.0f, 1.0f};
+        tangent = sub3(reference, scale3(n, dot3(n, reference)));
+    }
+    const V3 a = scale3(tangent, rsqrt_exact(dot3(tangent, tangent)));
+    *t1 = a;
+    *t2 = cross3(n, a);
+}
+
+__device__ __forceinline__ float uniform_value(float v, uint32_t lane) {   // `lane` is the same in every lane
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), int(lane)));
+}
+
 // ---- AssembleRows: one wavefront per environment (assemble_rows.cu:325-394, 200-214, 406-801, 122-186) ----
 __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataView d, AssembleRowsParams p) {
     extern __shared__ uint32_t lds_u[];
@@ -747,6 +846,7 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
     uint32_t* row_merge = row_link_b + CR;              // CR: both sides articulated with the same owner
     float* row_point = reinterpret_cast<float*>(row_merge + CR);   // 3 CR
     float* row_dir = row_point + 3u * CR;                // 3 CR, side A's direction (side B's is its negative)
+    float* row_gain = row_dir + 3u * CR;                 // CR: a compliant row's gain on the start velocity along it, else 0
     Row* rows = reinterpret_cast<Row*>(d.urows) + size_t{env} * R;
     float* lambda = d.lambda + size_t{env} * R;
     float* pen = d.row_penetration + size_t{env} * R;
@@ -781,7 +881,7 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
         lambda[local] = 0.0f; pen[local] = 0.0f; cj_link[local] = kInvalid; cj_link_b[local] = kInvalid;
         rows[local].flags = 0u;
     }
-    for (uint32_t local = lane; local < CR; local += kWave) { row_link_a[local] = kInvalid; row_link_b[local] = kInvalid; row_merge[local] = 0u; }
+    for (uint32_t local = lane; local < CR; local += kWave) { row_link_a[local] = kInvalid; row_link_b[local] = kInvalid; row_merge[local] = 0u; row_gain[local] = 0.0f; }
     if (lane == 0u) {
         d.contact_row_extent[2u * env] = previous_extent;
         d.contact_row_extent[2u * env + 1u] = extent;
@@ -818,40 +918,83 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
         }
         if (kind_a == kSideStatic) idx_a = kInvalid;
         if (kind_b == kSideStatic) idx_b = kInvalid;
-        // per-shape friction profile or the default 1.0, mixed by max at equal priority (scene/contact_filter.hpp:58-62, 108-111)
-        const float mu_a1 = sa.profile < m.profile_count ? m.profile_mu[2u * sa.profile] : 1.0f;
-        const float mu_a2 = sa.profile < m.profile_count ? m.profile_mu[2u * sa.profile + 1u] : 1.0f;
-        const float mu_b1 = sb.profile < m.profile_count ? m.profile_mu[2u * sb.profile] : 1.0f;
-        const float mu_b2 = sb.profile < m.profile_count ? m.profile_mu[2u * sb.profile + 1u] : 1.0f;
-        const float mu1 = fmaxf(mu_a1, mu_b1), mu2 = fmaxf(mu_a2, mu_b2);
-        d.contact_material[gid] = n_active > 0u ? contact_material_key(mu1, mu2, d.ucontact_law[gid]) : 0ull;   // :620-622
+        // the two sides' profiles merged (:540-594; scene/contact_filter.hpp:100-137); a side without one has the defaults
+        const uint32_t law = d.ucontact_law[gid];
+        const bool mujoco = law == kContactLawCompliant;   // :480
+        float side_a[11], side_b[11], merged[11];
+        profile_terms(m, sa.profile, side_a); profile_terms(m, sb.profile, side_b);
+        merge_contact_params(side_a, side_b, merged);
+        if (mujoco) { merged[0] = fmaxf(1.0e-5f, merged[0]); merged[1] = fmaxf(1.0e-5f, merged[1]); }   // :573-576
+        const float mu1 = merged[0], mu2 = merged[1];
+        const float* solref = merged + 2, *solimp = merged + 4;
+        const float margin = merged[9];
+        d.contact_material[gid] = n_active > 0u ? merged_material_key(merged, law, m.contact_cone) : 0ull;   // :620-623
+        // a compliant row's weight is the sum of its two bodies' reference weights, a link's through its own collidable row (:595-597)
+        float invweight = 0.0f;
+        if (mujoco) {
+            const float* weights = d.body_invweight0 + size_t{env} * m.bodies_per_env * 2u;
+            const uint32_t weight_a = kind_a == kSideArtic ? m.link_body[link_a - env * nl] : local_a;
+            const uint32_t weight_b = kind_b == kSideArtic ? m.link_body[link_b - env * nl] : local_b;
+            invweight = (weight_a < m.bodies_per_env ? weights[2u * weight_a] : 0.0f) + (weight_b < m.bodies_per_env ? weights[2u * weight_b] : 0.0f);
+        }
+        const bool pyramidal = mujoco && m.contact_cone == 0u;   // condim 3 (:598)
+        const float impratio = m.contact_impratio;
+        V3 frame_axis{0, 0, 0};   // :601-605: a capsule on a plane aligns the pyramid with the capsule's axis
+        if (pyramidal && sa.kind == 1u && sb.kind == 3u) frame_axis = make_prim(sa, load_xf(d.body_pose + (size_t{env} * m.bodies_per_env + local_a) * 7u)).cz;
+        if (pyramidal && sb.kind == 1u && sa.kind == 3u) frame_axis = make_prim(sb, load_xf(d.body_pose + (size_t{env} * m.bodies_per_env + local_b) * 7u)).cz;
         for (uint32_t pt = 0u; pt < P; ++pt) {
-            const bool live = pt < n_active && pt < 4u;
             const size_t mp = gid * 4u + pt;
-            const uint32_t row_of[3] = {base + pt, base + P + pt, base + 2u * P + pt};
-            V3 n{0, 0, 1}, point{0, 0, 0}, dirs[3];
-            dirs[1] = V3{1, 0, 0}; dirs[2] = V3{0, 1, 0};
+            // the velocity laws keep every point; a compliant point lives inside its margin (:625-626)
+            const bool live = pt < n_active && pt < 4u && (!mujoco || d.ucontact_depth[mp] + margin > 0.0f);
+            const uint32_t row_of[4] = {base + pt, base + P + pt, base + 2u * P + pt, base + 3u * P + pt};
+            V3 n{0, 0, 1}, point{0, 0, 0}, dirs[4];
+            V3 t0{1, 0, 0}, t1{0, 1, 0};
             float d0 = 0.0f;
             if (live) {
                 const V3 raw{d.ucontact_normal[3u * mp], d.ucontact_normal[3u * mp + 1u], d.ucontact_normal[3u * mp + 2u]};
                 const float len = sqrtf(raw.x * raw.x + raw.y * raw.y + raw.z * raw.z);
                 n = len < 1e-12f ? V3{0, 0, 0} : V3{raw.x / len, raw.y / len, raw.z / len};
                 point = V3{d.ucontact_point[3u * mp], d.ucontact_point[3u * mp + 1u], d.ucontact_point[3u * mp + 2u]};
-                contact_tangent_basis(raw, &dirs[1], &dirs[2]);
+                if (pyramidal) mujoco_contact_frame(raw, frame_axis, &t0, &t1);
+                else contact_tangent_basis(raw, &t0, &t1);
                 d0 = d.ucontact_depth[mp];
             }
-            dirs[0] = n;
-            for (uint32_t axis = 0u; axis < 3u; ++axis) {
+            // a pyramid has four scalar rows a point along n +- mu t (:651-690); the other cones a normal and two tangents
+            const uint32_t row_count = pyramidal ? 4u : 3u;
+            CompliantRow edge{};
+            float edge_invweight = 0.0f;
+            if (pyramidal) {
+                edge_invweight = (invweight + mu1 * mu1 * invweight) * 2.0f * mu1 * mu1 / impratio;
+                const float pos = -d0 - margin;
+                edge = compliant_row(solref, solimp, pos, pos, 0.0f, edge_invweight, p.dt, p.refsafe);
+                for (uint32_t k = 0u; k < 4u; ++k) {
+                    const float mu = k < 2u ? mu1 : mu2;
+                    const V3 tangent = k < 2u ? t0 : t1;
+                    dirs[k] = add3(n, scale3(tangent, (k & 1u) != 0u ? -mu : mu));
+                }
+            } else { dirs[0] = n; dirs[1] = t0; dirs[2] = t1; dirs[3] = V3{0, 0, 0}; }
+            for (uint32_t axis = 0u; axis < row_count; ++axis) {
                 const uint32_t rs = row_of[axis];
                 lambda[rs] = 0.0f; pen[rs] = 0.0f; cj_link[rs] = kInvalid; cj_link_b[rs] = kInvalid;
-                if (!live) { rows[rs].flags = 0u; continue; }
+                row_gain[rs] = 0.0f;
+                if (!live) {
+                    if (pyramidal) rows[rs] = Row{}; else rows[rs].flags = 0u;
+                    continue;
+                }
                 Row row{};
                 const V3 dir = dirs[axis];
                 row.group_first = env * R + base; row.group_normal_count = P; row.env = env;
                 row.mu = mu1; row.friction_secondary = mu2;
                 row.a.kind = kind_a; row.a.index = idx_a; row.a.jlin = dir; row.a.jang = V3{0, 0, 0};
                 row.b.kind = kind_b; row.b.index = idx_b; row.b.jlin = V3{-dir.x, -dir.y, -dir.z}; row.b.jang = V3{0, 0, 0};
-                if (axis == 0u) {
+                float gain = 0.0f, weight = 0.0f;
+                if (pyramidal) {
+                    row.flags = kRowActive | kRowMuJoCo | kRowPyramidal | (axis == 0u ? uint32_t(kRowContactNormal) : 0u);
+                    row.group_first = env * R + rs; row.group_normal_count = 1u;
+                    row.rhs = edge.bias; row.compliance_alpha = edge.R;
+                    row.lower = 0.0f; row.upper = FLT_MAX;
+                    gain = edge.gain; weight = edge_invweight;
+                } else if (axis == 0u) {
                     // speculative rows reserve the rounding of their projected endpoint positions (:703-713)
                     const V3 ext{fabsf(point.x) + fabsf(n.x * d0), fabsf(point.y) + fabsf(n.y * d0), fabsf(point.z) + fabsf(n.z * d0)};
                     const double gamma = 3.0 * double(FLT_EPSILON) / (1.0 - 3.0 * double(FLT_EPSILON));
@@ -860,14 +1003,33 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
                                                      fabs(double(n.z)) * (fabs(double(ext.z)) + fabs(double(ext.z))));
                     const float clearance = roundoff > 0.0 ? nextafterf(float(roundoff), FLT_MAX) : 0.0f;
                     const float depth = d0 + clearance;
-                    pen[rs] = depth;
-                    row.flags = kRowActive | kRowContactNormal | kRowBlockNormal | kRowSpeculative;
+                    pen[rs] = mujoco ? fmaxf(d0, 0.0f) : depth;
+                    row.flags = kRowActive | kRowContactNormal | kRowBlockNormal | (mujoco ? uint32_t(kRowMuJoCo) : uint32_t(kRowSpeculative));
                     row.rhs = (fminf(depth, 0.0f) + (p.position_pass != 0u ? 0.0f
                                : fminf(fmaxf(d0, 0.0f), p.overlap_recovery_velocity * p.dt))) / (p.dt * p.dt);
+                    if (mujoco) {   // :714-731: the spring-damper reference of the merged solref / solimp at this depth
+                        const float pos = -d0 - margin;
+                        const CompliantRow c = compliant_row(solref, solimp, pos, pos, 0.0f, invweight, p.dt, p.refsafe);
+                        row.rhs = c.bias; row.compliance_alpha = c.R;
+                        gain = c.gain; weight = invweight;
+                    }
                     row.lower = 0.0f; row.upper = FLT_MAX;
                 } else {
                     row.flags = kRowActive | kRowBlockTangent;
+                    if (mujoco) {   // :771-782: the tangent rows' compliance, which shapes the elliptic cone's metric
+                        const float mu = axis == 1u ? mu1 : mu2;
+                        weight = invweight / impratio * (mu1 * mu1) / (mu * mu);
+                        const CompliantRow c = compliant_row(solref, solimp, -d0 - margin, 0.0f, 0.0f, weight, p.dt, p.refsafe);
+                        row.flags |= kRowMuJoCo;
+                        row.compliance_alpha = c.R;
+                        gain = c.gain;
+                    }
                     row.lower = -FLT_MAX; row.upper = FLT_MAX;
+                }
+                if (mujoco) {
+                    d.row_reference_velocity_gain[size_t{env} * R + rs] = gain;
+                    d.row_invweight[size_t{env} * R + rs] = weight;
+                    row_gain[rs] = gain;
                 }
                 row_point[3u * rs] = point.x; row_point[3u * rs + 1u] = point.y; row_point[3u * rs + 2u] = point.z;
                 row_dir[3u * rs] = dir.x; row_dir[3u * rs + 1u] = dir.y; row_dir[3u * rs + 2u] = dir.z;
@@ -970,6 +1132,7 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
         }
     }
     const uint32_t bound = min(contact_row_bound(previous_extent, extent, CR), CR);
+    const float start_velocity = m.any_mujoco != 0u && lane < md ? d.step_qdot_flat[size_t{env} * md + lane] : 0.0f;
     for (uint32_t r = 0u; r < bound; ++r) {
         const uint32_t links[2] = {row_link_a[r], row_link_b[r]};
         if (links[0] == kInvalid && links[1] == kInvalid) continue;
@@ -993,6 +1156,19 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
         if (lane < md) {
             if (links[0] != kInvalid) d.chain_jacobian[(size_t{env} * R + r) * md + lane] = entries[0];
             if (links[1] != kInvalid) d.chain_jacobian_b[(size_t{env} * R + r) * md + lane] = entries[1];
+        }
+        // PrepareContactRowsKernel (:1134-1140): a compliant row's reference acceleration includes the damping of the
+        // velocity the step started from along the row, ContactReferenceVelocity (:1072-1100): side A's coordinates in
+        // order, then side B's
+        const float gain = row_gain[r];
+        if (gain != 0.0f) {
+            float velocity = 0.0f;
+            for (uint32_t side = 0u; side < 2u; ++side) {
+                if (links[side] == kInvalid) continue;
+                const float term = entries[side] * start_velocity;
+                for (uint32_t k = 0u; k < md; ++k) velocity += uniform_value(term, k);
+            }
+            if (lane == 0u) rows[r].rhs += gain * velocity;
         }
     }
 }
@@ -1051,7 +1227,7 @@ Status OpAssembleRows(const ModelView& m, const DataView& d, const void* params,
     if (p == nullptr) return Status::Failed;
     if (p->env_count == 0u || p->rows_per_env == 0u) return Status::Ok;
     if (p->max_dof > kMaxDof) return Status::InvalidArgument;
-    const size_t lds = (size_t{p->union_slot_count} * 2u + size_t{p->contact_rows_per_env} * 9u) * sizeof(uint32_t);
+    const size_t lds = (size_t{p->union_slot_count} * 2u + size_t{p->contact_rows_per_env} * 10u) * sizeof(uint32_t);
     if (lds > 150u * 1024u) return Status::InvalidArgument;
     hipLaunchKernelGGL(AssembleRowsKernel, dim3(p->env_count), dim3(kWave), lds, stream, m, d, *p);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
@@ -1400,7 +1576,34 @@ Status OpAccumulateStep(const ModelView&, const DataView& d, const void* params,
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 
-Status OpSnapshotStepVelocity(const ModelView&, const DataView&, const void*, hipStream_t) { return Status::Ok; }
+namespace {
+// PackQdotFlatMultiKernel (assemble_rows.cu:200-214) into step_qdot_flat
+__global__ void __launch_bounds__(256) SnapshotStepVelocityKernel(ModelView m, DataView d, uint32_t env_count) {
+    const uint32_t gid = blockIdx.x * 256u + threadIdx.x;
+    if (gid >= env_count * m.max_dof) return;
+    const uint32_t env = gid / m.max_dof, dof = gid - env * m.max_dof;
+    float value = 0.0f;
+    if (dof < m.dof) {
+        const uint32_t link = m.dof_link[dof], component = m.dof_component[dof];
+        value = component == kInvalid ? d.qdot[size_t{env} * m.links_per_env + link]
+                                      : d.link_velocity[(size_t{env} * m.links_per_env + link) * 6u + component];
+    }
+    d.step_qdot_flat[gid] = value;
+}
+}  // namespace
+
+// SnapshotStepVelocity (assemble_rows.cu:1457-1477): the generalized velocity the step starts from.  Only the
+// compliant rows of the MuJoCo contact law read it (PrepareContactRowsKernel :1134-1140), so a world without a
+// MuJoCo-sourced profile has nothing to record.
+Status OpSnapshotStepVelocity(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const SnapshotStepVelocityParams*>(params);
+    if (p == nullptr || p->env_count == 0u) return Status::Failed;
+    if (m.any_mujoco == 0u || m.max_dof == 0u) return Status::Ok;
+    if (p->max_dof != m.max_dof) return Status::InvalidArgument;
+    const uint32_t total = p->env_count * m.max_dof;
+    hipLaunchKernelGGL(SnapshotStepVelocityKernel, dim3((total + 255u) / 256u), dim3(256), 0, stream, m, d, p->env_count);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
 
 void InitContactKernels() {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(AssembleRowsKernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);

@@ -18,7 +18,9 @@ NKH_DECLARE_WIDTH(52) NKH_DECLARE_WIDTH(56) NKH_DECLARE_WIDTH(60) NKH_DECLARE_WI
 // Heads the solver's LDS holds: the contact heads (each stages three Jacobian rows) plus one unit head per joint row
 // slot.  Returns the contact-head capacity that fits `lds_budget_bytes`, 0 when not even one does.
 uint32_t SolverHeadCapacity(const ModelView& m, uint32_t slots, size_t lds_budget_bytes) {
-    const uint32_t want = slots * (m.max_points_per_slot == 0u ? kPointsPerSlot : m.max_points_per_slot);
+    // a contact point is one head, or four under the pyramidal cone of the MuJoCo law (one scalar head an edge)
+    const uint32_t heads_per_point = m.any_mujoco != 0u && m.contact_cone == 0u ? kRowsPerPoint : 1u;
+    const uint32_t want = slots * (m.max_points_per_slot == 0u ? kPointsPerSlot : m.max_points_per_slot) * heads_per_point;
     const uint32_t joint_heads = m.joint_limit_rows + m.joint_friction_rows + m.joint_drive_rows;
     for (uint32_t staged = want; staged >= 1u; --staged)
         if (size_t{solver::SolverLdsFloats(m.dof, staged + joint_heads, staged)} * sizeof(float) <= lds_budget_bytes) return staged;
@@ -95,11 +97,15 @@ Status OpBlockDescentSolve(const ModelView& m, const DataView& d, const void* pa
     // lets more blocks share a compute unit, environments with few contact points go to a launch of that capacity:
     // up to three such launches, for eight, four and two blocks a unit, before the full one.  Each launch takes the
     // environments whose contact points fall in its range; an environment's results do not depend on its launch.
-    const bool contacts_only = joint_heads == 0u && staged <= uint32_t(solver::kWave);
+    // (the elliptic cone of the MuJoCo law is answered by the general kernel only)
+    const bool contacts_only = joint_heads == 0u && staged <= uint32_t(solver::kWave) && !(m.any_mujoco != 0u && m.contact_cone == 1u);
     const SolverKernel kernel = kSolverKernels[contacts_only ? 1 : 0][solver::PaddedWidth(m.dof) / 4u - 1u];
     hipLaunchKernelGGL(OrderTilesKernel, dim3(1), dim3(1024), 0, stream, d, p->env_count);
     uint32_t first_points = 0u;
-    if (p->contact_slots_per_env != 0u) {
+    // (a launch takes its environments by their contact points, one head a point: not under the pyramidal cone, whose
+    // worlds go to the one full launch)
+    const bool one_head_a_point = !(m.any_mujoco != 0u && m.contact_cone == 0u);
+    if (p->contact_slots_per_env != 0u && one_head_a_point) {
         for (const size_t blocks : {size_t{8u}, size_t{4u}, size_t{2u}}) {
             if (blocks > most_blocks) continue;                            // more blocks than the waves allow
             if (blocks_per_unit(staged) >= blocks) break;                  // the full capacity does as well

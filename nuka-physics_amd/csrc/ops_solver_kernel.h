@@ -170,6 +170,38 @@ __device__ __forceinline__ void tangent_impulse(V3 dual, float rho, float res_y,
     tangent_impulse(dual, rho, res_y, res_z, normal_impulse, tangent_ratios(mu_first, mu_second), fy, fz, cyy, czz, cyz);
 }
 
+// ComputeEllipticResponse (augmented_row.hpp:48-55): residual scale k and dual scale s of the three axes
+struct EllipticResponse { float kx, ky, kz, sx, st; };
+__device__ __forceinline__ EllipticResponse elliptic_response(float cap, float cn, float cy, float cz) {
+    const double tangent = fmin(double(cy), double(cz));
+    const double normal_scale = 1.0 / (1.0 + double(cap) * cn);
+    const double tangent_scale = 1.0 / (1.0 + double(cap) * tangent);
+    return EllipticResponse{float(cap * normal_scale), float(cap * tangent_scale * tangent / cy), float(cap * tangent_scale * tangent / cz),
+                            float(normal_scale), float(tangent_scale)};
+}
+// EvaluateEllipticImpulse (augmented_row.hpp:58-80): the projection onto the friction cone in the metric that makes
+// its cross section a circle; curvature xx yy zz xy xz yz
+__device__ __forceinline__ void elliptic_impulse(V3 dual, float cap, float rx, float ry, float rz, float cn, float cy, float cz, float mu_first,
+                                                 float* f, float* cv) {
+    const EllipticResponse e = elliptic_response(cap, cn, cy, cz);
+    const float xx = fmaf(e.kx, rx, e.sx * dual.x), xy = fmaf(e.ky, ry, e.st * dual.y), xz = fmaf(e.kz, rz, e.st * dual.z);
+    const float root_x = sqrtf(e.kx), root_y = sqrtf(e.ky), root_z = sqrtf(e.kz);
+    const float m = mu_first * root_x / root_y;
+    const float p = xx / root_x, q1 = xy / root_y, q2 = xz / root_z;
+    const float t = hypotf(q1, q2);
+    f[0] = f[1] = f[2] = 0.0f;
+    cv[0] = cv[1] = cv[2] = cv[3] = cv[4] = cv[5] = 0.0f;
+    if (t <= m * p) { f[0] = xx; f[1] = xy; f[2] = xz; cv[0] = e.kx; cv[1] = e.ky; cv[2] = e.kz; return; }
+    if (m * t + p <= 0.0f) return;
+    const float a = 1.0f / (1.0f + m * m);
+    const float projected = (p + m * t) * a;
+    const float u1 = q1 / t, u2 = q2 / t;
+    const float b = m * projected / t, along = m * m * a;
+    f[0] = projected * root_x; f[1] = m * projected * u1 * root_y; f[2] = m * projected * u2 * root_z;
+    cv[0] = e.kx * a; cv[1] = e.ky * (along * u1 * u1 + b * u2 * u2); cv[2] = e.kz * (along * u2 * u2 + b * u1 * u1);
+    cv[3] = root_x * root_y * m * a * u1; cv[4] = root_x * root_z * m * a * u2; cv[5] = root_y * root_z * (along - b) * u1 * u2;
+}
+
 __device__ __forceinline__ uint32_t residual_bits(float value) { return __float_as_uint(value <= FLT_MAX ? fabsf(value) : FLT_MAX); }
 __device__ __forceinline__ float along_axis(float impulse, float velocity) { return impulse > 0.0f ? velocity : impulse < 0.0f ? -velocity : 0.0f; }
 
@@ -183,6 +215,13 @@ enum HeadField : uint32_t {
     hUnitValue,          // its Jacobian entry there
     hFieldCount
 };
+
+// A contact head under the elliptic cone of the MuJoCo law (block_descent_tile.cuh:645, 778) carries 4 in hAxes: three
+// axes, answered by elliptic_impulse.  Such a head has no relaxation state (its dual update takes the projection as it
+// is), so the first two words of hRelaxStep hold what it needs instead: the compliances of its two tangent rows.
+constexpr uint32_t kAxesElliptic = 4u;
+constexpr uint32_t hTangentCompliance = hRelaxStep;
+__device__ __forceinline__ bool block_axes(uint32_t axes) { return axes >= 3u; }
 
 // A head on one axis uses the first component of every three-component field and none of the block-only fields;
 // only block heads (three axes: contact points, which are listed first) use the rest.  The fields are therefore kept
@@ -221,6 +260,7 @@ struct Tile {
     mutable bool factor_current;     // no head's curvature has changed since hfac was factored: the Hessian is the same
     mutable uint32_t work;   // Newton steps and line probes of this solve, the next solve's scheduling key
     bool mass_valid;
+    bool elliptic;   // some head is under the elliptic cone: every response goes through the general functions
     bool units;      // some head is a unit head
     bool unit_lists; // every coordinate's unit heads fit its list
     uint32_t* unit_list;      // kUnitSlots x 64: lane's unit heads in head order, slot-major
@@ -246,12 +286,18 @@ struct Tile {
 // TileResponse (block_descent_tile.cuh:678-681) with the Coulomb branch of EvaluateAugmentedResponse (block_descent.cu:1593-1621)
 __device__ __forceinline__ void head_response(const Tile& c, uint32_t h, float mx, float my, float mz, float* f, float* cv) {
     const float rho = c.F(hRho, h);
+    if (c.elliptic && c.U(hAxes, h) == kAxesElliptic) {   // block_descent.cu:1595-1601
+        elliptic_impulse(V3{c.F(hDual, h), c.F(hDual + 1, h), c.F(hDual + 2, h)}, rho, c.F(hRes, h) - mx, c.F(hRes + 1, h) - my,
+                         c.F(hRes + 2, h) - mz, c.F(hCompliance, h), c.F(hTangentCompliance, h), c.F(hTangentCompliance + 1, h),
+                         c.F(hMu1, h), f, cv);
+        return;
+    }
     float ni, nc;
     scalar_impulse(c.F(hDual, h), rho, c.F(hRes, h) - mx, c.F(hCompliance, h), c.F(hLower, h), c.F(hUpper, h),
                    Response{c.F(hDualScale, h), c.F(hResidualScale, h)}, &ni, &nc);
     f[0] = ni; f[1] = f[2] = 0.0f;
     cv[0] = nc; cv[1] = cv[2] = cv[3] = cv[4] = cv[5] = 0.0f;
-    if (c.U(hAxes, h) != 3u) return;
+    if (!block_axes(c.U(hAxes, h))) return;
     tangent_impulse(V3{c.F(hDual, h), c.F(hDual + 1, h), c.F(hDual + 2, h)}, rho, c.F(hRes + 1, h) - my, c.F(hRes + 2, h) - mz,
                     c.F(hNormalBound, h), c.F(hMu1, h), c.F(hMu2, h), &f[1], &f[2], &cv[1], &cv[2], &cv[5]);
 }
@@ -505,7 +551,8 @@ __device__ __forceinline__ void add_head(const Tile& c, uint32_t h, bool coordin
 // One head's line-search inputs in registers: nothing in them changes between the probes of one search, and neither
 // do the parts of its response that do not depend on the probe (plain_line).
 struct HeadLine {
-    bool owned, contact, bounded, cone;
+    bool owned, contact, bounded, cone, elliptic;
+    float tangent_compliance[2], mu_first;
     float rho, compliance, lower, upper, bound;
     Response response;
     TangentRatios ratios;
@@ -517,7 +564,9 @@ __device__ __forceinline__ HeadLine load_head_line(const Tile& c, uint32_t h) {
     HeadLine l{};
     l.owned = h < c.heads && c.U(hOwned, h) != 0u;
     if (!l.owned) return l;
-    l.contact = c.U(hAxes, h) == 3u;
+    l.contact = block_axes(c.U(hAxes, h));
+    l.elliptic = c.elliptic && c.U(hAxes, h) == kAxesElliptic;
+    if (l.elliptic) { l.tangent_compliance[0] = c.F(hTangentCompliance, h); l.tangent_compliance[1] = c.F(hTangentCompliance + 1, h); l.mu_first = c.F(hMu1, h); }
     l.rho = c.F(hRho, h); l.compliance = c.F(hCompliance, h); l.lower = c.F(hLower, h); l.upper = c.F(hUpper, h);
     l.bound = c.F(hNormalBound, h);
     l.response = Response{c.F(hDualScale, h), c.F(hResidualScale, h)};
@@ -551,6 +600,12 @@ __device__ __forceinline__ void add_line_terms(const float (&f)[3], const float 
 __device__ __forceinline__ void line_terms(const HeadLine& l, float alpha, TileSum& row_slope, float& row_curvature, float& row_magnitude) {
     const float sx = l.step[0], sy = l.step[1], sz = l.step[2];
     float f[3] = {0.0f, 0.0f, 0.0f}, r[6] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    if (l.elliptic) {
+        elliptic_impulse(V3{l.dual[0], l.dual[1], l.dual[2]}, l.rho, l.res[0] - fmaf(alpha, sx, l.move[0]), l.res[1] - fmaf(alpha, sy, l.move[1]),
+                         l.res[2] - fmaf(alpha, sz, l.move[2]), l.compliance, l.tangent_compliance[0], l.tangent_compliance[1], l.mu_first, f, r);
+        add_line_terms(f, r, sx, sy, sz, row_slope, row_curvature, row_magnitude);
+        return;
+    }
     scalar_impulse(l.dual[0], l.rho, l.res[0] - fmaf(alpha, sx, l.move[0]), l.compliance, l.lower, l.upper, l.response, &f[0], &r[0]);
     if (l.contact)
         tangent_impulse(V3{l.dual[0], l.dual[1], l.dual[2]}, l.rho, l.res[1] - fmaf(alpha, sy, l.move[1]),
@@ -645,8 +700,9 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
 #pragma unroll
         for (int k = 0; k < 3; ++k) mn[k] = fabsf(mf[k]) + mc[k] * (fabsf(own.res[k]) + fabsf(own.move[k]));
     }
+    if (c.elliptic) head_terms(c, lane, mf, mc, mn);   // the cone's own response; the same values as above for every other head
     const bool mine = mf[0] != 0.0f || mf[1] != 0.0f || mf[2] != 0.0f || mc[0] != 0.0f || mc[1] != 0.0f || mc[2] != 0.0f || mc[5] != 0.0f ||
-                      mn[0] != 0.0f || mn[1] != 0.0f || mn[2] != 0.0f;
+                      mc[3] != 0.0f || mc[4] != 0.0f || mn[0] != 0.0f || mn[1] != 0.0f || mn[2] != 0.0f;
     const uint32_t my_axes = lane < c.heads ? c.U(hAxes, lane) : 0u;
     const uint32_t my_low = lane < c.heads ? c.U(hColumnsLow, lane) : 0u, my_high = lane < c.heads ? c.U(hColumnsHigh, lane) : 0u;
     // The Hessian M + sum J^T C J changes only through the heads' curvatures: every head keeps the curvature of its
@@ -880,7 +936,7 @@ __device__ __forceinline__ void plain_line_terms(const PlainLine& p, float alpha
     row_magnitude += fabsf(f[0] * sx) + fabsf(f[1] * sy) + fabsf(f[2] * sz);
     row_curvature += r[0] * sx * sx + r[1] * sy * sy + r[2] * sz * sz + 2.0f * r[5] * sy * sz;
 }
-// `general` (uniform): the block has more heads than lanes
+// `general` (uniform): the block has more heads than lanes, or some head is under the elliptic cone
 __device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& mine, const PlainLine& plain, bool general, float alpha,
                                  float inertial_slope, float inertial_curvature, float* slope, float* curvature, float* magnitude) {
     PROF_COUNT(c, 1);
@@ -914,7 +970,7 @@ __device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& 
 __device__ __forceinline__ float search_line(const Tile& c, float inertial_slope, float inertial_curvature) {
     float slope = 0.0f, curvature = 0.0f, magnitude = 0.0f;
     const HeadLine mine = load_head_line(c, c.lane);
-    const bool general = c.heads > uint32_t(kWave);
+    const bool general = c.heads > uint32_t(kWave) || c.elliptic;
     const PlainLine plain = plain_line(mine);
     line_derivatives(c, mine, plain, general, 0.0f, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
     const float initial = slope;
@@ -1092,13 +1148,13 @@ __device__ __forceinline__ void measure_primal(Tile& c, const float (&mrow)[N], 
         add_units(done, h);
         done = h + 1u;
         const uint32_t local = c.U(hSlot, h) - c.env * R, stride = c.U(hStride, h), axes = c.U(hAxes, h);
-        const float ix = lambda_env[local], iy = axes == 3u ? lambda_env[local + stride] : 0.0f,
-                    iz = axes == 3u ? lambda_env[local + 2u * stride] : 0.0f;
+        const float ix = lambda_env[local], iy = block_axes(axes) ? lambda_env[local + stride] : 0.0f,
+                    iz = block_axes(axes) ? lambda_env[local + 2u * stride] : 0.0f;
         if (!(ix != 0.0f || iy != 0.0f || iz != 0.0f)) continue;
         if (!coordinate) continue;
         const float* j = c.jac + first * c.ldj;
         balance += double(j[lane]) * ix;
-        if (axes == 3u) {
+        if (block_axes(axes)) {
             balance += double(j[c.ldj + lane]) * iy;
             balance += double(j[2u * c.ldj + lane]) * iz;
         }
@@ -1169,7 +1225,8 @@ __device__ __forceinline__ void update_duals(const Tile& c, float* lambda_env, u
     double restart = 0.0;
     for (uint32_t h = c.lane; h < c.heads; h += kWave) {
         const uint32_t slot = c.U(hSlot, h), local = slot - c.env * R, stride = c.U(hStride, h), axes = c.U(hAxes, h);
-        const bool contact = axes == 3u;
+        const bool contact = block_axes(axes);
+        const bool elliptic = c.elliptic && axes == kAxesElliptic;
         const float rho = c.F(hRho, h), compliance = c.F(hCompliance, h), lower = c.F(hLower, h), upper = c.F(hUpper, h);
         const float mu1 = c.F(hMu1, h), mu2 = c.F(hMu2, h);
         const Response response{c.F(hDualScale, h), c.F(hResidualScale, h)};
@@ -1181,7 +1238,13 @@ __device__ __forceinline__ void update_duals(const Tile& c, float* lambda_env, u
         V3 dual{normal, 0.0f, 0.0f};
         V3 rstep{0, 0, 0}, rpoint{0, 0, 0};
         float rweight = 0.0f;
-        if (contact) {   // ProjectRowDual (block_descent.cu:799-804) with RelaxContactImpulse (augmented_row.hpp:128-138)
+        float cone_y = 0.0f, cone_z = 0.0f;
+        if (elliptic) {   // :2509-2510: the projection onto the elliptic cone as it is
+            cone_y = c.F(hTangentCompliance, h); cone_z = c.F(hTangentCompliance + 1, h);
+            float f[3], cv[6];
+            elliptic_impulse(tdual, rho, residual.x, residual.y, residual.z, compliance, cone_y, cone_z, mu1, f, cv);
+            dual = V3{f[0], f[1], f[2]};
+        } else if (contact) {   // ProjectRowDual (block_descent.cu:799-804) with RelaxContactImpulse (augmented_row.hpp:128-138)
             float fy, fz, cyy, czz, cyz;
             tangent_impulse(tdual, rho, residual.y, residual.z, normal, mu1, mu2, &fy, &fz, &cyy, &czz, &cyz);
             const V3 next{normal, fy, fz};
@@ -1214,6 +1277,12 @@ __device__ __forceinline__ void update_duals(const Tile& c, float* lambda_env, u
             step_tangent = hypotf(first, second);
         }
         if (!commit && response.residual_scale > 0.0f) step_normal = fabsf(dual.x - tdual.x) / response.residual_scale;
+        EllipticResponse cone{};
+        if (elliptic) {   // EllipticMultiplierStep (augmented_row.hpp:104-108; :2516-2519)
+            cone = elliptic_response(rho, compliance, cone_y, cone_z);
+            step_normal = fabsf(dual.x - tdual.x) / cone.kx;
+            step_tangent = fmaxf(fabsf(dual.y - tdual.y) / cone.ky, fabsf(dual.z - tdual.z) / cone.kz);
+        }
         const V3 physical = commit ? dual : tdual;
         if (!contact) {
             const bool normal_row = (__float_as_uint(urows[size_t{slot} * kRowWords]) & kRowContactNormal) != 0u;
@@ -1224,15 +1293,22 @@ __device__ __forceinline__ void update_duals(const Tile& c, float* lambda_env, u
             else steps[2] = max(steps[2], residual_bits(value));
         } else {
             if (commit) {
-                c.F(hRelaxStep, h) = rstep.x; c.F(hRelaxStep + 1, h) = rstep.y; c.F(hRelaxStep + 2, h) = rstep.z;
-                c.F(hRelaxWeight, h) = rweight;
-                c.F(hRelaxPoint, h) = rpoint.x; c.F(hRelaxPoint + 1, h) = rpoint.y; c.F(hRelaxPoint + 2, h) = rpoint.z;
+                if (!elliptic) {   // an elliptic head keeps its tangent compliances where the others keep this state
+                    c.F(hRelaxStep, h) = rstep.x; c.F(hRelaxStep + 1, h) = rstep.y; c.F(hRelaxStep + 2, h) = rstep.z;
+                    c.F(hRelaxWeight, h) = rweight;
+                    c.F(hRelaxPoint, h) = rpoint.x; c.F(hRelaxPoint + 1, h) = rpoint.y; c.F(hRelaxPoint + 2, h) = rpoint.z;
+                }
                 lambda_env[local + stride] = dual.y;
                 lambda_env[local + 2u * stride] = dual.z;
             }
-            const V3 v{-residual.x + compliance * physical.x, -residual.y, -residual.z};
-            steps[0] = max(steps[0], residual_bits(physical.x > 0.0f ? fabsf(v.x) : fmaxf(-v.x, 0.0f)));
-            steps[1] = max(steps[1], residual_bits(fmaxf(step_tangent, fmaxf(along_axis(physical.y, v.y), along_axis(physical.z, v.z)))));
+            if (elliptic) {   // :2539-2542
+                steps[0] = max(steps[0], residual_bits(step_normal));
+                steps[1] = max(steps[1], residual_bits(step_tangent));
+            } else {
+                const V3 v{-residual.x + compliance * physical.x, -residual.y, -residual.z};
+                steps[0] = max(steps[0], residual_bits(physical.x > 0.0f ? fabsf(v.x) : fmaxf(-v.x, 0.0f)));
+                steps[1] = max(steps[1], residual_bits(fmaxf(step_tangent, fmaxf(along_axis(physical.y, v.y), along_axis(physical.z, v.z)))));
+            }
         }
         if (!commit) continue;
         if (velocity) lambda_env[local] = dual.x;
@@ -1241,7 +1317,8 @@ __device__ __forceinline__ void update_duals(const Tile& c, float* lambda_env, u
             const float friction = fmaxf(mu1, mu2);
             const float first = contact && mu1 > 0.0f ? mu1 / friction : 0.0f;
             const float second = contact && mu2 > 0.0f ? mu2 / friction : 0.0f;
-            const V3 metric{response.residual_scale, rho * first * first, rho * second * second};
+            V3 metric{response.residual_scale, rho * first * first, rho * second * second};
+            if (elliptic) metric = V3{cone.kx, cone.ky, cone.kz};   // :2555-2557
             restart += (metric.x > 0.0f ? (double(tdual.x) - dual.x) * (double(dual.x) - base.x) / metric.x : 0.0) +
                        (metric.y > 0.0f ? (double(tdual.y) - dual.y) * (double(dual.y) - base.y) / metric.y : 0.0) +
                        (metric.z > 0.0f ? (double(tdual.z) - dual.z) * (double(dual.z) - base.z) / metric.z : 0.0);
@@ -1261,7 +1338,7 @@ __device__ __forceinline__ void update_duals(const Tile& c, float* lambda_env, u
         momentum->beta = (momentum->t - 1.0f) / t;
         momentum->t = t;
         for (uint32_t h = c.lane; h < c.heads; h += kWave) {
-            const bool contact = c.U(hAxes, h) == 3u;
+            const bool contact = block_axes(c.U(hAxes, h));
             const bool extrapolate = contact || c.F(hDualScale, h) != 0.0f;
             const float beta = extrapolate ? momentum->beta : 0.0f;
             const V3 base{c.F(hMove, h), c.F(hMove + 1, h), c.F(hMove + 2, h)};
@@ -1320,7 +1397,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     Tile c;
     c.env = env; c.lane = lane; c.n = n; c.ld = uint32_t(N) + 1u; c.ldj = uint32_t(N); c.cap = cap; c.narrow = staged_cap; c.heads = 0u; c.iteration = 0u;
     c.tolerance = p.velocity_tolerance; c.failed = false; c.momentum = 0.0f; c.residual = 0.0f;
-    c.mass_inverse = 0.0f; c.mass_valid = false; c.work = 0u; c.units = false;
+    c.mass_inverse = 0.0f; c.mass_valid = false; c.work = 0u; c.units = false; c.elliptic = false;
     c.factor_current = false;
 #ifdef NKH_SOLVER_PROFILE
     for (int i = 0; i < 26; ++i) c.prof[i] = 0;
@@ -1641,6 +1718,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     PROF_END(c, 18);
     PROF_BEGIN(c, 19);
     // InitializeTileHead (:743-797), lane = head
+    bool any_elliptic = false;
     for (uint32_t base = 0u; base < heads; base += kWave) {
         const uint32_t h = base + lane;
         if (h < heads) {
@@ -1665,7 +1743,10 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
             const float compliance = row[5];
             const Response sr = scalar_response(rho, compliance);
             const uint32_t local = slot - env * R;
-            c.U(hStride, h) = stride; c.U(hAxes, h) = axes;
+            // three axes of a MuJoCo-law contact: the elliptic cone, with the compliances of the two tangent rows (:778-780)
+            const bool elliptic = !kContactsOnly && axes == 3u && (flags & kRowMuJoCo) != 0u;
+            any_elliptic = any_elliptic || elliptic;
+            c.U(hStride, h) = stride; c.U(hAxes, h) = elliptic ? kAxesElliptic : axes;
             c.U(hOwned, h) = (kind_a == kSideArtic || kind_b == kSideArtic) ? 1u : 0u;
             c.F(hRho, h) = rho; c.F(hCompliance, h) = compliance; c.F(hLower, h) = row[6]; c.F(hUpper, h) = row[7];
             c.F(hMu1, h) = row[8]; c.F(hMu2, h) = row[9]; c.F(hNormalBound, h) = 0.0f;
@@ -1677,8 +1758,13 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
 #pragma unroll
             for (int k = 0; k < 3; ++k) { c.F(hRes + k, h) = 0.0f; c.F(hMove + k, h) = 0.0f; c.F(hStep + k, h) = 0.0f; c.F(hRelaxStep + k, h) = 0.0f; c.F(hRelaxPoint + k, h) = 0.0f; }
             c.F(hRelaxWeight, h) = 0.0f;
+            if (elliptic) {
+                c.F(hTangentCompliance, h) = urows[size_t{slot + stride} * kRowWords + 5u];
+                c.F(hTangentCompliance + 1, h) = urows[size_t{slot + 2u * stride} * kRowWords + 5u];
+            }
         }
     }
+    c.elliptic = !kContactsOnly && __any(any_elliptic);
     __syncthreads();
     PROF_END(c, 19);
     PROF_BEGIN(c, 20);

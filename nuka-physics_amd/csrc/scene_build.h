@@ -294,6 +294,10 @@ struct Geom {
     int32_t group = 0;
     float friction = 1.0f;
     bool friction_authored = false;
+    // the MuJoCo contact law's terms of the geom (src/import/mjcf_importer.cpp:162-165, 1009-1015)
+    float solref[2] = {0.02f, 1.0f};
+    float solimp[5] = {0.9f, 0.95f, 0.001f, 0.5f, 2.0f};
+    float margin = 0.0f, gap = 0.0f;
 };
 struct Link {
     std::string name, joint_name;

@@ -21,6 +21,9 @@ constexpr uint32_t kPlaneContactsOnly = 1u;
 constexpr uint32_t kFixedBase = 2u;
 // A static ground plane z = 0 is added to the file's collidables (a URDF names none).
 constexpr uint32_t kGroundPlane = 4u;
+// MJCF: the geoms keep this library's native contact law (speculative velocity rows) instead of the MuJoCo law the
+// reference's importer gives every MJCF shape (src/import/mjcf_importer.cpp:790).
+constexpr uint32_t kNativeContactLaw = 8u;
 
 struct Scene {
     nuka_template_desc_t desc{};
@@ -29,7 +32,11 @@ struct Scene {
     std::vector<uint32_t> parent_link, body_role, body_link, shape_kind, shape_contype, shape_conaffinity, shape_group, shape_profile,
         excluded_pairs;   // [pair][2] collidable rows that never pair
     std::vector<float> joint_axis, link_local_pose, link_inertial_frame, link_mass, link_diag_inertia, joint_damping, joint_armature,
-        joint_stiffness, joint_spring_reference, joint_frictionloss, joint_limit_lower, joint_limit_upper, body_local, shape_params, profile_mu;
+        joint_stiffness, joint_spring_reference, joint_frictionloss, joint_limit_lower, joint_limit_upper, body_local, shape_params, profile_mu,
+        profile_solref, profile_solimp, profile_margin;
+    std::vector<uint32_t> profile_law;
+    uint32_t contact_cone = 0u;      // <option cone>: 0 pyramidal (MuJoCo's default), 1 elliptic
+    float contact_impratio = 1.0f;   // <option impratio>
     std::vector<float> initial_q, drive_stiffness, drive_damping, drive_force_limit, drive_joint_force_limit;
     std::array<float, 7> base_pose{0, 0, 0, 1, 0, 0, 0};
     bool floating_root = false;

@@ -65,7 +65,9 @@ struct HostModel {
         link_geom_kind, body_to_link, body_to_articulation, body_collidable_link, body_collidable_body;
     std::vector<uint64_t> link_dof_mask, excluded_pairs;
     std::vector<float> joint_axis, parent_offset, link_local_pose, link_inertial_frame, link_inertia, joint_damping, joint_armature,
-        joint_stiffness, joint_spring_reference, joint_limit_lower, joint_limit_upper, joint_frictionloss, link_geom_local, shape_table, body_collidable_local, body_init_pose, profile_mu;
+        joint_stiffness, joint_spring_reference, joint_limit_lower, joint_limit_upper, joint_frictionloss, link_geom_local, shape_table, body_collidable_local, body_init_pose, profile_mu,
+        profile_solref, profile_solimp, profile_margin;
+    std::vector<uint32_t> profile_law;
     std::vector<float> link_mass, link_diag_inertia;   // kept for nuka_world_set_param: a new mass rebuilds the spatial inertia
 };
 
@@ -154,6 +156,22 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
     m.body_collidable_local.resize(size_t{nb} * 7u);
     m.body_init_pose.resize(size_t{nb} * 7u);
     m.profile_mu.assign(d.profile_mu, d.profile_mu + 2u * d.profile_count);
+    // the MuJoCo-law terms of each profile, at the defaults of ContactParamsIn (scene/contact_filter.hpp:20-37) where not authored
+    m.profile_law.assign(d.profile_count, 0u);
+    m.profile_solref.resize(2u * d.profile_count); m.profile_solimp.resize(5u * d.profile_count); m.profile_margin.assign(2u * d.profile_count, 0.0f);
+    {
+        const float solimp[5] = {0.9f, 0.95f, 0.001f, 0.5f, 2.0f};
+        for (uint32_t i = 0u; i < d.profile_count; ++i) {
+            if (d.profile_law != nullptr) m.profile_law[i] = d.profile_law[i];
+            m.profile_solref[2u * i] = d.profile_solref != nullptr ? d.profile_solref[2u * i] : 0.02f;
+            m.profile_solref[2u * i + 1u] = d.profile_solref != nullptr ? d.profile_solref[2u * i + 1u] : 1.0f;
+            for (uint32_t k = 0u; k < 5u; ++k) m.profile_solimp[5u * i + k] = d.profile_solimp != nullptr ? d.profile_solimp[5u * i + k] : solimp[k];
+            for (uint32_t k = 0u; k < 2u; ++k) if (d.profile_margin != nullptr) m.profile_margin[2u * i + k] = d.profile_margin[2u * i + k];
+            if (m.profile_law[i] > 1u) throw std::invalid_argument("unknown profile law");
+            for (uint32_t k = 0u; k < 2u; ++k) if (!std::isfinite(m.profile_solref[2u * i + k]) || !std::isfinite(m.profile_margin[2u * i + k])) throw std::invalid_argument("invalid profile solref or margin");
+            for (uint32_t k = 0u; k < 5u; ++k) if (!std::isfinite(m.profile_solimp[5u * i + k])) throw std::invalid_argument("invalid profile solimp");
+        }
+    }
     auto bits = [](uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; };
     for (uint32_t b = 0u; b < nb; ++b) {
         const uint32_t role = d.body_role[b], link = d.body_link[b];
@@ -253,6 +271,11 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
     c.drive_mode = d.drive_rows != 0u ? d.drive_mode : uint32_t(kDriveTorque);
     c.rows_per_env = c.contact_rows_per_env + c.joint_limit_rows + c.joint_friction_rows + c.joint_drive_rows;
     c.profile_count = d.profile_count;
+    c.any_mujoco = 0u;
+    for (uint32_t law : m.profile_law) if (law == 1u) c.any_mujoco = 1u;
+    if (d.contact_cone > 1u) throw std::invalid_argument("unknown contact cone");
+    c.contact_cone = d.contact_cone;
+    c.contact_impratio = d.contact_impratio > 0.0f ? d.contact_impratio : 1.0f;
     c.floating_root = m.joint_type[0] == kFloatingBase ? 1u : 0u;
     c.max_points_per_slot = max_points;
     c.excluded_pair_count = uint32_t(m.excluded_pairs.size());
@@ -277,6 +300,8 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(contact_row_extent, kU32, E * 2) X(env_status, kU32, E) X(vbd_velocity_sweep_count, kU32, E) \
     X(solver_residual, kF32, E * 4) X(solver_penalty, kF32, E * R) X(solver_velocity, kF32, E * md) X(solver_free, kF32, E * md) \
     X(solver_cost, kU32, E) X(tile_order, kU32, E) X(row_unit, kU32, E * R) X(row_unit_value, kF32, E * R) \
+    X(body_invweight0, kF32, E * nb * 2) X(dof_invweight0, kF32, E * md) X(row_invweight, kF32, E * R) \
+    X(row_reference_velocity_gain, kF32, E * R) X(step_qdot_flat, kF32, E * md) \
     X(contact_material, kU64, E * S) X(contact_cache_pair, kU64, E * S * 4) X(contact_cache_feature, kU64, E * S * 4) \
     X(contact_cache_material, kU64, E * S * 4) X(contact_cache_lambda, kF32, E * S * 16) X(contact_cache_normal, kF32, E * S * 12) \
     X(contact_cache_age, kU32, E * S * 4) X(contact_cache_current_owner, kU32, E * S * 4) X(contact_cache_old_keep, kU32, E * S * 4) \
@@ -302,7 +327,7 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(link_dof, kU32) X(dof_link, kU32) X(dof_component, kU32) X(link_dof_mask, kU64) X(link_geom_kind, kU32) \
     X(link_geom_local, kF32) X(shape_table, kF32) X(body_to_link, kU32) X(body_to_articulation, kU32) \
     X(body_collidable_link, kU32) X(body_collidable_body, kU32) X(body_collidable_local, kF32) X(profile_mu, kF32) \
-    X(excluded_pairs, kU64)
+    X(profile_law, kU32) X(profile_solref, kF32) X(profile_solimp, kF32) X(profile_margin, kF32) X(excluded_pairs, kU64)
 
 uint32_t DtypeBytes(Dtype t) { return t == kU64 ? 8u : t == kU8 ? 1u : 4u; }
 
@@ -344,6 +369,7 @@ struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
     ContactWarmStartParams p_warm0{}, p_warm1{};
     BlockDescentSolveParams p_solve{};
     SnapshotStepVelocityParams p_snapshot{};
+    ReferenceWeightsParams p_reference_weights{};   // dispatched at creation, outside the step (nk/pipeline/world.cpp:553-561)
     NarrowphaseHeightfieldParams p_heightfield{};
     std::vector<AccumulateStepParams> p_accumulate;   // one per substep (pipeline.cpp:128-152)
     nuka_execution_mode_t mode = NUKA_EXECUTION_EAGER;
@@ -422,6 +448,8 @@ std::mutex g_static_reset_mutex;                            // guards the host s
 
 bool CheckpointKeeps(const char* name) {
     for (const char* kept : {"q", "qdot", "qddot", "tau", "base_pose", "link_pose", "link_velocity", "body_pose", "lambda", "link_wrench",
+                             "drive_target", "drive_stiffness", "drive_damping", "drive_force_limit", "drive_joint_force_limit",
+                             "velocity_target", "actuator_noload_speed",
                              "contact_cache_pair", "contact_cache_feature", "contact_cache_material", "contact_cache_lambda",
                              "contact_cache_normal", "contact_cache_age"})
         if (std::strcmp(name, kept) == 0) return true;
@@ -467,6 +495,8 @@ void BuildPipeline(World& w) {
     w.p_int_vel = {};
     w.p_int_vel.dt = dt; w.p_int_vel.total_link_count = E * nl; w.p_int_vel.articulation_count = E;
     std::memcpy(w.p_int_vel.gravity, cfg.gravity, sizeof(cfg.gravity));
+    w.p_snapshot = {E, E, m.max_dof, nl, E * nb, 0u};
+    w.p_reference_weights = {m.max_dof, E, E * nl, 1u, nb, E * nb};
     w.p_int_pos = {};
     w.p_int_pos.dt = dt; w.p_int_pos.total_link_count = E * nl; w.p_int_pos.articulation_count = E; w.p_int_pos.env_count = E;
     w.p_int_pos.pos_pass = (has_contacts && cfg.solver_pos_iters > 0u) ? 1u : 0u;
@@ -497,6 +527,10 @@ void BuildPipeline(World& w) {
     as.dt = dt; as.overlap_recovery_velocity = cfg.solver_overlap_recovery_velocity; as.contact_margin = contact_margin;
     as.joint_limit_rows_per_env = m.joint_limit_rows; as.joint_friction_rows_per_env = m.joint_friction_rows;
     as.joint_drive_rows_per_env = m.joint_drive_rows; as.baumgarte_max_velocity = cfg.solver_baumgarte_max_velocity;
+    // the MuJoCo law's world-wide terms (pipeline.cpp:880-886); a pair's solref and solimp come from its profiles
+    as.solref[0] = 0.02f; as.solref[1] = 1.0f;
+    as.solimp[0] = 0.9f; as.solimp[1] = 0.95f; as.solimp[2] = 0.001f; as.solimp[3] = 0.5f; as.solimp[4] = 2.0f;
+    as.impratio = m.contact_impratio; as.refsafe = true; as.cone = m.contact_cone;
     w.p_warm0 = {};
     w.p_warm0.env_count = E; w.p_warm0.slot_count = m.contact_slots; w.p_warm0.rows_per_env = m.rows_per_env;
     w.p_warm0.full_row_slot_count = m.contact_slots; w.p_warm0.decay_steps = 2u;
@@ -818,8 +852,21 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
             if (hc.drive_mode == kDrivePdPosition) ok = ok && put(w.data.drive_target, tile(scene->initial_q));   // hold the authored pose
             if (!ok) return Error(NUKA_RESULT_DEVICE_ERROR, "scene state upload failed");
         }
-        if (Iface(w.initial)->copy_from(w.initial, w.arena, 0u, 0u, w.arena_bytes) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "snapshot failed");
         BuildPipeline(w);
+        // nk/pipeline/world.cpp:553-561: creation exposes the poses of the initial state and the reference weights at
+        // them.  Only the MuJoCo contact law reads the weights; other worlds first compute their poses in their first step.
+        if (hc.any_mujoco != 0u) {
+            const nuka_phi_op_call at_creation[3] = {{uint16_t(NkOp::FkWorldPoses), &w.p_fk}, {uint16_t(NkOp::SyncLinkBodyPose), &w.p_sync},
+                                                     {uint16_t(NkOp::ReferenceWeights), &w.p_reference_weights}};
+            for (const nuka_phi_op_call& call : at_creation) {
+                if (call.op == uint16_t(NkOp::SyncLinkBodyPose) && nb == 0u) continue;
+                const uint8_t status = w.be->dispatch(w.backend, reinterpret_cast<const nuka_phi_model_view*>(&w.model),
+                                                      reinterpret_cast<const nuka_phi_data_view*>(&w.data), &call);
+                if (status != uint8_t(Status::Ok)) return Error(MapStatus(status), "reference weights failed");
+            }
+            if (w.be->synchronize(w.backend, nullptr) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "device error in the reference weights");
+        }
+        if (Iface(w.initial)->copy_from(w.initial, w.arena, 0u, 0u, w.arena_bytes) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "snapshot failed");
         if (w.be->synchronize(w.backend, nullptr) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "device error during world creation");
         *out = reinterpret_cast<nuka_world_handle>(world.release());
         return NUKA_RESULT_OK;
@@ -845,7 +892,7 @@ nuka_result_t nuka_scene_load_mjcf(const char* path, uint32_t flags, nuka_scene_
     if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
     *out = nullptr;
     if (path == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "path is null");
-    if ((flags & ~uint32_t(NUKA_SCENE_PLANE_CONTACTS_ONLY | NUKA_SCENE_GROUND_PLANE)) != 0u) return Error(NUKA_RESULT_INVALID_ARG, "unknown scene flag");
+    if ((flags & ~uint32_t(NUKA_SCENE_PLANE_CONTACTS_ONLY | NUKA_SCENE_GROUND_PLANE | NUKA_SCENE_NATIVE_CONTACT_LAW)) != 0u) return Error(NUKA_RESULT_INVALID_ARG, "unknown scene flag");
     try {
         *out = reinterpret_cast<nuka_scene_handle>(scene_file::LoadMjcf(path, flags).release());
         return NUKA_RESULT_OK;
@@ -1136,6 +1183,7 @@ nuka_result_t nuka_world_dispatch_op(nuka_world_handle world, uint16_t op, uint3
     for (const nuka_phi_op_call& call : w->calls) if (call.op == op) { params = call.params; break; }
     if (op == uint16_t(NkOp::ArticulationDynamics) && variant == 1u) params = &w->p_dynamics_probe;
     if (op == uint16_t(NkOp::ContactWarmStart) && variant == 1u) params = &w->p_warm1;
+    if (op == uint16_t(NkOp::ReferenceWeights)) params = &w->p_reference_weights;
     if (params == nullptr) return Error(NUKA_RESULT_NOT_SUPPORTED, "op is not part of this world's pipeline");
     const nuka_phi_op_call call{op, params};
     const uint8_t status = w->be->dispatch(w->backend, reinterpret_cast<const nuka_phi_model_view*>(&w->model),

@@ -1091,14 +1091,16 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
         const float mu_a2 = sa.profile < t->n_profiles ? t->profile_mu[2u * sa.profile + 1u] : 1.0f;
         const float mu_b1 = sb.profile < t->n_profiles ? t->profile_mu[2u * sb.profile] : 1.0f;
         const float mu_b2 = sb.profile < t->n_profiles ? t->profile_mu[2u * sb.profile + 1u] : 1.0f;
-        const float mu1 = mu_a1 > mu_b1 ? mu_a1 : mu_b1, mu2 = mu_a2 > mu_b2 ? mu_a2 : mu_b2;
         const int position_pass = w->cfg.solver_pos_iters > 0u;
         const uint32_t law = w->ucontact_law[gid];
         const int mujoco = law == 0u;   /* kContactLawCompliant (:480) */
+        float mu1 = mu_a1 > mu_b1 ? mu_a1 : mu_b1, mu2 = mu_a2 > mu_b2 ? mu_a2 : mu_b2;
+        if (mujoco) { mu1 = fmaxf(1.0e-5f, mu1); mu2 = fmaxf(1.0e-5f, mu2); }   /* :573-576 */
         /* the two sides' profiles merged (:540-594; contact_filter.hpp:100-137), a side without one at the defaults */
         float side_a[11], side_b[11], merged[11];
         profile_terms(t, sa.profile, side_a); profile_terms(t, sb.profile, side_b);
         nko_merge_contact_params(side_a, side_b, merged);
+        if (mujoco) { merged[0] = mu1; merged[1] = mu2; }   /* the clamp above is part of what the material key hashes */
         const float* solref = merged + 2, *solimp = merged + 4;
         const float margin = merged[9];
         const uint32_t weight_a = kind_a == NKO_SIDE_ARTIC ? t->link_body[link_a - env * t->nl] : local_a;
@@ -1110,8 +1112,7 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
         v3 frame_axis = v3_make(0, 0, 0);   /* :601-605: a capsule on a plane aligns the pyramid with the capsule's axis */
         if (pyramidal && sa.kind == 1u && sb.kind == 3u) frame_axis = nko_prim_rotate(xform_load(w->body_pose + ((size_t)env * t->nb + local_a) * 7u).r, v3_make(0, 0, 1));
         if (pyramidal && sb.kind == 1u && sa.kind == 3u) frame_axis = nko_prim_rotate(xform_load(w->body_pose + ((size_t)env * t->nb + local_b) * 7u).r, v3_make(0, 0, 1));
-        w->contact_material[gid] = n_active > 0u ? (mujoco ? nko_contact_material_merged(merged, law, t->cone)
-                                                           : nko_contact_material(mu1, mu2, law)) : 0u;   /* :620-623 */
+        w->contact_material[gid] = n_active > 0u ? nko_contact_material_merged(merged, law, t->cone) : 0u;   /* :620-623 */
         for (uint32_t p = 0u; p < P; ++p) {
             /* velocity_only keeps every point; a compliant point lives inside its margin (:625-626) */
             const int live = p < n_active && p < 4u && (!mujoco || w->ucontact_depth[gid * 4u + p] + margin > 0.0f);

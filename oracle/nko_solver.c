@@ -476,8 +476,9 @@ static int assemble_block(tile* c, const float* u, const float* free_v, float h[
                     scale[i] += fabsf(j0) * noise.x;
                     if (t->axes == 1u) {
                         const float a0 = j0 * cv[0];
-                        if (wide_tile(n)) for (uint32_t kk = i; kk < n; ++kk) h[i][kk] = fmaf(a0, j0r[kk], h[i][kk]);
-                        else for (uint32_t kk = 0u; kk < n; ++kk) h[i][kk] += a0 * j0r[kk];
+                        /* h += a0 j: one product added to the entry, which the reference's compiler contracts to one fused
+                         * multiply-add (:1581-1585) */
+                        for (uint32_t kk = wide_tile(n) ? i : 0u; kk < n; ++kk) h[i][kk] = fmaf(a0, j0r[kk], h[i][kk]);
                         continue;
                     }
                     const float j1 = j1r[i], j2 = j2r[i];

@@ -288,6 +288,7 @@ nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc*
     /* nk/pipeline/world.cpp:553-561: creation exposes the poses of the rest state and the reference weights at them */
     if (t->any_mujoco) {
         nko_fk_world_poses(w);
+        if (t->nb > 0u) nko_sync_link_body_pose(w);
         nko_reference_weights(w);
     }
     return w;

@@ -277,7 +277,21 @@ def test_contact_filtering_fixture_of_the_reference():
                     ("b2", abi.SHAPE_BOX, 10, 1, 0)]        # g_class_override: its own contype wins
     explicit = [r for r in range(len(owner)) if a["shape_kind"][r] != abi.INVALID][0]
     assert a["profile_mu"].reshape(-1, 2)[a["shape_profile"][explicit]][0] == np.float32(0.7)
-    assert a["shape_profile"][explicit + 1] == abi.INVALID                              # friction never authored: the default
+    # every geom is MuJoCo-sourced (mjcf_importer.cpp:790) and carries its solref, solimp, margin and gap; a class's
+    # solref reaches the geoms of the class, and an unauthored geom has the defaults
+    law, solref = a["profile_law"], a["profile_solref"].reshape(-1, 2)
+    solimp, margin = a["profile_solimp"].reshape(-1, 5), a["profile_margin"].reshape(-1, 2)
+    assert (law == abi.LAW_MUJOCO).all()
+    p_explicit, p_default, p_class = (a["shape_profile"][explicit + k] for k in range(3))
+    assert np.array_equal(solref[p_explicit], np.float32([0.01, 0.8])) and np.array_equal(solimp[p_explicit], np.float32([0.8, 0.9, 0.002, 0.4, 3]))
+    assert np.array_equal(margin[p_explicit], np.float32([0.01, 0.005]))
+    assert np.array_equal(solref[p_default], np.float32([0.02, 1.0])) and np.array_equal(solimp[p_default], np.float32([0.9, 0.95, 0.001, 0.5, 2]))
+    assert np.array_equal(margin[p_default], np.float32([0, 0])) and a["profile_mu"].reshape(-1, 2)[p_default][0] == 1.0
+    assert np.array_equal(solref[p_class], np.float32([0.005, 0.5])) and a["shape_profile"][explicit + 3] == p_class
+    assert a["contact_cone"] == abi.CONE_PYRAMIDAL and a["contact_impratio"] == 1.0
+    # with the native law kept, only an authored friction makes a profile
+    native = nk.Scene(os.path.join(GOLDEN, "contact_filtering.xml"), nk.SCENE_NATIVE_CONTACT_LAW).template_arrays()
+    assert native["shape_profile"][explicit + 1] == abi.INVALID and (native["profile_law"] == abi.LAW_NATIVE).all()
     excluded = {frozenset((owner[p[0]], owner[p[1]])) for p in a["excluded_pairs"].reshape(-1, 2)}
     assert excluded == {frozenset(("b1", "b2"))}
 
