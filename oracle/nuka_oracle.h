@@ -26,8 +26,13 @@
  *                             PrimitivePair is covered (sphere, capsule, box, plane, cylinder; box x box included)
  *   row math (AL impulses)  : pinned bit-exact against oracle/_ref (augmented_row.hpp), the committed vectors, and
  *                             the known answers in tests/math/test_contact_tangent.cpp; the compliant-row terms and
- *                             the elliptic cone (no device counterpart) likewise, with the hand-evaluated table of
+ *                             the elliptic cone likewise, with the hand-evaluated table of
  *                             tests/constraint/test_solref_solimp.cpp
+ *   MuJoCo contact law      : pinned (merged profile terms bit-exact against the reference's MergeContactParams in
+ *                             oracle/_ref; reference weights against the closed forms of a free body and a pendulum
+ *                             and a dense float64 J M^-1 J^T of a chain; the compliant normal, tangent and pyramid
+ *                             edge rows against the pinned row math and the geometry of the pyramid; a resting
+ *                             sphere's depth against the closed form of the spring-damper reference, both cones)
  *   chain Jacobian          : pinned (J qdot == contact point velocity of the float64 model)
  *   contact cache           : pinned by behaviour (seeding of a persisting contact, one-step retention and decay,
  *                             layout invariants); the merged profile terms of the material key against the
