@@ -116,6 +116,12 @@ typedef struct nuka_template_desc_t {
     const float* profile_margin;     /* [profile][2] margin, gap; nullable => 0, 0 */
     uint32_t contact_cone;           /* <option cone>: 0 pyramidal (four edge rows a point), 1 elliptic */
     float contact_impratio;          /* <option impratio>; 0 => 1 */
+    /* How two sides' profiles merge (src/scene/contact_filter.hpp:89-137), read only when struct_size covers them */
+    const int32_t* profile_priority; /* [profile] the higher priority gives friction and condim and all of the mixing
+                                        weight; nullable => 0 */
+    const float* profile_solmix;     /* [profile] mixing weight at equal priority; nullable => 1 */
+    const uint32_t* profile_condim;  /* [profile] 3: a normal and two friction rows a point; 1: the normal alone;
+                                        nullable => 3 */
 } nuka_template_desc_t;
 
 /* The world options of the cooked-template creator (the library's own descriptor; the reference's nuka_world_desc_t

@@ -226,6 +226,8 @@ class Scene:
                       shape_conaffinity=nb, shape_group=nb, shape_profile=nb, profile_mu=2 * npf, joint_limit_lower=nl,
                       profile_law=npf if d.profile_law else 0, profile_solref=2 * npf if d.profile_solref else 0,
                       profile_solimp=5 * npf if d.profile_solimp else 0, profile_margin=2 * npf if d.profile_margin else 0,
+                      profile_priority=npf if d.profile_priority else 0, profile_solmix=npf if d.profile_solmix else 0,
+                      profile_condim=npf if d.profile_condim else 0,
                       joint_limit_upper=nl, joint_limit_flags=nl, joint_frictionloss=nl, excluded_pairs=2 * d.excluded_pair_count)
         out = {name: np.ctypeslib.as_array(getattr(d, name), shape=(count,)).copy() if count else np.zeros(0, np.float32)
                for name, count in shapes.items()}

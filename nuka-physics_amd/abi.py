@@ -47,6 +47,7 @@ class TemplateDescC(C.Structure):
         ("excluded_pairs", _PU), ("excluded_pair_count", C.c_uint32), ("reserved1", C.c_uint32),
         ("profile_law", _PU), ("profile_solref", _PF), ("profile_solimp", _PF), ("profile_margin", _PF),
         ("contact_cone", C.c_uint32), ("contact_impratio", C.c_float),
+        ("profile_priority", C.POINTER(C.c_int32)), ("profile_solmix", _PF), ("profile_condim", _PU),
     ]
 
 
@@ -135,11 +136,11 @@ class Template:
         return len(self.links) - 1
 
     def add_profile(self, mu1, mu2=None, law=LAW_NATIVE, solref=(0.02, 1.0), solimp=(0.9, 0.95, 0.001, 0.5, 2.0), margin=0.0,
-                    gap=0.0):
+                    gap=0.0, priority=0, solmix=1.0, condim=3):
         """A contact profile; `law`, `solref`, `solimp`, `margin` and `gap` matter to MuJoCo-law contacts only
         (scene/contact_filter.hpp:20-37 holds the defaults)."""
         self.profiles.append(dict(mu=(mu1, mu1 if mu2 is None else mu2), law=law, solref=tuple(solref), solimp=tuple(solimp),
-                                  margin=(margin, gap)))
+                                  margin=(margin, gap), priority=priority, solmix=solmix, condim=condim))
         return len(self.profiles) - 1
 
     def add_body(self, role, link=None, kind=SHAPE_NONE, params=(0, 0, 0, 0), local_pos=(0, 0, 0),
@@ -195,6 +196,9 @@ class Template:
             profile_solref=np.array([p["solref"] for p in self.profiles], dtype=f32).reshape(-1),
             profile_solimp=np.array([p["solimp"] for p in self.profiles], dtype=f32).reshape(-1),
             profile_margin=np.array([p["margin"] for p in self.profiles], dtype=f32).reshape(-1),
+            profile_priority=np.array([p["priority"] for p in self.profiles], dtype=np.int32),
+            profile_solmix=np.array([p["solmix"] for p in self.profiles], dtype=f32),
+            profile_condim=np.array([p["condim"] for p in self.profiles], dtype=u32),
             excluded_pairs=np.array(self.excluded, dtype=u32).reshape(-1),
         )
 
@@ -208,7 +212,7 @@ class Template:
         d.drive_mode, d.drive_rows = self.drive_mode, 1 if self.drive_rows else 0
         d.excluded_pair_count = len(self.excluded)
         d.contact_cone, d.contact_impratio = self.contact_cone, self.contact_impratio
-        ctype = {np.dtype(np.float32): C.c_float, np.dtype(np.uint32): C.c_uint32, np.dtype(np.uint8): C.c_uint8}
+        ctype = {np.dtype(np.float32): C.c_float, np.dtype(np.uint32): C.c_uint32, np.dtype(np.uint8): C.c_uint8, np.dtype(np.int32): C.c_int32}
         for name, arr in a.items():
             arr = np.ascontiguousarray(arr)
             a[name] = arr

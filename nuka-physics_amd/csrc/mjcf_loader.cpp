@@ -48,7 +48,8 @@ struct GeomDefaults : Frame {
     float friction[3] = {1.0f, 0.005f, 0.0001f};
     float solref[2] = {0.02f, 1.0f};
     float solimp[5] = {0.9f, 0.95f, 0.001f, 0.5f, 2.0f};
-    float margin = 0.0f, gap = 0.0f;
+    float margin = 0.0f, gap = 0.0f, solmix = 1.0f;
+    long priority = 0, condim = 3;
     float density = 1000.0f, mass = -1.0f;
 };
 struct GeneralDefaults {
@@ -107,6 +108,9 @@ void ApplyGeomAttributes(const Element& e, GeomDefaults* g) {
     ParseFloats(e.Attribute("solimp"), g->solimp, 5);
     QueryFloat(e, "margin", &g->margin);
     QueryFloat(e, "gap", &g->gap);
+    QueryFloat(e, "solmix", &g->solmix);
+    QueryInt(e, "priority", &g->priority);
+    QueryInt(e, "condim", &g->condim);
     QueryFloat(e, "density", &g->density);
     QueryFloat(e, "mass", &g->mass);
 }
@@ -291,6 +295,14 @@ struct Builder : SceneParts {
             ParseFloats(e.Attribute("solimp"), g.solimp, 5);
             QueryFloat(e, "margin", &g.margin);
             QueryFloat(e, "gap", &g.gap);
+            long priority = gd.priority, condim = gd.condim;
+            g.solmix = gd.solmix;
+            QueryFloat(e, "solmix", &g.solmix);
+            QueryInt(e, "priority", &priority);
+            QueryInt(e, "condim", &condim);
+            g.priority = int32_t(priority);
+            // torsional and rolling friction (condim 4, 6) have no rows here: such a geom keeps its sliding friction
+            g.condim = condim == 1 ? 1u : 3u;
             float density = gd.density, geom_mass = gd.mass;
             QueryFloat(e, "density", &density);
             QueryFloat(e, "mass", &geom_mass);
@@ -630,6 +642,7 @@ void FlattenScene(const SceneParts& b, uint32_t flags, uint32_t drive_mode, Scen
             bool same = s.profile_mu[2u * i] == g.friction && s.profile_law[i] == law && s.profile_solref[2u * i] == g.solref[0] &&
                         s.profile_solref[2u * i + 1u] == g.solref[1] && s.profile_margin[2u * i] == g.margin && s.profile_margin[2u * i + 1u] == g.gap;
             for (size_t k = 0u; k < 5u; ++k) same = same && s.profile_solimp[5u * i + k] == g.solimp[k];
+            same = same && s.profile_priority[i] == g.priority && s.profile_solmix[i] == g.solmix && s.profile_condim[i] == g.condim;
             if (same) return uint32_t(i);
         }
         s.profile_mu.push_back(g.friction); s.profile_mu.push_back(g.friction);
@@ -637,6 +650,7 @@ void FlattenScene(const SceneParts& b, uint32_t flags, uint32_t drive_mode, Scen
         s.profile_solref.push_back(g.solref[0]); s.profile_solref.push_back(g.solref[1]);
         for (float v : g.solimp) s.profile_solimp.push_back(v);
         s.profile_margin.push_back(g.margin); s.profile_margin.push_back(g.gap);
+        s.profile_priority.push_back(g.priority); s.profile_solmix.push_back(g.solmix); s.profile_condim.push_back(g.condim);
         any_friction_profile = true;
         return uint32_t(s.profile_law.size() - 1u);
     };
@@ -736,6 +750,7 @@ void Scene::Bind() {
     if (!profile_law.empty()) {   // a loader that authors no law leaves every profile native
         desc.profile_law = profile_law.data(); desc.profile_solref = profile_solref.data();
         desc.profile_solimp = profile_solimp.data(); desc.profile_margin = profile_margin.data();
+        desc.profile_priority = profile_priority.data(); desc.profile_solmix = profile_solmix.data(); desc.profile_condim = profile_condim.data();
     }
     desc.contact_cone = contact_cone;
     desc.contact_impratio = contact_impratio;

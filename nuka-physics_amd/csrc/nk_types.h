@@ -110,6 +110,7 @@ struct ModelView {
     const float* profile_solref;      // [profile][2]
     const float* profile_solimp;      // [profile][5]
     const float* profile_margin;      // [profile][2] margin, gap
+    const float* profile_mix;         // [profile][3] priority, solmix, condim
     const uint64_t* excluded_pairs;   // sorted (a << 32 | b) keys of collidable rows that never pair, a < b
 };
 

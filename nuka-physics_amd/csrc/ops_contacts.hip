@@ -744,38 +744,54 @@ __device__ uint64_t contact_material_key(float mu1, float mu2, uint32_t law) {
     return h;
 }
 
-// The same hash of any merged profile (mu1, mu2, solref[2], solimp[5], margin, gap; condim 3, no friction slope),
-// then the law word for the velocity-only laws and the cone for the compliant law (:620-623).
-__device__ uint64_t merged_material_key(const float (&merged)[11], uint32_t law, uint32_t cone) {
+// The same hash of any merged profile (mu1, mu2, solref[2], solimp[5], margin, gap, condim; no friction slope), then
+// the law word for the velocity-only laws and the cone for the compliant law (:620-623).
+__device__ uint64_t merged_material_key(const float (&merged)[12], uint32_t law, uint32_t cone) {
     uint64_t h = 0x4e554b4150524f46ull;
     h = profile_word(h, 2u);
     h = profile_word(h, 1u);
     h = profile_word(h, __float_as_uint(merged[0])); h = profile_word(h, __float_as_uint(merged[1]));
     h = profile_word(h, __float_as_uint(0.005f)); h = profile_word(h, __float_as_uint(0.0001f));
     for (int i = 2; i < 11; ++i) h = profile_word(h, __float_as_uint(merged[i]));
-    h = profile_word(h, 3u);
+    h = profile_word(h, uint32_t(merged[11]));
     if (h == 0ull) h = 0x9e3779b97f4a7c15ull;
     if (law == kContactLawVelocity || law == kContactLawSpeculative) { h ^= uint64_t{law}; h *= 1099511628211ull; }
     if (law == kContactLawCompliant) { h ^= uint64_t{cone}; h *= 1099511628211ull; }
     return h;
 }
-// One shape's contact parameters as the merge takes them: mu1, mu2, solref[2], solimp[5], margin, gap; a shape without
-// a profile has the defaults of scene/contact_filter.hpp:20-37.
-__device__ void profile_terms(const ModelView& m, uint32_t profile, float (&out)[11]) {
+// One shape's contact parameters as the merge takes them: mu1, mu2, solref[2], solimp[5], margin, gap, priority,
+// solmix, condim; a shape without a profile has the defaults of scene/contact_filter.hpp:20-37.
+__device__ void profile_terms(const ModelView& m, uint32_t profile, float (&out)[14]) {
     out[0] = 1.0f; out[1] = 1.0f; out[2] = 0.02f; out[3] = 1.0f; out[4] = 0.9f; out[5] = 0.95f; out[6] = 0.001f; out[7] = 0.5f; out[8] = 2.0f;
-    out[9] = 0.0f; out[10] = 0.0f;
+    out[9] = 0.0f; out[10] = 0.0f; out[11] = 0.0f; out[12] = 1.0f; out[13] = 3.0f;
     if (profile >= m.profile_count) return;
     out[0] = m.profile_mu[2u * profile]; out[1] = m.profile_mu[2u * profile + 1u];
     out[2] = m.profile_solref[2u * profile]; out[3] = m.profile_solref[2u * profile + 1u];
     for (uint32_t k = 0u; k < 5u; ++k) out[4u + k] = m.profile_solimp[5u * profile + k];
     out[9] = m.profile_margin[2u * profile]; out[10] = m.profile_margin[2u * profile + 1u];
+    for (uint32_t k = 0u; k < 3u; ++k) out[11u + k] = m.profile_mix[3u * profile + k];
 }
-// MergeContactParams (scene/contact_filter.hpp:100-137) at equal priority and mixing weight: friction by max, solref
-// mixed half and half (or the minimum when either is in direct form), solimp mixed, margins and gaps added.
-__device__ void merge_contact_params(const float (&a)[11], const float (&b)[11], float (&out)[11]) {
-    const float mix = 1.0f / (1.0f + 1.0f), imix = 1.0f - mix;
-    out[0] = a[0] > b[0] ? a[0] : b[0];
-    out[1] = a[1] > b[1] ? a[1] : b[1];
+// MergeContactParams (scene/contact_filter.hpp:89-137) with arithmetic friction mixing: the side of higher priority
+// gives friction and condim and all of the mixing weight; at equal priority friction and condim take the larger and
+// the weight is solmix_a / (solmix_a + solmix_b), a side whose solmix is below 1e-15 deferring to the other.  solref
+// is mixed, or the minimum when either is in direct form; solimp is mixed; margins and gaps add.
+__device__ void merge_contact_params(const float (&a)[14], const float (&b)[14], float (&out)[12]) {
+    float mix;
+    if (a[11] != b[11]) {
+        const bool first = a[11] > b[11];
+        mix = first ? 1.0f : 0.0f;
+        out[11] = first ? a[13] : b[13]; out[0] = first ? a[0] : b[0]; out[1] = first ? a[1] : b[1];
+    } else {
+        out[11] = a[13] > b[13] ? a[13] : b[13];
+        out[0] = a[0] > b[0] ? a[0] : b[0];
+        out[1] = a[1] > b[1] ? a[1] : b[1];
+        const bool a_ok = a[12] >= 1e-15f, b_ok = b[12] >= 1e-15f;
+        if (a_ok && b_ok) mix = a[12] / (a[12] + b[12]);
+        else if (!a_ok && !b_ok) mix = 0.5f;
+        else if (!a_ok) mix = 0.0f;
+        else mix = 1.0f;
+    }
+    const float imix = 1.0f - mix;
     if (a[2] > 0.0f && b[2] > 0.0f) { out[2] = mix * a[2] + imix * b[2]; out[3] = mix * a[3] + imix * b[3]; }
     else { out[2] = a[2] < b[2] ? a[2] : b[2]; out[3] = a[3] < b[3] ? a[3] : b[3]; }
     for (int i = 0; i < 5; ++i) out[4 + i] = mix * a[4 + i] + imix * b[4 + i];
@@ -921,7 +937,7 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
         // the two sides' profiles merged (:540-594; scene/contact_filter.hpp:100-137); a side without one has the defaults
         const uint32_t law = d.ucontact_law[gid];
         const bool mujoco = law == kContactLawCompliant;   // :480
-        float side_a[11], side_b[11], merged[11];
+        float side_a[14], side_b[14], merged[12];
         profile_terms(m, sa.profile, side_a); profile_terms(m, sb.profile, side_b);
         merge_contact_params(side_a, side_b, merged);
         if (mujoco) { merged[0] = fmaxf(1.0e-5f, merged[0]); merged[1] = fmaxf(1.0e-5f, merged[1]); }   // :573-576
@@ -937,7 +953,8 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
             const uint32_t weight_b = kind_b == kSideArtic ? m.link_body[link_b - env * nl] : local_b;
             invweight = (weight_a < m.bodies_per_env ? weights[2u * weight_a] : 0.0f) + (weight_b < m.bodies_per_env ? weights[2u * weight_b] : 0.0f);
         }
-        const bool pyramidal = mujoco && m.contact_cone == 0u;   // condim 3 (:598)
+        const bool friction_rows = merged[11] == 3.0f;   // condim 3: a normal and two tangents, else the normal alone (:721, 763)
+        const bool pyramidal = mujoco && m.contact_cone == 0u && friction_rows;   // :598
         const float impratio = m.contact_impratio;
         V3 frame_axis{0, 0, 0};   // :601-605: a capsule on a plane aligns the pyramid with the capsule's axis
         if (pyramidal && sa.kind == 1u && sb.kind == 3u) frame_axis = make_prim(sa, load_xf(d.body_pose + (size_t{env} * m.bodies_per_env + local_a) * 7u)).cz;
@@ -961,6 +978,7 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
             }
             // a pyramid has four scalar rows a point along n +- mu t (:651-690); the other cones a normal and two tangents
             const uint32_t row_count = pyramidal ? 4u : 3u;
+            const bool emits[2] = {live, live && friction_rows};   // the normal row; the tangent rows
             CompliantRow edge{};
             float edge_invweight = 0.0f;
             if (pyramidal) {
@@ -977,7 +995,7 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
                 const uint32_t rs = row_of[axis];
                 lambda[rs] = 0.0f; pen[rs] = 0.0f; cj_link[rs] = kInvalid; cj_link_b[rs] = kInvalid;
                 row_gain[rs] = 0.0f;
-                if (!live) {
+                if (!(pyramidal ? live : emits[axis == 0u ? 0 : 1])) {
                     if (pyramidal) rows[rs] = Row{}; else rows[rs].flags = 0u;
                     continue;
                 }
@@ -1004,7 +1022,7 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
                     const float clearance = roundoff > 0.0 ? nextafterf(float(roundoff), FLT_MAX) : 0.0f;
                     const float depth = d0 + clearance;
                     pen[rs] = mujoco ? fmaxf(d0, 0.0f) : depth;
-                    row.flags = kRowActive | kRowContactNormal | kRowBlockNormal | (mujoco ? uint32_t(kRowMuJoCo) : uint32_t(kRowSpeculative));
+                    row.flags = kRowActive | kRowContactNormal | (friction_rows ? uint32_t(kRowBlockNormal) : 0u) | (mujoco ? uint32_t(kRowMuJoCo) : uint32_t(kRowSpeculative));
                     row.rhs = (fminf(depth, 0.0f) + (p.position_pass != 0u ? 0.0f
                                : fminf(fmaxf(d0, 0.0f), p.overlap_recovery_velocity * p.dt))) / (p.dt * p.dt);
                     if (mujoco) {   // :714-731: the spring-damper reference of the merged solref / solimp at this depth

@@ -297,7 +297,9 @@ struct Geom {
     // the MuJoCo contact law's terms of the geom (src/import/mjcf_importer.cpp:162-165, 1009-1015)
     float solref[2] = {0.02f, 1.0f};
     float solimp[5] = {0.9f, 0.95f, 0.001f, 0.5f, 2.0f};
-    float margin = 0.0f, gap = 0.0f;
+    float margin = 0.0f, gap = 0.0f, solmix = 1.0f;
+    int32_t priority = 0;
+    uint32_t condim = 3u;
 };
 struct Link {
     std::string name, joint_name;

@@ -33,8 +33,9 @@ struct Scene {
         excluded_pairs;   // [pair][2] collidable rows that never pair
     std::vector<float> joint_axis, link_local_pose, link_inertial_frame, link_mass, link_diag_inertia, joint_damping, joint_armature,
         joint_stiffness, joint_spring_reference, joint_frictionloss, joint_limit_lower, joint_limit_upper, body_local, shape_params, profile_mu,
-        profile_solref, profile_solimp, profile_margin;
-    std::vector<uint32_t> profile_law;
+        profile_solref, profile_solimp, profile_margin, profile_solmix;
+    std::vector<uint32_t> profile_law, profile_condim;
+    std::vector<int32_t> profile_priority;
     uint32_t contact_cone = 0u;      // <option cone>: 0 pyramidal (MuJoCo's default), 1 elliptic
     float contact_impratio = 1.0f;   // <option impratio>
     std::vector<float> initial_q, drive_stiffness, drive_damping, drive_force_limit, drive_joint_force_limit;

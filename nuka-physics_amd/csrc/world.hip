@@ -66,7 +66,7 @@ struct HostModel {
     std::vector<uint64_t> link_dof_mask, excluded_pairs;
     std::vector<float> joint_axis, parent_offset, link_local_pose, link_inertial_frame, link_inertia, joint_damping, joint_armature,
         joint_stiffness, joint_spring_reference, joint_limit_lower, joint_limit_upper, joint_frictionloss, link_geom_local, shape_table, body_collidable_local, body_init_pose, profile_mu,
-        profile_solref, profile_solimp, profile_margin;
+        profile_solref, profile_solimp, profile_margin, profile_mix;   // profile_mix: [profile][3] priority, solmix, condim
     std::vector<uint32_t> profile_law;
     std::vector<float> link_mass, link_diag_inertia;   // kept for nuka_world_set_param: a new mass rebuilds the spatial inertia
 };
@@ -167,6 +167,12 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
             m.profile_solref[2u * i + 1u] = d.profile_solref != nullptr ? d.profile_solref[2u * i + 1u] : 1.0f;
             for (uint32_t k = 0u; k < 5u; ++k) m.profile_solimp[5u * i + k] = d.profile_solimp != nullptr ? d.profile_solimp[5u * i + k] : solimp[k];
             for (uint32_t k = 0u; k < 2u; ++k) if (d.profile_margin != nullptr) m.profile_margin[2u * i + k] = d.profile_margin[2u * i + k];
+            m.profile_mix.push_back(d.profile_priority != nullptr ? float(d.profile_priority[i]) : 0.0f);
+            m.profile_mix.push_back(d.profile_solmix != nullptr ? d.profile_solmix[i] : 1.0f);
+            m.profile_mix.push_back(d.profile_condim != nullptr ? float(d.profile_condim[i]) : 3.0f);
+            if (d.profile_condim != nullptr && d.profile_condim[i] != 1u && d.profile_condim[i] != 3u)
+                throw NotSupported("contact dimensions other than 1 and 3 (torsional and rolling friction) are not built on this path");
+            if (!std::isfinite(m.profile_mix[3u * i + 1u]) || std::fabs(m.profile_mix[3u * i]) > 16777216.0f) throw std::invalid_argument("invalid profile solmix or priority");
             if (m.profile_law[i] > 1u) throw std::invalid_argument("unknown profile law");
             for (uint32_t k = 0u; k < 2u; ++k) if (!std::isfinite(m.profile_solref[2u * i + k]) || !std::isfinite(m.profile_margin[2u * i + k])) throw std::invalid_argument("invalid profile solref or margin");
             for (uint32_t k = 0u; k < 5u; ++k) if (!std::isfinite(m.profile_solimp[5u * i + k])) throw std::invalid_argument("invalid profile solimp");
@@ -327,7 +333,8 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(link_dof, kU32) X(dof_link, kU32) X(dof_component, kU32) X(link_dof_mask, kU64) X(link_geom_kind, kU32) \
     X(link_geom_local, kF32) X(shape_table, kF32) X(body_to_link, kU32) X(body_to_articulation, kU32) \
     X(body_collidable_link, kU32) X(body_collidable_body, kU32) X(body_collidable_local, kF32) X(profile_mu, kF32) \
-    X(profile_law, kU32) X(profile_solref, kF32) X(profile_solimp, kF32) X(profile_margin, kF32) X(excluded_pairs, kU64)
+    X(profile_law, kU32) X(profile_solref, kF32) X(profile_solimp, kF32) X(profile_margin, kF32) X(profile_mix, kF32) \
+    X(excluded_pairs, kU64)
 
 uint32_t DtypeBytes(Dtype t) { return t == kU64 ? 8u : t == kU8 ? 1u : 4u; }
 
@@ -748,9 +755,10 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
     constexpr size_t kTemplateBase = offsetof(nuka_template_desc_t, joint_limit_lower);
     constexpr size_t kTemplateJointRows = offsetof(nuka_template_desc_t, excluded_pairs);
     constexpr size_t kTemplateExcluded = offsetof(nuka_template_desc_t, profile_law);
+    constexpr size_t kTemplateLaw = offsetof(nuka_template_desc_t, profile_priority);
     constexpr size_t kWorldBase = offsetof(nuka_hip_world_desc_t, solver_fold_drive_damping);
     constexpr size_t kWorldDrives = offsetof(nuka_hip_world_desc_t, solver_substeps);
-    if ((tmpl->struct_size != sizeof(nuka_template_desc_t) && tmpl->struct_size != kTemplateExcluded && tmpl->struct_size != kTemplateJointRows &&
+    if ((tmpl->struct_size != sizeof(nuka_template_desc_t) && tmpl->struct_size != kTemplateLaw && tmpl->struct_size != kTemplateExcluded && tmpl->struct_size != kTemplateJointRows &&
          tmpl->struct_size != kTemplateBase) ||
         (desc->struct_size != sizeof(nuka_hip_world_desc_t) && desc->struct_size != kWorldDrives && desc->struct_size != kWorldBase))
         return Error(NUKA_RESULT_INVALID_ARG, "struct_size mismatch");

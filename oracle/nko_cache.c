@@ -36,16 +36,16 @@ uint64_t nko_contact_material(float mu1, float mu2, uint32_t law) {
     return h;
 }
 
-/* The same hash of any merged profile (mu1, mu2, solref[2], solimp[5], margin, gap; condim 3, no friction slope),
+/* The same hash of any merged profile (mu1, mu2, solref[2], solimp[5], margin, gap, condim; no friction slope),
  * then the law word for the velocity and speculative laws and the cone for the compliant law (:620-623) */
-uint64_t nko_contact_material_merged(const float merged[11], uint32_t law, uint32_t cone) {
+uint64_t nko_contact_material_merged(const float merged[12], uint32_t law, uint32_t cone) {
     uint64_t h = 0x4e554b4150524f46ull;
     h = profile_word(h, 2u);
     h = profile_word(h, 1u);
     h = profile_word(h, bits(merged[0])); h = profile_word(h, bits(merged[1]));
     h = profile_word(h, bits(0.005f)); h = profile_word(h, bits(0.0001f));
     for (int i = 2; i < 11; ++i) h = profile_word(h, bits(merged[i]));
-    h = profile_word(h, 3u);
+    h = profile_word(h, (uint32_t)merged[11]);   /* condim */
     if (h == 0u) h = 0x9e3779b97f4a7c15ull;
     if (law == 1u || law == 2u) { h ^= (uint64_t)law; h *= 1099511628211ull; }
     if (law == 0u) { h ^= (uint64_t)cone; h *= 1099511628211ull; }

@@ -911,22 +911,37 @@ static void chain_jacobian_row(const nko_world* w, uint32_t env, uint32_t link_g
 
 /* One shape's contact parameters as MergeContactParams takes them: mu1, mu2, solref[2], solimp[5], margin, gap; a
  * shape without a profile has the defaults (assemble_rows.cu:41-52 DefaultProfile, mu 1). */
-static void profile_terms(const nko_template* t, uint32_t profile, float out[11]) {
-    const float defaults[11] = {1.0f, 1.0f, 0.02f, 1.0f, 0.9f, 0.95f, 0.001f, 0.5f, 2.0f, 0.0f, 0.0f};
+static void profile_terms(const nko_template* t, uint32_t profile, float out[14]) {
+    const float defaults[14] = {1.0f, 1.0f, 0.02f, 1.0f, 0.9f, 0.95f, 0.001f, 0.5f, 2.0f, 0.0f, 0.0f, 0.0f, 1.0f, 3.0f};
     memcpy(out, defaults, sizeof(defaults));
     if (profile >= t->n_profiles) return;
     out[0] = t->profile_mu[2u * profile]; out[1] = t->profile_mu[2u * profile + 1u];
     out[2] = t->profile_solref[2u * profile]; out[3] = t->profile_solref[2u * profile + 1u];
     for (uint32_t k = 0u; k < 5u; ++k) out[4u + k] = t->profile_solimp[5u * profile + k];
     out[9] = t->profile_margin[2u * profile]; out[10] = t->profile_margin[2u * profile + 1u];
+    for (uint32_t k = 0u; k < 3u; ++k) out[11u + k] = t->profile_mix[3u * profile + k];
 }
-/* scene/contact_filter.hpp:100-137 MergeContactParams at equal priority and solmix 1 on both sides (mix 1/2), arithmetic
- * friction mixing: friction by max, solref mixed (or the minimum when one is in direct form), solimp mixed, margins
- * and gaps added */
-void nko_merge_contact_params(const float a[11], const float b[11], float out[11]) {
-    const float mix = 1.0f / (1.0f + 1.0f), imix = 1.0f - mix;
-    out[0] = a[0] > b[0] ? a[0] : b[0];
-    out[1] = a[1] > b[1] ? a[1] : b[1];
+/* scene/contact_filter.hpp:89-137 MergeContactParams with arithmetic friction mixing: the side of higher priority gives
+ * friction and condim and all of the mixing weight; at equal priority friction and condim take the larger and the weight
+ * is solmix_a / (solmix_a + solmix_b), a side whose solmix is below mjMINVAL deferring to the other.  solref is mixed, or
+ * the minimum when either is in direct form; solimp is mixed; margins and gaps add. */
+void nko_merge_contact_params(const float a[14], const float b[14], float out[12]) {
+    float mix;
+    if (a[11] != b[11]) {
+        const float* w = a[11] > b[11] ? a : b;
+        mix = a[11] > b[11] ? 1.0f : 0.0f;
+        out[11] = w[13]; out[0] = w[0]; out[1] = w[1];
+    } else {
+        out[11] = a[13] > b[13] ? a[13] : b[13];
+        out[0] = a[0] > b[0] ? a[0] : b[0];
+        out[1] = a[1] > b[1] ? a[1] : b[1];
+        const int a_ok = a[12] >= 1e-15f, b_ok = b[12] >= 1e-15f;
+        if (a_ok && b_ok) mix = a[12] / (a[12] + b[12]);
+        else if (!a_ok && !b_ok) mix = 0.5f;
+        else if (!a_ok) mix = 0.0f;
+        else mix = 1.0f;
+    }
+    const float imix = 1.0f - mix;
     if (a[2] > 0.0f && b[2] > 0.0f) { out[2] = mix * a[2] + imix * b[2]; out[3] = mix * a[3] + imix * b[3]; }
     else { out[2] = a[2] < b[2] ? a[2] : b[2]; out[3] = a[3] < b[3] ? a[3] : b[3]; }
     for (int i = 0; i < 5; ++i) out[4 + i] = mix * a[4 + i] + imix * b[4 + i];
@@ -1086,28 +1101,23 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
         }
         if (kind_a == NKO_SIDE_STATIC) idx_a = NKO_INVALID;
         if (kind_b == NKO_SIDE_STATIC) idx_b = NKO_INVALID;
-        /* friction: per-shape profile or the default 1.0; equal priority mixes by max (contact_filter.hpp:58-62, 108-111) */
-        const float mu_a1 = sa.profile < t->n_profiles ? t->profile_mu[2u * sa.profile] : 1.0f;
-        const float mu_a2 = sa.profile < t->n_profiles ? t->profile_mu[2u * sa.profile + 1u] : 1.0f;
-        const float mu_b1 = sb.profile < t->n_profiles ? t->profile_mu[2u * sb.profile] : 1.0f;
-        const float mu_b2 = sb.profile < t->n_profiles ? t->profile_mu[2u * sb.profile + 1u] : 1.0f;
         const int position_pass = w->cfg.solver_pos_iters > 0u;
         const uint32_t law = w->ucontact_law[gid];
         const int mujoco = law == 0u;   /* kContactLawCompliant (:480) */
-        float mu1 = mu_a1 > mu_b1 ? mu_a1 : mu_b1, mu2 = mu_a2 > mu_b2 ? mu_a2 : mu_b2;
-        if (mujoco) { mu1 = fmaxf(1.0e-5f, mu1); mu2 = fmaxf(1.0e-5f, mu2); }   /* :573-576 */
-        /* the two sides' profiles merged (:540-594; contact_filter.hpp:100-137), a side without one at the defaults */
-        float side_a[11], side_b[11], merged[11];
+        /* the two sides' profiles merged (:540-594; contact_filter.hpp:89-137), a side without one at the defaults */
+        float side_a[14], side_b[14], merged[12];
         profile_terms(t, sa.profile, side_a); profile_terms(t, sb.profile, side_b);
         nko_merge_contact_params(side_a, side_b, merged);
-        if (mujoco) { merged[0] = mu1; merged[1] = mu2; }   /* the clamp above is part of what the material key hashes */
+        if (mujoco) { merged[0] = fmaxf(1.0e-5f, merged[0]); merged[1] = fmaxf(1.0e-5f, merged[1]); }   /* :573-576 */
+        const float mu1 = merged[0], mu2 = merged[1];
+        const int friction_rows = merged[11] == 3.0f;   /* condim 3: a normal and two tangents, else the normal alone (:721, 763) */
         const float* solref = merged + 2, *solimp = merged + 4;
         const float margin = merged[9];
         const uint32_t weight_a = kind_a == NKO_SIDE_ARTIC ? t->link_body[link_a - env * t->nl] : local_a;
         const uint32_t weight_b = kind_b == NKO_SIDE_ARTIC ? t->link_body[link_b - env * t->nl] : local_b;
         const float* invweight0 = w->body_invweight0 + (size_t)env * t->nb * 2u;
         const float invweight = mujoco ? invweight0[2u * weight_a] + invweight0[2u * weight_b] : 0.0f;   /* :597 */
-        const int pyramidal = mujoco && t->cone == 0u;   /* condim 3 (:598) */
+        const int pyramidal = mujoco && t->cone == 0u && friction_rows;   /* :598 */
         const float impratio = t->impratio;
         v3 frame_axis = v3_make(0, 0, 0);   /* :601-605: a capsule on a plane aligns the pyramid with the capsule's axis */
         if (pyramidal && sa.kind == 1u && sb.kind == 3u) frame_axis = nko_prim_rotate(xform_load(w->body_pose + ((size_t)env * t->nb + local_a) * 7u).r, v3_make(0, 0, 1));
@@ -1175,7 +1185,7 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
                     const float clearance = roundoff > 0.0 ? nextafterf((float)roundoff, FLT_MAX) : 0.0f;
                     const float depth = d0 + clearance;
                     pen[normal_row] = mujoco ? fmaxf(d0, 0.0f) : depth;
-                    row.flags = NKO_ROW_ACTIVE | NKO_ROW_CONTACT_NORMAL | NKO_ROW_BLOCK_NORMAL | (mujoco ? NKO_ROW_MUJOCO : NKO_ROW_SPECULATIVE);
+                    row.flags = NKO_ROW_ACTIVE | NKO_ROW_CONTACT_NORMAL | (friction_rows ? NKO_ROW_BLOCK_NORMAL : 0u) | (mujoco ? NKO_ROW_MUJOCO : NKO_ROW_SPECULATIVE);
                     row.group_first = env * R + base; row.group_normal_count = P; row.env = env;
                     row.rhs = (fminf(depth, 0.0f) + (position_pass ? 0.0f : fminf(fmaxf(d0, 0.0f), w->cfg.solver_overlap_recovery_velocity * dt))) / (dt * dt);
                     row.compliance_alpha = 0.0f;   /* DiscretizeCompliantRow of a zero row: R = 0 (solref_solimp.hpp:40-44) */
@@ -1204,7 +1214,7 @@ void nko_env_assemble_rows(nko_world* w, uint32_t env) {
                 nko_row row; memset(&row, 0, sizeof(row));
                 row.a.kind = row.b.kind = NKO_SIDE_STATIC; row.a.index = row.b.index = NKO_INVALID;
                 lambda[rs] = 0.0f; pen[rs] = 0.0f; cj_link[rs] = NKO_INVALID; cj_link_b[rs] = NKO_INVALID;
-                if (live) {
+                if (live && friction_rows) {
                     const v3 dir = tdir[k];
                     row.flags = NKO_ROW_ACTIVE | NKO_ROW_BLOCK_TANGENT;
                     row.group_first = env * R + base; row.group_normal_count = P; row.env = env;

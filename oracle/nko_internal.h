@@ -82,6 +82,7 @@ typedef struct {
     float* profile_mu;            /* n_profiles*2 */
     /* MuJoCo-law profiles (scene_ir.hpp:116; contact_filter.hpp:20-37): law source, solref, solimp, margin and gap */
     uint32_t* profile_law;        /* n_profiles */
+    float* profile_mix;           /* n_profiles*3: priority, solmix, condim */
     float* profile_solref;        /* n_profiles*2 */
     float* profile_solimp;        /* n_profiles*5 */
     float* profile_margin;        /* n_profiles*2 */

@@ -89,7 +89,9 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
     t->profile_mu = ALLOC(float, t->n_profiles * 2u);
     if (t->n_profiles) memcpy(t->profile_mu, d->profile_mu, t->n_profiles * 2u * sizeof(float));
     {   /* MuJoCo-law profile terms, defaults of ContactParamsIn (contact_filter.hpp:20-37) where not authored */
-        const int has = d->struct_size >= sizeof(nko_template_desc);
+        const int has = d->struct_size >= offsetof(nko_template_desc, profile_priority);
+        const int has_mix = d->struct_size >= sizeof(nko_template_desc);
+        t->profile_mix = ALLOC(float, t->n_profiles * 3u);
         t->profile_law = ALLOC(uint32_t, t->n_profiles); t->profile_solref = ALLOC(float, t->n_profiles * 2u);
         t->profile_solimp = ALLOC(float, t->n_profiles * 5u); t->profile_margin = ALLOC(float, t->n_profiles * 2u);
         const float solimp[5] = {0.9f, 0.95f, 0.001f, 0.5f, 2.0f};
@@ -99,6 +101,9 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
             t->profile_solref[2u * i + 1u] = has && d->profile_solref ? d->profile_solref[2u * i + 1u] : 1.0f;
             for (uint32_t k = 0u; k < 5u; ++k) t->profile_solimp[5u * i + k] = has && d->profile_solimp ? d->profile_solimp[5u * i + k] : solimp[k];
             for (uint32_t k = 0u; k < 2u; ++k) t->profile_margin[2u * i + k] = has && d->profile_margin ? d->profile_margin[2u * i + k] : 0.0f;
+            t->profile_mix[3u * i] = has_mix && d->profile_priority ? (float)d->profile_priority[i] : 0.0f;
+            t->profile_mix[3u * i + 1u] = has_mix && d->profile_solmix ? d->profile_solmix[i] : 1.0f;
+            t->profile_mix[3u * i + 2u] = has_mix && d->profile_condim ? (float)d->profile_condim[i] : 3.0f;
             t->any_mujoco = t->any_mujoco || t->profile_law[i] == 1u;
         }
         t->cone = has ? d->contact_cone : 0u;
@@ -206,7 +211,7 @@ static void free_template(nko_template* t) {
     free(t->link_geom_local); free(t->link_geom_kind); free(t->shape_table); free(t->excluded_pairs); free(t->body_to_link);
     free(t->body_to_articulation); free(t->body_collidable_link); free(t->body_collidable_body);
     free(t->body_collidable_local); free(t->body_init_pose); free(t->profile_mu);
-    free(t->profile_law); free(t->profile_solref); free(t->profile_solimp); free(t->profile_margin);
+    free(t->profile_mix); free(t->profile_law); free(t->profile_solref); free(t->profile_solimp); free(t->profile_margin);
 }
 
 nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc* desc) {

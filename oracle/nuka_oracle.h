@@ -110,6 +110,9 @@ typedef struct nko_template_desc {
     const float* profile_margin;
     uint32_t contact_cone;
     float contact_impratio;
+    const int32_t* profile_priority;
+    const float* profile_solmix;
+    const uint32_t* profile_condim;
 } nko_template_desc;
 
 typedef struct nko_world_desc {
@@ -164,10 +167,10 @@ void nko_world_step(nko_world* w);
  * once at the template's rest pose. */
 void nko_reference_weights(nko_world* w);
 void nko_snapshot_step_velocity(nko_world* w);
-/* scene/contact_filter.hpp:100-137 MergeContactParams of two profiles of equal priority and solmix:
- * out = mu1, mu2, solref[2], solimp[5], margin, gap */
-void nko_merge_contact_params(const float a[11], const float b[11], float out[11]);
-uint64_t nko_contact_material_merged(const float merged[11], uint32_t law, uint32_t cone);
+/* scene/contact_filter.hpp:100-137 MergeContactParams.  A side is mu1, mu2, solref[2], solimp[5], margin, gap, priority,
+ * solmix, condim; out = mu1, mu2, solref[2], solimp[5], margin, gap, condim */
+void nko_merge_contact_params(const float a[14], const float b[14], float out[12]);
+uint64_t nko_contact_material_merged(const float merged[12], uint32_t law, uint32_t cone);
 
 /* Stand-alone pieces exposed for unit pins. */
 void nko_make_spatial_inertia(float mass, const float diag[3], const float inertial_frame[7], float out[36]);

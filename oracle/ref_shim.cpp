@@ -180,22 +180,23 @@ void ref_merged_profile(float mu_a, float mu_b, float* out) {
     out[15] = m.solreffriction[0]; out[16] = m.solreffriction[1];
 }
 
-// MergeContactParams of two profiles of equal priority and solmix, packed mu1 mu2 solref[2] solimp[5] margin gap
+// MergeContactParams of two profiles packed mu1 mu2 solref[2] solimp[5] margin gap priority solmix condim; out without
+// priority and solmix
 void ref_merge_params(const float* pa, const float* pb, float* out) {
     scene::ContactParamsIn a, b;
     const float* in[2] = {pa, pb};
     scene::ContactParamsIn* side[2] = {&a, &b};
     for (int s = 0; s < 2; ++s) {
         side[s]->mu1 = in[s][0]; side[s]->mu2 = in[s][1];
-        side[s]->friction_mu = in[s][0];
         side[s]->solref[0] = in[s][2]; side[s]->solref[1] = in[s][3];
         for (int i = 0; i < 5; ++i) side[s]->solimp[i] = in[s][4 + i];
         side[s]->margin = in[s][9]; side[s]->gap = in[s][10];
+        side[s]->priority = int32_t(in[s][11]); side[s]->solmix = in[s][12]; side[s]->condim = uint8_t(in[s][13]);
     }
     const auto m = scene::MergeContactParams(a, b);
     out[0] = m.mu1; out[1] = m.mu2; out[2] = m.solref[0]; out[3] = m.solref[1];
     for (int i = 0; i < 5; ++i) out[4 + i] = m.solimp[i];
-    out[9] = m.margin; out[10] = m.gap;
+    out[9] = m.margin; out[10] = m.gap; out[11] = float(m.condim);
 }
 
 int ref_shape_filter_admits(uint32_t ta, uint32_t aa, uint32_t ga, uint32_t tb, uint32_t ab, uint32_t gb) {

@@ -203,3 +203,53 @@ def test_resting_spheres_sink_to_the_depth_of_the_spring_reference(oracle_py, de
         lo, hi = (mid, hi) if terms[5] / terms[4] < force else (lo, mid)
     assert np.abs(depth / (0.5 * (lo + hi)) - 1.0).max() < 0.03
     world.close()
+
+
+@pytest.mark.parametrize("law", [abi.LAW_NATIVE, abi.LAW_MUJOCO])
+def test_priority_solmix_and_frictionless_profiles(oracle_py, device, law):
+    """The merge's other branches on the device: the plane and the feet carry different profiles - a higher priority on
+    one side, unequal solmix on equal priority, a direct-form solref, condim 1 - and every merged outcome (material key,
+    row flags and terms, the steps that follow) matches the oracle."""
+    E = 16
+    variants = [dict(priority=2), dict(solmix=3.0, solref=(0.05, 0.7)), dict(solref=(-400.0, -30.0)), dict(condim=1), dict(priority=1, condim=1)]
+    for variant in variants:
+        cfg = nk.synthetic.config(2, E)
+        t = cfg.template
+        feet = dict(t.profiles[0])
+        feet.update(law=law, mu=(0.5, 0.5), solref=(0.03, 1.1), solimp=(0.8, 0.9, 0.002, 0.5, 2.0), margin=(0.002, 0.0))
+        feet.update(variant)
+        t.profiles[0].update(law=law, mu=(0.9, 0.9))
+        t.profiles.append(feet)
+        for body in t.bodies:
+            if body["kind"] == abi.SHAPE_SPHERE:
+                body["profile"] = 1
+        t.contact_cone = abi.CONE_ELLIPTIC
+        desc = abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters)
+        oracle = oracle_py.OracleWorld(t, desc, threads=8)
+        world = nk.World(device, t, desc)
+        state = cfg.state()
+        state["base_pose"][:, 2] -= 0.12
+        oracle.set_state(state); world.set_state(state)
+        for name in UPSTREAM:
+            oracle.op(*ORACLE_OPS[name])
+            world.op(name)
+        world.synchronize()
+        R = world.rows_per_env
+        assert np.array_equal(world.download("contact_material"), oracle.download("contact_material")), variant
+        got = world.download("urows").view(np.uint32).reshape(E, R, ROW_WORDS)
+        expect = oracle.download("urows").view(np.uint32).reshape(E, R, ROW_WORDS)
+        assert np.array_equal(got[:, :, [0, 1, 2, 3, 10, 11, 18, 19]], expect[:, :, [0, 1, 2, 3, 10, 11, 18, 19]]), variant
+        active = (expect[:, :, 0] & 1) != 0
+        assert active.sum() >= E
+        # condim 1 prevails only from the side of higher priority; at equal priority the larger condim does
+        frictionless = variant.get("condim") == 1 and variant.get("priority", 0) > 0
+        assert (((expect[:, :, 0] & ((1 << 2) | (1 << 3)))[active] == 0).all()) == frictionless
+        for word in (4, 5, 8, 9):
+            a = np.where(active, got.view(np.float32)[:, :, word], 0.0)
+            b = np.where(active, expect.view(np.float32)[:, :, word], 0.0)
+            assert per_env_error(a, b, E).max() <= TOL, (variant, word)
+        oracle.step(4); world.step(4); world.synchronize()
+        assert np.array_equal(world.download("env_status"), oracle.download("env_status")) and (oracle.download("env_status") == 0).all()
+        for name in ("q", "qdot", "link_velocity"):
+            close(world, oracle, name, tol=5e-4)
+        oracle.close(); world.close()

@@ -289,6 +289,8 @@ def test_contact_filtering_fixture_of_the_reference():
     assert np.array_equal(margin[p_default], np.float32([0, 0])) and a["profile_mu"].reshape(-1, 2)[p_default][0] == 1.0
     assert np.array_equal(solref[p_class], np.float32([0.005, 0.5])) and a["shape_profile"][explicit + 3] == p_class
     assert a["contact_cone"] == abi.CONE_PYRAMIDAL and a["contact_impratio"] == 1.0
+    assert (a["profile_priority"][p_explicit], a["profile_solmix"][p_explicit], a["profile_condim"][p_explicit]) == (5, np.float32(0.5), 1)
+    assert (a["profile_priority"][p_default], a["profile_solmix"][p_default], a["profile_condim"][p_default]) == (0, 1.0, 3)
     # with the native law kept, only an authored friction makes a profile
     native = nk.Scene(os.path.join(GOLDEN, "contact_filtering.xml"), nk.SCENE_NATIVE_CONTACT_LAW).template_arrays()
     assert native["shape_profile"][explicit + 1] == abi.INVALID and (native["profile_law"] == abi.LAW_NATIVE).all()

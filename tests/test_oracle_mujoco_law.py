@@ -20,29 +20,53 @@ def farr(values):
 
 
 def test_profile_merge_matches_the_reference(oracle_py, ref_lib):
-    """MergeContactParams (scene/contact_filter.hpp:100-137) at equal priority and solmix, the reference's own header
-    beside the restatement; direct-form (non-positive) solref entries take the minimum branch."""
+    """MergeContactParams (scene/contact_filter.hpp:89-137), the reference's own header beside the restatement, on
+    random profiles: equal and different priorities, solmix weights down to the deferring zero, direct-form solref
+    (the minimum branch), condim 1 and 3; then the known answers of tests/scene/test_filter_precedence.cpp."""
     L = oracle_py.lib()
     g = np.random.default_rng(5)
-    for case in range(200):
+    for case in range(400):
         sides = []
         for _ in range(2):
             solref = g.uniform(0.005, 0.1, 2) if g.random() < 0.7 else -g.uniform(10.0, 500.0, 2)
+            solmix = 0.0 if g.random() < 0.15 else g.uniform(0.1, 2.0)
             sides.append(np.concatenate([g.uniform(0.1, 1.5, 2), solref, g.uniform(0.5, 0.99, 2), g.uniform(1e-4, 1e-2, 1),
-                                         g.uniform(0.1, 0.9, 1), g.uniform(1.0, 3.0, 1), g.uniform(0.0, 0.01, 2)]).astype(np.float32))
-        mine, theirs = (F * 11)(), (F * 11)()
+                                         g.uniform(0.1, 0.9, 1), g.uniform(1.0, 3.0, 1), g.uniform(0.0, 0.01, 2),
+                                         [g.integers(-1, 2), solmix, g.choice([1, 3])]]).astype(np.float32))
+        mine, theirs = (F * 12)(), (F * 12)()
         L.nko_merge_contact_params(farr(sides[0]), farr(sides[1]), mine)
         ref_lib.ref_merge_params(farr(sides[0]), farr(sides[1]), theirs)
         assert np.array_equal(np.array(mine[:], np.float32).view(np.uint32), np.array(theirs[:], np.float32).view(np.uint32)), case
-    # the known answers of tests/scene/test_filter_precedence.cpp:119-145 that do not depend on solmix
-    a = [1, 1, -3.0, -50.0, 0.9, 0.95, 0.001, 0.5, 2.0, 0, 0]
-    b = [1, 1, -5.0, -10.0, 0.9, 0.95, 0.001, 0.5, 2.0, 0, 0]
-    c = [1, 1, 0.2, 4.0, 0.9, 0.95, 0.001, 0.5, 2.0, 0, 0]
-    out = (F * 11)()
-    L.nko_merge_contact_params(farr(a), farr(b), out)
-    assert (out[2], out[3]) == (-5.0, -50.0)
-    L.nko_merge_contact_params(farr(c), farr(b), out)
-    assert (out[2], out[3]) == (-5.0, -10.0)
+
+    def merged(a, b):
+        out = (F * 12)()
+        L.nko_merge_contact_params(farr(a), farr(b), out)
+        return np.array(out[:], np.float32)
+
+    def side(mu=1.0, solref=(0.02, 1.0), solimp=(0.9, 0.95, 0.001, 0.5, 2.0), margin=0.0, gap=0.0, priority=0, solmix=1.0, condim=3):
+        return [mu, mu, *solref, *solimp, margin, gap, priority, solmix, condim]
+
+    # :37-74 equal priority: friction and condim by max, solref and solimp by solmix 1 : 3
+    m = merged(side(0.3, (0.1, 2.0), (0,) * 5, 0.01, 0.02, 2, 1.0, 3), side(0.7, (0.2, 4.0), (1,) * 5, 0.03, 0.05, 2, 3.0, 1))
+    assert m[0] == np.float32(0.7) and m[11] == 3
+    # (EXPECT_FLOAT_EQ there: four units in the last place)
+    assert m[2] == pytest.approx(0.175, rel=3e-7) and m[3] == np.float32(3.5) and (m[4:9] == np.float32(0.75)).all()
+    # :80-113 the higher priority supplies friction and condim and, through the weight, solref and solimp
+    hi = side(0.9, (0.07, 1.5), (0.1, 0.2, 0.3, 0.4, 0.5), 0.09, 0.08, 5, 1.0, 1)
+    lo = side(0.2, (0.5, 9.0), (0.99,) * 5, 0.001, 0.002, 1, 1.0, 3)
+    for m in (merged(hi, lo), merged(lo, hi)):
+        assert m[0] == np.float32(0.9) and m[11] == 1 and m[2] == np.float32(0.07) and m[3] == np.float32(1.5)
+        assert np.array_equal(m[4:9], np.float32([0.1, 0.2, 0.3, 0.4, 0.5]))
+    # :119-145 a direct-form solref on either side takes the elementwise minimum
+    assert tuple(merged(side(solref=(-3.0, -50.0)), side(solref=(-5.0, -10.0)))[2:4]) == (-5.0, -50.0)
+    assert tuple(merged(side(solref=(0.2, 4.0)), side(solref=(-5.0, -10.0)))[2:4]) == (-5.0, -10.0)
+    # :153-183 a zero solmix defers to the other side; two valid ones mix
+    a, b = side(solref=(0.1, 1.0), solimp=(0.9, 0.95, 0.001, 0.5, 2.0)), side(solref=(0.3, 9.0), solimp=(0.5, 0.95, 0.001, 0.5, 2.0), solmix=0.0)
+    for m in (merged(a, b), merged(b, a)):
+        assert m[2] == np.float32(0.1) and m[3] == np.float32(1.0) and m[4] == np.float32(0.9)
+    b[12] = 1.0
+    m = merged(a, b)
+    assert m[2] == np.float32(0.5 * np.float32(0.1) + 0.5 * np.float32(0.3)) and m[4] == np.float32(0.5 * np.float32(0.9) + 0.5 * np.float32(0.5))
 
 
 def weights_world(oracle_py, template, q=None, base=None):
@@ -312,3 +336,23 @@ def test_a_resting_sphere_sinks_to_the_depth_of_the_spring_reference(oracle_py, 
             hi = mid
     assert depth == pytest.approx(0.5 * (lo + hi), rel=0.03), (depth, lo)
     w.close()
+
+
+def test_frictionless_contacts_have_the_normal_row_alone(oracle_py):
+    """condim 1 (assemble_rows.cu:721, 763): the normal row is a single-axis head, no tangent rows; both laws."""
+    E = 2
+    for law, cone in ((abi.LAW_NATIVE, abi.CONE_PYRAMIDAL), (abi.LAW_MUJOCO, abi.CONE_PYRAMIDAL), (abi.LAW_MUJOCO, abi.CONE_ELLIPTIC)):
+        cfg = nk.synthetic.config(2, E)
+        for p in cfg.template.profiles:
+            p.update(law=law, condim=1)
+        cfg.template.contact_cone = cone
+        w, _ = assembled(oracle_py, cfg, E)
+        R = w.rows_per_env
+        flags = w.download("urows").view(np.uint32).reshape(E, R, ROW_WORDS)[:, :, 0]
+        active = flags[(flags & ACTIVE) != 0]
+        assert active.size >= E
+        assert ((active & (BLOCK_NORMAL | BLOCK_TANGENT | PYRAMIDAL)) == 0).all() and ((active & CONTACT_NORMAL) != 0).all()
+        assert (((active & MUJOCO) != 0) == (law == abi.LAW_MUJOCO)).all()
+        w.step(20)   # and the solve runs on such heads
+        assert (w.download("env_status") == 0).all()
+        w.close()
