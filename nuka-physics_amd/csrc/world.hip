@@ -11,6 +11,7 @@
 #include <cstring>
 #include <exception>
 #include <memory>
+#include <atomic>
 #include <mutex>
 #include <stdexcept>
 #include <string>
@@ -345,6 +346,7 @@ struct DeviceRecord {   // src/c_abi/internal.hpp:57-69
 
 struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
     DeviceRecord* device = nullptr;
+    uint64_t id = 0u;   // creation number, unique in the process
     nuka_phi_backend* backend = nullptr;
     const nuka_phi_backend_i* be = nullptr;
     HostModel host;
@@ -405,12 +407,23 @@ struct CheckpointSegments {
     char* live[kMaxCheckpointSegments];
     char* kept[kMaxCheckpointSegments];
 };
+// What nuka_world_set_param can change after creation (src/c_abi/checkpoint.cpp:18-24 keeps link_inertia and
+// joint_armature beside the state; here every live parameter), in the order of the parameter table: a few words a link,
+// held on the host.
+struct LiveParams {
+    std::vector<double> values;   // [parameter][element], flattened
+    bool operator==(const LiveParams& o) const { return values == o.values; }
+};
 struct Checkpoint {
     World* owner = nullptr;
+    uint64_t owner_id = 0u;        // the world's creation number: a destroyed world's address may be used again
+    uint64_t layout_hash = 0u;     // of the owner, taken at capture
     nuka_phi_buffer* store = nullptr;
     CheckpointSegments segments{};
     uint64_t bytes = 0u;
+    LiveParams params;
 };
+bool OwnedBy(const Checkpoint* cp, const World* w) { return cp->owner == w && cp->owner_id == w->id; }
 
 // blockIdx.y picks the segment, blockIdx.x strides over its 16-byte units.
 __global__ void __launch_bounds__(256) CheckpointCopyKernel(CheckpointSegments s, uint32_t restore) {
@@ -771,6 +784,8 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
     try {
         auto world = std::make_unique<World>();
         World& w = *world;
+        static std::atomic<uint64_t> created{0u};
+        w.id = ++created;
         w.device = reinterpret_cast<DeviceRecord*>(device);
         w.backend = reinterpret_cast<nuka_phi_backend*>(w.device->backend);
         w.be = reinterpret_cast<nuka_phi_backend_head*>(w.backend)->iface;
@@ -1345,7 +1360,7 @@ nuka_result_t nuka_world_time_steps(nuka_world_handle world, nuka_checkpoint_han
     auto* w = reinterpret_cast<World*>(world);
     if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
     if (out_total_ms == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
-    if (from != nullptr && reinterpret_cast<Checkpoint*>(from)->owner != w) return Error(NUKA_RESULT_INVALID_ARG, "checkpoint belongs to another world");
+    if (from != nullptr && !OwnedBy(reinterpret_cast<Checkpoint*>(from), w)) return Error(NUKA_RESULT_INVALID_ARG, "checkpoint belongs to another world");
     nuka_phi_event* start = w->be->event_new(w->backend);
     nuka_phi_event* stop = w->be->event_new(w->backend);
     if (start == nullptr || stop == nullptr) return Error(NUKA_RESULT_DEVICE_ERROR, "event creation failed");
@@ -1370,7 +1385,7 @@ nuka_result_t nuka_world_profile_ops(nuka_world_handle world, nuka_checkpoint_ha
     auto* w = reinterpret_cast<World*>(world);
     if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
     if (out_ms == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
-    if (from != nullptr && reinterpret_cast<Checkpoint*>(from)->owner != w) return Error(NUKA_RESULT_INVALID_ARG, "checkpoint belongs to another world");
+    if (from != nullptr && !OwnedBy(reinterpret_cast<Checkpoint*>(from), w)) return Error(NUKA_RESULT_INVALID_ARG, "checkpoint belongs to another world");
     const size_t n = w->calls.size();
     std::vector<nuka_phi_event*> events(n + 1u, nullptr);
     for (auto& e : events) e = w->be->event_new(w->backend);
@@ -1433,6 +1448,7 @@ nuka_result_t NewCheckpoint(World* w, std::unique_ptr<Checkpoint>* out) {
     auto cp = std::unique_ptr<Checkpoint>(new (std::nothrow) Checkpoint{});
     if (!cp) return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
     cp->owner = w;
+    cp->owner_id = w->id;
     size_t total = 0u;
     for (const Field& f : w->fields) {
         if (f.is_template || f.count == 0u || !(CheckpointKeeps(f.name) || CheckpointClears(f.name))) continue;
@@ -1480,8 +1496,45 @@ uint64_t CheckpointLayoutHash(const World& w) {
     }
     return hash;
 }
-struct CheckpointFileHeader { char magic[8]; uint64_t layout_hash, bytes; };
-constexpr char kCheckpointMagic[8] = {'N', 'K', 'H', 'C', 'K', 'P', 'T', '1'};
+struct CheckpointFileHeader { char magic[8]; uint64_t layout_hash, bytes, param_values; };
+constexpr char kCheckpointMagic[8] = {'N', 'K', 'H', 'C', 'K', 'P', 'T', '2'};
+
+// Every live parameter of the world as the public getters report it.
+nuka_result_t ReadLiveParams(World* w, LiveParams* out) {
+    out->values.clear();
+    uint32_t count = 0u;
+    if (const nuka_result_t r = nuka_world_param_count(reinterpret_cast<nuka_world_handle>(w), &count); r != NUKA_RESULT_OK) return r;
+    std::vector<nuka_param_info_t> infos(count);
+    for (auto& info : infos) { info.struct_size = sizeof(info); info.schema_version = NUKA_PARAM_INFO_VERSION; }
+    if (const nuka_result_t r = nuka_world_get_param_infos(reinterpret_cast<nuka_world_handle>(w), infos.data(), count); r != NUKA_RESULT_OK) return r;
+    for (uint32_t p = 0u; p < count; ++p)
+        for (uint32_t e = 0u; e < infos[p].count; ++e) {
+            double value = 0.0;
+            if (const nuka_result_t r = nuka_world_get_param(reinterpret_cast<nuka_world_handle>(w), p, e, &value); r != NUKA_RESULT_OK) return r;
+            out->values.push_back(value);
+        }
+    return NUKA_RESULT_OK;
+}
+// Brings the world's live parameters to `wanted` through the public setter (which keeps the device tables, the reset
+// snapshot and the host mirrors in step); nothing happens when they already agree, as on every restore of a
+// checkpoint taken since the last parameter change.
+nuka_result_t ApplyLiveParams(World* w, const LiveParams& wanted) {
+    LiveParams current;
+    if (const nuka_result_t r = ReadLiveParams(w, &current); r != NUKA_RESULT_OK) return r;
+    if (current == wanted) return NUKA_RESULT_OK;
+    if (current.values.size() != wanted.values.size()) return Error(NUKA_RESULT_INVALID_ARG, "the checkpoint holds another number of parameters");
+    uint32_t count = 0u;
+    if (const nuka_result_t r = nuka_world_param_count(reinterpret_cast<nuka_world_handle>(w), &count); r != NUKA_RESULT_OK) return r;
+    std::vector<nuka_param_info_t> infos(count);
+    for (auto& info : infos) { info.struct_size = sizeof(info); info.schema_version = NUKA_PARAM_INFO_VERSION; }
+    if (const nuka_result_t r = nuka_world_get_param_infos(reinterpret_cast<nuka_world_handle>(w), infos.data(), count); r != NUKA_RESULT_OK) return r;
+    size_t at = 0u;
+    for (uint32_t p = 0u; p < count; ++p)
+        for (uint32_t e = 0u; e < infos[p].count; ++e, ++at)
+            if (current.values[at] != wanted.values[at])
+                if (const nuka_result_t r = nuka_world_set_param(reinterpret_cast<nuka_world_handle>(w), p, e, wanted.values[at]); r != NUKA_RESULT_OK) return r;
+    return NUKA_RESULT_OK;
+}
 }  // namespace
 }  // namespace nkh
 
@@ -1497,6 +1550,8 @@ nuka_result_t nuka_world_checkpoint_capture(nuka_world_handle world, nuka_checkp
         Iface(cp->store)->free(cp->store);
         return Error(NUKA_RESULT_DEVICE_ERROR, "checkpoint capture failed");
     }
+    cp->layout_hash = CheckpointLayoutHash(*w);
+    if (const nuka_result_t r = ReadLiveParams(w, &cp->params); r != NUKA_RESULT_OK) { Iface(cp->store)->free(cp->store); return r; }
     *out = reinterpret_cast<nuka_checkpoint_handle>(cp.release());
     return NUKA_RESULT_OK;
 }
@@ -1511,11 +1566,13 @@ nuka_result_t nuka_checkpoint_write(nuka_checkpoint_handle checkpoint, const cha
             return Error(NUKA_RESULT_DEVICE_ERROR, "checkpoint download failed");
         CheckpointFileHeader header{};
         std::memcpy(header.magic, kCheckpointMagic, sizeof(header.magic));
-        header.layout_hash = CheckpointLayoutHash(*cp->owner);
+        header.layout_hash = cp->layout_hash;   // taken at capture: the world may be gone by now
         header.bytes = cp->bytes;
+        header.param_values = cp->params.values.size();
         std::FILE* file = std::fopen(path, "wb");
         if (file == nullptr) return Error(NUKA_RESULT_INVALID_ARG, std::string("cannot open ") + path);
-        const bool ok = std::fwrite(&header, sizeof(header), 1u, file) == 1u && (bytes.empty() || std::fwrite(bytes.data(), bytes.size(), 1u, file) == 1u);
+        const bool ok = std::fwrite(&header, sizeof(header), 1u, file) == 1u && (bytes.empty() || std::fwrite(bytes.data(), bytes.size(), 1u, file) == 1u) &&
+                        (cp->params.values.empty() || std::fwrite(cp->params.values.data(), cp->params.values.size() * sizeof(double), 1u, file) == 1u);
         if (std::fclose(file) != 0 || !ok) return Error(NUKA_RESULT_INTERNAL, std::string("write failed: ") + path);
     } catch (const std::bad_alloc&) {
         return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
@@ -1544,6 +1601,13 @@ nuka_result_t nuka_world_checkpoint_read(nuka_world_handle world, const char* pa
                 result = Error(NUKA_RESULT_INVALID_ARG, "truncated checkpoint file");
             else if (!bytes.empty() && Iface(cp->store)->upload(cp->store, bytes.data(), 0u, bytes.size()) != uint8_t(Status::Ok))
                 result = Error(NUKA_RESULT_DEVICE_ERROR, "checkpoint upload failed");
+            if (result == NUKA_RESULT_OK) {
+                cp->layout_hash = header.layout_hash;
+                cp->params.values.resize(header.param_values < (1u << 24u) ? header.param_values : 0u);
+                if (cp->params.values.size() != header.param_values ||
+                    (!cp->params.values.empty() && std::fread(cp->params.values.data(), cp->params.values.size() * sizeof(double), 1u, file) != 1u))
+                    result = Error(NUKA_RESULT_INVALID_ARG, "truncated checkpoint file");
+            }
             if (result == NUKA_RESULT_OK && nuka_world_synchronize(world) != NUKA_RESULT_OK) result = NUKA_RESULT_DEVICE_ERROR;
             if (result != NUKA_RESULT_OK) Iface(cp->store)->free(cp->store);
             else *out = reinterpret_cast<nuka_checkpoint_handle>(cp.release());
@@ -1578,7 +1642,8 @@ nuka_result_t nuka_world_checkpoint_restore(nuka_world_handle world, nuka_checkp
     auto* w = reinterpret_cast<World*>(world);
     auto* cp = reinterpret_cast<Checkpoint*>(checkpoint);
     if (w == nullptr || cp == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world or checkpoint is null");
-    if (cp->owner != w) return Error(NUKA_RESULT_INVALID_ARG, "checkpoint belongs to another world");
+    if (!OwnedBy(cp, w)) return Error(NUKA_RESULT_INVALID_ARG, "checkpoint belongs to another world");
+    if (const nuka_result_t r = ApplyLiveParams(w, cp->params); r != NUKA_RESULT_OK) return r;
     hipLaunchKernelGGL(CheckpointCopyKernel, dim3(256, cp->segments.count), dim3(256), 0, BackendStream(w->device->backend), cp->segments, 1u);
     return hipGetLastError() == hipSuccess ? NUKA_RESULT_OK : Error(NUKA_RESULT_DEVICE_ERROR, "checkpoint restore failed");
 }
@@ -1613,7 +1678,7 @@ nuka_result_t nuka_checkpoint_equal(nuka_checkpoint_handle a, nuka_checkpoint_ha
         if (x->bytes > 0u && (Iface(x->store)->download(x->store, left.data(), 0u, x->bytes) != uint8_t(Status::Ok) ||
                               Iface(y->store)->download(y->store, right.data(), 0u, y->bytes) != uint8_t(Status::Ok)))
             return Error(NUKA_RESULT_DEVICE_ERROR, "checkpoint download failed");
-        *out_equal = left == right ? 1u : 0u;
+        *out_equal = left == right && x->params == y->params ? 1u : 0u;
     } catch (const std::bad_alloc&) {
         return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
     }
@@ -1648,6 +1713,9 @@ nuka_result_t nuka_world_state_hash(nuka_world_handle world, uint64_t* out_hash)
     } catch (const std::bad_alloc&) {
         return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
     }
+    LiveParams params;   // a world that differs in a live parameter alone is another state
+    if (const nuka_result_t r = ReadLiveParams(w, &params); r != NUKA_RESULT_OK) return r;
+    if (!params.values.empty()) mix(params.values.data(), params.values.size() * sizeof(double));
     *out_hash = hash;
     return NUKA_RESULT_OK;
 }

@@ -163,9 +163,33 @@ def test_pose_refresh_state_hash_and_checkpoint_equality(oracle_py, device):
     world.step(1)
     moved, other = world.checkpoint(), twin.checkpoint()
     assert not world.checkpoints_equal(kept, moved) and world.checkpoints_equal(kept, other)
-    for handle in (kept, again, moved, other):
+    # drive fields and live parameters are state too: a change moves the hash and a restore takes it back
+    base = world.checkpoint()
+    before = world.state_hash()
+    target = world.download("drive_target")
+    world.upload("drive_target", target + 0.25)
+    assert world.state_hash() != before
+    world.restore(base); world.synchronize()
+    assert world.state_hash() == before and np.array_equal(world.download("drive_target"), target)
+    mass, damping = world.get_param("link_mass", 2), world.get_param("joint_damping", 3)
+    world.set_param("link_mass", 2, 2.0 * mass)
+    world.set_param("joint_damping", 3, damping + 0.5)
+    changed = world.checkpoint()
+    assert world.state_hash() != before and not world.checkpoints_equal(base, changed)
+    world.restore(base); world.synchronize()
+    assert world.get_param("link_mass", 2) == mass and world.get_param("joint_damping", 3) == damping
+    assert world.state_hash() == before
+    world.step(2)
+    twin.restore(twin.checkpoint()); twin.set_state(state); twin.forward_kinematics()
+    # a checkpoint of a world that is gone, or of another world, is refused by address and creation number
+    stale = twin.checkpoint()
+    twin.close()
+    fresh = nk.World(device, cfg.template, desc)
+    assert nk.lib().nuka_world_checkpoint_restore(fresh._h, stale) == abi.RESULT_INVALID_ARG
+    assert nk.lib().nuka_world_checkpoint_restore(world._h, stale) == abi.RESULT_INVALID_ARG
+    for handle in (kept, again, moved, other, base, changed, stale):
         nk.lib().nuka_checkpoint_destroy(handle)
-    for w in (world, twin, oracle):
+    for w in (world, fresh, oracle):
         w.close()
 
 
@@ -189,10 +213,11 @@ def test_checkpoint_files_and_execution_info(device, tmp_path):
     world.write_checkpoint(kept, path)
     size = C.c_uint64()
     nk.lib().nuka_checkpoint_byte_size(kept, C.byref(size))
-    assert path.stat().st_size == 24 + size.value
+    live_values = 2 + 6 * cfg.template.link_count            # gravity, sweeps, six per-link parameters
+    assert path.stat().st_size == 32 + size.value + 8 * live_values
     read = other.read_checkpoint(path)
-    other.set_velocity_iterations(5)
-    other.restore(read); other.synchronize()
+    other.restore(read); other.synchronize()               # the live parameters come with it: five sweeps
+    assert other.get_param("velocity_iterations") == 5
     assert other.state_hash() == world.state_hash()
     world.restore(kept)                                    # a restore also clears the solver's carried history: both start from it
     world.step(2); other.step(2)
