@@ -123,12 +123,23 @@ def cpu_baseline(nk, cfg, desc, budget_s=12.0):
             "sample": f"{steps} steps of the first {E} environments of the same seeded batch in {elapsed:.1f} s, gcc -O2 -fopenmp"}
 
 
-def measure(nk, device, index, envs, steps, warmup, mode, cpu_budget_s):
+def apply_contact_law(nk, cfg, law):
+    """`native` keeps the configuration as published; `elliptic` / `pyramidal` give every contact profile the MuJoCo law
+    with that cone (the contact law of an imported MJCF file)."""
+    if law == "native":
+        return
+    for profile in cfg.template.profiles:
+        profile["law"] = nk.abi.LAW_MUJOCO
+    cfg.template.contact_cone = nk.abi.CONE_ELLIPTIC if law == "elliptic" else nk.abi.CONE_PYRAMIDAL
+
+
+def measure(nk, device, index, envs, steps, warmup, mode, cpu_budget_s, law="native"):
     """One configuration: warm-up, the timed steps (wall clock around back-to-back submissions and one final
     synchronisation), device events on the launch stream, per-op device times, and what the batch did - live
     contacts, sweeps used, environments at the sweep cap, environments that raised a status bit."""
     import numpy as np
     cfg = nk.synthetic.config(index, envs or None)
+    apply_contact_law(nk, cfg, law)
     E = cfg.env_count
     desc = nk.abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters)
     world = nk.World(device, cfg.template, desc)
@@ -173,7 +184,8 @@ def measure(nk, device, index, envs, steps, warmup, mode, cpu_budget_s):
     out = {
         "value": E * 1e3 / wall_ms, "ms_per_step": wall_ms, "steps": steps, "warmup": warmup,
         "config": {"workload": f"{cfg.name}: {nl} links, {nv} DoF, {nc} contact spheres, {E} envs, dt {cfg.dt:.6f}, "
-                               f"{cfg.vel_iters} block-descent sweeps{live}", "config_index": index, "envs": E,
+                               f"{cfg.vel_iters} block-descent sweeps{live}" + ("" if law == "native" else f"; MuJoCo contact law, {law} cone"),
+                   "config_index": index, "envs": E,
                    "execution": mode, "event_ms_per_step": event_ms,
                    "each_step_from": "seeded batch (checkpoint restore inside the timed region)", **batch},
         "roofline": {"bound": "hbm", "kernel": kernel, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -202,6 +214,8 @@ def main():
     ap.add_argument("--envs", type=int, default=0)
     ap.add_argument("--mode", choices=("eager", "graph"), default="graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--contact-law", choices=("native", "elliptic", "pyramidal"), default="native",
+                    help="with --only: the configuration's contacts under the MuJoCo law with this cone instead of the native law")
     ap.add_argument("--only", action="store_true", help="the named configuration alone, without the short runs of the others")
     ap.add_argument("--seeded-only", action="store_true",
                     help="kept for the profile commands: every launch of a run is a step from the seeded batch")
@@ -218,7 +232,10 @@ def main():
         scene_run(nk, args)
         return
     device = nk.Device(0)
-    head = measure(nk, device, args.config, args.envs, args.steps, args.warmup, args.mode, 0.0 if args.no_cpu_baseline else 12.0)
+    if args.contact_law != "native" and not args.only:
+        sys.exit("bench.py: --contact-law goes with --only (the published configurations use the native law)")
+    head = measure(nk, device, args.config, args.envs, args.steps, args.warmup, args.mode, 0.0 if args.no_cpu_baseline else 12.0,
+                   args.contact_law)
     result = {
         "metric": "env-steps/sec", "value": head["value"], "unit": "env-steps/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True,
