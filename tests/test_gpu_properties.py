@@ -209,6 +209,39 @@ def test_single_environment_and_contact_free_worlds(oracle_py, device):
         oracle.close()
 
 
+@pytest.mark.parametrize("index", [2, 3])
+def test_a_non_finite_environment_is_flagged_and_alone(oracle_py, device, index):
+    """Environments that start from a coordinate, a velocity, a base height or a torque that is not a number raise
+    their own status word (as the oracle does) and change nothing in any other environment: every other environment's
+    state after three steps equals, bit for bit, that of a batch without them."""
+    E = 256
+    cfg = nk.synthetic.config(index, E)
+    desc = abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters)
+    clean, dirty, oracle = nk.World(device, cfg.template, desc), nk.World(device, cfg.template, desc), oracle_py.OracleWorld(cfg.template, desc, threads=8)
+    state = cfg.state()
+    clean.set_state(state)
+    bad = cfg.state()
+    bad["q"][7, 3] = np.nan
+    bad["qdot"][11, 2] = np.inf
+    bad["base_pose"][13, 2] = np.nan
+    bad["tau"][17, 4] = np.inf
+    poisoned = [7, 11, 13, 17]
+    dirty.set_state(bad)
+    oracle.set_state(bad)
+    for w in (clean, dirty, oracle):
+        w.step(3)
+    dirty.synchronize(); clean.synchronize()
+    status = dirty.download("env_status")
+    assert (status[poisoned] != 0).all() and np.array_equal(status[poisoned], oracle.download("env_status")[poisoned])
+    others = np.setdiff1d(np.arange(E), poisoned)
+    assert (status[others] == 0).all()
+    for name in ("q", "qdot", "base_pose", "link_velocity", "lambda"):
+        got, expect = dirty.download(name).reshape(E, -1), clean.download(name).reshape(E, -1)
+        assert np.array_equal(got[others].view(np.uint32), expect[others].view(np.uint32)), name
+    for w in (clean, dirty, oracle):
+        w.close()
+
+
 def box_template(plane_first):
     t = abi.Template()
     t.add_link(abi.JOINT_FLOATING, None, mass=1.2, diag_inertia=(0.004, 0.006, 0.005))
