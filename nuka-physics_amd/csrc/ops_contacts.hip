@@ -1149,7 +1149,8 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
             mode = component < 3u ? 3u : 4u;
         }
     }
-    const uint32_t bound = min(contact_row_bound(previous_extent, extent, CR), CR);
+    // only the rows below this step's extent can have a link; the rows up to the previous extent were cleared above
+    const uint32_t bound = min(extent - 1u, CR);
     const float start_velocity = m.any_mujoco != 0u && lane < md ? d.step_qdot_flat[size_t{env} * md + lane] : 0.0f;
     for (uint32_t r = 0u; r < bound; ++r) {
         const uint32_t links[2] = {row_link_a[r], row_link_b[r]};

@@ -1430,8 +1430,11 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     }
     PROF_BEGIN(c, 16);
     // ListTileHeads (:1250-1296): active rows that are not block tangents, in slot order
-    const uint32_t previous = d.contact_row_extent[2u * env], current = d.contact_row_extent[2u * env + 1u];
-    const uint32_t bound = previous == 0u || current == 0u ? p.contact_rows_per_env : min(max(previous, current) - 1u, p.contact_rows_per_env);
+    // The reference scans the rows below the larger of the last two row extents (all of them when either is unknown,
+    // as after a reset).  The rows between this step's extent and that bound were cleared by this step's row assembly
+    // and hold no head, so the scan stops at this step's extent: the same heads from a fraction of the row records.
+    const uint32_t current = d.contact_row_extent[2u * env + 1u];
+    const uint32_t bound = current == 0u ? p.contact_rows_per_env : min(current - 1u, p.contact_rows_per_env);
     const uint32_t total = bound + (R - p.contact_rows_per_env);
     uint32_t heads = 0u;
     bool overflow = false;
