@@ -122,6 +122,18 @@ typedef struct nuka_template_desc_t {
     const float* profile_solmix;     /* [profile] mixing weight at equal priority; nullable => 1 */
     const uint32_t* profile_condim;  /* [profile] 3: a normal and two friction rows a point; 1: the normal alone;
                                         nullable => 3 */
+    /* MuJoCo-sourced joints and integrator (src/scene/cook/cook_to_model.cpp:662-693; src/nk/pipeline/pipeline.cpp:264-265,
+     * 939-951), read only when struct_size covers them.  Such a joint's limit and dry-friction rows are compliant rows
+     * of its own solref / solimp (src/phi/backend_cuda/ops/assemble_rows.cu:860-877, 921-931). */
+    const uint8_t* joint_law;              /* [link] 0 native, 1 MuJoCo-sourced; nullable */
+    const float* joint_limit_margin;       /* [link]; nullable => 0 */
+    const float* joint_limit_reference;    /* [link][7] solref[2], solimp[5] of the limit rows; nullable => 0.02 1, 0.9 0.95 0.001 0.5 2 */
+    const float* joint_friction_reference; /* [link][7] of the dry-friction row; nullable => the same */
+    uint32_t integrator;                   /* 0 native (damping of drives folded into the solve); 1 MuJoCo's Euler: joint
+                                              damping applied implicitly after the solve, the step's velocity change
+                                              through (M + dt D)^-1 M; 2 implicit / implicitfast: the servos' velocity
+                                              gains join D */
+    uint32_t reserved2;
 } nuka_template_desc_t;
 
 /* The world options of the cooked-template creator (the library's own descriptor; the reference's nuka_world_desc_t
@@ -220,6 +232,11 @@ typedef struct nuka_scene_t* nuka_scene_handle;
  * MuJoCo-sourced, as in the reference's importer (src/import/mjcf_importer.cpp:790): its friction, solref, solimp,
  * margin and gap make a contact profile of the MuJoCo law, with the cone and impratio of <option>. */
 #define NUKA_SCENE_NATIVE_CONTACT_LAW 8u
+/* MJCF only: the joints keep the native limit and dry-friction rows and the native integrator.  Without it every joint is
+ * MuJoCo-sourced (src/import/mjcf_importer.cpp:1193, 1720): its limit rows are compliant rows of margin / solreflimit /
+ * solimplimit, its dry friction of solreffriction / solimpfriction, and joint damping is applied implicitly after the
+ * solve as <option integrator> says (Euler by default; implicit and implicitfast add the servos' velocity gains). */
+#define NUKA_SCENE_NATIVE_JOINT_LAW 16u
 nuka_result_t nuka_scene_load_mjcf(const char* path, uint32_t flags, nuka_scene_handle* out);
 nuka_result_t nuka_scene_load_urdf(const char* path, uint32_t flags, nuka_scene_handle* out);
 void nuka_scene_destroy(nuka_scene_handle scene);

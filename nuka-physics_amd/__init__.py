@@ -39,6 +39,7 @@ SCENE_PLANE_CONTACTS_ONLY = 1
 SCENE_FIXED_BASE = 2
 SCENE_GROUND_PLANE = 4
 SCENE_NATIVE_CONTACT_LAW = 8
+SCENE_NATIVE_JOINT_LAW = 16
 
 
 class ParamInfoC(C.Structure):
@@ -227,11 +228,13 @@ class Scene:
                       profile_law=npf if d.profile_law else 0, profile_solref=2 * npf if d.profile_solref else 0,
                       profile_solimp=5 * npf if d.profile_solimp else 0, profile_margin=2 * npf if d.profile_margin else 0,
                       profile_priority=npf if d.profile_priority else 0, profile_solmix=npf if d.profile_solmix else 0,
-                      profile_condim=npf if d.profile_condim else 0,
+                      profile_condim=npf if d.profile_condim else 0, joint_law=nl if d.joint_law else 0,
+                      joint_limit_margin=nl if d.joint_limit_margin else 0, joint_limit_reference=7 * nl if d.joint_limit_reference else 0,
+                      joint_friction_reference=7 * nl if d.joint_friction_reference else 0,
                       joint_limit_upper=nl, joint_limit_flags=nl, joint_frictionloss=nl, excluded_pairs=2 * d.excluded_pair_count)
         out = {name: np.ctypeslib.as_array(getattr(d, name), shape=(count,)).copy() if count else np.zeros(0, np.float32)
                for name, count in shapes.items()}
-        out.update(drive_mode=d.drive_mode, drive_rows=d.drive_rows, contact_cone=d.contact_cone, contact_impratio=d.contact_impratio)
+        out.update(drive_mode=d.drive_mode, drive_rows=d.drive_rows, contact_cone=d.contact_cone, contact_impratio=d.contact_impratio, integrator=d.integrator)
         return out
 
     def initial_state(self):

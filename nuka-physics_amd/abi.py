@@ -19,6 +19,9 @@ ROLE_STATIC, ROLE_LINK_BODY, ROLE_PROXY = 0, 1, 2
 # constraint/law_source.hpp: where a shape's contact law comes from; nk/solve/row_types.hpp cone of the MuJoCo law
 LAW_NATIVE, LAW_MUJOCO = 0, 1
 CONE_PYRAMIDAL, CONE_ELLIPTIC = 0, 1
+# the integrator of the step: native, MuJoCo's Euler (joint damping implicit after the solve), implicit / implicitfast
+INTEGRATOR_NATIVE, INTEGRATOR_MUJOCO_EULER, INTEGRATOR_MUJOCO_IMPLICIT = 0, 1, 2
+SOLVER_REFERENCE = (0.02, 1.0, 0.9, 0.95, 0.001, 0.5, 2.0)   # solref, solimp of constraint::SolverReference
 
 # phi/articulation_contract.hpp:16-23
 DRIVE_PD_POSITION, DRIVE_TORQUE, DRIVE_VELOCITY, DRIVE_COMPUTED_TORQUE, DRIVE_OSC, DRIVE_ACTUATOR = 0, 1, 2, 3, 4, 5
@@ -48,6 +51,8 @@ class TemplateDescC(C.Structure):
         ("profile_law", _PU), ("profile_solref", _PF), ("profile_solimp", _PF), ("profile_margin", _PF),
         ("contact_cone", C.c_uint32), ("contact_impratio", C.c_float),
         ("profile_priority", C.POINTER(C.c_int32)), ("profile_solmix", _PF), ("profile_condim", _PU),
+        ("joint_law", _PB), ("joint_limit_margin", _PF), ("joint_limit_reference", _PF), ("joint_friction_reference", _PF),
+        ("integrator", C.c_uint32), ("reserved2", C.c_uint32),
     ]
 
 
@@ -124,15 +129,18 @@ class Template:
         self.excluded = []        # pairs of collidable rows that never pair (rows of one link are excluded by the cook)
         self.contact_cone = CONE_PYRAMIDAL   # friction cone of MuJoCo-law contacts (<option cone>)
         self.contact_impratio = 1.0          # <option impratio>
+        self.integrator = INTEGRATOR_NATIVE  # <option integrator> of a MuJoCo-sourced scene
 
     def add_link(self, joint_type, parent, axis=(0, 0, 1), local_pos=(0, 0, 0), local_rot=(1, 0, 0, 0), mass=1.0,
                  diag_inertia=(0.01, 0.01, 0.01), com=(0, 0, 0), damping=0.0, armature=0.0, stiffness=0.0,
-                 spring_ref=0.0, parent_offset=(0, 0, 0), lower=None, upper=None, frictionloss=0.0):
+                 spring_ref=0.0, parent_offset=(0, 0, 0), lower=None, upper=None, frictionloss=0.0, law=LAW_NATIVE,
+                 limit_margin=0.0, limit_reference=SOLVER_REFERENCE, friction_reference=SOLVER_REFERENCE):
         self.links.append(dict(joint_type=joint_type, parent=INVALID if parent is None else parent, axis=axis,
                                local=list(local_pos) + list(local_rot), mass=mass, diag=diag_inertia,
                                inertial=list(com) + [1, 0, 0, 0], damping=damping, armature=armature,
                                stiffness=stiffness, spring_ref=spring_ref, parent_offset=parent_offset,
-                               lower=lower, upper=upper, frictionloss=frictionloss))
+                               lower=lower, upper=upper, frictionloss=frictionloss, law=law, limit_margin=limit_margin,
+                               limit_reference=tuple(limit_reference), friction_reference=tuple(friction_reference)))
         return len(self.links) - 1
 
     def add_profile(self, mu1, mu2=None, law=LAW_NATIVE, solref=(0.02, 1.0), solimp=(0.9, 0.95, 0.001, 0.5, 2.0), margin=0.0,
@@ -182,6 +190,10 @@ class Template:
             joint_limit_upper=np.array([0.0 if l["upper"] is None else l["upper"] for l in L], dtype=f32),
             joint_limit_flags=np.array([(l["lower"] is not None) + 2 * (l["upper"] is not None) for l in L], dtype=np.uint8),
             joint_frictionloss=np.array([l["frictionloss"] for l in L], dtype=f32),
+            joint_law=np.array([l["law"] for l in L], dtype=np.uint8),
+            joint_limit_margin=np.array([l["limit_margin"] for l in L], dtype=f32),
+            joint_limit_reference=np.array([l["limit_reference"] for l in L], dtype=f32).reshape(-1),
+            joint_friction_reference=np.array([l["friction_reference"] for l in L], dtype=f32).reshape(-1),
             body_role=np.array([b["role"] for b in B], dtype=u32),
             body_link=np.array([b["link"] for b in B], dtype=u32),
             body_local=np.array([b["local"] for b in B], dtype=f32).reshape(-1),
@@ -212,6 +224,7 @@ class Template:
         d.drive_mode, d.drive_rows = self.drive_mode, 1 if self.drive_rows else 0
         d.excluded_pair_count = len(self.excluded)
         d.contact_cone, d.contact_impratio = self.contact_cone, self.contact_impratio
+        d.integrator = self.integrator
         ctype = {np.dtype(np.float32): C.c_float, np.dtype(np.uint32): C.c_uint32, np.dtype(np.uint8): C.c_uint8, np.dtype(np.int32): C.c_int32}
         for name, arr in a.items():
             arr = np.ascontiguousarray(arr)

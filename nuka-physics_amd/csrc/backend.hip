@@ -50,6 +50,7 @@ void RegisterOps() {
     set(NkOp::ReadoutContactWrench, &OpReadoutContactWrench);
     set(NkOp::AccumulateStep, &OpAccumulateStep);
     set(NkOp::ReferenceWeights, &OpReferenceWeights);
+    set(NkOp::ArticulationDamping, &OpArticulationDamping);
 }
 
 void Fail(nuka_phi_execution_error* error, Status status, uint16_t op, int native, const char* message) {

@@ -34,6 +34,9 @@ struct JointDefaults {
     bool has_range = false;
     int limited = -1;
     float damping = 0.0f, armature = 0.0f, frictionloss = 0.0f, actuator_force_limit = 0.0f, stiffness = 0.0f, spring_reference = 0.0f;
+    float limit_margin = 0.0f;
+    float limit_reference[7] = {0.02f, 1.0f, 0.9f, 0.95f, 0.001f, 0.5f, 2.0f};      // solreflimit, solimplimit
+    float friction_reference[7] = {0.02f, 1.0f, 0.9f, 0.95f, 0.001f, 0.5f, 2.0f};   // solreffriction, solimpfriction
 };
 struct Frame {
     V3 position;
@@ -80,6 +83,11 @@ void ApplyJointAttributes(const Element& e, JointDefaults* j) {
     QueryFloat(e, "damping", &j->damping);
     QueryFloat(e, "armature", &j->armature);
     QueryFloat(e, "frictionloss", &j->frictionloss);
+    QueryFloat(e, "margin", &j->limit_margin);   // mjcf_importer.cpp:334-338, 1209-1213
+    ParseFloats(e.Attribute("solreflimit"), j->limit_reference, 2);
+    ParseFloats(e.Attribute("solimplimit"), j->limit_reference + 2, 5);
+    ParseFloats(e.Attribute("solreffriction"), j->friction_reference, 2);
+    ParseFloats(e.Attribute("solimpfriction"), j->friction_reference + 2, 5);
     ParseActuatorForceRange(e, &j->actuator_force_limit);
     QueryFloat(e, "stiffness", &j->stiffness);
     QueryFloat(e, "springref", &j->spring_reference);
@@ -423,6 +431,8 @@ struct Builder : SceneParts {
             link.joint_type = j.type == JointKind::Slide ? 1u : 0u;
             link.axis = j.axis;
             link.damping = j.damping; link.armature = j.armature; link.frictionloss = j.frictionloss;
+            link.limit_margin = j.limit_margin;
+            for (int i = 0; i < 7; ++i) { link.limit_reference[i] = j.limit_reference[i]; link.friction_reference[i] = j.friction_reference[i]; }
             link.stiffness = j.stiffness; link.spring_reference = j.spring_reference;
             link.actuator_force_limit = j.actuator_force_limit;
             link.lower = j.lower; link.upper = j.upper;
@@ -539,6 +549,7 @@ std::unique_ptr<Scene> LoadMjcf(const std::string& path, uint32_t flags) {
     b.context.flags = flags;
     auto scene = std::make_unique<Scene>();
     scene->timestep = 0.002f;   // MuJoCo's default
+    scene->integrator = 1u;     // Euler, MuJoCo's default: joint damping implicit after the solve (pipeline.cpp:264-265)
     scene->gravity[0] = 0.0f; scene->gravity[1] = 0.0f; scene->gravity[2] = -9.81f;
     if (const Element* option = mujoco->First("option")) {
         QueryFloat(*option, "timestep", &scene->timestep);
@@ -549,6 +560,13 @@ std::unique_ptr<Scene> LoadMjcf(const std::string& path, uint32_t flags) {
             else throw std::runtime_error("MJCF: invalid option cone");
         }
         QueryFloat(*option, "impratio", &scene->contact_impratio);
+        if (const char* integrator = option->Attribute("integrator")) {
+            const std::string name(integrator);
+            if (name == "Euler") scene->integrator = 1u;
+            else if (name == "implicit" || name == "implicitfast") scene->integrator = 2u;
+            else if (name == "RK4") throw Unsupported("MJCF: the RK4 integrator is not built on this path");
+            else throw std::runtime_error("MJCF: invalid option integrator");
+        }
     }
     if (const Element* compiler = mujoco->First("compiler")) {
         if (const char* angle = compiler->Attribute("angle")) {
@@ -591,6 +609,7 @@ std::unique_ptr<Scene> LoadMjcf(const std::string& path, uint32_t flags) {
     });
     uint32_t drive_mode = 1u;
     b.ParseActuators(*mujoco, &drive_mode);
+    if ((flags & kNativeJointLaw) != 0u) scene->integrator = 0u;
     FlattenScene(b, flags, drive_mode, scene.get());
     return scene;
 }
@@ -619,6 +638,10 @@ void FlattenScene(const SceneParts& b, uint32_t flags, uint32_t drive_mode, Scen
         s.joint_damping.push_back(k.damping); s.joint_armature.push_back(k.armature);
         s.joint_stiffness.push_back(k.stiffness); s.joint_spring_reference.push_back(k.spring_reference);
         s.joint_frictionloss.push_back(k.frictionloss);
+        s.joint_law.push_back((flags & kNativeJointLaw) != 0u ? 0u : 1u);
+        s.joint_limit_margin.push_back(k.limit_margin);
+        for (float v : k.limit_reference) s.joint_limit_reference.push_back(v);
+        for (float v : k.friction_reference) s.joint_friction_reference.push_back(v);
         s.joint_limit_lower.push_back(k.limited ? k.lower : 0.0f); s.joint_limit_upper.push_back(k.limited ? k.upper : 0.0f);
         s.joint_limit_flags.push_back(k.limited ? 3u : 0u);
         s.initial_q.push_back(k.initial_position);
@@ -754,6 +777,11 @@ void Scene::Bind() {
     }
     desc.contact_cone = contact_cone;
     desc.contact_impratio = contact_impratio;
+    if (!joint_law.empty()) {
+        desc.joint_law = joint_law.data(); desc.joint_limit_margin = joint_limit_margin.data();
+        desc.joint_limit_reference = joint_limit_reference.data(); desc.joint_friction_reference = joint_friction_reference.data();
+    }
+    desc.integrator = integrator;
 }
 
 }  // namespace scene_file

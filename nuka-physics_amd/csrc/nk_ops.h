@@ -28,6 +28,7 @@ Status OpBlockDescentSolve(const ModelView&, const DataView&, const void*, hipSt
 Status OpReadoutDrives(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpReadoutContactWrench(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpAccumulateStep(const ModelView&, const DataView&, const void*, hipStream_t);
+Status OpArticulationDamping(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpReferenceWeights(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpSnapshotStepVelocity(const ModelView&, const DataView&, const void*, hipStream_t);
 

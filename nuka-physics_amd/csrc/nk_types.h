@@ -74,6 +74,7 @@ struct ModelView {
     // the MuJoCo contact law: some profile is MuJoCo-sourced; the cone of its contacts (0 pyramidal, 1 elliptic) and impratio
     uint32_t any_mujoco, contact_cone;
     float contact_impratio;
+    uint32_t integrator;   // 0 native; 1, 2: ArticulationDamping follows the solve (2: with the servos' velocity gains)
     const uint8_t* joint_type;
     const uint32_t* parent_link;
     const float* joint_axis;
@@ -89,6 +90,10 @@ struct ModelView {
     const float* joint_limit_upper;
     const float* joint_frictionloss;
     const uint8_t* joint_limit_flags;   // bit 0: lower bound authored, bit 1: upper
+    const uint8_t* joint_law;           // 1: MuJoCo-sourced joint rows
+    const float* joint_limit_margin;
+    const float* joint_limit_reference;     // [link][7] solref, solimp
+    const float* joint_friction_reference;  // [link][7]
     const uint32_t* link_body;
     const uint32_t* link_tree_depth;
     const uint32_t* link_child_range;
@@ -199,6 +204,15 @@ struct ReferenceWeightsParams {   // op_schema.hpp:123-130
     uint32_t articulations_per_env;
     uint32_t bodies_per_env;
     uint32_t total_body_count;
+};
+struct ArticulationDampingParams {   // op_schema.hpp:132-141
+    float dt;
+    uint32_t max_dof;
+    uint32_t articulation_count;
+    uint32_t total_link_count;
+    uint32_t actuator_derivative;
+    uint32_t mode;
+    uint32_t readout_drives = 0u;
 };
 struct IntegrateVelocityParams {   // op_schema.hpp:143-150
     float dt;

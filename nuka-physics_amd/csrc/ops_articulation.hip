@@ -687,6 +687,92 @@ Status OpReferenceWeights(const ModelView& m, const DataView& d, const void* par
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 
+namespace {
+// ActuatorVelocityDerivative (articulation.cu:942-948): what a servo's effort changes per unit joint velocity, none
+// while its own force limit clamps it
+__device__ float actuator_velocity_derivative(const DataView& d, uint32_t mode, size_t link) {
+    if (d.drive_force_limit[link] > 0.0f && fabsf(d.drive_command[link] - d.joint_gravity_force[link]) > d.drive_force_limit[link]) return 0.0f;
+    return mode == kDrivePdPosition ? d.drive_damping[link] : mode == kDriveVelocity ? d.drive_stiffness[link] : 0.0f;
+}
+
+// ArticulationDampingKernel (articulation.cu:950-1000), one wavefront an environment: contacts were solved with the plain
+// mass; the step's velocity change now goes through (M + dt D)^-1 M, D the joint damping and, for the implicit
+// integrators, the unclamped servo velocity gains.  M + dt D is factored as L D L^T in LDS, lane = row; every entry takes
+// its pivots' updates in pivot order (FactorMass, articulation_mass.cuh:269-335), and the solve runs forward by
+// columns, divides, and substitutes back serially (SolveMassBlock :357-396).
+__global__ void __launch_bounds__(kWave) ArticulationDampingKernel(ModelView m, DataView d, ArticulationDampingParams p) {
+    extern __shared__ float lds[];
+    const uint32_t env = blockIdx.x, lane = threadIdx.x, n = m.dof, stride = m.max_dof, nl = m.links_per_env, ld = n + 1u;
+    float* A = lds;               // n x (n + 1)
+    float* change = A + n * ld;   // n
+    const size_t lbase = size_t{env} * nl, base = size_t{env} * stride;
+    const bool coordinate = lane < n;
+    uint32_t link = 0u, component = kInvalid;
+    float value = 0.0f, velocity = 0.0f, damping = 0.0f;
+    if (coordinate) {
+        link = m.dof_link[lane]; component = m.dof_component[lane];
+        const bool scalar = component == kInvalid;
+        value = scalar ? m.joint_damping[link] : 0.0f;
+        if (scalar && p.actuator_derivative != 0u) value += actuator_velocity_derivative(d, p.mode, lbase + link);
+        velocity = scalar ? d.qdot[lbase + link] : d.link_velocity[(lbase + link) * 6u + component];
+        damping = p.dt * value;
+        change[lane] = damping * (velocity - d.step_qdot_flat[base + lane]);
+    }
+    if (!__any(coordinate && value != 0.0f)) return;
+    if (coordinate)
+        for (uint32_t j = 0u; j <= lane; ++j) A[lane * ld + j] = d.m[(base + lane) * stride + j] + (j == lane ? damping : 0.0f);
+    for (uint32_t k = 0u; k < n; ++k) {
+        __syncthreads();
+        const float diagonal = fmaxf(A[k * ld + k], 1.0e-6f);
+        __syncthreads();
+        float l = 0.0f;
+        if (coordinate && lane > k) { l = A[lane * ld + k] / diagonal; A[lane * ld + k] = l; }
+        if (lane == k) A[k * ld + k] = diagonal;
+        __syncthreads();
+        if (coordinate && lane > k)
+            for (uint32_t j = k + 1u; j <= lane; ++j) A[lane * ld + j] -= l * A[j * ld + k] * diagonal;
+    }
+    for (uint32_t j = 0u; j < n; ++j) {   // forward by columns
+        __syncthreads();
+        const float solved = change[j];
+        if (coordinate && lane > j) change[lane] -= A[lane * ld + j] * solved;
+    }
+    __syncthreads();
+    if (coordinate) change[lane] = change[lane] / A[lane * ld + lane];
+    __syncthreads();
+    if (lane == 0u)
+        for (uint32_t end = n; end > 0u; --end) {
+            const uint32_t i = end - 1u;
+            float sum = change[i];
+            for (uint32_t j = i + 1u; j < n; ++j) sum -= A[j * ld + i] * change[j];
+            change[i] = sum;
+        }
+    __syncthreads();
+    if (!coordinate) return;
+    velocity -= change[lane];
+    if (component == kInvalid) d.qdot[lbase + link] = velocity; else d.link_velocity[(lbase + link) * 6u + component] = velocity;
+    d.qdot_flat[base + lane] = velocity;
+    if (component == kInvalid && p.actuator_derivative != 0u && p.readout_drives != 0u) {
+        const float derivative = actuator_velocity_derivative(d, p.mode, lbase + link);
+        const float correction = derivative * (velocity - d.step_qdot_flat[base + lane]);
+        d.actuator_effort_requested[lbase + link] -= correction;
+        d.actuator_effort[lbase + link] -= correction;
+        d.tau[lbase + link] -= correction;
+    }
+}
+}  // namespace
+
+// ArticulationDamping (op_schema.hpp:132-141): the op a MuJoCo integrator adds after the constraint solve.
+Status OpArticulationDamping(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
+    const auto* p = static_cast<const ArticulationDampingParams*>(params);
+    if (p == nullptr) return Status::Failed;
+    if (p->articulation_count == 0u || p->total_link_count == 0u || m.dof == 0u) return Status::Ok;
+    if (m.dof > kMaxDof || p->max_dof != m.max_dof || p->total_link_count != p->articulation_count * m.links_per_env) return Status::InvalidArgument;
+    const size_t lds = size_t{m.dof} * (m.dof + 2u) * sizeof(float);
+    hipLaunchKernelGGL(ArticulationDampingKernel, dim3(p->articulation_count), dim3(kWave), lds, stream, m, d, *p);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
 Status OpIntegratePosition(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
     const auto* p = static_cast<const IntegratePositionParams*>(params);
     if (p == nullptr) return Status::Failed;

@@ -1072,7 +1072,7 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
             const uint32_t rs = CR + slot;
             Row row{};
             cj_link[rs] = kInvalid; cj_link_b[rs] = kInvalid; pen[rs] = 0.0f;
-            float jacobian = 0.0f, impulse = 0.0f;
+            float jacobian = 0.0f, impulse = 0.0f, joint_gain = 0.0f, joint_weight = 0.0f;
             uint32_t l;
             if (slot < limit_rows) {   // EmitJointLimitRow :805-882
                 l = slot / 2u;
@@ -1089,6 +1089,17 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
                     jacobian = side == 0u ? 1.0f : -1.0f;
                     pen[rs] = fmaxf(-signed_distance, 0.0f);
                     impulse = lambda[rs];   // an active limit row keeps its multiplier
+                    if (m.joint_law[l] == 1u) {   // :860-877: a compliant row inside its margin, on the nearer bound only
+                        const float pos = signed_distance - m.joint_limit_margin[l];
+                        const float* reference = m.joint_limit_reference + 7u * l;
+                        const float invweight = d.dof_invweight0[size_t{env} * md + m.link_dof[l]];
+                        const CompliantRow c = compliant_row(reference, reference + 2u, pos, pos, 0.0f, invweight, p.dt, p.refsafe);
+                        row.flags |= kRowMuJoCo;
+                        const bool lower_nearest = q - m.joint_limit_lower[l] < m.joint_limit_upper[l] - q;
+                        if (pos >= 0.0f || lower_nearest != (side == 0u)) { row.flags &= ~uint32_t(kRowActive); impulse = 0.0f; }
+                        row.rhs = c.bias; row.compliance_alpha = c.R;
+                        joint_gain = c.gain; joint_weight = invweight;
+                    }
                 }
             } else if (slot < limit_rows + friction_rows) {   // EmitJointFrictionRows :886-934
                 l = slot - limit_rows;
@@ -1097,6 +1108,14 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
                     row.flags = kRowActive | kRowVelocityOnly;
                     row.lower = -friction * p.dt; row.upper = friction * p.dt;
                     jacobian = 1.0f;
+                    if (m.joint_law[l] == 1u) {   // :921-931: dry friction regularised by its own solref / solimp
+                        const float* reference = m.joint_friction_reference + 7u * l;
+                        const float invweight = d.dof_invweight0[size_t{env} * md + m.link_dof[l]];
+                        const CompliantRow c = compliant_row(reference, reference + 2u, 0.0f, 0.0f, 0.0f, invweight, p.dt, p.refsafe);
+                        row.flags |= kRowMuJoCo;
+                        row.compliance_alpha = c.R;
+                        joint_gain = c.gain; joint_weight = invweight;
+                    }
                 }
             } else {   // EmitJointDriveRows :938-971
                 l = slot - limit_rows - friction_rows;
@@ -1111,7 +1130,14 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
             if (row.flags != 0u) {
                 row.group_first = env * R + rs; row.group_normal_count = 1u; row.env = env;
                 row.a.kind = kSideArtic; row.a.index = env;
-                ++active_rows;
+                if ((row.flags & kRowActive) != 0u) ++active_rows;
+                if ((row.flags & kRowMuJoCo) != 0u) {
+                    d.row_reference_velocity_gain[size_t{env} * R + rs] = joint_gain;
+                    d.row_invweight[size_t{env} * R + rs] = joint_weight;
+                    // PrepareContactRowsKernel (:1134-1140): the row's one entry times the start velocity of its coordinate
+                    if ((row.flags & kRowActive) != 0u)
+                        row.rhs += joint_gain * (0.0f + jacobian * d.step_qdot_flat[size_t{env} * md + m.link_dof[l]]);
+                }
             }
             lambda[rs] = impulse;
             if (joint_dof(m.joint_type[l]) == 1u) d.chain_jacobian[(size_t{env} * R + rs) * md + m.link_dof[l]] = jacobian;
@@ -1612,12 +1638,12 @@ __global__ void __launch_bounds__(256) SnapshotStepVelocityKernel(ModelView m, D
 }  // namespace
 
 // SnapshotStepVelocity (assemble_rows.cu:1457-1477): the generalized velocity the step starts from.  Only the
-// compliant rows of the MuJoCo contact law read it (PrepareContactRowsKernel :1134-1140), so a world without a
-// MuJoCo-sourced profile has nothing to record.
+// compliant rows of the MuJoCo law read it (PrepareContactRowsKernel :1134-1140) and the damping a MuJoCo integrator
+// applies after the solve, so a world with neither has nothing to record.
 Status OpSnapshotStepVelocity(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
     const auto* p = static_cast<const SnapshotStepVelocityParams*>(params);
     if (p == nullptr || p->env_count == 0u) return Status::Failed;
-    if (m.any_mujoco == 0u || m.max_dof == 0u) return Status::Ok;
+    if ((m.any_mujoco == 0u && m.integrator == 0u) || m.max_dof == 0u) return Status::Ok;
     if (p->max_dof != m.max_dof) return Status::InvalidArgument;
     const uint32_t total = p->env_count * m.max_dof;
     hipLaunchKernelGGL(SnapshotStepVelocityKernel, dim3((total + 255u) / 256u), dim3(256), 0, stream, m, d, p->env_count);

@@ -314,6 +314,10 @@ struct Link {
     float damping = 0.0f, armature = 0.0f, frictionloss = 0.0f, stiffness = 0.0f, spring_reference = 0.0f;
     float lower = 0.0f, upper = 0.0f;
     bool limited = false;
+    // a MuJoCo-sourced joint's limit margin and the solref[2], solimp[5] of its limit and dry-friction rows
+    float limit_margin = 0.0f;
+    float limit_reference[7] = {0.02f, 1.0f, 0.9f, 0.95f, 0.001f, 0.5f, 2.0f};
+    float friction_reference[7] = {0.02f, 1.0f, 0.9f, 0.95f, 0.001f, 0.5f, 2.0f};
     float initial_position = 0.0f;
     float actuator_force_limit = 0.0f;
     V3 anchor_shift;   // what the body authors in its own frame moves by this: minus its joint anchor

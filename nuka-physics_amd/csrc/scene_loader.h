@@ -24,20 +24,24 @@ constexpr uint32_t kGroundPlane = 4u;
 // MJCF: the geoms keep this library's native contact law (speculative velocity rows) instead of the MuJoCo law the
 // reference's importer gives every MJCF shape (src/import/mjcf_importer.cpp:790).
 constexpr uint32_t kNativeContactLaw = 8u;
+// MJCF: the joints keep the native limit and friction rows and the native integrator (drive damping folded into the
+// solve) instead of MuJoCo-sourced rows and the MuJoCo integrator of <option> (mjcf_importer.cpp:1193, 1720).
+constexpr uint32_t kNativeJointLaw = 16u;
 
 struct Scene {
     nuka_template_desc_t desc{};
     std::vector<std::string> link_names, joint_names;
-    std::vector<uint8_t> joint_type, joint_limit_flags;
+    std::vector<uint8_t> joint_type, joint_limit_flags, joint_law;
     std::vector<uint32_t> parent_link, body_role, body_link, shape_kind, shape_contype, shape_conaffinity, shape_group, shape_profile,
         excluded_pairs;   // [pair][2] collidable rows that never pair
     std::vector<float> joint_axis, link_local_pose, link_inertial_frame, link_mass, link_diag_inertia, joint_damping, joint_armature,
         joint_stiffness, joint_spring_reference, joint_frictionloss, joint_limit_lower, joint_limit_upper, body_local, shape_params, profile_mu,
-        profile_solref, profile_solimp, profile_margin, profile_solmix;
+        profile_solref, profile_solimp, profile_margin, profile_solmix, joint_limit_margin, joint_limit_reference, joint_friction_reference;
     std::vector<uint32_t> profile_law, profile_condim;
     std::vector<int32_t> profile_priority;
     uint32_t contact_cone = 0u;      // <option cone>: 0 pyramidal (MuJoCo's default), 1 elliptic
     float contact_impratio = 1.0f;   // <option impratio>
+    uint32_t integrator = 0u;        // 0 native; 1 MuJoCo's Euler; 2 implicit / implicitfast (<option integrator>)
     std::vector<float> initial_q, drive_stiffness, drive_damping, drive_force_limit, drive_joint_force_limit;
     std::array<float, 7> base_pose{0, 0, 0, 1, 0, 0, 0};
     bool floating_root = false;

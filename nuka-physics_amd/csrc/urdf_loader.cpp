@@ -180,7 +180,9 @@ std::unique_ptr<Scene> LoadUrdf(const std::string& path, uint32_t flags) {
 
     auto scene = std::make_unique<Scene>();
     scene->timestep = 1.0f / 240.0f;   // the format names none: the library's default step
-    FlattenScene(parts, flags, drive_mode, scene.get());
+    // a URDF carries no MuJoCo law: its shapes and joints keep the native rows (only the MJCF and USD importers of the
+    // reference mark theirs MuJoCo-sourced)
+    FlattenScene(parts, flags | kNativeContactLaw | kNativeJointLaw, drive_mode, scene.get());
     return scene;
 }
 

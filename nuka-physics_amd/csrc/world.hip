@@ -61,13 +61,14 @@ uint32_t JointWidth(uint8_t type) { return type <= kPrismatic ? 1u : type == kFl
 
 struct HostModel {
     ModelView counts{};   // scalar members only
-    std::vector<uint8_t> joint_type, joint_limit_flags;
+    std::vector<uint8_t> joint_type, joint_limit_flags, joint_law;
     std::vector<uint32_t> parent_link, link_body, link_tree_depth, link_child_range, link_children, link_dof, dof_link, dof_component,
         link_geom_kind, body_to_link, body_to_articulation, body_collidable_link, body_collidable_body;
     std::vector<uint64_t> link_dof_mask, excluded_pairs;
     std::vector<float> joint_axis, parent_offset, link_local_pose, link_inertial_frame, link_inertia, joint_damping, joint_armature,
         joint_stiffness, joint_spring_reference, joint_limit_lower, joint_limit_upper, joint_frictionloss, link_geom_local, shape_table, body_collidable_local, body_init_pose, profile_mu,
-        profile_solref, profile_solimp, profile_margin, profile_mix;   // profile_mix: [profile][3] priority, solmix, condim
+        profile_solref, profile_solimp, profile_margin, profile_mix,   // profile_mix: [profile][3] priority, solmix, condim
+        joint_limit_margin, joint_limit_reference, joint_friction_reference;
     std::vector<uint32_t> profile_law;
     std::vector<float> link_mass, link_diag_inertia;   // kept for nuka_world_set_param: a new mass rebuilds the spatial inertia
 };
@@ -101,6 +102,22 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
     m.joint_limit_lower = CopyOrZero(d.joint_limit_lower, nl);
     m.joint_limit_upper = CopyOrZero(d.joint_limit_upper, nl);
     m.joint_frictionloss = CopyOrZero(d.joint_frictionloss, nl);
+    // MuJoCo-sourced joints (scene/cook/cook_to_model.cpp:662-693)
+    m.joint_law = d.joint_law != nullptr ? std::vector<uint8_t>(d.joint_law, d.joint_law + nl) : std::vector<uint8_t>(nl, 0u);
+    m.joint_limit_margin = CopyOrZero(d.joint_limit_margin, nl);
+    {
+        const float reference[7] = {0.02f, 1.0f, 0.9f, 0.95f, 0.001f, 0.5f, 2.0f};
+        m.joint_limit_reference.resize(7u * nl); m.joint_friction_reference.resize(7u * nl);
+        for (uint32_t l = 0u; l < nl; ++l)
+            for (uint32_t k = 0u; k < 7u; ++k) {
+                m.joint_limit_reference[7u * l + k] = d.joint_limit_reference != nullptr ? d.joint_limit_reference[7u * l + k] : reference[k];
+                m.joint_friction_reference[7u * l + k] = d.joint_friction_reference != nullptr ? d.joint_friction_reference[7u * l + k] : reference[k];
+                if (!std::isfinite(m.joint_limit_reference[7u * l + k]) || !std::isfinite(m.joint_friction_reference[7u * l + k]))
+                    throw std::invalid_argument("invalid joint solref or solimp");
+            }
+        for (uint32_t l = 0u; l < nl; ++l)
+            if (m.joint_law[l] > 1u || !std::isfinite(m.joint_limit_margin[l])) throw std::invalid_argument("invalid joint law or limit margin");
+    }
     m.joint_limit_flags = d.joint_limit_flags != nullptr ? std::vector<uint8_t>(d.joint_limit_flags, d.joint_limit_flags + nl) : std::vector<uint8_t>(nl, 0u);
     m.link_inertia.resize(36u * nl);
     m.link_mass.assign(d.link_mass, d.link_mass + nl);
@@ -280,6 +297,9 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
     c.profile_count = d.profile_count;
     c.any_mujoco = 0u;
     for (uint32_t law : m.profile_law) if (law == 1u) c.any_mujoco = 1u;
+    for (uint8_t law : m.joint_law) if (law == 1u) c.any_mujoco = 1u;
+    if (d.integrator > 2u) throw std::invalid_argument("unknown integrator");
+    c.integrator = d.integrator;
     if (d.contact_cone > 1u) throw std::invalid_argument("unknown contact cone");
     c.contact_cone = d.contact_cone;
     c.contact_impratio = d.contact_impratio > 0.0f ? d.contact_impratio : 1.0f;
@@ -330,7 +350,8 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(joint_type, kU8) X(parent_link, kU32) X(joint_axis, kF32) X(parent_offset, kF32) X(link_local_pose, kF32) \
     X(link_inertial_frame, kF32) X(link_inertia, kF32) X(joint_damping, kF32) X(joint_armature, kF32) X(joint_stiffness, kF32) \
     X(joint_spring_reference, kF32) X(joint_limit_lower, kF32) X(joint_limit_upper, kF32) X(joint_frictionloss, kF32) \
-    X(joint_limit_flags, kU8) X(link_body, kU32) X(link_tree_depth, kU32) X(link_child_range, kU32) X(link_children, kU32) \
+    X(joint_limit_flags, kU8) X(joint_law, kU8) X(joint_limit_margin, kF32) X(joint_limit_reference, kF32) \
+    X(joint_friction_reference, kF32) X(link_body, kU32) X(link_tree_depth, kU32) X(link_child_range, kU32) X(link_children, kU32) \
     X(link_dof, kU32) X(dof_link, kU32) X(dof_component, kU32) X(link_dof_mask, kU64) X(link_geom_kind, kU32) \
     X(link_geom_local, kF32) X(shape_table, kF32) X(body_to_link, kU32) X(body_to_articulation, kU32) \
     X(body_collidable_link, kU32) X(body_collidable_body, kU32) X(body_collidable_local, kF32) X(profile_mu, kF32) \
@@ -378,6 +399,7 @@ struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
     ContactWarmStartParams p_warm0{}, p_warm1{};
     BlockDescentSolveParams p_solve{};
     SnapshotStepVelocityParams p_snapshot{};
+    ArticulationDampingParams p_damping{};
     ReferenceWeightsParams p_reference_weights{};   // dispatched at creation, outside the step (nk/pipeline/world.cpp:553-561)
     NarrowphaseHeightfieldParams p_heightfield{};
     std::vector<AccumulateStepParams> p_accumulate;   // one per substep (pipeline.cpp:128-152)
@@ -500,7 +522,8 @@ void BuildPipeline(World& w) {
     w.p_drives.dt = dt; w.p_drives.total_link_count = E * nl; w.p_drives.links_per_env = nl;
     w.p_drives.mode = m.drive_mode; w.p_drives.articulation_count = E; w.p_drives.bodies_per_env = nb;
     const bool drives = m.joint_drive_rows > 0u;
-    const bool fold = drives && cfg.solver_fold_drive_damping != 0xFFFFFFFFu;   // pipeline.cpp:380-381
+    // pipeline.cpp:380-381; a MuJoCo integrator keeps the damping explicit in the solve and applies it afterwards (:264-265)
+    const bool fold = drives && cfg.solver_fold_drive_damping != 0xFFFFFFFFu && m.integrator == 0u;
     w.p_drives.defer_velocity_damping = fold ? 1u : 0u;
     std::memcpy(w.p_drives.gravity, cfg.gravity, sizeof(cfg.gravity));
     w.p_readout_drives = {dt, E * nl, nl, m.rows_per_env, m.contact_rows_per_env + m.joint_limit_rows + m.joint_friction_rows};
@@ -592,6 +615,8 @@ void BuildPipeline(World& w) {
         if (m.contact_slots > 0u) add(NkOp::ContactWarmStart, &w.p_warm1);
     }
     if (drives) add(NkOp::ReadoutDrives, &w.p_readout_drives);   // pipeline.cpp:929-937
+    w.p_damping = {dt, m.max_dof, E, E * nl, m.integrator == 2u ? 1u : 0u, m.drive_mode, drives ? 1u : 0u};
+    if (m.integrator != 0u) add(NkOp::ArticulationDamping, &w.p_damping);   // pipeline.cpp:939-951
     add(NkOp::IntegratePosition, &w.p_int_pos);
     add(NkOp::FkWorldPoses, &w.p_fk);
     add(NkOp::FkLinkVelocities, &w.p_fk_velocity);
@@ -769,9 +794,10 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
     constexpr size_t kTemplateJointRows = offsetof(nuka_template_desc_t, excluded_pairs);
     constexpr size_t kTemplateExcluded = offsetof(nuka_template_desc_t, profile_law);
     constexpr size_t kTemplateLaw = offsetof(nuka_template_desc_t, profile_priority);
+    constexpr size_t kTemplateMerge = offsetof(nuka_template_desc_t, joint_law);
     constexpr size_t kWorldBase = offsetof(nuka_hip_world_desc_t, solver_fold_drive_damping);
     constexpr size_t kWorldDrives = offsetof(nuka_hip_world_desc_t, solver_substeps);
-    if ((tmpl->struct_size != sizeof(nuka_template_desc_t) && tmpl->struct_size != kTemplateLaw && tmpl->struct_size != kTemplateExcluded && tmpl->struct_size != kTemplateJointRows &&
+    if ((tmpl->struct_size != sizeof(nuka_template_desc_t) && tmpl->struct_size != kTemplateMerge && tmpl->struct_size != kTemplateLaw && tmpl->struct_size != kTemplateExcluded && tmpl->struct_size != kTemplateJointRows &&
          tmpl->struct_size != kTemplateBase) ||
         (desc->struct_size != sizeof(nuka_hip_world_desc_t) && desc->struct_size != kWorldDrives && desc->struct_size != kWorldBase))
         return Error(NUKA_RESULT_INVALID_ARG, "struct_size mismatch");
@@ -915,7 +941,7 @@ nuka_result_t nuka_scene_load_mjcf(const char* path, uint32_t flags, nuka_scene_
     if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
     *out = nullptr;
     if (path == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "path is null");
-    if ((flags & ~uint32_t(NUKA_SCENE_PLANE_CONTACTS_ONLY | NUKA_SCENE_GROUND_PLANE | NUKA_SCENE_NATIVE_CONTACT_LAW)) != 0u) return Error(NUKA_RESULT_INVALID_ARG, "unknown scene flag");
+    if ((flags & ~uint32_t(NUKA_SCENE_PLANE_CONTACTS_ONLY | NUKA_SCENE_GROUND_PLANE | NUKA_SCENE_NATIVE_CONTACT_LAW | NUKA_SCENE_NATIVE_JOINT_LAW)) != 0u) return Error(NUKA_RESULT_INVALID_ARG, "unknown scene flag");
     try {
         *out = reinterpret_cast<nuka_scene_handle>(scene_file::LoadMjcf(path, flags).release());
         return NUKA_RESULT_OK;

@@ -1001,7 +1001,24 @@ void nko_env_joint_rows(nko_world* w, uint32_t env) {
                 row.a.kind = NKO_SIDE_ARTIC; row.a.index = env;
                 J[t->link_dof[l]] = sign;
                 w->row_penetration[rs] = fmaxf(-signed_distance, 0.0f);
-                w->row_count[env] += 1u;
+                if (t->joint_law[l] == 1u) {   /* :860-877: the limit as a compliant row inside its margin, on the nearer bound only */
+                    const float pos = signed_distance - t->joint_limit_margin[l];
+                    const float* reference = t->joint_limit_reference + 7u * l;
+                    const float invweight = w->dof_invweight0[(size_t)env * md + t->link_dof[l]];
+                    float terms[6], discrete[3];
+                    nko_compliant_row_terms(reference, reference + 2u, pos, pos, 0.0f, invweight, dt, 1, terms);
+                    nko_discretize_compliant_row(terms[4], terms[5], terms[1], dt, discrete);
+                    row.flags |= NKO_ROW_MUJOCO;
+                    const int lower_nearest = w->q[link] - t->joint_limit_lower[l] < t->joint_limit_upper[l] - w->q[link];
+                    if (pos >= 0.0f || lower_nearest != (side == 0u)) {
+                        row.flags &= ~NKO_ROW_ACTIVE;
+                        w->lambda[rs] = 0.0f;
+                    }
+                    row.rhs = discrete[1]; row.compliance_alpha = discrete[0];
+                    w->row_reference_velocity_gain[rs] = discrete[2];
+                    w->row_invweight[rs] = invweight;
+                }
+                if (row.flags & NKO_ROW_ACTIVE) w->row_count[env] += 1u;
             } else w->lambda[rs] = 0.0f;
         } else if (slot < limit_rows + friction_rows) {   /* EmitJointFrictionRows :886-934 */
             const uint32_t l = slot - limit_rows;
@@ -1013,6 +1030,17 @@ void nko_env_joint_rows(nko_world* w, uint32_t env) {
                 row.lower = -friction * dt; row.upper = friction * dt;
                 row.a.kind = NKO_SIDE_ARTIC; row.a.index = env;
                 J[t->link_dof[l]] = 1.0f;
+                if (t->joint_law[l] == 1u) {   /* :921-931: dry friction regularised by its own solref / solimp */
+                    const float* reference = t->joint_friction_reference + 7u * l;
+                    const float invweight = w->dof_invweight0[(size_t)env * md + t->link_dof[l]];
+                    float terms[6], discrete[3];
+                    nko_compliant_row_terms(reference, reference + 2u, 0.0f, 0.0f, 0.0f, invweight, dt, 1, terms);
+                    nko_discretize_compliant_row(terms[4], terms[5], terms[1], dt, discrete);
+                    row.flags |= NKO_ROW_MUJOCO;
+                    row.compliance_alpha = discrete[0];
+                    w->row_reference_velocity_gain[rs] = discrete[2];
+                    w->row_invweight[rs] = invweight;
+                }
                 w->row_count[env] += 1u;
             }
         } else {   /* EmitJointDriveRows :938-971 */

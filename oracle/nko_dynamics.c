@@ -795,3 +795,54 @@ void nko_env_reference_weights(nko_world* w, uint32_t env) {
         if (body < nb) { weights[2u * body] = weight[0] / 3.0f; weights[2u * body + 1u] = weight[1] / 3.0f; }
     }
 }
+
+/* ActuatorVelocityDerivative (articulation.cu:942-948): what a servo's effort changes per unit joint velocity, none while
+ * its own force limit clamps it */
+static float actuator_velocity_derivative(const nko_world* w, size_t link) {
+    if (w->drive_force_limit[link] > 0.0f && fabsf(w->drive_command[link] - w->joint_gravity_force[link]) > w->drive_force_limit[link]) return 0.0f;
+    return w->t.drive_mode == NKO_DRIVE_PD_POSITION ? w->drive_damping[link] : w->t.drive_mode == NKO_DRIVE_VELOCITY ? w->drive_stiffness[link] : 0.0f;
+}
+
+/* ArticulationDampingKernel (articulation.cu:950-1000): contacts are solved with the plain mass; afterwards the step's
+ * velocity change goes through (M + dt D)^-1 M, D the joint damping and, for the implicit integrators, the unclamped
+ * servo velocity gains. */
+void nko_env_articulation_damping(nko_world* w, uint32_t env) {
+    const nko_template* t = &w->t;
+    const uint32_t nl = t->nl, stride = t->max_dof, dof = t->nv;
+    const size_t lbase = (size_t)env * nl, base = (size_t)env * stride;
+    const float dt = w->cfg.fixed_dt;
+    const int actuator_derivative = t->integrator == 2u, readout_drives = t->joint_drive_rows > 0u;
+    float change[NKO_MAX_DOF], damping[NKO_MAX_DOF];
+    int damped = 0;
+    for (uint32_t d = 0u; d < dof; ++d) {
+        const uint32_t link = t->dof_link[d], component = t->dof_component[d];
+        const int scalar = component == NKO_INVALID;
+        float value = scalar ? t->joint_damping[link] : 0.0f;
+        if (scalar && actuator_derivative) value += actuator_velocity_derivative(w, lbase + link);
+        const float velocity = scalar ? w->qdot[lbase + link] : w->link_velocity[(lbase + link) * 6u + component];
+        damping[d] = dt * value;
+        change[d] = damping[d] * (velocity - w->step_qdot_flat[base + d]);
+        damped |= value != 0.0f;
+    }
+    if (!damped) return;
+    float* mass = (float*)malloc(sizeof(float) * (size_t)stride * stride * 2u);
+    float* factor = mass + (size_t)stride * stride;
+    memcpy(mass, w->m + base * stride, sizeof(float) * (size_t)stride * stride);
+    for (uint32_t d = 0u; d < dof; ++d) mass[(size_t)d * stride + d] = mass[(size_t)d * stride + d] + damping[d];   /* FactorMass: `add` joins the diagonal */
+    nko_factor_mass(mass, factor, dof, stride);
+    nko_solve_mass(factor, change, dof, stride);
+    for (uint32_t d = 0u; d < dof; ++d) {
+        const uint32_t link = t->dof_link[d], component = t->dof_component[d];
+        float* velocity = component == NKO_INVALID ? &w->qdot[lbase + link] : &w->link_velocity[(lbase + link) * 6u + component];
+        *velocity -= change[d];
+        w->qdot_flat[base + d] = *velocity;
+        if (component == NKO_INVALID && actuator_derivative && readout_drives) {
+            const float derivative = actuator_velocity_derivative(w, lbase + link);
+            const float correction = derivative * (*velocity - w->step_qdot_flat[base + d]);
+            w->actuator_effort_requested[lbase + link] -= correction;
+            w->actuator_effort[lbase + link] -= correction;
+            w->tau[lbase + link] -= correction;
+        }
+    }
+    free(mass);
+}

@@ -83,6 +83,9 @@ typedef struct {
     /* MuJoCo-law profiles (scene_ir.hpp:116; contact_filter.hpp:20-37): law source, solref, solimp, margin and gap */
     uint32_t* profile_law;        /* n_profiles */
     float* profile_mix;           /* n_profiles*3: priority, solmix, condim */
+    uint8_t* joint_law;           /* nl: 1 MuJoCo-sourced joint rows */
+    float *joint_limit_margin, *joint_limit_reference, *joint_friction_reference;   /* nl, nl*7 (solref, solimp), nl*7 */
+    uint32_t integrator;          /* 0 native; 1 MuJoCo Euler (implicit joint damping after the solve); 2 with actuator derivatives */
     float* profile_solref;        /* n_profiles*2 */
     float* profile_solimp;        /* n_profiles*5 */
     float* profile_margin;        /* n_profiles*2 */
@@ -174,6 +177,7 @@ void nko_env_readout_contact_wrench(nko_world* w, uint32_t env);
 void nko_env_dynamics(nko_world* w, uint32_t env, uint32_t integrate_velocity);
 void nko_env_integrate_position(nko_world* w, uint32_t env);
 void nko_env_link_velocities(nko_world* w, uint32_t env);
+void nko_env_articulation_damping(nko_world* w, uint32_t env);
 void nko_env_reference_weights(nko_world* w, uint32_t env);
 /* the generalized force of a force f and a moment tau applied at `point`, added into one link's coordinates */
 void nko_accumulate_chain(const nko_world* w, uint32_t env, uint32_t link_local, uint32_t dof_index, v3 point, v3 f, v3 tau, float* out);

@@ -90,7 +90,7 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
     if (t->n_profiles) memcpy(t->profile_mu, d->profile_mu, t->n_profiles * 2u * sizeof(float));
     {   /* MuJoCo-law profile terms, defaults of ContactParamsIn (contact_filter.hpp:20-37) where not authored */
         const int has = d->struct_size >= offsetof(nko_template_desc, profile_priority);
-        const int has_mix = d->struct_size >= sizeof(nko_template_desc);
+        const int has_mix = d->struct_size >= offsetof(nko_template_desc, joint_law);
         t->profile_mix = ALLOC(float, t->n_profiles * 3u);
         t->profile_law = ALLOC(uint32_t, t->n_profiles); t->profile_solref = ALLOC(float, t->n_profiles * 2u);
         t->profile_solimp = ALLOC(float, t->n_profiles * 5u); t->profile_margin = ALLOC(float, t->n_profiles * 2u);
@@ -108,6 +108,22 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
         }
         t->cone = has ? d->contact_cone : 0u;
         t->impratio = has && d->contact_impratio > 0.0f ? d->contact_impratio : 1.0f;
+    }
+    {   /* MuJoCo-sourced joints: limit margin and the solref / solimp of the limit and friction rows */
+        const int has_joints = d->struct_size >= sizeof(nko_template_desc);
+        const float reference[7] = {0.02f, 1.0f, 0.9f, 0.95f, 0.001f, 0.5f, 2.0f};
+        t->joint_law = ALLOC(uint8_t, nl); t->joint_limit_margin = ALLOC(float, nl);
+        t->joint_limit_reference = ALLOC(float, nl * 7u); t->joint_friction_reference = ALLOC(float, nl * 7u);
+        for (uint32_t l = 0u; l < nl; ++l) {
+            t->joint_law[l] = has_joints && d->joint_law ? d->joint_law[l] : 0u;
+            t->joint_limit_margin[l] = has_joints && d->joint_limit_margin ? d->joint_limit_margin[l] : 0.0f;
+            for (uint32_t k = 0u; k < 7u; ++k) {
+                t->joint_limit_reference[7u * l + k] = has_joints && d->joint_limit_reference ? d->joint_limit_reference[7u * l + k] : reference[k];
+                t->joint_friction_reference[7u * l + k] = has_joints && d->joint_friction_reference ? d->joint_friction_reference[7u * l + k] : reference[k];
+            }
+            t->any_mujoco = t->any_mujoco || t->joint_law[l] == 1u;
+        }
+        t->integrator = has_joints ? d->integrator : 0u;
     }
     for (uint32_t b = 0u; b < nb; ++b) {
         const uint32_t role = d->body_role[b], link = d->body_link[b];
@@ -211,6 +227,7 @@ static void free_template(nko_template* t) {
     free(t->link_geom_local); free(t->link_geom_kind); free(t->shape_table); free(t->excluded_pairs); free(t->body_to_link);
     free(t->body_to_articulation); free(t->body_collidable_link); free(t->body_collidable_body);
     free(t->body_collidable_local); free(t->body_init_pose); free(t->profile_mu);
+    free(t->joint_law); free(t->joint_limit_margin); free(t->joint_limit_reference); free(t->joint_friction_reference);
     free(t->profile_mix); free(t->profile_law); free(t->profile_solref); free(t->profile_solimp); free(t->profile_margin);
 }
 
@@ -231,6 +248,7 @@ nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc*
     /* pipeline.hpp:48-49: velocity feedback of a drive is solved implicitly unless switched off */
     w->fold_drive_damping = 1;
     if (desc->struct_size >= offsetof(nko_world_desc, solver_substeps) && desc->solver_fold_drive_damping == 0xFFFFFFFFu) w->fold_drive_damping = 0;
+    if (w->t.integrator != 0u) w->fold_drive_damping = 0;   /* pipeline.cpp:380-381: a MuJoCo integrator keeps the damping explicit in the solve */
     /* pipeline.cpp:63-69: every op of the interval runs at dt / substeps */
     w->substeps = desc->struct_size >= sizeof(nko_world_desc) && desc->solver_substeps > 1u ? desc->solver_substeps : 1u;
     w->outer_dt = w->cfg.fixed_dt;
@@ -414,6 +432,7 @@ void nko_contact_warm_start(nko_world* w, uint32_t phase) {
 void nko_block_descent_solve(nko_world* w) { FOR_ENVS(nko_env_solve(w, env)) }
 void nko_integrate_position(nko_world* w) { FOR_ENVS(nko_env_integrate_position(w, env)) }
 void nko_fk_link_velocities(nko_world* w) { FOR_ENVS(nko_env_link_velocities(w, env)) }
+void nko_articulation_damping(nko_world* w) { FOR_ENVS(nko_env_articulation_damping(w, env)) }
 void nko_reference_weights(nko_world* w) {
     const int fold = w->fold_drive_damping;
     w->fold_drive_damping = 0;   /* ComputeArticulationMass without drive damping (articulation.cu:452-453) */
@@ -438,7 +457,7 @@ void nko_snapshot_step_velocity(nko_world* w) {
 }
 
 static void step_interval(nko_world* w) {
-    if (w->t.rows_per_env > 0u) nko_snapshot_step_velocity(w);
+    if (w->t.rows_per_env > 0u || w->t.integrator != 0u) nko_snapshot_step_velocity(w);   /* pipeline.cpp:367 */
     nko_fk_world_poses(w);
     if (w->t.joint_drive_rows > 0u) nko_apply_drives(w);
     nko_articulation_dynamics(w, 1u);
@@ -455,6 +474,7 @@ static void step_interval(nko_world* w) {
         nko_contact_warm_start(w, 1u);
     }
     if (w->t.joint_drive_rows > 0u) nko_readout_drives(w);   /* pipeline.cpp:929-937 */
+    if (w->t.integrator != 0u) nko_articulation_damping(w);  /* pipeline.cpp:939-951 */
     nko_integrate_position(w);
     nko_fk_world_poses(w);
     nko_fk_link_velocities(w);

@@ -113,6 +113,13 @@ typedef struct nko_template_desc {
     const int32_t* profile_priority;
     const float* profile_solmix;
     const uint32_t* profile_condim;
+    /* MuJoCo-sourced joints and integrator; read only when struct_size covers them */
+    const uint8_t* joint_law;
+    const float* joint_limit_margin;
+    const float* joint_limit_reference;
+    const float* joint_friction_reference;
+    uint32_t integrator;
+    uint32_t reserved2;
 } nko_template_desc;
 
 typedef struct nko_world_desc {
@@ -167,6 +174,8 @@ void nko_world_step(nko_world* w);
  * once at the template's rest pose. */
 void nko_reference_weights(nko_world* w);
 void nko_snapshot_step_velocity(nko_world* w);
+/* ArticulationDamping (articulation.cu:950-1000): the step's velocity change through (M + dt D)^-1 M */
+void nko_articulation_damping(nko_world* w);
 /* scene/contact_filter.hpp:100-137 MergeContactParams.  A side is mu1, mu2, solref[2], solimp[5], margin, gap, priority,
  * solmix, condim; out = mu1, mu2, solref[2], solimp[5], margin, gap, condim */
 void nko_merge_contact_params(const float a[14], const float b[14], float out[12]);

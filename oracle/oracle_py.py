@@ -49,7 +49,8 @@ def lib():
         L.nko_world_rows_per_env.restype = C.c_uint32
         for name in ("fk_world_poses", "sync_link_body_pose", "build_aabbs", "query_pairs", "narrowphase",
                      "assemble_rows", "block_descent_solve", "integrate_position", "fk_link_velocities", "apply_drives",
-                     "readout_drives", "readout_contact_wrench", "reference_weights", "snapshot_step_velocity"):
+                     "readout_drives", "readout_contact_wrench", "reference_weights", "snapshot_step_velocity",
+                     "articulation_damping"):
             getattr(L, "nko_" + name).argtypes = [C.c_void_p]
         L.nko_articulation_dynamics.argtypes = [C.c_void_p, C.c_uint32]
         L.nko_contact_warm_start.argtypes = [C.c_void_p, C.c_uint32]

@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_struct_layouts_match_the_header():
     # 6 u32 + 22 pointers, then 4 pointers + 2 u32 of joint rows, then a pointer + 2 u32 of excluded pairs; 15 4-byte words
-    assert C.sizeof(nk.abi.TemplateDescC) == 6 * 4 + 22 * 8 + 4 * 8 + 2 * 4 + 8 + 2 * 4 + 4 * 8 + 2 * 4 + 3 * 8
+    assert C.sizeof(nk.abi.TemplateDescC) == 6 * 4 + 22 * 8 + 4 * 8 + 2 * 4 + 8 + 2 * 4 + 4 * 8 + 2 * 4 + 3 * 8 + 4 * 8 + 2 * 4
     assert C.sizeof(nk.abi.WorldDescC) == 17 * 4
 
 

@@ -253,3 +253,124 @@ def test_priority_solmix_and_frictionless_profiles(oracle_py, device, law):
         for name in ("q", "qdot", "link_velocity"):
             close(world, oracle, name, tol=5e-4)
         oracle.close(); world.close()
+
+
+def mujoco_joint_pair(oracle_py, device, index, E, integrator, mode=abi.DRIVE_PD_POSITION, seed=5):
+    """A benchmark configuration as an imported MJCF would have it: every joint MuJoCo-sourced with ranges around the
+    nominal pose (some seeded joints start beyond them), dry friction, passive damping, servos, and the MuJoCo
+    integrator."""
+    import copy
+    cfg = nk.synthetic.config(index, E)
+    t = copy.deepcopy(cfg.template)
+    t.drive_rows, t.drive_mode, t.integrator = True, mode, integrator
+    for p in t.profiles:
+        p.update(law=abi.LAW_MUJOCO)
+    t.contact_cone = abi.CONE_ELLIPTIC
+    rng = np.random.default_rng(seed)
+    for l, link in enumerate(t.links):
+        if link["joint_type"] != abi.JOINT_REVOLUTE:
+            continue
+        link["law"] = abi.LAW_MUJOCO
+        link["damping"] = 0.3 + 0.05 * (l % 4)
+        if l % 3 != 0:
+            link["lower"], link["upper"] = float(cfg.nominal_q[l]) - 0.2, float(cfg.nominal_q[l]) + 0.25
+            link["limit_margin"] = 0.01 * (l % 2)
+            link["limit_reference"] = (0.02 + 0.005 * (l % 3), 1.0, 0.9, 0.95, 0.001, 0.5, 2.0)
+        if l % 2 == 0:
+            link["frictionloss"] = 0.15
+            link["friction_reference"] = (0.01, 1.0, 0.85, 0.95, 0.001, 0.5, 2.0)
+    desc = abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters)
+    oracle = oracle_py.OracleWorld(t, desc, threads=8)
+    world = nk.World(device, t, desc)
+    state = cfg.state()
+    state["base_pose"][:, 2] -= 0.1 if index == 2 else 0.03
+    nl = t.link_count
+    gains = dict(drive_target=cfg.nominal_q[None, :] + rng.normal(0, 0.2, (E, nl)), drive_stiffness=rng.uniform(20, 80, (E, nl)),
+                 drive_damping=rng.uniform(0.5, 3, (E, nl)), drive_force_limit=np.where(rng.uniform(size=(E, nl)) < 0.5, rng.uniform(5, 30, (E, nl)), 0.0),
+                 velocity_target=rng.normal(0, 0.5, (E, nl)))
+    for w in (oracle, world):
+        w.set_state(state)
+        for name, values in gains.items():
+            w.upload(name, values.astype(np.float32))
+    return cfg, t, oracle, world
+
+
+@pytest.mark.parametrize("index,integrator", [(2, abi.INTEGRATOR_MUJOCO_EULER), (3, abi.INTEGRATOR_MUJOCO_EULER), (3, abi.INTEGRATOR_MUJOCO_IMPLICIT)])
+def test_mujoco_joint_rows_and_integrator(oracle_py, device, index, integrator):
+    """Compliant limit and dry-friction rows (assemble_rows.cu:860-877, 921-931) and ArticulationDamping
+    (articulation.cu:950-1000), op by op and then over whole steps."""
+    E = 64
+    cfg, t, oracle, world = mujoco_joint_pair(oracle_py, device, index, E, integrator)
+    R = world.rows_per_env
+    first = world.info.contact_slots_per_env * 16
+    sequence = [("SnapshotStepVelocity", ("snapshot_step_velocity",)), ("FkWorldPoses", ("fk_world_poses",)), ("ApplyDrives", ("apply_drives",)),
+                ("ArticulationDynamics", ("articulation_dynamics", 1)), ("SyncLinkBodyPose", ("sync_link_body_pose",)),
+                ("BuildAabbs", ("build_aabbs",)), ("LbvhQueryPairs", ("query_pairs",)), ("NarrowphasePrimitives", ("narrowphase",)),
+                ("AssembleRows", ("assemble_rows",))]
+    for name, call in sequence:
+        oracle.op(*call)
+        world.op(name)
+    world.synchronize()
+    got = world.download("urows").view(np.uint32).reshape(E, R, ROW_WORDS)
+    expect = oracle.download("urows").view(np.uint32).reshape(E, R, ROW_WORDS)
+    assert np.array_equal(got[:, first:, [0, 1, 2, 3, 10, 11]], expect[:, first:, [0, 1, 2, 3, 10, 11]])
+    joint_flags = expect[:, first:, 0]
+    mujoco_rows = (joint_flags & (1 << 11)) != 0
+    assert ((joint_flags & 1) != 0)[mujoco_rows].sum() >= E and (mujoco_rows & ((joint_flags & 1) == 0)).sum() > 0   # live ones, and limits left off
+    active = (expect[:, :, 0] & 1) != 0
+    for word in (4, 5, 6, 7):   # rhs (with the start-velocity forcing), compliance, bounds
+        a = np.where(active, got.view(np.float32)[:, :, word], 0.0)
+        b = np.where(active, expect.view(np.float32)[:, :, word], 0.0)
+        a, b = np.clip(a, -1e30, 1e30), np.clip(b, -1e30, 1e30)
+        assert per_env_error(a, b, E).max() <= TOL, word
+    assert np.array_equal(world.download("lambda").reshape(E, R)[:, first:] != 0, oracle.download("lambda").reshape(E, R)[:, first:] != 0)
+    for name, call in (("ContactWarmStart", ("contact_warm_start", 0)), ("BlockDescentSolve", ("block_descent_solve",))):
+        oracle.op(*call)
+        world.op(name)
+    oracle.op("contact_warm_start", 1); world.op("ContactWarmStart", 1)
+    oracle.op("readout_drives"); world.op("ReadoutDrives")
+    world.synchronize()
+    close(world, oracle, "qdot", tol=2e-4)
+    before = world.download("qdot").copy()
+    oracle.op("articulation_damping"); world.op("ArticulationDamping")
+    world.synchronize()
+    assert np.abs(world.download("qdot") - before).max() > 1e-4          # the op did something
+    for name in ("qdot", "link_velocity", "qdot_flat", "actuator_effort", "tau"):
+        close(world, oracle, name, tol=2e-4)
+    oracle.close(); world.close()
+    cfg, t, oracle, world = mujoco_joint_pair(oracle_py, device, index, E, integrator)
+    oracle.step(6); world.step(6); world.synchronize()
+    assert np.array_equal(world.download("env_status"), oracle.download("env_status")) and (oracle.download("env_status") == 0).all()
+    for name in ("q", "qdot", "base_pose", "link_velocity", "actuator_effort"):
+        close(world, oracle, name, tol=1e-3)
+    oracle.close(); world.close()
+
+
+def test_mjcf_scene_runs_the_mujoco_joint_law_unless_told_otherwise(oracle_py, device):
+    """An MJCF file's joints and integrator (mjcf_importer.cpp:1193, 1720): MuJoCo-sourced by default, native with the
+    scene flags; either way the device follows the oracle."""
+    import os
+    path = os.path.join(os.path.dirname(__file__), "data", "capsule_walker.xml")
+    for flags, law, integrator in ((0, abi.LAW_MUJOCO, abi.INTEGRATOR_MUJOCO_EULER),
+                                   (nk.SCENE_NATIVE_JOINT_LAW | nk.SCENE_NATIVE_CONTACT_LAW, abi.LAW_NATIVE, abi.INTEGRATOR_NATIVE)):
+        scene = nk.Scene(path, flags)
+        arrays = scene.template_arrays()
+        assert (arrays["joint_law"] == law).all() and arrays["integrator"] == integrator
+        E = 16
+        desc = abi.world_desc(E, scene.info.timestep, vel_iters=8)
+        oracle, world = oracle_py.OracleWorld(scene, desc, threads=8), nk.World(device, scene, desc)
+        state = scene.initial_state()
+        for w in (oracle, world):
+            for name in ("q", "drive_stiffness", "drive_damping", "drive_force_limit", "drive_joint_force_limit"):
+                w.upload(name, np.tile(state[name], E))
+            w.upload("base_pose", np.tile(state["base_pose"], E))
+            w.upload("drive_target", np.tile(state["q"], E))
+        oracle.op("fk_world_poses"); oracle.op("sync_link_body_pose"); oracle.op("reference_weights")
+        world.op("FkWorldPoses"); world.op("SyncLinkBodyPose")
+        if law == abi.LAW_MUJOCO:
+            world.op("ReferenceWeights")
+        oracle.step(20); world.step(20); world.synchronize()
+        assert np.array_equal(world.download("env_status"), oracle.download("env_status"))
+        for name in ("q", "qdot", "base_pose"):
+            close(world, oracle, name, tol=1e-3)
+        oracle.close(); world.close()

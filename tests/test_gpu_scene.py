@@ -140,7 +140,10 @@ def test_urdf_world_matches_the_oracle(oracle_py, device):
     assert np.abs(oracle.download("actuator_effort")).max() <= 30.0 + 1e-3 and (oracle.download("actuator_saturated") != 0).any()
     for name in ("q", "qdot", "base_pose", "link_pose", "actuator_effort", "joint_limit_impulse"):
         error = relative_error(world.download(name), oracle.download(name))
-        assert error <= 5 * TOL, f"{name}: {error:.2e}"
+        # the knee limits' multipliers move by 6.7e-4 in the oracle itself when its inputs move by one unit in the last
+        # place (measured on this scenario); they are held to four times that, everything else to 5 TOL
+        bound = 4 * 6.7e-4 if name == "joint_limit_impulse" else 5 * TOL
+        assert error <= bound, f"{name}: {error:.2e}"
     world.close(); oracle.close()
 
 

@@ -314,3 +314,40 @@ def test_errors(tmp_path):
         with pytest.raises(nk.NukaError) as err:
             nk.Scene(str(path))
         assert err.value.code == abi.RESULT_INVALID_ARG, name
+
+
+def test_joint_law_attributes_and_integrator(tmp_path):
+    """mjcf_importer.cpp:334-338, 1193-1213, 1720-1728: every joint is MuJoCo-sourced with its limit margin and the solref /
+    solimp of its limit and friction rows (class defaults, then the joint's own; a partial list keeps the rest), the
+    scene runs MuJoCo's integrator (Euler unless <option> names implicit or implicitfast; RK4 is refused), and the
+    native flag turns both off.  A URDF is native throughout."""
+    text = """<mujoco><option integrator="{integrator}"/>
+      <default><default class="soft"><joint solreflimit="0.05 0.8" solimplimit="0.8" margin="0.02" solreffriction="0.03"/></default></default>
+      <worldbody><body name="a"><inertial mass="1" pos="0 0 0" diaginertia="1 1 1"/>
+        <joint name="j0" type="hinge" axis="0 1 0" range="-1 1" class="soft" solimplimit="0.7 0.9"/>
+        <body name="b" pos="0 0 1"><inertial mass="1" pos="0 0 0" diaginertia="1 1 1"/>
+          <joint name="j1" type="hinge" axis="0 1 0" solimpfriction="0.6 0.7 0.003" frictionloss="0.1"/></body></body></worldbody></mujoco>"""
+    default = [0.02, 1.0, 0.9, 0.95, 0.001, 0.5, 2.0]
+    for integrator, expect in (("Euler", abi.INTEGRATOR_MUJOCO_EULER), ("implicitfast", abi.INTEGRATOR_MUJOCO_IMPLICIT), ("implicit", abi.INTEGRATOR_MUJOCO_IMPLICIT)):
+        path = tmp_path / f"{integrator}.xml"
+        path.write_text(text.format(integrator=integrator))
+        a = nk.Scene(str(path)).template_arrays()
+        assert a["integrator"] == expect and (a["joint_law"] == abi.LAW_MUJOCO).all()
+        limit, friction = a["joint_limit_reference"].reshape(-1, 7), a["joint_friction_reference"].reshape(-1, 7)
+        j0, j1 = 1, 2                                              # link 0 is the world
+        assert np.allclose(limit[j0], [0.05, 0.8, 0.7, 0.9, 0.001, 0.5, 2.0]) and np.isclose(a["joint_limit_margin"][j0], 0.02)
+        assert np.allclose(friction[j0], [0.03, 1.0, 0.9, 0.95, 0.001, 0.5, 2.0])
+        assert np.allclose(limit[j1], default) and a["joint_limit_margin"][j1] == 0.0
+        assert np.allclose(friction[j1], [0.02, 1.0, 0.6, 0.7, 0.003, 0.5, 2.0])
+    native = nk.Scene(str(tmp_path / "Euler.xml"), nk.SCENE_NATIVE_JOINT_LAW).template_arrays()
+    assert native["integrator"] == abi.INTEGRATOR_NATIVE and (native["joint_law"] == abi.LAW_NATIVE).all()
+    plain = tmp_path / "plain.xml"
+    plain.write_text(text.replace('<option integrator="{integrator}"/>', ""))
+    assert nk.Scene(str(plain)).template_arrays()["integrator"] == abi.INTEGRATOR_MUJOCO_EULER
+    rk4 = tmp_path / "rk4.xml"
+    rk4.write_text(text.format(integrator="RK4"))
+    with pytest.raises(nk.NukaError) as err:
+        nk.Scene(str(rk4))
+    assert err.value.code == abi.RESULT_INVALID_ARG and "RK4" in str(err.value)   # the scene loader's code for every refusal
+    urdf = nk.Scene(os.path.join(ROOT, "tests", "golden", "urdf", "minimal_arm.urdf")).template_arrays()
+    assert urdf["integrator"] == abi.INTEGRATOR_NATIVE and (urdf["joint_law"] == abi.LAW_NATIVE).all() and urdf["profile_law"].size == 0 or (urdf["profile_law"] == abi.LAW_NATIVE).all()

@@ -356,3 +356,110 @@ def test_frictionless_contacts_have_the_normal_row_alone(oracle_py):
         w.step(20)   # and the solve runs on such heads
         assert (w.download("env_status") == 0).all()
         w.close()
+
+
+def hinge(law, **joint):
+    """A fixed base and one hinge about y carrying a point-like link: M = I_yy + m r^2 + armature."""
+    t = abi.Template()
+    t.add_link(abi.JOINT_FIXED, None, mass=1.0)
+    t.add_link(abi.JOINT_REVOLUTE, 0, axis=(0, 1, 0), mass=1.5, diag_inertia=(0.01, 0.03, 0.02), com=(0.2, 0, 0), armature=0.01, law=law, **joint)
+    return t, 0.03 + 1.5 * 0.2 * 0.2 + 0.01
+
+
+def test_a_compliant_joint_limit_gives_way_as_the_spring_reference_says(oracle_py):
+    """A constant torque presses a MuJoCo-sourced hinge against its upper limit (assemble_rows.cu:860-877): at rest the
+    row equation a + R f = aref holds with a = 0 and f the torque, with the coordinate's reference weight 1 / M as the
+    row's weight, which fixes how far the joint passes its limit.  The lower row of the same joint stays inactive."""
+    L = oracle_py.lib()
+    reference, torque, dt, upper = (0.03, 1.0, 0.85, 0.96, 0.002, 0.5, 2.0), 2.0, 0.002, 0.3
+    t, M = hinge(abi.LAW_MUJOCO, lower=-0.4, upper=upper, damping=0.4, limit_reference=reference, limit_margin=0.0)
+    w = oracle_py.OracleWorld(t, abi.world_desc(1, dt, gravity=(0, 0, 0), vel_iters=16, velocity_tolerance=1e-7))
+    assert w.download("dof_invweight0")[0] == pytest.approx(1.0 / M, rel=1e-5)
+    w.upload("q", np.array([0.0, 0.25], np.float32))
+    tau = np.array([0.0, torque], np.float32)
+    for _ in range(3000):
+        w.upload("tau", tau)
+        w.step()
+    assert w.download("env_status")[0] == 0 and abs(w.download("qdot")[1]) < 1e-5
+    R = w.rows_per_env
+    flags = w.download("urows").view(np.uint32).reshape(R, ROW_WORDS)[:, 0]
+    # two limit row slots a link: the hinge's are 2 and 3; its lower bound is off, its upper bound on
+    assert flags[2] == (1 << 4) | MUJOCO and flags[3] == ACTIVE | (1 << 5) | MUJOCO
+    assert w.download("lambda")[3] / dt == pytest.approx(torque, rel=1e-3)
+    passed = w.download("q")[1] - upper
+    lo, hi = 0.0, 0.05
+    for _ in range(60):
+        mid = 0.5 * (lo + hi)
+        terms = (F * 6)()
+        L.nko_compliant_row_terms(farr(reference[:2]), farr(reference[2:]), F(-mid), F(-mid), F(0.0), F(1.0 / M), F(dt), 1, terms)
+        lo, hi = (mid, hi) if terms[5] / terms[4] < torque else (lo, mid)
+    assert passed == pytest.approx(0.5 * (lo + hi), rel=0.03)
+    w.close()
+
+
+def test_mujoco_dry_friction_row_carries_its_reference(oracle_py):
+    """assemble_rows.cu:921-931: the friction row of a MuJoCo-sourced joint is regularised by its own solref / solimp
+    at the coordinate's reference weight; a torque below the friction loss leaves the joint at rest but for the slip the
+    regularisation admits, R times the held impulse."""
+    L = oracle_py.lib()
+    reference, dt, loss, torque = (0.01, 1.0, 0.9, 0.95, 0.001, 0.5, 2.0), 0.002, 0.5, 0.3
+    t, M = hinge(abi.LAW_MUJOCO, frictionloss=loss, friction_reference=reference)
+    w = oracle_py.OracleWorld(t, abi.world_desc(1, dt, gravity=(0, 0, 0), vel_iters=16, velocity_tolerance=1e-8))
+    w.upload("tau", np.array([0.0, torque], np.float32))
+    w.step()
+    rows = w.download("urows").view(np.uint32).reshape(-1, ROW_WORDS)
+    assert rows[1, 0] == ACTIVE | (1 << 7) | MUJOCO          # one friction row slot a link: the hinge's is 1
+    terms, discrete = (F * 6)(), (F * 3)()
+    L.nko_compliant_row_terms(farr(reference[:2]), farr(reference[2:]), F(0.0), F(0.0), F(0.0), F(1.0 / M), F(dt), 1, terms)
+    L.nko_discretize_compliant_row(F(terms[4]), F(terms[5]), F(terms[1]), F(dt), discrete)
+    assert rows.view(np.float32)[1, 5] == np.float32(discrete[0]) and discrete[0] > 0.0
+    # the friction holds (its impulse stays inside the bounds) and the momentum balance M v = dt torque + lambda closes;
+    # what the regularisation lets through is a small slip along the torque, where the native row holds v = 0
+    lam, v = float(w.download("lambda")[1]), float(w.download("qdot")[1])
+    assert -loss * dt < lam < 0.0
+    assert M * v == pytest.approx(dt * torque + lam, rel=1e-3, abs=1e-8)
+    assert 0.0 < v < 0.2 * dt * torque / M
+    w.close()
+    t, _ = hinge(abi.LAW_NATIVE, frictionloss=loss)
+    w = oracle_py.OracleWorld(t, abi.world_desc(1, dt, gravity=(0, 0, 0), vel_iters=16, velocity_tolerance=1e-8))
+    w.upload("tau", np.array([0.0, torque], np.float32))
+    w.step()
+    assert abs(float(w.download("qdot")[1])) < 1e-7
+    w.close()
+
+
+def test_mujoco_integrator_applies_joint_damping_implicitly(oracle_py):
+    """ArticulationDamping (articulation.cu:950-1000) on one hinge: v+ = v + dt (tau - b v) / (M + dt b), the implicit
+    Euler step of the damping, against the explicit one of the native integrator; then on the seven-joint chain the
+    step's velocity change against (M + dt D)^-1 M applied densely in float64."""
+    dt, b, torque = 0.01, 3.0, 0.7
+    t, M = hinge(abi.LAW_NATIVE, damping=b)
+    for integrator in (abi.INTEGRATOR_NATIVE, abi.INTEGRATOR_MUJOCO_EULER):
+        t.integrator = integrator
+        w = oracle_py.OracleWorld(t, abi.world_desc(1, dt, gravity=(0, 0, 0)))
+        v = 0.0
+        for _ in range(50):
+            w.upload("tau", np.array([0.0, torque], np.float32))
+            w.step()
+            v = v + dt * (torque - b * v) / (M + (dt * b if integrator else 0.0))
+            assert w.download("qdot")[1] == pytest.approx(v, rel=2e-5)
+        w.close()
+    cfg = nk.synthetic.config(1, 2)
+    for link in cfg.template.links[1:]:
+        link["damping"] = 0.8
+    cfg.template.integrator = abi.INTEGRATOR_MUJOCO_EULER
+    w = oracle_py.OracleWorld(cfg.template, abi.world_desc(2, cfg.dt))
+    state = cfg.state(2)
+    w.set_state(state)
+    w.op("snapshot_step_velocity"); w.op("fk_world_poses"); w.op("articulation_dynamics", 1)
+    n = w.dof
+    before, solved = state["qdot"][:, 1:].astype(np.float64), w.download("qdot").reshape(2, -1)[:, 1:].astype(np.float64)
+    mass = w.download("m").reshape(2, n, n).astype(np.float64)
+    w.op("articulation_damping")
+    after = w.download("qdot").reshape(2, -1)[:, 1:]
+    for e in range(2):
+        D = cfg.dt * 0.8 * np.eye(n)
+        expect = before[e] + np.linalg.solve(mass[e] + D, mass[e] @ (solved[e] - before[e]))
+        assert np.allclose(after[e], expect, rtol=2e-4, atol=1e-6)
+    assert np.abs(after - solved).max() > 1e-4
+    w.close()
