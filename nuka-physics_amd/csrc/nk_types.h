@@ -98,6 +98,7 @@ struct ModelView {
     const uint32_t* link_tree_depth;
     const uint32_t* link_child_range;
     const uint32_t* link_children;
+    const uint32_t* link_push_order;   // children in the order the composite-inertia pass adds them to their parents, then kInvalid
     const uint32_t* link_dof;
     const uint32_t* dof_link;
     const uint32_t* dof_component;

@@ -126,16 +126,26 @@ __global__ void __launch_bounds__(kWave) FkWorldPosesKernel(ModelView m, DataVie
     if (env >= env_count) return;
     float* pose = lds;   // nl * 7
     const float* q = d.q + size_t{env} * nl;
+    // A link's frame in its parent does not wait on the tree: every lane computes its own link's before the sweep, which
+    // then only composes a depth at a time (links past the 64th compute theirs when their depth comes).
+    struct Placed { uint32_t depth, parent; Xf frame; };
+    auto place = [&](uint32_t l) {
+        const uint8_t type = m.joint_type[l];
+        const uint32_t parent = m.parent_link[l];
+        const Xf relative = joint_relative_frame(type, load3(m.joint_axis + 3u * l), load_xf(m.link_local_pose + 7u * l),
+                                                 load3(m.parent_offset + 3u * l), q[l]);
+        return Placed{m.link_tree_depth[l], parent, parent == kInvalid && type == kFloatingBase ? load_xf(d.base_pose + size_t{env} * 7u) : relative};
+    };
+    auto compose = [&](uint32_t l, const Placed& t) {
+        store_xf(pose + 7u * l, t.parent == kInvalid ? t.frame : compose_frame(load_xf(pose + 7u * t.parent), t.frame));
+    };
+    Placed own{kInvalid, kInvalid, Xf{}};
+    if (lane < nl) own = place(lane);
     for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
-        for (uint32_t l = lane; l < nl; l += kWave) {
-            if (m.link_tree_depth[l] != depth) continue;
-            const Xf relative = joint_relative_frame(m.joint_type[l], load3(m.joint_axis + 3u * l),
-                load_xf(m.link_local_pose + 7u * l), load3(m.parent_offset + 3u * l), q[l]);
-            const uint32_t parent = m.parent_link[l];
-            Xf out;
-            if (parent == kInvalid) out = m.joint_type[l] == kFloatingBase ? load_xf(d.base_pose + size_t{env} * 7u) : relative;
-            else out = compose_frame(load_xf(pose + 7u * parent), relative);
-            store_xf(pose + 7u * l, out);
+        if (own.depth == depth) compose(lane, own);
+        for (uint32_t l = lane + kWave; l < nl; l += kWave) {
+            const Placed t = place(l);
+            if (t.depth == depth) compose(l, t);
         }
         __syncthreads();
     }
@@ -176,6 +186,13 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
     float* qd = d.qdot + lbase;
     const V3 gravity{p.gravity[0], p.gravity[1], p.gravity[2]};
     const Q4 base_rot = load_xf(d.base_pose + size_t{env} * 7u).r;
+    // A lane's own link: its place in the tree and its joint rate, read once.  The passes below visit the tree a depth at
+    // a time and every visit would otherwise wait on these loads again (links past the 64th read theirs at each visit).
+    struct LinkTree { uint32_t depth, parent, child_begin, child_end; uint8_t type; float rate; };
+    auto tree_of = [&](uint32_t l) {
+        return LinkTree{m.link_tree_depth[l], m.parent_link[l], m.link_child_range[2u * l], m.link_child_range[2u * l + 1u], m.joint_type[l], qd[l]};
+    };
+    const LinkTree own = lane < nl ? tree_of(lane) : LinkTree{kInvalid, kInvalid, 0u, 0u, uint8_t(0), 0.0f};
 
     // link twists of the state enter LDS (a floating root's twist is state; the rest is rebuilt)
     for (uint32_t e = lane; e < nl * 6u; e += kWave) v[e] = d.link_velocity[lbase * 6u + e];
@@ -195,16 +212,17 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
     // velocities root to leaf (:334-363)
     for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
         for (uint32_t l = lane; l < nl; l += kWave) {
-            if (m.link_tree_depth[l] != depth) continue;
-            const uint32_t parent = m.parent_link[l];
-            if (parent == kInvalid && m.joint_type[l] == kFloatingBase) continue;
+            const LinkTree t = l == lane ? own : tree_of(l);
+            if (t.depth != depth) continue;
+            const uint32_t parent = t.parent;
+            if (parent == kInvalid && t.type == kFloatingBase) continue;
             float vp[6] = {0, 0, 0, 0, 0, 0}, tp[6], jv[6], vl[6];
             if (parent != kInvalid) {
 #pragma unroll
                 for (int i = 0; i < 6; ++i) vp[i] = v[6u * parent + i];
             }
             mat66_vec(xup + 36u * l, vp, tp);
-            const float qdl = qd[l];
+            const float qdl = t.rate;
 #pragma unroll
             for (int i = 0; i < 6; ++i) { jv[i] = S[6u * l + i] * qdl; vl[i] = tp[i] + jv[i]; }
 #pragma unroll
@@ -237,15 +255,16 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
     // bias accelerations with gravity as base acceleration (:526-547)
     for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
         for (uint32_t l = lane; l < nl; l += kWave) {
-            if (m.link_tree_depth[l] != depth) continue;
+            const LinkTree t = l == lane ? own : tree_of(l);
+            if (t.depth != depth) continue;
             float al[6];
-            const uint32_t parent = m.parent_link[l];
+            const uint32_t parent = t.parent;
             if (parent != kInvalid) {
                 float ap[6];
 #pragma unroll
                 for (int i = 0; i < 6; ++i) ap[i] = a[6u * parent + i];
                 mat66_vec(xup + 36u * l, ap, al);
-            } else if (m.joint_type[l] == kFloatingBase) {
+            } else if (t.type == kFloatingBase) {
                 const V3 g = rotate_inverse(base_rot, gravity);
                 al[0] = al[1] = al[2] = 0.0f; al[3] = -g.x; al[4] = -g.y; al[5] = -g.z;
             } else {
@@ -270,8 +289,9 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
     // leaf to root, children in CSR order (:557-569)
     for (uint32_t remaining = m.max_depth + 1u; remaining > 0u; --remaining) {
         for (uint32_t l = lane; l < nl; l += kWave) {
-            if (m.link_tree_depth[l] != remaining - 1u) continue;
-            for (uint32_t i = m.link_child_range[2u * l]; i < m.link_child_range[2u * l + 1u]; ++i) {
+            const LinkTree t = l == lane ? own : tree_of(l);
+            if (t.depth != remaining - 1u) continue;
+            for (uint32_t i = t.child_begin; i < t.child_end; ++i) {
                 const uint32_t child = m.link_children[i];
                 float pc[6], f[6];
 #pragma unroll
@@ -305,30 +325,28 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
     for (uint32_t e = lane; e < nl * 36u; e += kWave) ic[e] = m.link_inertia[e];
     for (uint32_t e = lane; e < n * ld; e += kWave) A[e] = 0.0f;
     __syncthreads();
-    for (uint32_t depth = m.max_depth; depth > 0u; --depth) {
-        for (uint32_t l = 0u; l < nl; ++l) {
-            if (m.link_tree_depth[l] + 1u != depth) continue;
-            for (uint32_t i = m.link_child_range[2u * l]; i < m.link_child_range[2u * l + 1u]; ++i) {
-                const uint32_t child = m.link_children[i];
-                const float* X = xup + 36u * child;
-                const float* C = ic + 36u * child;
-                const uint32_t row = lane / 6u, col = lane % 6u;
-                if (lane < 36u) {
-                    float value = 0.0f;
+    // deepest parents first, parents of one depth in link order, a parent's children in list order: the cooked visiting list
+    for (uint32_t visit = 0u; visit < nl; ++visit) {
+        const uint32_t child = m.link_push_order[visit];
+        if (child == kInvalid) break;
+        const uint32_t l = m.parent_link[child];
+        const float* X = xup + 36u * child;
+        const float* C = ic + 36u * child;
+        const uint32_t row = lane / 6u, col = lane % 6u;
+        if (lane < 36u) {
+            float value = 0.0f;
 #pragma unroll
-                    for (int k = 0; k < 6; ++k) value += C[row * 6u + k] * X[k * 6u + col];
-                    tmp[lane] = value;
-                }
-                __syncthreads();
-                if (lane < 36u) {
-                    float value = 0.0f;
-#pragma unroll
-                    for (int k = 0; k < 6; ++k) value += X[k * 6u + row] * tmp[k * 6u + col];
-                    ic[36u * l + lane] += value;
-                }
-                __syncthreads();
-            }
+            for (int k = 0; k < 6; ++k) value += C[row * 6u + k] * X[k * 6u + col];
+            tmp[lane] = value;
         }
+        __syncthreads();
+        if (lane < 36u) {
+            float value = 0.0f;
+#pragma unroll
+            for (int k = 0; k < 6; ++k) value += X[k * 6u + row] * tmp[k * 6u + col];
+            ic[36u * l + lane] += value;
+        }
+        __syncthreads();
     }
     const bool floating_root = m.floating_root != 0u;
     if (floating_root && lane < 36u) A[(lane / 6u) * ld + lane % 6u] = ic[lane];
@@ -461,10 +479,11 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
     // final link accelerations (:617-644)
     for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
         for (uint32_t l = lane; l < nl; l += kWave) {
-            if (m.link_tree_depth[l] != depth) continue;
+            const LinkTree t = l == lane ? own : tree_of(l);
+            if (t.depth != depth) continue;
             float al[6];
-            const uint32_t parent = m.parent_link[l];
-            if (m.joint_type[l] == kFloatingBase) {
+            const uint32_t parent = t.parent;
+            if (t.type == kFloatingBase) {
                 const V3 g = rotate_inverse(base_rot, gravity);
 #pragma unroll
                 for (int c = 0; c < 6; ++c) al[c] = acc[c];
@@ -479,7 +498,7 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
                     const float world[6] = {0.0f, 0.0f, 0.0f, -gravity.x, -gravity.y, -gravity.z};
                     mat66_vec(xup + 36u * l, world, al);
                 }
-                const float qdd = joint_dof(m.joint_type[l]) == 1u ? acc[m.link_dof[l]] : 0.0f;
+                const float qdd = joint_dof(t.type) == 1u ? acc[m.link_dof[l]] : 0.0f;
 #pragma unroll
                 for (int c = 0; c < 6; ++c) al[c] += vb[6u * l + c] + S[6u * l + c] * qdd;
             }
@@ -527,22 +546,40 @@ __global__ void __launch_bounds__(kWave) FkLinkVelocitiesKernel(ModelView m, Dat
     const size_t lbase = size_t{env} * nl;
     for (uint32_t e = lane; e < nl * 6u; e += kWave) v[e] = d.link_velocity[lbase * 6u + e];
     __syncthreads();
+    // the joint transform and the joint's own twist do not wait on the tree: a lane prepares its link's before the sweep
+    struct Jointed { uint32_t depth, parent; bool state; float X[36], own[6]; };
+    auto prepare = [&](uint32_t l, Jointed& t) {
+        const uint8_t type = m.joint_type[l];
+        t.depth = m.link_tree_depth[l]; t.parent = m.parent_link[l];
+        t.state = t.parent == kInvalid && type == kFloatingBase;   // a floating root's twist is state
+        if (t.state) return;
+        float s[6];
+        joint_transform(m, l, d.q[lbase + l], t.X);
+        motion_subspace(type, load3(m.joint_axis + 3u * l), s);
+        const float qdl = d.qdot[lbase + l];
+#pragma unroll
+        for (int c = 0; c < 6; ++c) t.own[c] = s[c] * qdl;
+    };
+    auto propagate = [&](uint32_t l, const Jointed& t) {
+        if (t.state) return;
+        float pv[6] = {0, 0, 0, 0, 0, 0}, vl[6];
+        if (t.parent != kInvalid) {
+#pragma unroll
+            for (int i = 0; i < 6; ++i) pv[i] = v[6u * t.parent + i];
+        }
+        mat66_vec(t.X, pv, vl);
+#pragma unroll
+        for (int c = 0; c < 6; ++c) v[6u * l + c] = vl[c] + t.own[c];
+    };
+    Jointed own;
+    own.depth = kInvalid; own.parent = kInvalid; own.state = true;
+    if (lane < nl) prepare(lane, own);
     for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
-        for (uint32_t l = lane; l < nl; l += kWave) {
-            if (m.link_tree_depth[l] != depth) continue;
-            const uint32_t parent = m.parent_link[l];
-            if (parent == kInvalid && m.joint_type[l] == kFloatingBase) continue;
-            float pv[6] = {0, 0, 0, 0, 0, 0}, X[36], s[6], vl[6];
-            if (parent != kInvalid) {
-#pragma unroll
-                for (int i = 0; i < 6; ++i) pv[i] = v[6u * parent + i];
-            }
-            joint_transform(m, l, d.q[lbase + l], X);
-            motion_subspace(m.joint_type[l], load3(m.joint_axis + 3u * l), s);
-            mat66_vec(X, pv, vl);
-            const float qdl = d.qdot[lbase + l];
-#pragma unroll
-            for (int c = 0; c < 6; ++c) v[6u * l + c] = vl[c] + s[c] * qdl;
+        if (own.depth == depth) propagate(lane, own);
+        for (uint32_t l = lane + kWave; l < nl; l += kWave) {
+            Jointed t;
+            prepare(l, t);
+            if (t.depth == depth) propagate(l, t);
         }
         __syncthreads();
     }
