@@ -966,19 +966,65 @@ __device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& 
     PROF_END(c, 25);
 }
 
+// The search always evaluates the line at 0 and then at 1.  With at most sixteen heads, none of them general, the rows
+// of sixteen lanes hold copies of the same heads (lane & 15) and the row sums stay within a row: the first row
+// evaluates the line at 0 while the others evaluate it at 1, one pass for both points with the numbers either gives
+// alone.  Each point's sums come out in its row's lanes.
+struct LinePoint { float slope, curvature, magnitude; };
+__device__ __forceinline__ void line_derivatives_pair(const Tile& c, const PlainLine& plain, float inertial_slope, float inertial_curvature,
+                                                      LinePoint* at_zero, LinePoint* at_one) {
+    PROF_COUNT(c, 1);
+    const float alpha = c.lane < 16u ? 0.0f : 1.0f;
+    TileSum row_slope{0.0f, 0.0f};
+    float row_curvature = 0.0f, row_magnitude = 0.0f;
+    plain_line_terms(plain, alpha, row_slope, row_curvature, row_magnitude);
+    TileSum total{-row_slope.value, -row_slope.error};
+    if ((c.lane & 15u) == 0u) {
+        tile_add_product(total, alpha, inertial_curvature);
+        tile_add(total, inertial_slope);
+    }
+    tile_merge(total, dpp_move<kDppXor1>(total.value), dpp_move<kDppXor1>(total.error));
+    tile_merge(total, dpp_move<kDppXor2>(total.value), dpp_move<kDppXor2>(total.error));
+    tile_merge(total, dpp_move<kDppHalfMirror>(total.value), dpp_move<kDppHalfMirror>(total.error));
+    tile_merge(total, dpp_move<kDppMirror>(total.value), dpp_move<kDppMirror>(total.error));
+    float cv = row_curvature, mg = row_magnitude;
+    cv += dpp_move<kDppXor1>(cv); cv += dpp_move<kDppXor2>(cv); cv += dpp_move<kDppHalfMirror>(cv); cv += dpp_move<kDppMirror>(cv);
+    mg += dpp_move<kDppXor1>(mg); mg += dpp_move<kDppXor2>(mg); mg += dpp_move<kDppHalfMirror>(mg); mg += dpp_move<kDppMirror>(mg);
+    at_zero->slope = row_value(total.value, 0) + row_value(total.error, 0);
+    at_zero->curvature = inertial_curvature + row_value(cv, 0);
+    at_zero->magnitude = fabsf(inertial_slope) + 0.0f * inertial_curvature + row_value(mg, 0);
+    at_one->slope = row_value(total.value, 1) + row_value(total.error, 1);
+    at_one->curvature = inertial_curvature + row_value(cv, 1);
+    at_one->magnitude = fabsf(inertial_slope) + 1.0f * inertial_curvature + row_value(mg, 1);
+}
+
 // SearchTileLine (:2089-2125)
 __device__ __forceinline__ float search_line(const Tile& c, float inertial_slope, float inertial_curvature) {
     float slope = 0.0f, curvature = 0.0f, magnitude = 0.0f;
-    const HeadLine mine = load_head_line(c, c.lane);
     const bool general = c.heads > uint32_t(kWave) || c.elliptic;
+    const bool paired = !general && c.heads <= 16u;
+    const HeadLine mine = load_head_line(c, paired ? (c.lane & 15u) : c.lane);
     const PlainLine plain = plain_line(mine);
-    line_derivatives(c, mine, plain, general, 0.0f, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
+    LinePoint at_one{0.0f, 0.0f, 0.0f};
+    if (paired) {
+        LinePoint at_zero;
+        line_derivatives_pair(c, plain, inertial_slope, inertial_curvature, &at_zero, &at_one);
+        c.work += 1u;
+        slope = at_zero.slope;
+    } else {
+        line_derivatives(c, mine, plain, general, 0.0f, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
+    }
     const float initial = slope;
     if (!(initial < 0.0f)) return 0.0f;
     float low = 0.0f, high = 0.0f, alpha = 1.0f;
     bool bounded = false;
     for (uint32_t step = 0u; step < kLineSearchSteps; ++step) {
-        line_derivatives(c, mine, plain, general, alpha, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
+        if (paired && step == 0u) {
+            slope = at_one.slope; curvature = at_one.curvature; magnitude = at_one.magnitude;
+            c.work += 1u;
+        } else {
+            line_derivatives(c, mine, plain, general, alpha, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
+        }
         if (!isfinite(slope) || !isfinite(curvature)) {
             high = alpha; bounded = true; alpha = 0.5f * (low + high);
             continue;
