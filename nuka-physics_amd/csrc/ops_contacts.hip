@@ -863,6 +863,10 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
     float* row_point = reinterpret_cast<float*>(row_merge + CR);   // 3 CR
     float* row_dir = row_point + 3u * CR;                // 3 CR, side A's direction (side B's is its negative)
     float* row_gain = row_dir + 3u * CR;                 // CR: a compliant row's gain on the start velocity along it, else 0
+    // nl: the coordinates on each link's path to the root (2 S + 10 CR words come before: an even count, so 8-byte aligned);
+    // the chain Jacobian pass asks for a link's mask once a row and side and would wait on the table each time
+    uint64_t* link_mask = reinterpret_cast<uint64_t*>(row_gain + CR);
+    for (uint32_t l = lane; l < nl; l += kWave) link_mask[l] = m.link_dof_mask[l];
     Row* rows = reinterpret_cast<Row*>(d.urows) + size_t{env} * R;
     float* lambda = d.lambda + size_t{env} * R;
     float* pen = d.row_penetration + size_t{env} * R;
@@ -1178,42 +1182,64 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
     // only the rows below this step's extent can have a link; the rows up to the previous extent were cleared above
     const uint32_t bound = min(extent - 1u, CR);
     const float start_velocity = m.any_mujoco != 0u && lane < md ? d.step_qdot_flat[size_t{env} * md + lane] : 0.0f;
-    for (uint32_t r = 0u; r < bound; ++r) {
-        const uint32_t links[2] = {row_link_a[r], row_link_b[r]};
-        if (links[0] == kInvalid && links[1] == kInvalid) continue;
-        const V3 point{row_point[3u * r], row_point[3u * r + 1u], row_point[3u * r + 2u]};
-        const V3 dir_a{row_dir[3u * r], row_dir[3u * r + 1u], row_dir[3u * r + 2u]};
-        float entries[2] = {0.0f, 0.0f};
-        for (uint32_t side = 0u; side < 2u; ++side) {
-            if (links[side] == kInvalid) continue;
-            const uint32_t link = links[side] - env * nl;
-            const V3 dir = side == 0u ? dir_a : V3{-dir_a.x, -dir_a.y, -dir_a.z};
-            float entry = 0.0f;
-            if (lane < m.dof && ((m.link_dof_mask[link] >> lane) & 1ull) != 0ull) {
-                if (mode == 1u) entry = dot3(cross3(axis_world, sub3(point, origin)), dir) + dot3(axis_world, V3{0, 0, 0});
-                else if (mode == 2u) entry = dot3(axis_world, dir);
-                else if (mode == 3u) entry = dot3(cross3(axis_world, sub3(point, origin)), dir) + dot3(axis_world, V3{0, 0, 0});
-                else if (mode == 4u) entry = dot3(axis_world, dir);
+    // Sixty-four rows at a time: every lane first fetches one row's endpoints, point, direction, gain and its links' masks
+    // (one round of LDS reads, all in flight together), then the rows go by in turn with their values handed round as
+    // lane reads - a row no longer waits on its own chain of dependent reads.
+    auto uniform_word = [](uint32_t v, uint32_t from) { return uint32_t(__builtin_amdgcn_readlane(int(v), int(from))); };
+    for (uint32_t first = 0u; first < bound; first += kWave) {
+        const uint32_t mine = first + lane;
+        uint32_t my_link[2] = {kInvalid, kInvalid}, my_merge = 0u, my_mask[2][2] = {{0u, 0u}, {0u, 0u}};
+        float my_point[3] = {0.0f, 0.0f, 0.0f}, my_dir[3] = {0.0f, 0.0f, 0.0f}, my_gain = 0.0f;
+        if (mine < bound) {
+            my_link[0] = row_link_a[mine]; my_link[1] = row_link_b[mine]; my_merge = row_merge[mine]; my_gain = row_gain[mine];
+#pragma unroll
+            for (int k = 0; k < 3; ++k) { my_point[k] = row_point[3u * mine + k]; my_dir[k] = row_dir[3u * mine + k]; }
+#pragma unroll
+            for (int side = 0; side < 2; ++side) {
+                if (my_link[side] == kInvalid) continue;
+                const uint64_t mask = link_mask[my_link[side] - env * nl];
+                my_mask[side][0] = uint32_t(mask); my_mask[side][1] = uint32_t(mask >> 32u);
             }
-            entries[side] = entry;
         }
-        if (row_merge[r] != 0u) { entries[0] += entries[1]; entries[1] = 0.0f; }   // shared owner (:172-186)
-        if (lane < md) {
-            if (links[0] != kInvalid) d.chain_jacobian[(size_t{env} * R + r) * md + lane] = entries[0];
-            if (links[1] != kInvalid) d.chain_jacobian_b[(size_t{env} * R + r) * md + lane] = entries[1];
-        }
-        // PrepareContactRowsKernel (:1134-1140): a compliant row's reference acceleration includes the damping of the
-        // velocity the step started from along the row, ContactReferenceVelocity (:1072-1100): side A's coordinates in
-        // order, then side B's
-        const float gain = row_gain[r];
-        if (gain != 0.0f) {
-            float velocity = 0.0f;
-            for (uint32_t side = 0u; side < 2u; ++side) {
+        const uint32_t count = min(uint32_t(kWave), bound - first);
+        for (uint32_t i = 0u; i < count; ++i) {
+            const uint32_t r = first + i;
+            const uint32_t links[2] = {uniform_word(my_link[0], i), uniform_word(my_link[1], i)};
+            if (links[0] == kInvalid && links[1] == kInvalid) continue;
+            const V3 point{uniform_value(my_point[0], i), uniform_value(my_point[1], i), uniform_value(my_point[2], i)};
+            const V3 dir_a{uniform_value(my_dir[0], i), uniform_value(my_dir[1], i), uniform_value(my_dir[2], i)};
+            float entries[2] = {0.0f, 0.0f};
+#pragma unroll
+            for (int side = 0; side < 2; ++side) {
                 if (links[side] == kInvalid) continue;
-                const float term = entries[side] * start_velocity;
-                for (uint32_t k = 0u; k < md; ++k) velocity += uniform_value(term, k);
+                const uint64_t mask = (uint64_t(uniform_word(my_mask[side][1], i)) << 32u) | uint64_t(uniform_word(my_mask[side][0], i));
+                const V3 dir = side == 0 ? dir_a : V3{-dir_a.x, -dir_a.y, -dir_a.z};
+                // a turning coordinate (hinge, base angular) takes the moment of the direction about its axis, a sliding
+                // one (prismatic, base linear) the direction along it: both evaluated, one selected, so that lanes of
+                // different kinds do not take turns
+                const float turning = dot3(cross3(axis_world, sub3(point, origin)), dir) + dot3(axis_world, V3{0, 0, 0});
+                const float sliding = dot3(axis_world, dir);
+                const bool on_path = lane < m.dof && ((mask >> lane) & 1ull) != 0ull;
+                entries[side] = !on_path || mode == 0u ? 0.0f : ((mode & 1u) != 0u ? turning : sliding);
             }
-            if (lane == 0u) rows[r].rhs += gain * velocity;
+            if (uniform_word(my_merge, i) != 0u) { entries[0] += entries[1]; entries[1] = 0.0f; }   // shared owner (:172-186)
+            if (lane < md) {
+                if (links[0] != kInvalid) d.chain_jacobian[(size_t{env} * R + r) * md + lane] = entries[0];
+                if (links[1] != kInvalid) d.chain_jacobian_b[(size_t{env} * R + r) * md + lane] = entries[1];
+            }
+            // PrepareContactRowsKernel (:1134-1140): a compliant row's reference acceleration includes the damping of the
+            // velocity the step started from along the row, ContactReferenceVelocity (:1072-1100): side A's coordinates
+            // in order, then side B's
+            const float gain = uniform_value(my_gain, i);
+            if (gain != 0.0f) {
+                float velocity = 0.0f;
+                for (uint32_t side = 0u; side < 2u; ++side) {
+                    if (links[side] == kInvalid) continue;
+                    const float term = entries[side] * start_velocity;
+                    for (uint32_t k = 0u; k < md; ++k) velocity += uniform_value(term, k);
+                }
+                if (lane == 0u) rows[r].rhs += gain * velocity;
+            }
         }
     }
 }
@@ -1272,7 +1298,7 @@ Status OpAssembleRows(const ModelView& m, const DataView& d, const void* params,
     if (p == nullptr) return Status::Failed;
     if (p->env_count == 0u || p->rows_per_env == 0u) return Status::Ok;
     if (p->max_dof > kMaxDof) return Status::InvalidArgument;
-    const size_t lds = (size_t{p->union_slot_count} * 2u + size_t{p->contact_rows_per_env} * 10u) * sizeof(uint32_t);
+    const size_t lds = (size_t{p->union_slot_count} * 2u + size_t{p->contact_rows_per_env} * 10u + size_t{m.links_per_env} * 2u) * sizeof(uint32_t);
     if (lds > 150u * 1024u) return Status::InvalidArgument;
     hipLaunchKernelGGL(AssembleRowsKernel, dim3(p->env_count), dim3(kWave), lds, stream, m, d, *p);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
