@@ -325,28 +325,36 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
     for (uint32_t e = lane; e < nl * 36u; e += kWave) ic[e] = m.link_inertia[e];
     for (uint32_t e = lane; e < n * ld; e += kWave) A[e] = 0.0f;
     __syncthreads();
-    // deepest parents first, parents of one depth in link order, a parent's children in list order: the cooked visiting list
-    for (uint32_t visit = 0u; visit < nl; ++visit) {
-        const uint32_t child = m.link_push_order[visit];
-        if (child == kInvalid) break;
-        const uint32_t l = m.parent_link[child];
-        const float* X = xup + 36u * child;
-        const float* C = ic + 36u * child;
-        const uint32_t row = lane / 6u, col = lane % 6u;
-        if (lane < 36u) {
-            float value = 0.0f;
-#pragma unroll
-            for (int k = 0; k < 6; ++k) value += C[row * 6u + k] * X[k * 6u + col];
-            tmp[lane] = value;
+    // deepest parents first, parents of one depth in link order, a parent's children in list order: the cooked visiting
+    // list, sixty-four visits at a time - a lane reads one visit's child and parent, the visits take theirs as lane reads
+    for (uint32_t first = 0u; first < nl; first += kWave) {
+        uint32_t my_child = kInvalid, my_parent = 0u;
+        if (first + lane < nl) {
+            my_child = m.link_push_order[first + lane];
+            if (my_child != kInvalid) my_parent = m.parent_link[my_child];
         }
-        __syncthreads();
-        if (lane < 36u) {
-            float value = 0.0f;
+        for (uint32_t visit = 0u; visit < uint32_t(kWave); ++visit) {
+            const uint32_t child = uint32_t(__builtin_amdgcn_readlane(int(my_child), int(visit)));
+            if (child == kInvalid) break;
+            const uint32_t l = uint32_t(__builtin_amdgcn_readlane(int(my_parent), int(visit)));
+            const float* X = xup + 36u * child;
+            const float* C = ic + 36u * child;
+            const uint32_t row = lane / 6u, col = lane % 6u;
+            if (lane < 36u) {
+                float value = 0.0f;
 #pragma unroll
-            for (int k = 0; k < 6; ++k) value += X[k * 6u + row] * tmp[k * 6u + col];
-            ic[36u * l + lane] += value;
+                for (int k = 0; k < 6; ++k) value += C[row * 6u + k] * X[k * 6u + col];
+                tmp[lane] = value;
+            }
+            __syncthreads();
+            if (lane < 36u) {
+                float value = 0.0f;
+#pragma unroll
+                for (int k = 0; k < 6; ++k) value += X[k * 6u + row] * tmp[k * 6u + col];
+                ic[36u * l + lane] += value;
+            }
+            __syncthreads();
         }
-        __syncthreads();
     }
     const bool floating_root = m.floating_root != 0u;
     if (floating_root && lane < 36u) A[(lane / 6u) * ld + lane % 6u] = ic[lane];
