@@ -69,6 +69,7 @@ struct ModelView {
     uint32_t profile_count, floating_root;
     uint32_t max_points_per_slot;   // most points a manifold of the template's admitted pairs can hold (sizes the solver's staged rows)
     uint32_t excluded_pair_count;
+    uint32_t pairable_count;   // collidable rows that can pass the shape filter with some partner (pairable_rows, ascending)
     // joint row slots after the contact rows: 2 per link, 1 per link, 1 per link, or 0 (scene/cook/cook_to_model.cpp:706-719)
     uint32_t joint_limit_rows, joint_friction_rows, joint_drive_rows, drive_mode;
     // the MuJoCo contact law: some profile is MuJoCo-sourced; the cone of its contacts (0 pyramidal, 1 elliptic) and impratio
@@ -111,6 +112,7 @@ struct ModelView {
     const uint32_t* body_collidable_link;
     const uint32_t* body_collidable_body;
     const float* body_collidable_local;
+    const uint32_t* pairable_rows;
     const float* profile_mu;
     const uint32_t* profile_law;      // [profile] 1: MuJoCo-sourced (constraint/law_source.hpp)
     const float* profile_solref;      // [profile][2]

@@ -114,18 +114,22 @@ __device__ bool pair_excluded(const ModelView& m, uint32_t a, uint32_t b) {
 }
 
 // ---- candidate pairs: one wavefront per env walks the (i, j) grid in row-major order; the ballot rank of an
-// emitting lane is its slot, which is the ascending (a, b) order the reference reaches by sorting. ----
+// emitting lane is its slot, which is the ascending (a, b) order the reference reaches by sorting.  The grid runs over
+// the rows that can pass the shape filter at all (a row with empty type and affinity masks pairs with nothing): a
+// humanoid's 31 shapeless link rows leave a grid of 13 x 13 out of 44 x 44. ----
 __global__ void __launch_bounds__(kWave) QueryPairsKernel(ModelView m, DataView d, LbvhQueryPairsParams p) {
-    const uint32_t env = blockIdx.x, lane = threadIdx.x, N = p.bodies_per_env;
-    const size_t bbase = size_t{env} * N;
+    const uint32_t env = blockIdx.x, lane = threadIdx.x, N = m.pairable_count;
+    const size_t bbase = size_t{env} * p.bodies_per_env;
     const uint32_t capacity = min(p.rigid_slot_cap, p.max_pairs);
     uint32_t* pairs = d.candidate_pairs + size_t{env} * p.max_contacts_per_env * 2u;
     uint32_t count = 0u;
     bool overflow = false;
     for (uint32_t base = 0u; base < N * N; base += kWave) {
-        const uint32_t item = base + lane, i = item / N, j = item % N;
+        const uint32_t item = base + lane, at_i = item / N, at_j = item % N;
         bool emit = false;
-        if (i < j && i < N) {
+        uint32_t i = 0u, j = 0u;
+        if (at_i < at_j && at_i < N) {
+            i = m.pairable_rows[at_i]; j = m.pairable_rows[at_j];
             const float* alo = d.body_aabb_lo + (bbase + i) * 3u, *ahi = d.body_aabb_hi + (bbase + i) * 3u;
             const float* blo = d.body_aabb_lo + (bbase + j) * 3u, *bhi = d.body_aabb_hi + (bbase + j) * 3u;
             const bool overlap = !(ahi[0] < blo[0] || alo[0] > bhi[0] || ahi[1] < blo[1] || alo[1] > bhi[1] ||

@@ -63,7 +63,7 @@ struct HostModel {
     ModelView counts{};   // scalar members only
     std::vector<uint8_t> joint_type, joint_limit_flags, joint_law;
     std::vector<uint32_t> parent_link, link_body, link_tree_depth, link_child_range, link_children, link_push_order, link_dof, dof_link, dof_component,
-        link_geom_kind, body_to_link, body_to_articulation, body_collidable_link, body_collidable_body;
+        link_geom_kind, body_to_link, body_to_articulation, body_collidable_link, body_collidable_body, pairable_rows;
     std::vector<uint64_t> link_dof_mask, excluded_pairs;
     std::vector<float> joint_axis, parent_offset, link_local_pose, link_inertial_frame, link_inertia, joint_damping, joint_armature,
         joint_stiffness, joint_spring_reference, joint_limit_lower, joint_limit_upper, joint_frictionloss, link_geom_local, shape_table, body_collidable_local, body_init_pose, profile_mu,
@@ -315,6 +315,12 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
     c.floating_root = m.joint_type[0] == kFloatingBase ? 1u : 0u;
     c.max_points_per_slot = max_points;
     c.excluded_pair_count = uint32_t(m.excluded_pairs.size());
+    // rows whose type and affinity masks are both empty pass the filter with no partner (shape_kind.hpp:26-33): the pair
+    // query walks the grid of the other rows only, in the same ascending order
+    m.pairable_rows.clear();
+    for (uint32_t b = 0u; b < nb; ++b) if ((d.shape_contype[b] | d.shape_conaffinity[b]) != 0u) m.pairable_rows.push_back(b);
+    c.pairable_count = uint32_t(m.pairable_rows.size());
+    m.pairable_rows.resize(nb, kInvalid);
 }
 
 enum Dtype : uint8_t { kF32 = 0, kU32 = 1, kU64 = 2, kU8 = 3 };
@@ -363,7 +369,7 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(joint_friction_reference, kF32) X(link_body, kU32) X(link_tree_depth, kU32) X(link_child_range, kU32) X(link_children, kU32) X(link_push_order, kU32) \
     X(link_dof, kU32) X(dof_link, kU32) X(dof_component, kU32) X(link_dof_mask, kU64) X(link_geom_kind, kU32) \
     X(link_geom_local, kF32) X(shape_table, kF32) X(body_to_link, kU32) X(body_to_articulation, kU32) \
-    X(body_collidable_link, kU32) X(body_collidable_body, kU32) X(body_collidable_local, kF32) X(profile_mu, kF32) \
+    X(body_collidable_link, kU32) X(body_collidable_body, kU32) X(body_collidable_local, kF32) X(pairable_rows, kU32) X(profile_mu, kF32) \
     X(profile_law, kU32) X(profile_solref, kF32) X(profile_solimp, kF32) X(profile_margin, kF32) X(profile_mix, kF32) \
     X(excluded_pairs, kU64)
 
