@@ -252,7 +252,7 @@ __device__ void reduce_and_emit_spread(const V3* position, const float* pen, con
 // collision/primitive_surface.hpp:28-122 QueryPrimitiveSurface: signed distance (positive outside), outward normal,
 // closest surface point and feature of a point in the primitive's own frame
 struct Surface { float distance; V3 normal, point; uint32_t feature; bool valid; };
-__device__ Surface query_surface(uint32_t kind, V3 par, V3 pos) {
+__device__ __forceinline__ Surface query_surface(uint32_t kind, V3 par, V3 pos) {
     Surface r{0.0f, V3{1, 0, 0}, V3{0, 0, 0}, 0u, false};
     if (kind == kShapeSphere || kind == kShapeCapsule) {
         if (!(par.x >= 0.0f)) return r;
@@ -308,10 +308,10 @@ __device__ Surface query_surface(uint32_t kind, V3 par, V3 pos) {
     return r;
 }
 
-__device__ void emit_one(Manifold* out, V3 position, V3 normal, float pen, uint32_t key) {
+__device__ __forceinline__ void emit_one(Manifold* out, V3 position, V3 normal, float pen, uint32_t key) {
     out->position[0] = position; out->normal = normal; out->penetration[0] = pen; out->key[0] = key; out->count = 1u;
 }
-__device__ void sphere_sphere(const Prim& a, const Prim& b, float query, Manifold* out) {   // :416-429
+__device__ __forceinline__ void sphere_sphere(const Prim& a, const Prim& b, float query, Manifold* out) {   // :416-429
     out->count = 0u;
     const V3 delta = sub3(a.t, b.t);
     const float dist = sqrtf(delta.x * delta.x + delta.y * delta.y + delta.z * delta.z);
@@ -320,7 +320,7 @@ __device__ void sphere_sphere(const Prim& a, const Prim& b, float query, Manifol
     const V3 n = norm_or(delta, V3{0, 1, 0});
     emit_one(out, add3(b.t, scale3(n, b.radius - 0.5f * pen)), n, pen, 0u);
 }
-__device__ void sphere_box(const Prim& sph, const Prim& box, float query, Manifold* out) {   // :434-448
+__device__ __forceinline__ void sphere_box(const Prim& sph, const Prim& box, float query, Manifold* out) {   // :434-448
     out->count = 0u;
     const Surface s = query_surface(kShapeBox, box.half, frame_world_to_local(box, sph.t));
     if (!s.valid) return;
@@ -329,7 +329,7 @@ __device__ void sphere_box(const Prim& sph, const Prim& box, float query, Manifo
     const V3 normal = frame_dir_to_world(box, s.normal);
     emit_one(out, sub3(frame_local_to_world(box, s.point), scale3(normal, 0.5f * pen)), normal, pen, 0u);
 }
-__device__ void sphere_plane(const Prim& sph, const Prim& plane, float query, Manifold* out) {   // :451-463
+__device__ __forceinline__ void sphere_plane(const Prim& sph, const Prim& plane, float query, Manifold* out) {   // :451-463
     out->count = 0u;
     const V3 n = norm_or(plane.cz, V3{0, 0, 1});
     const float signed_dist = dot3(sub3(sph.t, plane.t), n);
@@ -368,7 +368,7 @@ __device__ void capsule_plane(const Prim& cap, const Prim& plane, float query, M
     }
     reduce_and_emit(position, pen, feature, ncand, n, out);
 }
-__device__ void capsule_sphere(const Prim& cap, const Prim& sph, float query, Manifold* out) {   // :764-778
+__device__ __forceinline__ void capsule_sphere(const Prim& cap, const Prim& sph, float query, Manifold* out) {   // :764-778
     out->count = 0u;
     const Surface s = query_surface(kShapeCapsule, V3{cap.radius, cap.half_height, 0.0f}, frame_world_to_local(cap, sph.t));
     if (!s.valid) return;
@@ -406,7 +406,7 @@ __device__ void cylinder_plane(const Prim& cyl, const Prim& plane, float query, 
     }
     reduce_and_emit_spread(position, pen, feature, ncand, n, out);
 }
-__device__ void cylinder_sphere(const Prim& cyl, const Prim& sph, float query, Manifold* out) {   // :819-834
+__device__ __forceinline__ void cylinder_sphere(const Prim& cyl, const Prim& sph, float query, Manifold* out) {   // :819-834
     out->count = 0u;
     const Surface s = query_surface(kShapeCylinder, V3{cyl.radius, cyl.half_height, 0.0f}, frame_world_to_local(cyl, sph.t));
     if (!s.valid) return;
@@ -417,7 +417,7 @@ __device__ void cylinder_sphere(const Prim& cyl, const Prim& sph, float query, M
 }
 // :841-896 ClosestPtSegmentSegment (fixed branch order)
 __device__ __forceinline__ float clamp01(float v) { return v < 0.0f ? 0.0f : (v > 1.0f ? 1.0f : v); }
-__device__ float closest_segment_segment(V3 p1, V3 q1, V3 p2, V3 q2, V3* c1_out, V3* c2_out) {
+__device__ __forceinline__ float closest_segment_segment(V3 p1, V3 q1, V3 p2, V3 q2, V3* c1_out, V3* c2_out) {
     const V3 d1 = sub3(q1, p1), d2 = sub3(q2, p2), r = sub3(p1, p2);
     const float a = dot3(d1, d1), e = dot3(d2, d2), f = dot3(d2, r);
     float s = 0.0f, t = 0.0f;
@@ -441,7 +441,7 @@ __device__ float closest_segment_segment(V3 p1, V3 q1, V3 p2, V3 q2, V3* c1_out,
     const V3 dv = sub3(c1, c2);
     return dot3(dv, dv);
 }
-__device__ void capsule_capsule(const Prim& a, const Prim& b, float query, Manifold* out) {   // :905-932
+__device__ __forceinline__ void capsule_capsule(const Prim& a, const Prim& b, float query, Manifold* out) {   // :905-932
     out->count = 0u;
     const V3 a0 = add3(a.t, scale3(a.cz, a.half_height)), a1 = sub3(a.t, scale3(a.cz, a.half_height));
     const V3 b0 = add3(b.t, scale3(b.cz, b.half_height)), b1 = sub3(b.t, scale3(b.cz, b.half_height));
@@ -601,6 +601,25 @@ __device__ void primitive_pair(uint32_t ka, const Prim& a, uint32_t kb, const Pr
     out->normal = V3{-out->normal.x, -out->normal.y, -out->normal.z};
 }
 
+// The pairs whose manifold is one point at most: a sphere against anything, capsule against capsule.  A world whose
+// admitted pairs are all of these (ModelView::max_points_per_slot == 1) runs the narrowphase on this dispatch alone:
+// nothing in it indexes a local array by a run-time value, so the manifold stays in registers and the kernel takes no
+// scratch memory (the general dispatch clips polygons and reduces candidate lists in local arrays).
+__device__ __forceinline__ void primitive_pair_single(uint32_t ka, const Prim& a, uint32_t kb, const Prim& b, float query, Manifold* out) {
+    out->count = 0u;
+    if (ka == kShapeSphere && kb == kShapeSphere) { sphere_sphere(a, b, query, out); return; }
+    if (ka == kShapeSphere && kb == kShapeBox) { sphere_box(a, b, query, out); return; }
+    if (ka == kShapeSphere && kb == kShapePlane) { sphere_plane(a, b, query, out); return; }
+    if (ka == kShapeCapsule && kb == kShapeSphere) { capsule_sphere(a, b, query, out); return; }
+    if (ka == kShapeCapsule && kb == kShapeCapsule) { capsule_capsule(a, b, query, out); return; }
+    if (ka == kShapeCylinder && kb == kShapeSphere) { cylinder_sphere(a, b, query, out); return; }
+    if (ka == kShapeBox && kb == kShapeSphere) sphere_box(b, a, query, out);
+    else if (ka == kShapePlane && kb == kShapeSphere) sphere_plane(b, a, query, out);
+    else if (ka == kShapeSphere && kb == kShapeCapsule) capsule_sphere(b, a, query, out);
+    else if (ka == kShapeSphere && kb == kShapeCylinder) cylinder_sphere(b, a, query, out);
+    out->normal = V3{-out->normal.x, -out->normal.y, -out->normal.z};
+}
+
 // nk/contact/contact_identity.hpp:98-157
 __device__ __forceinline__ int32_t quantize_coord(float value) {
     const float scaled = value * 4096.0f;
@@ -622,8 +641,10 @@ __device__ V3 inverse_transform_point(Xf xf, V3 wp) {   // prims_types.cuh:98-10
 }
 
 // ---- NarrowphasePrimitives: one thread per (env, slot) (narrowphase_prims.cu:181-366, analytic route) ----
-__device__ uint32_t NarrowphaseSlot(const ModelView& m, const DataView& d, const NarrowphasePrimitivesParams& p, uint32_t env,
-                                    uint32_t slot) {
+template <bool kSinglePoint>
+__device__ __forceinline__ uint32_t NarrowphaseSlot(const ModelView& m, const DataView& d, const NarrowphasePrimitivesParams& p, uint32_t env,
+                                                    uint32_t slot) {
+    constexpr uint32_t kPoints = kSinglePoint ? 1u : 4u;
     const size_t gid = size_t{env} * p.union_slot_count + slot;
     const size_t bbase = size_t{env} * p.bodies_per_env;
     const float separation = fmaxf(p.contact_margin, 0.0005f);
@@ -647,12 +668,18 @@ __device__ uint32_t NarrowphaseSlot(const ModelView& m, const DataView& d, const
             query_margin = margin_a + margin_b;
         }
         const float query = fmaxf(query_margin, fminf(motion_radius(2.0f * separation, p.dt, 0.0f, 0.0f, 0.9f), p.query_reach));
-        primitive_pair(sa.kind, pa, sb.kind, pb, query, &mf);
-        if (law != kContactLawCompliant) for (uint32_t i = 0u; i < mf.count; ++i) mf.penetration[i] += separation;
+        if constexpr (kSinglePoint) primitive_pair_single(sa.kind, pa, sb.kind, pb, query, &mf);
+        else primitive_pair(sa.kind, pa, sb.kind, pb, query, &mf);
+        if (law != kContactLawCompliant) {
+#pragma unroll
+            for (uint32_t i = 0u; i < kPoints; ++i) if (i < mf.count) mf.penetration[i] += separation;
+        }
     }
     d.ucontact_count[gid] = mf.count;
     d.ucontact_law[gid] = law;
-    for (uint32_t i = 0u; i < mf.count; ++i) {
+#pragma unroll
+    for (uint32_t i = 0u; i < kPoints; ++i) {
+        if (i >= mf.count) break;
         const size_t at = gid * 4u + i;
         d.ucontact_point[3u * at] = mf.position[i].x; d.ucontact_point[3u * at + 1u] = mf.position[i].y; d.ucontact_point[3u * at + 2u] = mf.position[i].z;
         d.ucontact_normal[3u * at] = mf.normal.x; d.ucontact_normal[3u * at + 1u] = mf.normal.y; d.ucontact_normal[3u * at + 2u] = mf.normal.z;
@@ -671,12 +698,13 @@ __device__ uint32_t NarrowphaseSlot(const ModelView& m, const DataView& d, const
 
 // One wavefront per environment; its lanes take the environment's slots in strides of 64, and the per-environment
 // contact count is a wave sum (no atomics).
+template <bool kSinglePoint>
 __global__ void __launch_bounds__(64) NarrowphaseKernel(ModelView m, DataView d, NarrowphasePrimitivesParams p) {
     const uint32_t env = blockIdx.x, lane = threadIdx.x;
     uint32_t contacts = 0u;
     for (uint32_t first = 0u; first < p.rigid_slot_cap; first += 64u) {
         const uint32_t slot = first + lane;
-        if (slot < p.rigid_slot_cap) contacts += NarrowphaseSlot(m, d, p, env, slot);
+        if (slot < p.rigid_slot_cap) contacts += NarrowphaseSlot<kSinglePoint>(m, d, p, env, slot);
     }
     contacts = wave_sum_u(contacts);
     if (lane == 0u) d.contact_count[env] = contacts;
@@ -854,7 +882,8 @@ __device__ __forceinline__ float uniform_value(float v, uint32_t lane) {   // `l
 }
 
 // ---- AssembleRows: one wavefront per environment (assemble_rows.cu:325-394, 200-214, 406-801, 122-186) ----
-__global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataView d, AssembleRowsParams p) {
+// four waves a SIMD (128 registers a lane): sixteen environments a compute unit are resident at once at 4096 environments
+__global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4, 4))) AssembleRowsKernel(ModelView m, DataView d, AssembleRowsParams p) {
     extern __shared__ uint32_t lds_u[];
     const uint32_t env = blockIdx.x, lane = threadIdx.x;
     const uint32_t R = p.rows_per_env, S = p.union_slot_count, CR = p.contact_rows_per_env, md = p.max_dof, nl = m.links_per_env;
@@ -971,8 +1000,9 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
             const size_t mp = gid * 4u + pt;
             // the velocity laws keep every point; a compliant point lives inside its margin (:625-626)
             const bool live = pt < n_active && pt < 4u && (!mujoco || d.ucontact_depth[mp] + margin > 0.0f);
-            const uint32_t row_of[4] = {base + pt, base + P + pt, base + 2u * P + pt, base + 3u * P + pt};
-            V3 n{0, 0, 1}, point{0, 0, 0}, dirs[4];
+            // the rows' directions as four values selected by the row's place, not an array indexed by it: an array
+            // indexed at run time lives in scratch memory, and every row would wait on it
+            V3 n{0, 0, 1}, point{0, 0, 0}, dir0{0, 0, 0}, dir1{0, 0, 0}, dir2{0, 0, 0}, dir3{0, 0, 0};
             V3 t0{1, 0, 0}, t1{0, 1, 0};
             float d0 = 0.0f;
             if (live) {
@@ -993,14 +1023,11 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
                 edge_invweight = (invweight + mu1 * mu1 * invweight) * 2.0f * mu1 * mu1 / impratio;
                 const float pos = -d0 - margin;
                 edge = compliant_row(solref, solimp, pos, pos, 0.0f, edge_invweight, p.dt, p.refsafe);
-                for (uint32_t k = 0u; k < 4u; ++k) {
-                    const float mu = k < 2u ? mu1 : mu2;
-                    const V3 tangent = k < 2u ? t0 : t1;
-                    dirs[k] = add3(n, scale3(tangent, (k & 1u) != 0u ? -mu : mu));
-                }
-            } else { dirs[0] = n; dirs[1] = t0; dirs[2] = t1; dirs[3] = V3{0, 0, 0}; }
+                dir0 = add3(n, scale3(t0, mu1)); dir1 = add3(n, scale3(t0, -mu1));
+                dir2 = add3(n, scale3(t1, mu2)); dir3 = add3(n, scale3(t1, -mu2));
+            } else { dir0 = n; dir1 = t0; dir2 = t1; }
             for (uint32_t axis = 0u; axis < row_count; ++axis) {
-                const uint32_t rs = row_of[axis];
+                const uint32_t rs = base + axis * P + pt;
                 lambda[rs] = 0.0f; pen[rs] = 0.0f; cj_link[rs] = kInvalid; cj_link_b[rs] = kInvalid;
                 row_gain[rs] = 0.0f;
                 if (!(pyramidal ? live : emits[axis == 0u ? 0 : 1])) {
@@ -1008,7 +1035,7 @@ __global__ void __launch_bounds__(kWave) AssembleRowsKernel(ModelView m, DataVie
                     continue;
                 }
                 Row row{};
-                const V3 dir = dirs[axis];
+                const V3 dir = axis == 0u ? dir0 : axis == 1u ? dir1 : axis == 2u ? dir2 : dir3;
                 row.group_first = env * R + base; row.group_normal_count = P; row.env = env;
                 row.mu = mu1; row.friction_secondary = mu2;
                 row.a.kind = kind_a; row.a.index = idx_a; row.a.jlin = dir; row.a.jang = V3{0, 0, 0};
@@ -1288,7 +1315,8 @@ Status OpNarrowphasePrimitives(const ModelView& m, const DataView& d, const void
     const auto* p = static_cast<const NarrowphasePrimitivesParams*>(params);
     if (p == nullptr) return Status::Failed;
     if (p->env_count == 0u || p->union_slot_count == 0u || p->rigid_slot_cap == 0u) return Status::Ok;
-    hipLaunchKernelGGL(NarrowphaseKernel, dim3(p->env_count), dim3(64), 0, stream, m, d, *p);
+    if (m.max_points_per_slot <= 1u) hipLaunchKernelGGL(NarrowphaseKernel<true>, dim3(p->env_count), dim3(64), 0, stream, m, d, *p);
+    else hipLaunchKernelGGL(NarrowphaseKernel<false>, dim3(p->env_count), dim3(64), 0, stream, m, d, *p);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 
