@@ -154,29 +154,38 @@ __global__ void __launch_bounds__(kWave) FkWorldPosesKernel(ModelView m, DataVie
 }
 
 // ---- ArticulationDynamics -------------------------------------------------------------------------------
-// The link accelerations and bias forces are dead while the composite inertias live (mass-matrix assembly) and the
-// other way round, so the two share their words: less LDS a block, more blocks a compute unit for a kernel that
-// waits on tree sweeps.
+// Two wavefronts an environment.  The bias forces (velocities, bias accelerations, the leaf-to-root force pass) and the
+// mass matrix with its factor (composite inertias, columns, LDL^T) do not depend on each other, and each is a chain of
+// tree sweeps that keeps a few lanes busy: the first wavefront takes the one, the second the other, side by side, and
+// they meet before the solve.  Each keeps to its own words of LDS in between.
 __host__ __device__ inline uint32_t DynamicsLdsFloats(uint32_t nl, uint32_t n) {
-    return nl * (36u + 36u + 3u * 6u) + n * (n + 1u) + 2u * n + 64u;
+    return nl * (36u + 36u + 5u * 6u) + n * (n + 1u) + 2u * n + 64u;
+}
+// Orders one wavefront's LDS writes before its later reads: its lanes run in step and the LDS takes a wavefront's
+// accesses in order, so only the compiler could move them - a fence of wavefront scope holds it without a wait
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // Compiled per padded DoF width N (a multiple of 4): the LDL^T factorisation and the solve keep one matrix row per
 // lane in registers, fully unrolled, and pass pivots and multipliers between lanes as scalar lane reads.
 template <int N>
-__global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m, DataView d, ArticulationDynamicsParams p,
-                                                                   uint32_t env_count) {
+__global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelView m, DataView d, ArticulationDynamicsParams p,
+                                                                       uint32_t env_count) {
     extern __shared__ float lds[];
-    const uint32_t env = blockIdx.x, lane = threadIdx.x, nl = m.links_per_env, n = m.dof, stride = m.max_dof;
+    const uint32_t env = blockIdx.x, lane = threadIdx.x % kWave, nl = m.links_per_env, n = m.dof, stride = m.max_dof;
+    const bool forces = threadIdx.x < uint32_t(kWave);   // the first wavefront: bias forces; the second: mass matrix, factor, solve
     if (env >= env_count) return;
     float* xup = lds;
     float* S = xup + nl * 36u;
     float* vb = S + nl * 6u;
     float* v = vb + nl * 6u;
-    float* ic = v + nl * 6u;          // composite inertias, from the mass-matrix assembly until its columns are done
-    float* a = ic;                    // link accelerations: bias pass, and again the final pass
-    float* pf = a + nl * 6u;          // bias forces: until the generalized bias is taken
-    float* A = ic + nl * 36u;         // n x (n + 1): mass matrix, then its factor
+    float* ic = v + nl * 6u;          // composite inertias (second wavefront)
+    float* a = ic + nl * 36u;         // link accelerations: bias pass (first wavefront), and again the final pass (second)
+    float* pf = a + nl * 6u;          // bias forces (first wavefront)
+    float* A = pf + nl * 6u;          // n x (n + 1): mass matrix, then its factor (second wavefront)
     float* vel = A + n * (n + 1u);
     float* acc = vel + n;
     float* tmp = acc + n;             // 36 floats of the inertia push, padded to 64
@@ -194,10 +203,14 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
     };
     const LinkTree own = lane < nl ? tree_of(lane) : LinkTree{kInvalid, kInvalid, 0u, 0u, uint8_t(0), 0.0f};
 
+    if (!forces) {   // what the mass matrix starts from, while the first wavefront builds the joint transforms
+        for (uint32_t e = lane; e < nl * 36u; e += kWave) ic[e] = m.link_inertia[e];
+        for (uint32_t e = lane; e < n * ld; e += kWave) A[e] = 0.0f;
+    }
     // link twists of the state enter LDS (a floating root's twist is state; the rest is rebuilt)
-    for (uint32_t e = lane; e < nl * 6u; e += kWave) v[e] = d.link_velocity[lbase * 6u + e];
+    for (uint32_t e = lane; forces && e < nl * 6u; e += kWave) v[e] = d.link_velocity[lbase * 6u + e];
     // joint transforms and motion subspaces (articulation.cu:318-332)
-    for (uint32_t l = lane; l < nl; l += kWave) {
+    for (uint32_t l = lane; forces && l < nl; l += kWave) {
         if (m.parent_link[l] == kInvalid && m.joint_type[l] == kFloatingBase) {
             const float id[9] = {1, 0, 0, 0, 1, 0, 0, 0, 1};
             store_motion_transform(id, V3{0.0f, 0.0f, 0.0f}, xup + 36u * l);
@@ -209,237 +222,238 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
         motion_subspace(m.joint_type[l], load3(m.joint_axis + 3u * l), S + 6u * l);
     }
     __syncthreads();
-    // velocities root to leaf (:334-363)
-    for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
-        for (uint32_t l = lane; l < nl; l += kWave) {
-            const LinkTree t = l == lane ? own : tree_of(l);
-            if (t.depth != depth) continue;
-            const uint32_t parent = t.parent;
-            if (parent == kInvalid && t.type == kFloatingBase) continue;
-            float vp[6] = {0, 0, 0, 0, 0, 0}, tp[6], jv[6], vl[6];
-            if (parent != kInvalid) {
-#pragma unroll
-                for (int i = 0; i < 6; ++i) vp[i] = v[6u * parent + i];
-            }
-            mat66_vec(xup + 36u * l, vp, tp);
-            const float qdl = t.rate;
-#pragma unroll
-            for (int i = 0; i < 6; ++i) { jv[i] = S[6u * l + i] * qdl; vl[i] = tp[i] + jv[i]; }
-#pragma unroll
-            for (int i = 0; i < 6; ++i) v[6u * l + i] = vl[i];
-            motion_cross(vl, jv, vb + 6u * l);
-        }
-        __syncthreads();
-    }
-    // p = v x* (I v) - external wrench (:364-374, 279-295)
-    for (uint32_t l = lane; l < nl; l += kWave) {
-        float vl[6], iv[6], bf[6];
-#pragma unroll
-        for (int i = 0; i < 6; ++i) vl[i] = v[6u * l + i];
-        mat66_vec(m.link_inertia + 36u * l, vl, iv);
-        force_cross(vl, iv, bf);
-        if (p.apply_link_wrench != 0u) {
-            const float* wr = d.link_wrench + (lbase + l) * 6u;
-            if (wr[0] != 0.0f || wr[1] != 0.0f || wr[2] != 0.0f || wr[3] != 0.0f || wr[4] != 0.0f || wr[5] != 0.0f) {
-                const Q4 rot = load_xf(d.link_pose + (lbase + l) * 7u).r;
-                const V3 force = rotate_inverse(rot, V3{wr[0], wr[1], wr[2]});
-                const V3 torque = rotate_inverse(rot, V3{wr[3], wr[4], wr[5]});
-                const V3 moment = add3(torque, cross3(load_xf(m.link_inertial_frame + 7u * l).p, force));
-                bf[0] -= moment.x; bf[1] -= moment.y; bf[2] -= moment.z; bf[3] -= force.x; bf[4] -= force.y; bf[5] -= force.z;
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < 6; ++i) pf[6u * l + i] = bf[i];
-    }
-    __syncthreads();
-    // bias accelerations with gravity as base acceleration (:526-547)
-    for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
-        for (uint32_t l = lane; l < nl; l += kWave) {
-            const LinkTree t = l == lane ? own : tree_of(l);
-            if (t.depth != depth) continue;
-            float al[6];
-            const uint32_t parent = t.parent;
-            if (parent != kInvalid) {
-                float ap[6];
-#pragma unroll
-                for (int i = 0; i < 6; ++i) ap[i] = a[6u * parent + i];
-                mat66_vec(xup + 36u * l, ap, al);
-            } else if (t.type == kFloatingBase) {
-                const V3 g = rotate_inverse(base_rot, gravity);
-                al[0] = al[1] = al[2] = 0.0f; al[3] = -g.x; al[4] = -g.y; al[5] = -g.z;
-            } else {
-                const float world[6] = {0.0f, 0.0f, 0.0f, -gravity.x, -gravity.y, -gravity.z};
-                mat66_vec(xup + 36u * l, world, al);
-            }
-#pragma unroll
-            for (int i = 0; i < 6; ++i) a[6u * l + i] = al[i] + vb[6u * l + i];
-        }
-        __syncthreads();
-    }
-    // p += I a (:548-555)
-    for (uint32_t l = lane; l < nl; l += kWave) {
-        float al[6], f[6];
-#pragma unroll
-        for (int i = 0; i < 6; ++i) al[i] = a[6u * l + i];
-        mat66_vec(m.link_inertia + 36u * l, al, f);
-#pragma unroll
-        for (int i = 0; i < 6; ++i) pf[6u * l + i] += f[i];
-    }
-    __syncthreads();
-    // leaf to root, children in CSR order (:557-569)
-    for (uint32_t remaining = m.max_depth + 1u; remaining > 0u; --remaining) {
-        for (uint32_t l = lane; l < nl; l += kWave) {
-            const LinkTree t = l == lane ? own : tree_of(l);
-            if (t.depth != remaining - 1u) continue;
-            for (uint32_t i = t.child_begin; i < t.child_end; ++i) {
-                const uint32_t child = m.link_children[i];
-                float pc[6], f[6];
-#pragma unroll
-                for (int c = 0; c < 6; ++c) pc[c] = pf[6u * child + c];
-                mat66t_vec(xup + 36u * child, pc, f);
-#pragma unroll
-                for (int c = 0; c < 6; ++c) pf[6u * l + c] += f[c];
-            }
-        }
-        __syncthreads();
-    }
-    // generalized bias and right-hand side, lane = DoF (:570-585)
-    float* bias = d.articulation_bias + size_t{env} * stride;
-    if (lane < stride) {
-        if (lane >= n) bias[lane] = 0.0f;
-        else {
-            const uint32_t link = m.dof_link[lane], component = m.dof_component[lane];
-            const bool scalar = component == kInvalid;
-            const float velocity = scalar ? qd[link] : v[6u * link + component];
-            float b = scalar ? dot6(S + 6u * link, pf + 6u * link) : pf[6u * link + component];
-            if (scalar) b += d.joint_gravity_force[lbase + link];   // zero unless uploaded
-            const float damping = scalar ? m.joint_damping[link] + (p.fold_drive_damping != 0u ? d.drive_dissipation[lbase + link] : 0.0f) : 0.0f;
-            const float spring = scalar ? m.joint_stiffness[link] * (q[link] - m.joint_spring_reference[link]) : 0.0f;
-            vel[lane] = velocity;
-            bias[lane] = b;
-            acc[lane] = (scalar ? d.tau[lbase + link] : 0.0f) - b - damping * velocity - spring;
-        }
-    }
-    __syncthreads();   // the bias forces have been read: their words now take the composite inertias
-    // CRBA: composite inertias leaf to root; the push X^T Ic X runs entry-parallel on 36 lanes (articulation_mass.cuh:146-165)
-    for (uint32_t e = lane; e < nl * 36u; e += kWave) ic[e] = m.link_inertia[e];
-    for (uint32_t e = lane; e < n * ld; e += kWave) A[e] = 0.0f;
-    __syncthreads();
-    // deepest parents first, parents of one depth in link order, a parent's children in list order: the cooked visiting
-    // list, sixty-four visits at a time - a lane reads one visit's child and parent, the visits take theirs as lane reads
-    for (uint32_t first = 0u; first < nl; first += kWave) {
-        uint32_t my_child = kInvalid, my_parent = 0u;
-        if (first + lane < nl) {
-            my_child = m.link_push_order[first + lane];
-            if (my_child != kInvalid) my_parent = m.parent_link[my_child];
-        }
-        for (uint32_t visit = 0u; visit < uint32_t(kWave); ++visit) {
-            const uint32_t child = uint32_t(__builtin_amdgcn_readlane(int(my_child), int(visit)));
-            if (child == kInvalid) break;
-            const uint32_t l = uint32_t(__builtin_amdgcn_readlane(int(my_parent), int(visit)));
-            const float* X = xup + 36u * child;
-            const float* C = ic + 36u * child;
-            const uint32_t row = lane / 6u, col = lane % 6u;
-            if (lane < 36u) {
-                float value = 0.0f;
-#pragma unroll
-                for (int k = 0; k < 6; ++k) value += C[row * 6u + k] * X[k * 6u + col];
-                tmp[lane] = value;
-            }
-            __syncthreads();
-            if (lane < 36u) {
-                float value = 0.0f;
-#pragma unroll
-                for (int k = 0; k < 6; ++k) value += X[k * 6u + row] * tmp[k * 6u + col];
-                ic[36u * l + lane] += value;
-            }
-            __syncthreads();
-        }
-    }
     const bool floating_root = m.floating_root != 0u;
-    if (floating_root && lane < 36u) A[(lane / 6u) * ld + lane % 6u] = ic[lane];
-    __syncthreads();
-    // mass columns: each jointed link pushes Ic S to the root (:183-252)
-    for (uint32_t l = lane; l < nl; l += kWave) {
-        if (joint_dof(m.joint_type[l]) == 0u) continue;
-        if (l == 0u && floating_root) continue;
-        const uint32_t dof_i = m.link_dof[l];
-        float force[6], sl[6];
+    float row[N];   // the second wavefront's row of the mass matrix, then of its factor
+    if (forces) {
+        // velocities root to leaf (:334-363)
+        for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
+            for (uint32_t l = lane; l < nl; l += kWave) {
+                const LinkTree t = l == lane ? own : tree_of(l);
+                if (t.depth != depth) continue;
+                const uint32_t parent = t.parent;
+                if (parent == kInvalid && t.type == kFloatingBase) continue;
+                float vp[6] = {0, 0, 0, 0, 0, 0}, tp[6], jv[6], vl[6];
+                if (parent != kInvalid) {
 #pragma unroll
-        for (int i = 0; i < 6; ++i) sl[i] = S[6u * l + i];
-        mat66_vec(ic + 36u * l, sl, force);
-        float diagonal = dot6(sl, force);
-        diagonal += m.joint_armature[l];
-        if (p.fold_drive_damping != 0u) diagonal += p.dt * d.drive_dissipation[lbase + l];   // articulation_mass.cuh:206-208
-        A[dof_i * ld + dof_i] = diagonal;
-        uint32_t walk = l;
-        for (;;) {
-            const uint32_t parent = m.parent_link[walk];
-            if (parent == kInvalid) break;
-            float pushed[6];
-            mat66t_vec(xup + 36u * walk, force, pushed);
+                    for (int i = 0; i < 6; ++i) vp[i] = v[6u * parent + i];
+                }
+                mat66_vec(xup + 36u * l, vp, tp);
+                const float qdl = t.rate;
 #pragma unroll
-            for (int i = 0; i < 6; ++i) force[i] = pushed[i];
-            walk = parent;
-            if (joint_dof(m.joint_type[walk]) == 0u) continue;
-            const uint32_t dof_j = m.link_dof[walk];
-            if (walk == 0u && floating_root) {
+                for (int i = 0; i < 6; ++i) { jv[i] = S[6u * l + i] * qdl; vl[i] = tp[i] + jv[i]; }
 #pragma unroll
-                for (int b = 0; b < 6; ++b) { A[dof_i * ld + b] = force[b]; A[b * ld + dof_i] = force[b]; }
-                continue;
+                for (int i = 0; i < 6; ++i) v[6u * l + i] = vl[i];
+                motion_cross(vl, jv, vb + 6u * l);
             }
-            const float entry = dot6(S + 6u * walk, force);
-            A[dof_i * ld + dof_j] = entry;
-            A[dof_j * ld + dof_i] = entry;
+            wave_sync();
         }
-    }
-    __syncthreads();
-    // the dense mass tile reaches HBM once, in row-major runs
-    float* M = d.m + size_t{env} * stride * stride;
-    for (uint32_t e = lane; e < stride * stride; e += kWave) {
-        const uint32_t i = e / stride, j = e % stride;
-        M[e] = i < n && j < n ? A[i * ld + j] : 0.0f;
-    }
-    // LDL^T, right-looking, lane = row in registers; the strict lower triangle becomes L and the diagonal D (:269-335).
-    // Rows and columns n..N-1 are those of the identity.  Entry (i, j) loses (L_ik L_jk) D_k for k = 0, 1, ... as the
-    // serial loop does; what a lane computes above its diagonal is never read.
-    float row[N];
-    {
-        const uint32_t ll = local_lane(lane);
+        // p = v x* (I v) - external wrench (:364-374, 279-295)
+        for (uint32_t l = lane; l < nl; l += kWave) {
+            float vl[6], iv[6], bf[6];
 #pragma unroll
-        for (int k = 0; k < N; ++k)
-            row[k] = ll < n && uint32_t(k) < n ? A[ll * ld + k] : (ll == uint32_t(k) ? 1.0f : 0.0f);
-    }
-    __syncthreads();
-    {
-        const uint32_t ll = local_lane(lane);
+            for (int i = 0; i < 6; ++i) vl[i] = v[6u * l + i];
+            mat66_vec(m.link_inertia + 36u * l, vl, iv);
+            force_cross(vl, iv, bf);
+            if (p.apply_link_wrench != 0u) {
+                const float* wr = d.link_wrench + (lbase + l) * 6u;
+                if (wr[0] != 0.0f || wr[1] != 0.0f || wr[2] != 0.0f || wr[3] != 0.0f || wr[4] != 0.0f || wr[5] != 0.0f) {
+                    const Q4 rot = load_xf(d.link_pose + (lbase + l) * 7u).r;
+                    const V3 force = rotate_inverse(rot, V3{wr[0], wr[1], wr[2]});
+                    const V3 torque = rotate_inverse(rot, V3{wr[3], wr[4], wr[5]});
+                    const V3 moment = add3(torque, cross3(load_xf(m.link_inertial_frame + 7u * l).p, force));
+                    bf[0] -= moment.x; bf[1] -= moment.y; bf[2] -= moment.z; bf[3] -= force.x; bf[4] -= force.y; bf[5] -= force.z;
+                }
+            }
 #pragma unroll
-        for (int k = 0; k < N; ++k) {
-            const float diagonal = fmaxf(lane_value(row[k], k), 1.0e-6f);
-            const float lik = row[k] / diagonal;
-            row[k] = ll > uint32_t(k) ? lik : (ll == uint32_t(k) ? diagonal : row[k]);
+            for (int i = 0; i < 6; ++i) pf[6u * l + i] = bf[i];
+        }
+        wave_sync();
+        // bias accelerations with gravity as base acceleration (:526-547)
+        for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
+            for (uint32_t l = lane; l < nl; l += kWave) {
+                const LinkTree t = l == lane ? own : tree_of(l);
+                if (t.depth != depth) continue;
+                float al[6];
+                const uint32_t parent = t.parent;
+                if (parent != kInvalid) {
+                    float ap[6];
 #pragma unroll
-            for (int j0 = k + 1; j0 < N; j0 += 8) {
-                float l[8];
+                    for (int i = 0; i < 6; ++i) ap[i] = a[6u * parent + i];
+                    mat66_vec(xup + 36u * l, ap, al);
+                } else if (t.type == kFloatingBase) {
+                    const V3 g = rotate_inverse(base_rot, gravity);
+                    al[0] = al[1] = al[2] = 0.0f; al[3] = -g.x; al[4] = -g.y; al[5] = -g.z;
+                } else {
+                    const float world[6] = {0.0f, 0.0f, 0.0f, -gravity.x, -gravity.y, -gravity.z};
+                    mat66_vec(xup + 36u * l, world, al);
+                }
 #pragma unroll
-                for (int t = 0; t < 8; ++t) l[t] = j0 + t < N ? lane_value(lik, j0 + t) : 0.0f;
+                for (int i = 0; i < 6; ++i) a[6u * l + i] = al[i] + vb[6u * l + i];
+            }
+            wave_sync();
+        }
+        // p += I a (:548-555)
+        for (uint32_t l = lane; l < nl; l += kWave) {
+            float al[6], f[6];
 #pragma unroll
-                for (int t = 0; t < 8; ++t)
-                    if (j0 + t < N) row[j0 + t] -= lik * l[t] * diagonal;
+            for (int i = 0; i < 6; ++i) al[i] = a[6u * l + i];
+            mat66_vec(m.link_inertia + 36u * l, al, f);
+#pragma unroll
+            for (int i = 0; i < 6; ++i) pf[6u * l + i] += f[i];
+        }
+        wave_sync();
+        // leaf to root, children in CSR order (:557-569)
+        for (uint32_t remaining = m.max_depth + 1u; remaining > 0u; --remaining) {
+            for (uint32_t l = lane; l < nl; l += kWave) {
+                const LinkTree t = l == lane ? own : tree_of(l);
+                if (t.depth != remaining - 1u) continue;
+                for (uint32_t i = t.child_begin; i < t.child_end; ++i) {
+                    const uint32_t child = m.link_children[i];
+                    float pc[6], f[6];
+#pragma unroll
+                    for (int c = 0; c < 6; ++c) pc[c] = pf[6u * child + c];
+                    mat66t_vec(xup + 36u * child, pc, f);
+#pragma unroll
+                    for (int c = 0; c < 6; ++c) pf[6u * l + c] += f[c];
+                }
+            }
+            wave_sync();
+        }
+        // generalized bias and right-hand side, lane = DoF (:570-585)
+        float* bias = d.articulation_bias + size_t{env} * stride;
+        if (lane < stride) {
+            if (lane >= n) bias[lane] = 0.0f;
+            else {
+                const uint32_t link = m.dof_link[lane], component = m.dof_component[lane];
+                const bool scalar = component == kInvalid;
+                const float velocity = scalar ? qd[link] : v[6u * link + component];
+                float b = scalar ? dot6(S + 6u * link, pf + 6u * link) : pf[6u * link + component];
+                if (scalar) b += d.joint_gravity_force[lbase + link];   // zero unless uploaded
+                const float damping = scalar ? m.joint_damping[link] + (p.fold_drive_damping != 0u ? d.drive_dissipation[lbase + link] : 0.0f) : 0.0f;
+                const float spring = scalar ? m.joint_stiffness[link] * (q[link] - m.joint_spring_reference[link]) : 0.0f;
+                vel[lane] = velocity;
+                bias[lane] = b;
+                acc[lane] = (scalar ? d.tau[lbase + link] : 0.0f) - b - damping * velocity - spring;
             }
         }
-        if (ll < n) {
+    } else {
+        // CRBA: composite inertias leaf to root; the push X^T Ic X runs entry-parallel on 36 lanes (articulation_mass.cuh:146-165)
+        // deepest parents first, parents of one depth in link order, a parent's children in list order: the cooked visiting
+        // list, sixty-four visits at a time - a lane reads one visit's child and parent, the visits take theirs as lane reads
+        for (uint32_t first = 0u; first < nl; first += kWave) {
+            uint32_t my_child = kInvalid, my_parent = 0u;
+            if (first + lane < nl) {
+                my_child = m.link_push_order[first + lane];
+                if (my_child != kInvalid) my_parent = m.parent_link[my_child];
+            }
+            for (uint32_t visit = 0u; visit < uint32_t(kWave); ++visit) {
+                const uint32_t child = uint32_t(__builtin_amdgcn_readlane(int(my_child), int(visit)));
+                if (child == kInvalid) break;
+                const uint32_t l = uint32_t(__builtin_amdgcn_readlane(int(my_parent), int(visit)));
+                const float* X = xup + 36u * child;
+                const float* C = ic + 36u * child;
+                const uint32_t row = lane / 6u, col = lane % 6u;
+                if (lane < 36u) {
+                    float value = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < 6; ++k) value += C[row * 6u + k] * X[k * 6u + col];
+                    tmp[lane] = value;
+                }
+                wave_sync();
+                if (lane < 36u) {
+                    float value = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < 6; ++k) value += X[k * 6u + row] * tmp[k * 6u + col];
+                    ic[36u * l + lane] += value;
+                }
+                wave_sync();
+            }
+        }
+        if (floating_root && lane < 36u) A[(lane / 6u) * ld + lane % 6u] = ic[lane];
+        wave_sync();
+        // mass columns: each jointed link pushes Ic S to the root (:183-252)
+        for (uint32_t l = lane; l < nl; l += kWave) {
+            if (joint_dof(m.joint_type[l]) == 0u) continue;
+            if (l == 0u && floating_root) continue;
+            const uint32_t dof_i = m.link_dof[l];
+            float force[6], sl[6];
+#pragma unroll
+            for (int i = 0; i < 6; ++i) sl[i] = S[6u * l + i];
+            mat66_vec(ic + 36u * l, sl, force);
+            float diagonal = dot6(sl, force);
+            diagonal += m.joint_armature[l];
+            if (p.fold_drive_damping != 0u) diagonal += p.dt * d.drive_dissipation[lbase + l];   // articulation_mass.cuh:206-208
+            A[dof_i * ld + dof_i] = diagonal;
+            uint32_t walk = l;
+            for (;;) {
+                const uint32_t parent = m.parent_link[walk];
+                if (parent == kInvalid) break;
+                float pushed[6];
+                mat66t_vec(xup + 36u * walk, force, pushed);
+#pragma unroll
+                for (int i = 0; i < 6; ++i) force[i] = pushed[i];
+                walk = parent;
+                if (joint_dof(m.joint_type[walk]) == 0u) continue;
+                const uint32_t dof_j = m.link_dof[walk];
+                if (walk == 0u && floating_root) {
+#pragma unroll
+                    for (int b = 0; b < 6; ++b) { A[dof_i * ld + b] = force[b]; A[b * ld + dof_i] = force[b]; }
+                    continue;
+                }
+                const float entry = dot6(S + 6u * walk, force);
+                A[dof_i * ld + dof_j] = entry;
+                A[dof_j * ld + dof_i] = entry;
+            }
+        }
+        wave_sync();
+        // the dense mass tile reaches HBM once, in row-major runs
+        float* M = d.m + size_t{env} * stride * stride;
+        for (uint32_t e = lane; e < stride * stride; e += kWave) {
+            const uint32_t i = e / stride, j = e % stride;
+            M[e] = i < n && j < n ? A[i * ld + j] : 0.0f;
+        }
+        // LDL^T, right-looking, lane = row in registers; the strict lower triangle becomes L and the diagonal D (:269-335).
+        // Rows and columns n..N-1 are those of the identity.  Entry (i, j) loses (L_ik L_jk) D_k for k = 0, 1, ... as the
+        // serial loop does; what a lane computes above its diagonal is never read.
+        {
+            const uint32_t ll = local_lane(lane);
 #pragma unroll
             for (int k = 0; k < N; ++k)
-                if (uint32_t(k) < n) A[ll * ld + k] = row[k];
+                row[k] = ll < n && uint32_t(k) < n ? A[ll * ld + k] : (ll == uint32_t(k) ? 1.0f : 0.0f);
+        }
+        wave_sync();
+        {
+            const uint32_t ll = local_lane(lane);
+#pragma unroll
+            for (int k = 0; k < N; ++k) {
+                const float diagonal = fmaxf(lane_value(row[k], k), 1.0e-6f);
+                const float lik = row[k] / diagonal;
+                row[k] = ll > uint32_t(k) ? lik : (ll == uint32_t(k) ? diagonal : row[k]);
+#pragma unroll
+                for (int j0 = k + 1; j0 < N; j0 += 8) {
+                    float l[8];
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) l[t] = j0 + t < N ? lane_value(lik, j0 + t) : 0.0f;
+#pragma unroll
+                    for (int t = 0; t < 8; ++t)
+                        if (j0 + t < N) row[j0 + t] -= lik * l[t] * diagonal;
+                }
+            }
+            if (ll < n) {
+#pragma unroll
+                for (int k = 0; k < N; ++k)
+                    if (uint32_t(k) < n) A[ll * ld + k] = row[k];
+            }
+        }
+        wave_sync();
+        float* factor = d.m_factor + size_t{env} * stride * stride;
+        for (uint32_t e = lane; e < stride * stride; e += kWave) {
+            const uint32_t i = e / stride, j = e % stride;
+            if (j <= i) factor[e] = i < n ? A[i * ld + j] : (i == j ? 1.0e-6f : 0.0f);
         }
     }
-    __syncthreads();
-    float* factor = d.m_factor + size_t{env} * stride * stride;
-    for (uint32_t e = lane; e < stride * stride; e += kWave) {
-        const uint32_t i = e / stride, j = e % stride;
-        if (j <= i) factor[e] = i < n ? A[i * ld + j] : (i == j ? 1.0e-6f : 0.0f);
-    }
+    __syncthreads();   // the right-hand side (first wavefront) meets the factor (second)
+    if (forces) return;
     // solve L D L^T x = rhs: forward by rows, scale, backward by columns (:357-396)
     float x = lane < n ? acc[lane] : 0.0f;
     {
@@ -461,7 +475,7 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
     }
     if (lane < stride) d.articulation_qdd[size_t{env} * stride + lane] = lane < n ? x : 0.0f;
     if (lane < n) acc[lane] = x;
-    __syncthreads();
+    wave_sync();
     // write back accelerations and the unconstrained velocity update (:597-615)
     for (uint32_t l = lane; l < nl; l += kWave) {
         const uint8_t type = m.joint_type[l];
@@ -483,7 +497,7 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
         const float transport = component < 3u ? 0.0f : vel[j] * vel[3u + k] - vel[k] * vel[3u + j];
         v[component] = vel[lane] + p.dt * (acc[lane] + transport);
     }
-    __syncthreads();
+    wave_sync();
     // final link accelerations (:617-644)
     for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
         for (uint32_t l = lane; l < nl; l += kWave) {
@@ -513,7 +527,7 @@ __global__ void __launch_bounds__(kWave) ArticulationDynamicsKernel(ModelView m,
 #pragma unroll
             for (int c = 0; c < 6; ++c) a[6u * l + c] = al[c];
         }
-        __syncthreads();
+        wave_sync();
     }
     for (uint32_t e = lane; e < nl * 6u; e += kWave) {
         d.link_velocity[lbase * 6u + e] = v[e];
@@ -622,7 +636,7 @@ Status OpArticulationDynamics(const ModelView& m, const DataView& d, const void*
         p->total_link_count != p->articulation_count * m.links_per_env) return Status::InvalidArgument;
     const size_t lds = size_t{DynamicsLdsFloats(m.links_per_env, m.dof)} * sizeof(float);
     if (lds > 160u * 1024u) return Status::InvalidArgument;
-    hipLaunchKernelGGL(kDynamicsKernels[((m.dof + 3u) & ~3u) / 4u - 1u], dim3(p->articulation_count), dim3(kWave), lds, stream, m, d,
+    hipLaunchKernelGGL(kDynamicsKernels[((m.dof + 3u) & ~3u) / 4u - 1u], dim3(p->articulation_count), dim3(2 * kWave), lds, stream, m, d,
                        *p, p->articulation_count);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
