@@ -24,7 +24,7 @@ DOMINANT_OP = "BlockDescentSolve"
 DOMINANT_KERNEL = "BlockDescentTileKernel"
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, scaled
 # by the same counters' reading of a plain copy of known size); keyed by (config, envs).  None where not measured.
-MEASURED_TRAFFIC_BYTES = {(3, 4096): 80.9e6, (2, 4096): 29.8e6, (3, 65536): 1244.9e6, (5, 8192): 496.9e6}   # profiles/counters_*.txt
+MEASURED_TRAFFIC_BYTES = {(3, 4096): 81.0e6, (2, 4096): 29.8e6, (3, 65536): 1244.9e6, (5, 8192): 497.2e6}   # profiles/counters_*.txt
 # What the same counter runs say limits the dominant kernel (not measured by this script): vector instructions a
 # launch issues and the share of a wave's resident cycles spent issuing them, at two waves a SIMD (one for the rope).
 MEASURED_ISSUE = {
