@@ -48,9 +48,24 @@ __global__ void __launch_bounds__(1024) OrderTilesKernel(DataView d, uint32_t en
     const uint32_t scale = top / 256u + 1u;
     for (uint32_t e = t; e < env_count; e += 1024u) atomicAdd(&bins[255u - min(d.solver_cost[e] / scale, 255u)], 1u);
     __syncthreads();
-    if (t == 0u) {
-        uint32_t running = 0u;
-        for (uint32_t b = 0u; b < 256u; ++b) { const uint32_t count = bins[b]; bins[b] = running; running += count; }
+    // exclusive prefix of the 256 counts: a scan inside each of the first four wavefronts, then their totals
+    __shared__ uint32_t wave_total[4];
+    uint32_t count = 0u, through = 0u;
+    if (t < 256u) {
+        count = bins[t];
+        through = count;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t other = __shfl_up(through, o, 64);
+            if (int(t & 63u) >= o) through += other;
+        }
+        if ((t & 63u) == 63u) wave_total[t >> 6u] = through;
+    }
+    __syncthreads();
+    if (t < 256u) {
+        uint32_t before = 0u;
+        for (uint32_t w = 0u; w < (t >> 6u); ++w) before += wave_total[w];
+        bins[t] = before + through - count;
     }
     __syncthreads();
     for (uint32_t e = t; e < env_count; e += 1024u) d.tile_order[atomicAdd(&bins[255u - min(d.solver_cost[e] / scale, 255u)], 1u)] = e;
