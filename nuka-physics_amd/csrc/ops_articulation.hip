@@ -336,6 +336,14 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
                 acc[lane] = (scalar ? d.tau[lbase + link] : 0.0f) - b - damping * velocity - spring;
             }
         }
+        __syncthreads();   // the second wavefront has the mass matrix in LDS
+        // the dense mass tile reaches HBM once, in row-major runs
+        float* M = d.m + size_t{env} * stride * stride;
+        for (uint32_t e = lane; e < stride * stride; e += kWave) {
+            const uint32_t i = e / stride, j = e % stride;
+            M[e] = i < n && j < n ? A[i * ld + j] : 0.0f;
+        }
+        __syncthreads();   // ... and may now overwrite it with the factor
     } else {
         // CRBA: composite inertias leaf to root; the push X^T Ic X runs entry-parallel on 36 lanes (articulation_mass.cuh:146-165)
         // deepest parents first, parents of one depth in link order, a parent's children in list order: the cooked visiting
@@ -405,13 +413,7 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
                 A[dof_j * ld + dof_i] = entry;
             }
         }
-        wave_sync();
-        // the dense mass tile reaches HBM once, in row-major runs
-        float* M = d.m + size_t{env} * stride * stride;
-        for (uint32_t e = lane; e < stride * stride; e += kWave) {
-            const uint32_t i = e / stride, j = e % stride;
-            M[e] = i < n && j < n ? A[i * ld + j] : 0.0f;
-        }
+        __syncthreads();   // the mass matrix stands in LDS: the first wavefront carries it to HBM while this one factors it
         // LDL^T, right-looking, lane = row in registers; the strict lower triangle becomes L and the diagonal D (:269-335).
         // Rows and columns n..N-1 are those of the identity.  Entry (i, j) loses (L_ik L_jk) D_k for k = 0, 1, ... as the
         // serial loop does; what a lane computes above its diagonal is never read.
@@ -421,7 +423,6 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
             for (int k = 0; k < N; ++k)
                 row[k] = ll < n && uint32_t(k) < n ? A[ll * ld + k] : (ll == uint32_t(k) ? 1.0f : 0.0f);
         }
-        wave_sync();
         {
             const uint32_t ll = local_lane(lane);
 #pragma unroll
@@ -439,21 +440,23 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
                         if (j0 + t < N) row[j0 + t] -= lik * l[t] * diagonal;
                 }
             }
+            __syncthreads();   // the first wavefront has read the mass matrix: its words take the factor
             if (ll < n) {
 #pragma unroll
                 for (int k = 0; k < N; ++k)
                     if (uint32_t(k) < n) A[ll * ld + k] = row[k];
             }
         }
-        wave_sync();
+    }
+    __syncthreads();   // the factor stands in LDS, and the right-hand side (first wavefront) meets it (second)
+    if (forces) {
         float* factor = d.m_factor + size_t{env} * stride * stride;
         for (uint32_t e = lane; e < stride * stride; e += kWave) {
             const uint32_t i = e / stride, j = e % stride;
             if (j <= i) factor[e] = i < n ? A[i * ld + j] : (i == j ? 1.0e-6f : 0.0f);
         }
+        return;
     }
-    __syncthreads();   // the right-hand side (first wavefront) meets the factor (second)
-    if (forces) return;
     // solve L D L^T x = rhs: forward by rows, scale, backward by columns (:357-396)
     float x = lane < n ? acc[lane] : 0.0f;
     {
