@@ -1,7 +1,8 @@
 // Articulation ops for gfx950: forward kinematics, forward dynamics (RNEA bias + CRBA + LDL^T solve), position
-// integration and link twists.  One 64-lane wavefront owns one environment: lanes are links in the tree sweeps,
-// matrix entries in the 6x6 inertia pushes, and matrix rows in the factorisation; every per-link quantity of the
-// environment lives in LDS between the sweeps and reaches HBM once, in contiguous env-major blocks.
+// integration and link twists.  One 64-lane wavefront owns one environment (the forward dynamics runs two, its bias
+// forces and its mass matrix side by side): lanes are links in the tree sweeps, matrix entries in the 6x6 inertia
+// pushes, and matrix rows in the factorisation; every per-link quantity of the environment lives in LDS between the
+// sweeps and reaches HBM once, in contiguous env-major blocks.
 //
 // Replaces src/phi/backend_cuda/ops/articulation.cu (UpdateWorldLinkPosesKernel :1561-1596,
 // ArticulationDynamicsKernel :505-645, IntegratePositionArticulationKernel :764-791, FkLinkVelocitiesKernel
