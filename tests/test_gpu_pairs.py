@@ -200,3 +200,43 @@ def test_supports_carry_the_weight(oracle_py, device, shape):
         assert relative_error(world.download(name), oracle.download(name)) <= TOL, name
     world.close()
     oracle.close()
+
+
+def test_single_point_dispatch_gives_the_general_dispatch_its_manifolds(device):
+    """A world whose admitted pairs give one point at most runs the narrowphase on its own dispatch of those manifolds.
+    The same world with one box added far above everything (its pair with the plane is admitted, so the general dispatch
+    runs, and never in reach) must report the same contacts for the pairs both worlds have, bit for bit."""
+    E = 256
+    cfg = nk.synthetic.config(3, E)
+    import copy
+    plain = cfg.template
+    boxed = copy.deepcopy(plain)
+    boxed.add_body(abi.ROLE_PROXY, link=0, kind=BOX, params=SHAPE_PARAMS[BOX], local_pos=(0.0, 0.0, 5.0), contype=1, conaffinity=2,
+                   profile=0)
+    boxed.max_contacts_per_env = plain.max_contacts_per_env + 1
+    results = []
+    for template in (plain, boxed):
+        world = nk.World(device, template, abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters))
+        world.set_state(cfg.state())
+        for op in ("FkWorldPoses", "SyncLinkBodyPose", "BuildAabbs", "LbvhQueryPairs", "NarrowphasePrimitives"):
+            world.op(op)
+        world.synchronize()
+        S = world.info.contact_slots_per_env
+        live = world.download("pair_count")
+        pairs = world.download("candidate_pairs").reshape(E, S, 2)
+        fields = {name: world.download(name).reshape(E, S, 4, -1) for name in ("ucontact_point", "ucontact_normal", "ucontact_depth",
+                                                                              "ucontact_id_feature", "ucontact_id_pair")}
+        counts = world.download("ucontact_count").reshape(E, S)
+        found = {}
+        for e in range(E):
+            for s in range(live[e]):
+                found[(e, int(pairs[e, s, 0]), int(pairs[e, s, 1]))] = (int(counts[e, s]),) + tuple(fields[n][e, s, 0].tobytes() for n in fields)
+        results.append(found)
+        world.close()
+    plain_found, boxed_found = results
+    assert len(plain_found) > 4 * E and sum(v[0] for v in plain_found.values()) > 2 * E, "the batch must hold contacts"
+    nb = len(plain.bodies)
+    shared = {k: v for k, v in boxed_found.items() if k[1] < nb and k[2] < nb}
+    assert shared.keys() == plain_found.keys()
+    differing = [k for k in plain_found if plain_found[k][0] != shared[k][0] or (plain_found[k][0] and plain_found[k][1:] != shared[k][1:])]
+    assert not differing, f"{len(differing)} pairs differ between the two dispatches, first {differing[:3]}"
