@@ -151,6 +151,19 @@ Status DispatchOn(Backend* be, const ModelView& m, const DataView& d, const nuka
     return fn(m, d, call.params, be->stream);
 }
 
+// IntegratePosition, FkWorldPoses, FkLinkVelocities and, if it follows, SyncLinkBodyPose at the head of `calls` as one
+// launch: the number of calls served, 0 when the head is something else or the ops must run one by one.
+int MergeStepTail(Backend* be, const ModelView& m, const DataView& d, const nuka_phi_op_call* calls, int n) {
+    if (n < 3 || calls[0].op != uint16_t(NkOp::IntegratePosition) || calls[1].op != uint16_t(NkOp::FkWorldPoses) ||
+        calls[2].op != uint16_t(NkOp::FkLinkVelocities)) return 0;
+    const bool bodies = n >= 4 && calls[3].op == uint16_t(NkOp::SyncLinkBodyPose);
+    const Status status = OpStepTail(m, d, static_cast<const IntegratePositionParams*>(calls[0].params),
+                                     static_cast<const FkWorldPosesParams*>(calls[1].params),
+                                     static_cast<const FkLinkVelocitiesParams*>(calls[2].params),
+                                     bodies ? static_cast<const SyncLinkBodyPoseParams*>(calls[3].params) : nullptr, be->stream);
+    return status == Status::Ok ? (bodies ? 4 : 3) : 0;
+}
+
 uint8_t BeDispatch(nuka_phi_backend* b, const nuka_phi_model_view* m, const nuka_phi_data_view* d, const nuka_phi_op_call* call) {
     if (b == nullptr || m == nullptr || d == nullptr || call == nullptr) return uint8_t(Status::InvalidArgument);
     return uint8_t(DispatchOn(reinterpret_cast<Backend*>(b), *reinterpret_cast<const ModelView*>(m),
@@ -185,8 +198,14 @@ nuka_phi_plan* BePlanCreate(nuka_phi_backend* b, const nuka_phi_model_view* m, c
     if (e != hipSuccess) { Fail(error, Status::Failed, uint16_t(NkOp::Count), int(e), hipGetErrorString(e)); return nullptr; }
     Status status = Status::Ok;
     uint16_t failed = uint16_t(NkOp::Count);
+    const ModelView& model = *reinterpret_cast<const ModelView*>(m);
+    const DataView& data = *reinterpret_cast<const DataView*>(d);
     for (int i = 0; i < n_calls && status == Status::Ok; ++i) {
-        status = DispatchOn(be, *reinterpret_cast<const ModelView*>(m), *reinterpret_cast<const DataView*>(d), calls[i]);
+        // The ops after the solve each take about a launch's time: where the list holds them in a row, one kernel runs
+        // the four (ops_articulation.hip StepTailKernel); where it cannot, they go one by one as dispatched.
+        const int merged = MergeStepTail(be, model, data, calls + i, n_calls - i);
+        if (merged > 0) { i += merged - 1; continue; }
+        status = DispatchOn(be, model, data, calls[i]);
         if (status != Status::Ok) failed = calls[i].op;
     }
     hipGraph_t graph = nullptr;

@@ -32,4 +32,9 @@ Status OpArticulationDamping(const ModelView&, const DataView&, const void*, hip
 Status OpReferenceWeights(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpSnapshotStepVelocity(const ModelView&, const DataView&, const void*, hipStream_t);
 
+// IntegratePosition, FkWorldPoses, FkLinkVelocities and (when `bodies` is not null) SyncLinkBodyPose as one launch, for
+// a plan whose op list holds them in a row; Unsupported when they must run one by one.
+Status OpStepTail(const ModelView&, const DataView&, const IntegratePositionParams*, const FkWorldPosesParams*,
+                  const FkLinkVelocitiesParams*, const SyncLinkBodyPoseParams*, hipStream_t);
+
 }  // namespace nkh

@@ -9,6 +9,7 @@
 // :647-689) and articulation_mass.cuh (ComputeArticulationMass :124-253, FactorMass :269-335,
 // SolveMassBlock :357-396).
 #include "nk_device_math.h"
+#include "nk_body_pose.h"
 #include "backend.h"
 #include "nk_ops.h"
 
@@ -17,6 +18,14 @@ namespace nkh {
 namespace {
 
 constexpr int kWave = 64;
+
+// Orders one wavefront's LDS writes before its later reads: its lanes run in step and the LDS takes a wavefront's
+// accesses in order, so only the compiler could move them - a fence of wavefront scope holds it without a wait
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 
 __device__ __forceinline__ V3 load3(const float* p) { return V3{p[0], p[1], p[2]}; }
 
@@ -121,11 +130,9 @@ __device__ void motion_subspace(uint8_t type, V3 axis, float* s) {
 }
 
 // ---- FkWorldPoses ---------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(kWave) FkWorldPosesKernel(ModelView m, DataView d, uint32_t env_count) {
-    extern __shared__ float lds[];
-    const uint32_t env = blockIdx.x, lane = threadIdx.x, nl = m.links_per_env;
-    if (env >= env_count) return;
-    float* pose = lds;   // nl * 7
+// One wavefront, one environment; `pose` holds nl * 7 words of LDS
+__device__ __forceinline__ void world_poses_of_env(const ModelView& m, const DataView& d, uint32_t env, uint32_t lane, float* pose) {
+    const uint32_t nl = m.links_per_env;
     const float* q = d.q + size_t{env} * nl;
     // A link's frame in its parent does not wait on the tree: every lane computes its own link's before the sweep, which
     // then only composes a depth at a time (links past the 64th compute theirs when their depth comes).
@@ -148,10 +155,15 @@ __global__ void __launch_bounds__(kWave) FkWorldPosesKernel(ModelView m, DataVie
             const Placed t = place(l);
             if (t.depth == depth) compose(l, t);
         }
-        __syncthreads();
+        wave_sync();
     }
     float* out = d.link_pose + size_t{env} * nl * 7u;
     for (uint32_t e = lane; e < nl * 7u; e += kWave) out[e] = pose[e];
+}
+__global__ void __launch_bounds__(kWave) FkWorldPosesKernel(ModelView m, DataView d, uint32_t env_count) {
+    extern __shared__ float lds[];
+    if (blockIdx.x >= env_count) return;
+    world_poses_of_env(m, d, blockIdx.x, threadIdx.x, lds);
 }
 
 // ---- ArticulationDynamics -------------------------------------------------------------------------------
@@ -161,13 +173,6 @@ __global__ void __launch_bounds__(kWave) FkWorldPosesKernel(ModelView m, DataVie
 // they meet before the solve.  Each keeps to its own words of LDS in between.
 __host__ __device__ inline uint32_t DynamicsLdsFloats(uint32_t nl, uint32_t n) {
     return nl * (36u + 36u + 5u * 6u) + n * (n + 1u) + 2u * n + 64u;
-}
-// Orders one wavefront's LDS writes before its later reads: its lanes run in step and the LDS takes a wavefront's
-// accesses in order, so only the compiler could move them - a fence of wavefront scope holds it without a wait
-__device__ __forceinline__ void wave_sync() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // Compiled per padded DoF width N (a multiple of 4): the LDL^T factorisation and the solve keep one matrix row per
@@ -540,10 +545,9 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
 }
 
 // ---- IntegratePosition: one thread per (env, link) (articulation.cu:732-791) ------------------------------
-__global__ void IntegratePositionKernel(ModelView m, DataView d, IntegratePositionParams p) {
-    const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
-    if (gid >= p.total_link_count) return;
-    const uint32_t nl = m.links_per_env, env = gid / nl, l = gid % nl;
+__device__ __forceinline__ void integrate_position_of_link(const ModelView& m, const DataView& d, const IntegratePositionParams& p,
+                                                            uint32_t env, uint32_t l) {
+    const uint32_t gid = env * m.links_per_env + l;
     const float dt = p.dt;
     if (p.pos_pass != 0u) d.q[gid] += (d.qdot[gid] + d.qdot_pseudo[gid]) * dt;
     else d.q[gid] += d.qdot[gid] * dt;
@@ -562,16 +566,19 @@ __global__ void IntegratePositionKernel(ModelView m, DataView d, IntegratePositi
         store_xf(d.base_pose + size_t{env} * 7u, pose);
     }
 }
+__global__ void IntegratePositionKernel(ModelView m, DataView d, IntegratePositionParams p) {
+    const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= p.total_link_count) return;
+    integrate_position_of_link(m, d, p, gid / m.links_per_env, gid % m.links_per_env);
+}
 
 // ---- FkLinkVelocities (articulation.cu:647-689) ---------------------------------------------------------
-__global__ void __launch_bounds__(kWave) FkLinkVelocitiesKernel(ModelView m, DataView d, uint32_t env_count) {
-    extern __shared__ float lds[];
-    const uint32_t env = blockIdx.x, lane = threadIdx.x, nl = m.links_per_env;
-    if (env >= env_count) return;
-    float* v = lds;   // nl * 6
+// One wavefront, one environment; `v` holds nl * 6 words of LDS
+__device__ __forceinline__ void link_velocities_of_env(const ModelView& m, const DataView& d, uint32_t env, uint32_t lane, float* v) {
+    const uint32_t nl = m.links_per_env;
     const size_t lbase = size_t{env} * nl;
     for (uint32_t e = lane; e < nl * 6u; e += kWave) v[e] = d.link_velocity[lbase * 6u + e];
-    __syncthreads();
+    wave_sync();
     // the joint transform and the joint's own twist do not wait on the tree: a lane prepares its link's before the sweep
     struct Jointed { uint32_t depth, parent; bool state; float X[36], own[6]; };
     auto prepare = [&](uint32_t l, Jointed& t) {
@@ -607,9 +614,33 @@ __global__ void __launch_bounds__(kWave) FkLinkVelocitiesKernel(ModelView m, Dat
             prepare(l, t);
             if (t.depth == depth) propagate(l, t);
         }
-        __syncthreads();
+        wave_sync();
     }
     for (uint32_t e = lane; e < nl * 6u; e += kWave) d.link_velocity[lbase * 6u + e] = v[e];
+}
+__global__ void __launch_bounds__(kWave) FkLinkVelocitiesKernel(ModelView m, DataView d, uint32_t env_count) {
+    extern __shared__ float lds[];
+    if (blockIdx.x >= env_count) return;
+    link_velocities_of_env(m, d, blockIdx.x, threadIdx.x, lds);
+}
+
+// What follows the solve in a step - positions integrated, world poses, link twists, the bodies' poses - as one kernel,
+// one wavefront an environment: four kernels that each take about the time of a launch become one, running the same
+// device code in the same order (IntegratePosition, FkWorldPoses, FkLinkVelocities, SyncLinkBodyPose).  A plan takes this
+// route when its op list holds the four in a row (backend.hip); an op dispatched by itself runs its own kernel.
+__global__ void __launch_bounds__(2 * kWave) StepTailKernel(ModelView m, DataView d, IntegratePositionParams p, uint32_t env_count,
+                                                            uint32_t sync_bodies) {
+    extern __shared__ float lds[];
+    const uint32_t env = blockIdx.x, lane = threadIdx.x % kWave, nl = m.links_per_env;
+    const bool twists = threadIdx.x >= uint32_t(kWave);   // world poses and link twists do not depend on each other: a wavefront each
+    if (env >= env_count) return;
+    if (!twists) for (uint32_t l = lane; l < nl; l += kWave) integrate_position_of_link(m, d, p, env, l);
+    __syncthreads();   // the new coordinates, base pose and root twist are in memory for both wavefronts
+    if (twists) { link_velocities_of_env(m, d, env, lane, lds + nl * 7u); return; }
+    world_poses_of_env(m, d, env, lane, lds);
+    if (sync_bodies == 0u) return;
+    wave_sync();
+    for (uint32_t b = lane; b < m.bodies_per_env; b += kWave) sync_body_pose(m, d, env, b, lds);
 }
 
 }  // namespace
@@ -622,6 +653,22 @@ Status OpFkWorldPoses(const ModelView& m, const DataView& d, const void* params,
     if (m.links_per_env == 0u || p->total_link_count != p->articulation_count * m.links_per_env) return Status::InvalidArgument;
     const size_t lds = size_t{m.links_per_env} * 7u * sizeof(float);
     hipLaunchKernelGGL(FkWorldPosesKernel, dim3(p->articulation_count), dim3(kWave), lds, stream, m, d, p->articulation_count);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
+// The four ops after the solve as one launch; Unsupported when any of them would not run its kernel as dispatched
+// (the caller then dispatches them one by one).
+Status OpStepTail(const ModelView& m, const DataView& d, const IntegratePositionParams* integrate, const FkWorldPosesParams* poses,
+                  const FkLinkVelocitiesParams* twists, const SyncLinkBodyPoseParams* bodies, hipStream_t stream) {
+    if (integrate == nullptr || poses == nullptr || twists == nullptr) return Status::Unsupported;
+    const uint32_t E = poses->articulation_count, links = E * m.links_per_env;
+    if (E == 0u || m.links_per_env == 0u || integrate->dt <= 0.0f || integrate->total_link_count != links ||
+        poses->total_link_count != links || poses->selected_env_count != 0u || twists->articulation_count != E ||
+        twists->total_link_count != links) return Status::Unsupported;
+    if (bodies != nullptr && (bodies->env_count != E || bodies->bodies_per_env != m.bodies_per_env || bodies->bodies_per_env == 0u ||
+                              bodies->selected_env_count != 0u)) return Status::Unsupported;
+    const size_t lds = size_t{m.links_per_env} * 13u * sizeof(float);
+    hipLaunchKernelGGL(StepTailKernel, dim3(E), dim3(2 * kWave), lds, stream, m, d, *integrate, E, bodies != nullptr ? 1u : 0u);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 

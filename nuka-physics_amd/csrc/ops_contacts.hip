@@ -10,6 +10,7 @@
 // :408-474 plus the canonical radix sort :478-542, 630-680), narrowphase_prims.cu (PairDrivenNarrowphaseKernel<false>
 // :181-366) and assemble_rows.cu (:122-214, 325-801, 1479-1605).
 #include "nk_device_math.h"
+#include "nk_body_pose.h"
 #include "nk_ops.h"
 
 namespace nkh {
@@ -40,18 +41,8 @@ __device__ __forceinline__ float motion_radius(float base, float dt, float sa, f
 __global__ void SyncLinkBodyPoseKernel(ModelView m, DataView d, uint32_t total_bodies) {
     const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
     if (gid >= total_bodies) return;
-    const uint32_t nb = m.bodies_per_env, env = gid / nb, b = gid % nb;
-    const uint32_t own = m.body_to_link[b], proxy = m.body_collidable_link[b];
-    if (own != kInvalid) {
-        if (m.link_body[own] != b) return;
-        Xf world = load_xf(d.link_pose + (size_t{env} * m.links_per_env + own) * 7u);
-        if (m.link_geom_kind[own] != 0u) world = compose_collidable(world, load_xf(m.link_geom_local + 7u * own));
-        store_xf(d.body_pose + size_t{gid} * 7u, world);
-    } else if (proxy != kInvalid && proxy < m.links_per_env) {
-        store_xf(d.body_pose + size_t{gid} * 7u,
-                 compose_collidable(load_xf(d.link_pose + (size_t{env} * m.links_per_env + proxy) * 7u),
-                                    load_xf(m.body_collidable_local + 7u * b)));
-    }
+    const uint32_t env = gid / m.bodies_per_env;
+    sync_body_pose(m, d, env, gid % m.bodies_per_env, d.link_pose + size_t{env} * m.links_per_env * 7u);
 }
 
 // broadphase.cu:154-170

@@ -504,3 +504,24 @@ def test_reset_envs_restores_the_selected_environments_only(device):
         assert np.array_equal(world.download(n).reshape(E, -1)[picked], fresh.download(n).reshape(E, -1)[picked]), n
     fresh.close()
     world.close()
+
+
+@pytest.mark.parametrize("index,E", [(3, 512), (1, 64), (5, 64)])
+def test_a_plan_steps_bit_for_bit_like_the_ops_one_by_one(device, index, E):
+    """A plan may run neighbouring ops as one launch (the four after the solve); whatever it merges, the state after
+    any number of steps must be the state the ops leave when each is dispatched by itself."""
+    cfg = nk.synthetic.config(index, E)
+    hashes = []
+    fields = {}
+    for graph in (False, True):
+        world = nk.World(device, cfg.template, abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters))
+        world.set_state(cfg.state())
+        world.set_execution_mode(graph)
+        world.step(5)
+        world.synchronize()
+        hashes.append(world.state_hash())
+        fields[graph] = {name: world.download(name).copy() for name in ("q", "qdot", "base_pose", "link_pose", "link_velocity", "body_pose")}
+        world.close()
+    for name in fields[False]:
+        assert np.array_equal(fields[False][name].view(np.uint32), fields[True][name].view(np.uint32)), name
+    assert hashes[0] == hashes[1]
