@@ -164,6 +164,18 @@ int MergeStepTail(Backend* be, const ModelView& m, const DataView& d, const nuka
     return status == Status::Ok ? (bodies ? 4 : 3) : 0;
 }
 
+// SyncLinkBodyPose, BuildAabbs, LbvhBuild, LbvhQueryPairs, NarrowphasePrimitives at the head of `calls` as one launch
+int MergeCollisionHead(Backend* be, const ModelView& m, const DataView& d, const nuka_phi_op_call* calls, int n) {
+    if (n < 5 || calls[0].op != uint16_t(NkOp::SyncLinkBodyPose) || calls[1].op != uint16_t(NkOp::BuildAabbs) ||
+        calls[2].op != uint16_t(NkOp::LbvhBuild) || calls[3].op != uint16_t(NkOp::LbvhQueryPairs) ||
+        calls[4].op != uint16_t(NkOp::NarrowphasePrimitives) || calls[2].params == nullptr) return 0;
+    const Status status = OpCollisionHead(m, d, static_cast<const SyncLinkBodyPoseParams*>(calls[0].params),
+                                          static_cast<const BuildAabbsParams*>(calls[1].params),
+                                          static_cast<const LbvhQueryPairsParams*>(calls[3].params),
+                                          static_cast<const NarrowphasePrimitivesParams*>(calls[4].params), be->stream);
+    return status == Status::Ok ? 5 : 0;
+}
+
 uint8_t BeDispatch(nuka_phi_backend* b, const nuka_phi_model_view* m, const nuka_phi_data_view* d, const nuka_phi_op_call* call) {
     if (b == nullptr || m == nullptr || d == nullptr || call == nullptr) return uint8_t(Status::InvalidArgument);
     return uint8_t(DispatchOn(reinterpret_cast<Backend*>(b), *reinterpret_cast<const ModelView*>(m),
@@ -201,9 +213,11 @@ nuka_phi_plan* BePlanCreate(nuka_phi_backend* b, const nuka_phi_model_view* m, c
     const ModelView& model = *reinterpret_cast<const ModelView*>(m);
     const DataView& data = *reinterpret_cast<const DataView*>(d);
     for (int i = 0; i < n_calls && status == Status::Ok; ++i) {
-        // The ops after the solve each take about a launch's time: where the list holds them in a row, one kernel runs
-        // the four (ops_articulation.hip StepTailKernel); where it cannot, they go one by one as dispatched.
-        const int merged = MergeStepTail(be, model, data, calls + i, n_calls - i);
+        // The ops after the solve, and those between the dynamics and the row assembly, each take about a launch's time:
+        // where the list holds them in a row, one kernel runs them (StepTailKernel, CollisionHeadKernel); where it cannot,
+        // they go one by one as dispatched.
+        int merged = MergeStepTail(be, model, data, calls + i, n_calls - i);
+        if (merged == 0) merged = MergeCollisionHead(be, model, data, calls + i, n_calls - i);
         if (merged > 0) { i += merged - 1; continue; }
         status = DispatchOn(be, model, data, calls[i]);
         if (status != Status::Ok) failed = calls[i].op;

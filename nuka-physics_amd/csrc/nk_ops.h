@@ -36,5 +36,8 @@ Status OpSnapshotStepVelocity(const ModelView&, const DataView&, const void*, hi
 // a plan whose op list holds them in a row; Unsupported when they must run one by one.
 Status OpStepTail(const ModelView&, const DataView&, const IntegratePositionParams*, const FkWorldPosesParams*,
                   const FkLinkVelocitiesParams*, const SyncLinkBodyPoseParams*, hipStream_t);
+// SyncLinkBodyPose, BuildAabbs, LbvhBuild, LbvhQueryPairs and NarrowphasePrimitives as one launch, likewise.
+Status OpCollisionHead(const ModelView&, const DataView&, const SyncLinkBodyPoseParams*, const BuildAabbsParams*,
+                       const LbvhQueryPairsParams*, const NarrowphasePrimitivesParams*, hipStream_t);
 
 }  // namespace nkh

@@ -54,9 +54,7 @@ __device__ V3 rot_abs(Q4 q, V3 v) {
 
 // ---- BuildAabbs (broadphase.cu:173-270).  Link-owned collidables carry no body velocity on this path, so the
 // motion term of the margin is zero. ----
-__global__ void BuildAabbsKernel(ModelView m, DataView d, BuildAabbsParams p) {
-    const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
-    if (gid >= p.env_count * p.bodies_per_env) return;
+__device__ __forceinline__ void build_aabb_of_body(const ModelView& m, const DataView& d, const BuildAabbsParams& p, uint32_t gid) {
     const uint32_t b = gid % p.bodies_per_env;
     const ShapeRow s = load_shape(m.shape_table, b);
     const Xf xf = load_xf(d.body_pose + size_t{gid} * 7u);
@@ -85,6 +83,11 @@ __global__ void BuildAabbsKernel(ModelView m, DataView d, BuildAabbsParams p) {
     lo[0] = c.x - he.x - mg; lo[1] = c.y - he.y - mg; lo[2] = c.z - he.z - mg;
     hi[0] = c.x + he.x + mg; hi[1] = c.y + he.y + mg; hi[2] = c.z + he.z + mg;
 }
+__global__ void BuildAabbsKernel(ModelView m, DataView d, BuildAabbsParams p) {
+    const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= p.env_count * p.bodies_per_env) return;
+    build_aabb_of_body(m, d, p, gid);
+}
 
 // collision/shape_kind.hpp:26-33
 __device__ __forceinline__ bool shape_filter_admits(uint32_t ta, uint32_t aa, uint32_t ga_, uint32_t tb, uint32_t ab, uint32_t gb_) {
@@ -108,8 +111,9 @@ __device__ bool pair_excluded(const ModelView& m, uint32_t a, uint32_t b) {
 // emitting lane is its slot, which is the ascending (a, b) order the reference reaches by sorting.  The grid runs over
 // the rows that can pass the shape filter at all (a row with empty type and affinity masks pairs with nothing): a
 // humanoid's 31 shapeless link rows leave a grid of 13 x 13 out of 44 x 44. ----
-__global__ void __launch_bounds__(kWave) QueryPairsKernel(ModelView m, DataView d, LbvhQueryPairsParams p) {
-    const uint32_t env = blockIdx.x, lane = threadIdx.x, N = m.pairable_count;
+__device__ __forceinline__ void query_pairs_of_env(const ModelView& m, const DataView& d, const LbvhQueryPairsParams& p, uint32_t env,
+                                                    uint32_t lane) {
+    const uint32_t N = m.pairable_count;
     const size_t bbase = size_t{env} * p.bodies_per_env;
     const uint32_t capacity = min(p.rigid_slot_cap, p.max_pairs);
     uint32_t* pairs = d.candidate_pairs + size_t{env} * p.max_contacts_per_env * 2u;
@@ -146,6 +150,9 @@ __global__ void __launch_bounds__(kWave) QueryPairsKernel(ModelView m, DataView 
         const uint32_t status = d.env_status[env] & ~kEnvStatusPairOverflow;
         d.env_status[env] = overflow ? status | kEnvStatusPairOverflow : status;
     }
+}
+__global__ void __launch_bounds__(kWave) QueryPairsKernel(ModelView m, DataView d, LbvhQueryPairsParams p) {
+    query_pairs_of_env(m, d, p, blockIdx.x, threadIdx.x);
 }
 
 // ---- manifolds (collision/analytical_manifold.hpp) ------------------------------------------------------
@@ -690,8 +697,8 @@ __device__ __forceinline__ uint32_t NarrowphaseSlot(const ModelView& m, const Da
 // One wavefront per environment; its lanes take the environment's slots in strides of 64, and the per-environment
 // contact count is a wave sum (no atomics).
 template <bool kSinglePoint>
-__global__ void __launch_bounds__(64) NarrowphaseKernel(ModelView m, DataView d, NarrowphasePrimitivesParams p) {
-    const uint32_t env = blockIdx.x, lane = threadIdx.x;
+__device__ __forceinline__ void narrowphase_of_env(const ModelView& m, const DataView& d, const NarrowphasePrimitivesParams& p, uint32_t env,
+                                                   uint32_t lane) {
     uint32_t contacts = 0u;
     for (uint32_t first = 0u; first < p.rigid_slot_cap; first += 64u) {
         const uint32_t slot = first + lane;
@@ -699,6 +706,27 @@ __global__ void __launch_bounds__(64) NarrowphaseKernel(ModelView m, DataView d,
     }
     contacts = wave_sum_u(contacts);
     if (lane == 0u) d.contact_count[env] = contacts;
+}
+template <bool kSinglePoint>
+__global__ void __launch_bounds__(64) NarrowphaseKernel(ModelView m, DataView d, NarrowphasePrimitivesParams p) {
+    narrowphase_of_env<kSinglePoint>(m, d, p, blockIdx.x, threadIdx.x);
+}
+
+// What stands between the dynamics and the row assembly - the bodies' poses, their boxes, the candidate pairs, the
+// manifolds - as one kernel, one wavefront an environment: four kernels of about a launch's time each become one, running
+// the same device code in the same order.  Single-point worlds only (the general manifolds keep their candidate lists in
+// scratch memory).  A plan takes this route when its op list holds the ops in a row (backend.hip).
+__global__ void __launch_bounds__(kWave) CollisionHeadKernel(ModelView m, DataView d, BuildAabbsParams boxes, LbvhQueryPairsParams query,
+                                                             NarrowphasePrimitivesParams narrow) {
+    const uint32_t env = blockIdx.x, lane = threadIdx.x, nb = m.bodies_per_env;
+    const float* link_pose = d.link_pose + size_t{env} * m.links_per_env * 7u;
+    for (uint32_t b = lane; b < nb; b += kWave) sync_body_pose(m, d, env, b, link_pose);
+    __syncthreads();   // the poses are in memory for every lane
+    for (uint32_t b = lane; b < nb; b += kWave) build_aabb_of_body(m, d, boxes, env * nb + b);
+    __syncthreads();
+    query_pairs_of_env(m, d, query, env, lane);
+    __syncthreads();
+    narrowphase_of_env<true>(m, d, narrow, env, lane);
 }
 // math/cuda_vec_ops.cuh:150-183
 __device__ void contact_tangent_basis(V3 normal, V3* t1, V3* t2) {
@@ -1308,6 +1336,20 @@ Status OpNarrowphasePrimitives(const ModelView& m, const DataView& d, const void
     if (p->env_count == 0u || p->union_slot_count == 0u || p->rigid_slot_cap == 0u) return Status::Ok;
     if (m.max_points_per_slot <= 1u) hipLaunchKernelGGL(NarrowphaseKernel<true>, dim3(p->env_count), dim3(64), 0, stream, m, d, *p);
     else hipLaunchKernelGGL(NarrowphaseKernel<false>, dim3(p->env_count), dim3(64), 0, stream, m, d, *p);
+    return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+}
+
+// SyncLinkBodyPose, BuildAabbs, LbvhBuild (no tree is built on this path), LbvhQueryPairs and NarrowphasePrimitives as one
+// launch; Unsupported when any of them would not run its kernel as dispatched, or the world has many-point manifolds.
+Status OpCollisionHead(const ModelView& m, const DataView& d, const SyncLinkBodyPoseParams* bodies, const BuildAabbsParams* boxes,
+                       const LbvhQueryPairsParams* query, const NarrowphasePrimitivesParams* narrow, hipStream_t stream) {
+    if (bodies == nullptr || boxes == nullptr || query == nullptr || narrow == nullptr || m.max_points_per_slot > 1u) return Status::Unsupported;
+    const uint32_t E = bodies->env_count, nb = m.bodies_per_env;
+    if (E == 0u || nb == 0u || bodies->bodies_per_env != nb || bodies->selected_env_count != 0u || boxes->env_count != E ||
+        boxes->bodies_per_env != nb || query->env_count != E || query->bodies_per_env != nb || query->excluded_count != 0u ||
+        narrow->env_count != E || narrow->bodies_per_env != nb || narrow->union_slot_count == 0u || narrow->rigid_slot_cap == 0u)
+        return Status::Unsupported;
+    hipLaunchKernelGGL(CollisionHeadKernel, dim3(E), dim3(kWave), 0, stream, m, d, *boxes, *query, *narrow);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
 
