@@ -34,6 +34,7 @@ enum class NkOp : uint16_t {
 const char* OpName(NkOp op);
 
 constexpr uint32_t kInvalid = 0xFFFFFFFFu;
+constexpr uint32_t kSweepLinks = 10u;      // links a pass of the dynamics' tree sweeps: six lanes a link
 constexpr uint32_t kMaxDof = 64u;          // src/phi/articulation_contract.hpp:25
 constexpr uint32_t kShapeStride = 13u;     // src/phi/op_schema.hpp:26
 constexpr uint32_t kRowWords = 26u;        // src/nk/solve/nk_row.hpp:99-100
@@ -69,6 +70,7 @@ struct ModelView {
     uint32_t profile_count, floating_root;
     uint32_t max_points_per_slot;   // most points a manifold of the template's admitted pairs can hold (sizes the solver's staged rows)
     uint32_t excluded_pair_count;
+    uint32_t sweep_passes;     // passes of the dynamics' tree sweeps (sweep_links)
     uint32_t pairable_count;   // collidable rows that can pass the shape filter with some partner (pairable_rows, ascending)
     // joint row slots after the contact rows: 2 per link, 1 per link, 1 per link, or 0 (scene/cook/cook_to_model.cpp:706-719)
     uint32_t joint_limit_rows, joint_friction_rows, joint_drive_rows, drive_mode;
@@ -99,6 +101,7 @@ struct ModelView {
     const uint32_t* link_tree_depth;
     const uint32_t* link_child_range;
     const uint32_t* link_children;
+    const uint32_t* sweep_links;       // [sweep_passes][kSweepLinks]: the links a depth at a time, ten a pass, kInvalid where a pass ends early
     const uint32_t* link_push_order;   // children in the order the composite-inertia pass adds them to their parents, then kInvalid
     const uint32_t* link_dof;
     const uint32_t* dof_link;

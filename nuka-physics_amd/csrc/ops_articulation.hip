@@ -171,12 +171,15 @@ __global__ void __launch_bounds__(kWave) FkWorldPosesKernel(ModelView m, DataVie
 // mass matrix with its factor (composite inertias, columns, LDL^T) do not depend on each other, and each is a chain of
 // tree sweeps that keeps a few lanes busy: the first wavefront takes the one, the second the other, side by side, and
 // they meet before the solve.  Each keeps to its own words of LDS in between.
-__host__ __device__ inline uint32_t DynamicsLdsFloats(uint32_t nl, uint32_t n) {
-    return nl * (36u + 36u + 5u * 6u) + n * (n + 1u) + 2u * n + 64u;
+__host__ __device__ inline uint32_t DynamicsLdsFloats(uint32_t nl, uint32_t n, uint32_t sweep_passes) {
+    return nl * (36u + 36u + 5u * 6u) + n * (n + 1u) + 2u * n + 64u + nl * 7u + sweep_passes * kSweepLinks;
 }
 
 // Compiled per padded DoF width N (a multiple of 4): the LDL^T factorisation and the solve keep one matrix row per
 // lane in registers, fully unrolled, and pass pivots and multipliers between lanes as scalar lane reads.
+// The tree sweeps run six lanes a link - a lane a row of the link's 6x6 products - and ten links a pass, a depth at a
+// time from the cooked pass list (ModelView::sweep_links): a pass costs about a third of the instructions of a lane a
+// link carrying all six rows, and each row sums in the order the whole product does.
 template <int N>
 __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelView m, DataView d, ArticulationDynamicsParams p,
                                                                        uint32_t env_count) {
@@ -195,23 +198,37 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
     float* vel = A + n * (n + 1u);
     float* acc = vel + n;
     float* tmp = acc + n;             // 36 floats of the inertia push, padded to 64
+    // the tree as the sweeps read it, a word a link each: parent, joint type, first coordinate, child range, children, rate
+    uint32_t* t_parent = reinterpret_cast<uint32_t*>(tmp + 64u);
+    uint32_t* t_type = t_parent + nl;
+    uint32_t* t_dof = t_type + nl;
+    uint32_t* t_child_begin = t_dof + nl;
+    uint32_t* t_child_end = t_child_begin + nl;
+    uint32_t* t_children = t_child_end + nl;
+    float* t_rate = reinterpret_cast<float*>(t_children + nl);
+    uint32_t* sweep = reinterpret_cast<uint32_t*>(t_rate + nl);   // sweep_passes x kSweepLinks links, kInvalid where a pass ends early
+    const uint32_t passes = m.sweep_passes;
     const uint32_t ld = n + 1u;
     const size_t lbase = size_t{env} * nl;
     const float* q = d.q + lbase;
     float* qd = d.qdot + lbase;
     const V3 gravity{p.gravity[0], p.gravity[1], p.gravity[2]};
     const Q4 base_rot = load_xf(d.base_pose + size_t{env} * 7u).r;
-    // A lane's own link: its place in the tree and its joint rate, read once.  The passes below visit the tree a depth at
-    // a time and every visit would otherwise wait on these loads again (links past the 64th read theirs at each visit).
-    struct LinkTree { uint32_t depth, parent, child_begin, child_end; uint8_t type; float rate; };
-    auto tree_of = [&](uint32_t l) {
-        return LinkTree{m.link_tree_depth[l], m.parent_link[l], m.link_child_range[2u * l], m.link_child_range[2u * l + 1u], m.joint_type[l], qd[l]};
-    };
-    const LinkTree own = lane < nl ? tree_of(lane) : LinkTree{kInvalid, kInvalid, 0u, 0u, uint8_t(0), 0.0f};
+    const uint32_t slot = lane / 6u, srow = lane - 6u * slot;   // of the sweeps: lanes 60..63 sit them out
+    const uint32_t ri = srow % 3u, rj = (ri + 1u) % 3u, rk = (ri + 2u) % 3u;
+    auto link_of_pass = [&](uint32_t pass) { return lane < 6u * kSweepLinks ? sweep[pass * kSweepLinks + slot] : kInvalid; };
+    const V3 gravity_in_base = rotate_inverse(base_rot, gravity);
+    const float gravity_in_base_row = srow < 3u ? 0.0f : (srow == 3u ? gravity_in_base.x : srow == 4u ? gravity_in_base.y : gravity_in_base.z);
 
-    if (!forces) {   // what the mass matrix starts from, while the first wavefront builds the joint transforms
+    if (!forces) {   // what the mass matrix starts from and the sweeps' tables, while the first wavefront builds the joint transforms
         for (uint32_t e = lane; e < nl * 36u; e += kWave) ic[e] = m.link_inertia[e];
         for (uint32_t e = lane; e < n * ld; e += kWave) A[e] = 0.0f;
+        for (uint32_t l = lane; l < nl; l += kWave) {
+            t_parent[l] = m.parent_link[l]; t_type[l] = m.joint_type[l]; t_dof[l] = m.link_dof[l];
+            t_child_begin[l] = m.link_child_range[2u * l]; t_child_end[l] = m.link_child_range[2u * l + 1u];
+            t_children[l] = m.link_children[l]; t_rate[l] = qd[l];
+        }
+        for (uint32_t e = lane; e < passes * kSweepLinks; e += kWave) sweep[e] = m.sweep_links[e];
     }
     // link twists of the state enter LDS (a floating root's twist is state; the rest is rebuilt)
     for (uint32_t e = lane; forces && e < nl * 6u; e += kWave) v[e] = d.link_velocity[lbase * 6u + e];
@@ -232,27 +249,27 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
     float row[N];   // the second wavefront's row of the mass matrix, then of its factor
     if (forces) {
         // velocities root to leaf (:334-363)
-        for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
-            for (uint32_t l = lane; l < nl; l += kWave) {
-                const LinkTree t = l == lane ? own : tree_of(l);
-                if (t.depth != depth) continue;
-                const uint32_t parent = t.parent;
-                if (parent == kInvalid && t.type == kFloatingBase) continue;
-                float vp[6] = {0, 0, 0, 0, 0, 0}, tp[6], jv[6], vl[6];
-                if (parent != kInvalid) {
+        for (uint32_t pass = 0u; pass < passes; ++pass) {
+            const uint32_t l = link_of_pass(pass);
+            const bool moves = l != kInvalid && !(t_parent[l] == kInvalid && t_type[l] == kFloatingBase);   // a floating root's twist is state
+            if (moves) {
+                const uint32_t parent = t_parent[l];
+                const float* X = xup + 36u * l + 6u * srow;
+                float through = 0.0f;
 #pragma unroll
-                    for (int i = 0; i < 6; ++i) vp[i] = v[6u * parent + i];
-                }
-                mat66_vec(xup + 36u * l, vp, tp);
-                const float qdl = t.rate;
-#pragma unroll
-                for (int i = 0; i < 6; ++i) { jv[i] = S[6u * l + i] * qdl; vl[i] = tp[i] + jv[i]; }
-#pragma unroll
-                for (int i = 0; i < 6; ++i) v[6u * l + i] = vl[i];
-                motion_cross(vl, jv, vb + 6u * l);
+                for (int c = 0; c < 6; ++c) through += X[c] * (parent != kInvalid ? v[6u * parent + c] : 0.0f);
+                v[6u * l + srow] = through + S[6u * l + srow] * t_rate[l];
             }
             wave_sync();
+            if (moves) {   // the link's twist crossed with its joint's own twist, row by row (motion_cross)
+                const float* vl = v + 6u * l, *s6 = S + 6u * l;
+                const float rate = t_rate[l];
+                const float first = vl[rj] * (s6[(srow < 3u ? 0u : 3u) + rk] * rate) - vl[rk] * (s6[(srow < 3u ? 0u : 3u) + rj] * rate);
+                const float second = vl[3u + rj] * (s6[rk] * rate) - vl[3u + rk] * (s6[rj] * rate);
+                vb[6u * l + srow] = srow < 3u ? first : first + second;
+            }
         }
+        wave_sync();
         // p = v x* (I v) - external wrench (:364-374, 279-295)
         for (uint32_t l = lane; l < nl; l += kWave) {
             float vl[6], iv[6], bf[6];
@@ -275,26 +292,19 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
         }
         wave_sync();
         // bias accelerations with gravity as base acceleration (:526-547)
-        for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
-            for (uint32_t l = lane; l < nl; l += kWave) {
-                const LinkTree t = l == lane ? own : tree_of(l);
-                if (t.depth != depth) continue;
-                float al[6];
-                const uint32_t parent = t.parent;
-                if (parent != kInvalid) {
-                    float ap[6];
+        for (uint32_t pass = 0u; pass < passes; ++pass) {
+            const uint32_t l = link_of_pass(pass);
+            if (l != kInvalid) {
+                const uint32_t parent = t_parent[l];
+                float al;
+                if (parent == kInvalid && t_type[l] == kFloatingBase) al = srow < 3u ? 0.0f : -gravity_in_base_row;
+                else {
+                    const float* X = xup + 36u * l + 6u * srow;
+                    al = 0.0f;
 #pragma unroll
-                    for (int i = 0; i < 6; ++i) ap[i] = a[6u * parent + i];
-                    mat66_vec(xup + 36u * l, ap, al);
-                } else if (t.type == kFloatingBase) {
-                    const V3 g = rotate_inverse(base_rot, gravity);
-                    al[0] = al[1] = al[2] = 0.0f; al[3] = -g.x; al[4] = -g.y; al[5] = -g.z;
-                } else {
-                    const float world[6] = {0.0f, 0.0f, 0.0f, -gravity.x, -gravity.y, -gravity.z};
-                    mat66_vec(xup + 36u * l, world, al);
+                    for (int c = 0; c < 6; ++c) al += X[c] * (parent != kInvalid ? a[6u * parent + c] : (c < 3 ? 0.0f : (c == 3 ? -gravity.x : c == 4 ? -gravity.y : -gravity.z)));
                 }
-#pragma unroll
-                for (int i = 0; i < 6; ++i) a[6u * l + i] = al[i] + vb[6u * l + i];
+                a[6u * l + srow] = al + vb[6u * l + srow];
             }
             wave_sync();
         }
@@ -308,20 +318,20 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
             for (int i = 0; i < 6; ++i) pf[6u * l + i] += f[i];
         }
         wave_sync();
-        // leaf to root, children in CSR order (:557-569)
-        for (uint32_t remaining = m.max_depth + 1u; remaining > 0u; --remaining) {
-            for (uint32_t l = lane; l < nl; l += kWave) {
-                const LinkTree t = l == lane ? own : tree_of(l);
-                if (t.depth != remaining - 1u) continue;
-                for (uint32_t i = t.child_begin; i < t.child_end; ++i) {
-                    const uint32_t child = m.link_children[i];
-                    float pc[6], f[6];
+        // leaf to root, children in CSR order (:557-569): the passes backwards, a lane a row of every child's X^T p
+        for (uint32_t pass = passes; pass-- > 0u;) {
+            const uint32_t l = link_of_pass(pass);
+            if (l != kInvalid) {
+                float total = pf[6u * l + srow];
+                for (uint32_t i = t_child_begin[l]; i < t_child_end[l]; ++i) {
+                    const uint32_t child = t_children[i];
+                    const float* X = xup + 36u * child + srow, *pc = pf + 6u * child;
+                    float pushed = 0.0f;
 #pragma unroll
-                    for (int c = 0; c < 6; ++c) pc[c] = pf[6u * child + c];
-                    mat66t_vec(xup + 36u * child, pc, f);
-#pragma unroll
-                    for (int c = 0; c < 6; ++c) pf[6u * l + c] += f[c];
+                    for (int c = 0; c < 6; ++c) pushed += X[6 * c] * pc[c];
+                    total += pushed;
                 }
+                pf[6u * l + srow] = total;
             }
             wave_sync();
         }
@@ -366,18 +376,18 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
                 const uint32_t l = uint32_t(__builtin_amdgcn_readlane(int(my_parent), int(visit)));
                 const float* X = xup + 36u * child;
                 const float* C = ic + 36u * child;
-                const uint32_t row = lane / 6u, col = lane % 6u;
+                const uint32_t entry_row = lane / 6u, entry_col = lane % 6u;
                 if (lane < 36u) {
                     float value = 0.0f;
 #pragma unroll
-                    for (int k = 0; k < 6; ++k) value += C[row * 6u + k] * X[k * 6u + col];
+                    for (int k = 0; k < 6; ++k) value += C[entry_row * 6u + k] * X[k * 6u + entry_col];
                     tmp[lane] = value;
                 }
                 wave_sync();
                 if (lane < 36u) {
                     float value = 0.0f;
 #pragma unroll
-                    for (int k = 0; k < 6; ++k) value += X[k * 6u + row] * tmp[k * 6u + col];
+                    for (int k = 0; k < 6; ++k) value += X[k * 6u + entry_row] * tmp[k * 6u + entry_col];
                     ic[36u * l + lane] += value;
                 }
                 wave_sync();
@@ -508,33 +518,21 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
     }
     wave_sync();
     // final link accelerations (:617-644)
-    for (uint32_t depth = 0u; depth <= m.max_depth; ++depth) {
-        for (uint32_t l = lane; l < nl; l += kWave) {
-            const LinkTree t = l == lane ? own : tree_of(l);
-            if (t.depth != depth) continue;
-            float al[6];
-            const uint32_t parent = t.parent;
-            if (t.type == kFloatingBase) {
-                const V3 g = rotate_inverse(base_rot, gravity);
+    for (uint32_t pass = 0u; pass < passes; ++pass) {
+        const uint32_t l = link_of_pass(pass);
+        if (l != kInvalid) {
+            const uint32_t parent = t_parent[l], type = t_type[l];
+            float al;
+            if (type == kFloatingBase) al = srow < 3u ? acc[srow] : acc[srow] - gravity_in_base_row;
+            else {
+                const float* X = xup + 36u * l + 6u * srow;
+                al = 0.0f;
 #pragma unroll
-                for (int c = 0; c < 6; ++c) al[c] = acc[c];
-                al[3] -= g.x; al[4] -= g.y; al[5] -= g.z;
-            } else {
-                if (parent != kInvalid) {
-                    float ap[6];
-#pragma unroll
-                    for (int i = 0; i < 6; ++i) ap[i] = a[6u * parent + i];
-                    mat66_vec(xup + 36u * l, ap, al);
-                } else {
-                    const float world[6] = {0.0f, 0.0f, 0.0f, -gravity.x, -gravity.y, -gravity.z};
-                    mat66_vec(xup + 36u * l, world, al);
-                }
-                const float qdd = joint_dof(t.type) == 1u ? acc[m.link_dof[l]] : 0.0f;
-#pragma unroll
-                for (int c = 0; c < 6; ++c) al[c] += vb[6u * l + c] + S[6u * l + c] * qdd;
+                for (int c = 0; c < 6; ++c) al += X[c] * (parent != kInvalid ? a[6u * parent + c] : (c < 3 ? 0.0f : (c == 3 ? -gravity.x : c == 4 ? -gravity.y : -gravity.z)));
+                const float qdd = joint_dof(uint8_t(type)) == 1u ? acc[t_dof[l]] : 0.0f;
+                al += vb[6u * l + srow] + S[6u * l + srow] * qdd;
             }
-#pragma unroll
-            for (int c = 0; c < 6; ++c) a[6u * l + c] = al[c];
+            a[6u * l + srow] = al;
         }
         wave_sync();
     }
@@ -685,7 +683,7 @@ Status OpArticulationDynamics(const ModelView& m, const DataView& d, const void*
     if (p->articulation_count == 0u || p->total_link_count == 0u) return Status::Ok;
     if (m.dof > kMaxDof || m.dof == 0u || p->max_dof != m.max_dof ||
         p->total_link_count != p->articulation_count * m.links_per_env) return Status::InvalidArgument;
-    const size_t lds = size_t{DynamicsLdsFloats(m.links_per_env, m.dof)} * sizeof(float);
+    const size_t lds = size_t{DynamicsLdsFloats(m.links_per_env, m.dof, m.sweep_passes)} * sizeof(float);
     if (lds > 160u * 1024u) return Status::InvalidArgument;
     hipLaunchKernelGGL(kDynamicsKernels[((m.dof + 3u) & ~3u) / 4u - 1u], dim3(p->articulation_count), dim3(2 * kWave), lds, stream, m, d,
                        *p, p->articulation_count);

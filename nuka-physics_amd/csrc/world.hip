@@ -62,7 +62,7 @@ uint32_t JointWidth(uint8_t type) { return type <= kPrismatic ? 1u : type == kFl
 struct HostModel {
     ModelView counts{};   // scalar members only
     std::vector<uint8_t> joint_type, joint_limit_flags, joint_law;
-    std::vector<uint32_t> parent_link, link_body, link_tree_depth, link_child_range, link_children, link_push_order, link_dof, dof_link, dof_component,
+    std::vector<uint32_t> parent_link, link_body, link_tree_depth, link_child_range, link_children, link_push_order, sweep_links, link_dof, dof_link, dof_component,
         link_geom_kind, body_to_link, body_to_articulation, body_collidable_link, body_collidable_body, pairable_rows;
     std::vector<uint64_t> link_dof_mask, excluded_pairs;
     std::vector<float> joint_axis, parent_offset, link_local_pose, link_inertial_frame, link_inertia, joint_damping, joint_armature,
@@ -175,6 +175,18 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
             for (uint32_t i = m.link_child_range[2u * l]; i < m.link_child_range[2u * l + 1u]; ++i) m.link_push_order.push_back(m.link_children[i]);
         }
     m.link_push_order.resize(nl, kInvalid);
+    // the dynamics' tree sweeps: the links of one depth, ten a pass (a pass that ends early is filled with kInvalid)
+    m.sweep_links.clear();
+    for (uint32_t depth = 0u; depth <= max_depth; ++depth) {
+        uint32_t in_pass = 0u;
+        for (uint32_t l = 0u; l < nl; ++l) {
+            if (m.link_tree_depth[l] != depth) continue;
+            m.sweep_links.push_back(l);
+            in_pass = (in_pass + 1u) % kSweepLinks;
+        }
+        while (in_pass != 0u) { m.sweep_links.push_back(kInvalid); in_pass = (in_pass + 1u) % kSweepLinks; }
+    }
+    m.counts.sweep_passes = uint32_t(m.sweep_links.size() / kSweepLinks);
     m.shape_table.assign(size_t{nb} * kShapeStride, 0.0f);
     m.body_to_link.assign(nb, kInvalid);
     m.body_to_articulation.assign(nb, kInvalid);
@@ -366,7 +378,7 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(link_inertial_frame, kF32) X(link_inertia, kF32) X(joint_damping, kF32) X(joint_armature, kF32) X(joint_stiffness, kF32) \
     X(joint_spring_reference, kF32) X(joint_limit_lower, kF32) X(joint_limit_upper, kF32) X(joint_frictionloss, kF32) \
     X(joint_limit_flags, kU8) X(joint_law, kU8) X(joint_limit_margin, kF32) X(joint_limit_reference, kF32) \
-    X(joint_friction_reference, kF32) X(link_body, kU32) X(link_tree_depth, kU32) X(link_child_range, kU32) X(link_children, kU32) X(link_push_order, kU32) \
+    X(joint_friction_reference, kF32) X(link_body, kU32) X(link_tree_depth, kU32) X(link_child_range, kU32) X(link_children, kU32) X(link_push_order, kU32) X(sweep_links, kU32) \
     X(link_dof, kU32) X(dof_link, kU32) X(dof_component, kU32) X(link_dof_mask, kU64) X(link_geom_kind, kU32) \
     X(link_geom_local, kF32) X(shape_table, kF32) X(body_to_link, kU32) X(body_to_articulation, kU32) \
     X(body_collidable_link, kU32) X(body_collidable_body, kU32) X(body_collidable_local, kF32) X(pairable_rows, kU32) X(profile_mu, kF32) \
