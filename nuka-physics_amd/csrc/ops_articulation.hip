@@ -397,9 +397,9 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
         wave_sync();
         // mass columns: each jointed link pushes Ic S to the root (:183-252)
         for (uint32_t l = lane; l < nl; l += kWave) {
-            if (joint_dof(m.joint_type[l]) == 0u) continue;
+            if (joint_dof(uint8_t(t_type[l])) == 0u) continue;
             if (l == 0u && floating_root) continue;
-            const uint32_t dof_i = m.link_dof[l];
+            const uint32_t dof_i = t_dof[l];
             float force[6], sl[6];
 #pragma unroll
             for (int i = 0; i < 6; ++i) sl[i] = S[6u * l + i];
@@ -410,15 +410,15 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
             A[dof_i * ld + dof_i] = diagonal;
             uint32_t walk = l;
             for (;;) {
-                const uint32_t parent = m.parent_link[walk];
+                const uint32_t parent = t_parent[walk];   // the walk reads the tree from LDS: a table load a hop would be its latency
                 if (parent == kInvalid) break;
                 float pushed[6];
                 mat66t_vec(xup + 36u * walk, force, pushed);
 #pragma unroll
                 for (int i = 0; i < 6; ++i) force[i] = pushed[i];
                 walk = parent;
-                if (joint_dof(m.joint_type[walk]) == 0u) continue;
-                const uint32_t dof_j = m.link_dof[walk];
+                if (joint_dof(uint8_t(t_type[walk])) == 0u) continue;
+                const uint32_t dof_j = t_dof[walk];
                 if (walk == 0u && floating_root) {
 #pragma unroll
                     for (int b = 0; b < 6; ++b) { A[dof_i * ld + b] = force[b]; A[b * ld + dof_i] = force[b]; }
