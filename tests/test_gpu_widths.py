@@ -56,3 +56,22 @@ def test_steps_at_wide_widths_stay_with_the_oracle(oracle_py, device, dof, float
             close(world, oracle, name, tol=TOL if step == 0 else 3 * TOL)
     world.close()
     oracle.close()
+
+
+@pytest.mark.parametrize("dof,floating,limb_joints", [(48, True, 3), (40, True, 2), (64, True, 4)])
+def test_trees_wider_than_a_sweep_pass_match_the_oracle(oracle_py, device, dof, floating, limb_joints):
+    """Bushy trees: more links at one depth (14, 17 and 15) than a pass of the dynamics' tree sweeps holds (ten), so a depth
+    takes several passes; every op against the oracle as above."""
+    E = 32
+    tree, desc, state = tree_case(oracle_py, dof, floating, True, seed=5 * dof + limb_joints, E=E, limb_joints=limb_joints)
+    oracle = oracle_py.OracleWorld(tree.template, desc, threads=8)
+    world = nk.World(device, tree.template, desc)
+    assert world.dof == dof
+    oracle.set_state(state)
+    world.set_state(state)
+    sens = one_ulp_sensitivity(oracle_py, tree.template, desc, state)
+    compare_ops(oracle, world, E, sens, state)
+    close(world, oracle, "link_velocity", tol=bar(sens, "velocity"))
+    close(world, oracle, "link_acceleration", tol=bar(sens, "qdd"))
+    world.close()
+    oracle.close()
