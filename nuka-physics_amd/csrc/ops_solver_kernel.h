@@ -936,14 +936,18 @@ __device__ __forceinline__ void plain_line_terms(const PlainLine& p, float alpha
     row_magnitude += fabsf(f[0] * sx) + fabsf(f[1] * sy) + fabsf(f[2] * sz);
     row_curvature += r[0] * sx * sx + r[1] * sy * sy + r[2] * sz * sz + 2.0f * r[5] * sy * sz;
 }
-// `general` (uniform): the block has more heads than lanes, or some head is under the elliptic cone
-__device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& mine, const PlainLine& plain, bool general, float alpha,
+// The line search runs in one of three modes, the same for every probe of a solve: general (the block has more heads
+// than lanes, or some head is under the elliptic cone), plain with the terms in the first sixteen lanes (narrow), plain
+// over the whole wavefront.  The mode is a template argument so that the probes carry no branch on it.
+enum LineMode : int { kLineGeneral = 0, kLineWide = 1, kLineNarrow = 2 };
+template <LineMode kMode>
+__device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& mine, const PlainLine& plain, float alpha,
                                  float inertial_slope, float inertial_curvature, float* slope, float* curvature, float* magnitude) {
     PROF_COUNT(c, 1);
     c.work += 1u;
     TileSum row_slope{0.0f, 0.0f};
     float row_curvature = 0.0f, row_magnitude = 0.0f;
-    if (general) {
+    if constexpr (kMode == kLineGeneral) {
         if (mine.owned) line_terms(mine, alpha, row_slope, row_curvature, row_magnitude);
         for (uint32_t h = c.lane + kWave; h < c.heads; h += kWave) {
             const HeadLine extra = load_head_line(c, h);
@@ -958,18 +962,25 @@ __device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& 
         tile_add_product(total, alpha, inertial_curvature);
         tile_add(total, inertial_slope);
     }
-    // with at most sixteen heads every term sits in the first row of lanes; (t + 0) + (0 + 0) is t, so the sums agree
-    const bool narrow = c.heads <= 16u;
-    *slope = wave_total(total, narrow);
-    *curvature = inertial_curvature + (narrow ? first_row_sum(row_curvature) : wave_sum(row_curvature));
-    *magnitude = fabsf(inertial_slope) + alpha * inertial_curvature + (narrow ? first_row_sum(row_magnitude) : wave_sum(row_magnitude));
+    if constexpr (kMode == kLineNarrow) {
+        // with at most sixteen heads every term sits in the first row of lanes; (t + 0) + (0 + 0) is t, so the sums agree
+        *slope = wave_total(total, true);
+        *curvature = inertial_curvature + first_row_sum(row_curvature);
+        *magnitude = fabsf(inertial_slope) + alpha * inertial_curvature + first_row_sum(row_magnitude);
+    } else {
+        // the general mode takes the first-row sums too when its heads fit the first sixteen lanes
+        const bool narrow = c.heads <= 16u;
+        *slope = wave_total(total, narrow);
+        *curvature = inertial_curvature + (narrow ? first_row_sum(row_curvature) : wave_sum(row_curvature));
+        *magnitude = fabsf(inertial_slope) + alpha * inertial_curvature + (narrow ? first_row_sum(row_magnitude) : wave_sum(row_magnitude));
+    }
     PROF_END(c, 25);
 }
 
-// The search always evaluates the line at 0 and then at 1.  With at most sixteen heads, none of them general, the rows
-// of sixteen lanes hold copies of the same heads (lane & 15) and the row sums stay within a row: the first row
-// evaluates the line at 0 while the others evaluate it at 1, one pass for both points with the numbers either gives
-// alone.  Each point's sums come out in its row's lanes.
+// The search always evaluates the line at 0 and then at 1.  In the narrow mode the rows of sixteen lanes hold copies of
+// the same heads (lane & 15) and the row sums stay within a row: the first row evaluates the line at 0 while the others
+// evaluate it at 1, one pass for both points with the numbers either gives alone.  Each point's sums come out in its
+// row's lanes.
 struct LinePoint { float slope, curvature, magnitude; };
 __device__ __forceinline__ void line_derivatives_pair(const Tile& c, const PlainLine& plain, float inertial_slope, float inertial_curvature,
                                                       LinePoint* at_zero, LinePoint* at_one) {
@@ -999,45 +1010,57 @@ __device__ __forceinline__ void line_derivatives_pair(const Tile& c, const Plain
 }
 
 // SearchTileLine (:2089-2125)
-__device__ __forceinline__ float search_line(const Tile& c, float inertial_slope, float inertial_curvature) {
+template <LineMode kMode>
+__device__ __forceinline__ float search_line_in(const Tile& c, float inertial_slope, float inertial_curvature) {
+    constexpr bool kPaired = kMode == kLineNarrow;
     float slope = 0.0f, curvature = 0.0f, magnitude = 0.0f;
-    const bool general = c.heads > uint32_t(kWave) || c.elliptic;
-    const bool paired = !general && c.heads <= 16u;
-    const HeadLine mine = load_head_line(c, paired ? (c.lane & 15u) : c.lane);
+    const HeadLine mine = load_head_line(c, kPaired ? (c.lane & 15u) : c.lane);
     const PlainLine plain = plain_line(mine);
-    LinePoint at_one{0.0f, 0.0f, 0.0f};
-    if (paired) {
-        LinePoint at_zero;
-        line_derivatives_pair(c, plain, inertial_slope, inertial_curvature, &at_zero, &at_one);
-        c.work += 1u;
-        slope = at_zero.slope;
-    } else {
-        line_derivatives(c, mine, plain, general, 0.0f, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
-    }
-    const float initial = slope;
-    if (!(initial < 0.0f)) return 0.0f;
     float low = 0.0f, high = 0.0f, alpha = 1.0f;
     bool bounded = false;
-    for (uint32_t step = 0u; step < kLineSearchSteps; ++step) {
-        if (paired && step == 0u) {
-            slope = at_one.slope; curvature = at_one.curvature; magnitude = at_one.magnitude;
-            c.work += 1u;
-        } else {
-            line_derivatives(c, mine, plain, general, alpha, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
-        }
+    float initial;
+    uint32_t step = 0u;
+    // one turn of the search on the line's slope and curvature at alpha: true when the search ends, with its answer
+    auto turn = [&](float* answer) {
         if (!isfinite(slope) || !isfinite(curvature)) {
             high = alpha; bounded = true; alpha = 0.5f * (low + high);
-            continue;
+            return false;
         }
-        if (fabsf(slope) <= fmaxf(kLineTolerance * -initial, kRoundings * FLT_EPSILON * magnitude)) return alpha;
+        if (fabsf(slope) <= fmaxf(kLineTolerance * -initial, kRoundings * FLT_EPSILON * magnitude)) { *answer = alpha; return true; }
         if (slope < 0.0f) low = alpha;
         else { high = alpha; bounded = true; }
-        if (bounded && high - low <= FLT_EPSILON * high) break;
+        if (bounded && high - low <= FLT_EPSILON * high) { *answer = low; return true; }
         float next = alpha - slope / curvature;
         if (!(next > low && (!bounded || next < high))) next = bounded ? 0.5f * (low + high) : 2.0f * alpha;
         alpha = next;
+        return false;
+    };
+    float answer = 0.0f;
+    if constexpr (kPaired) {
+        LinePoint at_zero, at_one;
+        line_derivatives_pair(c, plain, inertial_slope, inertial_curvature, &at_zero, &at_one);
+        c.work += 1u;
+        initial = at_zero.slope;
+        if (!(initial < 0.0f)) return 0.0f;
+        slope = at_one.slope; curvature = at_one.curvature; magnitude = at_one.magnitude;
+        c.work += 1u;
+        if (turn(&answer)) return answer;
+        step = 1u;
+    } else {
+        line_derivatives<kMode>(c, mine, plain, 0.0f, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
+        initial = slope;
+        if (!(initial < 0.0f)) return 0.0f;
+    }
+    for (; step < kLineSearchSteps; ++step) {
+        line_derivatives<kMode>(c, mine, plain, alpha, inertial_slope, inertial_curvature, &slope, &curvature, &magnitude);
+        if (turn(&answer)) return answer;
     }
     return low;
+}
+__device__ __forceinline__ float search_line(const Tile& c, float inertial_slope, float inertial_curvature) {
+    if (c.heads > uint32_t(kWave) || c.elliptic) return search_line_in<kLineGeneral>(c, inertial_slope, inertial_curvature);
+    if (c.heads <= 16u) return search_line_in<kLineNarrow>(c, inertial_slope, inertial_curvature);
+    return search_line_in<kLineWide>(c, inertial_slope, inertial_curvature);
 }
 
 __device__ __forceinline__ void apply_moves(const Tile& c, float alpha) {
