@@ -15,6 +15,7 @@
 // Not built: free rigid 6x6 blocks, mimic couplings, elliptic (MuJoCo-law) cones.
 #pragma once
 
+#include <utility>
 #include "nk_device_math.h"
 #include "backend.h"
 #include "nk_ops.h"
@@ -504,8 +505,78 @@ __device__ __forceinline__ float solve_tile_mass(const Tile& c, float force) {
     return substitute<N>(c.lane, row, col, c.mass_inverse, c.lane < c.n ? force : 0.0f);
 }
 
+// The LDS byte address of a pointer into the block's shared memory.
+__device__ __forceinline__ uint32_t lds_address(const float* p) {
+    return uint32_t(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const float*)p));
+}
+
+// Four columns of a head's Hessian term, taken or left as a whole on a uniform mask, with the products and sums the
+// plain loops of add_head form.  Three rows: h += a0 x0 + a1 x1 + a2 x2 as a product, two fused multiply-adds and a
+// sum.  A single row: one fused multiply-add into h.  Written out because the compiled form of such a conditional
+// update carries the whole row through the head loop twice and copies one set of registers into the other at every
+// branch, about as many moves as the update has arithmetic.  Here the row's registers change in place, and the words
+// come from LDS (`kFirst`, `kSecond`, `kThird` bytes past `row_address`) into twelve registers that the block takes for
+// itself, v244-v255.  Only for widths that run two waves a SIMD: their kernels leave those registers free.  The waits
+// count LDS reads only as far as those return in order; scalar loads in flight make them wait longer, never shorter.
+template <int kFirst, int kSecond, int kThird>
+__device__ __forceinline__ void add_columns_if(uint32_t live, uint32_t single, uint32_t row_address, float a0, float a1, float a2, float& h0,
+                                               float& h1, float& h2, float& h3) {
+    asm volatile(
+        "s_cmp_eq_u32 %[live], 0\n\t"
+        "s_cbranch_scc1 .Lcolumns_done_%=\n\t"
+        "s_cmp_eq_u32 %[single], 0\n\t"
+        "s_cbranch_scc0 .Lcolumns_single_%=\n\t"
+        "ds_read_b128 v[244:247], %[at] offset:%[first]\n\t"
+        "ds_read_b128 v[248:251], %[at] offset:%[second]\n\t"
+        "ds_read_b128 v[252:255], %[at] offset:%[third]\n\t"
+        "s_waitcnt lgkmcnt(2)\n\t"
+        "v_mul_f32 v244, %[a0], v244\n\t"
+        "v_mul_f32 v245, %[a0], v245\n\t"
+        "v_mul_f32 v246, %[a0], v246\n\t"
+        "v_mul_f32 v247, %[a0], v247\n\t"
+        "s_waitcnt lgkmcnt(1)\n\t"
+        "v_fmac_f32 v244, %[a1], v248\n\t"
+        "v_fmac_f32 v245, %[a1], v249\n\t"
+        "v_fmac_f32 v246, %[a1], v250\n\t"
+        "v_fmac_f32 v247, %[a1], v251\n\t"
+        "s_waitcnt lgkmcnt(0)\n\t"
+        "v_fmac_f32 v244, %[a2], v252\n\t"
+        "v_fmac_f32 v245, %[a2], v253\n\t"
+        "v_fmac_f32 v246, %[a2], v254\n\t"
+        "v_fmac_f32 v247, %[a2], v255\n\t"
+        "v_add_f32 %[h0], %[h0], v244\n\t"
+        "v_add_f32 %[h1], %[h1], v245\n\t"
+        "v_add_f32 %[h2], %[h2], v246\n\t"
+        "v_add_f32 %[h3], %[h3], v247\n\t"
+        "s_branch .Lcolumns_done_%=\n"
+        ".Lcolumns_single_%=:\n\t"
+        "ds_read_b128 v[244:247], %[at] offset:%[first]\n\t"
+        "s_waitcnt lgkmcnt(0)\n\t"
+        "v_fmac_f32 %[h0], %[a0], v244\n\t"
+        "v_fmac_f32 %[h1], %[a0], v245\n\t"
+        "v_fmac_f32 %[h2], %[a0], v246\n\t"
+        "v_fmac_f32 %[h3], %[a0], v247\n"
+        ".Lcolumns_done_%=:"
+        : [h0] "+v"(h0), [h1] "+v"(h1), [h2] "+v"(h2), [h3] "+v"(h3)
+        : [live] "s"(live), [single] "s"(single), [at] "v"(row_address), [a0] "v"(a0), [a1] "v"(a1), [a2] "v"(a2), [first] "n"(kFirst),
+          [second] "n"(kSecond), [third] "n"(kThird)
+        : "v244", "v245", "v246", "v247", "v248", "v249", "v250", "v251", "v252", "v253", "v254", "v255", "scc");
+}
+template <int N, int... Q>
+__device__ __forceinline__ void add_column_groups(std::integer_sequence<int, Q...>, uint64_t columns, uint32_t single, uint32_t row_address,
+                                                  float a0, float a1, float a2, float (&hrow)[N]) {
+    // the mask and the flag are uniform; the lane read says so where they come out of LDS
+    const uint32_t low = uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(columns))));
+    const uint32_t high = uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(columns >> 32u))));
+    const uint64_t uniform_columns = (uint64_t(high) << 32u) | uint64_t(low);
+    single = uint32_t(__builtin_amdgcn_readfirstlane(int(single)));
+    (add_columns_if<16 * Q, 16 * Q + 4 * N, 16 * Q + 8 * N>(uint32_t(uniform_columns >> (4 * Q)) & 0xFu, single, row_address, a0, a1, a2, hrow[4 * Q],
+                                                            hrow[4 * Q + 1], hrow[4 * Q + 2], hrow[4 * Q + 3]), ...);
+}
+
 // One head's part of the block: g += J^T f and H += J^T C J for lane's row, skipping the column blocks the head's
-// Jacobian rows leave at exact zero.  All head values are uniform.
+// Jacobian rows leave at exact zero.  All head values are uniform.  Widths that run two waves a SIMD update the row
+// through add_columns_if, wider ones through the plain loops.
 template <int N>
 __device__ __forceinline__ void add_head(const Tile& c, uint32_t h, bool coordinate, const float (&f)[3], const float (&cv)[6],
                                          const float (&noise)[3], uint32_t axes, uint64_t columns, float (&hrow)[N], TileSum& g,
@@ -515,6 +586,21 @@ __device__ __forceinline__ void add_head(const Tile& c, uint32_t h, bool coordin
     tile_add_product(g, j0, f[0]);
     scale += fabsf(j0) * noise[0];
     const float4* r0 = reinterpret_cast<const float4*>(j0r);
+    if constexpr (N <= kTwoWaveWidth) {
+        float a0 = j0 * cv[0], a1 = 0.0f, a2 = 0.0f;
+        if (axes != 1u) {
+            const float j1 = coordinate ? j0r[N + c.lane] : 0.0f, j2 = coordinate ? j0r[2 * N + c.lane] : 0.0f;
+            const float cxx = cv[0], cyy = cv[1], czz = cv[2], cxy = cv[3], cxz = cv[4], cyz = cv[5];
+            tile_add_product(g, j1, f[1]);
+            tile_add_product(g, j2, f[2]);
+            scale += fabsf(j1) * noise[1] + fabsf(j2) * noise[2];
+            a0 = (j0 * cxx + j1 * cxy) + j2 * cxz;
+            a1 = (j1 * cyy + j2 * cyz) + j0 * cxy;
+            a2 = (j2 * czz + j1 * cyz) + j0 * cxz;
+        }
+        add_column_groups<N>(std::make_integer_sequence<int, N / 4>{}, columns, axes == 1u ? 1u : 0u, lds_address(j0r), a0, a1, a2, hrow);
+        return;
+    }
     if (axes == 1u) {
         const float a0 = j0 * cv[0];
 #pragma unroll
