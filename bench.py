@@ -24,15 +24,15 @@ DOMINANT_OP = "BlockDescentSolve"
 DOMINANT_KERNEL = "BlockDescentTileKernel"
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, scaled
 # by the same counters' reading of a plain copy of known size); keyed by (config, envs).  None where not measured.
-MEASURED_TRAFFIC_BYTES = {(3, 4096): 81.0e6, (2, 4096): 29.8e6, (3, 65536): 1244.9e6, (5, 8192): 497.2e6}   # profiles/counters_*.txt
+MEASURED_TRAFFIC_BYTES = {(3, 4096): 80.9e6, (2, 4096): 29.7e6, (3, 65536): 1244.4e6, (5, 8192): 495.5e6}   # profiles/counters_*.txt
 # What the same counter runs say limits the dominant kernel (not measured by this script): vector instructions a
 # launch issues and the share of a wave's resident cycles spent issuing them, at two waves a SIMD (one for the rope).
 MEASURED_ISSUE = {
-    (3, 4096): {"limiter": "valu_issue", "valu_instructions_per_env": 174000, "wave_cycles_issuing_valu": 0.49, "waves_per_simd": 2,
+    (3, 4096): {"limiter": "valu_issue", "valu_instructions_per_env": 167000, "wave_cycles_issuing_valu": 0.47, "waves_per_simd": 2,
                 "scratch_bytes_per_lane": 0, "source": "profiles/counters_humanoid_4096.txt"},
-    (2, 4096): {"limiter": "valu_issue", "valu_instructions_per_env": 133000, "wave_cycles_issuing_valu": 0.50, "waves_per_simd": 2,
+    (2, 4096): {"limiter": "valu_issue", "valu_instructions_per_env": 128000, "wave_cycles_issuing_valu": 0.50, "waves_per_simd": 2,
                 "scratch_bytes_per_lane": 0, "source": "profiles/counters_quadruped_4096.txt"},
-    (3, 65536): {"limiter": "valu_issue", "valu_instructions_per_env": 174000, "wave_cycles_issuing_valu": 0.48, "waves_per_simd": 2,
+    (3, 65536): {"limiter": "valu_issue", "valu_instructions_per_env": 167000, "wave_cycles_issuing_valu": 0.47, "waves_per_simd": 2,
                  "scratch_bytes_per_lane": 0, "source": "profiles/counters_humanoid_65536.txt"},
     (5, 8192): {"limiter": "valu_issue", "valu_instructions_per_env": 287000, "wave_cycles_issuing_valu": 0.48, "waves_per_simd": 1,
                 "source": "profiles/counters_rope_8192.txt"},
