@@ -1,6 +1,6 @@
 """Features that other tests cover one at a time, here together and at widths the benchmark configurations do not reach:
 joint rows (unit heads) in the wide one-wave-per-SIMD kernels, the MuJoCo contact law with either cone at wide widths,
-MuJoCo-sourced joint rows with the integrator's damping pass, the split-impulse position pass past 36 coordinates.
+MuJoCo-sourced joint rows with the integrator's damping pass, the split-impulse position pass at narrow and wide widths.
 Every case steps the device world and the CPU oracle side by side from one seeded state."""
 import copy
 
@@ -25,6 +25,10 @@ CASES = [
     (48, True, False, dict(cone=abi.CONE_PYRAMIDAL)),
     (28, True, True, dict(cone=abi.CONE_ELLIPTIC, limits=True, friction=0.1, joint_law=True, integrator=abi.INTEGRATOR_MUJOCO_EULER, damping=0.4)),
     (56, True, True, dict(limits=True, friction=0.1, pos_iters=2)),
+    # the position pass at widths whose block assembly updates the Hessian row by the written-out column groups: its
+    # contact heads are single rows, with and without joint rows beside them
+    (20, True, True, dict(pos_iters=2)),
+    (32, False, True, dict(limits=True, friction=0.1, pos_iters=3)),
     (36, False, True, dict(cone=abi.CONE_PYRAMIDAL, drive=abi.DRIVE_VELOCITY, limits=True)),
 ]
 
