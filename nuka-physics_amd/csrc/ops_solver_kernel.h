@@ -12,7 +12,7 @@
 // the helpers it takes from block_descent.cu (:735-820, 1593-1621, 1726-1753) and nk/solve/augmented_row.hpp.
 // Blocks: one articulation per environment.  Rows on a single coordinate (joint limit, friction and drive rows) are
 // "unit" rows (:799-833): they stage no Jacobian row and touch one diagonal entry and one force entry.
-// Not built: free rigid 6x6 blocks, mimic couplings, elliptic (MuJoCo-law) cones.
+// Not built: free rigid 6x6 blocks, mimic couplings.
 #pragma once
 
 #include <utility>
@@ -50,36 +50,38 @@ constexpr uint32_t kUnitSlots = 6u;
 #define PROF_COUNT(c, i)
 #endif
 
-struct TileSum { float value, error; };   // block_descent_tile.cuh:15-31
-__device__ __forceinline__ void tile_add(TileSum& s, float x) {
-    const float sum = s.value + x;
-    const float part = sum - s.value;
-    s.error += (s.value - (sum - part)) + (x - part);
-    s.value = sum;
+// The reference sums its gradients, slopes and decrements as two-float compensated sums (TileSum, block_descent_tile.cuh
+// :15-46).  Here the same sums run in double: a product of two floats is exact in double, the vector unit executes a
+// double multiply-add at the rate of a float one, and one instruction replaces the nine of a compensated step.  The
+// rounded result is at least as close to the exact sum as the two-float one.
+struct TileSum { double value; };
+__device__ __forceinline__ void tile_add(TileSum& s, float x) { s.value += double(x); }
+__device__ __forceinline__ void tile_add_product(TileSum& s, float a, float b) { s.value = fma(double(a), double(b), s.value); }
+template <int Ctrl>
+__device__ __forceinline__ double dpp_move_d(double v) {
+    const uint64_t bits = uint64_t(__double_as_longlong(v));
+    const uint32_t low = uint32_t(__builtin_amdgcn_update_dpp(0, int(uint32_t(bits)), Ctrl, 0xF, 0xF, false));
+    const uint32_t high = uint32_t(__builtin_amdgcn_update_dpp(0, int(uint32_t(bits >> 32u)), Ctrl, 0xF, 0xF, false));
+    return __longlong_as_double((long long)((uint64_t(high) << 32u) | uint64_t(low)));
 }
-__device__ __forceinline__ void tile_add_product(TileSum& s, float a, float b) {
-    const float product = a * b;
-    s.error += fmaf(a, b, -product);
-    tile_add(s, product);
+__device__ __forceinline__ double row_value_d(double v, int row) {
+    const uint64_t bits = uint64_t(__double_as_longlong(v));
+    const uint32_t low = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(bits)), 16 * row));
+    const uint32_t high = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(bits >> 32u)), 16 * row));
+    return __longlong_as_double((long long)((uint64_t(high) << 32u) | uint64_t(low)));
 }
-// block_descent_tile.cuh:34-46 over 64 lanes: rows of 16 by DPP, then the four rows as scalars; uniform result
-__device__ __forceinline__ void tile_merge(TileSum& s, float value, float error) {
-    s.error += error;
-    tile_add(s, value);
+// every lane of a row of sixteen ends with the row's sum
+__device__ __forceinline__ double row_total_d(double v) {
+    v += dpp_move_d<kDppXor1>(v); v += dpp_move_d<kDppXor2>(v); v += dpp_move_d<kDppHalfMirror>(v); v += dpp_move_d<kDppMirror>(v);
+    return v;
 }
+// the sum over the wave: rows of 16 by DPP, then the four rows as scalars; uniform result
 __device__ __forceinline__ float wave_total(TileSum s, bool first_row_only = false) {
-    tile_merge(s, dpp_move<kDppXor1>(s.value), dpp_move<kDppXor1>(s.error));
-    tile_merge(s, dpp_move<kDppXor2>(s.value), dpp_move<kDppXor2>(s.error));
-    tile_merge(s, dpp_move<kDppHalfMirror>(s.value), dpp_move<kDppHalfMirror>(s.error));
-    tile_merge(s, dpp_move<kDppMirror>(s.value), dpp_move<kDppMirror>(s.error));
-    TileSum a{row_value(s.value, 0), row_value(s.error, 0)};
-    // lanes 16..63 hold exact zeros when only the first sixteen lanes carry terms: merging them changes nothing
-    if (first_row_only) return a.value + a.error;
-    TileSum b{row_value(s.value, 2), row_value(s.error, 2)};
-    tile_merge(a, row_value(s.value, 1), row_value(s.error, 1));
-    tile_merge(b, row_value(s.value, 3), row_value(s.error, 3));
-    tile_merge(a, b.value, b.error);
-    return a.value + a.error;
+    const double v = row_total_d(s.value);
+    const double a = row_value_d(v, 0);
+    // the copies of the first row's heads in lanes 16..63 are left out when only the first sixteen lanes carry terms
+    if (first_row_only) return float(a);
+    return float((a + row_value_d(v, 1)) + (row_value_d(v, 2) + row_value_d(v, 3)));
 }
 __device__ __forceinline__ float first_row_sum(float v) {
     v += dpp_move<kDppXor1>(v); v += dpp_move<kDppXor2>(v); v += dpp_move<kDppHalfMirror>(v); v += dpp_move<kDppMirror>(v);
@@ -303,6 +305,12 @@ __device__ __forceinline__ void head_response(const Tile& c, uint32_t h, float m
                     c.F(hNormalBound, h), c.F(hMu1, h), c.F(hMu2, h), &f[1], &f[2], &cv[1], &cv[2], &cv[5]);
 }
 
+// A pivot's reciprocal square root by the hardware approximation (an ulp or so): the pivot's place in the factor is
+// pivot * scale and its reciprocal is scale, two instructions on the chain every later pivot waits for where a
+// correctly rounded root and quotient take about fifteen.  The factor differs from the correctly rounded one by a
+// backward error of a few ulp in the matrix, which a Newton direction does not see.
+__device__ __forceinline__ float pivot_scale(float pivot) { return __builtin_amdgcn_rsqf(pivot); }
+
 // FactorTileBlock (:1622-1645) on register rows: lane i holds row i of the symmetric matrix; on return its entries
 // k <= i are row i of the Cholesky factor.  Element (i, j) loses L_ik L_jk for k = 0, 1, ... in that order, as the
 // reference's serial inner loop does; each product and subtraction is one fused multiply-add (the reference is
@@ -314,11 +322,11 @@ __device__ __forceinline__ bool factor_rows(uint32_t lane, float (&row)[N], floa
     float inverse = 0.0f;
 #pragma unroll
     for (int k = 0; k < N; ++k) {
-        // the pivot's square root and reciprocal: every pivot of a valid block lies in the normal range
+        // the pivot's square root and reciprocal
         const float pivot = lane_value(row[k], k);
         valid = valid && pivot > 0.0f && pivot <= FLT_MAX;
-        const float root = sqrt_rn_normal(valid ? pivot : 1.0f);
-        const float scale = div_by(1.0f, make_recip(root));
+        const float scale = pivot_scale(valid ? pivot : 1.0f);
+        const float root = pivot * scale;
         row[k] = lane == uint32_t(k) ? root : row[k] * scale;
         if (lane == uint32_t(k)) inverse = scale;
         // lane reads in batches of eight ahead of their multiply-adds: a scalar read has to settle for two cycles
@@ -356,8 +364,8 @@ __device__ __forceinline__ bool factor_rows_up(uint32_t lane, float (&row)[N], f
     for (int k = N - 1; k >= 0; --k) {
         const float pivot = lane_value(row[k], k);
         valid = valid && pivot > 0.0f && pivot <= FLT_MAX;
-        const float root = sqrt_rn_normal(valid ? pivot : 1.0f);
-        const float scale = div_by(1.0f, make_recip(root));
+        const float scale = pivot_scale(valid ? pivot : 1.0f);
+        const float root = pivot * scale;
         row[k] = lane == uint32_t(k) ? root : row[k] * scale;
         if (lane == uint32_t(k)) inverse = scale;
         const uint64_t reach = __ballot(lane < uint32_t(k) && row[k] != 0.0f);
@@ -772,11 +780,10 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
                                float* inertia, bool* converged) {
     const uint32_t lane = c.lane;
     const bool coordinate = lane < c.n;
-    const float difference = u - free_v;
-    const float part = difference - u;
-    const float difference_error = (u - (difference - part)) + (-free_v - part);
-    float* dvec = c.vec, *evec = c.vec + 64, *uvec = c.vec + 128;
-    dvec[lane] = difference; evec[lane] = difference_error; uvec[lane] = fabsf(u);
+    // the difference of two floats, exact in double (the reference carries it as a float and its rounding error)
+    double* dvec = reinterpret_cast<double*>(c.vec);
+    float* uvec = c.vec + 128;
+    dvec[lane] = double(u) - double(free_v); uvec[lane] = fabsf(u);
     PROF_BEGIN(c, 10);
     // lane's own head (the first 64 heads) from its constants, without a branch; a lane without an owned head gets zeros
     float mf[3], mc[6], mn[3];
@@ -817,24 +824,21 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
     PROF_BEGIN(c, 11);
     // Padded columns (k >= n) hold exact zeros in the mass row, the vectors and the Jacobian rows: their terms add
     // nothing to any of the sums below.
-    TileSum inertial{0.0f, 0.0f};
-    float scale = 0.0f;
-    const float4* d4 = reinterpret_cast<const float4*>(dvec);
-    const float4* e4 = reinterpret_cast<const float4*>(evec);
+    TileSum inertial{0.0};
+    double inertial_scale = 0.0;
+    const double2* d2 = reinterpret_cast<const double2*>(dvec);
 #pragma unroll
-    for (int q = 0; q < N / 4; ++q) {
-        const float4 dv = d4[q], ev = e4[q];
-        const float dk[4] = {dv.x, dv.y, dv.z, dv.w}, ek[4] = {ev.x, ev.y, ev.z, ev.w};
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const float mass = mrow[4 * q + t];
-            hrow[4 * q + t] = mass;
-            tile_add_product(inertial, mass, dk[t]);
-            tile_add_product(inertial, mass, ek[t]);
-            scale += fabsf(mass) * fabsf(dk[t]);
-        }
+    for (int q = 0; q < N / 2; ++q) {
+        const double2 dv = d2[q];
+        const double m0 = double(mrow[2 * q]), m1 = double(mrow[2 * q + 1]);
+        hrow[2 * q] = mrow[2 * q]; hrow[2 * q + 1] = mrow[2 * q + 1];
+        inertial.value = fma(m0, dv.x, inertial.value);
+        inertial.value = fma(m1, dv.y, inertial.value);
+        inertial_scale = fma(fabs(m0), fabs(dv.x), inertial_scale);
+        inertial_scale = fma(fabs(m1), fabs(dv.y), inertial_scale);
     }
-    TileSum g{-inertial.value, -inertial.error};
+    float scale = float(inertial_scale);
+    TileSum g{-inertial.value};
     PROF_END(c, 11);
     PROF_BEGIN(c, 12);
     if (!c.units) {   // staged heads only: plain head order
@@ -923,8 +927,8 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
     }
     PROF_END(c, 12);
     PROF_BEGIN(c, 13);
-    *force = coordinate ? g.value + g.error : 0.0f;
-    *inertia = coordinate ? inertial.value + inertial.error : 0.0f;
+    *force = coordinate ? float(g.value) : 0.0f;
+    *inertia = coordinate ? float(inertial.value) : 0.0f;
     bool finite = isfinite(*force);
     const float4* u4 = reinterpret_cast<const float4*>(uvec);
 #pragma unroll
@@ -1031,7 +1035,7 @@ __device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& 
                                  float inertial_slope, float inertial_curvature, float* slope, float* curvature, float* magnitude) {
     PROF_COUNT(c, 1);
     c.work += 1u;
-    TileSum row_slope{0.0f, 0.0f};
+    TileSum row_slope{0.0};
     float row_curvature = 0.0f, row_magnitude = 0.0f;
     if constexpr (kMode == kLineGeneral) {
         if (mine.owned) line_terms(mine, alpha, row_slope, row_curvature, row_magnitude);
@@ -1043,7 +1047,7 @@ __device__ __forceinline__ void line_derivatives(const Tile& c, const HeadLine& 
         plain_line_terms(plain, alpha, row_slope, row_curvature, row_magnitude);
     }
     PROF_BEGIN(c, 25);
-    TileSum total{-row_slope.value, -row_slope.error};
+    TileSum total{-row_slope.value};
     if (c.lane == 0u) {
         tile_add_product(total, alpha, inertial_curvature);
         tile_add(total, inertial_slope);
@@ -1072,25 +1076,22 @@ __device__ __forceinline__ void line_derivatives_pair(const Tile& c, const Plain
                                                       LinePoint* at_zero, LinePoint* at_one) {
     PROF_COUNT(c, 1);
     const float alpha = c.lane < 16u ? 0.0f : 1.0f;
-    TileSum row_slope{0.0f, 0.0f};
+    TileSum row_slope{0.0};
     float row_curvature = 0.0f, row_magnitude = 0.0f;
     plain_line_terms(plain, alpha, row_slope, row_curvature, row_magnitude);
-    TileSum total{-row_slope.value, -row_slope.error};
+    TileSum total{-row_slope.value};
     if ((c.lane & 15u) == 0u) {
         tile_add_product(total, alpha, inertial_curvature);
         tile_add(total, inertial_slope);
     }
-    tile_merge(total, dpp_move<kDppXor1>(total.value), dpp_move<kDppXor1>(total.error));
-    tile_merge(total, dpp_move<kDppXor2>(total.value), dpp_move<kDppXor2>(total.error));
-    tile_merge(total, dpp_move<kDppHalfMirror>(total.value), dpp_move<kDppHalfMirror>(total.error));
-    tile_merge(total, dpp_move<kDppMirror>(total.value), dpp_move<kDppMirror>(total.error));
+    const double slopes = row_total_d(total.value);
     float cv = row_curvature, mg = row_magnitude;
     cv += dpp_move<kDppXor1>(cv); cv += dpp_move<kDppXor2>(cv); cv += dpp_move<kDppHalfMirror>(cv); cv += dpp_move<kDppMirror>(cv);
     mg += dpp_move<kDppXor1>(mg); mg += dpp_move<kDppXor2>(mg); mg += dpp_move<kDppHalfMirror>(mg); mg += dpp_move<kDppMirror>(mg);
-    at_zero->slope = row_value(total.value, 0) + row_value(total.error, 0);
+    at_zero->slope = float(row_value_d(slopes, 0));
     at_zero->curvature = inertial_curvature + row_value(cv, 0);
     at_zero->magnitude = fabsf(inertial_slope) + 0.0f * inertial_curvature + row_value(mg, 0);
-    at_one->slope = row_value(total.value, 1) + row_value(total.error, 1);
+    at_one->slope = float(row_value_d(slopes, 1));
     at_one->curvature = inertial_curvature + row_value(cv, 1);
     at_one->magnitude = fabsf(inertial_slope) + 1.0f * inertial_curvature + row_value(mg, 1);
 }
@@ -1192,7 +1193,7 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], f
     if (c.iteration == 0u && has_free) {   // first-sweep segment search (:2165-2209)
         const float dd = coordinate ? free_v - u : 0.0f;
         const float mass_step = mass_times<N>(c, mrow, dd);
-        TileSum curvature{0.0f, 0.0f};
+        TileSum curvature{0.0};
         if (coordinate) tile_add_product(curvature, dd, mass_step);
         const float inertial_curvature = wave_total(curvature);
         if (inertial_curvature > 0.0f && isfinite(inertial_curvature)) {
@@ -1216,7 +1217,7 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], f
         PROF_BEGIN(c, 8);
         const float mass_step = mass_times<N>(c, mrow, dd);
         PROF_END(c, 8);
-        TileSum decrement{0, 0}, slope{0, 0}, curvature{0, 0};
+        TileSum decrement{0.0}, slope{0.0}, curvature{0.0};
         if (coordinate) {
             tile_add_product(decrement, force, dd);
             tile_add_product(slope, inertia, dd);

@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 
 from conftest import nk, relative_error
+from test_gpu_parity import one_ulp_sensitivity
 from test_oracle_pairs import box_on_slab, floating, floating_state, rail_state, rails
 
 pytestmark = pytest.mark.gpu
@@ -138,8 +139,13 @@ def test_every_analytic_pair_matches_the_oracle(oracle_py, device, ka, kb):
     oracle.op("block_descent_solve"); world.op("BlockDescentSolve")
     world.synchronize()
     assert np.array_equal(world.download("env_status")[same], oracle.download("env_status")[same])
-    for name in ("qdot", "lambda"):
-        assert relative_error(world.download(name).reshape(E, -1)[same], oracle.download(name).reshape(E, -1)[same]) <= TOL, name
+    # A manifold of several points on one rigid body splits its impulse over the points indeterminately to first
+    # order: the multipliers are held to what the oracle's own answer moves by when its inputs move by one ulp (where
+    # that is more than the tolerance), the velocities they produce to the tolerance itself.
+    sens = one_ulp_sensitivity(oracle_py, t, desc, state)
+    for name, bound in (("qdot", TOL), ("lambda", max(TOL, 4.0 * sens["lambda"]))):
+        error = relative_error(world.download(name).reshape(E, -1)[same], oracle.download(name).reshape(E, -1)[same])
+        assert error <= bound, (name, error, bound)
     world.close()
     oracle.close()
 

@@ -73,10 +73,24 @@ def test_humanoid_4096_contact_solution_properties(device):
     world.close()
 
 
-@pytest.mark.parametrize("index,E", [(2, 4096), (4, 16384)])
+@pytest.mark.parametrize("index,E", [(2, 4096), (4, 1024), (4, 16384), (4, 65536)])
 def test_full_size_batches_step_cleanly(device, index, E):
+    """Every environment count of the humanoid sweep (and the quadruped batch) steps twice without a status bit, with
+    finite state and unit quaternions; the first 64 environments of the batch equal a 64-environment world bit for
+    bit, whatever the batch size and the launch order the larger batch gives them."""
     cfg, world = stepped(device, index, E)
-    world.step(2)
+    _, small = stepped(device, index, 64)
+    world.step()
+    small.step()
+    world.synchronize()
+    small.synchronize()
+    nl, R = world.link_count, world.rows_per_env
+    for name, per in (("q", nl), ("qdot", nl), ("lambda", R), ("link_pose", nl * 7), ("candidate_pairs", None)):
+        big, few = world.download(name), small.download(name)
+        per = per if per is not None else few.size // 64
+        assert np.array_equal(big.reshape(E, per)[:64], few.reshape(64, per)), name
+    small.close()
+    world.step()
     world.synchronize()
     assert np.all(world.download("env_status") == 0)
     for name in ("q", "qdot", "link_pose", "lambda"):
@@ -84,6 +98,8 @@ def test_full_size_batches_step_cleanly(device, index, E):
     pose = world.download("link_pose").reshape(E, -1, 7)
     assert np.abs(np.linalg.norm(pose[:, :, 3:], axis=2) - 1).max() < 1e-5      # unit quaternions
     assert np.all(world.download("pair_count") <= world.info.contact_slots_per_env)
+    sweeps = world.download("vbd_velocity_sweep_count")
+    assert sweeps.min() >= 1 and sweeps.max() <= cfg.vel_iters
     world.close()
 
 
