@@ -450,6 +450,9 @@ nuka_result_t nuka_world_download_field(nuka_world_handle world, nuka_state_fiel
 /* Counts of the cooked world. */
 typedef struct nuka_world_info_t {
     uint32_t env_count, links_per_env, bodies_per_env, dof, max_dof, contact_slots_per_env, rows_per_env, op_count;
+    /* coordinates the sweeps of the contact solve work on: dof, or fewer where no contact of the world can reach the
+     * later coordinates and the solve eliminates those once per step */
+    uint32_t solver_width;
 } nuka_world_info_t;
 nuka_result_t nuka_world_get_info(nuka_world_handle world, nuka_world_info_t* out);
 

@@ -19,5 +19,7 @@ void InitArticulationKernels();
 void InitSolverKernels();
 void InitContactKernels();
 uint32_t SolverHeadCapacity(const ModelView& m, uint32_t slots, size_t lds_budget_bytes);
+// the width the sweeps of the world's block-descent solve run at: its coordinates, or fewer for a reduced block
+uint32_t SolverSweepWidth(const ModelView& m);
 
 }  // namespace nkh

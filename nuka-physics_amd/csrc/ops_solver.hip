@@ -12,6 +12,13 @@ NKH_DECLARE_WIDTH(4) NKH_DECLARE_WIDTH(8) NKH_DECLARE_WIDTH(12) NKH_DECLARE_WIDT
 NKH_DECLARE_WIDTH(28) NKH_DECLARE_WIDTH(32) NKH_DECLARE_WIDTH(36) NKH_DECLARE_WIDTH(40) NKH_DECLARE_WIDTH(44) NKH_DECLARE_WIDTH(48)
 NKH_DECLARE_WIDTH(52) NKH_DECLARE_WIDTH(56) NKH_DECLARE_WIDTH(60) NKH_DECLARE_WIDTH(64)
 #undef NKH_DECLARE_WIDTH
+// reduced blocks (contact heads only): width N with the sweeps K wide
+#define NKH_DECLARE_REDUCED(N, K) \
+    extern template __global__ void BlockDescentTileKernel<N, true, K>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+NKH_DECLARE_REDUCED(24, 12) NKH_DECLARE_REDUCED(28, 16) NKH_DECLARE_REDUCED(32, 16) NKH_DECLARE_REDUCED(36, 20) NKH_DECLARE_REDUCED(40, 20)
+NKH_DECLARE_REDUCED(44, 24) NKH_DECLARE_REDUCED(48, 24) NKH_DECLARE_REDUCED(52, 28) NKH_DECLARE_REDUCED(56, 28) NKH_DECLARE_REDUCED(60, 32)
+NKH_DECLARE_REDUCED(64, 32)
+#undef NKH_DECLARE_REDUCED
 }  // namespace solver
 
 
@@ -82,6 +89,14 @@ using SolverKernel = void (*)(ModelView, DataView, BlockDescentSolveParams, uint
     BlockDescentTileKernel<52, V>, BlockDescentTileKernel<56, V>, BlockDescentTileKernel<60, V>, BlockDescentTileKernel<64, V>
 const SolverKernel kSolverKernels[2][16] = {{NKH_WIDTHS(false)}, {NKH_WIDTHS(true)}};
 #undef NKH_WIDTHS
+// One reduced instantiation per padded width from 24 on: the sweeps run at about half the width.  A world takes it
+// when no contact can reach a coordinate from that width on (ModelView::contact_dof_end).
+struct ReducedKernel { uint32_t width, reduced; SolverKernel kernel; };
+const ReducedKernel kReducedKernels[] = {
+    {24u, 12u, BlockDescentTileKernel<24, true, 12>}, {28u, 16u, BlockDescentTileKernel<28, true, 16>}, {32u, 16u, BlockDescentTileKernel<32, true, 16>},
+    {36u, 20u, BlockDescentTileKernel<36, true, 20>}, {40u, 20u, BlockDescentTileKernel<40, true, 20>}, {44u, 24u, BlockDescentTileKernel<44, true, 24>},
+    {48u, 24u, BlockDescentTileKernel<48, true, 24>}, {52u, 28u, BlockDescentTileKernel<52, true, 28>}, {56u, 28u, BlockDescentTileKernel<56, true, 28>},
+    {60u, 32u, BlockDescentTileKernel<60, true, 32>}, {64u, 32u, BlockDescentTileKernel<64, true, 32>}};
 }  // namespace
 
 void InitSolverKernels() {
@@ -91,6 +106,30 @@ void InitSolverKernels() {
             (void)hipGetLastError();
         }
     }
+    for (const ReducedKernel& reduced : kReducedKernels) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(reduced.kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipGetLastError();
+    }
+}
+
+// The width the sweeps of a world's solve run at: its coordinates, or the K of a reduced block where no contact of the
+// world reaches the coordinates from K on and a kernel is compiled for that.
+static uint32_t SolverWorkingWidth(const ModelView& m, bool contacts_only) {
+    if (contacts_only)
+        for (const ReducedKernel& reduced : kReducedKernels)
+            if (reduced.width == solver::PaddedWidth(m.dof) && m.contact_dof_end <= reduced.reduced && reduced.reduced <= m.dof) return reduced.reduced;
+    return m.dof;
+}
+// worlds whose heads are contact heads only, at most one a lane (the elliptic cone of the MuJoCo law is answered by the
+// general kernel only)
+static bool ContactHeadsOnly(const ModelView& m, uint32_t staged) {
+    const uint32_t joint_heads = m.joint_limit_rows + m.joint_friction_rows + m.joint_drive_rows;
+    return joint_heads == 0u && staged <= uint32_t(solver::kWave) && !(m.any_mujoco != 0u && m.contact_cone == 1u);
+}
+uint32_t SolverSweepWidth(const ModelView& m) {
+    if (m.rows_per_env == 0u || m.dof == 0u) return m.dof;
+    const uint32_t staged = SolverHeadCapacity(m, std::max(m.contact_slots, 1u), 150u * 1024u);
+    return SolverWorkingWidth(m, staged != 0u && ContactHeadsOnly(m, staged));
 }
 
 Status OpBlockDescentSolve(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
@@ -103,18 +142,23 @@ Status OpBlockDescentSolve(const ModelView& m, const DataView& d, const void* pa
     const uint32_t staged = SolverHeadCapacity(m, p->contact_slots_per_env == 0u ? 1u : p->contact_slots_per_env, budget);
     if (staged == 0u) return Status::InvalidArgument;
     const uint32_t joint_heads = m.joint_limit_rows + m.joint_friction_rows + m.joint_drive_rows;
-    const auto lds_bytes = [&](uint32_t contact_heads) { return size_t{solver::SolverLdsFloats(m.dof, contact_heads + joint_heads, contact_heads)} * sizeof(float); };
+    const bool contacts_only = ContactHeadsOnly(m, staged);
+    const uint32_t width = SolverWorkingWidth(m, contacts_only);
+    const auto lds_bytes = [&](uint32_t contact_heads) {
+        return size_t{solver::ReducedSolverLdsFloats(m.dof, width, contact_heads + joint_heads, contact_heads)} * sizeof(float);
+    };
     // widths past kTwoWaveWidth run one wave a SIMD: four blocks a compute unit at most, whatever their LDS
-    const size_t most_blocks = solver::PaddedWidth(m.dof) > uint32_t(solver::kTwoWaveWidth) ? 4u : 8u;
+    const size_t most_blocks = solver::PaddedWidth(width) > uint32_t(solver::kTwoWaveWidth) ? 4u : 8u;
     const auto blocks_per_unit = [&](uint32_t contact_heads) { return std::min<size_t>(most_blocks, (160u * 1024u) / lds_bytes(contact_heads)); };
     // The LDS a block needs grows with the contact heads it can stage, and a scene's slots (every pair that may ever
     // touch, at its largest manifold) outnumber the contacts an environment usually has.  Where a smaller capacity
     // lets more blocks share a compute unit, environments with few contact points go to a launch of that capacity:
     // up to three such launches, for eight, four and two blocks a unit, before the full one.  Each launch takes the
     // environments whose contact points fall in its range; an environment's results do not depend on its launch.
-    // (the elliptic cone of the MuJoCo law is answered by the general kernel only)
-    const bool contacts_only = joint_heads == 0u && staged <= uint32_t(solver::kWave) && !(m.any_mujoco != 0u && m.contact_cone == 1u);
-    const SolverKernel kernel = kSolverKernels[contacts_only ? 1 : 0][solver::PaddedWidth(m.dof) / 4u - 1u];
+    SolverKernel kernel = kSolverKernels[contacts_only ? 1 : 0][solver::PaddedWidth(m.dof) / 4u - 1u];
+    if (width != m.dof)
+        for (const ReducedKernel& reduced : kReducedKernels)
+            if (reduced.width == solver::PaddedWidth(m.dof) && reduced.reduced == width) kernel = reduced.kernel;
     hipLaunchKernelGGL(OrderTilesKernel, dim3(1), dim3(1024), 0, stream, d, p->env_count);
     uint32_t first_points = 0u;
     // (a launch takes its environments by their contact points, one head a point: not under the pyramidal cone, whose

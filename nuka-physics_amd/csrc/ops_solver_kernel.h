@@ -70,6 +70,12 @@ __device__ __forceinline__ double row_value_d(double v, int row) {
     const uint32_t high = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(bits >> 32u)), 16 * row));
     return __longlong_as_double((long long)((uint64_t(high) << 32u) | uint64_t(low)));
 }
+__device__ __forceinline__ double lane_value_d(double v, int lane) {   // `lane` a compile-time constant at every call site
+    const uint64_t bits = uint64_t(__double_as_longlong(v));
+    const uint32_t low = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(bits)), lane));
+    const uint32_t high = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(bits >> 32u)), lane));
+    return __longlong_as_double((long long)((uint64_t(high) << 32u) | uint64_t(low)));
+}
 // every lane of a row of sixteen ends with the row's sum
 __device__ __forceinline__ double row_total_d(double v) {
     v += dpp_move_d<kDppXor1>(v); v += dpp_move_d<kDppXor2>(v); v += dpp_move_d<kDppHalfMirror>(v); v += dpp_move_d<kDppMirror>(v);
@@ -253,6 +259,7 @@ constexpr uint32_t kWideStride = kWideFields | 1u, kNarrowStride = kNarrowFields
 
 struct Tile {
     uint32_t env, lane, n, ld, ldj, heads, cap, narrow, iteration;
+    uint32_t n_all;   // n, or past it the coordinates that follow the block's own (a reduced block, described above mass_times)
     float tolerance;
     float* mfac;     // N x ld: Cholesky factor of the mass matrix (rows; columns are read transposed)
     float* hfac;     // N x ld: Cholesky factor of the current Newton Hessian
@@ -355,13 +362,15 @@ constexpr bool kLeavesFirst = N > 32;
 // FactorTileColumns on register rows: lane i holds row i of the symmetric matrix; on return its entries k >= i are
 // row i of U.  Column k leaves exact zeros in the rows of other branches of the tree, and the update of a column by
 // an exact zero changes nothing: such columns are skipped four at a time.
-template <int N>
+// With kStop > 0 the elimination ends after pivot kStop: rows and columns below it then hold the Schur complement of the
+// eliminated coordinates, rows below it hold their coupling to them in the columns from kStop on.
+template <int N, int kStop = 0>
 __device__ __forceinline__ bool factor_rows_up(uint32_t lane, float (&row)[N], float* inverse_out) {
     lane = local_lane(lane);
     bool valid = true;
     float inverse = 0.0f;
 #pragma unroll
-    for (int k = N - 1; k >= 0; --k) {
+    for (int k = N - 1; k >= kStop; --k) {
         const float pivot = lane_value(row[k], k);
         valid = valid && pivot > 0.0f && pivot <= FLT_MAX;
         const float scale = pivot_scale(valid ? pivot : 1.0f);
@@ -775,9 +784,12 @@ __device__ __forceinline__ float uniform_lane_value(float v, uint32_t lane) {   
 // AssembleTileBlock (:1507-1618): lane i assembles row i of H = M + sum J^T C J in `hrow` and its force g_i.  The
 // first 64 heads evaluate their response one per lane and hand it to the row lanes as scalar lane reads; heads beyond
 // 64 pass theirs through the head fields.
-template <int N>
-__device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow)[N], float u, float free_v, float (&hrow)[N], float* force,
-                               float* inertia, bool* converged) {
+// In a reduced block (kFollow) the mass row is the sum of two floats, `mrow` and `mlow`: the Schur complement as it comes
+// out of the double-precision elimination.  The force takes both parts, so that the velocity the block converges to
+// balances the momentum against the mass matrix itself; the Hessian takes the first.
+template <int N, bool kFollow>
+__device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow)[N], const float (&mlow)[N], float u, float free_v, float (&hrow)[N],
+                               float* force, float* inertia, bool* converged) {
     const uint32_t lane = c.lane;
     const bool coordinate = lane < c.n;
     // the difference of two floats, exact in double (the reference carries it as a float and its rounding error)
@@ -834,6 +846,10 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
         hrow[2 * q] = mrow[2 * q]; hrow[2 * q + 1] = mrow[2 * q + 1];
         inertial.value = fma(m0, dv.x, inertial.value);
         inertial.value = fma(m1, dv.y, inertial.value);
+        if constexpr (kFollow) {
+            inertial.value = fma(double(mlow[2 * q]), dv.x, inertial.value);
+            inertial.value = fma(double(mlow[2 * q + 1]), dv.y, inertial.value);
+        }
         inertial_scale = fma(fabs(m0), fabs(dv.x), inertial_scale);
         inertial_scale = fma(fabs(m1), fabs(dv.y), inertial_scale);
     }
@@ -951,17 +967,45 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
 
 enum Failure : uint32_t { kFailNone = 0u, kFailEquation, kFailFactor, kFailDirection, kFailCandidate };
 
+// A reduced block.  Where no contact of the world reaches the coordinates from K on (the arms of a humanoid that
+// stands on its feet), those coordinates enter the block's objective through the mass matrix alone and the minimiser
+// over them is linear in the others: u_U = free_U - P (u_T - free_T), P = M_UU^-1 M_UT.  Eliminating them once per
+// solve leaves the same problem on the K coordinates T with the Schur complement M_TT - M_TU M_UU^-1 M_UT as its mass
+// matrix: every Newton block, factorisation and substitution of the solve is K wide instead of N.  The lanes K..n-1
+// ("followers") hold a row of -P where the block's lanes hold a mass row, so that the product every Newton step
+// takes with the mass rows (mass_times) hands each follower its own move, and the tests the reference makes over all
+// coordinates (step below rounding, largest step, mass-normalised residual) still see all of them.  The minimiser of
+// each block is the one the full-width block has; the iterates on the way differ by rounding.
+// mass_step_i = sum_k M_ik d_k in coordinate order (:2177-2187, 2228-2238).  In a reduced block the lanes past the
+// block's coordinates hold a row of -P instead of a mass row, and get their own move -P d from the same products.
+template <int N>
+__device__ __forceinline__ float mass_times(const Tile& c, const float (&mrow)[N], float d) {
+    float* dvec = c.vec + 192;
+    dvec[c.lane] = d;
+    __syncthreads();
+    float out = 0.0f;
+    const float4* d4 = reinterpret_cast<const float4*>(dvec);
+#pragma unroll
+    for (int q = 0; q < N / 4; ++q) {
+        const float4 dv = d4[q];
+        out += mrow[4 * q] * dv.x; out += mrow[4 * q + 1] * dv.y; out += mrow[4 * q + 2] * dv.z; out += mrow[4 * q + 3] * dv.w;
+    }
+    __syncthreads();
+    return c.lane < c.n_all ? out : 0.0f;
+}
+
+
 // TileNewtonDirection (:1935-1992).  The reference re-assembles the block after the mass-normalised
 // convergence test because its mass factor overwrites the Hessian storage; here the two live apart and the
 // assembled row, force and inertia (which the second assembly would reproduce bit for bit) are simply kept.
-template <int N>
-__device__ __forceinline__ Failure newton_direction(const Tile& c, const float (&mrow)[N], float u, float free_v, float* force, float* inertia,
-                                    float* d, bool* converged) {
+template <int N, bool kFollow>
+__device__ __forceinline__ Failure newton_direction(const Tile& c, const float (&mrow)[N], const float (&mlow)[N], float u, float free_v, float* force,
+                                    float* inertia, float* d, bool* converged) {
     PROF_COUNT(c, 0);
     c.work += 16u;
     float hrow[N];
     PROF_BEGIN(c, 1);
-    const bool assembled = assemble_block<N>(c, mrow, u, free_v, hrow, force, inertia, converged);
+    const bool assembled = assemble_block<N, kFollow>(c, mrow, mlow, u, free_v, hrow, force, inertia, converged);
     PROF_END(c, 1);
     if (!assembled) return kFailEquation;
     if (*converged && c.tolerance > 0.0f) {
@@ -970,7 +1014,12 @@ __device__ __forceinline__ Failure newton_direction(const Tile& c, const float (
         const float direction = solve_tile_mass<N>(c, *force);
         PROF_END(c, 3);
         *d = direction;
-        *converged = __all(c.lane >= c.n || fabsf(direction) < c.tolerance);
+        bool small = c.lane >= c.n || fabsf(direction) < c.tolerance;
+        if constexpr (kFollow) {
+            const float follow = mass_times<N>(c, mrow, c.lane < c.n ? direction : 0.0f);
+            if (c.lane >= c.n && c.lane < c.n_all) small = fabsf(follow) < c.tolerance;
+        }
+        *converged = __all(small);
         if (*converged) return kFailNone;
     }
     if (*converged) return kFailNone;
@@ -1159,40 +1208,31 @@ __device__ __forceinline__ void apply_moves(const Tile& c, float alpha) {
     __syncthreads();
 }
 
-// mass_step_i = sum_k M_ik d_k in coordinate order (:2177-2187, 2228-2238)
-template <int N>
-__device__ __forceinline__ float mass_times(const Tile& c, const float (&mrow)[N], float d) {
-    float* dvec = c.vec + 192;
-    dvec[c.lane] = d;
-    __syncthreads();
-    float out = 0.0f;
-    const float4* d4 = reinterpret_cast<const float4*>(dvec);
-#pragma unroll
-    for (int q = 0; q < N / 4; ++q) {
-        const float4 dv = d4[q];
-        out += mrow[4 * q] * dv.x; out += mrow[4 * q + 1] * dv.y; out += mrow[4 * q + 2] * dv.z; out += mrow[4 * q + 3] * dv.w;
-    }
-    __syncthreads();
-    return c.lane < c.n ? out : 0.0f;
-}
-
 // DescendTileBlock (:2145-2301).  `u` is lane i's block coordinate; `has_free` is false in the position pass.
-template <int N>
-__device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], float* u_io, float free_in, bool has_free, DataView d) {
+template <int N, bool kFollow>
+__device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], const float (&mlow)[N], float* u_io, float free_in, bool has_free,
+                                              DataView d) {
     const uint32_t lane = c.lane, n = c.n;
     const bool coordinate = lane < n;
+    const bool follower = kFollow && lane >= n && lane < c.n_all;
+    const bool moving = coordinate || follower;
     for (uint32_t h = lane; h < c.heads; h += kWave) {   // StartTileBlock (:1386-1397)
         if (c.U(hOwned, h) == 0u) continue;
         c.F(hNormalBound, h) = c.F(hDual, h);
         c.F(hMove, h) = 0.0f; c.F(hMove + 1, h) = 0.0f; c.F(hMove + 2, h) = 0.0f;
     }
     __syncthreads();
-    const float start = coordinate ? *u_io : 0.0f;
-    const float free_v = coordinate && has_free ? free_in : 0.0f;
+    float start = coordinate ? *u_io : 0.0f;
+    const float free_v = moving && has_free ? free_in : 0.0f;
+    if constexpr (kFollow) {   // the followers start where the block's coordinates put them
+        const float follow = mass_times<N>(c, mrow, coordinate ? start - free_v : 0.0f);
+        if (follower) start = free_v + follow;
+    }
     float u = start;
     if (c.iteration == 0u && has_free) {   // first-sweep segment search (:2165-2209)
-        const float dd = coordinate ? free_v - u : 0.0f;
+        float dd = coordinate ? free_v - u : 0.0f;
         const float mass_step = mass_times<N>(c, mrow, dd);
+        if (follower) dd = mass_step;
         TileSum curvature{0.0};
         if (coordinate) tile_add_product(curvature, dd, mass_step);
         const float inertial_curvature = wave_total(curvature);
@@ -1210,12 +1250,13 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], f
     for (uint32_t step = 0u; step < kNewtonSteps; ++step) {
         float force = 0.0f, inertia = 0.0f, dd = 0.0f;
         bool converged = false;
-        failure = newton_direction<N>(c, mrow, u, free_v, &force, &inertia, &dd, &converged);
+        failure = newton_direction<N, kFollow>(c, mrow, mlow, u, free_v, &force, &inertia, &dd, &converged);
         if (converged) primal = 0.0f;
         if (failure != kFailNone || converged) break;
         if (!coordinate) dd = 0.0f;
         PROF_BEGIN(c, 8);
         const float mass_step = mass_times<N>(c, mrow, dd);
+        if (follower) dd = mass_step;
         PROF_END(c, 8);
         TileSum decrement{0.0}, slope{0.0}, curvature{0.0};
         if (coordinate) {
@@ -1235,10 +1276,10 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], f
         const float alpha = search_line(c, inertial_slope, inertial_curvature);
         PROF_END(c, 5);
         const float after = fmaf(alpha, dd, u);
-        const bool rounded = __all(!coordinate || after == u);
-        if (!__all(!coordinate || isfinite(after))) { failure = kFailCandidate; break; }
+        const bool rounded = __all(!moving || after == u);
+        if (!__all(!moving || isfinite(after))) { failure = kFailCandidate; break; }
         primal = 0.0f;
-        if (coordinate && !rounded) primal = fmaxf(primal, fabsf(alpha * dd));
+        if (moving && !rounded) primal = fmaxf(primal, fabsf(alpha * dd));
         if (!(alpha > 0.0f)) break;
         u = after;
         apply_moves(c, alpha);
@@ -1255,19 +1296,20 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], f
         if (lane == 0u) d.env_status[c.env] |= kEnvStatusSolverFailure;
     }
     float moved = failure == kFailNone ? 0.0f : FLT_MAX;
-    if (coordinate) moved = fmaxf(moved, __uint_as_float(residual_bits(u - start)));
+    if (moving) moved = fmaxf(moved, __uint_as_float(residual_bits(u - start)));
     c.momentum = fmaxf(c.momentum, wave_max(moved));
     if (failure != kFailNone) primal = FLT_MAX;
     c.residual = fmaxf(c.residual, wave_max(primal));   // one block per environment: no coupled heads
-    if (coordinate) *u_io = u;
+    if (moving) *u_io = u;
 }
 
 // MeasureTilePrimal (:2378-2489): the mass-normalised momentum balance in double
-template <int N>
-__device__ __forceinline__ void measure_primal(Tile& c, const float (&mrow)[N], float* velocity_io, float free_v, const float* lambda_env, uint32_t R,
-                               bool reconstruct, DataView d) {
+template <int N, bool kFollow>
+__device__ __forceinline__ void measure_primal(Tile& c, const float (&mrow)[N], const float (&mlow)[N], float* velocity_io, float free_v,
+                               const float* lambda_env, uint32_t R, bool reconstruct, DataView d) {
     const uint32_t lane = c.lane, n = c.n;
     const bool coordinate = lane < n;
+    const bool follower = kFollow && lane >= n && lane < c.n_all;
     float* dvec = c.vec;
     dvec[lane] = coordinate ? *velocity_io : 0.0f;
     c.vec[64 + lane] = coordinate ? free_v : 0.0f;
@@ -1279,6 +1321,7 @@ __device__ __forceinline__ void measure_primal(Tile& c, const float (&mrow)[N], 
         // ahead of the sweeps, and holds two registers an entry from there on
         const float mass = opaque(mrow[j]);
         balance -= double(mass) * (double(dvec[j]) - c.vec[64 + j]);   // padded terms are exact zeros
+        if constexpr (kFollow) balance -= double(opaque(mlow[j])) * (double(dvec[j]) - c.vec[64 + j]);
     }
     // heads with an impulse add J^T lambda in head order (:2402-2436).  A unit head touches one coordinate: that
     // lane takes it from its own list when it comes up between the staged heads
@@ -1327,12 +1370,17 @@ __device__ __forceinline__ void measure_primal(Tile& c, const float (&mrow)[N], 
     }
     float residual = failure == kFailNone ? 0.0f : FLT_MAX;
     if (failure != kFailNone && lane == 0u) d.env_status[c.env] |= kEnvStatusSolverFailure;
-    if (failure == kFailNone && coordinate) residual = fmaxf(residual, isfinite(direction) ? fabsf(direction) : FLT_MAX);
+    if constexpr (kFollow) {   // the followers' part of M^-1 (balance, 0) is -P times the block's part
+        const float follow = failure == kFailNone ? mass_times<N>(c, mrow, coordinate ? direction : 0.0f) : 0.0f;
+        if (follower) direction = follow;
+    }
+    const bool moving = coordinate || follower;
+    if (failure == kFailNone && moving) residual = fmaxf(residual, isfinite(direction) ? fabsf(direction) : FLT_MAX);
     residual = wave_max(residual);
     c.residual = fmaxf(c.residual, residual);
     if (reconstruct && failure == kFailNone) {
-        if (!__all(!coordinate || isfinite(*velocity_io + direction))) { c.residual = FLT_MAX; return; }
-        if (coordinate) *velocity_io += direction;
+        if (!__all(!moving || isfinite(*velocity_io + direction))) { c.residual = FLT_MAX; return; }
+        if (moving) *velocity_io += direction;
         c.momentum = fmaxf(c.momentum, residual);
     }
 }
@@ -1519,9 +1567,16 @@ __device__ __forceinline__ void update_duals(const Tile& c, float* lambda_env, u
 }
 
 __host__ __device__ inline uint32_t PaddedWidth(uint32_t n) { return (n + 3u) & ~3u; }
+// `n`: the width the solve works at - the block's coordinates, or the K of a reduced block
 __host__ __device__ inline uint32_t FactorRegionFloats(uint32_t n) {
     const uint32_t N = PaddedWidth(n);
     return 2u * N * (N + 1u);   // a multiple of 4 since N is
+}
+// what the set-up of a reduced block passes through LDS ahead of everything else: the eliminated coordinates' factor
+// and their coupling to the others, transposed
+__host__ __device__ inline uint32_t ReductionScratchFloats(uint32_t full, uint32_t reduced) {
+    const uint32_t N = PaddedWidth(full);
+    return reduced >= full ? 0u : 2u * (N - reduced) * N;   // doubles
 }
 __host__ __device__ inline uint32_t HeadFieldFloats(uint32_t cap, uint32_t narrow) {
     return (kWideStride * cap + kNarrowStride * (narrow + 1u) + 3u) & ~3u;
@@ -1533,14 +1588,115 @@ __host__ __device__ inline uint32_t SolverLdsFloats(uint32_t n, uint32_t cap, ui
     // the block keeps the footprint that lets eight of them share a compute unit's LDS
     return FactorRegionFloats(n) + 3u * staged * N + HeadFieldFloats(cap, staged) + 256u + (cap > staged ? kUnitSlots * uint32_t(kWave) : 0u);
 }
+__host__ __device__ inline uint32_t ReducedSolverLdsFloats(uint32_t full, uint32_t reduced, uint32_t cap, uint32_t staged) {
+    const uint32_t solve = SolverLdsFloats(reduced, cap, staged), scratch = ReductionScratchFloats(full, reduced);
+    return solve > scratch ? solve : scratch;
+}
 
 // DescendTile (:2941-3087).  kContactsOnly is the instantiation for worlds without joint rows whose heads fit one a
 // lane (cap <= 64, every head a staged contact head): the unit-head paths and the loops over heads beyond the first
 // 64 are compiled out, which leaves the hot loop shorter and with fewer values to keep live.
-template <int N, bool kContactsOnly>
-__global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(N <= kTwoWaveWidth ? 2 : 1, N <= kTwoWaveWidth ? 2 : 1)))
+// The set-up of a reduced block, in double.  Lane i < n comes with row i of the mass matrix at `mass` (md words a row).
+// The coordinates N-1 .. K are eliminated leaves first (FactorTileColumns' order): the lanes below K are left with
+// their rows of the Schur complement S = M_TT - M_TU M_UU^-1 M_UT and of U_TU = M_TU U_UU^-T, the followers with their
+// rows of the factor M_UU = U_UU U_UU^T.  P = M_UU^-1 M_UT = U_UU^-T U_TU^T then follows by forward substitution over the
+// followers in ascending order, its two operands passing through LDS to be read transposed.  On return a lane below K
+// holds its row of S as the sum mrow + mlow of two floats, a follower its row of -P rounded to float in mrow.
+// Double because these rows stand in for the mass matrix over the whole solve: a Schur complement eliminated in
+// single precision moves the velocities the solve converges to by a few 1e-5 of the contact impulse's effect.
+template <int N, int K>
+__device__ __forceinline__ bool reduce_block(uint32_t lane, uint32_t n, const float* mass, uint32_t md, float* lds, float (&mrow)[K], float (&mlow)[K]) {
+    constexpr int kFollowers = N - K;
+    const bool row_lane = lane < n;
+    double full[N];
+    {
+        float fetched[N];
+        if (md % 4u == 0u && md >= uint32_t(N)) {
+#pragma unroll
+            for (int q = 0; q < N / 4; ++q) {
+                const float4 m4 = reinterpret_cast<const float4*>(mass)[q];
+                fetched[4 * q] = m4.x; fetched[4 * q + 1] = m4.y; fetched[4 * q + 2] = m4.z; fetched[4 * q + 3] = m4.w;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < N; ++k) fetched[k] = uint32_t(k) < n ? mass[k] : 0.0f;
+        }
+#pragma unroll
+        for (int k = 0; k < N; ++k)   // rows and columns n..N-1 are those of the identity
+            full[k] = row_lane && uint32_t(k) < n ? double(fetched[k]) : (lane == uint32_t(k) && lane < uint32_t(N) ? 1.0 : 0.0);
+    }
+    const uint32_t at = local_lane(lane);
+    bool valid = true;
+    double own_scale = 0.0;
+#pragma unroll
+    for (int k = N - 1; k >= K; --k) {
+        const double pivot = lane_value_d(full[k], k);
+        valid = valid && pivot > 0.0 && pivot <= double(FLT_MAX);
+        // the reciprocal root: the single-precision approximation and two Newton steps
+        const double safe = valid ? pivot : 1.0;
+        double scale = double(__builtin_amdgcn_rsqf(float(safe)));
+        scale = scale * fma(-0.5 * safe, scale * scale, 1.5);
+        scale = scale * fma(-0.5 * safe, scale * scale, 1.5);
+        full[k] = at == uint32_t(k) ? safe * scale : full[k] * scale;
+        if (at == uint32_t(k)) own_scale = scale;
+        const uint64_t reach = __ballot(at < uint32_t(k) && full[k] != 0.0);
+#pragma unroll
+        for (int q = (k - 1) / 4; q >= 0; --q) {
+            if (((reach >> (4 * q)) & 0xFull) == 0ull) continue;
+            double u[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) u[t] = 4 * q + t <= k - 1 ? lane_value_d(full[k], 4 * q + t) : 0.0;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                if (4 * q + t <= k - 1) full[4 * q + t] = fma(-full[k], u[t], full[4 * q + t]);
+        }
+    }
+    double* coupling = reinterpret_cast<double*>(lds);   // [follower][coordinate below K]: U_TU transposed
+    double* corner = coupling + kFollowers * K;           // [follower i][follower k]: U_UU[i][k], zero below the diagonal
+    if (lane < uint32_t(K)) {
+#pragma unroll
+        for (int k = K; k < N; ++k) coupling[(k - K) * K + int(lane)] = full[k];
+    } else if (lane < uint32_t(N)) {
+#pragma unroll
+        for (int k = K; k < N; ++k) corner[(int(lane) - K) * kFollowers + (k - K)] = uint32_t(k) >= lane ? full[k] : 0.0;
+    }
+    __syncthreads();
+    const uint32_t slot = lane >= uint32_t(K) && lane < uint32_t(N) ? lane - uint32_t(K) : 0u;
+    double prow[K], column[kFollowers];
+#pragma unroll
+    for (int q = 0; q < K / 2; ++q) {
+        const double2 v = reinterpret_cast<const double2*>(coupling + slot * uint32_t(K))[q];
+        prow[2 * q] = v.x; prow[2 * q + 1] = v.y;
+    }
+#pragma unroll
+    for (int i = 0; i < kFollowers; ++i) column[i] = corner[i * kFollowers + int(slot)];
+#pragma unroll
+    for (int i = K; i < N; ++i) {
+#pragma unroll
+        for (int c0 = 0; c0 < K; ++c0) {
+            const double y = lane_value_d(prow[c0] * own_scale, i);
+            prow[c0] = at > uint32_t(i) ? fma(-column[i - K], y, prow[c0]) : prow[c0];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const double entry = lane < uint32_t(K) ? full[k] : (lane < n ? -(prow[k] * own_scale) : 0.0);
+        mrow[k] = float(entry);
+        mlow[k] = lane < uint32_t(K) ? float(entry - double(mrow[k])) : 0.0f;
+    }
+    __syncthreads();
+    return valid;
+}
+
+// K < N is a reduced block (described above mass_times): no contact of the world reaches the coordinates K..n-1, which are
+// eliminated once in the set-up, and the sweeps run K wide.  K is a multiple of 4 with K <= n, contact heads only.
+template <int N, bool kContactsOnly, int K = N>
+__global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(K <= kTwoWaveWidth ? 2 : 1, K <= kTwoWaveWidth ? 2 : 1)))
 BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint32_t cap, uint32_t staged_cap, uint32_t points_lo,
                        uint32_t points_hi) {
+    constexpr bool kReduced = K < N;
+    constexpr int W = K;   // the width of the sweeps
+    static_assert(K % 4 == 0 && K <= N && (!kReduced || kContactsOnly), "a reduced block holds contact heads only");
     extern __shared__ __align__(16) float lds[];
     const uint32_t env = d.tile_order[blockIdx.x], lane = threadIdx.x;
     // A world whose contact slots outnumber the contacts it usually has is solved by two launches of different LDS
@@ -1551,7 +1707,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     }
     const uint32_t R = p.rows_per_env, md = p.max_dof, n = m.dof, nl = m.links_per_env, S = p.contact_slots_per_env;
     Tile c;
-    c.env = env; c.lane = lane; c.n = n; c.ld = uint32_t(N) + 1u; c.ldj = uint32_t(N); c.cap = cap; c.narrow = staged_cap; c.heads = 0u; c.iteration = 0u;
+    c.env = env; c.lane = lane; c.n = kReduced ? uint32_t(K) : n; c.n_all = n; c.ld = uint32_t(W) + 1u; c.ldj = uint32_t(W); c.cap = cap; c.narrow = staged_cap; c.heads = 0u; c.iteration = 0u;
     c.tolerance = p.velocity_tolerance; c.failed = false; c.momentum = 0.0f; c.residual = 0.0f;
     c.mass_inverse = 0.0f; c.mass_valid = false; c.work = 0u; c.units = false; c.elliptic = false;
     c.factor_current = false;
@@ -1563,10 +1719,20 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     PROF_BEGIN(c, 9);
     PROF_BEGIN(c, 0);
     c.mfac = lds;
-    c.hfac = c.mfac + uint32_t(N) * c.ld;
-    c.jac = lds + FactorRegionFloats(n);
+    c.hfac = c.mfac + uint32_t(W) * c.ld;
+    c.jac = lds + FactorRegionFloats(uint32_t(W));
     c.fields = c.jac + 3u * staged_cap * c.ldj;
     c.vec = c.fields + HeadFieldFloats(cap, staged_cap);
+    // The block's mass rows: lane's row of M, or in a reduced block lane's row of the Schur complement (lanes below K)
+    // and of -P (the followers).
+    float mrow[W], mlow[W];
+    bool reduction_valid = true;
+    if constexpr (kReduced) {
+        reduction_valid = reduce_block<N, K>(lane, n, d.m + size_t{env} * md * md + size_t{lane < n ? lane : 0u} * md, md, lds, mrow, mlow);
+    } else {
+#pragma unroll
+        for (int k = 0; k < W; ++k) mlow[k] = 0.0f;   // never read
+    }
     if (lane < kNarrowFields) c.fields[kWideStride * cap + staged_cap * kNarrowStride + lane] = 0.0f;   // what a narrow field reads beyond its heads
     c.unit_list = reinterpret_cast<uint32_t*>(c.vec + 256);
     c.unit_lists = true; c.unit_count = 0u; c.staged_end = 0u; c.individual_end = 0u;
@@ -1702,6 +1868,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     __syncthreads();
     // CopyTileRows (:836-869): the staged heads' rows, their loads in flight together
 
+    bool stray = false;   // a reduced block: an entry past the block's coordinates
     for (uint32_t h0 = 0u; h0 < c.staged_end; h0 += 4u) {   // four heads at a time: 24 reads in flight
         uint32_t first[4];
         float value[4][3];
@@ -1728,10 +1895,16 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
                 if (staged && lane < c.ldj) c.jac[(first[t] + axis) * c.ldj + lane] = value[t][axis];   // padded columns hold zeros
             // the columns this head touches at all: a contact on one limb leaves most coordinates out, and the Hessian
             // update skips their exact-zero products four columns at a time
-            const uint64_t columns = __ballot(value[t][0] != 0.0f || value[t][1] != 0.0f || value[t][2] != 0.0f);
+            uint64_t columns = __ballot(value[t][0] != 0.0f || value[t][1] != 0.0f || value[t][2] != 0.0f);
+            if constexpr (kReduced) {
+                stray = stray || (columns >> uint32_t(W)) != 0ull;
+                columns &= (uint64_t{1} << uint32_t(W)) - 1ull;
+            }
             if (lane == 0u) { c.U(hColumnsLow, h) = uint32_t(columns); c.U(hColumnsHigh, h) = uint32_t(columns >> 32u); }
         }
     }
+    // a contact that reaches a coordinate the world's reduction left out: the launch was given the wrong width
+    if (stray && lane == 0u) d.env_status[env] |= kEnvStatusSolverFailure;
     __syncthreads();
     PROF_END(c, 17);
     PROF_BEGIN(c, 18);
@@ -1739,7 +1912,6 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     // (ForwardMass + MassDot, articulation_mass.cuh:414-431).  lane = DoF: the unit-lower factor row sits in
     // registers with zeros from the diagonal on, each y_j travels as a scalar lane read, so row i subtracts
     // L_ij y_j for j = 0, 1, ... exactly as the serial loop does; the ordered sum of y_i^2 / D_i follows the same way.
-    float mrow[N];
     {
         // Lane's own rows of the mass matrix and of its LDL^T factor (StageTileMass :2127-2142) straight into registers:
         // one row is md contiguous words, so every read of both rows is in flight at once, as 16-byte words where the
@@ -1747,27 +1919,42 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         const size_t tile = size_t{env} * md * md + size_t{coordinate ? lane : 0u} * md;
         const float* factor = d.m_factor + tile;
         const float* mass = d.m + tile;
-        float lrow[N], fetched[N];
-        if (md % 4u == 0u && md >= uint32_t(N)) {
+        float lrow[N];
+        if constexpr (kReduced) {   // the mass rows were taken, and reduced, at the start
+            if (md % 4u == 0u && md >= uint32_t(N)) {
 #pragma unroll
-            for (int q = 0; q < N / 4; ++q) {
-                const float4 f4 = reinterpret_cast<const float4*>(factor)[q], m4 = reinterpret_cast<const float4*>(mass)[q];
-                lrow[4 * q] = f4.x; lrow[4 * q + 1] = f4.y; lrow[4 * q + 2] = f4.z; lrow[4 * q + 3] = f4.w;
-                fetched[4 * q] = m4.x; fetched[4 * q + 1] = m4.y; fetched[4 * q + 2] = m4.z; fetched[4 * q + 3] = m4.w;
+                for (int q = 0; q < N / 4; ++q) {
+                    const float4 f4 = reinterpret_cast<const float4*>(factor)[q];
+                    lrow[4 * q] = f4.x; lrow[4 * q + 1] = f4.y; lrow[4 * q + 2] = f4.z; lrow[4 * q + 3] = f4.w;
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < N; ++k) lrow[k] = uint32_t(k) < n ? factor[k] : 0.0f;
             }
         } else {
+            float fetched[N];
+            if (md % 4u == 0u && md >= uint32_t(N)) {
 #pragma unroll
-            for (int k = 0; k < N; ++k) {
-                lrow[k] = uint32_t(k) < n ? factor[k] : 0.0f;
-                fetched[k] = uint32_t(k) < n ? mass[k] : 0.0f;
+                for (int q = 0; q < N / 4; ++q) {
+                    const float4 f4 = reinterpret_cast<const float4*>(factor)[q], m4 = reinterpret_cast<const float4*>(mass)[q];
+                    lrow[4 * q] = f4.x; lrow[4 * q + 1] = f4.y; lrow[4 * q + 2] = f4.z; lrow[4 * q + 3] = f4.w;
+                    fetched[4 * q] = m4.x; fetched[4 * q + 1] = m4.y; fetched[4 * q + 2] = m4.z; fetched[4 * q + 3] = m4.w;
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < N; ++k) {
+                    lrow[k] = uint32_t(k) < n ? factor[k] : 0.0f;
+                    fetched[k] = uint32_t(k) < n ? mass[k] : 0.0f;
+                }
             }
+#pragma unroll
+            for (int k = 0; k < W; ++k)   // rows and columns n..N-1 of the mass matrix are those of the identity
+                mrow[k] = coordinate && uint32_t(k) < n ? fetched[k] : (lane == uint32_t(k) && lane < uint32_t(N) ? 1.0f : 0.0f);
         }
         float pivot = 1.0f;
 #pragma unroll
         for (int k = 0; k < N; ++k) {
             if (coordinate && lane == uint32_t(k)) pivot = lrow[k];
-            // rows and columns n..N-1 of the mass matrix are those of the identity
-            mrow[k] = coordinate && uint32_t(k) < n ? fetched[k] : (lane == uint32_t(k) && lane < uint32_t(N) ? 1.0f : 0.0f);
             lrow[k] = coordinate && uint32_t(k) < lane ? lrow[k] : 0.0f;
         }
         // y = L^-1 a, then the ordered sum of y_i^2 / D_i
@@ -1803,7 +1990,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
                 const float unit_value = c.F(hUnitValue, h);
                 skip[t] = share_units && unit != kInvalid && fabsf(unit_value) == 1.0f && !apart[t];
                 if (coordinate && (artic_a || artic_b) && !apart[t] && !skip[t])
-                    a[t] = first != kInvalid ? c.jac[first * c.ldj + lane] : (lane == unit ? unit_value : 0.0f);
+                    a[t] = first != kInvalid ? (lane < c.ldj ? c.jac[first * c.ldj + lane] : 0.0f) : (lane == unit ? unit_value : 0.0f);
             }
             if (skip[0] && skip[1] && skip[2] && skip[3]) continue;
 #pragma unroll
@@ -1928,10 +2115,10 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     PROF_END(c, 19);
     PROF_BEGIN(c, 20);
     // the one factorisation of the mass matrix
-    c.mass_valid = factor_mass<N>(c, mrow);
+    c.mass_valid = factor_mass<W>(c, mrow) && reduction_valid;
     PROF_END(c, 20);
     PROF_BEGIN(c, 21);
-    initialize_residuals<N>(c, velocity, urows, p.dt);
+    initialize_residuals<W>(c, velocity, urows, p.dt);
     PROF_END(c, 21);
     PROF_END(c, 0);
     float residual4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -1942,22 +2129,22 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         c.iteration = sweeps++;
         c.momentum = 0.0f; c.residual = 0.0f;
         PROF_COUNT(c, 2);
-        descend_block<N>(c, mrow, &velocity, free_v, true, d);
+        descend_block<W, kReduced>(c, mrow, mlow, &velocity, free_v, true, d);
         float rowsr[3];
         PROF_BEGIN(c, 6);
         update_duals(c, lambda_env, R, urows, &momentum, true, true, rowsr);
         PROF_END(c, 6);
         PROF_BEGIN(c, 7);
         if (sweeps == p.iterations || fmaxf(fmaxf(rowsr[0], rowsr[1]), fmaxf(rowsr[2], c.residual)) < tol)
-            measure_primal<N>(c, mrow, &velocity, free_v, lambda_env, R, false, d);
+            measure_primal<W, kReduced>(c, mrow, mlow, &velocity, free_v, lambda_env, R, false, d);
         PROF_END(c, 7);
         if (fmaxf(fmaxf(rowsr[0], rowsr[1]), rowsr[2]) < tol && c.residual >= tol && c.residual < FLT_MAX) {
-            measure_primal<N>(c, mrow, &velocity, free_v, lambda_env, R, true, d);
+            measure_primal<W, kReduced>(c, mrow, mlow, &velocity, free_v, lambda_env, R, true, d);
             if (c.residual < FLT_MAX) {
-                initialize_residuals<N>(c, velocity, urows, p.dt);
+                initialize_residuals<W>(c, velocity, urows, p.dt);
                 update_duals(c, lambda_env, R, urows, nullptr, true, false, rowsr);
                 c.residual = 0.0f;
-                measure_primal<N>(c, mrow, &velocity, free_v, lambda_env, R, false, d);
+                measure_primal<W, kReduced>(c, mrow, mlow, &velocity, free_v, lambda_env, R, false, d);
             }
         }
         residual4[0] = rowsr[0]; residual4[1] = rowsr[1]; residual4[2] = rowsr[2]; residual4[3] = c.residual;
@@ -2075,7 +2262,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
             const uint32_t positions = 1u;   // no head couples two moving blocks here, so one solve (:2716)
             for (uint32_t iteration = 0u; iteration < positions; ++iteration) {
                 c.iteration = sweeps + iteration;
-                descend_block<N>(c, mrow, &pseudo, 0.0f, false, d);
+                descend_block<W, kReduced>(c, mrow, mlow, &pseudo, 0.0f, false, d);
             }
         }
         // FinishTilePositions (:2720-2744)

@@ -326,6 +326,13 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
     c.contact_impratio = d.contact_impratio > 0.0f ? d.contact_impratio : 1.0f;
     c.floating_root = m.joint_type[0] == kFloatingBase ? 1u : 0u;
     c.max_points_per_slot = max_points;
+    // the coordinates a contact can act on: those on the way to the root from a link that carries a shape that can pair
+    c.contact_dof_end = 0u;
+    for (uint32_t b = 0u; b < nb; ++b) {
+        if (d.body_role[b] == 0u || d.shape_kind[b] == kInvalid || d.body_link[b] >= nl) continue;
+        const uint64_t mask = m.link_dof_mask[d.body_link[b]];
+        for (uint32_t k = 0u; k < nv; ++k) if ((mask >> k) & 1ull) c.contact_dof_end = std::max(c.contact_dof_end, k + 1u);
+    }
     c.excluded_pair_count = uint32_t(m.excluded_pairs.size());
     // rows whose type and affinity masks are both empty pass the filter with no partner (shape_kind.hpp:26-33): the pair
     // query walks the grid of the other rows only, in the same ascending order
@@ -1405,7 +1412,8 @@ nuka_result_t nuka_world_get_info(nuka_world_handle world, nuka_world_info_t* ou
     if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
     if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
     const ModelView& m = w->model;
-    *out = {w->env_count, m.links_per_env, m.bodies_per_env, m.dof, m.max_dof, m.contact_slots, m.rows_per_env, uint32_t(w->calls.size())};
+    *out = {w->env_count, m.links_per_env, m.bodies_per_env, m.dof, m.max_dof, m.contact_slots, m.rows_per_env, uint32_t(w->calls.size()),
+            SolverSweepWidth(m)};
     return NUKA_RESULT_OK;
 }
 

@@ -15,9 +15,11 @@ class Tree:
         self.link_count = template.link_count
 
 
-def make_tree(dof, floating, branched, seed, mu=0.7, root_height=0.0, limb_joints=7):
+def make_tree(dof, floating, branched, seed, mu=0.7, root_height=0.0, limb_joints=7, sphere_limbs=None):
     """A tree with `dof` coordinates: a floating or fixed root and revolute joints, laid out as one serial chain or as
-    limbs of at most `limb_joints` (seven) joints fanning out of the root.  Every limb's last two links carry a contact sphere."""
+    limbs of at most `limb_joints` (seven) joints fanning out of the root.  Every limb's last two links carry a contact
+    sphere, or only those of the first `sphere_limbs` limbs: the later limbs then carry no shape, like the arms of a
+    robot that stands on its feet."""
     g = np.random.default_rng(seed)
     t = abi.Template()
     if floating:
@@ -26,7 +28,7 @@ def make_tree(dof, floating, branched, seed, mu=0.7, root_height=0.0, limb_joint
         t.add_link(abi.JOINT_FIXED, None, local_pos=(0, 0, root_height), mass=1.0)
     joints = dof - (6 if floating else 0)
     limb = limb_joints if branched else joints
-    sphere_links, made = [], 0
+    sphere_links, made, limbs = [], 0, 0
     while made < joints:
         count = min(limb, joints - made)
         parent = 0
@@ -40,9 +42,10 @@ def make_tree(dof, floating, branched, seed, mu=0.7, root_height=0.0, limb_joint
             parent = t.add_link(abi.JOINT_REVOLUTE, parent, axis=AXES[(made + k) % 3], local_pos=tuple(offset), mass=mass,
                                 diag_inertia=tuple(mass * g.uniform(0.004, 0.02, 3)), com=tuple(0.5 * length * direction),
                                 armature=0.02)
-            if k >= count - 2:
+            if k >= count - 2 and (sphere_limbs is None or limbs < sphere_limbs):
                 sphere_links.append((parent, tuple(length * direction), SPHERE_RADIUS))
         made += count
+        limbs += 1
     profile = t.add_profile(mu)
     t.add_body(abi.ROLE_STATIC, kind=abi.SHAPE_PLANE, contype=2, conaffinity=1, profile=profile)
     for link in range(t.link_count):
@@ -66,12 +69,12 @@ def sphere_heights(oracle_py, tree, desc, state):
     return z
 
 
-def tree_case(oracle_py, dof, floating, branched, seed, E, dt=1.0 / 240.0, vel_iters=8, limb_joints=7):
+def tree_case(oracle_py, dof, floating, branched, seed, E, dt=1.0 / 240.0, vel_iters=8, limb_joints=7, sphere_limbs=None):
     """(tree, desc, state): seeded joint angles, rates and torques; the root is placed so that each environment's
     lowest sphere presses a few millimetres into the plane (floating root), or so that half of the environments touch
     it (fixed root: the anchor height belongs to the template)."""
     g = np.random.default_rng(seed + 1000)
-    tree = make_tree(dof, floating, branched, seed, limb_joints=limb_joints)
+    tree = make_tree(dof, floating, branched, seed, limb_joints=limb_joints, sphere_limbs=sphere_limbs)
     nl = tree.link_count
     desc = abi.world_desc(E, dt, vel_iters=vel_iters, contact_margin=0.1)   # spheres a hand above the plane get speculative rows
     q = g.normal(0.0, 0.3, (E, nl)).astype(np.float32)
@@ -89,5 +92,6 @@ def tree_case(oracle_py, dof, floating, branched, seed, E, dt=1.0 / 240.0, vel_i
     if floating:
         base[:, 2] = (SPHERE_RADIUS - lowest - g.uniform(0.0, 0.004, E)).astype(np.float32)
     else:
-        tree = make_tree(dof, floating, branched, seed, root_height=float(SPHERE_RADIUS - np.median(lowest)), limb_joints=limb_joints)
+        tree = make_tree(dof, floating, branched, seed, root_height=float(SPHERE_RADIUS - np.median(lowest)), limb_joints=limb_joints,
+                         sphere_limbs=sphere_limbs)
     return tree, desc, state
