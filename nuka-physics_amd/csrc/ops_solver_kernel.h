@@ -651,9 +651,75 @@ __device__ __forceinline__ void add_head(const Tile& c, uint32_t h, bool coordin
     }
 }
 
+// v[lane & 31] + v[32 + (lane & 31)] in every lane: the two halves of the wavefront swapped against each other
+__device__ __forceinline__ float halves_sum(float v) {
+    const auto pair = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(pair[0]) + __uint_as_float(pair[1]);
+}
+__device__ __forceinline__ double halves_sum(double v) {
+    const uint64_t bits = uint64_t(__double_as_longlong(v));
+    const auto low = __builtin_amdgcn_permlane32_swap(uint32_t(bits), uint32_t(bits), false, false);
+    const auto high = __builtin_amdgcn_permlane32_swap(uint32_t(bits >> 32u), uint32_t(bits >> 32u), false, false);
+    return __longlong_as_double((long long)((uint64_t(high[0]) << 32u) | uint64_t(low[0]))) +
+           __longlong_as_double((long long)((uint64_t(high[1]) << 32u) | uint64_t(low[1])));
+}
+
+// Two heads in one pass, for blocks of at most 32 coordinates: lanes 0..31 add head `ha` to their rows, lanes 32..63
+// add head `hb` (kInvalid: none) to rows of their own that start at zero, row = lane & 31 in both halves; the caller
+// sums the halves afterwards (halves_sum).  A head's values come from its own lane (lane = head) through the lane
+// permute, its Jacobian words from the head's own rows in LDS; a column group is taken when either head reaches it
+// (the other then adds exact zeros).  The sums add in another order than head after head: the last place may differ.
+template <int N>
+__device__ __forceinline__ void add_head_pair(const Tile& c, uint32_t ha, uint32_t hb, const float (&mf)[3], const float (&mc)[6], const float (&mn)[3],
+                                              uint32_t my_first, uint32_t my_low, uint32_t my_high, float (&hrow)[N], TileSum& g, float& scale) {
+    static_assert(N <= 32, "both halves of the wavefront hold every row");
+    const uint32_t row = c.lane & 31u;
+    const bool none = c.lane >= 32u && hb == kInvalid;
+    const int source = int(c.lane >= 32u ? (hb == kInvalid ? ha : hb) : ha);
+    float f[3], cv[6], noise[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { f[k] = __shfl(mf[k], source, kWave); noise[k] = __shfl(mn[k], source, kWave); }
+#pragma unroll
+    for (int k = 0; k < 6; ++k) cv[k] = __shfl(mc[k], source, kWave);
+    const uint32_t first = uint32_t(__shfl(int(my_first), source, kWave));
+    const float* j0r = c.jac + first * uint32_t(N);
+    const bool live = !none && row < c.n;
+    const float j0 = live ? j0r[row] : 0.0f, j1 = live ? j0r[N + row] : 0.0f, j2 = live ? j0r[2 * N + row] : 0.0f;
+    tile_add_product(g, j0, f[0]);
+    tile_add_product(g, j1, f[1]);
+    tile_add_product(g, j2, f[2]);
+    scale += (fabsf(j0) * noise[0] + fabsf(j1) * noise[1]) + fabsf(j2) * noise[2];
+    const float cxx = cv[0], cyy = cv[1], czz = cv[2], cxy = cv[3], cxz = cv[4], cyz = cv[5];
+    const float a0 = (j0 * cxx + j1 * cxy) + j2 * cxz;
+    const float a1 = (j1 * cyy + j2 * cyz) + j0 * cxy;
+    const float a2 = (j2 * czz + j1 * cyz) + j0 * cxz;
+    uint64_t columns = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_high), int(ha)))) << 32u) |
+                       uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_low), int(ha))));
+    if (hb != kInvalid)
+        columns |= (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_high), int(hb)))) << 32u) |
+                   uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_low), int(hb))));
+    if constexpr (N <= kTwoWaveWidth) {
+        add_column_groups<N>(std::make_integer_sequence<int, N / 4>{}, columns, 0u, lds_address(j0r), a0, a1, a2, hrow);
+    } else {
+        const float4* r0 = reinterpret_cast<const float4*>(j0r);
+        const float4* r1 = reinterpret_cast<const float4*>(j0r + N);
+        const float4* r2 = reinterpret_cast<const float4*>(j0r + 2 * N);
+#pragma unroll
+        for (int q = 0; q < N / 4; ++q) {
+            if (((columns >> (4 * q)) & 0xFull) == 0ull) continue;
+            const float4 x0 = r0[q], x1 = r1[q], x2 = r2[q];
+            hrow[4 * q] += fmaf(a2, x2.x, fmaf(a1, x1.x, a0 * x0.x));
+            hrow[4 * q + 1] += fmaf(a2, x2.y, fmaf(a1, x1.y, a0 * x0.y));
+            hrow[4 * q + 2] += fmaf(a2, x2.z, fmaf(a1, x1.z, a0 * x0.z));
+            hrow[4 * q + 3] += fmaf(a2, x2.w, fmaf(a1, x1.w, a0 * x0.w));
+        }
+    }
+}
+
 // One head's line-search inputs in registers: nothing in them changes between the probes of one search, and neither
 // do the parts of its response that do not depend on the probe (plain_line).
 struct HeadLine {
+    uint32_t head;
     bool owned, contact, bounded, cone, elliptic;
     float tangent_compliance[2], mu_first;
     float rho, compliance, lower, upper, bound;
@@ -665,6 +731,7 @@ struct HeadLine {
 };
 __device__ __forceinline__ HeadLine load_head_line(const Tile& c, uint32_t h) {
     HeadLine l{};
+    l.head = h;
     l.owned = h < c.heads && c.U(hOwned, h) != 0u;
     if (!l.owned) return l;
     l.contact = block_axes(c.U(hAxes, h));
@@ -720,15 +787,21 @@ __device__ __forceinline__ void line_terms(const HeadLine& l, float alpha, TileS
 // cone argument, a cone of radius zero gives no tangent impulse and no curvature) is made here once, by handing the
 // probe constants on which the general formulas give those results exactly - zeros for what must come out as zero.
 // A lane without an owned head gets zeros throughout and adds exact zeros to every sum.
+// The cone argument dual / mu + rho mu residual (ConeArgument, augmented_row.hpp:302-318) is kept by the reference as
+// compensated float pairs; here the same two constants are doubles (the sums of the reference's pairs) and the
+// argument is one double multiply-add.  Everything but `move` and `step` is constant over a block descent.
 struct PlainLine {
     float k, k_bounded, dual_part, lower, upper;
     float res[3], move[3], step[3];
-    ConeAxis y, z;
+    double cone_y, cone_z, gain_y, gain_z;
     float mu_y, mu_z, radius, rho_radius, radius_y, radius_z, inside_yy, inside_zz;
+    uint32_t head;   // the head the constants belong to, kInvalid for none: `move` and `step` are then never read
 };
 __device__ __forceinline__ PlainLine plain_line(const HeadLine& l) {
     PlainLine p{};
+    p.head = kInvalid;
     if (!l.owned || l.rho <= 0.0f) return p;   // no penalty: no impulse and no curvature (scalar_impulse, tangent_impulse)
+    p.head = l.head;
     p.k = l.response.residual_scale; p.k_bounded = l.bounded ? p.k : 0.0f; p.dual_part = l.dual_part; p.lower = l.lower; p.upper = l.upper;
 #pragma unroll
     for (int k = 0; k < 3; ++k) { p.res[k] = l.res[k]; p.move[k] = l.move[k]; p.step[k] = l.step[k]; }
@@ -736,32 +809,56 @@ __device__ __forceinline__ PlainLine plain_line(const HeadLine& l) {
     if (!(l.rho == l.rho && l.dual[0] == l.dual[0] && l.compliance == l.compliance && l.lower == l.lower && l.upper == l.upper)) p.dual_part = nanf("");
     if (!l.contact) return p;
     p.mu_y = l.ratios.mu_y; p.mu_z = l.ratios.mu_z;
-    if (p.mu_y != 0.0f) p.y = l.y;
-    if (p.mu_z != 0.0f) p.z = l.z;
+    if (p.mu_y != 0.0f) { p.cone_y = double(l.y.dd) + double(l.y.d_low); p.gain_y = double(l.y.p) + double(l.y.p_low); }
+    if (p.mu_z != 0.0f) { p.cone_z = double(l.z.dd) + double(l.z.d_low); p.gain_z = double(l.z.p) + double(l.z.p_low); }
     p.radius = l.radius; p.rho_radius = l.rho_radius; p.radius_y = l.radius_y; p.radius_z = l.radius_z;
     if (l.cone) { p.inside_yy = l.inside_yy; p.inside_zz = l.inside_zz; }
     return p;
 }
 // The response of a head from its constants: scalar_impulse and tangent_impulse operation for operation, both sides
-// of the cone computed and one selected, the three quotients by the tangent norm sharing one reciprocal.  A residual
+// of the cone computed and one selected, the three quotients by the tangent norm sharing one reciprocal (the answers
+// differ from the general functions' in the last place or two).  A residual
 // that is not a number comes out as an impulse that is not a number, as in the general functions.  plain_line_terms
 // is TileLineDerivatives (:2048-2086) on it, with at most one head a lane.
 __device__ __forceinline__ void plain_response(const PlainLine& p, float mx, float my, float mz, float (&f)[3], float (&r)[6]) {
     const float x = fmaf(p.k, p.res[0] - mx, p.dual_part);
     f[0] = x < p.lower ? p.lower : (x > p.upper ? p.upper : x);
     r[0] = x >= p.lower && x <= p.upper ? p.k_bounded : 0.0f;
-    const float q_y = cone_value(p.y, p.res[1] - my);
-    const float q_z = cone_value(p.z, p.res[2] - mz);
-    const float norm = hypotf(q_y, q_z);
+    const float q_y = float(fma(p.gain_y, double(p.res[1] - my), p.cone_y));
+    const float q_z = float(fma(p.gain_z, double(p.res[2] - mz), p.cone_z));
+    // the norm and its reciprocal by the hardware root and reciprocal (an ulp each): impulses lie far inside the range
+    // where the squares neither overflow nor vanish
+    const float norm = __builtin_amdgcn_sqrtf(fmaf(q_y, q_y, q_z * q_z));
     const bool inside = norm <= p.radius;
-    const Recip by_norm = make_recip(inside ? 1.0f : norm);
-    const float dy = div_by(q_y, by_norm), dz = div_by(q_z, by_norm), cs = div_by(p.rho_radius, by_norm);
+    const float by_norm = __builtin_amdgcn_rcpf(inside ? 1.0f : norm);
+    const float dy = q_y * by_norm, dz = q_z * by_norm, cs = p.rho_radius * by_norm;
     f[1] = inside ? p.mu_y * q_y : p.radius_y * dy;
     f[2] = inside ? p.mu_z * q_z : p.radius_z * dz;
     r[1] = inside ? p.inside_yy : cs * p.mu_y * p.mu_y * dz * dz;
     r[2] = inside ? p.inside_zz : cs * p.mu_z * p.mu_z * dy * dy;
     r[3] = 0.0f; r[4] = 0.0f;
     r[5] = inside ? 0.0f : -cs * p.mu_y * p.mu_z * dy * dz;
+}
+// The constants of lane's own head for one block descent.  With at most sixteen heads the four rows of sixteen lanes
+// hold copies of the heads (lane & 15), which the line search uses to evaluate several points of a line in one pass;
+// the block assembly then takes the copies of the first row only.  `move` and `step` change with every Newton step
+// and are read again where they are used.
+// Widths whose register rows leave room keep the constants in registers over the whole block descent; the others
+// (28 to 36, at two waves a SIMD) compute them again at each use, which costs less than the spills would.
+template <int N>
+constexpr bool kKeepLine = N <= 24 || N > kTwoWaveWidth;
+__device__ __forceinline__ PlainLine own_line(const Tile& c) {
+    return plain_line(load_head_line(c, c.heads <= 16u ? (c.lane & 15u) : c.lane));
+}
+__device__ __forceinline__ void refresh_moves(const Tile& c, PlainLine& p) {
+    if (p.head == kInvalid) return;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) p.move[k] = c.F(hMove + k, p.head);
+}
+__device__ __forceinline__ void refresh_steps(const Tile& c, PlainLine& p) {
+    if (p.head == kInvalid) return;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { p.move[k] = c.F(hMove + k, p.head); p.step[k] = c.F(hStep + k, p.head); }
 }
 // A head's response at its current move with the rounding noise of each axis; false when nothing of it is non-zero.
 __device__ __forceinline__ bool head_terms(const Tile& c, uint32_t h, float (&f)[3], float (&cv)[6], float (&noise)[3]) {
@@ -788,8 +885,8 @@ __device__ __forceinline__ float uniform_lane_value(float v, uint32_t lane) {   
 // out of the double-precision elimination.  The force takes both parts, so that the velocity the block converges to
 // balances the momentum against the mass matrix itself; the Hessian takes the first.
 template <int N, bool kFollow>
-__device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow)[N], const float (&mlow)[N], float u, float free_v, float (&hrow)[N],
-                               float* force, float* inertia, bool* converged) {
+__device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow)[N], const float (&mlow)[N], PlainLine& own, float u, float free_v,
+                               float (&hrow)[N], float* force, float* inertia, bool* converged) {
     const uint32_t lane = c.lane;
     const bool coordinate = lane < c.n;
     // the difference of two floats, exact in double (the reference carries it as a float and its rounding error)
@@ -800,14 +897,16 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
     // lane's own head (the first 64 heads) from its constants, without a branch; a lane without an owned head gets zeros
     float mf[3], mc[6], mn[3];
     {
-        const PlainLine own = plain_line(load_head_line(c, lane));
+        if constexpr (kKeepLine<N>) refresh_moves(c, own);
+        else own = own_line(c);
         plain_response(own, own.move[0], own.move[1], own.move[2], mf, mc);
 #pragma unroll
         for (int k = 0; k < 3; ++k) mn[k] = fabsf(mf[k]) + mc[k] * (fabsf(own.res[k]) + fabsf(own.move[k]));
     }
     if (c.elliptic) head_terms(c, lane, mf, mc, mn);   // the cone's own response; the same values as above for every other head
-    const bool mine = mf[0] != 0.0f || mf[1] != 0.0f || mf[2] != 0.0f || mc[0] != 0.0f || mc[1] != 0.0f || mc[2] != 0.0f || mc[5] != 0.0f ||
-                      mc[3] != 0.0f || mc[4] != 0.0f || mn[0] != 0.0f || mn[1] != 0.0f || mn[2] != 0.0f;
+    // (lanes from the heads' count on hold copies of the first sixteen heads when there are no more than that)
+    const bool mine = lane < c.heads && (mf[0] != 0.0f || mf[1] != 0.0f || mf[2] != 0.0f || mc[0] != 0.0f || mc[1] != 0.0f || mc[2] != 0.0f || mc[5] != 0.0f ||
+                      mc[3] != 0.0f || mc[4] != 0.0f || mn[0] != 0.0f || mn[1] != 0.0f || mn[2] != 0.0f);
     const uint32_t my_axes = lane < c.heads ? c.U(hAxes, lane) : 0u;
     const uint32_t my_low = lane < c.heads ? c.U(hColumnsLow, lane) : 0u, my_high = lane < c.heads ? c.U(hColumnsHigh, lane) : 0u;
     // The Hessian M + sum J^T C J changes only through the heads' curvatures: every head keeps the curvature of its
@@ -857,7 +956,33 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
     TileSum g{-inertial.value};
     PROF_END(c, 11);
     PROF_BEGIN(c, 12);
-    if (!c.units) {   // staged heads only: plain head order
+    bool paired = false;
+    if constexpr (N <= 32) {
+        // two or more contributing heads (all of them staged, one a lane): two a pass, the second half of the
+        // wavefront collecting its heads in rows of its own
+        const uint64_t all = __ballot(mine);
+        paired = !c.units && c.heads <= uint32_t(kWave) && (all & (all - 1ull)) != 0ull;
+        if (paired) {
+            if (lane >= 32u) {
+#pragma unroll
+                for (int k = 0; k < N; ++k) hrow[k] = 0.0f;
+                g.value = 0.0; scale = 0.0f;
+            }
+            const uint32_t my_first = lane < c.heads ? c.U(hRow, lane) : 0u;
+            for (uint64_t rest = all; rest != 0ull;) {
+                const uint32_t ha = uint32_t(__builtin_ctzll(rest));
+                rest &= rest - 1ull;
+                const uint32_t hb = rest != 0ull ? uint32_t(__builtin_ctzll(rest)) : kInvalid;
+                rest &= rest - 1ull;   // zero stays zero
+                add_head_pair<N>(c, ha, hb, mf, mc, mn, my_first, my_low, my_high, hrow, g, scale);
+            }
+#pragma unroll
+            for (int k = 0; k < N; ++k) hrow[k] = halves_sum(hrow[k]);
+            g.value = halves_sum(g.value); scale = halves_sum(scale);
+        }
+    }
+    if (paired) {
+    } else if (!c.units) {   // staged heads only: plain head order
         for (uint64_t rest = __ballot(mine); rest != 0ull; rest &= rest - 1ull) {
             const uint32_t h = uint32_t(__builtin_ctzll(rest));
             float f[3], cv[6], noise[3];
@@ -999,13 +1124,13 @@ __device__ __forceinline__ float mass_times(const Tile& c, const float (&mrow)[N
 // convergence test because its mass factor overwrites the Hessian storage; here the two live apart and the
 // assembled row, force and inertia (which the second assembly would reproduce bit for bit) are simply kept.
 template <int N, bool kFollow>
-__device__ __forceinline__ Failure newton_direction(const Tile& c, const float (&mrow)[N], const float (&mlow)[N], float u, float free_v, float* force,
-                                    float* inertia, float* d, bool* converged) {
+__device__ __forceinline__ Failure newton_direction(const Tile& c, const float (&mrow)[N], const float (&mlow)[N], PlainLine& line, float u, float free_v,
+                                    float* force, float* inertia, float* d, bool* converged) {
     PROF_COUNT(c, 0);
     c.work += 16u;
     float hrow[N];
     PROF_BEGIN(c, 1);
-    const bool assembled = assemble_block<N, kFollow>(c, mrow, mlow, u, free_v, hrow, force, inertia, converged);
+    const bool assembled = assemble_block<N, kFollow>(c, mrow, mlow, line, u, free_v, hrow, force, inertia, converged);
     PROF_END(c, 1);
     if (!assembled) return kFailEquation;
     if (*converged && c.tolerance > 0.0f) {
@@ -1146,12 +1271,14 @@ __device__ __forceinline__ void line_derivatives_pair(const Tile& c, const Plain
 }
 
 // SearchTileLine (:2089-2125)
-template <LineMode kMode>
-__device__ __forceinline__ float search_line_in(const Tile& c, float inertial_slope, float inertial_curvature) {
+template <LineMode kMode, bool kKept>
+__device__ __forceinline__ float search_line_in(const Tile& c, PlainLine& plain, float inertial_slope, float inertial_curvature) {
     constexpr bool kPaired = kMode == kLineNarrow;
     float slope = 0.0f, curvature = 0.0f, magnitude = 0.0f;
-    const HeadLine mine = load_head_line(c, kPaired ? (c.lane & 15u) : c.lane);
-    const PlainLine plain = plain_line(mine);
+    HeadLine mine{};
+    if constexpr (kMode == kLineGeneral) mine = load_head_line(c, c.lane);
+    else if constexpr (kKept) refresh_steps(c, plain);
+    else plain = own_line(c);
     float low = 0.0f, high = 0.0f, alpha = 1.0f;
     bool bounded = false;
     float initial;
@@ -1166,7 +1293,7 @@ __device__ __forceinline__ float search_line_in(const Tile& c, float inertial_sl
         if (slope < 0.0f) low = alpha;
         else { high = alpha; bounded = true; }
         if (bounded && high - low <= FLT_EPSILON * high) { *answer = low; return true; }
-        float next = alpha - slope / curvature;
+        float next = alpha - slope * __builtin_amdgcn_rcpf(curvature);
         if (!(next > low && (!bounded || next < high))) next = bounded ? 0.5f * (low + high) : 2.0f * alpha;
         alpha = next;
         return false;
@@ -1193,10 +1320,11 @@ __device__ __forceinline__ float search_line_in(const Tile& c, float inertial_sl
     }
     return low;
 }
-__device__ __forceinline__ float search_line(const Tile& c, float inertial_slope, float inertial_curvature) {
-    if (c.heads > uint32_t(kWave) || c.elliptic) return search_line_in<kLineGeneral>(c, inertial_slope, inertial_curvature);
-    if (c.heads <= 16u) return search_line_in<kLineNarrow>(c, inertial_slope, inertial_curvature);
-    return search_line_in<kLineWide>(c, inertial_slope, inertial_curvature);
+template <bool kKept>
+__device__ __forceinline__ float search_line(const Tile& c, PlainLine& line, float inertial_slope, float inertial_curvature) {
+    if (c.heads > uint32_t(kWave) || c.elliptic) return search_line_in<kLineGeneral, kKept>(c, line, inertial_slope, inertial_curvature);
+    if (c.heads <= 16u) return search_line_in<kLineNarrow, kKept>(c, line, inertial_slope, inertial_curvature);
+    return search_line_in<kLineWide, kKept>(c, line, inertial_slope, inertial_curvature);
 }
 
 __device__ __forceinline__ void apply_moves(const Tile& c, float alpha) {
@@ -1222,6 +1350,8 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], c
         c.F(hMove, h) = 0.0f; c.F(hMove + 1, h) = 0.0f; c.F(hMove + 2, h) = 0.0f;
     }
     __syncthreads();
+    PlainLine line{};   // the heads' constants over this block descent
+    if constexpr (kKeepLine<N>) line = own_line(c);
     float start = coordinate ? *u_io : 0.0f;
     const float free_v = moving && has_free ? free_in : 0.0f;
     if constexpr (kFollow) {   // the followers start where the block's coordinates put them
@@ -1238,7 +1368,7 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], c
         const float inertial_curvature = wave_total(curvature);
         if (inertial_curvature > 0.0f && isfinite(inertial_curvature)) {
             row_steps<N>(c, dd);
-            const float alpha = search_line(c, -inertial_curvature, inertial_curvature);
+            const float alpha = search_line<kKeepLine<N>>(c, line, -inertial_curvature, inertial_curvature);
             if (alpha > 0.0f) {
                 u = fmaf(alpha, dd, u);
                 apply_moves(c, alpha);
@@ -1250,7 +1380,7 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], c
     for (uint32_t step = 0u; step < kNewtonSteps; ++step) {
         float force = 0.0f, inertia = 0.0f, dd = 0.0f;
         bool converged = false;
-        failure = newton_direction<N, kFollow>(c, mrow, mlow, u, free_v, &force, &inertia, &dd, &converged);
+        failure = newton_direction<N, kFollow>(c, mrow, mlow, line, u, free_v, &force, &inertia, &dd, &converged);
         if (converged) primal = 0.0f;
         if (failure != kFailNone || converged) break;
         if (!coordinate) dd = 0.0f;
@@ -1273,7 +1403,7 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], c
         row_steps<N>(c, dd);
         PROF_END(c, 4);
         PROF_BEGIN(c, 5);
-        const float alpha = search_line(c, inertial_slope, inertial_curvature);
+        const float alpha = search_line<kKeepLine<N>>(c, line, inertial_slope, inertial_curvature);
         PROF_END(c, 5);
         const float after = fmaf(alpha, dd, u);
         const bool rounded = __all(!moving || after == u);

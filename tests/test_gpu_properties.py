@@ -351,7 +351,7 @@ def test_environments_on_either_side_of_the_capacity_split_match_the_oracle(orac
         assert np.array_equal(world.download(name), oracle.download(name)), name
     assert not world.download("env_status").any()
     # an environment whose residual sits at the tolerance may stop a sweep earlier or later under other rounding
-    assert np.mean(world.download("vbd_velocity_sweep_count") != oracle.download("vbd_velocity_sweep_count")) <= 0.03
+    assert np.mean(world.download("vbd_velocity_sweep_count") != oracle.download("vbd_velocity_sweep_count")) <= 0.05
     for name in ("qdot", "link_velocity", "base_pose"):
         error = per_env_error(world.download(name), oracle.download(name), E)
         assert error.max() <= 2e-4, (name, float(error.max()), int(counts[error.argmax()]))       # two steps
