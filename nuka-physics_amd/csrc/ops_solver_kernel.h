@@ -757,6 +757,16 @@ __device__ __forceinline__ HeadLine load_head_line(const Tile& c, uint32_t h) {
     return l;
 }
 
+// What the rounding of a head's residual and trial move does to its term of the slope: the impulse is curvature times
+// (residual - move) plus a constant, so each of the two carries its own ulp into the impulse at the rate of the
+// curvature - the noise the reference's block assembly allows its forces (AssembleTileBlock :1568-1572: impulse plus
+// curvature times (|residual| + |move|)).  The reference's line search measures its slopes against the impulses alone
+// (:2075-2083): where a stiff row nearly cancels its residual the slope then moves in steps many times the tolerance, no
+// point of the line meets it, and the search halves its bracket down to one ulp, some twenty probes for nothing.
+// Here the tolerance sees that noise; the accepted step differs from the reference's below the slope's own rounding.
+__device__ __forceinline__ float line_noise(const float (&r)[6], float rx, float ry, float rz, float mx, float my, float mz, float sx, float sy, float sz) {
+    return r[0] * (fabsf(rx) + fabsf(mx)) * fabsf(sx) + r[1] * (fabsf(ry) + fabsf(my)) * fabsf(sy) + r[2] * (fabsf(rz) + fabsf(mz)) * fabsf(sz);
+}
 __device__ __forceinline__ void add_line_terms(const float (&f)[3], const float (&r)[6], float sx, float sy, float sz, TileSum& row_slope,
                                                float& row_curvature, float& row_magnitude) {
     tile_add_product(row_slope, f[0], sx);
@@ -774,6 +784,7 @@ __device__ __forceinline__ void line_terms(const HeadLine& l, float alpha, TileS
         elliptic_impulse(V3{l.dual[0], l.dual[1], l.dual[2]}, l.rho, l.res[0] - fmaf(alpha, sx, l.move[0]), l.res[1] - fmaf(alpha, sy, l.move[1]),
                          l.res[2] - fmaf(alpha, sz, l.move[2]), l.compliance, l.tangent_compliance[0], l.tangent_compliance[1], l.mu_first, f, r);
         add_line_terms(f, r, sx, sy, sz, row_slope, row_curvature, row_magnitude);
+        row_magnitude += line_noise(r, l.res[0], l.res[1], l.res[2], fmaf(alpha, sx, l.move[0]), fmaf(alpha, sy, l.move[1]), fmaf(alpha, sz, l.move[2]), sx, sy, sz);
         return;
     }
     scalar_impulse(l.dual[0], l.rho, l.res[0] - fmaf(alpha, sx, l.move[0]), l.compliance, l.lower, l.upper, l.response, &f[0], &r[0]);
@@ -781,6 +792,7 @@ __device__ __forceinline__ void line_terms(const HeadLine& l, float alpha, TileS
         tangent_impulse(V3{l.dual[0], l.dual[1], l.dual[2]}, l.rho, l.res[1] - fmaf(alpha, sy, l.move[1]),
                         l.res[2] - fmaf(alpha, sz, l.move[2]), l.bound, l.ratios, &f[1], &f[2], &r[1], &r[2], &r[5]);
     add_line_terms(f, r, sx, sy, sz, row_slope, row_curvature, row_magnitude);
+    row_magnitude += line_noise(r, l.res[0], l.res[1], l.res[2], fmaf(alpha, sx, l.move[0]), fmaf(alpha, sy, l.move[1]), fmaf(alpha, sz, l.move[2]), sx, sy, sz);
 }
 // A head's line-search constants as numbers only, so that the probes run without a branch: every selection the
 // response makes on a constant of the head (a single-axis head has no tangent part, a friction ratio of zero takes no
@@ -1193,11 +1205,12 @@ __device__ __forceinline__ void row_steps(const Tile& c, float d) {
 __device__ __forceinline__ void plain_line_terms(const PlainLine& p, float alpha, TileSum& row_slope, float& row_curvature, float& row_magnitude) {
     const float sx = p.step[0], sy = p.step[1], sz = p.step[2];
     float f[3], r[6];
-    plain_response(p, fmaf(alpha, sx, p.move[0]), fmaf(alpha, sy, p.move[1]), fmaf(alpha, sz, p.move[2]), f, r);
+    const float mx = fmaf(alpha, sx, p.move[0]), my = fmaf(alpha, sy, p.move[1]), mz = fmaf(alpha, sz, p.move[2]);
+    plain_response(p, mx, my, mz, f, r);
     tile_add_product(row_slope, f[0], sx);
     tile_add_product(row_slope, f[1], sy);
     tile_add_product(row_slope, f[2], sz);
-    row_magnitude += fabsf(f[0] * sx) + fabsf(f[1] * sy) + fabsf(f[2] * sz);
+    row_magnitude += fabsf(f[0] * sx) + fabsf(f[1] * sy) + fabsf(f[2] * sz) + line_noise(r, p.res[0], p.res[1], p.res[2], mx, my, mz, sx, sy, sz);
     row_curvature += r[0] * sx * sx + r[1] * sy * sy + r[2] * sz * sz + 2.0f * r[5] * sy * sz;
 }
 // The line search runs in one of three modes, the same for every probe of a solve: general (the block has more heads

