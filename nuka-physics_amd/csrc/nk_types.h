@@ -158,6 +158,7 @@ struct DataView {
     float *contact_point, *contact_normal, *contact_force, *ucontact_impulse, *link_contact_wrench;
     uint32_t *contact_side_a_kind, *contact_side_b_kind, *contact_side_a_index, *contact_side_b_index, *contact_link;
     uint32_t *reset_env_ids;                // staging of nuka_world_reset_envs
+    float* solver_mass_factor;              // [env][FactorFloats]: the solve's own factor of the mass matrix, for blocks too wide to keep it in LDS
     uint32_t *solver_cost, *tile_order;     // decaying maximum of the solves' work per environment; launch order of the next solve (costliest first)
     uint32_t *row_unit;                     // per row: the one coordinate a single-coordinate row acts on, ~0u otherwise
     float *row_unit_value;                  // its Jacobian entry there

@@ -126,6 +126,11 @@ static bool ContactHeadsOnly(const ModelView& m, uint32_t staged) {
     const uint32_t joint_heads = m.joint_limit_rows + m.joint_friction_rows + m.joint_drive_rows;
     return joint_heads == 0u && staged <= uint32_t(solver::kWave) && !(m.any_mujoco != 0u && m.contact_cone == 1u);
 }
+uint32_t SolverMassFactorFloats(const ModelView& m) {
+    if (m.rows_per_env == 0u || m.dof == 0u) return 0u;
+    const uint32_t width = SolverSweepWidth(m);
+    return solver::MassFactorInMemory(width) ? solver::FactorFloats(solver::PaddedWidth(width)) : 0u;
+}
 uint32_t SolverSweepWidth(const ModelView& m) {
     if (m.rows_per_env == 0u || m.dof == 0u) return m.dof;
     const uint32_t staged = SolverHeadCapacity(m, std::max(m.contact_slots, 1u), 150u * 1024u);

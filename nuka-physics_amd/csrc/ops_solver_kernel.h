@@ -359,6 +359,16 @@ __device__ __forceinline__ bool factor_rows(uint32_t lane, float (&row)[N], floa
 template <int N>
 constexpr bool kLeavesFirst = N > 32;
 
+// Where a factor is kept for its transposed reads.  Root first: rows of N + 1 words.  Leaves first: lane i's row of
+// U holds the entries k >= i only, and the rows are packed - row i starts at i N - i (i - 1) / 2 and is N - i words
+// long - which halves the storage; a column's words for consecutive lanes are consecutive.
+__host__ __device__ constexpr uint32_t FactorFloats(uint32_t N) { return N > 32u ? (N * (N + 1u) / 2u + 3u) & ~3u : N * (N + 1u); }
+template <int N>
+__device__ __forceinline__ uint32_t factor_at(uint32_t i, uint32_t k) {   // leaves first: k >= i
+    if constexpr (kLeavesFirst<N>) return i * uint32_t(N) - (i * (i - 1u)) / 2u + (k - i);
+    else return i * uint32_t(N + 1) + k;
+}
+
 // FactorTileColumns on register rows: lane i holds row i of the symmetric matrix; on return its entries k >= i are
 // row i of U.  Column k leaves exact zeros in the rows of other branches of the tree, and the update of a column by
 // an exact zero changes nothing: such columns are skipped four at a time.
@@ -405,12 +415,13 @@ __device__ __forceinline__ float substitute_up(uint32_t lane, const float (&row)
         r = lane < uint32_t(j) ? fmaf(-row[j], y, r) : r;
     }
     r *= inverse;
-    const float* column = factor + (lane < uint32_t(N) ? lane : 0u);
+    const uint32_t mine = lane < uint32_t(N) ? lane : 0u;
 #pragma unroll
     for (int j0 = 0; j0 < N; j0 += 8) {
         float u[8];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) u[t] = j0 + t < N ? column[(j0 + t) * (N + 1)] : 0.0f;
+        for (int t = 0; t < 8; ++t)   // U[j][lane] for the lanes past j; the others read a word they do not use
+            u[t] = j0 + t < N ? factor[mine >= uint32_t(j0 + t) ? factor_at<N>(uint32_t(j0 + t), mine) : 0u] : 0.0f;
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
             if (j0 + t >= N) continue;
@@ -447,14 +458,15 @@ __device__ __forceinline__ void store_rows(float* a, uint32_t lane, const float 
     lane = local_lane(lane);
     if (lane < uint32_t(N)) {
 #pragma unroll
-        for (int k = 0; k < N; ++k) a[lane * (N + 1) + k] = row[k];
+        for (int k = 0; k < N; ++k)
+            if (!kLeavesFirst<N> || uint32_t(k) >= lane) a[factor_at<N>(lane, uint32_t(k))] = row[k];
     }
 }
 template <int N>
 __device__ __forceinline__ void load_rows(const float* a, uint32_t lane, float (&row)[N]) {
     lane = local_lane(lane);
 #pragma unroll
-    for (int k = 0; k < N; ++k) row[k] = lane < uint32_t(N) ? a[lane * (N + 1) + k] : 0.0f;
+    for (int k = 0; k < N; ++k) row[k] = lane < uint32_t(N) && (!kLeavesFirst<N> || uint32_t(k) >= lane) ? a[factor_at<N>(lane, uint32_t(k))] : 0.0f;
 }
 template <int N>
 __device__ __forceinline__ void load_columns(const float* a, uint32_t lane, float (&col)[N]) {
@@ -482,7 +494,7 @@ __device__ __forceinline__ bool cholesky_solve(const Tile& c, float (&hrow)[N], 
     } else {
         // rows and the reciprocal diagonal come back from hfac (the factor's own reciprocal is 1 / its diagonal
         // entry, the same division)
-        inverse = row < uint32_t(N) ? 1.0f / c.hfac[row * (N + 1) + row] : 0.0f;
+        inverse = row < uint32_t(N) ? 1.0f / c.hfac[factor_at<N>(row, row)] : 0.0f;
         load_rows<N>(c.hfac, c.lane, hrow);
     }
     PROF_BEGIN(c, 15);
@@ -1711,9 +1723,13 @@ __device__ __forceinline__ void update_duals(const Tile& c, float* lambda_env, u
 
 __host__ __device__ inline uint32_t PaddedWidth(uint32_t n) { return (n + 3u) & ~3u; }
 // `n`: the width the solve works at - the block's coordinates, or the K of a reduced block
+// The factor of the Newton Hessian, and at the widths that run two waves a SIMD the factor of the mass matrix beside
+// it; wider blocks keep the mass factor, which a solve reads a few times a sweep, in device memory instead
+// (DataView::solver_mass_factor), so that two of them fit a compute unit's LDS.
+__host__ __device__ inline bool MassFactorInMemory(uint32_t n) { return PaddedWidth(n) > uint32_t(kTwoWaveWidth); }
 __host__ __device__ inline uint32_t FactorRegionFloats(uint32_t n) {
     const uint32_t N = PaddedWidth(n);
-    return 2u * N * (N + 1u);   // a multiple of 4 since N is
+    return (MassFactorInMemory(n) ? 1u : 2u) * FactorFloats(N);   // a multiple of 4
 }
 // what the set-up of a reduced block passes through LDS ahead of everything else: the eliminated coordinates' factor
 // and their coupling to the others, transposed
@@ -1861,8 +1877,13 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
 #endif
     PROF_BEGIN(c, 9);
     PROF_BEGIN(c, 0);
-    c.mfac = lds;
-    c.hfac = c.mfac + uint32_t(W) * c.ld;
+    if constexpr (W > kTwoWaveWidth) {
+        c.mfac = d.solver_mass_factor + size_t{env} * FactorFloats(uint32_t(W));
+        c.hfac = lds;
+    } else {
+        c.mfac = lds;
+        c.hfac = c.mfac + FactorFloats(uint32_t(W));
+    }
     c.jac = lds + FactorRegionFloats(uint32_t(W));
     c.fields = c.jac + 3u * staged_cap * c.ldj;
     c.vec = c.fields + HeadFieldFloats(cap, staged_cap);

@@ -361,6 +361,7 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(contact_row_extent, kU32, E * 2) X(env_status, kU32, E) X(vbd_velocity_sweep_count, kU32, E) \
     X(solver_residual, kF32, E * 4) X(solver_penalty, kF32, E * R) X(solver_velocity, kF32, E * md) X(solver_free, kF32, E * md) \
     X(solver_cost, kU32, E) X(tile_order, kU32, E) X(row_unit, kU32, E * R) X(row_unit_value, kF32, E * R) \
+    X(solver_mass_factor, kF32, E * mf) \
     X(body_invweight0, kF32, E * nb * 2) X(dof_invweight0, kF32, E * md) X(row_invweight, kF32, E * R) \
     X(row_reference_velocity_gain, kF32, E * R) X(step_qdot_flat, kF32, E * md) \
     X(contact_material, kU64, E * S) X(contact_cache_pair, kU64, E * S * 4) X(contact_cache_feature, kU64, E * S * 4) \
@@ -866,6 +867,7 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
         w.env_count = desc->env_count;
         const ModelView& hc = w.host.counts;
         const size_t E = w.env_count, nl = hc.links_per_env, nb = hc.bodies_per_env, md = hc.max_dof, S = hc.contact_slots, R = hc.rows_per_env;
+        const size_t mf = SolverMassFactorFloats(hc);
         if (E * std::max<size_t>(R, 1u) > 0xFFFFFFFFull / 2u || E * nl * 7u > 0xFFFFFFFFull) throw std::invalid_argument("world too large for 32-bit row indices");
         if (hc.rows_per_env > 0u && SolverHeadCapacity(hc, std::max(hc.contact_slots, 1u), 150u * 1024u) == 0u) throw std::invalid_argument("solver tile does not fit LDS");
         // arena layout: template tables first, then the env-major fields, each on a 256-byte boundary (buffer.hpp:39)
