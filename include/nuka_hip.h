@@ -303,12 +303,14 @@ nuka_result_t nuka_world_synchronize(nuka_world_handle world);   /* nuka.h:376 *
 nuka_result_t nuka_world_reset(nuka_world_handle world);         /* nuka.h:380 */
 /* nuka.h:381-385: duplicates are ignored, count 0 is a no-op, an id out of range returns INVALID_ARG and changes nothing */
 nuka_result_t nuka_world_reset_envs(nuka_world_handle world, const uint32_t* env_ids, uint32_t count);
-/* No counterpart in the reference.  nuka_world_reset_envs for callers that cannot allocate (code under HIP graph
- * capture, tight serving loops, harnesses that forbid hipMalloc): the same kernel and the same result, with the ids
- * staged in a device array of static storage, NUKA_RESET_ENVS_STATIC_MAX words that each GPU the library has opened
- * holds until the process ends, instead of in memory the library allocates.  Takes no device memory and no host heap
- * memory.  More ids than the maximum are refused with NUKA_RESULT_INVALID_ARG (nuka_last_error_message says so).  Every
- * call on one GPU shares that GPU's array: calls that overlap on one GPU race; a call reads only the ids it staged. */
+/* No counterpart in the reference.  nuka_world_reset_envs for callers that cannot allocate (tight serving loops,
+ * harnesses that forbid hipMalloc): the same kernel and the same result, with the ids staged in a device array of
+ * static storage, NUKA_RESET_ENVS_STATIC_MAX words that each GPU the library has opened holds until the process ends,
+ * instead of in memory the library allocates.  Takes no device memory and no host heap memory.  More ids than the
+ * maximum are refused with NUKA_RESULT_INVALID_ARG (nuka_last_error_message says so).  The call blocks the host on the
+ * world's stream (it waits for the stream before it stages the ids and again before it returns), so it does not belong
+ * inside a stream capture.  Every call on one GPU shares that GPU's array; the library serialises such calls on a
+ * process-wide lock held until the call's reset has finished, so they do not overlap. */
 #define NUKA_RESET_ENVS_STATIC_MAX 16384u
 nuka_result_t nuka_world_reset_envs_static(nuka_world_handle world, const uint32_t* env_ids, uint32_t count);
 

@@ -152,8 +152,10 @@ Status DispatchOn(Backend* be, const ModelView& m, const DataView& d, const nuka
 }
 
 // IntegratePosition, FkWorldPoses, FkLinkVelocities and, if it follows, SyncLinkBodyPose at the head of `calls` as one
-// launch: the number of calls served, 0 when the head is something else or the ops must run one by one.
-int MergeStepTail(Backend* be, const ModelView& m, const DataView& d, const nuka_phi_op_call* calls, int n) {
+// launch: the number of calls served, 0 when the head is something else or the merged kernel does not serve these
+// parameters (Unsupported: the ops then run one by one).  Any other failure of the merged launch is the plan's
+// failure and comes back through `status`, never as a quiet fall back that would dispatch the ops a second time.
+int MergeStepTail(Backend* be, const ModelView& m, const DataView& d, const nuka_phi_op_call* calls, int n, Status* failure) {
     if (n < 3 || calls[0].op != uint16_t(NkOp::IntegratePosition) || calls[1].op != uint16_t(NkOp::FkWorldPoses) ||
         calls[2].op != uint16_t(NkOp::FkLinkVelocities)) return 0;
     const bool bodies = n >= 4 && calls[3].op == uint16_t(NkOp::SyncLinkBodyPose);
@@ -161,11 +163,12 @@ int MergeStepTail(Backend* be, const ModelView& m, const DataView& d, const nuka
                                      static_cast<const FkWorldPosesParams*>(calls[1].params),
                                      static_cast<const FkLinkVelocitiesParams*>(calls[2].params),
                                      bodies ? static_cast<const SyncLinkBodyPoseParams*>(calls[3].params) : nullptr, be->stream);
+    if (status != Status::Ok && status != Status::Unsupported) *failure = status;
     return status == Status::Ok ? (bodies ? 4 : 3) : 0;
 }
 
 // SyncLinkBodyPose, BuildAabbs, LbvhBuild, LbvhQueryPairs, NarrowphasePrimitives at the head of `calls` as one launch
-int MergeCollisionHead(Backend* be, const ModelView& m, const DataView& d, const nuka_phi_op_call* calls, int n) {
+int MergeCollisionHead(Backend* be, const ModelView& m, const DataView& d, const nuka_phi_op_call* calls, int n, Status* failure) {
     if (n < 5 || calls[0].op != uint16_t(NkOp::SyncLinkBodyPose) || calls[1].op != uint16_t(NkOp::BuildAabbs) ||
         calls[2].op != uint16_t(NkOp::LbvhBuild) || calls[3].op != uint16_t(NkOp::LbvhQueryPairs) ||
         calls[4].op != uint16_t(NkOp::NarrowphasePrimitives) || calls[2].params == nullptr) return 0;
@@ -173,6 +176,7 @@ int MergeCollisionHead(Backend* be, const ModelView& m, const DataView& d, const
                                           static_cast<const BuildAabbsParams*>(calls[1].params),
                                           static_cast<const LbvhQueryPairsParams*>(calls[3].params),
                                           static_cast<const NarrowphasePrimitivesParams*>(calls[4].params), be->stream);
+    if (status != Status::Ok && status != Status::Unsupported) *failure = status;
     return status == Status::Ok ? 5 : 0;
 }
 
@@ -216,8 +220,9 @@ nuka_phi_plan* BePlanCreate(nuka_phi_backend* b, const nuka_phi_model_view* m, c
         // The ops after the solve, and those between the dynamics and the row assembly, each take about a launch's time:
         // where the list holds them in a row, one kernel runs them (StepTailKernel, CollisionHeadKernel); where it cannot,
         // they go one by one as dispatched.
-        int merged = MergeStepTail(be, model, data, calls + i, n_calls - i);
-        if (merged == 0) merged = MergeCollisionHead(be, model, data, calls + i, n_calls - i);
+        int merged = MergeStepTail(be, model, data, calls + i, n_calls - i, &status);
+        if (merged == 0 && status == Status::Ok) merged = MergeCollisionHead(be, model, data, calls + i, n_calls - i, &status);
+        if (status != Status::Ok) { failed = calls[i].op; break; }
         if (merged > 0) { i += merged - 1; continue; }
         status = DispatchOn(be, model, data, calls[i]);
         if (status != Status::Ok) failed = calls[i].op;

@@ -6,8 +6,9 @@
 // Not read: meshes, height fields, materials, cameras, lights, sensors, sites, equalities, <contact> pairs, ball
 // joints (rejected), tendons.  Geoms carry the MuJoCo contact law as in the reference's importer (every MJCF shape is
 // MuJoCo-sourced, mjcf_importer.cpp:790): friction, solref, solimp, margin and gap go into contact profiles, and
-// <option cone impratio> selects the cone.  The joint rows keep this library's native law: the solref / solimp
-// compliant limit and friction rows the reference attaches to MJCF joints are not built.
+// <option cone impratio> selects the cone.  Joints carry the MuJoCo law too (margin, solreflimit / solimplimit,
+// solreffriction / solimpfriction: compliant limit and friction rows), and <option integrator> selects the damping
+// pass after the solve.
 #include "scene_loader.h"
 
 #include "scene_build.h"
@@ -309,8 +310,11 @@ struct Builder : SceneParts {
             QueryInt(e, "priority", &priority);
             QueryInt(e, "condim", &condim);
             g.priority = int32_t(priority);
-            // torsional and rolling friction (condim 4, 6) have no rows here: such a geom keeps its sliding friction
-            g.condim = condim == 1 ? 1u : 3u;
+            // the contact dimensions the path has rows for (scene/cook/cook_to_model.cpp:188-196 and nk/model/model.cpp:66
+            // refuse every other value; torsional and rolling friction, condim 4 and 6, get no rows in assemble_rows.cu)
+            if (condim != 1 && condim != 3) throw Unsupported("MJCF: geom condim " + std::to_string(condim) + " is not supported on this path (1 or 3)");
+            g.condim = uint32_t(condim);
+            if (!(g.margin >= 0.0f) || !(g.gap >= 0.0f)) throw std::runtime_error("MJCF: geom margin and gap must not be negative");
             float density = gd.density, geom_mass = gd.mass;
             QueryFloat(e, "density", &density);
             QueryFloat(e, "mass", &geom_mass);

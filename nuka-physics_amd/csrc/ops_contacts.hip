@@ -1117,7 +1117,8 @@ __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4, 4
     }
     // joint rows (EmitJointRowsKernel, assemble_rows.cu:803-1026): stable per-link slots after the contact rows - lower
     // and upper limit (two a link), dry friction, drive.  Each acts on one coordinate, J = +-e_joint; the rest of
-    // its Jacobian row is never written and stays at the zeros it was allocated with.  Native law only.
+    // its Jacobian row is never written and stays at the zeros it was allocated with.  A MuJoCo-sourced joint gets its
+    // limit and friction rows as compliant rows (margin, solref, solimp at the coordinate's reference weight).
     {
         const uint32_t limit_rows = p.joint_limit_rows_per_env, friction_rows = p.joint_friction_rows_per_env;
         const uint32_t joint_slots = limit_rows + friction_rows + p.joint_drive_rows_per_env;

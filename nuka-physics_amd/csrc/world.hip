@@ -442,6 +442,7 @@ struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
     nuka_phi_plan* plan = nullptr;
     std::vector<float> drive_stiffness, drive_force_limit;   // per template link: what nuka_world_get_param reports
     uint64_t capture_attempts = 0u, graph_replays = 0u;      // nuka_world_get_execution_info
+    uint64_t param_version = 0u;   // counts the calls that may have changed a live parameter: a checkpoint taken at the current count holds the current values
     nuka_phi_execution_error last_error{};
 
     ~World() {
@@ -479,6 +480,7 @@ struct Checkpoint {
     CheckpointSegments segments{};
     uint64_t bytes = 0u;
     LiveParams params;
+    uint64_t param_version = ~0ull;   // the owner's count when `params` was last known to equal its live parameters
 };
 bool OwnedBy(const Checkpoint* cp, const World* w) { return cp->owner == w && cp->owner_id == w->id; }
 
@@ -1154,6 +1156,7 @@ nuka_result_t nuka_world_set_velocity_iterations(nuka_world_handle world, uint32
     if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
     if (iterations == 0u || iterations > 65535u) return Error(NUKA_RESULT_INVALID_ARG, "iterations must be in 1..65535");
     if (w->be->synchronize(w->backend, nullptr) != uint8_t(Status::Ok)) return Error(NUKA_RESULT_DEVICE_ERROR, "device error");
+    ++w->param_version;
     w->cfg.solver_vel_iters = iterations;
     w->p_solve.iterations = iterations;
     InvalidatePlan(*w);   // a changed value invalidates the execution graph (nuka.h:287-288)
@@ -1615,6 +1618,7 @@ nuka_result_t nuka_world_checkpoint_capture(nuka_world_handle world, nuka_checkp
     }
     cp->layout_hash = CheckpointLayoutHash(*w);
     if (const nuka_result_t r = ReadLiveParams(w, &cp->params); r != NUKA_RESULT_OK) { Iface(cp->store)->free(cp->store); return r; }
+    cp->param_version = w->param_version;
     *out = reinterpret_cast<nuka_checkpoint_handle>(cp.release());
     return NUKA_RESULT_OK;
 }
@@ -1706,7 +1710,12 @@ nuka_result_t nuka_world_checkpoint_restore(nuka_world_handle world, nuka_checkp
     auto* cp = reinterpret_cast<Checkpoint*>(checkpoint);
     if (w == nullptr || cp == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world or checkpoint is null");
     if (!OwnedBy(cp, w)) return Error(NUKA_RESULT_INVALID_ARG, "checkpoint belongs to another world");
-    if (const nuka_result_t r = ApplyLiveParams(w, cp->params); r != NUKA_RESULT_OK) return r;
+    // no parameter call since the checkpoint's values were last seen to be the world's: nothing to compare, the restore
+    // only enqueues its copy
+    if (cp->param_version != w->param_version) {
+        if (const nuka_result_t r = ApplyLiveParams(w, cp->params); r != NUKA_RESULT_OK) return r;
+        cp->param_version = w->param_version;
+    }
     hipLaunchKernelGGL(CheckpointCopyKernel, dim3(256, cp->segments.count), dim3(256), 0, BackendStream(w->device->backend), cp->segments, 1u);
     return hipGetLastError() == hipSuccess ? NUKA_RESULT_OK : Error(NUKA_RESULT_DEVICE_ERROR, "checkpoint restore failed");
 }
@@ -1950,6 +1959,7 @@ nuka_result_t nuka_world_set_param(nuka_world_handle world, uint32_t param, uint
     auto* w = reinterpret_cast<World*>(world);
     if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
     if (param >= kParamCount) return Error(NUKA_RESULT_INVALID_ARG, "unknown parameter");
+    ++w->param_version;
     try {
         return SetParam(*w, world, param, element, value);
     } catch (const std::bad_alloc&) {

@@ -541,3 +541,42 @@ def test_a_plan_steps_bit_for_bit_like_the_ops_one_by_one(device, index, E):
     for name in fields[False]:
         assert np.array_equal(fields[False][name].view(np.uint32), fields[True][name].view(np.uint32)), name
     assert hashes[0] == hashes[1]
+
+
+@pytest.mark.parametrize("case", ["substeps", "mujoco_integrator"])
+def test_a_plan_merges_ops_inside_substeps_and_ahead_of_the_damping_pass(device, case):
+    """The same identity where the ops a plan merges stand elsewhere in the list: inside an interval that repeats
+    (two substeps, each closed by AccumulateStep), and with ArticulationDamping between the solve and the ops after it
+    (the MuJoCo integrator on MuJoCo-sourced joints with servos)."""
+    import copy
+    E = 128
+    cfg = nk.synthetic.config(3, E)
+    t = copy.deepcopy(cfg.template)
+    gains = {}
+    if case == "mujoco_integrator":
+        t.drive_rows, t.drive_mode, t.integrator = True, abi.DRIVE_PD_POSITION, abi.INTEGRATOR_MUJOCO_EULER
+        for l, link in enumerate(t.links):
+            if link["joint_type"] == abi.JOINT_REVOLUTE:
+                link["law"] = abi.LAW_MUJOCO
+                link["damping"] = 0.3
+                link["lower"], link["upper"] = float(cfg.nominal_q[l]) - 0.4, float(cfg.nominal_q[l]) + 0.4
+        rng = np.random.default_rng(3)
+        nl = t.link_count
+        gains = dict(drive_target=np.tile(cfg.nominal_q, (E, 1)), drive_stiffness=rng.uniform(20, 80, (E, nl)), drive_damping=rng.uniform(0.5, 3, (E, nl)))
+    desc = abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters, substeps=2 if case == "substeps" else 0)
+    fields, hashes = {}, []
+    for graph in (False, True):
+        world = nk.World(device, t, desc)
+        world.set_state(cfg.state())
+        for name, values in gains.items():
+            world.upload(name, values.astype(np.float32))
+        world.set_execution_mode(graph)
+        world.step(4)
+        world.synchronize()
+        assert not world.download("env_status").any()
+        hashes.append(world.state_hash())
+        fields[graph] = {name: world.download(name).copy() for name in ("q", "qdot", "base_pose", "link_pose", "link_velocity", "body_pose", "lambda")}
+        world.close()
+    for name in fields[False]:
+        assert np.array_equal(fields[False][name].view(np.uint32), fields[True][name].view(np.uint32)), name
+    assert hashes[0] == hashes[1]

@@ -308,12 +308,25 @@ def test_errors(tmp_path):
         "xml": '<mujoco><worldbody><body></worldbody></mujoco>',
         "root": '<robot/>',
     }
+    # contact dimensions other than 1 and 3, and negative margins or gaps, are refused as the reference's cook refuses
+    # them (scene/cook/cook_to_model.cpp:188-196, nk/model/model.cpp:66), not read as something else
+    geom = '<mujoco><worldbody><body><freejoint/><geom type="sphere" size="0.1" %s/></body></worldbody></mujoco>'
+    for condim in (0, 2, 4, 6):
+        cases[f"condim{condim}"] = geom % f'condim="{condim}"'
+    cases["margin"] = geom % 'margin="-0.01"'
+    cases["gap"] = geom % 'gap="-0.01"'
+    expected = {"margin": "margin and gap", "gap": "margin and gap", **{f"condim{c}": f"condim {c}" for c in (0, 2, 4, 6)}}
     for name, text in cases.items():
         path = tmp_path / f"{name}.xml"
         path.write_text(text)
         with pytest.raises(nk.NukaError) as err:
             nk.Scene(str(path))
         assert err.value.code == abi.RESULT_INVALID_ARG, name
+        assert expected.get(name, "") in str(err.value), (name, str(err.value))
+    for attributes in ('condim="1"', 'condim="3"', 'margin="0.01" gap="0.002"'):
+        path = tmp_path / "accepted.xml"
+        path.write_text(geom % attributes)
+        assert nk.Scene(str(path)).link_count == 1
 
 
 def test_joint_law_attributes_and_integrator(tmp_path):
