@@ -15,7 +15,7 @@
 static const uint32_t kDecaySteps = 2u;
 
 static uint64_t profile_word(uint64_t hash, uint32_t word) { hash ^= (uint64_t)word; hash *= 0x100000001b3ull; return hash; }
-static uint32_t bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static uint32_t bits(float f) { return f2u(f); }
 
 /* HashMergedContactProfile (:88-105) of two default-authored profiles that differ in friction only
  * (scene/contact_filter.hpp:16-31, 72-130: equal priorities and solmix leave every other term at its default), then

@@ -156,8 +156,13 @@ static inline xform xform_load(const float* p) {
 static inline void xform_store(float* p, xform t) {
     p[0] = t.p.x; p[1] = t.p.y; p[2] = t.p.z; p[3] = t.r.w; p[4] = t.r.x; p[5] = t.r.y; p[6] = t.r.z;
 }
-static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
-static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+/* 32-bit patterns kept in scalar words.  In the double-precision build (nko_double.h) the word is a double that holds
+ * the single-precision value of the pattern exactly, NaN payloads and subnormals included. */
+#ifndef NKO_DOUBLE
+typedef float nko_f32;
+#endif
+static inline uint32_t f2u(float f) { const nko_f32 g = (nko_f32)f; uint32_t u; memcpy(&u, &g, 4); return u; }
+static inline float u2f(uint32_t u) { nko_f32 g; memcpy(&g, &u, 4); return g; }
 
 quat nko_quat_mul(quat a, quat b);
 quat nko_quat_normalize_rsqrt(quat q, float eps);

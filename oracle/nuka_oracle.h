@@ -149,6 +149,7 @@ int nko_world_field(nko_world* w, const char* name, void** ptr, size_t* bytes);
 /* Comma-separated list of the field names nko_world_field serves. */
 const char* nko_world_field_names(void);
 void nko_world_set_threads(nko_world* w, int threads);
+uint32_t nko_real_bytes(void);
 uint32_t nko_world_dof(const nko_world* w);
 uint32_t nko_world_rows_per_env(const nko_world* w);
 

@@ -7,6 +7,7 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "_build", "libnuka_oracle.so")
+LIB64_PATH = os.path.join(HERE, "_build", "libnuka_oracle_f64.so")   # the same sources with every scalar a double
 REF_PATH = os.path.join(HERE, "_ref", "libnuka_ref.so")
 
 U32_FIELDS = {"candidate_pairs", "pair_count", "ucontact_count", "ucontact_a", "ucontact_b", "ucontact_law",
@@ -23,13 +24,80 @@ U64_FIELDS = {"ucontact_id_pair", "ucontact_id_feature", "contact_material", "co
 def build(force=False):
     """Compiles the oracle (and, where the reference tree is mounted, the reference-header shim)."""
     # make compares the sources' and headers' times with the library's: an up-to-date library costs nothing
-    subprocess.run(["make", "-C", HERE, "_build/libnuka_oracle.so"] + (["-B"] if force else []), check=True,
+    subprocess.run(["make", "-C", HERE, "_build/libnuka_oracle.so", "_build/libnuka_oracle_f64.so"] + (["-B"] if force else []), check=True,
                    stdout=subprocess.DEVNULL)
     if os.path.isdir("/root/reference/src") and (force or not os.path.exists(REF_PATH)):
         subprocess.run(["make", "-C", HERE, "ref"], check=True, stdout=subprocess.DEVNULL)
 
 
 _lib = None
+_lib64 = None
+
+
+def lib64():
+    """The double-precision build: the world entry points only (what steps a world and reads its fields)."""
+    global _lib64
+    if _lib64 is None:
+        build()
+        L = C.CDLL(LIB64_PATH)
+        _declare_world_entry_points(L)
+        assert L.nko_real_bytes() == 8
+        _lib64 = L
+    return _lib64
+
+
+def _declare_world_entry_points(L):
+    L.nko_world_create.restype = C.c_void_p
+    L.nko_world_create.argtypes = [C.c_void_p, C.c_void_p]
+    L.nko_world_destroy.argtypes = [C.c_void_p]
+    L.nko_world_field.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t)]
+    L.nko_world_field_names.restype = C.c_char_p
+    L.nko_world_set_threads.argtypes = [C.c_void_p, C.c_int]
+    L.nko_world_dof.argtypes = [C.c_void_p]
+    L.nko_world_dof.restype = C.c_uint32
+    L.nko_world_rows_per_env.argtypes = [C.c_void_p]
+    L.nko_world_rows_per_env.restype = C.c_uint32
+    L.nko_real_bytes.restype = C.c_uint32
+    for name in ("fk_world_poses", "sync_link_body_pose", "build_aabbs", "query_pairs", "narrowphase",
+                 "assemble_rows", "block_descent_solve", "integrate_position", "fk_link_velocities", "apply_drives",
+                 "readout_drives", "readout_contact_wrench", "reference_weights", "snapshot_step_velocity",
+                 "articulation_damping"):
+        getattr(L, "nko_" + name).argtypes = [C.c_void_p]
+    L.nko_articulation_dynamics.argtypes = [C.c_void_p, C.c_uint32]
+    L.nko_contact_warm_start.argtypes = [C.c_void_p, C.c_uint32]
+    L.nko_world_step.argtypes = [C.c_void_p]
+
+
+def widened(struct, arrays=None):
+    """A descriptor struct for the double-precision build: the same members in the same order with every float a
+    double, arrays of floats converted (`arrays`: the float32 arrays behind the struct's pointers, by member name).
+    Returns the struct and what must stay alive with it."""
+    fields, keep = [], []
+    for name, ctype in struct._fields_:
+        if ctype is C.c_float:
+            ctype = C.c_double
+        elif isinstance(ctype, type) and issubclass(ctype, C.Array) and ctype._type_ is C.c_float:
+            ctype = C.c_double * ctype._length_
+        elif ctype == C.POINTER(C.c_float):
+            ctype = C.POINTER(C.c_double)
+        fields.append((name, ctype))
+    wide = type(type(struct).__name__ + "F64", (C.Structure,), {"_fields_": fields})()
+    for (name, old), (_, new) in zip(struct._fields_, fields):
+        value = getattr(struct, name)
+        if new == C.POINTER(C.c_double):
+            source = None if arrays is None else arrays.get(name)
+            if source is not None and source.size:
+                converted = np.ascontiguousarray(source, dtype=np.float64)
+                keep.append(converted)
+                setattr(wide, name, converted.ctypes.data_as(new))
+        elif isinstance(new, type) and issubclass(new, C.Array):
+            for i in range(new._length_):
+                getattr(wide, name)[i] = value[i]
+        else:
+            setattr(wide, name, value)
+    if hasattr(wide, "struct_size"):
+        wide.struct_size = C.sizeof(wide)
+    return wide, keep
 
 
 def lib():
@@ -61,9 +129,15 @@ def lib():
 
 
 class OracleWorld:
-    def __init__(self, template, desc, threads=1):
-        L = lib()
+    def __init__(self, template, desc, threads=1, double=False):
+        """`double`: the double-precision build of the same sources - every field then reads and writes as float64."""
+        self._double = double
+        L = self._lib = lib64() if double else lib()
         tdesc, self._keep = template.to_c()
+        if double:
+            tdesc, kept = widened(tdesc, self._keep)
+            desc, _ = widened(desc)
+            self._keep = (self._keep, kept)
         self._h = L.nko_world_create(C.byref(tdesc), C.byref(desc))
         if not self._h:
             raise RuntimeError("oracle: template rejected")
@@ -75,7 +149,7 @@ class OracleWorld:
 
     def close(self):
         if self._h:
-            lib().nko_world_destroy(self._h)
+            self._lib.nko_world_destroy(self._h)
             self._h = None
 
     def __del__(self):
@@ -83,9 +157,9 @@ class OracleWorld:
 
     def field(self, name):
         ptr, nbytes = C.c_void_p(), C.c_size_t()
-        if lib().nko_world_field(self._h, name.encode(), C.byref(ptr), C.byref(nbytes)) != 0:
+        if self._lib.nko_world_field(self._h, name.encode(), C.byref(ptr), C.byref(nbytes)) != 0:
             raise KeyError(name)
-        dtype = np.uint32 if name in U32_FIELDS else np.uint64 if name in U64_FIELDS else np.float32
+        dtype = np.uint32 if name in U32_FIELDS else np.uint64 if name in U64_FIELDS else np.float64 if self._double else np.float32
         count = nbytes.value // np.dtype(dtype).itemsize
         if count == 0:
             return np.zeros(0, dtype)
@@ -109,8 +183,8 @@ class OracleWorld:
         lv[:, 0, :] = state["root_twist"]
 
     def op(self, name, *args):
-        getattr(lib(), "nko_" + name)(self._h, *args)
+        getattr(self._lib, "nko_" + name)(self._h, *args)
 
     def step(self, n=1):
         for _ in range(n):
-            lib().nko_world_step(self._h)
+            self._lib.nko_world_step(self._h)
