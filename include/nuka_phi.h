@@ -131,6 +131,45 @@ const char* nuka_hip_op_name(uint16_t op);
 /* -1 when the name is not an op of this backend. */
 int nuka_hip_op_from_name(const char* name);
 
+/* ModelView / DataView (src/nk/model/generated/views.hpp:34-36; forward-declared in src/phi/backend.hpp) are flat
+ * aggregates of device pointers, one per field of src/nk/model/fields.yaml.  This backend's two views hold the fields
+ * its ops touch under the same names, element types and per-entity widths, plus a few of its own; a host that keeps
+ * the reference's field table fills them through the calls below instead of by struct layout.  All of them are also
+ * reached through RegistryEntryI::get_proc_address under their own names (src/phi/backend.hpp:124).
+ *
+ * One member of a view.  `reference_name` is the field of fields.yaml the member stands for (mostly the member's own
+ * name; dof_link is dof_to_link there), NULL for a member of this backend's own, which a host gives memory from its
+ * solver scratch (block_descent_scratch in fields.yaml).  `dtype` is the scalar the elements are made of (0 float32,
+ * 1 uint32, 2 uint64, 3 uint8), `per` the entity the field has one element group for, `scalars_per_entity` the scalars
+ * of a group (a transform per link: 7), 0 where the field is sized by a count of its own (per scalar).  Model fields
+ * are read for one environment: where the host replicates them per environment, the first copy serves. */
+enum { NUKA_HIP_PER_ENV = 0, NUKA_HIP_PER_LINK, NUKA_HIP_PER_BODY, NUKA_HIP_PER_DOF, NUKA_HIP_PER_DOF2, NUKA_HIP_PER_CONTACT_SLOT,
+       NUKA_HIP_PER_ROW_SLOT, NUKA_HIP_PER_ROW_DOF, NUKA_HIP_PER_SCALAR };
+typedef struct nuka_hip_view_field_t {
+    const char* name;
+    const char* reference_name;
+    uint8_t owner;   /* 0 model view, 1 data view */
+    uint8_t dtype;
+    uint8_t per;
+    uint32_t scalars_per_entity;
+} nuka_hip_view_field_t;
+uint32_t nuka_hip_view_field_count(void);
+/* 0 on success, -1 past the last field */
+int nuka_hip_view_field(uint32_t index, nuka_hip_view_field_t* out);
+/* bytes of the two view structs, for a host that allocates them as opaque storage (zero them first) */
+size_t nuka_hip_model_view_bytes(void);
+size_t nuka_hip_data_view_bytes(void);
+/* Sets the member of either view that stands for each named field (`names[i]`: a name of fields.yaml, or a member's own
+ * name) to `pointers[i]`; names no member stands for are ignored.  Returns the number of members still null afterwards
+ * and writes their names, comma separated, to `missing` (as far as `missing_bytes` allows; may be NULL). */
+int nuka_hip_bind_views(const char* const* names, void* const* pointers, uint32_t count, nuka_phi_model_view* model, nuka_phi_data_view* data,
+                        char* missing, size_t missing_bytes);
+/* The per-environment counts at the head of the model view, by name (links_per_env, bodies_per_env, dof, max_dof,
+ * max_depth, contact_slots, rows_per_env, contact_rows_per_env, profile_count, floating_root, max_points_per_slot,
+ * excluded_pair_count, joint_limit_rows, joint_friction_rows, joint_drive_rows, drive_mode, any_mujoco, contact_cone,
+ * integrator, contact_dof_end).  0 on success, -1 for an unknown name. */
+int nuka_hip_model_view_set_count(nuka_phi_model_view* model, const char* name, uint32_t value);
+
 #ifdef __cplusplus
 }
 #endif

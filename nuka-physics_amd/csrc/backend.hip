@@ -350,6 +350,13 @@ void* RegGetProcAddress(nuka_phi_registry_entry*, const char* name) {
     if (name == nullptr) return nullptr;
     if (std::strcmp(name, "nuka_hip_op_name") == 0) return reinterpret_cast<void*>(&nuka_hip_op_name);
     if (std::strcmp(name, "nuka_hip_op_from_name") == 0) return reinterpret_cast<void*>(&nuka_hip_op_from_name);
+    // the views by field name
+    if (std::strcmp(name, "nuka_hip_view_field_count") == 0) return reinterpret_cast<void*>(&nuka_hip_view_field_count);
+    if (std::strcmp(name, "nuka_hip_view_field") == 0) return reinterpret_cast<void*>(&nuka_hip_view_field);
+    if (std::strcmp(name, "nuka_hip_model_view_bytes") == 0) return reinterpret_cast<void*>(&nuka_hip_model_view_bytes);
+    if (std::strcmp(name, "nuka_hip_data_view_bytes") == 0) return reinterpret_cast<void*>(&nuka_hip_data_view_bytes);
+    if (std::strcmp(name, "nuka_hip_bind_views") == 0) return reinterpret_cast<void*>(&nuka_hip_bind_views);
+    if (std::strcmp(name, "nuka_hip_model_view_set_count") == 0) return reinterpret_cast<void*>(&nuka_hip_model_view_set_count);
     return nullptr;
 }
 const nuka_phi_registry_entry_i kRegistryI = {RegName, RegDeviceCount, RegGetDevice, RegGetProcAddress};

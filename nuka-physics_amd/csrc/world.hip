@@ -1280,6 +1280,120 @@ nuka_result_t nuka_world_dispatch_op(nuka_world_handle world, uint16_t op, uint3
     return NUKA_RESULT_OK;
 }
 
+// ---- the views by field name (include/nuka_phi.h) -----------------------------------------------------------------
+namespace nkh {
+namespace {
+struct ViewField { const char* name; const char* reference_name; uint8_t owner, dtype, per; uint32_t scalars; size_t offset; };
+// Members that stand for a field of fields.yaml under another name there, and members of the backend's own (no
+// counterpart: nullptr).  Every other member carries the reference's name.
+const char* ReferenceName(const char* name) {
+    static const char* const renamed[][2] = {{"dof_link", "dof_to_link"}, {"dof_component", "dof_to_component"}};
+    static const char* const own[] = {"joint_law", "link_push_order", "sweep_links", "link_dof", "link_dof_mask", "pairable_rows", "profile_mu",
+                                      "profile_law", "profile_solref", "profile_solimp", "profile_margin", "profile_mix", "articulation_qdd",
+                                      "solver_penalty", "solver_velocity", "solver_free", "solver_cost", "tile_order", "row_unit",
+                                      "row_unit_value", "solver_mass_factor", "contact_cache_match"};
+    for (const auto& pair : renamed) if (std::strcmp(name, pair[0]) == 0) return pair[1];
+    for (const char* mine : own) if (std::strcmp(name, mine) == 0) return nullptr;
+    return name;
+}
+// The model tables' element groups: entity and scalars a group (the data fields' follow from their counts).
+struct ModelShape { const char* name; uint8_t per; uint32_t scalars; };
+constexpr ModelShape kModelShapes[] = {
+    {"joint_type", NUKA_HIP_PER_LINK, 1u}, {"parent_link", NUKA_HIP_PER_LINK, 1u}, {"joint_axis", NUKA_HIP_PER_LINK, 3u}, {"parent_offset", NUKA_HIP_PER_LINK, 3u},
+    {"link_local_pose", NUKA_HIP_PER_LINK, 7u}, {"link_inertial_frame", NUKA_HIP_PER_LINK, 7u}, {"link_inertia", NUKA_HIP_PER_LINK, 36u},
+    {"joint_damping", NUKA_HIP_PER_LINK, 1u}, {"joint_armature", NUKA_HIP_PER_LINK, 1u}, {"joint_stiffness", NUKA_HIP_PER_LINK, 1u},
+    {"joint_spring_reference", NUKA_HIP_PER_LINK, 1u}, {"joint_limit_lower", NUKA_HIP_PER_LINK, 1u}, {"joint_limit_upper", NUKA_HIP_PER_LINK, 1u},
+    {"joint_frictionloss", NUKA_HIP_PER_LINK, 1u}, {"joint_limit_flags", NUKA_HIP_PER_LINK, 1u}, {"joint_law", NUKA_HIP_PER_LINK, 1u},
+    {"joint_limit_margin", NUKA_HIP_PER_LINK, 1u}, {"joint_limit_reference", NUKA_HIP_PER_LINK, 7u}, {"joint_friction_reference", NUKA_HIP_PER_LINK, 7u},
+    {"link_body", NUKA_HIP_PER_LINK, 1u}, {"link_tree_depth", NUKA_HIP_PER_LINK, 1u}, {"link_child_range", NUKA_HIP_PER_LINK, 2u},
+    {"link_children", NUKA_HIP_PER_LINK, 1u}, {"link_push_order", NUKA_HIP_PER_LINK, 1u}, {"sweep_links", NUKA_HIP_PER_SCALAR, 0u},
+    {"link_dof", NUKA_HIP_PER_LINK, 1u}, {"dof_link", NUKA_HIP_PER_DOF, 1u}, {"dof_component", NUKA_HIP_PER_DOF, 1u}, {"link_dof_mask", NUKA_HIP_PER_LINK, 1u},
+    {"link_geom_kind", NUKA_HIP_PER_LINK, 1u}, {"link_geom_local", NUKA_HIP_PER_LINK, 7u}, {"shape_table", NUKA_HIP_PER_SCALAR, 0u},
+    {"body_to_link", NUKA_HIP_PER_BODY, 1u}, {"body_to_articulation", NUKA_HIP_PER_BODY, 1u}, {"body_collidable_link", NUKA_HIP_PER_BODY, 1u},
+    {"body_collidable_body", NUKA_HIP_PER_BODY, 1u}, {"body_collidable_local", NUKA_HIP_PER_BODY, 7u}, {"pairable_rows", NUKA_HIP_PER_BODY, 1u},
+    {"profile_mu", NUKA_HIP_PER_SCALAR, 0u}, {"profile_law", NUKA_HIP_PER_SCALAR, 0u}, {"profile_solref", NUKA_HIP_PER_SCALAR, 0u},
+    {"profile_solimp", NUKA_HIP_PER_SCALAR, 0u}, {"profile_margin", NUKA_HIP_PER_SCALAR, 0u}, {"profile_mix", NUKA_HIP_PER_SCALAR, 0u},
+    {"excluded_pairs", NUKA_HIP_PER_SCALAR, 0u}};
+// A data field's entity and group from its count, evaluated at counts that are distinct primes past any group size:
+// the primes that divide the count name the entity, what is left is the group.
+void DataShape(size_t count, uint8_t* per, uint32_t* scalars) {
+    constexpr size_t kEnvs = 2u, kLinks = 101u, kBodies = 103u, kDof = 107u, kSlots = 109u, kRows = 113u, kOwn = 127u;
+    size_t rest = count / kEnvs;
+    auto takes = [&](size_t prime) { if (rest % prime != 0u) return false; rest /= prime; return true; };
+    if (takes(kOwn)) { *per = NUKA_HIP_PER_SCALAR; *scalars = 0u; return; }
+    if (takes(kLinks)) *per = NUKA_HIP_PER_LINK;
+    else if (takes(kBodies)) *per = NUKA_HIP_PER_BODY;
+    else if (takes(kSlots)) *per = NUKA_HIP_PER_CONTACT_SLOT;
+    else if (takes(kRows)) *per = takes(kDof) ? NUKA_HIP_PER_ROW_DOF : NUKA_HIP_PER_ROW_SLOT;
+    else if (takes(kDof)) *per = takes(kDof) ? NUKA_HIP_PER_DOF2 : NUKA_HIP_PER_DOF;
+    else *per = NUKA_HIP_PER_ENV;
+    *scalars = uint32_t(rest);
+}
+const std::vector<ViewField>& ViewFields() {
+    static const std::vector<ViewField> fields = [] {
+        std::vector<ViewField> out;
+#define X(field, dtype) { uint8_t per = NUKA_HIP_PER_SCALAR; uint32_t scalars = 0u; \
+            for (const ModelShape& shape : kModelShapes) if (std::strcmp(shape.name, #field) == 0) { per = shape.per; scalars = shape.scalars; } \
+            out.push_back({#field, ReferenceName(#field), 0u, uint8_t(dtype), per, scalars, offsetof(ModelView, field)}); }
+        NKH_MODEL_FIELDS(X)
+#undef X
+        const size_t E = 2u, nl = 101u, nb = 103u, md = 107u, S = 109u, R = 113u, mf = 127u;
+#define X(field, dtype, count) { uint8_t per = 0u; uint32_t scalars = 0u; DataShape(size_t(count), &per, &scalars); \
+            out.push_back({#field, ReferenceName(#field), 1u, uint8_t(dtype), per, scalars, offsetof(DataView, field)}); }
+        NKH_DATA_FIELDS(X)
+#undef X
+        return out;
+    }();
+    return fields;
+}
+}  // namespace
+}  // namespace nkh
+
+uint32_t nuka_hip_view_field_count(void) { return uint32_t(nkh::ViewFields().size()); }
+int nuka_hip_view_field(uint32_t index, nuka_hip_view_field_t* out) {
+    const auto& fields = nkh::ViewFields();
+    if (out == nullptr || index >= fields.size()) return -1;
+    const nkh::ViewField& f = fields[index];
+    *out = {f.name, f.reference_name, f.owner, f.dtype, f.per, f.scalars};
+    return 0;
+}
+size_t nuka_hip_model_view_bytes(void) { return sizeof(nkh::ModelView); }
+size_t nuka_hip_data_view_bytes(void) { return sizeof(nkh::DataView); }
+int nuka_hip_bind_views(const char* const* names, void* const* pointers, uint32_t count, nuka_phi_model_view* model, nuka_phi_data_view* data,
+                        char* missing, size_t missing_bytes) {
+    if (model == nullptr || data == nullptr || (count != 0u && (names == nullptr || pointers == nullptr))) return -1;
+    int unset = 0;
+    size_t written = 0u;
+    if (missing != nullptr && missing_bytes != 0u) missing[0] = '\0';
+    for (const nkh::ViewField& f : nkh::ViewFields()) {
+        void** member = reinterpret_cast<void**>(reinterpret_cast<char*>(f.owner == 0u ? static_cast<void*>(model) : static_cast<void*>(data)) + f.offset);
+        for (uint32_t i = 0u; i < count; ++i) {
+            if (names[i] == nullptr) continue;
+            if (std::strcmp(names[i], f.name) == 0 || (f.reference_name != nullptr && std::strcmp(names[i], f.reference_name) == 0)) *member = pointers[i];
+        }
+        if (*member != nullptr) continue;
+        ++unset;
+        const size_t length = std::strlen(f.name);
+        if (missing != nullptr && written + length + 2u <= missing_bytes) {
+            if (written != 0u) missing[written++] = ',';
+            std::memcpy(missing + written, f.name, length + 1u);
+            written += length;
+        }
+    }
+    return unset;
+}
+int nuka_hip_model_view_set_count(nuka_phi_model_view* model, const char* name, uint32_t value) {
+    if (model == nullptr || name == nullptr) return -1;
+    auto* m = reinterpret_cast<nkh::ModelView*>(model);
+#define COUNT(member) if (std::strcmp(name, #member) == 0) { m->member = value; return 0; }
+    COUNT(links_per_env) COUNT(bodies_per_env) COUNT(dof) COUNT(max_dof) COUNT(max_depth) COUNT(contact_slots) COUNT(rows_per_env)
+    COUNT(contact_rows_per_env) COUNT(profile_count) COUNT(floating_root) COUNT(max_points_per_slot) COUNT(excluded_pair_count)
+    COUNT(sweep_passes) COUNT(pairable_count) COUNT(contact_dof_end) COUNT(joint_limit_rows) COUNT(joint_friction_rows) COUNT(joint_drive_rows)
+    COUNT(drive_mode) COUNT(any_mujoco) COUNT(contact_cone) COUNT(integrator)
+#undef COUNT
+    return -1;
+}
+
 const char* nuka_field_names(void) {
 #define X(name, ...) #name ","
     return NKH_MODEL_FIELDS(X) NKH_DATA_FIELDS(X) "";
