@@ -22,21 +22,35 @@ import __graft_entry__ as entry  # noqa: E402
 HBM_PEAK_GBPS = 8000.0
 DOMINANT_OP = "BlockDescentSolve"
 DOMINANT_KERNEL = "BlockDescentTileKernel"
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, scaled
-# by the same counters' reading of a plain copy of known size); keyed by (config, envs).  None where not measured.
-MEASURED_TRAFFIC_BYTES = {(3, 4096): 80.9e6, (2, 4096): 29.7e6, (3, 65536): 1244.4e6, (5, 8192): 495.5e6}   # profiles/counters_*.txt
-# What the same counter runs say limits the dominant kernel (not measured by this script): vector instructions a
-# launch issues and the share of a wave's resident cycles spent issuing them, at two waves a SIMD (one for the rope).
-MEASURED_ISSUE = {
-    (3, 4096): {"limiter": "valu_issue", "valu_instructions_per_env": 167000, "wave_cycles_issuing_valu": 0.47, "waves_per_simd": 2,
-                "scratch_bytes_per_lane": 0, "source": "profiles/counters_humanoid_4096.txt"},
-    (2, 4096): {"limiter": "valu_issue", "valu_instructions_per_env": 128000, "wave_cycles_issuing_valu": 0.50, "waves_per_simd": 2,
-                "scratch_bytes_per_lane": 0, "source": "profiles/counters_quadruped_4096.txt"},
-    (3, 65536): {"limiter": "valu_issue", "valu_instructions_per_env": 167000, "wave_cycles_issuing_valu": 0.47, "waves_per_simd": 2,
-                 "scratch_bytes_per_lane": 0, "source": "profiles/counters_humanoid_65536.txt"},
-    (5, 8192): {"limiter": "valu_issue", "valu_instructions_per_env": 287000, "wave_cycles_issuing_valu": 0.48, "waves_per_simd": 1,
-                "source": "profiles/counters_rope_8192.txt"},
-}
+SOLVER_SOURCES = ("nuka-physics_amd/csrc/ops_solver_kernel.h", "nuka-physics_amd/csrc/ops_solver.hip")
+
+
+def solver_source_digest():
+    """Names the dominant kernel's source as it stands: a counter summary is quoted only for the source it was taken on."""
+    import hashlib
+    digest = hashlib.sha256()
+    for relative in SOLVER_SOURCES:
+        with open(os.path.join(ROOT, relative), "rb") as handle:
+            digest.update(handle.read())
+    return digest.hexdigest()[:16]
+
+
+def profiled_figures(name, envs):
+    """What this script cannot measure itself - HBM bytes per launch of the dominant kernel and its instruction issue,
+    from rocprofv3 --pmc runs - read from the committed summary of this workload (its `figures:` line), with the file it
+    comes from and whether the kernel source is still the one the counters were taken on.  None without a summary."""
+    relative = os.path.join("profiles", f"counters_{name}_{envs}.txt")
+    try:
+        with open(os.path.join(ROOT, relative)) as handle:
+            lines = [line for line in handle if line.startswith("figures: ")]
+    except OSError:
+        return None
+    if not lines:
+        return None
+    figures = json.loads(lines[-1][len("figures: "):])
+    figures["from"] = relative
+    figures["taken_on_this_source"] = figures.get("solver_source_sha256") == solver_source_digest()
+    return figures
 
 
 def algorithmic_bytes(nl, nv, nc, floating):
@@ -155,7 +169,7 @@ def measure(nk, device, index, envs, steps, warmup, mode, cpu_budget_s, law="nat
     wall_ms = (time.perf_counter() - start) * 1e3 / steps
     event_ms = world.time_steps(steps, seeded) / steps            # device events on the world's own stream
 
-    nl, nv = world.link_count, world.dof
+    nl, nv, solver_width = world.link_count, world.dof, world.info.solver_width
     nc = world.info.contact_slots_per_env
     batch = {"failed_envs": int((world.download("env_status") != 0).sum())}
     if world.rows_per_env:
@@ -175,7 +189,13 @@ def measure(nk, device, index, envs, steps, warmup, mode, cpu_budget_s, law="nat
     else:
         kernel, kernel_ms, kernel_bytes = DOMINANT_KERNEL, dominant_ms, solver_bytes(nv, nc)
     achieved = kernel_bytes * E / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
+    survey_gbps = b_alg * E / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0   # the whole step's bytes over the kernel's time
     step_gbps = b_alg * E / (wall_ms * 1e-3) / 1e9
+    profiled = profiled_figures(cfg.name, E) if kernel == DOMINANT_KERNEL else None
+    traffic = profiled.pop("traffic_bytes_per_launch", None) if profiled else None
+    if profiled and not profiled["taken_on_this_source"]:
+        traffic = None                                            # counters of an older kernel say nothing of this one
+    blocks_per_cu = world.info.solver_blocks_per_cu
     live = ""
     if "contacts_mean" in batch:
         live = (f"; live contacts {batch['contacts_mean']:.1f} of {nc} slots per env, {batch['sweeps_mean']:.2f} sweeps used on "
@@ -184,14 +204,17 @@ def measure(nk, device, index, envs, steps, warmup, mode, cpu_budget_s, law="nat
     out = {
         "value": E * 1e3 / wall_ms, "ms_per_step": wall_ms, "steps": steps, "warmup": warmup,
         "config": {"workload": f"{cfg.name}: {nl} links, {nv} DoF, {nc} contact spheres, {E} envs, dt {cfg.dt:.6f}, "
-                               f"{cfg.vel_iters} block-descent sweeps{live}" + ("" if law == "native" else f"; MuJoCo contact law, {law} cone"),
+                               f"{cfg.vel_iters} block-descent sweeps{live}" + (f"; {cfg.note}" if cfg.note else "")
+                               + ("" if law == "native" else f"; MuJoCo contact law, {law} cone"),
                    "config_index": index, "envs": E,
                    "execution": mode, "event_ms_per_step": event_ms,
                    "each_step_from": "seeded batch (checkpoint restore inside the timed region)", **batch},
         "roofline": {"bound": "hbm", "kernel": kernel, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get((3 if index == 4 else index, E)),
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
                      "algorithmic_bytes_per_launch": kernel_bytes * E, "kernel_ms": kernel_ms,
-                     "profiled": MEASURED_ISSUE.get((3 if index == 4 else index, E))},
+                     "frac_survey": survey_gbps / HBM_PEAK_GBPS, "survey_bytes_per_launch": b_alg * E,
+                     "solver_width": solver_width, "blocks_per_cu": blocks_per_cu, "waves_per_simd": blocks_per_cu / 4.0,
+                     "profiled": profiled},
         "roofline_step": {"algorithmic_bytes_per_env_step": b_alg, "state_io_bytes_per_env_step": tier_a,
                           "achieved": step_gbps, "unit": "GB/s", "frac": step_gbps / HBM_PEAK_GBPS},
         "per_op_ms": {k: round(v, 4) for k, v in per_op.items() if v >= 0.001},

@@ -455,6 +455,9 @@ typedef struct nuka_world_info_t {
     /* coordinates the sweeps of the contact solve work on: dof, or fewer where no contact of the world can reach the
      * later coordinates and the solve eliminates those once per step */
     uint32_t solver_width;
+    /* one-wavefront blocks of the contact solve's full-capacity launch that a compute unit (four SIMDs) holds at once,
+     * by the runtime's occupancy query for that kernel and its LDS; 0 for a world without a contact solve */
+    uint32_t solver_blocks_per_cu;
 } nuka_world_info_t;
 nuka_result_t nuka_world_get_info(nuka_world_handle world, nuka_world_info_t* out);
 

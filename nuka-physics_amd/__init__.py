@@ -27,7 +27,7 @@ class NukaError(RuntimeError):
 
 class WorldInfoC(C.Structure):
     _fields_ = [(n, C.c_uint32) for n in ("env_count", "links_per_env", "bodies_per_env", "dof", "max_dof",
-                                          "contact_slots_per_env", "rows_per_env", "op_count", "solver_width")]
+                                          "contact_slots_per_env", "rows_per_env", "op_count", "solver_width", "solver_blocks_per_cu")]
 
 
 class SceneInfoC(C.Structure):

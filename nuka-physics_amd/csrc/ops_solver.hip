@@ -126,6 +126,30 @@ static bool ContactHeadsOnly(const ModelView& m, uint32_t staged) {
     const uint32_t joint_heads = m.joint_limit_rows + m.joint_friction_rows + m.joint_drive_rows;
     return joint_heads == 0u && staged <= uint32_t(solver::kWave) && !(m.any_mujoco != 0u && m.contact_cone == 1u);
 }
+static SolverKernel KernelOfWidth(const ModelView& m, bool contacts_only, uint32_t width) {
+    if (width != m.dof)
+        for (const ReducedKernel& reduced : kReducedKernels)
+            if (reduced.width == solver::PaddedWidth(m.dof) && reduced.reduced == width) return reduced.kernel;
+    return kSolverKernels[contacts_only ? 1 : 0][solver::PaddedWidth(m.dof) / 4u - 1u];
+}
+// Blocks (one wavefront, one environment each) of a world's full-capacity solve launch that a compute unit holds at
+// once, as the runtime's occupancy query answers for the kernel and the LDS the launch asks for; 0 without a solve.
+uint32_t SolverBlocksPerUnit(const ModelView& m) {
+    if (m.rows_per_env == 0u || m.dof == 0u) return 0u;
+    const uint32_t staged = SolverHeadCapacity(m, std::max(m.contact_slots, 1u), 150u * 1024u);
+    if (staged == 0u) return 0u;
+    const uint32_t joint_heads = m.joint_limit_rows + m.joint_friction_rows + m.joint_drive_rows;
+    const bool contacts_only = ContactHeadsOnly(m, staged);
+    const uint32_t width = SolverWorkingWidth(m, contacts_only);
+    const size_t lds = size_t{solver::ReducedSolverLdsFloats(m.dof, width, staged + joint_heads, staged)} * sizeof(float);
+    int blocks = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, reinterpret_cast<const void*>(KernelOfWidth(m, contacts_only, width)),
+                                                     solver::kWave, lds) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0u;
+    }
+    return uint32_t(std::max(blocks, 0));
+}
 uint32_t SolverMassFactorFloats(const ModelView& m) {
     if (m.rows_per_env == 0u || m.dof == 0u) return 0u;
     const uint32_t width = SolverSweepWidth(m);
@@ -160,10 +184,7 @@ Status OpBlockDescentSolve(const ModelView& m, const DataView& d, const void* pa
     // lets more blocks share a compute unit, environments with few contact points go to a launch of that capacity:
     // up to three such launches, for eight, four and two blocks a unit, before the full one.  Each launch takes the
     // environments whose contact points fall in its range; an environment's results do not depend on its launch.
-    SolverKernel kernel = kSolverKernels[contacts_only ? 1 : 0][solver::PaddedWidth(m.dof) / 4u - 1u];
-    if (width != m.dof)
-        for (const ReducedKernel& reduced : kReducedKernels)
-            if (reduced.width == solver::PaddedWidth(m.dof) && reduced.reduced == width) kernel = reduced.kernel;
+    const SolverKernel kernel = KernelOfWidth(m, contacts_only, width);
     hipLaunchKernelGGL(OrderTilesKernel, dim3(1), dim3(1024), 0, stream, d, p->env_count);
     uint32_t first_points = 0u;
     // (a launch takes its environments by their contact points, one head a point: not under the pyramidal cone, whose
