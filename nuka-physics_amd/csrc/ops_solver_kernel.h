@@ -37,6 +37,8 @@ constexpr float kPenaltyConditionCap = 1.0e2f;   // block_descent.cu:71
 // Unit heads a coordinate can list for itself (lower limit, upper limit, friction, drive, and room to spare); a block
 // with more on one coordinate walks its unit heads serially instead.
 constexpr uint32_t kUnitSlots = 6u;
+// contributing heads from which a wide block takes the heads' curvature by way of the links (add_heads_through_links)
+constexpr uint32_t kLinkHeads = 4u;
 
 // Phase timers for development builds (-DNKH_SOLVER_PROFILE): cycles per phase and event counts per environment,
 // written over the environment's solver_penalty words at the end of the solve.
@@ -279,6 +281,17 @@ struct Tile {
     uint32_t individual_end;  // one past the last head whose inertial response is computed for itself
     float momentum, residual;
     bool failed;
+    // what add_heads_through_links needs (wide blocks only)
+    bool through_links;       // every staged head acts on the block through one link: the heads' curvature may go by way of the links
+    float* axes;              // 64 x 12: a coordinate's motion axis about `pivot`, then the contact stiffness it carries times that axis
+    uint32_t path_low, path_high;     // lane = coordinate: the coordinates on the way from its link to the root, itself included
+    uint32_t under_low, under_high;   // the coordinates whose way to the root passes through lane's
+    V3 pivot;                 // the point the axes and the heads' wrenches are taken about: the root link's origin
+    const float* rows;        // the environment-major row records, row points and row links of device memory
+    const float* row_point_a, *row_point_b;
+    const uint32_t* row_link_a, *row_link_b;
+    const uint64_t* link_paths;
+    uint32_t first_link;      // index of the environment's first link
 #ifdef NKH_SOLVER_PROFILE
     mutable long long prof[26];
     mutable uint32_t prof_count[4];
@@ -902,6 +915,119 @@ __device__ __forceinline__ float uniform_lane_value(float v, uint32_t lane) {   
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), int(lane)));
 }
 
+// One head's part of the force only: g += J^T f for lane's coordinate, with the rounding scale of that sum.
+template <int N>
+__device__ __forceinline__ void add_head_force(const Tile& c, uint32_t first_row, bool coordinate, const float (&f)[3], const float (&noise)[3],
+                                               uint32_t axes, TileSum& g, float& scale) {
+    const float* j0r = c.jac + first_row * uint32_t(N);
+    const float j0 = coordinate ? j0r[c.lane] : 0.0f;
+    tile_add_product(g, j0, f[0]);
+    scale += fabsf(j0) * noise[0];
+    if (axes == 1u) return;
+    const float j1 = coordinate ? j0r[N + c.lane] : 0.0f, j2 = coordinate ? j0r[2 * N + c.lane] : 0.0f;
+    tile_add_product(g, j1, f[1]);
+    tile_add_product(g, j2, f[2]);
+    scale += fabsf(j1) * noise[1] + fabsf(j2) * noise[2];
+}
+
+// The heads' curvature sum_h J_h^T C_h J_h by way of the links, for blocks whose staged heads each act through one link.
+// A row of such a head is a wrench w = [(p - o) x n; n] about a point o, met by every coordinate j on the way from the
+// head's link to the root with its motion axis s_j = [a_j; (r_j - o) x a_j] (a sliding coordinate: [0; a_j]):
+// J_j = s_j . w, the entry the row assembly wrote (assemble_rows.cu:122-169).  The head's term in H_ij is therefore
+// s_i^T (W C W^T) s_j when both i and j lie on that way, else zero; and of two coordinates that share any head one lies
+// on the other's way to the root.  With K_i the sum of W C W^T over the heads whose way to the root holds i - the
+// contact stiffness coordinate i carries, as a composite inertia is the inertia it carries -
+//     H_ij += (K_i s_i) . s_j   for j on i's way to the root,      (K_j s_j) . s_i   for i on j's,
+// which takes 21 words a head and 12 a column where the plain sum over heads takes 3 N words a head.  The two forms
+// of one entry multiply and add the same numbers in the same order: the rows stay each other's transposes to the bit.
+// lane = head on the way in (mc: its curvature, `mine`: it contributes), lane = coordinate from the sums on.
+template <int N>
+__device__ __forceinline__ void add_heads_through_links(const Tile& c, bool mine, const float (&mc)[6], float (&hrow)[N]) {
+    const uint32_t lane = c.lane;
+    float k[21];
+#pragma unroll
+    for (int e = 0; e < 21; ++e) k[e] = 0.0f;
+    uint32_t way_low = 0u, way_high = 0u;
+    if (mine) {
+        const uint32_t slot = c.U(hSlot, lane), stride = c.U(hStride, lane), axes = c.U(hAxes, lane);
+        const bool second = c.U(hSourceA, lane) == kInvalid;   // the side that moves is the row's second
+        const uint64_t way = c.link_paths[(second ? c.row_link_b : c.row_link_a)[slot] - c.first_link];
+        way_low = uint32_t(way); way_high = uint32_t(way >> 32u);
+        float w[3][6];
+#pragma unroll
+        for (uint32_t a = 0u; a < 3u; ++a) {
+#pragma unroll
+            for (int t = 0; t < 6; ++t) w[a][t] = 0.0f;
+            if (a != 0u && axes == 1u) continue;
+            const size_t rs = size_t{slot} + a * stride;
+            const float* row = c.rows + rs * kRowWords + 12u;          // the first side's direction; the second side's is its negative,
+            const float* at = (second ? c.row_point_b : c.row_point_a) + 3u * rs;   // and W C W^T does not see the sign
+            const V3 n{row[0], row[1], row[2]};
+            const V3 arm = sub3(V3{at[0], at[1], at[2]}, c.pivot);
+            const V3 moment = cross3(arm, n);
+            w[a][0] = moment.x; w[a][1] = moment.y; w[a][2] = moment.z; w[a][3] = n.x; w[a][4] = n.y; w[a][5] = n.z;
+        }
+        const float cxx = mc[0], cyy = mc[1], czz = mc[2], cxy = mc[3], cxz = mc[4], cyz = mc[5];
+        float u[3][6];
+#pragma unroll
+        for (int t = 0; t < 6; ++t) {
+            u[0][t] = (cxx * w[0][t] + cxy * w[1][t]) + cxz * w[2][t];
+            u[1][t] = (cxy * w[0][t] + cyy * w[1][t]) + cyz * w[2][t];
+            u[2][t] = (cxz * w[0][t] + cyz * w[1][t]) + czz * w[2][t];
+        }
+        int e = 0;
+#pragma unroll
+        for (int r = 0; r < 6; ++r) {
+#pragma unroll
+            for (int t = r; t < 6; ++t) k[e++] = (w[0][r] * u[0][t] + w[1][r] * u[1][t]) + w[2][r] * u[2][t];
+        }
+    }
+    // lane = coordinate: the stiffness of every head whose way to the root passes through it
+    float carried[21];
+#pragma unroll
+    for (int e = 0; e < 21; ++e) carried[e] = 0.0f;
+    for (uint64_t rest = __ballot(mine); rest != 0ull; rest &= rest - 1ull) {
+        const int h = __builtin_ctzll(rest);
+        const uint64_t way = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(way_high), h))) << 32u) |
+                             uint64_t(uint32_t(__builtin_amdgcn_readlane(int(way_low), h)));
+        const bool through = ((way >> lane) & 1ull) != 0ull;
+#pragma unroll
+        for (int e = 0; e < 21; ++e) {
+            const float term = uniform_lane_value(k[e], uint32_t(h));
+            if (through) carried[e] += term;
+        }
+    }
+    float4* table = reinterpret_cast<float4*>(c.axes);
+    float s[6], y[6];
+    {
+        const float4 a = table[3u * lane], b = table[3u * lane + 1u];
+        s[0] = a.x; s[1] = a.y; s[2] = a.z; s[3] = a.w; s[4] = b.x; s[5] = b.y;
+        // y = K s, K symmetric with its upper triangle in `carried`, rows first
+        auto entry = [&](int r, int t) { return r <= t ? carried[r * 6 - r * (r - 1) / 2 + (t - r)] : carried[t * 6 - t * (t - 1) / 2 + (r - t)]; };
+#pragma unroll
+        for (int r = 0; r < 6; ++r) {
+            float sum = entry(r, 0) * s[0];
+#pragma unroll
+            for (int t = 1; t < 6; ++t) sum = fmaf(entry(r, t), s[t], sum);
+            y[r] = sum;
+        }
+        table[3u * lane + 1u] = float4{b.x, b.y, y[0], y[1]};
+        table[3u * lane + 2u] = float4{y[2], y[3], y[4], y[5]};
+    }
+    __syncthreads();
+    const uint64_t path = (uint64_t(c.path_high) << 32u) | uint64_t(c.path_low), under = (uint64_t(c.under_high) << 32u) | uint64_t(c.under_low);
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        const float4 a = table[3 * j], b = table[3 * j + 1], d = table[3 * j + 2];
+        // (K_i s_i) . s_j and (K_j s_j) . s_i, each the stiffness-times-axis of the coordinate further from the root first
+        const float mine_first = fmaf(y[5], b.y, fmaf(y[4], b.x, fmaf(y[3], a.w, fmaf(y[2], a.z, fmaf(y[1], a.y, y[0] * a.x)))));
+        const float other_first = fmaf(d.w, s[5], fmaf(d.z, s[4], fmaf(d.y, s[3], fmaf(d.x, s[2], fmaf(b.w, s[1], b.z * s[0])))));
+        const bool on_my_way = ((path >> j) & 1ull) != 0ull, through_me = ((under >> j) & 1ull) != 0ull;
+        hrow[j] += on_my_way ? mine_first : (through_me ? other_first : 0.0f);
+    }
+    __syncthreads();
+}
+
 // AssembleTileBlock (:1507-1618): lane i assembles row i of H = M + sum J^T C J in `hrow` and its force g_i.  The
 // first 64 heads evaluate their response one per lane and hand it to the row lanes as scalar lane reads; heads beyond
 // 64 pass theirs through the head fields.
@@ -1006,6 +1132,18 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
         }
     }
     if (paired) {
+    } else if (N > kTwoWaveWidth && c.through_links && __popcll(__ballot(mine)) >= int(kLinkHeads)) {
+        // enough heads that their curvature is cheaper by way of the links; the force takes the staged rows as ever
+        const uint32_t my_first = lane < c.heads ? c.U(hRow, lane) : 0u;
+        for (uint64_t rest = __ballot(mine); rest != 0ull; rest &= rest - 1ull) {
+            const uint32_t h = uint32_t(__builtin_ctzll(rest));
+            float f[3], noise[3];
+#pragma unroll
+            for (int k = 0; k < 3; ++k) { f[k] = uniform_lane_value(mf[k], h); noise[k] = uniform_lane_value(mn[k], h); }
+            add_head_force<N>(c, uint32_t(__builtin_amdgcn_readlane(int(my_first), int(h))), coordinate, f, noise,
+                              uint32_t(__builtin_amdgcn_readlane(int(my_axes), int(h))), g, scale);
+        }
+        add_heads_through_links<N>(c, mine, mc, hrow);
     } else if (!c.units) {   // staged heads only: plain head order
         for (uint64_t rest = __ballot(mine); rest != 0ull; rest &= rest - 1ull) {
             const uint32_t h = uint32_t(__builtin_ctzll(rest));
@@ -1737,6 +1875,8 @@ __host__ __device__ inline uint32_t ReductionScratchFloats(uint32_t full, uint32
     const uint32_t N = PaddedWidth(full);
     return reduced >= full ? 0u : 2u * (N - reduced) * N;   // doubles
 }
+// the coordinates' motion axes of a wide block (Tile::axes), twelve words a coordinate
+__host__ __device__ inline uint32_t LinkAxisFloats(uint32_t n) { return PaddedWidth(n) > uint32_t(kTwoWaveWidth) ? 12u * uint32_t(kWave) : 0u; }
 __host__ __device__ inline uint32_t HeadFieldFloats(uint32_t cap, uint32_t narrow) {
     return (kWideStride * cap + kNarrowStride * (narrow + 1u) + 3u) & ~3u;
 }
@@ -1745,7 +1885,8 @@ __host__ __device__ inline uint32_t SolverLdsFloats(uint32_t n, uint32_t cap, ui
     const uint32_t N = PaddedWidth(n);
     // the per-coordinate unit lists exist only when some head beyond the staged ones can be listed; without joint rows
     // the block keeps the footprint that lets eight of them share a compute unit's LDS
-    return FactorRegionFloats(n) + 3u * staged * N + HeadFieldFloats(cap, staged) + 256u + (cap > staged ? kUnitSlots * uint32_t(kWave) : 0u);
+    return FactorRegionFloats(n) + 3u * staged * N + HeadFieldFloats(cap, staged) + 256u + (cap > staged ? kUnitSlots * uint32_t(kWave) : 0u) +
+           LinkAxisFloats(n);
 }
 __host__ __device__ inline uint32_t ReducedSolverLdsFloats(uint32_t full, uint32_t reduced, uint32_t cap, uint32_t staged) {
     const uint32_t solve = SolverLdsFloats(reduced, cap, staged), scratch = ReductionScratchFloats(full, reduced);
@@ -1900,6 +2041,12 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     if (lane < kNarrowFields) c.fields[kWideStride * cap + staged_cap * kNarrowStride + lane] = 0.0f;   // what a narrow field reads beyond its heads
     c.unit_list = reinterpret_cast<uint32_t*>(c.vec + 256);
     c.unit_lists = true; c.unit_count = 0u; c.staged_end = 0u; c.individual_end = 0u;
+    c.through_links = false;
+    c.axes = c.vec + 256 + (cap > staged_cap ? kUnitSlots * uint32_t(kWave) : 0u);
+    c.path_low = c.path_high = c.under_low = c.under_high = 0u;
+    c.rows = d.urows; c.row_point_a = d.row_cj_point; c.row_point_b = d.row_cj_point_b; c.row_link_a = d.row_cj_link; c.row_link_b = d.row_cj_link_b;
+    c.link_paths = m.link_dof_mask; c.first_link = env * nl;
+    c.pivot = V3{0.0f, 0.0f, 0.0f};
     const bool coordinate = lane < n;
     const float* urows = d.urows;
     float* lambda_env = d.lambda + size_t{env} * R;
@@ -2030,6 +2177,59 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         PROF_END(c, 23);
     }
     __syncthreads();
+    if constexpr (W > kTwoWaveWidth && kContactsOnly) {
+        // The coordinates' motion axes about the root link's origin, for add_heads_through_links: a hinge or an angular
+        // coordinate of a floating root turns about its axis through the joint's origin, a sliding one moves along it
+        // (the columns the row assembly wrote, assemble_rows.cu:122-169, before the dot with a row's direction).
+        const float* root = d.link_pose + lbase * 7u;
+        c.pivot = V3{root[0], root[1], root[2]};
+        float axis[6] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        uint64_t path = 0ull;
+        bool plain = true;
+        if (coordinate) {
+            V3 along, at;
+            bool turning;
+            if (my_component == kInvalid) {
+                const Xf pose = load_xf(d.link_pose + (lbase + my_link) * 7u);
+                along = rotate_normalized(pose.r, V3{m.joint_axis[3u * my_link], m.joint_axis[3u * my_link + 1u], m.joint_axis[3u * my_link + 2u]});
+                at = pose.p;
+                turning = m.joint_type[my_link] != kPrismatic;
+            } else {
+                const Xf base = load_xf(d.base_pose + size_t{env} * 7u);
+                const uint32_t k = my_component % 3u;
+                along = rotate_normalized(base.r, V3{k == 0u ? 1.0f : 0.0f, k == 1u ? 1.0f : 0.0f, k == 2u ? 1.0f : 0.0f});
+                at = base.p;
+                turning = my_component < 3u;
+                plain = my_component < 6u;
+            }
+            if (turning) {
+                const V3 arm = cross3(sub3(at, c.pivot), along);
+                axis[0] = along.x; axis[1] = along.y; axis[2] = along.z; axis[3] = arm.x; axis[4] = arm.y; axis[5] = arm.z;
+            } else {
+                axis[3] = along.x; axis[4] = along.y; axis[5] = along.z;
+            }
+            path = m.link_dof_mask[my_link];
+        }
+        float4* table = reinterpret_cast<float4*>(c.axes);
+        table[3u * lane] = float4{axis[0], axis[1], axis[2], axis[3]};
+        table[3u * lane + 1u] = float4{axis[4], axis[5], 0.0f, 0.0f};
+        table[3u * lane + 2u] = float4{0.0f, 0.0f, 0.0f, 0.0f};
+        c.path_low = uint32_t(path); c.path_high = uint32_t(path >> 32u);
+        uint64_t under = 0ull;
+        for (uint32_t i = 0u; i < n; ++i) {
+            const uint64_t holders = __ballot(((path >> i) & 1ull) != 0ull);   // the coordinates whose way to the root holds i
+            if (lane == i) under = holders;
+        }
+        c.under_low = uint32_t(under); c.under_high = uint32_t(under >> 32u);
+        // every staged head with exactly one side that moves
+        bool one_link = true;
+        if (lane < heads) {
+            const bool side_a = c.U(hSourceA, lane) != kInvalid, side_b = c.U(hSourceB, lane) != kInvalid;
+            one_link = !(side_a && side_b) && (!(side_a || side_b) || c.U(hRow, lane) != kInvalid);
+        }
+        c.through_links = heads <= uint32_t(kWave) && !c.units && __all(plain && one_link);
+        __syncthreads();
+    }
     // CopyTileRows (:836-869): the staged heads' rows, their loads in flight together
 
     bool stray = false;   // a reduced block: an entry past the block's coordinates
