@@ -915,19 +915,31 @@ __device__ __forceinline__ float uniform_lane_value(float v, uint32_t lane) {   
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), int(lane)));
 }
 
-// One head's part of the force only: g += J^T f for lane's coordinate, with the rounding scale of that sum.
+// The heads' part of the force only: g += J^T f for lane's coordinate, with the rounding scale of that sum.  A staged
+// head has three rows in LDS whatever its axes (those it does not have hold zeros, as its response does), and the
+// padded columns hold zeros: every head reads its three words without a condition, the next head's ahead of this
+// one's arithmetic.  lane = head on the way in (mf, mn, my_first), lane = coordinate for the sums.
 template <int N>
-__device__ __forceinline__ void add_head_force(const Tile& c, uint32_t first_row, bool coordinate, const float (&f)[3], const float (&noise)[3],
-                                               uint32_t axes, TileSum& g, float& scale) {
-    const float* j0r = c.jac + first_row * uint32_t(N);
-    const float j0 = coordinate ? j0r[c.lane] : 0.0f;
-    tile_add_product(g, j0, f[0]);
-    scale += fabsf(j0) * noise[0];
-    if (axes == 1u) return;
-    const float j1 = coordinate ? j0r[N + c.lane] : 0.0f, j2 = coordinate ? j0r[2 * N + c.lane] : 0.0f;
-    tile_add_product(g, j1, f[1]);
-    tile_add_product(g, j2, f[2]);
-    scale += fabsf(j1) * noise[1] + fabsf(j2) * noise[2];
+__device__ __forceinline__ void add_heads_force(const Tile& c, uint64_t heads, const float (&mf)[3], const float (&mn)[3], uint32_t my_first,
+                                                TileSum& g, float& scale) {
+    const uint32_t column = c.lane < uint32_t(N) ? c.lane : uint32_t(N - 1);
+    auto rows_of = [&](uint32_t h, float (&j)[3]) {
+        const float* at = c.jac + uint32_t(__builtin_amdgcn_readlane(int(my_first), int(h))) * uint32_t(N) + column;
+        j[0] = at[0]; j[1] = at[N]; j[2] = at[2 * N];
+    };
+    float next[3] = {0.0f, 0.0f, 0.0f};
+    if (heads != 0ull) rows_of(uint32_t(__builtin_ctzll(heads)), next);
+    while (heads != 0ull) {
+        const uint32_t h = uint32_t(__builtin_ctzll(heads));
+        heads &= heads - 1ull;
+        const float j[3] = {next[0], next[1], next[2]};
+        if (heads != 0ull) rows_of(uint32_t(__builtin_ctzll(heads)), next);
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            tile_add_product(g, j[k], uniform_lane_value(mf[k], h));
+            scale += fabsf(j[k]) * uniform_lane_value(mn[k], h);
+        }
+    }
 }
 
 // The heads' curvature sum_h J_h^T C_h J_h by way of the links, for blocks whose staged heads each act through one link.
@@ -990,12 +1002,10 @@ __device__ __forceinline__ void add_heads_through_links(const Tile& c, bool mine
         const int h = __builtin_ctzll(rest);
         const uint64_t way = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(way_high), h))) << 32u) |
                              uint64_t(uint32_t(__builtin_amdgcn_readlane(int(way_low), h)));
-        const bool through = ((way >> lane) & 1ull) != 0ull;
+        // one multiply-add an entry with a weight of one or zero: a conditional sum compiles to an add and two copies
+        const float through = ((way >> lane) & 1ull) != 0ull ? 1.0f : 0.0f;
 #pragma unroll
-        for (int e = 0; e < 21; ++e) {
-            const float term = uniform_lane_value(k[e], uint32_t(h));
-            if (through) carried[e] += term;
-        }
+        for (int e = 0; e < 21; ++e) carried[e] = fmaf(through, uniform_lane_value(k[e], uint32_t(h)), carried[e]);
     }
     float4* table = reinterpret_cast<float4*>(c.axes);
     float s[6], y[6];
@@ -1134,15 +1144,7 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
     if (paired) {
     } else if (N > kTwoWaveWidth && c.through_links && __popcll(__ballot(mine)) >= int(kLinkHeads)) {
         // enough heads that their curvature is cheaper by way of the links; the force takes the staged rows as ever
-        const uint32_t my_first = lane < c.heads ? c.U(hRow, lane) : 0u;
-        for (uint64_t rest = __ballot(mine); rest != 0ull; rest &= rest - 1ull) {
-            const uint32_t h = uint32_t(__builtin_ctzll(rest));
-            float f[3], noise[3];
-#pragma unroll
-            for (int k = 0; k < 3; ++k) { f[k] = uniform_lane_value(mf[k], h); noise[k] = uniform_lane_value(mn[k], h); }
-            add_head_force<N>(c, uint32_t(__builtin_amdgcn_readlane(int(my_first), int(h))), coordinate, f, noise,
-                              uint32_t(__builtin_amdgcn_readlane(int(my_axes), int(h))), g, scale);
-        }
+        add_heads_force<N>(c, __ballot(mine), mf, mn, lane < c.heads ? c.U(hRow, lane) : 0u, g, scale);
         add_heads_through_links<N>(c, mine, mc, hrow);
     } else if (!c.units) {   // staged heads only: plain head order
         for (uint64_t rest = __ballot(mine); rest != 0ull; rest &= rest - 1ull) {
