@@ -73,6 +73,10 @@ struct ModelView {
     uint32_t sweep_passes;     // passes of the dynamics' tree sweeps (sweep_links)
     uint32_t pairable_count;   // collidable rows that can pass the shape filter with some partner (pairable_rows, ascending)
     uint32_t contact_dof_end;  // one past the last coordinate on the path to the root of any link that carries a shape: no contact row reaches a later one
+    // 1: every contact row acts on the articulation through one link (no admitted pair joins two of its links' shapes) and
+    // every coordinate is a hinge, a slider or one of a floating root's six: a contact row's entries then follow from the
+    // row's wrench and the coordinates' motion axes, and the solve of a wide block need not keep the rows themselves
+    uint32_t rows_from_links;
     // joint row slots after the contact rows: 2 per link, 1 per link, 1 per link, or 0 (scene/cook/cook_to_model.cpp:706-719)
     uint32_t joint_limit_rows, joint_friction_rows, joint_drive_rows, drive_mode;
     // the MuJoCo contact law: some profile is MuJoCo-sourced; the cone of its contacts (0 pyramidal, 1 elliptic) and impratio

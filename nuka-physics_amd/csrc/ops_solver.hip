@@ -141,7 +141,8 @@ uint32_t SolverBlocksPerUnit(const ModelView& m) {
     const uint32_t joint_heads = m.joint_limit_rows + m.joint_friction_rows + m.joint_drive_rows;
     const bool contacts_only = ContactHeadsOnly(m, staged);
     const uint32_t width = SolverWorkingWidth(m, contacts_only);
-    const size_t lds = size_t{solver::ReducedSolverLdsFloats(m.dof, width, staged + joint_heads, staged)} * sizeof(float);
+    const size_t lds = size_t{solver::ReducedSolverLdsFloats(m.dof, width, staged + joint_heads, staged,
+                                                             solver::RowsFromLinks(width, contacts_only, m.rows_from_links))} * sizeof(float);
     int blocks = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, reinterpret_cast<const void*>(KernelOfWidth(m, contacts_only, width)),
                                                      solver::kWave, lds) != hipSuccess) {
@@ -174,7 +175,8 @@ Status OpBlockDescentSolve(const ModelView& m, const DataView& d, const void* pa
     const bool contacts_only = ContactHeadsOnly(m, staged);
     const uint32_t width = SolverWorkingWidth(m, contacts_only);
     const auto lds_bytes = [&](uint32_t contact_heads) {
-        return size_t{solver::ReducedSolverLdsFloats(m.dof, width, contact_heads + joint_heads, contact_heads)} * sizeof(float);
+        return size_t{solver::ReducedSolverLdsFloats(m.dof, width, contact_heads + joint_heads, contact_heads,
+                                                     solver::RowsFromLinks(width, contacts_only, m.rows_from_links))} * sizeof(float);
     };
     // widths past kTwoWaveWidth run one wave a SIMD: four blocks a compute unit at most, whatever their LDS
     const size_t most_blocks = solver::PaddedWidth(width) > uint32_t(solver::kTwoWaveWidth) ? 4u : 8u;

@@ -39,6 +39,8 @@ constexpr float kPenaltyConditionCap = 1.0e2f;   // block_descent.cu:71
 constexpr uint32_t kUnitSlots = 6u;
 // contributing heads from which a wide block takes the heads' curvature by way of the links (add_heads_through_links)
 constexpr uint32_t kLinkHeads = 4u;
+// words a head of Tile::wrench: 3 x 6 wrench components, the two words of its way to the root, one more for an odd stride
+constexpr uint32_t kWrenchStride = 21u;
 
 // Phase timers for development builds (-DNKH_SOLVER_PROFILE): cycles per phase and event counts per environment,
 // written over the environment's solver_penalty words at the end of the solve.
@@ -282,6 +284,8 @@ struct Tile {
     float momentum, residual;
     bool failed;
     // what add_heads_through_links needs (wide blocks only)
+    bool from_links;          // the block keeps no contact rows: their entries follow from `wrench` and `axes` wherever a row is read
+    float* wrench;            // cap x kWrenchStride: a head's three rows as wrenches about `pivot`, then its way to the root (two words)
     bool through_links;       // every staged head acts on the block through one link: the heads' curvature may go by way of the links
     float* axes;              // 64 x 12: a coordinate's motion axis about `pivot`, then the contact stiffness it carries times that axis
     uint32_t path_low, path_high;     // lane = coordinate: the coordinates on the way from its link to the root, itself included
@@ -942,6 +946,86 @@ __device__ __forceinline__ void add_heads_force(const Tile& c, uint64_t heads, c
     }
 }
 
+// Blocks that keep no contact rows (Tile::from_links).  Entry j of a head's row is s_j . w where j lies on the head's
+// way to the root, s_j the coordinate's motion axis (Tile::axes) and w the row's wrench (Tile::wrench); elsewhere zero.
+// lane = head: the motion of the head's link, sum over the coordinates j on its way of s_j x_j, for a vector x in LDS.
+template <int N>
+__device__ __forceinline__ void link_motion(const Tile& c, uint64_t way, const float* x, float (&motion)[6]) {
+    const float4* table = reinterpret_cast<const float4*>(c.axes);
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+#pragma unroll
+    for (int k = 0; k < 6; ++k) motion[k] = 0.0f;
+    const uint32_t low = uint32_t(way), high = uint32_t(way >> 32u);
+#pragma unroll
+    for (int q = 0; q < N / 4; ++q) {
+        const float4 xq = x4[q];
+        const float xs[4] = {xq.x, xq.y, xq.z, xq.w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int j = 4 * q + t;
+            const float4 a = table[3 * j], b = table[3 * j + 1];
+            const float on = ((j < 32 ? low >> j : high >> (j - 32)) & 1u) != 0u ? xs[t] : 0.0f;
+            motion[0] = fmaf(a.x, on, motion[0]); motion[1] = fmaf(a.y, on, motion[1]); motion[2] = fmaf(a.z, on, motion[2]);
+            motion[3] = fmaf(a.w, on, motion[3]); motion[4] = fmaf(b.x, on, motion[4]); motion[5] = fmaf(b.y, on, motion[5]);
+        }
+    }
+}
+// lane = head: row `axis` of head h times the vector whose link motion is `motion`
+__device__ __forceinline__ float wrench_dot(const Tile& c, uint32_t h, uint32_t axis, const float (&motion)[6]) {
+    const float* w = c.wrench + h * kWrenchStride + 6u * axis;
+    return fmaf(w[5], motion[5], fmaf(w[4], motion[4], fmaf(w[3], motion[3], fmaf(w[2], motion[2], fmaf(w[1], motion[1], w[0] * motion[0])))));
+}
+__device__ __forceinline__ uint64_t way_of(const Tile& c, uint32_t h) {
+    const uint32_t* w = reinterpret_cast<const uint32_t*>(c.wrench + h * kWrenchStride + 18u);
+    return (uint64_t(w[1]) << 32u) | uint64_t(w[0]);
+}
+// lane = coordinate: sum over the heads `heads` (a uniform mask of the first 64) of J^T x, x one value an axis held by
+// lane = head, in double: the heads' wrenches weighted by x summed over the heads whose way holds the coordinate, then
+// taken against the coordinate's motion axis.  With `weights` (the magnitudes that go with x) also the rounding scale
+// of that sum, an upper bound: sum |s_j| . sum |w| weights.
+template <bool kScale>
+__device__ __forceinline__ double rows_transposed_times(const Tile& c, uint64_t heads, const float (&x)[3], const float (&weights)[3], float* scale) {
+    const uint32_t lane = c.lane;
+    float sum[6] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f}, bound[6] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    uint32_t way_low = 0u, way_high = 0u;
+    if (lane < c.heads && ((heads >> lane) & 1ull) != 0ull) {
+        const float* w = c.wrench + lane * kWrenchStride;
+#pragma unroll
+        for (int k = 0; k < 6; ++k) {
+            sum[k] = (w[k] * x[0] + w[6 + k] * x[1]) + w[12 + k] * x[2];
+            if constexpr (kScale) bound[k] = (fabsf(w[k]) * weights[0] + fabsf(w[6 + k]) * weights[1]) + fabsf(w[12 + k]) * weights[2];
+        }
+        const uint64_t way = way_of(c, lane);
+        way_low = uint32_t(way); way_high = uint32_t(way >> 32u);
+    }
+    double carried[6] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
+    float carried_bound[6] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    for (uint64_t rest = heads; rest != 0ull; rest &= rest - 1ull) {
+        const int h = __builtin_ctzll(rest);
+        const uint64_t way = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(way_high), h))) << 32u) |
+                             uint64_t(uint32_t(__builtin_amdgcn_readlane(int(way_low), h)));
+        const float through = ((way >> lane) & 1ull) != 0ull ? 1.0f : 0.0f;
+#pragma unroll
+        for (int k = 0; k < 6; ++k) {
+            carried[k] = fma(double(through), double(uniform_lane_value(sum[k], uint32_t(h))), carried[k]);
+            if constexpr (kScale) carried_bound[k] = fmaf(through, uniform_lane_value(bound[k], uint32_t(h)), carried_bound[k]);
+        }
+    }
+    const float4* table = reinterpret_cast<const float4*>(c.axes);
+    const float4 a = table[3u * lane], b = table[3u * lane + 1u];
+    const float s[6] = {a.x, a.y, a.z, a.w, b.x, b.y};
+    double total = 0.0;
+#pragma unroll
+    for (int k = 0; k < 6; ++k) total = fma(double(s[k]), carried[k], total);
+    if constexpr (kScale) {
+        float magnitude = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 6; ++k) magnitude = fmaf(fabsf(s[k]), carried_bound[k], magnitude);
+        *scale += magnitude;
+    }
+    return total;
+}
+
 // The heads' curvature sum_h J_h^T C_h J_h by way of the links, for blocks whose staged heads each act through one link.
 // A row of such a head is a wrench w = [(p - o) x n; n] about a point o, met by every coordinate j on the way from the
 // head's link to the root with its motion axis s_j = [a_j; (r_j - o) x a_j] (a sliding coordinate: [0; a_j]):
@@ -963,11 +1047,16 @@ __device__ __forceinline__ void add_heads_through_links(const Tile& c, bool mine
     if (mine) {
         const uint32_t slot = c.U(hSlot, lane), stride = c.U(hStride, lane), axes = c.U(hAxes, lane);
         const bool second = c.U(hSourceA, lane) == kInvalid;   // the side that moves is the row's second
-        const uint64_t way = c.link_paths[(second ? c.row_link_b : c.row_link_a)[slot] - c.first_link];
+        const uint64_t way = c.from_links ? way_of(c, lane) : c.link_paths[(second ? c.row_link_b : c.row_link_a)[slot] - c.first_link];
         way_low = uint32_t(way); way_high = uint32_t(way >> 32u);
         float w[3][6];
 #pragma unroll
         for (uint32_t a = 0u; a < 3u; ++a) {
+            if (c.from_links) {
+#pragma unroll
+                for (int t = 0; t < 6; ++t) w[a][t] = c.wrench[lane * kWrenchStride + 6u * a + uint32_t(t)];
+                continue;
+            }
 #pragma unroll
             for (int t = 0; t < 6; ++t) w[a][t] = 0.0f;
             if (a != 0u && axes == 1u) continue;
@@ -1142,6 +1231,13 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
         }
     }
     if (paired) {
+    } else if (N > kTwoWaveWidth && c.from_links) {
+        if (__ballot(mine) != 0ull) {
+            float weighted = 0.0f;
+            g.value += rows_transposed_times<true>(c, __ballot(mine), mf, mn, &weighted);
+            scale += weighted;
+            add_heads_through_links<N>(c, mine, mc, hrow);
+        }
     } else if (N > kTwoWaveWidth && c.through_links && __popcll(__ballot(mine)) >= int(kLinkHeads)) {
         // enough heads that their curvature is cheaper by way of the links; the force takes the staged rows as ever
         add_heads_force<N>(c, __ballot(mine), mf, mn, lane < c.heads ? c.U(hRow, lane) : 0u, g, scale);
@@ -1345,8 +1441,18 @@ __device__ __forceinline__ void row_steps(const Tile& c, float d) {
             c.F(hStep, h) = c.F(hUnitValue, h) * dvec[unit]; c.F(hStep + 1, h) = 0.0f; c.F(hStep + 2, h) = 0.0f;
             continue;
         }
-        const float* j = c.jac + c.U(hRow, h) * uint32_t(N);
         const uint32_t axes = c.U(hAxes, h);
+        if constexpr (N > kTwoWaveWidth) {
+            if (c.from_links) {
+                float motion[6];
+                link_motion<N>(c, way_of(c, h), dvec, motion);
+                c.F(hStep, h) = wrench_dot(c, h, 0u, motion);
+                c.F(hStep + 1, h) = axes > 1u ? wrench_dot(c, h, 1u, motion) : 0.0f;
+                c.F(hStep + 2, h) = axes > 2u ? wrench_dot(c, h, 2u, motion) : 0.0f;
+                continue;
+            }
+        }
+        const float* j = c.jac + c.U(hRow, h) * uint32_t(N);
         c.F(hStep, h) = row_dot_fma<N>(j, dvec);
         c.F(hStep + 1, h) = axes > 1u ? row_dot_fma<N>(j + N, dvec) : 0.0f;
         c.F(hStep + 2, h) = axes > 2u ? row_dot_fma<N>(j + 2 * N, dvec) : 0.0f;
@@ -1636,7 +1742,21 @@ __device__ __forceinline__ void measure_primal(Tile& c, const float (&mrow)[N], 
             if (c.U(hOwned, h) != 0u && c.U(hUnit, h) == lane) balance += double(c.F(hUnitValue, h)) * lambda_env[c.U(hSlot, h) - c.env * R];
     };
     uint32_t done = 0u;
-    for (uint32_t h = 0u; h < c.staged_end; ++h) {
+    bool rows_taken = false;
+    if constexpr (N > kTwoWaveWidth) {
+        if (c.from_links) {   // lane = head holds its impulse; the sum goes by way of the links
+            float impulse[3] = {0.0f, 0.0f, 0.0f};
+            if (lane < c.heads && c.U(hOwned, lane) != 0u) {
+                const uint32_t local = c.U(hSlot, lane) - c.env * R, stride = c.U(hStride, lane), axes = c.U(hAxes, lane);
+                impulse[0] = lambda_env[local];
+                if (block_axes(axes)) { impulse[1] = lambda_env[local + stride]; impulse[2] = lambda_env[local + 2u * stride]; }
+            }
+            const double sum = rows_transposed_times<false>(c, __ballot(impulse[0] != 0.0f || impulse[1] != 0.0f || impulse[2] != 0.0f), impulse, impulse, nullptr);
+            if (coordinate) balance += sum;
+            rows_taken = true;
+        }
+    }
+    for (uint32_t h = 0u; h < (rows_taken ? 0u : c.staged_end); ++h) {
         const uint32_t first = c.U(hRow, h);
         if (first == kInvalid || c.U(hOwned, h) == 0u) continue;
         add_units(done, h);
@@ -1695,6 +1815,15 @@ __device__ __forceinline__ void initialize_residuals(const Tile& c, float veloci
             c.F(hRes, h) = urows[size_t{slot} * kRowWords + 4u] * dt - (0.0f + along);
             c.F(hRes + 1, h) = 0.0f; c.F(hRes + 2, h) = 0.0f;
             continue;
+        }
+        if constexpr (N > kTwoWaveWidth) {
+            if (c.from_links) {
+                float motion[6];
+                link_motion<N>(c, way_of(c, h), dvec, motion);
+                for (uint32_t axis = 0u; axis < 3u; ++axis)
+                    c.F(hRes + axis, h) = axis < axes ? urows[size_t{slot + axis * stride} * kRowWords + 4u] * dt - wrench_dot(c, h, axis, motion) : 0.0f;
+                continue;
+            }
         }
         for (uint32_t axis = 0u; axis < 3u; ++axis) {
             float residual = 0.0f;
@@ -1883,15 +2012,23 @@ __host__ __device__ inline uint32_t HeadFieldFloats(uint32_t cap, uint32_t narro
     return (kWideStride * cap + kNarrowStride * (narrow + 1u) + 3u) & ~3u;
 }
 // `cap` heads carry fields; `staged` of them (the contact heads) carry three Jacobian rows each.
-__host__ __device__ inline uint32_t SolverLdsFloats(uint32_t n, uint32_t cap, uint32_t staged) {
+// A block that keeps no contact rows (the world's contact rows each act through one link, ModelView::rows_from_links;
+// a wide block of contact heads only) holds a wrench record a head in their place.
+__host__ __device__ inline bool RowsFromLinks(uint32_t n, bool contacts_only, uint32_t world_flag) {
+    return PaddedWidth(n) > uint32_t(kTwoWaveWidth) && contacts_only && world_flag != 0u;
+}
+__host__ __device__ inline uint32_t RowFloats(uint32_t N, uint32_t staged, bool from_links) {
+    return from_links ? (kWrenchStride * staged + 3u) & ~3u : 3u * staged * N;
+}
+__host__ __device__ inline uint32_t SolverLdsFloats(uint32_t n, uint32_t cap, uint32_t staged, bool from_links = false) {
     const uint32_t N = PaddedWidth(n);
     // the per-coordinate unit lists exist only when some head beyond the staged ones can be listed; without joint rows
     // the block keeps the footprint that lets eight of them share a compute unit's LDS
-    return FactorRegionFloats(n) + 3u * staged * N + HeadFieldFloats(cap, staged) + 256u + (cap > staged ? kUnitSlots * uint32_t(kWave) : 0u) +
-           LinkAxisFloats(n);
+    return FactorRegionFloats(n) + RowFloats(N, staged, from_links) + HeadFieldFloats(cap, staged) + 256u +
+           (cap > staged ? kUnitSlots * uint32_t(kWave) : 0u) + LinkAxisFloats(n);
 }
-__host__ __device__ inline uint32_t ReducedSolverLdsFloats(uint32_t full, uint32_t reduced, uint32_t cap, uint32_t staged) {
-    const uint32_t solve = SolverLdsFloats(reduced, cap, staged), scratch = ReductionScratchFloats(full, reduced);
+__host__ __device__ inline uint32_t ReducedSolverLdsFloats(uint32_t full, uint32_t reduced, uint32_t cap, uint32_t staged, bool from_links = false) {
+    const uint32_t solve = SolverLdsFloats(reduced, cap, staged, from_links), scratch = ReductionScratchFloats(full, reduced);
     return solve > scratch ? solve : scratch;
 }
 
@@ -2027,8 +2164,10 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         c.mfac = lds;
         c.hfac = c.mfac + FactorFloats(uint32_t(W));
     }
+    c.from_links = RowsFromLinks(uint32_t(W), kContactsOnly, m.rows_from_links);
     c.jac = lds + FactorRegionFloats(uint32_t(W));
-    c.fields = c.jac + 3u * staged_cap * c.ldj;
+    c.wrench = c.jac;   // one or the other
+    c.fields = c.jac + RowFloats(uint32_t(W), staged_cap, c.from_links);
     c.vec = c.fields + HeadFieldFloats(cap, staged_cap);
     // The block's mass rows: lane's row of M, or in a reduced block lane's row of the Schur complement (lanes below K)
     // and of -P (the followers).
@@ -2230,12 +2369,46 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
             one_link = !(side_a && side_b) && (!(side_a || side_b) || c.U(hRow, lane) != kInvalid);
         }
         c.through_links = heads <= uint32_t(kWave) && !c.units && __all(plain && one_link);
+        if (c.from_links) {
+            // the world was cooked as one whose contact rows each act through one link: an environment that holds
+            // anything else was given the wrong kernel
+            if (!c.through_links && lane == 0u) d.env_status[env] |= kEnvStatusSolverFailure;
+            // lane = head: its rows as wrenches about the pivot, [(p - o) x n; n] with n the direction of the side that
+            // moves, and its way to the root
+            if (lane < heads) {
+                float* record = c.wrench + lane * kWrenchStride;
+                const uint32_t slot = c.U(hSlot, lane);
+                const float* row = urows + size_t{slot} * kRowWords;
+                const uint32_t stride = __float_as_uint(row[2]);
+                const uint32_t axes = (__float_as_uint(row[0]) & kRowBlockNormal) != 0u ? 3u : 1u;
+                const bool side_a = c.U(hSourceA, lane) != kInvalid, side_b = c.U(hSourceB, lane) != kInvalid;
+                const bool second = !side_a;
+                uint64_t way = 0ull;
+                if (side_a != side_b) way = m.link_dof_mask[(second ? d.row_cj_link_b : d.row_cj_link)[slot] - env * nl];
+                for (uint32_t a = 0u; a < 3u; ++a) {
+                    float w[6] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+                    if (a < axes && side_a != side_b) {
+                        const size_t rs = size_t{slot} + a * stride;
+                        const float* side = urows + rs * kRowWords + (second ? 20u : 12u);
+                        const float* at = (second ? d.row_cj_point_b : d.row_cj_point) + 3u * rs;
+                        const V3 n{side[0], side[1], side[2]};
+                        const V3 moment = cross3(sub3(V3{at[0], at[1], at[2]}, c.pivot), n);
+                        w[0] = moment.x; w[1] = moment.y; w[2] = moment.z; w[3] = n.x; w[4] = n.y; w[5] = n.z;
+                    }
+#pragma unroll
+                    for (int t = 0; t < 6; ++t) record[6u * a + uint32_t(t)] = w[t];
+                }
+                reinterpret_cast<uint32_t*>(record)[18] = uint32_t(way);
+                reinterpret_cast<uint32_t*>(record)[19] = uint32_t(way >> 32u);
+                c.U(hColumnsLow, lane) = uint32_t(way); c.U(hColumnsHigh, lane) = uint32_t(way >> 32u);
+            }
+        }
         __syncthreads();
     }
     // CopyTileRows (:836-869): the staged heads' rows, their loads in flight together
 
     bool stray = false;   // a reduced block: an entry past the block's coordinates
-    for (uint32_t h0 = 0u; h0 < c.staged_end; h0 += 4u) {   // four heads at a time: 24 reads in flight
+    for (uint32_t h0 = 0u; h0 < (c.from_links ? 0u : c.staged_end); h0 += 4u) {   // four heads at a time: 24 reads in flight
         uint32_t first[4];
         float value[4][3];
 #pragma unroll
@@ -2355,8 +2528,17 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
                 const uint32_t first = c.U(hRow, h), unit = c.U(hUnit, h);
                 const float unit_value = c.F(hUnitValue, h);
                 skip[t] = share_units && unit != kInvalid && fabsf(unit_value) == 1.0f && !apart[t];
-                if (coordinate && (artic_a || artic_b) && !apart[t] && !skip[t])
-                    a[t] = first != kInvalid ? (lane < c.ldj ? c.jac[first * c.ldj + lane] : 0.0f) : (lane == unit ? unit_value : 0.0f);
+                if (coordinate && (artic_a || artic_b) && !apart[t] && !skip[t]) {
+                    if (W > kTwoWaveWidth && c.from_links) {   // the first row's entry: the coordinate's axis against the row's wrench
+                        const float4* table = reinterpret_cast<const float4*>(c.axes);
+                        const float4 sa = table[3u * lane], sb = table[3u * lane + 1u];
+                        const float* w = c.wrench + h * kWrenchStride;
+                        const float entry = fmaf(sb.y, w[5], fmaf(sb.x, w[4], fmaf(sa.w, w[3], fmaf(sa.z, w[2], fmaf(sa.y, w[1], sa.x * w[0])))));
+                        a[t] = ((way_of(c, h) >> lane) & 1ull) != 0ull ? entry : 0.0f;
+                    } else {
+                        a[t] = first != kInvalid ? (lane < c.ldj ? c.jac[first * c.ldj + lane] : 0.0f) : (lane == unit ? unit_value : 0.0f);
+                    }
+                }
             }
             if (skip[0] && skip[1] && skip[2] && skip[3]) continue;
 #pragma unroll

@@ -271,6 +271,7 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
         return ka == kShapeCapsule && kb == kShapeCapsule ? 1u : 0u;
     };
     uint32_t admitted = 0u, max_points = 1u;
+    bool link_pairs = false;   // some admitted pair joins the shapes of two links
     for (uint32_t i = 0u; i < nb; ++i) {
         const uint32_t kind = d.shape_kind[i];
         if (kind != kInvalid && kind != kShapeSphere && kind != kShapeCapsule && kind != kShapeBox && kind != kShapePlane && kind != kShapeCylinder)
@@ -290,6 +291,7 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
             if (points == 0u) throw NotSupported("admitted collidable pair has no analytic manifold (capsule or cylinder against box, capsule x cylinder, cylinder x cylinder)");
             max_points = std::max(max_points, points);
             ++admitted;
+            if (d.body_role[i] != 0u && d.body_role[j] != 0u) link_pairs = true;
         }
     }
     const uint32_t slots = d.max_contacts_per_env != 0u ? d.max_contacts_per_env : admitted;
@@ -332,6 +334,11 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
         if (d.body_role[b] == 0u || d.shape_kind[b] == kInvalid || d.body_link[b] >= nl) continue;
         const uint64_t mask = m.link_dof_mask[d.body_link[b]];
         for (uint32_t k = 0u; k < nv; ++k) if ((mask >> k) & 1ull) c.contact_dof_end = std::max(c.contact_dof_end, k + 1u);
+    }
+    c.rows_from_links = link_pairs ? 0u : 1u;
+    for (uint32_t l = 0u; l < nl; ++l) {
+        const uint8_t type = m.joint_type[l];
+        if (!(type == kRevolute || type == kPrismatic || type == kFixed || (type == kFloatingBase && l == 0u))) c.rows_from_links = 0u;
     }
     c.excluded_pair_count = uint32_t(m.excluded_pairs.size());
     // rows whose type and affinity masks are both empty pass the filter with no partner (shape_kind.hpp:26-33): the pair
@@ -1388,7 +1395,7 @@ int nuka_hip_model_view_set_count(nuka_phi_model_view* model, const char* name, 
 #define COUNT(member) if (std::strcmp(name, #member) == 0) { m->member = value; return 0; }
     COUNT(links_per_env) COUNT(bodies_per_env) COUNT(dof) COUNT(max_dof) COUNT(max_depth) COUNT(contact_slots) COUNT(rows_per_env)
     COUNT(contact_rows_per_env) COUNT(profile_count) COUNT(floating_root) COUNT(max_points_per_slot) COUNT(excluded_pair_count)
-    COUNT(sweep_passes) COUNT(pairable_count) COUNT(contact_dof_end) COUNT(joint_limit_rows) COUNT(joint_friction_rows) COUNT(joint_drive_rows)
+    COUNT(sweep_passes) COUNT(pairable_count) COUNT(contact_dof_end) COUNT(rows_from_links) COUNT(joint_limit_rows) COUNT(joint_friction_rows) COUNT(joint_drive_rows)
     COUNT(drive_mode) COUNT(any_mujoco) COUNT(contact_cone) COUNT(integrator)
 #undef COUNT
     return -1;
