@@ -2511,7 +2511,42 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         // wants exactly the staged sum of its two sides' rows.  Unit heads with an entry of +-1 are left to the
         // per-coordinate pass below: y(-e) = -y(e), so every such head of one coordinate has the same response.
         const bool share_units = c.units && c.unit_lists;
-        for (uint32_t h0 = 0u; h0 < (share_units ? c.individual_end : heads); h0 += 4u) {
+        bool by_heads = false;
+        if constexpr (W > kTwoWaveWidth && kContactsOnly) {
+            if (c.from_links && c.through_links) {
+                // Every head at once, lane = head: its first row sits in the lane's registers (the coordinates' axes against
+                // the row's wrench), the factor's entries are the same for every lane, and the substitution and the ordered
+                // sum run down the coordinates with the operations of the loop below, head beside head instead of
+                // four heads a pass.
+                by_heads = true;
+                const float* factor_rows = d.m_factor + size_t{env} * md * md;
+                const bool owned = lane < heads && (c.U(hSourceA, lane) != kInvalid || c.U(hSourceB, lane) != kInvalid);
+                const uint64_t way = owned ? way_of(c, lane) : 0ull;
+                float w[6];
+#pragma unroll
+                for (int t = 0; t < 6; ++t) w[t] = owned ? c.wrench[lane * kWrenchStride + uint32_t(t)] : 0.0f;
+                const float4* table = reinterpret_cast<const float4*>(c.axes);
+                float y[N];
+                float total = 0.0f;
+#pragma unroll
+                for (int i = 0; i < N; ++i) {
+                    if (uint32_t(i) >= n) { y[i] = 0.0f; continue; }
+                    const float4 sa = table[3 * i], sb = table[3 * i + 1];
+                    const float entry = fmaf(sb.y, w[5], fmaf(sb.x, w[4], fmaf(sa.w, w[3], fmaf(sa.z, w[2], fmaf(sa.y, w[1], sa.x * w[0])))));
+                    float v = ((way >> i) & 1ull) != 0ull ? entry : 0.0f;
+                    const float* factor_row = factor_rows + size_t(i) * md;
+#pragma unroll
+                    for (int j = 0; j < i; ++j) v -= factor_row[j] * y[j];
+                    y[i] = v;
+                    total += v * v / factor_row[i];
+                }
+                if (lane < heads) {
+                    const bool second = c.U(hSourceA, lane) == kInvalid;
+                    c.F(hStep, lane) = second ? 0.0f : total; c.F(hMove, lane) = second ? total : 0.0f;
+                }
+            }
+        }
+        for (uint32_t h0 = 0u; h0 < (by_heads ? 0u : share_units ? c.individual_end : heads); h0 += 4u) {
             float a[4], term[4], total[4];
             bool second[4], apart[4], skip[4];
 #pragma unroll
