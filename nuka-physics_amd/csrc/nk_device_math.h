@@ -239,6 +239,10 @@ __device__ __forceinline__ float opaque(float v) {
     asm volatile("" : "+v"(v));
     return v;
 }
+__device__ __forceinline__ uint32_t opaque_word(uint32_t v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
 __device__ __forceinline__ bool wave_all(bool p) { return __all(p); }
 __device__ __forceinline__ bool wave_any(bool p) { return __any(p); }
 

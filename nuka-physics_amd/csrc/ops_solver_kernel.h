@@ -1114,7 +1114,10 @@ __device__ __forceinline__ void add_heads_through_links(const Tile& c, bool mine
         table[3u * lane + 2u] = float4{y[2], y[3], y[4], y[5]};
     }
     __syncthreads();
-    const uint64_t path = (uint64_t(c.path_high) << 32u) | uint64_t(c.path_low), under = (uint64_t(c.under_high) << 32u) | uint64_t(c.under_low);
+    // (through the barrier so that the sixty-four lane masks of each are made here, two instructions a column, instead of
+    // ahead of the sweeps and kept in scalar registers the kernel does not have)
+    const uint64_t path = (uint64_t(opaque_word(c.path_high)) << 32u) | uint64_t(opaque_word(c.path_low));
+    const uint64_t under = (uint64_t(opaque_word(c.under_high)) << 32u) | uint64_t(opaque_word(c.under_low));
 #pragma unroll
     for (int j = 0; j < N; ++j) {
         const float4 a = table[3 * j], b = table[3 * j + 1], d = table[3 * j + 2];
@@ -1190,7 +1193,11 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
 #pragma unroll
     for (int q = 0; q < N / 2; ++q) {
         const double2 dv = d2[q];
-        const double m0 = double(mrow[2 * q]), m1 = double(mrow[2 * q + 1]);
+        // (the mass rows do not change over the solve: left to itself the compiler widens them to double once, ahead of
+        // the sweeps, and holds two registers an entry from there on - which pays while they fit, and a wide block
+        // has no room for)
+        const double m0 = double(N > kTwoWaveWidth ? opaque(mrow[2 * q]) : mrow[2 * q]);
+        const double m1 = double(N > kTwoWaveWidth ? opaque(mrow[2 * q + 1]) : mrow[2 * q + 1]);
         hrow[2 * q] = mrow[2 * q]; hrow[2 * q + 1] = mrow[2 * q + 1];
         inertial.value = fma(m0, dv.x, inertial.value);
         inertial.value = fma(m1, dv.y, inertial.value);
