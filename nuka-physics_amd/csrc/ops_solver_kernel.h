@@ -955,16 +955,17 @@ __device__ __forceinline__ void link_motion(const Tile& c, uint64_t way, const f
     const float4* x4 = reinterpret_cast<const float4*>(x);
 #pragma unroll
     for (int k = 0; k < 6; ++k) motion[k] = 0.0f;
-    const uint32_t low = uint32_t(way), high = uint32_t(way >> 32u);
-#pragma unroll
-    for (int q = 0; q < N / 4; ++q) {
+    // a loop that stays a loop: unrolled, all of the table is fetched ahead of the first product, into registers the
+    // block does not have
+#pragma unroll 1
+    for (uint32_t q = 0u; q < uint32_t(N / 4); ++q) {
         const float4 xq = x4[q];
         const float xs[4] = {xq.x, xq.y, xq.z, xq.w};
+        const uint32_t four = uint32_t(way >> (4u * q)) & 0xFu;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const int j = 4 * q + t;
-            const float4 a = table[3 * j], b = table[3 * j + 1];
-            const float on = ((j < 32 ? low >> j : high >> (j - 32)) & 1u) != 0u ? xs[t] : 0.0f;
+        for (uint32_t t = 0u; t < 4u; ++t) {
+            const float4 a = table[3u * (4u * q + t)], b = table[3u * (4u * q + t) + 1u];
+            const float on = ((four >> t) & 1u) != 0u ? xs[t] : 0.0f;
             motion[0] = fmaf(a.x, on, motion[0]); motion[1] = fmaf(a.y, on, motion[1]); motion[2] = fmaf(a.z, on, motion[2]);
             motion[3] = fmaf(a.w, on, motion[3]); motion[4] = fmaf(b.x, on, motion[4]); motion[5] = fmaf(b.y, on, motion[5]);
         }
