@@ -38,6 +38,30 @@ def test_every_op_at_every_width_matches_the_oracle(oracle_py, device, dof, floa
     oracle.close()
 
 
+@pytest.mark.parametrize("dof,floating,limb_joints", [(44, True, 7), (64, False, 16), (28, True, 7)])
+def test_wide_blocks_with_rows_between_links_match_the_oracle(oracle_py, device, dof, floating, limb_joints):
+    """Worlds whose spheres also collide with one another: some contact rows have the articulation on both sides, so a
+    wide block keeps its rows staged instead of deriving them from the links, and takes the heads' curvature by way of
+    the links only in environments where every live row happens to be one-sided."""
+    E = 48
+    tree, desc, state = tree_case(oracle_py, dof, floating, True, seed=3 * dof + 1, E=E, limb_joints=limb_joints, sphere_pairs=True)
+    oracle = oracle_py.OracleWorld(tree.template, desc, threads=8)
+    world = nk.World(device, tree.template, desc)
+    assert world.dof == dof
+    oracle.set_state(state)
+    world.set_state(state)
+    sens = one_ulp_sensitivity(oracle_py, tree.template, desc, state)
+    compare_ops(oracle, world, E, sens, state)
+    rows = oracle.download("urows").reshape(E, -1, 26).view(np.uint32)
+    active = (rows[:, :, 0] & 1) != 0
+    two_sided = active & (rows[:, :, 10] == 1) & (rows[:, :, 18] == 1)
+    print(f"dof {dof}: environments with a row between two links {int(two_sided.any(1).sum())} of {E}, contacts per env "
+          f"{oracle.download('contact_count').mean():.1f}")
+    close(world, oracle, "link_velocity", tol=bar(sens, "velocity"))
+    world.close()
+    oracle.close()
+
+
 @pytest.mark.parametrize("dof,floating,branched", [(40, True, True), (56, False, False), (64, True, True)])
 def test_steps_at_wide_widths_stay_with_the_oracle(oracle_py, device, dof, floating, branched):
     """Three whole steps (contact cache and carried solver velocities included) through the graph-less pipeline."""

@@ -15,11 +15,12 @@ class Tree:
         self.link_count = template.link_count
 
 
-def make_tree(dof, floating, branched, seed, mu=0.7, root_height=0.0, limb_joints=7, sphere_limbs=None):
+def make_tree(dof, floating, branched, seed, mu=0.7, root_height=0.0, limb_joints=7, sphere_limbs=None, sphere_pairs=False):
     """A tree with `dof` coordinates: a floating or fixed root and revolute joints, laid out as one serial chain or as
     limbs of at most `limb_joints` (seven) joints fanning out of the root.  Every limb's last two links carry a contact
     sphere, or only those of the first `sphere_limbs` limbs: the later limbs then carry no shape, like the arms of a
-    robot that stands on its feet."""
+    robot that stands on its feet.  With `sphere_pairs` the spheres of different links also collide with one another,
+    so that some contact rows have the articulation on both sides."""
     g = np.random.default_rng(seed)
     t = abi.Template()
     if floating:
@@ -50,10 +51,13 @@ def make_tree(dof, floating, branched, seed, mu=0.7, root_height=0.0, limb_joint
     t.add_body(abi.ROLE_STATIC, kind=abi.SHAPE_PLANE, contype=2, conaffinity=1, profile=profile)
     for link in range(t.link_count):
         t.add_body(abi.ROLE_LINK_BODY, link=link, kind=abi.SHAPE_NONE, contype=0, conaffinity=0)
-    for link, offset, radius in sphere_links:
+    for k, (link, offset, radius) in enumerate(sphere_links):
+        # (a negative group never pairs within itself, shape_kind.hpp:26-33: the two spheres of one limb, which sit a
+        # link apart, stay out of each other's way and only spheres of different limbs meet)
         t.add_body(abi.ROLE_PROXY, link=link, kind=abi.SHAPE_SPHERE, params=(radius, 0, 0, 0), local_pos=offset,
-                   contype=1, conaffinity=2, profile=profile)
-    t.max_contacts_per_env = len(sphere_links)
+                   contype=1, conaffinity=3 if sphere_pairs else 2, group=(-(k // 2 + 1)) & 0xFFFFFFFF if sphere_pairs else 0,
+                   profile=profile)
+    t.max_contacts_per_env = 0 if sphere_pairs else len(sphere_links)   # 0: a slot for every admitted pair
     return Tree(t, floating, sphere_links)
 
 
@@ -69,12 +73,12 @@ def sphere_heights(oracle_py, tree, desc, state):
     return z
 
 
-def tree_case(oracle_py, dof, floating, branched, seed, E, dt=1.0 / 240.0, vel_iters=8, limb_joints=7, sphere_limbs=None):
+def tree_case(oracle_py, dof, floating, branched, seed, E, dt=1.0 / 240.0, vel_iters=8, limb_joints=7, sphere_limbs=None, sphere_pairs=False):
     """(tree, desc, state): seeded joint angles, rates and torques; the root is placed so that each environment's
     lowest sphere presses a few millimetres into the plane (floating root), or so that half of the environments touch
     it (fixed root: the anchor height belongs to the template)."""
     g = np.random.default_rng(seed + 1000)
-    tree = make_tree(dof, floating, branched, seed, limb_joints=limb_joints, sphere_limbs=sphere_limbs)
+    tree = make_tree(dof, floating, branched, seed, limb_joints=limb_joints, sphere_limbs=sphere_limbs, sphere_pairs=sphere_pairs)
     nl = tree.link_count
     desc = abi.world_desc(E, dt, vel_iters=vel_iters, contact_margin=0.1)   # spheres a hand above the plane get speculative rows
     q = g.normal(0.0, 0.3, (E, nl)).astype(np.float32)
@@ -93,5 +97,5 @@ def tree_case(oracle_py, dof, floating, branched, seed, E, dt=1.0 / 240.0, vel_i
         base[:, 2] = (SPHERE_RADIUS - lowest - g.uniform(0.0, 0.004, E)).astype(np.float32)
     else:
         tree = make_tree(dof, floating, branched, seed, root_height=float(SPHERE_RADIUS - np.median(lowest)), limb_joints=limb_joints,
-                         sphere_limbs=sphere_limbs)
+                         sphere_limbs=sphere_limbs, sphere_pairs=sphere_pairs)
     return tree, desc, state
