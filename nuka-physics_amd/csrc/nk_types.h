@@ -72,7 +72,7 @@ struct ModelView {
     uint32_t excluded_pair_count;
     uint32_t sweep_passes;     // passes of the dynamics' tree sweeps (sweep_links)
     uint32_t pairable_count;   // collidable rows that can pass the shape filter with some partner (pairable_rows, ascending)
-    uint32_t contact_dof_end;  // one past the last coordinate on the path to the root of any link that carries a shape: no contact row reaches a later one
+    uint32_t contact_dof_end;  // one past the last coordinate on the path to the root of any link that carries a shape: no contact row reaches a later one (0: not known)
     // 1: every contact row acts on the articulation through one link (no admitted pair joins two of its links' shapes) and
     // every coordinate is a hinge, a slider or one of a floating root's six: a contact row's entries then follow from the
     // row's wrench and the coordinates' motion axes, and the solve of a wide block need not keep the rows themselves

@@ -117,7 +117,8 @@ void InitSolverKernels() {
 static uint32_t SolverWorkingWidth(const ModelView& m, bool contacts_only) {
     if (contacts_only)
         for (const ReducedKernel& reduced : kReducedKernels)
-            if (reduced.width == solver::PaddedWidth(m.dof) && m.contact_dof_end <= reduced.reduced && reduced.reduced <= m.dof) return reduced.reduced;
+            if (reduced.width == solver::PaddedWidth(m.dof) && m.contact_dof_end != 0u && m.contact_dof_end <= reduced.reduced &&
+                reduced.reduced <= m.dof) return reduced.reduced;   // (0: a host that did not say; the full width is always right)
     return m.dof;
 }
 // worlds whose heads are contact heads only, at most one a lane (the elliptic cone of the MuJoCo law is answered by the

@@ -6,7 +6,13 @@
 // multipliers travel between lanes as scalar lane reads, and LDS only carries what must be read transposed (the
 // factor columns of the backward substitution) or broadcast (Jacobian rows, small vectors, read as 16-byte words).
 // The mass matrix is constant over a solve, so its factor is built once.  A lane is a head row in the per-head
-// phases.  Cross-lane sums use the compensated two-float butterfly; nothing is exchanged between environments.
+// phases.  Sums that the reference carries as compensated two-float pairs are double accumulators here (a double
+// multiply-add issues at the rate of a float one on this device); nothing is exchanged between environments.
+// Two instantiations go beyond the plain block.  A reduced block (template argument K < N) eliminates, once per
+// solve, the coordinates from K on that no contact of the world reaches, and sweeps K wide (described above
+// mass_times).  A wide block (more than kTwoWaveWidth coordinates) of a world whose contact rows each act through one
+// link keeps no Jacobian rows: every entry follows from the row's wrench and the coordinates' motion axes (described
+// above link_motion and add_heads_through_links).
 //
 // Replaces src/phi/backend_cuda/ops/block_descent_tile.cuh (DescendTile :2941-3087 and everything it calls) and
 // the helpers it takes from block_descent.cu (:735-820, 1593-1621, 1726-1753) and nk/solve/augmented_row.hpp.
@@ -262,11 +268,11 @@ static_assert(kNarrowFields <= 64u, "one lane clears the shared word of each nar
 constexpr uint32_t kWideStride = kWideFields | 1u, kNarrowStride = kNarrowFields | 1u;
 
 struct Tile {
-    uint32_t env, lane, n, ld, ldj, heads, cap, narrow, iteration;
+    uint32_t env, lane, n, ldj, heads, cap, narrow, iteration;
     uint32_t n_all;   // n, or past it the coordinates that follow the block's own (a reduced block, described above mass_times)
     float tolerance;
-    float* mfac;     // N x ld: Cholesky factor of the mass matrix (rows; columns are read transposed)
-    float* hfac;     // N x ld: Cholesky factor of the current Newton Hessian
+    float* mfac;     // FactorFloats(N) words: Cholesky factor of the mass matrix (rows; columns are read transposed); device memory for a wide block
+    float* hfac;     // FactorFloats(N) words: Cholesky factor of the current Newton Hessian
     float* jac;      // 3 * staged capacity rows x ldj, ldj = N
     float* fields;   // cap x kWideStride, then (narrow + 1) x kNarrowStride
     float* vec;      // 4 x 64 scratch vectors, 16-byte aligned
@@ -2154,7 +2160,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     }
     const uint32_t R = p.rows_per_env, md = p.max_dof, n = m.dof, nl = m.links_per_env, S = p.contact_slots_per_env;
     Tile c;
-    c.env = env; c.lane = lane; c.n = kReduced ? uint32_t(K) : n; c.n_all = n; c.ld = uint32_t(W) + 1u; c.ldj = uint32_t(W); c.cap = cap; c.narrow = staged_cap; c.heads = 0u; c.iteration = 0u;
+    c.env = env; c.lane = lane; c.n = kReduced ? uint32_t(K) : n; c.n_all = n; c.ldj = uint32_t(W); c.cap = cap; c.narrow = staged_cap; c.heads = 0u; c.iteration = 0u;
     c.tolerance = p.velocity_tolerance; c.failed = false; c.momentum = 0.0f; c.residual = 0.0f;
     c.mass_inverse = 0.0f; c.mass_valid = false; c.work = 0u; c.units = false; c.elliptic = false;
     c.factor_current = false;
