@@ -303,7 +303,7 @@ struct Tile {
     const uint64_t* link_paths;
     uint32_t first_link;      // index of the environment's first link
 #ifdef NKH_SOLVER_PROFILE
-    mutable long long prof[26];
+    mutable long long prof[32];
     mutable uint32_t prof_count[4];
 #endif
     // with a constant field, as at nearly every call, the place of the field folds to a constant
@@ -1629,6 +1629,7 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], c
     const bool coordinate = lane < n;
     const bool follower = kFollow && lane >= n && lane < c.n_all;
     const bool moving = coordinate || follower;
+    PROF_BEGIN(c, 26);
     for (uint32_t h = lane; h < c.heads; h += kWave) {   // StartTileBlock (:1386-1397)
         if (c.U(hOwned, h) == 0u) continue;
         c.F(hNormalBound, h) = c.F(hDual, h);
@@ -1660,6 +1661,7 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], c
             }
         }
     }
+    PROF_END(c, 26);
     Failure failure = kFailNone;
     float primal = FLT_MAX;
     for (uint32_t step = 0u; step < kNewtonSteps; ++step) {
@@ -1673,6 +1675,7 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], c
         const float mass_step = mass_times<N>(c, mrow, dd);
         if (follower) dd = mass_step;
         PROF_END(c, 8);
+        PROF_BEGIN(c, 27);
         TileSum decrement{0.0}, slope{0.0}, curvature{0.0};
         if (coordinate) {
             tile_add_product(decrement, force, dd);
@@ -1684,12 +1687,14 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], c
         const float inertial_curvature = wave_total(curvature);
         if (!isfinite(total_decrement) || !isfinite(inertial_slope) || !isfinite(inertial_curvature)) { failure = kFailDirection; break; }
         if (!(total_decrement > 0.0f)) break;
+        PROF_END(c, 27);
         PROF_BEGIN(c, 4);
         row_steps<N>(c, dd);
         PROF_END(c, 4);
         PROF_BEGIN(c, 5);
         const float alpha = search_line<kKeepLine<N>>(c, line, inertial_slope, inertial_curvature);
         PROF_END(c, 5);
+        PROF_BEGIN(c, 28);
         const float after = fmaf(alpha, dd, u);
         const bool rounded = __all(!moving || after == u);
         if (!__all(!moving || isfinite(after))) { failure = kFailCandidate; break; }
@@ -1698,8 +1703,10 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], c
         if (!(alpha > 0.0f)) break;
         u = after;
         apply_moves(c, alpha);
+        PROF_END(c, 28);
         if (rounded) break;
     }
+    PROF_BEGIN(c, 29);
     for (uint32_t h = lane; h < c.heads; h += kWave) {   // EndTileBlock (:1400-1409)
         if (c.U(hOwned, h) == 0u) continue;
 #pragma unroll
@@ -1716,6 +1723,7 @@ __device__ __forceinline__ void descend_block(Tile& c, const float (&mrow)[N], c
     if (failure != kFailNone) primal = FLT_MAX;
     c.residual = fmaxf(c.residual, wave_max(primal));   // one block per environment: no coupled heads
     if (moving) *u_io = u;
+    PROF_END(c, 29);
 }
 
 // MeasureTilePrimal (:2378-2489): the mass-normalised momentum balance in double
@@ -2165,7 +2173,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     c.mass_inverse = 0.0f; c.mass_valid = false; c.work = 0u; c.units = false; c.elliptic = false;
     c.factor_current = false;
 #ifdef NKH_SOLVER_PROFILE
-    for (int i = 0; i < 26; ++i) c.prof[i] = 0;
+    for (int i = 0; i < 32; ++i) c.prof[i] = 0;
     for (int i = 0; i < 4; ++i) c.prof_count[i] = 0u;
     const long long prof_wall_start = wall_clock64();
 #endif
@@ -2764,6 +2772,7 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
         for (int i = 0; i < 10; ++i) d.solver_penalty[size_t{env} * R + i] = float(c.prof[i]);
         for (int i = 0; i < 4; ++i) d.solver_penalty[size_t{env} * R + 10 + i] = float(c.prof_count[i]);
         for (int i = 10; i < 26; ++i) d.solver_penalty[size_t{env} * R + 4 + i] = float(c.prof[i]);
+        for (int i = 26; i < 32; ++i) if (uint32_t(7 + i) < R) d.solver_penalty[size_t{env} * R + 7 + i] = float(c.prof[i]);
         // launch slot and the wave's first and last moment on the constant 100 MHz clock, as raw words
         d.solver_penalty[size_t{env} * R + 30] = __uint_as_float(uint32_t(prof_wall_start));
         d.solver_penalty[size_t{env} * R + 31] = __uint_as_float(uint32_t(wall_clock64()));
