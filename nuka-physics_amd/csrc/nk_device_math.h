@@ -239,6 +239,13 @@ __device__ __forceinline__ float opaque(float v) {
     asm volatile("" : "+v"(v));
     return v;
 }
+// The same for a value that does not change over a loop, tied to one that does (`with`): what is computed from the
+// result cannot leave the loop, and since the statement has no side effect of its own it orders nothing - reads and
+// arithmetic around it are scheduled freely, where the plain barrier above keeps every memory access on its side.
+__device__ __forceinline__ float opaque_with(float v, float with) {
+    asm("" : "+v"(v) : "v"(with));
+    return v;
+}
 __device__ __forceinline__ uint32_t opaque_word(uint32_t v) {
     asm volatile("" : "+v"(v));
     return v;

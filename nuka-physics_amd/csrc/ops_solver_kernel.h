@@ -1203,14 +1203,16 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
         // (the mass rows do not change over the solve: left to itself the compiler widens them to double once, ahead of
         // the sweeps, and holds two registers an entry from there on - which pays while they fit, and a wide block
         // has no room for)
-        const double m0 = double(N > kTwoWaveWidth ? opaque(mrow[2 * q]) : mrow[2 * q]);
-        const double m1 = double(N > kTwoWaveWidth ? opaque(mrow[2 * q + 1]) : mrow[2 * q + 1]);
+        const double m0 = double(N > kTwoWaveWidth ? opaque_with(mrow[2 * q], u) : mrow[2 * q]);
+        const double m1 = double(N > kTwoWaveWidth ? opaque_with(mrow[2 * q + 1], u) : mrow[2 * q + 1]);
         hrow[2 * q] = mrow[2 * q]; hrow[2 * q + 1] = mrow[2 * q + 1];
         inertial.value = fma(m0, dv.x, inertial.value);
         inertial.value = fma(m1, dv.y, inertial.value);
         if constexpr (kFollow) {
-            inertial.value = fma(double(mlow[2 * q]), dv.x, inertial.value);
-            inertial.value = fma(double(mlow[2 * q + 1]), dv.y, inertial.value);
+            // (the low parts widened here, at every assembly: held widened over the solve beside the high parts they
+            // take the block past its registers)
+            inertial.value = fma(double(opaque_with(mlow[2 * q], u)), dv.x, inertial.value);
+            inertial.value = fma(double(opaque_with(mlow[2 * q + 1], u)), dv.y, inertial.value);
         }
         inertial_scale = fma(fabs(m0), fabs(dv.x), inertial_scale);
         inertial_scale = fma(fabs(m1), fabs(dv.y), inertial_scale);
@@ -1733,18 +1735,24 @@ __device__ __forceinline__ void measure_primal(Tile& c, const float (&mrow)[N], 
     const uint32_t lane = c.lane, n = c.n;
     const bool coordinate = lane < n;
     const bool follower = kFollow && lane >= n && lane < c.n_all;
-    float* dvec = c.vec;
-    dvec[lane] = coordinate ? *velocity_io : 0.0f;
-    c.vec[64 + lane] = coordinate ? free_v : 0.0f;
+    // every coordinate's distance from its free velocity, exact in double, through LDS
+    double* apart = reinterpret_cast<double*>(c.vec);
+    const float here = coordinate ? *velocity_io : 0.0f;
+    apart[lane] = coordinate ? double(here) - double(free_v) : 0.0;
     __syncthreads();
     double balance = 0.0;
+    const double2* apart2 = reinterpret_cast<const double2*>(apart);
 #pragma unroll
-    for (int j = 0; j < N; ++j) {
+    for (int q = 0; q < N / 2; ++q) {
         // the mass row does not change over the solve: left to itself the compiler widens all of it to double once,
         // ahead of the sweeps, and holds two registers an entry from there on
-        const float mass = opaque(mrow[j]);
-        balance -= double(mass) * (double(dvec[j]) - c.vec[64 + j]);   // padded terms are exact zeros
-        if constexpr (kFollow) balance -= double(opaque(mlow[j])) * (double(dvec[j]) - c.vec[64 + j]);
+        const double2 dv = apart2[q];   // padded terms are exact zeros
+        balance = fma(-double(opaque_with(mrow[2 * q], here)), dv.x, balance);
+        balance = fma(-double(opaque_with(mrow[2 * q + 1], here)), dv.y, balance);
+        if constexpr (kFollow) {
+            balance = fma(-double(opaque_with(mlow[2 * q], here)), dv.x, balance);
+            balance = fma(-double(opaque_with(mlow[2 * q + 1], here)), dv.y, balance);
+        }
     }
     // heads with an impulse add J^T lambda in head order (:2402-2436).  A unit head touches one coordinate: that
     // lane takes it from its own list when it comes up between the staged heads
