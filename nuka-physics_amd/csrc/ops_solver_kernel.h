@@ -634,14 +634,18 @@ __device__ __forceinline__ void add_head(const Tile& c, uint32_t h, bool coordin
                                          const float (&noise)[3], uint32_t axes, uint64_t columns, float (&hrow)[N], TileSum& g,
                                          float& scale) {
     const float* j0r = c.jac + c.U(hRow, h) * uint32_t(N);
-    const float j0 = coordinate ? j0r[c.lane] : 0.0f;
+    // (the lane's words read whether or not it is a coordinate: a read under a condition compiles to a branch a word)
+    const uint32_t column = c.lane < uint32_t(N) ? c.lane : uint32_t(N - 1);
+    const float w0 = j0r[column];
+    const float j0 = coordinate ? w0 : 0.0f;
     tile_add_product(g, j0, f[0]);
     scale += fabsf(j0) * noise[0];
     const float4* r0 = reinterpret_cast<const float4*>(j0r);
     if constexpr (N <= kTwoWaveWidth) {
         float a0 = j0 * cv[0], a1 = 0.0f, a2 = 0.0f;
         if (axes != 1u) {
-            const float j1 = coordinate ? j0r[N + c.lane] : 0.0f, j2 = coordinate ? j0r[2 * N + c.lane] : 0.0f;
+            const float w1 = j0r[N + column], w2 = j0r[2 * N + column];
+            const float j1 = coordinate ? w1 : 0.0f, j2 = coordinate ? w2 : 0.0f;
             const float cxx = cv[0], cyy = cv[1], czz = cv[2], cxy = cv[3], cxz = cv[4], cyz = cv[5];
             tile_add_product(g, j1, f[1]);
             tile_add_product(g, j2, f[2]);
@@ -719,7 +723,10 @@ __device__ __forceinline__ void add_head_pair(const Tile& c, uint32_t ha, uint32
     const uint32_t first = uint32_t(__shfl(int(my_first), source, kWave));
     const float* j0r = c.jac + first * uint32_t(N);
     const bool live = !none && row < c.n;
-    const float j0 = live ? j0r[row] : 0.0f, j1 = live ? j0r[N + row] : 0.0f, j2 = live ? j0r[2 * N + row] : 0.0f;
+    // (read whether or not the lane uses them: a read under a condition compiles to a branch a word)
+    const uint32_t column = row < uint32_t(N) ? row : uint32_t(N - 1);
+    const float w0 = j0r[column], w1 = j0r[N + column], w2 = j0r[2 * N + column];
+    const float j0 = live ? w0 : 0.0f, j1 = live ? w1 : 0.0f, j2 = live ? w2 : 0.0f;
     tile_add_product(g, j0, f[0]);
     tile_add_product(g, j1, f[1]);
     tile_add_product(g, j2, f[2]);
@@ -749,6 +756,72 @@ __device__ __forceinline__ void add_head_pair(const Tile& c, uint32_t ha, uint32
             hrow[4 * q + 3] += fmaf(a2, x2.w, fmaf(a1, x1.w, a0 * x0.w));
         }
     }
+}
+
+// Heads a pass where three or four copies of the block's rows fit the wavefront (kGroups<N> of N lanes each): the
+// lanes of group g add head `heads[g]` (kInvalid: none) to rows of their own, row = lane - g N; groups past the first
+// start at zero and the caller adds the groups' rows together afterwards (groups_sum).  Otherwise as add_head_pair.
+template <int N>
+constexpr int kGroups = N <= 16 ? 4 : (N <= 20 ? 3 : 2);
+template <int N>
+__device__ __forceinline__ void add_head_group(const Tile& c, const uint32_t (&heads)[4], const float (&mf)[3], const float (&mc)[6],
+                                               const float (&mn)[3], uint32_t my_first, uint32_t my_low, uint32_t my_high, float (&hrow)[N],
+                                               TileSum& g, float& scale) {
+    constexpr int G = kGroups<N>;
+    static_assert(G >= 3 && G * N <= 64, "three or four copies of the rows fit the wavefront");
+    const uint32_t group = c.lane / uint32_t(N), row = c.lane - group * uint32_t(N);
+    uint32_t mine = kInvalid;
+#pragma unroll
+    for (int k = 0; k < G; ++k) mine = group == uint32_t(k) ? heads[k] : mine;
+    const bool none = mine == kInvalid;   // also the lanes past the last group
+    const int source = int(none ? heads[0] : mine);
+    float f[3], cv[6], noise[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { f[k] = __shfl(mf[k], source, kWave); noise[k] = __shfl(mn[k], source, kWave); }
+#pragma unroll
+    for (int k = 0; k < 6; ++k) cv[k] = __shfl(mc[k], source, kWave);
+    const uint32_t first = uint32_t(__shfl(int(my_first), source, kWave));
+    const float* j0r = c.jac + first * uint32_t(N);
+    const bool live = !none && row < c.n;
+    const uint32_t column = row < uint32_t(N) ? row : uint32_t(N - 1);
+    const float w0 = j0r[column], w1 = j0r[N + column], w2 = j0r[2 * N + column];
+    const float j0 = live ? w0 : 0.0f, j1 = live ? w1 : 0.0f, j2 = live ? w2 : 0.0f;
+    tile_add_product(g, j0, f[0]);
+    tile_add_product(g, j1, f[1]);
+    tile_add_product(g, j2, f[2]);
+    scale += (fabsf(j0) * noise[0] + fabsf(j1) * noise[1]) + fabsf(j2) * noise[2];
+    const float cxx = cv[0], cyy = cv[1], czz = cv[2], cxy = cv[3], cxz = cv[4], cyz = cv[5];
+    const float a0 = (j0 * cxx + j1 * cxy) + j2 * cxz;
+    const float a1 = (j1 * cyy + j2 * cyz) + j0 * cxy;
+    const float a2 = (j2 * czz + j1 * cyz) + j0 * cxz;
+    uint64_t columns = 0ull;
+#pragma unroll
+    for (int k = 0; k < G; ++k) {
+        if (heads[k] == kInvalid) continue;
+        columns |= (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_high), int(heads[k])))) << 32u) |
+                   uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_low), int(heads[k]))));
+    }
+    add_column_groups<N>(std::make_integer_sequence<int, N / 4>{}, columns, 0u, lds_address(j0r), a0, a1, a2, hrow);
+}
+// v[lane] + v[lane + N] + ... over the groups of add_head_group, in the lanes of the first group
+template <int N>
+__device__ __forceinline__ float groups_sum(uint32_t lane, float v) {
+    float total = v;
+#pragma unroll
+    for (int k = 1; k < kGroups<N>; ++k) total += __shfl(v, int(lane) + k * N, kWave);
+    return total;
+}
+template <int N>
+__device__ __forceinline__ double groups_sum(uint32_t lane, double v) {
+    const uint64_t bits = uint64_t(__double_as_longlong(v));
+    double total = v;
+#pragma unroll
+    for (int k = 1; k < kGroups<N>; ++k) {
+        const uint32_t low = uint32_t(__shfl(int(uint32_t(bits)), int(lane) + k * N, kWave));
+        const uint32_t high = uint32_t(__shfl(int(uint32_t(bits >> 32u)), int(lane) + k * N, kWave));
+        total += __longlong_as_double((long long)((uint64_t(high) << 32u) | uint64_t(low)));
+    }
+    return total;
 }
 
 // One head's line-search inputs in registers: nothing in them changes between the probes of one search, and neither
@@ -1221,13 +1294,40 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
     TileSum g{-inertial.value};
     PROF_END(c, 11);
     PROF_BEGIN(c, 12);
-    bool paired = false;
+    bool paired = false, grouped = false;
     if constexpr (N <= 32) {
         // two or more contributing heads (all of them staged, one a lane): two a pass, the second half of the
         // wavefront collecting its heads in rows of its own
         const uint64_t all = __ballot(mine);
         paired = !c.units && c.heads <= uint32_t(kWave) && (all & (all - 1ull)) != 0ull;
-        if (paired) {
+        if constexpr (N <= 20 && N <= kTwoWaveWidth) {
+            // where three or four copies of the rows fit the wavefront, that many heads a pass - when it takes fewer
+            // passes than two a pass would (adding the groups' rows together costs more than adding two halves)
+            const int contributing = __popcll(all);
+            if (paired && (contributing + kGroups<N> - 1) / kGroups<N> < (contributing + 1) / 2) {
+                if (lane >= uint32_t(N)) {
+#pragma unroll
+                    for (int k = 0; k < N; ++k) hrow[k] = 0.0f;
+                    g.value = 0.0; scale = 0.0f;
+                }
+                const uint32_t my_first = lane < c.heads ? c.U(hRow, lane) : 0u;
+                for (uint64_t rest = all; rest != 0ull;) {
+                    uint32_t taken[4] = {kInvalid, kInvalid, kInvalid, kInvalid};
+#pragma unroll
+                    for (int k = 0; k < kGroups<N>; ++k) {
+                        if (rest == 0ull) break;
+                        taken[k] = uint32_t(__builtin_ctzll(rest));
+                        rest &= rest - 1ull;
+                    }
+                    add_head_group<N>(c, taken, mf, mc, mn, my_first, my_low, my_high, hrow, g, scale);
+                }
+#pragma unroll
+                for (int k = 0; k < N; ++k) hrow[k] = groups_sum<N>(lane, hrow[k]);
+                g.value = groups_sum<N>(lane, g.value); scale = groups_sum<N>(lane, scale);
+                grouped = true;
+            }
+        }
+        if (paired && !grouped) {
             if (lane >= 32u) {
 #pragma unroll
                 for (int k = 0; k < N; ++k) hrow[k] = 0.0f;
