@@ -35,6 +35,12 @@ constexpr int kWave = 64;
 #define NKH_TWO_WAVE_WIDTH 36
 #endif
 constexpr int kTwoWaveWidth = NKH_TWO_WAVE_WIDTH;
+// From this width on a block widens its mass rows to double where it uses them; below it the widened rows are kept over
+// the solve (two registers an entry), which pays while they fit.
+#ifndef NKH_WIDEN_AT_USE
+#define NKH_WIDEN_AT_USE 24
+#endif
+constexpr int kWidenAtUse = NKH_WIDEN_AT_USE;
 constexpr uint32_t kNewtonSteps = 16u;        // block_descent_dense.cuh:14
 constexpr uint32_t kLineSearchSteps = 32u;    // block_descent_dense.cuh:15
 constexpr float kLineTolerance = 1.0e-6f;     // block_descent_dense.cuh:17
@@ -1276,8 +1282,8 @@ __device__ __forceinline__ bool assemble_block(const Tile& c, const float (&mrow
         // (the mass rows do not change over the solve: left to itself the compiler widens them to double once, ahead of
         // the sweeps, and holds two registers an entry from there on - which pays while they fit, and a wide block
         // has no room for)
-        const double m0 = double(N > kTwoWaveWidth ? opaque_with(mrow[2 * q], u) : mrow[2 * q]);
-        const double m1 = double(N > kTwoWaveWidth ? opaque_with(mrow[2 * q + 1], u) : mrow[2 * q + 1]);
+        const double m0 = double(N >= kWidenAtUse ? opaque_with(mrow[2 * q], u) : mrow[2 * q]);
+        const double m1 = double(N >= kWidenAtUse ? opaque_with(mrow[2 * q + 1], u) : mrow[2 * q + 1]);
         hrow[2 * q] = mrow[2 * q]; hrow[2 * q + 1] = mrow[2 * q + 1];
         inertial.value = fma(m0, dv.x, inertial.value);
         inertial.value = fma(m1, dv.y, inertial.value);
