@@ -491,17 +491,33 @@ __device__ __forceinline__ void store_rows(float* a, uint32_t lane, const float 
             if (!kLeavesFirst<N> || uint32_t(k) >= lane) a[factor_at<N>(lane, uint32_t(k))] = row[k];
     }
 }
+// (Every word is read whether or not the lane keeps it - a read under a condition compiles to a branch a word - from
+// a place inside the factor: a lane past the rows reads the last row's, and a packed row's words left of its diagonal
+// fall in the rows before it.)
 template <int N>
 __device__ __forceinline__ void load_rows(const float* a, uint32_t lane, float (&row)[N]) {
     lane = local_lane(lane);
+    const uint32_t from = lane < uint32_t(N) ? lane : uint32_t(N - 1);
 #pragma unroll
-    for (int k = 0; k < N; ++k) row[k] = lane < uint32_t(N) && (!kLeavesFirst<N> || uint32_t(k) >= lane) ? a[factor_at<N>(lane, uint32_t(k))] : 0.0f;
+    for (int k = 0; k < N; ++k) {
+        const bool kept = lane < uint32_t(N) && (!kLeavesFirst<N> || uint32_t(k) >= lane);
+        if constexpr (N > kTwoWaveWidth) {   // such a block's mass factor is in device memory: only the words that are kept
+            row[k] = kept ? a[factor_at<N>(lane, uint32_t(k))] : 0.0f;
+        } else {
+            const float word = a[factor_at<N>(from, uint32_t(k))];
+            row[k] = kept ? word : 0.0f;
+        }
+    }
 }
 template <int N>
 __device__ __forceinline__ void load_columns(const float* a, uint32_t lane, float (&col)[N]) {
     lane = local_lane(lane);
+    const uint32_t from = lane < uint32_t(N) ? lane : uint32_t(N - 1);
 #pragma unroll
-    for (int j = 0; j < N; ++j) col[j] = lane < uint32_t(N) ? a[j * (N + 1) + lane] : 0.0f;
+    for (int j = 0; j < N; ++j) {
+        const float word = a[j * (N + 1) + from];
+        col[j] = lane < uint32_t(N) ? word : 0.0f;
+    }
 }
 
 // Cholesky of the Newton Hessian held in `hrow`, then d = H^-1 g.  The factor passes through LDS once, for the
