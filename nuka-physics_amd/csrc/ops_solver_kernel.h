@@ -537,6 +537,7 @@ __device__ __forceinline__ bool cholesky_solve(const Tile& c, float (&hrow)[N], 
         PROF_END(c, 24);
         c.factor_current = true;
     } else {
+        PROF_COUNT(c, 3);
         // rows and the reciprocal diagonal come back from hfac (the factor's own reciprocal is 1 / its diagonal
         // entry, the same division)
         inverse = row < uint32_t(N) ? 1.0f / c.hfac[factor_at<N>(row, row)] : 0.0f;
