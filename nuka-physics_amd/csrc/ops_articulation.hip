@@ -434,10 +434,15 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
         // Rows and columns n..N-1 are those of the identity.  Entry (i, j) loses (L_ik L_jk) D_k for k = 0, 1, ... as the
         // serial loop does; what a lane computes above its diagonal is never read.
         {
+            // (every word read whether or not the lane keeps it, from a place inside the matrix: a read under a condition
+            // compiles to a branch a word)
             const uint32_t ll = local_lane(lane);
+            const uint32_t from = (ll < n ? ll : 0u) * ld;
 #pragma unroll
-            for (int k = 0; k < N; ++k)
-                row[k] = ll < n && uint32_t(k) < n ? A[ll * ld + k] : (ll == uint32_t(k) ? 1.0f : 0.0f);
+            for (int k = 0; k < N; ++k) {
+                const float word = A[from + (uint32_t(k) < n ? uint32_t(k) : 0u)];
+                row[k] = ll < n && uint32_t(k) < n ? word : (ll == uint32_t(k) ? 1.0f : 0.0f);
+            }
         }
         {
             const uint32_t ll = local_lane(lane);
@@ -479,7 +484,10 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
         const uint32_t ll = local_lane(lane);
         float col[N];
 #pragma unroll
-        for (int i = 0; i < N; ++i) col[i] = ll < uint32_t(i) && uint32_t(i) < n ? A[i * ld + ll] : 0.0f;
+        for (int i = 0; i < N; ++i) {
+            const float word = A[(uint32_t(i) < n ? uint32_t(i) : 0u) * ld + (ll < n ? ll : 0u)];
+            col[i] = ll < uint32_t(i) && uint32_t(i) < n ? word : 0.0f;
+        }
 #pragma unroll
         for (int j = 0; j < N; ++j) {
             const float solved = lane_value(x, j);
