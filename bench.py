@@ -73,7 +73,10 @@ def scene_run(nk, args):
     settles for --settle steps from the authored pose with a small random push per environment, then --steps
     free-running steps are timed; environments that are flagged or not finite are counted, not hidden."""
     import numpy as np
-    scene = nk.Scene(args.scene, nk.SCENE_GROUND_PLANE | nk.SCENE_PLANE_CONTACTS_ONLY if args.scene.endswith(".urdf") else 0)
+    flags = nk.SCENE_GROUND_PLANE | nk.SCENE_PLANE_CONTACTS_ONLY if args.scene.endswith(".urdf") else 0
+    if args.native_laws:            # an MJCF file's contacts and joint rows under the native laws instead of MuJoCo's
+        flags |= nk.SCENE_NATIVE_CONTACT_LAW | nk.SCENE_NATIVE_JOINT_LAW
+    scene = nk.Scene(args.scene, flags)
     E = args.envs or 4096
     device = nk.Device(0)
     world = nk.World(device, scene, nk.abi.world_desc(E, 0.0, vel_iters=8))
@@ -104,7 +107,8 @@ def scene_run(nk, args):
         "warmup": args.settle, "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{os.path.basename(args.scene)}: {nl} links, {world.dof} DoF, {world.info.contact_slots_per_env} contact slots, "
-                               f"{E} envs, free-running after {args.settle} settling steps", "envs": E, "execution": args.mode,
+                               f"{E} envs, free-running after {args.settle} settling steps" + (", native contact and joint laws" if args.native_laws else ""),
+                   "envs": E, "execution": args.mode,
                    "event_ms_per_step": event_ms, "failed_envs": failed, "contacts_mean": float(world.download("contact_count").mean()),
                    "sweeps_mean": float(sweeps.mean()), "envs_using_every_sweep": int((sweeps == sweeps.max()).sum())},
         "per_op_ms": {k: round(v, 4) for k, v in per_op.items() if v >= 0.001},
@@ -243,6 +247,8 @@ def main():
     ap.add_argument("--seeded-only", action="store_true",
                     help="kept for the profile commands: every launch of a run is a step from the seeded batch")
     ap.add_argument("--scene", default="", help="a scene file instead of a benchmark configuration: its robot left to itself (see scene_run)")
+    ap.add_argument("--native-laws", action="store_true",
+                    help="with --scene: the file's contacts and joint rows under the native laws (an MJCF file's are MuJoCo's by default)")
     ap.add_argument("--settle", type=int, default=600)
     ap.add_argument("--base-height", type=float, default=0.0, help="with --scene: height of the root link at the start, 0 keeps the file's")
     args = ap.parse_args()
