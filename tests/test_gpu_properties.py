@@ -208,6 +208,18 @@ def test_rope_full_batch_steps(device):
     world.close()
 
 
+def test_a_world_reports_the_width_and_the_occupancy_of_its_solve(device):
+    """What the benchmark line quotes as `solver_width` and `blocks_per_cu`: the humanoid's contacts reach the root and the
+    legs (18 coordinates), so its sweeps run 20 wide, eight blocks a compute unit like the quadruped's; the rope's block
+    is 64 wide, keeps no contact rows and runs four a unit (one wavefront a SIMD); a world without contacts has no solve."""
+    expected = {1: (7, 0), 2: (18, 8), 3: (20, 8), 5: (64, 4)}
+    for index, (width, blocks) in expected.items():
+        cfg = nk.synthetic.config(index, 8)
+        world = nk.World(device, cfg.template, abi.world_desc(8, cfg.dt, vel_iters=cfg.vel_iters))
+        assert (world.info.solver_width, world.info.solver_blocks_per_cu) == (width, blocks), f"config {index}"
+        world.close()
+
+
 def test_single_environment_and_contact_free_worlds(oracle_py, device):
     for index in (1, 3):
         cfg = nk.synthetic.config(index, 1)
