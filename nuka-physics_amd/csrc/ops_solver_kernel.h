@@ -2262,10 +2262,13 @@ __device__ __forceinline__ bool reduce_block(uint32_t lane, uint32_t n, const fl
     }
 #pragma unroll
     for (int i = 0; i < kFollowers; ++i) column[i] = corner[i * kFollowers + int(slot)];
+    // Column by column (the columns do not meet in the substitution).  A column of the coupling that is zero in every
+    // follower's row stays zero - a leg's coordinate and an arm's share no link - and is left out, on a uniform test.
 #pragma unroll
-    for (int i = K; i < N; ++i) {
+    for (int c0 = 0; c0 < K; ++c0) {
+        if (__ballot(lane >= uint32_t(K) && lane < uint32_t(N) && prow[c0] != 0.0) == 0ull) continue;
 #pragma unroll
-        for (int c0 = 0; c0 < K; ++c0) {
+        for (int i = K; i < N; ++i) {
             const double y = lane_value_d(prow[c0] * own_scale, i);
             prow[c0] = at > uint32_t(i) ? fma(-column[i - K], y, prow[c0]) : prow[c0];
         }
@@ -2327,7 +2330,9 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     float mrow[W], mlow[W];
     bool reduction_valid = true;
     if constexpr (kReduced) {
+        PROF_BEGIN(c, 30);
         reduction_valid = reduce_block<N, K>(lane, n, d.m + size_t{env} * md * md + size_t{lane < n ? lane : 0u} * md, md, lds, mrow, mlow);
+        PROF_END(c, 30);
     } else {
 #pragma unroll
         for (int k = 0; k < W; ++k) mlow[k] = 0.0f;   // never read
