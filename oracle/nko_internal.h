@@ -99,6 +99,7 @@ struct nko_world {
     nko_world_desc cfg;
     uint32_t env_count;
     int threads;
+    int line_rule;   /* nko_world_set_line_rule */
     uint64_t step_index;
     /* env-major state */
     float *q, *qdot, *qddot, *tau, *base_pose, *link_pose, *link_velocity, *link_acceleration, *link_wrench;

@@ -579,6 +579,9 @@ static void line_derivatives(tile* c, float alpha, float inertial_slope, float i
         tile_add_product(&row_slope, f.y, t->step.y);
         tile_add_product(&row_slope, f.z, t->step.z);
         row_magnitude += fabsf(f.x * t->step.x) + fabsf(f.y * t->step.y) + fabsf(f.z * t->step.z);
+        if (c->w->line_rule != 0)   /* not the reference's: nko_world_set_line_rule */
+            row_magnitude += r[0] * (fabsf(t->residual.x) + fabsf(trial.x)) * fabsf(t->step.x) + r[1] * (fabsf(t->residual.y) + fabsf(trial.y)) * fabsf(t->step.y) +
+                             r[2] * (fabsf(t->residual.z) + fabsf(trial.z)) * fabsf(t->step.z);
         row_curvature += r[0] * t->step.x * t->step.x + r[1] * t->step.y * t->step.y + r[2] * t->step.z * t->step.z +
                          2.0f * r[5] * t->step.y * t->step.z + 2.0f * r[3] * t->step.x * t->step.y + 2.0f * r[4] * t->step.x * t->step.z;
     }

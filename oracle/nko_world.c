@@ -406,6 +406,7 @@ const char* nko_world_field_names(void) {
 }
 
 void nko_world_set_threads(nko_world* w, int threads) { w->threads = threads > 0 ? threads : 1; }
+void nko_world_set_line_rule(nko_world* w, int rule) { w->line_rule = rule != 0 ? 1 : 0; }
 /* bytes of the scalar type of this build: 4, or 8 for the double-precision build */
 uint32_t nko_real_bytes(void) { return (uint32_t)sizeof(float); }
 uint32_t nko_world_dof(const nko_world* w) { return w->t.nv; }

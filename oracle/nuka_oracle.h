@@ -149,6 +149,11 @@ int nko_world_field(nko_world* w, const char* name, void** ptr, size_t* bytes);
 /* Comma-separated list of the field names nko_world_field serves. */
 const char* nko_world_field_names(void);
 void nko_world_set_threads(nko_world* w, int threads);
+/* The line search's stopping rule.  0 (the default): the reference's (SearchTileLine, block_descent_tile.cuh:2089-2125),
+ * whose rounding magnitude counts the heads' responses.  1: the magnitude also counts the rounding of the heads'
+ * residuals, curvature x (|residual| + |move|) x |step| a head axis - the rule the HIP kernels apply - so that a test
+ * can tell the kernels' arithmetic from that one deliberate difference. */
+void nko_world_set_line_rule(nko_world* w, int rule);
 uint32_t nko_real_bytes(void);
 uint32_t nko_world_dof(const nko_world* w);
 uint32_t nko_world_rows_per_env(const nko_world* w);

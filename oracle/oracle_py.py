@@ -53,6 +53,7 @@ def _declare_world_entry_points(L):
     L.nko_world_field.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t)]
     L.nko_world_field_names.restype = C.c_char_p
     L.nko_world_set_threads.argtypes = [C.c_void_p, C.c_int]
+    L.nko_world_set_line_rule.argtypes = [C.c_void_p, C.c_int]
     L.nko_world_dof.argtypes = [C.c_void_p]
     L.nko_world_dof.restype = C.c_uint32
     L.nko_world_rows_per_env.argtypes = [C.c_void_p]
@@ -111,6 +112,7 @@ def lib():
         L.nko_world_field.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t)]
         L.nko_world_field_names.restype = C.c_char_p
         L.nko_world_set_threads.argtypes = [C.c_void_p, C.c_int]
+        L.nko_world_set_line_rule.argtypes = [C.c_void_p, C.c_int]
         L.nko_world_dof.argtypes = [C.c_void_p]
         L.nko_world_dof.restype = C.c_uint32
         L.nko_world_rows_per_env.argtypes = [C.c_void_p]
@@ -146,6 +148,10 @@ class OracleWorld:
         self.link_count = template.link_count
         self.dof = L.nko_world_dof(self._h)
         self.rows_per_env = L.nko_world_rows_per_env(self._h)
+
+    def set_line_rule(self, rule):
+        """1: the line search stops by the rule of the HIP kernels instead of the reference's (nuka_oracle.h)."""
+        self._lib.nko_world_set_line_rule(self._h, int(rule))
 
     def close(self):
         if self._h:

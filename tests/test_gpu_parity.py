@@ -303,6 +303,36 @@ def distances_to_double(oracle_py, device, index, E):
     return out, sweeps, int(same.sum())
 
 
+@pytest.mark.parametrize("index,E", [(2, 512), (3, 512)])
+def test_the_kernels_line_rule_in_the_oracle_changes_nothing_that_is_compared(oracle_py, device, index, E):
+    """The kernels' line search stops by a rule that is not the reference's (its rounding magnitude also counts the
+    heads' residuals).  The oracle switched to that rule must stand to the device as the oracle under the reference's
+    rule does: sweep counts equal on at least 99 % of the environments either way, velocities within the bar either way."""
+    cfg = nk.synthetic.config(index, E)
+    desc = nk.abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters)
+    state = cfg.state()
+    world = nk.World(device, cfg.template, desc)
+    world.set_state(state)
+    for name in UPSTREAM + ["BlockDescentSolve"]:
+        world.op(name)
+    world.synchronize()
+    got, sweeps = world.download("qdot_flat").reshape(E, -1), world.download("vbd_velocity_sweep_count").astype(int)
+    for rule in (0, 1):
+        oracle = oracle_py.OracleWorld(cfg.template, desc, threads=8)
+        oracle.set_line_rule(rule)
+        oracle.set_state(state)
+        for name in UPSTREAM + ["BlockDescentSolve"]:
+            oracle.op(*ORACLE_OPS[name])
+        expect, taken = oracle.download("qdot_flat").reshape(E, -1), oracle.download("vbd_velocity_sweep_count").astype(int)
+        equal = sweeps == taken
+        error = np.abs(got - expect).max(1) / np.maximum(np.abs(expect).max(1), 1e-6)
+        print(f"config {index}, line rule {rule}: sweep counts equal on {equal.mean():.4f}, velocity worst {error[equal].max():.2e}")
+        assert equal.mean() >= 0.99 and np.abs(sweeps - taken).max() <= 1
+        assert error[equal].max() <= TOL
+        oracle.close()
+    world.close()
+
+
 @pytest.mark.parametrize("index,E", [(2, 512), (3, 512), (5, 64)])
 def test_the_device_is_as_close_to_the_double_precision_answer_as_the_oracle(oracle_py, device, index, E):
     """The bars above that exceed 1e-4 rest on the single-precision oracle's own sensitivity; this is the measure
