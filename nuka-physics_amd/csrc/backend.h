@@ -21,8 +21,9 @@ void InitContactKernels();
 uint32_t SolverHeadCapacity(const ModelView& m, uint32_t slots, size_t lds_budget_bytes);
 // the width the sweeps of the world's block-descent solve run at: its coordinates, or fewer for a reduced block
 uint32_t SolverSweepWidth(const ModelView& m);
-// blocks of the world's full-capacity solve launch that one compute unit holds at once (runtime occupancy query)
-uint32_t SolverBlocksPerUnit(const ModelView& m);
+// blocks of the world's full-capacity solve launch that one compute unit holds at once (runtime occupancy query for
+// the kernel a batch of `env_count` environments takes)
+uint32_t SolverBlocksPerUnit(const ModelView& m, uint32_t env_count);
 // words per environment of DataView::solver_mass_factor: the solve's factor of the mass matrix where its block is too
 // wide to keep it in LDS, else none
 uint32_t SolverMassFactorFloats(const ModelView& m);

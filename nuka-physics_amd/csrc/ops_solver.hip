@@ -19,6 +19,17 @@ NKH_DECLARE_REDUCED(24, 12) NKH_DECLARE_REDUCED(28, 16) NKH_DECLARE_REDUCED(32, 
 NKH_DECLARE_REDUCED(44, 24) NKH_DECLARE_REDUCED(48, 24) NKH_DECLARE_REDUCED(52, 28) NKH_DECLARE_REDUCED(56, 28) NKH_DECLARE_REDUCED(60, 32)
 NKH_DECLARE_REDUCED(64, 32)
 #undef NKH_DECLARE_REDUCED
+// The dense build of the same template (ops_solver_kernel.h compiled with NKH_SOLVER_DENSE: three waves a SIMD), for the
+// widths it is instantiated at in ops_solver_d*.hip.
+namespace dense {
+template <int N, bool kContactsOnly, int K = N>
+__global__ void BlockDescentTileKernel(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+#define NKH_DECLARE_DENSE(N, K) \
+    extern template __global__ void BlockDescentTileKernel<N, true, K>(ModelView, DataView, BlockDescentSolveParams, uint32_t, uint32_t, uint32_t, uint32_t);
+NKH_DECLARE_DENSE(4, 4) NKH_DECLARE_DENSE(8, 8) NKH_DECLARE_DENSE(12, 12) NKH_DECLARE_DENSE(16, 16) NKH_DECLARE_DENSE(20, 20)
+NKH_DECLARE_DENSE(24, 12) NKH_DECLARE_DENSE(28, 16) NKH_DECLARE_DENSE(32, 16) NKH_DECLARE_DENSE(36, 20) NKH_DECLARE_DENSE(40, 20)
+#undef NKH_DECLARE_DENSE
+}  // namespace dense
 }  // namespace solver
 
 
@@ -97,6 +108,22 @@ const ReducedKernel kReducedKernels[] = {
     {36u, 20u, BlockDescentTileKernel<36, true, 20>}, {40u, 20u, BlockDescentTileKernel<40, true, 20>}, {44u, 24u, BlockDescentTileKernel<44, true, 24>},
     {48u, 24u, BlockDescentTileKernel<48, true, 24>}, {52u, 28u, BlockDescentTileKernel<52, true, 28>}, {56u, 28u, BlockDescentTileKernel<56, true, 28>},
     {60u, 32u, BlockDescentTileKernel<60, true, 32>}, {64u, 32u, BlockDescentTileKernel<64, true, 32>}};
+// The dense kernels: (padded width of the block, width of the sweeps), contact heads only.
+const ReducedKernel kDenseKernels[] = {
+    {4u, 4u, dense::BlockDescentTileKernel<4, true, 4>}, {8u, 8u, dense::BlockDescentTileKernel<8, true, 8>},
+    {12u, 12u, dense::BlockDescentTileKernel<12, true, 12>}, {16u, 16u, dense::BlockDescentTileKernel<16, true, 16>},
+    {20u, 20u, dense::BlockDescentTileKernel<20, true, 20>}, {24u, 12u, dense::BlockDescentTileKernel<24, true, 12>},
+    {28u, 16u, dense::BlockDescentTileKernel<28, true, 16>}, {32u, 16u, dense::BlockDescentTileKernel<32, true, 16>},
+    {36u, 20u, dense::BlockDescentTileKernel<36, true, 20>}, {40u, 20u, dense::BlockDescentTileKernel<40, true, 20>}};
+// Batches from this many environments on take a dense kernel where there is one: twice the 3072 wave slots three waves
+// a SIMD make of 256 compute units.  A dense wave runs slower than a two-wave one (fewer registers, some spilled), so
+// below that the launch is over sooner with the two-wave kernel: its length is then the longest environment's, not the
+// machine's throughput.  Measured on the 36-coordinate humanoid: 4096 environments +9 % with the dense kernel, 5120
+// +1 %, 6144 -8 %, 8192 -8 %, 65536 -9 %; the 18-coordinate quadruped -9 % at 6144 and -14 % at 65536.
+#ifndef NKH_DENSE_BATCH
+#define NKH_DENSE_BATCH 6144
+#endif
+constexpr uint32_t kDenseBatch = NKH_DENSE_BATCH;
 }  // namespace
 
 void InitSolverKernels() {
@@ -108,6 +135,10 @@ void InitSolverKernels() {
     }
     for (const ReducedKernel& reduced : kReducedKernels) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(reduced.kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipGetLastError();
+    }
+    for (const ReducedKernel& dense : kDenseKernels) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(dense.kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         (void)hipGetLastError();
     }
 }
@@ -127,7 +158,15 @@ static bool ContactHeadsOnly(const ModelView& m, uint32_t staged) {
     const uint32_t joint_heads = m.joint_limit_rows + m.joint_friction_rows + m.joint_drive_rows;
     return joint_heads == 0u && staged <= uint32_t(solver::kWave) && !(m.any_mujoco != 0u && m.contact_cone == 1u);
 }
-static SolverKernel KernelOfWidth(const ModelView& m, bool contacts_only, uint32_t width) {
+// `dense_out`: whether the kernel is a dense one (three waves a SIMD)
+static SolverKernel KernelOfWidth(const ModelView& m, bool contacts_only, uint32_t width, uint32_t env_count, bool* dense_out = nullptr) {
+    if (dense_out != nullptr) *dense_out = false;
+    if (contacts_only && env_count >= kDenseBatch)
+        for (const ReducedKernel& dense : kDenseKernels)
+            if (dense.width == solver::PaddedWidth(m.dof) && dense.reduced == solver::PaddedWidth(width) && (width == m.dof || dense.reduced == width)) {
+                if (dense_out != nullptr) *dense_out = true;
+                return dense.kernel;
+            }
     if (width != m.dof)
         for (const ReducedKernel& reduced : kReducedKernels)
             if (reduced.width == solver::PaddedWidth(m.dof) && reduced.reduced == width) return reduced.kernel;
@@ -135,7 +174,7 @@ static SolverKernel KernelOfWidth(const ModelView& m, bool contacts_only, uint32
 }
 // Blocks (one wavefront, one environment each) of a world's full-capacity solve launch that a compute unit holds at
 // once, as the runtime's occupancy query answers for the kernel and the LDS the launch asks for; 0 without a solve.
-uint32_t SolverBlocksPerUnit(const ModelView& m) {
+uint32_t SolverBlocksPerUnit(const ModelView& m, uint32_t env_count) {
     if (m.rows_per_env == 0u || m.dof == 0u) return 0u;
     const uint32_t staged = SolverHeadCapacity(m, std::max(m.contact_slots, 1u), 150u * 1024u);
     if (staged == 0u) return 0u;
@@ -145,7 +184,7 @@ uint32_t SolverBlocksPerUnit(const ModelView& m) {
     const size_t lds = size_t{solver::ReducedSolverLdsFloats(m.dof, width, staged + joint_heads, staged,
                                                              solver::RowsFromLinks(width, contacts_only, m.rows_from_links))} * sizeof(float);
     int blocks = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, reinterpret_cast<const void*>(KernelOfWidth(m, contacts_only, width)),
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, reinterpret_cast<const void*>(KernelOfWidth(m, contacts_only, width, env_count)),
                                                      solver::kWave, lds) != hipSuccess) {
         (void)hipGetLastError();
         return 0u;
@@ -179,22 +218,24 @@ Status OpBlockDescentSolve(const ModelView& m, const DataView& d, const void* pa
         return size_t{solver::ReducedSolverLdsFloats(m.dof, width, contact_heads + joint_heads, contact_heads,
                                                      solver::RowsFromLinks(width, contacts_only, m.rows_from_links))} * sizeof(float);
     };
-    // widths past kTwoWaveWidth run one wave a SIMD: four blocks a compute unit at most, whatever their LDS
-    const size_t most_blocks = solver::PaddedWidth(width) > uint32_t(solver::kTwoWaveWidth) ? 4u : 8u;
+    bool dense = false;
+    const SolverKernel kernel = KernelOfWidth(m, contacts_only, width, p->env_count, &dense);
+    // widths past kTwoWaveWidth run one wave a SIMD: four blocks a compute unit at most, whatever their LDS; the dense
+    // kernels run three, twelve blocks
+    const size_t most_blocks = dense ? 12u : solver::PaddedWidth(width) > uint32_t(solver::kTwoWaveWidth) ? 4u : 8u;
     const auto blocks_per_unit = [&](uint32_t contact_heads) { return std::min<size_t>(most_blocks, (160u * 1024u) / lds_bytes(contact_heads)); };
     // The LDS a block needs grows with the contact heads it can stage, and a scene's slots (every pair that may ever
     // touch, at its largest manifold) outnumber the contacts an environment usually has.  Where a smaller capacity
     // lets more blocks share a compute unit, environments with few contact points go to a launch of that capacity:
     // up to three such launches, for eight, four and two blocks a unit, before the full one.  Each launch takes the
     // environments whose contact points fall in its range; an environment's results do not depend on its launch.
-    const SolverKernel kernel = KernelOfWidth(m, contacts_only, width);
     hipLaunchKernelGGL(OrderTilesKernel, dim3(1), dim3(1024), 0, stream, d, p->env_count);
     uint32_t first_points = 0u;
     // (a launch takes its environments by their contact points, one head a point: not under the pyramidal cone, whose
     // worlds go to the one full launch)
     const bool one_head_a_point = !(m.any_mujoco != 0u && m.contact_cone == 0u);
     if (p->contact_slots_per_env != 0u && one_head_a_point) {
-        for (const size_t blocks : {size_t{8u}, size_t{4u}, size_t{2u}}) {
+        for (const size_t blocks : {size_t{12u}, size_t{8u}, size_t{4u}, size_t{2u}}) {
             if (blocks > most_blocks) continue;                            // more blocks than the waves allow
             if (blocks_per_unit(staged) >= blocks) break;                  // the full capacity does as well
             uint32_t few = staged;

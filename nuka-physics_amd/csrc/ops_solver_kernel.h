@@ -28,6 +28,14 @@
 
 namespace nkh {
 namespace solver {
+// This header compiles two ways.  Plainly, a block of up to kTwoWaveWidth coordinates runs two waves a SIMD with up to 256
+// registers each.  With NKH_SOLVER_DENSE defined (ops_solver_d*.hip) everything below sits in namespace `dense` and a block
+// of up to kThreeWaveWidth coordinates is compiled for three waves a SIMD: 168 registers, a few dozen values a lane in
+// scratch memory, the same arithmetic.  A long environment runs a tenth slower that way and a full machine gets a tenth
+// more done, so the launcher takes the dense kernels for batches that fill the machine several times over.
+#ifdef NKH_SOLVER_DENSE
+namespace dense {
+#endif
 
 constexpr int kWave = 64;
 // Widths up to this run two waves per SIMD (at most 256 registers each); wider rows need the whole register file.
@@ -35,6 +43,13 @@ constexpr int kWave = 64;
 #define NKH_TWO_WAVE_WIDTH 36
 #endif
 constexpr int kTwoWaveWidth = NKH_TWO_WAVE_WIDTH;
+// Widths up to this run three waves per SIMD in the dense build (none in the plain one).
+#ifdef NKH_SOLVER_DENSE
+constexpr int kThreeWaveWidth = 20;
+#else
+constexpr int kThreeWaveWidth = 0;
+#endif
+constexpr int WavesPerSimd(int width) { return width <= kThreeWaveWidth ? 3 : (width <= kTwoWaveWidth ? 2 : 1); }
 // From this width on a block widens its mass rows to double where it uses them; below it the widened rows are kept over
 // the solve (two registers an entry), which pays while they fit.
 #ifndef NKH_WIDEN_AT_USE
@@ -593,6 +608,52 @@ __device__ __forceinline__ uint32_t lds_address(const float* p) {
 // come from LDS (`kFirst`, `kSecond`, `kThird` bytes past `row_address`) into twelve registers that the block takes for
 // itself, v244-v255.  Only for widths that run two waves a SIMD: their kernels leave those registers free.  The waits
 // count LDS reads only as far as those return in order; scalar loads in flight make them wait longer, never shorter.
+#ifdef NKH_SOLVER_DENSE   // the same block on registers inside the dense build's 168: v152-v163
+template <int kFirst, int kSecond, int kThird>
+__device__ __forceinline__ void add_columns_if(uint32_t live, uint32_t single, uint32_t row_address, float a0, float a1, float a2, float& h0,
+                                               float& h1, float& h2, float& h3) {
+    asm volatile(
+        "s_cmp_eq_u32 %[live], 0\n\t"
+        "s_cbranch_scc1 .Lcolumns_done_%=\n\t"
+        "s_cmp_eq_u32 %[single], 0\n\t"
+        "s_cbranch_scc0 .Lcolumns_single_%=\n\t"
+        "ds_read_b128 v[152:155], %[at] offset:%[first]\n\t"
+        "ds_read_b128 v[156:159], %[at] offset:%[second]\n\t"
+        "ds_read_b128 v[160:163], %[at] offset:%[third]\n\t"
+        "s_waitcnt lgkmcnt(2)\n\t"
+        "v_mul_f32 v152, %[a0], v152\n\t"
+        "v_mul_f32 v153, %[a0], v153\n\t"
+        "v_mul_f32 v154, %[a0], v154\n\t"
+        "v_mul_f32 v155, %[a0], v155\n\t"
+        "s_waitcnt lgkmcnt(1)\n\t"
+        "v_fmac_f32 v152, %[a1], v156\n\t"
+        "v_fmac_f32 v153, %[a1], v157\n\t"
+        "v_fmac_f32 v154, %[a1], v158\n\t"
+        "v_fmac_f32 v155, %[a1], v159\n\t"
+        "s_waitcnt lgkmcnt(0)\n\t"
+        "v_fmac_f32 v152, %[a2], v160\n\t"
+        "v_fmac_f32 v153, %[a2], v161\n\t"
+        "v_fmac_f32 v154, %[a2], v162\n\t"
+        "v_fmac_f32 v155, %[a2], v163\n\t"
+        "v_add_f32 %[h0], %[h0], v152\n\t"
+        "v_add_f32 %[h1], %[h1], v153\n\t"
+        "v_add_f32 %[h2], %[h2], v154\n\t"
+        "v_add_f32 %[h3], %[h3], v155\n\t"
+        "s_branch .Lcolumns_done_%=\n"
+        ".Lcolumns_single_%=:\n\t"
+        "ds_read_b128 v[152:155], %[at] offset:%[first]\n\t"
+        "s_waitcnt lgkmcnt(0)\n\t"
+        "v_fmac_f32 %[h0], %[a0], v152\n\t"
+        "v_fmac_f32 %[h1], %[a0], v153\n\t"
+        "v_fmac_f32 %[h2], %[a0], v154\n\t"
+        "v_fmac_f32 %[h3], %[a0], v155\n"
+        ".Lcolumns_done_%=:"
+        : [h0] "+v"(h0), [h1] "+v"(h1), [h2] "+v"(h2), [h3] "+v"(h3)
+        : [live] "s"(live), [single] "s"(single), [at] "v"(row_address), [a0] "v"(a0), [a1] "v"(a1), [a2] "v"(a2), [first] "n"(kFirst),
+          [second] "n"(kSecond), [third] "n"(kThird)
+        : "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", "v163", "scc");
+}
+#else
 template <int kFirst, int kSecond, int kThird>
 __device__ __forceinline__ void add_columns_if(uint32_t live, uint32_t single, uint32_t row_address, float a0, float a1, float a2, float& h0,
                                                float& h1, float& h2, float& h3) {
@@ -637,6 +698,7 @@ __device__ __forceinline__ void add_columns_if(uint32_t live, uint32_t single, u
           [second] "n"(kSecond), [third] "n"(kThird)
         : "v244", "v245", "v246", "v247", "v248", "v249", "v250", "v251", "v252", "v253", "v254", "v255", "scc");
 }
+#endif
 template <int N, int... Q>
 __device__ __forceinline__ void add_column_groups(std::integer_sequence<int, Q...>, uint64_t columns, uint32_t single, uint32_t row_address,
                                                   float a0, float a1, float a2, float (&hrow)[N]) {
@@ -2286,7 +2348,7 @@ __device__ __forceinline__ bool reduce_block(uint32_t lane, uint32_t n, const fl
 // K < N is a reduced block (described above mass_times): no contact of the world reaches the coordinates K..n-1, which are
 // eliminated once in the set-up, and the sweeps run K wide.  K is a multiple of 4 with K <= n, contact heads only.
 template <int N, bool kContactsOnly, int K = N>
-__global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(K <= kTwoWaveWidth ? 2 : 1, K <= kTwoWaveWidth ? 2 : 1)))
+__global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(WavesPerSimd(K), WavesPerSimd(K))))
 BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint32_t cap, uint32_t staged_cap, uint32_t points_lo,
                        uint32_t points_hi) {
     constexpr bool kReduced = K < N;
@@ -3015,5 +3077,8 @@ BlockDescentTileKernel(ModelView m, DataView d, BlockDescentSolveParams p, uint3
     }
 }
 
+#ifdef NKH_SOLVER_DENSE
+}  // namespace dense
+#endif
 }  // namespace solver
 }  // namespace nkh

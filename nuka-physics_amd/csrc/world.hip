@@ -1539,7 +1539,7 @@ nuka_result_t nuka_world_get_info(nuka_world_handle world, nuka_world_info_t* ou
     if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
     const ModelView& m = w->model;
     *out = {w->env_count, m.links_per_env, m.bodies_per_env, m.dof, m.max_dof, m.contact_slots, m.rows_per_env, uint32_t(w->calls.size()),
-            SolverSweepWidth(m), SolverBlocksPerUnit(m)};
+            SolverSweepWidth(m), SolverBlocksPerUnit(m, w->env_count)};
     return NUKA_RESULT_OK;
 }
 

@@ -171,3 +171,44 @@ def test_steps_of_reduced_blocks_stay_with_the_oracle(oracle_py, device, dof, fl
             close(world, oracle, name, tol=TOL if step == 0 else 3 * TOL)
     world.close()
     oracle.close()
+
+
+# (coordinates, floating root, joints a limb, limbs that carry spheres or None, width of the sweeps): every kernel of
+# the dense build, full blocks up to 20 coordinates and the reduced blocks that sweep at up to 20
+DENSE = [(4, False, 7, None, 4), (8, True, 7, None, 8), (11, True, 7, None, 11), (16, False, 7, None, 16), (20, True, 7, None, 20),
+         (24, True, 6, 1, 12), (28, True, 7, 1, 16), (32, True, 7, 1, 16), (36, True, 7, 2, 20), (40, True, 7, 2, 20)]
+
+
+@pytest.mark.parametrize("dof,floating,limb_joints,sphere_limbs,width", DENSE)
+def test_large_batches_take_the_dense_kernels_and_give_the_same_bits(oracle_py, device, dof, floating, limb_joints, sphere_limbs, width):
+    """From 6144 environments on, worlds of contact heads only whose sweeps are at most 20 wide run the kernels compiled
+    for three waves a SIMD (twelve blocks a compute unit instead of eight).  They are the same arithmetic in fewer
+    registers: a batch of 6144 made of 128 copies of 48 seeded environments must give, in every copy, the bits the 48
+    give alone with the two-wave kernel, and those stay with the oracle."""
+    E, copies = 48, 128
+    tree, desc, state = tree_case(oracle_py, dof, floating, True, seed=5 * dof + 1, E=E, limb_joints=limb_joints, sphere_limbs=sphere_limbs)
+    small = nk.World(device, tree.template, desc)
+    assert small.dof == dof and small.info.solver_width == width and small.info.solver_blocks_per_cu == 8
+    small.set_state(state)
+    small.step()
+    small.synchronize()
+    big_desc = nk.abi.world_desc(E * copies, 1.0 / 240.0, vel_iters=8, contact_margin=0.1)
+    big = nk.World(device, tree.template, big_desc)
+    assert big.info.solver_width == width and big.info.solver_blocks_per_cu > 8, big.info.solver_blocks_per_cu
+    big.set_state({k: np.tile(v, (copies, 1)) for k, v in state.items()})
+    big.step()
+    big.synchronize()
+    assert (small.download("contact_count") > 0).mean() >= 0.4, "the case must exercise the contact solve"
+    for name in ("qdot", "q", "lambda", "link_velocity", "vbd_velocity_sweep_count", "env_status"):
+        alone = small.download(name).reshape(1, -1)
+        batch = big.download(name).reshape(copies, -1)
+        assert np.array_equal(np.broadcast_to(alone, batch.shape), batch), name
+    small.close()
+    small = nk.World(device, tree.template, desc)       # and the two-wave kernel's results against the oracle's, op by op
+    small.set_state(state)
+    oracle = oracle_py.OracleWorld(tree.template, desc, threads=8)
+    oracle.set_state(state)
+    compare_ops(oracle, small, E, one_ulp_sensitivity(oracle_py, tree.template, desc, state), state)
+    small.close()
+    big.close()
+    oracle.close()
