@@ -51,9 +51,14 @@ constexpr int kThreeWaveWidth = 0;
 #endif
 constexpr int WavesPerSimd(int width) { return width <= kThreeWaveWidth ? 3 : (width <= kTwoWaveWidth ? 2 : 1); }
 // From this width on a block widens its mass rows to double where it uses them; below it the widened rows are kept over
-// the solve (two registers an entry), which pays while they fit.
+// the solve (two registers an entry), which pays while they fit.  In the dense build's 168 registers they never do:
+// kept, they are what spills (96 B a lane at 20 coordinates, none widened at use; 65536 quadrupeds 6.74 -> 6.48 ms).
 #ifndef NKH_WIDEN_AT_USE
+#ifdef NKH_SOLVER_DENSE
+#define NKH_WIDEN_AT_USE 0
+#else
 #define NKH_WIDEN_AT_USE 24
+#endif
 #endif
 constexpr int kWidenAtUse = NKH_WIDEN_AT_USE;
 constexpr uint32_t kNewtonSteps = 16u;        // block_descent_dense.cuh:14
