@@ -353,11 +353,17 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
             }
         }
         __syncthreads();   // the second wavefront has the mass matrix in LDS
-        // the dense mass tile reaches HBM once, in row-major runs
+        // the dense mass tile reaches HBM once, in row-major runs (row and column of a lane's word step with it: a
+        // division by the stride a word costs more than the word)
         float* M = d.m + size_t{env} * stride * stride;
-        for (uint32_t e = lane; e < stride * stride; e += kWave) {
-            const uint32_t i = e / stride, j = e % stride;
-            M[e] = i < n && j < n ? A[i * ld + j] : 0.0f;
+        const uint32_t rows_a_step = uint32_t(kWave) / stride, columns_a_step = uint32_t(kWave) % stride;
+        {
+            uint32_t i = lane / stride, j = lane % stride;
+            for (uint32_t e = lane; e < stride * stride; e += kWave) {
+                M[e] = i < n && j < n ? A[i * ld + j] : 0.0f;
+                i += rows_a_step; j += columns_a_step;
+                if (j >= stride) { j -= stride; ++i; }
+            }
         }
         __syncthreads();   // ... and may now overwrite it with the factor
     } else {
@@ -432,7 +438,9 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
         __syncthreads();   // the mass matrix stands in LDS: the first wavefront carries it to HBM while this one factors it
         // LDL^T, right-looking, lane = row in registers; the strict lower triangle becomes L and the diagonal D (:269-335).
         // Rows and columns n..N-1 are those of the identity.  Entry (i, j) loses (L_ik L_jk) D_k for k = 0, 1, ... as the
-        // serial loop does; what a lane computes above its diagonal is never read.
+        // serial loop does (the products in the reference's order: fused into one multiply-add an entry the factor
+        // differs in its last place, and of 4096 humanoids one then ends its eight sweeps 2e-4 from the oracle's);
+        // what a lane computes above its diagonal is never read.
         {
             // (every word read whether or not the lane keeps it, from a place inside the matrix: a read under a condition
             // compiles to a branch a word)
@@ -472,9 +480,12 @@ __global__ void __launch_bounds__(2 * kWave) ArticulationDynamicsKernel(ModelVie
     __syncthreads();   // the factor stands in LDS, and the right-hand side (first wavefront) meets it (second)
     if (forces) {
         float* factor = d.m_factor + size_t{env} * stride * stride;
+        const uint32_t rows_a_step = uint32_t(kWave) / stride, columns_a_step = uint32_t(kWave) % stride;
+        uint32_t i = lane / stride, j = lane % stride;
         for (uint32_t e = lane; e < stride * stride; e += kWave) {
-            const uint32_t i = e / stride, j = e % stride;
             if (j <= i) factor[e] = i < n ? A[i * ld + j] : (i == j ? 1.0e-6f : 0.0f);
+            i += rows_a_step; j += columns_a_step;
+            if (j >= stride) { j -= stride; ++i; }
         }
         return;
     }
