@@ -456,7 +456,9 @@ typedef struct nuka_world_info_t {
      * later coordinates and the solve eliminates those once per step */
     uint32_t solver_width;
     /* one-wavefront blocks of the contact solve's full-capacity launch that a compute unit (four SIMDs) holds at once,
-     * by the runtime's occupancy query for that kernel and its LDS; 0 for a world without a contact solve */
+     * by the runtime's occupancy query for that kernel and its LDS (a world of 6144 environments or more takes the
+     * kernels built for three waves a SIMD where there is one for its width: 12 instead of 8); 0 for a world without
+     * a contact solve */
     uint32_t solver_blocks_per_cu;
 } nuka_world_info_t;
 nuka_result_t nuka_world_get_info(nuka_world_handle world, nuka_world_info_t* out);

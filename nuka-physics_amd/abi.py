@@ -52,7 +52,7 @@ class TemplateDescC(C.Structure):
         ("contact_cone", C.c_uint32), ("contact_impratio", C.c_float),
         ("profile_priority", C.POINTER(C.c_int32)), ("profile_solmix", _PF), ("profile_condim", _PU),
         ("joint_law", _PB), ("joint_limit_margin", _PF), ("joint_limit_reference", _PF), ("joint_friction_reference", _PF),
-        ("integrator", C.c_uint32), ("reserved2", C.c_uint32),
+        ("integrator", C.c_uint32), ("free_body", C.c_uint32),
     ]
 
 
@@ -130,6 +130,7 @@ class Template:
         self.contact_cone = CONE_PYRAMIDAL   # friction cone of MuJoCo-law contacts (<option cone>)
         self.contact_impratio = 1.0          # <option impratio>
         self.integrator = INTEGRATOR_NATIVE  # <option integrator> of a MuJoCo-sourced scene
+        self.free_body = False    # True: the template's one link (floating root) is a free rigid body (rigid-body ops)
 
     def add_link(self, joint_type, parent, axis=(0, 0, 1), local_pos=(0, 0, 0), local_rot=(1, 0, 0, 0), mass=1.0,
                  diag_inertia=(0.01, 0.01, 0.01), com=(0, 0, 0), damping=0.0, armature=0.0, stiffness=0.0,
@@ -225,6 +226,7 @@ class Template:
         d.excluded_pair_count = len(self.excluded)
         d.contact_cone, d.contact_impratio = self.contact_cone, self.contact_impratio
         d.integrator = self.integrator
+        d.free_body = 1 if self.free_body else 0
         ctype = {np.dtype(np.float32): C.c_float, np.dtype(np.uint32): C.c_uint32, np.dtype(np.uint8): C.c_uint8, np.dtype(np.int32): C.c_int32}
         for name, arr in a.items():
             arr = np.ascontiguousarray(arr)

@@ -60,7 +60,8 @@ static float contact_query_reach(float thickness, float margin) { return fmaxf(0
 static float contact_motion_radius(float base, float dt, float sa, float sb, float relax) { return base + dt * (sa + sb) * (2.0f / relax); }
 
 /* ---- BuildAabbs (broadphase.cu:173-270). Link-owned collidables keep zero body velocity and
- * zero previous motion on this path (nothing writes them for inv_mass 0 rows), so speed = 0. ---- */
+ * zero previous motion on this path (nothing writes them for inv_mass 0 rows), so speed = 0; a free
+ * body's row carries the body's velocities. ---- */
 void nko_env_aabbs(nko_world* w, uint32_t env) {
     const nko_template* t = &w->t;
     const size_t bbase = (size_t)env * t->nb;
@@ -89,7 +90,13 @@ void nko_env_aabbs(nko_world* w, uint32_t env) {
             lo[0] = lo[1] = lo[2] = FLT_MAX; hi[0] = hi[1] = hi[2] = -FLT_MAX;
             continue;
         }
-        const float speed = 0.0f;
+        /* :262-264: a free body's own row moves with it - its speed, and its turning rate over the shape's radius */
+        float speed = 0.0f;
+        if (t->free_body && b == t->link_body[0]) {
+            const float* lv = w->body_linear_velocity + (size_t)env * 3u, *av = w->body_angular_velocity + (size_t)env * 3u;
+            const float radius = sqrtf(he.x * he.x + he.y * he.y + he.z * he.z) + sqrtf(0.0f);
+            speed = fmaxf(0.0f, sqrtf(lv[0] * lv[0] + lv[1] * lv[1] + lv[2] * lv[2]) + sqrtf(av[0] * av[0] + av[1] * av[1] + av[2] * av[2]) * radius);
+        }
         const float m = fmaxf(margin, fminf(contact_motion_radius(margin, w->cfg.fixed_dt, speed, 0.0f, 0.9f), reach));
         const v3 c = xf.p;
         lo[0] = c.x - he.x - m; lo[1] = c.y - he.y - m; lo[2] = c.z - he.z - m;
@@ -768,8 +775,20 @@ void nko_env_narrowphase(nko_world* w, uint32_t env) {
                 const float margin_b = has_b ? t->profile_margin[2u * sb.profile] + t->profile_margin[2u * sb.profile + 1u] : 0.0f;
                 query_margin = margin_a + margin_b;
             }
-            /* :243-250 query band; both speeds are zero for link-owned collidables */
-            const float query = fmaxf(query_margin, fminf(contact_motion_radius(2.0f * separation, w->cfg.fixed_dt, 0.0f, 0.0f, 0.9f), reach));
+            /* :236-250 query band; both speeds are zero for link-owned collidables, a free body's own row moves with it */
+            float speeds[2] = {0.0f, 0.0f};
+            const uint32_t ends[2] = {a, b};
+            for (uint32_t side = 0u; side < 2u && t->free_body; ++side) {
+                if (ends[side] != t->link_body[0]) continue;
+                const size_t at = bbase + ends[side];
+                const float* center = w->body_pose + at * 7u, *lo = w->body_aabb_lo + at * 3u, *hi = w->body_aabb_hi + at * 3u;
+                const v3 extent = v3_make(fmaxf(fabsf(lo[0] - center[0]), fabsf(hi[0] - center[0])), fmaxf(fabsf(lo[1] - center[1]), fabsf(hi[1] - center[1])),
+                                          fmaxf(fabsf(lo[2] - center[2]), fabsf(hi[2] - center[2])));
+                const float* lv = w->body_linear_velocity + (size_t)env * 3u, *av = w->body_angular_velocity + (size_t)env * 3u;
+                speeds[side] = fmaxf(0.0f, sqrtf(lv[0] * lv[0] + lv[1] * lv[1] + lv[2] * lv[2]) +
+                                           sqrtf((av[0] * av[0] + av[1] * av[1] + av[2] * av[2]) * (extent.x * extent.x + extent.y * extent.y + extent.z * extent.z)));
+            }
+            const float query = fmaxf(query_margin, fminf(contact_motion_radius(2.0f * separation, w->cfg.fixed_dt, speeds[0], speeds[1], 0.9f), reach));
             primitive_pair(sa.kind, &pa, sb.kind, &pb, query, &m);
             if (law != 0u) for (uint32_t i = 0u; i < m.count; ++i) m.penetration[i] += separation;   /* :295-296 */
         }
@@ -871,6 +890,20 @@ void nko_accumulate_chain(const nko_world* w, uint32_t env, uint32_t link_local,
     const nko_template* t = &w->t;
     const uint32_t stride = t->max_dof;
     const uint8_t type = t->joint_type[link_local];
+    if (type == NKO_FLOATING && t->free_body) {
+        /* a free body's six coordinates: its linear velocity, then its angular velocity about the centre of mass, in world
+         * axes - the row's jlin and jang = (point - com) x jlin (assemble_rows.cu:537-538, 680-681; TileBlock::Jacobian,
+         * block_descent_tile.cuh:556-563) */
+        float com[3];
+        nko_body_center_of_mass(w, env, com);
+        const v3 jang = v3_add(v3_cross(v3_sub(point, v3_make(com[0], com[1], com[2])), f), zero);
+        const float lin[3] = {f.x, f.y, f.z}, ang[3] = {jang.x, jang.y, jang.z};
+        for (uint32_t b = 0u; b < 3u; ++b) {
+            if (dof_index + b < stride) out[dof_index + b] += lin[b];
+            if (dof_index + 3u + b < stride) out[dof_index + 3u + b] += ang[b];
+        }
+        return;
+    }
     if (type == NKO_FLOATING) {
         const xform base = xform_load(w->base_pose + (size_t)env * 7u);
         const v3 lever = v3_sub(point, base.p);

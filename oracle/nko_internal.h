@@ -27,7 +27,7 @@ enum {
     NKO_ROW_MUJOCO = 1u << 11, NKO_ROW_PYRAMIDAL = 1u << 12, NKO_ROW_FRICTION = 1u << 1
 };
 /* phi/op_schema.hpp:36-52 */
-enum { NKO_STATUS_PAIR_OVERFLOW = 1u << 0, NKO_STATUS_DOF_OVERFLOW = 1u << 2, NKO_STATUS_INVALID_ENDPOINT = 1u << 6,
+enum { NKO_STATUS_PAIR_OVERFLOW = 1u << 0, NKO_STATUS_DOF_OVERFLOW = 1u << 2, NKO_STATUS_GYRO_FAILURE = 1u << 5, NKO_STATUS_INVALID_ENDPOINT = 1u << 6,
        NKO_STATUS_CONTROL_FAILURE = 1u << 10, NKO_STATUS_SOLVER_FAILURE = 1u << 13 };
 /* phi/articulation_contract.hpp:16-23 */
 enum { NKO_DRIVE_PD_POSITION = 0, NKO_DRIVE_TORQUE = 1, NKO_DRIVE_VELOCITY = 2, NKO_DRIVE_COMPUTED_TORQUE = 3,
@@ -92,6 +92,9 @@ typedef struct {
     uint32_t cone;                /* constraint::FrictionCone: 0 pyramidal, 1 elliptic */
     float impratio;
     int any_mujoco;
+    /* the template's one link is a free rigid body, stepped by the reference's rigid-body ops (nko_rigid.c) */
+    int free_body;
+    float body_mass, body_diag_inertia[3];
 } nko_template;
 
 struct nko_world {
@@ -106,6 +109,9 @@ struct nko_world {
     float *articulation_bias, *articulation_qdd, *m, *m_factor, *qdot_flat;
     float *qdot_pseudo, *link_velocity_pseudo;
     float *body_pose, *body_aabb_lo, *body_aabb_hi;
+    /* the free body of a free_body world, one an environment (fields.yaml:102-103, 569; articulation.cu:1068-1070) */
+    float *body_linear_velocity, *body_angular_velocity, *body_world_inv_inertia, *body_gyro_residual;
+    uint32_t *body_gyro_iterations, *body_gyro_status;
     uint32_t *candidate_pairs, *pair_count;
     uint32_t *ucontact_count, *ucontact_a, *ucontact_b, *ucontact_law, *ucontact_row_range;
     float *ucontact_point, *ucontact_normal, *ucontact_depth;
@@ -182,6 +188,10 @@ void nko_env_joint_rows(nko_world* w, uint32_t env);
 void nko_env_readout_contact_wrench(nko_world* w, uint32_t env);
 void nko_env_dynamics(nko_world* w, uint32_t env, uint32_t integrate_velocity);
 void nko_env_integrate_position(nko_world* w, uint32_t env);
+void nko_env_body_integrate_velocity(nko_world* w, uint32_t env);
+void nko_env_body_integrate_position(nko_world* w, uint32_t env);
+void nko_body_center_of_mass(const nko_world* w, uint32_t env, float out[3]);
+void nko_factor_mass(const float* mass, float* factor, uint32_t n, uint32_t stride);
 void nko_env_link_velocities(nko_world* w, uint32_t env);
 void nko_env_articulation_damping(nko_world* w, uint32_t env);
 void nko_env_reference_weights(nko_world* w, uint32_t env);

@@ -1,0 +1,243 @@
+/*
+ * CPU oracle (test infrastructure; see nuka_oracle.h): the free rigid body of a world whose template says free_body.
+ *
+ * The reference steps such a body with its own ops - BodyIntegrateVelocityKernel before the contact solve, a six by six
+ * block of the tile in it (block_descent_rigid.cuh, block_descent_tile.cuh:541-603), BodyIntegratePositionKernel with the
+ * free-rotation solve after it.  The body's coordinates are its linear velocity and its angular velocity about the
+ * centre of mass, both in world axes.  Here the body is the one link of the template: `base_pose` is the body's pose,
+ * `body_linear_velocity` / `body_angular_velocity` its state, and the six coordinates pass through the link's twist
+ * words (`link_velocity`: linear first, then angular) to the row assembly and the block descent, which take the block's
+ * mass matrix and factor from `m` / `m_factor` as they do for an articulation.
+ */
+#include "nko_internal.h"
+
+/* math/symmetric_mat3.hpp:31-47 FromRotatedDiagonal: R diag(d) R^T of the rotation of q, as xx yy zz xy xz yz */
+static void from_rotated_diagonal(v3 d, quat q, float out[6]) {
+    const float norm_sq = q.w * q.w + q.x * q.x + q.y * q.y + q.z * q.z;
+    const float s = norm_sq > 1.0e-12f ? 2.0f / norm_sq : 0.0f;
+    const v3 x = v3_make(1.0f - s * (q.y * q.y + q.z * q.z), s * (q.x * q.y - q.w * q.z), s * (q.x * q.z + q.w * q.y));
+    const v3 y = v3_make(s * (q.x * q.y + q.w * q.z), 1.0f - s * (q.x * q.x + q.z * q.z), s * (q.y * q.z - q.w * q.x));
+    const v3 z = v3_make(s * (q.x * q.z - q.w * q.y), s * (q.y * q.z + q.w * q.x), 1.0f - s * (q.x * q.x + q.y * q.y));
+    out[0] = d.x * x.x * x.x + d.y * x.y * x.y + d.z * x.z * x.z;
+    out[1] = d.x * y.x * y.x + d.y * y.y * y.y + d.z * y.z * y.z;
+    out[2] = d.x * z.x * z.x + d.y * z.y * z.y + d.z * z.z * z.z;
+    out[3] = d.x * x.x * y.x + d.y * x.y * y.y + d.z * x.z * y.z;
+    out[4] = d.x * x.x * z.x + d.y * x.y * z.y + d.z * x.z * z.z;
+    out[5] = d.x * y.x * z.x + d.y * y.y * z.y + d.z * y.z * z.z;
+}
+
+/* math/symmetric_mat3.hpp:25-29 Multiply */
+static v3 sym_multiply(const float* m, v3 v) {
+    return v3_make(m[0] * v.x + m[3] * v.y + m[4] * v.z, m[3] * v.x + m[1] * v.y + m[5] * v.z, m[4] * v.x + m[5] * v.y + m[2] * v.z);
+}
+
+/* nk/solve/vertex_block.hpp:139-153 Invert (floor 0): cofactors in double, rounded once */
+static int sym_invert(const float* m, float out[6]) {
+    const double xx = m[0], yy = m[1], zz = m[2], xy = m[3], xz = m[4], yz = m[5];
+    const double cxx = yy * zz - yz * yz, cyy = xx * zz - xz * xz;
+    const double czz = xx * yy - xy * xy, cxy = xz * yz - xy * zz;
+    const double cxz = xy * yz - xz * yy, cyz = xy * xz - xx * yz;
+    const double det = xx * cxx + xy * cxy + xz * cxz;
+    if (!(det > 0.0 && det <= DBL_MAX)) return 0;
+    const double inv = 1.0 / det;
+    const double values[6] = {cxx * inv, cyy * inv, czz * inv, cxy * inv, cxz * inv, cyz * inv};
+    for (uint32_t i = 0u; i < 6u; ++i) {
+        if (!(values[i] >= -FLT_MAX && values[i] <= FLT_MAX)) return 0;
+        out[i] = (float)values[i];
+    }
+    return 1;
+}
+
+/* rigid_types.cuh:10-14 BodyCenterOfMass, :16-21 BodyWorldInverseInertia */
+static v3 body_center_of_mass(xform pose, xform frame) { return v3_add(pose.p, nko_rotate_normalized(pose.r, frame.p)); }
+static void body_world_inverse_inertia(xform pose, xform frame, v3 inv_i, float out[6]) {
+    from_rotated_diagonal(inv_i, nko_quat_mul(pose.r, frame.r), out);
+}
+void nko_body_center_of_mass(const nko_world* w, uint32_t env, float out[3]) {
+    const v3 c = body_center_of_mass(xform_load(w->base_pose + (size_t)env * 7u), xform_load(w->t.link_inertial_frame));
+    out[0] = c.x; out[1] = c.y; out[2] = c.z;
+}
+
+static float max_abs(v3 v) { return fmaxf(fabsf(v.x), fmaxf(fabsf(v.y), fabsf(v.z))); }
+static int finite_vector(v3 v) { return isfinite(v.x) && isfinite(v.y) && isfinite(v.z); }
+
+/* rigid_types.cuh:38-121 SolveFreeRotation: the implicit midpoint rule of Euler's equations in the principal frame,
+ * on the angular momentum scaled to unit size, by Newton steps with halving; `midpoint` is the angular velocity at the
+ * middle of the step */
+typedef struct { v3 midpoint; float residual; uint32_t iterations, status; } gyro_result;
+static v3 gyro_residual(v3 u0, v3 c, v3 u) {
+    const v3 mid = v3_scale(v3_add(u0, u), 0.5f);
+    return v3_make(u.x - u0.x + c.x * mid.y * mid.z, u.y - u0.y + c.y * mid.z * mid.x, u.z - u0.z + c.z * mid.x * mid.y);
+}
+static gyro_result solve_free_rotation(v3 w0, v3 inv_i, float dt) {
+    gyro_result out;
+    memset(&out, 0, sizeof(out));
+    if (!finite_vector(w0) || !finite_vector(inv_i) || inv_i.x <= 0.0f || inv_i.y <= 0.0f || inv_i.z <= 0.0f) {
+        out.status = 2u; out.residual = INFINITY;   /* kBodyGyroInvalidInput */
+        return out;
+    }
+    const v3 m0 = v3_make(w0.x / inv_i.x, w0.y / inv_i.y, w0.z / inv_i.z);
+    const float scale = max_abs(m0);
+    if (!finite_vector(m0)) { out.status = 2u; out.residual = INFINITY; return out; }
+    if (scale == 0.0f) return out;
+    const v3 u0 = v3_scale(m0, 1.0f / scale);
+    const v3 a = v3_scale(inv_i, scale);
+    const v3 c = v3_make(dt * (a.y - a.z), dt * (a.z - a.x), dt * (a.x - a.y));
+    const float tolerance = 1.0e-6f;
+    const uint32_t max_iterations = 12u, max_backtracks = 8u;
+    v3 u = u0;
+    for (uint32_t iteration = 0u; iteration <= max_iterations; ++iteration) {
+        const v3 r = gyro_residual(u0, c, u);
+        out.residual = finite_vector(r) ? max_abs(r) : INFINITY;
+        if (out.residual <= tolerance) {
+            const v3 mid = v3_scale(v3_add(u0, u), 0.5f);
+            out.midpoint = v3_make(a.x * mid.x, a.y * mid.y, a.z * mid.z);
+            return out;
+        }
+        if (iteration == max_iterations || !isfinite(out.residual)) break;
+        const v3 mid = v3_scale(v3_add(u0, u), 0.5f);
+        float j[3][4] = {{1.0f, 0.5f * c.x * mid.z, 0.5f * c.x * mid.y, r.x},
+                         {0.5f * c.y * mid.z, 1.0f, 0.5f * c.y * mid.x, r.y},
+                         {0.5f * c.z * mid.y, 0.5f * c.z * mid.x, 1.0f, r.z}};
+        int valid = 1;
+        for (uint32_t column = 0u; column < 3u; ++column) {
+            uint32_t pivot = column;
+            for (uint32_t row = column + 1u; row < 3u; ++row)
+                if (fabsf(j[row][column]) > fabsf(j[pivot][column])) pivot = row;
+            if (!isfinite(j[pivot][column]) || fabsf(j[pivot][column]) < 1.0e-12f) { valid = 0; break; }
+            for (uint32_t col = column; col < 4u; ++col) {
+                const float value = j[column][col];
+                j[column][col] = j[pivot][col];
+                j[pivot][col] = value;
+            }
+            for (uint32_t row = column + 1u; row < 3u; ++row) {
+                const float factor = j[row][column] / j[column][column];
+                for (uint32_t col = column + 1u; col < 4u; ++col) j[row][col] -= factor * j[column][col];
+            }
+        }
+        ++out.iterations;
+        if (!valid) break;
+        v3 delta;
+        delta.z = j[2][3] / j[2][2];
+        delta.y = (j[1][3] - j[1][2] * delta.z) / j[1][1];
+        delta.x = (j[0][3] - j[0][1] * delta.y - j[0][2] * delta.z) / j[0][0];
+        int accepted = 0;
+        float alpha = 1.0f;
+        for (uint32_t backtrack = 0u; backtrack < max_backtracks; ++backtrack) {
+            const v3 trial = v3_sub(u, v3_scale(delta, alpha));
+            const v3 trial_r = gyro_residual(u0, c, trial);
+            if (finite_vector(trial_r) && max_abs(trial_r) < out.residual) { u = trial; accepted = 1; break; }
+            alpha *= 0.5f;
+        }
+        if (!accepted) break;
+    }
+    out.status = 1u;   /* kBodyGyroNotConverged */
+    return out;
+}
+/* the free-rotation solve alone, for the tests: returns the status, writes the midpoint angular velocity (principal
+ * frame), the residual and the Newton steps taken */
+uint32_t nko_solve_free_rotation(const float w0[3], const float inv_i[3], float dt, float midpoint[3], float* residual, uint32_t* iterations) {
+    const gyro_result g = solve_free_rotation(v3_make(w0[0], w0[1], w0[2]), v3_make(inv_i[0], inv_i[1], inv_i[2]), dt);
+    midpoint[0] = g.midpoint.x; midpoint[1] = g.midpoint.y; midpoint[2] = g.midpoint.z;
+    *residual = g.residual; *iterations = g.iterations;
+    return g.status;
+}
+
+static v3 inverse_inertia_of(const nko_template* t) {   /* cook: body_inv_inertia = 1 / principal moment, 0 for none */
+    const float* d = t->body_diag_inertia;
+    return v3_make(d[0] > 0.0f ? 1.0f / d[0] : 0.0f, d[1] > 0.0f ? 1.0f / d[1] : 0.0f, d[2] > 0.0f ? 1.0f / d[2] : 0.0f);
+}
+
+/* BodyIntegrateVelocityKernel (articulation.cu:1019-1049): the world inverse inertia at the step's pose, gravity and the
+ * applied force on the linear velocity, the applied torque on the angular velocity (no gyroscopic term here: the
+ * position update carries it).  `link_wrench` holds the applied force and torque about the centre of mass, world axes,
+ * and is cleared.  Then the block the tile will descend on (InitializeRigidBlock, block_descent_rigid.cuh:4-48): mass
+ * matrix diag(m, m, m) and the inverse of the world inverse inertia, its L D L^T factor for the heads' inertial
+ * response, and the six coordinates in the link's twist words. */
+void nko_env_body_integrate_velocity(nko_world* w, uint32_t env) {
+    const nko_template* t = &w->t;
+    const float dt = w->cfg.fixed_dt;
+    float* lin = w->body_linear_velocity + (size_t)env * 3u, *ang = w->body_angular_velocity + (size_t)env * 3u;
+    float* wrench = w->link_wrench + (size_t)env * 6u;
+    float* inverse = w->body_world_inv_inertia + (size_t)env * 6u;
+    const v3 force = v3_make(wrench[0], wrench[1], wrench[2]), torque = v3_make(wrench[3], wrench[4], wrench[5]);
+    for (uint32_t i = 0u; i < 6u; ++i) wrench[i] = 0.0f;
+    const float inv_mass = t->body_mass > 0.0f ? 1.0f / t->body_mass : 0.0f;
+    const uint32_t md = t->max_dof;
+    float* M = w->m + (size_t)env * md * md, *F = w->m_factor + (size_t)env * md * md;
+    for (uint32_t i = 0u; i < md * md; ++i) { M[i] = 0.0f; F[i] = 0.0f; }
+    if (inv_mass <= 0.0f) {
+        for (uint32_t i = 0u; i < 6u; ++i) inverse[i] = 0.0f;
+    } else {
+        const xform pose = xform_load(w->base_pose + (size_t)env * 7u), frame = xform_load(t->link_inertial_frame);
+        body_world_inverse_inertia(pose, frame, inverse_inertia_of(t), inverse);
+        const v3 g = v3_make(w->cfg.gravity[0], w->cfg.gravity[1], w->cfg.gravity[2]);
+        const v3 dv = v3_scale(v3_add(v3_scale(g, 1.0f - 0.0f), v3_scale(force, inv_mass)), dt);
+        lin[0] += dv.x; lin[1] += dv.y; lin[2] += dv.z;
+        const v3 dw = v3_scale(sym_multiply(inverse, torque), dt);
+        ang[0] += dw.x; ang[1] += dw.y; ang[2] += dw.z;
+    }
+    float inertia[6];
+    const float mass = (float)(1.0 / (double)inv_mass);
+    const int valid = inv_mass > 0.0f && sym_invert(inverse, inertia) && inertia[0] > 0.0f && inertia[1] > 0.0f && inertia[2] > 0.0f &&
+                      (double)inertia[0] * inertia[1] > (double)inertia[3] * inertia[3] && isfinite(lin[0]) && isfinite(lin[1]) &&
+                      isfinite(lin[2]) && isfinite(ang[0]) && isfinite(ang[1]) && isfinite(ang[2]);
+    if (!valid) { w->env_status[env] |= NKO_STATUS_SOLVER_FAILURE; for (uint32_t i = 0u; i < 6u; ++i) inertia[i] = i < 3u ? 1.0f : 0.0f; }
+    const float rotational[3][3] = {{inertia[0], inertia[3], inertia[4]}, {inertia[3], inertia[1], inertia[5]}, {inertia[4], inertia[5], inertia[2]}};
+    for (uint32_t r = 0u; r < 6u; ++r)
+        for (uint32_t c = 0u; c < 6u; ++c) {
+            float value = 0.0f;
+            if (r < 3u && c < 3u && r == c) value = valid ? mass : 1.0f;
+            if (r >= 3u && c >= 3u) value = rotational[r - 3u][c - 3u];
+            M[(size_t)r * md + c] = value;
+        }
+    nko_factor_mass(M, F, 6u, md);
+    float* twist = w->link_velocity + (size_t)env * 6u;
+    for (uint32_t i = 0u; i < 3u; ++i) { twist[i] = lin[i]; twist[3u + i] = ang[i]; }
+    for (uint32_t i = 0u; i < md; ++i) { w->articulation_qdd[(size_t)env * md + i] = 0.0f; w->articulation_bias[(size_t)env * md + i] = 0.0f; }
+}
+
+/* BodyIntegratePositionKernel (articulation.cu:1058-1117): the solve's velocities from the link's twist words; the
+ * angular momentum is carried through the step in world axes while the pose turns by the midpoint angular velocity of
+ * the free-rotation solve (and by the position pass's pseudo velocity, which moves the pose only); the centre of mass
+ * moves with the linear velocity. */
+void nko_env_body_integrate_position(nko_world* w, uint32_t env) {
+    const nko_template* t = &w->t;
+    const float dt = w->cfg.fixed_dt;
+    const int pos_pass = w->cfg.solver_pos_iters > 0u && t->rows_per_env > 0u;
+    float* lin = w->body_linear_velocity + (size_t)env * 3u, *ang = w->body_angular_velocity + (size_t)env * 3u;
+    float* twist = w->link_velocity + (size_t)env * 6u;
+    if (t->rows_per_env > 0u) for (uint32_t i = 0u; i < 3u; ++i) { lin[i] = twist[i]; ang[i] = twist[3u + i]; }
+    w->body_gyro_residual[env] = 0.0f; w->body_gyro_iterations[env] = 0u; w->body_gyro_status[env] = 0u;
+    if (!(t->body_mass > 0.0f)) return;
+    xform pose = xform_load(w->base_pose + (size_t)env * 7u);
+    const xform frame = xform_load(t->link_inertial_frame);
+    const v3 inv_i = inverse_inertia_of(t);
+    const quat principal = nko_quat_normalize_rsqrt(nko_quat_mul(pose.r, frame.r), 1.0e-12f);
+    const quat inverse = quat_make(principal.w, -principal.x, -principal.y, -principal.z);
+    const v3 w0 = nko_rotate_normalized(inverse, v3_make(ang[0], ang[1], ang[2]));
+    const gyro_result gyro = solve_free_rotation(w0, inv_i, dt);
+    w->body_gyro_residual[env] = gyro.residual; w->body_gyro_iterations[env] = gyro.iterations; w->body_gyro_status[env] = gyro.status;
+    if (gyro.status != 0u) { w->env_status[env] |= NKO_STATUS_GYRO_FAILURE; return; }
+    const v3 momentum = nko_rotate_normalized(principal, v3_make(w0.x / inv_i.x, w0.y / inv_i.y, w0.z / inv_i.z));
+    v3 v = v3_make(lin[0], lin[1], lin[2]);
+    const v3 wm = nko_rotate_normalized(principal, gyro.midpoint);
+    const v3 center = body_center_of_mass(pose, frame);
+    const quat dq = quat_make(1.0f, 0.5f * dt * wm.x, 0.5f * dt * wm.y, 0.5f * dt * wm.z);
+    quat q = nko_quat_normalize_rsqrt(nko_quat_mul(dq, pose.r), 1.0e-12f);
+    if (pos_pass) {
+        const float* pseudo = w->link_velocity_pseudo + (size_t)env * 6u;
+        v = v3_add(v, v3_make(pseudo[0], pseudo[1], pseudo[2]));
+        const quat turn = quat_make(1.0f, 0.5f * dt * pseudo[3], 0.5f * dt * pseudo[4], 0.5f * dt * pseudo[5]);
+        q = nko_quat_normalize_rsqrt(nko_quat_mul(turn, q), 1.0e-12f);
+    }
+    pose.r = q;
+    const v3 offset = nko_rotate_normalized(q, frame.p);
+    pose.p = v3_sub(v3_add(center, v3_scale(v, dt)), offset);
+    xform_store(w->base_pose + (size_t)env * 7u, pose);
+    float* world_inverse = w->body_world_inv_inertia + (size_t)env * 6u;
+    body_world_inverse_inertia(pose, frame, inv_i, world_inverse);
+    const v3 turned = sym_multiply(world_inverse, momentum);
+    ang[0] = turned.x; ang[1] = turned.y; ang[2] = turned.z;
+    for (uint32_t i = 0u; i < 3u; ++i) { twist[i] = lin[i]; twist[3u + i] = ang[i]; }
+}

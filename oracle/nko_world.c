@@ -61,6 +61,12 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
     if (nv > NKO_MAX_DOF) return -1;
     t->nv = nv; t->max_dof = nv;
     t->floating = nl > 0u && t->joint_type[0] == NKO_FLOATING && t->parent_link[0] == NKO_INVALID;
+    t->free_body = d->struct_size >= sizeof(nko_template_desc) && d->free_body != 0u;
+    if (t->free_body) {
+        if (nl != 1u || !t->floating) return -1;   /* one free body an environment, the template's one link */
+        t->body_mass = d->link_mass[0];
+        for (uint32_t k = 0u; k < 3u; ++k) t->body_diag_inertia[k] = d->link_diag_inertia[k];
+    }
     t->dof_link = ALLOC(uint32_t, nv); t->dof_component = ALLOC(uint32_t, nv);
     for (uint32_t l = 0u; l < nl; ++l) {
         const uint32_t width = nko_joint_dof(t->joint_type[l]);
@@ -264,6 +270,9 @@ nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc*
     w->m = ALLOC(float, E * md * md); w->m_factor = ALLOC(float, E * md * md); w->qdot_flat = ALLOC(float, E * md);
     w->qdot_pseudo = ALLOC(float, E * nl); w->link_velocity_pseudo = ALLOC(float, E * nl * 6u);
     w->body_pose = ALLOC(float, E * nb * 7u); w->body_aabb_lo = ALLOC(float, E * nb * 3u); w->body_aabb_hi = ALLOC(float, E * nb * 3u);
+    w->body_linear_velocity = ALLOC(float, E * 3u); w->body_angular_velocity = ALLOC(float, E * 3u);
+    w->body_world_inv_inertia = ALLOC(float, E * 6u); w->body_gyro_residual = ALLOC(float, E);
+    w->body_gyro_iterations = ALLOC(uint32_t, E); w->body_gyro_status = ALLOC(uint32_t, E);
     w->candidate_pairs = ALLOC(uint32_t, E * S * 2u); w->pair_count = ALLOC(uint32_t, E);
     w->ucontact_count = ALLOC(uint32_t, E * S); w->ucontact_a = ALLOC(uint32_t, E * S * 4u); w->ucontact_b = ALLOC(uint32_t, E * S * 4u);
     w->ucontact_law = ALLOC(uint32_t, E * S); w->ucontact_row_range = ALLOC(uint32_t, E * S * 2u);
@@ -378,7 +387,9 @@ void nko_world_destroy(nko_world* w) {
     X(contact_point, float, E * S * 3u) X(contact_normal, float, E * S * 3u) X(contact_force, float, E * S * 3u) \
     X(ucontact_impulse, float, E * S * 12u) X(link_contact_wrench, float, E * nl * 6u) \
     X(contact_side_a_kind, uint32_t, E * S) X(contact_side_b_kind, uint32_t, E * S) X(contact_side_a_index, uint32_t, E * S) \
-    X(contact_side_b_index, uint32_t, E * S) X(contact_link, uint32_t, E * S)
+    X(contact_side_b_index, uint32_t, E * S) X(contact_link, uint32_t, E * S) \
+    X(body_linear_velocity, float, E * 3u) X(body_angular_velocity, float, E * 3u) X(body_world_inv_inertia, float, E * 6u) \
+    X(body_gyro_residual, float, E) X(body_gyro_iterations, uint32_t, E) X(body_gyro_status, uint32_t, E)
 
 #define TEMPLATE_LIST(X) \
     X(link_inertia, float, nl * 36u) X(link_tree_depth, uint32_t, nl) X(link_child_range, uint32_t, nl * 2u) \
@@ -434,6 +445,8 @@ void nko_contact_warm_start(nko_world* w, uint32_t phase) {
 }
 void nko_block_descent_solve(nko_world* w) { FOR_ENVS(nko_env_solve(w, env)) }
 void nko_integrate_position(nko_world* w) { FOR_ENVS(nko_env_integrate_position(w, env)) }
+void nko_body_integrate_velocity(nko_world* w) { FOR_ENVS(nko_env_body_integrate_velocity(w, env)) }
+void nko_body_integrate_position(nko_world* w) { FOR_ENVS(nko_env_body_integrate_position(w, env)) }
 void nko_fk_link_velocities(nko_world* w) { FOR_ENVS(nko_env_link_velocities(w, env)) }
 void nko_articulation_damping(nko_world* w) { FOR_ENVS(nko_env_articulation_damping(w, env)) }
 void nko_reference_weights(nko_world* w) {
@@ -459,7 +472,37 @@ void nko_snapshot_step_velocity(nko_world* w) {
         }
 }
 
+/* pipeline.cpp:434-443, 600-606, 955-986 for a world of free bodies: the velocity update, the contact pipeline on the
+ * bodies' poses, the solve on their six by six blocks, the position update */
+static void step_free_body(nko_world* w) {
+    for (size_t e = 0u; e < w->env_count; ++e)   /* the six coordinates as the state holds them */
+        for (uint32_t i = 0u; i < 3u; ++i) {
+            w->link_velocity[e * 6u + i] = w->body_linear_velocity[e * 3u + i];
+            w->link_velocity[e * 6u + 3u + i] = w->body_angular_velocity[e * 3u + i];
+        }
+    if (w->t.rows_per_env > 0u) nko_snapshot_step_velocity(w);
+    nko_body_integrate_velocity(w);
+    nko_fk_world_poses(w);
+    if (w->t.rows_per_env > 0u) {
+        if (w->t.slots > 0u) {
+            nko_sync_link_body_pose(w);
+            nko_build_aabbs(w);
+            nko_query_pairs(w);
+            nko_narrowphase(w);
+        }
+        nko_assemble_rows(w);
+        nko_contact_warm_start(w, 0u);
+        nko_block_descent_solve(w);
+        nko_contact_warm_start(w, 1u);
+    }
+    nko_body_integrate_position(w);
+    nko_fk_world_poses(w);
+    if (w->t.nb > 0u) nko_sync_link_body_pose(w);
+    if (w->readout_in_step && w->t.rows_per_env > 0u && w->t.slots > 0u) nko_readout_contact_wrench(w);
+}
+
 static void step_interval(nko_world* w) {
+    if (w->t.free_body) { step_free_body(w); return; }
     if (w->t.rows_per_env > 0u || w->t.integrator != 0u) nko_snapshot_step_velocity(w);   /* pipeline.cpp:367 */
     nko_fk_world_poses(w);
     if (w->t.joint_drive_rows > 0u) nko_apply_drives(w);

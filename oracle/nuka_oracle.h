@@ -44,6 +44,11 @@
  *                             to the generalized impulse the solve applied)
  *   substeps                : pinned (n substeps of dt are n steps of dt / n bit for bit; the step's status, joint limit
  *                             impulses and link contact wrenches are the or, the sum and the time average of those steps')
+ *   free rigid body         : pinned (free flight: the parabola of the centre of mass, angular momentum and kinetic
+ *                             energy of a tumbling body over thousands of steps, the precession rate of a symmetric top
+ *                             against its closed form, the free-rotation solve against the midpoint rule's own
+ *                             equation; the row entries J [v; w] against the velocity of the contact point; a box at rest
+ *                             on a plane carries its weight; a sliding box stops by Coulomb's law)
  *   UABD fixed point        : pinned (closed-form resting, falling, sticking and sliding ball; Coulomb / KKT
  *                             conditions and momentum balance of converged solves)
  *   UABD iterate path       : PARITY UNPINNED - penalty heuristic, first-sweep segment search, FISTA
@@ -119,7 +124,7 @@ typedef struct nko_template_desc {
     const float* joint_limit_reference;
     const float* joint_friction_reference;
     uint32_t integrator;
-    uint32_t reserved2;
+    uint32_t free_body;   /* 1: the template's one link (floating root) is a free rigid body, stepped by the rigid-body ops */
 } nko_template_desc;
 
 typedef struct nko_world_desc {
@@ -173,6 +178,11 @@ void nko_readout_drives(nko_world* w);
 void nko_readout_contact_wrench(nko_world* w);   /* on demand: not part of nko_world_step until it has been called once,
                                                     then every interval ends with it (nk/pipeline/world.cpp:905-975) */
 void nko_integrate_position(nko_world* w);
+/* a free_body world's ops (articulation.cu:1019-1049 BodyIntegrateVelocityKernel with the tile's rigid block,
+ * :1058-1117 BodyIntegratePositionKernel) and the free-rotation solve alone (rigid_types.cuh:38-121) */
+void nko_body_integrate_velocity(nko_world* w);
+void nko_body_integrate_position(nko_world* w);
+uint32_t nko_solve_free_rotation(const float w0[3], const float inv_i[3], float dt, float midpoint[3], float* residual, uint32_t* iterations);
 void nko_fk_link_velocities(nko_world* w);
 /* The whole op list of one step, in the reference's order. */
 void nko_world_step(nko_world* w);

@@ -16,7 +16,8 @@ U32_FIELDS = {"candidate_pairs", "pair_count", "ucontact_count", "ucontact_a", "
               "link_child_range", "link_children", "link_dof", "dof_link", "dof_component", "link_body",
               "body_to_link", "body_collidable_link", "body_collidable_body", "contact_cache_age",
               "contact_cache_current_owner", "contact_cache_old_keep", "contact_cache_extent", "contact_warm_start_counts",
-              "contact_side_a_kind", "contact_side_b_kind", "contact_side_a_index", "contact_side_b_index", "contact_link"}
+              "contact_side_a_kind", "contact_side_b_kind", "contact_side_a_index", "contact_side_b_index", "contact_link",
+              "body_gyro_iterations", "body_gyro_status"}
 U64_FIELDS = {"ucontact_id_pair", "ucontact_id_feature", "contact_material", "contact_cache_pair", "contact_cache_feature",
               "contact_cache_material"}
 
@@ -62,7 +63,7 @@ def _declare_world_entry_points(L):
     for name in ("fk_world_poses", "sync_link_body_pose", "build_aabbs", "query_pairs", "narrowphase",
                  "assemble_rows", "block_descent_solve", "integrate_position", "fk_link_velocities", "apply_drives",
                  "readout_drives", "readout_contact_wrench", "reference_weights", "snapshot_step_velocity",
-                 "articulation_damping"):
+                 "articulation_damping", "body_integrate_velocity", "body_integrate_position"):
         getattr(L, "nko_" + name).argtypes = [C.c_void_p]
     L.nko_articulation_dynamics.argtypes = [C.c_void_p, C.c_uint32]
     L.nko_contact_warm_start.argtypes = [C.c_void_p, C.c_uint32]
@@ -120,7 +121,7 @@ def lib():
         for name in ("fk_world_poses", "sync_link_body_pose", "build_aabbs", "query_pairs", "narrowphase",
                      "assemble_rows", "block_descent_solve", "integrate_position", "fk_link_velocities", "apply_drives",
                      "readout_drives", "readout_contact_wrench", "reference_weights", "snapshot_step_velocity",
-                     "articulation_damping"):
+                     "articulation_damping", "body_integrate_velocity", "body_integrate_position"):
             getattr(L, "nko_" + name).argtypes = [C.c_void_p]
         L.nko_articulation_dynamics.argtypes = [C.c_void_p, C.c_uint32]
         L.nko_contact_warm_start.argtypes = [C.c_void_p, C.c_uint32]

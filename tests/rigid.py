@@ -1,0 +1,27 @@
+"""Templates of a free rigid body for the tests: a box (the body's own collidable row) over an optional static plane."""
+import numpy as np
+
+from conftest import nk
+
+abi = nk.abi
+
+
+def box_template(half=(0.2, 0.2, 0.1), mass=1.0, diag=(0.01, 0.01, 0.01), com=(0.0, 0.0, 0.0), mu=0.7, plane=True):
+    t = abi.Template()
+    t.free_body = True
+    t.add_link(abi.JOINT_FLOATING, None, mass=mass, diag_inertia=diag, com=com)
+    profile = t.add_profile(mu)
+    if plane:
+        t.add_body(abi.ROLE_STATIC, kind=abi.SHAPE_PLANE, contype=2, conaffinity=1, profile=profile)
+    t.add_body(abi.ROLE_LINK_BODY, link=0, kind=abi.SHAPE_BOX, params=(half[0], half[1], half[2], 0.0), contype=1, conaffinity=2,
+               profile=profile)
+    t.max_contacts_per_env = 1 if plane else 0
+    return t
+
+
+def rotation_matrix(q):
+    """Rotation matrix of a quaternion w x y z, in float64."""
+    w, x, y, z = np.asarray(q, np.float64) / np.linalg.norm(q)
+    return np.array([[1 - 2 * (y * y + z * z), 2 * (x * y - w * z), 2 * (x * z + w * y)],
+                     [2 * (x * y + w * z), 1 - 2 * (x * x + z * z), 2 * (y * z - w * x)],
+                     [2 * (x * z - w * y), 2 * (y * z + w * x), 1 - 2 * (x * x + y * y)]])
