@@ -133,7 +133,16 @@ typedef struct nuka_template_desc_t {
                                               damping applied implicitly after the solve, the step's velocity change
                                               through (M + dt D)^-1 M; 2 implicit / implicitfast: the servos' velocity
                                               gains join D */
-    uint32_t reserved2;
+    uint32_t free_body;                    /* 1: the template's one link (link_count 1, a floating root) is a free rigid body.
+                                              The reference's rigid-body ops step it (BodyIntegrateVelocityKernel,
+                                              src/phi/backend_cuda/ops/articulation.cu:1019-1049; the six by six block of the
+                                              tile, ops/block_descent_rigid.cuh:4-48, ops/block_descent_tile.cuh:541-603;
+                                              BodyIntegratePositionKernel with the free-rotation solve, articulation.cu:1058-1117,
+                                              ops/rigid_types.cuh:38-121): base_pose is the body's pose, link_mass,
+                                              link_diag_inertia and link_inertial_frame its inertial parameters,
+                                              BODY_LINEAR_VELOCITY / BODY_ANGULAR_VELOCITY its state (world axes, about the
+                                              centre of mass), link_wrench the force and torque applied at the centre of
+                                              mass.  One free body an environment; statics beside it */
 } nuka_template_desc_t;
 
 /* The world options of the cooked-template creator (the library's own descriptor; the reference's nuka_world_desc_t
@@ -400,6 +409,8 @@ typedef enum nuka_state_field_t {
     NUKA_FIELD_CONTACT_FORCE = 18,
     NUKA_FIELD_CONTACT_LINK = 19,
     NUKA_FIELD_JOINT_FEEDFORWARD = 22,          /* joint_f */
+    NUKA_FIELD_BODY_LINEAR_VELOCITY = 25,       /* per body row; a free body's values in its own row */
+    NUKA_FIELD_BODY_ANGULAR_VELOCITY = 26,
     NUKA_FIELD_JOINT_LIMIT_IMPULSE = 27,
     NUKA_FIELD_ACTUATOR_EFFORT_REQUESTED = 28,
     NUKA_FIELD_ACTUATOR_EFFORT = 29,

@@ -94,6 +94,7 @@ PUBLIC_FIELDS = {
     "VELOCITY_TARGET": (13, "velocity_target", 4), "ACTUATOR_NOLOAD_SPEED": (14, "actuator_noload_speed", 4),
     "LINK_CONTACT_WRENCH": (16, "link_contact_wrench", 24), "CONTACT_NORMAL": (17, "contact_normal", 12),
     "CONTACT_FORCE": (18, "contact_force", 12), "CONTACT_LINK": (19, "contact_link", 4), "JOINT_FEEDFORWARD": (22, "joint_f", 4),
+    "BODY_LINEAR_VELOCITY": (25, "body_linear_velocity", 12), "BODY_ANGULAR_VELOCITY": (26, "body_angular_velocity", 12),
     "JOINT_LIMIT_IMPULSE": (27, "joint_limit_impulse", 8), "ACTUATOR_EFFORT_REQUESTED": (28, "actuator_effort_requested", 4),
     "ACTUATOR_EFFORT": (29, "actuator_effort", 4), "ACTUATOR_SATURATED": (30, "actuator_saturated", 4),
     "CONTACT_SIDE_A_KIND": (33, "contact_side_a_kind", 4), "CONTACT_SIDE_B_KIND": (34, "contact_side_b_kind", 4),

@@ -32,6 +32,10 @@ Status OpArticulationDamping(const ModelView&, const DataView&, const void*, hip
 Status OpReferenceWeights(const ModelView&, const DataView&, const void*, hipStream_t);
 Status OpSnapshotStepVelocity(const ModelView&, const DataView&, const void*, hipStream_t);
 
+// A free body's part of IntegrateVelocity and IntegratePosition (ModelView::free_body; ops_rigid.hip)
+Status BodyIntegrateVelocity(const ModelView&, const DataView&, const IntegrateVelocityParams&, hipStream_t);
+Status BodyIntegratePosition(const ModelView&, const DataView&, const IntegratePositionParams&, hipStream_t);
+
 // IntegratePosition, FkWorldPoses, FkLinkVelocities and (when `bodies` is not null) SyncLinkBodyPose as one launch, for
 // a plan whose op list holds them in a row; Unsupported when they must run one by one.
 Status OpStepTail(const ModelView&, const DataView&, const IntegratePositionParams*, const FkWorldPosesParams*,

@@ -56,7 +56,7 @@ enum : uint32_t {
 };
 // src/phi/op_schema.hpp:36-52
 enum : uint32_t {
-    kEnvStatusPairOverflow = 1u << 0, kEnvStatusDofOverflow = 1u << 2, kEnvStatusInvalidEndpoint = 1u << 6,
+    kEnvStatusPairOverflow = 1u << 0, kEnvStatusDofOverflow = 1u << 2, kEnvStatusGyroFailure = 1u << 5, kEnvStatusInvalidEndpoint = 1u << 6,
     kEnvStatusControlFailure = 1u << 10, kEnvStatusSolverFailure = 1u << 13
 };
 // src/phi/articulation_contract.hpp:16-23
@@ -83,6 +83,10 @@ struct ModelView {
     uint32_t any_mujoco, contact_cone;
     float contact_impratio;
     uint32_t integrator;   // 0 native; 1, 2: ArticulationDamping follows the solve (2: with the servos' velocity gains)
+    // 1: the template's one link is a free rigid body, stepped by the rigid-body ops (ops_rigid.hip): its six coordinates
+    // are its linear velocity and its angular velocity about the centre of mass, in world axes
+    uint32_t free_body;
+    float body_inv_mass, body_inv_inertia[3];   // 1 / mass and 1 / principal moments (src/nk/model/fields.yaml:17, 108)
     const uint8_t* joint_type;
     const uint32_t* parent_link;
     const float* joint_axis;
@@ -136,6 +140,9 @@ struct DataView {
     float *q, *qdot, *qddot, *tau, *base_pose, *link_pose, *link_velocity, *link_acceleration, *link_wrench;
     float *articulation_bias, *articulation_qdd, *m, *m_factor, *qdot_flat, *qdot_pseudo, *link_velocity_pseudo;
     float *body_pose, *body_aabb_lo, *body_aabb_hi;
+    // the free body of a free_body world, one an environment (fields.yaml:102-103, 569; articulation.cu:1068-1070)
+    float *body_linear_velocity, *body_angular_velocity, *body_world_inv_inertia, *body_gyro_residual;
+    uint32_t *body_gyro_iterations, *body_gyro_status;
     uint32_t *candidate_pairs, *pair_count;
     uint32_t *ucontact_count, *ucontact_a, *ucontact_b, *ucontact_law, *ucontact_row_range;
     float *ucontact_point, *ucontact_normal, *ucontact_depth;

@@ -904,6 +904,7 @@ Status OpIntegratePosition(const ModelView& m, const DataView& d, const void* pa
     const auto* p = static_cast<const IntegratePositionParams*>(params);
     if (p == nullptr) return Status::Failed;
     if (p->dt <= 0.0f || p->total_link_count == 0u) return Status::Ok;
+    if (m.free_body != 0u) return BodyIntegratePosition(m, d, *p, stream);
     const uint32_t blocks = (p->total_link_count + 255u) / 256u;
     hipLaunchKernelGGL(IntegratePositionKernel, dim3(blocks), dim3(256), 0, stream, m, d, *p);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
@@ -1022,7 +1023,7 @@ __global__ void __launch_bounds__(256) ReadoutDrivesKernel(ModelView m, DataView
 }
 
 // OpApplyDrives (articulation.cu:1604-1620).  Without drive rows in the cooked world tau is the applied generalized
-// force and the op only validates; free bodies do not exist on this path, so IntegrateVelocity only validates too.
+// force and the op only validates; IntegrateVelocity acts on a free body only (ops_rigid.hip).
 Status OpApplyDrives(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
     const auto* p = static_cast<const ApplyDrivesParams*>(params);
     if (p == nullptr || p->mode > kDriveActuator) return Status::InvalidArgument;
@@ -1044,9 +1045,11 @@ Status OpReadoutDrives(const ModelView& m, const DataView& d, const void* params
     hipLaunchKernelGGL(ReadoutDrivesKernel, dim3((p->total_link_count + 255u) / 256u), dim3(256), 0, stream, m, d, *p);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
-Status OpIntegrateVelocity(const ModelView&, const DataView&, const void* params, hipStream_t) {
+Status OpIntegrateVelocity(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
     const auto* p = static_cast<const IntegrateVelocityParams*>(params);
     if (p == nullptr) return Status::Failed;
+    if (p->dt <= 0.0f) return Status::Ok;
+    if (m.free_body != 0u && p->total_body_count > 0u) return BodyIntegrateVelocity(m, d, *p, stream);
     return Status::Ok;
 }
 

@@ -53,7 +53,7 @@ __device__ V3 rot_abs(Q4 q, V3 v) {
 }
 
 // ---- BuildAabbs (broadphase.cu:173-270).  Link-owned collidables carry no body velocity on this path, so the
-// motion term of the margin is zero. ----
+// motion term of the margin is zero; a free body's row carries the body's velocities. ----
 __device__ __forceinline__ void build_aabb_of_body(const ModelView& m, const DataView& d, const BuildAabbsParams& p, uint32_t gid) {
     const uint32_t b = gid % p.bodies_per_env;
     const ShapeRow s = load_shape(m.shape_table, b);
@@ -78,7 +78,14 @@ __device__ __forceinline__ void build_aabb_of_body(const ModelView& m, const Dat
         lo[0] = lo[1] = lo[2] = FLT_MAX; hi[0] = hi[1] = hi[2] = -FLT_MAX;
         return;
     }
-    const float mg = fmaxf(p.margin, fminf(motion_radius(p.margin, p.dt, 0.0f, 0.0f, 0.9f), p.query_reach));
+    // (:262-264) a free body's own row moves with it - its speed, and its turning rate over the shape's radius
+    float speed = 0.0f;
+    if (m.free_body != 0u && b == m.link_body[0]) {
+        const float* lv = d.body_linear_velocity + size_t{gid} * 3u, *av = d.body_angular_velocity + size_t{gid} * 3u;
+        const float radius = sqrtf(he.x * he.x + he.y * he.y + he.z * he.z) + sqrtf(0.0f);
+        speed = fmaxf(0.0f, sqrtf(lv[0] * lv[0] + lv[1] * lv[1] + lv[2] * lv[2]) + sqrtf(av[0] * av[0] + av[1] * av[1] + av[2] * av[2]) * radius);
+    }
+    const float mg = fmaxf(p.margin, fminf(motion_radius(p.margin, p.dt, speed, 0.0f, 0.9f), p.query_reach));
     const V3 c = xf.p;
     lo[0] = c.x - he.x - mg; lo[1] = c.y - he.y - mg; lo[2] = c.z - he.z - mg;
     hi[0] = c.x + he.x + mg; hi[1] = c.y + he.y + mg; hi[2] = c.z + he.z + mg;
@@ -665,7 +672,23 @@ __device__ __forceinline__ uint32_t NarrowphaseSlot(const ModelView& m, const Da
             const float margin_b = has_b ? m.profile_margin[2u * sb.profile] + m.profile_margin[2u * sb.profile + 1u] : 0.0f;
             query_margin = margin_a + margin_b;
         }
-        const float query = fmaxf(query_margin, fminf(motion_radius(2.0f * separation, p.dt, 0.0f, 0.0f, 0.9f), p.query_reach));
+        // (:236-250) the gap both sides can close within the step: link-owned rows carry no body velocity, a free body's own
+        // row moves with it
+        float speeds[2] = {0.0f, 0.0f};
+        if (m.free_body != 0u) {
+            const uint32_t ends[2] = {a, b};
+            for (uint32_t side = 0u; side < 2u; ++side) {
+                if (ends[side] != m.link_body[0]) continue;
+                const size_t at = bbase + ends[side];
+                const float* center = d.body_pose + at * 7u, *lo = d.body_aabb_lo + at * 3u, *hi = d.body_aabb_hi + at * 3u;
+                const V3 extent{fmaxf(fabsf(lo[0] - center[0]), fabsf(hi[0] - center[0])), fmaxf(fabsf(lo[1] - center[1]), fabsf(hi[1] - center[1])),
+                                fmaxf(fabsf(lo[2] - center[2]), fabsf(hi[2] - center[2]))};
+                const float* lv = d.body_linear_velocity + at * 3u, *av = d.body_angular_velocity + at * 3u;
+                speeds[side] = fmaxf(0.0f, sqrtf(lv[0] * lv[0] + lv[1] * lv[1] + lv[2] * lv[2]) +
+                                           sqrtf((av[0] * av[0] + av[1] * av[1] + av[2] * av[2]) * (extent.x * extent.x + extent.y * extent.y + extent.z * extent.z)));
+            }
+        }
+        const float query = fmaxf(query_margin, fminf(motion_radius(2.0f * separation, p.dt, speeds[0], speeds[1], 0.9f), p.query_reach));
         if constexpr (kSinglePoint) primitive_pair_single(sa.kind, pa, sb.kind, pb, query, &mf);
         else primitive_pair(sa.kind, pa, sb.kind, pb, query, &mf);
         if (law != kContactLawCompliant) {
@@ -1225,9 +1248,18 @@ __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4, 4
         } else {
             const Xf base = load_xf(d.base_pose + size_t{env} * 7u);
             const uint32_t k = component % 3u;
-            axis_world = rotate_normalized(base.r, V3{k == 0u ? 1.0f : 0.0f, k == 1u ? 1.0f : 0.0f, k == 2u ? 1.0f : 0.0f});
-            origin = base.p;
-            mode = component < 3u ? 3u : 4u;
+            const V3 unit{k == 0u ? 1.0f : 0.0f, k == 1u ? 1.0f : 0.0f, k == 2u ? 1.0f : 0.0f};
+            if (m.free_body != 0u) {
+                // a free body's coordinates: linear velocity, then angular velocity about the centre of mass, world axes -
+                // the row's jlin and jang = (point - com) x jlin (assemble_rows.cu:537-538, 680-681)
+                axis_world = unit;
+                origin = add3(base.p, rotate_normalized(base.r, V3{m.link_inertial_frame[0], m.link_inertial_frame[1], m.link_inertial_frame[2]}));
+                mode = component < 3u ? 4u : 3u;
+            } else {
+                axis_world = rotate_normalized(base.r, unit);
+                origin = base.p;
+                mode = component < 3u ? 3u : 4u;
+            }
         }
     }
     // only the rows below this step's extent can have a link; the rows up to the previous extent were cleared above

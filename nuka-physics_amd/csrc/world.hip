@@ -327,6 +327,23 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
     c.contact_cone = d.contact_cone;
     c.contact_impratio = d.contact_impratio > 0.0f ? d.contact_impratio : 1.0f;
     c.floating_root = m.joint_type[0] == kFloatingBase ? 1u : 0u;
+    // a free rigid body: the template's one link, stepped by the rigid-body ops
+    c.free_body = d.struct_size >= sizeof(nuka_template_desc_t) && d.free_body != 0u ? 1u : 0u;
+    c.body_inv_mass = 0.0f;
+    c.body_inv_inertia[0] = c.body_inv_inertia[1] = c.body_inv_inertia[2] = 0.0f;
+    if (c.free_body != 0u) {
+        if (nl != 1u || c.floating_root == 0u) throw std::invalid_argument("a free body is a template of one link with a floating root");
+        if (c.joint_limit_rows + c.joint_friction_rows + c.joint_drive_rows != 0u || c.integrator != 0u)
+            throw std::invalid_argument("a free body has no joint rows, drives or joint integrator");
+        if (c.any_mujoco != 0u) throw NotSupported("a free body takes the native contact law on this path");
+        if (m.link_body[0] == kInvalid) throw std::invalid_argument("a free body needs its own body row: its state lives there");
+        if (!(d.link_mass[0] > 0.0f) || !std::isfinite(d.link_mass[0])) throw std::invalid_argument("a free body needs a positive mass");
+        c.body_inv_mass = 1.0f / d.link_mass[0];
+        for (uint32_t k = 0u; k < 3u; ++k) {
+            if (!(d.link_diag_inertia[k] > 0.0f) || !std::isfinite(d.link_diag_inertia[k])) throw std::invalid_argument("a free body needs positive principal moments");
+            c.body_inv_inertia[k] = 1.0f / d.link_diag_inertia[k];
+        }
+    }
     c.max_points_per_slot = max_points;
     // the coordinates a contact can act on: those on the way to the root from a link that carries a shape that can pair
     c.contact_dof_end = 0u;
@@ -386,7 +403,9 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(contact_side_b_kind, kU32, E * S) X(contact_side_a_index, kU32, E * S) X(contact_side_b_index, kU32, E * S) \
     X(contact_link, kU32, E * S) \
     X(step_env_status, kU32, E) X(step_link_impulse, kF32, E * nl * 3) X(step_link_moment, kF32, E * nl * 3) \
-    X(step_joint_limit_impulse, kF32, E * nl * 2)
+    X(step_joint_limit_impulse, kF32, E * nl * 2) \
+    X(body_linear_velocity, kF32, E * nb * 3) X(body_angular_velocity, kF32, E * nb * 3) X(body_world_inv_inertia, kF32, E * nb * 6) \
+    X(body_gyro_residual, kF32, E * nb) X(body_gyro_iterations, kU32, E * nb) X(body_gyro_status, kU32, E * nb)
 
 #define NKH_MODEL_FIELDS(X) \
     X(joint_type, kU8) X(parent_link, kU32) X(joint_axis, kF32) X(parent_offset, kF32) X(link_local_pose, kF32) \
@@ -534,6 +553,7 @@ std::mutex g_static_reset_mutex;                            // guards the host s
 
 bool CheckpointKeeps(const char* name) {
     for (const char* kept : {"q", "qdot", "qddot", "tau", "base_pose", "link_pose", "link_velocity", "body_pose", "lambda", "link_wrench",
+                             "body_linear_velocity", "body_angular_velocity",
                              "drive_target", "drive_stiffness", "drive_damping", "drive_force_limit", "drive_joint_force_limit",
                              "velocity_target", "actuator_noload_speed",
                              "contact_cache_pair", "contact_cache_feature", "contact_cache_material", "contact_cache_lambda",
@@ -640,10 +660,19 @@ void BuildPipeline(World& w) {
         w.calls.push_back({uint16_t(op), params});
     };
     add(NkOp::SnapshotStepVelocity, &w.p_snapshot);
-    add(NkOp::FkWorldPoses, &w.p_fk);
-    add(NkOp::ApplyDrives, &w.p_drives);
-    add(NkOp::ArticulationDynamics, &w.p_dynamics);
-    add(NkOp::IntegrateVelocity, &w.p_int_vel);
+    if (m.free_body != 0u) {
+        // a world of free bodies (pipeline.cpp:434-443, 600-606): the bodies' velocity update, with the block the solve
+        // descends on, then the poses of their collidable rows
+        w.p_int_vel.total_body_count = E * nb > 0u ? E * nb : E;
+        w.p_int_pos.total_body_count = w.p_int_vel.total_body_count;
+        add(NkOp::IntegrateVelocity, &w.p_int_vel);
+        add(NkOp::FkWorldPoses, &w.p_fk);
+    } else {
+        add(NkOp::FkWorldPoses, &w.p_fk);
+        add(NkOp::ApplyDrives, &w.p_drives);
+        add(NkOp::ArticulationDynamics, &w.p_dynamics);
+        add(NkOp::IntegrateVelocity, &w.p_int_vel);
+    }
     if (has_contacts) {   // rows of any kind: contact slots, joint limits, joint friction, drives (pipeline.cpp:207)
         if (m.contact_slots > 0u) {
             add(NkOp::SyncLinkBodyPose, &w.p_sync);
@@ -663,7 +692,7 @@ void BuildPipeline(World& w) {
     if (m.integrator != 0u) add(NkOp::ArticulationDamping, &w.p_damping);   // pipeline.cpp:939-951
     add(NkOp::IntegratePosition, &w.p_int_pos);
     add(NkOp::FkWorldPoses, &w.p_fk);
-    add(NkOp::FkLinkVelocities, &w.p_fk_velocity);
+    if (m.free_body == 0u) add(NkOp::FkLinkVelocities, &w.p_fk_velocity);   // a free body's twist words hold its six coordinates
     if (nb > 0u) add(NkOp::SyncLinkBodyPose, &w.p_sync);
     // a pure readout, part of the step only once a consumer has asked for one of its fields (pipeline.cpp:990-1005)
     w.p_readout_contacts = {};
@@ -1396,7 +1425,7 @@ int nuka_hip_model_view_set_count(nuka_phi_model_view* model, const char* name, 
     COUNT(links_per_env) COUNT(bodies_per_env) COUNT(dof) COUNT(max_dof) COUNT(max_depth) COUNT(contact_slots) COUNT(rows_per_env)
     COUNT(contact_rows_per_env) COUNT(profile_count) COUNT(floating_root) COUNT(max_points_per_slot) COUNT(excluded_pair_count)
     COUNT(sweep_passes) COUNT(pairable_count) COUNT(contact_dof_end) COUNT(rows_from_links) COUNT(joint_limit_rows) COUNT(joint_friction_rows) COUNT(joint_drive_rows)
-    COUNT(drive_mode) COUNT(any_mujoco) COUNT(contact_cone) COUNT(integrator)
+    COUNT(drive_mode) COUNT(any_mujoco) COUNT(contact_cone) COUNT(integrator) COUNT(free_body)
 #undef COUNT
     return -1;
 }
@@ -1445,6 +1474,7 @@ constexpr PublicField kPublicFields[] = {
     {NUKA_FIELD_UCONTACT_SIDE_B, "ucontact_b", 16u}, {NUKA_FIELD_UCONTACT_IMPULSE, "ucontact_impulse", 48u},
     {NUKA_FIELD_JOINT_GRAVITY_FORCE, "joint_gravity_force", 4u}, {NUKA_FIELD_ROW_PENETRATION, "row_penetration", 4u},
     {NUKA_FIELD_ROW_LAMBDA, "lambda", 4u},
+    {NUKA_FIELD_BODY_LINEAR_VELOCITY, "body_linear_velocity", 12u}, {NUKA_FIELD_BODY_ANGULAR_VELOCITY, "body_angular_velocity", 12u},
 };
 
 // The world's field a public or library id stands for and the stride of its view; null when the id is not served.
@@ -2003,6 +2033,7 @@ nuka_result_t SetParam(World& w, nuka_world_handle handle, uint32_t p, uint32_t 
     bool ok = false;
     switch (p) {
         case kLinkMass: {   // the centre of mass and the rotational inertia about it stay (params.cpp:112-121)
+            if (w.model.free_body != 0u) return Error(NUKA_RESULT_NOT_SUPPORTED, "a free body's mass changes through a rebuild in this world");
             float inertia[36];
             MakeSpatialInertia(f, w.host.link_diag_inertia.data() + 3u * element, w.host.link_inertial_frame.data() + 7u * element, inertia);
             ok = PutTemplate(w, "link_inertia", size_t{36u} * element, inertia, 36u);

@@ -93,7 +93,7 @@ void nko_env_aabbs(nko_world* w, uint32_t env) {
         /* :262-264: a free body's own row moves with it - its speed, and its turning rate over the shape's radius */
         float speed = 0.0f;
         if (t->free_body && b == t->link_body[0]) {
-            const float* lv = w->body_linear_velocity + (size_t)env * 3u, *av = w->body_angular_velocity + (size_t)env * 3u;
+            const float* lv = w->body_linear_velocity + (bbase + b) * 3u, *av = w->body_angular_velocity + (bbase + b) * 3u;
             const float radius = sqrtf(he.x * he.x + he.y * he.y + he.z * he.z) + sqrtf(0.0f);
             speed = fmaxf(0.0f, sqrtf(lv[0] * lv[0] + lv[1] * lv[1] + lv[2] * lv[2]) + sqrtf(av[0] * av[0] + av[1] * av[1] + av[2] * av[2]) * radius);
         }
@@ -784,7 +784,7 @@ void nko_env_narrowphase(nko_world* w, uint32_t env) {
                 const float* center = w->body_pose + at * 7u, *lo = w->body_aabb_lo + at * 3u, *hi = w->body_aabb_hi + at * 3u;
                 const v3 extent = v3_make(fmaxf(fabsf(lo[0] - center[0]), fabsf(hi[0] - center[0])), fmaxf(fabsf(lo[1] - center[1]), fabsf(hi[1] - center[1])),
                                           fmaxf(fabsf(lo[2] - center[2]), fabsf(hi[2] - center[2])));
-                const float* lv = w->body_linear_velocity + (size_t)env * 3u, *av = w->body_angular_velocity + (size_t)env * 3u;
+                const float* lv = w->body_linear_velocity + at * 3u, *av = w->body_angular_velocity + at * 3u;
                 speeds[side] = fmaxf(0.0f, sqrtf(lv[0] * lv[0] + lv[1] * lv[1] + lv[2] * lv[2]) +
                                            sqrtf((av[0] * av[0] + av[1] * av[1] + av[2] * av[2]) * (extent.x * extent.x + extent.y * extent.y + extent.z * extent.z)));
             }

@@ -5,9 +5,10 @@
  * block of the tile in it (block_descent_rigid.cuh, block_descent_tile.cuh:541-603), BodyIntegratePositionKernel with the
  * free-rotation solve after it.  The body's coordinates are its linear velocity and its angular velocity about the
  * centre of mass, both in world axes.  Here the body is the one link of the template: `base_pose` is the body's pose,
- * `body_linear_velocity` / `body_angular_velocity` its state, and the six coordinates pass through the link's twist
- * words (`link_velocity`: linear first, then angular) to the row assembly and the block descent, which take the block's
- * mass matrix and factor from `m` / `m_factor` as they do for an articulation.
+ * `body_linear_velocity` / `body_angular_velocity` (per body row, as in the reference: the link's own row holds them)
+ * its state, and the six coordinates pass through the link's twist words (`link_velocity`: linear first, then angular)
+ * to the row assembly and the block descent, which take the block's mass matrix and factor from `m` / `m_factor` as
+ * they do for an articulation.
  */
 #include "nko_internal.h"
 
@@ -157,9 +158,10 @@ static v3 inverse_inertia_of(const nko_template* t) {   /* cook: body_inv_inerti
 void nko_env_body_integrate_velocity(nko_world* w, uint32_t env) {
     const nko_template* t = &w->t;
     const float dt = w->cfg.fixed_dt;
-    float* lin = w->body_linear_velocity + (size_t)env * 3u, *ang = w->body_angular_velocity + (size_t)env * 3u;
+    const size_t body = (size_t)env * t->nb + t->link_body[0];   /* the body's row among the environment's bodies */
+    float* lin = w->body_linear_velocity + body * 3u, *ang = w->body_angular_velocity + body * 3u;
     float* wrench = w->link_wrench + (size_t)env * 6u;
-    float* inverse = w->body_world_inv_inertia + (size_t)env * 6u;
+    float* inverse = w->body_world_inv_inertia + body * 6u;
     const v3 force = v3_make(wrench[0], wrench[1], wrench[2]), torque = v3_make(wrench[3], wrench[4], wrench[5]);
     for (uint32_t i = 0u; i < 6u; ++i) wrench[i] = 0.0f;
     const float inv_mass = t->body_mass > 0.0f ? 1.0f / t->body_mass : 0.0f;
@@ -205,10 +207,11 @@ void nko_env_body_integrate_position(nko_world* w, uint32_t env) {
     const nko_template* t = &w->t;
     const float dt = w->cfg.fixed_dt;
     const int pos_pass = w->cfg.solver_pos_iters > 0u && t->rows_per_env > 0u;
-    float* lin = w->body_linear_velocity + (size_t)env * 3u, *ang = w->body_angular_velocity + (size_t)env * 3u;
+    const size_t body = (size_t)env * t->nb + t->link_body[0];
+    float* lin = w->body_linear_velocity + body * 3u, *ang = w->body_angular_velocity + body * 3u;
     float* twist = w->link_velocity + (size_t)env * 6u;
     if (t->rows_per_env > 0u) for (uint32_t i = 0u; i < 3u; ++i) { lin[i] = twist[i]; ang[i] = twist[3u + i]; }
-    w->body_gyro_residual[env] = 0.0f; w->body_gyro_iterations[env] = 0u; w->body_gyro_status[env] = 0u;
+    w->body_gyro_residual[body] = 0.0f; w->body_gyro_iterations[body] = 0u; w->body_gyro_status[body] = 0u;
     if (!(t->body_mass > 0.0f)) return;
     xform pose = xform_load(w->base_pose + (size_t)env * 7u);
     const xform frame = xform_load(t->link_inertial_frame);
@@ -217,7 +220,7 @@ void nko_env_body_integrate_position(nko_world* w, uint32_t env) {
     const quat inverse = quat_make(principal.w, -principal.x, -principal.y, -principal.z);
     const v3 w0 = nko_rotate_normalized(inverse, v3_make(ang[0], ang[1], ang[2]));
     const gyro_result gyro = solve_free_rotation(w0, inv_i, dt);
-    w->body_gyro_residual[env] = gyro.residual; w->body_gyro_iterations[env] = gyro.iterations; w->body_gyro_status[env] = gyro.status;
+    w->body_gyro_residual[body] = gyro.residual; w->body_gyro_iterations[body] = gyro.iterations; w->body_gyro_status[body] = gyro.status;
     if (gyro.status != 0u) { w->env_status[env] |= NKO_STATUS_GYRO_FAILURE; return; }
     const v3 momentum = nko_rotate_normalized(principal, v3_make(w0.x / inv_i.x, w0.y / inv_i.y, w0.z / inv_i.z));
     v3 v = v3_make(lin[0], lin[1], lin[2]);
@@ -235,7 +238,7 @@ void nko_env_body_integrate_position(nko_world* w, uint32_t env) {
     const v3 offset = nko_rotate_normalized(q, frame.p);
     pose.p = v3_sub(v3_add(center, v3_scale(v, dt)), offset);
     xform_store(w->base_pose + (size_t)env * 7u, pose);
-    float* world_inverse = w->body_world_inv_inertia + (size_t)env * 6u;
+    float* world_inverse = w->body_world_inv_inertia + body * 6u;
     body_world_inverse_inertia(pose, frame, inv_i, world_inverse);
     const v3 turned = sym_multiply(world_inverse, momentum);
     ang[0] = turned.x; ang[1] = turned.y; ang[2] = turned.z;

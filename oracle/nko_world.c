@@ -221,6 +221,7 @@ static int cook_template(nko_template* t, const nko_template_desc* d) {
     t->joint_friction_rows = any_friction ? nl : 0u;
     t->joint_drive_rows = has_joint_rows && d->drive_rows != 0u ? nl : 0u;
     t->rows_per_env = t->contact_rows_per_env + t->joint_limit_rows + t->joint_friction_rows + t->joint_drive_rows;
+    if (t->free_body && t->link_body[0] == NKO_INVALID) return -1;   /* the body's state lives in its own body row */
     return 0;
 }
 
@@ -270,9 +271,9 @@ nko_world* nko_world_create(const nko_template_desc* tmpl, const nko_world_desc*
     w->m = ALLOC(float, E * md * md); w->m_factor = ALLOC(float, E * md * md); w->qdot_flat = ALLOC(float, E * md);
     w->qdot_pseudo = ALLOC(float, E * nl); w->link_velocity_pseudo = ALLOC(float, E * nl * 6u);
     w->body_pose = ALLOC(float, E * nb * 7u); w->body_aabb_lo = ALLOC(float, E * nb * 3u); w->body_aabb_hi = ALLOC(float, E * nb * 3u);
-    w->body_linear_velocity = ALLOC(float, E * 3u); w->body_angular_velocity = ALLOC(float, E * 3u);
-    w->body_world_inv_inertia = ALLOC(float, E * 6u); w->body_gyro_residual = ALLOC(float, E);
-    w->body_gyro_iterations = ALLOC(uint32_t, E); w->body_gyro_status = ALLOC(uint32_t, E);
+    w->body_linear_velocity = ALLOC(float, E * nb * 3u); w->body_angular_velocity = ALLOC(float, E * nb * 3u);
+    w->body_world_inv_inertia = ALLOC(float, E * nb * 6u); w->body_gyro_residual = ALLOC(float, E * nb);
+    w->body_gyro_iterations = ALLOC(uint32_t, E * nb); w->body_gyro_status = ALLOC(uint32_t, E * nb);
     w->candidate_pairs = ALLOC(uint32_t, E * S * 2u); w->pair_count = ALLOC(uint32_t, E);
     w->ucontact_count = ALLOC(uint32_t, E * S); w->ucontact_a = ALLOC(uint32_t, E * S * 4u); w->ucontact_b = ALLOC(uint32_t, E * S * 4u);
     w->ucontact_law = ALLOC(uint32_t, E * S); w->ucontact_row_range = ALLOC(uint32_t, E * S * 2u);
@@ -388,8 +389,8 @@ void nko_world_destroy(nko_world* w) {
     X(ucontact_impulse, float, E * S * 12u) X(link_contact_wrench, float, E * nl * 6u) \
     X(contact_side_a_kind, uint32_t, E * S) X(contact_side_b_kind, uint32_t, E * S) X(contact_side_a_index, uint32_t, E * S) \
     X(contact_side_b_index, uint32_t, E * S) X(contact_link, uint32_t, E * S) \
-    X(body_linear_velocity, float, E * 3u) X(body_angular_velocity, float, E * 3u) X(body_world_inv_inertia, float, E * 6u) \
-    X(body_gyro_residual, float, E) X(body_gyro_iterations, uint32_t, E) X(body_gyro_status, uint32_t, E)
+    X(body_linear_velocity, float, E * nb * 3u) X(body_angular_velocity, float, E * nb * 3u) X(body_world_inv_inertia, float, E * nb * 6u) \
+    X(body_gyro_residual, float, E * nb) X(body_gyro_iterations, uint32_t, E * nb) X(body_gyro_status, uint32_t, E * nb)
 
 #define TEMPLATE_LIST(X) \
     X(link_inertia, float, nl * 36u) X(link_tree_depth, uint32_t, nl) X(link_child_range, uint32_t, nl * 2u) \
@@ -477,8 +478,9 @@ void nko_snapshot_step_velocity(nko_world* w) {
 static void step_free_body(nko_world* w) {
     for (size_t e = 0u; e < w->env_count; ++e)   /* the six coordinates as the state holds them */
         for (uint32_t i = 0u; i < 3u; ++i) {
-            w->link_velocity[e * 6u + i] = w->body_linear_velocity[e * 3u + i];
-            w->link_velocity[e * 6u + 3u + i] = w->body_angular_velocity[e * 3u + i];
+            const size_t body = e * w->t.nb + w->t.link_body[0];
+            w->link_velocity[e * 6u + i] = w->body_linear_velocity[body * 3u + i];
+            w->link_velocity[e * 6u + 3u + i] = w->body_angular_velocity[body * 3u + i];
         }
     if (w->t.rows_per_env > 0u) nko_snapshot_step_velocity(w);
     nko_body_integrate_velocity(w);

@@ -25,3 +25,19 @@ def rotation_matrix(q):
     return np.array([[1 - 2 * (y * y + z * z), 2 * (x * y - w * z), 2 * (x * z + w * y)],
                      [2 * (x * y + w * z), 1 - 2 * (x * x + z * z), 2 * (y * z - w * x)],
                      [2 * (x * z - w * y), 2 * (y * z + w * x), 1 - 2 * (x * x + y * y)]])
+
+
+def body_field(template, values):
+    """A per-body field of a free-body world from the free body's values [E][k]: the body's own row (the last one of
+    box_template) holds them, the other rows zeros."""
+    values = np.asarray(values, np.float32)
+    nb = len(template.bodies)
+    out = np.zeros((values.shape[0], nb) + values.shape[1:], np.float32)
+    out[:, nb - 1] = values
+    return out
+
+
+def of_body(template, field, E):
+    """The free body's values of a per-body field as downloaded."""
+    nb = len(template.bodies)
+    return np.asarray(field).reshape(E, nb, -1)[:, nb - 1]

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 from conftest import nk
-from rigid import box_template, rotation_matrix
+from rigid import body_field, box_template, of_body, rotation_matrix
 
 abi = nk.abi
 
@@ -62,14 +62,14 @@ def test_free_flight_follows_the_parabola_and_keeps_momentum_and_energy(oracle_p
     pose[:, 3:] /= np.linalg.norm(pose[:, 3:], axis=1, keepdims=True)
     v0 = g.normal(0.0, 1.0, (E, 3)).astype(np.float32)
     w0 = g.normal(0.0, 4.0, (E, 3)).astype(np.float32)
-    w.upload("base_pose", pose); w.upload("body_linear_velocity", v0); w.upload("body_angular_velocity", w0)
+    w.upload("base_pose", pose); w.upload("body_linear_velocity", body_field(t, v0)); w.upload("body_angular_velocity", body_field(t, w0))
     inertia = np.diag([0.02, 0.05, 0.035])
 
     def measures():
         p = w.download("base_pose").reshape(E, 7).astype(np.float64)
         R = np.stack([rotation_matrix(q) for q in p[:, 3:]])
         centre = p[:, :3] + np.einsum("eij,j->ei", R, np.array(com))
-        omega = w.download("body_angular_velocity").reshape(E, 3).astype(np.float64)
+        omega = of_body(t, w.download("body_angular_velocity"), E).astype(np.float64)
         world_inertia = np.einsum("eij,jk,elk->eil", R, inertia, R)
         momentum = np.einsum("eij,ej->ei", world_inertia, omega)
         return centre, momentum, 0.5 * np.einsum("ei,ei->e", omega, momentum)
@@ -81,7 +81,7 @@ def test_free_flight_follows_the_parabola_and_keeps_momentum_and_energy(oracle_p
     n = steps
     expect = c0 + n * dt * v0.astype(np.float64) + np.array([0.0, 0.0, -9.81]) * dt * dt * n * (n + 1) / 2.0
     assert np.abs(c1 - expect).max() <= 2e-4 * np.abs(expect).max()
-    assert np.allclose(w.download("body_linear_velocity").reshape(E, 3), v0 + np.array([0, 0, -9.81]) * dt * n, rtol=2e-5, atol=1e-4)
+    assert np.allclose(of_body(t, w.download("body_linear_velocity"), E), v0 + np.array([0, 0, -9.81]) * dt * n, rtol=2e-5, atol=1e-4)
     # (single precision over two thousand steps: the momentum is rebuilt from the angular velocity at every step)
     assert np.abs(l1 - l0).max() <= 1e-3 * np.abs(l0).max()
     assert np.abs(k1 - k0).max() <= 2e-3 * k0.max()
@@ -98,10 +98,10 @@ def test_symmetric_top_precesses_at_the_closed_form_rate(oracle_py):
     t = box_template(half=(0.1, 0.1, 0.1), mass=1.0, diag=(i1, i1, i3), plane=False)
     w, _ = make(oracle_py, t, 1, dt, gravity=(0.0, 0.0, 0.0))
     w3, wt = 6.0, 1.5
-    w.upload("body_angular_velocity", np.array([[wt, 0.0, w3]], np.float32))
+    w.upload("body_angular_velocity", body_field(t, np.array([[wt, 0.0, w3]], np.float32)))
     w.step(steps)
     pose = w.download("base_pose").reshape(7).astype(np.float64)
-    body = rotation_matrix(pose[3:]).T @ w.download("body_angular_velocity").reshape(3).astype(np.float64)
+    body = rotation_matrix(pose[3:]).T @ of_body(t, w.download("body_angular_velocity"), 1)[0].astype(np.float64)
     rate = (i3 - i1) / i1 * w3
     angle = rate * dt * steps
     # Euler: dw1/dt = -(I3 - I1)/I1 w3 w2, dw2/dt = +(I3 - I1)/I1 w3 w1: the transverse part turns by +rate about axis 3
@@ -125,7 +125,7 @@ def test_row_entries_times_the_coordinates_are_the_contact_point_velocity(oracle
     pose[:, 3:] /= np.linalg.norm(pose[:, 3:], axis=1, keepdims=True)
     v = g.normal(0.0, 0.3, (E, 3)).astype(np.float32)
     om = g.normal(0.0, 1.0, (E, 3)).astype(np.float32)
-    w.upload("base_pose", pose); w.upload("body_linear_velocity", v); w.upload("body_angular_velocity", om)
+    w.upload("base_pose", pose); w.upload("body_linear_velocity", body_field(t, v)); w.upload("body_angular_velocity", body_field(t, om))
     zero_gravity = w
     for name in ("body_integrate_velocity", "fk_world_poses", "sync_link_body_pose", "build_aabbs", "query_pairs", "narrowphase", "assemble_rows"):
         zero_gravity.op(name)
@@ -136,8 +136,8 @@ def test_row_entries_times_the_coordinates_are_the_contact_point_velocity(oracle
     points = w.download("row_cj_point").reshape(E, R, 3).astype(np.float64) + 0.0
     points_b = w.download("row_cj_point_b").reshape(E, R, 3).astype(np.float64)
     link_a = w.download("row_cj_link").reshape(E, R)
-    vel = w.download("body_linear_velocity").reshape(E, 3).astype(np.float64)
-    omega = w.download("body_angular_velocity").reshape(E, 3).astype(np.float64)
+    vel = of_body(t, w.download("body_linear_velocity"), E).astype(np.float64)
+    omega = of_body(t, w.download("body_angular_velocity"), E).astype(np.float64)
     p = w.download("base_pose").reshape(E, 7).astype(np.float64)
     checked = 0
     for e in range(E):
@@ -165,7 +165,7 @@ def test_a_box_at_rest_carries_its_weight_and_a_sliding_box_stops_by_coulombs_la
     pose[:, 2] = 0.1; pose[:, 3] = 1.0
     v = np.zeros((E, 3), np.float32)
     v[1, 0] = 1.0                                       # the second box slides along x
-    w.upload("base_pose", pose); w.upload("body_linear_velocity", v)
+    w.upload("base_pose", pose); w.upload("body_linear_velocity", body_field(t, v))
     R = w.rows_per_env
     n = 30
     w.step(n)
@@ -175,10 +175,10 @@ def test_a_box_at_rest_carries_its_weight_and_a_sliding_box_stops_by_coulombs_la
     normal = (rows[:, :, 0] & (1 << 6)) != 0
     support = np.where(normal, lam, 0.0).sum(1) / dt     # the rows' impulses over the step: a force
     assert np.allclose(support, mass * 9.81, rtol=2e-3), support
-    speeds = w.download("body_linear_velocity").reshape(E, 3)
+    speeds = of_body(t, w.download("body_linear_velocity"), E)
     assert np.abs(speeds[0]).max() <= 1e-4                                   # at rest stays at rest
     assert abs(speeds[1, 0] - (1.0 - mu * 9.81 * n * dt)) <= 5e-3, speeds[1]  # Coulomb: deceleration mu g
     assert abs(w.download("base_pose").reshape(E, 7)[0, 2] - 0.1) <= 1e-3
     w.step(80)                                                               # ... and comes to a stop, not back
-    assert np.abs(w.download("body_linear_velocity").reshape(E, 3)[1]).max() <= 2e-3
+    assert np.abs(of_body(t, w.download("body_linear_velocity"), E)[1]).max() <= 2e-3
     w.close()
