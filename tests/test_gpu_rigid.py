@@ -126,3 +126,71 @@ def test_a_free_body_refuses_what_it_does_not_build(device):
     t.add_link(abi.JOINT_REVOLUTE, 0)
     with pytest.raises(Exception):
         nk.World(device, t, abi.world_desc(4, 1.0 / 240.0))
+
+
+def shaped_template(kind, params, mu=0.6):
+    t = abi.Template()
+    t.free_body = True
+    t.add_link(abi.JOINT_FLOATING, None, mass=1.5, diag_inertia=(0.012, 0.015, 0.02), com=(0.01, 0.0, 0.005))
+    profile = t.add_profile(mu)
+    t.add_body(abi.ROLE_STATIC, kind=abi.SHAPE_PLANE, contype=2, conaffinity=1, profile=profile)
+    t.add_body(abi.ROLE_LINK_BODY, link=0, kind=kind, params=params, contype=1, conaffinity=2, profile=profile)
+    t.max_contacts_per_env = 1
+    return t
+
+
+@pytest.mark.parametrize("kind,params,height", [(abi.SHAPE_SPHERE, (0.1, 0, 0, 0), 0.1), (abi.SHAPE_CAPSULE, (0.06, 0.1, 0, 0), 0.06),
+                                                (abi.SHAPE_CYLINDER, (0.08, 0.1, 0, 0), 0.08)])
+def test_other_shapes_of_a_free_body_follow_the_oracle(oracle_py, device, kind, params, height):
+    """A ball, a lying capsule and a lying cylinder (the single-point pairs take the merged collision kernel, the others
+    the general one): forty steps of rolling and sliding on the plane, in graph mode."""
+    E = 96
+    t = shaped_template(kind, params)
+    world, oracle = pair(oracle_py, device, t, E, vel_iters=8, pos_iters=4, contact_margin=0.02)
+    pose, v, w = seeded_boxes(E, 5 + kind, height=height, spread=0.02, tilt=0.0, speed=0.5, spin=2.0)
+    if kind != abi.SHAPE_SPHERE:   # lying on its side: the axis along x
+        pose[:, 3:] = np.array([np.sqrt(0.5), 0.0, np.sqrt(0.5), 0.0], np.float32)
+    put(world, oracle, t, pose, v, w)
+    world.set_execution_mode(True)
+    for steps in (1, 39):
+        world.step(steps); world.synchronize()
+        oracle.step(steps)
+        assert np.array_equal(world.download("env_status"), oracle.download("env_status"))
+        assert np.array_equal(world.download("contact_count"), oracle.download("contact_count"))
+        tol = TOL if steps == 1 else 20 * TOL
+        close_env(world, oracle, "base_pose", E, tol=tol)
+        got, expect = of_body(t, world.download("body_angular_velocity"), E), of_body(t, oracle.download("body_angular_velocity"), E)
+        assert np.abs(got - expect).max() <= 20 * tol * max(1.0, np.abs(expect).max())
+    assert (oracle.download("contact_count") > 0).mean() >= 0.5
+    world.close(); oracle.close()
+
+
+def test_checkpoint_reset_and_large_batches_of_free_bodies(oracle_py, device):
+    """The body's state is part of a checkpoint and of a reset; a batch of 8192 boxes (the solve's kernels for three waves
+    a SIMD) gives in every copy the bits a batch of 64 gives."""
+    E, copies = 64, 128
+    t = box_template(half=(0.2, 0.15, 0.1), mass=3.0, diag=(0.03, 0.04, 0.05), mu=0.6)
+    desc = abi.world_desc(E, 1.0 / 240.0, vel_iters=8, pos_iters=4, contact_margin=0.02)
+    small = nk.World(device, t, desc)
+    pose, v, w = seeded_boxes(E, 21)
+    small.upload("base_pose", pose); small.upload("body_linear_velocity", body_field(t, v)); small.upload("body_angular_velocity", body_field(t, w))
+    start = small.checkpoint()
+    small.step(5); small.synchronize()
+    after = {name: small.download(name) for name in ("base_pose", "body_linear_velocity", "body_angular_velocity", "lambda")}
+    small.restore(start)
+    assert np.array_equal(of_body(t, small.download("body_linear_velocity"), E), v) and np.array_equal(small.download("base_pose").reshape(E, 7), pose)
+    small.step(5); small.synchronize()
+    for name, value in after.items():
+        assert np.array_equal(small.download(name), value), name
+    big = nk.World(device, t, abi.world_desc(E * copies, 1.0 / 240.0, vel_iters=8, pos_iters=4, contact_margin=0.02))
+    assert big.info.solver_blocks_per_cu > 8
+    big.upload("base_pose", np.tile(pose, (copies, 1)))
+    big.upload("body_linear_velocity", np.tile(body_field(t, v), (copies, 1, 1)))
+    big.upload("body_angular_velocity", np.tile(body_field(t, w), (copies, 1, 1)))
+    big.step(5); big.synchronize()
+    for name, value in after.items():
+        batch = big.download(name).reshape(copies, -1)
+        assert np.array_equal(np.broadcast_to(value.reshape(1, -1), batch.shape), batch), name
+    small.reset(); small.synchronize()
+    assert not small.download("body_linear_velocity").any() and not small.download("body_angular_velocity").any()
+    small.close(); big.close()
