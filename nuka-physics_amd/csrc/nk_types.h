@@ -86,7 +86,6 @@ struct ModelView {
     // 1: the template's one link is a free rigid body, stepped by the rigid-body ops (ops_rigid.hip): its six coordinates
     // are its linear velocity and its angular velocity about the centre of mass, in world axes
     uint32_t free_body;
-    float body_inv_mass, body_inv_inertia[3];   // 1 / mass and 1 / principal moments (src/nk/model/fields.yaml:17, 108)
     const uint8_t* joint_type;
     const uint32_t* parent_link;
     const float* joint_axis;
@@ -142,6 +141,7 @@ struct DataView {
     float *body_pose, *body_aabb_lo, *body_aabb_hi;
     // the free body of a free_body world, one an environment (fields.yaml:102-103, 569; articulation.cu:1068-1070)
     float *body_linear_velocity, *body_angular_velocity, *body_world_inv_inertia, *body_gyro_residual;
+    float *body_inv_mass, *body_inv_inertia, *body_inertial_frame;   // fields.yaml:17, 108, 568: 1 / mass, 1 / principal moments, the inertial frame in the body's
     uint32_t *body_gyro_iterations, *body_gyro_status;
     uint32_t *candidate_pairs, *pair_count;
     uint32_t *ucontact_count, *ucontact_a, *ucontact_b, *ucontact_law, *ucontact_row_range;

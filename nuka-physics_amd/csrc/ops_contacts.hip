@@ -1253,7 +1253,8 @@ __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4, 4
                 // a free body's coordinates: linear velocity, then angular velocity about the centre of mass, world axes -
                 // the row's jlin and jang = (point - com) x jlin (assemble_rows.cu:537-538, 680-681)
                 axis_world = unit;
-                origin = add3(base.p, rotate_normalized(base.r, V3{m.link_inertial_frame[0], m.link_inertial_frame[1], m.link_inertial_frame[2]}));
+                const float* frame = d.body_inertial_frame + (size_t{env} * m.bodies_per_env + m.link_body[0]) * 7u;
+                origin = add3(base.p, rotate_normalized(base.r, V3{frame[0], frame[1], frame[2]}));
                 mode = component < 3u ? 4u : 3u;
             } else {
                 axis_world = rotate_normalized(base.r, unit);

@@ -148,14 +148,15 @@ __global__ void __launch_bounds__(256) BodyIntegrateVelocityKernel(ModelView m, 
     const V3 force{wrench[0], wrench[1], wrench[2]}, torque{wrench[3], wrench[4], wrench[5]};
     if (p.clear_body_forces != 0u)
         for (uint32_t i = 0u; i < 6u; ++i) wrench[i] = 0.0f;
-    const float inv_mass = m.body_inv_mass;
+    const float inv_mass = d.body_inv_mass[body];
     const uint32_t md = m.max_dof;
     float* M = d.m + size_t{env} * md * md, *F = d.m_factor + size_t{env} * md * md;
     V3 v{lin[0], lin[1], lin[2]}, w{ang[0], ang[1], ang[2]};
     float world_inverse[6] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     if (inv_mass > 0.0f) {
-        const Xf pose = load_xf(d.base_pose + size_t{env} * 7u), frame = load_xf(m.link_inertial_frame);
-        body_world_inverse_inertia(pose, frame, V3{m.body_inv_inertia[0], m.body_inv_inertia[1], m.body_inv_inertia[2]}, world_inverse);
+        const Xf pose = load_xf(d.base_pose + size_t{env} * 7u), frame = load_xf(d.body_inertial_frame + body * 7u);
+        const float* inv_i = d.body_inv_inertia + body * 3u;
+        body_world_inverse_inertia(pose, frame, V3{inv_i[0], inv_i[1], inv_i[2]}, world_inverse);
         const V3 g{p.gravity[0], p.gravity[1], p.gravity[2]};
         v = add3(v, scale3(add3(scale3(g, 1.0f - 0.0f), scale3(force, inv_mass)), p.dt));
         w = add3(w, scale3(sym_multiply(world_inverse, torque), p.dt));
@@ -216,10 +217,10 @@ __global__ void __launch_bounds__(256) BodyIntegratePositionKernel(ModelView m, 
     if (m.rows_per_env > 0u)
         for (uint32_t i = 0u; i < 3u; ++i) { lin[i] = twist[i]; ang[i] = twist[3u + i]; }
     d.body_gyro_residual[body] = 0.0f; d.body_gyro_iterations[body] = 0u; d.body_gyro_status[body] = 0u;
-    if (!(m.body_inv_mass > 0.0f)) return;
+    if (!(d.body_inv_mass[body] > 0.0f)) return;
     Xf pose = load_xf(d.base_pose + size_t{env} * 7u);
-    const Xf frame = load_xf(m.link_inertial_frame);
-    const V3 inv_i{m.body_inv_inertia[0], m.body_inv_inertia[1], m.body_inv_inertia[2]};
+    const Xf frame = load_xf(d.body_inertial_frame + body * 7u);
+    const V3 inv_i{d.body_inv_inertia[body * 3u], d.body_inv_inertia[body * 3u + 1u], d.body_inv_inertia[body * 3u + 2u]};
     const Q4 principal = qnormalize_le(qmul(pose.r, frame.r), 1.0e-12f);
     const Q4 inverse{principal.w, -principal.x, -principal.y, -principal.z};
     const V3 w0 = rotate_normalized(inverse, V3{ang[0], ang[1], ang[2]});

@@ -329,8 +329,6 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
     c.floating_root = m.joint_type[0] == kFloatingBase ? 1u : 0u;
     // a free rigid body: the template's one link, stepped by the rigid-body ops
     c.free_body = d.struct_size >= sizeof(nuka_template_desc_t) && d.free_body != 0u ? 1u : 0u;
-    c.body_inv_mass = 0.0f;
-    c.body_inv_inertia[0] = c.body_inv_inertia[1] = c.body_inv_inertia[2] = 0.0f;
     if (c.free_body != 0u) {
         if (nl != 1u || c.floating_root == 0u) throw std::invalid_argument("a free body is a template of one link with a floating root");
         if (c.joint_limit_rows + c.joint_friction_rows + c.joint_drive_rows != 0u || c.integrator != 0u)
@@ -338,11 +336,8 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
         if (c.any_mujoco != 0u) throw NotSupported("a free body takes the native contact law on this path");
         if (m.link_body[0] == kInvalid) throw std::invalid_argument("a free body needs its own body row: its state lives there");
         if (!(d.link_mass[0] > 0.0f) || !std::isfinite(d.link_mass[0])) throw std::invalid_argument("a free body needs a positive mass");
-        c.body_inv_mass = 1.0f / d.link_mass[0];
-        for (uint32_t k = 0u; k < 3u; ++k) {
+        for (uint32_t k = 0u; k < 3u; ++k)
             if (!(d.link_diag_inertia[k] > 0.0f) || !std::isfinite(d.link_diag_inertia[k])) throw std::invalid_argument("a free body needs positive principal moments");
-            c.body_inv_inertia[k] = 1.0f / d.link_diag_inertia[k];
-        }
     }
     c.max_points_per_slot = max_points;
     // the coordinates a contact can act on: those on the way to the root from a link that carries a shape that can pair
@@ -405,7 +400,8 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(step_env_status, kU32, E) X(step_link_impulse, kF32, E * nl * 3) X(step_link_moment, kF32, E * nl * 3) \
     X(step_joint_limit_impulse, kF32, E * nl * 2) \
     X(body_linear_velocity, kF32, E * nb * 3) X(body_angular_velocity, kF32, E * nb * 3) X(body_world_inv_inertia, kF32, E * nb * 6) \
-    X(body_gyro_residual, kF32, E * nb) X(body_gyro_iterations, kU32, E * nb) X(body_gyro_status, kU32, E * nb)
+    X(body_gyro_residual, kF32, E * nb) X(body_gyro_iterations, kU32, E * nb) X(body_gyro_status, kU32, E * nb) \
+    X(body_inv_mass, kF32, E * nb) X(body_inv_inertia, kF32, E * nb * 3) X(body_inertial_frame, kF32, E * nb * 7)
 
 #define NKH_MODEL_FIELDS(X) \
     X(joint_type, kU8) X(parent_link, kU32) X(joint_axis, kF32) X(parent_offset, kF32) X(link_local_pose, kF32) \
@@ -949,6 +945,20 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
                 if (bytes == 0u) return true;
                 return Iface(w.arena)->upload(w.arena, src, size_t(static_cast<char*>(field) - base), bytes) == uint8_t(Status::Ok);
             };
+            // the bodies' inertial parameters (fields.yaml:17, 108, 568): a free body's in its own row - 1 / mass, 1 / principal
+            // moments, the inertial frame - and zero mass (a body the rigid-body ops leave alone) in every other row
+            std::vector<float> inv_mass(E * nb, 0.0f), inv_inertia(E * nb * 3u, 0.0f), inertial_frame(E * nb * 7u, 0.0f);
+            for (size_t e = 0u; e < E; ++e)
+                for (size_t b = 0u; b < nb; ++b) {
+                    inertial_frame[(e * nb + b) * 7u + 3u] = 1.0f;
+                    if (hc.free_body == 0u || b != w.host.link_body[0]) continue;
+                    inv_mass[e * nb + b] = 1.0f / w.host.link_mass[0];
+                    for (size_t k = 0u; k < 3u; ++k) inv_inertia[(e * nb + b) * 3u + k] = 1.0f / w.host.link_diag_inertia[k];
+                    std::memcpy(&inertial_frame[(e * nb + b) * 7u], w.host.link_inertial_frame.data(), 7u * sizeof(float));
+                }
+            if (!put(w.data.body_inv_mass, inv_mass.data(), inv_mass.size() * 4u) || !put(w.data.body_inv_inertia, inv_inertia.data(), inv_inertia.size() * 4u) ||
+                !put(w.data.body_inertial_frame, inertial_frame.data(), inertial_frame.size() * 4u))
+                return Error(NUKA_RESULT_DEVICE_ERROR, "initial state upload failed");
             if (!put(w.data.base_pose, base_pose.data(), base_pose.size() * 4u) || !put(w.data.link_pose, link_pose.data(), link_pose.size() * 4u) ||
                 !put(w.data.body_pose, body_pose.data(), body_pose.size() * 4u) || !put(w.data.row_cj_link, invalid.data(), invalid.size() * 4u) ||
                 !put(w.data.row_cj_link_b, invalid.data(), invalid.size() * 4u) || !put(w.data.row_unit, invalid.data(), invalid.size() * 4u))
