@@ -167,7 +167,7 @@ int nuka_hip_bind_views(const char* const* names, void* const* pointers, uint32_
 /* The per-environment counts at the head of the model view, by name (links_per_env, bodies_per_env, dof, max_dof,
  * max_depth, contact_slots, rows_per_env, contact_rows_per_env, profile_count, floating_root, max_points_per_slot,
  * excluded_pair_count, joint_limit_rows, joint_friction_rows, joint_drive_rows, drive_mode, any_mujoco, contact_cone,
- * integrator, contact_dof_end, rows_from_links).  0 on success, -1 for an unknown name. */
+ * integrator, contact_dof_end, rows_from_links, free_body).  0 on success, -1 for an unknown name. */
 int nuka_hip_model_view_set_count(nuka_phi_model_view* model, const char* name, uint32_t value);
 
 #ifdef __cplusplus
