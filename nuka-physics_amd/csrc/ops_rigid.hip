@@ -56,79 +56,98 @@ __device__ bool sym_invert(const float* m, float* out) {
 __device__ V3 body_center_of_mass(Xf pose, Xf frame) { return add3(pose.p, rotate_normalized(pose.r, frame.p)); }
 __device__ void body_world_inverse_inertia(Xf pose, Xf frame, V3 inv_i, float* out) { from_rotated_diagonal(inv_i, qmul(pose.r, frame.r), out); }
 
-__device__ float max_abs(V3 v) { return fmaxf(fabsf(v.x), fmaxf(fabsf(v.y), fabsf(v.z))); }
 __device__ bool finite3(V3 v) { return isfinite(v.x) && isfinite(v.y) && isfinite(v.z); }
 
-// rigid_types.cuh:38-121 SolveFreeRotation: the implicit midpoint rule of Euler's equations in the principal frame on
-// the angular momentum scaled to unit size, by Newton steps with halving; `midpoint` is the angular velocity at the
-// middle of the step
-struct GyroResult { V3 midpoint; float residual; uint32_t iterations, status; };
-__device__ V3 gyro_residual(V3 u0, V3 c, V3 u) {
-    const V3 mid = scale3(add3(u0, u), 0.5f);
-    return V3{u.x - u0.x + c.x * mid.y * mid.z, u.y - u0.y + c.y * mid.z * mid.x, u.z - u0.z + c.z * mid.x * mid.y};
-}
-__device__ GyroResult solve_free_rotation(V3 w0, V3 inv_i, float dt) {
-    GyroResult out{V3{0.0f, 0.0f, 0.0f}, 0.0f, 0u, 0u};
-    if (!finite3(w0) || !finite3(inv_i) || inv_i.x <= 0.0f || inv_i.y <= 0.0f || inv_i.z <= 0.0f) {
-        out.status = 2u; out.residual = INFINITY;   // kBodyGyroInvalidInput
-        return out;
+// The free-rotation step (rigid_types.cuh:38-121 SolveFreeRotation): Euler's equations in the principal frame by the
+// implicit midpoint rule, m1 - m0 = dt (m_mid x w_mid), solved for the end-of-step angular momentum.  The unknown is the
+// momentum scaled to unit size, `g(u) = u - u0 + c o (mid_y mid_z, mid_z mid_x, mid_x mid_y)` with mid = (u0 + u) / 2
+// and c = dt (a_y - a_z, a_z - a_x, a_x - a_y), a = scaled inverse moments; Newton steps on g with a halved step while
+// the residual does not fall, at most twelve, to a residual of 1e-6.  Returns the angular velocity at the middle of the
+// step, which turns the pose.
+struct FreeRotation { V3 midpoint; float residual; uint32_t iterations, status; };
+enum : uint32_t { kGyroConverged = 0u, kGyroNotConverged = 1u, kGyroInvalidInput = 2u };   // op_schema.hpp:53-54
+
+struct MidpointRule {
+    float start[3], coupling[3];
+    __device__ void residual(const float (&u)[3], float (&g)[3]) const {
+        const float mid[3] = {(start[0] + u[0]) * 0.5f, (start[1] + u[1]) * 0.5f, (start[2] + u[2]) * 0.5f};
+#pragma unroll
+        for (int k = 0; k < 3; ++k) g[k] = u[k] - start[k] + coupling[k] * mid[(k + 1) % 3] * mid[(k + 2) % 3];
     }
-    const V3 m0{w0.x / inv_i.x, w0.y / inv_i.y, w0.z / inv_i.z};
-    const float scale = max_abs(m0);
-    if (!finite3(m0)) { out.status = 2u; out.residual = INFINITY; return out; }
-    if (scale == 0.0f) return out;
-    const V3 u0 = scale3(m0, 1.0f / scale);
-    const V3 a = scale3(inv_i, scale);
-    const V3 c{dt * (a.y - a.z), dt * (a.z - a.x), dt * (a.x - a.y)};
-    constexpr float tolerance = 1.0e-6f;
-    constexpr uint32_t max_iterations = 12u, max_backtracks = 8u;
-    V3 u = u0;
-    for (uint32_t iteration = 0u; iteration <= max_iterations; ++iteration) {
-        const V3 r = gyro_residual(u0, c, u);
-        out.residual = finite3(r) ? max_abs(r) : INFINITY;
-        if (out.residual <= tolerance) {
-            const V3 mid = scale3(add3(u0, u), 0.5f);
-            out.midpoint = V3{a.x * mid.x, a.y * mid.y, a.z * mid.z};
+    // dg/du: the identity and half the coupling times the other two midpoint components
+    __device__ void jacobian(const float (&u)[3], float (&j)[3][3]) const {
+        const float mid[3] = {(start[0] + u[0]) * 0.5f, (start[1] + u[1]) * 0.5f, (start[2] + u[2]) * 0.5f};
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            j[k][k] = 1.0f;
+            j[k][(k + 1) % 3] = 0.5f * coupling[k] * mid[(k + 2) % 3];
+            j[k][(k + 2) % 3] = 0.5f * coupling[k] * mid[(k + 1) % 3];
+        }
+    }
+};
+__device__ float largest3(const float (&v)[3]) { return fmaxf(fabsf(v[0]), fmaxf(fabsf(v[1]), fabsf(v[2]))); }
+__device__ bool all_finite3(const float (&v)[3]) { return isfinite(v[0]) && isfinite(v[1]) && isfinite(v[2]); }
+// x of a x = b by elimination with row pivoting, columns left to right; false when a pivot is below 1e-12 or not finite
+__device__ bool solve3(float (&a)[3][3], float (&b)[3], float (&x)[3]) {
+    for (int column = 0; column < 3; ++column) {
+        int best = column;
+        for (int row = column + 1; row < 3; ++row)
+            if (fabsf(a[row][column]) > fabsf(a[best][column])) best = row;
+        if (!isfinite(a[best][column]) || fabsf(a[best][column]) < 1.0e-12f) return false;
+        for (int k = column; k < 3; ++k) { const float held = a[column][k]; a[column][k] = a[best][k]; a[best][k] = held; }
+        { const float held = b[column]; b[column] = b[best]; b[best] = held; }
+        for (int row = column + 1; row < 3; ++row) {
+            const float ratio = a[row][column] / a[column][column];
+            for (int k = column + 1; k < 3; ++k) a[row][k] -= ratio * a[column][k];
+            b[row] -= ratio * b[column];
+        }
+    }
+    x[2] = b[2] / a[2][2];
+    x[1] = (b[1] - a[1][2] * x[2]) / a[1][1];
+    x[0] = (b[0] - a[0][1] * x[1] - a[0][2] * x[2]) / a[0][0];
+    return true;
+}
+__device__ FreeRotation solve_free_rotation(V3 w0, V3 inv_i, float dt) {
+    FreeRotation out{V3{0.0f, 0.0f, 0.0f}, 0.0f, 0u, kGyroConverged};
+    const float rate[3] = {w0.x, w0.y, w0.z}, inverse[3] = {inv_i.x, inv_i.y, inv_i.z};
+    float momentum[3];
+    bool usable = all_finite3(rate) && all_finite3(inverse);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { usable = usable && inverse[k] > 0.0f; momentum[k] = rate[k] / inverse[k]; }
+    if (!usable || !all_finite3(momentum)) { out.status = kGyroInvalidInput; out.residual = INFINITY; return out; }
+    const float size = largest3(momentum);
+    if (size == 0.0f) return out;   // nothing turns
+    const float to_unit = 1.0f / size;
+    const float a[3] = {inverse[0] * size, inverse[1] * size, inverse[2] * size};
+    MidpointRule rule;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { rule.start[k] = momentum[k] * to_unit; rule.coupling[k] = dt * (a[(k + 1) % 3] - a[(k + 2) % 3]); }
+    float u[3] = {rule.start[0], rule.start[1], rule.start[2]};
+    constexpr uint32_t kMostSteps = 12u, kMostHalvings = 8u;
+    for (uint32_t step = 0u; step <= kMostSteps; ++step) {
+        float g[3];
+        rule.residual(u, g);
+        out.residual = all_finite3(g) ? largest3(g) : INFINITY;
+        if (out.residual <= 1.0e-6f) {
+            out.midpoint = V3{a[0] * ((rule.start[0] + u[0]) * 0.5f), a[1] * ((rule.start[1] + u[1]) * 0.5f), a[2] * ((rule.start[2] + u[2]) * 0.5f)};
             return out;
         }
-        if (iteration == max_iterations || !isfinite(out.residual)) break;
-        const V3 mid = scale3(add3(u0, u), 0.5f);
-        float j[3][4] = {{1.0f, 0.5f * c.x * mid.z, 0.5f * c.x * mid.y, r.x},
-                         {0.5f * c.y * mid.z, 1.0f, 0.5f * c.y * mid.x, r.y},
-                         {0.5f * c.z * mid.y, 0.5f * c.z * mid.x, 1.0f, r.z}};
-        bool valid = true;
-        for (uint32_t column = 0u; column < 3u; ++column) {
-            uint32_t pivot = column;
-            for (uint32_t row = column + 1u; row < 3u; ++row)
-                if (fabsf(j[row][column]) > fabsf(j[pivot][column])) pivot = row;
-            if (!isfinite(j[pivot][column]) || fabsf(j[pivot][column]) < 1.0e-12f) { valid = false; break; }
-            for (uint32_t col = column; col < 4u; ++col) {
-                const float value = j[column][col];
-                j[column][col] = j[pivot][col];
-                j[pivot][col] = value;
-            }
-            for (uint32_t row = column + 1u; row < 3u; ++row) {
-                const float factor = j[row][column] / j[column][column];
-                for (uint32_t col = column + 1u; col < 4u; ++col) j[row][col] -= factor * j[column][col];
-            }
-        }
+        if (step == kMostSteps || !isfinite(out.residual)) break;
+        float j[3][3], change[3];
+        rule.jacobian(u, j);
         ++out.iterations;
-        if (!valid) break;
-        V3 delta;
-        delta.z = j[2][3] / j[2][2];
-        delta.y = (j[1][3] - j[1][2] * delta.z) / j[1][1];
-        delta.x = (j[0][3] - j[0][1] * delta.y - j[0][2] * delta.z) / j[0][0];
-        bool accepted = false;
-        float alpha = 1.0f;
-        for (uint32_t backtrack = 0u; backtrack < max_backtracks; ++backtrack) {
-            const V3 trial = sub3(u, scale3(delta, alpha));
-            const V3 trial_r = gyro_residual(u0, c, trial);
-            if (finite3(trial_r) && max_abs(trial_r) < out.residual) { u = trial; accepted = true; break; }
-            alpha *= 0.5f;
+        if (!solve3(j, g, change)) break;
+        bool fell = false;
+        float length = 1.0f;
+        for (uint32_t halving = 0u; halving < kMostHalvings && !fell; ++halving, length *= 0.5f) {
+            const float trial[3] = {u[0] - change[0] * length, u[1] - change[1] * length, u[2] - change[2] * length};
+            float at_trial[3];
+            rule.residual(trial, at_trial);
+            if (all_finite3(at_trial) && largest3(at_trial) < out.residual) { u[0] = trial[0]; u[1] = trial[1]; u[2] = trial[2]; fell = true; }
         }
-        if (!accepted) break;
+        if (!fell) break;
     }
-    out.status = 1u;   // kBodyGyroNotConverged
+    out.status = kGyroNotConverged;
     return out;
 }
 
@@ -224,7 +243,7 @@ __global__ void __launch_bounds__(256) BodyIntegratePositionKernel(ModelView m, 
     const Q4 principal = qnormalize_le(qmul(pose.r, frame.r), 1.0e-12f);
     const Q4 inverse{principal.w, -principal.x, -principal.y, -principal.z};
     const V3 w0 = rotate_normalized(inverse, V3{ang[0], ang[1], ang[2]});
-    const GyroResult gyro = solve_free_rotation(w0, inv_i, p.dt);
+    const FreeRotation gyro = solve_free_rotation(w0, inv_i, p.dt);
     d.body_gyro_residual[body] = gyro.residual; d.body_gyro_iterations[body] = gyro.iterations; d.body_gyro_status[body] = gyro.status;
     if (gyro.status != 0u) { atomicOr(d.env_status + env, uint32_t(kEnvStatusGyroFailure)); return; }
     const V3 momentum = rotate_normalized(principal, V3{w0.x / inv_i.x, w0.y / inv_i.y, w0.z / inv_i.z});

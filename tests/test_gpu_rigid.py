@@ -55,6 +55,8 @@ def test_free_flight_matches_the_oracle_over_many_steps(oracle_py, device):
         for name in ("base_pose", "body_linear_velocity", "body_angular_velocity", "body_pose"):
             close_env(world, oracle, name, E, tol=TOL if steps == 1 else 5 * TOL)
     assert np.array_equal(world.download("body_gyro_status"), oracle.download("body_gyro_status"))
+    iterations = oracle.download("body_gyro_iterations")
+    assert iterations.max() >= 1 and np.array_equal(world.download("body_gyro_iterations"), iterations)   # the Newton steps of the free-rotation solve
     assert not world.download("env_status").any()
     world.close(); oracle.close()
 
