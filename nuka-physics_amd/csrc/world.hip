@@ -399,9 +399,9 @@ struct Field { const char* name; Dtype dtype; uint32_t elem_bytes; size_t count;
     X(contact_link, kU32, E * S) \
     X(step_env_status, kU32, E) X(step_link_impulse, kF32, E * nl * 3) X(step_link_moment, kF32, E * nl * 3) \
     X(step_joint_limit_impulse, kF32, E * nl * 2) \
-    X(body_linear_velocity, kF32, E * nb * 3) X(body_angular_velocity, kF32, E * nb * 3) X(body_world_inv_inertia, kF32, E * nb * 6) \
-    X(body_gyro_residual, kF32, E * nb) X(body_gyro_iterations, kU32, E * nb) X(body_gyro_status, kU32, E * nb) \
-    X(body_inv_mass, kF32, E * nb) X(body_inv_inertia, kF32, E * nb * 3) X(body_inertial_frame, kF32, E * nb * 7)
+    X(body_linear_velocity, kF32, E * fb * 3) X(body_angular_velocity, kF32, E * fb * 3) X(body_world_inv_inertia, kF32, E * fb * 6) \
+    X(body_gyro_residual, kF32, E * fb) X(body_gyro_iterations, kU32, E * fb) X(body_gyro_status, kU32, E * fb) \
+    X(body_inv_mass, kF32, E * fb) X(body_inv_inertia, kF32, E * fb * 3) X(body_inertial_frame, kF32, E * fb * 7)
 
 #define NKH_MODEL_FIELDS(X) \
     X(joint_type, kU8) X(parent_link, kU32) X(joint_axis, kF32) X(parent_offset, kF32) X(link_local_pose, kF32) \
@@ -902,6 +902,7 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
         const ModelView& hc = w.host.counts;
         const size_t E = w.env_count, nl = hc.links_per_env, nb = hc.bodies_per_env, md = hc.max_dof, S = hc.contact_slots, R = hc.rows_per_env;
         const size_t mf = SolverMassFactorFloats(hc);
+        const size_t fb = hc.free_body != 0u ? nb : 0u;   // the rigid-body fields have their rows in a world of free bodies only
         if (E * std::max<size_t>(R, 1u) > 0xFFFFFFFFull / 2u || E * nl * 7u > 0xFFFFFFFFull) throw std::invalid_argument("world too large for 32-bit row indices");
         if (hc.rows_per_env > 0u && SolverHeadCapacity(hc, std::max(hc.contact_slots, 1u), 150u * 1024u) == 0u) throw std::invalid_argument("solver tile does not fit LDS");
         // arena layout: template tables first, then the env-major fields, each on a 256-byte boundary (buffer.hpp:39)
@@ -947,9 +948,9 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
             };
             // the bodies' inertial parameters (fields.yaml:17, 108, 568): a free body's in its own row - 1 / mass, 1 / principal
             // moments, the inertial frame - and zero mass (a body the rigid-body ops leave alone) in every other row
-            std::vector<float> inv_mass(E * nb, 0.0f), inv_inertia(E * nb * 3u, 0.0f), inertial_frame(E * nb * 7u, 0.0f);
+            std::vector<float> inv_mass(E * fb, 0.0f), inv_inertia(E * fb * 3u, 0.0f), inertial_frame(E * fb * 7u, 0.0f);
             for (size_t e = 0u; e < E; ++e)
-                for (size_t b = 0u; b < nb; ++b) {
+                for (size_t b = 0u; b < fb; ++b) {
                     inertial_frame[(e * nb + b) * 7u + 3u] = 1.0f;
                     if (hc.free_body == 0u || b != w.host.link_body[0]) continue;
                     inv_mass[e * nb + b] = 1.0f / w.host.link_mass[0];
@@ -1383,7 +1384,7 @@ const std::vector<ViewField>& ViewFields() {
             out.push_back({#field, ReferenceName(#field), 0u, uint8_t(dtype), per, scalars, offsetof(ModelView, field)}); }
         NKH_MODEL_FIELDS(X)
 #undef X
-        const size_t E = 2u, nl = 101u, nb = 103u, md = 107u, S = 109u, R = 113u, mf = 127u;
+        const size_t E = 2u, nl = 101u, nb = 103u, md = 107u, S = 109u, R = 113u, mf = 127u, fb = nb;
 #define X(field, dtype, count) { uint8_t per = 0u; uint32_t scalars = 0u; DataShape(size_t(count), &per, &scalars); \
             out.push_back({#field, ReferenceName(#field), 1u, uint8_t(dtype), per, scalars, offsetof(DataView, field)}); }
         NKH_DATA_FIELDS(X)
