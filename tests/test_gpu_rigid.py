@@ -196,3 +196,34 @@ def test_checkpoint_reset_and_large_batches_of_free_bodies(oracle_py, device):
     small.reset(); small.synchronize()
     assert not small.download("body_linear_velocity").any() and not small.download("body_angular_velocity").any()
     small.close(); big.close()
+
+
+def test_the_box_is_as_close_to_the_double_precision_answer_as_the_oracle(oracle_py, device):
+    """One step of boxes meeting the plane on the device, in the single-precision oracle and in the oracle built in double:
+    the device's velocities and poses lie within 1e-4 of the double-precision answer, or no further from it than twice
+    the single-precision oracle does (median, 95th percentile and largest over the batch)."""
+    E = 256
+    t = box_template(half=(0.2, 0.15, 0.1), mass=3.0, diag=(0.03, 0.04, 0.05), com=(0.03, 0.01, -0.02), mu=0.6)
+    desc = abi.world_desc(E, 1.0 / 240.0, vel_iters=8, pos_iters=4, contact_margin=0.02)
+    world, single, double = nk.World(device, t, desc), oracle_py.OracleWorld(t, desc, threads=8), oracle_py.OracleWorld(t, desc, threads=8, double=True)
+    pose, v, w = seeded_boxes(E, 31)
+    put(world, single, t, pose, v, w)
+    double.upload("base_pose", pose); double.upload("body_linear_velocity", body_field(t, v)); double.upload("body_angular_velocity", body_field(t, w))
+    world.step(); world.synchronize(); single.step(); double.step()
+    assert (single.download("contact_count") > 0).mean() >= 0.5
+
+    def coordinates(side):
+        return np.concatenate([of_body(t, side.download("body_linear_velocity"), E), of_body(t, side.download("body_angular_velocity"), E)], axis=1).astype(np.float64)
+
+    exact = coordinates(double)
+    scale = np.maximum(np.abs(exact).max(1), 0.05)
+    for name, field in (("velocity", coordinates), ("pose", lambda side: side.download("base_pose").reshape(E, 7).astype(np.float64))):
+        reference = field(double)
+        size = scale if name == "velocity" else np.maximum(np.abs(reference).max(1), 1e-3)
+        dev = np.abs(field(world) - reference).max(1) / size
+        ora = np.abs(field(single) - reference).max(1) / size
+        for what, measure in (("median", np.median), ("95th percentile", lambda x: np.percentile(x, 95)), ("largest", np.max)):
+            d, o = float(measure(dev)), float(measure(ora))
+            assert d <= max(TOL, 2.0 * o), f"{name} {what}: device {d:.2e} from the double-precision answer, oracle {o:.2e}"
+        print(f"{name}: device {dev.max():.1e} (median {np.median(dev):.1e}), oracle {ora.max():.1e} (median {np.median(ora):.1e})")
+    world.close(); single.close(); double.close()
