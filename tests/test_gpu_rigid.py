@@ -227,3 +227,37 @@ def test_the_box_is_as_close_to_the_double_precision_answer_as_the_oracle(oracle
             assert d <= max(TOL, 2.0 * o), f"{name} {what}: device {d:.2e} from the double-precision answer, oracle {o:.2e}"
         print(f"{name}: device {dev.max():.1e} (median {np.median(dev):.1e}), oracle {ora.max():.1e} (median {np.median(ora):.1e})")
     world.close(); single.close(); double.close()
+
+
+def test_a_scene_files_lone_free_body_is_a_free_rigid_body(oracle_py, device):
+    """A body on a free joint that no joint hangs a child on is no articulation in the reference
+    (articulation_cooker.cpp:148-151): loaded with the native laws the scene's template says free_body, and the world
+    steps it with the rigid-body ops as the oracle does on the same template.  Under MuJoCo-sourced profiles it stays a
+    one-link articulation."""
+    import os
+    from conftest import ROOT
+    path = os.path.join(ROOT, "tests", "data", "free_box.xml")
+    assert nk.Scene(path).to_c()[0].free_body == 0                      # MuJoCo laws by default
+    scene = nk.Scene(path, nk.SCENE_NATIVE_CONTACT_LAW | nk.SCENE_NATIVE_JOINT_LAW)
+    tdesc = scene.to_c()[0]
+    assert tdesc.free_body == 1 and tdesc.link_count == 1 and tdesc.drive_rows == 0
+    E = 64
+    desc = abi.world_desc(E, scene.info.timestep, gravity=tuple(scene.info.gravity), vel_iters=8, pos_iters=4)
+    world, oracle = nk.World(device, scene, desc), oracle_py.OracleWorld(scene, desc, threads=8)
+    oracle.upload("base_pose", world.download("base_pose"))          # the pose the file authors, in every environment
+    nb = tdesc.body_count
+    g = np.random.default_rng(4)
+    spin = np.zeros((E, nb, 3), np.float32)
+    own = int(np.argmax(np.ctypeslib.as_array(tdesc.body_role, shape=(nb,)) == abi.ROLE_LINK_BODY))
+    spin[:, own] = g.normal(0.0, 0.5, (E, 3))
+    for side in (world, oracle):
+        side.upload("body_angular_velocity", spin)
+    world.set_execution_mode(True)
+    for steps in (1, 59):
+        world.step(steps); world.synchronize()
+        oracle.step(steps)
+        assert np.array_equal(world.download("env_status"), oracle.download("env_status")) and not oracle.download("env_status").any()
+        assert np.array_equal(world.download("contact_count"), oracle.download("contact_count"))
+        close_env(world, oracle, "base_pose", E, tol=TOL if steps == 1 else 20 * TOL)
+    assert (oracle.download("contact_count") >= 3).mean() >= 0.8     # the crates lie on the floor
+    world.close(); oracle.close()
