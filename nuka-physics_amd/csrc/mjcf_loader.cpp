@@ -788,14 +788,12 @@ void Scene::Bind() {
     desc.integrator = integrator;
     // A lone body on a free joint is no articulation in the reference: CookArticulations passes over a root that no joint
     // hangs a child on (src/runtime/articulation/articulation_cooker.cpp:148-151), and the body stays a free rigid body of
-    // the rigid-body ops.  So it is here, where the scene keeps the native laws; under MuJoCo-sourced profiles the
-    // compliant rows' reference weights exist for articulations only, and the body is stepped as a one-link articulation.
-    bool native = integrator == 0u;
-    for (uint32_t law : profile_law) native = native && law == 0u;
-    for (uint8_t law : joint_law) native = native && law == 0u;
-    if (desc.link_count == 1u && floating_root && native) {
+    // the rigid-body ops.  It has no joint for a joint law or the joints' integrator to act on.
+    if (desc.link_count == 1u && floating_root) {
         desc.free_body = 1u;
         desc.drive_rows = 0u;
+        desc.integrator = 0u;
+        desc.joint_law = nullptr;
     }
 }
 

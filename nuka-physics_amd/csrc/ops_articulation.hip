@@ -795,9 +795,24 @@ __global__ void __launch_bounds__(kWave) ReferenceWeightsKernel(ModelView m, Dat
 // ReferenceWeights (op_schema.hpp:123-130; articulation.cu:425-500): the mass matrix at the current poses without
 // drive damping, its factor, and the reference weights from it.  World creation and reset dispatch it after the poses
 // are refreshed (nk/pipeline/world.cpp:553-561).
+// BodyReferenceWeightsKernel (articulation.cu:425-432): a free body's weights are its inverse mass and the mean of its
+// inverse principal moments; rows without mass weigh nothing
+__global__ void __launch_bounds__(256) BodyReferenceWeightsKernel(DataView d, uint32_t count) {
+    const uint32_t body = blockIdx.x * 256u + threadIdx.x;
+    if (body >= count) return;
+    const float* inverse = d.body_inv_inertia + size_t{body} * 3u;
+    d.body_invweight0[2u * body] = d.body_inv_mass[body];
+    d.body_invweight0[2u * body + 1u] = (inverse[0] + inverse[1] + inverse[2]) / 3.0f;
+}
+
 Status OpReferenceWeights(const ModelView& m, const DataView& d, const void* params, hipStream_t stream) {
     const auto* p = static_cast<const ReferenceWeightsParams*>(params);
     if (p == nullptr) return Status::Failed;
+    if (m.free_body != 0u) {
+        if (p->total_body_count == 0u) return Status::Ok;
+        hipLaunchKernelGGL(BodyReferenceWeightsKernel, dim3((p->total_body_count + 255u) / 256u), dim3(256), 0, stream, d, p->total_body_count);
+        return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
+    }
     if (p->articulation_count == 0u || p->total_link_count == 0u) return Status::Ok;
     if (p->articulations_per_env != 1u || p->max_dof != m.max_dof || p->bodies_per_env != m.bodies_per_env ||
         p->total_link_count != p->articulation_count * m.links_per_env) return Status::InvalidArgument;

@@ -1753,7 +1753,10 @@ __global__ void __launch_bounds__(256) SnapshotStepVelocityKernel(ModelView m, D
     if (gid >= env_count * m.max_dof) return;
     const uint32_t env = gid / m.max_dof, dof = gid - env * m.max_dof;
     float value = 0.0f;
-    if (dof < m.dof) {
+    if (dof < m.dof && m.free_body != 0u) {   // a free body's six coordinates as its state holds them: linear, then angular velocity
+        const size_t body = size_t{env} * m.bodies_per_env + m.link_body[0];
+        value = dof < 3u ? d.body_linear_velocity[body * 3u + dof] : d.body_angular_velocity[body * 3u + dof - 3u];
+    } else if (dof < m.dof) {
         const uint32_t link = m.dof_link[dof], component = m.dof_component[dof];
         value = component == kInvalid ? d.qdot[size_t{env} * m.links_per_env + link]
                                       : d.link_velocity[(size_t{env} * m.links_per_env + link) * 6u + component];

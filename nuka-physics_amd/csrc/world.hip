@@ -333,7 +333,6 @@ void Cook(const nuka_template_desc_t& d, HostModel* out) {
         if (nl != 1u || c.floating_root == 0u) throw std::invalid_argument("a free body is a template of one link with a floating root");
         if (c.joint_limit_rows + c.joint_friction_rows + c.joint_drive_rows != 0u || c.integrator != 0u)
             throw std::invalid_argument("a free body has no joint rows, drives or joint integrator");
-        if (c.any_mujoco != 0u) throw NotSupported("a free body takes the native contact law on this path");
         if (m.link_body[0] == kInvalid) throw std::invalid_argument("a free body needs its own body row: its state lives there");
         if (!(d.link_mass[0] > 0.0f) || !std::isfinite(d.link_mass[0])) throw std::invalid_argument("a free body needs a positive mass");
         for (uint32_t k = 0u; k < 3u; ++k)

@@ -757,6 +757,14 @@ void nko_env_reference_weights(nko_world* w, uint32_t env) {
     const uint32_t nl = t->nl, nb = t->nb, md = t->max_dof, dof = t->nv;
     float* weights = w->body_invweight0 + (size_t)env * nb * 2u;
     for (uint32_t b = 0u; b < nb; ++b) weights[2u * b] = weights[2u * b + 1u] = 0.0f;   /* static rows: inverse mass zero */
+    if (t->free_body) {   /* BodyReferenceWeightsKernel (articulation.cu:425-432): the inverse mass, the mean inverse principal moment */
+        const uint32_t body = t->link_body[0];
+        const float* d = t->body_diag_inertia;
+        const float inverse[3] = {d[0] > 0.0f ? 1.0f / d[0] : 0.0f, d[1] > 0.0f ? 1.0f / d[1] : 0.0f, d[2] > 0.0f ? 1.0f / d[2] : 0.0f};
+        weights[2u * body] = t->body_mass > 0.0f ? 1.0f / t->body_mass : 0.0f;
+        weights[2u * body + 1u] = (inverse[0] + inverse[1] + inverse[2]) / 3.0f;
+        return;
+    }
     if (dof == 0u) return;
     nko_env_dynamics(w, env, 0u);   /* m, m_factor at the current pose; the caller has switched the damping fold off */
     const float* factor = w->m_factor + (size_t)env * md * md;

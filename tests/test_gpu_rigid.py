@@ -229,29 +229,40 @@ def test_the_box_is_as_close_to_the_double_precision_answer_as_the_oracle(oracle
     world.close(); single.close(); double.close()
 
 
-def test_a_scene_files_lone_free_body_is_a_free_rigid_body(oracle_py, device):
+@pytest.mark.parametrize("flags,cone", [("native", None), ("mujoco", "pyramidal"), ("mujoco", "elliptic")])
+def test_a_scene_files_lone_free_body_is_a_free_rigid_body(oracle_py, device, flags, cone, tmp_path):
     """A body on a free joint that no joint hangs a child on is no articulation in the reference
-    (articulation_cooker.cpp:148-151): loaded with the native laws the scene's template says free_body, and the world
-    steps it with the rigid-body ops as the oracle does on the same template.  Under MuJoCo-sourced profiles it stays a
-    one-link articulation."""
+    (articulation_cooker.cpp:148-151): the scene's template says free_body, and the world steps it with the rigid-body
+    ops as the oracle does on the same template - under the native laws and under the file's own MuJoCo contact law
+    (compliant rows weighted by BodyReferenceWeightsKernel's inverse mass; both cones)."""
     import os
     from conftest import ROOT
     path = os.path.join(ROOT, "tests", "data", "free_box.xml")
-    assert nk.Scene(path).to_c()[0].free_body == 0                      # MuJoCo laws by default
-    scene = nk.Scene(path, nk.SCENE_NATIVE_CONTACT_LAW | nk.SCENE_NATIVE_JOINT_LAW)
+    if cone == "elliptic":
+        text = open(path).read().replace('<option timestep="0.004"', '<option cone="elliptic" timestep="0.004"')
+        path = str(tmp_path / "free_box_elliptic.xml")
+        open(path, "w").write(text)
+    scene = nk.Scene(path, nk.SCENE_NATIVE_CONTACT_LAW | nk.SCENE_NATIVE_JOINT_LAW if flags == "native" else 0)
     tdesc = scene.to_c()[0]
-    assert tdesc.free_body == 1 and tdesc.link_count == 1 and tdesc.drive_rows == 0
+    assert tdesc.free_body == 1 and tdesc.link_count == 1 and tdesc.drive_rows == 0 and tdesc.integrator == 0
+    assert (scene.template_arrays()["profile_law"] == (0 if flags == "native" else 1)).all()
     E = 64
     desc = abi.world_desc(E, scene.info.timestep, gravity=tuple(scene.info.gravity), vel_iters=8, pos_iters=4)
     world, oracle = nk.World(device, scene, desc), oracle_py.OracleWorld(scene, desc, threads=8)
     oracle.upload("base_pose", world.download("base_pose"))          # the pose the file authors, in every environment
     nb = tdesc.body_count
-    g = np.random.default_rng(4)
-    spin = np.zeros((E, nb, 3), np.float32)
     own = int(np.argmax(np.ctypeslib.as_array(tdesc.body_role, shape=(nb,)) == abi.ROLE_LINK_BODY))
+    if flags == "mujoco":
+        weights = world.download("body_invweight0").reshape(E, nb, 2)
+        assert np.allclose(weights[:, own], [1.0 / 2.5, (1 / 0.03 + 1 / 0.045 + 1 / 0.05) / 3.0], rtol=1e-6) and not np.delete(weights, own, axis=1).any()
+        assert np.array_equal(weights, oracle.download("body_invweight0").reshape(E, nb, 2))
+    g = np.random.default_rng(4)
+    spin, push = np.zeros((E, nb, 3), np.float32), np.zeros((E, nb, 3), np.float32)
     spin[:, own] = g.normal(0.0, 0.5, (E, 3))
+    push[:, own] = g.normal(0.0, 0.3, (E, 3))
     for side in (world, oracle):
         side.upload("body_angular_velocity", spin)
+        side.upload("body_linear_velocity", push)
     world.set_execution_mode(True)
     for steps in (1, 59):
         world.step(steps); world.synchronize()

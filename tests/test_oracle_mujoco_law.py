@@ -304,20 +304,25 @@ def resting_sphere(cone, solref, solimp):
     return t
 
 
+@pytest.mark.parametrize("free_body", [False, True])
 @pytest.mark.parametrize("cone", [abi.CONE_ELLIPTIC, abi.CONE_PYRAMIDAL])
-def test_a_resting_sphere_sinks_to_the_depth_of_the_spring_reference(oracle_py, cone):
+def test_a_resting_sphere_sinks_to_the_depth_of_the_spring_reference(oracle_py, cone, free_body):
     """At rest the contact force is the weight and the row equation a + R f = aref holds with a = 0: f = aref / R with
     aref = k imp depth and R = invweight (1 - imp) / imp (constraint/solref_solimp.hpp:55-86), which fixes the depth.
-    A pyramid's four edges share the load and each is softer, with the edge weight of assemble_rows.cu:652."""
+    A pyramid's four edges share the load and each is softer, with the edge weight of assemble_rows.cu:652.  The ball as
+    a one-link articulation and as a free rigid body (the rigid-body ops, BodyReferenceWeightsKernel's inverse mass)."""
     L = oracle_py.lib()
     solref, solimp, dt, mass, g = (0.02, 1.0), (0.9, 0.95, 0.001, 0.5, 2.0), 0.002, 3.0, 9.81
     t = resting_sphere(cone, solref, solimp)
+    t.free_body = free_body
     w = oracle_py.OracleWorld(t, abi.world_desc(1, dt, vel_iters=16, velocity_tolerance=1e-7))
     w.upload("base_pose", np.array([0, 0, 0.0999, 1, 0, 0, 0], np.float32))
     w.step(1500)
     assert w.download("env_status")[0] == 0
     height = w.download("base_pose")[2]
-    assert abs(w.download("link_velocity")[5]) < 1e-4
+    assert abs(w.download("body_linear_velocity").reshape(2, 3)[1, 2] if free_body else w.download("link_velocity")[5]) < 1e-4
+    if free_body:
+        assert np.allclose(w.download("body_invweight0").reshape(2, 2)[1], [1.0 / mass, 1.0 / 0.02], rtol=1e-6)
     depth = 0.1 - height
     mu = 0.9
     invweight = 1.0 / mass
