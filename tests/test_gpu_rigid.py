@@ -193,6 +193,16 @@ def test_checkpoint_reset_and_large_batches_of_free_bodies(oracle_py, device):
     for name, value in after.items():
         batch = big.download(name).reshape(copies, -1)
         assert np.array_equal(np.broadcast_to(value.reshape(1, -1), batch.shape), batch), name
+    # a masked reset returns the chosen environments' bodies to the state of creation and leaves the others alone
+    before = {name: small.download(name).reshape(E, -1) for name in ("base_pose", "body_linear_velocity", "body_angular_velocity")}
+    chosen = np.array([3, 17, 40], np.uint32)
+    small.reset_envs(chosen); small.synchronize()
+    others = np.setdiff1d(np.arange(E), chosen)
+    for name, value in before.items():
+        now = small.download(name).reshape(E, -1)
+        assert np.array_equal(now[others], value[others]), name
+        expect = np.array([0, 0, 0, 1, 0, 0, 0], np.float32) if name == "base_pose" else 0.0
+        assert np.array_equal(now[chosen], np.broadcast_to(expect, now[chosen].shape)), name
     small.reset(); small.synchronize()
     assert not small.download("body_linear_velocity").any() and not small.download("body_angular_velocity").any()
     small.close(); big.close()
