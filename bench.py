@@ -83,7 +83,16 @@ def scene_run(nk, args):
     nl = scene.link_count
     twist = np.zeros((E, nl, 6), np.float32)
     twist[:, 0] = np.random.default_rng(11).normal(0, 0.3, (E, 6))
-    world.upload("link_velocity", twist)
+    template = scene.to_c()[0]
+    if template.free_body:          # a lone free body's state is its own row of the per-body velocity fields
+        nb = template.body_count
+        own = int(np.argmax(np.ctypeslib.as_array(template.body_role, shape=(nb,)) == nk.abi.ROLE_LINK_BODY))
+        for name, part in (("body_linear_velocity", twist[:, 0, 3:]), ("body_angular_velocity", twist[:, 0, :3])):
+            values = np.zeros((E, nb, 3), np.float32)
+            values[:, own] = part
+            world.upload(name, values)
+    else:
+        world.upload("link_velocity", twist)
     if args.base_height > 0.0:
         base = world.download("base_pose").reshape(E, 7).copy()
         base[:, 2] = args.base_height
