@@ -59,80 +59,90 @@ void nko_body_center_of_mass(const nko_world* w, uint32_t env, float out[3]) {
     out[0] = c.x; out[1] = c.y; out[2] = c.z;
 }
 
-static float max_abs(v3 v) { return fmaxf(fabsf(v.x), fmaxf(fabsf(v.y), fabsf(v.z))); }
-static int finite_vector(v3 v) { return isfinite(v.x) && isfinite(v.y) && isfinite(v.z); }
-
-/* rigid_types.cuh:38-121 SolveFreeRotation: the implicit midpoint rule of Euler's equations in the principal frame,
- * on the angular momentum scaled to unit size, by Newton steps with halving; `midpoint` is the angular velocity at the
- * middle of the step */
+/* The free-rotation step (rigid_types.cuh:38-121 SolveFreeRotation): Euler's equations in the principal frame by the
+ * implicit midpoint rule, m1 - m0 = dt (m_mid x w_mid), solved for the end-of-step angular momentum.  The unknown is the
+ * momentum scaled to unit size, g(u) = u - u0 + c o (mid_y mid_z, mid_z mid_x, mid_x mid_y) with mid = (u0 + u) / 2 and
+ * c = dt (a_y - a_z, a_z - a_x, a_x - a_y), a = scaled inverse moments; Newton steps on g, each halved while the residual
+ * does not fall, at most twelve, to a residual of 1e-6.  `midpoint` is the angular velocity at the middle of the step. */
 typedef struct { v3 midpoint; float residual; uint32_t iterations, status; } gyro_result;
-static v3 gyro_residual(v3 u0, v3 c, v3 u) {
-    const v3 mid = v3_scale(v3_add(u0, u), 0.5f);
-    return v3_make(u.x - u0.x + c.x * mid.y * mid.z, u.y - u0.y + c.y * mid.z * mid.x, u.z - u0.z + c.z * mid.x * mid.y);
+enum { GYRO_CONVERGED = 0, GYRO_NOT_CONVERGED = 1, GYRO_INVALID_INPUT = 2 };   /* op_schema.hpp:53-54 */
+typedef struct { float start[3], coupling[3]; } midpoint_rule;
+
+static void rule_residual(const midpoint_rule* r, const float u[3], float g[3]) {
+    const float mid[3] = {(r->start[0] + u[0]) * 0.5f, (r->start[1] + u[1]) * 0.5f, (r->start[2] + u[2]) * 0.5f};
+    for (int k = 0; k < 3; ++k) g[k] = u[k] - r->start[k] + r->coupling[k] * mid[(k + 1) % 3] * mid[(k + 2) % 3];
+}
+/* dg/du: the identity and half the coupling times the other two midpoint components */
+static void rule_jacobian(const midpoint_rule* r, const float u[3], float j[3][3]) {
+    const float mid[3] = {(r->start[0] + u[0]) * 0.5f, (r->start[1] + u[1]) * 0.5f, (r->start[2] + u[2]) * 0.5f};
+    for (int k = 0; k < 3; ++k) {
+        j[k][k] = 1.0f;
+        j[k][(k + 1) % 3] = 0.5f * r->coupling[k] * mid[(k + 2) % 3];
+        j[k][(k + 2) % 3] = 0.5f * r->coupling[k] * mid[(k + 1) % 3];
+    }
+}
+static float largest3(const float v[3]) { return fmaxf(fabsf(v[0]), fmaxf(fabsf(v[1]), fabsf(v[2]))); }
+static int all_finite3(const float v[3]) { return isfinite(v[0]) && isfinite(v[1]) && isfinite(v[2]); }
+/* x of a x = b by elimination with row pivoting, columns left to right; 0 when a pivot is below 1e-12 or not finite */
+static int solve3(float a[3][3], float b[3], float x[3]) {
+    for (int column = 0; column < 3; ++column) {
+        int best = column;
+        for (int row = column + 1; row < 3; ++row)
+            if (fabsf(a[row][column]) > fabsf(a[best][column])) best = row;
+        if (!isfinite(a[best][column]) || fabsf(a[best][column]) < 1.0e-12f) return 0;
+        for (int k = column; k < 3; ++k) { const float held = a[column][k]; a[column][k] = a[best][k]; a[best][k] = held; }
+        { const float held = b[column]; b[column] = b[best]; b[best] = held; }
+        for (int row = column + 1; row < 3; ++row) {
+            const float ratio = a[row][column] / a[column][column];
+            for (int k = column + 1; k < 3; ++k) a[row][k] -= ratio * a[column][k];
+            b[row] -= ratio * b[column];
+        }
+    }
+    x[2] = b[2] / a[2][2];
+    x[1] = (b[1] - a[1][2] * x[2]) / a[1][1];
+    x[0] = (b[0] - a[0][1] * x[1] - a[0][2] * x[2]) / a[0][0];
+    return 1;
 }
 static gyro_result solve_free_rotation(v3 w0, v3 inv_i, float dt) {
     gyro_result out;
     memset(&out, 0, sizeof(out));
-    if (!finite_vector(w0) || !finite_vector(inv_i) || inv_i.x <= 0.0f || inv_i.y <= 0.0f || inv_i.z <= 0.0f) {
-        out.status = 2u; out.residual = INFINITY;   /* kBodyGyroInvalidInput */
-        return out;
-    }
-    const v3 m0 = v3_make(w0.x / inv_i.x, w0.y / inv_i.y, w0.z / inv_i.z);
-    const float scale = max_abs(m0);
-    if (!finite_vector(m0)) { out.status = 2u; out.residual = INFINITY; return out; }
-    if (scale == 0.0f) return out;
-    const v3 u0 = v3_scale(m0, 1.0f / scale);
-    const v3 a = v3_scale(inv_i, scale);
-    const v3 c = v3_make(dt * (a.y - a.z), dt * (a.z - a.x), dt * (a.x - a.y));
-    const float tolerance = 1.0e-6f;
-    const uint32_t max_iterations = 12u, max_backtracks = 8u;
-    v3 u = u0;
-    for (uint32_t iteration = 0u; iteration <= max_iterations; ++iteration) {
-        const v3 r = gyro_residual(u0, c, u);
-        out.residual = finite_vector(r) ? max_abs(r) : INFINITY;
-        if (out.residual <= tolerance) {
-            const v3 mid = v3_scale(v3_add(u0, u), 0.5f);
-            out.midpoint = v3_make(a.x * mid.x, a.y * mid.y, a.z * mid.z);
+    const float rate[3] = {w0.x, w0.y, w0.z}, inverse[3] = {inv_i.x, inv_i.y, inv_i.z};
+    float momentum[3];
+    int usable = all_finite3(rate) && all_finite3(inverse);
+    for (int k = 0; k < 3; ++k) { usable = usable && inverse[k] > 0.0f; momentum[k] = rate[k] / inverse[k]; }
+    if (!usable || !all_finite3(momentum)) { out.status = GYRO_INVALID_INPUT; out.residual = INFINITY; return out; }
+    const float size = largest3(momentum);
+    if (size == 0.0f) return out;   /* nothing turns */
+    const float to_unit = 1.0f / size;
+    const float a[3] = {inverse[0] * size, inverse[1] * size, inverse[2] * size};
+    midpoint_rule rule;
+    for (int k = 0; k < 3; ++k) { rule.start[k] = momentum[k] * to_unit; rule.coupling[k] = dt * (a[(k + 1) % 3] - a[(k + 2) % 3]); }
+    float u[3] = {rule.start[0], rule.start[1], rule.start[2]};
+    const uint32_t most_steps = 12u, most_halvings = 8u;
+    for (uint32_t step = 0u; step <= most_steps; ++step) {
+        float g[3];
+        rule_residual(&rule, u, g);
+        out.residual = all_finite3(g) ? largest3(g) : INFINITY;
+        if (out.residual <= 1.0e-6f) {
+            out.midpoint = v3_make(a[0] * ((rule.start[0] + u[0]) * 0.5f), a[1] * ((rule.start[1] + u[1]) * 0.5f), a[2] * ((rule.start[2] + u[2]) * 0.5f));
             return out;
         }
-        if (iteration == max_iterations || !isfinite(out.residual)) break;
-        const v3 mid = v3_scale(v3_add(u0, u), 0.5f);
-        float j[3][4] = {{1.0f, 0.5f * c.x * mid.z, 0.5f * c.x * mid.y, r.x},
-                         {0.5f * c.y * mid.z, 1.0f, 0.5f * c.y * mid.x, r.y},
-                         {0.5f * c.z * mid.y, 0.5f * c.z * mid.x, 1.0f, r.z}};
-        int valid = 1;
-        for (uint32_t column = 0u; column < 3u; ++column) {
-            uint32_t pivot = column;
-            for (uint32_t row = column + 1u; row < 3u; ++row)
-                if (fabsf(j[row][column]) > fabsf(j[pivot][column])) pivot = row;
-            if (!isfinite(j[pivot][column]) || fabsf(j[pivot][column]) < 1.0e-12f) { valid = 0; break; }
-            for (uint32_t col = column; col < 4u; ++col) {
-                const float value = j[column][col];
-                j[column][col] = j[pivot][col];
-                j[pivot][col] = value;
-            }
-            for (uint32_t row = column + 1u; row < 3u; ++row) {
-                const float factor = j[row][column] / j[column][column];
-                for (uint32_t col = column + 1u; col < 4u; ++col) j[row][col] -= factor * j[column][col];
-            }
-        }
+        if (step == most_steps || !isfinite(out.residual)) break;
+        float j[3][3], change[3];
+        rule_jacobian(&rule, u, j);
         ++out.iterations;
-        if (!valid) break;
-        v3 delta;
-        delta.z = j[2][3] / j[2][2];
-        delta.y = (j[1][3] - j[1][2] * delta.z) / j[1][1];
-        delta.x = (j[0][3] - j[0][1] * delta.y - j[0][2] * delta.z) / j[0][0];
-        int accepted = 0;
-        float alpha = 1.0f;
-        for (uint32_t backtrack = 0u; backtrack < max_backtracks; ++backtrack) {
-            const v3 trial = v3_sub(u, v3_scale(delta, alpha));
-            const v3 trial_r = gyro_residual(u0, c, trial);
-            if (finite_vector(trial_r) && max_abs(trial_r) < out.residual) { u = trial; accepted = 1; break; }
-            alpha *= 0.5f;
+        if (!solve3(j, g, change)) break;
+        int fell = 0;
+        float length = 1.0f;
+        for (uint32_t halving = 0u; halving < most_halvings && !fell; ++halving, length *= 0.5f) {
+            const float trial[3] = {u[0] - change[0] * length, u[1] - change[1] * length, u[2] - change[2] * length};
+            float at_trial[3];
+            rule_residual(&rule, trial, at_trial);
+            if (all_finite3(at_trial) && largest3(at_trial) < out.residual) { u[0] = trial[0]; u[1] = trial[1]; u[2] = trial[2]; fell = 1; }
         }
-        if (!accepted) break;
+        if (!fell) break;
     }
-    out.status = 1u;   /* kBodyGyroNotConverged */
+    out.status = GYRO_NOT_CONVERGED;
     return out;
 }
 /* the free-rotation solve alone, for the tests: returns the status, writes the midpoint angular velocity (principal
