@@ -1,6 +1,6 @@
 """Headline benchmark: env-steps/s of the batched articulation step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 3] [--envs 4096] [--mode eager|graph] [--only]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1..6] [--envs 4096] [--mode eager|graph] [--only]
 
 One "step" is one pass of the whole pipeline (FK, dynamics, contacts, block-descent solve, integration, FK) over
 every environment of the batch, state resident in HBM.  Every timed step starts from the same seeded batch: the
@@ -216,7 +216,7 @@ def measure(nk, device, index, envs, steps, warmup, mode, cpu_budget_s, law="nat
     world.close()
     out = {
         "value": E * 1e3 / wall_ms, "ms_per_step": wall_ms, "steps": steps, "warmup": warmup,
-        "config": {"workload": f"{cfg.name}: {nl} links, {nv} DoF, {nc} contact spheres, {E} envs, dt {cfg.dt:.6f}, "
+        "config": {"workload": f"{cfg.name}: {nl} links, {nv} DoF, {nc} contact " + ("slots of up to four points" if index == 6 else "spheres") + f", {E} envs, dt {cfg.dt:.6f}, "
                                f"{cfg.vel_iters} block-descent sweeps{live}" + (f"; {cfg.note}" if cfg.note else "")
                                + ("" if law == "native" else f"; MuJoCo contact law, {law} cone"),
                    "config_index": index, "envs": E,

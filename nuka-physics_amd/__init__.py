@@ -309,6 +309,9 @@ class World:
         lv = np.zeros((E, nl, 6), np.float32)
         lv[:, 0, :] = state["root_twist"]
         self.upload("link_velocity", lv)
+        for name in ("body_linear_velocity", "body_angular_velocity"):   # a free body's state, per body row
+            if name in state:
+                self.upload(name, state[name])
 
     def op(self, name, variant=0):
         op = lib().nuka_hip_op_from_name(name.encode())

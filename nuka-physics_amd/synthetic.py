@@ -12,7 +12,7 @@ import math
 import numpy as np
 
 from .abi import (JOINT_FIXED, JOINT_FLOATING, JOINT_REVOLUTE, ROLE_LINK_BODY, ROLE_PROXY, ROLE_STATIC,
-                  SHAPE_NONE, SHAPE_PLANE, SHAPE_SPHERE, Template)
+                  SHAPE_BOX, SHAPE_NONE, SHAPE_PLANE, SHAPE_SPHERE, Template)
 
 SEED = 0xC0FFEE
 X, Y, Z = (1, 0, 0), (0, 1, 0), (0, 0, 1)
@@ -233,7 +233,37 @@ def rope(env_count=8192):
     return Config(5, "rope64", t, 1.0 / 500.0, 16, env_count, sample, np.zeros(nl, np.float32), False, note)
 
 
+def free_box(env_count=4096):
+    """Not one of the published configurations: a free rigid body, a box of 0.4 x 0.3 x 0.2 m with its centre of mass off
+    the middle, dropped a few millimetres onto the plane with a small tilt, push and spin (four-point manifolds)."""
+    t = Template()
+    t.free_body = True
+    t.add_link(JOINT_FLOATING, None, mass=3.0, diag_inertia=(0.03, 0.04, 0.05), com=(0.03, 0.01, -0.02))
+    profile = t.add_profile(0.6)
+    t.add_body(ROLE_STATIC, kind=SHAPE_PLANE, contype=2, conaffinity=1, profile=profile)
+    t.add_body(ROLE_LINK_BODY, link=0, kind=SHAPE_BOX, params=(0.2, 0.15, 0.1, 0.0), contype=1, conaffinity=2, profile=profile)
+    t.max_contacts_per_env = 1
+
+    def sample(E):
+        pose = np.zeros((E, 7), np.float32)
+        pose[:, :2] = _rng(6, 0).normal(0.0, 0.5, (E, 2))
+        pose[:, 2] = 0.1 + _rng(6, 1).uniform(-0.004, 0.01, E)
+        pose[:, 3] = 1.0
+        pose[:, 4:] = 0.5 * _rng(6, 2).normal(0.0, 0.03, (E, 3))
+        pose[:, 3:] /= np.linalg.norm(pose[:, 3:], axis=1, keepdims=True)
+        linear, angular = np.zeros((E, 2, 3), np.float32), np.zeros((E, 2, 3), np.float32)   # per body row: the plane's, the box's
+        linear[:, 1] = _rng(6, 3).normal(0.0, 0.3, (E, 3))
+        angular[:, 1] = _rng(6, 4).normal(0.0, 1.0, (E, 3))
+        zeros = np.zeros((E, 1), np.float32)
+        return dict(q=zeros, qdot=zeros.copy(), tau=zeros.copy(), base_pose=pose, root_twist=np.zeros((E, 6), np.float32),
+                    body_linear_velocity=linear, body_angular_velocity=angular)
+
+    return Config(6, "free_box", t, 1.0 / 240.0, 8, env_count, sample, np.zeros(1, np.float32), True,
+                  note="a free rigid body stepped by the rigid-body ops, outside the published configurations")
+
+
 def config(index, env_count=None):
-    """Benchmark configuration by number 1..5; 4 is the humanoid at a swept environment count."""
-    makers = {1: chain7, 2: quadruped, 3: humanoid, 4: lambda e=4096: humanoid(e, 4), 5: rope}
+    """Benchmark configuration by number 1..5; 4 is the humanoid at a swept environment count; 6 is a free rigid box,
+    outside the published table."""
+    makers = {1: chain7, 2: quadruped, 3: humanoid, 4: lambda e=4096: humanoid(e, 4), 5: rope, 6: free_box}
     return makers[index]() if env_count is None else makers[index](env_count)

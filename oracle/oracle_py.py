@@ -188,6 +188,9 @@ class OracleWorld:
         lv = self.field("link_velocity").reshape(E, nl, 6)
         lv[:] = 0.0
         lv[:, 0, :] = state["root_twist"]
+        for name in ("body_linear_velocity", "body_angular_velocity"):   # a free body's state, per body row
+            if name in state:
+                self.upload(name, state[name])
 
     def op(self, name, *args):
         getattr(self._lib, "nko_" + name)(self._h, *args)
