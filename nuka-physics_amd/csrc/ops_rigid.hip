@@ -4,10 +4,10 @@
 // by six block of the tile in it (block_descent_rigid.cuh:4-48, block_descent_tile.cuh:541-603) and
 // BodyIntegratePositionKernel with the free-rotation solve after it (articulation.cu:1058-1117, rigid_types.cuh:38-121).
 // Here the body is the template's one link: `base_pose` is its pose, `body_linear_velocity` / `body_angular_velocity`
-// (per body row, as in the reference: the link's own row holds them) its state, and the six coordinates - linear velocity, then angular velocity about the centre of mass, world axes -
-// pass through the link's twist words to the row assembly and the block descent, which take the block's mass matrix
-// and its factor from `m` / `m_factor` as for an articulation.  One thread an environment: the work is a few hundred
-// operations on a body.
+// (per body row, as in the reference: the link's own row holds them) its state, and the six coordinates - linear
+// velocity, then angular velocity about the centre of mass, world axes - pass through the link's twist words to the row
+// assembly and the block descent, which take the block's mass matrix and its factor from `m` / `m_factor` as for an
+// articulation.  One thread an environment: the work is a few hundred operations on a body.
 #include <cfloat>
 
 #include "nk_device_math.h"
@@ -177,7 +177,7 @@ __global__ void __launch_bounds__(256) BodyIntegrateVelocityKernel(ModelView m, 
         const float* inv_i = d.body_inv_inertia + body * 3u;
         body_world_inverse_inertia(pose, frame, V3{inv_i[0], inv_i[1], inv_i[2]}, world_inverse);
         const V3 g{p.gravity[0], p.gravity[1], p.gravity[2]};
-        v = add3(v, scale3(add3(scale3(g, 1.0f - 0.0f), scale3(force, inv_mass)), p.dt));
+        v = add3(v, scale3(add3(g, scale3(force, inv_mass)), p.dt));
         w = add3(w, scale3(sym_multiply(world_inverse, torque), p.dt));
     }
     for (uint32_t i = 0u; i < 6u; ++i) inverse[i] = world_inverse[i];

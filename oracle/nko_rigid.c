@@ -184,7 +184,7 @@ void nko_env_body_integrate_velocity(nko_world* w, uint32_t env) {
         const xform pose = xform_load(w->base_pose + (size_t)env * 7u), frame = xform_load(t->link_inertial_frame);
         body_world_inverse_inertia(pose, frame, inverse_inertia_of(t), inverse);
         const v3 g = v3_make(w->cfg.gravity[0], w->cfg.gravity[1], w->cfg.gravity[2]);
-        const v3 dv = v3_scale(v3_add(v3_scale(g, 1.0f - 0.0f), v3_scale(force, inv_mass)), dt);
+        const v3 dv = v3_scale(v3_add(g, v3_scale(force, inv_mass)), dt);
         lin[0] += dv.x; lin[1] += dv.y; lin[2] += dv.z;
         const v3 dw = v3_scale(sym_multiply(inverse, torque), dt);
         ang[0] += dw.x; ang[1] += dw.y; ang[2] += dw.z;
