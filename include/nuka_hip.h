@@ -460,6 +460,72 @@ nuka_result_t nuka_world_upload_field(nuka_world_handle world, nuka_state_field_
 nuka_result_t nuka_world_download_field(nuka_world_handle world, nuka_state_field_t field, void* bytes, size_t nbytes,
                                         size_t byte_offset);
 
+/* What a caller binds names, columns and its own stream to (nuka.h:34-40, 292-299, 478-494, 1222-1281, 1283-1301;
+ * src/c_abi/error.cpp:69-72, cuda_interop.cpp:20-58, world.cpp:759-768, 1170-1294, 1345-1413), under the reference's
+ * names, layouts and error behaviour. */
+typedef struct nuka_version_t {
+    uint16_t major;
+    uint16_t minor;
+    uint16_t patch;
+} nuka_version_t;
+nuka_version_t nuka_get_version(void);   /* the version of the C ABI this header follows: 0.1.0 */
+enum { NUKA_RUNTIME_INFO_VERSION = 1 };
+typedef struct nuka_runtime_info_t {
+    uint32_t struct_size;
+    uint32_t schema_version;
+    int32_t cuda_runtime_version;   /* here: hipRuntimeGetVersion */
+    int32_t cuda_driver_version;    /* here: hipDriverGetVersion */
+} nuka_runtime_info_t;
+/* struct_size and schema_version are set by the caller, else INVALID_ARG */
+nuka_result_t nuka_get_runtime_info(nuka_runtime_info_t* out);
+/* The stream the world executes on (a hipStream_t), and a caller's hipEvent_t recorded on it after all submitted work */
+nuka_result_t nuka_world_get_stream(nuka_world_handle world, void** out_stream);
+nuka_result_t nuka_world_record_event(nuka_world_handle world, void* cuda_event);
+typedef struct nuka_solver_options_t {
+    uint32_t cone;         /* constraint/solver_contract.hpp:8: 0 pyramidal, 1 elliptic */
+    uint32_t integrator;   /* :9: 0 Euler, 3 implicitfast (what the template's integrator 2 runs) */
+    float impratio;
+    uint32_t refsafe;
+} nuka_solver_options_t;
+nuka_result_t nuka_world_get_solver_options(nuka_world_handle world, nuka_solver_options_t* out);
+/* The name of the joint whose child is link `link_index` (any environment's copy: env-concatenated link order), else
+ * the link's own name.  `out` null is a size query; a `cap` too small for name + NUL is INVALID_ARG with *out_len still
+ * set; NOT_SUPPORTED for a world that was not created from a scene file. */
+nuka_result_t nuka_world_get_dof_name(nuka_world_handle world, uint32_t link_index, char* out, size_t cap, size_t* out_len);
+typedef enum nuka_kinematic_joint_t {
+    NUKA_KINEMATIC_ROOT = 0,
+    NUKA_KINEMATIC_FIXED = 1,
+    NUKA_KINEMATIC_REVOLUTE = 2,
+    NUKA_KINEMATIC_PRISMATIC = 3,
+    NUKA_KINEMATIC_SPHERICAL = 4    /* never reported: this path builds no ball joints */
+} nuka_kinematic_joint_t;
+typedef struct nuka_kinematic_link_t {
+    uint32_t parent_index;          /* UINT32_MAX for a root */
+    uint32_t articulation_index;
+    nuka_kinematic_joint_t joint_type;
+    float local_pose[7];            /* parent to child at coordinate zero (xyz, wxyz); identity for a root */
+    float axis[3];                  /* in the child frame */
+} nuka_kinematic_link_t;
+nuka_result_t nuka_world_get_kinematic_link(nuka_world_handle world, uint32_t link_index, nuka_kinematic_link_t* out);
+typedef struct nuka_link_binding_t {
+    uint32_t body_index;            /* the link's own collidable row, UINT32_MAX without one */
+    uint32_t articulation_index;
+    uint32_t is_root;
+    uint32_t is_floating;
+} nuka_link_binding_t;
+nuka_result_t nuka_world_get_link_binding(nuka_world_handle world, uint32_t link_index, nuka_link_binding_t* out);
+/* One collision shape of the template with its pose in an environment now (xyz, wxyz): a link's shape follows the
+ * link's pose of the last forward kinematics, any other row its own body pose. */
+typedef struct nuka_collider_t {
+    uint32_t kind;
+    uint32_t is_static;
+    float params[4];
+    float pose[7];
+} nuka_collider_t;
+/* `out` null: *out_count = rows only; a capacity below the rows or an environment out of range is INVALID_ARG */
+nuka_result_t nuka_world_get_colliders(nuka_world_handle world, uint32_t env_index, nuka_collider_t* out, uint32_t capacity,
+                                       uint32_t* out_count);
+
 /* Counts of the cooked world. */
 typedef struct nuka_world_info_t {
     uint32_t env_count, links_per_env, bodies_per_env, dof, max_dof, contact_slots_per_env, rows_per_env, op_count;

@@ -56,6 +56,39 @@ class ExecutionInfoC(C.Structure):
                 ("native_error", C.c_int32), ("message", C.c_char * 256)]
 
 
+class VersionC(C.Structure):
+    """nuka_version_t"""
+    _fields_ = [("major", C.c_uint16), ("minor", C.c_uint16), ("patch", C.c_uint16)]
+
+
+class RuntimeInfoC(C.Structure):
+    """nuka_runtime_info_t"""
+    _fields_ = [("struct_size", C.c_uint32), ("schema_version", C.c_uint32), ("cuda_runtime_version", C.c_int32),
+                ("cuda_driver_version", C.c_int32)]
+
+
+class SolverOptionsC(C.Structure):
+    """nuka_solver_options_t"""
+    _fields_ = [("cone", C.c_uint32), ("integrator", C.c_uint32), ("impratio", C.c_float), ("refsafe", C.c_uint32)]
+
+
+class KinematicLinkC(C.Structure):
+    """nuka_kinematic_link_t"""
+    _fields_ = [("parent_index", C.c_uint32), ("articulation_index", C.c_uint32), ("joint_type", C.c_int), ("local_pose", C.c_float * 7),
+                ("axis", C.c_float * 3)]
+
+
+class LinkBindingC(C.Structure):
+    """nuka_link_binding_t"""
+    _fields_ = [(n, C.c_uint32) for n in ("body_index", "articulation_index", "is_root", "is_floating")]
+
+
+class ColliderC(C.Structure):
+    """nuka_collider_t"""
+    _fields_ = [("kind", C.c_uint32), ("is_static", C.c_uint32), ("params", C.c_float * 4), ("pose", C.c_float * 7)]
+
+
+KINEMATIC_ROOT, KINEMATIC_FIXED, KINEMATIC_REVOLUTE, KINEMATIC_PRISMATIC = 0, 1, 2, 3
 PARAM_INFO_VERSION = 1
 PARAM_LIVE, PARAM_REBUILD = 0, 1
 PARAMS = ("gravity_z", "velocity_iterations", "link_mass", "joint_damping", "joint_armature", "joint_frictionloss", "drive_stiffness",
@@ -83,6 +116,8 @@ EXPORTS = [
     "nuka_checkpoint_equal", "nuka_world_state_hash", "nuka_world_forward_kinematics", "nuka_world_param_count", "nuka_world_get_param_infos",
     "nuka_world_get_param", "nuka_world_set_param", "nuka_world_set_link_mass", "nuka_world_set_gravity_z",
     "nuka_checkpoint_write", "nuka_world_checkpoint_read", "nuka_world_get_execution_info",
+    "nuka_get_version", "nuka_get_runtime_info", "nuka_world_get_stream", "nuka_world_record_event", "nuka_world_get_solver_options",
+    "nuka_world_get_dof_name", "nuka_world_get_kinematic_link", "nuka_world_get_link_binding", "nuka_world_get_colliders",
 ]
 
 
@@ -162,6 +197,15 @@ def lib():
         L.nuka_checkpoint_write.argtypes = [C.c_void_p, C.c_char_p]
         L.nuka_world_checkpoint_read.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]
         L.nuka_world_get_execution_info.argtypes = [C.c_void_p, C.POINTER(ExecutionInfoC)]
+        L.nuka_get_version.restype = VersionC
+        L.nuka_get_runtime_info.argtypes = [C.POINTER(RuntimeInfoC)]
+        L.nuka_world_get_stream.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        L.nuka_world_record_event.argtypes = [C.c_void_p, C.c_void_p]
+        L.nuka_world_get_solver_options.argtypes = [C.c_void_p, C.POINTER(SolverOptionsC)]
+        L.nuka_world_get_dof_name.argtypes = [C.c_void_p, C.c_uint32, C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t)]
+        L.nuka_world_get_kinematic_link.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(KinematicLinkC)]
+        L.nuka_world_get_link_binding.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(LinkBindingC)]
+        L.nuka_world_get_colliders.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(ColliderC), C.c_uint32, C.POINTER(C.c_uint32)]
         _lib = L
     return _lib
 
@@ -169,6 +213,19 @@ def lib():
 def _check(code):
     if code != 0:
         raise NukaError(code, lib().nuka_last_error_message().decode() or lib().nuka_result_message(code).decode())
+
+
+def version():
+    """nuka_get_version as (major, minor, patch)."""
+    v = lib().nuka_get_version()
+    return v.major, v.minor, v.patch
+
+
+def runtime_info():
+    """nuka_get_runtime_info: the HIP runtime and driver versions in the reference's record."""
+    info = RuntimeInfoC(C.sizeof(RuntimeInfoC), 1, 0, 0)
+    _check(lib().nuka_get_runtime_info(C.byref(info)))
+    return info
 
 
 class Device:
@@ -385,6 +442,47 @@ class World:
         info.struct_size, info.schema_version = C.sizeof(ExecutionInfoC), 1
         _check(lib().nuka_world_get_execution_info(self._h, C.byref(info)))
         return info
+
+    def stream(self):
+        """nuka_world_get_stream: the hipStream_t the world executes on, as an integer address."""
+        out = C.c_void_p()
+        _check(lib().nuka_world_get_stream(self._h, C.byref(out)))
+        return out.value
+
+    def record_event(self, event):
+        """nuka_world_record_event: records the caller's hipEvent_t (an address) after the work submitted so far."""
+        _check(lib().nuka_world_record_event(self._h, C.c_void_p(event)))
+
+    def solver_options(self):
+        out = SolverOptionsC()
+        _check(lib().nuka_world_get_solver_options(self._h, C.byref(out)))
+        return out
+
+    def dof_name(self, link_index):
+        """nuka_world_get_dof_name by its two calls: the size query, then the name."""
+        length = C.c_size_t()
+        _check(lib().nuka_world_get_dof_name(self._h, link_index, None, 0, C.byref(length)))
+        buffer = C.create_string_buffer(length.value + 1)
+        _check(lib().nuka_world_get_dof_name(self._h, link_index, buffer, length.value + 1, C.byref(length)))
+        return buffer.value.decode()
+
+    def kinematic_link(self, link_index):
+        out = KinematicLinkC()
+        _check(lib().nuka_world_get_kinematic_link(self._h, link_index, C.byref(out)))
+        return out
+
+    def link_binding(self, link_index):
+        out = LinkBindingC()
+        _check(lib().nuka_world_get_link_binding(self._h, link_index, C.byref(out)))
+        return out
+
+    def colliders(self, env_index):
+        """nuka_world_get_colliders: the count query, then the records of one environment."""
+        count = C.c_uint32()
+        _check(lib().nuka_world_get_colliders(self._h, env_index, None, 0, C.byref(count)))
+        records = (ColliderC * max(count.value, 1))()
+        _check(lib().nuka_world_get_colliders(self._h, env_index, records, count.value, C.byref(count)))
+        return list(records)[:count.value]
 
     def param_infos(self):
         """nuka_world_get_param_infos as a list of dicts, in parameter order."""

@@ -464,6 +464,8 @@ struct World {   // src/c_abi/internal.hpp:153-165 WorldRecord + nk::World
     std::vector<float> drive_stiffness, drive_force_limit;   // per template link: what nuka_world_get_param reports
     uint64_t capture_attempts = 0u, graph_replays = 0u;      // nuka_world_get_execution_info
     uint64_t param_version = 0u;   // counts the calls that may have changed a live parameter: a checkpoint taken at the current count holds the current values
+    bool from_scene = false;                            // created from a scene file: the names below are the file's
+    std::vector<std::string> link_names, joint_names;   // per template link; a joint's name sits at its child link
     nuka_phi_execution_error last_error{};
 
     ~World() {
@@ -985,6 +987,7 @@ nuka_result_t CreateWorld(nuka_device_handle device, const nuka_template_desc_t*
             if (hc.drive_mode == kDrivePdPosition) ok = ok && put(w.data.drive_target, tile(scene->initial_q));   // hold the authored pose
             if (!ok) return Error(NUKA_RESULT_DEVICE_ERROR, "scene state upload failed");
         }
+        if (scene != nullptr) { w.from_scene = true; w.link_names = scene->link_names; w.joint_names = scene->joint_names; }
         BuildPipeline(w);
         // nk/pipeline/world.cpp:553-561: creation exposes the poses of the initial state and the reference weights at
         // them.  Only the MuJoCo contact law reads the weights; other worlds first compute their poses in their first step.
@@ -1375,7 +1378,7 @@ void DataShape(size_t count, uint8_t* per, uint32_t* scalars) {
     else *per = NUKA_HIP_PER_ENV;
     *scalars = uint32_t(rest);
 }
-const std::vector<ViewField>& ViewFields() {
+extern "C++" const std::vector<ViewField>& ViewFields() {   // (a C++ return type: not a C function, though the file's entry points around it are)
     static const std::vector<ViewField> fields = [] {
         std::vector<ViewField> out;
 #define X(field, dtype) { uint8_t per = NUKA_HIP_PER_SCALAR; uint32_t scalars = 0u; \
@@ -1581,6 +1584,172 @@ nuka_result_t nuka_world_get_info(nuka_world_handle world, nuka_world_info_t* ou
     *out = {w->env_count, m.links_per_env, m.bodies_per_env, m.dof, m.max_dof, m.contact_slots, m.rows_per_env, uint32_t(w->calls.size()),
             SolverSweepWidth(m), SolverBlocksPerUnit(m, w->env_count)};
     return NUKA_RESULT_OK;
+}
+
+nuka_version_t nuka_get_version(void) { return {0u, 1u, 0u}; }   // src/c_abi/error.cpp:69-72
+
+nuka_result_t nuka_get_runtime_info(nuka_runtime_info_t* out) {   // src/c_abi/cuda_interop.cpp:40-56
+    if (out == nullptr || out->struct_size != sizeof(*out) || out->schema_version != NUKA_RUNTIME_INFO_VERSION) return NUKA_RESULT_INVALID_ARG;
+    *out = {};
+    out->struct_size = sizeof(*out);
+    out->schema_version = NUKA_RUNTIME_INFO_VERSION;
+    int runtime_version = 0, driver_version = 0;
+    if (hipRuntimeGetVersion(&runtime_version) != hipSuccess || hipDriverGetVersion(&driver_version) != hipSuccess) return NUKA_RESULT_DEVICE_ERROR;
+    out->cuda_runtime_version = runtime_version;
+    out->cuda_driver_version = driver_version;
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_get_stream(nuka_world_handle world, void** out_stream) {   // cuda_interop.cpp:20-28
+    if (out_stream == nullptr) return NUKA_RESULT_INVALID_ARG;
+    *out_stream = nullptr;
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    *out_stream = BackendStream(w->device->backend);
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_record_event(nuka_world_handle world, void* cuda_event) {   // cuda_interop.cpp:30-38
+    if (cuda_event == nullptr) return NUKA_RESULT_INVALID_ARG;
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    return hipEventRecord(static_cast<hipEvent_t>(cuda_event), BackendStream(w->device->backend)) == hipSuccess
+               ? NUKA_RESULT_OK : Error(NUKA_RESULT_DEVICE_ERROR, "event record failed");
+}
+
+nuka_result_t nuka_world_get_solver_options(nuka_world_handle world, nuka_solver_options_t* out) {   // world.cpp:759-768
+    if (out == nullptr) return NUKA_RESULT_INVALID_ARG;
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    // the template's integrator 0 (native) and 1 (MuJoCo's Euler) are both Euler steps; 2 runs implicitfast
+    *out = {w->model.contact_cone, w->model.integrator == 2u ? 3u : 0u, w->model.contact_impratio, 1u};
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_get_dof_name(nuka_world_handle world, uint32_t link_index, char* out, size_t cap, size_t* out_len) {   // world.cpp:1170-1225
+    if (out_len != nullptr) *out_len = 0u;
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (!w->from_scene) return Error(NUKA_RESULT_NOT_SUPPORTED, "the world was not created from a scene file: its links have no names");
+    const uint32_t nl = w->model.links_per_env;
+    if (uint64_t{link_index} >= uint64_t{nl} * w->env_count) return Error(NUKA_RESULT_INVALID_ARG, "link index out of range");
+    const uint32_t l = link_index % nl;
+    std::string name = l < w->joint_names.size() ? w->joint_names[l] : std::string();
+    if (name.empty() && l < w->link_names.size()) name = w->link_names[l];
+    if (out_len != nullptr) *out_len = name.size();
+    if (out == nullptr) return NUKA_RESULT_OK;   // size query
+    if (name.size() + 1u > cap) return Error(NUKA_RESULT_INVALID_ARG, "the buffer cannot hold the name and its terminator");
+    std::memcpy(out, name.c_str(), name.size() + 1u);
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_get_kinematic_link(nuka_world_handle world, uint32_t link_index, nuka_kinematic_link_t* out) {   // world.cpp:1227-1276
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (out == nullptr) return NUKA_RESULT_INVALID_ARG;
+    const HostModel& h = w->host;
+    if (link_index >= w->model.links_per_env) return Error(NUKA_RESULT_INVALID_ARG, "link index out of range");
+    nuka_kinematic_link_t result{};
+    result.parent_index = h.parent_link[link_index];
+    result.articulation_index = 0u;
+    result.local_pose[3] = 1.0f;
+    if (result.parent_index == kInvalid) {
+        result.joint_type = NUKA_KINEMATIC_ROOT;
+    } else {
+        switch (h.joint_type[link_index]) {
+            case kFixed: result.joint_type = NUKA_KINEMATIC_FIXED; break;
+            case kRevolute: result.joint_type = NUKA_KINEMATIC_REVOLUTE; break;
+            case kPrismatic: result.joint_type = NUKA_KINEMATIC_PRISMATIC; break;
+            default: return Error(NUKA_RESULT_NOT_SUPPORTED, "joint type without a kinematic record");
+        }
+        const float* local = h.link_local_pose.data() + 7u * link_index;
+        for (int k = 0; k < 3; ++k) result.local_pose[k] = local[k] + h.parent_offset[3u * link_index + k];
+        for (int k = 3; k < 7; ++k) result.local_pose[k] = local[k];
+        for (int k = 0; k < 3; ++k) result.axis[k] = h.joint_axis[3u * link_index + k];
+    }
+    *out = result;
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_get_link_binding(nuka_world_handle world, uint32_t link_index, nuka_link_binding_t* out) {   // world.cpp:1278-1294
+    if (out == nullptr) return NUKA_RESULT_INVALID_ARG;
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    const HostModel& h = w->host;
+    if (link_index >= w->model.links_per_env) return Error(NUKA_RESULT_INVALID_ARG, "link index out of range");
+    out->body_index = h.link_body[link_index];
+    out->articulation_index = 0u;
+    out->is_root = h.parent_link[link_index] == kInvalid ? 1u : 0u;
+    out->is_floating = out->is_root != 0u && h.joint_type[link_index] == kFloatingBase ? 1u : 0u;
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_get_colliders(nuka_world_handle world, uint32_t env_index, nuka_collider_t* out, uint32_t capacity,
+                                       uint32_t* out_count) {   // world.cpp:1345-1413
+    if (out_count == nullptr) return NUKA_RESULT_INVALID_ARG;
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    const HostModel& h = w->host;
+    const uint32_t nb = w->model.bodies_per_env, nl = w->model.links_per_env;
+    *out_count = nb;
+    if (out == nullptr) return NUKA_RESULT_OK;
+    if (capacity < nb || env_index >= w->env_count) return Error(NUKA_RESULT_INVALID_ARG, "capacity below the shape rows, or environment out of range");
+    try {
+        std::vector<float> body_pose(size_t{nb} * 7u), link_pose(size_t{nl} * 7u);
+        const nuka_result_t synced = nuka_world_synchronize(world);
+        if (synced != NUKA_RESULT_OK) return synced;
+        auto fetch = [&](const float* field, std::vector<float>& host, uint32_t per_env) {
+            if (per_env == 0u) return true;
+            const char* base = static_cast<const char*>(Iface(w->arena)->base(w->arena));
+            const size_t offset = size_t(reinterpret_cast<const char*>(field) - base) + size_t{env_index} * per_env * sizeof(float);
+            return Iface(w->arena)->download(w->arena, host.data(), offset, size_t{per_env} * sizeof(float)) == uint8_t(Status::Ok);
+        };
+        if (!fetch(w->data.body_pose, body_pose, nb * 7u) || !fetch(w->data.link_pose, link_pose, nl * 7u)) return Error(NUKA_RESULT_INTERNAL, "pose download failed");
+        // parent * child: the child's origin carried by the parent, the rotations multiplied and normalised (math/transform.hpp:37-42)
+        auto compose = [](const float* parent, const float* child, float* result) {
+            const float w0 = parent[3], x0 = parent[4], y0 = parent[5], z0 = parent[6];
+            const float v[3] = {child[0], child[1], child[2]};
+            const float t[3] = {2.0f * (y0 * v[2] - z0 * v[1]), 2.0f * (z0 * v[0] - x0 * v[2]), 2.0f * (x0 * v[1] - y0 * v[0])};
+            result[0] = parent[0] + v[0] + w0 * t[0] + (y0 * t[2] - z0 * t[1]);
+            result[1] = parent[1] + v[1] + w0 * t[1] + (z0 * t[0] - x0 * t[2]);
+            result[2] = parent[2] + v[2] + w0 * t[2] + (x0 * t[1] - y0 * t[0]);
+            const float w1 = child[3], x1 = child[4], y1 = child[5], z1 = child[6];
+            float q[4] = {w0 * w1 - x0 * x1 - y0 * y1 - z0 * z1, w0 * x1 + x0 * w1 + y0 * z1 - z0 * y1,
+                          w0 * y1 - x0 * z1 + y0 * w1 + z0 * x1, w0 * z1 + x0 * y1 - y0 * x1 + z0 * w1};
+            const float norm = std::sqrt(q[0] * q[0] + q[1] * q[1] + q[2] * q[2] + q[3] * q[3]);
+            for (int k = 0; k < 4; ++k) result[3 + k] = norm > 0.0f ? q[k] / norm : (k == 0 ? 1.0f : 0.0f);
+        };
+        for (uint32_t row = 0u; row < nb; ++row) {
+            const float* shape = h.shape_table.data() + size_t{row} * kShapeStride;
+            nuka_collider_t& collider = out[row];
+            std::memcpy(&collider.kind, shape, sizeof(uint32_t));
+            std::memcpy(collider.params, shape + 1, 4u * sizeof(float));
+            int32_t body_id;
+            std::memcpy(&body_id, shape + 8, sizeof(body_id));
+            float pose[7] = {0.0f, 0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 0.0f};
+            bool is_static = true;
+            if (body_id >= 0) {
+                const uint32_t body = uint32_t(body_id);
+                const uint32_t link = body < h.body_to_link.size() ? h.body_to_link[body] : kInvalid;
+                const uint32_t owner = body < h.body_collidable_link.size() ? h.body_collidable_link[body] : kInvalid;
+                if (link != kInvalid || owner != kInvalid) {
+                    // a link's own row hangs off the link by the link's shape frame, a further row of a link by its own
+                    if (owner != kInvalid) compose(link_pose.data() + 7u * owner, h.body_collidable_local.data() + 7u * body, pose);
+                    else compose(link_pose.data() + 7u * link, h.link_geom_local.data() + 7u * link, pose);
+                    is_static = false;
+                } else {
+                    std::memcpy(pose, body_pose.data() + 7u * body, sizeof(pose));
+                }
+            } else if (row < nb) {
+                std::memcpy(pose, body_pose.data() + 7u * row, sizeof(pose));
+            }
+            collider.is_static = is_static ? 1u : 0u;
+            std::memcpy(collider.pose, pose, sizeof(pose));
+        }
+        return NUKA_RESULT_OK;
+    } catch (const std::bad_alloc&) {
+        return Error(NUKA_RESULT_OUT_OF_MEMORY, "host allocation failed");
+    }
 }
 
 nuka_result_t nuka_world_time_steps(nuka_world_handle world, nuka_checkpoint_handle from, uint32_t step_count, float* out_total_ms) {
