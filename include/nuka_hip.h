@@ -526,6 +526,36 @@ typedef struct nuka_collider_t {
 nuka_result_t nuka_world_get_colliders(nuka_world_handle world, uint32_t env_index, nuka_collider_t* out, uint32_t capacity,
                                        uint32_t* out_count);
 
+/* Memory and execution figures (nuka.h:343-374; src/c_abi/device.cpp:101-108, world.cpp:910-990), through the backend's
+ * own resource_info and plan_metrics entries.  A null handle or out pointer is refused here (NULL_HANDLE, INVALID_ARG). */
+typedef struct nuka_device_resource_info_t {
+    uint64_t free_bytes, total_bytes, thread_stack_limit_bytes;
+    uint64_t graph_used_bytes, graph_reserved_bytes;
+    uint32_t compute_units, threads_per_unit;
+} nuka_device_resource_info_t;
+typedef struct nuka_world_resource_info_t {
+    uint64_t model_bytes, persistent_bytes, scratch_bytes;   /* the template's tables; what a checkpoint keeps; the rest of the arena */
+    uint32_t env_count, contacts_per_env, rows_per_env, dofs_per_articulation;
+    uint32_t bodies_per_env, particles_per_env;              /* particles: always 0 on this path */
+} nuka_world_resource_info_t;
+typedef struct nuka_resource_field_t {
+    char name[64];           /* the reference's field name where it has one, else this library's */
+    uint64_t offset, bytes;  /* place in the world's one arena */
+    uint32_t owner, arena;   /* owner 0: the template (model), 1: per-environment data; arena 0 persistent, 1 scratch */
+} nuka_resource_field_t;
+typedef struct nuka_execution_window_t {
+    double gpu_ms;           /* device time between begin and end on the world's stream */
+    uint64_t graph_replays, nodes, kernels, clears, copies;   /* replays inside the window; the captured graph's make-up */
+} nuka_execution_window_t;
+nuka_result_t nuka_device_get_resource_info(nuka_device_handle device, nuka_device_resource_info_t* out);
+nuka_result_t nuka_world_get_resource_info(nuka_world_handle world, nuka_world_resource_info_t* out);
+uint32_t nuka_world_resource_field_count(nuka_world_handle world);
+/* the caller allocates nuka_world_resource_field_count entries */
+nuka_result_t nuka_world_get_resource_fields(nuka_world_handle world, nuka_resource_field_t* out);
+nuka_result_t nuka_world_begin_execution_window(nuka_world_handle world, void** window);
+/* ends and frees the window; waits for the work inside it */
+nuka_result_t nuka_world_end_execution_window(nuka_world_handle world, void* window, nuka_execution_window_t* out);
+
 /* Counts of the cooked world. */
 typedef struct nuka_world_info_t {
     uint32_t env_count, links_per_env, bodies_per_env, dof, max_dof, contact_slots_per_env, rows_per_env, op_count;

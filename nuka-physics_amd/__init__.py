@@ -88,6 +88,29 @@ class ColliderC(C.Structure):
     _fields_ = [("kind", C.c_uint32), ("is_static", C.c_uint32), ("params", C.c_float * 4), ("pose", C.c_float * 7)]
 
 
+class DeviceResourceInfoC(C.Structure):
+    """nuka_device_resource_info_t"""
+    _fields_ = [(n, C.c_uint64) for n in ("free_bytes", "total_bytes", "thread_stack_limit_bytes", "graph_used_bytes",
+                                          "graph_reserved_bytes")] + [("compute_units", C.c_uint32), ("threads_per_unit", C.c_uint32)]
+
+
+class WorldResourceInfoC(C.Structure):
+    """nuka_world_resource_info_t"""
+    _fields_ = [(n, C.c_uint64) for n in ("model_bytes", "persistent_bytes", "scratch_bytes")] + \
+               [(n, C.c_uint32) for n in ("env_count", "contacts_per_env", "rows_per_env", "dofs_per_articulation", "bodies_per_env",
+                                          "particles_per_env")]
+
+
+class ResourceFieldC(C.Structure):
+    """nuka_resource_field_t"""
+    _fields_ = [("name", C.c_char * 64), ("offset", C.c_uint64), ("bytes", C.c_uint64), ("owner", C.c_uint32), ("arena", C.c_uint32)]
+
+
+class ExecutionWindowC(C.Structure):
+    """nuka_execution_window_t"""
+    _fields_ = [("gpu_ms", C.c_double)] + [(n, C.c_uint64) for n in ("graph_replays", "nodes", "kernels", "clears", "copies")]
+
+
 KINEMATIC_ROOT, KINEMATIC_FIXED, KINEMATIC_REVOLUTE, KINEMATIC_PRISMATIC = 0, 1, 2, 3
 PARAM_INFO_VERSION = 1
 PARAM_LIVE, PARAM_REBUILD = 0, 1
@@ -118,6 +141,8 @@ EXPORTS = [
     "nuka_checkpoint_write", "nuka_world_checkpoint_read", "nuka_world_get_execution_info",
     "nuka_get_version", "nuka_get_runtime_info", "nuka_world_get_stream", "nuka_world_record_event", "nuka_world_get_solver_options",
     "nuka_world_get_dof_name", "nuka_world_get_kinematic_link", "nuka_world_get_link_binding", "nuka_world_get_colliders",
+    "nuka_device_get_resource_info", "nuka_world_get_resource_info", "nuka_world_resource_field_count", "nuka_world_get_resource_fields",
+    "nuka_world_begin_execution_window", "nuka_world_end_execution_window",
 ]
 
 
@@ -206,6 +231,13 @@ def lib():
         L.nuka_world_get_kinematic_link.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(KinematicLinkC)]
         L.nuka_world_get_link_binding.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(LinkBindingC)]
         L.nuka_world_get_colliders.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(ColliderC), C.c_uint32, C.POINTER(C.c_uint32)]
+        L.nuka_device_get_resource_info.argtypes = [C.c_void_p, C.POINTER(DeviceResourceInfoC)]
+        L.nuka_world_get_resource_info.argtypes = [C.c_void_p, C.POINTER(WorldResourceInfoC)]
+        L.nuka_world_resource_field_count.argtypes = [C.c_void_p]
+        L.nuka_world_resource_field_count.restype = C.c_uint32
+        L.nuka_world_get_resource_fields.argtypes = [C.c_void_p, C.POINTER(ResourceFieldC)]
+        L.nuka_world_begin_execution_window.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        L.nuka_world_end_execution_window.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(ExecutionWindowC)]
         _lib = L
     return _lib
 
@@ -240,6 +272,12 @@ class Device:
         if self._h:
             lib().nuka_device_destroy(self._h)
             self._h = C.c_void_p()
+
+    def resource_info(self):
+        """nuka_device_get_resource_info: free and total device memory, compute units and threads a unit."""
+        out = DeviceResourceInfoC()
+        _check(lib().nuka_device_get_resource_info(self._h, C.byref(out)))
+        return out
 
     def copy_bandwidth(self, nbytes=1 << 30, repeats=10):
         out = C.c_float()
@@ -442,6 +480,27 @@ class World:
         info.struct_size, info.schema_version = C.sizeof(ExecutionInfoC), 1
         _check(lib().nuka_world_get_execution_info(self._h, C.byref(info)))
         return info
+
+    def resource_info(self):
+        out = WorldResourceInfoC()
+        _check(lib().nuka_world_get_resource_info(self._h, C.byref(out)))
+        return out
+
+    def resource_fields(self):
+        """nuka_world_get_resource_fields: every field's place in the world's arena."""
+        records = (ResourceFieldC * max(lib().nuka_world_resource_field_count(self._h), 1))()
+        _check(lib().nuka_world_get_resource_fields(self._h, records))
+        return list(records)[:lib().nuka_world_resource_field_count(self._h)]
+
+    def begin_execution_window(self):
+        window = C.c_void_p()
+        _check(lib().nuka_world_begin_execution_window(self._h, C.byref(window)))
+        return window
+
+    def end_execution_window(self, window):
+        out = ExecutionWindowC()
+        _check(lib().nuka_world_end_execution_window(self._h, window, C.byref(out)))
+        return out
 
     def stream(self):
         """nuka_world_get_stream: the hipStream_t the world executes on, as an integer address."""

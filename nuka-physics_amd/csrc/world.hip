@@ -1752,6 +1752,104 @@ nuka_result_t nuka_world_get_colliders(nuka_world_handle world, uint32_t env_ind
     }
 }
 
+nuka_result_t nuka_device_get_resource_info(nuka_device_handle device, nuka_device_resource_info_t* out) {   // src/c_abi/device.cpp:101-108
+    auto* record = reinterpret_cast<DeviceRecord*>(device);
+    if (record == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "device is null");
+    if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    auto* backend = reinterpret_cast<nuka_phi_backend*>(record->backend);
+    const nuka_phi_resource_info info = reinterpret_cast<nuka_phi_backend_head*>(backend)->iface->resource_info(backend);
+    *out = {info.free_bytes, info.total_bytes, info.thread_stack_limit_bytes, info.graph_used_bytes, info.graph_reserved_bytes,
+            info.compute_units, info.threads_per_unit};
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_get_resource_info(nuka_world_handle world, nuka_world_resource_info_t* out) {   // src/c_abi/world.cpp:917-929
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    uint64_t model = 0u, persistent = 0u, scratch = 0u;
+    for (const Field& f : w->fields) {
+        const uint64_t bytes = (uint64_t{f.count} * f.elem_bytes + 255u) & ~uint64_t{255u};   // as the arena places it
+        (f.is_template ? model : CheckpointKeeps(f.name) ? persistent : scratch) += bytes;
+    }
+    const ModelView& m = w->model;
+    *out = {model, persistent, scratch, w->env_count, m.contact_slots, m.rows_per_env, m.dof, m.bodies_per_env, 0u};
+    return NUKA_RESULT_OK;
+}
+
+uint32_t nuka_world_resource_field_count(nuka_world_handle world) {   // world.cpp:931-936
+    auto* w = reinterpret_cast<World*>(world);
+    return w == nullptr ? 0u : uint32_t(w->fields.size());
+}
+
+nuka_result_t nuka_world_get_resource_fields(nuka_world_handle world, nuka_resource_field_t* out) {   // world.cpp:938-959
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "out is null");
+    uint32_t index = 0u;
+    for (const bool template_pass : {true, false})   // the model's fields first, as the reference lists them
+        for (const Field& f : w->fields) {
+            if (f.is_template != template_pass) continue;
+            nuka_resource_field_t& field = out[index++];
+            const char* reference_name = ReferenceName(f.name);
+            std::snprintf(field.name, sizeof(field.name), "%s", reference_name != nullptr && reference_name[0] != '\0' ? reference_name : f.name);
+            field.offset = f.offset;
+            field.bytes = uint64_t{f.count} * f.elem_bytes;
+            field.owner = f.is_template ? 0u : 1u;
+            field.arena = f.is_template || CheckpointKeeps(f.name) ? 0u : 1u;
+        }
+    return NUKA_RESULT_OK;
+}
+
+namespace nkh {
+namespace {
+struct ExecutionWindow {   // world.cpp:910-914
+    nuka_phi_event* start;
+    nuka_phi_event* end;
+    uint64_t replays;
+    uint64_t owner_id;
+};
+}  // namespace
+}  // namespace nkh
+
+nuka_result_t nuka_world_begin_execution_window(nuka_world_handle world, void** window) {   // world.cpp:961-969
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    if (window == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "window is null");
+    *window = nullptr;
+    auto interval = std::make_unique<nkh::ExecutionWindow>();
+    interval->start = w->be->event_new(w->backend);
+    interval->end = w->be->event_new(w->backend);
+    if (interval->start == nullptr || interval->end == nullptr) {
+        if (interval->start != nullptr) w->be->event_free(w->backend, interval->start);
+        if (interval->end != nullptr) w->be->event_free(w->backend, interval->end);
+        return Error(NUKA_RESULT_DEVICE_ERROR, "event creation failed");
+    }
+    interval->replays = w->graph_replays;
+    interval->owner_id = w->id;
+    w->be->event_record(w->backend, interval->start);
+    *window = interval.release();
+    return NUKA_RESULT_OK;
+}
+
+nuka_result_t nuka_world_end_execution_window(nuka_world_handle world, void* window, nuka_execution_window_t* out) {   // world.cpp:971-990
+    auto* w = reinterpret_cast<World*>(world);
+    if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");
+    auto* interval = static_cast<nkh::ExecutionWindow*>(window);
+    if (interval == nullptr || out == nullptr) return Error(NUKA_RESULT_INVALID_ARG, "window and out are required");
+    if (interval->owner_id != w->id) return Error(NUKA_RESULT_INVALID_ARG, "the window was opened on another world");
+    w->be->event_record(w->backend, interval->end);
+    const uint8_t waited = w->be->synchronize(w->backend, nullptr);   // the elapsed time exists once the end event has completed
+    nuka_phi_plan_metrics metrics{};
+    if (w->plan != nullptr) metrics = w->be->plan_metrics(w->backend, w->plan);
+    *out = {double(w->be->event_elapsed_ms(w->backend, interval->start, interval->end)), w->graph_replays - interval->replays, metrics.nodes,
+            metrics.kernels, metrics.clears, metrics.copies};
+    w->be->event_free(w->backend, interval->start);
+    w->be->event_free(w->backend, interval->end);
+    delete interval;
+    return waited == uint8_t(Status::Ok) ? NUKA_RESULT_OK : Error(NUKA_RESULT_DEVICE_ERROR, "device error inside the window");
+}
+
 nuka_result_t nuka_world_time_steps(nuka_world_handle world, nuka_checkpoint_handle from, uint32_t step_count, float* out_total_ms) {
     auto* w = reinterpret_cast<World*>(world);
     if (w == nullptr) return Error(NUKA_RESULT_NULL_HANDLE, "world is null");

@@ -209,3 +209,82 @@ def test_colliders_carry_the_shape_table_and_the_live_poses(device):
     assert L.nuka_world_get_colliders(world._h, 0, records, nb, None) == INVALID_ARG
     assert L.nuka_world_get_colliders(None, 0, records, nb, C.byref(count)) == NULL_HANDLE
     world.close(); scene.close()
+
+
+def test_resource_records_add_up_to_the_arena(device):
+    """nuka_device_get_resource_info, nuka_world_get_resource_info and the field list (nuka.h:343-371): the fields tile
+    the world's one arena without overlap, their sums are the three totals, and the counts are the world's."""
+    gpu = device.resource_info()
+    assert gpu.total_bytes >= 200 << 30 and 0 < gpu.free_bytes <= gpu.total_bytes      # an MI355X: 288 GB of HBM
+    assert gpu.compute_units == 256 and gpu.threads_per_unit >= 1024
+    E = 64
+    cfg = nk.synthetic.config(3, E)
+    before = device.resource_info().free_bytes
+    world = nk.World(device, cfg.template, abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters))
+    info = world.resource_info()
+    assert (info.env_count, info.rows_per_env, info.dofs_per_articulation, info.bodies_per_env, info.particles_per_env) == \
+           (E, world.rows_per_env, world.dof, world.info.bodies_per_env, 0)
+    assert info.contacts_per_env == world.info.contact_slots_per_env
+    fields = world.resource_fields()
+    assert len(fields) == nk.lib().nuka_world_resource_field_count(world._h) > 100
+    names = [f.name.decode() for f in fields]
+    assert len(set(names)) == len(names)
+    for expected in ("q", "qdot", "link_pose", "m", "m_factor", "lambda", "urows", "chain_jacobian", "parent_link", "link_inertia"):
+        assert expected in names, expected
+    # the model's tables come first, then the data; placed ranges do not overlap
+    owners = [f.owner for f in fields]
+    assert owners == sorted(owners) and set(owners) == {0, 1}
+    placed = sorted((f.offset, f.offset + f.bytes) for f in fields if f.bytes)
+    assert all(a_end <= b_start for (_, a_end), (b_start, _) in zip(placed, placed[1:]))
+    pad = lambda n: (n + 255) & ~255
+    assert sum(pad(f.bytes) for f in fields if f.owner == 0) == info.model_bytes
+    assert sum(pad(f.bytes) for f in fields if f.owner == 1 and f.arena == 0) == info.persistent_bytes
+    assert sum(pad(f.bytes) for f in fields if f.owner == 1 and f.arena == 1) == info.scratch_bytes
+    by_name = {f.name.decode(): f for f in fields}
+    assert by_name["q"].bytes == E * world.link_count * 4 and by_name["q"].arena == 0      # state a checkpoint keeps
+    assert by_name["urows"].arena == 1                                                      # rebuilt every step
+    # the arena and its reset copy came out of the device's free memory
+    taken = before - device.resource_info().free_bytes
+    total = info.model_bytes + info.persistent_bytes + info.scratch_bytes
+    assert taken >= total
+    L = nk.lib()
+    assert L.nuka_world_get_resource_info(world._h, None) == INVALID_ARG
+    assert L.nuka_world_get_resource_info(None, C.byref(nk.WorldResourceInfoC())) == NULL_HANDLE
+    assert L.nuka_world_resource_field_count(None) == 0
+    assert L.nuka_device_get_resource_info(None, C.byref(nk.DeviceResourceInfoC())) == NULL_HANDLE
+    world.close()
+
+
+def test_an_execution_window_times_the_steps_inside_it(device):
+    """nuka_world_begin_execution_window / nuka_world_end_execution_window (src/c_abi/world.cpp:961-990): device time
+    and graph replays between the two calls, and the make-up of the captured graph."""
+    E = 1024
+    cfg = nk.synthetic.config(3, E)
+    world = nk.World(device, cfg.template, abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters))
+    world.set_state(cfg.state())
+    world.set_execution_mode(True)
+    world.step(3); world.synchronize()                     # the graph is captured
+    empty = world.end_execution_window(world.begin_execution_window())
+    assert empty.graph_replays == 0 and 0.0 <= empty.gpu_ms < 1.0
+    import time
+    started = time.perf_counter()
+    window = world.begin_execution_window()
+    world.step(10)
+    inside = world.end_execution_window(window)
+    wall_ms = (time.perf_counter() - started) * 1e3
+    assert inside.graph_replays == 10
+    assert inside.nodes >= 8 and inside.kernels >= 8       # a step is a graph of about a dozen kernels
+    assert 10 * 0.2 < inside.gpu_ms < 10 * 20.0            # ten humanoid steps: milliseconds, not microseconds or seconds
+    assert inside.gpu_ms <= wall_ms                        # the host waited for the window's end
+    eager = nk.World(device, cfg.template, abi.world_desc(E, cfg.dt, vel_iters=cfg.vel_iters))
+    window = eager.begin_execution_window()
+    eager.step(2)
+    plain = eager.end_execution_window(window)
+    assert plain.graph_replays == 0 and plain.nodes == 0 and plain.gpu_ms > 0.0
+    L = nk.lib()
+    other = world.begin_execution_window()
+    assert L.nuka_world_end_execution_window(eager._h, other, C.byref(nk.ExecutionWindowC())) == INVALID_ARG   # another world's window
+    world.end_execution_window(other)
+    assert L.nuka_world_begin_execution_window(world._h, None) == INVALID_ARG
+    assert L.nuka_world_end_execution_window(world._h, None, C.byref(nk.ExecutionWindowC())) == INVALID_ARG
+    world.close(); eager.close()
