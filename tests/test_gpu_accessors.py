@@ -181,9 +181,13 @@ def test_the_kinematic_records_rebuild_the_worlds_link_poses(device):
     world.close(); scene.close()
 
 
-def test_colliders_carry_the_shape_table_and_the_live_poses(device):
+FREE_BOX = os.path.join(ROOT, "tests", "data", "free_box.xml")
+
+
+@pytest.mark.parametrize("path", [WALKER, FREE_BOX], ids=["walker", "free_box"])
+def test_colliders_carry_the_shape_table_and_the_live_poses(device, path):
     E = 4
-    scene = nk.Scene(WALKER, 0)
+    scene = nk.Scene(path, 0)
     world = nk.World(device, scene, abi.world_desc(E, 0.0, gravity=(0.0, 0.0, 0.0), vel_iters=4))
     world.step(3)
     world.synchronize()
