@@ -734,6 +734,18 @@ template <bool kSinglePoint>
 __global__ void __launch_bounds__(64) NarrowphaseKernel(ModelView m, DataView d, NarrowphasePrimitivesParams p) {
     narrowphase_of_env<kSinglePoint>(m, d, p, blockIdx.x, threadIdx.x);
 }
+// Worlds of at most 32 slots an environment: `width` lanes (a power of two, at least the slots) an environment and
+// 64 / width environments a wavefront, so that a world of one or two slots does not leave 62 lanes of every wavefront
+// idle.  The same slot code; an environment's contact count is the sum over its lanes (integers: any order).
+template <bool kSinglePoint>
+__global__ void __launch_bounds__(64) NarrowphasePackedKernel(ModelView m, DataView d, NarrowphasePrimitivesParams p, uint32_t width) {
+    const uint32_t lane = threadIdx.x;
+    const uint32_t env = blockIdx.x * (64u / width) + lane / width, slot = lane % width;
+    uint32_t contacts = 0u;
+    if (env < p.env_count && slot < p.rigid_slot_cap) contacts = NarrowphaseSlot<kSinglePoint>(m, d, p, env, slot);
+    for (uint32_t o = width >> 1u; o != 0u; o >>= 1u) contacts += uint32_t(__shfl_xor(int(contacts), int(o), 64));
+    if (slot == 0u && env < p.env_count) d.contact_count[env] = contacts;
+}
 
 // What stands between the dynamics and the row assembly - the bodies' poses, their boxes, the candidate pairs, the
 // manifolds - as one kernel, one wavefront an environment: four kernels of about a launch's time each become one, running
@@ -1368,7 +1380,13 @@ Status OpNarrowphasePrimitives(const ModelView& m, const DataView& d, const void
     const auto* p = static_cast<const NarrowphasePrimitivesParams*>(params);
     if (p == nullptr) return Status::Failed;
     if (p->env_count == 0u || p->union_slot_count == 0u || p->rigid_slot_cap == 0u) return Status::Ok;
-    if (m.max_points_per_slot <= 1u) hipLaunchKernelGGL(NarrowphaseKernel<true>, dim3(p->env_count), dim3(64), 0, stream, m, d, *p);
+    if (p->rigid_slot_cap <= 32u) {
+        uint32_t width = 1u;
+        while (width < p->rigid_slot_cap) width <<= 1u;
+        const uint32_t blocks = (p->env_count + 64u / width - 1u) / (64u / width);
+        if (m.max_points_per_slot <= 1u) hipLaunchKernelGGL(NarrowphasePackedKernel<true>, dim3(blocks), dim3(64), 0, stream, m, d, *p, width);
+        else hipLaunchKernelGGL(NarrowphasePackedKernel<false>, dim3(blocks), dim3(64), 0, stream, m, d, *p, width);
+    } else if (m.max_points_per_slot <= 1u) hipLaunchKernelGGL(NarrowphaseKernel<true>, dim3(p->env_count), dim3(64), 0, stream, m, d, *p);
     else hipLaunchKernelGGL(NarrowphaseKernel<false>, dim3(p->env_count), dim3(64), 0, stream, m, d, *p);
     return hipGetLastError() == hipSuccess ? Status::Ok : Status::Failed;
 }
