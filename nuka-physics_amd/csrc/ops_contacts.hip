@@ -1003,13 +1003,18 @@ __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4, 4
         d.qdot_flat[size_t{env} * md + lane] = value;
     }
     __syncthreads();
-    // contact rows, one lane per slot (:453-801; speculative law, condim 3)
+    // contact rows (:453-801; speculative law, condim 3): a lane a slot where every slot has one point at most, else a
+    // lane a (slot, point) - a slot's points share nothing but the slot's own values, which each of their lanes works
+    // out for itself
     uint32_t active_rows = 0u;
     bool invalid_endpoint = false;
-    for (uint32_t slot = lane; slot < S; slot += kWave) {
+    const uint32_t fan = m.max_points_per_slot > 1u ? 4u : 1u;
+    for (uint32_t item = lane; item < S * fan; item += kWave) {
+        const uint32_t slot = item / fan, own_point = item - slot * fan;
         const size_t gid = size_t{env} * S + slot;
         const uint32_t base = range_first[slot], P = range_points[slot];
-        if (P == 0u) continue;
+        if (P == 0u || (fan > 1u && own_point >= P)) continue;
+        const bool slot_lane = own_point == 0u;   // the one lane that writes what belongs to the slot as a whole
         uint32_t n_active = P;
         const uint32_t local_a = d.ucontact_a[gid * 4u], local_b = d.ucontact_b[gid * 4u];
         ShapeRow sa{}, sb{};
@@ -1035,7 +1040,7 @@ __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4, 4
         const float mu1 = merged[0], mu2 = merged[1];
         const float* solref = merged + 2, *solimp = merged + 4;
         const float margin = merged[9];
-        d.contact_material[gid] = n_active > 0u ? merged_material_key(merged, law, m.contact_cone) : 0ull;   // :620-623
+        if (slot_lane) d.contact_material[gid] = n_active > 0u ? merged_material_key(merged, law, m.contact_cone) : 0ull;   // :620-623
         // a compliant row's weight is the sum of its two bodies' reference weights, a link's through its own collidable row (:595-597)
         float invweight = 0.0f;
         if (mujoco) {
@@ -1050,7 +1055,7 @@ __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4, 4
         V3 frame_axis{0, 0, 0};   // :601-605: a capsule on a plane aligns the pyramid with the capsule's axis
         if (pyramidal && sa.kind == 1u && sb.kind == 3u) frame_axis = make_prim(sa, load_xf(d.body_pose + (size_t{env} * m.bodies_per_env + local_a) * 7u)).cz;
         if (pyramidal && sb.kind == 1u && sa.kind == 3u) frame_axis = make_prim(sb, load_xf(d.body_pose + (size_t{env} * m.bodies_per_env + local_b) * 7u)).cz;
-        for (uint32_t pt = 0u; pt < P; ++pt) {
+        for (uint32_t pt = fan > 1u ? own_point : 0u; pt < (fan > 1u ? own_point + 1u : P); ++pt) {
             const size_t mp = gid * 4u + pt;
             // the velocity laws keep every point; a compliant point lives inside its margin (:625-626)
             const bool live = pt < n_active && pt < 4u && (!mujoco || d.ucontact_depth[mp] + margin > 0.0f);
